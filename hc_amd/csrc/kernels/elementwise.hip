@@ -1,0 +1,158 @@
+// Elementwise maps: c = a + b (fp32) and d = a * b + c (fp16 storage, fp32
+// arithmetic).  HBM-bound: every element is read once and written once.
+//
+// Flat kernels treat a contiguous tensor as one vector of 16-byte words.  A
+// workgroup owns VPT * 256 consecutive words; thread t takes words t, t+256,
+// ... so every wave-level access covers 1 KiB of consecutive bytes.  Workgroups
+// that lie wholly inside the array run without any bounds test (a scalar
+// branch); only the last workgroup predicates per word and finishes the
+// sub-word tail per element, so tail masking costs nothing on the bulk.
+#include "common.h"
+
+using namespace hcamd;
+
+namespace {
+constexpr int kThreads = 256;
+
+struct AddF32 {
+  using Vec = f32x4;
+  using Elem = float;
+  static constexpr int kElems = 4;
+  static constexpr int kInputs = 2;
+  static __device__ __forceinline__ Vec apply(const Vec *in) {
+    return in[0] + in[1];
+  }
+  static __device__ __forceinline__ Elem apply1(const Elem *in) {
+    return in[0] + in[1];
+  }
+};
+
+struct FmaF16 {
+  using Vec = f16x8;
+  using Elem = _Float16;
+  static constexpr int kElems = 8;
+  static constexpr int kInputs = 3;
+  static __device__ __forceinline__ Elem apply1(const Elem *in) {
+    // fp16 x fp16 is exact in fp32 (11+11 significand bits), so the rounding
+    // of the separate multiply never happens and mul+add equals a fused
+    // multiply-add; the only roundings are the fp32 add and the final
+    // fp32->fp16 conversion (nearest even).
+    return (_Float16)((float)in[0] * (float)in[1] + (float)in[2]);
+  }
+  static __device__ __forceinline__ Vec apply(const Vec *in) {
+    Vec r;
+#pragma unroll
+    for (int i = 0; i < kElems; ++i) {
+      Elem e[3] = {in[0][i], in[1][i], in[2][i]};
+      r[i] = apply1(e);
+    }
+    return r;
+  }
+};
+
+struct Ptrs3 {
+  const void *in[3];
+  void *out;
+};
+
+template <class Op, int VPT, bool NT>
+__device__ __forceinline__ void flat_map(const Ptrs3 &p, size_t n) {
+  using Vec = typename Op::Vec;
+  using Elem = typename Op::Elem;
+  const size_t nvec = n / Op::kElems;
+  const size_t first = (size_t)blockIdx.x * (kThreads * VPT) + threadIdx.x;
+  const Vec *in[Op::kInputs];
+#pragma unroll
+  for (int a = 0; a < Op::kInputs; ++a)
+    in[a] = static_cast<const Vec *>(p.in[a]);
+  Vec *out = static_cast<Vec *>(p.out);
+
+  if (((size_t)blockIdx.x + 1) * (kThreads * VPT) <= nvec) {
+    Vec v[VPT][Op::kInputs];
+#pragma unroll
+    for (int a = 0; a < Op::kInputs; ++a)
+#pragma unroll
+      for (int j = 0; j < VPT; ++j)
+        v[j][a] = ldg<NT>(in[a] + first + (size_t)j * kThreads);
+#pragma unroll
+    for (int j = 0; j < VPT; ++j)
+      stg<NT>(out + first + (size_t)j * kThreads, Op::apply(v[j]));
+    return;
+  }
+
+  // Last workgroup: per-word predicate, then the elements past the last
+  // whole word, one per thread.
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const size_t w = first + (size_t)j * kThreads;
+    if (w < nvec) {
+      Vec v[Op::kInputs];
+#pragma unroll
+      for (int a = 0; a < Op::kInputs; ++a)
+        v[a] = in[a][w];
+      out[w] = Op::apply(v);
+    }
+  }
+  const size_t e = nvec * Op::kElems + threadIdx.x;
+  if (threadIdx.x < Op::kElems && e < n) {
+    Elem s[Op::kInputs];
+#pragma unroll
+    for (int a = 0; a < Op::kInputs; ++a)
+      s[a] = static_cast<const Elem *>(p.in[a])[e];
+    static_cast<Elem *>(p.out)[e] = Op::apply1(s);
+  }
+}
+} // namespace
+
+#define HCAMD_FLAT_ADD(NAME, VPT, NT)                                          \
+  extern "C" __global__ __launch_bounds__(256) void NAME(                      \
+      const float *a, const float *b, float *c, size_t n) {                    \
+    Ptrs3 p{{a, b, nullptr}, c};                                               \
+    flat_map<AddF32, VPT, NT>(p, n);                                           \
+  }
+
+#define HCAMD_FLAT_FMA(NAME, VPT, NT)                                          \
+  extern "C" __global__ __launch_bounds__(256) void NAME(                      \
+      const _Float16 *a, const _Float16 *b, const _Float16 *c, _Float16 *d,    \
+      size_t n) {                                                              \
+    Ptrs3 p{{a, b, c}, d};                                                     \
+    flat_map<FmaF16, VPT, NT>(p, n);                                           \
+  }
+
+HCAMD_FLAT_ADD(hcamd_add_f32_v1, 1, false)
+HCAMD_FLAT_ADD(hcamd_add_f32_v2, 2, false)
+HCAMD_FLAT_ADD(hcamd_add_f32_v4, 4, false)
+HCAMD_FLAT_ADD(hcamd_add_f32_v8, 8, false)
+HCAMD_FLAT_ADD(hcamd_add_f32_v1_nt, 1, true)
+HCAMD_FLAT_ADD(hcamd_add_f32_v2_nt, 2, true)
+HCAMD_FLAT_ADD(hcamd_add_f32_v4_nt, 4, true)
+HCAMD_FLAT_ADD(hcamd_add_f32_v8_nt, 8, true)
+
+HCAMD_FLAT_FMA(hcamd_fma_f16_v1, 1, false)
+HCAMD_FLAT_FMA(hcamd_fma_f16_v2, 2, false)
+HCAMD_FLAT_FMA(hcamd_fma_f16_v4, 4, false)
+HCAMD_FLAT_FMA(hcamd_fma_f16_v1_nt, 1, true)
+HCAMD_FLAT_FMA(hcamd_fma_f16_v2_nt, 2, true)
+HCAMD_FLAT_FMA(hcamd_fma_f16_v4_nt, 4, true)
+
+// General path: any base alignment, any leading dimensions.  One element per
+// work-item; x runs along the row so a wave reads consecutive elements.
+extern "C" __global__ __launch_bounds__(256) void hcamd_add_f32_scalar(
+    const float *a, const float *b, float *c, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n)
+    c[i] = a[i] + b[i];
+}
+
+extern "C" __global__ __launch_bounds__(256) void hcamd_fma_f16_2d(
+    const _Float16 *a, size_t lda, const _Float16 *b, size_t ldb,
+    const _Float16 *c, size_t ldc, _Float16 *d, size_t ldd, size_t rows,
+    size_t cols) {
+  const size_t col = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t row = blockIdx.y;
+  if (col < cols && row < rows) {
+    _Float16 e[3] = {a[row * lda + col], b[row * ldb + col],
+                     c[row * ldc + col]};
+    d[row * ldd + col] = FmaF16::apply1(e);
+  }
+}

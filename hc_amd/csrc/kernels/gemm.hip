@@ -1,0 +1,256 @@
+// C[M,N] = A[M,K] * B[K,N], bf16 inputs, fp32 accumulation on MFMA, bf16
+// output (round to nearest even).  A is row-major; B is column-major and is
+// passed as Bt[N,K] row-major, so both operands are K-contiguous.
+//
+// Tiled kernel.  A workgroup of WM x WN waves owns a BM x BN tile of C and walks
+// K in steps of 64.  Each step's A and B panels (BM x 64 and BN x 64 bf16) live
+// in LDS, double buffered: while the MFMAs consume buffer b, the global loads
+// for the next step are in flight into registers and are written to buffer b^1
+// afterwards; one barrier per step.
+//
+// LDS layout: a panel row is 64 bf16 = 128 bytes = eight 16-byte chunks.  Chunk
+// c of row r is stored at chunk position c ^ swz(r), so that the sixteen lanes
+// of an MFMA operand read (sixteen consecutive rows, same logical chunk) fall
+// into different banks, and so do the eight lanes that write one row.
+//
+// MFMA: v_mfma_f32_16x16x32_bf16.  Lane l supplies row (l % 16) and the eight
+// K values 8*(l/16)..8*(l/16)+7 of each 16 x 32 operand block, i.e. exactly
+// one 16-byte chunk of a panel row.  The Bt block is given as the first
+// operand and the A block as the second, which yields the transposed product:
+// lane l then holds C[m = l % 16][n = 4*(l/16) .. 4*(l/16)+3], four consecutive
+// columns that are stored as one 8-byte word.
+//
+// Workgroup order: consecutive workgroup ids go to different XCDs (each with a
+// private L2), so ids are first regrouped to give each XCD a contiguous range
+// and the range is then walked in GROUP_M-row bands; an XCD's concurrent tiles
+// form a compact block that shares A and B panels in its L2.
+#include "common.h"
+
+using namespace hcamd;
+
+namespace {
+
+constexpr int kBK = 64;         // K step (bf16 elements)
+constexpr int kRowBytes = 128;  // kBK * 2
+constexpr int kChunks = 8;      // 16-byte chunks per panel row
+constexpr int kXcds = 8;
+constexpr int kGroupM = 4;
+
+template <int SH> __device__ __forceinline__ int swz(int row) {
+  return (row >> SH) & 7;
+}
+
+__device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n,
+                                                  int &tm, int &tn) {
+  const int n_wg = tiles_m * tiles_n;
+  int wg = blockIdx.x;
+  if (n_wg % kXcds == 0)
+    wg = (wg % kXcds) * (n_wg / kXcds) + wg / kXcds;
+  const int band = kGroupM * tiles_n;
+  const int first_m = (wg / band) * kGroupM;
+  const int rows = min(tiles_m - first_m, kGroupM);
+  const int in_band = wg % band;
+  tm = first_m + in_band % rows;
+  tn = in_band / rows;
+}
+
+template <int BM, int BN, int WM, int WN, int SH>
+__device__ __forceinline__ void gemm_tile(const __bf16 *__restrict__ A,
+                                          size_t lda,
+                                          const __bf16 *__restrict__ Bt,
+                                          size_t ldb, __bf16 *__restrict__ C,
+                                          size_t ldc, int M, int N, int K) {
+  constexpr int kThreads = WM * WN * kWave;
+  constexpr int kWaveM = BM / WM;
+  constexpr int kWaveN = BN / WN;
+  constexpr int kMI = kWaveM / 16;
+  constexpr int kNI = kWaveN / 16;
+  constexpr int kALoads = BM * kChunks / kThreads;
+  constexpr int kBLoads = BN * kChunks / kThreads;
+  static_assert(BM * kChunks % kThreads == 0 && BN * kChunks % kThreads == 0,
+                "panel chunks must divide evenly over the threads");
+  constexpr int kABytes = BM * kRowBytes;
+  constexpr int kStageBytes = (BM + BN) * kRowBytes;
+
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kStageBytes];
+
+  int tm, tn;
+  tile_of_workgroup(M / BM, N / BN, tm, tn);
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave;
+  const int wave = tid / kWave;
+  const int wave_m = (wave / WN) * kWaveM;
+  const int wave_n = (wave % WN) * kWaveN;
+
+  // ---- global -> register -> LDS staging ---------------------------------
+  // chunk id = tid + i * kThreads: row = id / 8, chunk = id % 8
+  const __bf16 *a_src[kALoads];
+  const __bf16 *b_src[kBLoads];
+  int a_dst[kALoads], b_dst[kBLoads];
+#pragma unroll
+  for (int i = 0; i < kALoads; ++i) {
+    const int id = tid + i * kThreads;
+    const int r = id / kChunks, c = id % kChunks;
+    a_src[i] = A + (size_t)(tm * BM + r) * lda + c * 8;
+    a_dst[i] = r * kRowBytes + ((c ^ swz<SH>(r)) * 16);
+  }
+#pragma unroll
+  for (int i = 0; i < kBLoads; ++i) {
+    const int id = tid + i * kThreads;
+    const int r = id / kChunks, c = id % kChunks;
+    b_src[i] = Bt + (size_t)(tn * BN + r) * ldb + c * 8;
+    b_dst[i] = kABytes + r * kRowBytes + ((c ^ swz<SH>(r)) * 16);
+  }
+
+  // ---- LDS -> operand registers -------------------------------------------
+  // operand block row = base + lane % 16, logical chunk = 4*ks + lane / 16
+  int a_off[kMI], b_off[kNI];
+  const int lrow = lane % 16, lchunk = lane / 16;
+#pragma unroll
+  for (int i = 0; i < kMI; ++i)
+    a_off[i] = (wave_m + i * 16 + lrow) * kRowBytes;
+#pragma unroll
+  for (int i = 0; i < kNI; ++i)
+    b_off[i] = kABytes + (wave_n + i * 16 + lrow) * kRowBytes;
+  // rows base+lrow with base % 16 == 0: swz depends on lrow only
+  const int lswz = swz<SH>(lrow);
+
+  f32x4 acc[kMI][kNI];
+#pragma unroll
+  for (int i = 0; i < kMI; ++i)
+#pragma unroll
+    for (int j = 0; j < kNI; ++j)
+      acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  u32x4 a_reg[kALoads], b_reg[kBLoads];
+  auto load_global = [&](int kt) {
+    const size_t k0 = (size_t)kt * kBK;
+#pragma unroll
+    for (int i = 0; i < kALoads; ++i)
+      a_reg[i] = *reinterpret_cast<const u32x4 *>(a_src[i] + k0);
+#pragma unroll
+    for (int i = 0; i < kBLoads; ++i)
+      b_reg[i] = *reinterpret_cast<const u32x4 *>(b_src[i] + k0);
+  };
+  auto store_lds = [&](int buf) {
+    unsigned char *base = lds + buf * kStageBytes;
+#pragma unroll
+    for (int i = 0; i < kALoads; ++i)
+      *reinterpret_cast<u32x4 *>(base + a_dst[i]) = a_reg[i];
+#pragma unroll
+    for (int i = 0; i < kBLoads; ++i)
+      *reinterpret_cast<u32x4 *>(base + b_dst[i]) = b_reg[i];
+  };
+  auto compute = [&](int buf) {
+    const unsigned char *base = lds + buf * kStageBytes;
+#pragma unroll
+    for (int ks = 0; ks < kBK / 32; ++ks) {
+      const int coff = ((ks * 4 + lchunk) ^ lswz) * 16;
+      bf16x8 af[kMI], bfr[kNI];
+#pragma unroll
+      for (int i = 0; i < kMI; ++i)
+        af[i] = *reinterpret_cast<const bf16x8 *>(base + a_off[i] + coff);
+#pragma unroll
+      for (int j = 0; j < kNI; ++j)
+        bfr[j] = *reinterpret_cast<const bf16x8 *>(base + b_off[j] + coff);
+#pragma unroll
+      for (int i = 0; i < kMI; ++i)
+#pragma unroll
+        for (int j = 0; j < kNI; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              bfr[j], af[i], acc[i][j], 0, 0, 0);
+    }
+  };
+
+  const int KT = K / kBK;
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+  for (int kt = 0; kt < KT; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < KT)
+      load_global(kt + 1);
+    compute(buf);
+    if (kt + 1 < KT)
+      store_lds(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: fp32 -> bf16 (nearest even), 8-byte stores ---------------
+  const int m_base = tm * BM + wave_m + lrow;
+  const int n_base = tn * BN + wave_n + lchunk * 4;
+#pragma unroll
+  for (int i = 0; i < kMI; ++i) {
+    __bf16 *crow = C + (size_t)(m_base + i * 16) * ldc + n_base;
+#pragma unroll
+    for (int j = 0; j < kNI; ++j) {
+      bf16x4 o;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        o[r] = (__bf16)acc[i][j][r];
+      *reinterpret_cast<bf16x4 *>(crow + j * 16) = o;
+    }
+  }
+}
+} // namespace
+
+#define HCAMD_GEMM(NAME, BM, BN, WM, WN, SH)                                   \
+  extern "C" __global__ __launch_bounds__(WM * WN * 64) void NAME(             \
+      const __bf16 *A, size_t lda, const __bf16 *Bt, size_t ldb, __bf16 *C,    \
+      size_t ldc, int M, int N, int K) {                                       \
+    gemm_tile<BM, BN, WM, WN, SH>(A, lda, Bt, ldb, C, ldc, M, N, K);           \
+  }
+
+HCAMD_GEMM(hcamd_gemm_bf16_256x256_w2x4_s0, 256, 256, 2, 4, 0)
+HCAMD_GEMM(hcamd_gemm_bf16_256x256_w2x4_s1, 256, 256, 2, 4, 1)
+HCAMD_GEMM(hcamd_gemm_bf16_256x256_w4x2_s0, 256, 256, 4, 2, 0)
+HCAMD_GEMM(hcamd_gemm_bf16_256x256_w2x2_s0, 256, 256, 2, 2, 0)
+HCAMD_GEMM(hcamd_gemm_bf16_128x128_w2x2_s0, 128, 128, 2, 2, 0)
+HCAMD_GEMM(hcamd_gemm_bf16_256x128_w2x2_s0, 256, 128, 2, 2, 0)
+
+// General kernel: any M, N, K, any leading dimensions and alignment.  A
+// 64 x 64 tile of C per workgroup, a 4 x 4 block per thread, fp32 FMAs on
+// LDS-staged 64 x 16 panels, every access bounds-checked.  Correct everywhere,
+// fast nowhere; it exists for the shapes the tiled kernel does not take.
+extern "C" __global__ __launch_bounds__(256) void hcamd_gemm_bf16_general(
+    const __bf16 *A, size_t lda, const __bf16 *Bt, size_t ldb, __bf16 *C,
+    size_t ldc, int M, int N, int K) {
+  constexpr int T = 64, KB = 16;
+  __shared__ float sa[KB][T + 1];
+  __shared__ float sb[KB][T + 1];
+  const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+  const int m0 = blockIdx.y * T, n0 = blockIdx.x * T;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += KB) {
+    for (int e = threadIdx.x; e < T * KB; e += 256) {
+      const int r = e / KB, k = e % KB;
+      const int gm = m0 + r, gn = n0 + r, gk = k0 + k;
+      sa[k][r] = (gm < M && gk < K) ? (float)A[(size_t)gm * lda + gk] : 0.f;
+      sb[k][r] = (gn < N && gk < K) ? (float)Bt[(size_t)gn * ldb + gk] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < KB; ++k) {
+      float av[4], bv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        av[i] = sa[k][ty * 4 + i];
+        bv[i] = sb[k][tx * 4 + i];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int gm = m0 + ty * 4 + i, gn = n0 + tx * 4 + j;
+      if (gm < M && gn < N)
+        C[(size_t)gm * ldc + gn] = (__bf16)acc[i][j];
+    }
+}

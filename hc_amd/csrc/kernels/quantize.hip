@@ -1,0 +1,222 @@
+// Row-wise symmetric int8 quantisation of fp16 rows:
+//   scale[r] = max|x[r,:]| / 127            (fp32, IEEE division)
+//   q[r,c]   = clamp(rint((float)x[r,c] / scale[r]), -127, 127)   (int8)
+// with round-half-even and a correctly rounded fp32 quotient, so that the int8
+// output is bit-identical to the whole-array NumPy expression.
+//
+// Layout: a thread owns chunks of 16 consecutive fp16 values (two 16-byte
+// loads) and produces 16 int8 values (one 16-byte store).  TPR threads share a
+// row; TPR = 256 is one workgroup per row, TPR = 64 is one wave per row and
+// four rows per workgroup.  The row stays in VGPRs between the absmax
+// reduction and the quantisation, so HBM sees one read and one write.
+//
+// absmax is computed on the fp16 bit patterns with the sign cleared: for
+// non-negative fp16 the unsigned integer order equals the numeric order, and
+// every NaN pattern (0x7c01..0x7fff) sorts above infinity, so a NaN anywhere in
+// the row makes the scale NaN, as numpy.max does.  Two values share one
+// 32-bit lane operation.
+//
+// Division: with EXACT_DIV the quotient is the compiler's IEEE fp32 division.
+// Otherwise the row's correctly rounded reciprocal y = fl(1/scale) is formed
+// once and each element takes q0 = x*y; r = fma(-q0, scale, x); q = fma(r, y,
+// q0): the residual r is exact and the corrected q equals the correctly rounded
+// quotient.  That equality was checked on the CPU for every one of the
+// 1,007,713,278 (x, absmax) pairs of finite fp16 values with |x| <= absmax; the
+// only difference is the sign of a zero quotient for x = -0, which the integer
+// conversion drops.  The same sweep shows |rint(q)| <= 127 always: for finite
+// rows the clamp never acts.
+#include "common.h"
+
+using namespace hcamd;
+
+namespace {
+constexpr int kThreads = 256;
+
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t absmax_bits(uint32_t m, uint32_t w) {
+  const u16x2 a = __builtin_bit_cast(u16x2, m);
+  const u16x2 b = __builtin_bit_cast(u16x2, w & 0x7fff7fffu);
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));
+}
+
+__device__ __forceinline__ float half_bits_to_float(uint32_t bits) {
+  return (float)__builtin_bit_cast(_Float16, (unsigned short)bits);
+}
+
+template <bool EXACT_DIV>
+__device__ __forceinline__ float quotient(float x, float scale, float rcp) {
+  if constexpr (EXACT_DIV) {
+    return x / scale;
+  } else {
+    const float q0 = x * rcp;
+    const float r = __builtin_fmaf(-q0, scale, x);
+    return __builtin_fmaf(r, rcp, q0);
+  }
+}
+
+// rint + clamp + int8 pack of four quotients into one 32-bit word.
+__device__ __forceinline__ uint32_t pack4(float a, float b, float c, float d) {
+  const int ia = (int)__builtin_amdgcn_fmed3f(__builtin_rintf(a), -127.f, 127.f);
+  const int ib = (int)__builtin_amdgcn_fmed3f(__builtin_rintf(b), -127.f, 127.f);
+  const int ic = (int)__builtin_amdgcn_fmed3f(__builtin_rintf(c), -127.f, 127.f);
+  const int id = (int)__builtin_amdgcn_fmed3f(__builtin_rintf(d), -127.f, 127.f);
+  return (uint32_t)(ia & 0xff) | ((uint32_t)(ib & 0xff) << 8) |
+         ((uint32_t)(ic & 0xff) << 16) | ((uint32_t)id << 24);
+}
+
+// Rows whose absmax is inf or NaN: a NaN quotient (inf/inf, x/NaN) maps to 0,
+// which is what a NaN -> int8 conversion yields on the host.
+__device__ __forceinline__ int8_t quant_special(float x, float scale) {
+  const float qf = x / scale;
+  if (qf != qf)
+    return 0;
+  return (int8_t)(int)__builtin_amdgcn_fmed3f(__builtin_rintf(qf), -127.f,
+                                              127.f);
+}
+
+template <int TPR, int VPT, bool EXACT_DIV, bool NT>
+__device__ __forceinline__ void quantize_regs(const _Float16 *x, size_t ldx,
+                                              int8_t *q, size_t ldq,
+                                              float *scale_out, size_t rows,
+                                              size_t cols) {
+  constexpr int kRowsPerGroup = kThreads / TPR;
+  constexpr int kWaves = TPR / kWave;
+  __shared__ uint32_t smax[kRowsPerGroup * kWaves];
+
+  const int t = threadIdx.x % TPR;
+  const int rg = threadIdx.x / TPR;
+  const size_t row = (size_t)blockIdx.x * kRowsPerGroup + rg;
+  const bool row_ok = row < rows; // uniform per wave
+  const _Float16 *xr = x + row * ldx;
+  int8_t *qr = q + row * ldq;
+
+  // chunk j of this thread starts at column ((j*TPR)+t)*16
+  u32x4 v[VPT][2];
+  uint32_t m = 0;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const size_t c = ((size_t)j * TPR + t) * 16;
+    v[j][0] = u32x4{0, 0, 0, 0};
+    v[j][1] = u32x4{0, 0, 0, 0};
+    if (row_ok) {
+      if (c + 16 <= cols) {
+        v[j][0] = ldg<NT>(reinterpret_cast<const u32x4 *>(xr + c));
+        v[j][1] = ldg<NT>(reinterpret_cast<const u32x4 *>(xr + c + 8));
+      } else if (c < cols) {
+        // ragged last chunk: element loads, zero fill (zero never raises the
+        // absmax and is never stored)
+        unsigned short e[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          e[i] = (c + i < cols)
+                     ? reinterpret_cast<const unsigned short *>(xr)[c + i]
+                     : (unsigned short)0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          v[j][0][i] = (uint32_t)e[2 * i] | ((uint32_t)e[2 * i + 1] << 16);
+          v[j][1][i] =
+              (uint32_t)e[8 + 2 * i] | ((uint32_t)e[8 + 2 * i + 1] << 16);
+        }
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        m = absmax_bits(m, v[j][h][i]);
+  }
+  m = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
+  m = group_reduce<UMaxOp, kWaves>(m, smax + rg * kWaves);
+
+  const float amax = half_bits_to_float(m);
+  const float scale = amax / 127.0f;
+  if (row_ok && t == 0)
+    scale_out[row] = scale;
+  const bool special = !(amax < INFINITY); // inf or NaN, uniform per row
+  // An all-zero row divides by 1 instead of 0: every quotient is 0.
+  const float div = (amax == 0.0f) ? 1.0f : scale;
+  const float rcp = 1.0f / div;
+
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const size_t c = ((size_t)j * TPR + t) * 16;
+    if (!row_ok || c >= cols)
+      continue;
+    if (special) {
+      for (int i = 0; i < 16 && c + i < cols; ++i) {
+        const uint32_t w = v[j][i / 8][(i % 8) / 2];
+        const uint32_t bits = (i & 1) ? (w >> 16) : (w & 0xffffu);
+        qr[c + i] = quant_special(half_bits_to_float(bits), scale);
+      }
+      continue;
+    }
+    u32x4 o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      // output word k holds elements 4k..4k+3 = input words 2k, 2k+1
+      const uint32_t w0 = v[j][k / 2][(2 * k) % 4];
+      const uint32_t w1 = v[j][k / 2][(2 * k) % 4 + 1];
+      const float f0 = half_bits_to_float(w0 & 0xffffu);
+      const float f1 = half_bits_to_float(w0 >> 16);
+      const float f2 = half_bits_to_float(w1 & 0xffffu);
+      const float f3 = half_bits_to_float(w1 >> 16);
+      o[k] = pack4(quotient<EXACT_DIV>(f0, div, rcp),
+                   quotient<EXACT_DIV>(f1, div, rcp),
+                   quotient<EXACT_DIV>(f2, div, rcp),
+                   quotient<EXACT_DIV>(f3, div, rcp));
+    }
+    if (c + 16 <= cols) {
+      stg<NT>(reinterpret_cast<u32x4 *>(qr + c), o);
+    } else {
+      for (int i = 0; i < 16 && c + i < cols; ++i)
+        qr[c + i] = (int8_t)((o[i / 4] >> (8 * (i % 4))) & 0xff);
+    }
+  }
+}
+} // namespace
+
+#define HCAMD_QUANT(NAME, TPR, VPT, EXACT, NT)                                 \
+  extern "C" __global__ __launch_bounds__(256) void NAME(                      \
+      const _Float16 *x, size_t ldx, int8_t *q, size_t ldq, float *scale,      \
+      size_t rows, size_t cols) {                                              \
+    quantize_regs<TPR, VPT, EXACT, NT>(x, ldx, q, ldq, scale, rows, cols);     \
+  }
+
+HCAMD_QUANT(hcamd_quant_f16_i8_w64_v1, 64, 1, false, false)
+HCAMD_QUANT(hcamd_quant_f16_i8_w64_v2, 64, 2, false, false)
+HCAMD_QUANT(hcamd_quant_f16_i8_w64_v4, 64, 4, false, false)
+HCAMD_QUANT(hcamd_quant_f16_i8_w64_v4_nt, 64, 4, false, true)
+HCAMD_QUANT(hcamd_quant_f16_i8_w64_v4_div, 64, 4, true, false)
+HCAMD_QUANT(hcamd_quant_f16_i8_g256_v1, 256, 1, false, false)
+HCAMD_QUANT(hcamd_quant_f16_i8_g256_v1_nt, 256, 1, false, true)
+HCAMD_QUANT(hcamd_quant_f16_i8_g256_v1_div, 256, 1, true, false)
+HCAMD_QUANT(hcamd_quant_f16_i8_g256_v2, 256, 2, false, false)
+HCAMD_QUANT(hcamd_quant_f16_i8_g256_v4, 256, 4, false, false)
+HCAMD_QUANT(hcamd_quant_f16_i8_g256_v8, 256, 8, false, false)
+
+// Streaming kernel: one workgroup per row, two sweeps (absmax, quantise) with
+// element accesses and the compiler's IEEE division.  Any alignment, any
+// number of columns.
+extern "C" __global__ __launch_bounds__(256) void hcamd_quant_f16_i8_stream(
+    const _Float16 *x, size_t ldx, int8_t *q, size_t ldq, float *scale_out,
+    size_t rows, size_t cols) {
+  __shared__ uint32_t smax[kThreads / kWave];
+  const size_t row = blockIdx.x;
+  const unsigned short *xr =
+      reinterpret_cast<const unsigned short *>(x) + row * ldx;
+  int8_t *qr = q + row * ldq;
+  uint32_t m = 0;
+  for (size_t c = threadIdx.x; c < cols; c += kThreads) {
+    const uint32_t b = xr[c] & 0x7fffu;
+    m = b > m ? b : m;
+  }
+  m = group_reduce<UMaxOp, kThreads / kWave>(m, smax);
+  const float amax = half_bits_to_float(m);
+  const float scale = amax / 127.0f;
+  if (threadIdx.x == 0)
+    scale_out[row] = scale;
+  const float div = (amax == 0.0f) ? 1.0f : scale;
+  for (size_t c = threadIdx.x; c < cols; c += kThreads)
+    qr[c] = quant_special(half_bits_to_float(xr[c]), div);
+}

@@ -1,0 +1,1050 @@
+// libhc_amd_runtime.so: the offload ABI (ol*), the launch half of the Python
+// runtime ABI (hcgpu*) and the typed launchers (hcamd*) for one MI355X, written
+// directly on the HIP module API: hipModuleLoadData, hipModuleGetFunction,
+// hipModuleLaunchKernel, one stream per queue, hipMalloc.  The signatures and
+// the reference interfaces they replace are documented in
+// include/hc_amd_runtime.h.
+#include "hc_amd_runtime.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// Call tracing (Loader.cpp:41-149, PyRuntime.cpp:12-34): "<fn> enter" /
+// "<fn> exit" on stdout, flushed, so that a trace interleaves correctly with
+// Python's own output.
+// ---------------------------------------------------------------------------
+bool g_traceLoader = false;
+bool g_tracePy = false;
+
+struct Scope {
+  Scope(const char *fn, bool on) : name(fn), enabled(on) {
+    if (enabled) {
+      std::fprintf(stdout, "%s enter\n", name);
+      std::fflush(stdout);
+    }
+  }
+  Scope(const char *fn, bool on, const char *fmt, ...) : name(fn), enabled(on) {
+    if (!enabled)
+      return;
+    std::fprintf(stdout, "%s ", name);
+    va_list ap;
+    va_start(ap, fmt);
+    std::vfprintf(stdout, fmt, ap);
+    va_end(ap);
+    std::fprintf(stdout, "\n");
+    std::fflush(stdout);
+  }
+  Scope(const Scope &) = delete;
+  ~Scope() {
+    if (enabled) {
+      std::fprintf(stdout, "%s exit\n", name);
+      std::fflush(stdout);
+    }
+  }
+  const char *name;
+  bool enabled;
+};
+#define OL_TRACE() Scope scope_(__func__, g_traceLoader)
+#define PY_TRACE() Scope scope_(__func__, g_tracePy)
+
+std::vector<std::string> g_searchPaths;
+
+// ---------------------------------------------------------------------------
+// Handles
+// ---------------------------------------------------------------------------
+struct Device {
+  OlErrorCallback callback = nullptr;
+  void *ctx = nullptr;
+  int index = 0;
+  // built-in modules and kernels, loaded on first use
+  std::unordered_map<std::string, hipModule_t> modules;
+  std::unordered_map<std::string, struct Kernel *> kernels;
+
+  void report(const char *fmt, ...) {
+    if (!callback)
+      return;
+    char buf[256] = {0};
+    va_list ap;
+    va_start(ap, fmt);
+    std::vsnprintf(buf, sizeof(buf) - 1, fmt, ap);
+    va_end(ap);
+    callback(ctx, OL_SEVERITY_ERROR, buf);
+  }
+  // 0 on success; otherwise reports "'<expr>' failed with '<hipErrorName>'"
+  int check(const char *expr, hipError_t err) {
+    if (err == hipSuccess)
+      return 0;
+    const char *name = hipGetErrorName(err);
+    report("'%s' failed with '%s'\n", expr, name ? name : "<unknown>");
+    return 1;
+  }
+  int makeCurrent() { return check("hipSetDevice(index)", hipSetDevice(index)); }
+  ~Device();
+};
+#define HIP_CHECK(dev, expr) (dev)->check(#expr, (expr))
+
+struct Module {
+  Device *device = nullptr;
+  hipModule_t module = nullptr;
+};
+
+struct Kernel {
+  Device *device = nullptr;
+  hipFunction_t function = nullptr;
+  std::string name;
+};
+
+struct Queue {
+  Device *device = nullptr;
+  hipStream_t stream = nullptr;
+};
+
+struct Event {
+  Device *device = nullptr;
+  hipStream_t stream = nullptr;
+  hipEvent_t event = nullptr;
+};
+
+Device::~Device() {
+  for (auto &kv : kernels)
+    delete kv.second;
+  for (auto &kv : modules)
+    if (kv.second)
+      (void)hipModuleUnload(kv.second);
+}
+
+// ---------------------------------------------------------------------------
+// Built-in code objects, linked in by blobs.S.
+// ---------------------------------------------------------------------------
+#define HCAMD_BLOB(n)                                                          \
+  extern "C" const unsigned char hcamd_blob_##n##_begin[];                     \
+  extern "C" const unsigned char hcamd_blob_##n##_end[];
+HCAMD_BLOB(copy)
+HCAMD_BLOB(elementwise)
+HCAMD_BLOB(softmax)
+HCAMD_BLOB(quantize)
+HCAMD_BLOB(gemm)
+#undef HCAMD_BLOB
+
+struct Blob {
+  const char *name;
+  const unsigned char *begin;
+  const unsigned char *end;
+};
+#define HCAMD_BLOB(n) {#n, hcamd_blob_##n##_begin, hcamd_blob_##n##_end}
+const Blob kBlobs[] = {HCAMD_BLOB(copy), HCAMD_BLOB(elementwise),
+                       HCAMD_BLOB(softmax), HCAMD_BLOB(quantize),
+                       HCAMD_BLOB(gemm)};
+#undef HCAMD_BLOB
+constexpr size_t kNumBlobs = sizeof(kBlobs) / sizeof(kBlobs[0]);
+
+Kernel *builtinKernel(Device *dev, const char *moduleName,
+                      const char *kernelName) {
+  std::string key = std::string(moduleName) + ":" + kernelName;
+  auto it = dev->kernels.find(key);
+  if (it != dev->kernels.end())
+    return it->second;
+  if (dev->makeCurrent())
+    return nullptr;
+  hipModule_t mod = nullptr;
+  auto mit = dev->modules.find(moduleName);
+  if (mit != dev->modules.end()) {
+    mod = mit->second;
+  } else {
+    const Blob *blob = nullptr;
+    for (const Blob &b : kBlobs)
+      if (std::strcmp(b.name, moduleName) == 0)
+        blob = &b;
+    if (!blob) {
+      dev->report("Unknown built-in module '%s'", moduleName);
+      return nullptr;
+    }
+    if (HIP_CHECK(dev, hipModuleLoadData(&mod, blob->begin)))
+      return nullptr;
+    dev->modules.emplace(moduleName, mod);
+  }
+  hipFunction_t fn = nullptr;
+  if (dev->check(kernelName, hipModuleGetFunction(&fn, mod, kernelName)))
+    return nullptr;
+  auto *k = new Kernel{dev, fn, kernelName};
+  dev->kernels.emplace(std::move(key), k);
+  return k;
+}
+
+// ---------------------------------------------------------------------------
+// Launch helper shared by olLaunchKernel and the typed launchers.
+// ---------------------------------------------------------------------------
+thread_local const char *t_lastKernel = "";
+
+int launch(Queue *q, Kernel *k, const size_t grid[3], const size_t block[3],
+           void **args, size_t sharedMem) {
+  Device *dev = q->device;
+  for (int i = 0; i < 3; ++i) {
+    if (grid[i] == 0 || block[i] == 0) {
+      dev->report("Empty launch dimension for '%s'", k->name.c_str());
+      return 1;
+    }
+  }
+  if (grid[0] > 0x7fffffffull || grid[1] > 65535 || grid[2] > 65535 ||
+      block[0] * block[1] * block[2] > 1024) {
+    dev->report("Launch geometry out of range for '%s': grid %zu,%zu,%zu "
+                "block %zu,%zu,%zu",
+                k->name.c_str(), grid[0], grid[1], grid[2], block[0], block[1],
+                block[2]);
+    return 1;
+  }
+  t_lastKernel = k->name.c_str();
+  return HIP_CHECK(
+      dev, hipModuleLaunchKernel(k->function, (unsigned)grid[0],
+                                 (unsigned)grid[1], (unsigned)grid[2],
+                                 (unsigned)block[0], (unsigned)block[1],
+                                 (unsigned)block[2], (unsigned)sharedMem,
+                                 q->stream, args, nullptr));
+}
+
+int launch1d(Queue *q, const char *module, const char *name, size_t groups,
+             size_t threads, void **args) {
+  Kernel *k = builtinKernel(q->device, module, name);
+  if (!k)
+    return 1;
+  const size_t grid[3] = {groups, 1, 1}, block[3] = {threads, 1, 1};
+  return launch(q, k, grid, block, args, 0);
+}
+
+inline bool aligned16(const void *p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+inline size_t ceilDiv(size_t a, size_t b) { return (a + b - 1) / b; }
+
+uint32_t upPow2(uint32_t x) {
+  x--;
+  x |= x >> 1;
+  x |= x >> 2;
+  x |= x >> 4;
+  x |= x >> 8;
+  x |= x >> 16;
+  return x + 1;
+}
+
+// kernel-variant overrides (0 = choose by shape)
+std::unordered_map<std::string, int> &variants() {
+  static std::unordered_map<std::string, int> v{
+      {"add", 0},     {"fma", 0},  {"softmax", 0},
+      {"quantize", 0}, {"gemm", 0}, {"copy", 0}};
+  return v;
+}
+int variantOf(const char *family) { return variants()[family]; }
+
+// ---------------------------------------------------------------------------
+// Process-wide device and queue of the hcgpu* entry points
+// (GpuRuntime.cpp:23-24).
+// ---------------------------------------------------------------------------
+OlDevice g_device = nullptr;
+OlQueue g_queue = nullptr;
+
+void stderrCallback(void *, OlSeverity sev, const char *desc) {
+  static const char *const kinds[] = {"error", "warning", "message"};
+  const char *kind = (sev >= 0 && sev <= 2) ? kinds[sev] : "error";
+  std::fprintf(stderr, "Offload %s: %s\n", kind, desc);
+  std::fflush(stderr);
+}
+
+[[noreturn]] void fatal(const char *desc) {
+  stderrCallback(nullptr, OL_SEVERITY_ERROR, desc);
+  std::abort();
+}
+
+// 0 ok, otherwise the name of the step that failed
+const char *ensureDefaultQueue(const char *deviceDesc) {
+  if (g_device)
+    return nullptr;
+  OlDevice dev = olCreateDevice(deviceDesc, &stderrCallback, nullptr);
+  if (!dev)
+    return "olCreateDevice failed";
+  OlQueue q = olCreateQueue(dev);
+  if (!q) {
+    olReleaseDevice(dev);
+    return "olCreateSyncQueue failed";
+  }
+  g_device = dev;
+  g_queue = q;
+  return nullptr;
+}
+
+} // namespace
+
+// ===========================================================================
+// 1. Offload ABI
+// ===========================================================================
+extern "C" {
+
+void setGPULoaderSearchPaths(const char *paths[], size_t count) noexcept {
+  g_searchPaths.clear();
+  for (size_t i = 0; i < count; ++i)
+    g_searchPaths.emplace_back(paths[i] ? paths[i] : "");
+}
+
+void enableFuncTracing(int val) noexcept { g_traceLoader = val != 0; }
+
+OlDevice olCreateDevice(const char *desc, OlErrorCallback errCallback,
+                        void *ctx) noexcept {
+  OL_TRACE();
+  auto fail = [&](const std::string &msg) -> OlDevice {
+    if (errCallback)
+      errCallback(ctx, OL_SEVERITY_ERROR, msg.c_str());
+    return nullptr;
+  };
+  if (!desc)
+    return fail("Invalid device desc: <null>");
+  const std::string d(desc);
+  const size_t sep = d.find(':');
+  if (sep == std::string::npos)
+    return fail("Invalid device desc: " + d);
+  const std::string runtime = d.substr(0, sep);
+  if (runtime != "hip")
+    return fail("Runtime not found: " + runtime);
+  const std::string id = d.substr(sep + 1);
+  if (id.empty() || id.find_first_not_of("0123456789") != std::string::npos ||
+      id.size() > 6)
+    return fail("Invalid device id");
+
+  auto dev = std::make_unique<Device>();
+  dev->callback = errCallback;
+  dev->ctx = ctx;
+  dev->index = std::atoi(id.c_str());
+  if (dev->makeCurrent())
+    return nullptr;
+  return dev.release();
+}
+
+void olReleaseDevice(OlDevice dev) noexcept {
+  OL_TRACE();
+  delete static_cast<Device *>(dev);
+}
+
+OlModule olCreateModule(OlDevice dev, const void *data,
+                        size_t /*len*/) noexcept {
+  OL_TRACE();
+  auto *device = static_cast<Device *>(dev);
+  if (!device)
+    return nullptr;
+  if (!data) {
+    device->report("olCreateModule: null code object");
+    return nullptr;
+  }
+  if (device->makeCurrent())
+    return nullptr;
+  hipModule_t mod = nullptr;
+  if (HIP_CHECK(device, hipModuleLoadData(&mod, data)))
+    return nullptr;
+  return new Module{device, mod};
+}
+
+void olReleaseModule(OlModule mod) noexcept {
+  OL_TRACE();
+  auto *m = static_cast<Module *>(mod);
+  if (!m)
+    return;
+  if (m->module)
+    HIP_CHECK(m->device, hipModuleUnload(m->module));
+  delete m;
+}
+
+OlKernel olGetKernel(OlModule mod, const char *name) noexcept {
+  OL_TRACE();
+  auto *m = static_cast<Module *>(mod);
+  if (!m || !name)
+    return nullptr;
+  hipFunction_t fn = nullptr;
+  if (HIP_CHECK(m->device, hipModuleGetFunction(&fn, m->module, name)))
+    return nullptr;
+  return new Kernel{m->device, fn, name};
+}
+
+void olReleaseKernel(OlKernel k) noexcept {
+  OL_TRACE();
+  delete static_cast<Kernel *>(k);
+}
+
+int olSuggestBlockSize(OlKernel /*k*/, const size_t *globalsSizes,
+                       size_t *blockSizesRet, size_t nDims) noexcept {
+  OL_TRACE();
+  if (nDims < 1 || nDims > 3 || !globalsSizes || !blockSizesRet)
+    return 1;
+  size_t budget = 1024;
+  for (size_t i = 0; i < nDims; ++i) {
+    const size_t g = globalsSizes[i];
+    if (g > 1) {
+      // budget stays a power of two >= 1: l <= budget implies
+      // upPow2(l) <= budget
+      const size_t l = std::min(g, budget);
+      blockSizesRet[i] = l;
+      budget /= upPow2(static_cast<uint32_t>(l));
+    } else {
+      blockSizesRet[i] = 1;
+    }
+  }
+  return 0;
+}
+
+OlQueue olCreateQueue(OlDevice dev) noexcept {
+  OL_TRACE();
+  auto *device = static_cast<Device *>(dev);
+  if (!device || device->makeCurrent())
+    return nullptr;
+  hipStream_t stream = nullptr;
+  if (HIP_CHECK(device, hipStreamCreate(&stream)))
+    return nullptr;
+  return new Queue{device, stream};
+}
+
+void olReleaseQueue(OlQueue q) noexcept {
+  OL_TRACE();
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return;
+  if (queue->stream)
+    HIP_CHECK(queue->device, hipStreamDestroy(queue->stream));
+  delete queue;
+}
+
+int olSyncQueue(OlQueue q) noexcept {
+  OL_TRACE();
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  return HIP_CHECK(queue->device, hipStreamSynchronize(queue->stream));
+}
+
+void *olAllocDevice(OlQueue q, size_t size, size_t /*align*/) noexcept {
+  OL_TRACE();
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue || queue->device->makeCurrent())
+    return nullptr;
+  void *ptr = nullptr;
+  if (HIP_CHECK(queue->device, hipMalloc(&ptr, size)))
+    return nullptr;
+  return ptr;
+}
+
+void olDeallocDevice(OlQueue q, void *data) noexcept {
+  OL_TRACE();
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return;
+  HIP_CHECK(queue->device, hipFree(data));
+}
+
+int olLaunchKernel(OlQueue q, OlKernel k, const size_t *gridSizes,
+                   const size_t *blockSizes, size_t nDims, void **args,
+                   size_t nArgs, size_t sharedMemSize) noexcept {
+  Scope scope_(__func__, g_traceLoader,
+               "grid: [%zu, %zu, %zu], blocks [%zu, %zu, %zu], nargs %zu, "
+               "shMem %zu",
+               nDims > 0 ? gridSizes[0] : 0, nDims > 1 ? gridSizes[1] : 0,
+               nDims > 2 ? gridSizes[2] : 0, nDims > 0 ? blockSizes[0] : 0,
+               nDims > 1 ? blockSizes[1] : 0, nDims > 2 ? blockSizes[2] : 0,
+               nArgs, sharedMemSize);
+  auto *queue = static_cast<Queue *>(q);
+  auto *kernel = static_cast<Kernel *>(k);
+  if (!queue || !kernel)
+    return 1;
+  if (nDims != 3) {
+    queue->device->report("Invalid launch dims: %d", static_cast<int>(nDims));
+    return 1;
+  }
+  return launch(queue, kernel, gridSizes, blockSizes, args, sharedMemSize);
+}
+
+// ===========================================================================
+// 2. Python-runtime ABI, launch half
+// ===========================================================================
+void hcgpuEnableTraceFunctions(int val) noexcept { g_tracePy = val != 0; }
+
+void *hcgpuGetKernel(void **handle, const char *deviceDesc, const void *data,
+                     size_t dataSize, const char *kernelName) noexcept {
+  PY_TRACE();
+  if (handle && *handle)
+    return *handle;
+  if (const char *err = ensureDefaultQueue(deviceDesc))
+    fatal(err);
+  // The module is intentionally kept for the life of the process: the kernel
+  // handle cached by the caller borrows from it (GpuRuntime.cpp:41-50).
+  OlModule module = olCreateModule(g_device, data, dataSize);
+  if (!module)
+    fatal("olCreateModule failed");
+  OlKernel kernel = olGetKernel(module, kernelName);
+  if (!kernel)
+    fatal("olGetKernel failed");
+  if (handle)
+    *handle = kernel;
+  return kernel;
+}
+
+void hcgpuSuggestBlockSize(void *kernel, const size_t *globalSizes,
+                           size_t *blockSizesRet, size_t nDim) noexcept {
+  PY_TRACE();
+  if (olSuggestBlockSize(kernel, globalSizes, blockSizesRet, nDim))
+    fatal("olSuggestBlockSize failed");
+}
+
+void hcgpuLaunchKernel(void *kernel, const size_t *gridSizes,
+                       const size_t *blockSizes, size_t nDim, void **args,
+                       size_t nArgs, size_t sharedMemSize) noexcept {
+  PY_TRACE();
+  if (!g_queue)
+    fatal("olLaunchKernel failed");
+  if (olLaunchKernel(g_queue, kernel, gridSizes, blockSizes, nDim, args, nArgs,
+                     sharedMemSize))
+    fatal("olLaunchKernel failed");
+  if (olSyncQueue(g_queue))
+    fatal("olSyncQueue failed");
+}
+
+// ===========================================================================
+// 3. Additions
+// ===========================================================================
+OlQueue hcamdGetDefaultQueue(const char *deviceDesc) noexcept {
+  if (const char *err = ensureDefaultQueue(deviceDesc)) {
+    stderrCallback(nullptr, OL_SEVERITY_ERROR, err);
+    return nullptr;
+  }
+  return g_queue;
+}
+
+OlDevice hcamdGetDefaultDevice(const char *deviceDesc) noexcept {
+  return hcamdGetDefaultQueue(deviceDesc) ? g_device : nullptr;
+}
+
+OlDevice hcamdQueueDevice(OlQueue q) noexcept {
+  return q ? static_cast<Queue *>(q)->device : nullptr;
+}
+
+size_t hcamdBuiltinModuleCount(void) noexcept { return kNumBlobs; }
+
+int hcamdGetBuiltinModule(size_t index, const char **name, const void **data,
+                          size_t *len) noexcept {
+  if (index >= kNumBlobs)
+    return 1;
+  if (name)
+    *name = kBlobs[index].name;
+  if (data)
+    *data = kBlobs[index].begin;
+  if (len)
+    *len = static_cast<size_t>(kBlobs[index].end - kBlobs[index].begin);
+  return 0;
+}
+
+OlKernel hcamdGetBuiltinKernel(OlDevice dev, const char *moduleName,
+                               const char *kernelName) noexcept {
+  if (!dev || !moduleName || !kernelName)
+    return nullptr;
+  return builtinKernel(static_cast<Device *>(dev), moduleName, kernelName);
+}
+
+int hcamdMemcpy(OlQueue q, void *dst, const void *src, size_t bytes,
+                int kind) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  static const hipMemcpyKind kinds[] = {hipMemcpyHostToDevice,
+                                        hipMemcpyDeviceToHost,
+                                        hipMemcpyDeviceToDevice};
+  if (kind < 0 || kind > 2) {
+    queue->device->report("Invalid copy kind: %d", kind);
+    return 1;
+  }
+  if (bytes == 0)
+    return 0;
+  return HIP_CHECK(queue->device,
+                   hipMemcpyAsync(dst, src, bytes, kinds[kind], queue->stream));
+}
+
+int hcamdFill32(OlQueue q, void *dst, uint32_t value, size_t count) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  if (count == 0)
+    return 0;
+  void *args[] = {&dst, &value, &count};
+  return launch1d(queue, "copy", "hcamd_fill32", ceilDiv(count, 256), 256,
+                  args);
+}
+
+HcamdEvent hcamdEventCreate(OlQueue q) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue || queue->device->makeCurrent())
+    return nullptr;
+  hipEvent_t ev = nullptr;
+  if (HIP_CHECK(queue->device, hipEventCreate(&ev)))
+    return nullptr;
+  return new Event{queue->device, queue->stream, ev};
+}
+
+void hcamdEventDestroy(HcamdEvent e) noexcept {
+  auto *ev = static_cast<Event *>(e);
+  if (!ev)
+    return;
+  HIP_CHECK(ev->device, hipEventDestroy(ev->event));
+  delete ev;
+}
+
+int hcamdEventRecord(HcamdEvent e) noexcept {
+  auto *ev = static_cast<Event *>(e);
+  if (!ev)
+    return 1;
+  return HIP_CHECK(ev->device, hipEventRecord(ev->event, ev->stream));
+}
+
+int hcamdEventSynchronize(HcamdEvent e) noexcept {
+  auto *ev = static_cast<Event *>(e);
+  if (!ev)
+    return 1;
+  return HIP_CHECK(ev->device, hipEventSynchronize(ev->event));
+}
+
+int hcamdEventElapsedMs(HcamdEvent start, HcamdEvent stop,
+                        float *ms) noexcept {
+  auto *a = static_cast<Event *>(start);
+  auto *b = static_cast<Event *>(stop);
+  if (!a || !b || !ms)
+    return 1;
+  return HIP_CHECK(a->device, hipEventElapsedTime(ms, a->event, b->event));
+}
+
+int hcamdDeviceInfo(OlDevice dev, int *computeUnits, int *clockKHz,
+                    int *memClockKHz, int *memBusBits, size_t *totalMem,
+                    char *archName, size_t archLen) noexcept {
+  auto *device = static_cast<Device *>(dev);
+  if (!device)
+    return 1;
+  hipDeviceProp_t prop;
+  if (HIP_CHECK(device, hipGetDeviceProperties(&prop, device->index)))
+    return 1;
+  if (computeUnits)
+    *computeUnits = prop.multiProcessorCount;
+  if (clockKHz)
+    *clockKHz = prop.clockRate;
+  if (memClockKHz)
+    *memClockKHz = prop.memoryClockRate;
+  if (memBusBits)
+    *memBusBits = prop.memoryBusWidth;
+  if (totalMem)
+    *totalMem = prop.totalGlobalMem;
+  if (archName && archLen) {
+    std::strncpy(archName, prop.gcnArchName, archLen - 1);
+    archName[archLen - 1] = '\0';
+  }
+  return 0;
+}
+
+int hcamdSetVariant(const char *family, int variant) noexcept {
+  if (!family)
+    return 1;
+  auto &v = variants();
+  auto it = v.find(family);
+  if (it == v.end())
+    return 1;
+  it->second = variant;
+  return 0;
+}
+
+const char *hcamdLastKernelName(void) noexcept { return t_lastKernel; }
+
+// ---------------------------------------------------------------------------
+// Typed launchers
+// ---------------------------------------------------------------------------
+int hcamdLaunchCopy2D(OlQueue q, size_t elemSize, const void *src,
+                      size_t srcRows, size_t srcCols, ptrdiff_t ss0,
+                      ptrdiff_t ss1, void *dst, size_t dstRows, size_t dstCols,
+                      ptrdiff_t ds0, ptrdiff_t ds1) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  const char *suffix = nullptr;
+  switch (elemSize) {
+  case 1: suffix = "b1"; break;
+  case 2: suffix = "b2"; break;
+  case 4: suffix = "b4"; break;
+  case 8: suffix = "b8"; break;
+  case 16: suffix = "b16"; break;
+  default:
+    dev->report("hcamdLaunchCopy2D: unsupported element size %zu", elemSize);
+    return 1;
+  }
+  size_t rows = std::min(srcRows, dstRows);
+  size_t cols = std::min(srcCols, dstCols);
+  if (rows == 0 || cols == 0)
+    return 0;
+  if (!src || !dst) {
+    dev->report("hcamdLaunchCopy2D: null pointer");
+    return 1;
+  }
+  if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) %
+      elemSize) {
+    dev->report("hcamdLaunchCopy2D: pointer not aligned to the element size");
+    return 1;
+  }
+  // Window covers whole rows of both arrays and both are dense: one vector.
+  const bool dense = ss1 == 1 && ds1 == 1 &&
+                     (rows == 1 || (ss0 == (ptrdiff_t)cols &&
+                                    ds0 == (ptrdiff_t)cols));
+  const int variant = variantOf("copy");
+  if (dense && aligned16(src) && aligned16(dst) && variant != 9) {
+    static const char *const names[] = {
+        "hcamd_copy_flat_v4",    "hcamd_copy_flat_v1",    "hcamd_copy_flat_v2",
+        "hcamd_copy_flat_v4",    "hcamd_copy_flat_v8",    "hcamd_copy_flat_v1_nt",
+        "hcamd_copy_flat_v2_nt", "hcamd_copy_flat_v4_nt", "hcamd_copy_flat_v8_nt"};
+    static const int vpt[] = {4, 1, 2, 4, 8, 1, 2, 4, 8};
+    const int v = (variant >= 0 && variant <= 8) ? variant : 0;
+    size_t nbytes = rows * cols * elemSize;
+    const size_t words = ceilDiv(nbytes, 16);
+    void *args[] = {&src, &dst, &nbytes};
+    return launch1d(queue, "copy", names[v], ceilDiv(words, 256 * (size_t)vpt[v]),
+                    256, args);
+  }
+  const std::string name = std::string("hcamd_copy2d_") + suffix;
+  Kernel *k = builtinKernel(dev, "copy", name.c_str());
+  if (!k)
+    return 1;
+  // rows go to grid.y (at most 65535 per launch): split tall windows
+  const size_t bx = cols >= 256 ? 256 : 64, by = 256 / bx;
+  for (size_t r0 = 0; r0 < rows; r0 += 65535 * by) {
+    size_t nr = std::min(rows - r0, (size_t)65535 * by);
+    const char *s = static_cast<const char *>(src) +
+                    (ptrdiff_t)r0 * ss0 * (ptrdiff_t)elemSize;
+    char *d = static_cast<char *>(dst) + (ptrdiff_t)r0 * ds0 * (ptrdiff_t)elemSize;
+    void *args[] = {&s, &ss0, &ss1, &d, &ds0, &ds1, &nr, &cols};
+    const size_t grid[3] = {ceilDiv(cols, bx), ceilDiv(nr, by), 1};
+    const size_t block[3] = {bx, by, 1};
+    if (launch(queue, k, grid, block, args, 0))
+      return 1;
+  }
+  return 0;
+}
+
+int hcamdLaunchCopy2DTiled(OlQueue q, size_t elemSize, const void *src,
+                           void *dst, size_t rows, size_t cols, ptrdiff_t ss0,
+                           ptrdiff_t ds0, size_t blockX, size_t blockY,
+                           size_t unroll) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  const char *suffix = nullptr;
+  switch (elemSize) {
+  case 1: suffix = "b1"; break;
+  case 2: suffix = "b2"; break;
+  case 4: suffix = "b4"; break;
+  case 8: suffix = "b8"; break;
+  case 16: suffix = "b16"; break;
+  default:
+    dev->report("hcamdLaunchCopy2DTiled: unsupported element size %zu",
+                elemSize);
+    return 1;
+  }
+  if (rows == 0 || cols == 0)
+    return 0;
+  if (!src || !dst || blockX == 0 || blockY == 0 || unroll == 0 ||
+      blockX * blockY > 1024) {
+    dev->report("hcamdLaunchCopy2DTiled: invalid argument");
+    return 1;
+  }
+  const std::string name = std::string("hcamd_copy2d_tiled_") + suffix;
+  Kernel *k = builtinKernel(dev, "copy", name.c_str());
+  if (!k)
+    return 1;
+  int64_t u = (int64_t)unroll, s0 = ss0, d0 = ds0, r = (int64_t)rows,
+          c = (int64_t)cols;
+  void *args[] = {&u, &s0, &src, &r, &c, &d0, &dst};
+  const size_t grid[3] = {ceilDiv(cols, blockX * unroll), ceilDiv(rows, blockY),
+                          1};
+  const size_t block[3] = {blockX, blockY, 1};
+  return launch(queue, k, grid, block, args, 0);
+}
+
+int hcamdLaunchAddF32(OlQueue q, const float *a, const float *b, float *c,
+                      size_t n) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  if (n == 0)
+    return 0;
+  if (!a || !b || !c) {
+    queue->device->report("hcamdLaunchAddF32: null pointer");
+    return 1;
+  }
+  void *args[] = {&a, &b, &c, &n};
+  const int variant = variantOf("add");
+  if (!(aligned16(a) && aligned16(b) && aligned16(c)) || variant == 9)
+    return launch1d(queue, "elementwise", "hcamd_add_f32_scalar",
+                    ceilDiv(n, 256), 256, args);
+  static const char *const names[] = {
+      "hcamd_add_f32_v4",    "hcamd_add_f32_v1",    "hcamd_add_f32_v2",
+      "hcamd_add_f32_v4",    "hcamd_add_f32_v8",    "hcamd_add_f32_v1_nt",
+      "hcamd_add_f32_v2_nt", "hcamd_add_f32_v4_nt", "hcamd_add_f32_v8_nt"};
+  static const int vpt[] = {4, 1, 2, 4, 8, 1, 2, 4, 8};
+  const int v = (variant >= 0 && variant <= 8) ? variant : 0;
+  const size_t words = ceilDiv(n, 4);
+  return launch1d(queue, "elementwise", names[v],
+                  ceilDiv(words, 256 * (size_t)vpt[v]), 256, args);
+}
+
+int hcamdLaunchFmaF16(OlQueue q, const void *a, size_t lda, const void *b,
+                      size_t ldb, const void *c, size_t ldc, void *d,
+                      size_t ldd, size_t rows, size_t cols) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  if (rows == 0 || cols == 0)
+    return 0;
+  if (!a || !b || !c || !d) {
+    dev->report("hcamdLaunchFmaF16: null pointer");
+    return 1;
+  }
+  if (rows > 1 && (lda < cols || ldb < cols || ldc < cols || ldd < cols)) {
+    dev->report("hcamdLaunchFmaF16: leading dimension smaller than cols");
+    return 1;
+  }
+  const bool dense = rows == 1 || (lda == cols && ldb == cols && ldc == cols &&
+                                   ldd == cols);
+  const int variant = variantOf("fma");
+  if (dense && aligned16(a) && aligned16(b) && aligned16(c) && aligned16(d) &&
+      variant != 7) {
+    static const char *const names[] = {
+        "hcamd_fma_f16_v2",    "hcamd_fma_f16_v1",    "hcamd_fma_f16_v2",
+        "hcamd_fma_f16_v4",    "hcamd_fma_f16_v1_nt", "hcamd_fma_f16_v2_nt",
+        "hcamd_fma_f16_v4_nt"};
+    static const int vpt[] = {2, 1, 2, 4, 1, 2, 4};
+    const int v = (variant >= 0 && variant <= 6) ? variant : 0;
+    size_t n = rows * cols;
+    const size_t words = ceilDiv(n, 8);
+    void *args[] = {&a, &b, &c, &d, &n};
+    return launch1d(queue, "elementwise", names[v],
+                    ceilDiv(words, 256 * (size_t)vpt[v]), 256, args);
+  }
+  Kernel *k = builtinKernel(dev, "elementwise", "hcamd_fma_f16_2d");
+  if (!k)
+    return 1;
+  for (size_t r0 = 0; r0 < rows; r0 += 65535) {
+    size_t nr = std::min(rows - r0, (size_t)65535);
+    const char *pa = static_cast<const char *>(a) + r0 * lda * 2;
+    const char *pb = static_cast<const char *>(b) + r0 * ldb * 2;
+    const char *pc = static_cast<const char *>(c) + r0 * ldc * 2;
+    char *pd = static_cast<char *>(d) + r0 * ldd * 2;
+    void *args[] = {&pa, &lda, &pb, &ldb, &pc, &ldc, &pd, &ldd, &nr, &cols};
+    const size_t grid[3] = {ceilDiv(cols, 256), nr, 1};
+    const size_t block[3] = {256, 1, 1};
+    if (launch(queue, k, grid, block, args, 0))
+      return 1;
+  }
+  return 0;
+}
+
+int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,
+                          size_t ldy, size_t rows, size_t cols) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  if (rows == 0 || cols == 0)
+    return 0;
+  if (!x || !y) {
+    dev->report("hcamdLaunchSoftmaxF32: null pointer");
+    return 1;
+  }
+  if (rows > 1 && (ldx < cols || ldy < cols)) {
+    dev->report("hcamdLaunchSoftmaxF32: leading dimension smaller than cols");
+    return 1;
+  }
+  if (rows > 0x7fffffffull) {
+    dev->report("hcamdLaunchSoftmaxF32: too many rows");
+    return 1;
+  }
+  void *args[] = {&x, &ldx, &y, &ldy, &rows, &cols};
+  const int variant = variantOf("softmax");
+  const bool vec_ok = aligned16(x) && aligned16(y) &&
+                      (rows == 1 || (ldx % 4 == 0 && ldy % 4 == 0));
+  if (!vec_ok || cols > 16384 || variant == 1)
+    return launch1d(queue, "softmax", "hcamd_softmax_f32_stream", rows, 256,
+                    args);
+  const char *name;
+  size_t groups = rows;
+  if (cols <= 1024) {
+    name = cols <= 256   ? "hcamd_softmax_f32_w64_v1"
+           : cols <= 512 ? "hcamd_softmax_f32_w64_v2"
+                         : "hcamd_softmax_f32_w64_v4";
+    groups = ceilDiv(rows, 4);
+  } else if (cols <= 2048) {
+    name = (cols == 2048 && variant != 2) ? "hcamd_softmax_f32_g256_v2_full"
+                                          : "hcamd_softmax_f32_g256_v2";
+  } else if (cols <= 4096) {
+    name = (cols == 4096 && variant != 2) ? "hcamd_softmax_f32_g256_v4_full"
+                                          : "hcamd_softmax_f32_g256_v4";
+  } else if (cols <= 8192) {
+    name = (cols == 8192 && variant != 2)
+               ? (variant == 3 ? "hcamd_softmax_f32_g256_v8_full_nt"
+                               : "hcamd_softmax_f32_g256_v8_full")
+               : "hcamd_softmax_f32_g256_v8";
+  } else {
+    name = "hcamd_softmax_f32_g256_v16";
+  }
+  return launch1d(queue, "softmax", name, groups, 256, args);
+}
+
+int hcamdLaunchQuantizeF16I8(OlQueue q, const void *x, size_t ldx, int8_t *qout,
+                             size_t ldq, float *scale, size_t rows,
+                             size_t cols) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  if (rows == 0)
+    return 0;
+  if (!x || !qout || !scale) {
+    dev->report("hcamdLaunchQuantizeF16I8: null pointer");
+    return 1;
+  }
+  if (cols == 0) {
+    // no elements: the absmax of an empty row is taken as 0
+    return hcamdFill32(q, scale, 0u, rows);
+  }
+  if (rows > 1 && (ldx < cols || ldq < cols)) {
+    dev->report("hcamdLaunchQuantizeF16I8: leading dimension smaller than cols");
+    return 1;
+  }
+  if (rows > 0x7fffffffull) {
+    dev->report("hcamdLaunchQuantizeF16I8: too many rows");
+    return 1;
+  }
+  void *args[] = {&x, &ldx, &qout, &ldq, &scale, &rows, &cols};
+  const int variant = variantOf("quantize");
+  const bool vec_ok = aligned16(x) && aligned16(qout) &&
+                      (rows == 1 || (ldx % 8 == 0 && ldq % 16 == 0));
+  if (!vec_ok || cols > 32768 || variant == 1)
+    return launch1d(queue, "quantize", "hcamd_quant_f16_i8_stream", rows, 256,
+                    args);
+  const char *name;
+  size_t groups = rows;
+  bool per_wave = false;
+  if (cols <= 1024) {
+    name = "hcamd_quant_f16_i8_w64_v1";
+    per_wave = true;
+  } else if (cols <= 2048) {
+    name = "hcamd_quant_f16_i8_w64_v2";
+    per_wave = true;
+  } else if (cols <= 4096) {
+    switch (variant) {
+    case 2: name = "hcamd_quant_f16_i8_w64_v4"; per_wave = true; break;
+    case 3: name = "hcamd_quant_f16_i8_g256_v1_nt"; break;
+    case 4: name = "hcamd_quant_f16_i8_w64_v4_nt"; per_wave = true; break;
+    case 5: name = "hcamd_quant_f16_i8_g256_v1_div"; break;
+    case 6: name = "hcamd_quant_f16_i8_w64_v4_div"; per_wave = true; break;
+    default: name = "hcamd_quant_f16_i8_g256_v1"; break;
+    }
+  } else if (cols <= 8192) {
+    name = "hcamd_quant_f16_i8_g256_v2";
+  } else if (cols <= 16384) {
+    name = "hcamd_quant_f16_i8_g256_v4";
+  } else {
+    name = "hcamd_quant_f16_i8_g256_v8";
+  }
+  if (per_wave)
+    groups = ceilDiv(rows, 4);
+  return launch1d(queue, "quantize", name, groups, 256, args);
+}
+
+int hcamdLaunchGemmBF16(OlQueue q, const void *a, size_t lda, const void *bt,
+                        size_t ldb, void *c, size_t ldc, size_t m, size_t n,
+                        size_t k) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  if (m == 0 || n == 0)
+    return 0;
+  if (!a || !bt || !c) {
+    dev->report("hcamdLaunchGemmBF16: null pointer");
+    return 1;
+  }
+  if (k == 0) {
+    dev->report("hcamdLaunchGemmBF16: K must be at least 1");
+    return 1;
+  }
+  if ((m > 1 && lda < k) || (n > 1 && ldb < k) || (m > 1 && ldc < n)) {
+    dev->report("hcamdLaunchGemmBF16: leading dimension too small");
+    return 1;
+  }
+  if (m > 0x7fffffffull || n > 0x7fffffffull || k > 0x7fffffffull) {
+    dev->report("hcamdLaunchGemmBF16: dimension exceeds 2^31-1");
+    return 1;
+  }
+  int M = (int)m, N = (int)n, K = (int)k;
+  void *args[] = {&a, &lda, &bt, &ldb, &c, &ldc, &M, &N, &K};
+
+  struct Tiled {
+    const char *name;
+    int bm, bn, threads;
+  };
+  static const Tiled tiled[] = {
+      {"hcamd_gemm_bf16_256x256_w2x4_s0", 256, 256, 512},
+      {"hcamd_gemm_bf16_256x256_w2x4_s1", 256, 256, 512},
+      {"hcamd_gemm_bf16_256x256_w4x2_s0", 256, 256, 512},
+      {"hcamd_gemm_bf16_256x256_w2x2_s0", 256, 256, 256},
+      {"hcamd_gemm_bf16_128x128_w2x2_s0", 128, 128, 256},
+      {"hcamd_gemm_bf16_256x128_w2x2_s0", 256, 128, 256},
+  };
+  constexpr int kNumTiled = sizeof(tiled) / sizeof(tiled[0]);
+  const int variant = variantOf("gemm");
+  const bool vec_ok = aligned16(a) && aligned16(bt) && aligned16(c) &&
+                      lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 &&
+                      k % 64 == 0;
+  const Tiled *pick = nullptr;
+  if (vec_ok && variant != 7) {
+    if (variant >= 1 && variant <= kNumTiled) {
+      const Tiled &t = tiled[variant - 1];
+      if (m % t.bm == 0 && n % t.bn == 0)
+        pick = &t;
+    } else {
+      if (m % 256 == 0 && n % 256 == 0)
+        pick = &tiled[0];
+      else if (m % 128 == 0 && n % 128 == 0)
+        pick = &tiled[4];
+    }
+  }
+  if (pick) {
+    Kernel *kn = builtinKernel(dev, "gemm", pick->name);
+    if (!kn)
+      return 1;
+    const size_t grid[3] = {(m / pick->bm) * (n / pick->bn), 1, 1};
+    const size_t block[3] = {(size_t)pick->threads, 1, 1};
+    return launch(queue, kn, grid, block, args, 0);
+  }
+  Kernel *kn = builtinKernel(dev, "gemm", "hcamd_gemm_bf16_general");
+  if (!kn)
+    return 1;
+  const size_t gy = ceilDiv(m, 64);
+  if (gy > 65535) {
+    dev->report("hcamdLaunchGemmBF16: M too large for the general kernel");
+    return 1;
+  }
+  const size_t grid[3] = {ceilDiv(n, 64), gy, 1};
+  const size_t block[3] = {256, 1, 1};
+  return launch(queue, kn, grid, block, args, 0);
+}
+
+} // extern "C"

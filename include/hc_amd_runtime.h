@@ -1,0 +1,279 @@
+/*
+ * hc_amd_runtime.h - C ABI of libhc_amd_runtime.so
+ *
+ * One shared library for one MI355X (gfx950).  It exports three groups of
+ * entry points:
+ *
+ *   1. ol*     - the 13-function offload ABI of the reference
+ *                (gpu-runtime/common/include/offload_api.h:27-63), implemented
+ *                directly on the HIP module API.  The library is therefore both
+ *                "the loader" and "the hip backend" of the reference
+ *                (gpu-runtime/loader/src/Loader.cpp:326-444,
+ *                gpu-runtime/hip-runtime/src/Runtime.cpp:100-248).
+ *   2. hcgpu*  - the entry points JIT'd host code and ctypes bind in the
+ *                reference (python/cpp/py-runtime/src/PyRuntime.cpp:36-94).
+ *                The two functions that take a PyObject* live in the companion
+ *                library libhc_amd_pyabi.so (hc_amd_pyabi.h) so that this
+ *                library has no CPython dependency.
+ *   3. hcamd*  - additions that have no counterpart in the reference: access
+ *                to the built-in gfx950 code objects, typed launchers for the
+ *                hand-written kernels, copies and events.  The reference has
+ *                none of these because its device code is compiler generated
+ *                and its buffers are torch allocations
+ *                (python/hckernel/tests/test_e2e.py:32-33).
+ *
+ * Conventions: plain pointers and sizes only; every function is noexcept;
+ * handle-returning functions return NULL on error and int-returning functions
+ * return non-zero on error, after calling the device's error callback with a
+ * message of at most 255 characters (offload_api.h:29-31).  No function takes
+ * a lock: callers serialise, as the reference's do
+ * (python/cpp/py-runtime/src/GpuRuntime.cpp:23-24).
+ */
+#ifndef HC_AMD_RUNTIME_H
+#define HC_AMD_RUNTIME_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#define HCAMD_NOEXCEPT noexcept
+#else
+#define HCAMD_NOEXCEPT
+#endif
+
+/* ---------------------------------------------------------------------------
+ * 1. Offload ABI.  offload_api.h:9-20 (handle and callback types).
+ * ------------------------------------------------------------------------ */
+typedef void *OlDevice;
+typedef void *OlModule;
+typedef void *OlKernel;
+typedef void *OlQueue;
+
+/* offload_api.h:14-18 declares `enum class OlSeverity : int`; an int carries
+ * the same values through a C signature. */
+typedef int OlSeverity;
+#define OL_SEVERITY_ERROR 0
+#define OL_SEVERITY_WARNING 1
+#define OL_SEVERITY_MESSAGE 2
+
+typedef void (*OlErrorCallback)(void *ctx, OlSeverity sev, const char *desc);
+
+/* offload_api.h:32-35; hip-runtime/src/Runtime.cpp:100-126.  `desc` is
+ * "hip:<index>".  A prefix other than "hip" reports "Runtime not found: <p>"
+ * (Loader.cpp:357-359), a missing ':' reports "Invalid device desc: <desc>"
+ * (Loader.cpp:331-335), an unparsable index reports "Invalid device id"
+ * (Runtime.cpp:115-119).  Makes the device current (hipSetDevice). */
+OlDevice olCreateDevice(const char *desc, OlErrorCallback errCallback,
+                        void *ctx) HCAMD_NOEXCEPT;
+/* offload_api.h:35; Runtime.cpp:127-129. */
+void olReleaseDevice(OlDevice dev) HCAMD_NOEXCEPT;
+
+/* offload_api.h:38-40; Runtime.cpp:131-145.  `data` is an ELF code object for
+ * gfx950 (hipModuleLoadData); `len` is not needed by HIP and is ignored, as in
+ * the reference. */
+OlModule olCreateModule(OlDevice dev, const void *data,
+                        size_t len) HCAMD_NOEXCEPT;
+void olReleaseModule(OlModule mod) HCAMD_NOEXCEPT;
+
+/* offload_api.h:42-44; Runtime.cpp:147-159 (hipModuleGetFunction).  The module
+ * must outlive the kernel.  olReleaseKernel frees the small handle. */
+OlKernel olGetKernel(OlModule mod, const char *name) HCAMD_NOEXCEPT;
+void olReleaseKernel(OlKernel k) HCAMD_NOEXCEPT;
+
+/* offload_api.h:46-49; Runtime.cpp:161-191.  globalsSizes is x-first (the last
+ * Python dimension first, mlir/lib/Transforms/LowerHKernel.cpp:296-305).
+ * Budget 1024 work-items: for each dim with size > 1 take min(size, budget)
+ * and divide the budget by that value rounded up to a power of two; other dims
+ * get 1.  Returns 1 when nDims is not 1..3.  `k` may be NULL: the heuristic
+ * does not look at the kernel. */
+int olSuggestBlockSize(OlKernel k, const size_t *globalsSizes,
+                       size_t *blockSizesRet, size_t nDims) HCAMD_NOEXCEPT;
+
+/* offload_api.h:51-53; Runtime.cpp:193-212.  One HIP stream at the default
+ * priority. */
+OlQueue olCreateQueue(OlDevice dev) HCAMD_NOEXCEPT;
+void olReleaseQueue(OlQueue q) HCAMD_NOEXCEPT;
+int olSyncQueue(OlQueue q) HCAMD_NOEXCEPT;
+
+/* offload_api.h:55-57; Runtime.cpp:214-231 (hipMalloc / hipFree; `align` is
+ * satisfied by hipMalloc's 256-byte alignment). */
+void *olAllocDevice(OlQueue q, size_t size, size_t align) HCAMD_NOEXCEPT;
+void olDeallocDevice(OlQueue q, void *data) HCAMD_NOEXCEPT;
+
+/* offload_api.h:59-63; Runtime.cpp:233-248.  nDims must be 3 ("Invalid launch
+ * dims: <n>" otherwise); gridSizes/blockSizes are x,y,z; `args` is an array of
+ * nArgs pointers, one to each kernel argument
+ * (mlir/lib/Transforms/GpuToGpuRuntime.cpp:279-292).  Asynchronous on the
+ * queue's stream (hipModuleLaunchKernel). */
+int olLaunchKernel(OlQueue q, OlKernel k, const size_t *gridSizes,
+                   const size_t *blockSizes, size_t nDims, void **args,
+                   size_t nArgs, size_t sharedMemSize) HCAMD_NOEXCEPT;
+
+/* Loader extras: gpu-runtime/loader/src/Loader.cpp:20-45.  The backend is
+ * built in, so the search paths are recorded but never searched.  Tracing
+ * prints "<fn> enter" / "<fn> exit" on stdout for every ol* call and the
+ * launch geometry for olLaunchKernel (Loader.cpp:433-438). */
+void setGPULoaderSearchPaths(const char *paths[], size_t count) HCAMD_NOEXCEPT;
+void enableFuncTracing(int val) HCAMD_NOEXCEPT;
+
+/* ---------------------------------------------------------------------------
+ * 2. Python-runtime ABI (launch half).  PyRuntime.cpp:36-94.
+ * ------------------------------------------------------------------------ */
+
+/* PyRuntime.cpp:36-39.  "<fn> enter/exit" on stdout for every hcgpu* call. */
+void hcgpuEnableTraceFunctions(int val) HCAMD_NOEXCEPT;
+
+/* PyRuntime.cpp:73-78; GpuRuntime.cpp:26-51.  Returns *handle when it is set.
+ * Otherwise creates the process-wide device and queue from deviceDesc on first
+ * use (the first desc wins for the life of the process), loads the code
+ * object, looks the kernel up, stores it in *handle and returns it.  Any
+ * failure prints "Offload error: <msg>" on stderr and aborts
+ * (GpuRuntime.cpp:11-21). */
+void *hcgpuGetKernel(void **handle, const char *deviceDesc, const void *data,
+                     size_t dataSize, const char *kernelName) HCAMD_NOEXCEPT;
+
+/* PyRuntime.cpp:80-85; GpuRuntime.cpp:53-58.  olSuggestBlockSize, abort on
+ * failure. */
+void hcgpuSuggestBlockSize(void *kernel, const size_t *globalSizes,
+                           size_t *blockSizesRet, size_t nDim) HCAMD_NOEXCEPT;
+
+/* PyRuntime.cpp:87-94; GpuRuntime.cpp:60-69.  olLaunchKernel on the
+ * process-wide queue followed by olSyncQueue: synchronous on return.  Abort on
+ * failure. */
+void hcgpuLaunchKernel(void *kernel, const size_t *gridSizes,
+                       const size_t *blockSizes, size_t nDim, void **args,
+                       size_t nArgs, size_t sharedMemSize) HCAMD_NOEXCEPT;
+
+/* ---------------------------------------------------------------------------
+ * 3. Additions (no counterpart in the reference).
+ * ------------------------------------------------------------------------ */
+
+/* The process-wide device and queue hcgpuGetKernel uses, created on first use
+ * from deviceDesc.  Unlike hcgpu*, failures return NULL after the
+ * "Offload error" line instead of aborting. */
+OlQueue hcamdGetDefaultQueue(const char *deviceDesc) HCAMD_NOEXCEPT;
+OlDevice hcamdGetDefaultDevice(const char *deviceDesc) HCAMD_NOEXCEPT;
+/* The device a queue belongs to. */
+OlDevice hcamdQueueDevice(OlQueue q) HCAMD_NOEXCEPT;
+
+/* Built-in gfx950 code objects, embedded in the library the way JIT'd host
+ * code embeds its blob (GpuToGpuRuntime.cpp:161-169).  Index 0..count-1;
+ * returns 0 and fills name/data/len, or 1 when the index is out of range.
+ * The blobs can be handed to olCreateModule / hcgpuGetKernel. */
+size_t hcamdBuiltinModuleCount(void) HCAMD_NOEXCEPT;
+int hcamdGetBuiltinModule(size_t index, const char **name, const void **data,
+                          size_t *len) HCAMD_NOEXCEPT;
+/* Kernel handle from the built-in modules, loaded once per device and cached.
+ * The handle is owned by the device: do not release it. */
+OlKernel hcamdGetBuiltinKernel(OlDevice dev, const char *moduleName,
+                               const char *kernelName) HCAMD_NOEXCEPT;
+
+/* Copies on the queue's stream.  kind: 0 host-to-device, 1 device-to-host,
+ * 2 device-to-device.  Asynchronous for pinned host memory; pageable host
+ * memory is staged by HIP.  hcamdFill32 writes `count` 32-bit words with a
+ * small kernel (safe under stream capture). */
+int hcamdMemcpy(OlQueue q, void *dst, const void *src, size_t bytes,
+                int kind) HCAMD_NOEXCEPT;
+int hcamdFill32(OlQueue q, void *dst, uint32_t value,
+                size_t count) HCAMD_NOEXCEPT;
+
+/* Events on the queue's stream, for timing kernels where they run. */
+typedef void *HcamdEvent;
+HcamdEvent hcamdEventCreate(OlQueue q) HCAMD_NOEXCEPT;
+void hcamdEventDestroy(HcamdEvent e) HCAMD_NOEXCEPT;
+int hcamdEventRecord(HcamdEvent e) HCAMD_NOEXCEPT;
+int hcamdEventSynchronize(HcamdEvent e) HCAMD_NOEXCEPT;
+int hcamdEventElapsedMs(HcamdEvent start, HcamdEvent stop,
+                        float *ms) HCAMD_NOEXCEPT;
+
+/* Device facts used for roofline arithmetic: compute units, engine clock in
+ * kHz, memory clock in kHz, memory bus width in bits, bytes of device memory,
+ * and the gcn arch name (copied into archName, NUL terminated, at most
+ * archLen bytes). */
+int hcamdDeviceInfo(OlDevice dev, int *computeUnits, int *clockKHz,
+                    int *memClockKHz, int *memBusBits, size_t *totalMem,
+                    char *archName, size_t archLen) HCAMD_NOEXCEPT;
+
+/* ---- Typed launchers for the hand-written kernels -------------------------
+ * All are asynchronous on the queue's stream and return 0 / non-zero.  They
+ * validate shapes and alignment on the host and pick the launch geometry;
+ * pointers are device pointers.  Leading dimensions (ld*) are in elements.
+ * Element types are given by size for copies and are fixed for the rest.
+ */
+
+/* Masked 2-D tile copy, the one kernel the reference's compiled path can
+ * express (python/hckernel/tests/test_e2e.py:57-136; semantics of
+ * CurrentGroup.load/store, python/hckernel/kernel_api.py:297-342): copies the
+ * window [0,min(srcRows,dstRows)) x [0,min(srcCols,dstCols)) and leaves every
+ * other byte of dst untouched.  elemSize is 1, 2, 4, 8 or 16.  Strides in
+ * elements; either may be non-unit. */
+int hcamdLaunchCopy2D(OlQueue q, size_t elemSize, const void *src,
+                      size_t srcRows, size_t srcCols, ptrdiff_t srcStride0,
+                      ptrdiff_t srcStride1, void *dst, size_t dstRows,
+                      size_t dstCols, ptrdiff_t dstStride0,
+                      ptrdiff_t dstStride1) HCAMD_NOEXCEPT;
+
+/* The same copy launched with the reference's own geometry and kernel argument
+ * list (tests/Transforms/gpu-to-gpu-runtime.mlir:34-37): grid =
+ * (ceil(cols/(bx*unroll)), ceil(rows/by), 1), block = (bx, by, 1), one element
+ * per work-item per load, `unroll` loads per work-item along the row
+ * (test_e2e.py:80-136).  Present so that the reference's tile decomposition
+ * can be checked on the GPU; hcamdLaunchCopy2D is the fast path. */
+int hcamdLaunchCopy2DTiled(OlQueue q, size_t elemSize, const void *src,
+                           void *dst, size_t rows, size_t cols,
+                           ptrdiff_t srcStride0, ptrdiff_t dstStride0,
+                           size_t blockX, size_t blockY,
+                           size_t unroll) HCAMD_NOEXCEPT;
+
+/* c[i] = a[i] + b[i], fp32, i < n.  One IEEE add per element. */
+int hcamdLaunchAddF32(OlQueue q, const float *a, const float *b, float *c,
+                      size_t n) HCAMD_NOEXCEPT;
+
+/* d = (half)((float)a * (float)b + (float)c) over a rows x cols window of
+ * row-major fp16 arrays; round to nearest even on the final conversion, fp16
+ * denormals kept.  When all four arrays are contiguous (ld == cols) the window
+ * is processed as one flat vector of rows*cols elements. */
+int hcamdLaunchFmaF16(OlQueue q, const void *a, size_t lda, const void *b,
+                      size_t ldb, const void *c, size_t ldc, void *d,
+                      size_t ldd, size_t rows, size_t cols) HCAMD_NOEXCEPT;
+
+/* Row softmax, fp32: y[r,:] = exp(x[r,:]-max(x[r,:])) / sum(exp(...)).
+ * Expression of python/hckernel/tests/test_examples.py:330-335. */
+int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,
+                          size_t ldy, size_t rows,
+                          size_t cols) HCAMD_NOEXCEPT;
+
+/* Row-wise symmetric int8 quantisation of fp16 rows:
+ * scale[r] = max|x[r,:]| / 127 (fp32), q = clamp(rint((float)x / scale[r]),
+ * -127, 127) with IEEE division and round-half-even.  A row whose absmax is
+ * zero gets scale 0 and q 0.  A row holding NaN gets scale NaN and q 0; an
+ * infinite absmax gives scale inf, q 0 for finite x and 0 for the infinite
+ * entries too (inf/inf is NaN). */
+int hcamdLaunchQuantizeF16I8(OlQueue q, const void *x, size_t ldx, int8_t *qout,
+                             size_t ldq, float *scale, size_t rows,
+                             size_t cols) HCAMD_NOEXCEPT;
+
+/* C[M,N] = A[M,K] * B[K,N]; A row-major bf16 (lda), B column-major bf16 given
+ * as Bt[N,K] row-major (ldb), fp32 accumulation on MFMA, C row-major bf16
+ * (ldc), round to nearest even.  Any M, N, K >= 1; K-contiguous rows must be
+ * 16-byte aligned for the fast path (ld % 8 == 0 and aligned base), otherwise
+ * a slower general kernel runs. */
+int hcamdLaunchGemmBF16(OlQueue q, const void *a, size_t lda, const void *bt,
+                        size_t ldb, void *c, size_t ldc, size_t m, size_t n,
+                        size_t k) HCAMD_NOEXCEPT;
+
+/* Chooses between kernel variants of one family by number (0 = default
+ * choice by shape).  For tuning and measurement; family names are "add",
+ * "fma", "softmax", "quantize", "gemm", "copy". Returns 1 for an unknown
+ * family. */
+int hcamdSetVariant(const char *family, int variant) HCAMD_NOEXCEPT;
+
+/* Name and launch geometry of the kernel the most recent typed launcher
+ * enqueued on this thread (for reports and profiles). */
+const char *hcamdLastKernelName(void) HCAMD_NOEXCEPT;
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+#endif /* HC_AMD_RUNTIME_H */
