@@ -1,0 +1,301 @@
+#!/usr/bin/env python3
+"""Benchmark of the five hc_amd kernels on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1..c5|all]
+
+A "step" is one launch of a workload's kernel over its full synthetic input,
+already resident in HBM.  Each workload cycles through ROTATE distinct buffer
+sets so that consecutive launches never find their inputs in the 256 MiB
+memory-side cache.  Timing: W warm-up launches, then exactly K launches between
+two HIP events recorded on the stream the kernels run on, with a host
+synchronisation and a wall clock around the same region.
+
+Prints ONE JSON line.  The top-level metric is the fused fp16 elementwise
+workload (d = a*b + c, 8191 x 8193); the `configs` object carries the same
+fields for all five workloads, each with its roofline and its NumPy CPU
+baseline timed on this machine's host cores in the same run.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
+ROTATE = 4
+
+# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
+# scaled by a copy kernel of known size; filled in from profiles/*.txt.
+MEASURED_TRAFFIC = {"c1": None, "c2": None, "c3": None, "c4": None, "c5": None}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+class Workload:
+    """name, algorithmic work, how to build device buffers, launch and check."""
+
+    def __init__(self, key, title, kernel_dtype, bound, work, unit):
+        self.key, self.title, self.dtype = key, title, kernel_dtype
+        self.bound, self.work, self.unit = bound, work, unit
+
+    def setup(self, rt):            # -> list of ROTATE argument tuples
+        raise NotImplementedError
+
+    def plan(self, rt, args):       # -> hc_amd.runtime.Plan (one foreign call per launch)
+        raise NotImplementedError
+
+    def check(self, rt, args):      # -> dict(parity=..., detail=...)
+        raise NotImplementedError
+
+    def cpu(self):                  # -> (seconds best-of-n, sample description, cores)
+        raise NotImplementedError
+
+
+def _best_of(fn, repeats=5):
+    fn()
+    best = float("inf")
+    for _ in range(repeats):
+        t = time.perf_counter()
+        fn()
+        best = min(best, time.perf_counter() - t)
+    return best
+
+
+def _blas_threads():
+    try:
+        from threadpoolctl import threadpool_info
+        return max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+    except Exception:
+        return int(os.environ.get("OPENBLAS_NUM_THREADS", os.cpu_count() or 1))
+
+
+def make_workloads(rt, wl):
+    from hc_amd import workloads as W
+
+    class C1(Workload):
+        def setup(self, rt):
+            self.a, self.b = W.inputs_c1()
+            return [(rt.to_device(self.a), rt.to_device(self.b),
+                     rt.DeviceArray(self.a.shape, np.float32)) for _ in range(ROTATE)]
+
+        def plan(self, rt, s):
+            return rt.plan_add_f32(s[0], s[1], s[2])
+
+        def check(self, rt, s):
+            from oracle import closed_forms as cf
+            ok = np.array_equal(s[2].to_host().view(np.uint32),
+                                cf.np_add(self.a, self.b).view(np.uint32))
+            return {"parity": "bit-exact" if ok else "MISMATCH", "ok": bool(ok)}
+
+        def cpu(self):
+            from oracle import closed_forms as cf
+            return _best_of(lambda: cf.np_add(self.a, self.b)), "full size, a + b", 1
+
+    class C2(Workload):
+        def setup(self, rt):
+            self.a, self.b, self.c = W.inputs_c2()
+            return [(rt.to_device(self.a), rt.to_device(self.b), rt.to_device(self.c),
+                     rt.DeviceArray(self.a.shape, np.float16)) for _ in range(ROTATE)]
+
+        def plan(self, rt, s):
+            return rt.plan_fma_f16(s[0], s[1], s[2], s[3])
+
+        def check(self, rt, s):
+            from oracle import closed_forms as cf
+            ok = np.array_equal(s[3].to_host().view(np.uint16),
+                                cf.np_fma_f16(self.a, self.b, self.c).view(np.uint16))
+            return {"parity": "bit-exact" if ok else "MISMATCH", "ok": bool(ok)}
+
+        def cpu(self):
+            from oracle import closed_forms as cf
+            return (_best_of(lambda: cf.np_fma_f16(self.a, self.b, self.c), 3),
+                    "full size, (a32*b32+c32).astype(f16)", 1)
+
+    class C3(Workload):
+        def setup(self, rt):
+            (self.x,) = W.inputs_c3()
+            return [(rt.to_device(self.x), rt.DeviceArray(self.x.shape, np.float32))
+                    for _ in range(ROTATE)]
+
+        def plan(self, rt, s):
+            return rt.plan_softmax_f32(s[0], s[1])
+
+        def check(self, rt, s):
+            from oracle import closed_forms as cf
+            y, want = s[1].to_host(), cf.np_softmax(self.x)
+            ok = np.allclose(y, want, rtol=1e-5, atol=1e-9)
+            rel = float(np.max(np.abs(y - want) / np.maximum(np.abs(want), 1e-30)))
+            return {"parity": "rtol 1e-5" if ok else "MISMATCH", "ok": bool(ok),
+                    "max_rel_err": rel}
+
+        def cpu(self):
+            from oracle import closed_forms as cf
+            return _best_of(lambda: cf.np_softmax(self.x), 3), "full size, np_softmax", 1
+
+    class C4(Workload):
+        def setup(self, rt):
+            (self.x,) = W.inputs_c4()
+            return [(rt.to_device(self.x), rt.DeviceArray(self.x.shape, np.int8),
+                     rt.DeviceArray((self.x.shape[0],), np.float32)) for _ in range(ROTATE)]
+
+        def plan(self, rt, s):
+            return rt.plan_quantize_f16_i8(s[0], s[1], s[2])
+
+        def check(self, rt, s):
+            from oracle import closed_forms as cf
+            q, sc = cf.np_quantize(self.x)
+            ok = (np.array_equal(s[1].to_host(), q) and
+                  np.array_equal(s[2].to_host().view(np.uint32), sc.view(np.uint32)))
+            return {"parity": "bit-exact" if ok else "MISMATCH", "ok": bool(ok)}
+
+        def cpu(self):
+            from oracle import closed_forms as cf
+            return _best_of(lambda: cf.np_quantize(self.x), 3), "full size, np_quantize", 1
+
+    class C5(Workload):
+        def setup(self, rt):
+            self.a, self.bt = W.inputs_c5()
+            m, n = self.a.shape[0], self.bt.shape[0]
+            return [(rt.to_device(self.a, bf16=True), rt.to_device(self.bt, bf16=True),
+                     rt.DeviceArray((m, n), np.uint16, bf16=True)) for _ in range(ROTATE)]
+
+        def plan(self, rt, s):
+            return rt.plan_gemm_bf16(s[0], s[1], s[2])
+
+        def check(self, rt, s):
+            from oracle import closed_forms as cf
+            got = W.bf16_bits_to_f32(s[2].to_host())
+            want = cf.np_gemm_bf16(self.a, self.bt, np.float32)
+            ok = np.allclose(got, want, rtol=1e-2, atol=2.6e-4)
+            return {"parity": "rtol 1e-2 vs fp32 accumulation" if ok else "MISMATCH",
+                    "ok": bool(ok), "max_abs_err": float(np.max(np.abs(got - want)))}
+
+        def cpu(self):
+            from oracle import closed_forms as cf
+            t = _best_of(lambda: cf.np_gemm_bf16(self.a, self.bt, np.float32), 2)
+            return t, "full size, OpenBLAS sgemm on bf16-rounded inputs", _blas_threads()
+
+    table = {
+        "c1": C1("c1", "vadd fp32 N=16777259", "f32", "hbm", W.work_c1(), "GB/s"),
+        "c2": C2("c2", "fma fp16 8191x8193 (fp32 math)", "f16", "hbm", W.work_c2(), "GB/s"),
+        "c3": C3("c3", "row softmax fp32 4096x8192", "f32", "hbm", W.work_c3(), "GB/s"),
+        "c4": C4("c4", "row absmax int8 quantize fp16 16384x4096", "f16->i8", "hbm",
+                 W.work_c4(), "GB/s"),
+        "c5": C5("c5", "GEMM bf16 4096^3 (fp32 acc)", "bf16", "mfma", W.work_c5(), "TFLOP/s"),
+    }
+    keys = list(table) if wl == "all" else [wl]
+    return [table[k] for k in keys]
+
+
+def run_one(rt, ctx, w, steps, warmup, want_cpu):
+    log(f"[bench] {w.key}: {w.title}: building inputs")
+    sets = w.setup(rt)
+    plans = [w.plan(rt, s) for s in sets]
+    launches = [p.launch for p in plans]
+    ctx.synchronize()
+    for i in range(warmup):
+        launches[i % ROTATE]()
+    ctx.synchronize()
+    kernel = rt.last_kernel_name()
+    start, stop = rt.Event(ctx), rt.Event(ctx)
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(steps):
+        launches[i % ROTATE]()
+    stop.record()
+    ctx.synchronize()
+    wall = time.perf_counter() - t0
+    ev_ms = start.elapsed_ms(stop)
+    ms_step = wall * 1e3 / steps
+    kern_ms = ev_ms / steps
+    scale = 1e-9 if w.unit == "GB/s" else 1e-12
+    value = w.work * scale / (wall / steps)
+    achieved = w.work * scale / (kern_ms * 1e-3)
+    peak = HBM_PEAK_GBS if w.bound == "hbm" else BF16_PEAK_TFLOPS
+    res = {
+        "workload": w.title, "kernel": kernel, "dtype": w.dtype,
+        "value": round(value, 2), "unit": w.unit, "ms_per_step": round(ms_step, 5),
+        "roofline": {"bound": w.bound, "achieved": round(achieved, 2), "peak": peak,
+                     "unit": w.unit, "frac": round(achieved / peak, 4),
+                     "traffic": MEASURED_TRAFFIC[w.key],
+                     "kernel_avg_us": round(kern_ms * 1e3, 3),
+                     "algorithmic_work": w.work},
+    }
+    log(f"[bench] {w.key}: {kernel}: {kern_ms * 1e3:.2f} us/launch, "
+        f"{achieved:.1f} {w.unit} = {100 * achieved / peak:.1f}% of peak; checking parity")
+    res["parity"] = w.check(rt, sets[(steps - 1) % ROTATE])
+    if want_cpu:
+        sec, sample, cores = w.cpu()
+        res["cpu_baseline"] = {"value": round(w.work * scale / sec, 3), "unit": w.unit,
+                               "cores": cores, "kind": "port", "sample": sample,
+                               "seconds": round(sec, 5)}
+        log(f"[bench] {w.key}: cpu {res['cpu_baseline']['value']} {w.unit} on {cores} core(s)")
+    for s in sets:
+        for a in s:
+            a.free()
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="all", choices=["all", "c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no "
+                 "sharding); run with --gpus 1")
+    if args.steps < 1:
+        sys.exit("--steps must be at least 1")
+
+    from hc_amd import runtime as rt          # fails loudly without the native library
+    ctx = rt.default_context("hip:0")
+    info = ctx.info()
+    log(f"[bench] device {info}")
+
+    results = {}
+    for w in make_workloads(rt, args.workload):
+        results[w.key] = run_one(rt, ctx, w, args.steps, args.warmup, not args.no_cpu)
+
+    head_key = "c2" if "c2" in results else next(iter(results))
+    head = results[head_key]
+    out = {
+        "metric": "HBM GB/s (elementwise/softmax/quant) + bf16 GEMM TFLOP/s, 1 MI355X",
+        "value": head["value"], "unit": head["unit"], "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": head["dtype"], "data": "synthetic",
+        "config": {"workload": head["workload"], "headline": head_key,
+                   "rotating_buffer_sets": ROTATE, "device": info["arch"],
+                   "compute_units": info["compute_units"],
+                   "host_cpus": os.cpu_count(),
+                   "host_cpus_usable": len(os.sched_getaffinity(0)),
+                   "numpy": np.__version__},
+        "roofline": head["roofline"],
+        "parity": head["parity"],
+        "configs": results,
+    }
+    if "cpu_baseline" in head:
+        out["cpu_baseline"] = head["cpu_baseline"]
+    print(json.dumps(out), flush=True)
+    bad = [k for k, r in results.items() if not r["parity"]["ok"]]
+    if bad:
+        sys.exit(f"bench.py: parity failed for {bad}")
+
+
+if __name__ == "__main__":
+    main()

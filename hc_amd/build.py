@@ -64,7 +64,7 @@ def _run(cmd: list[str]) -> None:
 def build_kernel_module(name: str, keep_asm: bool = False) -> Path:
     src = CSRC / "kernels" / f"{name}.hip"
     out = BUILD / f"{name}.hsaco"
-    cmd = [_hipcc(), "--genco", *DEVICE_FLAGS, "-I", str(CSRC / "kernels"),
+    cmd = [_hipcc(), "--genco", "--no-gpu-bundle-output", *DEVICE_FLAGS, "-I", str(CSRC / "kernels"),
            "-o", str(out), str(src)]
     if keep_asm:
         cmd.insert(2, "-save-temps=obj")

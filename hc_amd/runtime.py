@@ -1,0 +1,497 @@
+"""Thin Python layer over the C ABI of libhc_amd_runtime.so.
+
+Everything that touches the GPU goes through the exported C functions declared
+in include/hc_amd_runtime.h: device memory (olAllocDevice), copies
+(hcamdMemcpy), the typed kernel launchers (hcamdLaunch*), events and the
+generic module/kernel/launch calls.  There is no CPU fallback here: without the
+native library the import of hc_amd.py_runtime fails, and without a GPU the
+first call raises HcRuntimeError.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import numpy as np
+
+from . import py_runtime
+
+_rt = py_runtime.runtime_lib
+_py = py_runtime.pyabi_lib
+
+
+class HcRuntimeError(RuntimeError):
+    """An ol*/hcamd* call reported failure; carries the runtime's message."""
+
+
+# ---------------------------------------------------------------------------
+# ctypes signatures (one place, mirrors include/hc_amd_runtime.h)
+# ---------------------------------------------------------------------------
+_vp, _sz, _ssz, _int = C.c_void_p, C.c_size_t, C.c_ssize_t, C.c_int
+ERROR_CALLBACK = C.CFUNCTYPE(None, _vp, _int, C.c_char_p)
+
+
+def _sig(lib, name, restype, *argtypes):
+    fn = getattr(lib, name)
+    fn.restype = restype
+    fn.argtypes = list(argtypes)
+    return fn
+
+
+_sz_p = C.POINTER(_sz)
+olCreateDevice = _sig(_rt, "olCreateDevice", _vp, C.c_char_p, ERROR_CALLBACK, _vp)
+olReleaseDevice = _sig(_rt, "olReleaseDevice", None, _vp)
+olCreateModule = _sig(_rt, "olCreateModule", _vp, _vp, _vp, _sz)
+olReleaseModule = _sig(_rt, "olReleaseModule", None, _vp)
+olGetKernel = _sig(_rt, "olGetKernel", _vp, _vp, C.c_char_p)
+olReleaseKernel = _sig(_rt, "olReleaseKernel", None, _vp)
+olSuggestBlockSize = _sig(_rt, "olSuggestBlockSize", _int, _vp, _sz_p, _sz_p, _sz)
+olCreateQueue = _sig(_rt, "olCreateQueue", _vp, _vp)
+olReleaseQueue = _sig(_rt, "olReleaseQueue", None, _vp)
+olSyncQueue = _sig(_rt, "olSyncQueue", _int, _vp)
+olAllocDevice = _sig(_rt, "olAllocDevice", _vp, _vp, _sz, _sz)
+olDeallocDevice = _sig(_rt, "olDeallocDevice", None, _vp, _vp)
+olLaunchKernel = _sig(_rt, "olLaunchKernel", _int, _vp, _vp, _sz_p, _sz_p, _sz,
+                      C.POINTER(_vp), _sz, _sz)
+hcgpuGetKernel = _sig(_rt, "hcgpuGetKernel", _vp, C.POINTER(_vp), C.c_char_p, _vp,
+                      _sz, C.c_char_p)
+hcgpuSuggestBlockSize = _sig(_rt, "hcgpuSuggestBlockSize", None, _vp, _sz_p, _sz_p, _sz)
+hcgpuLaunchKernel = _sig(_rt, "hcgpuLaunchKernel", None, _vp, _sz_p, _sz_p, _sz,
+                         C.POINTER(_vp), _sz, _sz)
+hcamdGetDefaultQueue = _sig(_rt, "hcamdGetDefaultQueue", _vp, C.c_char_p)
+hcamdGetDefaultDevice = _sig(_rt, "hcamdGetDefaultDevice", _vp, C.c_char_p)
+hcamdQueueDevice = _sig(_rt, "hcamdQueueDevice", _vp, _vp)
+hcamdBuiltinModuleCount = _sig(_rt, "hcamdBuiltinModuleCount", _sz)
+hcamdGetBuiltinModule = _sig(_rt, "hcamdGetBuiltinModule", _int, _sz,
+                             C.POINTER(C.c_char_p), C.POINTER(_vp), _sz_p)
+hcamdGetBuiltinKernel = _sig(_rt, "hcamdGetBuiltinKernel", _vp, _vp, C.c_char_p,
+                             C.c_char_p)
+hcamdMemcpy = _sig(_rt, "hcamdMemcpy", _int, _vp, _vp, _vp, _sz, _int)
+hcamdFill32 = _sig(_rt, "hcamdFill32", _int, _vp, _vp, C.c_uint32, _sz)
+hcamdEventCreate = _sig(_rt, "hcamdEventCreate", _vp, _vp)
+hcamdEventDestroy = _sig(_rt, "hcamdEventDestroy", None, _vp)
+hcamdEventRecord = _sig(_rt, "hcamdEventRecord", _int, _vp)
+hcamdEventSynchronize = _sig(_rt, "hcamdEventSynchronize", _int, _vp)
+hcamdEventElapsedMs = _sig(_rt, "hcamdEventElapsedMs", _int, _vp, _vp,
+                           C.POINTER(C.c_float))
+hcamdDeviceInfo = _sig(_rt, "hcamdDeviceInfo", _int, _vp, C.POINTER(_int),
+                       C.POINTER(_int), C.POINTER(_int), C.POINTER(_int), _sz_p,
+                       C.c_char_p, _sz)
+hcamdSetVariant = _sig(_rt, "hcamdSetVariant", _int, C.c_char_p, _int)
+hcamdLastKernelName = _sig(_rt, "hcamdLastKernelName", C.c_char_p)
+hcamdLaunchCopy2D = _sig(_rt, "hcamdLaunchCopy2D", _int, _vp, _sz, _vp, _sz, _sz,
+                         _ssz, _ssz, _vp, _sz, _sz, _ssz, _ssz)
+hcamdLaunchCopy2DTiled = _sig(_rt, "hcamdLaunchCopy2DTiled", _int, _vp, _sz, _vp, _vp,
+                              _sz, _sz, _ssz, _ssz, _sz, _sz, _sz)
+hcamdLaunchAddF32 = _sig(_rt, "hcamdLaunchAddF32", _int, _vp, _vp, _vp, _vp, _sz)
+hcamdLaunchFmaF16 = _sig(_rt, "hcamdLaunchFmaF16", _int, _vp, _vp, _sz, _vp, _sz, _vp,
+                         _sz, _vp, _sz, _sz, _sz)
+hcamdLaunchSoftmaxF32 = _sig(_rt, "hcamdLaunchSoftmaxF32", _int, _vp, _vp, _sz, _vp,
+                             _sz, _sz, _sz)
+hcamdLaunchQuantizeF16I8 = _sig(_rt, "hcamdLaunchQuantizeF16I8", _int, _vp, _vp, _sz,
+                                _vp, _sz, _vp, _sz, _sz)
+hcamdLaunchGemmBF16 = _sig(_rt, "hcamdLaunchGemmBF16", _int, _vp, _vp, _sz, _vp, _sz,
+                           _vp, _sz, _sz, _sz, _sz)
+hcamdConvertPyArray = _sig(_py, "hcamdConvertPyArray", _int, C.py_object, _int, _vp,
+                           _sz_p, C.c_char_p, _sz)
+hcamdConvertPyInt64 = _sig(_py, "hcamdConvertPyInt64", _int, C.py_object,
+                           C.POINTER(C.c_int64), C.c_char_p, _sz)
+
+H2D, D2H, D2D = 0, 1, 2
+
+
+# ---------------------------------------------------------------------------
+# Device / queue with a Python error callback
+# ---------------------------------------------------------------------------
+class Context:
+    """One device and one queue (stream).  Error messages from the runtime's
+    callback are collected and raised as HcRuntimeError."""
+
+    def __init__(self, desc: str = "hip:0"):
+        self.desc = desc
+        self.messages: list[str] = []
+
+        def on_error(_ctx, _sev, text):
+            self.messages.append(text.decode(errors="replace").rstrip())
+
+        self._cb = ERROR_CALLBACK(on_error)     # keep alive
+        self.device = olCreateDevice(desc.encode(), self._cb, None)
+        if not self.device:
+            raise HcRuntimeError(self._drain() or f"olCreateDevice({desc!r}) failed")
+        self.queue = olCreateQueue(self.device)
+        if not self.queue:
+            msg = self._drain()
+            olReleaseDevice(self.device)
+            raise HcRuntimeError(msg or "olCreateQueue failed")
+
+    def _drain(self) -> str:
+        msg = "; ".join(self.messages)
+        self.messages.clear()
+        return msg
+
+    def check(self, rc: int, what: str) -> None:
+        if rc:
+            raise HcRuntimeError(f"{what}: {self._drain() or 'failed'}")
+
+    def synchronize(self) -> None:
+        self.check(olSyncQueue(self.queue), "olSyncQueue")
+
+    def info(self) -> dict:
+        cu, clk, mclk, bus = _int(), _int(), _int(), _int()
+        mem = _sz()
+        arch = C.create_string_buffer(64)
+        self.check(hcamdDeviceInfo(self.device, C.byref(cu), C.byref(clk), C.byref(mclk),
+                                   C.byref(bus), C.byref(mem), arch, 64), "hcamdDeviceInfo")
+        return {"compute_units": cu.value, "clock_khz": clk.value,
+                "mem_clock_khz": mclk.value, "mem_bus_bits": bus.value,
+                "total_mem": mem.value, "arch": arch.value.decode()}
+
+
+_default: Context | None = None
+
+
+def default_context(desc: str = "hip:0") -> Context:
+    """Process-wide context; the first device description wins, as in the
+    reference (python/cpp/py-runtime/src/GpuRuntime.cpp:31-39)."""
+    global _default
+    if _default is None:
+        _default = Context(desc)
+    return _default
+
+
+# ---------------------------------------------------------------------------
+# Arrays
+# ---------------------------------------------------------------------------
+@dataclass
+class Memref:
+    """ptr / shape / strides (elements) / itemsize of any array-like, obtained
+    through the PyObject* half of the C ABI (hcamdConvertPyArray)."""
+    ptr: int
+    shape: tuple
+    strides: tuple
+    itemsize: int
+
+    @property
+    def size(self) -> int:
+        return int(np.prod(self.shape, dtype=np.int64)) if self.shape else 1
+
+    def is_contiguous(self) -> bool:
+        acc = 1
+        for n, s in zip(reversed(self.shape), reversed(self.strides)):
+            if n != 1 and s != acc:
+                return False
+            acc *= n
+        return True
+
+
+def as_memref(obj, rank: int | None = None) -> Memref:
+    if rank is None:
+        rank = len(obj.shape)
+    words = (C.c_int64 * (3 + 2 * max(rank, 1)))()
+    item = _sz()
+    err = C.create_string_buffer(256)
+    if hcamdConvertPyArray(obj, rank, C.cast(words, _vp), C.byref(item), err, 256):
+        raise HcRuntimeError(err.value.decode(errors="replace"))
+    return Memref(ptr=int(words[1]) & (2 ** 64 - 1),
+                  shape=tuple(int(words[3 + i]) for i in range(rank)),
+                  strides=tuple(int(words[3 + rank + i]) for i in range(rank)),
+                  itemsize=int(item.value))
+
+
+_TYPESTR = {"float32": "<f4", "float16": "<f2", "int8": "|i1", "uint8": "|u1",
+            "int16": "<i2", "uint16": "<u2", "int32": "<i4", "uint32": "<u4",
+            "int64": "<i8", "uint64": "<u8", "float64": "<f8"}
+
+
+class DeviceArray:
+    """Dense row-major array in device memory owned by this object.  bf16 data
+    is held as uint16 bit patterns with `bf16=True` (NumPy has no bfloat16)."""
+
+    def __init__(self, shape, dtype, ctx: Context | None = None, bf16: bool = False):
+        self.ctx = ctx or default_context()
+        self.shape = tuple(int(s) for s in (shape if hasattr(shape, "__iter__") else (shape,)))
+        self.dtype = np.dtype(dtype)
+        self.bf16 = bool(bf16)
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
+        self.ptr = olAllocDevice(self.ctx.queue, max(self.nbytes, 16), 256)
+        if not self.ptr:
+            raise HcRuntimeError(self.ctx._drain() or "olAllocDevice failed")
+
+    # dense row-major strides in elements
+    @property
+    def strides(self):
+        out, acc = [], 1
+        for n in reversed(self.shape):
+            out.append(acc)
+            acc *= n
+        return tuple(reversed(out))
+
+    @property
+    def __cuda_array_interface__(self):
+        return {"shape": self.shape, "typestr": _TYPESTR[self.dtype.name],
+                "data": (int(self.ptr), False), "strides": None, "version": 2}
+
+    def copy_from_host(self, host: np.ndarray) -> "DeviceArray":
+        host = np.ascontiguousarray(host)
+        if host.nbytes != self.nbytes:
+            raise ValueError("size mismatch in copy_from_host")
+        self.ctx.check(hcamdMemcpy(self.ctx.queue, self.ptr, host.ctypes.data, self.nbytes, H2D),
+                       "hcamdMemcpy(H2D)")
+        self.ctx.synchronize()
+        return self
+
+    def to_host(self) -> np.ndarray:
+        out = np.empty(self.shape, self.dtype)
+        self.ctx.synchronize()
+        self.ctx.check(hcamdMemcpy(self.ctx.queue, out.ctypes.data, self.ptr, self.nbytes, D2H),
+                       "hcamdMemcpy(D2H)")
+        self.ctx.synchronize()
+        return out
+
+    def fill_bytes32(self, word: int) -> "DeviceArray":
+        self.ctx.check(hcamdFill32(self.ctx.queue, self.ptr, word & 0xFFFFFFFF,
+                                   (self.nbytes + 3) // 4), "hcamdFill32")
+        return self
+
+    def free(self) -> None:
+        if getattr(self, "ptr", None):
+            olDeallocDevice(self.ctx.queue, self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def to_device(host: np.ndarray, ctx: Context | None = None, bf16: bool = False) -> DeviceArray:
+    host = np.ascontiguousarray(host)
+    return DeviceArray(host.shape, host.dtype, ctx, bf16).copy_from_host(host)
+
+
+def empty_like(a: DeviceArray) -> DeviceArray:
+    return DeviceArray(a.shape, a.dtype, a.ctx, a.bf16)
+
+
+# ---------------------------------------------------------------------------
+# Typed launchers
+# ---------------------------------------------------------------------------
+def _ctx_of(*arrays) -> Context:
+    for a in arrays:
+        ctx = getattr(a, "ctx", None)
+        if isinstance(ctx, Context):
+            return ctx
+    return default_context()
+
+
+class Plan:
+    """A validated launch: the C entry point and its argument values.  Building
+    a plan does the Python-side checks and pointer extraction once; launch()
+    is then a single foreign call, which keeps the host out of the way when the
+    same kernel is enqueued many times."""
+
+    __slots__ = ("ctx", "fn", "args", "what", "keep")
+
+    def __init__(self, ctx, fn, args, what, keep=()):
+        self.ctx, self.fn, self.args, self.what, self.keep = ctx, fn, args, what, keep
+
+    def launch(self, sync: bool = False) -> None:
+        rc = self.fn(*self.args)
+        if rc:
+            self.ctx.check(rc, self.what)
+        if sync:
+            self.ctx.synchronize()
+
+
+def _rows_cols(m: Memref):
+    if len(m.shape) == 1:
+        return 1, m.shape[0], m.shape[0]
+    if len(m.shape) == 2:
+        if m.strides[1] != 1 and m.shape[1] > 1:
+            raise HcRuntimeError("rows must be contiguous (last stride 1)")
+        return m.shape[0], m.shape[1], (m.strides[0] if m.shape[0] > 1 else m.shape[1])
+    raise HcRuntimeError("expected a 1-D or 2-D array")
+
+
+def _expect(m: Memref, itemsize: int, name: str):
+    if m.itemsize != itemsize:
+        raise HcRuntimeError(f"{name}: element size {m.itemsize}, expected {itemsize}")
+
+
+def plan_copy2d(src, dst) -> Plan:
+    ctx = _ctx_of(src, dst)
+    s, d = as_memref(src), as_memref(dst)
+    if s.itemsize != d.itemsize or len(s.shape) != len(d.shape) or len(s.shape) not in (1, 2):
+        raise HcRuntimeError("copy2d: element size / rank mismatch")
+    if len(s.shape) == 1:
+        s = Memref(s.ptr, (1,) + s.shape, (0,) + s.strides, s.itemsize)
+        d = Memref(d.ptr, (1,) + d.shape, (0,) + d.strides, d.itemsize)
+    return Plan(ctx, hcamdLaunchCopy2D,
+                (ctx.queue, s.itemsize, s.ptr, s.shape[0], s.shape[1], s.strides[0],
+                 s.strides[1], d.ptr, d.shape[0], d.shape[1], d.strides[0], d.strides[1]),
+                "hcamdLaunchCopy2D", (src, dst))
+
+
+def plan_copy2d_tiled(src, dst, block_x: int, block_y: int, unroll: int = 1) -> Plan:
+    ctx = _ctx_of(src, dst)
+    s, d = as_memref(src, 2), as_memref(dst, 2)
+    if s.itemsize != d.itemsize or s.strides[1] != 1 or d.strides[1] != 1:
+        raise HcRuntimeError("copy2d_tiled: unit inner stride and equal element size required")
+    rows, cols = min(s.shape[0], d.shape[0]), min(s.shape[1], d.shape[1])
+    return Plan(ctx, hcamdLaunchCopy2DTiled,
+                (ctx.queue, s.itemsize, s.ptr, d.ptr, rows, cols, s.strides[0], d.strides[0],
+                 block_x, block_y, unroll), "hcamdLaunchCopy2DTiled", (src, dst))
+
+
+def plan_add_f32(a, b, c) -> Plan:
+    ctx = _ctx_of(a, b, c)
+    ma, mb, mc = as_memref(a), as_memref(b), as_memref(c)
+    for m, n in ((ma, "a"), (mb, "b"), (mc, "c")):
+        _expect(m, 4, n)
+        if not m.is_contiguous():
+            raise HcRuntimeError("add_f32: arrays must be contiguous")
+    if not (ma.size == mb.size == mc.size):
+        raise HcRuntimeError("add_f32: size mismatch")
+    return Plan(ctx, hcamdLaunchAddF32, (ctx.queue, ma.ptr, mb.ptr, mc.ptr, ma.size),
+                "hcamdLaunchAddF32", (a, b, c))
+
+
+def plan_fma_f16(a, b, c, d) -> Plan:
+    ctx = _ctx_of(a, b, c, d)
+    ms = [as_memref(v) for v in (a, b, c, d)]
+    geo = []
+    for m, n in zip(ms, "abcd"):
+        _expect(m, 2, n)
+        geo.append(_rows_cols(m))
+    rows, cols = geo[0][0], geo[0][1]
+    if any(g[0] != rows or g[1] != cols for g in geo):
+        raise HcRuntimeError("fma_f16: shape mismatch")
+    return Plan(ctx, hcamdLaunchFmaF16,
+                (ctx.queue, ms[0].ptr, geo[0][2], ms[1].ptr, geo[1][2], ms[2].ptr, geo[2][2],
+                 ms[3].ptr, geo[3][2], rows, cols), "hcamdLaunchFmaF16", (a, b, c, d))
+
+
+def plan_softmax_f32(x, y) -> Plan:
+    ctx = _ctx_of(x, y)
+    mx, my = as_memref(x, 2), as_memref(y, 2)
+    _expect(mx, 4, "x")
+    _expect(my, 4, "y")
+    rx, cx, ldx = _rows_cols(mx)
+    ry, cy, ldy = _rows_cols(my)
+    if (rx, cx) != (ry, cy):
+        raise HcRuntimeError("softmax_f32: shape mismatch")
+    return Plan(ctx, hcamdLaunchSoftmaxF32, (ctx.queue, mx.ptr, ldx, my.ptr, ldy, rx, cx),
+                "hcamdLaunchSoftmaxF32", (x, y))
+
+
+def plan_quantize_f16_i8(x, q, scale) -> Plan:
+    ctx = _ctx_of(x, q, scale)
+    mx, mq, ms = as_memref(x, 2), as_memref(q, 2), as_memref(scale, 1)
+    _expect(mx, 2, "x")
+    _expect(mq, 1, "q")
+    _expect(ms, 4, "scale")
+    rx, cx, ldx = _rows_cols(mx)
+    rq, cq, ldq = _rows_cols(mq)
+    if (rx, cx) != (rq, cq) or ms.shape[0] != rx or not ms.is_contiguous():
+        raise HcRuntimeError("quantize_f16_i8: shape mismatch")
+    return Plan(ctx, hcamdLaunchQuantizeF16I8,
+                (ctx.queue, mx.ptr, ldx, mq.ptr, ldq, ms.ptr, rx, cx),
+                "hcamdLaunchQuantizeF16I8", (x, q, scale))
+
+
+def plan_gemm_bf16(a, bt, c) -> Plan:
+    """C[M,N] = A[M,K] @ Bt[N,K].T, bf16 bit patterns in 2-byte arrays."""
+    ctx = _ctx_of(a, bt, c)
+    ma, mb, mc = as_memref(a, 2), as_memref(bt, 2), as_memref(c, 2)
+    for m, n in ((ma, "a"), (mb, "bt"), (mc, "c")):
+        _expect(m, 2, n)
+    m_, k_, lda = _rows_cols(ma)
+    n_, k2, ldb = _rows_cols(mb)
+    m2, n2, ldc = _rows_cols(mc)
+    if k_ != k2 or m_ != m2 or n_ != n2:
+        raise HcRuntimeError("gemm_bf16: shape mismatch")
+    return Plan(ctx, hcamdLaunchGemmBF16,
+                (ctx.queue, ma.ptr, lda, mb.ptr, ldb, mc.ptr, ldc, m_, n_, k_),
+                "hcamdLaunchGemmBF16", (a, bt, c))
+
+
+# Call-and-wait forms: a kernel call is synchronous on return by default, as in
+# the reference (python/cpp/py-runtime/src/GpuRuntime.cpp:60-69).
+def copy2d(src, dst, sync: bool = True) -> None:
+    plan_copy2d(src, dst).launch(sync)
+
+
+def copy2d_tiled(src, dst, block_x: int, block_y: int, unroll: int = 1, sync: bool = True) -> None:
+    plan_copy2d_tiled(src, dst, block_x, block_y, unroll).launch(sync)
+
+
+def add_f32(a, b, c, sync: bool = True) -> None:
+    plan_add_f32(a, b, c).launch(sync)
+
+
+def fma_f16(a, b, c, d, sync: bool = True) -> None:
+    plan_fma_f16(a, b, c, d).launch(sync)
+
+
+def softmax_f32(x, y, sync: bool = True) -> None:
+    plan_softmax_f32(x, y).launch(sync)
+
+
+def quantize_f16_i8(x, q, scale, sync: bool = True) -> None:
+    plan_quantize_f16_i8(x, q, scale).launch(sync)
+
+
+def gemm_bf16(a, bt, c, sync: bool = True) -> None:
+    plan_gemm_bf16(a, bt, c).launch(sync)
+
+
+def set_variant(family: str, variant: int) -> None:
+    if hcamdSetVariant(family.encode(), int(variant)):
+        raise HcRuntimeError(f"unknown kernel family {family!r}")
+
+
+def last_kernel_name() -> str:
+    return (hcamdLastKernelName() or b"").decode()
+
+
+# ---------------------------------------------------------------------------
+# Events
+# ---------------------------------------------------------------------------
+class Event:
+    def __init__(self, ctx: Context | None = None):
+        self.ctx = ctx or default_context()
+        self.handle = hcamdEventCreate(self.ctx.queue)
+        if not self.handle:
+            raise HcRuntimeError(self.ctx._drain() or "hcamdEventCreate failed")
+
+    def record(self):
+        self.ctx.check(hcamdEventRecord(self.handle), "hcamdEventRecord")
+
+    def synchronize(self):
+        self.ctx.check(hcamdEventSynchronize(self.handle), "hcamdEventSynchronize")
+
+    def elapsed_ms(self, stop: "Event") -> float:
+        ms = C.c_float()
+        self.ctx.check(hcamdEventElapsedMs(self.handle, stop.handle, C.byref(ms)),
+                       "hcamdEventElapsedMs")
+        return float(ms.value)
+
+    def __del__(self):
+        try:
+            if self.handle:
+                hcamdEventDestroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+def builtin_modules() -> dict[str, tuple[int, int]]:
+    """name -> (address, length) of the embedded gfx950 code objects."""
+    out = {}
+    for i in range(hcamdBuiltinModuleCount()):
+        name, data, n = C.c_char_p(), _vp(), _sz()
+        hcamdGetBuiltinModule(i, C.byref(name), C.byref(data), C.byref(n))
+        out[name.value.decode()] = (int(data.value), int(n.value))
+    return out

@@ -1,0 +1,568 @@
+"""GPU parity: every kernel, called through the C ABI (hc_amd.runtime is a ctypes
+shim over libhc_amd_runtime.so), against the CPU oracle on the same seeded
+inputs.  Integer / byte / fp16 results are compared bit for bit; fp32 softmax
+within rtol 1e-5; bf16 GEMM within rtol 1e-2 of an fp32 accumulation (and bit
+for bit where the arithmetic is exact).  Full benchmark sizes are covered by
+the NumPy closed forms and by size-independent properties."""
+
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+from numpy.testing import assert_allclose, assert_array_equal
+
+from hc_amd import runtime as rt
+from oracle import c_oracle as co
+from oracle import closed_forms as cf
+
+pytestmark = pytest.mark.gpu
+
+POISON32 = 0xA5A5A5A5
+
+
+def say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = rt.default_context("hip:0")
+    say("device:", c.info())
+    return c
+
+
+@pytest.fixture(autouse=True)
+def default_variants():
+    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy"):
+        rt.set_variant(fam, 0)
+    yield
+    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy"):
+        rt.set_variant(fam, 0)
+
+
+def dev(a, **kw):
+    return rt.to_device(a, **kw)
+
+
+def poisoned(shape, dtype):
+    return rt.DeviceArray(shape, dtype).fill_bytes32(POISON32)
+
+
+def poison_value(dtype):
+    return np.frombuffer(np.array([POISON32] * 4, np.uint32).tobytes(), dtype)[0]
+
+
+class _View:
+    """A window of a DeviceArray, exposed through __cuda_array_interface__."""
+
+    def __init__(self, base, shape, offset_elems=0, strides=None):
+        self.shape = tuple(shape)
+        self.ctx = base.ctx
+        item = base.dtype.itemsize
+        self.__cuda_array_interface__ = {
+            "shape": self.shape, "typestr": rt._TYPESTR[base.dtype.name],
+            "data": (int(base.ptr) + offset_elems * item, False),
+            "strides": None if strides is None else tuple(s * item for s in strides),
+            "version": 2}
+
+
+def _view(base, n, offset=0):
+    return _View(base, (n,), offset)
+
+
+# ---------------------------------------------------------------------------
+# runtime plumbing
+# ---------------------------------------------------------------------------
+def test_device_is_gfx950(ctx):
+    info = ctx.info()
+    assert info["arch"].startswith("gfx950"), info
+    assert info["compute_units"] >= 200
+
+
+def test_memcpy_round_trip_and_fill(ctx):
+    a = np.random.default_rng(0).integers(0, 255, 1_000_003, dtype=np.uint8)
+    d = dev(a)
+    assert_array_equal(d.to_host(), a)
+    p = poisoned((1000,), np.uint32)
+    assert_array_equal(p.to_host(), np.full(1000, POISON32, np.uint32))
+
+
+def test_generic_module_kernel_launch_path(ctx):
+    """olCreateModule / olGetKernel / olLaunchKernel with an embedded code
+    object, the way the reference's generated host code drives the runtime
+    (hcgpuGetKernel / hcgpuLaunchKernel), using the reference's kernel argument
+    list for a 2-D copy: (i64, i64 stride, ptr, i64 rows, i64 cols, i64 stride,
+    ptr)."""
+    rows, cols = 111, 813
+    a = np.arange(rows * cols, dtype=np.int32).reshape(rows, cols)
+    src, dst = dev(a), poisoned((rows, cols), np.int32)
+    addr, n = rt.builtin_modules()["copy"]
+    mod = rt.olCreateModule(ctx.device, addr, n)
+    assert mod
+    k = rt.olGetKernel(mod, b"hcamd_copy2d_tiled_b4")
+    assert k
+    # geometry exactly as the reference derives it: block from the suggestion
+    # for the reversed work shape, grid = reversed group counts
+    g = (C.c_size_t * 2)(cols, rows)
+    b = (C.c_size_t * 2)()
+    assert rt.olSuggestBlockSize(k, g, b, 2) == 0
+    assert tuple(b) == (813, 1)
+    grid = (C.c_size_t * 3)(-(-cols // b[0]), -(-rows // b[1]), 1)
+    block = (C.c_size_t * 3)(b[0], b[1], 1)
+    vals = [C.c_int64(1), C.c_int64(cols), C.c_void_p(src.ptr), C.c_int64(rows),
+            C.c_int64(cols), C.c_int64(cols), C.c_void_p(dst.ptr)]
+    args = (C.c_void_p * len(vals))(*[C.cast(C.pointer(v), C.c_void_p) for v in vals])
+    assert rt.olLaunchKernel(ctx.queue, k, grid, block, 3, args, len(vals), 0) == 0
+    ctx.synchronize()
+    assert_array_equal(dst.to_host(), a)
+    # nDims != 3 is rejected with the reference's message
+    assert rt.olLaunchKernel(ctx.queue, k, grid, block, 2, args, len(vals), 0) == 1
+    assert "Invalid launch dims: 2" in ctx._drain()
+    # unknown kernel name
+    assert rt.olGetKernel(mod, b"no_such_kernel") is None
+    assert "hipModuleGetFunction" in ctx._drain()
+    rt.olReleaseKernel(k)
+    rt.olReleaseModule(mod)
+
+
+def test_hcgpu_entry_points_cache_and_launch_synchronously(ctx):
+    rows, cols = 10, 20
+    a = np.arange(rows * cols, dtype=np.int32).reshape(rows, cols)
+    src, dst = dev(a), poisoned((rows, cols), np.int32)
+    addr, n = rt.builtin_modules()["copy"]
+    handle = C.c_void_p()
+    k = rt.hcgpuGetKernel(C.byref(handle), b"hip:0", addr, n, b"hcamd_copy2d_tiled_b4")
+    assert k and handle.value == k
+    assert rt.hcgpuGetKernel(C.byref(handle), b"hip:0", None, 0, b"ignored") == k   # cached
+    grid = (C.c_size_t * 3)(1, rows, 1)
+    block = (C.c_size_t * 3)(cols, 1, 1)
+    vals = [C.c_int64(1), C.c_int64(cols), C.c_void_p(src.ptr), C.c_int64(rows),
+            C.c_int64(cols), C.c_int64(cols), C.c_void_p(dst.ptr)]
+    args = (C.c_void_p * len(vals))(*[C.cast(C.pointer(v), C.c_void_p) for v in vals])
+    rt.hcgpuLaunchKernel(k, grid, block, 3, args, len(vals), 0)
+    # no explicit synchronisation: the call returns after the kernel finished
+    out = np.empty_like(a)
+    assert rt.hcamdMemcpy(ctx.queue, out.ctypes.data, dst.ptr, out.nbytes, rt.D2H) == 0
+    ctx.synchronize()
+    assert_array_equal(out, a)
+
+
+# ---------------------------------------------------------------------------
+# W0 masked tile copy (python/hckernel/tests/test_e2e.py:46-136)
+# ---------------------------------------------------------------------------
+E2E_SHAPES = [(1, 27), (1, 72), (1, 128), (10, 20), (111, 813), (256, 64), (256, 1024)]
+
+
+@pytest.mark.parametrize("shape", E2E_SHAPES)
+def test_copy_e2e_shapes_flat_path(ctx, shape):
+    a = np.arange(shape[0] * shape[1], dtype=np.int32).reshape(shape)
+    src, dst = dev(a), dev(np.zeros_like(a))
+    rt.copy2d(src, dst)
+    assert rt.last_kernel_name().startswith("hcamd_copy_flat")
+    assert_array_equal(dst.to_host(), a)
+
+
+@pytest.mark.parametrize("shape", E2E_SHAPES)
+@pytest.mark.parametrize("unroll", [1, 2, 4])
+def test_copy_e2e_shapes_reference_geometry(ctx, shape, unroll):
+    """Tile decomposition of the reference: work_shape (W, ceil(H/V)), group
+    shape from olSuggestBlockSize, each group copies a (gs0, gs1*V) tile."""
+    rows, cols = shape
+    a = np.arange(rows * cols, dtype=np.int32).reshape(shape)
+    src, dst = dev(a), poisoned(shape, np.int32)
+    work = (rows, -(-cols // unroll))
+    gs = cf.default_group_shape(work)
+    rt.copy2d_tiled(src, dst, block_x=gs[1], block_y=gs[0], unroll=unroll)
+    assert_array_equal(dst.to_host(), a)
+
+
+@pytest.mark.parametrize("itemsize,dtype", [(1, np.uint8), (2, np.uint16), (4, np.int32),
+                                            (8, np.int64)])
+def test_copy_window_smaller_than_destination_leaves_rest_untouched(ctx, itemsize, dtype):
+    rng = np.random.default_rng(itemsize)
+    a = rng.integers(0, 200, (37, 101)).astype(dtype)
+    src, dst = dev(a), poisoned((50, 130), dtype)
+    rt.copy2d(src, dst)                       # window 37 x 101 of a 50 x 130 array
+    assert rt.last_kernel_name() == f"hcamd_copy2d_b{itemsize}"
+    want = cf.np_copy_window(a, np.full((50, 130), poison_value(dtype), dtype))
+    assert_array_equal(dst.to_host(), want)
+    big = dev(rng.integers(0, 200, (64, 140)).astype(dtype))
+    small = poisoned((5, 9), dtype)
+    rt.copy2d(big, small)                     # source larger than destination
+    assert_array_equal(small.to_host(), big.to_host()[:5, :9])
+
+
+def test_copy_large_flat_all_variants(ctx):
+    a = np.random.default_rng(1).integers(0, 2 ** 31, 4_000_037, dtype=np.int32)[None, :]
+    src = dev(a)
+    for v in range(0, 9):
+        rt.set_variant("copy", v)
+        dst = poisoned((1, a.size + 16), np.int32)
+        rt.copy2d(src, dst)
+        out = dst.to_host()
+        assert_array_equal(out[:, :a.size], a)
+        assert (out[:, a.size:] == np.int32(poison_value(np.int32))).all(), rt.last_kernel_name()
+
+
+# ---------------------------------------------------------------------------
+# W1 c = a + b
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("n", [1, 3, 4, 255, 1024, 4099, 262_144, 1_000_003])
+def test_add_bit_exact_with_untouched_tail(ctx, n):
+    a, b = cf.inputs_c1(n)
+    want = cf.np_add(a, b)
+    assert_array_equal(want.view(np.uint32), co.add_f32(a, b).view(np.uint32))
+    da, db = dev(a), dev(b)
+    for v in range(0, 10):
+        rt.set_variant("add", v)
+        dc = poisoned((n + 8,), np.float32)
+        rt.add_f32(da, db, _view(dc, n))
+        out = dc.to_host()
+        assert_array_equal(out[:n].view(np.uint32), want.view(np.uint32))
+        assert (out[n:].view(np.uint32) == POISON32).all(), (v, rt.last_kernel_name())
+
+
+def test_add_misaligned_pointers_take_the_scalar_kernel(ctx):
+    n = 10_001
+    a, b = cf.inputs_c1(n + 1)
+    da, db, dc = dev(a), dev(b), poisoned((n + 9,), np.float32)
+    rt.add_f32(_view(da, n, 1), _view(db, n, 1), _view(dc, n, 1))
+    assert rt.last_kernel_name() == "hcamd_add_f32_scalar"
+    out = dc.to_host()
+    assert_array_equal(out[1:n + 1].view(np.uint32), (a[1:] + b[1:]).view(np.uint32))
+    assert out.view(np.uint32)[0] == POISON32 and (out.view(np.uint32)[n + 1:] == POISON32).all()
+
+
+def test_add_full_benchmark_size(ctx):
+    a, b = cf.inputs_c1()
+    assert a.size == 16_777_259
+    dc = rt.DeviceArray(a.shape, np.float32)
+    rt.add_f32(dev(a), dev(b), dc)
+    assert_array_equal(dc.to_host().view(np.uint32), cf.np_add(a, b).view(np.uint32))
+
+
+def test_add_special_values(ctx):
+    f = np.float32
+    a = np.array([np.inf, -np.inf, np.inf, 1e-45, -0.0, 3e38, 1.0, 16777216.0], f)
+    b = np.array([1.0, 1.0, -np.inf, 1e-45, 0.0, 3e38, 2.0 ** -24, 1.0], f)
+    dc = rt.DeviceArray(a.shape, f)
+    rt.add_f32(dev(a), dev(b), dc)
+    with np.errstate(all="ignore"):
+        want = a + b
+    out = dc.to_host()
+    assert_array_equal(np.isnan(out), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert_array_equal(out[ok].view(np.uint32), want[ok].view(np.uint32))   # denormals kept
+
+
+# ---------------------------------------------------------------------------
+# W2 d = a * b + c (fp16 storage, fp32 arithmetic)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (1, 4099), (17, 4099), (129, 1031)])
+def test_fma_bit_exact_all_variants(ctx, shape):
+    a, b, c = cf.inputs_c2(shape)
+    want = cf.np_fma_f16(a, b, c)
+    assert_array_equal(want.view(np.uint16), co.fma_f16(a, b, c).view(np.uint16))
+    da, db, dc = dev(a), dev(b), dev(c)
+    for v in range(0, 8):
+        rt.set_variant("fma", v)
+        dd = poisoned((shape[0] * shape[1] + 16,), np.float16)
+        out_view = _View(dd, shape)
+        rt.fma_f16(da, db, dc, out_view)
+        out = dd.to_host()
+        assert_array_equal(out[:want.size].view(np.uint16), want.ravel().view(np.uint16))
+        assert (out[want.size:].view(np.uint16) == 0xA5A5).all(), (v, rt.last_kernel_name())
+
+
+def test_fma_strided_rows(ctx):
+    rows, cols, ld = 33, 1000, 1024
+    a, b, c = cf.inputs_c2((rows, ld))
+    da, db, dc = dev(a), dev(b), dev(c)
+    dd = poisoned((rows, ld), np.float16)
+    views = [_View(x, (rows, cols), 0, (ld, 1)) for x in (da, db, dc, dd)]
+    rt.fma_f16(*views)
+    assert rt.last_kernel_name() == "hcamd_fma_f16_2d"
+    out = dd.to_host()
+    assert_array_equal(out[:, :cols].view(np.uint16),
+                       cf.np_fma_f16(a[:, :cols], b[:, :cols], c[:, :cols]).view(np.uint16))
+    assert (out[:, cols:].view(np.uint16) == 0xA5A5).all()
+
+
+def test_fma_special_values(ctx):
+    h = np.float16
+    a = np.array([[6e-8, 6e-8, 300, -300, 0.0, 1.0, 2.0 ** -14, 65504, 1.0]], h)
+    b = np.array([[1.0, 0.5, 300, 300, -1.0, 1.0, 0.5, 1.0, 1.0]], h)
+    c = np.array([[0.0, 0.0, 0.0, 0.0, 0.0, 2.0 ** -11, 0.0, 15.9, 2.0 ** -10]], h)
+    dd = rt.DeviceArray(a.shape, h)
+    rt.fma_f16(dev(a), dev(b), dev(c), dd)
+    with np.errstate(over="ignore"):
+        want = cf.np_fma_f16(a, b, c)
+    assert_array_equal(dd.to_host().view(np.uint16), want.view(np.uint16))
+
+
+def test_fma_full_benchmark_size(ctx):
+    a, b, c = cf.inputs_c2()
+    assert a.shape == (8191, 8193)
+    dd = rt.DeviceArray(a.shape, np.float16)
+    rt.fma_f16(dev(a), dev(b), dev(c), dd)
+    assert rt.last_kernel_name().startswith("hcamd_fma_f16_v")
+    assert_array_equal(dd.to_host().view(np.uint16), cf.np_fma_f16(a, b, c).view(np.uint16))
+
+
+# ---------------------------------------------------------------------------
+# W3 row softmax
+# ---------------------------------------------------------------------------
+SOFTMAX_RTOL = 1e-5      # the tolerance the task states for fp32 results
+SOFTMAX_ATOL = 1e-9
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (5, 7), (33, 256), (7, 257), (64, 1000), (16, 1024),
+                                   (8, 2048), (9, 4097), (12, 8192), (5, 8190), (3, 16384),
+                                   (3, 12345), (2, 20000), (1030, 512)])
+def test_softmax_against_both_oracles(ctx, shape):
+    (x,) = cf.inputs_c3(shape)
+    dy = poisoned(shape, np.float32)
+    rt.softmax_f32(dev(x), dy)
+    say("softmax", shape, rt.last_kernel_name())
+    y = dy.to_host()
+    assert_allclose(y, cf.np_softmax(x), rtol=SOFTMAX_RTOL, atol=SOFTMAX_ATOL)
+    assert_allclose(y, co.softmax(x, f64=True), rtol=4e-6, atol=SOFTMAX_ATOL)
+    assert_allclose(y.astype(np.float64).sum(1), 1.0, atol=2e-6)
+
+
+def test_softmax_variants_and_strided_rows(ctx):
+    rows, cols, ld = 19, 8192, 8200
+    (x,) = cf.inputs_c3((rows, ld))
+    want = cf.np_softmax(x[:, :cols])
+    dx = dev(x)
+    for v in (0, 1, 2, 3):
+        rt.set_variant("softmax", v)
+        dy = poisoned((rows, ld), np.float32)
+        rt.softmax_f32(_View(dx, (rows, cols), 0, (ld, 1)), _View(dy, (rows, cols), 0, (ld, 1)))
+        say("softmax variant", v, rt.last_kernel_name())
+        out = dy.to_host()
+        assert_allclose(out[:, :cols], want, rtol=SOFTMAX_RTOL, atol=SOFTMAX_ATOL)
+        assert (out[:, cols:].view(np.uint32) == POISON32).all()
+    # unaligned base pointer -> streaming kernel
+    rt.set_variant("softmax", 0)
+    dy = poisoned((rows, ld), np.float32)
+    rt.softmax_f32(_View(dx, (rows, 1000), 1, (ld, 1)), _View(dy, (rows, 1000), 1, (ld, 1)))
+    assert rt.last_kernel_name() == "hcamd_softmax_f32_stream"
+    assert_allclose(dy.to_host()[:, 1:1001], cf.np_softmax(x[:, 1:1001]), rtol=SOFTMAX_RTOL,
+                    atol=SOFTMAX_ATOL)
+
+
+def test_softmax_extreme_and_special_rows(ctx):
+    f = np.float32
+    x = np.zeros((6, 1024), f)
+    x[0, :] = 1.25                                   # constant row: exactly 1/1024
+    x[1, :] = np.linspace(-80, 80, 1024)             # wide range, tiny tails
+    x[2, 5] = np.nan                                 # NaN anywhere -> NaN row
+    x[3, 7] = np.inf                                 # +inf -> NaN row (inf - inf)
+    x[4, :] = -np.inf                                # all -inf -> NaN row
+    x[5, :] = -1e30
+    x[5, 3] = 0.0                                    # one-hot
+    dy = rt.DeviceArray(x.shape, f)
+    rt.softmax_f32(dev(x), dy)
+    y = dy.to_host()
+    assert_array_equal(y[0], np.full(1024, 1 / 1024, f))
+    with np.errstate(all="ignore"):
+        want = cf.np_softmax(x)
+    assert_allclose(y[1], want[1], rtol=SOFTMAX_RTOL, atol=1e-30)
+    assert np.isnan(y[2]).all() and np.isnan(y[3]).all() and np.isnan(y[4]).all()
+    assert np.isnan(want[2]).all() and np.isnan(want[3]).all() and np.isnan(want[4]).all()
+    assert y[5, 3] == 1.0 and y[5].sum() == 1.0
+
+
+def test_softmax_reference_test_input(ctx):
+    # python/hckernel/tests/test_examples.py:322-335 (float64 there)
+    m, n = 30, 25
+    a = (2 * np.arange(m * n).reshape(m, n) / (m * n)).astype(np.float32)
+    dy = rt.DeviceArray(a.shape, np.float32)
+    rt.softmax_f32(dev(a), dy)
+    assert_allclose(dy.to_host(), cf.np_softmax(a.astype(np.float64)), rtol=2e-6)
+
+
+def test_softmax_full_benchmark_size(ctx):
+    (x,) = cf.inputs_c3()
+    assert x.shape == (4096, 8192)
+    dy = rt.DeviceArray(x.shape, np.float32)
+    rt.softmax_f32(dev(x), dy)
+    assert rt.last_kernel_name().startswith("hcamd_softmax_f32_g256_v8_full")
+    y = dy.to_host()
+    assert_allclose(y, cf.np_softmax(x), rtol=SOFTMAX_RTOL, atol=SOFTMAX_ATOL)
+    assert_allclose(y.astype(np.float64).sum(1), 1.0, atol=2e-6)
+    assert_array_equal(y.argmax(1), x.argmax(1))
+
+
+# ---------------------------------------------------------------------------
+# W4 row absmax int8 quantisation
+# ---------------------------------------------------------------------------
+def run_quantize(x, ld=None):
+    rows, cols = x.shape
+    ld = ld or cols
+    ldq = ld if ld == cols else (ld + 15) // 16 * 16
+    xp = np.zeros((rows, ld), np.float16)
+    xp[:, :cols] = x
+    dq = poisoned((rows, ldq), np.int8)
+    ds = poisoned((rows,), np.float32)
+    dx = dev(xp)
+    rt.quantize_f16_i8(_View(dx, (rows, cols), 0, (ld, 1)), _View(dq, (rows, cols), 0, (ldq, 1)), ds)
+    q = dq.to_host()
+    assert (q[:, cols:].view(np.uint8) == 0xA5).all(), "wrote past the row"
+    return q[:, :cols], ds.to_host()
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (3, 15), (5, 16), (7, 1000), (33, 1024), (9, 2047),
+                                   (64, 4096), (11, 4100), (6, 8192), (3, 16400), (2, 32768),
+                                   (2, 40000), (1027, 64)])
+def test_quantize_bit_exact(ctx, shape):
+    (x,) = cf.inputs_c4(shape)
+    q, s = run_quantize(x)
+    say("quantize", shape, rt.last_kernel_name())
+    q_np, s_np = cf.np_quantize(x)
+    assert_array_equal(q, q_np)
+    assert_array_equal(s.view(np.uint32), s_np.view(np.uint32))
+    if x.size < 200_000:
+        q_c, s_c = co.quantize(x)
+        assert_array_equal(q, q_c)
+
+
+def test_quantize_variants_and_strides(ctx):
+    (x,) = cf.inputs_c4((301, 4096))
+    q_np, s_np = cf.np_quantize(x)
+    for v in range(0, 7):
+        rt.set_variant("quantize", v)
+        for ld in (4096, 4096 + 64):
+            q, s = run_quantize(x, ld)
+            say("quantize variant", v, ld, rt.last_kernel_name())
+            assert_array_equal(q, q_np)
+            assert_array_equal(s.view(np.uint32), s_np.view(np.uint32))
+
+
+def test_quantize_every_fp16_value_against_many_scales(ctx):
+    """Each row holds an absmax and 4095 arbitrary finite fp16 values below it,
+    drawn from the bit patterns directly so that every exponent (subnormals
+    included) and rounding position is hit; 4096 rows, 16.7 M quotients, bit for
+    bit against the IEEE-division statement."""
+    rng = np.random.default_rng(44)
+    rows, cols = 4096, 4096
+    amax_bits = rng.integers(1, 0x7C00, rows).astype(np.uint16)
+    frac = rng.random((rows, cols))
+    bits = (frac * (amax_bits[:, None].astype(np.float64) + 1)).astype(np.uint16)
+    bits = np.minimum(bits, amax_bits[:, None])
+    bits[:, 0] = amax_bits
+    bits |= (rng.integers(0, 2, (rows, cols)).astype(np.uint16) << 15)
+    x = bits.view(np.float16)
+    q_np, s_np = cf.np_quantize(x)
+    for v in (0, 2):
+        rt.set_variant("quantize", v)
+        q, s = run_quantize(x)
+        assert_array_equal(q, q_np)
+        assert_array_equal(s.view(np.uint32), s_np.view(np.uint32))
+
+
+def test_quantize_ties_and_special_rows(ctx):
+    h = np.float16
+    for e in (-3, 0, 2):
+        ks = np.array([0, 1, 2, 3, 4, 125, 126], np.float32)
+        x = (np.concatenate([ks + 0.5, -(ks + 0.5), [127.0]]) * 2.0 ** e).astype(h)[None, :]
+        q, s = run_quantize(np.repeat(x, 3, 0))
+        assert s[0] == np.float32(2.0 ** e)
+        assert_array_equal(q[0], [0, 2, 2, 4, 4, 126, 126, 0, -2, -2, -4, -4, -126, -126, 127])
+    rows = np.zeros((4, 64), h)
+    rows[1, 3], rows[1, 5] = np.nan, 2.0
+    rows[2, 0], rows[2, 1], rows[2, 2] = np.inf, 1.0, -np.inf
+    rows[3, :3] = [6e-8, -6e-8, 3e-8]
+    q, s = run_quantize(rows)
+    q_np, s_np = cf.np_quantize(rows)
+    assert s[0] == 0 and np.isnan(s[1]) and np.isinf(s[2])
+    assert_array_equal(q, q_np)
+    assert_array_equal(q[3, :3], [127, -127, 127])
+
+
+def test_quantize_full_benchmark_size(ctx):
+    (x,) = cf.inputs_c4()
+    assert x.shape == (16384, 4096)
+    q, s = run_quantize(x)
+    q_np, s_np = cf.np_quantize(x)
+    assert_array_equal(q, q_np)
+    assert_array_equal(s.view(np.uint32), s_np.view(np.uint32))
+    # size-independent property: dequantisation error is at most half a step
+    err = np.abs(q.astype(np.float32) * s[:, None] - x.astype(np.float32))
+    assert (err <= 0.5000001 * s[:, None]).all()
+
+
+# ---------------------------------------------------------------------------
+# W5 GEMM
+# ---------------------------------------------------------------------------
+GEMM_RTOL = 1e-2
+
+
+def run_gemm(ab, bb, ldc_pad=0):
+    m, n = ab.shape[0], bb.shape[0]
+    dc = poisoned((m, n + ldc_pad), np.uint16)
+    rt.gemm_bf16(dev(ab), dev(bb), _View(dc, (m, n), 0, (n + ldc_pad, 1)))
+    out = dc.to_host()
+    if ldc_pad:
+        assert (out[:, n:] == 0xA5A5).all()
+    return out[:, :n]
+
+
+@pytest.mark.parametrize("mnk", [(256, 256, 64), (256, 512, 128), (512, 256, 256), (128, 128, 64),
+                                 (384, 128, 192), (33, 47, 96), (100, 200, 300), (1, 1, 1),
+                                 (64, 64, 8), (257, 255, 130)])
+def test_gemm_exact_integer_matrices_bit_for_bit(ctx, mnk):
+    m, n, k = mnk
+    rng = np.random.default_rng(m * 7 + n)
+    a = rng.integers(-4, 5, (m, k)).astype(np.float32)
+    bt = rng.integers(-4, 5, (n, k)).astype(np.float32)
+    want = cf.f32_to_bf16_bits((a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32))
+    got = run_gemm(cf.f32_to_bf16_bits(a), cf.f32_to_bf16_bits(bt))
+    say("gemm", mnk, rt.last_kernel_name())
+    assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("mnk", [(256, 256, 256), (512, 768, 1024), (128, 384, 512),
+                                 (100, 200, 300), (77, 33, 4097)])
+def test_gemm_random_within_tolerance(ctx, mnk):
+    ab, bb = cf.inputs_c5(mnk)
+    got = cf.bf16_bits_to_f32(run_gemm(ab, bb))
+    want = cf.np_gemm_bf16(ab, bb, np.float32)
+    sigma = 0.02 * 0.02 * np.sqrt(mnk[2])
+    assert_allclose(got, want, rtol=GEMM_RTOL, atol=1e-2 * sigma)
+    # the result is the fp64 product rounded to bf16, give or take one bf16 ulp
+    exact = cf.np_gemm_bf16(ab, bb, np.float64)
+    assert np.abs(got - exact).max() <= 2.0 ** -8 * np.abs(exact).max()
+    if mnk[0] * mnk[1] * mnk[2] <= 256 ** 3:
+        _, c32 = co.gemm_bf16(ab, bb)
+        assert_allclose(got, c32, rtol=GEMM_RTOL, atol=1e-2 * sigma)
+
+
+def test_gemm_all_variants_and_padded_output(ctx):
+    ab, bb = cf.inputs_c5((512, 512, 256))
+    want = cf.np_gemm_bf16(ab, bb, np.float32)
+    sigma = 0.02 * 0.02 * 16
+    for v in range(0, 8):
+        rt.set_variant("gemm", v)
+        got = cf.bf16_bits_to_f32(run_gemm(ab, bb, ldc_pad=8))
+        say("gemm variant", v, rt.last_kernel_name())
+        assert_allclose(got, want, rtol=GEMM_RTOL, atol=1e-2 * sigma)
+
+
+def test_gemm_full_benchmark_size_and_linearity(ctx):
+    ab, bb = cf.inputs_c5()
+    assert ab.shape == (4096, 4096) and bb.shape == (4096, 4096)
+    got_bits = run_gemm(ab, bb)
+    assert rt.last_kernel_name().startswith("hcamd_gemm_bf16_256x256")
+    got = cf.bf16_bits_to_f32(got_bits)
+    want = cf.np_gemm_bf16(ab, bb, np.float32)
+    assert_allclose(got, want, rtol=GEMM_RTOL, atol=2.6e-4)
+    # linearity: scaling A by 2 is exact in bf16 and in every partial sum
+    a2 = cf.f32_to_bf16_bits(cf.bf16_bits_to_f32(ab) * np.float32(2))
+    got2 = cf.bf16_bits_to_f32(run_gemm(a2, bb))
+    assert_array_equal(got2, got * np.float32(2))
+    # identity: A @ I = A exactly
+    eye = cf.f32_to_bf16_bits(np.eye(4096, dtype=np.float32))
+    assert_array_equal(run_gemm(ab, eye), ab)
