@@ -1,0 +1,394 @@
+"""Matches a traced per-group program against the hand-written gfx950 kernels.
+
+The reference lowers a kernel body through its compiler; this build has a fixed
+set of hand-written kernels instead, so a traced body is recognised
+structurally:
+
+    copy       store(load a)
+    add        store(load a + load b)                                  fp32
+    fma        store((f32 a * f32 b + f32 c) -> f16)                   fp16 storage
+    softmax    store(exp(x - max_row x) / sum_row exp(x - max_row x))  fp32 rows
+    quantize   store(int8 clip(rint(f32 x / s), -127, 127)), s = max_row|x| / 127
+    gemm       store(sum_k dot(load A[m, k-chunk], load Bt[n, k-chunk].T))   bf16
+
+Every load and the store must walk their buffers tile by tile: the start along a
+dimension is either 0 or group_id[i] * tile_extent, so that the tiles of all
+groups are disjoint and their union is a window [0, rows) x [0, cols) of the
+buffer.  That window, not the user's tile shape, is what the native kernel
+receives: it re-tiles the window for the hardware (16-byte accesses, wave64
+reductions, MFMA blocks).  A body that matches nothing raises NoNativeKernel;
+there is no interpreter or CPU path behind it.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+from . import runtime as rt
+from .kernel_api import Affine, BufferView, Tile, TraceError
+
+
+class NoNativeKernel(RuntimeError):
+    """The traced kernel body does not correspond to a hand-written kernel."""
+
+
+# ---------------------------------------------------------------------------
+# Windows
+# ---------------------------------------------------------------------------
+@dataclass
+class Window:
+    """Union over all groups of one tiled access: [0, extent[d]) per dim."""
+    buffer: int          # argument index
+    extent: tuple        # elements per dim
+    driver: tuple        # group dim that walks each buffer dim, or None
+    tile: tuple
+
+
+def _coeffs(a: Affine, rank: int):
+    return tuple(a.coeffs) + (0,) * (rank - len(a.coeffs))
+
+
+def window_of(view: BufferView, tile_shape, n_groups) -> Window:
+    rank = len(n_groups)
+    extent, driver = [], []
+    used = set()
+    for d, (start, t) in enumerate(zip(view.starts, tile_shape)):
+        co = _coeffs(start, rank)
+        nz = [i for i, c in enumerate(co) if c]
+        size = view.base.shape[d]
+        if not nz:
+            if start.const != 0:
+                raise NoNativeKernel(f"{view.base.name}: constant offset {start.const} along "
+                                     f"dim {d} (only whole-extent or tiled access is bound)")
+            extent.append(min(t, size))
+            driver.append(None)
+        elif len(nz) == 1 and start.const == 0 and co[nz[0]] == t and nz[0] not in used:
+            used.add(nz[0])
+            extent.append(min(n_groups[nz[0]] * t, size))
+            driver.append(nz[0])
+        else:
+            raise NoNativeKernel(
+                f"{view.base.name}: offset {start!r} along dim {d} with tile extent {t} is "
+                "not a disjoint tiling (need group_id * tile_extent)")
+    return Window(view.base.index, tuple(extent), tuple(driver), tuple(tile_shape))
+
+
+# ---------------------------------------------------------------------------
+# Tiny structural matcher
+# ---------------------------------------------------------------------------
+def _is(t: Tile, op: str, n: int | None = None) -> bool:
+    return isinstance(t, Tile) and t.op == op and (n is None or len(t.args) == n)
+
+
+def _const(t: Tile, value=None) -> bool:
+    if not (_is(t, "const") or _is(t, "full")):
+        return False
+    return value is None or t.attrs.get("value") == float(value)
+
+
+def _strip_cast(t: Tile, to: str) -> Tile:
+    return t.args[0] if _is(t, "astype", 1) and t.dtype_name == to else t
+
+
+def _f32(t: Tile):
+    """The load behind `x.astype(float32)` (or x itself if already fp32)."""
+    if _is(t, "astype", 1) and t.dtype_name == "float32" and _is(t.args[0], "load"):
+        return t.args[0]
+    if _is(t, "load") and t.dtype_name == "float32":
+        return t
+    return None
+
+
+def _same(a: Tile, b: Tile) -> bool:
+    """Structural equality of two expression trees (loads by identity of the
+    window they read)."""
+    if a is b:
+        return True
+    if a.op != b.op or a.shape != b.shape or a.dtype_name != b.dtype_name:
+        return False
+    if a.op == "load":
+        va, vb = a.attrs["view"], b.attrs["view"]
+        return va.base.index == vb.base.index and va.starts == vb.starts
+    if {k: v for k, v in a.attrs.items()} != {k: v for k, v in b.attrs.items()}:
+        return False
+    return len(a.args) == len(b.args) and all(_same(x, y) for x, y in zip(a.args, b.args))
+
+
+def _row_reduce(t: Tile, op: str):
+    """x if t == x.<op>(axis=1, keepdims=True) on a 2-D tile."""
+    if _is(t, op, 1) and t.attrs.get("axes") == (1,) and t.attrs.get("keepdims") \
+            and len(t.args[0].shape) == 2:
+        return t.args[0]
+    return None
+
+
+# ---------------------------------------------------------------------------
+# Patterns.  Each returns a function(memrefs, ctx) -> list[rt.Plan] or None.
+# ---------------------------------------------------------------------------
+def _check_same_window(wins):
+    w0 = wins[0]
+    for w in wins[1:]:
+        if w.extent != w0.extent or w.driver != w0.driver:
+            raise NoNativeKernel("loads and the store walk different windows")
+    return w0
+
+
+def _region2d(extent):
+    if len(extent) == 1:
+        return 1, extent[0]
+    if len(extent) == 2:
+        return extent
+    raise NoNativeKernel("only 1-D and 2-D buffers have native kernels")
+
+
+def _sub(m: rt.Memref, extent) -> rt.Memref:
+    return rt.Memref(m.ptr, tuple(extent), m.strides, m.itemsize)
+
+
+class _Arr:
+    """Memref wrapper accepted by the runtime's plan_* functions."""
+
+    def __init__(self, m: rt.Memref, ctx):
+        self.shape, self.ctx = m.shape, ctx
+        code = {1: "|u1", 2: "<u2", 4: "<u4", 8: "<u8", 16: "|V16"}[m.itemsize]
+        self.__cuda_array_interface__ = {
+            "shape": m.shape, "typestr": code, "data": (m.ptr, False),
+            "strides": tuple(s * m.itemsize for s in m.strides), "version": 2}
+
+
+def match_copy(dst_view, value, n_groups):
+    if not _is(value, "load"):
+        return None
+    src = value.attrs["view"]
+    if src.base.dtype_name != dst_view.base.dtype_name:
+        return None
+    ws = window_of(src, value.shape, n_groups)
+    wd = window_of(dst_view, value.shape, n_groups)
+    if ws.driver != wd.driver:
+        raise NoNativeKernel("load and store walk different windows")
+    extent = tuple(min(a, b) for a, b in zip(ws.extent, wd.extent))
+    if len(extent) > 2:
+        raise NoNativeKernel("only 1-D and 2-D copies have a native kernel")
+
+    def make(mem, ctx):
+        return [rt.plan_copy2d(_Arr(_sub(mem[ws.buffer], extent), ctx),
+                               _Arr(_sub(mem[wd.buffer], extent), ctx))]
+    return make
+
+
+def match_add(dst_view, value, n_groups):
+    value = _strip_cast(value, dst_view.base.dtype_name)
+    if not (_is(value, "add", 2) and all(_is(a, "load") for a in value.args)):
+        return None
+    if {a.dtype_name for a in value.args} | {dst_view.base.dtype_name} != {"float32"}:
+        return None
+    wins = [window_of(a.attrs["view"], a.shape, n_groups) for a in value.args]
+    wins.append(window_of(dst_view, value.shape, n_groups))
+    w = _check_same_window(wins)
+
+    def make(mem, ctx):
+        ms = [mem[x.buffer] for x in wins]
+        if all(m.shape == w.extent and m.is_contiguous() for m in ms):
+            return [rt.plan_add_f32(*[_Arr(m, ctx) for m in ms])]
+        raise NoNativeKernel("c = a + b is bound for whole contiguous arrays only")
+    return make
+
+
+def match_fma(dst_view, value, n_groups):
+    if dst_view.base.dtype_name != "float16":
+        return None
+    value = _strip_cast(value, "float16")
+    if not (_is(value, "add", 2) and value.dtype_name == "float32"):
+        return None
+    for prod, addend in (value.args, value.args[::-1]):
+        c = _f32(addend)
+        if c is None or not _is(prod, "mul", 2):
+            continue
+        a, b = _f32(prod.args[0]), _f32(prod.args[1])
+        if a is None or b is None:
+            continue
+        if {a.dtype_name, b.dtype_name, c.dtype_name} != {"float16"}:
+            return None
+        wins = [window_of(t.attrs["view"], t.shape, n_groups) for t in (a, b, c)]
+        wins.append(window_of(dst_view, value.shape, n_groups))
+        w = _check_same_window(wins)
+        if len(w.extent) > 2:
+            raise NoNativeKernel("only 1-D and 2-D buffers have native kernels")
+
+        def make(mem, ctx):
+            return [rt.plan_fma_f16(*[_Arr(_sub(mem[x.buffer], w.extent), ctx) for x in wins])]
+        return make
+    return None
+
+
+def match_softmax(dst_view, value, n_groups):
+    if dst_view.base.dtype_name != "float32" or not _is(value, "div", 2):
+        return None
+    e, s = value.args
+    if _row_reduce(s, "sum") is None or not _same(_row_reduce(s, "sum"), e):
+        return None
+    if not (_is(e, "exp", 1) and _is(e.args[0], "sub", 2)):
+        return None
+    x, m = e.args[0].args
+    if not (_is(x, "load") and x.dtype_name == "float32" and _row_reduce(m, "max") is x):
+        return None
+    wx = window_of(x.attrs["view"], x.shape, n_groups)
+    wy = window_of(dst_view, value.shape, n_groups)
+    w = _check_same_window([wx, wy])
+    if len(w.extent) != 2 or w.driver[1] is not None or w.extent[1] != x.attrs["view"].base.shape[1]:
+        raise NoNativeKernel("row softmax needs tiles that hold whole rows")
+
+    def make(mem, ctx):
+        return [rt.plan_softmax_f32(_Arr(_sub(mem[wx.buffer], w.extent), ctx),
+                                    _Arr(_sub(mem[wy.buffer], w.extent), ctx))]
+    return make
+
+
+def _quant_parts(value):
+    """(x load, scale tile) if value == int8(clip(rint(f32 x / scale), -127, 127))."""
+    v = _strip_cast(value, "int8")
+    if not (_is(v, "clip", 1) and v.attrs["lo"] == -127.0 and v.attrs["hi"] == 127.0):
+        return None
+    r = v.args[0]
+    if not (_is(r, "rint", 1) and _is(r.args[0], "div", 2)):
+        return None
+    xf, scale = r.args[0].args
+    x = _f32(xf)
+    if x is None or x.dtype_name != "float16":
+        return None
+    if not (_is(scale, "div", 2) and _const(scale.args[1], 127) and scale.dtype_name == "float32"):
+        return None
+    amax = _row_reduce(scale.args[0], "max")
+    if amax is None or not (_is(amax, "abs", 1) and _f32(amax.args[0]) is x):
+        return None
+    return x, scale
+
+
+def match_quantize(stores, n_groups):
+    """Two stores: the int8 matrix and the per-row scale vector."""
+    if len(stores) != 2:
+        return None
+    for (qv, qval), (sv, sval) in (stores, stores[::-1]):
+        if qv.base.dtype_name != "int8" or sv.base.dtype_name != "float32":
+            continue
+        parts = _quant_parts(qval)
+        if parts is None:
+            continue
+        x, scale = parts
+        # the scale may be stored as (rows, 1), or flattened to (rows,)
+        s = sval
+        while _is(s, "slice", 1) or _is(s, "reshape", 1):
+            s = s.args[0]
+        if not _same(s, scale):
+            continue
+        wx = window_of(x.attrs["view"], x.shape, n_groups)
+        wq = window_of(qv, qval.shape, n_groups)
+        w = _check_same_window([wx, wq])
+        if len(w.extent) != 2 or w.driver[1] is not None or \
+                w.extent[1] != x.attrs["view"].base.shape[1]:
+            raise NoNativeKernel("row quantisation needs tiles that hold whole rows")
+        ws = window_of(sv, (x.shape[0],) + (1,) * (sv.base.ndim - 1), n_groups)
+        if ws.extent[0] != w.extent[0] or ws.driver[0] != w.driver[0]:
+            raise NoNativeKernel("scale vector and matrix walk different rows")
+
+        def make(mem, ctx, wx=wx, wq=wq, ws=ws, w=w):
+            sm = mem[ws.buffer]
+            scale_arr = rt.Memref(sm.ptr, (w.extent[0],), (sm.strides[0],), sm.itemsize)
+            return [rt.plan_quantize_f16_i8(_Arr(_sub(mem[wx.buffer], w.extent), ctx),
+                                            _Arr(_sub(mem[wq.buffer], w.extent), ctx),
+                                            _Arr(scale_arr, ctx))]
+        return make
+    return None
+
+
+def _flatten_sum(t: Tile, out: list):
+    if _is(t, "add", 2):
+        _flatten_sum(t.args[0], out)
+        _flatten_sum(t.args[1], out)
+    else:
+        out.append(t)
+
+
+def match_gemm(dst_view, value, n_groups):
+    if dst_view.base.dtype_name != "bfloat16":
+        return None
+    value = _strip_cast(value, "bfloat16")
+    terms: list = []
+    _flatten_sum(value, terms)
+    dots = [t for t in terms if not _const(t, 0)]
+    if not dots or not all(_is(d, "dot", 2) or
+                           (_is(d, "astype", 1) and _is(d.args[0], "dot", 2)) for d in dots):
+        return None
+    chunks, wa0, wb0, a_idx, b_idx = [], None, None, None, None
+    for d in dots:
+        d = d.args[0] if d.op == "astype" else d
+        la, lbt = d.args
+        if not (_is(la, "load") and _is(lbt, "transpose", 1) and _is(lbt.args[0], "load")):
+            raise NoNativeKernel("GEMM is bound for dot(load A[m, k], load Bt[n, k].T): B must "
+                                 "be column-major, passed as Bt[N, K]")
+        lb = lbt.args[0]
+        if la.dtype_name != "bfloat16" or lb.dtype_name != "bfloat16":
+            return None
+        va, vb = la.attrs["view"], lb.attrs["view"]
+        ka, kb = va.starts[1], vb.starts[1]
+        if not (ka.is_const and kb.is_const and ka.const == kb.const and
+                la.shape[1] == lb.shape[1]):
+            raise NoNativeKernel("A and Bt tiles of one dot must cover the same K range")
+        chunks.append((ka.const, la.shape[1]))
+        # windows along M and N: evaluate with the K offset removed
+        va0 = BufferView(va.base, (va.starts[0], Affine(0, ka.coeffs)))
+        vb0 = BufferView(vb.base, (vb.starts[0], Affine(0, kb.coeffs)))
+        wa = window_of(va0, (la.shape[0], va.base.shape[1]), n_groups)
+        wb = window_of(vb0, (lb.shape[0], vb.base.shape[1]), n_groups)
+        if wa0 is None:
+            wa0, wb0, a_idx, b_idx = wa, wb, va.base.index, vb.base.index
+        elif (wa.extent, wa.driver, wb.extent, wb.driver, va.base.index, vb.base.index) != \
+                (wa0.extent, wa0.driver, wb0.extent, wb0.driver, a_idx, b_idx):
+            raise NoNativeKernel("dot terms walk different A / Bt windows")
+    k_total = wa0.extent[1]
+    if wb0.extent[1] != k_total:
+        raise NoNativeKernel("A and Bt have different K extents")
+    chunks.sort()
+    pos = 0
+    for start, length in chunks:
+        if start != pos:
+            raise NoNativeKernel("K chunks of the dot terms are not contiguous")
+        pos += length
+    if pos < k_total:
+        raise NoNativeKernel("the dot terms do not cover all of K")
+    wc = window_of(dst_view, value.shape, n_groups)
+    if wc.driver != (wa0.driver[0], wb0.driver[0]) or wc.driver[0] == wc.driver[1]:
+        raise NoNativeKernel("C tiles must be walked by the A-row and Bt-row group dims")
+    m, n = min(wc.extent[0], wa0.extent[0]), min(wc.extent[1], wb0.extent[0])
+
+    def make(mem, ctx):
+        return [rt.plan_gemm_bf16(_Arr(_sub(mem[a_idx], (m, k_total)), ctx),
+                                  _Arr(_sub(mem[b_idx], (n, k_total)), ctx),
+                                  _Arr(_sub(mem[wc.buffer], (m, n)), ctx))]
+    return make
+
+
+def bind(stores, n_groups):
+    """stores: list of (BufferView, Tile) from one traced execution.  Returns a
+    list of plan makers; raises NoNativeKernel when nothing matches."""
+    if not stores:
+        raise NoNativeKernel("the kernel body stores nothing")
+    try:
+        q = match_quantize(stores, n_groups)
+        if q is not None:
+            return [q]
+        makers = []
+        for view, value in stores:
+            for matcher in (match_copy, match_add, match_fma, match_softmax, match_gemm):
+                mk = matcher(view, value, n_groups)
+                if mk is not None:
+                    makers.append(mk)
+                    break
+            else:
+                raise NoNativeKernel(
+                    f"no hand-written kernel matches the value stored to {view.base.name} "
+                    f"({value!r}); bound patterns: copy, a+b (fp32), a*b+c (fp16 storage, fp32 "
+                    "math), row softmax (fp32), row absmax int8 quantisation, bf16 GEMM")
+        return makers
+    except TraceError as exc:
+        raise NoNativeKernel(str(exc)) from exc

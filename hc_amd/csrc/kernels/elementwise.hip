@@ -35,9 +35,15 @@ struct FmaF16 {
   static __device__ __forceinline__ Elem apply1(const Elem *in) {
     // fp16 x fp16 is exact in fp32 (11+11 significand bits), so the rounding
     // of the separate multiply never happens and mul+add equals a fused
-    // multiply-add; the only roundings are the fp32 add and the final
-    // fp32->fp16 conversion (nearest even).
-    return (_Float16)((float)in[0] * (float)in[1] + (float)in[2]);
+    // multiply-add.  Two roundings remain and both are required: the fp32 sum
+    // (nearest even) and then the fp32->fp16 conversion (nearest even).  The
+    // one-instruction form v_fma_mixlo_f16 rounds the exact sum straight to
+    // fp16 and differs from that in about one element in 70,000 (an fp32
+    // result that lands on an fp16 tie), so the fp32 value is pinned in a
+    // register before it is converted.
+    float r = __builtin_fmaf((float)in[0], (float)in[1], (float)in[2]);
+    asm volatile("" : "+v"(r));
+    return (_Float16)r;
   }
   static __device__ __forceinline__ Vec apply(const Vec *in) {
     Vec r;

@@ -705,7 +705,7 @@ int hcamdLaunchCopy2D(OlQueue q, size_t elemSize, const void *src,
   const int variant = variantOf("copy");
   if (dense && aligned16(src) && aligned16(dst) && variant != 9) {
     static const char *const names[] = {
-        "hcamd_copy_flat_v4",    "hcamd_copy_flat_v1",    "hcamd_copy_flat_v2",
+        "hcamd_copy_flat_v4_nt", "hcamd_copy_flat_v1",    "hcamd_copy_flat_v2",
         "hcamd_copy_flat_v4",    "hcamd_copy_flat_v8",    "hcamd_copy_flat_v1_nt",
         "hcamd_copy_flat_v2_nt", "hcamd_copy_flat_v4_nt", "hcamd_copy_flat_v8_nt"};
     static const int vpt[] = {4, 1, 2, 4, 8, 1, 2, 4, 8};
@@ -793,7 +793,7 @@ int hcamdLaunchAddF32(OlQueue q, const float *a, const float *b, float *c,
     return launch1d(queue, "elementwise", "hcamd_add_f32_scalar",
                     ceilDiv(n, 256), 256, args);
   static const char *const names[] = {
-      "hcamd_add_f32_v4",    "hcamd_add_f32_v1",    "hcamd_add_f32_v2",
+      "hcamd_add_f32_v4_nt", "hcamd_add_f32_v1",    "hcamd_add_f32_v2",
       "hcamd_add_f32_v4",    "hcamd_add_f32_v8",    "hcamd_add_f32_v1_nt",
       "hcamd_add_f32_v2_nt", "hcamd_add_f32_v4_nt", "hcamd_add_f32_v8_nt"};
   static const int vpt[] = {4, 1, 2, 4, 8, 1, 2, 4, 8};
@@ -826,10 +826,10 @@ int hcamdLaunchFmaF16(OlQueue q, const void *a, size_t lda, const void *b,
   if (dense && aligned16(a) && aligned16(b) && aligned16(c) && aligned16(d) &&
       variant != 7) {
     static const char *const names[] = {
-        "hcamd_fma_f16_v2",    "hcamd_fma_f16_v1",    "hcamd_fma_f16_v2",
+        "hcamd_fma_f16_v4_nt", "hcamd_fma_f16_v1",    "hcamd_fma_f16_v2",
         "hcamd_fma_f16_v4",    "hcamd_fma_f16_v1_nt", "hcamd_fma_f16_v2_nt",
         "hcamd_fma_f16_v4_nt"};
-    static const int vpt[] = {2, 1, 2, 4, 1, 2, 4};
+    static const int vpt[] = {4, 1, 2, 4, 1, 2, 4};
     const int v = (variant >= 0 && variant <= 6) ? variant : 0;
     size_t n = rows * cols;
     const size_t words = ceilDiv(n, 8);
@@ -897,8 +897,8 @@ int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,
                                           : "hcamd_softmax_f32_g256_v4";
   } else if (cols <= 8192) {
     name = (cols == 8192 && variant != 2)
-               ? (variant == 3 ? "hcamd_softmax_f32_g256_v8_full_nt"
-                               : "hcamd_softmax_f32_g256_v8_full")
+               ? (variant == 3 ? "hcamd_softmax_f32_g256_v8_full"
+                               : "hcamd_softmax_f32_g256_v8_full_nt")
                : "hcamd_softmax_f32_g256_v8";
   } else {
     name = "hcamd_softmax_f32_g256_v16";
@@ -950,11 +950,11 @@ int hcamdLaunchQuantizeF16I8(OlQueue q, const void *x, size_t ldx, int8_t *qout,
   } else if (cols <= 4096) {
     switch (variant) {
     case 2: name = "hcamd_quant_f16_i8_w64_v4"; per_wave = true; break;
-    case 3: name = "hcamd_quant_f16_i8_g256_v1_nt"; break;
+    case 3: name = "hcamd_quant_f16_i8_g256_v1"; break;
     case 4: name = "hcamd_quant_f16_i8_w64_v4_nt"; per_wave = true; break;
     case 5: name = "hcamd_quant_f16_i8_g256_v1_div"; break;
     case 6: name = "hcamd_quant_f16_i8_w64_v4_div"; per_wave = true; break;
-    default: name = "hcamd_quant_f16_i8_g256_v1"; break;
+    default: name = "hcamd_quant_f16_i8_g256_v1_nt"; break;
     }
   } else if (cols <= 8192) {
     name = "hcamd_quant_f16_i8_g256_v2";

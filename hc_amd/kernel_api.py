@@ -1,0 +1,555 @@
+"""The kernel programming model: group object, buffers, tiles.
+
+Host-side mirror of the reference's python/hckernel/kernel_api.py (the names a
+kernel body is written against: CurrentGroup.load/store/vload, allocators,
+work_offset, shape, Buffer, TunableParam, atomic_ref, create_mapping).  The
+reference compiles the body's source text; here the body is *run once* with a
+tracing group.  Group ids are symbolic, buffers are proxies, and tiles record
+the operations applied to them, so that one execution yields the whole
+per-group program: which windows are loaded, what is computed, what is stored.
+hc_amd.binding then matches that program against the hand-written gfx950
+kernels.  Nothing in this module computes array values.
+"""
+
+from __future__ import annotations
+
+import math
+from collections.abc import Iterable
+
+import numpy as np
+
+
+class TraceError(RuntimeError):
+    """The kernel body did something the tracer cannot express."""
+
+
+# ---------------------------------------------------------------------------
+# Small public types (kernel_api.py:35-40, 214-220, 231-252, 437-451)
+# ---------------------------------------------------------------------------
+class TunableParam:
+    def __init__(self, sym, default, vals, strategy=None):
+        self.sym, self.default, self.vals, self.strategy = sym, default, vals, strategy
+
+
+class Mapping:
+    def __init__(self, func):
+        self.func = func
+
+
+def create_mapping(func):
+    return Mapping(func)
+
+
+def atomic_ref(a):
+    return a
+
+
+class Buffer(type):
+    """`Buffer[d0, ..., dtype]`: annotation for an array argument; symbolic
+    dims are bound to the argument's shape at call time."""
+
+    def __class_getitem__(cls, spec):
+        assert len(spec) > 0, "Invalid shape and dtype"
+        return type("Buffer", (cls,), {"shape": tuple(spec[:-1]), "dtype": spec[-1]})
+
+
+class CurrentSubGroup:
+    def __init__(self, size, subgroup_id):
+        self._size, self._id = size, subgroup_id
+
+    def size(self):
+        return self._size
+
+    def subgroup_id(self):
+        return self._id
+
+
+class CurrentWorkitem:
+    def __init__(self, local_id, global_id):
+        self._lid, self._gid = local_id, global_id
+
+    def local_id(self):
+        return self._lid
+
+    def global_id(self):
+        return self._gid
+
+
+# ---------------------------------------------------------------------------
+# Affine index expressions in the group id
+# ---------------------------------------------------------------------------
+class Affine:
+    """const + sum(coeffs[i] * group_id[i]).  The only index arithmetic a tiled
+    kernel needs: offsets are group id times tile size plus constants."""
+
+    __slots__ = ("const", "coeffs")
+
+    def __init__(self, const, coeffs):
+        self.const, self.coeffs = int(const), tuple(int(c) for c in coeffs)
+
+    @staticmethod
+    def lift(v, rank):
+        if isinstance(v, Affine):
+            return v
+        try:
+            return Affine(int(v), (0,) * rank)
+        except (TypeError, ValueError):
+            raise TraceError(f"unsupported index value {v!r}") from None
+
+    @property
+    def is_const(self):
+        return not any(self.coeffs)
+
+    def __add__(self, o):
+        o = Affine.lift(o, len(self.coeffs))
+        return Affine(self.const + o.const, [a + b for a, b in zip(self.coeffs, o.coeffs)])
+
+    __radd__ = __add__
+
+    def __neg__(self):
+        return Affine(-self.const, [-c for c in self.coeffs])
+
+    def __sub__(self, o):
+        return self + (-Affine.lift(o, len(self.coeffs)))
+
+    def __rsub__(self, o):
+        return Affine.lift(o, len(self.coeffs)) - self
+
+    def __mul__(self, o):
+        if isinstance(o, Affine):
+            if o.is_const:
+                o = o.const
+            elif self.is_const:
+                return o * self.const
+            else:
+                raise TraceError("product of two group-id dependent indices")
+        try:
+            k = int(o)
+        except (TypeError, ValueError):
+            raise TraceError(f"unsupported index factor {o!r}") from None
+        return Affine(self.const * k, [c * k for c in self.coeffs])
+
+    __rmul__ = __mul__
+
+    def __index__(self):
+        if self.is_const:
+            return self.const
+        raise TraceError("a group-id dependent index was used where a number is needed "
+                         "(only offsets of loads and stores may depend on the group id)")
+
+    __int__ = __index__
+
+    def _unsupported(self, *_):
+        raise TraceError("only +, - and * by a constant are supported on group offsets")
+
+    __floordiv__ = __mod__ = __truediv__ = __lt__ = __le__ = __gt__ = __ge__ = _unsupported
+
+    def __eq__(self, o):
+        o = Affine.lift(o, len(self.coeffs)) if not isinstance(o, Affine) else o
+        return self.const == o.const and self.coeffs == o.coeffs
+
+    def __hash__(self):
+        return hash((self.const, self.coeffs))
+
+    def __repr__(self):
+        terms = [f"{c}*g{i}" for i, c in enumerate(self.coeffs) if c]
+        return " + ".join(terms + ([str(self.const)] if self.const or not terms else []))
+
+
+# ---------------------------------------------------------------------------
+# dtypes
+# ---------------------------------------------------------------------------
+def dtype_name(dt) -> str:
+    """Canonical name ('float32', 'float16', 'bfloat16', 'int8', ...) of a
+    NumPy dtype, a torch dtype, a type like np.float32, or a string."""
+    if isinstance(dt, str):
+        return dt.replace("torch.", "")
+    name = getattr(dt, "__name__", None)            # np.float32, float, int
+    if name in ("float", "int", "bool"):
+        return {"float": "float64", "int": "int64", "bool": "bool"}[name]
+    s = str(dt)
+    if s.startswith("torch."):
+        return s[6:]
+    try:
+        return np.dtype(dt).name
+    except TypeError:
+        raise TraceError(f"unknown dtype {dt!r}") from None
+
+
+_RANK = {"bool": 0, "int8": 1, "uint8": 1, "int16": 2, "uint16": 2, "int32": 3, "uint32": 3,
+         "int64": 4, "uint64": 4, "float16": 5, "bfloat16": 5, "float32": 6, "float64": 7}
+
+
+def promote(a: str, b: str) -> str:
+    """Result type of a binary operation between tiles (NumPy's rules for the
+    types the kernels use; mixing float16 with bfloat16 gives float32)."""
+    if a == b:
+        return a
+    if {a, b} == {"float16", "bfloat16"}:
+        return "float32"
+    fa, fb = _RANK[a] >= 5, _RANK[b] >= 5
+    if fa != fb:                       # int with float: the float wins if wide enough
+        f, i = (a, b) if fa else (b, a)
+        if _RANK[f] == 5 and _RANK[i] >= 2:
+            return "float32" if _RANK[i] == 2 else "float64"
+        return f
+    return a if _RANK[a] >= _RANK[b] else b
+
+
+# ---------------------------------------------------------------------------
+# Buffers and views
+# ---------------------------------------------------------------------------
+class BufferProxy:
+    """Stands for an array argument while the body is traced."""
+
+    def __init__(self, index, name, shape, strides, dtype, obj):
+        self.index, self.name = index, name
+        self.shape, self.strides = tuple(shape), tuple(strides)
+        self.dtype_name = dtype
+        self.obj = obj
+
+    @property
+    def dtype(self):
+        try:
+            return np.dtype(self.dtype_name)
+        except TypeError:
+            return self.dtype_name
+
+    @property
+    def ndim(self):
+        return len(self.shape)
+
+    def __getitem__(self, key):
+        if not isinstance(key, tuple):
+            key = (key,)
+        if len(key) > self.ndim:
+            raise TraceError(f"too many indices for {self.name}")
+        starts = []
+        for k in key:
+            if not isinstance(k, slice):
+                raise TraceError("buffers are indexed with slices `a[x:, y:]` inside a kernel")
+            if k.step not in (None, 1) or k.stop is not None:
+                raise TraceError("only `start:` slices are supported on buffers")
+            starts.append(0 if k.start is None else k.start)
+        starts += [0] * (self.ndim - len(starts))
+        rank = max((len(s.coeffs) for s in starts if isinstance(s, Affine)), default=0)
+        return BufferView(self, tuple(Affine.lift(s, rank) for s in starts))
+
+    def __setitem__(self, key, value):
+        raise TraceError("direct assignment to a buffer is not supported on the GPU path; "
+                         "use group.store")
+
+    def __repr__(self):
+        return f"<buffer {self.name} {self.shape} {self.dtype_name}>"
+
+
+class BufferView:
+    """`buffer[x:, y:]`: a window that starts at an (affine) offset."""
+
+    def __init__(self, base: BufferProxy, starts):
+        self.base, self.starts = base, starts
+
+    @property
+    def dtype(self):
+        return self.base.dtype
+
+    @property
+    def shape(self):
+        out = []
+        for n, s in zip(self.base.shape, self.starts):
+            if not s.is_const:
+                raise TraceError("the shape of a window that depends on the group id is "
+                                 "not a number")
+            out.append(max(n - s.const, 0))
+        return tuple(out)
+
+
+def _as_view(x) -> BufferView:
+    if isinstance(x, BufferView):
+        return x
+    if isinstance(x, BufferProxy):
+        return x[tuple(slice(None) for _ in x.shape)]
+    raise TraceError(f"expected a buffer window, got {type(x).__name__}")
+
+
+# ---------------------------------------------------------------------------
+# Tiles: nodes of the traced expression DAG
+# ---------------------------------------------------------------------------
+_UFUNC_OPS = {"add": "add", "subtract": "sub", "multiply": "mul", "true_divide": "div",
+              "divide": "div", "exp": "exp", "absolute": "abs", "fabs": "abs", "rint": "rint",
+              "negative": "neg", "maximum": "maximum", "minimum": "minimum", "sqrt": "sqrt"}
+
+
+def _result_dtype(a: "Tile", b: "Tile") -> str:
+    """Python scalars are weak (they adopt the tile's type unless that is an
+    integer type and the scalar a float); NumPy scalars and tiles promote."""
+    aw, bw = bool(a.attrs.get("weak")), bool(b.attrs.get("weak"))
+    if aw and not bw:
+        a, b, bw = b, a, True
+    elif aw and bw:
+        return promote(a.dtype_name, b.dtype_name)
+    if bw:
+        if _RANK[a.dtype_name] >= 5 or b.dtype_name != "float64":
+            return a.dtype_name
+        return "float64"
+    return promote(a.dtype_name, b.dtype_name)
+
+
+def _broadcast(a, b):
+    try:
+        return tuple(np.broadcast_shapes(tuple(a), tuple(b)))
+    except ValueError:
+        raise TraceError(f"shapes {a} and {b} do not broadcast") from None
+
+
+class Tile:
+    """A value in the per-group program.  `op` is 'load', 'const', an
+    elementwise operation, a reduction, 'astype', 'dot', 'transpose', 'clip' or
+    'slice'; `args` are Tiles; `attrs` holds the rest."""
+
+    __array_priority__ = 1000
+    _counter = 0
+
+    def __init__(self, op, args=(), shape=(), dtype="float32", **attrs):
+        self.op, self.args, self.shape = op, tuple(args), tuple(int(s) for s in shape)
+        self.dtype_name, self.attrs = dtype, attrs
+        Tile._counter += 1
+        self.uid = Tile._counter
+
+    # -- construction helpers ----------------------------------------------------
+    @staticmethod
+    def wrap(x, like: "Tile | None" = None) -> "Tile":
+        if isinstance(x, Tile):
+            return x
+        if isinstance(x, (bool, int, float, np.generic)):
+            if isinstance(x, np.generic):
+                dt, weak = x.dtype.name, False
+            else:
+                dt, weak = ("float64" if isinstance(x, float) else "int64"), True
+            return Tile("const", (), (), dt, value=float(x), weak=weak)
+        raise TraceError(f"cannot use {type(x).__name__} in a tile expression")
+
+    def _binary(self, other, op, reflected=False):
+        o = Tile.wrap(other)
+        a, b = (o, self) if reflected else (self, o)
+        return Tile(op, (a, b), _broadcast(a.shape, b.shape), _result_dtype(a, b))
+
+    def __add__(self, o): return self._binary(o, "add")
+    def __radd__(self, o): return self._binary(o, "add", True)
+    def __sub__(self, o): return self._binary(o, "sub")
+    def __rsub__(self, o): return self._binary(o, "sub", True)
+    def __mul__(self, o): return self._binary(o, "mul")
+    def __rmul__(self, o): return self._binary(o, "mul", True)
+    def __truediv__(self, o): return self._binary(o, "div")
+    def __rtruediv__(self, o): return self._binary(o, "div", True)
+    def __neg__(self): return Tile("neg", (self,), self.shape, self.dtype_name)
+    def __abs__(self): return Tile("abs", (self,), self.shape, self.dtype_name)
+
+    def __matmul__(self, o):
+        return _dot(self, Tile.wrap(o))
+
+    # -- NumPy protocol -----------------------------------------------------------
+    def __array_ufunc__(self, ufunc, method, *inputs, **kwargs):
+        op = _UFUNC_OPS.get(ufunc.__name__)
+        if method != "__call__" or op is None or kwargs:
+            raise TraceError(f"numpy.{ufunc.__name__} ({method}) is not supported in a GPU kernel")
+        if len(inputs) == 1:
+            x = Tile.wrap(inputs[0])
+            return Tile(op, (x,), x.shape, x.dtype_name)
+        a, b = inputs
+        if isinstance(a, Tile):
+            return a._binary(b, op)
+        return Tile.wrap(b)._binary(a, op, reflected=True)
+
+    def __array_function__(self, func, types, args, kwargs):
+        name = func.__name__
+        if name == "dot" and len(args) == 2:
+            return _dot(Tile.wrap(args[0]), Tile.wrap(args[1]))
+        if name == "clip":
+            x = Tile.wrap(args[0])
+            lo = kwargs.get("a_min", args[1] if len(args) > 1 else None)
+            hi = kwargs.get("a_max", args[2] if len(args) > 2 else None)
+            return Tile("clip", (x,), x.shape, x.dtype_name, lo=float(lo), hi=float(hi))
+        if name in ("amax", "max", "sum", "amin", "min"):
+            x = Tile.wrap(args[0])
+            return x._reduce({"amax": "max", "amin": "min"}.get(name, name),
+                             kwargs.get("axis", args[1] if len(args) > 1 else None),
+                             kwargs.get("keepdims", False))
+        if name == "transpose" and len(args) == 1:
+            return Tile.wrap(args[0]).T
+        raise TraceError(f"numpy.{name} is not supported in a GPU kernel")
+
+    # -- methods kernels use ---------------------------------------------------------
+    def _reduce(self, op, axis, keepdims):
+        if axis is None:
+            axes = tuple(range(len(self.shape)))
+        else:
+            axes = (axis,) if isinstance(axis, int) else tuple(axis)
+        axes = tuple(a % len(self.shape) for a in axes)
+        shape = tuple((1 if i in axes else n) for i, n in enumerate(self.shape)) if keepdims \
+            else tuple(n for i, n in enumerate(self.shape) if i not in axes)
+        return Tile(op, (self,), shape, self.dtype_name, axes=axes, keepdims=bool(keepdims))
+
+    def max(self, axis=None, keepdims=False): return self._reduce("max", axis, keepdims)
+    def min(self, axis=None, keepdims=False): return self._reduce("min", axis, keepdims)
+    def sum(self, axis=None, keepdims=False): return self._reduce("sum", axis, keepdims)
+
+    def astype(self, dt):
+        name = dtype_name(dt)
+        if name == self.dtype_name:
+            return self
+        return Tile("astype", (self,), self.shape, name)
+
+    @property
+    def T(self):
+        if len(self.shape) != 2:
+            raise TraceError(".T needs a 2-D tile")
+        return Tile("transpose", (self,), self.shape[::-1], self.dtype_name)
+
+    @property
+    def dtype(self):
+        try:
+            return np.dtype(self.dtype_name)
+        except TypeError:
+            return self.dtype_name
+
+    @property
+    def ndim(self):
+        return len(self.shape)
+
+    def __getitem__(self, key):
+        if not isinstance(key, tuple):
+            key = (key,)
+        key = key + (slice(None),) * (len(self.shape) - len(key))
+        shape = []
+        for k, n in zip(key, self.shape):
+            if isinstance(k, slice):
+                shape.append(len(range(*k.indices(n))))
+            else:
+                int(k)
+        norm = tuple((k.start, k.stop, k.step) if isinstance(k, slice) else int(k) for k in key)
+        return Tile("slice", (self,), shape, self.dtype_name, key=norm)
+
+    def reshape(self, *shape):
+        shape = shape[0] if len(shape) == 1 and isinstance(shape[0], Iterable) else shape
+        shape = tuple(int(s) for s in shape)
+        if -1 in shape:
+            known = -math.prod(shape)
+            shape = tuple(math.prod(self.shape) // known if s == -1 else s for s in shape)
+        if math.prod(shape) != math.prod(self.shape):
+            raise TraceError("reshape changes the number of elements")
+        return Tile("reshape", (self,), shape, self.dtype_name)
+
+    def __bool__(self):
+        raise TraceError("the value of a tile is not known while the kernel is traced; "
+                         "data-dependent control flow is not supported")
+
+    def __iter__(self):
+        raise TraceError("tiles cannot be iterated in a GPU kernel")
+
+    def __repr__(self):
+        return f"<tile {self.op} {self.shape} {self.dtype_name}>"
+
+
+def _dot(a: Tile, b: Tile) -> Tile:
+    if len(a.shape) != 2 or len(b.shape) != 2 or a.shape[1] != b.shape[0]:
+        raise TraceError(f"dot of shapes {a.shape} and {b.shape}")
+    return Tile("dot", (a, b), (a.shape[0], b.shape[1]), promote(a.dtype_name, b.dtype_name))
+
+
+# ---------------------------------------------------------------------------
+# The group object handed to the kernel body
+# ---------------------------------------------------------------------------
+class CurrentGroup:
+    """Tracing group (python/hckernel/kernel_api.py:255-434).  `id` and
+    `work_offset` are symbolic; `shape` and `size` are numbers."""
+
+    def __init__(self, group_shape, subgroup_size):
+        self._shape = tuple(int(s) for s in group_shape)
+        self._subgroup_size = subgroup_size
+        rank = len(self._shape)
+        self._id = tuple(Affine(0, [1 if j == i else 0 for j in range(rank)])
+                         for i in range(rank))
+        self.stores = []          # (BufferView, Tile) in program order
+
+    @property
+    def id(self):
+        return self._id
+
+    @property
+    def shape(self):
+        return self._shape
+
+    @property
+    def size(self):
+        return math.prod(self._shape)
+
+    @property
+    def work_offset(self):
+        return tuple(g * s for g, s in zip(self._id, self._shape))
+
+    # -- loads and stores ----------------------------------------------------------
+    def load(self, array, shape, mapping=None):
+        if mapping is not None:
+            raise TraceError("mapped (gathered) loads have no native kernel yet")
+        if not isinstance(shape, Iterable):
+            shape = (shape,)
+        shape = tuple(int(s) for s in shape)
+        if isinstance(array, Tile):
+            raise TraceError("loading from a tile (vload of a register tile) has no native "
+                             "kernel yet")
+        view = _as_view(array)
+        if len(shape) != view.base.ndim:
+            raise TraceError(f"load shape {shape} does not match the rank of {view.base.name}")
+        return Tile("load", (), shape, view.base.dtype_name, view=view)
+
+    def vload(self, array, shape, mapping=None):
+        return self.load(array, shape, mapping)
+
+    def store(self, dst, src, mapping=None):
+        if mapping is not None:
+            raise TraceError("mapped (scattered) stores have no native kernel yet")
+        self.stores.append((_as_view(dst), Tile.wrap(src)))
+
+    # -- allocators ------------------------------------------------------------------
+    def _alloc(self, shape, dtype, value):
+        if not isinstance(shape, Iterable):
+            shape = (shape,)
+        t = Tile("const", (), (), dtype_name(dtype), value=float(value), weak=False)
+        return Tile("full", (t,), shape, dtype_name(dtype), value=float(value))
+
+    def empty(self, shape, dtype): return self._alloc(shape, dtype, 0)
+    def zeros(self, shape, dtype): return self._alloc(shape, dtype, 0)
+    def ones(self, shape, dtype): return self._alloc(shape, dtype, 1)
+    def full(self, shape, dtype, fill_value): return self._alloc(shape, dtype, fill_value)
+    vempty, vzeros, vones, vfull = empty, zeros, ones, full
+
+    def vec(self, src, shape=None):
+        src = Tile.wrap(src)
+        if shape is None or tuple(shape) == src.shape:
+            return src
+        return src[tuple(slice(0, s) for s in shape)]
+
+    # -- nested scopes -----------------------------------------------------------------
+    def subgroups(self, func):
+        raise TraceError("explicit subgroup scopes have no native kernel: the hand-written "
+                         "kernels choose their own wave-level decomposition")
+
+    def workitems(self, func):
+        raise TraceError("explicit work-item scopes have no native kernel: the hand-written "
+                         "kernels choose their own per-lane decomposition")
+
+    def barrier(self):
+        return None
+
+
+class CurrentGroup1(CurrentGroup):
+    pass
+
+
+class CurrentGroup2(CurrentGroup):
+    pass
+
+
+class CurrentGroup3(CurrentGroup):
+    pass

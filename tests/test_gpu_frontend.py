@@ -1,0 +1,215 @@
+"""Kernels written against the reference's Python API, run on the GPU through
+`@kernel` (tracing front-end -> typed C entry points) and checked against the
+CPU oracle.  The three copy kernels are the bodies of the reference's own GPU
+end-to-end tests (python/hckernel/tests/test_e2e.py:57-136), imported through
+the reference's package name."""
+
+import numpy as np
+import pytest
+import sympy
+from numpy.testing import assert_allclose, assert_array_equal
+
+from hckernel.kernel import *          # noqa: F401,F403  (the reference's import line)
+from hc_amd import runtime as rt
+from oracle import closed_forms as cf
+from oracle.hcsim import kernel as sim_kernel
+
+pytestmark = pytest.mark.gpu
+
+DT = typename.DT
+_copy_shapes = [(1, 27), (1, 72), (1, 128), (10, 20), (111, 813), (256, 64), (256, 1024)]
+
+
+def cdiv(a, b):
+    return (a + b - 1) // b
+
+
+def dev_pair(shape):
+    a = np.arange(shape[0] * shape[1], dtype=np.int32).reshape(shape)
+    return a, rt.to_device(a), rt.to_device(np.zeros_like(a))
+
+
+@pytest.mark.parametrize("shape", _copy_shapes)
+def test_copy(shape):
+    W, H = sym.W, sym.H
+
+    @kernel(work_shape=(W, H), backend="rocm", device="hip:0")
+    def copy_kernel(group: CurrentGroup, src: Buffer[W, H, DT], dst: Buffer[W, H, DT]):
+        x, y = group.work_offset
+        val = group.load(src[x:, y:], shape=group.shape)
+        group.store(dst[x:, y:], val)
+
+    a, da, db = dev_pair(shape)
+    copy_kernel(da, db)
+    assert_array_equal(db.to_host(), a)
+
+
+@pytest.mark.parametrize("shape", _copy_shapes)
+@pytest.mark.parametrize("unroll", [1, 2, 4])
+@pytest.mark.parametrize("vec", [False, True])
+def test_copy_unroll_and_vec(shape, unroll, vec):
+    W, H, V = sym.W, sym.H, sym.V
+    H1 = sympy.ceiling(H / V)
+
+    @kernel(work_shape=(W, H1), backend="rocm", device="hip:0", literals=[V] if vec else ())
+    def copy_kernel(group: CurrentGroup, src: Buffer[W, H, DT], dst: Buffer[W, H, DT], v: V):
+        x, y = group.work_offset
+        ld = group.vload if vec else group.load
+        val = ld(src[x:, y * V:], shape=(group.shape[0], group.shape[1] * V))
+        group.store(dst[x:, y * V:], val)
+
+    a, da, db = dev_pair(shape)
+    copy_kernel(da, db, unroll)
+    assert_array_equal(db.to_host(), a)
+
+
+def test_copy_with_torch_tensors():
+    torch = pytest.importorskip("torch")
+    if not torch.cuda.is_available():
+        pytest.skip("torch sees no GPU")
+    W, H = sym.W, sym.H
+
+    @kernel(work_shape=(W, H))
+    def copy_kernel(group: CurrentGroup, src: Buffer[W, H, DT], dst: Buffer[W, H, DT]):
+        x, y = group.work_offset
+        group.store(dst[x:, y:], group.load(src[x:, y:], shape=group.shape))
+
+    a = torch.arange(111 * 813, dtype=torch.int32).reshape(111, 813).to("cuda")
+    b = torch.zeros_like(a)
+    torch.cuda.synchronize()
+    copy_kernel(a, b)
+    torch.testing.assert_close(b, a)
+    # a strided (non-contiguous) source window
+    c = torch.zeros((111, 400), dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    copy_kernel.plan(a[:, :400], c)
+    W2, H2 = sym.W2, sym.H2
+
+    @kernel(work_shape=(W2, H2))
+    def copy_window(group: CurrentGroup, src: Buffer[W2, H2, DT], dst: Buffer[W2, H2, DT]):
+        x, y = group.work_offset
+        group.store(dst[x:, y:], group.load(src[x:, y:], shape=group.shape))
+
+    copy_window(a[:, :400], c)
+    torch.testing.assert_close(c, a[:, :400])
+
+
+def test_vector_add_same_body_on_gpu_and_on_the_host_executor():
+    N = sym.N
+
+    def body(gr, a, b, c):
+        o = gr.work_offset[0]
+        gr.store(c[o:], gr.load(a[o:], shape=gr.shape[0]) + gr.load(b[o:], shape=gr.shape[0]))
+
+    def annotated(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], c: Buffer[N, DT]):
+        body(gr, a, b, c)
+
+    n = 100_003
+    a, b = cf.inputs_c1(n)
+    dc = rt.DeviceArray((n,), np.float32)
+    kernel(work_shape=N, group_shape=256)(annotated)(rt.to_device(a), rt.to_device(b), dc)
+    host = np.zeros(n, np.float32)
+    sim_kernel(work_shape=N, group_shape=256)(annotated)(a, b, host)     # tile by tile on the CPU
+    assert_array_equal(dc.to_host().view(np.uint32), host.view(np.uint32))
+    assert_array_equal(host.view(np.uint32), cf.np_add(a, b).view(np.uint32))
+
+
+def test_fused_multiply_add_2d_ragged():
+    R, Cc = sym.R, sym.C
+    f = np.float32
+
+    @kernel(work_shape=(R, Cc))
+    def fma(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT], c: Buffer[R, Cc, DT],
+            d: Buffer[R, Cc, DT]):
+        x, y = gr.work_offset
+        ta, tb, tc = (gr.load(v[x:, y:], shape=gr.shape) for v in (a, b, c))
+        gr.store(d[x:, y:], (ta.astype(f) * tb.astype(f) + tc.astype(f)).astype(np.float16))
+
+    a, b, c = cf.inputs_c2((127, 1031))
+    dd = rt.DeviceArray(a.shape, np.float16)
+    fma(rt.to_device(a), rt.to_device(b), rt.to_device(c), dd)
+    assert_array_equal(dd.to_host().view(np.uint16), cf.np_fma_f16(a, b, c).view(np.uint16))
+
+
+def test_softmax_body_of_the_reference_example():
+    M, N, GM, MI = sym.M, sym.N, sym.GM, sym.MI
+
+    @kernel(work_shape=cdiv(M, MI), group_shape=GM, tunables=TunableParam(MI, 1, range(1, 8)))
+    def softmax(gr: CurrentGroup, a: Buffer[M, N, DT], out: Buffer[M, N, DT], gshape: GM):
+        m_start = gr.work_offset[0] * MI
+        m_block = gr.shape[0] * MI
+        a_view = gr.load(a[m_start:, :], shape=(m_block, N))
+        exp = np.exp(a_view - a_view.max(axis=1, keepdims=True))
+        gr.store(out[m_start:, :], exp / (exp.sum(axis=1, keepdims=True)))
+
+    m, n = 30, 25                      # the reference's input, in fp32
+    a = (2 * np.arange(m * n).reshape(m, n) / (m * n)).astype(np.float32)
+    out = rt.DeviceArray(a.shape, np.float32)
+    softmax(rt.to_device(a), out, 8)
+    assert_allclose(out.to_host(), cf.np_softmax(a.astype(np.float64)), rtol=2e-6)
+    (x,) = cf.inputs_c3((257, 8192))
+    out = rt.DeviceArray(x.shape, np.float32)
+    softmax(rt.to_device(x), out, 8)
+    assert_allclose(out.to_host(), cf.np_softmax(x), rtol=1e-5, atol=1e-9)
+
+
+def test_row_quantize_bit_exact():
+    M, N, GM = sym.M, sym.N, sym.GM
+
+    @kernel(work_shape=M, group_shape=GM)
+    def quant(gr: CurrentGroup, x: Buffer[M, N, DT], q: Buffer[M, N, DT], scale: Buffer[M, DT],
+              g: GM):
+        m0 = gr.work_offset[0]
+        xf = gr.load(x[m0:, :], shape=(gr.shape[0], N)).astype(np.float32)
+        s = np.abs(xf).max(axis=1, keepdims=True) / np.float32(127)
+        gr.store(q[m0:, :], np.clip(np.rint(xf / s), -127, 127).astype(np.int8))
+        gr.store(scale[m0:], s[:, 0])
+
+    (x,) = cf.inputs_c4((513, 4096))
+    dq, ds = rt.DeviceArray(x.shape, np.int8), rt.DeviceArray((x.shape[0],), np.float32)
+    quant(rt.to_device(x), dq, ds, 4)
+    q, s = cf.np_quantize(x)
+    assert_array_equal(dq.to_host(), q)
+    assert_array_equal(ds.to_host().view(np.uint32), s.view(np.uint32))
+
+
+@pytest.mark.parametrize("mnk,gshape", [((512, 256, 256), (16, 16)), ((100, 200, 300), (8, 8))])
+def test_blocked_dot_binds_to_the_mfma_gemm(mnk, gshape):
+    M, N, K = sym.M, sym.N, sym.K
+    GM, GN, MI, NI, KB = sym.GM, sym.GN, sym.MI, sym.NI, sym.KB
+    tun = (TunableParam(MI, 4, range(1, 8)), TunableParam(NI, 4, range(1, 8)),
+           TunableParam(KB, 64, range(8, 128)))
+    KI = cdiv(K, KB)
+
+    @kernel(work_shape=(cdiv(M, MI), cdiv(N, NI)), group_shape=(GM, GN), tunables=tun)
+    def dot(gr: CurrentGroup, a: Buffer[M, K, DT], bt: Buffer[N, K, DT], out: Buffer[M, N, DT],
+            gshape: (GM, GN)):
+        m0, n0 = gr.work_offset[0] * MI, gr.work_offset[1] * NI
+        mb, nb = gr.shape[0] * MI, gr.shape[1] * NI
+        r = gr.zeros(shape=(mb, nb), dtype=np.float32)
+        for k in range(KI):
+            r += np.dot(gr.load(a[m0:, k * KB:], shape=(mb, KB)),
+                        gr.load(bt[n0:, k * KB:], shape=(nb, KB)).T)
+        gr.store(out[m0:, n0:], r)
+
+    ab, bb = cf.inputs_c5(mnk)
+    dc = rt.DeviceArray((mnk[0], mnk[1]), np.uint16, bf16=True)
+    dot(rt.to_device(ab, bf16=True), rt.to_device(bb, bf16=True), dc, gshape)
+    want = cf.np_gemm_bf16(ab, bb, np.float32)
+    assert_allclose(cf.bf16_bits_to_f32(dc.to_host()), want, rtol=1e-2,
+                    atol=1e-2 * 0.02 * 0.02 * np.sqrt(mnk[2]))
+
+
+def test_unsupported_body_raises_instead_of_running_on_the_cpu():
+    N = sym.N
+
+    @kernel(work_shape=N, group_shape=64)
+    def scaled(gr: CurrentGroup, a: Buffer[N, DT], c: Buffer[N, DT]):
+        o = gr.work_offset[0]
+        gr.store(c[o:], gr.load(a[o:], shape=gr.shape[0]) * 3.0)
+
+    a = rt.to_device(np.ones(1000, np.float32))
+    c = rt.to_device(np.zeros(1000, np.float32))
+    with pytest.raises(NoNativeKernel):
+        scaled(a, c)
+    assert_array_equal(c.to_host(), np.zeros(1000, np.float32))     # untouched

@@ -1,0 +1,281 @@
+"""The `@kernel` front-end without a GPU: symbol binding, launch-geometry
+defaults, tracing of kernel bodies written against the reference's API, and the
+binding of the traced program to the typed C entry points (which entry point,
+which pointers, leading dimensions and window sizes).  Arrays are stand-ins
+that expose __cuda_array_interface__ with made-up device addresses; nothing is
+launched."""
+
+import numpy as np
+import pytest
+import sympy
+
+from hc_amd import runtime as rt
+from hc_amd.kernel import (Buffer, CurrentGroup, NoNativeKernel, TunableParam, kernel,
+                           suggest_group_shape, sym, typename)
+from oracle import closed_forms as cf
+
+DT = typename.DT
+CODES = {"float32": "<f4", "float16": "<f2", "int8": "|i1", "int32": "<i4", "bfloat16": "<u2"}
+
+
+class FakeDev:
+    """Device-array stand-in: shape, dtype and a fake address."""
+    _next = 0x7F00_0000_0000
+
+    def __init__(self, shape, dtype, ld=None):
+        self.shape = tuple(shape)
+        self.bf16 = dtype == "bfloat16"
+        self.dtype = np.dtype("uint16" if self.bf16 else dtype)
+        item = self.dtype.itemsize
+        FakeDev._next += 1 << 32
+        self.ptr = FakeDev._next
+        strides = None
+        if ld is not None:
+            strides = (ld * item, item)
+        self.__cuda_array_interface__ = {"shape": self.shape, "typestr": CODES[str(dtype)],
+                                         "data": (self.ptr, False), "strides": strides,
+                                         "version": 2}
+
+
+@pytest.fixture
+def ctx():
+    c = rt.Context.__new__(rt.Context)      # no device behind it: plans are built, never launched
+    c.queue, c.device, c.messages = 0x1234, 0x5678, []
+    return c
+
+
+def cdiv(a, b):
+    return (a + b - 1) // b
+
+
+def test_default_group_shape_comes_from_the_block_size_suggestion():
+    for work in [(16_777_259,), (8191, 8193), (256, 64), (1, 27), (111, 813), (4, 5, 6)]:
+        assert suggest_group_shape(work) == cf.default_group_shape(work)
+
+
+def test_copy_kernel_of_the_reference_e2e_test_binds_to_copy2d(ctx):
+    W, H = sym.W, sym.H
+
+    @kernel(work_shape=(W, H))
+    def copy_kernel(group: CurrentGroup, src: Buffer[W, H, DT], dst: Buffer[W, H, DT]):
+        x, y = group.work_offset
+        val = group.load(src[x:, y:], shape=group.shape)
+        group.store(dst[x:, y:], val)
+
+    for shape in [(1, 27), (10, 20), (111, 813), (256, 1024)]:
+        a, b = FakeDev(shape, "int32"), FakeDev(shape, "int32")
+        (p,) = copy_kernel.plan(a, b, ctx=ctx)
+        assert p.fn is rt.hcamdLaunchCopy2D
+        assert p.args == (ctx.queue, 4, a.ptr, shape[0], shape[1], shape[1], 1,
+                          b.ptr, shape[0], shape[1], shape[1], 1)
+
+
+@pytest.mark.parametrize("literal", [False, True])
+@pytest.mark.parametrize("unroll", [1, 2, 4])
+def test_unrolled_copy_kernels_cover_the_same_window(ctx, unroll, literal):
+    W, H, V = sym.W, sym.H, sym.V
+    H1 = sympy.ceiling(H / V)
+
+    @kernel(work_shape=(W, H1), literals=[V] if literal else ())
+    def copy_kernel(group: CurrentGroup, src: Buffer[W, H, DT], dst: Buffer[W, H, DT], v: V):
+        x, y = group.work_offset
+        load = group.vload if literal else group.load
+        val = load(src[x:, y * V:], shape=(group.shape[0], group.shape[1] * V))
+        group.store(dst[x:, y * V:], val)
+
+    a, b = FakeDev((111, 813), "int32"), FakeDev((111, 813), "int32")
+    (p,) = copy_kernel.plan(a, b, unroll, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchCopy2D and p.args[3:5] == (111, 813)
+
+
+def test_copy_into_a_larger_destination_copies_the_common_window(ctx):
+    W, H, W2, H2 = sym.W, sym.H, sym.W2, sym.H2
+
+    @kernel(work_shape=(W2, H2), group_shape=(4, 64))
+    def k(group: CurrentGroup, src: Buffer[W, H, DT], dst: Buffer[W2, H2, DT]):
+        x, y = group.work_offset
+        group.store(dst[x:, y:], group.load(src[x:, y:], shape=group.shape))
+
+    a, b = FakeDev((37, 101), "float16"), FakeDev((50, 130), "float16", ld=136)
+    (p,) = k.plan(a, b, ctx=ctx)
+    assert p.args == (ctx.queue, 2, a.ptr, 37, 101, 101, 1, b.ptr, 37, 101, 136, 1)
+
+
+def test_vector_add_binds_to_add_f32(ctx):
+    N = sym.N
+
+    @kernel(work_shape=N, group_shape=256)
+    def vadd(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], c: Buffer[N, DT]):
+        o = gr.work_offset[0]
+        gr.store(c[o:], gr.load(a[o:], shape=gr.shape[0]) + gr.load(b[o:], shape=gr.shape[0]))
+
+    n = 16_777_259
+    a, b, c = (FakeDev((n,), "float32") for _ in range(3))
+    (p,) = vadd.plan(a, b, c, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchAddF32 and p.args == (ctx.queue, a.ptr, b.ptr, c.ptr, n)
+    # second call: cached binding, fresh pointers
+    a2 = FakeDev((n,), "float32")
+    (p2,) = vadd.plan(a2, b, c, ctx=ctx)
+    assert p2.args[1] == a2.ptr and len(vadd._cache) == 1
+    with pytest.raises(NoNativeKernel):
+        vadd.plan(*(FakeDev((n,), "float16") for _ in range(3)), ctx=ctx)
+
+
+def test_fused_multiply_add_binds_to_fma_f16(ctx):
+    R, Cc = sym.R, sym.C
+    f = np.float32
+
+    @kernel(work_shape=(R, Cc))
+    def fma(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT], c: Buffer[R, Cc, DT],
+            d: Buffer[R, Cc, DT]):
+        x, y = gr.work_offset
+        ta, tb, tc = (gr.load(v[x:, y:], shape=gr.shape) for v in (a, b, c))
+        gr.store(d[x:, y:], (ta.astype(f) * tb.astype(f) + tc.astype(f)).astype(np.float16))
+
+    arrs = [FakeDev((8191, 8193), "float16") for _ in range(4)]
+    (p,) = fma.plan(*arrs, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchFmaF16
+    assert p.args == (ctx.queue, arrs[0].ptr, 8193, arrs[1].ptr, 8193, arrs[2].ptr, 8193,
+                      arrs[3].ptr, 8193, 8191, 8193)
+
+    # without the fp32 casts the arithmetic would round in fp16: no native kernel
+    @kernel(work_shape=(R, Cc))
+    def fma_half(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT],
+                 c: Buffer[R, Cc, DT], d: Buffer[R, Cc, DT]):
+        x, y = gr.work_offset
+        ta, tb, tc = (gr.load(v[x:, y:], shape=gr.shape) for v in (a, b, c))
+        gr.store(d[x:, y:], ta * tb + tc)
+
+    with pytest.raises(NoNativeKernel):
+        fma_half.plan(*arrs, ctx=ctx)
+
+
+def test_softmax_of_the_reference_example_binds_to_softmax_f32(ctx):
+    # body of python/hckernel/tests/test_examples.py:304-321
+    M, N, GM, MI = sym.M, sym.N, sym.GM, sym.MI
+
+    @kernel(work_shape=cdiv(M, MI), group_shape=GM, tunables=TunableParam(MI, 1, range(1, 8)))
+    def softmax(gr: CurrentGroup, a: Buffer[M, N, DT], out: Buffer[M, N, DT], gshape: GM):
+        m_start = gr.work_offset[0] * MI
+        m_block = gr.shape[0] * MI
+        a_view = gr.load(a[m_start:, :], shape=(m_block, N))
+        exp = np.exp(a_view - a_view.max(axis=1, keepdims=True))
+        gr.store(out[m_start:, :], exp / (exp.sum(axis=1, keepdims=True)))
+
+    x, y = FakeDev((4096, 8192), "float32"), FakeDev((4096, 8192), "float32")
+    (p,) = softmax.plan(x, y, 8, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchSoftmaxF32
+    assert p.args == (ctx.queue, x.ptr, 8192, y.ptr, 8192, 4096, 8192)
+    y2 = FakeDev((30, 25), "float32")
+    (p,) = softmax.parametrize({MI: 4}).plan(FakeDev((30, 25), "float32", ld=32), y2, 8, ctx=ctx)
+    assert p.args[2] == 32 and p.args[4] == 25 and p.args[5:] == (30, 25)
+
+
+def test_row_quantize_binds_to_quantize_f16_i8(ctx):
+    M, N, GM = sym.M, sym.N, sym.GM
+
+    @kernel(work_shape=M, group_shape=GM)
+    def quant(gr: CurrentGroup, x: Buffer[M, N, DT], q: Buffer[M, N, DT], scale: Buffer[M, DT],
+              g: GM):
+        m0 = gr.work_offset[0]
+        xf = gr.load(x[m0:, :], shape=(gr.shape[0], N)).astype(np.float32)
+        s = np.abs(xf).max(axis=1, keepdims=True) / np.float32(127)
+        gr.store(q[m0:, :], np.clip(np.rint(xf / s), -127, 127).astype(np.int8))
+        gr.store(scale[m0:], s[:, 0])
+
+    x, q, s = FakeDev((16384, 4096), "float16"), FakeDev((16384, 4096), "int8"), \
+        FakeDev((16384,), "float32")
+    (p,) = quant.plan(x, q, s, 1, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchQuantizeF16I8
+    assert p.args == (ctx.queue, x.ptr, 4096, q.ptr, 4096, s.ptr, 16384, 4096)
+
+
+@pytest.mark.parametrize("blocked", [True, False])
+def test_dot_kernel_binds_to_gemm_bf16(ctx, blocked):
+    # structure of python/hckernel/tests/test_examples.py:74-165 with B column-major
+    M, N, K = sym.M, sym.N, sym.K
+    GM, GN, MI, NI, KB = sym.GM, sym.GN, sym.MI, sym.NI, sym.KB
+    tun = (TunableParam(MI, 4, range(1, 8)), TunableParam(NI, 4, range(1, 8)),
+           TunableParam(KB, 64, range(8, 128)))
+    KI = cdiv(K, KB)
+
+    @kernel(work_shape=(cdiv(M, MI), cdiv(N, NI)), group_shape=(GM, GN), tunables=tun)
+    def dot(gr: CurrentGroup, a: Buffer[M, K, DT], bt: Buffer[N, K, DT], out: Buffer[M, N, DT],
+            gshape: (GM, GN)):
+        m0, n0 = gr.work_offset[0] * MI, gr.work_offset[1] * NI
+        mb, nb = gr.shape[0] * MI, gr.shape[1] * NI
+        r = gr.zeros(shape=(mb, nb), dtype=np.float32)
+        if blocked:
+            for k in range(KI):
+                r += np.dot(gr.load(a[m0:, k * KB:], shape=(mb, KB)),
+                            gr.load(bt[n0:, k * KB:], shape=(nb, KB)).T)
+        else:
+            r += np.dot(gr.load(a[m0:, :], shape=(mb, K)), gr.load(bt[n0:, :], shape=(nb, K)).T)
+        gr.store(out[m0:, n0:], r)
+
+    a, bt, c = (FakeDev((4096, 4096), "bfloat16") for _ in range(3))
+    (p,) = dot.plan(a, bt, c, (16, 16), ctx=ctx)
+    assert p.fn is rt.hcamdLaunchGemmBF16
+    assert p.args == (ctx.queue, a.ptr, 4096, bt.ptr, 4096, c.ptr, 4096, 4096, 4096, 4096)
+    a2, bt2, c2 = FakeDev((100, 300), "bfloat16"), FakeDev((200, 300), "bfloat16"), \
+        FakeDev((100, 200), "bfloat16")
+    (p,) = dot.plan(a2, bt2, c2, (8, 8), ctx=ctx)
+    assert p.args[7:] == (100, 200, 300)
+
+
+def test_symbol_conflicts_and_rank_errors_are_reported():
+    W, H = sym.W, sym.H
+
+    @kernel(work_shape=(W, H))
+    def k(group: CurrentGroup, src: Buffer[W, H, DT], dst: Buffer[W, H, DT]):
+        x, y = group.work_offset
+        group.store(dst[x:, y:], group.load(src[x:, y:], shape=group.shape))
+
+    with pytest.raises(RuntimeError, match="Symbol value conflict"):
+        k.plan(FakeDev((3, 4), "int32"), FakeDev((3, 5), "int32"), ctx=object())
+    with pytest.raises(RuntimeError, match="Invalid rank"):
+        k.plan(FakeDev((3,), "int32"), FakeDev((3, 5), "int32"), ctx=object())
+    with pytest.raises(RuntimeError, match="host array"):
+        k.plan(np.zeros((3, 4), np.int32), np.zeros((3, 4), np.int32), ctx=object())
+    with pytest.raises(RuntimeError, match="backend"):
+        kernel(work_shape=(W, H), backend="nvvm")(k.func).plan(FakeDev((3, 4), "int32"),
+                                                               FakeDev((3, 4), "int32"))
+
+
+def test_bodies_without_a_native_kernel_fail_loudly(ctx):
+    N = sym.N
+
+    @kernel(work_shape=N, group_shape=64)
+    def shifted(gr: CurrentGroup, a: Buffer[N, DT], c: Buffer[N, DT]):
+        o = gr.work_offset[0]
+        gr.store(c[o:], gr.load(a[o + 1:], shape=gr.shape[0]))       # not a disjoint tiling
+
+    @kernel(work_shape=N, group_shape=64)
+    def scaled(gr: CurrentGroup, a: Buffer[N, DT], c: Buffer[N, DT]):
+        o = gr.work_offset[0]
+        gr.store(c[o:], gr.load(a[o:], shape=gr.shape[0]) * 3.0)      # no such kernel
+
+    @kernel(work_shape=N, group_shape=64)
+    def nothing(gr: CurrentGroup, a: Buffer[N, DT], c: Buffer[N, DT]):
+        pass
+
+    @kernel(work_shape=N, group_shape=64)
+    def scoped(gr: CurrentGroup, a: Buffer[N, DT], c: Buffer[N, DT]):
+        @gr.workitems
+        def inner(wi):
+            pass
+        inner()
+
+    a, c = FakeDev((1000,), "float32"), FakeDev((1000,), "float32")
+    for k in (shifted, scaled, nothing, scoped):
+        with pytest.raises(NoNativeKernel):
+            k.plan(a, c, ctx=ctx)
+
+
+def test_decorator_argument_checks():
+    with pytest.raises(AssertionError):
+        kernel(work_shape=(1, 2, 3, 4))
+    with pytest.raises(AssertionError):
+        kernel(work_shape=(4, 4), group_shape=(2,))
+    with pytest.raises(AssertionError, match="Subgroup size"):
+        kernel(work_shape=4, subgroup_size=sym.SG)
