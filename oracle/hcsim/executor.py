@@ -253,7 +253,12 @@ def _bind(subs, symbol, value):
 
 def _binder_for(position, ann):
     """Returns f(subs, args) for one annotated parameter, or None."""
-    if ann in (CurrentGroup, CurrentSubGroup, CurrentWorkitem):
+    # Scope annotations bind nothing.  They are recognised by name as well as
+    # by identity so that a body annotated with another package's classes of
+    # the same names (the GPU front-end's) runs here unchanged.
+    if ann in (CurrentGroup, CurrentSubGroup, CurrentWorkitem) or \
+            getattr(ann, "__name__", "").startswith(("CurrentGroup", "CurrentSubGroup",
+                                                     "CurrentWorkitem")):
         return None
     if isinstance(ann, sympy.Symbol):
         return lambda subs, args: _bind(subs, ann, args[position])
@@ -269,7 +274,8 @@ def _binder_for(position, ann):
                     _bind(subs, s, v)
 
         return bind_tuple
-    if isinstance(ann, type) and issubclass(ann, Buffer):
+    if isinstance(ann, type) and (issubclass(ann, Buffer) or
+                                  (ann.__name__ == "Buffer" and hasattr(ann, "shape"))):
         def bind_buffer(subs, args):
             val = args[position]
             assert len(val.shape) == len(ann.shape)
