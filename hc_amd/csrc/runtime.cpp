@@ -1007,7 +1007,22 @@ int hcamdLaunchGemmBF16(OlQueue q, const void *a, size_t lda, const void *bt,
       {"hcamd_gemm_bf16_256x256_w2x2_s0", 256, 256, 256},
       {"hcamd_gemm_bf16_128x128_w2x2_s0", 128, 128, 256},
       {"hcamd_gemm_bf16_256x128_w2x2_s0", 256, 128, 256},
+      {nullptr, 0, 0, 0}, // 7: the general kernel
+      {"hcamd_gemm_bf16_p256x256_w2x4", 256, 256, 512},
+      {"hcamd_gemm_bf16_p256x256_w4x2", 256, 256, 512},
+      {"hcamd_gemm_bf16_p256x256_w2x2", 256, 256, 256},
+      {"hcamd_gemm_bf16_p128x128_w2x2", 128, 128, 256},
+      {"hcamd_gemm_bf16_p256x128_w2x2", 256, 128, 256},
+      {"hcamd_gemm_bf16_q256x256_w2x4", 256, 256, 512}, // 13
+      {"hcamd_gemm_bf16_q256x256_w4x2", 256, 256, 512},
+      {"hcamd_gemm_bf16_q256x256_w2x2", 256, 256, 256},
+      {"hcamd_gemm_bf16_q128x128_w2x2", 128, 128, 256},
+      {"hcamd_gemm_bf16_q256x128_w2x4", 256, 128, 512},
+      {"hcamd_gemm_bf16_pp256x256_w2x4", 256, 256, 512}, // 18
+      {"hcamd_gemm_bf16_pp256x256_w4x2", 256, 256, 512},
+      {"hcamd_gemm_bf16_r256x256", 256, 256, 256}, // 20
   };
+  constexpr int kFirstPipelined = 8; // variants from here need K >= 128
   constexpr int kNumTiled = sizeof(tiled) / sizeof(tiled[0]);
   const int variant = variantOf("gemm");
   const bool vec_ok = aligned16(a) && aligned16(bt) && aligned16(c) &&
@@ -1017,11 +1032,18 @@ int hcamdLaunchGemmBF16(OlQueue q, const void *a, size_t lda, const void *bt,
   if (vec_ok && variant != 7) {
     if (variant >= 1 && variant <= kNumTiled) {
       const Tiled &t = tiled[variant - 1];
-      if (m % t.bm == 0 && n % t.bn == 0)
+      if (t.name && m % t.bm == 0 && n % t.bn == 0 &&
+          (variant < kFirstPipelined || k >= 128))
         pick = &t;
     } else {
-      if (m % 256 == 0 && n % 256 == 0)
+      // default: the pipelined 256 x 256 kernel; smaller or K < 128 shapes fall
+      // back to the simpler tiled kernels
+      if (m % 256 == 0 && n % 256 == 0 && k >= 128)
+        pick = &tiled[kFirstPipelined - 1];
+      else if (m % 256 == 0 && n % 256 == 0)
         pick = &tiled[0];
+      else if (m % 128 == 0 && n % 128 == 0 && k >= 128)
+        pick = &tiled[10];
       else if (m % 128 == 0 && n % 128 == 0)
         pick = &tiled[4];
     }
