@@ -8,7 +8,9 @@ already resident in HBM.  Each workload cycles through ROTATE distinct buffer
 sets so that consecutive launches never find their inputs in the 256 MiB
 memory-side cache.  Timing: W warm-up launches, then exactly K launches between
 two HIP events recorded on the stream the kernels run on, with a host
-synchronisation and a wall clock around the same region.
+synchronisation and a wall clock around the same region.  Before the warm-up
+steps each workload runs untimed for a fraction of a second so that the GPU's
+clocks have settled.
 
 Prints ONE JSON line.  The top-level metric is the fused fp16 elementwise
 workload (d = a*b + c, 8191 x 8193); the `configs` object carries the same
@@ -33,10 +35,22 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
 ROTATE = 4
+PREWARM_SECONDS = 0.4        # untimed, per workload, before the W warm-up steps
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
 # scaled by a copy kernel of known size; filled in from profiles/*.txt.
-MEASURED_TRAFFIC = {"c1": None, "c2": None, "c3": None, "c4": None, "c5": None}
+# FETCH_SIZE reads half the true value on this device (a 256 MiB copy reads
+# 131,082 KiB), WRITE_SIZE reads true (262,215 KiB), so fetches are scaled by
+# 2.0 and writes by 1.0.  Source: profiles/hbm_traffic_pmc.txt.
+_KIB = 1024
+MEASURED_TRAFFIC = {
+    "c0": int((131085.1 * 2.0 + 262156.5) * _KIB),
+    "c1": int((65556.6 * 2.0 + 65536.2) * _KIB),     # algorithmic 201,327,108
+    "c2": int((196637.6 * 2.0 + 131072.0) * _KIB),   # algorithmic 536,870,904
+    "c3": int((65566.9 * 2.0 + 131125.1) * _KIB),    # algorithmic 268,435,456
+    "c4": int((65869.6 * 2.0 + 66048.0) * _KIB),     # algorithmic 201,392,128
+    "c5": int((98362.2 * 2.0 + 32768.0) * _KIB),     # 2.3 x the algorithmic 100,663,296 (L2 refetch)
+}
 
 
 def log(*a):
@@ -187,7 +201,30 @@ def make_workloads(rt, wl):
             t = _best_of(lambda: cf.np_gemm_bf16(self.a, self.bt, np.float32), 2)
             return t, "full size, OpenBLAS sgemm on bf16-rounded inputs", _blas_threads()
 
+    class C0(Workload):
+        """Plain copy of 256 MiB: the yardstick the hardware counters are scaled
+        by, and the practical ceiling of a read-once / write-once stream."""
+
+        def setup(self, rt):
+            self.n = 64 * 1024 * 1024
+            self.src = np.arange(self.n, dtype=np.int32)[None, :]
+            return [(rt.to_device(self.src), rt.DeviceArray((1, self.n), np.int32))
+                    for _ in range(ROTATE)]
+
+        def plan(self, rt, s):
+            return rt.plan_copy2d(s[0], s[1])
+
+        def check(self, rt, s):
+            ok = np.array_equal(s[1].to_host(), self.src)
+            return {"parity": "bit-exact" if ok else "MISMATCH", "ok": bool(ok)}
+
+        def cpu(self):
+            dst = np.empty_like(self.src)
+            return _best_of(lambda: np.copyto(dst, self.src)), "full size, numpy.copyto", 1
+
     table = {
+        "c0": C0("c0", "copy 256 MiB int32 (calibration)", "u32", "hbm", 2 * 4 * 64 * 1024 * 1024,
+                 "GB/s"),
         "c1": C1("c1", "vadd fp32 N=16777259", "f32", "hbm", W.work_c1(), "GB/s"),
         "c2": C2("c2", "fma fp16 8191x8193 (fp32 math)", "f16", "hbm", W.work_c2(), "GB/s"),
         "c3": C3("c3", "row softmax fp32 4096x8192", "f32", "hbm", W.work_c3(), "GB/s"),
@@ -195,16 +232,23 @@ def make_workloads(rt, wl):
                  W.work_c4(), "GB/s"),
         "c5": C5("c5", "GEMM bf16 4096^3 (fp32 acc)", "bf16", "mfma", W.work_c5(), "TFLOP/s"),
     }
-    keys = list(table) if wl == "all" else [wl]
+    keys = [k for k in table if k != "c0"] if wl == "all" else [wl]
     return [table[k] for k in keys]
 
 
-def run_one(rt, ctx, w, steps, warmup, want_cpu):
+def run_one(rt, ctx, w, steps, warmup, want_cpu, prewarm):
     log(f"[bench] {w.key}: {w.title}: building inputs")
     sets = w.setup(rt)
     plans = [w.plan(rt, s) for s in sets]
     launches = [p.launch for p in plans]
     ctx.synchronize()
+    # Untimed device warm-up: the GPU raises its clocks only under sustained
+    # load, so a short burst would time the ramp instead of the kernel.
+    t_end = time.perf_counter() + prewarm
+    while time.perf_counter() < t_end:
+        for i in range(50):
+            launches[i % ROTATE]()
+        ctx.synchronize()
     for i in range(warmup):
         launches[i % ROTATE]()
     ctx.synchronize()
@@ -253,8 +297,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="all", choices=["all", "c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="all", choices=["all", "c0", "c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy CPU baseline")
+    ap.add_argument("--prewarm", type=float, default=PREWARM_SECONDS,
+                    help="seconds of untimed device warm-up per workload")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no "
@@ -269,7 +315,8 @@ def main():
 
     results = {}
     for w in make_workloads(rt, args.workload):
-        results[w.key] = run_one(rt, ctx, w, args.steps, args.warmup, not args.no_cpu)
+        results[w.key] = run_one(rt, ctx, w, args.steps, args.warmup, not args.no_cpu,
+                                 args.prewarm)
 
     head_key = "c2" if "c2" in results else next(iter(results))
     head = results[head_key]

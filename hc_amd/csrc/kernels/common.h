@@ -81,16 +81,18 @@ __device__ __forceinline__ typename Op::T wave_reduce(typename Op::T v) {
       T, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
-// Workgroup reduction for WAVES waves: one LDS slot per wave, one barrier.
-// `slots` must hold WAVES floats and must not be reused for another reduction
-// without a barrier in between (callers pass a different slot array per step).
+// Reduction over the WAVES consecutive waves that share one row: one LDS slot
+// per wave, one barrier.  `slots` must hold WAVES values, belong to this row
+// only, and must not be reused for another reduction without a barrier in
+// between (callers pass a different slot array per step).  Every thread of the
+// workgroup must call it (the barrier is workgroup-wide).
 template <class Op, int WAVES>
 __device__ __forceinline__ typename Op::T group_reduce(typename Op::T v,
                                                        typename Op::T *slots) {
   v = wave_reduce<Op>(v);
   if constexpr (WAVES == 1)
     return v;
-  const int wave = threadIdx.x / kWave;
+  const int wave = (threadIdx.x / kWave) % WAVES;
   if ((threadIdx.x & (kWave - 1)) == 0)
     slots[wave] = v;
   __syncthreads();

@@ -32,7 +32,18 @@ __device__ __forceinline__ float exp_nonpos(float x) {
   return __builtin_fmaf(e, lo * kLn2, e);
 }
 
-template <int TPR, int VPT, bool FULL, bool NT>
+// exp(x - m) as 2^(x*log2(e) - m*log2(e)): one fma and one v_exp_f32.  The fma
+// rounds x*log2(e) - m*log2(e) once; with |x - m| <= 88 that is an absolute
+// error of at most 2^-18 in the exponent, i.e. a relative error below 3e-6 in
+// the result (1.3e-6 at |x - m| = 30); the rounding of m*log2(e) is common to
+// the whole row and cancels in the normalisation.  Results below 2^-126 flush to
+// zero.  NaN propagates; -inf (masked lanes) gives 0.
+__device__ __forceinline__ float exp_scaled(float x, float m_log2e) {
+  constexpr float kLog2e = 1.44269502162933349609375f;
+  return __builtin_amdgcn_exp2f(__builtin_fmaf(x, kLog2e, -m_log2e));
+}
+
+template <int TPR, int VPT, bool FULL, bool NT, bool FAST = true>
 __device__ __forceinline__ void softmax_regs(const float *x, size_t ldx,
                                              float *y, size_t ldy, size_t rows,
                                              size_t cols) {
@@ -77,11 +88,14 @@ __device__ __forceinline__ void softmax_regs(const float *x, size_t ldx,
   m = group_reduce<MaxOp, kWaves>(m, smax + rg * kWaves);
 
   float s = 0.0f;
+  // a row of -inf (or a masked-out row) has m = -inf: m*log2(e) - that would
+  // make fma(-inf, c, +inf) NaN, which is also what the plain expression gives
+  const float m_log2e = m * 1.44269502162933349609375f;
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      v[j][i] = exp_nonpos(v[j][i] - m);
+      v[j][i] = FAST ? exp_scaled(v[j][i], m_log2e) : exp_nonpos(v[j][i] - m);
       s += v[j][i];
     }
   }
@@ -112,7 +126,13 @@ __device__ __forceinline__ void softmax_regs(const float *x, size_t ldx,
   extern "C" __global__ __launch_bounds__(256) void NAME(                      \
       const float *x, size_t ldx, float *y, size_t ldy, size_t rows,           \
       size_t cols) {                                                           \
-    softmax_regs<TPR, VPT, FULL, NT>(x, ldx, y, ldy, rows, cols);              \
+    softmax_regs<TPR, VPT, FULL, NT, true>(x, ldx, y, ldy, rows, cols);        \
+  }
+#define HCAMD_SOFTMAX_ACC(NAME, TPR, VPT, FULL, NT)                            \
+  extern "C" __global__ __launch_bounds__(256) void NAME(                      \
+      const float *x, size_t ldx, float *y, size_t ldy, size_t rows,           \
+      size_t cols) {                                                           \
+    softmax_regs<TPR, VPT, FULL, NT, false>(x, ldx, y, ldy, rows, cols);       \
   }
 
 // masked (any cols up to the capacity, rows need 16-byte alignment only)
@@ -128,6 +148,72 @@ HCAMD_SOFTMAX(hcamd_softmax_f32_g256_v8_full, 256, 8, true, false)
 HCAMD_SOFTMAX(hcamd_softmax_f32_g256_v8_full_nt, 256, 8, true, true)
 HCAMD_SOFTMAX(hcamd_softmax_f32_g256_v4_full, 256, 4, true, false)
 HCAMD_SOFTMAX(hcamd_softmax_f32_g256_v2_full, 256, 2, true, false)
+// compensated exponential (about 1.5 ulp) instead of the two-instruction one
+HCAMD_SOFTMAX_ACC(hcamd_softmax_f32_g256_v8_full_nt_acc, 256, 8, true, true)
+HCAMD_SOFTMAX_ACC(hcamd_softmax_f32_g256_v8_acc, 256, 8, false, false)
+
+// Persistent form of the full-row kernel: a workgroup walks rows blockIdx.x,
+// blockIdx.x + gridDim.x, ... and requests the next row before it reduces the
+// current one, so that loads stay in flight during the reductions, the
+// exponentials and the stores, and reads and writes reach HBM interleaved
+// rather than in alternating bursts.
+template <int VPT, bool NT>
+__device__ __forceinline__ void softmax_persistent(const float *x, size_t ldx,
+                                                   float *y, size_t ldy,
+                                                   size_t rows) {
+  constexpr int kWaves = kThreads / kWave;
+  __shared__ float smax[kWaves];
+  __shared__ float ssum[kWaves];
+  const int t = threadIdx.x;
+  size_t row = blockIdx.x;
+  if (row >= rows)
+    return;
+  f32x4 cur[VPT], nxt[VPT];
+#pragma unroll
+  for (int j = 0; j < VPT; ++j)
+    nxt[j] = ldg<NT>(reinterpret_cast<const f32x4 *>(x + row * ldx) + j * kThreads + t);
+  for (; row < rows; row += gridDim.x) {
+#pragma unroll
+    for (int j = 0; j < VPT; ++j)
+      cur[j] = nxt[j];
+    const size_t next_row = row + gridDim.x;
+    if (next_row < rows) {
+#pragma unroll
+      for (int j = 0; j < VPT; ++j)
+        nxt[j] = ldg<NT>(reinterpret_cast<const f32x4 *>(x + next_row * ldx) + j * kThreads + t);
+    }
+    float m = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j)
+      m = fmaxf(fmaxf(fmaxf(m, cur[j][0]), fmaxf(cur[j][1], cur[j][2])), cur[j][3]);
+    m = group_reduce<MaxOp, kWaves>(m, smax);
+    const float m_log2e = m * 1.44269502162933349609375f;
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        cur[j][i] = exp_scaled(cur[j][i], m_log2e);
+        s += cur[j][i];
+      }
+    s = group_reduce<SumOp, kWaves>(s, ssum);
+    const float inv = 1.0f / s;
+    f32x4 *yr = reinterpret_cast<f32x4 *>(y + row * ldy);
+#pragma unroll
+    for (int j = 0; j < VPT; ++j)
+      stg<NT>(yr + j * kThreads + t, cur[j] * inv);
+  }
+}
+
+#define HCAMD_SOFTMAX_PERSIST(NAME, VPT, NT)                                   \
+  extern "C" __global__ __launch_bounds__(256) void NAME(                      \
+      const float *x, size_t ldx, float *y, size_t ldy, size_t rows,           \
+      size_t cols) {                                                           \
+    softmax_persistent<VPT, NT>(x, ldx, y, ldy, rows);                         \
+  }
+HCAMD_SOFTMAX_PERSIST(hcamd_softmax_f32_p256_v8_nt, 8, true)
+HCAMD_SOFTMAX_PERSIST(hcamd_softmax_f32_p256_v8, 8, false)
+HCAMD_SOFTMAX_PERSIST(hcamd_softmax_f32_p256_v4_nt, 4, true)
 
 // Streaming kernel: one workgroup per row, three sweeps over the row (max,
 // sum, write) with scalar accesses; the second and third sweeps hit L2.  Any

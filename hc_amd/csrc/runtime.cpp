@@ -68,6 +68,7 @@ struct Device {
   OlErrorCallback callback = nullptr;
   void *ctx = nullptr;
   int index = 0;
+  int computeUnits = 0; // filled in on first use
   // built-in modules and kernels, loaded on first use
   std::unordered_map<std::string, hipModule_t> modules;
   std::unordered_map<std::string, struct Kernel *> kernels;
@@ -221,6 +222,17 @@ int launch1d(Queue *q, const char *module, const char *name, size_t groups,
     return 1;
   const size_t grid[3] = {groups, 1, 1}, block[3] = {threads, 1, 1};
   return launch(q, k, grid, block, args, 0);
+}
+
+int computeUnitsOf(Device *dev) {
+  if (dev->computeUnits == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount,
+                              dev->index) != hipSuccess || n <= 0)
+      n = 256;
+    dev->computeUnits = n;
+  }
+  return dev->computeUnits;
 }
 
 inline bool aligned16(const void *p) {
@@ -896,10 +908,23 @@ int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,
     name = (cols == 4096 && variant != 2) ? "hcamd_softmax_f32_g256_v4_full"
                                           : "hcamd_softmax_f32_g256_v4";
   } else if (cols <= 8192) {
-    name = (cols == 8192 && variant != 2)
-               ? (variant == 3 ? "hcamd_softmax_f32_g256_v8_full"
-                               : "hcamd_softmax_f32_g256_v8_full_nt")
-               : "hcamd_softmax_f32_g256_v8";
+    const size_t cus = (size_t)computeUnitsOf(dev);
+    if (cols == 8192 && ((variant == 0 && rows >= 8 * cus) ||
+                         (variant >= 5 && variant <= 9))) {
+      // Full rows and enough of them: the persistent kernel, a fixed number of
+      // workgroups per compute unit, each prefetching its next row.
+      static const int per_cu[] = {4, 8, 2, 6, 3};
+      name = "hcamd_softmax_f32_p256_v8_nt";
+      groups = std::min<size_t>(rows, cus * per_cu[variant >= 5 ? variant - 5 : 0]);
+    } else if (variant == 4) {
+      name = cols == 8192 ? "hcamd_softmax_f32_g256_v8_full_nt_acc"
+                          : "hcamd_softmax_f32_g256_v8_acc";
+    } else {
+      name = (cols == 8192 && variant != 2)
+                 ? (variant == 3 ? "hcamd_softmax_f32_g256_v8_full"
+                                 : "hcamd_softmax_f32_g256_v8_full_nt")
+                 : "hcamd_softmax_f32_g256_v8";
+    }
   } else {
     name = "hcamd_softmax_f32_g256_v16";
   }
@@ -941,6 +966,7 @@ int hcamdLaunchQuantizeF16I8(OlQueue q, const void *x, size_t ldx, int8_t *qout,
   const char *name;
   size_t groups = rows;
   bool per_wave = false;
+  size_t rows_per_group = 1;
   if (cols <= 1024) {
     name = "hcamd_quant_f16_i8_w64_v1";
     per_wave = true;
@@ -954,6 +980,7 @@ int hcamdLaunchQuantizeF16I8(OlQueue q, const void *x, size_t ldx, int8_t *qout,
     case 4: name = "hcamd_quant_f16_i8_w64_v4_nt"; per_wave = true; break;
     case 5: name = "hcamd_quant_f16_i8_g256_v1_div"; break;
     case 6: name = "hcamd_quant_f16_i8_w64_v4_div"; per_wave = true; break;
+    case 7: name = "hcamd_quant_f16_i8_g128_v2_nt"; rows_per_group = 2; break;
     default: name = "hcamd_quant_f16_i8_g256_v1_nt"; break;
     }
   } else if (cols <= 8192) {
@@ -964,7 +991,8 @@ int hcamdLaunchQuantizeF16I8(OlQueue q, const void *x, size_t ldx, int8_t *qout,
     name = "hcamd_quant_f16_i8_g256_v8";
   }
   if (per_wave)
-    groups = ceilDiv(rows, 4);
+    rows_per_group = 4;
+  groups = ceilDiv(rows, rows_per_group);
   return launch1d(queue, "quantize", name, groups, 256, args);
 }
 
