@@ -14,6 +14,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <memory>
+#include <mutex>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -72,6 +73,7 @@ struct Device {
   // built-in modules and kernels, loaded on first use
   std::unordered_map<std::string, hipModule_t> modules;
   std::unordered_map<std::string, struct Kernel *> kernels;
+  std::mutex cacheLock; // guards the two maps
 
   void report(const char *fmt, ...) {
     if (!callback)
@@ -154,6 +156,7 @@ constexpr size_t kNumBlobs = sizeof(kBlobs) / sizeof(kBlobs[0]);
 Kernel *builtinKernel(Device *dev, const char *moduleName,
                       const char *kernelName) {
   std::string key = std::string(moduleName) + ":" + kernelName;
+  std::lock_guard<std::mutex> guard(dev->cacheLock);
   auto it = dev->kernels.find(key);
   if (it != dev->kernels.end())
     return it->second;
@@ -280,6 +283,8 @@ void stderrCallback(void *, OlSeverity sev, const char *desc) {
 
 // 0 ok, otherwise the name of the step that failed
 const char *ensureDefaultQueue(const char *deviceDesc) {
+  static std::mutex lock;
+  std::lock_guard<std::mutex> guard(lock);
   if (g_device)
     return nullptr;
   OlDevice dev = olCreateDevice(deviceDesc, &stderrCallback, nullptr);
