@@ -393,6 +393,213 @@ __device__ __forceinline__ void gemm_tile_pipelined(
   }
 }
 // ---------------------------------------------------------------------------
+// The pipelined kernel again, with the MFMA block size as a parameter: MF = 32
+// uses v_mfma_f32_32x32x16_bf16 (two K sub-steps of 16 per half-step), half as
+// many matrix instructions for the same operand reads.  Same barriers, same
+// load schedule as gemm_tile_pipelined.
+// ---------------------------------------------------------------------------
+template <int BM, int BN, int WM, int WN, int MF, int ABL = 0>
+__device__ __forceinline__ void gemm_tile_pipelined_mf(
+    const __bf16 *__restrict__ A, size_t lda, const __bf16 *__restrict__ Bt,
+    size_t ldb, __bf16 *__restrict__ C, size_t ldc, int M, int N, int K) {
+  constexpr int kWaves = WM * WN;
+  constexpr int kWaveM = BM / WM;
+  constexpr int kWaveN = BN / WN;
+  constexpr int SH = 0;
+  constexpr int kMI = kWaveM / MF;
+  constexpr int kNI = kWaveN / MF;
+  constexpr int kSub = MF == 16 ? 1 : 2;      // K sub-steps per half-step
+  constexpr int kAccRegs = MF == 16 ? 4 : 16;
+  typedef float acc_t __attribute__((ext_vector_type(kAccRegs)));
+  constexpr int kALoads = BM / (8 * kWaves); // wave-level loads per panel
+  constexpr int kBLoads = BN / (8 * kWaves);
+  static_assert(BM % (8 * kWaves) == 0 && BN % (8 * kWaves) == 0, "panel rows");
+  constexpr int kABytes = BM * kRowBytes;
+  constexpr int kStageBytes = (BM + BN) * kRowBytes;
+  constexpr int kMfma = kMI * kNI * kSub;  // MFMAs per half-step
+  constexpr int kReads = (kMI + kNI) * kSub; // ds_read_b128 per half-step
+
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kStageBytes];
+
+  int tm, tn;
+  tile_of_workgroup(M / BM, N / BN, tm, tn);
+  const int lane = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int wave_m = (wave / WN) * kWaveM;
+  const int wave_n = (wave % WN) * kWaveN;
+
+  // ---- global -> LDS ---------------------------------------------------------
+  // load i of this wave fills panel rows (i*kWaves + wave)*8 .. +8
+  const int ld_row = lane / 8, ld_pchunk = lane % 8;
+  const __bf16 *a_src[kALoads];
+  const __bf16 *b_src[kBLoads];
+#pragma unroll
+  for (int i = 0; i < kALoads; ++i) {
+    const int r = (i * kWaves + wave) * 8 + ld_row;
+    a_src[i] = A + (size_t)(tm * BM + r) * lda + ((ld_pchunk ^ swz<SH>(r)) * 8);
+  }
+#pragma unroll
+  for (int i = 0; i < kBLoads; ++i) {
+    const int r = (i * kWaves + wave) * 8 + ld_row;
+    b_src[i] = Bt + (size_t)(tn * BN + r) * ldb + ((ld_pchunk ^ swz<SH>(r)) * 8);
+  }
+  auto issue_loads = [&](int kt, int buf) {
+    const size_t k0 = (size_t)kt * kBK;
+    unsigned char *base = lds + buf * kStageBytes + wave * 1024;
+#pragma unroll
+    for (int i = 0; i < kALoads; ++i)
+      __builtin_amdgcn_global_load_lds((global_cptr)(a_src[i] + k0),
+                                       (lds_ptr)(base + i * kWaves * 1024), 16,
+                                       0, 0);
+#pragma unroll
+    for (int i = 0; i < kBLoads; ++i)
+      __builtin_amdgcn_global_load_lds(
+          (global_cptr)(b_src[i] + k0),
+          (lds_ptr)(base + kABytes + i * kWaves * 1024), 16, 0, 0);
+  };
+
+  // ---- LDS -> operand registers ------------------------------------------------
+  // lane l supplies row l % MF; its chunk in half-step h, sub-step u is
+  // 4*h + (kSub == 1 ? l / 16 : 2*u + l / 32)
+  const int lrow = lane % MF, lchunk = lane / MF;
+  const int lswz = swz<SH>(lrow);
+  int a_off[kMI], b_off[kNI];
+#pragma unroll
+  for (int i = 0; i < kMI; ++i)
+    a_off[i] = (wave_m + i * MF + lrow) * kRowBytes;
+#pragma unroll
+  for (int i = 0; i < kNI; ++i)
+    b_off[i] = kABytes + (wave_n + i * MF + lrow) * kRowBytes;
+  int coff[2][kSub];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int u = 0; u < kSub; ++u)
+      coff[h][u] = ((4 * h + (kSub == 1 ? lchunk : 2 * u + lchunk)) ^ lswz) * 16;
+
+  bf16x8 fa[2][kSub][kMI], fb[2][kSub][kNI];
+  auto read_frags = [&](int buf, int ks, auto slot) {
+    constexpr int S = decltype(slot)::value;
+#pragma unroll
+    for (int u = 0; u < kSub; ++u) {
+      const unsigned char *base = lds + buf * kStageBytes + (ks ? coff[1][u] : coff[0][u]);
+#pragma unroll
+      for (int j = 0; j < kNI; ++j)
+        fb[S][u][j] = *reinterpret_cast<const bf16x8 *>(base + b_off[j]);
+#pragma unroll
+      for (int i = 0; i < kMI; ++i)
+        fa[S][u][i] = *reinterpret_cast<const bf16x8 *>(base + a_off[i]);
+    }
+  };
+
+  acc_t acc[kMI][kNI];
+#pragma unroll
+  for (int i = 0; i < kMI; ++i)
+#pragma unroll
+    for (int j = 0; j < kNI; ++j)
+#pragma unroll
+      for (int e = 0; e < kAccRegs; ++e)
+        acc[i][j][e] = 0.f;
+  auto mma = [&](auto slot) {
+    constexpr int S = decltype(slot)::value;
+#pragma unroll
+    for (int u = 0; u < kSub; ++u)
+#pragma unroll
+      for (int i = 0; i < kMI; ++i)
+#pragma unroll
+        for (int j = 0; j < kNI; ++j) {
+          if constexpr (MF == 16)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                fb[S][u][j], fa[S][u][i], acc[i][j], 0, 0, 0);
+          else
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                fb[S][u][j], fa[S][u][i], acc[i][j], 0, 0, 0);
+        }
+  };
+  using Slot0 = std::integral_constant<int, 0>;
+  using Slot1 = std::integral_constant<int, 1>;
+
+  // Order inside a half-step: one LDS read per MFMA from the start, so the last
+  // read is out after kReads MFMAs and has the rest of the sequence to land;
+  // the global->LDS loads follow, one per MFMA.
+  auto interleave = [&](auto vmem) {
+    constexpr int V = decltype(vmem)::value;
+#pragma unroll
+    for (int i = 0; i < kMfma; ++i) {
+      constexpr int kVFirst = kMfma >= kReads + V ? kReads : 0;
+      if (i < kReads)
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
+      if (i >= kVFirst && i - kVFirst < V)
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // VMEM read
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+    }
+  };
+  using NoVmem = std::integral_constant<int, 0>;
+  using WithVmem = std::integral_constant<int, kALoads + kBLoads>;
+
+  const int KT = K / kBK; // host guarantees KT >= 2
+  issue_loads(0, 0);
+  issue_loads(1, 1);
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(kALoads + kBLoads, kNoLgkm));
+  __builtin_amdgcn_s_barrier();
+  read_frags(0, 0, Slot0{});
+
+  auto tile_step = [&](int t, auto load_next2, auto read_next) {
+    constexpr bool LOAD = decltype(load_next2)::value;
+    constexpr bool READ = decltype(read_next)::value;
+    const int buf = t & 1;
+    // even half-step: consume slot 0 (requested a whole half-step ago, so the
+    // wait is free and makes the later waits exact), fetch slot 1
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoVm, 0));
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(buf, 1, Slot1{});
+    mma(Slot0{});
+    interleave(NoVmem{});
+    // odd half-step; the fences keep the MFMAs above on this side of the wait
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (LOAD)
+      issue_loads(t + 2, buf);
+    if constexpr (READ)
+      read_frags(buf ^ 1, 0, Slot0{});
+    mma(Slot1{});
+    if constexpr (LOAD && READ)
+      interleave(WithVmem{});
+    else if constexpr (READ)
+      interleave(NoVmem{});
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  int t = 0;
+  for (; t < KT - 2; ++t)
+    tile_step(t, std::true_type{}, std::true_type{});
+  tile_step(t, std::false_type{}, std::true_type{});
+  tile_step(t + 1, std::false_type{}, std::false_type{});
+
+  // ---- epilogue ------------------------------------------------------------------
+  const int m_base = tm * BM + wave_m + lrow;
+  const int n_base = tn * BN + wave_n + lchunk * 4;
+#pragma unroll
+  for (int i = 0; i < kMI; ++i) {
+    __bf16 *crow = C + (size_t)(m_base + i * MF) * ldc + n_base;
+#pragma unroll
+    for (int j = 0; j < kNI; ++j) {
+#pragma unroll
+      for (int g = 0; g < kAccRegs / 4; ++g) {
+        bf16x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          o[e] = (__bf16)acc[i][j][4 * g + e];
+        if constexpr (ABL & 16) // measurement only: no stores
+          asm volatile("" ::"v"(o));
+        else
+          *reinterpret_cast<bf16x4 *>(crow + j * MF + g * 8) = o;
+      }
+    }
+  }
+}
+// ---------------------------------------------------------------------------
 // Pipelined kernel on v_mfma_f32_32x32x16_bf16.  A 32 x 32 output block per
 // instruction halves the number of MFMA issues and of operand reads per flop
 // compared with 16 x 16 x 32, and two independent accumulators already keep the
@@ -980,7 +1187,273 @@ __device__ __forceinline__ void gemm_tile_staged(
     }
   }
 }
+// ---------------------------------------------------------------------------
+// Ring kernel.  256 x 256 tile, K walked in slices of 32, and a ring of SLOTS
+// LDS slots of 32 KiB (A slice 256 x 32, then the B slice).  A slice is
+// requested SLOTS-1 slices before its fragments are read, so a request that
+// misses L2 has about three slices of MFMA time to come back instead of one;
+// with only two 64-wide stages the slowest of a tile's 512 requests decides
+// when the whole workgroup may go on.
+//
+//   step s:  wait until this wave's loads of slice s+1 have landed and its
+//            fragment reads of slice s are complete; barrier; request slice
+//            s+SLOTS into the slot slice s occupied; read the fragments of
+//            slice s+1 into the other register set; MFMAs on slice s.
+//
+// A slice row is 32 bf16 = 64 bytes = four chunks; chunk c of row r sits at
+// chunk position c ^ ((r >> 1) & 3), which makes the eight lanes served per
+// clock by a 16-byte LDS read hit eight different 16-byte bank groups.  A
+// wave-level direct load fills 1 KiB = 16 slice rows; lane l lands in row l/4,
+// position l%4, and therefore fetches logical chunk (l%4) ^ ((l>>3) & 3).
+// A 16 x 16 x 32 MFMA operand is exactly 16 slice rows.
+// ---------------------------------------------------------------------------
+template <int WM, int WN, int SLOTS, int MF, int ABL = 0, int SKEW = 0>
+__device__ __forceinline__ void gemm_tile_ring(
+    const __bf16 *__restrict__ A, size_t lda, const __bf16 *__restrict__ Bt,
+    size_t ldb, __bf16 *__restrict__ C, size_t ldc, int M, int N, int K) {
+  // MF = 16: v_mfma_f32_16x16x32_bf16, one K sub-step per slice.
+  // MF = 32: v_mfma_f32_32x32x16_bf16, two K sub-steps of 16 per slice.
+  // ABL (measurement only, results are wrong when non-zero) removes one part of
+  // the steady-state loop: 1 global loads, 2 LDS reads, 4 MFMAs, 8 barriers.
+  static_assert(MF == 16 || MF == 32, "MFMA block size");
+  constexpr int BM = 256, BN = 256, BK = 32;
+  constexpr int kRow = BK * 2; // bytes
+  constexpr int kWaves = WM * WN;
+  constexpr int kWaveM = BM / WM;
+  constexpr int kWaveN = BN / WN;
+  constexpr int kMI = kWaveM / MF;
+  constexpr int kNI = kWaveN / MF;
+  constexpr int kSub = MF == 16 ? 1 : 2;      // K sub-steps per slice
+  constexpr int kAccRegs = MF == 16 ? 4 : 16; // fp32 per lane per block
+  constexpr int kALoads = BM / (16 * kWaves); // wave-level loads per slice
+  constexpr int kBLoads = BN / (16 * kWaves);
+  constexpr int kLoads = kALoads + kBLoads;
+  constexpr int kABytes = BM * kRow;
+  constexpr int kSlotBytes = (BM + BN) * kRow;
+  constexpr int kMfma = kMI * kNI * kSub;
+  constexpr int kReads = (kMI + kNI) * kSub;
+  static_assert((SLOTS & (SLOTS - 1)) == 0, "slot index is s & (SLOTS-1)");
+  typedef float acc_t __attribute__((ext_vector_type(kAccRegs)));
+
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[SLOTS * kSlotBytes];
+
+  int tm, tn;
+  tile_of_workgroup(M / BM, N / BN, tm, tn);
+  const int lane = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int wave_m = (wave / WN) * kWaveM;
+  const int wave_n = (wave % WN) * kWaveN;
+
+  // ---- global -> LDS ---------------------------------------------------------
+  // load i of this wave fills slice rows (i*kWaves + wave)*16 .. +16; the byte
+  // offset of a lane inside the panel fits 32 bits (checked by the host)
+  const int ld_row = lane / 4;
+  const int ld_chunk = (lane % 4) ^ ((lane >> 3) & 3);
+  const char *a_base = reinterpret_cast<const char *>(A + (size_t)tm * BM * lda);
+  const char *b_base = reinterpret_cast<const char *>(Bt + (size_t)tn * BN * ldb);
+  uint32_t a_off[kALoads], b_off[kBLoads];
+#pragma unroll
+  for (int i = 0; i < kALoads; ++i)
+    a_off[i] = (uint32_t)(((i * kWaves + wave) * 16 + ld_row) * lda * 2 + ld_chunk * 16);
+#pragma unroll
+  for (int i = 0; i < kBLoads; ++i)
+    b_off[i] = (uint32_t)(((i * kWaves + wave) * 16 + ld_row) * ldb * 2 + ld_chunk * 16);
+  const int KS = K / BK; // host guarantees K % 64 == 0 and KS >= SLOTS
+  // Workgroups of one XCD start their walk over K at different slices (the sum
+  // over K is the same in any order): at a given moment they then fetch from
+  // different 64-byte columns of A and Bt, i.e. from different L2 channels.
+  const int skew = SKEW ? ((int)(blockIdx.x / kXcds) * SKEW) % KS : 0;
+  auto issue_loads = [&](int s) {
+    int sk = s + skew;
+    sk = sk >= KS ? sk - KS : sk;
+    const char *ga = a_base + (size_t)sk * kRow;
+    const char *gb = b_base + (size_t)sk * kRow;
+    unsigned char *base = lds + (s & (SLOTS - 1)) * kSlotBytes + wave * 1024;
+#pragma unroll
+    for (int i = 0; i < kALoads; ++i)
+      __builtin_amdgcn_global_load_lds((global_cptr)(ga + a_off[i]),
+                                       (lds_ptr)(base + i * kWaves * 1024), 16,
+                                       0, 0);
+#pragma unroll
+    for (int i = 0; i < kBLoads; ++i)
+      __builtin_amdgcn_global_load_lds(
+          (global_cptr)(gb + b_off[i]),
+          (lds_ptr)(base + kABytes + i * kWaves * 1024), 16, 0, 0);
+  };
+
+  // ---- LDS -> operand registers ------------------------------------------------
+  // lane l supplies row l % MF; its logical chunk in sub-step u is
+  // (kSub == 1 ? l / 16 : 2 * u + l / 32)
+  const int lrow = lane % MF, lhi = lane / MF;
+  const int lswz = (lrow >> 1) & 3;
+  int coff[kSub];
+#pragma unroll
+  for (int u = 0; u < kSub; ++u)
+    coff[u] = lrow * kRow + (((kSub == 1 ? lhi : 2 * u + lhi) ^ lswz) * 16);
+  const int fa_off = wave_m * kRow;
+  const int fb_off = kABytes + wave_n * kRow;
+  bf16x8 fa[2][kSub][kMI], fb[2][kSub][kNI];
+  auto read_frags = [&](int s, auto set) {
+    constexpr int S = decltype(set)::value;
+    const unsigned char *base = lds + (s & (SLOTS - 1)) * kSlotBytes;
+#pragma unroll
+    for (int u = 0; u < kSub; ++u) {
+#pragma unroll
+      for (int j = 0; j < kNI; ++j)
+        fb[S][u][j] = *reinterpret_cast<const bf16x8 *>(base + fb_off + coff[u] +
+                                                        j * MF * kRow);
+#pragma unroll
+      for (int i = 0; i < kMI; ++i)
+        fa[S][u][i] = *reinterpret_cast<const bf16x8 *>(base + fa_off + coff[u] +
+                                                        i * MF * kRow);
+    }
+  };
+
+  acc_t acc[kMI][kNI];
+#pragma unroll
+  for (int i = 0; i < kMI; ++i)
+#pragma unroll
+    for (int j = 0; j < kNI; ++j)
+#pragma unroll
+      for (int e = 0; e < kAccRegs; ++e)
+        acc[i][j][e] = 0.f;
+  auto mma = [&](auto set) {
+    constexpr int S = decltype(set)::value;
+#pragma unroll
+    for (int u = 0; u < kSub; ++u)
+#pragma unroll
+      for (int i = 0; i < kMI; ++i)
+#pragma unroll
+        for (int j = 0; j < kNI; ++j) {
+          if constexpr (MF == 16)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                fb[S][u][j], fa[S][u][i], acc[i][j], 0, 0, 0);
+          else
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                fb[S][u][j], fa[S][u][i], acc[i][j], 0, 0, 0);
+        }
+  };
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+
+  // LDS reads go out at the start of a step, at most one per MFMA and all
+  // within its first half; the global->LDS loads are spread over the rest.
+  auto interleave = [&](auto reads, auto vmem) {
+    constexpr int R = decltype(reads)::value;
+    constexpr int V = decltype(vmem)::value;
+    constexpr int kRStride = (kMfma / 2) / (R > 0 ? R : 1) > 0 ? (kMfma / 2) / (R > 0 ? R : 1) : 1;
+    constexpr int kRPer = R > kMfma / 2 ? (R + kMfma / 2 - 1) / (kMfma / 2) : 1;
+    constexpr int kVStride = V > 0 ? (kMfma - 2) / V : 1;
+#pragma unroll
+    for (int i = 0; i < kMfma; ++i) {
+      if (R > 0 && i % kRStride == 0 && (i / kRStride) * kRPer < R)
+        __builtin_amdgcn_sched_group_barrier(0x100, kRPer, 0); // DS read
+      if (V > 0 && i >= 1 && (i - 1) % kVStride == 0 && (i - 1) / kVStride < V)
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // VMEM read
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+    }
+  };
+
+  // VM = loads of this wave that may still be in flight at the top of the step
+  // (those of slices after s+1)
+  auto step = [&](int s, auto cur, auto nxt, auto load, auto read, auto vm) {
+    constexpr bool LOAD = decltype(load)::value;
+    constexpr bool READ = decltype(read)::value;
+    constexpr int VM = decltype(vm)::value;
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm((ABL & 1) ? 0 : VM, 0));
+    if constexpr (!(ABL & 8))
+      __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (LOAD && !(ABL & 1))
+      issue_loads(s + SLOTS);
+    if constexpr (READ && !(ABL & 2))
+      read_frags(s + 1, nxt);
+    if constexpr (!(ABL & 4)) {
+      mma(cur);
+      interleave(std::integral_constant < int, READ && !(ABL & 2) ? kReads : 0 > {},
+                 std::integral_constant < int, LOAD && !(ABL & 1) ? kLoads : 0 > {});
+    } else {
+      constexpr int C = decltype(cur)::value;
+#pragma unroll
+      for (int u = 0; u < kSub; ++u) {
+#pragma unroll
+        for (int j = 0; j < kNI; ++j)
+          asm volatile("" ::"v"(fb[C][u][j]));
+#pragma unroll
+        for (int i = 0; i < kMI; ++i)
+          asm volatile("" ::"v"(fa[C][u][i]));
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+#pragma unroll
+  for (int s = 0; s < SLOTS; ++s)
+    issue_loads(s);
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm((SLOTS - 1) * kLoads, kNoLgkm));
+  __builtin_amdgcn_s_barrier();
+  read_frags(0, Set0{});
+
+  using Yes = std::true_type;
+  using No = std::false_type;
+  constexpr int kSteady = (SLOTS - 2) * kLoads;
+  int s = 0;
+  for (; s < KS - SLOTS; s += 2) {
+    step(s, Set0{}, Set1{}, Yes{}, Yes{}, std::integral_constant<int, kSteady>{});
+    step(s + 1, Set1{}, Set0{}, Yes{}, Yes{}, std::integral_constant<int, kSteady>{});
+  }
+  // the last SLOTS slices: nothing left to request
+  static_assert(SLOTS == 4, "tail below is written for four slots");
+  step(s, Set0{}, Set1{}, No{}, Yes{}, std::integral_constant<int, 2 * kLoads>{});
+  step(s + 1, Set1{}, Set0{}, No{}, Yes{}, std::integral_constant<int, 1 * kLoads>{});
+  step(s + 2, Set0{}, Set1{}, No{}, Yes{}, std::integral_constant<int, 0>{});
+  step(s + 3, Set1{}, Set0{}, No{}, No{}, std::integral_constant<int, 0>{});
+
+  // ---- epilogue ------------------------------------------------------------------
+  // MF = 16: lane holds C[l % 16][4*(l/16) + e];  MF = 32: C[l % 32][8*g +
+  // 4*(l/32) + e] for accumulator element 4*g + e.
+  const int m_base = tm * BM + wave_m + lrow;
+  const int n_base = tn * BN + wave_n + lhi * 4;
+#pragma unroll
+  for (int i = 0; i < kMI; ++i) {
+    __bf16 *crow = C + (size_t)(m_base + i * MF) * ldc + n_base;
+#pragma unroll
+    for (int j = 0; j < kNI; ++j) {
+#pragma unroll
+      for (int g = 0; g < kAccRegs / 4; ++g) {
+        bf16x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          o[e] = (__bf16)acc[i][j][4 * g + e];
+        *reinterpret_cast<bf16x4 *>(crow + j * MF + g * 8) = o;
+      }
+    }
+  }
+}
 } // namespace
+
+#define HCAMD_GEMM_PM(NAME, WM, WN, MF)                                          \
+  extern "C" __global__ __launch_bounds__(WM *WN * 64) void NAME(              \
+      const __bf16 *A, size_t lda, const __bf16 *Bt, size_t ldb, __bf16 *C,    \
+      size_t ldc, int M, int N, int K) {                                       \
+    gemm_tile_pipelined_mf<256, 256, WM, WN, MF>(A, lda, Bt, ldb, C, ldc, M,   \
+                                                 N, K);                        \
+  }
+HCAMD_GEMM_PM(hcamd_gemm_bf16_pm32_256x256_w2x4, 2, 4, 32)
+HCAMD_GEMM_PM(hcamd_gemm_bf16_pm32_256x256_w4x2, 4, 2, 32)
+HCAMD_GEMM_PM(hcamd_gemm_bf16_pm16_256x256_w2x4, 2, 4, 16)
+
+#define HCAMD_GEMM_N(NAME, WM, WN, MF)                                           \
+  extern "C" __global__ __launch_bounds__(WM *WN * 64) void NAME(              \
+      const __bf16 *A, size_t lda, const __bf16 *Bt, size_t ldb, __bf16 *C,    \
+      size_t ldc, int M, int N, int K) {                                       \
+    gemm_tile_ring<WM, WN, 4, MF>(A, lda, Bt, ldb, C, ldc, M, N, K);           \
+  }
+HCAMD_GEMM_N(hcamd_gemm_bf16_n256x256_w2x2, 2, 2, 32)
+HCAMD_GEMM_N(hcamd_gemm_bf16_n256x256_w2x4, 2, 4, 16)
+HCAMD_GEMM_N(hcamd_gemm_bf16_n256x256_w4x2, 4, 2, 16)
+HCAMD_GEMM_N(hcamd_gemm_bf16_n32_256x256_w2x4, 2, 4, 32)
 
 #define HCAMD_GEMM_P(NAME, BM, BN, WM, WN, SH)                                 \
   extern "C" __global__ __launch_bounds__(WM * WN * 64) void NAME(             \

@@ -1054,8 +1054,18 @@ int hcamdLaunchGemmBF16(OlQueue q, const void *a, size_t lda, const void *bt,
       {"hcamd_gemm_bf16_pp256x256_w2x4", 256, 256, 512}, // 18
       {"hcamd_gemm_bf16_pp256x256_w4x2", 256, 256, 512},
       {"hcamd_gemm_bf16_r256x256", 256, 256, 256}, // 20
+      {"hcamd_gemm_bf16_n256x256_w2x2", 256, 256, 256},
+      {"hcamd_gemm_bf16_n256x256_w2x4", 256, 256, 512},
+      {"hcamd_gemm_bf16_n256x256_w4x2", 256, 256, 512},
+      {"hcamd_gemm_bf16_n32_256x256_w2x4", 256, 256, 512}, // 24
+      {"hcamd_gemm_bf16_pm32_256x256_w2x4", 256, 256, 512},
+      {"hcamd_gemm_bf16_pm32_256x256_w4x2", 256, 256, 512},
+      {"hcamd_gemm_bf16_pm16_256x256_w2x4", 256, 256, 512}, // 27
   };
   constexpr int kFirstPipelined = 8; // variants from here need K >= 128
+  // the ring kernels address a panel row with a 32-bit byte offset
+  constexpr int kFirstRing = 21, kLastRing = 24;
+  const bool ring_ok = lda < (size_t(1) << 22) && ldb < (size_t(1) << 22);
   constexpr int kNumTiled = sizeof(tiled) / sizeof(tiled[0]);
   const int variant = variantOf("gemm");
   const bool vec_ok = aligned16(a) && aligned16(bt) && aligned16(c) &&
@@ -1066,7 +1076,8 @@ int hcamdLaunchGemmBF16(OlQueue q, const void *a, size_t lda, const void *bt,
     if (variant >= 1 && variant <= kNumTiled) {
       const Tiled &t = tiled[variant - 1];
       if (t.name && m % t.bm == 0 && n % t.bn == 0 &&
-          (variant < kFirstPipelined || k >= 128))
+          (variant < kFirstPipelined || k >= 128) &&
+          (variant < kFirstRing || variant > kLastRing || ring_ok))
         pick = &t;
     } else {
       // default: the pipelined 256 x 256 kernel; smaller or K < 128 shapes fall
