@@ -1034,50 +1034,32 @@ int hcamdLaunchGemmBF16(OlQueue q, const void *a, size_t lda, const void *bt,
     int bm, bn, threads;
   };
   static const Tiled tiled[] = {
-      {"hcamd_gemm_bf16_256x256_w2x4_s0", 256, 256, 512},
+      {"hcamd_gemm_bf16_256x256_w2x4_s0", 256, 256, 512}, // 1
       {"hcamd_gemm_bf16_256x256_w2x4_s1", 256, 256, 512},
       {"hcamd_gemm_bf16_256x256_w4x2_s0", 256, 256, 512},
-      {"hcamd_gemm_bf16_256x256_w2x2_s0", 256, 256, 256},
       {"hcamd_gemm_bf16_128x128_w2x2_s0", 128, 128, 256},
       {"hcamd_gemm_bf16_256x128_w2x2_s0", 256, 128, 256},
-      {nullptr, 0, 0, 0}, // 7: the general kernel
-      {"hcamd_gemm_bf16_p256x256_w2x4", 256, 256, 512},
+      {nullptr, 0, 0, 0}, // 6: the general kernel
+      {"hcamd_gemm_bf16_p256x256_w2x4", 256, 256, 512}, // 7
       {"hcamd_gemm_bf16_p256x256_w4x2", 256, 256, 512},
-      {"hcamd_gemm_bf16_p256x256_w2x2", 256, 256, 256},
       {"hcamd_gemm_bf16_p128x128_w2x2", 128, 128, 256},
       {"hcamd_gemm_bf16_p256x128_w2x2", 256, 128, 256},
-      {"hcamd_gemm_bf16_q256x256_w2x4", 256, 256, 512}, // 13
-      {"hcamd_gemm_bf16_q256x256_w4x2", 256, 256, 512},
-      {"hcamd_gemm_bf16_q256x256_w2x2", 256, 256, 256},
-      {"hcamd_gemm_bf16_q128x128_w2x2", 128, 128, 256},
-      {"hcamd_gemm_bf16_q256x128_w2x4", 256, 128, 512},
-      {"hcamd_gemm_bf16_pp256x256_w2x4", 256, 256, 512}, // 18
-      {"hcamd_gemm_bf16_pp256x256_w4x2", 256, 256, 512},
-      {"hcamd_gemm_bf16_r256x256", 256, 256, 256}, // 20
-      {"hcamd_gemm_bf16_n256x256_w2x2", 256, 256, 256},
-      {"hcamd_gemm_bf16_n256x256_w2x4", 256, 256, 512},
-      {"hcamd_gemm_bf16_n256x256_w4x2", 256, 256, 512},
-      {"hcamd_gemm_bf16_n32_256x256_w2x4", 256, 256, 512}, // 24
-      {"hcamd_gemm_bf16_pm32_256x256_w2x4", 256, 256, 512},
-      {"hcamd_gemm_bf16_pm32_256x256_w4x2", 256, 256, 512},
-      {"hcamd_gemm_bf16_pm16_256x256_w2x4", 256, 256, 512}, // 27
+      {"hcamd_gemm_bf16_p32_256x256_w2x4", 256, 256, 512}, // 11
+      {"hcamd_gemm_bf16_p32_256x256_w4x2", 256, 256, 512},
   };
-  constexpr int kFirstPipelined = 8; // variants from here need K >= 128
-  // the ring kernels address a panel row with a 32-bit byte offset
-  constexpr int kFirstRing = 21, kLastRing = 24;
-  const bool ring_ok = lda < (size_t(1) << 22) && ldb < (size_t(1) << 22);
+  constexpr int kGeneral = 6;
+  constexpr int kFirstPipelined = 7; // variants from here need K >= 128
   constexpr int kNumTiled = sizeof(tiled) / sizeof(tiled[0]);
   const int variant = variantOf("gemm");
   const bool vec_ok = aligned16(a) && aligned16(bt) && aligned16(c) &&
                       lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 &&
                       k % 64 == 0;
   const Tiled *pick = nullptr;
-  if (vec_ok && variant != 7) {
+  if (vec_ok && variant != kGeneral) {
     if (variant >= 1 && variant <= kNumTiled) {
       const Tiled &t = tiled[variant - 1];
       if (t.name && m % t.bm == 0 && n % t.bn == 0 &&
-          (variant < kFirstPipelined || k >= 128) &&
-          (variant < kFirstRing || variant > kLastRing || ring_ok))
+          (variant < kFirstPipelined || k >= 128))
         pick = &t;
     } else {
       // default: the pipelined 256 x 256 kernel; smaller or K < 128 shapes fall
@@ -1087,9 +1069,9 @@ int hcamdLaunchGemmBF16(OlQueue q, const void *a, size_t lda, const void *bt,
       else if (m % 256 == 0 && n % 256 == 0)
         pick = &tiled[0];
       else if (m % 128 == 0 && n % 128 == 0 && k >= 128)
-        pick = &tiled[10];
+        pick = &tiled[8];
       else if (m % 128 == 0 && n % 128 == 0)
-        pick = &tiled[4];
+        pick = &tiled[3];
     }
   }
   if (pick) {

@@ -545,7 +545,7 @@ def test_gemm_all_variants_and_padded_output(ctx):
     ab, bb = cf.inputs_c5((512, 512, 256))
     want = cf.np_gemm_bf16(ab, bb, np.float32)
     sigma = 0.02 * 0.02 * 16
-    for v in range(0, 28):
+    for v in range(0, 13):
         rt.set_variant("gemm", v)
         got = cf.bf16_bits_to_f32(run_gemm(ab, bb, ldc_pad=8))
         say("gemm variant", v, rt.last_kernel_name())
