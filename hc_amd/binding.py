@@ -10,6 +10,9 @@ structurally:
     softmax    store(exp(x - max_row x) / sum_row exp(x - max_row x))  fp32 rows
     quantize   store(int8 clip(rint(f32 x / s), -127, 127)), s = max_row|x| / 127
     gemm       store(sum_k dot(load A[m, k-chunk], load Bt[n, k-chunk].T))   bf16
+    map        store(f(load a, load b, ...)) for any other elementwise f over up to
+               four fp32 / fp16 operands: compiled to a postfix program for the
+               fused map kernel
 
 Every load and the store must walk their buffers tile by tile: the start along a
 dimension is either 0 or group_id[i] * tile_extent, so that the tiles of all
@@ -186,11 +189,13 @@ def match_add(dst_view, value, n_groups):
     wins.append(window_of(dst_view, value.shape, n_groups))
     w = _check_same_window(wins)
 
+    general = match_map(dst_view, value, n_groups)
+
     def make(mem, ctx):
         ms = [mem[x.buffer] for x in wins]
         if all(m.shape == w.extent and m.is_contiguous() for m in ms):
             return [rt.plan_add_f32(*[_Arr(m, ctx) for m in ms])]
-        raise NoNativeKernel("c = a + b is bound for whole contiguous arrays only")
+        return general(mem, ctx)        # windows of larger or strided arrays
     return make
 
 
@@ -368,6 +373,149 @@ def match_gemm(dst_view, value, n_groups):
     return make
 
 
+# ---------------------------------------------------------------------------
+# Generic elementwise expressions -> postfix program for the fused map kernel
+# ---------------------------------------------------------------------------
+_MAP_BINARY = {"add": ("add", "add", True), "mul": ("mul", "mul", True),
+               "maximum": ("max", "max", True), "minimum": ("min", "min", True),
+               "sub": ("sub", "rsub", False), "div": ("div", "rdiv", False)}
+_MAP_UNARY = {"neg": "neg", "abs": "abs", "sqrt": "sqrt", "rint": "rint", "exp": "exp",
+              "log": "log", "tanh": "tanh"}
+_MAP_EXACT = {"neg", "abs", "maximum", "minimum", "clip"}   # fp16 in -> fp16 out, no rounding
+_MAP_FLOATS = ("float16", "float32")
+
+
+def _round_to(value: float, dtype: str) -> float:
+    import numpy as np
+    return float(np.float16(value)) if dtype == "float16" else float(np.float32(value))
+
+
+class _MapCompiler:
+    """Sethi-Ullman ordering: the operand that needs the deeper stack is
+    evaluated first, constants become immediates, so an expression with up to
+    eight distinct leaves in a balanced tree fits the four-entry stack."""
+
+    def __init__(self, n_groups):
+        self.n_groups = n_groups
+        self.inputs = []          # (buffer index, starts, Tile)
+        self.need_cache = {}
+
+    def operand(self, t: Tile) -> int:
+        v = t.attrs["view"]
+        for i, (b, st, _) in enumerate(self.inputs):
+            if b == v.base.index and st == v.starts:
+                return i
+        self.inputs.append((v.base.index, v.starts, t))
+        return len(self.inputs) - 1
+
+    def supported(self, t: Tile) -> bool:
+        if _const(t):
+            return True
+        if t.dtype_name not in _MAP_FLOATS:
+            return False
+        if _is(t, "load"):
+            return True
+        if _is(t, "astype", 1) or t.op in _MAP_UNARY or _is(t, "clip", 1):
+            return len(t.args) == 1 and self.supported(t.args[0])
+        if t.op in _MAP_BINARY and len(t.args) == 2:
+            if all(_const(a) for a in t.args):
+                return False
+            return all(self.supported(a) and (_const(a) or a.shape == t.shape) for a in t.args)
+        return False
+
+    def need(self, t: Tile) -> int:
+        if t.uid in self.need_cache:
+            return self.need_cache[t.uid]
+        if _is(t, "load") or _const(t):
+            n = 1
+        elif len(t.args) == 1:
+            n = self.need(t.args[0])
+        else:
+            a, b = t.args
+            if _const(a) or _const(b):
+                n = self.need(b if _const(a) else a)
+            else:
+                na, nb = self.need(a), self.need(b)
+                n = max(na, nb) if na != nb else na + 1
+        self.need_cache[t.uid] = n
+        return n
+
+    def emit(self, t: Tile, out: list):
+        half = t.dtype_name == "float16"
+        if _is(t, "load"):
+            out.append(("in", self.operand(t), 0.0))
+            return
+        if _const(t):
+            out.append(("const", 0, t.attrs["value"]))
+            return
+        if _is(t, "astype", 1):
+            self.emit(t.args[0], out)
+            if half and t.args[0].dtype_name != "float16":
+                out.append(("r16", 0, 0.0))
+            return
+        if _is(t, "clip", 1):
+            self.emit(t.args[0], out)
+            out.append(("maxi", 0, _round_to(t.attrs["lo"], t.dtype_name)))
+            out.append(("mini", 0, _round_to(t.attrs["hi"], t.dtype_name)))
+            return
+        if t.op in _MAP_UNARY:
+            self.emit(t.args[0], out)
+            out.append((_MAP_UNARY[t.op], 0, 0.0))
+        else:
+            fwd, rev, _ = _MAP_BINARY[t.op]
+            a, b = t.args
+            if _const(b):
+                self.emit(a, out)
+                out.append((fwd + "i", 0, _round_to(b.attrs["value"], t.dtype_name)))
+            elif _const(a):
+                self.emit(b, out)
+                out.append((rev + "i", 0, _round_to(a.attrs["value"], t.dtype_name)))
+            elif self.need(a) >= self.need(b):
+                self.emit(a, out)
+                self.emit(b, out)
+                out.append((fwd, 0, 0.0))
+            else:
+                self.emit(b, out)
+                self.emit(a, out)
+                out.append((rev, 0, 0.0))
+        if half and t.op not in _MAP_EXACT:
+            out.append(("r16", 0, 0.0))
+
+
+def match_map(dst_view, value, n_groups):
+    if dst_view.base.dtype_name not in _MAP_FLOATS:
+        return None
+    comp = _MapCompiler(n_groups)
+    if _const(value) or not comp.supported(value):
+        return None
+    if comp.need(value) > rt.MAP_STACK_DEPTH:
+        raise NoNativeKernel(f"elementwise expression stored to {dst_view.base.name} needs an "
+                             f"evaluation stack deeper than {rt.MAP_STACK_DEPTH}")
+    program: list = []
+    comp.emit(value, program)
+    if len(program) > rt.MAP_MAX_INSTRS:
+        raise NoNativeKernel(f"elementwise expression stored to {dst_view.base.name} compiles to "
+                             f"{len(program)} operations (at most {rt.MAP_MAX_INSTRS})")
+    if len(comp.inputs) > rt.MAP_MAX_INPUTS:
+        raise NoNativeKernel(f"elementwise expression stored to {dst_view.base.name} reads "
+                             f"{len(comp.inputs)} arrays (at most {rt.MAP_MAX_INPUTS})")
+    if not comp.inputs:
+        return None
+    wins = [window_of(t.attrs["view"], t.shape, n_groups) for _, _, t in comp.inputs]
+    wins.append(window_of(dst_view, value.shape, n_groups))
+    w = _check_same_window(wins)
+    if len(w.extent) > 2:
+        raise NoNativeKernel("only 1-D and 2-D buffers have native kernels")
+    types = [rt.F16 if t.dtype_name == "float16" else rt.F32 for _, _, t in comp.inputs]
+    types.append(rt.F16 if dst_view.base.dtype_name == "float16" else rt.F32)
+
+    def make(mem, ctx):
+        arrays = [_Arr(_sub(mem[x.buffer], w.extent), ctx) for x in wins]
+        return [rt.plan_map(program, arrays[:-1], arrays[-1], types)]
+    make.program = program
+    return make
+
+
 def bind(stores, n_groups):
     """stores: list of (BufferView, Tile) from one traced execution.  Returns a
     list of plan makers; raises NoNativeKernel when nothing matches."""
@@ -379,7 +527,8 @@ def bind(stores, n_groups):
             return [q]
         makers = []
         for view, value in stores:
-            for matcher in (match_copy, match_add, match_fma, match_softmax, match_gemm):
+            for matcher in (match_copy, match_add, match_fma, match_softmax, match_gemm,
+                            match_map):
                 mk = matcher(view, value, n_groups)
                 if mk is not None:
                     makers.append(mk)
@@ -388,7 +537,8 @@ def bind(stores, n_groups):
                 raise NoNativeKernel(
                     f"no hand-written kernel matches the value stored to {view.base.name} "
                     f"({value!r}); bound patterns: copy, a+b (fp32), a*b+c (fp16 storage, fp32 "
-                    "math), row softmax (fp32), row absmax int8 quantisation, bf16 GEMM")
+                    "math), row softmax (fp32), row absmax int8 quantisation, bf16 GEMM, elementwise "
+                    "expressions over fp32 / fp16 arrays")
         return makers
     except TraceError as exc:
         raise NoNativeKernel(str(exc)) from exc

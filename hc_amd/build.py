@@ -29,7 +29,7 @@ NATIVE = PKG / "_native"
 BUILD = NATIVE / "build"
 INCLUDE = PKG.parent / "include"
 
-KERNEL_MODULES = ("copy", "elementwise", "softmax", "quantize", "gemm")
+KERNEL_MODULES = ("copy", "elementwise", "map", "softmax", "quantize", "gemm")
 ARCH = "gfx950"
 
 # Packed fp32 VALU forms are kept out of every kernel.
@@ -40,6 +40,12 @@ DEVICE_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
+
+
+# The map kernel is an interpreter whose branches are all wave-uniform; left
+# alone, the compiler linearises them into a chain of guarded regions with
+# register copies at every join.
+MODULE_FLAGS = {"map": ["-mllvm", "--structurizecfg-skip-uniform-regions"]}
 
 
 def _hipcc() -> str:
@@ -64,7 +70,8 @@ def _run(cmd: list[str]) -> None:
 def build_kernel_module(name: str, keep_asm: bool = False) -> Path:
     src = CSRC / "kernels" / f"{name}.hip"
     out = BUILD / f"{name}.hsaco"
-    cmd = [_hipcc(), "--genco", "--no-gpu-bundle-output", *DEVICE_FLAGS, "-I", str(CSRC / "kernels"),
+    cmd = [_hipcc(), "--genco", "--no-gpu-bundle-output", *DEVICE_FLAGS,
+           *MODULE_FLAGS.get(name, []), "-I", str(CSRC / "kernels"),
            "-o", str(out), str(src)]
     if keep_asm:
         cmd.insert(2, "-save-temps=obj")

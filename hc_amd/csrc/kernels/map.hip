@@ -1,0 +1,424 @@
+// Fused elementwise map: out[i] = f(in0[i], ..., in3[i]) for an expression f
+// that is handed to the kernel as a short postfix program, so that a kernel body
+// made of loads, arithmetic and one store runs as ONE pass over HBM without any
+// code being generated at run time.
+//
+// The program runs on a four-entry evaluation stack of fp32 values.  The stack
+// pointer is uniform over the whole grid, so the interpreter switches on it and
+// on the opcode with scalar branches only, and every stack entry has a fixed
+// register in each arm: no indexed register access, no spills.  One pass of the
+// program serves eight elements per lane (the scalar unit issues one
+// instruction per SIMD every four cycles, and the two dozen scalar compares and
+// branches of a dispatch are what an interpreted instruction costs; more
+// elements per pass would amortise them, but the registers that takes cost more
+// in occupancy than it gains).  Operands stay packed in registers as
+// loaded (16 bytes per eight fp16, 32 per eight fp32) and are converted when
+// the program pushes them, which keeps the kernel at four waves per SIMD.
+//
+// Arithmetic is IEEE fp32 with no contraction (a*b+c is two roundings, as in
+// NumPy); R16 rounds the top of the stack to fp16 and back, which is how
+// arithmetic on fp16 tiles is expressed (for + - * / sqrt, rounding the fp32
+// result to fp16 equals computing in fp16 directly).  MAX/MIN propagate NaN like
+// numpy.maximum / numpy.minimum.
+//
+// Storage types: fp32 and fp16 per operand.  Flat form: all operands contiguous
+// and 16-byte aligned, treated as one vector.  Strided form: a rows x cols
+// window with a leading dimension per operand, any alignment, one scalar access
+// per element.
+#include "common.h"
+
+#pragma clang fp contract(off)
+
+using namespace hcamd;
+
+namespace {
+constexpr int kThreads = 256;
+constexpr int kDepth = 4;    // evaluation stack entries
+constexpr int kMaxIn = 4;    // operands
+constexpr int kMaxProg = 32; // instructions
+#ifndef HCAMD_MAP_CHUNKS
+#define HCAMD_MAP_CHUNKS 1
+#endif
+#ifndef HCAMD_MAP_WAVES
+#define HCAMD_MAP_WAVES 4 // resident waves per SIMD the flat kernel is compiled for
+#endif
+constexpr int kChunks = HCAMD_MAP_CHUNKS; // chunks of eight elements per lane per pass
+constexpr int kN = 8 * kChunks;           // elements per lane per pass
+
+// Opcodes.  The numbering is part of the C ABI (hcamdLaunchMap).
+enum : uint32_t {
+  OP_END = 0,
+  OP_IN = 1,    // push operand `arg`
+  OP_CONST = 2, // push imm
+  // pop b, pop a, push a op b
+  OP_ADD = 3,
+  OP_SUB = 4,
+  OP_MUL = 5,
+  OP_DIV = 6,
+  OP_MAX = 7,
+  OP_MIN = 8,
+  OP_RSUB = 9,  // b - a
+  OP_RDIV = 10, // b / a
+  // top = top op imm
+  OP_ADDI = 11,
+  OP_SUBI = 12,
+  OP_MULI = 13,
+  OP_DIVI = 14,
+  OP_MAXI = 15,
+  OP_MINI = 16,
+  OP_RSUBI = 17, // imm - top
+  OP_RDIVI = 18, // imm / top
+  // top = f(top)
+  OP_NEG = 19,
+  OP_ABS = 20,
+  OP_SQRT = 21,
+  OP_RINT = 22,
+  OP_EXP = 23,
+  OP_LOG = 24,
+  OP_TANH = 25,
+  OP_R16 = 26, // round to fp16 and back
+  OP_COUNT = 27,
+};
+
+struct Instr {
+  uint16_t op;
+  uint16_t arg;
+  float imm;
+};
+
+struct MapArgs {
+  const void *in[kMaxIn];
+  void *out;
+  size_t ld[kMaxIn]; // leading dimensions in elements (strided form)
+  size_t ldo;
+  size_t rows, cols; // flat form: rows = 1, cols = element count
+  uint32_t f16_mask; // bit i: operand i is fp16; bit 8: the output is fp16
+  uint32_t n_instr;
+  Instr prog[kMaxProg];
+};
+
+__device__ __forceinline__ float nan_max(float a, float b) {
+  float r = __builtin_fmaxf(a, b);
+  return (a != a || b != b) ? a + b : r;
+}
+__device__ __forceinline__ float nan_min(float a, float b) {
+  float r = __builtin_fminf(a, b);
+  return (a != a || b != b) ? a + b : r;
+}
+__device__ __forceinline__ float round16(float x) {
+  _Float16 h = (_Float16)x;
+  asm volatile("" : "+v"(h)); // keep the conversion pair from being folded
+  return (float)h;
+}
+
+template <int OP> __device__ __forceinline__ float binary(float a, float b) {
+  if constexpr (OP == OP_ADD) return a + b;
+  if constexpr (OP == OP_SUB) return a - b;
+  if constexpr (OP == OP_MUL) return a * b;
+  if constexpr (OP == OP_DIV) return a / b;
+  if constexpr (OP == OP_MAX) return nan_max(a, b);
+  if constexpr (OP == OP_MIN) return nan_min(a, b);
+  if constexpr (OP == OP_RSUB) return b - a;
+  if constexpr (OP == OP_RDIV) return b / a;
+  return a;
+}
+template <int OP> __device__ __forceinline__ float unary(float a) {
+  if constexpr (OP == OP_NEG) return -a;
+  if constexpr (OP == OP_ABS) return __builtin_fabsf(a);
+  if constexpr (OP == OP_SQRT) return __builtin_sqrtf(a);
+  if constexpr (OP == OP_RINT) return __builtin_rintf(a);
+  if constexpr (OP == OP_EXP) return expf(a);
+  if constexpr (OP == OP_LOG) return logf(a);
+  if constexpr (OP == OP_TANH) return tanhf(a);
+  if constexpr (OP == OP_R16) return round16(a);
+  return a;
+}
+
+// Operands of one pass, as loaded: per chunk eight fp16 in w[..][j][0], or
+// eight fp32 in w[..][j][0..1].
+struct Raw {
+  u32x4 w[kMaxIn][kChunks][2];
+};
+
+struct Stack {
+  float st[kDepth][kN];
+};
+
+__device__ __forceinline__ void unpack(const Raw &raw, int i, bool f16, float *dst) {
+  // The empty asm statements pin the conversion to the arm that pushes the
+  // operand: hoisted out of the interpreter loop it would hold eight more
+  // registers per operand and chunk for the whole pass.
+#pragma unroll
+  for (int j = 0; j < kChunks; ++j) {
+    if (f16) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        uint32_t w = raw.w[i][j][0][e];
+        asm volatile("" : "+v"(w));
+        dst[8 * j + 2 * e] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
+        dst[8 * j + 2 * e + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        uint32_t lo = raw.w[i][j][0][e], hi = raw.w[i][j][1][e];
+        asm volatile("" : "+v"(lo), "+v"(hi));
+        dst[8 * j + e] = __builtin_bit_cast(float, lo);
+        dst[8 * j + 4 + e] = __builtin_bit_cast(float, hi);
+      }
+    }
+  }
+}
+
+template <int SP, int OP> __device__ __forceinline__ void do_binary(Stack &r) {
+  if constexpr (SP >= 2) {
+#pragma unroll
+    for (int e = 0; e < kN; ++e)
+      r.st[SP - 2][e] = binary<OP>(r.st[SP - 2][e], r.st[SP - 1][e]);
+  }
+}
+template <int SP, int OP> __device__ __forceinline__ void do_imm(Stack &r, float imm) {
+  if constexpr (SP >= 1) {
+    // the same operation with the immediate as the second operand
+    constexpr int B = OP == OP_ADDI   ? OP_ADD
+                      : OP == OP_SUBI ? OP_SUB
+                      : OP == OP_MULI ? OP_MUL
+                      : OP == OP_DIVI ? OP_DIV
+                      : OP == OP_MAXI ? OP_MAX
+                      : OP == OP_MINI ? OP_MIN
+                      : OP == OP_RSUBI ? OP_RSUB
+                                       : OP_RDIV;
+#pragma unroll
+    for (int e = 0; e < kN; ++e)
+      r.st[SP - 1][e] = binary<B>(r.st[SP - 1][e], imm);
+  }
+}
+template <int SP, int OP> __device__ __forceinline__ void do_unary(Stack &r) {
+  if constexpr (SP >= 1) {
+#pragma unroll
+    for (int e = 0; e < kN; ++e)
+      r.st[SP - 1][e] = unary<OP>(r.st[SP - 1][e]);
+  }
+}
+
+// One instruction with SP entries on the stack; returns the new stack pointer.
+// The host has verified the program, so pushes never overflow and pops never
+// underflow; the guards only keep impossible arms out of the code.
+template <int SP>
+__device__ __forceinline__ int step(Stack &r, const Raw &raw, uint32_t f16_mask,
+                                    uint32_t op, uint32_t arg, float imm) {
+  switch (op) {
+  case OP_IN:
+    if constexpr (SP < kDepth) {
+      switch (arg) {
+      case 0: unpack(raw, 0, f16_mask & 1, r.st[SP]); break;
+      case 1: unpack(raw, 1, f16_mask & 2, r.st[SP]); break;
+      case 2: unpack(raw, 2, f16_mask & 4, r.st[SP]); break;
+      default: unpack(raw, 3, f16_mask & 8, r.st[SP]); break;
+      }
+    }
+    return SP + 1;
+  case OP_CONST:
+    if constexpr (SP < kDepth) {
+#pragma unroll
+      for (int e = 0; e < kN; ++e) r.st[SP][e] = imm;
+    }
+    return SP + 1;
+#define HCAMD_BIN(OP)                                                          \
+  case OP:                                                                     \
+    do_binary<SP, OP>(r);                                                      \
+    return SP - 1;
+    HCAMD_BIN(OP_ADD)
+    HCAMD_BIN(OP_SUB)
+    HCAMD_BIN(OP_MUL)
+    HCAMD_BIN(OP_DIV)
+    HCAMD_BIN(OP_MAX)
+    HCAMD_BIN(OP_MIN)
+    HCAMD_BIN(OP_RSUB)
+    HCAMD_BIN(OP_RDIV)
+#undef HCAMD_BIN
+#define HCAMD_IMM(OP)                                                          \
+  case OP:                                                                     \
+    do_imm<SP, OP>(r, imm);                                                    \
+    return SP;
+    HCAMD_IMM(OP_ADDI)
+    HCAMD_IMM(OP_SUBI)
+    HCAMD_IMM(OP_MULI)
+    HCAMD_IMM(OP_DIVI)
+    HCAMD_IMM(OP_MAXI)
+    HCAMD_IMM(OP_MINI)
+    HCAMD_IMM(OP_RSUBI)
+    HCAMD_IMM(OP_RDIVI)
+#undef HCAMD_IMM
+#define HCAMD_UN(OP)                                                           \
+  case OP:                                                                     \
+    do_unary<SP, OP>(r);                                                       \
+    return SP;
+    HCAMD_UN(OP_NEG)
+    HCAMD_UN(OP_ABS)
+    HCAMD_UN(OP_SQRT)
+    HCAMD_UN(OP_RINT)
+    HCAMD_UN(OP_EXP)
+    HCAMD_UN(OP_LOG)
+    HCAMD_UN(OP_TANH)
+    HCAMD_UN(OP_R16)
+#undef HCAMD_UN
+  default:
+    return SP;
+  }
+}
+
+// Runs the program; the result is r.st[0].  Instructions are fetched with
+// scalar loads from the argument block, the next one before the current one is
+// dispatched.
+__device__ __forceinline__ void run_program(const MapArgs &a, const Raw &raw,
+                                            uint32_t f16_mask, Stack &r) {
+  int sp = 0;
+  Instr next = a.prog[0];
+  for (uint32_t pc = 0; pc < a.n_instr; ++pc) {
+    const Instr cur = next;
+    next = a.prog[(pc + 1) & (kMaxProg - 1)];
+    const uint32_t op = cur.op, arg = cur.arg;
+    const float imm = cur.imm;
+    switch (sp) {
+    case 0: sp = step<0>(r, raw, f16_mask, op, arg, imm); break;
+    case 1: sp = step<1>(r, raw, f16_mask, op, arg, imm); break;
+    case 2: sp = step<2>(r, raw, f16_mask, op, arg, imm); break;
+    case 3: sp = step<3>(r, raw, f16_mask, op, arg, imm); break;
+    default: sp = step<4>(r, raw, f16_mask, op, arg, imm); break;
+    }
+  }
+}
+
+// ---- operand access -------------------------------------------------------------
+// chunk j of a pass that starts at chunk c is c + j * 256: a wave-level access
+// covers 1 KiB (fp16) or 2 KiB (fp32) of consecutive memory
+__device__ __forceinline__ void load_raw(const MapArgs &a, uint32_t n_in, size_t c,
+                                         size_t n_chunks, Raw &raw) {
+#pragma unroll
+  for (int i = 0; i < kMaxIn; ++i)
+    if (i < (int)n_in) {
+#pragma unroll
+      for (int j = 0; j < kChunks; ++j) {
+        const size_t chunk = c + (size_t)j * kThreads;
+        if (chunk < n_chunks) {
+          if ((a.f16_mask >> i) & 1) {
+            raw.w[i][j][0] = ldg<true>(static_cast<const u32x4 *>(a.in[i]) + chunk);
+          } else {
+            const u32x4 *q = static_cast<const u32x4 *>(a.in[i]) + 2 * chunk;
+            raw.w[i][j][0] = ldg<true>(q);
+            raw.w[i][j][1] = ldg<true>(q + 1);
+          }
+        }
+      }
+    }
+}
+__device__ __forceinline__ void store_chunk(void *p, bool f16, size_t chunk,
+                                            const float *src) {
+  if (f16) {
+    f16x8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (_Float16)src[e];
+    stg<true>(static_cast<f16x8 *>(p) + chunk, v);
+  } else {
+    f32x4 lo, hi;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      lo[e] = src[e];
+      hi[e] = src[4 + e];
+    }
+    f32x4 *q = static_cast<f32x4 *>(p) + 2 * chunk;
+    stg<true>(q, lo);
+    stg<true>(q + 1, hi);
+  }
+}
+__device__ __forceinline__ float load_elem(const void *p, bool f16, size_t i) {
+  return f16 ? (float)static_cast<const _Float16 *>(p)[i]
+             : static_cast<const float *>(p)[i];
+}
+__device__ __forceinline__ void store_elem(void *p, bool f16, size_t i, float v) {
+  if (f16)
+    static_cast<_Float16 *>(p)[i] = (_Float16)v;
+  else
+    static_cast<float *>(p)[i] = v;
+}
+// Element-wise gather of one pass: slot e of every operand from index idx(e),
+// zero where idx(e) is out of range; kept as fp32 whatever the operand type.
+template <class Index>
+__device__ __forceinline__ void gather(const MapArgs &a, uint32_t n_in, Raw &raw,
+                                       Index index) {
+#pragma unroll
+  for (int i = 0; i < kMaxIn; ++i)
+    if (i < (int)n_in) {
+#pragma unroll
+      for (int e = 0; e < kN; ++e) {
+        size_t off;
+        const bool ok = index(i, e, off);
+        const float v = ok ? load_elem(a.in[i], (a.f16_mask >> i) & 1, off) : 0.0f;
+        raw.w[i][e / 8][(e % 8) / 4][e % 4] = __builtin_bit_cast(uint32_t, v);
+      }
+    }
+}
+} // namespace
+
+// Flat form.  Chunk = eight consecutive elements; a workgroup owns kChunks * 256
+// consecutive chunks and lane t takes chunks t, t + 256, ...  All operand loads
+// of a pass are issued together and the program runs once they have landed;
+// the other resident waves cover the memory latency.  The elements after the
+// last whole chunk are finished by the last lane of the last workgroup, one by
+// one.
+extern "C" __global__ __launch_bounds__(256)
+__attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcamd_map_flat(
+    const MapArgs a, const uint32_t n_in) {
+  const size_t n = a.cols;
+  const size_t n_chunks = n / 8;
+  const bool out_f16 = (a.f16_mask >> 8) & 1;
+  const size_t c = (size_t)blockIdx.x * (kThreads * kChunks) + threadIdx.x;
+  Raw raw;
+  load_raw(a, n_in, c, n_chunks, raw);
+  Stack r;
+  run_program(a, raw, a.f16_mask, r);
+#pragma unroll
+  for (int j = 0; j < kChunks; ++j) {
+    const size_t chunk = c + (size_t)j * kThreads;
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = r.st[0][8 * j + e];
+    if (chunk < n_chunks)
+      store_chunk(a.out, out_f16, chunk, v);
+  }
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == kThreads - 1 && n_chunks * 8 < n) {
+    gather(a, n_in, raw, [&](int, int e, size_t &off) {
+      off = n_chunks * 8 + e;
+      return off < n;
+    });
+    run_program(a, raw, 0, r);
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      if (n_chunks * 8 + e < n)
+        store_elem(a.out, out_f16, n_chunks * 8 + e, r.st[0][e]);
+  }
+}
+
+// Strided form: blockIdx.y walks rows, x walks the columns of a row in runs of
+// 256 * kN; lane t takes columns t, t + 256, ... so a wave reads consecutive
+// elements.
+extern "C" __global__ __launch_bounds__(256) void hcamd_map_strided(
+    const MapArgs a, const uint32_t n_in) {
+  const size_t row = blockIdx.y;
+  const size_t col0 = (size_t)blockIdx.x * (kThreads * kN) + threadIdx.x;
+  Raw raw;
+  gather(a, n_in, raw, [&](int i, int e, size_t &off) {
+    const size_t col = col0 + (size_t)e * kThreads;
+    off = row * a.ld[i] + col;
+    return col < a.cols;
+  });
+  Stack r;
+  run_program(a, raw, 0, r);
+#pragma unroll
+  for (int e = 0; e < kN; ++e) {
+    const size_t col = col0 + (size_t)e * kThreads;
+    if (col < a.cols)
+      store_elem(a.out, (a.f16_mask >> 8) & 1, row * a.ldo + col, r.st[0][e]);
+  }
+}

@@ -136,6 +136,7 @@ Device::~Device() {
   extern "C" const unsigned char hcamd_blob_##n##_end[];
 HCAMD_BLOB(copy)
 HCAMD_BLOB(elementwise)
+HCAMD_BLOB(map)
 HCAMD_BLOB(softmax)
 HCAMD_BLOB(quantize)
 HCAMD_BLOB(gemm)
@@ -148,7 +149,7 @@ struct Blob {
 };
 #define HCAMD_BLOB(n) {#n, hcamd_blob_##n##_begin, hcamd_blob_##n##_end}
 const Blob kBlobs[] = {HCAMD_BLOB(copy), HCAMD_BLOB(elementwise),
-                       HCAMD_BLOB(softmax), HCAMD_BLOB(quantize),
+                       HCAMD_BLOB(map), HCAMD_BLOB(softmax), HCAMD_BLOB(quantize),
                        HCAMD_BLOB(gemm)};
 #undef HCAMD_BLOB
 constexpr size_t kNumBlobs = sizeof(kBlobs) / sizeof(kBlobs[0]);
@@ -257,7 +258,7 @@ uint32_t upPow2(uint32_t x) {
 std::unordered_map<std::string, int> &variants() {
   static std::unordered_map<std::string, int> v{
       {"add", 0},     {"fma", 0},  {"softmax", 0},
-      {"quantize", 0}, {"gemm", 0}, {"copy", 0}};
+      {"quantize", 0}, {"gemm", 0}, {"copy", 0}, {"map", 0}};
   return v;
 }
 int variantOf(const char *family) { return variants()[family]; }
@@ -865,6 +866,160 @@ int hcamdLaunchFmaF16(OlQueue q, const void *a, size_t lda, const void *b,
     char *pd = static_cast<char *>(d) + r0 * ldd * 2;
     void *args[] = {&pa, &lda, &pb, &ldb, &pc, &ldc, &pd, &ldd, &nr, &cols};
     const size_t grid[3] = {ceilDiv(cols, 256), nr, 1};
+    const size_t block[3] = {256, 1, 1};
+    if (launch(queue, k, grid, block, args, 0))
+      return 1;
+  }
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Fused elementwise map (kernels/map.hip)
+// ---------------------------------------------------------------------------
+namespace {
+constexpr size_t kMapMaxIn = HCAMD_MAP_MAX_INPUTS;
+constexpr size_t kMapMaxProg = HCAMD_MAP_MAX_INSTRS;
+constexpr int kMapDepth = HCAMD_MAP_STACK_DEPTH;
+
+// Kernel argument block; layout shared with kernels/map.hip.
+struct MapArgs {
+  const void *in[kMapMaxIn];
+  void *out;
+  size_t ld[kMapMaxIn];
+  size_t ldo;
+  size_t rows, cols;
+  uint32_t f16_mask;
+  uint32_t n_instr;
+  HcamdMapInstr prog[kMapMaxProg];
+};
+
+// Stack effect of an opcode: pops, pushes; -1 pops = unknown opcode.
+void mapStackEffect(unsigned op, int &pops, int &pushes) {
+  if (op == HCAMD_MAP_IN || op == HCAMD_MAP_CONST) {
+    pops = 0, pushes = 1;
+  } else if (op >= HCAMD_MAP_ADD && op <= HCAMD_MAP_RDIV) {
+    pops = 2, pushes = 1;
+  } else if (op >= HCAMD_MAP_ADDI && op <= HCAMD_MAP_R16) {
+    pops = 1, pushes = 1;
+  } else {
+    pops = -1, pushes = 0;
+  }
+}
+} // namespace
+
+int hcamdLaunchMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
+                   const void *const *inputs, const int *inputTypes,
+                   const size_t *inputLd, size_t nInputs, void *out,
+                   int outType, size_t ldo, size_t rows,
+                   size_t cols) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  if (!prog || nInstr == 0 || nInstr > kMapMaxProg) {
+    dev->report("hcamdLaunchMap: program of %zu instructions (1..%zu allowed)",
+                nInstr, kMapMaxProg);
+    return 1;
+  }
+  if (nInputs > kMapMaxIn || (nInputs && (!inputs || !inputTypes || !inputLd))) {
+    dev->report("hcamdLaunchMap: %zu operands (at most %zu)", nInputs,
+                kMapMaxIn);
+    return 1;
+  }
+  auto typeOk = [](int t) { return t == HCAMD_F32 || t == HCAMD_F16; };
+  if (!typeOk(outType)) {
+    dev->report("hcamdLaunchMap: unsupported output type %d", outType);
+    return 1;
+  }
+  // The program must keep the stack within bounds and leave one value.
+  int sp = 0;
+  for (size_t i = 0; i < nInstr; ++i) {
+    int pops, pushes;
+    mapStackEffect(prog[i].op, pops, pushes);
+    if (pops < 0) {
+      dev->report("hcamdLaunchMap: unknown opcode %u at %zu", prog[i].op, i);
+      return 1;
+    }
+    if (prog[i].op == HCAMD_MAP_IN && prog[i].arg >= nInputs) {
+      dev->report("hcamdLaunchMap: operand %u at %zu (only %zu given)",
+                  prog[i].arg, i, nInputs);
+      return 1;
+    }
+    if (sp < pops) {
+      dev->report("hcamdLaunchMap: stack underflow at %zu", i);
+      return 1;
+    }
+    sp += pushes - pops;
+    if (sp > kMapDepth) {
+      dev->report("hcamdLaunchMap: stack deeper than %d at %zu", kMapDepth, i);
+      return 1;
+    }
+  }
+  if (sp != 1) {
+    dev->report("hcamdLaunchMap: program leaves %d values, expected 1", sp);
+    return 1;
+  }
+  if (rows == 0 || cols == 0)
+    return 0;
+  if (!out) {
+    dev->report("hcamdLaunchMap: null pointer");
+    return 1;
+  }
+  MapArgs a{};
+  bool dense = rows == 1 || ldo == cols;
+  bool aligned = aligned16(out);
+  if (rows > 1 && ldo < cols) {
+    dev->report("hcamdLaunchMap: leading dimension smaller than cols");
+    return 1;
+  }
+  for (size_t i = 0; i < nInputs; ++i) {
+    if (!inputs[i]) {
+      dev->report("hcamdLaunchMap: null pointer");
+      return 1;
+    }
+    if (!typeOk(inputTypes[i])) {
+      dev->report("hcamdLaunchMap: unsupported operand type %d", inputTypes[i]);
+      return 1;
+    }
+    if (rows > 1 && inputLd[i] < cols) {
+      dev->report("hcamdLaunchMap: leading dimension smaller than cols");
+      return 1;
+    }
+    a.in[i] = inputs[i];
+    a.ld[i] = inputLd[i];
+    if (inputTypes[i] == HCAMD_F16)
+      a.f16_mask |= 1u << i;
+    dense = dense && (rows == 1 || inputLd[i] == cols);
+    aligned = aligned && aligned16(inputs[i]);
+  }
+  if (outType == HCAMD_F16)
+    a.f16_mask |= 1u << 8;
+  a.out = out;
+  a.ldo = ldo;
+  a.n_instr = static_cast<uint32_t>(nInstr);
+  std::memcpy(a.prog, prog, nInstr * sizeof(HcamdMapInstr));
+  uint32_t nIn = static_cast<uint32_t>(nInputs);
+  void *args[] = {&a, &nIn};
+  constexpr size_t kPerGroup = 256 * 8; // elements per workgroup: eight per lane
+  if (dense && aligned && variantOf("map") != 1) {
+    a.rows = 1;
+    a.cols = rows * cols;
+    const size_t groups = std::max(ceilDiv(a.cols, kPerGroup), (size_t)1);
+    return launch1d(queue, "map", "hcamd_map_flat", groups, 256, args);
+  }
+  Kernel *k = builtinKernel(dev, "map", "hcamd_map_strided");
+  if (!k)
+    return 1;
+  a.cols = cols;
+  const size_t esz_out = outType == HCAMD_F16 ? 2 : 4;
+  for (size_t r0 = 0; r0 < rows; r0 += 65535) {
+    const size_t nr = std::min(rows - r0, (size_t)65535);
+    a.rows = nr;
+    for (size_t i = 0; i < nInputs; ++i)
+      a.in[i] = static_cast<const char *>(inputs[i]) +
+                r0 * inputLd[i] * (inputTypes[i] == HCAMD_F16 ? 2 : 4);
+    a.out = static_cast<char *>(out) + r0 * ldo * esz_out;
+    const size_t grid[3] = {ceilDiv(cols, kPerGroup), nr, 1};
     const size_t block[3] = {256, 1, 1};
     if (launch(queue, k, grid, block, args, 0))
       return 1;

@@ -277,7 +277,8 @@ def _as_view(x) -> BufferView:
 # ---------------------------------------------------------------------------
 _UFUNC_OPS = {"add": "add", "subtract": "sub", "multiply": "mul", "true_divide": "div",
               "divide": "div", "exp": "exp", "absolute": "abs", "fabs": "abs", "rint": "rint",
-              "negative": "neg", "maximum": "maximum", "minimum": "minimum", "sqrt": "sqrt"}
+              "negative": "neg", "maximum": "maximum", "minimum": "minimum", "sqrt": "sqrt",
+              "log": "log", "tanh": "tanh"}
 
 
 def _result_dtype(a: "Tile", b: "Tile") -> str:

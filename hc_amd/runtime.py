@@ -93,6 +93,15 @@ hcamdLaunchQuantizeF16I8 = _sig(_rt, "hcamdLaunchQuantizeF16I8", _int, _vp, _vp,
                                 _vp, _sz, _vp, _sz, _sz)
 hcamdLaunchGemmBF16 = _sig(_rt, "hcamdLaunchGemmBF16", _int, _vp, _vp, _sz, _vp, _sz,
                            _vp, _sz, _sz, _sz, _sz)
+
+
+class MapInstr(C.Structure):
+    """HcamdMapInstr of include/hc_amd_runtime.h."""
+    _fields_ = [("op", C.c_uint16), ("arg", C.c_uint16), ("imm", C.c_float)]
+
+
+hcamdLaunchMap = _sig(_rt, "hcamdLaunchMap", _int, _vp, C.POINTER(MapInstr), _sz,
+                      C.POINTER(_vp), C.POINTER(_int), _sz_p, _sz, _vp, _int, _sz, _sz, _sz)
 hcamdConvertPyArray = _sig(_py, "hcamdConvertPyArray", _int, C.py_object, _int, _vp,
                            _sz_p, C.c_char_p, _sz)
 hcamdConvertPyInt64 = _sig(_py, "hcamdConvertPyInt64", _int, C.py_object,
@@ -371,6 +380,46 @@ def plan_fma_f16(a, b, c, d) -> Plan:
     return Plan(ctx, hcamdLaunchFmaF16,
                 (ctx.queue, ms[0].ptr, geo[0][2], ms[1].ptr, geo[1][2], ms[2].ptr, geo[2][2],
                  ms[3].ptr, geo[3][2], rows, cols), "hcamdLaunchFmaF16", (a, b, c, d))
+
+
+# Opcodes of the fused elementwise map (enum HcamdMapOp)
+MAP_OPS = {"in": 1, "const": 2, "add": 3, "sub": 4, "mul": 5, "div": 6, "max": 7, "min": 8,
+           "rsub": 9, "rdiv": 10, "addi": 11, "subi": 12, "muli": 13, "divi": 14, "maxi": 15,
+           "mini": 16, "rsubi": 17, "rdivi": 18, "neg": 19, "abs": 20, "sqrt": 21, "rint": 22,
+           "exp": 23, "log": 24, "tanh": 25, "r16": 26}
+MAP_MAX_INPUTS, MAP_MAX_INSTRS, MAP_STACK_DEPTH = 4, 32, 4
+F32, F16 = 0, 1
+
+
+def plan_map(program, inputs, out, types=None) -> Plan:
+    """out = f(inputs...) element by element; `program` is a sequence of
+    (opname, arg, imm) triples in postfix order (see MAP_OPS).  Arrays are
+    fp32 or fp16 (by element size, or `types` = list of F32/F16 for inputs
+    followed by the output), 1-D or 2-D with contiguous rows, all of one
+    shape."""
+    arrays = list(inputs) + [out]
+    ctx = _ctx_of(*arrays)
+    ms = [as_memref(v) for v in arrays]
+    geo = [_rows_cols(m) for m in ms]
+    rows, cols = geo[-1][0], geo[-1][1]
+    if any(g[0] != rows or g[1] != cols for g in geo):
+        raise HcRuntimeError("map: shape mismatch")
+    if types is None:
+        types = []
+        for m in ms:
+            if m.itemsize not in (2, 4):
+                raise HcRuntimeError(f"map: element size {m.itemsize} (fp32 and fp16 only)")
+            types.append(F16 if m.itemsize == 2 else F32)
+    n_in = len(inputs)
+    prog = (MapInstr * max(len(program), 1))()
+    for i, (name, arg, imm) in enumerate(program):
+        prog[i].op, prog[i].arg, prog[i].imm = MAP_OPS[name], int(arg), float(imm)
+    ptrs = (_vp * max(n_in, 1))(*[m.ptr for m in ms[:-1]])
+    tys = (_int * max(n_in, 1))(*types[:n_in])
+    lds = (_sz * max(n_in, 1))(*[g[2] for g in geo[:-1]])
+    return Plan(ctx, hcamdLaunchMap,
+                (ctx.queue, prog, len(program), ptrs, tys, lds, n_in, ms[-1].ptr, types[-1],
+                 geo[-1][2], rows, cols), "hcamdLaunchMap", (arrays, prog, ptrs, tys, lds))
 
 
 def plan_softmax_f32(x, y) -> Plan:

@@ -238,6 +238,61 @@ int hcamdLaunchFmaF16(OlQueue q, const void *a, size_t lda, const void *b,
                       size_t ldb, const void *c, size_t ldc, void *d,
                       size_t ldd, size_t rows, size_t cols) HCAMD_NOEXCEPT;
 
+/* Fused elementwise map: out = f(in_0 .. in_{n-1}) element by element over a
+ * rows x cols window, f given as a postfix program on a stack of fp32 values
+ * (at most HCAMD_MAP_STACK_DEPTH deep, HCAMD_MAP_MAX_INSTRS long, leaving one
+ * value).  This is what a kernel body made of loads, arithmetic and one store
+ * lowers to (python/hckernel/kernel_api.py:106-211 gives the tile operators
+ * their NumPy meaning): IEEE fp32 arithmetic without contraction; R16 rounds
+ * the top of the stack to fp16 and back (arithmetic on fp16 tiles); MAX / MIN
+ * propagate NaN like numpy.maximum / numpy.minimum; the store rounds to
+ * nearest even.  Operands are fp32 or fp16, each with its own leading
+ * dimension in elements.  The program is validated on the host; a malformed
+ * one is an error, not a launch. */
+enum HcamdElemType { HCAMD_F32 = 0, HCAMD_F16 = 1 };
+enum HcamdMapOp {
+  HCAMD_MAP_END = 0,
+  HCAMD_MAP_IN = 1,    /* push operand `arg` */
+  HCAMD_MAP_CONST = 2, /* push imm */
+  HCAMD_MAP_ADD = 3,   /* pop b, pop a, push a op b */
+  HCAMD_MAP_SUB = 4,
+  HCAMD_MAP_MUL = 5,
+  HCAMD_MAP_DIV = 6,
+  HCAMD_MAP_MAX = 7,
+  HCAMD_MAP_MIN = 8,
+  HCAMD_MAP_RSUB = 9,  /* b - a */
+  HCAMD_MAP_RDIV = 10, /* b / a */
+  HCAMD_MAP_ADDI = 11, /* top = top op imm */
+  HCAMD_MAP_SUBI = 12,
+  HCAMD_MAP_MULI = 13,
+  HCAMD_MAP_DIVI = 14,
+  HCAMD_MAP_MAXI = 15,
+  HCAMD_MAP_MINI = 16,
+  HCAMD_MAP_RSUBI = 17, /* imm - top */
+  HCAMD_MAP_RDIVI = 18, /* imm / top */
+  HCAMD_MAP_NEG = 19,   /* top = f(top) */
+  HCAMD_MAP_ABS = 20,
+  HCAMD_MAP_SQRT = 21,
+  HCAMD_MAP_RINT = 22,
+  HCAMD_MAP_EXP = 23,
+  HCAMD_MAP_LOG = 24,
+  HCAMD_MAP_TANH = 25,
+  HCAMD_MAP_R16 = 26
+};
+#define HCAMD_MAP_MAX_INPUTS 4
+#define HCAMD_MAP_MAX_INSTRS 32
+#define HCAMD_MAP_STACK_DEPTH 4
+typedef struct HcamdMapInstr {
+  uint16_t op;  /* HcamdMapOp */
+  uint16_t arg; /* operand index for HCAMD_MAP_IN */
+  float imm;    /* HCAMD_MAP_CONST and the *I forms */
+} HcamdMapInstr;
+int hcamdLaunchMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
+                   const void *const *inputs, const int *inputTypes,
+                   const size_t *inputLd, size_t nInputs, void *out,
+                   int outType, size_t ldo, size_t rows,
+                   size_t cols) HCAMD_NOEXCEPT;
+
 /* Row softmax, fp32: y[r,:] = exp(x[r,:]-max(x[r,:])) / sum(exp(...)).
  * Expression of python/hckernel/tests/test_examples.py:330-335. */
 int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,

@@ -33,4 +33,11 @@ Pinning status (what each part is checked against, see tests/test_oracle_*.py):
     tiles, domain masking of divide/sqrt/log, np.dot on masked tiles,
     compressed()/repr).  hcsim follows the documented numpy.ma rules for
     these, but no reference test or fixture fixes them.
+  * parity unpinned: a bare Python scalar next to a tile (`tile * 0.5`).
+    numpy.ma turns the scalar into a 0-d float64 array, so under NumPy >= 2
+    the simulator computes such an expression in float64, under NumPy 1.x in
+    the tile's type; the reference pins no NumPy version and no test covers
+    it.  The GPU front-end gives the scalar the tile's type (what a plain
+    ndarray does); tests that compare the two write scalars as np.float32(..)
+    / np.float16(..), which both sides treat alike.
 """

@@ -200,13 +200,132 @@ def test_blocked_dot_binds_to_the_mfma_gemm(mnk, gshape):
                     atol=1e-2 * 0.02 * 0.02 * np.sqrt(mnk[2]))
 
 
+# ---------------------------------------------------------------------------
+# arbitrary elementwise bodies: the same body on the GPU (fused map kernel) and
+# on the host executor, bit for bit
+# ---------------------------------------------------------------------------
+def random_expression(rng, depth, dtype):
+    """A Python function of three tiles built from operations whose fp32 / fp16
+    results are exactly defined (no transcendental functions), together with its
+    source text.  Denominators are kept away from zero: the host executor's
+    masked arithmetic would otherwise leave those elements unwritten.  Scalars
+    are written as K(value) with K the tiles' own type: a bare Python float
+    would make numpy.ma, and with it the host executor, compute in float64."""
+    def leaf():
+        return rng.choice(["a", "b", "c"])
+
+    def gen(d):
+        if d == 0 or rng.random() < 0.15:
+            return leaf()
+        kind = rng.integers(0, 12)
+        x = gen(d - 1)
+        if kind <= 2:
+            return f"({x} {rng.choice(['+', '-', '*'])} {gen(d - 1)})"
+        if kind == 3:
+            return f"({x} / (np.abs({gen(d - 1)}) + K(1.0)))"
+        if kind == 4:
+            return f"np.{rng.choice(['maximum', 'minimum'])}({x}, {gen(d - 1)})"
+        if kind == 5:
+            return f"(-{x})"
+        if kind == 6:
+            return f"np.abs({x})"
+        if kind == 7:
+            return f"np.sqrt(np.abs({x}))"
+        if kind == 8:
+            return f"np.rint({x} * K(3.0))"
+        if kind == 9:
+            return f"np.clip({x}, -1.5, 2.25)"
+        if kind == 10:
+            return f"(K({rng.choice(['0.3', '2.0', '-1.25'])}) {rng.choice(['+', '-', '*', '/'])} " \
+                   f"(np.abs({x}) + K(0.5)))"
+        return f"({x} {rng.choice(['+', '-', '*', '/'])} K({rng.choice(['0.7', '4.0', '-0.125'])}))"
+
+    text = gen(depth)
+    while text in ("a", "b", "c"):
+        text = gen(depth)
+    return eval(f"lambda a, b, c: {text}", {"np": np, "K": dtype}), text
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("layout", ["flat", "ragged2d", "window"])
+def test_random_elementwise_bodies_match_the_host_executor(dtype, layout):
+    rng = np.random.default_rng({"flat": 1, "ragged2d": 2, "window": 3}[layout] * 10 +
+                                np.dtype(dtype).itemsize)
+    N, R, Cc, R2, C2 = sym.N, sym.R, sym.C, sym.R2, sym.C2
+    if layout == "flat":
+        shape = big = (100_003,)
+    elif layout == "ragged2d":
+        shape = big = (37, 1031)
+    else:
+        shape, big = (36, 1024), (40, 1100)         # a window of larger arrays
+    vals = [(rng.uniform(0.5, 2.0, big) * rng.choice([-1.0, 1.0], big)).astype(dtype)
+            for _ in range(3)]
+    tried = bound = 0
+    while bound < 12:
+        expr, text = random_expression(rng, 3, dtype)
+        tried += 1
+
+        if len(shape) == 1:
+            def body(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], c: Buffer[N, DT],
+                     out: Buffer[N, DT]):
+                o, g = gr.work_offset[0], gr.shape[0]
+                gr.store(out[o:], expr(gr.load(a[o:], shape=g), gr.load(b[o:], shape=g),
+                                       gr.load(c[o:], shape=g)))
+            deco = dict(work_shape=N, group_shape=256)
+        else:
+            def body(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT],
+                     c: Buffer[R, Cc, DT], out: Buffer[R2, C2, DT]):
+                x, y = gr.work_offset
+                gr.store(out[x:, y:], expr(*(gr.load(v[x:, y:], shape=gr.shape)
+                                            for v in (a, b, c))))
+            deco = dict(work_shape=(shape[0], shape[1]), group_shape=(4, 64))
+        poison = np.full(shape if layout != "window" else (40, 1040), 7.5, dtype)
+        host = poison.copy()
+        with np.errstate(all="ignore"):
+            sim_kernel(**deco)(body)(*vals, host)
+        dout = rt.to_device(poison)
+        try:
+            kernel(**deco)(body)(*[rt.to_device(v) for v in vals], dout)
+        except NoNativeKernel as exc:                  # deeper than the stack: not bound
+            assert "stack" in str(exc) or "operations" in str(exc), text
+            continue
+        bound += 1
+        got = dout.to_host()
+        nan = np.isnan(host)
+        assert (np.isnan(got) == nan).all(), text
+        u = np.uint32 if dtype == np.float32 else np.uint16
+        assert_array_equal(got.view(u)[~nan], host.view(u)[~nan], err_msg=text)
+    assert tried < 40
+
+
+def test_elementwise_body_with_transcendental_functions():
+    N = sym.N
+
+    def body(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], out: Buffer[N, DT]):
+        o, g = gr.work_offset[0], gr.shape[0]
+        x, y = gr.load(a[o:], shape=g), gr.load(b[o:], shape=g)
+        one = np.float32(1)
+        gr.store(out[o:], x / (one + np.exp(-x)) + np.tanh(y) * np.log(np.abs(y) + one))
+
+    rng = np.random.default_rng(21)
+    n = 70_001
+    a, b = (rng.standard_normal(n).astype(np.float32) * 3 for _ in range(2))
+    host = np.zeros(n, np.float32)
+    sim_kernel(work_shape=N, group_shape=256)(body)(a, b, host)
+    dout = rt.DeviceArray((n,), np.float32)
+    kernel(work_shape=N, group_shape=256)(body)(rt.to_device(a), rt.to_device(b), dout)
+    # exp / tanh / log are within 2 ulp of NumPy's; the sum of two terms of
+    # either sign keeps that as an absolute error relative to the larger term
+    assert_allclose(dout.to_host(), host, rtol=2e-6, atol=2e-6)
+
+
 def test_unsupported_body_raises_instead_of_running_on_the_cpu():
     N = sym.N
 
     @kernel(work_shape=N, group_shape=64)
     def scaled(gr: CurrentGroup, a: Buffer[N, DT], c: Buffer[N, DT]):
         o = gr.work_offset[0]
-        gr.store(c[o:], gr.load(a[o:], shape=gr.shape[0]) * 3.0)
+        gr.store(c[o:], (gr.load(a[o:], shape=gr.shape[0]) * 3.0).sum())
 
     a = rt.to_device(np.ones(1000, np.float32))
     c = rt.to_device(np.zeros(1000, np.float32))

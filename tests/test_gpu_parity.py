@@ -34,10 +34,10 @@ def ctx():
 
 @pytest.fixture(autouse=True)
 def default_variants():
-    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy"):
+    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy", "map"):
         rt.set_variant(fam, 0)
     yield
-    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy"):
+    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy", "map"):
         rt.set_variant(fam, 0)
 
 
@@ -308,6 +308,170 @@ def test_fma_full_benchmark_size(ctx):
     rt.fma_f16(dev(a), dev(b), dev(c), dd)
     assert rt.last_kernel_name().startswith("hcamd_fma_f16_v")
     assert_array_equal(dd.to_host().view(np.uint16), cf.np_fma_f16(a, b, c).view(np.uint16))
+
+
+# ---------------------------------------------------------------------------
+# fused elementwise map (postfix programs)
+# ---------------------------------------------------------------------------
+def I(name, arg=0, imm=0.0):
+    return (name, arg, imm)
+
+
+def assert_same_floats(got, want, what=""):
+    """Bit for bit, except that any NaN matches any NaN (an invalid operation
+    yields a NaN whose sign differs between the host CPU and the GPU)."""
+    assert got.dtype == want.dtype and got.shape == want.shape
+    nan = np.isnan(want)
+    assert_array_equal(np.isnan(got), nan, what)
+    u = {2: np.uint16, 4: np.uint32}[got.dtype.itemsize]
+    assert_array_equal(got.view(u)[~nan], want.view(u)[~nan], what)
+
+
+FMA_PROGRAM = [I("in", 0), I("in", 1), I("mul"), I("in", 2), I("add")]
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (1, 4099), (17, 4099), (129, 1031)])
+@pytest.mark.parametrize("variant", [0, 1])
+def test_map_fma_program_equals_the_fma_kernel(ctx, shape, variant):
+    a, b, c = cf.inputs_c2(shape)
+    want = cf.np_fma_f16(a, b, c)
+    rt.set_variant("map", variant)                      # 1: always the strided kernel
+    d = poisoned(shape, np.float16)
+    rt.plan_map(FMA_PROGRAM, [dev(a), dev(b), dev(c)], d).launch(sync=True)
+    say("map", shape, rt.last_kernel_name())
+    assert rt.last_kernel_name() == ("hcamd_map_flat" if variant == 0 else "hcamd_map_strided")
+    assert_array_equal(d.to_host().view(np.uint16), want.view(np.uint16))
+    assert_array_equal(want.view(np.uint16), co.fma_f16(a, b, c).view(np.uint16))
+
+
+def test_map_window_of_larger_arrays_leaves_the_rest_untouched(ctx):
+    rows, cols = 37, 1031
+    a, b, c = cf.inputs_c2((rows, cols))
+    big = [np.zeros((40, 1100), np.float16) for _ in range(3)]
+    for dst, src in zip(big, (a, b, c)):
+        dst[:rows, :cols] = src
+    dbig = [dev(x) for x in big]
+    out = poisoned((40, 1040), np.float16)
+    views = [_View(x, (rows, cols), 0, (1100, 1)) for x in dbig]
+    rt.plan_map(FMA_PROGRAM, views, _View(out, (rows, cols), 0, (1040, 1))).launch(sync=True)
+    assert rt.last_kernel_name() == "hcamd_map_strided"
+    got = out.to_host()
+    assert_array_equal(got[:rows, :cols].view(np.uint16), cf.np_fma_f16(a, b, c).view(np.uint16))
+    p = poison_value(np.float16)
+    assert (got[rows:].view(np.uint16) == p.view(np.uint16)).all()
+    assert (got[:, cols:].view(np.uint16) == p.view(np.uint16)).all()
+
+
+def test_map_every_operation_against_numpy(ctx):
+    rng = np.random.default_rng(11)
+    n = 50_001
+    f = np.float32
+    x = rng.uniform(0.5, 2.0, n).astype(f) * rng.choice([-1, 1], n).astype(f)
+    y = rng.uniform(0.5, 2.0, n).astype(f) * rng.choice([-1, 1], n).astype(f)
+    x[:4] = [np.nan, 1.0, np.inf, -0.0]
+    y[:4] = [1.0, np.nan, -np.inf, 1.0]
+    dx, dy = dev(x), dev(y)
+    k = f(0.75)
+    exact = {
+        "add": x + y, "sub": x - y, "mul": x * y, "div": x / y,
+        "max": np.maximum(x, y), "min": np.minimum(x, y), "rsub": y - x, "rdiv": y / x,
+    }
+    with np.errstate(all="ignore"):
+        for name, want in exact.items():
+            out = poisoned((n,), f)
+            rt.plan_map([I("in", 0), I("in", 1), I(name)], [dx, dy], out).launch(sync=True)
+            assert_same_floats(out.to_host(), want.astype(f), name)
+        imm = {"addi": x + k, "subi": x - k, "muli": x * k, "divi": x / k,
+               "maxi": np.maximum(x, k), "mini": np.minimum(x, k), "rsubi": k - x,
+               "rdivi": k / x}
+        for name, want in imm.items():
+            out = poisoned((n,), f)
+            rt.plan_map([I("in", 0), I(name, 0, k)], [dx], out).launch(sync=True)
+            assert_same_floats(out.to_host(), want.astype(f), name)
+        unary = {"neg": -x, "abs": np.abs(x), "rint": np.rint(x * f(3)),
+                 "r16": x.astype(np.float16).astype(f)}
+        for name, want in unary.items():
+            pre = [I("muli", 0, 3.0)] if name == "rint" else []
+            out = poisoned((n,), f)
+            rt.plan_map([I("in", 0)] + pre + [I(name)], [dx], out).launch(sync=True)
+            assert_same_floats(out.to_host(), want, name)
+        # correctly rounded square root, bit for bit
+        out = poisoned((n,), f)
+        rt.plan_map([I("in", 0), I("abs"), I("sqrt")], [dx], out).launch(sync=True)
+        assert_same_floats(out.to_host(), np.sqrt(np.abs(x)), "sqrt")
+        # transcendental functions: within 2 ulp of NumPy's fp32 results
+        for name, fn, arg in (("exp", np.exp, x), ("log", np.log, np.abs(x)), ("tanh", np.tanh, x)):
+            out = poisoned((n,), f)
+            pre = [I("abs")] if name == "log" else []
+            rt.plan_map([I("in", 0)] + pre + [I(name)], [dx], out).launch(sync=True)
+            got, want = out.to_host(), fn(arg).astype(f)
+            ok = np.isfinite(want)
+            assert_array_equal(np.isnan(got), np.isnan(want), name)
+            assert_allclose(got[ok], want[ok], rtol=3e-7, atol=1e-45, err_msg=name)
+    # a constant pushed on the stack, and the deepest legal stack
+    out = poisoned((n,), f)
+    rt.plan_map([I("const", 0, 2.0), I("in", 0), I("const", 0, 3.0), I("in", 1), I("mul"),
+                 I("add"), I("mul")], [dx, dy], out).launch(sync=True)
+    with np.errstate(all="ignore"):
+        assert_same_floats(out.to_host(), f(2) * (x + f(3) * y), "stack")
+
+
+def test_map_no_contraction_two_roundings_in_fp32(ctx):
+    # a*b+c where the fused result differs from the twice-rounded one
+    rng = np.random.default_rng(12)
+    n = 1 << 20
+    a, b, c = (rng.standard_normal(n).astype(np.float32) for _ in range(3))
+    want = a * b + c
+    fused = (a.astype(np.float64) * b.astype(np.float64) + c.astype(np.float64)).astype(np.float32)
+    assert (want != fused).any()                      # the inputs do tell the two apart
+    out = poisoned((n,), np.float32)
+    rt.plan_map(FMA_PROGRAM, [dev(a), dev(b), dev(c)], out).launch(sync=True)
+    assert_array_equal(out.to_host().view(np.uint32), want.view(np.uint32))
+
+
+def test_map_mixed_storage_types(ctx):
+    rng = np.random.default_rng(13)
+    shape = (33, 517)
+    a = rng.standard_normal(shape).astype(np.float16)
+    b = rng.standard_normal(shape).astype(np.float32)
+    want32 = a.astype(np.float32) * b
+    for out_dtype in (np.float32, np.float16):
+        out = poisoned(shape, out_dtype)
+        rt.plan_map([I("in", 0), I("in", 1), I("mul")], [dev(a), dev(b)], out).launch(sync=True)
+        assert_array_equal(out.to_host(), want32.astype(out_dtype))
+
+
+def test_map_rejects_malformed_programs(ctx):
+    x = dev(np.ones(64, np.float32))
+    out = poisoned((64,), np.float32)
+    bad = {
+        "underflow": [I("in", 0), I("add")],
+        "leaves 2": [I("in", 0), I("in", 0)],
+        "deeper": [I("in", 0)] * 5 + [I("add")] * 4,
+        "operand 1": [I("in", 1)],
+    }
+    for what, prog in bad.items():
+        with pytest.raises(rt.HcRuntimeError, match=what):
+            rt.plan_map(prog, [x], out).launch(sync=True)
+    with pytest.raises(rt.HcRuntimeError, match="instructions"):
+        rt.plan_map([I("in", 0)] + [I("neg")] * 32, [x], out).launch(sync=True)
+    prog = (rt.MapInstr * 1)()
+    prog[0].op = 99
+    ptrs, tys, lds = (C.c_void_p * 1)(x.ptr), (C.c_int * 1)(0), (C.c_size_t * 1)(64)
+    assert rt.hcamdLaunchMap(ctx.queue, prog, 1, ptrs, tys, lds, 1, out.ptr, 0, 64, 1, 64) == 1
+    with pytest.raises(rt.HcRuntimeError, match="unknown opcode"):
+        ctx.check(1, "hcamdLaunchMap")
+    assert (out.to_host().view(np.uint32) == POISON32).all()      # nothing was launched
+    # empty windows are not an error
+    rt.plan_map([I("in", 0)], [_view(x, 0)], _view(out, 0)).launch(sync=True)
+
+
+def test_map_full_benchmark_size_fma(ctx):
+    a, b, c = cf.inputs_c2()
+    d = rt.DeviceArray(a.shape, np.float16)
+    rt.plan_map(FMA_PROGRAM, [dev(a), dev(b), dev(c)], d).launch(sync=True)
+    assert rt.last_kernel_name() == "hcamd_map_flat"
+    assert_array_equal(d.to_host().view(np.uint16), cf.np_fma_f16(a, b, c).view(np.uint16))
 
 
 # ---------------------------------------------------------------------------

@@ -117,8 +117,82 @@ def test_vector_add_binds_to_add_f32(ctx):
     a2 = FakeDev((n,), "float32")
     (p2,) = vadd.plan(a2, b, c, ctx=ctx)
     assert p2.args[1] == a2.ptr and len(vadd._cache) == 1
+    # fp16 arrays: no dedicated kernel, the fused map runs "add, round to fp16"
+    (p3,) = vadd.plan(*(FakeDev((n,), "float16") for _ in range(3)), ctx=ctx)
+    assert p3.fn is rt.hcamdLaunchMap
+    assert map_program(p3) == [("in", 0, 0.0), ("in", 1, 0.0), ("add", 0, 0.0), ("r16", 0, 0.0)]
     with pytest.raises(NoNativeKernel):
-        vadd.plan(*(FakeDev((n,), "float16") for _ in range(3)), ctx=ctx)
+        vadd.plan(*(FakeDev((n,), "int32") for _ in range(3)), ctx=ctx)
+
+
+def map_program(plan):
+    """(opname, arg, imm) triples of a hcamdLaunchMap plan."""
+    names = {v: k for k, v in rt.MAP_OPS.items()}
+    prog, n = plan.args[1], plan.args[2]
+    return [(names[prog[i].op], prog[i].arg, prog[i].imm) for i in range(n)]
+
+
+def stack_depth(program):
+    sp = deepest = 0
+    for name, _, _ in program:
+        code = rt.MAP_OPS[name]
+        sp += 1 if code <= 2 else (-1 if code <= 10 else 0)
+        deepest = max(deepest, sp)
+    assert sp == 1
+    return deepest
+
+
+def test_elementwise_expressions_compile_to_postfix_programs(ctx):
+    N = sym.N
+    f = np.float32
+
+    def kern(expr):
+        @kernel(work_shape=N, group_shape=256)
+        def k(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], c: Buffer[N, DT],
+              out: Buffer[N, DT]):
+            o, g = gr.work_offset[0], gr.shape[0]
+            gr.store(out[o:], expr(gr.load(a[o:], shape=g), gr.load(b[o:], shape=g),
+                                   gr.load(c[o:], shape=g)))
+        return k
+
+    arrs = [FakeDev((1000,), "float32") for _ in range(4)]
+    # constants fold into immediates; a reversed immediate form where the
+    # constant is on the left
+    (p,) = kern(lambda a, b, c: (2.0 - a) * b / 4).plan(*arrs, ctx=ctx)
+    assert map_program(p) == [("in", 0, 0.0), ("rsubi", 0, 2.0), ("in", 1, 0.0),
+                              ("mul", 0, 0.0), ("divi", 0, 4.0)]
+    assert p.args[6] == 2 and p.args[10:] == (1, 1000)        # two operands, 1 x 1000
+    # the deeper operand goes first: a - (b*c + a/b) evaluates the right side,
+    # then a, then "reversed subtract"
+    (p,) = kern(lambda a, b, c: a - (b * c + a / b)).plan(*arrs, ctx=ctx)
+    prog = map_program(p)
+    assert prog[-1][0] == "rsub" and prog[-2][0] == "in" and stack_depth(prog) == 3
+    assert p.args[3][prog[-2][1]] == arrs[0].ptr       # operands are numbered by first use
+    # ufuncs, clip, maximum with NaN propagation left to the kernel
+    (p,) = kern(lambda a, b, c: np.clip(np.exp(-np.abs(a)) + np.maximum(b, c), 0, 6)).plan(
+        *arrs, ctx=ctx)
+    assert [i[0] for i in map_program(p)] == ["in", "in", "max", "in", "abs", "neg", "exp",
+                                              "add", "maxi", "mini"]
+    # mixed storage: fp16 operands, fp32 math, fp16 result -> one rounding, at the store
+    half = [FakeDev((1000,), "float16") for _ in range(4)]
+    (p,) = kern(lambda a, b, c: (a.astype(f) * b.astype(f) - c.astype(f)).astype(np.float16)
+                ).plan(*half, ctx=ctx)
+    assert [i[0] for i in map_program(p)] == ["in", "in", "mul", "in", "sub", "r16"]
+    assert list(p.args[4][:3]) == [rt.F16] * 3 and p.args[8] == rt.F16
+    # arithmetic on fp16 tiles rounds after every operation, and a Python
+    # scalar is first rounded to fp16 like NumPy does
+    (p,) = kern(lambda a, b, c: a * 0.1 + b).plan(*half, ctx=ctx)
+    assert map_program(p) == [("in", 0, 0.0), ("muli", 0, float(np.float32(np.float16(0.1)))),
+                              ("r16", 0, 0.0), ("in", 1, 0.0), ("add", 0, 0.0), ("r16", 0, 0.0)]
+    # too deep for the four-entry stack: a balanced tree over 16 leaves
+    def deep(a, b, c):
+        l = [a, b, c, a * 2, b * 2, c * 2, a * 3, b * 3, c * 3, a * 4, b * 4, c * 4, a * 5, b * 5,
+             c * 5, a * 6]
+        while len(l) > 1:
+            l = [x / y for x, y in zip(l[::2], l[1::2])]
+        return l[0]
+    with pytest.raises(NoNativeKernel, match="stack"):
+        kern(deep).plan(*arrs, ctx=ctx)
 
 
 def test_fused_multiply_add_binds_to_fma_f16(ctx):
@@ -138,7 +212,8 @@ def test_fused_multiply_add_binds_to_fma_f16(ctx):
     assert p.args == (ctx.queue, arrs[0].ptr, 8193, arrs[1].ptr, 8193, arrs[2].ptr, 8193,
                       arrs[3].ptr, 8193, 8191, 8193)
 
-    # without the fp32 casts the arithmetic would round in fp16: no native kernel
+    # without the fp32 casts the arithmetic rounds to fp16 after the multiply as
+    # well: not the fma kernel, but the fused map with an extra rounding step
     @kernel(work_shape=(R, Cc))
     def fma_half(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT],
                  c: Buffer[R, Cc, DT], d: Buffer[R, Cc, DT]):
@@ -146,8 +221,9 @@ def test_fused_multiply_add_binds_to_fma_f16(ctx):
         ta, tb, tc = (gr.load(v[x:, y:], shape=gr.shape) for v in (a, b, c))
         gr.store(d[x:, y:], ta * tb + tc)
 
-    with pytest.raises(NoNativeKernel):
-        fma_half.plan(*arrs, ctx=ctx)
+    (p,) = fma_half.plan(*arrs, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchMap
+    assert [i[0] for i in map_program(p)] == ["in", "in", "mul", "r16", "in", "add", "r16"]
 
 
 def test_softmax_of_the_reference_example_binds_to_softmax_f32(ctx):
@@ -253,7 +329,7 @@ def test_bodies_without_a_native_kernel_fail_loudly(ctx):
     @kernel(work_shape=N, group_shape=64)
     def scaled(gr: CurrentGroup, a: Buffer[N, DT], c: Buffer[N, DT]):
         o = gr.work_offset[0]
-        gr.store(c[o:], gr.load(a[o:], shape=gr.shape[0]) * 3.0)      # no such kernel
+        gr.store(c[o:], (gr.load(a[o:], shape=gr.shape[0]) * 3.0).sum())   # a reduction
 
     @kernel(work_shape=N, group_shape=64)
     def nothing(gr: CurrentGroup, a: Buffer[N, DT], c: Buffer[N, DT]):
