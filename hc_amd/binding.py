@@ -390,6 +390,16 @@ def _round_to(value: float, dtype: str) -> float:
     return float(np.float16(value)) if dtype == "float16" else float(np.float32(value))
 
 
+def _leaf(t: Tile):
+    """The load behind t if pushing t is just reading an operand: a load, or a
+    load widened to fp32 (no rounding involved)."""
+    if _is(t, "load"):
+        return t
+    if _is(t, "astype", 1) and t.dtype_name == "float32" and _is(t.args[0], "load"):
+        return t.args[0]
+    return None
+
+
 class _MapCompiler:
     """Sethi-Ullman ordering: the operand that needs the deeper stack is
     evaluated first, constants become immediates, so an expression with up to
@@ -434,6 +444,8 @@ class _MapCompiler:
             a, b = t.args
             if _const(a) or _const(b):
                 n = self.need(b if _const(a) else a)
+            elif _leaf(b) is not None or _leaf(a) is not None:
+                n = self.need(a if _leaf(b) is not None else b)
             else:
                 na, nb = self.need(a), self.need(b)
                 n = max(na, nb) if na != nb else na + 1
@@ -470,6 +482,12 @@ class _MapCompiler:
             elif _const(a):
                 self.emit(b, out)
                 out.append((rev + "i", 0, _round_to(a.attrs["value"], t.dtype_name)))
+            elif _leaf(b) is not None:              # operand forms: one dispatch, no push
+                self.emit(a, out)
+                out.append((fwd + "_in", self.operand(_leaf(b)), 0.0))
+            elif _leaf(a) is not None:
+                self.emit(b, out)
+                out.append((rev + "_in", self.operand(_leaf(a)), 0.0))
             elif self.need(a) >= self.need(b):
                 self.emit(a, out)
                 self.emit(b, out)

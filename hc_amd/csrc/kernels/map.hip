@@ -77,7 +77,17 @@ enum : uint32_t {
   OP_LOG = 24,
   OP_TANH = 25,
   OP_R16 = 26, // round to fp16 and back
-  OP_COUNT = 27,
+  // top = top op operand `arg` (a binary operation whose right side is an
+  // operand: one dispatch instead of two)
+  OP_ADD_IN = 27,
+  OP_SUB_IN = 28,
+  OP_MUL_IN = 29,
+  OP_DIV_IN = 30,
+  OP_MAX_IN = 31,
+  OP_MIN_IN = 32,
+  OP_RSUB_IN = 33, // operand - top
+  OP_RDIV_IN = 34, // operand / top
+  OP_COUNT = 35,
 };
 
 struct Instr {
@@ -193,6 +203,23 @@ template <int SP, int OP> __device__ __forceinline__ void do_imm(Stack &r, float
       r.st[SP - 1][e] = binary<B>(r.st[SP - 1][e], imm);
   }
 }
+template <int SP, int OP>
+__device__ __forceinline__ void do_operand(Stack &r, const Raw &raw, uint32_t f16_mask,
+                                           uint32_t arg) {
+  if constexpr (SP >= 1) {
+    constexpr int B = OP - OP_ADD_IN + OP_ADD; // the plain binary operation
+    float t[kN];
+    switch (arg) {
+    case 0: unpack(raw, 0, f16_mask & 1, t); break;
+    case 1: unpack(raw, 1, f16_mask & 2, t); break;
+    case 2: unpack(raw, 2, f16_mask & 4, t); break;
+    default: unpack(raw, 3, f16_mask & 8, t); break;
+    }
+#pragma unroll
+    for (int e = 0; e < kN; ++e)
+      r.st[SP - 1][e] = binary<B>(r.st[SP - 1][e], t[e]);
+  }
+}
 template <int SP, int OP> __device__ __forceinline__ void do_unary(Stack &r) {
   if constexpr (SP >= 1) {
 #pragma unroll
@@ -263,6 +290,19 @@ __device__ __forceinline__ int step(Stack &r, const Raw &raw, uint32_t f16_mask,
     HCAMD_UN(OP_TANH)
     HCAMD_UN(OP_R16)
 #undef HCAMD_UN
+#define HCAMD_OPND(OP)                                                         \
+  case OP:                                                                     \
+    do_operand<SP, OP>(r, raw, f16_mask, arg);                                 \
+    return SP;
+    HCAMD_OPND(OP_ADD_IN)
+    HCAMD_OPND(OP_SUB_IN)
+    HCAMD_OPND(OP_MUL_IN)
+    HCAMD_OPND(OP_DIV_IN)
+    HCAMD_OPND(OP_MAX_IN)
+    HCAMD_OPND(OP_MIN_IN)
+    HCAMD_OPND(OP_RSUB_IN)
+    HCAMD_OPND(OP_RDIV_IN)
+#undef HCAMD_OPND
   default:
     return SP;
   }

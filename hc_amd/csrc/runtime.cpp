@@ -899,7 +899,7 @@ void mapStackEffect(unsigned op, int &pops, int &pushes) {
     pops = 0, pushes = 1;
   } else if (op >= HCAMD_MAP_ADD && op <= HCAMD_MAP_RDIV) {
     pops = 2, pushes = 1;
-  } else if (op >= HCAMD_MAP_ADDI && op <= HCAMD_MAP_R16) {
+  } else if (op >= HCAMD_MAP_ADDI && op <= HCAMD_MAP_RDIV_IN) {
     pops = 1, pushes = 1;
   } else {
     pops = -1, pushes = 0;
@@ -940,7 +940,10 @@ int hcamdLaunchMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
       dev->report("hcamdLaunchMap: unknown opcode %u at %zu", prog[i].op, i);
       return 1;
     }
-    if (prog[i].op == HCAMD_MAP_IN && prog[i].arg >= nInputs) {
+    const bool readsOperand =
+        prog[i].op == HCAMD_MAP_IN ||
+        (prog[i].op >= HCAMD_MAP_ADD_IN && prog[i].op <= HCAMD_MAP_RDIV_IN);
+    if (readsOperand && prog[i].arg >= nInputs) {
       dev->report("hcamdLaunchMap: operand %u at %zu (only %zu given)",
                   prog[i].arg, i, nInputs);
       return 1;

@@ -386,7 +386,9 @@ def plan_fma_f16(a, b, c, d) -> Plan:
 MAP_OPS = {"in": 1, "const": 2, "add": 3, "sub": 4, "mul": 5, "div": 6, "max": 7, "min": 8,
            "rsub": 9, "rdiv": 10, "addi": 11, "subi": 12, "muli": 13, "divi": 14, "maxi": 15,
            "mini": 16, "rsubi": 17, "rdivi": 18, "neg": 19, "abs": 20, "sqrt": 21, "rint": 22,
-           "exp": 23, "log": 24, "tanh": 25, "r16": 26}
+           "exp": 23, "log": 24, "tanh": 25, "r16": 26, "add_in": 27, "sub_in": 28,
+           "mul_in": 29, "div_in": 30, "max_in": 31, "min_in": 32, "rsub_in": 33,
+           "rdiv_in": 34}
 MAP_MAX_INPUTS, MAP_MAX_INSTRS, MAP_STACK_DEPTH = 4, 32, 4
 F32, F16 = 0, 1
 

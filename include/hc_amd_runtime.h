@@ -277,14 +277,22 @@ enum HcamdMapOp {
   HCAMD_MAP_EXP = 23,
   HCAMD_MAP_LOG = 24,
   HCAMD_MAP_TANH = 25,
-  HCAMD_MAP_R16 = 26
+  HCAMD_MAP_R16 = 26,
+  HCAMD_MAP_ADD_IN = 27, /* top = top op operand `arg` */
+  HCAMD_MAP_SUB_IN = 28,
+  HCAMD_MAP_MUL_IN = 29,
+  HCAMD_MAP_DIV_IN = 30,
+  HCAMD_MAP_MAX_IN = 31,
+  HCAMD_MAP_MIN_IN = 32,
+  HCAMD_MAP_RSUB_IN = 33, /* operand - top */
+  HCAMD_MAP_RDIV_IN = 34  /* operand / top */
 };
 #define HCAMD_MAP_MAX_INPUTS 4
 #define HCAMD_MAP_MAX_INSTRS 32
 #define HCAMD_MAP_STACK_DEPTH 4
 typedef struct HcamdMapInstr {
   uint16_t op;  /* HcamdMapOp */
-  uint16_t arg; /* operand index for HCAMD_MAP_IN */
+  uint16_t arg; /* operand index for HCAMD_MAP_IN and the *_IN forms */
   float imm;    /* HCAMD_MAP_CONST and the *I forms */
 } HcamdMapInstr;
 int hcamdLaunchMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,

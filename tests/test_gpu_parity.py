@@ -381,6 +381,10 @@ def test_map_every_operation_against_numpy(ctx):
             out = poisoned((n,), f)
             rt.plan_map([I("in", 0), I("in", 1), I(name)], [dx, dy], out).launch(sync=True)
             assert_same_floats(out.to_host(), want.astype(f), name)
+        for name, want in exact.items():                 # operand forms of the same
+            out = poisoned((n,), f)
+            rt.plan_map([I("in", 0), I(name + "_in", 1)], [dx, dy], out).launch(sync=True)
+            assert_same_floats(out.to_host(), want.astype(f), name + "_in")
         imm = {"addi": x + k, "subi": x - k, "muli": x * k, "divi": x / k,
                "maxi": np.maximum(x, k), "mini": np.minimum(x, k), "rsubi": k - x,
                "rdivi": k / x}

@@ -120,7 +120,7 @@ def test_vector_add_binds_to_add_f32(ctx):
     # fp16 arrays: no dedicated kernel, the fused map runs "add, round to fp16"
     (p3,) = vadd.plan(*(FakeDev((n,), "float16") for _ in range(3)), ctx=ctx)
     assert p3.fn is rt.hcamdLaunchMap
-    assert map_program(p3) == [("in", 0, 0.0), ("in", 1, 0.0), ("add", 0, 0.0), ("r16", 0, 0.0)]
+    assert map_program(p3) == [("in", 0, 0.0), ("add_in", 1, 0.0), ("r16", 0, 0.0)]
     with pytest.raises(NoNativeKernel):
         vadd.plan(*(FakeDev((n,), "int32") for _ in range(3)), ctx=ctx)
 
@@ -136,7 +136,7 @@ def stack_depth(program):
     sp = deepest = 0
     for name, _, _ in program:
         code = rt.MAP_OPS[name]
-        sp += 1 if code <= 2 else (-1 if code <= 10 else 0)
+        sp += 1 if code <= 2 else (-1 if code <= 10 else 0)     # the rest: one in, one out
         deepest = max(deepest, sp)
     assert sp == 1
     return deepest
@@ -159,35 +159,43 @@ def test_elementwise_expressions_compile_to_postfix_programs(ctx):
     # constants fold into immediates; a reversed immediate form where the
     # constant is on the left
     (p,) = kern(lambda a, b, c: (2.0 - a) * b / 4).plan(*arrs, ctx=ctx)
-    assert map_program(p) == [("in", 0, 0.0), ("rsubi", 0, 2.0), ("in", 1, 0.0),
-                              ("mul", 0, 0.0), ("divi", 0, 4.0)]
+    assert map_program(p) == [("in", 0, 0.0), ("rsubi", 0, 2.0), ("mul_in", 1, 0.0),
+                              ("divi", 0, 4.0)]
     assert p.args[6] == 2 and p.args[10:] == (1, 1000)        # two operands, 1 x 1000
-    # the deeper operand goes first: a - (b*c + a/b) evaluates the right side,
-    # then a, then "reversed subtract"
+    # an operand on one side of a binary operation is read by the operation
+    # itself: a - (b*c + a/b) evaluates the right side, then "a minus top"
     (p,) = kern(lambda a, b, c: a - (b * c + a / b)).plan(*arrs, ctx=ctx)
     prog = map_program(p)
-    assert prog[-1][0] == "rsub" and prog[-2][0] == "in" and stack_depth(prog) == 3
-    assert p.args[3][prog[-2][1]] == arrs[0].ptr       # operands are numbered by first use
+    assert [i[0] for i in prog] == ["in", "mul_in", "in", "div_in", "add", "rsub_in"]
+    assert stack_depth(prog) == 2
+    assert p.args[3][prog[-1][1]] == arrs[0].ptr       # operands are numbered by first use
+    # the deeper side goes first: (a*b - c*a) / (exp(a) / (b*c + a*a))
+    (p,) = kern(lambda a, b, c: (a * b - c * a) / (np.exp(a) / (b * c + a * a))).plan(
+        *arrs, ctx=ctx)
+    prog = map_program(p)
+    assert [i[0] for i in prog] == ["in", "mul_in", "in", "mul_in", "sub",        # numerator
+                                    "in", "mul_in", "in", "mul_in", "add",        # b*c + a*a
+                                    "in", "exp", "rdiv", "div"]
+    assert stack_depth(prog) == 3
     # ufuncs, clip, maximum with NaN propagation left to the kernel
     (p,) = kern(lambda a, b, c: np.clip(np.exp(-np.abs(a)) + np.maximum(b, c), 0, 6)).plan(
         *arrs, ctx=ctx)
-    assert [i[0] for i in map_program(p)] == ["in", "in", "max", "in", "abs", "neg", "exp",
-                                              "add", "maxi", "mini"]
+    assert [i[0] for i in map_program(p)] == ["in", "abs", "neg", "exp", "in", "max_in", "add",
+                                              "maxi", "mini"]
     # mixed storage: fp16 operands, fp32 math, fp16 result -> one rounding, at the store
     half = [FakeDev((1000,), "float16") for _ in range(4)]
     (p,) = kern(lambda a, b, c: (a.astype(f) * b.astype(f) - c.astype(f)).astype(np.float16)
                 ).plan(*half, ctx=ctx)
-    assert [i[0] for i in map_program(p)] == ["in", "in", "mul", "in", "sub", "r16"]
+    assert [i[0] for i in map_program(p)] == ["in", "mul_in", "sub_in", "r16"]
     assert list(p.args[4][:3]) == [rt.F16] * 3 and p.args[8] == rt.F16
     # arithmetic on fp16 tiles rounds after every operation, and a Python
     # scalar is first rounded to fp16 like NumPy does
     (p,) = kern(lambda a, b, c: a * 0.1 + b).plan(*half, ctx=ctx)
     assert map_program(p) == [("in", 0, 0.0), ("muli", 0, float(np.float32(np.float16(0.1)))),
-                              ("r16", 0, 0.0), ("in", 1, 0.0), ("add", 0, 0.0), ("r16", 0, 0.0)]
-    # too deep for the four-entry stack: a balanced tree over 16 leaves
+                              ("r16", 0, 0.0), ("add_in", 1, 0.0), ("r16", 0, 0.0)]
+    # too deep for the four-entry stack: a balanced tree over 16 sub-expressions
     def deep(a, b, c):
-        l = [a, b, c, a * 2, b * 2, c * 2, a * 3, b * 3, c * 3, a * 4, b * 4, c * 4, a * 5, b * 5,
-             c * 5, a * 6]
+        l = [np.abs(v) for v in (a, b, c) * 5 + (a,)]
         while len(l) > 1:
             l = [x / y for x, y in zip(l[::2], l[1::2])]
         return l[0]
@@ -223,7 +231,7 @@ def test_fused_multiply_add_binds_to_fma_f16(ctx):
 
     (p,) = fma_half.plan(*arrs, ctx=ctx)
     assert p.fn is rt.hcamdLaunchMap
-    assert [i[0] for i in map_program(p)] == ["in", "in", "mul", "r16", "in", "add", "r16"]
+    assert [i[0] for i in map_program(p)] == ["in", "mul_in", "r16", "add_in", "r16"]
 
 
 def test_softmax_of_the_reference_example_binds_to_softmax_f32(ctx):
