@@ -13,6 +13,8 @@ structurally:
     map        store(f(load a, load b, ...)) for any other elementwise f over up to
                four fp32 / fp16 operands: compiled to a postfix program for the
                fused map kernel
+    sum        atomic_ref(r)[i] += f(load a, ...).sum(): the same programs, reduced
+               with one fp32 atomic addition per workgroup
 
 Every load and the store must walk their buffers tile by tile: the start along a
 dimension is either 0 or group_id[i] * tile_extent, so that the tiles of all
@@ -534,12 +536,98 @@ def match_map(dst_view, value, n_groups):
     return make
 
 
-def bind(stores, n_groups):
-    """stores: list of (BufferView, Tile) from one traced execution.  Returns a
-    list of plan makers; raises NoNativeKernel when nothing matches."""
-    if not stores:
+# ---------------------------------------------------------------------------
+# atomic_ref(result)[i] += <elementwise expression>.sum()
+# ---------------------------------------------------------------------------
+def _merge_strided_loads(terms, n_groups):
+    """The idiom of python/hckernel/tests/test_examples.py:50-71: a group adds up
+    N tiles of `size` elements that start at g*N*size + i*size.  Together the N
+    loads tile the window [g*N*size, (g+1)*N*size); they are replaced by one
+    load of N*size elements.  Returns the new list of terms."""
+    loads = [t for t in terms if _is(t, "load") and len(t.shape) == 1]
+    rest = [t for t in terms if not (_is(t, "load") and len(t.shape) == 1)]
+    by_key = {}
+    for t in loads:
+        v = t.attrs["view"]
+        st = v.starts[0]
+        by_key.setdefault((v.base.index, tuple(st.coeffs), t.shape[0]), []).append(t)
+    out = list(rest)
+    for (_, coeffs, size), group in by_key.items():
+        consts = sorted(t.attrs["view"].starts[0].const for t in group)
+        nz = [c for c in coeffs if c]
+        n = len(group)
+        if n > 1 and len(nz) == 1 and nz[0] == n * size and \
+                consts == [i * size for i in range(n)]:
+            v = group[0].attrs["view"]
+            merged = BufferView(v.base, (Affine(0, coeffs),))
+            out.append(Tile("load", (), (n * size,), group[0].dtype_name, view=merged))
+        else:
+            out.extend(group)
+    return out
+
+
+def match_sum(proxy, index, value, n_groups):
+    if proxy.dtype_name != "float32":
+        raise NoNativeKernel(f"atomic accumulation into {proxy.name}: only float32 cells have "
+                             "a native kernel")
+    if not (value.op == "sum" and len(value.args) == 1 and
+            value.attrs.get("axes") == tuple(range(len(value.args[0].shape)))):
+        raise NoNativeKernel(f"atomic accumulation into {proxy.name}: the value must be "
+                             "`<tile expression>.sum()` over all axes")
+    n_cells = 1
+    for s in proxy.shape:
+        n_cells *= s
+    if not 0 <= index < n_cells:
+        raise NoNativeKernel(f"atomic accumulation into {proxy.name}: index {index} out of range")
+    # sum(x + y) = sum(x) + sum(y): every term of a top-level sum gets its own
+    # pass, which also covers tiles that were added up one by one
+    terms: list = []
+    _flatten_sum(value.args[0], terms)
+    terms = [t for t in terms if not _const(t, 0)]
+    terms = _merge_strided_loads(terms, n_groups)
+    if not terms:
+        raise NoNativeKernel("nothing to accumulate")
+    makers = []
+    for term in terms:
+        comp = _MapCompiler(n_groups)
+        if not comp.supported(term):
+            raise NoNativeKernel(f"atomic accumulation into {proxy.name}: {term!r} is not an "
+                                 "elementwise expression over fp32 / fp16 loads")
+        if comp.need(term) > rt.MAP_STACK_DEPTH:
+            raise NoNativeKernel("elementwise expression needs an evaluation stack deeper than "
+                                 f"{rt.MAP_STACK_DEPTH}")
+        program: list = []
+        comp.emit(term, program)
+        if len(program) > rt.MAP_MAX_INSTRS or len(comp.inputs) > rt.MAP_MAX_INPUTS or \
+                not comp.inputs:
+            raise NoNativeKernel("elementwise expression too large for the map kernel")
+        wins = [window_of(t.attrs["view"], t.shape, n_groups) for _, _, t in comp.inputs]
+        w = _check_same_window(wins)
+        if len(w.extent) > 2:
+            raise NoNativeKernel("only 1-D and 2-D buffers have native kernels")
+        types = [rt.F16 if t.dtype_name == "float16" else rt.F32 for _, _, t in comp.inputs]
+
+        def make(mem, ctx, program=program, wins=wins, w=w, types=types):
+            arrays = [_Arr(_sub(mem[x.buffer], w.extent), ctx) for x in wins]
+            return [rt.plan_map_sum(program, arrays, _Arr(mem[proxy.index], ctx), index, types)]
+        make.program = program
+        makers.append(make)
+    return makers
+
+
+def bind(stores, n_groups, atomics=()):
+    """stores: list of (BufferView, Tile) from one traced execution; atomics:
+    list of (BufferProxy, index, Tile) atomic additions.  Returns a list of plan
+    makers; raises NoNativeKernel when nothing matches."""
+    if not stores and not atomics:
         raise NoNativeKernel("the kernel body stores nothing")
     try:
+        if atomics:
+            if stores:
+                raise NoNativeKernel("a body that both stores tiles and accumulates "
+                                     "atomically has no native kernel")
+            return [mk for proxy, index, value in atomics
+                    for mk in match_sum(proxy, index, value, n_groups)]
         q = match_quantize(stores, n_groups)
         if q is not None:
             return [q]

@@ -462,3 +462,78 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_map_strided(
       store_elem(a.out, (a.f16_mask >> 8) & 1, row * a.ldo + col, r.st[0][e]);
   }
 }
+
+// ---------------------------------------------------------------------------
+// Map-reduce: *result += sum over the window of f(in0[i], ...).  Same programs,
+// same operand handling; the output pointer of the argument block is the fp32
+// accumulator cell.  A lane adds up the values of its own elements in fp32, a
+// wave folds its lanes with DPP, the four waves meet in LDS, and one lane per
+// workgroup issues a single hardware fp32 atomic add; the grid is capped so that
+// at most a few thousand atomics reach the cell.  The order of the additions
+// differs from run to run: the result is a correctly computed fp32 sum, not a
+// bit-reproducible one.
+// ---------------------------------------------------------------------------
+namespace {
+__device__ __forceinline__ void finish_sum(float acc, float *cell) {
+  __shared__ float slots[kThreads / kWave];
+  const float total = group_reduce<SumOp, kThreads / kWave>(acc, slots);
+  if (threadIdx.x == 0)
+    unsafeAtomicAdd(cell, total);
+}
+} // namespace
+
+extern "C" __global__ __launch_bounds__(256)
+__attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcamd_map_sum_flat(
+    const MapArgs a, const uint32_t n_in) {
+  const size_t n = a.cols;
+  const size_t n_chunks = n / 8;
+  const size_t stride = (size_t)gridDim.x * kThreads;
+  const size_t passes = (n_chunks + stride - 1) / stride; // same for every lane
+  size_t c = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  float acc = 0.0f;
+  Raw raw;
+  Stack r;
+  for (size_t p = 0; p < passes; ++p, c += stride) {
+    if (c < n_chunks)
+      load_raw(a, n_in, c, n_chunks, raw);
+    run_program(a, raw, a.f16_mask, r);
+    if (c < n_chunks) {
+#pragma unroll
+      for (int e = 0; e < kN; ++e)
+        acc += r.st[0][e];
+    }
+  }
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == kThreads - 1 && n_chunks * 8 < n) {
+    gather(a, n_in, raw, [&](int, int e, size_t &off) {
+      off = n_chunks * 8 + e;
+      return off < n;
+    });
+    run_program(a, raw, 0, r);
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      if (n_chunks * 8 + e < n)
+        acc += r.st[0][e];
+  }
+  finish_sum(acc, static_cast<float *>(a.out));
+}
+
+// Strided form: one workgroup per (row, run of 256 * kN columns).
+extern "C" __global__ __launch_bounds__(256) void hcamd_map_sum_strided(
+    const MapArgs a, const uint32_t n_in) {
+  const size_t row = blockIdx.y;
+  const size_t col0 = (size_t)blockIdx.x * (kThreads * kN) + threadIdx.x;
+  Raw raw;
+  gather(a, n_in, raw, [&](int i, int e, size_t &off) {
+    const size_t col = col0 + (size_t)e * kThreads;
+    off = row * a.ld[i] + col;
+    return col < a.cols;
+  });
+  Stack r;
+  run_program(a, raw, 0, r);
+  float acc = 0.0f;
+#pragma unroll
+  for (int e = 0; e < kN; ++e)
+    if (col0 + (size_t)e * kThreads < a.cols)
+      acc += r.st[0][e];
+  finish_sum(acc, static_cast<float *>(a.out));
+}

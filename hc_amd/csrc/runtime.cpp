@@ -907,28 +907,31 @@ void mapStackEffect(unsigned op, int &pops, int &pushes) {
 }
 } // namespace
 
-int hcamdLaunchMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
-                   const void *const *inputs, const int *inputTypes,
-                   const size_t *inputLd, size_t nInputs, void *out,
-                   int outType, size_t ldo, size_t rows,
-                   size_t cols) noexcept {
+namespace {
+// Shared by the map and the map-sum entry points.  `sum`: out is the fp32 cell
+// the sum of all results is added to; outType and ldo are not used.
+int launchMap(OlQueue q, bool sum, const HcamdMapInstr *prog, size_t nInstr,
+              const void *const *inputs, const int *inputTypes,
+              const size_t *inputLd, size_t nInputs, void *out, int outType,
+              size_t ldo, size_t rows, size_t cols) {
   auto *queue = static_cast<Queue *>(q);
   if (!queue)
     return 1;
   Device *dev = queue->device;
+  const char *who = sum ? "hcamdLaunchMapSum" : "hcamdLaunchMap";
   if (!prog || nInstr == 0 || nInstr > kMapMaxProg) {
-    dev->report("hcamdLaunchMap: program of %zu instructions (1..%zu allowed)",
+    dev->report("%s: program of %zu instructions (1..%zu allowed)", who,
                 nInstr, kMapMaxProg);
     return 1;
   }
   if (nInputs > kMapMaxIn || (nInputs && (!inputs || !inputTypes || !inputLd))) {
-    dev->report("hcamdLaunchMap: %zu operands (at most %zu)", nInputs,
+    dev->report("%s: %zu operands (at most %zu)", who, nInputs,
                 kMapMaxIn);
     return 1;
   }
   auto typeOk = [](int t) { return t == HCAMD_F32 || t == HCAMD_F16; };
   if (!typeOk(outType)) {
-    dev->report("hcamdLaunchMap: unsupported output type %d", outType);
+    dev->report("%s: unsupported output type %d", who, outType);
     return 1;
   }
   // The program must keep the stack within bounds and leave one value.
@@ -937,55 +940,55 @@ int hcamdLaunchMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
     int pops, pushes;
     mapStackEffect(prog[i].op, pops, pushes);
     if (pops < 0) {
-      dev->report("hcamdLaunchMap: unknown opcode %u at %zu", prog[i].op, i);
+      dev->report("%s: unknown opcode %u at %zu", who, prog[i].op, i);
       return 1;
     }
     const bool readsOperand =
         prog[i].op == HCAMD_MAP_IN ||
         (prog[i].op >= HCAMD_MAP_ADD_IN && prog[i].op <= HCAMD_MAP_RDIV_IN);
     if (readsOperand && prog[i].arg >= nInputs) {
-      dev->report("hcamdLaunchMap: operand %u at %zu (only %zu given)",
+      dev->report("%s: operand %u at %zu (only %zu given)", who,
                   prog[i].arg, i, nInputs);
       return 1;
     }
     if (sp < pops) {
-      dev->report("hcamdLaunchMap: stack underflow at %zu", i);
+      dev->report("%s: stack underflow at %zu", who, i);
       return 1;
     }
     sp += pushes - pops;
     if (sp > kMapDepth) {
-      dev->report("hcamdLaunchMap: stack deeper than %d at %zu", kMapDepth, i);
+      dev->report("%s: stack deeper than %d at %zu", who, kMapDepth, i);
       return 1;
     }
   }
   if (sp != 1) {
-    dev->report("hcamdLaunchMap: program leaves %d values, expected 1", sp);
+    dev->report("%s: program leaves %d values, expected 1", who, sp);
     return 1;
   }
   if (rows == 0 || cols == 0)
     return 0;
   if (!out) {
-    dev->report("hcamdLaunchMap: null pointer");
+    dev->report("%s: null pointer", who);
     return 1;
   }
   MapArgs a{};
-  bool dense = rows == 1 || ldo == cols;
-  bool aligned = aligned16(out);
-  if (rows > 1 && ldo < cols) {
-    dev->report("hcamdLaunchMap: leading dimension smaller than cols");
+  bool dense = sum || rows == 1 || ldo == cols;
+  bool aligned = sum || aligned16(out);
+  if (!sum && rows > 1 && ldo < cols) {
+    dev->report("%s: leading dimension smaller than cols", who);
     return 1;
   }
   for (size_t i = 0; i < nInputs; ++i) {
     if (!inputs[i]) {
-      dev->report("hcamdLaunchMap: null pointer");
+      dev->report("%s: null pointer", who);
       return 1;
     }
     if (!typeOk(inputTypes[i])) {
-      dev->report("hcamdLaunchMap: unsupported operand type %d", inputTypes[i]);
+      dev->report("%s: unsupported operand type %d", who, inputTypes[i]);
       return 1;
     }
     if (rows > 1 && inputLd[i] < cols) {
-      dev->report("hcamdLaunchMap: leading dimension smaller than cols");
+      dev->report("%s: leading dimension smaller than cols", who);
       return 1;
     }
     a.in[i] = inputs[i];
@@ -1007,10 +1010,14 @@ int hcamdLaunchMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
   if (dense && aligned && variantOf("map") != 1) {
     a.rows = 1;
     a.cols = rows * cols;
-    const size_t groups = std::max(ceilDiv(a.cols, kPerGroup), (size_t)1);
-    return launch1d(queue, "map", "hcamd_map_flat", groups, 256, args);
+    size_t groups = std::max(ceilDiv(a.cols, kPerGroup), (size_t)1);
+    if (sum) // persistent: one atomic per workgroup, at most 8 groups per CU
+      groups = std::min(groups, (size_t)computeUnitsOf(dev) * 8);
+    return launch1d(queue, "map", sum ? "hcamd_map_sum_flat" : "hcamd_map_flat",
+                    groups, 256, args);
   }
-  Kernel *k = builtinKernel(dev, "map", "hcamd_map_strided");
+  Kernel *k = builtinKernel(dev, "map",
+                            sum ? "hcamd_map_sum_strided" : "hcamd_map_strided");
   if (!k)
     return 1;
   a.cols = cols;
@@ -1021,13 +1028,31 @@ int hcamdLaunchMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
     for (size_t i = 0; i < nInputs; ++i)
       a.in[i] = static_cast<const char *>(inputs[i]) +
                 r0 * inputLd[i] * (inputTypes[i] == HCAMD_F16 ? 2 : 4);
-    a.out = static_cast<char *>(out) + r0 * ldo * esz_out;
+    a.out = sum ? out : static_cast<char *>(out) + r0 * ldo * esz_out;
     const size_t grid[3] = {ceilDiv(cols, kPerGroup), nr, 1};
     const size_t block[3] = {256, 1, 1};
     if (launch(queue, k, grid, block, args, 0))
       return 1;
   }
   return 0;
+}
+} // namespace
+
+int hcamdLaunchMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
+                   const void *const *inputs, const int *inputTypes,
+                   const size_t *inputLd, size_t nInputs, void *out,
+                   int outType, size_t ldo, size_t rows,
+                   size_t cols) noexcept {
+  return launchMap(q, false, prog, nInstr, inputs, inputTypes, inputLd, nInputs,
+                   out, outType, ldo, rows, cols);
+}
+
+int hcamdLaunchMapSum(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
+                      const void *const *inputs, const int *inputTypes,
+                      const size_t *inputLd, size_t nInputs, float *cell,
+                      size_t rows, size_t cols) noexcept {
+  return launchMap(q, true, prog, nInstr, inputs, inputTypes, inputLd, nInputs,
+                   cell, HCAMD_F32, cols, rows, cols);
 }
 
 int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,

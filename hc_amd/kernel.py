@@ -208,12 +208,15 @@ class GpuKernel:
                 proxies.append(BufferProxy(i, names[i] if i < len(names) else f"arg{i}",
                                            m.shape, m.strides, _array_dtype(a), a))
         group_obj = [CurrentGroup1, CurrentGroup2, CurrentGroup3][len(work) - 1](group, sg)
+        for p in proxies:
+            if isinstance(p, BufferProxy):
+                p.group = group_obj
         body = _resolve_symbols(self.func, subs)
         try:
             body(group_obj, *proxies)
         except TraceError as exc:
             raise NoNativeKernel(f"{self.func.__name__}: {exc}") from exc
-        return bind(group_obj.stores, n_groups)
+        return bind(group_obj.stores, n_groups, group_obj.atomics)
 
     def plan(self, *args, ctx=None):
         """Everything a call does short of launching: returns the list of

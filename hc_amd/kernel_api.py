@@ -40,8 +40,57 @@ def create_mapping(func):
     return Mapping(func)
 
 
+_ATOMIC_DONE = object()      # what `cell += v` leaves behind for the `ref[i] = ...` that follows
+
+
+class _AtomicCell:
+    def __init__(self, ref, index):
+        self.ref, self.index = ref, index
+
+    def __iadd__(self, value):
+        self.ref.record(self.index, value)
+        return _ATOMIC_DONE
+
+    def _unsupported(self, *_):
+        raise TraceError("only `atomic_ref(buffer)[i] += value` is supported on the GPU path")
+
+    __isub__ = __imul__ = __itruediv__ = __add__ = __radd__ = _unsupported
+
+
+class AtomicRef:
+    """`atomic_ref(buffer)`: element updates through it are atomic
+    (python/hckernel/kernel_api.py:450-451 returns the array itself because the
+    simulator runs the groups one after another).  Traced: `ref[i] += value`
+    records an atomic addition of `value` to element i."""
+
+    def __init__(self, proxy):
+        self.proxy = proxy
+
+    def __getitem__(self, index):
+        if isinstance(index, tuple) and len(index) == 1:
+            index = index[0]
+        if isinstance(index, Affine):
+            if not index.is_const:
+                raise TraceError("atomic updates of an element chosen by the group id have no "
+                                 "native kernel yet")
+            index = index.const
+        if not isinstance(index, (int, np.integer)):
+            raise TraceError("atomic_ref(buffer)[i]: i must be an integer")
+        return _AtomicCell(self, int(index))
+
+    def __setitem__(self, index, value):
+        if value is not _ATOMIC_DONE:
+            raise TraceError("only `atomic_ref(buffer)[i] += value` is supported on the GPU path")
+
+    def record(self, index, value):
+        group = getattr(self.proxy, "group", None)
+        if group is None:
+            raise TraceError("atomic_ref outside a kernel body")
+        group.atomics.append((self.proxy, index, Tile.wrap(value)))
+
+
 def atomic_ref(a):
-    return a
+    return AtomicRef(a) if isinstance(a, BufferProxy) else a
 
 
 class Buffer(type):
@@ -472,6 +521,7 @@ class CurrentGroup:
         self._id = tuple(Affine(0, [1 if j == i else 0 for j in range(rank)])
                          for i in range(rank))
         self.stores = []          # (BufferView, Tile) in program order
+        self.atomics = []         # (BufferProxy, element index, Tile) atomic additions
 
     @property
     def id(self):

@@ -102,6 +102,8 @@ class MapInstr(C.Structure):
 
 hcamdLaunchMap = _sig(_rt, "hcamdLaunchMap", _int, _vp, C.POINTER(MapInstr), _sz,
                       C.POINTER(_vp), C.POINTER(_int), _sz_p, _sz, _vp, _int, _sz, _sz, _sz)
+hcamdLaunchMapSum = _sig(_rt, "hcamdLaunchMapSum", _int, _vp, C.POINTER(MapInstr), _sz,
+                         C.POINTER(_vp), C.POINTER(_int), _sz_p, _sz, _vp, _sz, _sz)
 hcamdConvertPyArray = _sig(_py, "hcamdConvertPyArray", _int, C.py_object, _int, _vp,
                            _sz_p, C.c_char_p, _sz)
 hcamdConvertPyInt64 = _sig(_py, "hcamdConvertPyInt64", _int, C.py_object,
@@ -422,6 +424,42 @@ def plan_map(program, inputs, out, types=None) -> Plan:
     return Plan(ctx, hcamdLaunchMap,
                 (ctx.queue, prog, len(program), ptrs, tys, lds, n_in, ms[-1].ptr, types[-1],
                  geo[-1][2], rows, cols), "hcamdLaunchMap", (arrays, prog, ptrs, tys, lds))
+
+
+def plan_map_sum(program, inputs, cell, index: int = 0, types=None) -> Plan:
+    """cell[index] += sum of f(inputs...) over all elements (fp32 atomic
+    accumulation); `cell` is an fp32 array, the inputs are as for plan_map."""
+    arrays = list(inputs)
+    ctx = _ctx_of(*arrays, cell)
+    ms = [as_memref(v) for v in arrays]
+    mc = as_memref(cell)
+    _expect(mc, 4, "cell")
+    n_cells = 1
+    for s in mc.shape:
+        n_cells *= s
+    if not mc.is_contiguous() or not 0 <= index < n_cells:
+        raise HcRuntimeError("map_sum: the accumulator must be a contiguous fp32 array and "
+                             "the index inside it")
+    geo = [_rows_cols(m) for m in ms]
+    rows, cols = geo[0][0], geo[0][1]
+    if any(g[0] != rows or g[1] != cols for g in geo):
+        raise HcRuntimeError("map_sum: shape mismatch")
+    if types is None:
+        types = []
+        for m in ms:
+            if m.itemsize not in (2, 4):
+                raise HcRuntimeError(f"map_sum: element size {m.itemsize} (fp32 and fp16 only)")
+            types.append(F16 if m.itemsize == 2 else F32)
+    n_in = len(arrays)
+    prog = (MapInstr * max(len(program), 1))()
+    for i, (name, arg, imm) in enumerate(program):
+        prog[i].op, prog[i].arg, prog[i].imm = MAP_OPS[name], int(arg), float(imm)
+    ptrs = (_vp * n_in)(*[m.ptr for m in ms])
+    tys = (_int * n_in)(*types[:n_in])
+    lds = (_sz * n_in)(*[g[2] for g in geo])
+    return Plan(ctx, hcamdLaunchMapSum,
+                (ctx.queue, prog, len(program), ptrs, tys, lds, n_in, mc.ptr + 4 * index,
+                 rows, cols), "hcamdLaunchMapSum", (arrays, cell, prog, ptrs, tys, lds))
 
 
 def plan_softmax_f32(x, y) -> Plan:

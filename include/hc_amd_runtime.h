@@ -301,6 +301,17 @@ int hcamdLaunchMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
                    int outType, size_t ldo, size_t rows,
                    size_t cols) HCAMD_NOEXCEPT;
 
+/* Map-reduce: *cell += sum over the window of f(in_0 .. in_{n-1}), fp32, with
+ * one hardware atomic add per workgroup.  This is the reference's reduction
+ * idiom `atomic_ref(result)[0] += tile.sum()` with the tile an elementwise
+ * expression of loads (python/hckernel/tests/test_examples.py:31-71;
+ * atomic_ref: kernel_api.py:450-451).  The order of the additions is not
+ * fixed, so two runs may differ in the last bits. */
+int hcamdLaunchMapSum(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
+                      const void *const *inputs, const int *inputTypes,
+                      const size_t *inputLd, size_t nInputs, float *cell,
+                      size_t rows, size_t cols) HCAMD_NOEXCEPT;
+
 /* Row softmax, fp32: y[r,:] = exp(x[r,:]-max(x[r,:])) / sum(exp(...)).
  * Expression of python/hckernel/tests/test_examples.py:330-335. */
 int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,

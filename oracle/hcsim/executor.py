@@ -348,7 +348,10 @@ class Kernel:
         self.tunables = tunables
         self.tuned = dict(tuned or {})
         self._binders = _collect_binders(func)
-        if isinstance(tunables, TunableParam):
+        # (by attribute, so that the GPU front-end's own TunableParam class,
+        # used by kernels written once and run on both sides, is accepted)
+        if isinstance(tunables, TunableParam) or (hasattr(tunables, "sym") and
+                                                  hasattr(tunables, "default")):
             tunables = (tunables,)
         assert isinstance(tunables, Iterable), "Unsupported tunables"
         self._defaults = {t.sym: t.default for t in tunables}

@@ -319,6 +319,77 @@ def test_elementwise_body_with_transcendental_functions():
     assert_allclose(dout.to_host(), host, rtol=2e-6, atol=2e-6)
 
 
+# ---------------------------------------------------------------------------
+# reductions through atomic_ref (python/hckernel/tests/test_examples.py:31-71)
+# ---------------------------------------------------------------------------
+def _reduction_kernels(deco):
+    WS, GS, N = sym.WS, sym.GS, sym.N
+    TN = TunableParam(N, 2, range(1, 64))
+
+    def reduction_1(gr: CurrentGroup, a: Buffer[WS, DT], result: Buffer[1, DT], gshape: GS):
+        a_view = gr.load(a[gr.work_offset[0] * N:], shape=gr.size * N)
+        atomic_ref(result)[0] += a_view.sum()
+
+    def reduction_2(group: CurrentGroup, a: Buffer[WS, DT], result: Buffer[1, DT], gshape: GS):
+        temp_result = group.zeros(group.size, dtype=a.dtype)
+        for i in range(N):
+            work_offset = group.work_offset[0] * N + i * group.size
+            a_view = group.load(a[work_offset:], shape=group.size)
+            temp_result += a_view
+        atomic_ref(result)[0] += temp_result.sum()
+
+    args = dict(work_shape=cdiv(WS, N), group_shape=GS, tunables=TN)
+    return [deco(**args)(f) for f in (reduction_1, reduction_2)]
+
+
+def test_reference_reductions_known_answer():
+    a = np.arange(0, 20).astype(np.float32)          # the reference's input; the sum is exact
+    for gpu, host in zip(_reduction_kernels(kernel), _reduction_kernels(sim_kernel)):
+        result = rt.to_device(np.zeros(1, np.float32))
+        gpu(rt.to_device(a), result, 8)
+        want = np.zeros(1, np.float32)
+        host(a, want, 8)
+        assert result.to_host()[0] == want[0] == a.sum() == 190.0
+        gpu(rt.to_device(a), result, 8)               # += : accumulates on top
+        assert result.to_host()[0] == 380.0
+
+
+@pytest.mark.parametrize("n", [1, 7, 8, 2047, 100_003, 16_777_259])
+def test_reductions_of_random_data_within_fp32_summation_error(n):
+    rng = np.random.default_rng(n)
+    a = rng.standard_normal(n).astype(np.float32)
+    exact = float(a.astype(np.float64).sum())
+    # any order of n fp32 additions is within n * 2^-24 * sum|a| of the exact sum;
+    # the kernel adds eight values per lane, then trees: far inside that bound
+    bound = 64 * 2.0 ** -24 * float(np.abs(a).astype(np.float64).sum()) + 1e-30
+    for k in _reduction_kernels(kernel):
+        result = rt.to_device(np.zeros(1, np.float32))
+        k.parametrize({sym.N: 4})(rt.to_device(a), result, 64)
+        assert abs(float(result.to_host()[0]) - exact) <= bound
+
+
+def test_dot_product_through_the_map_sum_kernel():
+    WS = sym.WS
+
+    def dot(gr: CurrentGroup, a: Buffer[WS, DT], b: Buffer[WS, DT], result: Buffer[4, DT]):
+        o, g = gr.work_offset[0], gr.shape[0]
+        atomic_ref(result)[2] += (gr.load(a[o:], shape=g) * gr.load(b[o:], shape=g)).sum()
+
+    rng = np.random.default_rng(33)
+    n = 1_000_003
+    for dtype in (np.float32, np.float16):
+        a, b = (rng.standard_normal(n).astype(dtype) for _ in range(2))
+        result = rt.to_device(np.array([1, 2, 3, 4], np.float32))
+        kernel(work_shape=WS, group_shape=256)(dot)(rt.to_device(a), rt.to_device(b), result)
+        got = result.to_host()
+        assert_array_equal(got[[0, 1, 3]], [1, 2, 4])            # neighbours untouched
+        if dtype == np.float16:                                   # fp16 tiles: the product rounds
+            prod = (a * b).astype(np.float64)
+        else:
+            prod = (a * b).astype(np.float64)                     # fp32 product, then summed
+        assert abs(float(got[2]) - 3.0 - prod.sum()) <= 64 * 2.0 ** -24 * np.abs(prod).sum()
+
+
 def test_unsupported_body_raises_instead_of_running_on_the_cpu():
     N = sym.N
 

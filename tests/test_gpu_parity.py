@@ -470,6 +470,38 @@ def test_map_rejects_malformed_programs(ctx):
     rt.plan_map([I("in", 0)], [_view(x, 0)], _view(out, 0)).launch(sync=True)
 
 
+def test_map_sum_flat_strided_and_accumulation(ctx):
+    rng = np.random.default_rng(14)
+    shape = (37, 1031)
+    a = rng.standard_normal(shape).astype(np.float16)
+    b = rng.standard_normal(shape).astype(np.float32)
+    terms = (a.astype(np.float32) * b).astype(np.float64)          # fp32 products
+    bound = 64 * 2.0 ** -24 * np.abs(terms).sum()
+    prog = [I("in", 0), I("mul_in", 1)]
+    cell = dev(np.array([0.0, 10.0], np.float32))
+    rt.plan_map_sum(prog, [dev(a), dev(b)], cell, 1).launch(sync=True)
+    assert rt.last_kernel_name() == "hcamd_map_sum_flat"
+    got = cell.to_host()
+    assert got[0] == 0.0 and abs(float(got[1]) - 10.0 - terms.sum()) <= bound
+    # a window of larger arrays goes through the strided kernel; adds on top
+    big_a, big_b = np.zeros((40, 1100), np.float16), np.zeros((40, 1100), np.float32)
+    big_a[:37, :1031], big_b[:37, :1031] = a, b
+    big_a[37:], big_b[:, 1031:] = 9.0, 9.0                          # must not be read as data
+    da, db = dev(big_a), dev(big_b)
+    views = [_View(da, shape, 0, (1100, 1)), _View(db, shape, 0, (1100, 1))]
+    rt.plan_map_sum(prog, views, cell, 1).launch(sync=True)
+    assert rt.last_kernel_name() == "hcamd_map_sum_strided"
+    assert abs(float(cell.to_host()[1]) - 10.0 - 2 * terms.sum()) <= 2 * bound
+    # constants survive the tail handling: sum(x * 0 + 1) counts the elements
+    for n in (1, 5, 8, 4099, 70_001):
+        x = dev(np.ones(n, np.float32))
+        c = dev(np.zeros(1, np.float32))
+        rt.plan_map_sum([I("in", 0), I("muli", 0, 0.0), I("addi", 0, 1.0)], [x], c).launch(sync=True)
+        assert c.to_host()[0] == n
+    with pytest.raises(rt.HcRuntimeError, match="underflow"):
+        rt.plan_map_sum([I("add")], [da], cell).launch(sync=True)
+
+
 def test_map_full_benchmark_size_fma(ctx):
     a, b, c = cf.inputs_c2()
     d = rt.DeviceArray(a.shape, np.float16)

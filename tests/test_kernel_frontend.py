@@ -10,7 +10,7 @@ import pytest
 import sympy
 
 from hc_amd import runtime as rt
-from hc_amd.kernel import (Buffer, CurrentGroup, NoNativeKernel, TunableParam, kernel,
+from hc_amd.kernel import (Buffer, CurrentGroup, NoNativeKernel, TunableParam, atomic_ref, kernel,
                            suggest_group_shape, sym, typename)
 from oracle import closed_forms as cf
 
@@ -363,3 +363,59 @@ def test_decorator_argument_checks():
         kernel(work_shape=(4, 4), group_shape=(2,))
     with pytest.raises(AssertionError, match="Subgroup size"):
         kernel(work_shape=4, subgroup_size=sym.SG)
+
+
+def test_reference_reduction_bodies_bind_to_the_map_sum_kernel(ctx):
+    # bodies of python/hckernel/tests/test_examples.py:31-71
+    WS, GS, N = sym.WS, sym.GS, sym.N
+    TN = TunableParam(N, 2, range(1, 64))
+
+    @kernel(work_shape=cdiv(WS, N), group_shape=GS, tunables=TN)
+    def reduction_1(gr: CurrentGroup, a: Buffer[WS, DT], result: Buffer[1, DT], gshape: GS):
+        a_view = gr.load(a[gr.work_offset[0] * N:], shape=gr.size * N)
+        atomic_ref(result)[0] += a_view.sum()
+
+    @kernel(work_shape=cdiv(WS, N), group_shape=GS, tunables=TN)
+    def reduction_2(group: CurrentGroup, a: Buffer[WS, DT], result: Buffer[1, DT], gshape: GS):
+        temp_result = group.zeros(group.size, dtype=a.dtype)
+        for i in range(N):
+            work_offset = group.work_offset[0] * N + i * group.size
+            a_view = group.load(a[work_offset:], shape=group.size)
+            temp_result += a_view
+        atomic_ref(result)[0] += temp_result.sum()
+
+    a, res = FakeDev((20,), "float32"), FakeDev((1,), "float32")
+    for k in (reduction_1, reduction_2, reduction_2.parametrize({N: 4})):
+        (p,) = k.plan(a, res, 8, ctx=ctx)
+        assert p.fn is rt.hcamdLaunchMapSum
+        assert map_program(p) == [("in", 0, 0.0)]
+        assert p.args[3][0] == a.ptr and p.args[7] == res.ptr and p.args[8:] == (1, 20)
+
+    # a dot product: one pass, the product is formed by the program
+    @kernel(work_shape=WS, group_shape=256)
+    def dot(gr: CurrentGroup, a: Buffer[WS, DT], b: Buffer[WS, DT], result: Buffer[4, DT]):
+        o, g = gr.work_offset[0], gr.shape[0]
+        atomic_ref(result)[2] += (gr.load(a[o:], shape=g) * gr.load(b[o:], shape=g)).sum()
+
+    res4 = FakeDev((4,), "float32")
+    (p,) = dot.plan(a, FakeDev((20,), "float32"), res4, ctx=ctx)
+    assert map_program(p) == [("in", 0, 0.0), ("mul_in", 1, 0.0)] and p.args[7] == res4.ptr + 8
+
+    # what has no kernel says so
+    @kernel(work_shape=WS, group_shape=256)
+    def per_group(gr: CurrentGroup, a: Buffer[WS, DT], result: Buffer[4, DT]):
+        atomic_ref(result)[gr.id[0]] += gr.load(a[gr.work_offset[0]:], shape=gr.shape[0]).sum()
+
+    @kernel(work_shape=WS, group_shape=256)
+    def not_a_sum(gr: CurrentGroup, a: Buffer[WS, DT], result: Buffer[4, DT]):
+        atomic_ref(result)[0] += gr.load(a[gr.work_offset[0]:], shape=gr.shape[0]).max()
+
+    @kernel(work_shape=WS, group_shape=256)
+    def assigned(gr: CurrentGroup, a: Buffer[WS, DT], result: Buffer[4, DT]):
+        atomic_ref(result)[0] = gr.load(a[gr.work_offset[0]:], shape=gr.shape[0]).sum()
+
+    for k in (per_group, not_a_sum, assigned):
+        with pytest.raises(NoNativeKernel):
+            k.plan(a, res4, ctx=ctx)
+    with pytest.raises(NoNativeKernel, match="float32"):
+        reduction_1.plan(a, FakeDev((1,), "float16"), 8, ctx=ctx)
