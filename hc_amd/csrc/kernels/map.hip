@@ -36,14 +36,10 @@ constexpr int kThreads = 256;
 constexpr int kDepth = 4;    // evaluation stack entries
 constexpr int kMaxIn = 4;    // operands
 constexpr int kMaxProg = 32; // instructions
-#ifndef HCAMD_MAP_CHUNKS
-#define HCAMD_MAP_CHUNKS 1
-#endif
 #ifndef HCAMD_MAP_WAVES
 #define HCAMD_MAP_WAVES 4 // resident waves per SIMD the flat kernel is compiled for
 #endif
-constexpr int kChunks = HCAMD_MAP_CHUNKS; // chunks of eight elements per lane per pass
-constexpr int kN = 8 * kChunks;           // elements per lane per pass
+constexpr int kN = 8; // elements per lane per run of the program (one chunk)
 
 // Opcodes.  The numbering is part of the C ABI (hcamdLaunchMap).
 enum : uint32_t {
@@ -144,10 +140,10 @@ template <int OP> __device__ __forceinline__ float unary(float a) {
   return a;
 }
 
-// Operands of one pass, as loaded: per chunk eight fp16 in w[..][j][0], or
-// eight fp32 in w[..][j][0..1].
+// Operands of one chunk, as loaded: eight fp16 in w[..][0], or eight fp32 in
+// w[..][0..1].
 struct Raw {
-  u32x4 w[kMaxIn][kChunks][2];
+  u32x4 w[kMaxIn][2];
 };
 
 struct Stack {
@@ -157,25 +153,22 @@ struct Stack {
 __device__ __forceinline__ void unpack(const Raw &raw, int i, bool f16, float *dst) {
   // The empty asm statements pin the conversion to the arm that pushes the
   // operand: hoisted out of the interpreter loop it would hold eight more
-  // registers per operand and chunk for the whole pass.
+  // registers per operand for the whole pass.
+  if (f16) {
 #pragma unroll
-  for (int j = 0; j < kChunks; ++j) {
-    if (f16) {
+    for (int e = 0; e < 4; ++e) {
+      uint32_t w = raw.w[i][0][e];
+      asm volatile("" : "+v"(w));
+      dst[2 * e] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
+      dst[2 * e + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+    }
+  } else {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        uint32_t w = raw.w[i][j][0][e];
-        asm volatile("" : "+v"(w));
-        dst[8 * j + 2 * e] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
-        dst[8 * j + 2 * e + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
-      }
-    } else {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        uint32_t lo = raw.w[i][j][0][e], hi = raw.w[i][j][1][e];
-        asm volatile("" : "+v"(lo), "+v"(hi));
-        dst[8 * j + e] = __builtin_bit_cast(float, lo);
-        dst[8 * j + 4 + e] = __builtin_bit_cast(float, hi);
-      }
+    for (int e = 0; e < 4; ++e) {
+      uint32_t lo = raw.w[i][0][e], hi = raw.w[i][1][e];
+      asm volatile("" : "+v"(lo), "+v"(hi));
+      dst[e] = __builtin_bit_cast(float, lo);
+      dst[4 + e] = __builtin_bit_cast(float, hi);
     }
   }
 }
@@ -331,28 +324,6 @@ __device__ __forceinline__ void run_program(const MapArgs &a, const Raw &raw,
 }
 
 // ---- operand access -------------------------------------------------------------
-// chunk j of a pass that starts at chunk c is c + j * 256: a wave-level access
-// covers 1 KiB (fp16) or 2 KiB (fp32) of consecutive memory
-__device__ __forceinline__ void load_raw(const MapArgs &a, uint32_t n_in, size_t c,
-                                         size_t n_chunks, Raw &raw) {
-#pragma unroll
-  for (int i = 0; i < kMaxIn; ++i)
-    if (i < (int)n_in) {
-#pragma unroll
-      for (int j = 0; j < kChunks; ++j) {
-        const size_t chunk = c + (size_t)j * kThreads;
-        if (chunk < n_chunks) {
-          if ((a.f16_mask >> i) & 1) {
-            raw.w[i][j][0] = ldg<true>(static_cast<const u32x4 *>(a.in[i]) + chunk);
-          } else {
-            const u32x4 *q = static_cast<const u32x4 *>(a.in[i]) + 2 * chunk;
-            raw.w[i][j][0] = ldg<true>(q);
-            raw.w[i][j][1] = ldg<true>(q + 1);
-          }
-        }
-      }
-    }
-}
 __device__ __forceinline__ void store_chunk(void *p, bool f16, size_t chunk,
                                             const float *src) {
   if (f16) {
@@ -382,7 +353,7 @@ __device__ __forceinline__ void store_elem(void *p, bool f16, size_t i, float v)
   else
     static_cast<float *>(p)[i] = v;
 }
-// Element-wise gather of one pass: slot e of every operand from index idx(e),
+// Element-wise gather of one chunk: slot e of every operand from index idx(e),
 // zero where idx(e) is out of range; kept as fp32 whatever the operand type.
 template <class Index>
 __device__ __forceinline__ void gather(const MapArgs &a, uint32_t n_in, Raw &raw,
@@ -395,39 +366,189 @@ __device__ __forceinline__ void gather(const MapArgs &a, uint32_t n_in, Raw &raw
         size_t off;
         const bool ok = index(i, e, off);
         const float v = ok ? load_elem(a.in[i], (a.f16_mask >> i) & 1, off) : 0.0f;
-        raw.w[i][e / 8][(e % 8) / 4][e % 4] = __builtin_bit_cast(uint32_t, v);
+        raw.w[i][e / 4][e % 4] = __builtin_bit_cast(uint32_t, v);
       }
     }
 }
+
+template <int T> __device__ __forceinline__ void finish_sum(float acc, float *cell) {
+  __shared__ float slots[T / kWave];
+  const float total = group_reduce<SumOp, T / kWave>(acc, slots);
+  if (threadIdx.x == 0)
+    unsafeAtomicAdd(cell, total);
+}
+
+// Flat form of the map-reduce (SUM = true: all results added up into one fp32
+// cell; SUM = false, one stored result per element, is kept for measurements).
+//
+// Chunk = eight consecutive elements.  A pass of a lane covers U chunks, 256
+// apart; workgroup g starts at chunk g * 256 * U and strides by gridDim.x * 256
+// * U.  The loads of all U chunks are issued together, then the program runs on
+// one chunk after the other, so a lane keeps U times the bytes in flight for the
+// same number of registers when there are few operands (NIN) or all of them are
+// fp16 (HALF).  The staged chunks are shifted down one place per run instead of
+// being indexed, and the loop over them is kept rolled, which keeps a single
+// copy of the interpreter in the code.  Every lane makes the same number of
+// passes and runs; out-of-range ones are predicated off, so the interpreter's
+// control flow stays uniform.  The elements after the last whole chunk are
+// finished by the last lane of the last workgroup, one by one.
+template <int NIN, int U, bool HALF, bool SUM>
+__device__ __forceinline__ void map_flat(const MapArgs &a, const uint32_t n_in) {
+  // The reduction runs with 1024 lanes per workgroup: one workgroup fills a CU,
+  // so a launch ends in a few hundred atomic additions to the one cell, not
+  // thousands (they are served one after the other, some 15 ns each).
+  constexpr int kThreads = SUM ? 1024 : 256;
+  constexpr int W = HALF ? 1 : 2;
+  const size_t n = a.cols;
+  const size_t n_chunks = n / 8;
+  const size_t stride = (size_t)gridDim.x * (kThreads * U);
+  const size_t passes = (n_chunks + stride - 1) / stride;
+  const bool out_f16 = (a.f16_mask >> 8) & 1;
+  size_t c0 = (size_t)blockIdx.x * (kThreads * U) + threadIdx.x;
+  float acc = 0.0f;
+  Raw raw;
+  Stack r;
+  for (size_t p = 0; p < passes; ++p, c0 += stride) {
+    u32x4 staged[NIN][U][W];
+#pragma unroll
+    for (int i = 0; i < NIN; ++i)
+      if (i < (int)n_in) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const size_t chunk = c0 + (size_t)u * kThreads;
+          if (chunk < n_chunks) {
+            const bool f16 = HALF || ((a.f16_mask >> i) & 1);
+            const u32x4 *q = static_cast<const u32x4 *>(a.in[i]) + (f16 ? chunk : 2 * chunk);
+            staged[i][u][0] = ldg<true>(q);
+            if constexpr (!HALF)
+              if (!f16)
+                staged[i][u][1] = ldg<true>(q + 1);
+          }
+        }
+      }
+#pragma nounroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int i = 0; i < NIN; ++i) {
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+          raw.w[i][w] = staged[i][0][w];
+#pragma unroll
+          for (int k = 0; k + 1 < U; ++k)
+            staged[i][k][w] = staged[i][k + 1][w];
+        }
+      }
+      run_program(a, raw, a.f16_mask, r);
+      const size_t chunk = c0 + (size_t)u * kThreads;
+      if (chunk < n_chunks) {
+        if constexpr (SUM) {
+#pragma unroll
+          for (int e = 0; e < kN; ++e)
+            acc += r.st[0][e];
+        } else {
+          store_chunk(a.out, out_f16, chunk, r.st[0]);
+        }
+      }
+    }
+  }
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == kThreads - 1 && n_chunks * 8 < n) {
+    gather(a, n_in, raw, [&](int, int e, size_t &off) {
+      off = n_chunks * 8 + e;
+      return off < n;
+    });
+    run_program(a, raw, 0, r);
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      if (n_chunks * 8 + e < n) {
+        if constexpr (SUM)
+          acc += r.st[0][e];
+        else
+          store_elem(a.out, out_f16, n_chunks * 8 + e, r.st[0][e]);
+      }
+  }
+  if constexpr (SUM)
+    finish_sum<kThreads>(acc, static_cast<float *>(a.out));
+}
+
+// Strided form: blockIdx.y walks rows, x walks the columns of a row in runs of
+// 256 * 8; lane t takes columns t, t + 256, ... so a wave reads consecutive
+// elements.
+template <bool SUM>
+__device__ __forceinline__ void map_strided(const MapArgs &a, const uint32_t n_in) {
+  const size_t row = blockIdx.y;
+  const size_t col0 = (size_t)blockIdx.x * (kThreads * kN) + threadIdx.x;
+  Raw raw;
+  gather(a, n_in, raw, [&](int i, int e, size_t &off) {
+    const size_t col = col0 + (size_t)e * kThreads;
+    off = row * a.ld[i] + col;
+    return col < a.cols;
+  });
+  Stack r;
+  run_program(a, raw, 0, r);
+  float acc = 0.0f;
+#pragma unroll
+  for (int e = 0; e < kN; ++e) {
+    const size_t col = col0 + (size_t)e * kThreads;
+    if (col < a.cols) {
+      if constexpr (SUM)
+        acc += r.st[0][e];
+      else
+        store_elem(a.out, (a.f16_mask >> 8) & 1, row * a.ldo + col, r.st[0][e]);
+    }
+  }
+  if constexpr (SUM)
+    finish_sum<kThreads>(acc, static_cast<float *>(a.out));
+}
 } // namespace
 
-// Flat form.  Chunk = eight consecutive elements; a workgroup owns kChunks * 256
-// consecutive chunks and lane t takes chunks t, t + 256, ...  All operand loads
-// of a pass are issued together and the program runs once they have landed;
-// the other resident waves cover the memory latency.  The elements after the
-// last whole chunk are finished by the last lane of the last workgroup, one by
-// one.
+// Map-reduce note: a lane adds up the values of its own elements in fp32, a wave
+// folds its lanes with DPP, the four waves meet in LDS, and one lane per
+// workgroup issues a single hardware fp32 atomic add; the host caps the grid so
+// that at most a few thousand atomics reach the cell.  The order of the
+// additions differs from run to run: the result is a correctly computed fp32
+// sum, not a bit-reproducible one.
+#define HCAMD_MAP_FLAT(NAME, NIN, U, HALF, SUM)                                \
+  extern "C" __global__ __launch_bounds__(SUM ? 1024 : 256) __attribute__((    \
+      amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void             \
+  NAME(const MapArgs a, const uint32_t n_in) {                                 \
+    map_flat<NIN, U, HALF, SUM>(a, n_in);                                      \
+  }
+// name: operands it can take / chunks per pass; h = all operands fp16
+HCAMD_MAP_FLAT(hcamd_map_sum_flat_n4u1, 4, 1, false, true)
+HCAMD_MAP_FLAT(hcamd_map_sum_flat_n2u2, 2, 2, false, true)
+HCAMD_MAP_FLAT(hcamd_map_sum_flat_n1u4, 1, 4, false, true)
+HCAMD_MAP_FLAT(hcamd_map_sum_flat_n4u2h, 4, 2, true, true)
+HCAMD_MAP_FLAT(hcamd_map_sum_flat_n2u4h, 2, 4, true, true)
+
+// The map itself: one chunk per lane, one pass, no loop around the interpreter
+// (several chunks per pass, or a persistent grid, measured slower here: the
+// stores of one workgroup already overlap the loads of the next).
 extern "C" __global__ __launch_bounds__(256)
 __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcamd_map_flat(
     const MapArgs a, const uint32_t n_in) {
   const size_t n = a.cols;
   const size_t n_chunks = n / 8;
   const bool out_f16 = (a.f16_mask >> 8) & 1;
-  const size_t c = (size_t)blockIdx.x * (kThreads * kChunks) + threadIdx.x;
+  const size_t c = (size_t)blockIdx.x * 256 + threadIdx.x;
   Raw raw;
-  load_raw(a, n_in, c, n_chunks, raw);
+  if (c < n_chunks) {
+#pragma unroll
+    for (int i = 0; i < kMaxIn; ++i)
+      if (i < (int)n_in) {
+        if ((a.f16_mask >> i) & 1) {
+          raw.w[i][0] = ldg<true>(static_cast<const u32x4 *>(a.in[i]) + c);
+        } else {
+          const u32x4 *q = static_cast<const u32x4 *>(a.in[i]) + 2 * c;
+          raw.w[i][0] = ldg<true>(q);
+          raw.w[i][1] = ldg<true>(q + 1);
+        }
+      }
+  }
   Stack r;
   run_program(a, raw, a.f16_mask, r);
-#pragma unroll
-  for (int j = 0; j < kChunks; ++j) {
-    const size_t chunk = c + (size_t)j * kThreads;
-    float v[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = r.st[0][8 * j + e];
-    if (chunk < n_chunks)
-      store_chunk(a.out, out_f16, chunk, v);
-  }
-  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == kThreads - 1 && n_chunks * 8 < n) {
+  if (c < n_chunks)
+    store_chunk(a.out, out_f16, c, r.st[0]);
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 255 && n_chunks * 8 < n) {
     gather(a, n_in, raw, [&](int, int e, size_t &off) {
       off = n_chunks * 8 + e;
       return off < n;
@@ -440,100 +561,11 @@ __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcam
   }
 }
 
-// Strided form: blockIdx.y walks rows, x walks the columns of a row in runs of
-// 256 * kN; lane t takes columns t, t + 256, ... so a wave reads consecutive
-// elements.
 extern "C" __global__ __launch_bounds__(256) void hcamd_map_strided(
     const MapArgs a, const uint32_t n_in) {
-  const size_t row = blockIdx.y;
-  const size_t col0 = (size_t)blockIdx.x * (kThreads * kN) + threadIdx.x;
-  Raw raw;
-  gather(a, n_in, raw, [&](int i, int e, size_t &off) {
-    const size_t col = col0 + (size_t)e * kThreads;
-    off = row * a.ld[i] + col;
-    return col < a.cols;
-  });
-  Stack r;
-  run_program(a, raw, 0, r);
-#pragma unroll
-  for (int e = 0; e < kN; ++e) {
-    const size_t col = col0 + (size_t)e * kThreads;
-    if (col < a.cols)
-      store_elem(a.out, (a.f16_mask >> 8) & 1, row * a.ldo + col, r.st[0][e]);
-  }
+  map_strided<false>(a, n_in);
 }
-
-// ---------------------------------------------------------------------------
-// Map-reduce: *result += sum over the window of f(in0[i], ...).  Same programs,
-// same operand handling; the output pointer of the argument block is the fp32
-// accumulator cell.  A lane adds up the values of its own elements in fp32, a
-// wave folds its lanes with DPP, the four waves meet in LDS, and one lane per
-// workgroup issues a single hardware fp32 atomic add; the grid is capped so that
-// at most a few thousand atomics reach the cell.  The order of the additions
-// differs from run to run: the result is a correctly computed fp32 sum, not a
-// bit-reproducible one.
-// ---------------------------------------------------------------------------
-namespace {
-__device__ __forceinline__ void finish_sum(float acc, float *cell) {
-  __shared__ float slots[kThreads / kWave];
-  const float total = group_reduce<SumOp, kThreads / kWave>(acc, slots);
-  if (threadIdx.x == 0)
-    unsafeAtomicAdd(cell, total);
-}
-} // namespace
-
-extern "C" __global__ __launch_bounds__(256)
-__attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcamd_map_sum_flat(
-    const MapArgs a, const uint32_t n_in) {
-  const size_t n = a.cols;
-  const size_t n_chunks = n / 8;
-  const size_t stride = (size_t)gridDim.x * kThreads;
-  const size_t passes = (n_chunks + stride - 1) / stride; // same for every lane
-  size_t c = (size_t)blockIdx.x * kThreads + threadIdx.x;
-  float acc = 0.0f;
-  Raw raw;
-  Stack r;
-  for (size_t p = 0; p < passes; ++p, c += stride) {
-    if (c < n_chunks)
-      load_raw(a, n_in, c, n_chunks, raw);
-    run_program(a, raw, a.f16_mask, r);
-    if (c < n_chunks) {
-#pragma unroll
-      for (int e = 0; e < kN; ++e)
-        acc += r.st[0][e];
-    }
-  }
-  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == kThreads - 1 && n_chunks * 8 < n) {
-    gather(a, n_in, raw, [&](int, int e, size_t &off) {
-      off = n_chunks * 8 + e;
-      return off < n;
-    });
-    run_program(a, raw, 0, r);
-#pragma unroll
-    for (int e = 0; e < 8; ++e)
-      if (n_chunks * 8 + e < n)
-        acc += r.st[0][e];
-  }
-  finish_sum(acc, static_cast<float *>(a.out));
-}
-
-// Strided form: one workgroup per (row, run of 256 * kN columns).
 extern "C" __global__ __launch_bounds__(256) void hcamd_map_sum_strided(
     const MapArgs a, const uint32_t n_in) {
-  const size_t row = blockIdx.y;
-  const size_t col0 = (size_t)blockIdx.x * (kThreads * kN) + threadIdx.x;
-  Raw raw;
-  gather(a, n_in, raw, [&](int i, int e, size_t &off) {
-    const size_t col = col0 + (size_t)e * kThreads;
-    off = row * a.ld[i] + col;
-    return col < a.cols;
-  });
-  Stack r;
-  run_program(a, raw, 0, r);
-  float acc = 0.0f;
-#pragma unroll
-  for (int e = 0; e < kN; ++e)
-    if (col0 + (size_t)e * kThreads < a.cols)
-      acc += r.st[0][e];
-  finish_sum(acc, static_cast<float *>(a.out));
+  map_strided<true>(a, n_in);
 }

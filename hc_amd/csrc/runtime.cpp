@@ -1010,11 +1010,30 @@ int launchMap(OlQueue q, bool sum, const HcamdMapInstr *prog, size_t nInstr,
   if (dense && aligned && variantOf("map") != 1) {
     a.rows = 1;
     a.cols = rows * cols;
-    size_t groups = std::max(ceilDiv(a.cols, kPerGroup), (size_t)1);
-    if (sum) // persistent: one atomic per workgroup, at most 8 groups per CU
-      groups = std::min(groups, (size_t)computeUnitsOf(dev) * 8);
-    return launch1d(queue, "map", sum ? "hcamd_map_sum_flat" : "hcamd_map_flat",
-                    groups, 256, args);
+    // The reduction picks its kernel by operand count and storage type: fewer
+    // or narrower operands leave registers for more chunks in flight per lane.
+    const bool half = nInputs > 0 && (a.f16_mask & 0xffu) == (1u << nInputs) - 1u;
+    const char *name = "hcamd_map_flat";
+    size_t u = 1;
+    if (sum && half) {
+      name = nInputs <= 2 ? "hcamd_map_sum_flat_n2u4h" : "hcamd_map_sum_flat_n4u2h";
+      u = nInputs <= 2 ? 4 : 2;
+    } else if (sum && nInputs <= 1) {
+      name = "hcamd_map_sum_flat_n1u4";
+      u = 4;
+    } else if (sum && nInputs <= 2) {
+      name = "hcamd_map_sum_flat_n2u2";
+      u = 2;
+    } else if (sum) {
+      name = "hcamd_map_sum_flat_n4u1";
+    }
+    // the reduction: 1024-lane workgroups, one per CU, each striding over the
+    // vector and ending in one atomic addition
+    const size_t threads = sum ? 1024 : 256;
+    size_t groups = std::max(ceilDiv(a.cols, threads * 8 * u), (size_t)1);
+    if (sum)
+      groups = std::min(groups, (size_t)computeUnitsOf(dev));
+    return launch1d(queue, "map", name, groups, threads, args);
   }
   Kernel *k = builtinKernel(dev, "map",
                             sum ? "hcamd_map_sum_strided" : "hcamd_map_strided");

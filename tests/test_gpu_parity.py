@@ -480,7 +480,7 @@ def test_map_sum_flat_strided_and_accumulation(ctx):
     prog = [I("in", 0), I("mul_in", 1)]
     cell = dev(np.array([0.0, 10.0], np.float32))
     rt.plan_map_sum(prog, [dev(a), dev(b)], cell, 1).launch(sync=True)
-    assert rt.last_kernel_name() == "hcamd_map_sum_flat"
+    assert rt.last_kernel_name() == "hcamd_map_sum_flat_n2u2"
     got = cell.to_host()
     assert got[0] == 0.0 and abs(float(got[1]) - 10.0 - terms.sum()) <= bound
     # a window of larger arrays goes through the strided kernel; adds on top
