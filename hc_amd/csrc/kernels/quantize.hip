@@ -182,7 +182,77 @@ __device__ __forceinline__ void quantize_regs(const _Float16 *x, size_t ldx,
     }
   }
 }
+// Persistent form for rows of exactly 256 * 16 columns, 16-byte aligned: a
+// workgroup strides over the rows, and the loads of its next row are issued
+// before the absmax reduction of the current one, so requests stay in flight
+// across the reduction and its barrier.  The two LDS slot sets alternate from
+// row to row, which makes the one barrier inside the reduction sufficient.
+template <bool NT>
+__device__ __forceinline__ void quantize_persistent(const _Float16 *x, size_t ldx,
+                                                    int8_t *q, size_t ldq,
+                                                    float *scale_out, size_t rows) {
+  constexpr int kWaves = kThreads / kWave;
+  __shared__ uint32_t smax[2][kWaves];
+  const int t = threadIdx.x;
+  size_t row = blockIdx.x;
+  u32x4 cur[2], nxt[2];
+  if (row < rows) {
+    const u32x4 *p = reinterpret_cast<const u32x4 *>(x + row * ldx + (size_t)t * 16);
+    cur[0] = ldg<NT>(p);
+    cur[1] = ldg<NT>(p + 1);
+  }
+  for (int it = 0; row < rows; row += gridDim.x, ++it) {
+    const size_t next = row + gridDim.x;
+    if (next < rows) {
+      const u32x4 *p = reinterpret_cast<const u32x4 *>(x + next * ldx + (size_t)t * 16);
+      nxt[0] = ldg<NT>(p);
+      nxt[1] = ldg<NT>(p + 1);
+    }
+    uint32_t m = 0;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        m = absmax_bits(m, cur[h][i]);
+    m = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
+    m = group_reduce<UMaxOp, kWaves>(m, smax[it & 1]);
+    const float amax = half_bits_to_float(m);
+    const float scale = amax / 127.0f;
+    if (t == 0)
+      scale_out[row] = scale;
+    int8_t *qr = q + row * ldq + (size_t)t * 16;
+    if (!(amax < INFINITY)) { // inf or NaN in the row
+      for (int i = 0; i < 16; ++i) {
+        const uint32_t w = cur[i / 8][(i % 8) / 2];
+        const uint32_t bits = (i & 1) ? (w >> 16) : (w & 0xffffu);
+        qr[i] = quant_special(half_bits_to_float(bits), scale);
+      }
+    } else {
+      const float div = (amax == 0.0f) ? 1.0f : scale;
+      const float rcp = 1.0f / div;
+      u32x4 o;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t w0 = cur[k / 2][(2 * k) % 4];
+        const uint32_t w1 = cur[k / 2][(2 * k) % 4 + 1];
+        o[k] = pack4(quotient<false>(half_bits_to_float(w0 & 0xffffu), div, rcp),
+                     quotient<false>(half_bits_to_float(w0 >> 16), div, rcp),
+                     quotient<false>(half_bits_to_float(w1 & 0xffffu), div, rcp),
+                     quotient<false>(half_bits_to_float(w1 >> 16), div, rcp));
+      }
+      stg<NT>(reinterpret_cast<u32x4 *>(qr), o);
+    }
+    cur[0] = nxt[0];
+    cur[1] = nxt[1];
+  }
+}
 } // namespace
+
+extern "C" __global__ __launch_bounds__(256) void hcamd_quant_f16_i8_p256_v1_nt(
+    const _Float16 *x, size_t ldx, int8_t *q, size_t ldq, float *scale,
+    size_t rows, size_t cols) {
+  quantize_persistent<true>(x, ldx, q, ldq, scale, rows);
+}
 
 #define HCAMD_QUANT(NAME, TPR, VPT, EXACT, NT)                                 \
   extern "C" __global__ __launch_bounds__(256) void NAME(                      \

@@ -1200,6 +1200,13 @@ int hcamdLaunchQuantizeF16I8(OlQueue q, const void *x, size_t ldx, int8_t *qout,
   if (per_wave)
     rows_per_group = 4;
   groups = ceilDiv(rows, rows_per_group);
+  // variants 8..11: persistent kernel for rows of exactly 4096 columns, with
+  // 4 / 8 / 6 / 12 workgroups per CU
+  if (cols == 4096 && variant >= 8 && variant <= 11) {
+    static const size_t per_cu[] = {4, 8, 6, 12};
+    name = "hcamd_quant_f16_i8_p256_v1_nt";
+    groups = std::min(rows, (size_t)computeUnitsOf(dev) * per_cu[variant - 8]);
+  }
   return launch1d(queue, "quantize", name, groups, 256, args);
 }
 

@@ -632,7 +632,7 @@ def test_quantize_bit_exact(ctx, shape):
 def test_quantize_variants_and_strides(ctx):
     (x,) = cf.inputs_c4((301, 4096))
     q_np, s_np = cf.np_quantize(x)
-    for v in range(0, 8):
+    for v in range(0, 12):
         rt.set_variant("quantize", v)
         for ld in (4096, 4096 + 64):
             q, s = run_quantize(x, ld)
