@@ -94,6 +94,46 @@ def test_copy_with_torch_tensors():
     torch.testing.assert_close(c, a[:, :400])
 
 
+def test_elementwise_and_reduction_bodies_on_torch_tensors():
+    torch = pytest.importorskip("torch")
+    if not torch.cuda.is_available():
+        pytest.skip("torch sees no GPU")
+    R, Cc, N = sym.R, sym.C, sym.N
+
+    @kernel(work_shape=(R, Cc))
+    def gated(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT], out: Buffer[R, Cc, DT]):
+        x, y = gr.work_offset
+        ta, tb = gr.load(a[x:, y:], shape=gr.shape), gr.load(b[x:, y:], shape=gr.shape)
+        gr.store(out[x:, y:], np.maximum(ta, np.float32(0)) * tb + ta)
+
+    g = torch.Generator(device="cuda").manual_seed(3)
+    a = torch.randn(257, 1031, device="cuda", generator=g)
+    b = torch.randn(257, 1031, device="cuda", generator=g)
+    out = torch.full_like(a, 7.0)
+    torch.cuda.synchronize()
+    gated(a, b, out)
+    want = torch.clamp_min(a, 0) * b + a              # two roundings, like the kernel
+    assert torch.equal(out, want)
+    # a column window of the tensors: strided rows
+    out2 = torch.full_like(a, 7.0)
+    torch.cuda.synchronize()
+    gated(a[:, :500], b[:, :500], out2[:, :500])
+    assert torch.equal(out2[:, :500], want[:, :500]) and bool((out2[:, 500:] == 7.0).all())
+
+    @kernel(work_shape=N, group_shape=256)
+    def sumsq(gr: CurrentGroup, x: Buffer[N, DT], result: Buffer[1, DT]):
+        o, t = gr.work_offset[0], None
+        t = gr.load(x[o:], shape=gr.shape[0])
+        atomic_ref(result)[0] += (t * t).sum()
+
+    v = torch.randn(1_000_003, device="cuda", generator=g, dtype=torch.float16)
+    res = torch.zeros(1, device="cuda")
+    torch.cuda.synchronize()
+    sumsq(v, res)
+    sq = (v * v).double()                              # fp16 products, as the tile arithmetic does
+    assert abs(res.item() - sq.sum().item()) <= 64 * 2.0 ** -24 * sq.sum().item()
+
+
 def test_vector_add_same_body_on_gpu_and_on_the_host_executor():
     N = sym.N
 
