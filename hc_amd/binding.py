@@ -15,6 +15,7 @@ structurally:
                fused map kernel
     sum        atomic_ref(r)[i] += f(load a, ...).sum(): the same programs, reduced
                with one fp32 atomic addition per workgroup
+    distance   store(norm(a[:, None, :] - b[None, :, :], axis=2))          fp32
 
 Every load and the store must walk their buffers tile by tile: the start along a
 dimension is either 0 or group_id[i] * tile_extent, so that the tiles of all
@@ -536,6 +537,40 @@ def match_map(dst_view, value, n_groups):
     return make
 
 
+def match_pairwise(dst_view, value, n_groups):
+    """out[m, n] = ||a[m, :] - b[n, :]||: the body of
+    python/hckernel/tests/test_examples.py:270-301."""
+    if not (_is(value, "norm", 1) and value.attrs.get("axes") == (2,) and
+            not value.attrs.get("keepdims") and _is(value.args[0], "sub", 2)):
+        return None
+    ea, eb = value.args[0].args
+    if not (_is(ea, "slice", 1) and _is(eb, "slice", 1) and
+            ea.attrs["key"] == ((None, None, None), "new", (None, None, None)) and
+            eb.attrs["key"] == ("new", (None, None, None), (None, None, None))):
+        return None
+    la, lb = ea.args[0], eb.args[0]
+    if not (_is(la, "load") and _is(lb, "load")):
+        return None
+    if {la.dtype_name, lb.dtype_name, dst_view.base.dtype_name} != {"float32"}:
+        raise NoNativeKernel("pairwise distances have a native kernel for float32 only")
+    wa = window_of(la.attrs["view"], la.shape, n_groups)
+    wb = window_of(lb.attrs["view"], lb.shape, n_groups)
+    wo = window_of(dst_view, value.shape, n_groups)
+    d = wa.extent[1]
+    if wa.driver[1] is not None or wb.driver[1] is not None or wb.extent[1] != d or \
+            d != la.attrs["view"].base.shape[1] or d != lb.attrs["view"].base.shape[1]:
+        raise NoNativeKernel("pairwise distances need tiles that hold whole rows of a and b")
+    if wo.driver != (wa.driver[0], wb.driver[0]) or wo.driver[0] == wo.driver[1]:
+        raise NoNativeKernel("the output tiles must be walked by the a-row and b-row group dims")
+    m, n = min(wo.extent[0], wa.extent[0]), min(wo.extent[1], wb.extent[0])
+
+    def make(mem, ctx):
+        return [rt.plan_pairwise_dist_f32(_Arr(_sub(mem[wa.buffer], (m, d)), ctx),
+                                          _Arr(_sub(mem[wb.buffer], (n, d)), ctx),
+                                          _Arr(_sub(mem[wo.buffer], (m, n)), ctx))]
+    return make
+
+
 # ---------------------------------------------------------------------------
 # atomic_ref(result)[i] += <elementwise expression>.sum()
 # ---------------------------------------------------------------------------
@@ -634,7 +669,7 @@ def bind(stores, n_groups, atomics=()):
         makers = []
         for view, value in stores:
             for matcher in (match_copy, match_add, match_fma, match_softmax, match_gemm,
-                            match_map):
+                            match_pairwise, match_map):
                 mk = matcher(view, value, n_groups)
                 if mk is not None:
                     makers.append(mk)

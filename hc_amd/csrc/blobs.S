@@ -18,6 +18,7 @@ hcamd_blob_\name\()_end:
         hcamd_blob copy
         hcamd_blob elementwise
         hcamd_blob map
+        hcamd_blob distance
         hcamd_blob softmax
         hcamd_blob quantize
         hcamd_blob gemm

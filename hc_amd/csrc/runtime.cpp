@@ -137,6 +137,7 @@ Device::~Device() {
 HCAMD_BLOB(copy)
 HCAMD_BLOB(elementwise)
 HCAMD_BLOB(map)
+HCAMD_BLOB(distance)
 HCAMD_BLOB(softmax)
 HCAMD_BLOB(quantize)
 HCAMD_BLOB(gemm)
@@ -149,7 +150,8 @@ struct Blob {
 };
 #define HCAMD_BLOB(n) {#n, hcamd_blob_##n##_begin, hcamd_blob_##n##_end}
 const Blob kBlobs[] = {HCAMD_BLOB(copy), HCAMD_BLOB(elementwise),
-                       HCAMD_BLOB(map), HCAMD_BLOB(softmax), HCAMD_BLOB(quantize),
+                       HCAMD_BLOB(map), HCAMD_BLOB(distance),
+                       HCAMD_BLOB(softmax), HCAMD_BLOB(quantize),
                        HCAMD_BLOB(gemm)};
 #undef HCAMD_BLOB
 constexpr size_t kNumBlobs = sizeof(kBlobs) / sizeof(kBlobs[0]);
@@ -1072,6 +1074,38 @@ int hcamdLaunchMapSum(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
                       size_t rows, size_t cols) noexcept {
   return launchMap(q, true, prog, nInstr, inputs, inputTypes, inputLd, nInputs,
                    cell, HCAMD_F32, cols, rows, cols);
+}
+
+int hcamdLaunchPairwiseDistF32(OlQueue q, const float *a, size_t lda,
+                               const float *b, size_t ldb, float *out,
+                               size_t ldo, size_t m, size_t n,
+                               size_t d) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  if (m == 0 || n == 0)
+    return 0;
+  if (!a || !b || !out) {
+    dev->report("hcamdLaunchPairwiseDistF32: null pointer");
+    return 1;
+  }
+  if ((m > 1 && lda < d) || (n > 1 && ldb < d) || (m > 1 && ldo < n)) {
+    dev->report("hcamdLaunchPairwiseDistF32: leading dimension smaller than the row");
+    return 1;
+  }
+  const size_t gy = ceilDiv(m, 64);
+  if (gy > 65535) {
+    dev->report("hcamdLaunchPairwiseDistF32: more than 65535 x 64 rows");
+    return 1;
+  }
+  Kernel *k = builtinKernel(dev, "distance", "hcamd_pairwise_dist_f32");
+  if (!k)
+    return 1;
+  void *args[] = {&a, &lda, &b, &ldb, &out, &ldo, &m, &n, &d};
+  const size_t grid[3] = {ceilDiv(n, 64), gy, 1};
+  const size_t block[3] = {256, 1, 1};
+  return launch(queue, k, grid, block, args, 0);
 }
 
 int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,

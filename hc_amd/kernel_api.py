@@ -427,6 +427,10 @@ class Tile:
                              kwargs.get("keepdims", False))
         if name == "transpose" and len(args) == 1:
             return Tile.wrap(args[0]).T
+        if name == "norm" and kwargs.get("ord", args[1] if len(args) > 1 else None) is None:
+            x = Tile.wrap(args[0])             # numpy.linalg.norm: the 2-norm along an axis
+            return x._reduce("norm", kwargs.get("axis", args[2] if len(args) > 2 else None),
+                             kwargs.get("keepdims", False))
         raise TraceError(f"numpy.{name} is not supported in a GPU kernel")
 
     # -- methods kernels use ---------------------------------------------------------
@@ -470,14 +474,19 @@ class Tile:
     def __getitem__(self, key):
         if not isinstance(key, tuple):
             key = (key,)
-        key = key + (slice(None),) * (len(self.shape) - len(key))
-        shape = []
-        for k, n in zip(key, self.shape):
-            if isinstance(k, slice):
-                shape.append(len(range(*k.indices(n))))
+        n_old = sum(1 for k in key if k is not None)
+        key = key + (slice(None),) * (len(self.shape) - n_old)
+        shape, dims = [], iter(self.shape)
+        for k in key:
+            if k is None:                      # numpy.newaxis
+                shape.append(1)
+            elif isinstance(k, slice):
+                shape.append(len(range(*k.indices(next(dims)))))
             else:
                 int(k)
-        norm = tuple((k.start, k.stop, k.step) if isinstance(k, slice) else int(k) for k in key)
+                next(dims)
+        norm = tuple("new" if k is None else
+                     (k.start, k.stop, k.step) if isinstance(k, slice) else int(k) for k in key)
         return Tile("slice", (self,), shape, self.dtype_name, key=norm)
 
     def reshape(self, *shape):

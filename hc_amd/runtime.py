@@ -102,6 +102,8 @@ class MapInstr(C.Structure):
 
 hcamdLaunchMap = _sig(_rt, "hcamdLaunchMap", _int, _vp, C.POINTER(MapInstr), _sz,
                       C.POINTER(_vp), C.POINTER(_int), _sz_p, _sz, _vp, _int, _sz, _sz, _sz)
+hcamdLaunchPairwiseDistF32 = _sig(_rt, "hcamdLaunchPairwiseDistF32", _int, _vp, _vp, _sz, _vp,
+                                  _sz, _vp, _sz, _sz, _sz, _sz)
 hcamdLaunchMapSum = _sig(_rt, "hcamdLaunchMapSum", _int, _vp, C.POINTER(MapInstr), _sz,
                          C.POINTER(_vp), C.POINTER(_int), _sz_p, _sz, _vp, _sz, _sz)
 hcamdConvertPyArray = _sig(_py, "hcamdConvertPyArray", _int, C.py_object, _int, _vp,
@@ -460,6 +462,20 @@ def plan_map_sum(program, inputs, cell, index: int = 0, types=None) -> Plan:
     return Plan(ctx, hcamdLaunchMapSum,
                 (ctx.queue, prog, len(program), ptrs, tys, lds, n_in, mc.ptr + 4 * index,
                  rows, cols), "hcamdLaunchMapSum", (arrays, cell, prog, ptrs, tys, lds))
+
+
+def plan_pairwise_dist_f32(a, b, out) -> Plan:
+    """out[i, j] = ||a[i, :] - b[j, :]||_2 for fp32 a[m, d], b[n, d], out[m, n]."""
+    ctx = _ctx_of(a, b, out)
+    ma, mb, mo = as_memref(a, 2), as_memref(b, 2), as_memref(out, 2)
+    for m, n in ((ma, "a"), (mb, "b"), (mo, "out")):
+        _expect(m, 4, n)
+    (m, d, lda), (n, d2, ldb), (mo_r, mo_c, ldo) = _rows_cols(ma), _rows_cols(mb), _rows_cols(mo)
+    if d != d2 or (mo_r, mo_c) != (m, n):
+        raise HcRuntimeError("pairwise_dist_f32: shape mismatch")
+    return Plan(ctx, hcamdLaunchPairwiseDistF32,
+                (ctx.queue, ma.ptr, lda, mb.ptr, ldb, mo.ptr, ldo, m, n, d),
+                "hcamdLaunchPairwiseDistF32", (a, b, out))
 
 
 def plan_softmax_f32(x, y) -> Plan:

@@ -312,6 +312,16 @@ int hcamdLaunchMapSum(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
                       const size_t *inputLd, size_t nInputs, float *cell,
                       size_t rows, size_t cols) HCAMD_NOEXCEPT;
 
+/* Pairwise Euclidean distances, fp32: out[i, j] = sqrt(sum_k (a[i,k] - b[j,k])^2)
+ * for a[m, d], b[n, d] row-major, out[m, n].  The expression of
+ * python/hckernel/tests/test_examples.py:270-301
+ * (numpy.linalg.norm(a[:, None, :] - b[None, :, :], axis=2)); differences are
+ * formed explicitly, sums run over d in ascending order per output. */
+int hcamdLaunchPairwiseDistF32(OlQueue q, const float *a, size_t lda,
+                               const float *b, size_t ldb, float *out,
+                               size_t ldo, size_t m, size_t n,
+                               size_t d) HCAMD_NOEXCEPT;
+
 /* Row softmax, fp32: y[r,:] = exp(x[r,:]-max(x[r,:])) / sum(exp(...)).
  * Expression of python/hckernel/tests/test_examples.py:330-335. */
 int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,

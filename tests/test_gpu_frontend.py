@@ -430,6 +430,33 @@ def test_dot_product_through_the_map_sum_kernel():
         assert abs(float(got[2]) - 3.0 - prod.sum()) <= 64 * 2.0 ** -24 * np.abs(prod).sum()
 
 
+def test_pairwise_distance_body_of_the_reference_example():
+    from test_kernel_frontend import _pairwise_kernel
+    m, n, d = 16, 32, 8                                 # the reference's input, in fp32
+    a = (2 * np.arange(m * d).reshape(m, d) / (m * d)).astype(np.float32)
+    b = (np.arange(n * d).reshape(n, d) / (n * d)).astype(np.float32)
+    out = rt.to_device(np.full((m, n), -1, np.float32))
+    _pairwise_kernel(kernel)(rt.to_device(a), rt.to_device(b), out, (8, 8))
+    host = np.zeros((m, n), np.float32)
+    _pairwise_kernel(sim_kernel)(a, b, host, (8, 8))
+    want = np.linalg.norm(a[:, None, :].astype(np.float64) - b[None, :, :], axis=2)
+    assert_allclose(host, want, rtol=1e-6)
+    assert_allclose(out.to_host(), want, rtol=1e-6, atol=1e-7)
+    # ragged sizes, several panels of d, tunables
+    rng = np.random.default_rng(41)
+    m, n, d = 201, 333, 77
+    a, b = rng.standard_normal((m, d)).astype(np.float32), rng.standard_normal((n, d)).astype(np.float32)
+    out = rt.to_device(np.full((m, n), -1, np.float32))
+    _pairwise_kernel(kernel).parametrize({sym.MI: 2, sym.NI: 3})(rt.to_device(a), rt.to_device(b),
+                                                               out, (8, 4))
+    want = np.linalg.norm(a[:, None, :].astype(np.float64) - b[None, :, :], axis=2)
+    assert_allclose(out.to_host(), want, rtol=2e-6)
+    # a point and itself: exactly zero, not the residue of a cancellation
+    out = rt.to_device(np.full((m, m), -1, np.float32))
+    _pairwise_kernel(kernel)(rt.to_device(a), rt.to_device(a), out, (8, 8))
+    assert (np.diag(out.to_host()) == 0).all()
+
+
 def test_unsupported_body_raises_instead_of_running_on_the_cpu():
     N = sym.N
 

@@ -311,6 +311,30 @@ def test_fma_full_benchmark_size(ctx):
 
 
 # ---------------------------------------------------------------------------
+# pairwise distances
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("mnd", [(1, 1, 1), (5, 7, 3), (64, 64, 32), (65, 130, 33), (300, 200, 128),
+                                 (1000, 1, 500)])
+def test_pairwise_distances_against_fp64(ctx, mnd):
+    m, n, d = mnd
+    rng = np.random.default_rng(sum(mnd))
+    a = rng.standard_normal((m, d)).astype(np.float32)
+    b = rng.standard_normal((n, d)).astype(np.float32)
+    out = poisoned((m + 3, n + 5), np.float32)
+    rt.plan_pairwise_dist_f32(dev(a), dev(b), _View(out, (m, n), 0, (n + 5, 1))).launch(sync=True)
+    got = out.to_host()
+    want = np.sqrt(((a[:, None, :].astype(np.float64) - b[None, :, :]) ** 2).sum(axis=2))
+    # d fused multiply-adds in fp32, then a correctly rounded square root
+    assert_allclose(got[:m, :n], want, rtol=(d + 2) * 2.0 ** -24)
+    p = poison_value(np.float32)
+    assert (got[m:].view(np.uint32) == p.view(np.uint32)).all()
+    assert (got[:, n:].view(np.uint32) == p.view(np.uint32)).all()
+    # what NumPy itself computes in fp32 is equally close to the exact result
+    ref32 = np.linalg.norm(a[:, None, :] - b[None, :, :], axis=2)
+    assert_allclose(ref32, want, rtol=(d + 2) * 2.0 ** -24)
+
+
+# ---------------------------------------------------------------------------
 # fused elementwise map (postfix programs)
 # ---------------------------------------------------------------------------
 def I(name, arg=0, imm=0.0):

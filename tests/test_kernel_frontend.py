@@ -419,3 +419,32 @@ def test_reference_reduction_bodies_bind_to_the_map_sum_kernel(ctx):
             k.plan(a, res4, ctx=ctx)
     with pytest.raises(NoNativeKernel, match="float32"):
         reduction_1.plan(a, FakeDev((1,), "float16"), 8, ctx=ctx)
+
+
+def _pairwise_kernel(deco):
+    # body of python/hckernel/tests/test_examples.py:270-292
+    M, N, D, GM, GN, MI, NI = sym.M, sym.N, sym.D, sym.GM, sym.GN, sym.MI, sym.NI
+    tun = (TunableParam(MI, 1, range(1, 8)), TunableParam(NI, 1, range(1, 8)))
+
+    @deco(work_shape=(cdiv(M, MI), cdiv(N, NI)), group_shape=(GM, GN), tunables=tun)
+    def pw_distance(gr: CurrentGroup, a: Buffer[M, D, DT], b: Buffer[N, D, DT],
+                    out: Buffer[M, N, DT], gshape: (GM, GN)):
+        m_start, n_start = gr.work_offset[0] * MI, gr.work_offset[1] * NI
+        m_block, n_block = gr.shape[0] * MI, gr.shape[1] * NI
+        a_view = gr.load(a[m_start:, :], shape=(m_block, D))
+        b_view = gr.load(b[n_start:, :], shape=(n_block, D))
+        diff = a_view[:, None, :] - b_view[None, :, :]
+        gr.store(out[m_start:, n_start:], np.linalg.norm(diff, axis=2))
+    return pw_distance
+
+
+def test_pairwise_distance_example_binds_to_the_distance_kernel(ctx):
+    k = _pairwise_kernel(kernel)
+    a, b, out = FakeDev((16, 8), "float32"), FakeDev((32, 8), "float32"), FakeDev((16, 32), "float32")
+    (p,) = k.plan(a, b, out, (8, 8), ctx=ctx)
+    assert p.fn is rt.hcamdLaunchPairwiseDistF32
+    assert p.args == (ctx.queue, a.ptr, 8, b.ptr, 8, out.ptr, 32, 16, 32, 8)
+    (p,) = k.parametrize({sym.MI: 2, sym.NI: 4}).plan(a, b, out, (4, 2), ctx=ctx)
+    assert p.args[7:] == (16, 32, 8)
+    with pytest.raises(NoNativeKernel, match="float32"):
+        k.plan(*(FakeDev(s, "float16") for s in ((16, 8), (32, 8), (16, 32))), (8, 8), ctx=ctx)
