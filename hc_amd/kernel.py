@@ -32,6 +32,7 @@ from collections.abc import Iterable
 import sympy
 
 from . import runtime as rt
+from .autotune import TunedParams, autotune
 from .binding import NoNativeKernel, bind
 from .indexing import sym
 from .kernel_api import (Buffer, BufferProxy, CurrentGroup, CurrentGroup1, CurrentGroup2,
@@ -41,7 +42,8 @@ from .typename import Typename, typename
 
 __all__ = ["kernel", "sym", "typename", "Buffer", "CurrentGroup", "CurrentGroup1",
            "CurrentGroup2", "CurrentGroup3", "CurrentSubGroup", "CurrentWorkitem",
-           "TunableParam", "atomic_ref", "create_mapping", "NoNativeKernel", "TraceError"]
+           "TunableParam", "atomic_ref", "create_mapping", "NoNativeKernel", "TraceError",
+           "autotune", "TunedParams"]
 
 DEFAULT_SUBGROUP_SIZE = 64      # mlir/lib/Transforms/LowerHKernel.cpp:539-544
 
@@ -173,11 +175,18 @@ class GpuKernel:
         self._defaults = {t.sym: t.default for t in tun}
         self._cache = {}
         self.last_plans = []
+        self.variants = {}              # {kernel family: variant number}
 
     def parametrize(self, tuned):
-        return GpuKernel(self.func, self.work_shape, self.group_shape, self.subgroup_size,
-                         self.literals, self.tunables, self.backend, self.device,
-                         {**self.tuned, **tuned})
+        """A copy of the kernel with tunable symbols fixed ({symbol: value},
+        python/hckernel/kernel_sim.py:165-175).  The result of
+        hc_amd.autotune.autotune() also carries the variants of the hand-written
+        kernels to use; they are selected around every call."""
+        k = GpuKernel(self.func, self.work_shape, self.group_shape, self.subgroup_size,
+                      self.literals, self.tunables, self.backend, self.device,
+                      {**self.tuned, **tuned})
+        k.variants = {**self.variants, **getattr(tuned, "variants", {})}
+        return k
 
     # -- the work ------------------------------------------------------------------
     def _signature(self, args, memrefs):
@@ -249,8 +258,14 @@ class GpuKernel:
 
     def __call__(self, *args, sync: bool = True):
         plans = self.plan(*args)
-        for p in plans:
-            p.launch()
+        for family, v in self.variants.items():
+            rt.set_variant(family, v)
+        try:
+            for p in plans:
+                p.launch()
+        finally:
+            for family in self.variants:
+                rt.set_variant(family, 0)
         self.last_plans = plans
         if sync and plans:
             plans[0].ctx.synchronize()

@@ -457,6 +457,51 @@ def test_pairwise_distance_body_of_the_reference_example():
     assert (np.diag(out.to_host()) == 0).all()
 
 
+def test_autotune_flow_of_the_language_reference(tmp_path):
+    # docs/langref.md:516-571: tunables on the decorator, autotune, parametrize, save / load
+    from hc_amd.kernel import autotune
+    WS, GS, N = sym.WS, sym.GS, sym.N
+    TP = TunableParam
+
+    @kernel(work_shape=cdiv(WS, N), group_shape=GS,
+            tunables=(TP(GS, 64, range(64, 1024, 320)), TP(N, 16, range(16, 256, 80))))
+    def reduction(group: CurrentGroup, a: Buffer[WS, DT], result: Buffer[1, DT]):
+        temp_result = group.zeros(group.size, dtype=a.dtype)
+        for i in range(N):
+            work_offset = group.work_offset[0] * N + i * group.size
+            temp_result += group.load(a[work_offset:], shape=group.size)
+        atomic_ref(result)[0] += temp_result.sum()
+
+    a = np.arange(200_000, dtype=np.float32) % 7
+    scratch = rt.to_device(np.zeros(1, np.float32))
+    tparams = autotune(reduction, rt.to_device(a), scratch, iters=3, warmup=1)
+    assert tparams[GS] in range(64, 1024, 320) and tparams[N] in range(16, 256, 80)
+    assert tparams.device.startswith("gfx950") and tparams.microseconds > 0
+    tparams.save(tmp_path / "reduction.json")
+    tuned = reduction.parametrize(autotune.load(tmp_path / "reduction.json"))
+    result = rt.to_device(np.zeros(1, np.float32))
+    tuned(rt.to_device(a), result)
+    assert result.to_host()[0] == a.sum()               # small integers: exact in any order
+
+    # a kernel family with variants: the chosen one is applied around the call
+    Nn = sym.NN
+
+    @kernel(work_shape=Nn, group_shape=256)
+    def vadd(gr: CurrentGroup, x: Buffer[Nn, DT], y: Buffer[Nn, DT], z: Buffer[Nn, DT]):
+        o, g = gr.work_offset[0], gr.shape[0]
+        gr.store(z[o:], gr.load(x[o:], shape=g) + gr.load(y[o:], shape=g))
+
+    x, y = cf.inputs_c1(1_000_003)
+    dx, dy, dz = rt.to_device(x), rt.to_device(y), rt.DeviceArray(x.shape, np.float32)
+    tp = autotune(vadd, dx, dy, dz, iters=5, warmup=1)
+    assert set(tp.variants) <= {"add"} and all(1 <= v <= 8 for v in tp.variants.values())
+    vadd.parametrize(tp)(dx, dy, dz)
+    assert_array_equal(dz.to_host().view(np.uint32), cf.np_add(x, y).view(np.uint32))
+    rt.set_variant("add", 0)
+    vadd(dx, dy, dz)
+    assert rt.last_kernel_name() == "hcamd_add_f32_v4_nt"     # the default is back
+
+
 def test_unsupported_body_raises_instead_of_running_on_the_cpu():
     N = sym.N
 

@@ -448,3 +448,27 @@ def test_pairwise_distance_example_binds_to_the_distance_kernel(ctx):
     assert p.args[7:] == (16, 32, 8)
     with pytest.raises(NoNativeKernel, match="float32"):
         k.plan(*(FakeDev(s, "float16") for s in ((16, 8), (32, 8), (16, 32))), (8, 8), ctx=ctx)
+
+
+def test_tuned_params_round_trip_and_parametrize(tmp_path, ctx):
+    from hc_amd.kernel import TunedParams, autotune
+    WS, GS, N = sym.WS, sym.GS, sym.N
+    t = TunedParams({N: 4, GS: 128}, {"add": 7}, "gfx950", 12.5)
+    t.save(tmp_path / "tuned.json")
+    back = autotune.load(tmp_path / "tuned.json")
+    assert dict(back) == {N: 4, GS: 128} and back.variants == {"add": 7}
+    assert back.device == "gfx950" and back.microseconds == 12.5
+
+    @kernel(work_shape=cdiv(WS, N), group_shape=GS,
+            tunables=(TunableParam(GS, 64, range(64, 1024, 64)), TunableParam(N, 16, range(16, 256, 16))))
+    def reduction(group: CurrentGroup, a: Buffer[WS, DT], result: Buffer[1, DT]):
+        temp_result = group.zeros(group.size, dtype=a.dtype)
+        for i in range(N):
+            work_offset = group.work_offset[0] * N + i * group.size
+            temp_result += group.load(a[work_offset:], shape=group.size)
+        atomic_ref(result)[0] += temp_result.sum()
+
+    tuned = reduction.parametrize(back)          # the spelling of docs/langref.md:540-550
+    assert tuned.tuned == {N: 4, GS: 128} and tuned.variants == {"add": 7}
+    (p,) = tuned.plan(FakeDev((5000,), "float32"), FakeDev((1,), "float32"), ctx=ctx)
+    assert p.fn is rt.hcamdLaunchMapSum and p.args[8:] == (1, 5000)
