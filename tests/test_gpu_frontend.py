@@ -502,6 +502,35 @@ def test_autotune_flow_of_the_language_reference(tmp_path):
     assert rt.last_kernel_name() == "hcamd_add_f32_v4_nt"     # the default is back
 
 
+def test_blocked_dot_on_torch_bfloat16_tensors():
+    torch = pytest.importorskip("torch")
+    if not torch.cuda.is_available():
+        pytest.skip("torch sees no GPU")
+    M, N, K, KB = sym.M, sym.N, sym.K, sym.KB
+    KI = cdiv(K, KB)
+
+    @kernel(work_shape=(cdiv(M, 4), cdiv(N, 4)), group_shape=(16, 16),
+            tunables=TunableParam(KB, 64, range(8, 128)))
+    def dot(gr: CurrentGroup, a: Buffer[M, K, DT], bt: Buffer[N, K, DT], out: Buffer[M, N, DT]):
+        m0, n0 = gr.work_offset[0] * 4, gr.work_offset[1] * 4
+        mb, nb = gr.shape[0] * 4, gr.shape[1] * 4
+        r = gr.zeros(shape=(mb, nb), dtype=np.float32)
+        for k in range(KI):
+            r += np.dot(gr.load(a[m0:, k * KB:], shape=(mb, KB)),
+                        gr.load(bt[n0:, k * KB:], shape=(nb, KB)).T)
+        gr.store(out[m0:, n0:], r)
+
+    g = torch.Generator(device="cuda").manual_seed(5)
+    a = (0.02 * torch.randn(512, 768, device="cuda", generator=g)).bfloat16()
+    bt = (0.02 * torch.randn(256, 768, device="cuda", generator=g)).bfloat16()
+    out = torch.zeros(512, 256, device="cuda", dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+    dot(a, bt, out)
+    assert rt.last_kernel_name().startswith("hcamd_gemm_bf16_p256x256")
+    want = a.float() @ bt.float().T
+    torch.testing.assert_close(out.float(), want, rtol=1e-2, atol=1e-2 * 0.02 * 0.02 * 768 ** 0.5)
+
+
 def test_unsupported_body_raises_instead_of_running_on_the_cpu():
     N = sym.N
 
