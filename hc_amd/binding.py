@@ -9,7 +9,7 @@ structurally:
     fma        store((f32 a * f32 b + f32 c) -> f16)                   fp16 storage
     softmax    store(exp(x - max_row x) / sum_row exp(x - max_row x))  fp32 rows
     quantize   store(int8 clip(rint(f32 x / s), -127, 127)), s = max_row|x| / 127
-    gemm       store(sum_k dot(load A[m, k-chunk], load Bt[n, k-chunk].T))   bf16
+    gemm       store(sum_k dot(load A[m, k-chunk], load Bt[n, k-chunk].T))   bf16 / fp16
     map        store(f(load a, load b, ...)) for any other elementwise f over up to
                four fp32 / fp16 operands: compiled to a postfix program for the
                fused map kernel
@@ -318,9 +318,10 @@ def _flatten_sum(t: Tile, out: list):
 
 
 def match_gemm(dst_view, value, n_groups):
-    if dst_view.base.dtype_name != "bfloat16":
+    elem = dst_view.base.dtype_name
+    if elem not in ("bfloat16", "float16"):
         return None
-    value = _strip_cast(value, "bfloat16")
+    value = _strip_cast(value, elem)
     terms: list = []
     _flatten_sum(value, terms)
     dots = [t for t in terms if not _const(t, 0)]
@@ -331,11 +332,20 @@ def match_gemm(dst_view, value, n_groups):
     for d in dots:
         d = d.args[0] if d.op == "astype" else d
         la, lbt = d.args
+        # operands may be widened to fp32 first (`load(...).astype(float32)`): the
+        # MFMA multiplies the stored values exactly and accumulates in fp32 anyway
+        if _leaf(la) is not None:
+            la = _leaf(la)
+        if _is(lbt, "transpose", 1) and _leaf(lbt.args[0]) is not None:
+            lbt = Tile("transpose", (_leaf(lbt.args[0]),), lbt.shape, lbt.dtype_name)
+        elif _is(lbt, "astype", 1) and lbt.dtype_name == "float32" and \
+                _is(lbt.args[0], "transpose", 1):
+            lbt = lbt.args[0]
         if not (_is(la, "load") and _is(lbt, "transpose", 1) and _is(lbt.args[0], "load")):
             raise NoNativeKernel("GEMM is bound for dot(load A[m, k], load Bt[n, k].T): B must "
                                  "be column-major, passed as Bt[N, K]")
         lb = lbt.args[0]
-        if la.dtype_name != "bfloat16" or lb.dtype_name != "bfloat16":
+        if la.dtype_name != elem or lb.dtype_name != elem:
             return None
         va, vb = la.attrs["view"], lb.attrs["view"]
         ka, kb = va.starts[1], vb.starts[1]
@@ -369,10 +379,12 @@ def match_gemm(dst_view, value, n_groups):
         raise NoNativeKernel("C tiles must be walked by the A-row and Bt-row group dims")
     m, n = min(wc.extent[0], wa0.extent[0]), min(wc.extent[1], wb0.extent[0])
 
+    plan = rt.plan_gemm_bf16 if elem == "bfloat16" else rt.plan_gemm_f16
+
     def make(mem, ctx):
-        return [rt.plan_gemm_bf16(_Arr(_sub(mem[a_idx], (m, k_total)), ctx),
-                                  _Arr(_sub(mem[b_idx], (n, k_total)), ctx),
-                                  _Arr(_sub(mem[wc.buffer], (m, n)), ctx))]
+        return [plan(_Arr(_sub(mem[a_idx], (m, k_total)), ctx),
+                     _Arr(_sub(mem[b_idx], (n, k_total)), ctx),
+                     _Arr(_sub(mem[wc.buffer], (m, n)), ctx))]
     return make
 
 

@@ -225,10 +225,29 @@ __device__ __forceinline__ void gemm_tile(const __bf16 *__restrict__ A,
 // ---------------------------------------------------------------------------
 typedef __attribute__((address_space(1))) const void *global_cptr;
 typedef __attribute__((address_space(3))) void *lds_ptr;
-template <int BM, int BN, int WM, int WN, int MF>
+// E is the storage type of A, Bt and C: __bf16 or _Float16 (same tiling, the
+// MFMA of the matching type, round-to-nearest-even on the way out).
+template <class E, int MF, class V, class Acc>
+__device__ __forceinline__ Acc mfma_block(V b, V a, Acc c) {
+  if constexpr (std::is_same<E, __bf16>::value) {
+    if constexpr (MF == 16)
+      return __builtin_amdgcn_mfma_f32_16x16x32_bf16(b, a, c, 0, 0, 0);
+    else
+      return __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, a, c, 0, 0, 0);
+  } else {
+    if constexpr (MF == 16)
+      return __builtin_amdgcn_mfma_f32_16x16x32_f16(b, a, c, 0, 0, 0);
+    else
+      return __builtin_amdgcn_mfma_f32_32x32x16_f16(b, a, c, 0, 0, 0);
+  }
+}
+
+template <class E, int BM, int BN, int WM, int WN, int MF>
 __device__ __forceinline__ void gemm_tile_pipelined(
-    const __bf16 *__restrict__ A, size_t lda, const __bf16 *__restrict__ Bt,
-    size_t ldb, __bf16 *__restrict__ C, size_t ldc, int M, int N, int K) {
+    const E *__restrict__ A, size_t lda, const E *__restrict__ Bt, size_t ldb,
+    E *__restrict__ C, size_t ldc, int M, int N, int K) {
+  typedef E ex8 __attribute__((ext_vector_type(8)));
+  typedef E ex4 __attribute__((ext_vector_type(4)));
   constexpr int kWaves = WM * WN;
   constexpr int kWaveM = BM / WM;
   constexpr int kWaveN = BN / WN;
@@ -258,8 +277,8 @@ __device__ __forceinline__ void gemm_tile_pipelined(
   // ---- global -> LDS ---------------------------------------------------------
   // load i of this wave fills panel rows (i*kWaves + wave)*8 .. +8
   const int ld_row = lane / 8, ld_pchunk = lane % 8;
-  const __bf16 *a_src[kALoads];
-  const __bf16 *b_src[kBLoads];
+  const E *a_src[kALoads];
+  const E *b_src[kBLoads];
 #pragma unroll
   for (int i = 0; i < kALoads; ++i) {
     const int r = (i * kWaves + wave) * 8 + ld_row;
@@ -304,7 +323,7 @@ __device__ __forceinline__ void gemm_tile_pipelined(
     for (int u = 0; u < kSub; ++u)
       coff[h][u] = ((4 * h + (kSub == 1 ? lchunk : 2 * u + lchunk)) ^ lswz) * 16;
 
-  bf16x8 fa[2][kSub][kMI], fb[2][kSub][kNI];
+  ex8 fa[2][kSub][kMI], fb[2][kSub][kNI];
   auto read_frags = [&](int buf, int ks, auto slot) {
     constexpr int S = decltype(slot)::value;
 #pragma unroll
@@ -312,10 +331,10 @@ __device__ __forceinline__ void gemm_tile_pipelined(
       const unsigned char *base = lds + buf * kStageBytes + (ks ? coff[1][u] : coff[0][u]);
 #pragma unroll
       for (int j = 0; j < kNI; ++j)
-        fb[S][u][j] = *reinterpret_cast<const bf16x8 *>(base + b_off[j]);
+        fb[S][u][j] = *reinterpret_cast<const ex8 *>(base + b_off[j]);
 #pragma unroll
       for (int i = 0; i < kMI; ++i)
-        fa[S][u][i] = *reinterpret_cast<const bf16x8 *>(base + a_off[i]);
+        fa[S][u][i] = *reinterpret_cast<const ex8 *>(base + a_off[i]);
     }
   };
 
@@ -335,12 +354,7 @@ __device__ __forceinline__ void gemm_tile_pipelined(
       for (int i = 0; i < kMI; ++i)
 #pragma unroll
         for (int j = 0; j < kNI; ++j) {
-          if constexpr (MF == 16)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                fb[S][u][j], fa[S][u][i], acc[i][j], 0, 0, 0);
-          else
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                fb[S][u][j], fa[S][u][i], acc[i][j], 0, 0, 0);
+          acc[i][j] = mfma_block<E, MF>(fb[S][u][j], fa[S][u][i], acc[i][j]);
         }
   };
   using Slot0 = std::integral_constant<int, 0>;
@@ -409,34 +423,37 @@ __device__ __forceinline__ void gemm_tile_pipelined(
   const int n_base = tn * BN + wave_n + lchunk * 4;
 #pragma unroll
   for (int i = 0; i < kMI; ++i) {
-    __bf16 *crow = C + (size_t)(m_base + i * MF) * ldc + n_base;
+    E *crow = C + (size_t)(m_base + i * MF) * ldc + n_base;
 #pragma unroll
     for (int j = 0; j < kNI; ++j) {
 #pragma unroll
       for (int g = 0; g < kAccRegs / 4; ++g) {
-        bf16x4 o;
+        ex4 o;
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          o[e] = (__bf16)acc[i][j][4 * g + e];
-        *reinterpret_cast<bf16x4 *>(crow + j * MF + g * 8) = o;
+          o[e] = (E)acc[i][j][4 * g + e];
+        *reinterpret_cast<ex4 *>(crow + j * MF + g * 8) = o;
       }
     }
   }
 }
 } // namespace
 
-#define HCAMD_GEMM_P(NAME, BM, BN, WM, WN, MF)                                 \
+#define HCAMD_GEMM_P(NAME, E, BM, BN, WM, WN, MF)                              \
   extern "C" __global__ __launch_bounds__(WM *WN * 64) void NAME(              \
-      const __bf16 *A, size_t lda, const __bf16 *Bt, size_t ldb, __bf16 *C,    \
-      size_t ldc, int M, int N, int K) {                                       \
-    gemm_tile_pipelined<BM, BN, WM, WN, MF>(A, lda, Bt, ldb, C, ldc, M, N, K); \
+      const E *A, size_t lda, const E *Bt, size_t ldb, E *C, size_t ldc,       \
+      int M, int N, int K) {                                                   \
+    gemm_tile_pipelined<E, BM, BN, WM, WN, MF>(A, lda, Bt, ldb, C, ldc, M, N,  \
+                                               K);                             \
   }
-HCAMD_GEMM_P(hcamd_gemm_bf16_p256x256_w2x4, 256, 256, 2, 4, 16)
-HCAMD_GEMM_P(hcamd_gemm_bf16_p256x256_w4x2, 256, 256, 4, 2, 16)
-HCAMD_GEMM_P(hcamd_gemm_bf16_p128x128_w2x2, 128, 128, 2, 2, 16)
-HCAMD_GEMM_P(hcamd_gemm_bf16_p256x128_w2x2, 256, 128, 2, 2, 16)
-HCAMD_GEMM_P(hcamd_gemm_bf16_p32_256x256_w2x4, 256, 256, 2, 4, 32)
-HCAMD_GEMM_P(hcamd_gemm_bf16_p32_256x256_w4x2, 256, 256, 4, 2, 32)
+HCAMD_GEMM_P(hcamd_gemm_bf16_p256x256_w2x4, __bf16, 256, 256, 2, 4, 16)
+HCAMD_GEMM_P(hcamd_gemm_bf16_p256x256_w4x2, __bf16, 256, 256, 4, 2, 16)
+HCAMD_GEMM_P(hcamd_gemm_bf16_p128x128_w2x2, __bf16, 128, 128, 2, 2, 16)
+HCAMD_GEMM_P(hcamd_gemm_bf16_p256x128_w2x2, __bf16, 256, 128, 2, 2, 16)
+HCAMD_GEMM_P(hcamd_gemm_bf16_p32_256x256_w2x4, __bf16, 256, 256, 2, 4, 32)
+HCAMD_GEMM_P(hcamd_gemm_bf16_p32_256x256_w4x2, __bf16, 256, 256, 4, 2, 32)
+HCAMD_GEMM_P(hcamd_gemm_f16_p256x256_w2x4, _Float16, 256, 256, 2, 4, 16)
+HCAMD_GEMM_P(hcamd_gemm_f16_p128x128_w2x2, _Float16, 128, 128, 2, 2, 16)
 
 #define HCAMD_GEMM(NAME, BM, BN, WM, WN, SH)                                   \
   extern "C" __global__ __launch_bounds__(WM * WN * 64) void NAME(             \
@@ -455,9 +472,10 @@ HCAMD_GEMM(hcamd_gemm_bf16_256x128_w2x2_s0, 256, 128, 2, 2, 0)
 // 64 x 64 tile of C per workgroup, a 4 x 4 block per thread, fp32 FMAs on
 // LDS-staged 64 x 16 panels, every access bounds-checked.  Correct everywhere,
 // fast nowhere; it exists for the shapes the tiled kernel does not take.
-extern "C" __global__ __launch_bounds__(256) void hcamd_gemm_bf16_general(
-    const __bf16 *A, size_t lda, const __bf16 *Bt, size_t ldb, __bf16 *C,
-    size_t ldc, int M, int N, int K) {
+template <class E>
+__device__ __forceinline__ void gemm_general(const E *A, size_t lda, const E *Bt,
+                                             size_t ldb, E *C, size_t ldc, int M,
+                                             int N, int K) {
   constexpr int T = 64, KB = 16;
   __shared__ float sa[KB][T + 1];
   __shared__ float sb[KB][T + 1];
@@ -494,6 +512,17 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_gemm_bf16_general(
     for (int j = 0; j < 4; ++j) {
       const int gm = m0 + ty * 4 + i, gn = n0 + tx * 4 + j;
       if (gm < M && gn < N)
-        C[(size_t)gm * ldc + gn] = (__bf16)acc[i][j];
+        C[(size_t)gm * ldc + gn] = (E)acc[i][j];
     }
+}
+
+extern "C" __global__ __launch_bounds__(256) void hcamd_gemm_bf16_general(
+    const __bf16 *A, size_t lda, const __bf16 *Bt, size_t ldb, __bf16 *C,
+    size_t ldc, int M, int N, int K) {
+  gemm_general<__bf16>(A, lda, Bt, ldb, C, ldc, M, N, K);
+}
+extern "C" __global__ __launch_bounds__(256) void hcamd_gemm_f16_general(
+    const _Float16 *A, size_t lda, const _Float16 *Bt, size_t ldb, _Float16 *C,
+    size_t ldc, int M, int N, int K) {
+  gemm_general<_Float16>(A, lda, Bt, ldb, C, ldc, M, N, K);
 }

@@ -1244,9 +1244,11 @@ int hcamdLaunchQuantizeF16I8(OlQueue q, const void *x, size_t ldx, int8_t *qout,
   return launch1d(queue, "quantize", name, groups, 256, args);
 }
 
-int hcamdLaunchGemmBF16(OlQueue q, const void *a, size_t lda, const void *bt,
-                        size_t ldb, void *c, size_t ldc, size_t m, size_t n,
-                        size_t k) noexcept {
+namespace {
+// Shared by the bf16 and fp16 entry points; `half` selects the fp16 kernels.
+int launchGemm(OlQueue q, bool half, const void *a, size_t lda, const void *bt,
+               size_t ldb, void *c, size_t ldc, size_t m, size_t n, size_t k) {
+  const char *who = half ? "hcamdLaunchGemmF16" : "hcamdLaunchGemmBF16";
   auto *queue = static_cast<Queue *>(q);
   if (!queue)
     return 1;
@@ -1254,19 +1256,19 @@ int hcamdLaunchGemmBF16(OlQueue q, const void *a, size_t lda, const void *bt,
   if (m == 0 || n == 0)
     return 0;
   if (!a || !bt || !c) {
-    dev->report("hcamdLaunchGemmBF16: null pointer");
+    dev->report("%s: null pointer", who);
     return 1;
   }
   if (k == 0) {
-    dev->report("hcamdLaunchGemmBF16: K must be at least 1");
+    dev->report("%s: K must be at least 1", who);
     return 1;
   }
   if ((m > 1 && lda < k) || (n > 1 && ldb < k) || (m > 1 && ldc < n)) {
-    dev->report("hcamdLaunchGemmBF16: leading dimension too small");
+    dev->report("%s: leading dimension too small", who);
     return 1;
   }
   if (m > 0x7fffffffull || n > 0x7fffffffull || k > 0x7fffffffull) {
-    dev->report("hcamdLaunchGemmBF16: dimension exceeds 2^31-1");
+    dev->report("%s: dimension exceeds 2^31-1", who);
     return 1;
   }
   int M = (int)m, N = (int)n, K = (int)k;
@@ -1298,7 +1300,16 @@ int hcamdLaunchGemmBF16(OlQueue q, const void *a, size_t lda, const void *bt,
                       lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 &&
                       k % 64 == 0;
   const Tiled *pick = nullptr;
-  if (vec_ok && variant != kGeneral) {
+  static const Tiled half256 = {"hcamd_gemm_f16_p256x256_w2x4", 256, 256, 512};
+  static const Tiled half128 = {"hcamd_gemm_f16_p128x128_w2x2", 128, 128, 256};
+  if (half) {
+    if (vec_ok && k >= 128 && variant != kGeneral) {
+      if (m % 256 == 0 && n % 256 == 0)
+        pick = &half256;
+      else if (m % 128 == 0 && n % 128 == 0)
+        pick = &half128;
+    }
+  } else if (vec_ok && variant != kGeneral) {
     if (variant >= 1 && variant <= kNumTiled) {
       const Tiled &t = tiled[variant - 1];
       if (t.name && m % t.bm == 0 && n % t.bn == 0 &&
@@ -1325,17 +1336,31 @@ int hcamdLaunchGemmBF16(OlQueue q, const void *a, size_t lda, const void *bt,
     const size_t block[3] = {(size_t)pick->threads, 1, 1};
     return launch(queue, kn, grid, block, args, 0);
   }
-  Kernel *kn = builtinKernel(dev, "gemm", "hcamd_gemm_bf16_general");
+  Kernel *kn = builtinKernel(dev, "gemm", half ? "hcamd_gemm_f16_general"
+                                               : "hcamd_gemm_bf16_general");
   if (!kn)
     return 1;
   const size_t gy = ceilDiv(m, 64);
   if (gy > 65535) {
-    dev->report("hcamdLaunchGemmBF16: M too large for the general kernel");
+    dev->report("%s: M too large for the general kernel", who);
     return 1;
   }
   const size_t grid[3] = {ceilDiv(n, 64), gy, 1};
   const size_t block[3] = {256, 1, 1};
   return launch(queue, kn, grid, block, args, 0);
+}
+} // namespace
+
+int hcamdLaunchGemmBF16(OlQueue q, const void *a, size_t lda, const void *bt,
+                        size_t ldb, void *c, size_t ldc, size_t m, size_t n,
+                        size_t k) noexcept {
+  return launchGemm(q, false, a, lda, bt, ldb, c, ldc, m, n, k);
+}
+
+int hcamdLaunchGemmF16(OlQueue q, const void *a, size_t lda, const void *bt,
+                       size_t ldb, void *c, size_t ldc, size_t m, size_t n,
+                       size_t k) noexcept {
+  return launchGemm(q, true, a, lda, bt, ldb, c, ldc, m, n, k);
 }
 
 } // extern "C"

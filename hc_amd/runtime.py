@@ -93,6 +93,8 @@ hcamdLaunchQuantizeF16I8 = _sig(_rt, "hcamdLaunchQuantizeF16I8", _int, _vp, _vp,
                                 _vp, _sz, _vp, _sz, _sz)
 hcamdLaunchGemmBF16 = _sig(_rt, "hcamdLaunchGemmBF16", _int, _vp, _vp, _sz, _vp, _sz,
                            _vp, _sz, _sz, _sz, _sz)
+hcamdLaunchGemmF16 = _sig(_rt, "hcamdLaunchGemmF16", _int, _vp, _vp, _sz, _vp, _sz,
+                          _vp, _sz, _sz, _sz, _sz)
 
 
 class MapInstr(C.Structure):
@@ -520,6 +522,22 @@ def plan_gemm_bf16(a, bt, c) -> Plan:
     return Plan(ctx, hcamdLaunchGemmBF16,
                 (ctx.queue, ma.ptr, lda, mb.ptr, ldb, mc.ptr, ldc, m_, n_, k_),
                 "hcamdLaunchGemmBF16", (a, bt, c))
+
+
+def plan_gemm_f16(a, bt, c) -> Plan:
+    """C[M,N] = A[M,K] @ Bt[N,K].T with fp16 storage and fp32 accumulation."""
+    ctx = _ctx_of(a, bt, c)
+    ma, mb, mc = as_memref(a, 2), as_memref(bt, 2), as_memref(c, 2)
+    for m, n in ((ma, "a"), (mb, "bt"), (mc, "c")):
+        _expect(m, 2, n)
+    m_, k_, lda = _rows_cols(ma)
+    n_, k2, ldb = _rows_cols(mb)
+    m2, n2, ldc = _rows_cols(mc)
+    if k_ != k2 or m_ != m2 or n_ != n2:
+        raise HcRuntimeError("gemm_f16: shape mismatch")
+    return Plan(ctx, hcamdLaunchGemmF16,
+                (ctx.queue, ma.ptr, lda, mb.ptr, ldb, mc.ptr, ldc, m_, n_, k_),
+                "hcamdLaunchGemmF16", (a, bt, c))
 
 
 # Call-and-wait forms: a kernel call is synchronous on return by default, as in

@@ -347,6 +347,14 @@ int hcamdLaunchGemmBF16(OlQueue q, const void *a, size_t lda, const void *bt,
                         size_t ldb, void *c, size_t ldc, size_t m, size_t n,
                         size_t k) HCAMD_NOEXCEPT;
 
+/* The same product with fp16 storage (A, Bt, C) and the fp16 MFMA: the dtype
+ * NumPy has natively, so the reference's blocked-dot example
+ * (python/hckernel/tests/test_examples.py:124-165, written with Bt) can be run
+ * on both sides. */
+int hcamdLaunchGemmF16(OlQueue q, const void *a, size_t lda, const void *bt,
+                       size_t ldb, void *c, size_t ldc, size_t m, size_t n,
+                       size_t k) HCAMD_NOEXCEPT;
+
 /* Chooses between kernel variants of one family by number (0 = default
  * choice by shape).  For tuning and measurement; family names are "add",
  * "fma", "softmax", "quantize", "gemm", "copy". Returns 1 for an unknown

@@ -531,6 +531,39 @@ def test_blocked_dot_on_torch_bfloat16_tensors():
     torch.testing.assert_close(out.float(), want, rtol=1e-2, atol=1e-2 * 0.02 * 0.02 * 768 ** 0.5)
 
 
+def test_blocked_dot_fp16_same_body_on_gpu_and_host_executor():
+    # the K-blocked dot of python/hckernel/tests/test_examples.py:124-165, with B given as Bt
+    M, N, K = sym.M, sym.N, sym.K
+    GM, GN, MI, NI, KB = sym.GM, sym.GN, sym.MI, sym.NI, sym.KB
+    tun = (TunableParam(MI, 4, range(1, 8)), TunableParam(NI, 4, range(1, 8)),
+           TunableParam(KB, 64, range(8, 128)))
+    KI = cdiv(K, KB)
+
+    def dot(gr: CurrentGroup, a: Buffer[M, K, DT], bt: Buffer[N, K, DT], out: Buffer[M, N, DT],
+            gshape: (GM, GN)):
+        m0, n0 = gr.work_offset[0] * MI, gr.work_offset[1] * NI
+        mb, nb = gr.shape[0] * MI, gr.shape[1] * NI
+        r = gr.zeros(shape=(mb, nb), dtype=np.float32)
+        for k in range(KI):
+            r += np.dot(gr.load(a[m0:, k * KB:], shape=(mb, KB)).astype(np.float32),
+                        gr.load(bt[n0:, k * KB:], shape=(nb, KB)).astype(np.float32).T)
+        gr.store(out[m0:, n0:], r)
+
+    deco = dict(work_shape=(cdiv(M, MI), cdiv(N, NI)), group_shape=(GM, GN), tunables=tun)
+    rng = np.random.default_rng(9)
+    m, n, k = 256, 128, 192
+    a = (0.5 * rng.standard_normal((m, k))).astype(np.float16)
+    bt = (0.5 * rng.standard_normal((n, k))).astype(np.float16)
+    host = np.zeros((m, n), np.float16)
+    sim_kernel(**deco)(dot)(a, bt, host, (16, 16))
+    out = rt.DeviceArray((m, n), np.float16)
+    kernel(**deco)(dot)(rt.to_device(a), rt.to_device(bt), out, (16, 16))
+    assert rt.last_kernel_name() == "hcamd_gemm_f16_p128x128_w2x2"
+    # both accumulate in fp32 (in different orders) and round once to fp16
+    assert_allclose(out.to_host().astype(np.float32), host.astype(np.float32),
+                    rtol=2.0 ** -10, atol=2.0 ** -10)
+
+
 def test_unsupported_body_raises_instead_of_running_on_the_cpu():
     N = sym.N
 

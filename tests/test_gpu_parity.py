@@ -765,6 +765,29 @@ def test_gemm_random_within_tolerance(ctx, mnk):
         assert_allclose(got, c32, rtol=GEMM_RTOL, atol=1e-2 * sigma)
 
 
+@pytest.mark.parametrize("mnk", [(256, 256, 128), (512, 256, 320), (128, 384, 192), (100, 70, 50),
+                                 (256, 256, 64)])
+def test_gemm_fp16_against_fp32_accumulation(ctx, mnk):
+    m, n, k = mnk
+    rng = np.random.default_rng(sum(mnk))
+    a = (0.5 * rng.standard_normal((m, k))).astype(np.float16)
+    bt = (0.5 * rng.standard_normal((n, k))).astype(np.float16)
+    c = poisoned((m, n + 8), np.float16)
+    rt.plan_gemm_f16(dev(a), dev(bt), _View(c, (m, n), 0, (n + 8, 1))).launch(sync=True)
+    say("gemm f16", mnk, rt.last_kernel_name())
+    got = c.to_host()
+    want = a.astype(np.float32) @ bt.astype(np.float32).T
+    # fp32 accumulation, one rounding to fp16 at the end
+    assert_allclose(got[:, :n].astype(np.float32), want, rtol=2.0 ** -10, atol=2.0 ** -10 * np.sqrt(k) * 0.25)
+    assert (got[:, n:].view(np.uint16) == poison_value(np.float16).view(np.uint16)).all()
+    # small integers: every product and partial sum is exact, so the result is too
+    ai = rng.integers(-3, 4, (m, k)).astype(np.float16)
+    bi = rng.integers(-3, 4, (n, k)).astype(np.float16)
+    c2 = rt.DeviceArray((m, n), np.float16)
+    rt.plan_gemm_f16(dev(ai), dev(bi), c2).launch(sync=True)
+    assert_array_equal(c2.to_host().astype(np.float32), ai.astype(np.float32) @ bi.astype(np.float32).T)
+
+
 def test_gemm_all_variants_and_padded_output(ctx):
     ab, bb = cf.inputs_c5((512, 512, 256))
     want = cf.np_gemm_bf16(ab, bb, np.float32)
