@@ -577,20 +577,23 @@ def test_softmax_variants_and_strided_rows(ctx):
                     atol=SOFTMAX_ATOL)
 
 
-def test_softmax_extreme_and_special_rows(ctx):
+@pytest.mark.parametrize("cols,variant", [(1024, 0), (8192, 0), (8192, 5)])
+def test_softmax_extreme_and_special_rows(ctx, cols, variant):
     f = np.float32
-    x = np.zeros((6, 1024), f)
-    x[0, :] = 1.25                                   # constant row: exactly 1/1024
-    x[1, :] = np.linspace(-80, 80, 1024)             # wide range, tiny tails
+    x = np.zeros((6, cols), f)
+    x[0, :] = 1.25                                   # constant row: exactly 1/cols
+    x[1, :] = np.linspace(-80, 80, cols)             # wide range, tiny tails
     x[2, 5] = np.nan                                 # NaN anywhere -> NaN row
     x[3, 7] = np.inf                                 # +inf -> NaN row (inf - inf)
     x[4, :] = -np.inf                                # all -inf -> NaN row
     x[5, :] = -1e30
     x[5, 3] = 0.0                                    # one-hot
     dy = rt.DeviceArray(x.shape, f)
+    rt.set_variant("softmax", variant)
     rt.softmax_f32(dev(x), dy)
+    say("softmax special rows", cols, variant, rt.last_kernel_name())
     y = dy.to_host()
-    assert_array_equal(y[0], np.full(1024, 1 / 1024, f))
+    assert_array_equal(y[0], np.full(cols, 1 / cols, f))
     with np.errstate(all="ignore"):
         want = cf.np_softmax(x)
     assert_allclose(y[1], want[1], rtol=SOFTMAX_RTOL, atol=1e-30)
