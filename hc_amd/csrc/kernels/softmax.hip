@@ -42,6 +42,15 @@ __device__ __forceinline__ float exp_scaled(float x, float m_log2e) {
   constexpr float kLog2e = 1.44269502162933349609375f;
   return __builtin_amdgcn_exp2f(__builtin_fmaf(x, kLog2e, -m_log2e));
 }
+// The fused form leaves the rounding error of m * log2(e) in every exponent of
+// the row.  It cancels in the normalisation as long as 2^error stays in range,
+// i.e. for |m| up to about 1e9; rows with a larger maximum take the plain
+// exp2((x - m) * log2(e)), one more operation per element.
+constexpr float kFusedMaxAbs = 1.0e6f;
+__device__ __forceinline__ float exp_shifted(float x, float m) {
+  constexpr float kLog2e = 1.44269502162933349609375f;
+  return __builtin_amdgcn_exp2f((x - m) * kLog2e);
+}
 
 template <int TPR, int VPT, bool FULL, bool NT, bool FAST = true>
 __device__ __forceinline__ void softmax_regs(const float *x, size_t ldx,
@@ -91,12 +100,23 @@ __device__ __forceinline__ void softmax_regs(const float *x, size_t ldx,
   // a row of -inf (or a masked-out row) has m = -inf: m*log2(e) - that would
   // make fma(-inf, c, +inf) NaN, which is also what the plain expression gives
   const float m_log2e = m * 1.44269502162933349609375f;
+  if (!FAST || __builtin_fabsf(m) < kFusedMaxAbs) { // uniform over the row
 #pragma unroll
-  for (int j = 0; j < VPT; ++j) {
+    for (int j = 0; j < VPT; ++j) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      v[j][i] = FAST ? exp_scaled(v[j][i], m_log2e) : exp_nonpos(v[j][i] - m);
-      s += v[j][i];
+      for (int i = 0; i < 4; ++i) {
+        v[j][i] = FAST ? exp_scaled(v[j][i], m_log2e) : exp_nonpos(v[j][i] - m);
+        s += v[j][i];
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[j][i] = exp_shifted(v[j][i], m);
+        s += v[j][i];
+      }
     }
   }
   s = group_reduce<SumOp, kWaves>(s, ssum + rg * kWaves);
@@ -189,13 +209,23 @@ __device__ __forceinline__ void softmax_persistent(const float *x, size_t ldx,
     m = group_reduce<MaxOp, kWaves>(m, smax);
     const float m_log2e = m * 1.44269502162933349609375f;
     float s = 0.0f;
+    if (__builtin_fabsf(m) < kFusedMaxAbs) { // uniform over the row
 #pragma unroll
-    for (int j = 0; j < VPT; ++j)
+      for (int j = 0; j < VPT; ++j)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        cur[j][i] = exp_scaled(cur[j][i], m_log2e);
-        s += cur[j][i];
-      }
+        for (int i = 0; i < 4; ++i) {
+          cur[j][i] = exp_scaled(cur[j][i], m_log2e);
+          s += cur[j][i];
+        }
+    } else {
+#pragma unroll
+      for (int j = 0; j < VPT; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          cur[j][i] = exp_shifted(cur[j][i], m);
+          s += cur[j][i];
+        }
+    }
     s = group_reduce<SumOp, kWaves>(s, ssum);
     const float inv = 1.0f / s;
     f32x4 *yr = reinterpret_cast<f32x4 *>(y + row * ldy);

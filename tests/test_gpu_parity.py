@@ -602,6 +602,29 @@ def test_softmax_extreme_and_special_rows(ctx, cols, variant):
     assert y[5, 3] == 1.0 and y[5].sum() == 1.0
 
 
+@pytest.mark.parametrize("cols,variant", [(1000, 0), (4096, 0), (8192, 0), (8192, 5)])
+def test_softmax_rows_of_huge_magnitude(ctx, cols, variant):
+    # a row's maximum may be far from 0: only differences matter
+    f = np.float32
+    rng = np.random.default_rng(cols)
+    base = rng.standard_normal((8, cols)).astype(f)
+    x = base.copy()
+    x[0] += f(1e30)                 # absorbed: every element becomes the same 1e30
+    x[1] = f(3e38)                  # constant, near the top of the range
+    x[2] = -x[1]
+    x[3] = base[3] * f(1e9)         # spread over +-4e9
+    x[4] = base[4] + f(2.5e7)       # fp32 spacing 2 at this magnitude
+    x[5] = base[5] - f(7e10)
+    rt.set_variant("softmax", variant)
+    dy = rt.DeviceArray(x.shape, f)
+    rt.softmax_f32(dev(x), dy)
+    say("softmax huge rows", cols, variant, rt.last_kernel_name())
+    with np.errstate(all="ignore"):
+        want = cf.np_softmax(x)
+    assert np.isfinite(want).all()
+    assert_allclose(dy.to_host(), want, rtol=SOFTMAX_RTOL, atol=1e-30)
+
+
 def test_softmax_reference_test_input(ctx):
     # python/hckernel/tests/test_examples.py:322-335 (float64 there)
     m, n = 30, 25
