@@ -34,6 +34,10 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
+# MI355X fp32 vector peak, published.  It counts packed fused multiply-adds; the
+# pairwise kernel issues one subtract and one unpacked multiply-add per term
+# (3 flop per 2 lane-instructions), so its own ceiling is well under this figure.
+FP32_VECTOR_PEAK_TFLOPS = 157.3
 ROTATE = 4
 PREWARM_SECONDS = 0.4        # untimed, per workload, before the W warm-up steps
 
@@ -222,6 +226,67 @@ def make_workloads(rt, wl):
             dst = np.empty_like(self.src)
             return _best_of(lambda: np.copyto(dst, self.src)), "full size, numpy.copyto", 1
 
+
+    # ---- beyond the five configurations: the generic paths, on request only ------
+    I = lambda name, arg=0, imm=0.0: (name, arg, imm)      # noqa: E731
+
+    class X1(C2):
+        """a*b+c on the C2 arrays through the fused map kernel (3 instructions)."""
+
+        def plan(self, rt, s):
+            return rt.plan_map([I("in", 0), I("mul_in", 1), I("add_in", 2)], s[:3], s[3])
+
+    class X2(Workload):
+        """fp32 dot product of the C1 vectors through the map-sum kernel."""
+
+        def setup(self, rt):
+            self.a, self.b = W.inputs_c1()
+            return [(rt.to_device(self.a), rt.to_device(self.b),
+                     rt.to_device(np.zeros(1, np.float32))) for _ in range(ROTATE)]
+
+        def plan(self, rt, s):
+            return rt.plan_map_sum([I("in", 0), I("mul_in", 1)], s[:2], s[2])
+
+        def check(self, rt, s):
+            cell = rt.to_device(np.zeros(1, np.float32))
+            rt.plan_map_sum([I("in", 0), I("mul_in", 1)], s[:2], cell).launch(sync=True)
+            prod = (self.a * self.b).astype(np.float64)
+            err = abs(float(cell.to_host()[0]) - prod.sum())
+            ok = err <= 64 * 2.0 ** -24 * np.abs(prod).sum()
+            return {"parity": "|err| <= 64 * 2^-24 * sum|x|" if ok else "MISMATCH", "ok": bool(ok),
+                    "abs_err": err}
+
+        def cpu(self):
+            return _best_of(lambda: np.dot(self.a, self.b)), "full size, numpy.dot", _blas_threads()
+
+    class X3(Workload):
+        """Pairwise distances of 8192 x 8192 points in 128 dimensions."""
+        M = N = 8192
+        D = 128
+
+        def setup(self, rt):
+            rng = np.random.default_rng(6)
+            self.a = rng.standard_normal((self.M, self.D)).astype(np.float32)
+            self.b = rng.standard_normal((self.N, self.D)).astype(np.float32)
+            return [(rt.to_device(self.a), rt.to_device(self.b),
+                     rt.DeviceArray((self.M, self.N), np.float32)) for _ in range(ROTATE)]
+
+        def plan(self, rt, s):
+            return rt.plan_pairwise_dist_f32(s[0], s[1], s[2])
+
+        def check(self, rt, s):
+            got = s[2].to_host()[:256, :512]
+            want = np.sqrt(((self.a[:256, None, :].astype(np.float64) - self.b[None, :512, :]) ** 2
+                            ).sum(axis=2))
+            ok = np.allclose(got, want, rtol=(self.D + 2) * 2.0 ** -24)
+            return {"parity": "rtol (d+2) * 2^-24 vs fp64 (256 x 512 block)" if ok else "MISMATCH",
+                    "ok": bool(ok)}
+
+        def cpu(self):
+            a, b = self.a[:512], self.b[:512]
+            t = _best_of(lambda: np.linalg.norm(a[:, None, :] - b[None, :, :], axis=2), 2)
+            return t * (self.M / 512) * (self.N / 512), "512 x 512 block scaled to full size", 1
+
     table = {
         "c0": C0("c0", "copy 256 MiB int32 (calibration)", "u32", "hbm", 2 * 4 * 64 * 1024 * 1024,
                  "GB/s"),
@@ -231,8 +296,18 @@ def make_workloads(rt, wl):
         "c4": C4("c4", "row absmax int8 quantize fp16 16384x4096", "f16->i8", "hbm",
                  W.work_c4(), "GB/s"),
         "c5": C5("c5", "GEMM bf16 4096^3 (fp32 acc)", "bf16", "mfma", W.work_c5(), "TFLOP/s"),
+        "x1": X1("x1", "map kernel: fma fp16 8191x8193 as a 3-instruction program", "f16", "hbm",
+                 W.work_c2(), "GB/s"),
+        "x2": X2("x2", "map-sum kernel: dot fp32 N=16777259", "f32", "hbm", 8 * W.C1_N, "GB/s"),
+        "x3": X3("x3", "pairwise distance fp32 8192x8192x128 (sub + fma per term)", "f32", "valu",
+                 3 * 8192 * 8192 * 128, "TFLOP/s"),
     }
-    keys = [k for k in table if k != "c0"] if wl == "all" else [wl]
+    if wl == "all":
+        keys = ["c1", "c2", "c3", "c4", "c5"]
+    elif wl == "extra":
+        keys = ["x1", "x2", "x3"]
+    else:
+        keys = [wl]
     return [table[k] for k in keys]
 
 
@@ -267,13 +342,13 @@ def run_one(rt, ctx, w, steps, warmup, want_cpu, prewarm):
     scale = 1e-9 if w.unit == "GB/s" else 1e-12
     value = w.work * scale / (wall / steps)
     achieved = w.work * scale / (kern_ms * 1e-3)
-    peak = HBM_PEAK_GBS if w.bound == "hbm" else BF16_PEAK_TFLOPS
+    peak = {"hbm": HBM_PEAK_GBS, "mfma": BF16_PEAK_TFLOPS, "valu": FP32_VECTOR_PEAK_TFLOPS}[w.bound]
     res = {
         "workload": w.title, "kernel": kernel, "dtype": w.dtype,
         "value": round(value, 2), "unit": w.unit, "ms_per_step": round(ms_step, 5),
         "roofline": {"bound": w.bound, "achieved": round(achieved, 2), "peak": peak,
                      "unit": w.unit, "frac": round(achieved / peak, 4),
-                     "traffic": MEASURED_TRAFFIC[w.key],
+                     "traffic": MEASURED_TRAFFIC.get(w.key),
                      "kernel_avg_us": round(kern_ms * 1e3, 3),
                      "algorithmic_work": w.work},
     }
@@ -297,7 +372,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="all", choices=["all", "c0", "c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="all", choices=["all", "c0", "c1", "c2", "c3", "c4", "c5", "extra", "x1", "x2", "x3"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy CPU baseline")
     ap.add_argument("--prewarm", type=float, default=PREWARM_SECONDS,
                     help="seconds of untimed device warm-up per workload")
