@@ -389,6 +389,232 @@ def match_gemm(dst_view, value, n_groups):
 
 
 # ---------------------------------------------------------------------------
+# Products of gathered tiles (mapped loads / stores)
+# ---------------------------------------------------------------------------
+class _Operand:
+    """One side of the product: the tile all dot terms read their chunks from.
+    `view` is the window it is loaded from, `func` maps (row, col) of the tile
+    to an index tuple inside the window (None: the identity of a plain 2-D
+    load), `shape` is the tile shape."""
+
+    def __init__(self, view, func, shape):
+        self.view, self.func, self.shape = view, func, tuple(shape)
+
+    def same_as(self, o):
+        return (self.view.base.index == o.view.base.index and self.func is o.func
+                and all(_same_index(a, b) for a, b in zip(self.view.starts, o.view.starts)))
+
+
+def _same_index(a, b):
+    return a is b or (isinstance(a, Affine) and isinstance(b, Affine) and a == b)
+
+
+def _region(t: Tile, axis_k: int):
+    """Follows slice / window nodes down to a load.  Returns (operand, origin,
+    limit): element e of `t` along each axis is element origin[axis] + e of the
+    operand tile, and holds data only while origin + e < limit[axis] (beyond that
+    it is an inactive zero).  A plain load whose K start is a constant is turned
+    into a chunk of the load with K start 0."""
+    if _is(t, "mapped_load"):
+        if len(t.shape) != 2:
+            raise NoNativeKernel("mapped loads are bound for 2-D tiles")
+        return _Operand(t.attrs["view"], t.attrs["mapping"], t.shape), [0, 0], list(t.shape)
+    if _is(t, "load"):
+        view = t.attrs["view"]
+        if view.base.ndim != 2 or len(t.shape) != 2:
+            raise NoNativeKernel("the operands of a dot are 2-D tiles")
+        k0 = view.starts[axis_k]
+        if not k0.is_const or k0.const < 0:
+            raise NoNativeKernel("the K offset of a dot operand must not depend on the group")
+        starts = list(view.starts)
+        starts[axis_k] = Affine(0, k0.coeffs)
+        shape = list(t.shape)
+        shape[axis_k] = None                       # filled in from the chunks
+        op = _Operand(BufferView(view.base, tuple(starts)), None, shape)
+        origin, limit = [0, 0], list(t.shape)
+        origin[axis_k] = k0.const
+        limit[axis_k] = k0.const + t.shape[axis_k]
+        return op, origin, limit
+    if _is(t, "astype", 1) and t.dtype_name == t.args[0].dtype_name:
+        return _region(t.args[0], axis_k)
+    if _is(t, "window", 1):
+        op, origin, limit = _region(t.args[0], axis_k)
+        limit = [min(l, o + n) for l, o, n in zip(limit, origin, t.shape)]
+        return op, origin, limit
+    if _is(t, "slice", 1):
+        src = t.args[0]
+        op, origin, limit = _region(src, axis_k)
+        key = t.attrs["key"]
+        if len(key) != 2 or any(not isinstance(k, tuple) for k in key):
+            raise NoNativeKernel("dot operands are sliced as tile[r0:r1, c0:c1]")
+        for ax, k in enumerate(key):
+            start, stop, step = slice(*k).indices(src.shape[ax])
+            if step != 1:
+                raise NoNativeKernel("strided slices of tiles have no native kernel")
+            limit[ax] = min(limit[ax], origin[ax] + max(stop, start))
+            origin[ax] += start
+        return op, origin, limit
+    raise NoNativeKernel(f"operand of a dot is {t!r}: bound for (slices of) loads")
+
+
+def _mapping_tables(func, rows, cols, ndim, name):
+    """Evaluates an index mapping on the whole tile.  Returns (row_index
+    [rows, ndim], col_index [cols, ndim]); every dimension must depend on one
+    tile coordinate only."""
+    import numpy as np
+    if func is None:
+        if ndim != 2:
+            raise NoNativeKernel(f"{name}: plain tiles of a product are 2-D")
+        r = np.zeros((rows, 2), np.int64)
+        c = np.zeros((cols, 2), np.int64)
+        r[:, 0] = np.arange(rows)
+        c[:, 1] = np.arange(cols)
+        return r, c
+    i = np.arange(rows, dtype=np.int64).reshape(rows, 1)
+    j = np.arange(cols, dtype=np.int64).reshape(1, cols)
+    try:
+        mapped = func(i, j)
+    except TraceError:
+        raise
+    except Exception as exc:
+        raise NoNativeKernel(f"{name}: the mapping cannot be evaluated on index arrays "
+                             f"({type(exc).__name__}: {exc})") from exc
+    if not isinstance(mapped, tuple) or len(mapped) != ndim:
+        raise NoNativeKernel(f"{name}: the mapping must return {ndim} indices")
+    r = np.zeros((rows, ndim), np.int64)
+    c = np.zeros((cols, ndim), np.int64)
+    for d, m in enumerate(mapped):
+        try:
+            full = np.broadcast_to(np.asarray(m), (rows, cols))
+            if full.dtype == object or full.dtype.kind == "f":
+                as_int = np.array([[int(v) for v in row] for row in full], dtype=np.int64)
+                if not all(v == w for v, w in zip(full.ravel(), as_int.ravel())):
+                    raise NoNativeKernel(f"{name}: the mapping gives fractional indices")
+                full = as_int
+            full = full.astype(np.int64)
+        except (TypeError, ValueError) as exc:
+            raise NoNativeKernel(f"{name}: mapping result of dimension {d} is not an integer "
+                                 f"array ({exc})") from exc
+        by_col = rows and cols and bool((full != full[:, :1]).any())
+        by_row = rows and cols and bool((full != full[:1, :]).any())
+        if by_col and by_row:
+            raise NoNativeKernel(f"{name}: index {d} of the mapping depends on both tile "
+                                 "coordinates (each index must follow the row or the column)")
+        if by_col:
+            c[:, d] = full[0, :]
+        elif rows and cols:
+            r[:, d] = full[:, 0]
+    return r, c
+
+
+def _group_starts(view, n_groups):
+    """Window start of every group, [n_groups, ndim], groups in row-major order."""
+    import numpy as np
+    from .kernel_api import evaluate_index
+    total = 1
+    for n in n_groups:
+        total *= n
+    ids = [g.reshape(-1) for g in np.indices(n_groups, dtype=np.int64)]
+    out = np.zeros((total, view.base.ndim), np.int64)
+    for d, s in enumerate(view.starts):
+        v = np.broadcast_to(np.asarray(evaluate_index(s, ids)), (total,))
+        if v.dtype == object:
+            if any(x != int(x) for x in v):
+                raise NoNativeKernel(f"{view.base.name}: fractional window start along dim {d}")
+            v = np.array([int(x) for x in v], dtype=np.int64)
+        if (v < 0).any():
+            raise NoNativeKernel(f"{view.base.name}: negative window start along dim {d}")
+        out[:, d] = v
+    return out
+
+
+def match_gather_gemm(dst_view, value, n_groups, out_func=None, plain=True):
+    """store(sum_k dot(A chunk, B chunk)) where the chunks are slices of one A
+    tile and one B tile, any of them loaded or stored through a mapping."""
+    value = _strip_cast(value, dst_view.base.dtype_name)
+    terms: list = []
+    _flatten_sum(value, terms)
+    dots = [t for t in terms if not _const(t, 0)]
+    if not dots or not all(_is(d, "dot", 2) for d in dots):
+        if plain:
+            return None
+        raise NoNativeKernel("a mapped store is bound for a sum of dot products")
+    if len(value.shape) != 2:
+        raise NoNativeKernel("the product tile must be 2-D")
+    tm, tn = value.shape
+    a_op = b_op = None
+    chunks = []
+    for d in dots:
+        oa, origin_a, limit_a = _region(d.args[0], 1)
+        ob, origin_b, limit_b = _region(d.args[1], 0)
+        if a_op is None:
+            a_op, b_op = oa, ob
+        elif not (a_op.same_as(oa) and b_op.same_as(ob)):
+            raise NoNativeKernel("the dot terms read different A / B tiles")
+        if origin_a[0] != 0 or origin_b[1] != 0 or d.args[0].shape[0] != tm or \
+                d.args[1].shape[1] != tn:
+            raise NoNativeKernel("dot terms must use all rows of A and all columns of B")
+        for op, got, ax in ((a_op, limit_a[0], 0), (b_op, limit_b[1], 1)):
+            if op.shape[ax] is not None and got < min(op.shape[ax], (tm, tn)[ax]):
+                raise NoNativeKernel("dot terms must use all rows of A and all columns of B")
+        if origin_a[1] != origin_b[0]:
+            raise NoNativeKernel("A and B chunks of one dot start at different K")
+        # beyond the shorter of the two chunks one factor is an inactive zero
+        length = min(limit_a[1] - origin_a[1], limit_b[0] - origin_b[0])
+        if length > 0:
+            chunks.append((origin_a[1], length))
+    chunks.sort()
+    pos = 0
+    for start, length in chunks:
+        if start != pos:
+            raise NoNativeKernel("K chunks of the dot terms are not contiguous from 0")
+        pos += length
+    k_total = pos
+    for op, ax in ((a_op, 1), (b_op, 0)):
+        if op.shape[ax] is None:
+            op.shape = tuple(k_total if i == ax else v for i, v in enumerate(op.shape))
+        elif op.shape[ax] != k_total:
+            raise NoNativeKernel("the dot terms do not cover all of K")
+    if a_op.shape[0] < tm or b_op.shape[1] < tn:
+        raise NoNativeKernel("the product tile is larger than its operands")
+    o_op = _Operand(dst_view, out_func, (tm, tn))
+    ops = (a_op, b_op, o_op)
+    names = tuple(o.view.base.name for o in ops)
+    if any(o.view.base.dtype_name != "float32" for o in ops):
+        raise NoNativeKernel("products of gathered tiles are bound for float32 buffers "
+                             f"({', '.join(o.view.base.dtype_name for o in ops)} given)")
+    dims = ((tm, k_total), (k_total, tn), (tm, tn))
+    tables = []
+    for o, (rows, cols), name in zip(ops, dims, names):
+        r, c = _mapping_tables(o.func, rows, cols, o.view.base.ndim, name)
+        tables.append((tuple(o.view.base.shape), tuple(o.view.base.strides),
+                       _group_starts(o.view, n_groups), r, c))
+    # two active elements of the out tile must not land on the same address
+    import numpy as np
+    so = np.asarray(o_op.view.base.strides, np.int64)
+    size = np.asarray(o_op.view.base.shape, np.int64)
+    ro, co = tables[2][3], tables[2][4]
+    ro = ro[((ro >= 0) & (ro < size)).all(axis=1)]          # rows / columns that can be active
+    co = co[((co >= 0) & (co < size)).all(axis=1)]
+    dest = (ro @ so)[:, None] + (co @ so)[None, :]
+    if len(np.unique(dest)) != dest.size:
+        raise NoNativeKernel(f"{names[2]}: the store mapping sends two tile elements to one "
+                             "destination")
+    total = 1
+    for n in n_groups:
+        total *= n
+    idx = tuple(o.view.base.index for o in ops)
+    cache = {}
+
+    def make(mem, ctx):
+        g = cache.get(id(ctx))
+        if g is None:
+            g = cache[id(ctx)] = rt.GatherGemm(ctx, *tables, total, tm, tn, k_total)
+        return [rt.plan_gather_gemm_f32(g, *[_Arr(mem[i], ctx) for i in idx])]
+    return make
+
+
+# ---------------------------------------------------------------------------
 # Generic elementwise expressions -> postfix program for the fused map kernel
 # ---------------------------------------------------------------------------
 _MAP_BINARY = {"add": ("add", "add", True), "mul": ("mul", "mul", True),
@@ -662,26 +888,28 @@ def match_sum(proxy, index, value, n_groups):
     return makers
 
 
-def bind(stores, n_groups, atomics=()):
+def bind(stores, n_groups, atomics=(), mapped_stores=()):
     """stores: list of (BufferView, Tile) from one traced execution; atomics:
-    list of (BufferProxy, index, Tile) atomic additions.  Returns a list of plan
-    makers; raises NoNativeKernel when nothing matches."""
-    if not stores and not atomics:
+    list of (BufferProxy, index, Tile) atomic additions; mapped_stores: list of
+    (BufferView, Tile, index function).  Returns a list of plan makers; raises
+    NoNativeKernel when nothing matches."""
+    if not stores and not atomics and not mapped_stores:
         raise NoNativeKernel("the kernel body stores nothing")
     try:
         if atomics:
-            if stores:
+            if stores or mapped_stores:
                 raise NoNativeKernel("a body that both stores tiles and accumulates "
                                      "atomically has no native kernel")
             return [mk for proxy, index, value in atomics
                     for mk in match_sum(proxy, index, value, n_groups)]
+        makers = [match_gather_gemm(view, value, n_groups, func, plain=False)
+                  for view, value, func in mapped_stores]
         q = match_quantize(stores, n_groups)
         if q is not None:
-            return [q]
-        makers = []
+            return makers + [q]
         for view, value in stores:
             for matcher in (match_copy, match_add, match_fma, match_softmax, match_gemm,
-                            match_pairwise, match_map):
+                            match_gather_gemm, match_pairwise, match_map):
                 mk = matcher(view, value, n_groups)
                 if mk is not None:
                     makers.append(mk)

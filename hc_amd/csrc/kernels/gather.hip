@@ -1,0 +1,170 @@
+// Matrix product of gathered tiles, fp32:
+//
+//   out[map_o(i, j)] = sum_k a[map_a(i, k)] * b[map_b(k, j)]      per group
+//
+// The operation behind a kernel body that loads its operands through index
+// mappings (python/hckernel/kernel_api.py:297-345 with mapping=..., as in the
+// implicit-GEMM convolution of python/hckernel/tests/test_examples.py:168-258)
+// and multiplies them with numpy.dot.  Every group has its own window into each
+// buffer (a start per dimension); inside the window the tile element (r, c)
+// sits at index row[r][d] + col[c][d] along dimension d, and each dimension is
+// driven by the tile row or by the tile column, never by both.  An element is
+// active if every index is inside the window, exactly the reference's bounds
+// test; inactive operand elements count as zero and inactive output elements
+// are not written.
+//
+// Tables (built and bounds-checked on the host):
+//   groups[g]  16 ints: {base, extent[4]} for a, b and out (base = element
+//              offset of the window, extent = buffer size - start per dim)
+//   *_rows[r], *_cols[c]  8 ints: {offset, index[4], unused[3]} (offset = sum
+//              of index * stride; dimensions the other coordinate drives hold 0)
+//
+// One workgroup of 256 lanes per group; the TM x TN tile is walked in 64 x 64
+// blocks, 4 x 4 outputs per lane, K in steps of 32 through LDS panels stored
+// k-major so that a lane's four operands are one 16-byte LDS read.  The gathers
+// of the next K step are issued before the multiply-adds of the current one.
+// Consecutive groups (which usually share operand data) go to the same XCD so
+// that they share its L2.
+#include "common.h"
+
+using namespace hcamd;
+
+namespace {
+constexpr int kTile = 64;
+constexpr int kStep = 32;
+constexpr int kPitch = kTile + 4;
+constexpr int kXcds = 8;
+
+struct GatherGemmArgs {
+  const float *a;
+  const float *b;
+  float *out;
+  const int32_t *groups;
+  const int32_t *a_rows, *a_cols, *b_rows, *b_cols, *o_rows, *o_cols;
+  uint32_t tm, tn, k, n_groups, per_xcd;
+};
+
+struct Window {
+  uint32_t base;
+  uint32_t ext[4];
+};
+
+// offset of a table entry if all of its indices are inside the window, else -1
+__device__ __forceinline__ int resolve(const int32_t *entry, const Window &w) {
+  const u32x4 lo = *reinterpret_cast<const u32x4 *>(entry);
+  const uint32_t i3 = static_cast<uint32_t>(entry[4]);
+  const bool ok = lo.y < w.ext[0] && lo.z < w.ext[1] && lo.w < w.ext[2] &&
+                  i3 < w.ext[3];
+  return ok ? static_cast<int>(lo.x) : -1;
+}
+
+__device__ __forceinline__ Window window_of(const int32_t *rec) {
+  Window w;
+  w.base = static_cast<uint32_t>(rec[0]);
+#pragma unroll
+  for (int d = 0; d < 4; ++d)
+    w.ext[d] = static_cast<uint32_t>(rec[1 + d]);
+  return w;
+}
+} // namespace
+
+extern "C" __global__ __launch_bounds__(256) void hcamd_gather_gemm_f32(
+    GatherGemmArgs p) {
+  __shared__ __attribute__((aligned(16))) float as[kStep][kPitch];
+  __shared__ __attribute__((aligned(16))) float bs[kStep][kPitch];
+  __shared__ int row_a[kTile], col_b[kTile], row_o[kTile], col_o[kTile];
+
+  const uint32_t g = (blockIdx.x % kXcds) * p.per_xcd + blockIdx.x / kXcds;
+  if (g >= p.n_groups)
+    return;
+  const int32_t *rec = p.groups + static_cast<size_t>(g) * 16;
+  const Window wa = window_of(rec), wb = window_of(rec + 5),
+               wo = window_of(rec + 10);
+  const float *a = p.a + wa.base;
+  const float *b = p.b + wb.base;
+  float *out = p.out + wo.base;
+
+  const int t = threadIdx.x;
+  const int tx = t % 16, ty = t / 16;
+  const int ld_k = t % kStep, ld_r = t / kStep;
+
+  for (uint32_t m0 = 0; m0 < p.tm; m0 += kTile)
+    for (uint32_t n0 = 0; n0 < p.tn; n0 += kTile) {
+      if (t < kTile) {
+        const uint32_t r = m0 + t;
+        row_a[t] = r < p.tm ? resolve(p.a_rows + 8 * (size_t)r, wa) : -1;
+        row_o[t] = r < p.tm ? resolve(p.o_rows + 8 * (size_t)r, wo) : -1;
+      } else if (t < 2 * kTile) {
+        const uint32_t c = n0 + t - kTile;
+        col_b[t - kTile] = c < p.tn ? resolve(p.b_cols + 8 * (size_t)c, wb) : -1;
+        col_o[t - kTile] = c < p.tn ? resolve(p.o_cols + 8 * (size_t)c, wo) : -1;
+      }
+      __syncthreads();
+
+      int ra[8], cb[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        ra[i] = row_a[ld_r + 8 * i];
+        cb[i] = col_b[ld_r + 8 * i];
+      }
+      float acc[4][4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = 0.0f;
+
+      float va[8], vb[8];
+      auto gather = [&](uint32_t k0) {
+        const uint32_t kk = k0 + ld_k;
+        int oa = -1, ob = -1;
+        if (kk < p.k) {
+          oa = resolve(p.a_cols + 8 * (size_t)kk, wa);
+          ob = resolve(p.b_rows + 8 * (size_t)kk, wb);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          // both offsets are non-negative when valid: the sign of the OR says
+          // whether either is the -1 marker
+          va[i] = (oa | ra[i]) >= 0 ? a[oa + ra[i]] : 0.0f;
+          vb[i] = (ob | cb[i]) >= 0 ? b[ob + cb[i]] : 0.0f;
+        }
+      };
+
+      if (p.k > 0)
+        gather(0);
+      for (uint32_t k0 = 0; k0 < p.k; k0 += kStep) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          as[ld_k][ld_r + 8 * i] = va[i];
+          bs[ld_k][ld_r + 8 * i] = vb[i];
+        }
+        __syncthreads();
+        if (k0 + kStep < p.k)
+          gather(k0 + kStep);
+#pragma unroll 8
+        for (int kk = 0; kk < kStep; ++kk) {
+          const f32x4 av = *reinterpret_cast<const f32x4 *>(&as[kk][4 * ty]);
+          const f32x4 bv = *reinterpret_cast<const f32x4 *>(&bs[kk][4 * tx]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
+        }
+        __syncthreads();
+      }
+
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int ro = row_o[4 * ty + i];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int co = col_o[4 * tx + j];
+          if ((ro | co) >= 0)
+            out[ro + co] = acc[i][j];
+        }
+      }
+      __syncthreads();
+    }
+}

@@ -15,6 +15,7 @@
 #include <cstring>
 #include <memory>
 #include <mutex>
+#include <new>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -138,6 +139,7 @@ HCAMD_BLOB(copy)
 HCAMD_BLOB(elementwise)
 HCAMD_BLOB(map)
 HCAMD_BLOB(distance)
+HCAMD_BLOB(gather)
 HCAMD_BLOB(softmax)
 HCAMD_BLOB(quantize)
 HCAMD_BLOB(gemm)
@@ -151,8 +153,8 @@ struct Blob {
 #define HCAMD_BLOB(n) {#n, hcamd_blob_##n##_begin, hcamd_blob_##n##_end}
 const Blob kBlobs[] = {HCAMD_BLOB(copy), HCAMD_BLOB(elementwise),
                        HCAMD_BLOB(map), HCAMD_BLOB(distance),
-                       HCAMD_BLOB(softmax), HCAMD_BLOB(quantize),
-                       HCAMD_BLOB(gemm)};
+                       HCAMD_BLOB(gather), HCAMD_BLOB(softmax),
+                       HCAMD_BLOB(quantize), HCAMD_BLOB(gemm)};
 #undef HCAMD_BLOB
 constexpr size_t kNumBlobs = sizeof(kBlobs) / sizeof(kBlobs[0]);
 
@@ -1106,6 +1108,245 @@ int hcamdLaunchPairwiseDistF32(OlQueue q, const float *a, size_t lda,
   const size_t grid[3] = {ceilDiv(n, 64), gy, 1};
   const size_t block[3] = {256, 1, 1};
   return launch(queue, k, grid, block, args, 0);
+}
+
+// ---------------------------------------------------------------------------
+// Matrix product of gathered tiles
+// ---------------------------------------------------------------------------
+struct HcamdGatherGemm_ {
+  Device *device = nullptr;
+  int32_t *tables = nullptr; // one device allocation holding all seven tables
+  size_t offGroups = 0, offRows[3] = {0, 0, 0}, offCols[3] = {0, 0, 0};
+  size_t elems[3] = {0, 0, 0}; // span of each buffer in elements
+  uint32_t tm = 0, tn = 0, k = 0, nGroups = 0;
+};
+
+namespace {
+// must match GatherGemmArgs in kernels/gather.hip
+struct GatherGemmArgs {
+  const float *a;
+  const float *b;
+  float *out;
+  const int32_t *groups;
+  const int32_t *a_rows, *a_cols, *b_rows, *b_cols, *o_rows, *o_cols;
+  uint32_t tm, tn, k, n_groups, per_xcd;
+};
+
+constexpr int kGatherEntry = 8;   // ints per row / column entry
+constexpr int kGatherRecord = 16; // ints per group record
+
+// Fills the entries of one tile axis of one operand.  `mine` says which
+// dimensions this axis drives (the others contribute index 0).
+void gatherEntries(const HcamdGatherOperand &op, const int32_t *index, size_t n,
+                   const bool mine[4], int32_t *dst) {
+  for (size_t r = 0; r < n; ++r) {
+    int32_t *e = dst + r * kGatherEntry;
+    int64_t off = 0;
+    bool inside = true;
+    for (int d = 0; d < 4; ++d) {
+      int32_t idx = 0;
+      if (d < op.ndim && mine[d])
+        idx = index[r * op.ndim + d];
+      e[1 + d] = idx;
+      const int64_t size = d < op.ndim ? (int64_t)op.shape[d] : 1;
+      if (idx < 0 || idx >= size)
+        inside = false;
+      else if (d < op.ndim)
+        off += (int64_t)idx * (int64_t)op.strides[d];
+    }
+    e[0] = inside ? (int32_t)off : 0; // never used when some index is outside
+    e[5] = e[6] = e[7] = 0;
+  }
+}
+} // namespace
+
+HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
+                                      const HcamdGatherOperand *b,
+                                      const HcamdGatherOperand *out,
+                                      size_t nGroups, size_t tm, size_t tn,
+                                      size_t k) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return nullptr;
+  Device *dev = queue->device;
+  if (!a || !b || !out) {
+    dev->report("hcamdGatherGemmCreate: null operand");
+    return nullptr;
+  }
+  if (nGroups == 0 || tm == 0 || tn == 0 || nGroups > 0x7ffffff0ull ||
+      tm > 0x7fffffffull || tn > 0x7fffffffull || k > 0x7fffffffull) {
+    dev->report("hcamdGatherGemmCreate: invalid sizes (groups %zu, tile %zu x "
+                "%zu x %zu)", nGroups, tm, tn, k);
+    return nullptr;
+  }
+  const HcamdGatherOperand *ops[3] = {a, b, out};
+  const size_t rows[3] = {tm, k, tm}, cols[3] = {k, tn, tn};
+  static const char *const names[3] = {"a", "b", "out"};
+  bool rowDim[3][4], colDim[3][4];
+  size_t span[3];
+  for (int o = 0; o < 3; ++o) {
+    const HcamdGatherOperand &op = *ops[o];
+    if (op.ndim < 1 || op.ndim > 4 || !op.starts ||
+        (rows[o] && !op.rowIndex) || (cols[o] && !op.colIndex)) {
+      dev->report("hcamdGatherGemmCreate: operand %s: rank %d or null table",
+                  names[o], op.ndim);
+      return nullptr;
+    }
+    size_t last = 0;
+    for (int d = 0; d < op.ndim; ++d) {
+      if (op.shape[d] == 0) {
+        dev->report("hcamdGatherGemmCreate: operand %s is empty", names[o]);
+        return nullptr;
+      }
+      last += (op.shape[d] - 1) * op.strides[d];
+    }
+    if (last >= 0x7fffffffull) {
+      dev->report("hcamdGatherGemmCreate: operand %s spans more than 2^31 "
+                  "elements", names[o]);
+      return nullptr;
+    }
+    span[o] = last + 1;
+    for (int d = 0; d < 4; ++d) {
+      bool r = false, c = false;
+      if (d < op.ndim) {
+        for (size_t i = 0; i < rows[o] && !r; ++i)
+          r = op.rowIndex[i * op.ndim + d] != 0;
+        for (size_t i = 0; i < cols[o] && !c; ++i)
+          c = op.colIndex[i * op.ndim + d] != 0;
+      }
+      if (r && c) {
+        dev->report("hcamdGatherGemmCreate: operand %s: dimension %d depends on "
+                    "both tile coordinates", names[o], d);
+        return nullptr;
+      }
+      colDim[o][d] = c;
+      rowDim[o][d] = !c; // constants (all-zero tables) ride with the row
+    }
+    for (size_t g = 0; g < nGroups; ++g)
+      for (int d = 0; d < op.ndim; ++d)
+        if (op.starts[g * op.ndim + d] < 0) {
+          dev->report("hcamdGatherGemmCreate: operand %s: negative window start",
+                      names[o]);
+          return nullptr;
+        }
+  }
+
+  auto plan = new (std::nothrow) HcamdGatherGemm_;
+  if (!plan)
+    return nullptr;
+  plan->device = dev;
+  plan->tm = (uint32_t)tm;
+  plan->tn = (uint32_t)tn;
+  plan->k = (uint32_t)k;
+  plan->nGroups = (uint32_t)nGroups;
+  size_t total = 0;
+  plan->offGroups = total;
+  total += nGroups * kGatherRecord;
+  for (int o = 0; o < 3; ++o) {
+    plan->elems[o] = span[o];
+    plan->offRows[o] = total;
+    total += rows[o] * kGatherEntry;
+    plan->offCols[o] = total;
+    total += cols[o] * kGatherEntry;
+  }
+  total += 4; // keeps the allocation non-empty and the last entry padded
+  std::vector<int32_t> host;
+  try {
+    host.assign(total, 0);
+  } catch (...) {
+    dev->report("hcamdGatherGemmCreate: out of host memory");
+    delete plan;
+    return nullptr;
+  }
+  for (size_t g = 0; g < nGroups; ++g) {
+    int32_t *rec = host.data() + plan->offGroups + g * kGatherRecord;
+    for (int o = 0; o < 3; ++o) {
+      const HcamdGatherOperand &op = *ops[o];
+      int32_t *w = rec + 5 * o;
+      int64_t base = 0;
+      bool empty = false;
+      for (int d = 0; d < 4; ++d) {
+        int64_t ext = 1;
+        if (d < op.ndim) {
+          const int64_t st = op.starts[g * op.ndim + d];
+          ext = (int64_t)op.shape[d] - st;
+          base += st * (int64_t)op.strides[d];
+        }
+        if (ext <= 0) {
+          ext = 0;
+          empty = true;
+        }
+        w[1 + d] = (int32_t)ext;
+      }
+      w[0] = empty ? 0 : (int32_t)base;
+    }
+  }
+  for (int o = 0; o < 3; ++o) {
+    gatherEntries(*ops[o], ops[o]->rowIndex, rows[o], rowDim[o],
+                  host.data() + plan->offRows[o]);
+    gatherEntries(*ops[o], ops[o]->colIndex, cols[o], colDim[o],
+                  host.data() + plan->offCols[o]);
+  }
+  if (dev->makeCurrent() ||
+      HIP_CHECK(dev, hipMalloc((void **)&plan->tables, total * sizeof(int32_t)))) {
+    delete plan;
+    return nullptr;
+  }
+  if (HIP_CHECK(dev, hipMemcpy(plan->tables, host.data(),
+                               total * sizeof(int32_t), hipMemcpyHostToDevice))) {
+    (void)hipFree(plan->tables);
+    delete plan;
+    return nullptr;
+  }
+  return plan;
+}
+
+int hcamdGatherGemmLaunchF32(OlQueue q, HcamdGatherGemm plan, const float *a,
+                             const float *b, float *out) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  if (!plan || plan->device != dev) {
+    dev->report("hcamdGatherGemmLaunchF32: the plan belongs to another device");
+    return 1;
+  }
+  if (!a || !b || !out) {
+    dev->report("hcamdGatherGemmLaunchF32: null pointer");
+    return 1;
+  }
+  Kernel *kern = builtinKernel(dev, "gather", "hcamd_gather_gemm_f32");
+  if (!kern)
+    return 1;
+  GatherGemmArgs args;
+  args.a = a;
+  args.b = b;
+  args.out = out;
+  const int32_t *t = plan->tables;
+  args.groups = t + plan->offGroups;
+  args.a_rows = t + plan->offRows[0];
+  args.a_cols = t + plan->offCols[0];
+  args.b_rows = t + plan->offRows[1];
+  args.b_cols = t + plan->offCols[1];
+  args.o_rows = t + plan->offRows[2];
+  args.o_cols = t + plan->offCols[2];
+  args.tm = plan->tm;
+  args.tn = plan->tn;
+  args.k = plan->k;
+  args.n_groups = plan->nGroups;
+  args.per_xcd = (plan->nGroups + 7) / 8;
+  void *params[] = {&args};
+  const size_t grid[3] = {(size_t)args.per_xcd * 8, 1, 1};
+  const size_t block[3] = {256, 1, 1};
+  return launch(queue, kern, grid, block, params, 0);
+}
+
+void hcamdGatherGemmRelease(HcamdGatherGemm plan) noexcept {
+  if (!plan)
+    return;
+  if (plan->tables && !plan->device->makeCurrent())
+    (void)hipFree(plan->tables);
+  delete plan;
 }
 
 int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,

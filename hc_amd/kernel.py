@@ -117,9 +117,17 @@ def _to_ints(expr, subs):
     return int(expr)
 
 
-def _resolve_symbols(func, subs):
+def _resolve_symbols(func, subs, _memo=None):
     """Clone func with sympy symbols / expressions in its closure and globals
-    replaced by their values (python/hckernel/kernel_api.py:43-90)."""
+    replaced by their values (python/hckernel/kernel_api.py:43-90); index
+    mappings found there are resolved the same way.  Each function is cloned
+    once per call (_memo), and a mapping that is reached again while it is being
+    cloned is left as it is, so module-level mappings that see each other
+    through their globals do not recurse."""
+    memo = {} if _memo is None else _memo
+    if id(func) in memo:
+        return memo[id(func)] or func
+    memo[id(func)] = None                       # in progress
 
     def value_of(v):
         if isinstance(v, sympy.Symbol):
@@ -128,20 +136,27 @@ def _resolve_symbols(func, subs):
             r = v.subs(subs)
             return int(r) if r.is_Integer else r
         if isinstance(v, Mapping):
-            return Mapping(_resolve_symbols(v.func, subs))
+            if memo.get(id(v.func), 0) is None:
+                return None
+            return Mapping(_resolve_symbols(v.func, subs, memo))
         return None
 
     closure = None
     if func.__closure__ is not None:
-        closure = tuple(c if value_of(c.cell_contents) is None
-                        else types.CellType(value_of(c.cell_contents))
-                        for c in func.__closure__)
-    new_globals = {k: (v if value_of(v) is None else value_of(v))
-                   for k, v in func.__globals__.items()}
+        cells = []
+        for c in func.__closure__:
+            r = value_of(c.cell_contents)
+            cells.append(c if r is None else types.CellType(r))
+        closure = tuple(cells)
+    new_globals = {}
+    for k, v in func.__globals__.items():
+        r = value_of(v)
+        new_globals[k] = v if r is None else r
     clone = types.FunctionType(func.__code__, new_globals, func.__name__,
                                func.__defaults__, closure)
     clone = functools.update_wrapper(clone, func)
     clone.__kwdefaults__ = func.__kwdefaults__
+    memo[id(func)] = clone
     return clone
 
 
@@ -225,7 +240,7 @@ class GpuKernel:
             body(group_obj, *proxies)
         except TraceError as exc:
             raise NoNativeKernel(f"{self.func.__name__}: {exc}") from exc
-        return bind(group_obj.stores, n_groups, group_obj.atomics)
+        return bind(group_obj.stores, n_groups, group_obj.atomics, group_obj.mapped_stores)
 
     def plan(self, *args, ctx=None):
         """Everything a call does short of launching: returns the list of

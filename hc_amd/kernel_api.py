@@ -14,7 +14,9 @@ kernels.  Nothing in this module computes array values.
 from __future__ import annotations
 
 import math
+import operator
 from collections.abc import Iterable
+from fractions import Fraction
 
 import numpy as np
 
@@ -127,9 +129,94 @@ class CurrentWorkitem:
 # ---------------------------------------------------------------------------
 # Affine index expressions in the group id
 # ---------------------------------------------------------------------------
+def _index_const(v):
+    """int or Fraction for a Python, NumPy or sympy rational number, else None."""
+    if isinstance(v, (bool, int, np.integer)):
+        return int(v)
+    if isinstance(v, Fraction):
+        return int(v) if v.denominator == 1 else v
+    p, q = getattr(v, "p", None), getattr(v, "q", None)      # sympy Integer / Rational
+    if isinstance(p, int) and isinstance(q, int) and q:
+        return p // q if p % q == 0 else Fraction(p, q)
+    return None
+
+
+class IndexExpr:
+    """An integer expression in the group id that is not affine: it contains a
+    floor division or a remainder (`w = idx % W_OUT; h = idx // W_OUT`).  Only
+    windows of mapped loads and stores may start at such an offset; their
+    kernels take the start of every group from a table."""
+
+    __slots__ = ("op", "args")
+    _OPS = {"add": operator.add, "sub": operator.sub, "mul": operator.mul,
+            "floordiv": operator.floordiv, "mod": operator.mod}
+
+    def __init__(self, op, args):
+        self.op, self.args = op, tuple(args)
+
+    @staticmethod
+    def _operand(v):
+        if isinstance(v, (Affine, IndexExpr)):
+            return v
+        c = _index_const(v)
+        if c is None:
+            raise TraceError(f"unsupported index value {v!r}")
+        return c
+
+    @classmethod
+    def make(cls, op, a, b):
+        return cls(op, (cls._operand(a), cls._operand(b)))
+
+    def __add__(self, o): return IndexExpr.make("add", self, o)
+    def __radd__(self, o): return IndexExpr.make("add", o, self)
+    def __sub__(self, o): return IndexExpr.make("sub", self, o)
+    def __rsub__(self, o): return IndexExpr.make("sub", o, self)
+    def __mul__(self, o): return IndexExpr.make("mul", self, o)
+    def __rmul__(self, o): return IndexExpr.make("mul", o, self)
+    def __floordiv__(self, o): return IndexExpr.make("floordiv", self, o)
+    def __rfloordiv__(self, o): return IndexExpr.make("floordiv", o, self)
+    def __mod__(self, o): return IndexExpr.make("mod", self, o)
+    def __rmod__(self, o): return IndexExpr.make("mod", o, self)
+    def __neg__(self): return IndexExpr.make("sub", 0, self)
+
+    def __index__(self):
+        raise TraceError("a group-id dependent index was used where a number is needed "
+                         "(only offsets of loads and stores may depend on the group id)")
+
+    __int__ = __index__
+
+    def _unsupported(self, *_):
+        raise TraceError("only + - * // and % are supported on group offsets")
+
+    __truediv__ = __rtruediv__ = __lt__ = __le__ = __gt__ = __ge__ = _unsupported
+
+    def __repr__(self):
+        sign = {"add": "+", "sub": "-", "mul": "*", "floordiv": "//", "mod": "%"}[self.op]
+        return f"({self.args[0]!r} {sign} {self.args[1]!r})"
+
+
+def evaluate_index(e, group_ids):
+    """Value of an index expression for many groups at once.  group_ids: one
+    integer array per group dimension, all of one shape; returns an array of
+    that shape (int64, or Python objects if fractions are involved)."""
+    if isinstance(e, Affine):
+        out = np.full(np.shape(group_ids[0]) if len(group_ids) else (), e.const, dtype=np.int64)
+        for c, g in zip(e.coeffs, group_ids):
+            if c:
+                out = out + c * g
+        return out
+    if isinstance(e, IndexExpr):
+        a, b = (evaluate_index(x, group_ids) for x in e.args)
+        if e.op in ("floordiv", "mod") and np.any(np.equal(b, 0)):
+            raise TraceError("division by zero in a group offset")
+        return IndexExpr._OPS[e.op](a, b)
+    return e
+
+
 class Affine:
-    """const + sum(coeffs[i] * group_id[i]).  The only index arithmetic a tiled
-    kernel needs: offsets are group id times tile size plus constants."""
+    """const + sum(coeffs[i] * group_id[i]).  The index arithmetic of a tiled
+    kernel: offsets are group id times tile size plus constants.  Floor
+    division and remainder leave the affine form and give an IndexExpr."""
 
     __slots__ = ("const", "coeffs")
 
@@ -140,6 +227,8 @@ class Affine:
     def lift(v, rank):
         if isinstance(v, Affine):
             return v
+        if isinstance(_index_const(v), Fraction):
+            raise TraceError(f"the index value {v} is not an integer")
         try:
             return Affine(int(v), (0,) * rank)
         except (TypeError, ValueError):
@@ -150,6 +239,8 @@ class Affine:
         return not any(self.coeffs)
 
     def __add__(self, o):
+        if isinstance(o, IndexExpr):
+            return NotImplemented
         o = Affine.lift(o, len(self.coeffs))
         return Affine(self.const + o.const, [a + b for a, b in zip(self.coeffs, o.coeffs)])
 
@@ -159,12 +250,20 @@ class Affine:
         return Affine(-self.const, [-c for c in self.coeffs])
 
     def __sub__(self, o):
+        if isinstance(o, IndexExpr):
+            return NotImplemented
         return self + (-Affine.lift(o, len(self.coeffs)))
 
     def __rsub__(self, o):
+        if isinstance(o, IndexExpr):
+            return NotImplemented
         return Affine.lift(o, len(self.coeffs)) - self
 
     def __mul__(self, o):
+        if isinstance(o, IndexExpr):
+            return NotImplemented
+        if isinstance(_index_const(o), Fraction):
+            return IndexExpr.make("mul", self, o)
         if isinstance(o, Affine):
             if o.is_const:
                 o = o.const
@@ -188,10 +287,15 @@ class Affine:
 
     __int__ = __index__
 
-    def _unsupported(self, *_):
-        raise TraceError("only +, - and * by a constant are supported on group offsets")
+    def __floordiv__(self, o): return IndexExpr.make("floordiv", self, o)
+    def __rfloordiv__(self, o): return IndexExpr.make("floordiv", o, self)
+    def __mod__(self, o): return IndexExpr.make("mod", self, o)
+    def __rmod__(self, o): return IndexExpr.make("mod", o, self)
 
-    __floordiv__ = __mod__ = __truediv__ = __lt__ = __le__ = __gt__ = __ge__ = _unsupported
+    def _unsupported(self, *_):
+        raise TraceError("only + - * // and % are supported on group offsets")
+
+    __truediv__ = __rtruediv__ = __lt__ = __le__ = __gt__ = __ge__ = _unsupported
 
     def __eq__(self, o):
         o = Affine.lift(o, len(self.coeffs)) if not isinstance(o, Affine) else o
@@ -282,7 +386,8 @@ class BufferProxy:
             starts.append(0 if k.start is None else k.start)
         starts += [0] * (self.ndim - len(starts))
         rank = max((len(s.coeffs) for s in starts if isinstance(s, Affine)), default=0)
-        return BufferView(self, tuple(Affine.lift(s, rank) for s in starts))
+        return BufferView(self, tuple(s if isinstance(s, IndexExpr) else Affine.lift(s, rank)
+                                      for s in starts))
 
     def __setitem__(self, key, value):
         raise TraceError("direct assignment to a buffer is not supported on the GPU path; "
@@ -299,6 +404,11 @@ class BufferView:
         self.base, self.starts = base, starts
 
     @property
+    def affine(self):
+        """False if a start contains // or % of the group id."""
+        return all(isinstance(s, Affine) for s in self.starts)
+
+    @property
     def dtype(self):
         return self.base.dtype
 
@@ -306,7 +416,7 @@ class BufferView:
     def shape(self):
         out = []
         for n, s in zip(self.base.shape, self.starts):
-            if not s.is_const:
+            if not (isinstance(s, Affine) and s.is_const):
                 raise TraceError("the shape of a window that depends on the group id is "
                                  "not a number")
             out.append(max(n - s.const, 0))
@@ -531,6 +641,7 @@ class CurrentGroup:
                          for i in range(rank))
         self.stores = []          # (BufferView, Tile) in program order
         self.atomics = []         # (BufferProxy, element index, Tile) atomic additions
+        self.mapped_stores = []   # (BufferView, Tile, index function) scattered stores
 
     @property
     def id(self):
@@ -550,15 +661,28 @@ class CurrentGroup:
 
     # -- loads and stores ----------------------------------------------------------
     def load(self, array, shape, mapping=None):
-        if mapping is not None:
-            raise TraceError("mapped (gathered) loads have no native kernel yet")
         if not isinstance(shape, Iterable):
             shape = (shape,)
         shape = tuple(int(s) for s in shape)
         if isinstance(array, Tile):
-            raise TraceError("loading from a tile (vload of a register tile) has no native "
-                             "kernel yet")
+            # a tile re-read at another shape: cropped, or padded with inactive
+            # (zero) elements, python/hckernel/kernel_api.py:312-314
+            if mapping is not None:
+                raise TraceError("a mapping on a load from a tile has no native kernel")
+            if len(shape) != len(array.shape):
+                raise TraceError(f"load shape {shape} does not match the rank of the tile")
+            if shape == array.shape:
+                return array
+            return Tile("window", (array,), shape, array.dtype_name)
         view = _as_view(array)
+        if mapping is not None:
+            if not isinstance(mapping, Mapping):
+                raise TraceError("mapping must come from create_mapping")
+            return Tile("mapped_load", (), shape, view.base.dtype_name, view=view,
+                        mapping=mapping.func)
+        if not view.affine:
+            raise TraceError("window offsets that use // or % of the group id are supported "
+                             "on mapped loads and stores only")
         if len(shape) != view.base.ndim:
             raise TraceError(f"load shape {shape} does not match the rank of {view.base.name}")
         return Tile("load", (), shape, view.base.dtype_name, view=view)
@@ -567,9 +691,16 @@ class CurrentGroup:
         return self.load(array, shape, mapping)
 
     def store(self, dst, src, mapping=None):
+        view = _as_view(dst)
         if mapping is not None:
-            raise TraceError("mapped (scattered) stores have no native kernel yet")
-        self.stores.append((_as_view(dst), Tile.wrap(src)))
+            if not isinstance(mapping, Mapping):
+                raise TraceError("mapping must come from create_mapping")
+            self.mapped_stores.append((view, Tile.wrap(src), mapping.func))
+            return
+        if not view.affine:
+            raise TraceError("window offsets that use // or % of the group id are supported "
+                             "on mapped loads and stores only")
+        self.stores.append((view, Tile.wrap(src)))
 
     # -- allocators ------------------------------------------------------------------
     def _alloc(self, shape, dtype, value):

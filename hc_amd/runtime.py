@@ -108,6 +108,18 @@ hcamdLaunchPairwiseDistF32 = _sig(_rt, "hcamdLaunchPairwiseDistF32", _int, _vp, 
                                   _sz, _vp, _sz, _sz, _sz, _sz)
 hcamdLaunchMapSum = _sig(_rt, "hcamdLaunchMapSum", _int, _vp, C.POINTER(MapInstr), _sz,
                          C.POINTER(_vp), C.POINTER(_int), _sz_p, _sz, _vp, _sz, _sz)
+class GatherOperand(C.Structure):
+    """HcamdGatherOperand of include/hc_amd_runtime.h."""
+    _fields_ = [("ndim", _int), ("shape", _sz * 4), ("strides", _sz * 4),
+                ("starts", C.POINTER(C.c_int32)), ("rowIndex", C.POINTER(C.c_int32)),
+                ("colIndex", C.POINTER(C.c_int32))]
+
+
+hcamdGatherGemmCreate = _sig(_rt, "hcamdGatherGemmCreate", _vp, _vp, C.POINTER(GatherOperand),
+                             C.POINTER(GatherOperand), C.POINTER(GatherOperand), _sz, _sz,
+                             _sz, _sz)
+hcamdGatherGemmLaunchF32 = _sig(_rt, "hcamdGatherGemmLaunchF32", _int, _vp, _vp, _vp, _vp, _vp)
+hcamdGatherGemmRelease = _sig(_rt, "hcamdGatherGemmRelease", None, _vp)
 hcamdConvertPyArray = _sig(_py, "hcamdConvertPyArray", _int, C.py_object, _int, _vp,
                            _sz_p, C.c_char_p, _sz)
 hcamdConvertPyInt64 = _sig(_py, "hcamdConvertPyInt64", _int, C.py_object,
@@ -478,6 +490,63 @@ def plan_pairwise_dist_f32(a, b, out) -> Plan:
     return Plan(ctx, hcamdLaunchPairwiseDistF32,
                 (ctx.queue, ma.ptr, lda, mb.ptr, ldb, mo.ptr, ldo, m, n, d),
                 "hcamdLaunchPairwiseDistF32", (a, b, out))
+
+
+class GatherGemm:
+    """Device tables of a product of gathered tiles (hcamdGatherGemmCreate).
+
+    Each operand is described by (shape, strides, starts, row_index,
+    col_index): shape / strides of the whole buffer in elements, starts an
+    int array [n_groups, ndim] with the window start of every group, row_index
+    [tile rows, ndim] and col_index [tile cols, ndim] the index each tile
+    coordinate contributes inside the window."""
+
+    def __init__(self, ctx, a, b, out, n_groups: int, tm: int, tn: int, k: int):
+        import numpy as np
+        self.ctx, self.handle = ctx, None
+        self.layouts = [(tuple(int(v) for v in o[0]), tuple(int(v) for v in o[1]))
+                        for o in (a, b, out)]
+        ops, keep = [], []
+        for shape, strides, starts, rows, cols in (a, b, out):
+            op = GatherOperand()
+            op.ndim = len(shape)
+            if not 1 <= op.ndim <= 4:
+                raise HcRuntimeError("gathered operands have 1 to 4 dimensions")
+            for d in range(op.ndim):
+                op.shape[d], op.strides[d] = int(shape[d]), int(strides[d])
+            tabs = []
+            for t in (starts, rows, cols):
+                t = np.ascontiguousarray(t, dtype=np.int64).reshape(-1, op.ndim)
+                if t.size and (t.max() > 0x7fffffff or t.min() < -0x80000000):
+                    raise HcRuntimeError("gather index out of the 32-bit range")
+                t = t.astype(np.int32)
+                keep.append(t)
+                tabs.append(t.ctypes.data_as(C.POINTER(C.c_int32)))
+            op.starts, op.rowIndex, op.colIndex = tabs
+            ops.append(op)
+        h = hcamdGatherGemmCreate(ctx.queue, C.byref(ops[0]), C.byref(ops[1]), C.byref(ops[2]),
+                                  n_groups, tm, tn, k)
+        if not h:
+            ctx.check(1, "hcamdGatherGemmCreate")
+        self.handle = h
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            hcamdGatherGemmRelease(self.handle)
+            self.handle = None
+
+
+def plan_gather_gemm_f32(tables: GatherGemm, a, b, out) -> Plan:
+    """One launch of a GatherGemm on fp32 buffers of the shapes it was built for."""
+    ctx = _ctx_of(a, b, out)
+    ma, mb, mo = as_memref(a), as_memref(b), as_memref(out)
+    for m, n, lay in zip((ma, mb, mo), ("a", "b", "out"), tables.layouts):
+        _expect(m, 4, n)
+        if (tuple(m.shape), tuple(m.strides)) != lay:
+            raise HcRuntimeError(f"gather_gemm_f32: {n} has shape {m.shape} strides {m.strides}, "
+                                 f"the tables were built for {lay[0]} {lay[1]}")
+    return Plan(ctx, hcamdGatherGemmLaunchF32, (ctx.queue, tables.handle, ma.ptr, mb.ptr, mo.ptr),
+                "hcamdGatherGemmLaunchF32", (tables, a, b, out))
 
 
 def plan_softmax_f32(x, y) -> Plan:

@@ -322,6 +322,48 @@ int hcamdLaunchPairwiseDistF32(OlQueue q, const float *a, size_t lda,
                                size_t ldo, size_t m, size_t n,
                                size_t d) HCAMD_NOEXCEPT;
 
+/* Matrix product of gathered tiles, fp32 -- the operation of a kernel body that
+ * loads its operands through index mappings and multiplies them
+ * (CurrentGroup.load / store with mapping=..., python/hckernel/kernel_api.py:297-345;
+ * the implicit-GEMM convolution of python/hckernel/tests/test_examples.py:168-258):
+ *
+ *     out_g[mo(i, j)] = sum_k a_g[ma(i, k)] * b_g[mb(k, j)]       for every group g
+ *
+ * x_g is the window of buffer x that starts at starts[g][d] along dimension d
+ * (the `x[s0:, s1:, ...]` of the body).  Element (r, c) of a tile sits at index
+ * rowIndex[r][d] + colIndex[c][d] of the window; for every dimension one of
+ * the two tables must be all zero (the index depends on the tile row or on the
+ * tile column, not on both).  An element is active if
+ * 0 <= index < shape[d] - starts[g][d] for every d, which is the reference's
+ * bounds test; inactive operand elements count as zero, inactive output
+ * elements are not written.  The a tile is tm x k, the b tile k x tn, the out
+ * tile tm x tn.  Two active out elements of one launch must not share a
+ * destination (their order is not defined).
+ *
+ * hcamdGatherGemmCreate checks the description, builds the device tables and
+ * returns a plan (NULL after reporting an error); it allocates device memory and
+ * synchronises.  hcamdGatherGemmLaunchF32 enqueues one launch of the plan on
+ * buffers that have the shapes and strides given at creation; it neither
+ * allocates nor synchronises.  All pointers in HcamdGatherOperand are host
+ * memory and are not kept. */
+typedef struct HcamdGatherOperand {
+  int ndim;               /* 1..4 */
+  size_t shape[4];        /* elements per dimension of the whole buffer */
+  size_t strides[4];      /* in elements */
+  const int32_t *starts;  /* [nGroups][ndim], >= 0 */
+  const int32_t *rowIndex; /* [tile rows][ndim] */
+  const int32_t *colIndex; /* [tile cols][ndim] */
+} HcamdGatherOperand;
+typedef struct HcamdGatherGemm_ *HcamdGatherGemm;
+HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
+                                      const HcamdGatherOperand *b,
+                                      const HcamdGatherOperand *out,
+                                      size_t nGroups, size_t tm, size_t tn,
+                                      size_t k) HCAMD_NOEXCEPT;
+int hcamdGatherGemmLaunchF32(OlQueue q, HcamdGatherGemm plan, const float *a,
+                             const float *b, float *out) HCAMD_NOEXCEPT;
+void hcamdGatherGemmRelease(HcamdGatherGemm plan) HCAMD_NOEXCEPT;
+
 /* Row softmax, fp32: y[r,:] = exp(x[r,:]-max(x[r,:])) / sum(exp(...)).
  * Expression of python/hckernel/tests/test_examples.py:330-335. */
 int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,

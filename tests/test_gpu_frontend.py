@@ -577,3 +577,79 @@ def test_unsupported_body_raises_instead_of_running_on_the_cpu():
     with pytest.raises(NoNativeKernel):
         scaled(a, c)
     assert_array_equal(c.to_host(), np.zeros(1000, np.float32))     # untouched
+
+
+# ---------------------------------------------------------------------------
+# mapped loads and stores (python/hckernel/tests/test_examples.py:168-258)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("n,c,nf,stride,tiles", [
+    (1, 1, 1, 1, {}), (2, 3, 2, 2, {}), (4, 3, 8, 3, {}), (4, 1, 8, 1, {}),
+    (3, 2, 5, 1, {sym.TN: 2, sym.TNF: 3}), (9, 3, 10, 2, {sym.TN: 4, sym.TNF: 7, sym.KB: 8})])
+def test_implicit_gemm_convolution_of_the_reference_examples(n, c, nf, stride, tiles):
+    from hc_amd.kernel import create_mapping
+    from oracle import hcsim
+    from test_kernel_frontend import _conv_kernel, conv_direct
+    rng = np.random.default_rng(n + 10 * c + 100 * nf + stride)
+    h = w = 4
+    hf = wf = 2
+    ho, wo = (h - hf) // stride + 1, (w - wf) // stride + 1
+    x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    f = rng.standard_normal((nf, c, hf, wf)).astype(np.float32)
+    out = rt.to_device(np.zeros((n, nf, ho, wo), np.float32))
+    k = _conv_kernel(kernel, create_mapping, stride).parametrize(tiles)
+    k(rt.to_device(x), rt.to_device(f), out)
+    assert rt.last_kernel_name() == "hcamd_gather_gemm_f32"
+    want = np.zeros((n, nf, ho, wo), np.float32)
+    _conv_kernel(sim_kernel, hcsim.create_mapping, stride).parametrize(tiles)(x, f, want)
+    # K = c * hf * wf <= 12 products per output, summed in fp32 in another order
+    assert_allclose(out.to_host(), want, rtol=1e-5, atol=1e-6)
+    assert_allclose(out.to_host(), conv_direct(x, f, stride), rtol=1e-5, atol=1e-5)
+
+
+def test_convolution_at_a_larger_size_with_full_tiles():
+    from hc_amd.kernel import create_mapping
+    from test_kernel_frontend import _conv_kernel, conv_direct
+    rng = np.random.default_rng(2024)
+    n, c, hw, nf, hf = 70, 6, 13, 66, 3          # (hw - hf) divisible by both strides
+    x = rng.standard_normal((n, c, hw, hw)).astype(np.float32)
+    f = rng.standard_normal((nf, c, hf, hf)).astype(np.float32)
+
+    # the example's mappings assume 2 x 2 filters only through HF * WF; 3 x 3 works the same
+    for stride, tiles in ((1, {sym.TN: 63, sym.TNF: 63, sym.KB: 16}), (2, {sym.TN: 32, sym.TNF: 40})):
+        ho = (hw - hf) // stride + 1
+        out = rt.to_device(np.full((n, nf, ho, ho), np.nan, np.float32))
+        _conv_kernel(kernel, create_mapping, stride).parametrize(tiles)(
+            rt.to_device(x), rt.to_device(f), out)
+        got = out.to_host()
+        assert not np.isnan(got).any()
+        assert_allclose(got, conv_direct(x, f, stride), rtol=1e-4, atol=(c * hf * hf + 2) * 2.0 ** -22)
+
+
+def test_float32_dot_with_row_major_b():
+    """The blocked dot of python/hckernel/tests/test_examples.py:74-121 on fp32
+    arrays: binds to the gathered product with identity mappings."""
+    M, N, K, GM, GN, KB = sym.M, sym.N, sym.K, sym.GM, sym.GN, sym.KB
+    KI = cdiv(K, KB)
+
+    def make(deco):
+        @deco(work_shape=(M, N), group_shape=(GM, GN), tunables=TunableParam(KB, 8, (8, 16)))
+        def dot(gr: CurrentGroup, a: Buffer[M, K, DT], b: Buffer[K, N, DT], out: Buffer[M, N, DT],
+                gshape: (GM, GN)):
+            m0, n0 = gr.work_offset
+            r = gr.zeros(shape=gr.shape, dtype=out.dtype)
+            for k in range(KI):
+                r += np.dot(gr.load(a[m0:, k * KB:], shape=(gr.shape[0], KB)),
+                            gr.load(b[k * KB:, n0:], shape=(KB, gr.shape[1])))
+            gr.store(out[m0:, n0:], r)
+        return dot
+
+    rng = np.random.default_rng(31)
+    a = rng.standard_normal((130, 77)).astype(np.float32)
+    b = rng.standard_normal((77, 95)).astype(np.float32)
+    out = rt.to_device(np.zeros((130, 95), np.float32))
+    make(kernel)(rt.to_device(a), rt.to_device(b), out, (64, 64))
+    assert rt.last_kernel_name() == "hcamd_gather_gemm_f32"
+    want = np.zeros((130, 95), np.float32)
+    make(sim_kernel)(a, b, want, (64, 64))
+    assert_allclose(out.to_host(), want, rtol=1e-4, atol=79 * 2.0 ** -22)
+    assert_allclose(out.to_host(), a.astype(np.float64) @ b, rtol=1e-4, atol=79 * 2.0 ** -22)

@@ -335,6 +335,114 @@ def test_pairwise_distances_against_fp64(ctx, mnd):
 
 
 # ---------------------------------------------------------------------------
+# product of gathered tiles
+# ---------------------------------------------------------------------------
+def _operand(arr_shape, starts, rows, cols, strides=None):
+    if strides is None:
+        strides = tuple(int(np.prod(arr_shape[d + 1:])) for d in range(len(arr_shape)))
+    return (tuple(arr_shape), strides, np.asarray(starts, np.int64).reshape(-1, len(arr_shape)),
+            np.asarray(rows, np.int64).reshape(-1, len(arr_shape)),
+            np.asarray(cols, np.int64).reshape(-1, len(arr_shape)))
+
+
+def _gather_reference(ops, n_groups, tm, tn, k, a, b, out):
+    from test_kernel_frontend import TablesOnly
+    t = TablesOnly(None, *ops, n_groups, tm, tn, k)
+    t.run(a, b, out)
+    return out
+
+
+@pytest.mark.parametrize("case", ["plain", "tails", "blocks", "transposed", "k0"])
+def test_gathered_product_against_the_table_semantics(ctx, case):
+    rng = np.random.default_rng(len(case))
+    # a[M, K] x b[K, N] walked by gm x gn groups of tm x tn tiles, written as tables
+    M, N, K, tm, tn = {"plain": (64, 64, 32, 64, 64), "tails": (70, 45, 37, 16, 24),
+                       "blocks": (150, 140, 70, 130, 70), "transposed": (33, 50, 19, 20, 20),
+                       "k0": (9, 9, 0, 8, 8)}[case]
+    gm, gn = -(-M // tm), -(-N // tn)
+    a = rng.standard_normal((M, max(K, 1))).astype(np.float32)[:, :K]
+    a = np.ascontiguousarray(a) if K else np.zeros((M, 1), np.float32)
+    kk = max(K, 1)
+    if case == "transposed":                       # b stored as [N, K], out as [N, M]
+        b = rng.standard_normal((N, kk)).astype(np.float32)
+        b_op = _operand(b.shape, [[gj * tn, 0] for gi in range(gm) for gj in range(gn)],
+                        [[0, r] for r in range(K)], [[c, 0] for c in range(tn)])
+        out_shape = (N, M)
+        o_op = _operand(out_shape, [[gj * tn, gi * tm] for gi in range(gm) for gj in range(gn)],
+                        [[0, r] for r in range(tm)], [[c, 0] for c in range(tn)])
+    else:
+        b = rng.standard_normal((kk, N)).astype(np.float32)
+        b_op = _operand(b.shape, [[0, gj * tn] for gi in range(gm) for gj in range(gn)],
+                        [[r, 0] for r in range(K)], [[0, c] for c in range(tn)])
+        out_shape = (M, N)
+        o_op = _operand(out_shape, [[gi * tm, gj * tn] for gi in range(gm) for gj in range(gn)],
+                        [[r, 0] for r in range(tm)], [[0, c] for c in range(tn)])
+    a_op = _operand(a.shape, [[gi * tm, 0] for gi in range(gm) for gj in range(gn)],
+                    [[r, 0] for r in range(tm)], [[0, c] for c in range(K)])
+    ops = (a_op, b_op, o_op)
+    tables = rt.GatherGemm(ctx, *ops, gm * gn, tm, tn, K)
+    out = poisoned(out_shape, np.float32)
+    say("gather", case, M, N, K, tm, tn)
+    rt.plan_gather_gemm_f32(tables, dev(a), dev(b), out).launch(sync=True)
+    got = out.to_host()
+    want = _gather_reference(ops, gm * gn, tm, tn, K, a, b, np.full(out_shape, np.nan, np.float32))
+    assert not np.isnan(want).any()
+    full = a[:, :K].astype(np.float64) @ (b[:, :K].T if case == "transposed" else b[:K]).astype(np.float64)
+    assert_allclose(want, full.T if case == "transposed" else full, rtol=1e-6, atol=1e-6)
+    assert_allclose(got, want, rtol=1e-5, atol=(K + 2) * 2.0 ** -22)
+
+
+def test_gathered_product_inactive_elements_and_untouched_memory(ctx):
+    """Windows that leave the buffer, negative and too-large indices, a start
+    beyond the end: inactive operands count as zero, inactive outputs keep
+    their bytes."""
+    rng = np.random.default_rng(77)
+    a = rng.standard_normal((3, 10, 7)).astype(np.float32)        # [batch, rows, k]
+    b = rng.standard_normal((7, 12)).astype(np.float32)
+    out_shape = (3, 12, 11)                                         # [batch, cols, rows + 1]
+    tm, tn, k = 6, 8, 9
+    groups = [(g0, g1) for g0 in range(4) for g1 in range(2)]       # batch 3 does not exist
+    a_op = _operand(a.shape, [[g0, 5 * g1, 0] for g0, g1 in groups],
+                    [[0, r - 1, 0] for r in range(tm)],             # row -1 is inactive
+                    [[0, 0, c] for c in range(k)])                  # k = 7, 8 are inactive
+    b_op = _operand(b.shape, [[0, 0] for _ in groups], [[r, 0] for r in range(k)],
+                    [[0, 2 * c] for c in range(tn)])                # every other column, 14 is inactive
+    o_op = _operand(out_shape, [[g0, 0, 6 * g1] for g0, g1 in groups],      # row 11 is inactive
+                    [[0, 0, r] for r in range(tm)], [[0, 11 - 2 * c, 0] for c in range(tn)])
+    ops = (a_op, b_op, o_op)
+    tables = rt.GatherGemm(ctx, *ops, len(groups), tm, tn, k)
+    out = poisoned(out_shape, np.float32)
+    rt.plan_gather_gemm_f32(tables, dev(a), dev(b), out).launch(sync=True)
+    got = out.to_host()
+    p = poison_value(np.float32)
+    want = _gather_reference(ops, len(groups), tm, tn, k, a, b, np.full(out_shape, p, np.float32))
+    written = want.view(np.uint32) != POISON32
+    assert written.any() and not written.all()
+    assert_array_equal(got.view(np.uint32)[~written], want.view(np.uint32)[~written])
+    assert_allclose(got[written], want[written], rtol=1e-5, atol=1e-5)
+
+
+def test_gathered_product_rejects_bad_descriptions(ctx):
+    ok = _operand((8, 8), [[0, 0]], [[r, 0] for r in range(4)], [[0, c] for c in range(4)])
+    both = _operand((8, 8), [[0, 0]], [[r, r] for r in range(4)], [[0, c] for c in range(4)])
+    neg = _operand((8, 8), [[-1, 0]], [[r, 0] for r in range(4)], [[0, c] for c in range(4)])
+    big = ((1 << 20, 1 << 12), (1 << 12, 1), ok[2], ok[3], ok[4])
+    for what, ops in {"both tile coordinates": (both, ok, ok), "negative window start": (ok, neg, ok),
+                      "2\\^31": (ok, ok, big)}.items():
+        with pytest.raises(rt.HcRuntimeError, match=what):
+            rt.GatherGemm(ctx, *ops, 1, 4, 4, 4)
+    with pytest.raises(rt.HcRuntimeError, match="invalid sizes"):
+        rt.GatherGemm(ctx, ok, ok, ok, 0, 4, 4, 4)
+    tables = rt.GatherGemm(ctx, ok, ok, ok, 1, 4, 4, 4)
+    x = dev(np.zeros((8, 8), np.float32))
+    with pytest.raises(rt.HcRuntimeError, match="built for"):
+        rt.plan_gather_gemm_f32(tables, x, x, dev(np.zeros((8, 9), np.float32)))
+    assert rt.hcamdGatherGemmLaunchF32(ctx.queue, tables.handle, x.ptr, None, x.ptr) == 1
+    with pytest.raises(rt.HcRuntimeError, match="null pointer"):
+        ctx.check(1, "hcamdGatherGemmLaunchF32")
+
+
+# ---------------------------------------------------------------------------
 # fused elementwise map (postfix programs)
 # ---------------------------------------------------------------------------
 def I(name, arg=0, imm=0.0):

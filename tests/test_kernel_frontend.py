@@ -472,3 +472,191 @@ def test_tuned_params_round_trip_and_parametrize(tmp_path, ctx):
     assert tuned.tuned == {N: 4, GS: 128} and tuned.variants == {"add": 7}
     (p,) = tuned.plan(FakeDev((5000,), "float32"), FakeDev((1,), "float32"), ctx=ctx)
     assert p.fn is rt.hcamdLaunchMapSum and p.args[8:] == (1, 5000)
+
+
+# ---------------------------------------------------------------------------
+# Mapped loads / stores: products of gathered tiles
+# ---------------------------------------------------------------------------
+def _conv_kernel(deco, make_mapping, stride):
+    """The implicit-GEMM convolution of python/hckernel/tests/test_examples.py:203-252:
+    a group owns TN images x TNF filters at one output position; the im2col
+    row of an image and the flattened filter are gathered through mappings."""
+    N, C, H, W, NF, HF, WF, KB = (sym.N, sym.C, sym.H, sym.W, sym.NF, sym.HF, sym.WF, sym.KB)
+    TN, TNF = sym.TN, sym.TNF
+    HO = (H - HF) / stride + 1
+    WO = (W - WF) / stride + 1
+    SZ = HF * WF * C
+    KI = cdiv(SZ, KB)
+    tun = (TunableParam(TN, 8, range(1, 64)), TunableParam(TNF, 8, range(1, 64)),
+           TunableParam(KB, 16, range(8, 128)))
+    x_map = make_mapping(lambda i, j: (i, j // (HF * WF), (j % (HF * WF)) % WF,
+                                       (j % (HF * WF)) // WF))
+    f_map = make_mapping(lambda i, j: (j, i // (HF * WF), i % WF, (i % (HF * WF)) // WF))
+    o_map = make_mapping(lambda i, j: (i, j, 0, 0))
+
+    @deco(work_shape=(N, NF, HO * WO), group_shape=(TN, TNF, 1), tunables=tun)
+    def conv(gr: CurrentGroup, xs: Buffer[N, C, H, W, DT], fs: Buffer[NF, C, HF, WF, DT],
+             out: Buffer[N, NF, HO, WO, DT]):
+        i0, o0, idx = gr.work_offset
+        p, q = idx % WO, idx // WO
+        xv = gr.load(xs[i0:, :, p * stride:, q * stride:], shape=(TN, SZ), mapping=x_map)
+        fv = gr.load(fs[o0:, :, :, :], shape=(SZ, TNF), mapping=f_map)
+        r = gr.zeros(shape=(xv.shape[0], fv.shape[1]), dtype=out.dtype)
+        for k in range(KI):
+            r += np.dot(gr.vload(xv[:, k * KB:], shape=(TN, KB)),
+                        gr.vload(fv[k * KB:, :], shape=(KB, TNF)))
+        gr.store(out[i0:, o0:, p:, q:], r, mapping=o_map)
+    return conv
+
+
+def conv_direct(x, f, stride):
+    """Valid cross-correlation, NCHW, square output walk as in the example."""
+    n, c, h, w = x.shape
+    nf, _, hf, wf = f.shape
+    ho, wo = (h - hf) // stride + 1, (w - wf) // stride + 1
+    out = np.zeros((n, nf, ho, wo), np.float64)
+    for p in range(ho):
+        for q in range(wo):
+            win = x[:, :, p * stride:p * stride + hf, q * stride:q * stride + wf]
+            out[:, :, p, q] = np.einsum("nchw,fchw->nf", win.astype(np.float64),
+                                        f.astype(np.float64))
+    return out
+
+
+class TablesOnly:
+    """Stands in for hc_amd.runtime.GatherGemm: keeps the host tables."""
+    last = None
+
+    def __init__(self, ctx, a, b, out, n_groups, tm, tn, k):
+        self.ctx, self.handle = ctx, 0xABCD
+        self.ops, self.n_groups, self.tm, self.tn, self.k = (a, b, out), n_groups, tm, tn, k
+        self.layouts = [(tuple(o[0]), tuple(o[1])) for o in (a, b, out)]
+        TablesOnly.last = self
+
+    def run(self, a, b, out):
+        """The meaning of the tables (include/hc_amd_runtime.h, HcamdGatherOperand):
+        element (r, c) of a group's tile sits at index rows[r] + cols[c] of the
+        window that starts at starts[g]; it is active while every index is
+        inside the window.  Products are summed in float64."""
+        def tile(op, arr, g, nr, nc):
+            shape, _, starts, rows, cols = op
+            idx = rows[:nr, None, :] + cols[None, :nc, :]
+            ok = ((idx >= 0) & (idx < np.asarray(shape) - starts[g])).all(-1)
+            src = np.where(ok[..., None], idx + starts[g], 0)
+            vals = arr[tuple(src[..., d] for d in range(len(shape)))]
+            return np.where(ok, vals, 0), ok, src
+
+        for g in range(self.n_groups):
+            ta, _, _ = tile(self.ops[0], a, g, self.tm, self.k)
+            tb, _, _ = tile(self.ops[1], b, g, self.k, self.tn)
+            _, ok, dst = tile(self.ops[2], out, g, self.tm, self.tn)
+            prod = ta.astype(np.float64) @ tb.astype(np.float64)
+            out[tuple(dst[ok][:, d] for d in range(dst.shape[-1]))] = prod[ok]
+
+
+@pytest.mark.parametrize("n,c,nf,stride,tiles", [
+    (1, 1, 1, 1, {}), (2, 3, 2, 2, {}), (4, 3, 8, 3, {}), (3, 2, 5, 1, {sym.TN: 2, sym.TNF: 3}),
+    (5, 3, 4, 1, {sym.TN: 4, sym.TNF: 4, sym.KB: 8})])
+def test_convolution_example_binds_to_the_gathered_product(ctx, monkeypatch, n, c, nf, stride, tiles):
+    from hc_amd.kernel import create_mapping
+    from oracle import hcsim
+    monkeypatch.setattr(rt, "GatherGemm", TablesOnly)
+    rng = np.random.default_rng(5)
+    h = w = 4
+    hf = wf = 2
+    ho, wo = (h - hf) // stride + 1, (w - wf) // stride + 1
+    x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    f = rng.standard_normal((nf, c, hf, wf)).astype(np.float32)
+
+    k = _conv_kernel(kernel, create_mapping, stride).parametrize(tiles)
+    dx, df, do = FakeDev(x.shape, "float32"), FakeDev(f.shape, "float32"), \
+        FakeDev((n, nf, ho, wo), "float32")
+    (p,) = k.plan(dx, df, do, ctx=ctx)
+    assert p.fn is rt.hcamdGatherGemmLaunchF32
+    t = TablesOnly.last
+    assert p.args == (ctx.queue, t.handle, dx.ptr, df.ptr, do.ptr)
+    tn, tnf = tiles.get(sym.TN, 8), tiles.get(sym.TNF, 8)
+    assert (t.tm, t.tn, t.k) == (tn, tnf, c * hf * wf)
+    got = np.full((n, nf, ho, wo), np.nan, np.float32)
+    t.run(x, f, got)
+
+    sim = hcsim.kernel
+    want = np.zeros((n, nf, ho, wo), np.float32)
+    _conv_kernel(sim, hcsim.create_mapping, stride).parametrize(tiles)(x, f, want)
+    assert not np.isnan(got).any()                       # every output was written
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(got, conv_direct(x, f, stride), rtol=1e-5, atol=1e-5)
+
+
+def test_plain_float32_dot_binds_to_the_gathered_product(ctx, monkeypatch):
+    monkeypatch.setattr(rt, "GatherGemm", TablesOnly)
+    M, N, K, GM, GN, KB = sym.M, sym.N, sym.K, sym.GM, sym.GN, sym.KB
+    KI = cdiv(K, KB)
+
+    @kernel(work_shape=(M, N), group_shape=(GM, GN), tunables=TunableParam(KB, 8, (8, 16)))
+    def dot(gr: CurrentGroup, a: Buffer[M, K, DT], b: Buffer[K, N, DT], out: Buffer[M, N, DT],
+            gshape: (GM, GN)):
+        m0, n0 = gr.work_offset
+        r = gr.zeros(shape=gr.shape, dtype=out.dtype)
+        for k in range(KI):
+            r += np.dot(gr.load(a[m0:, k * KB:], shape=(gr.shape[0], KB)),
+                        gr.load(b[k * KB:, n0:], shape=(KB, gr.shape[1])))
+        gr.store(out[m0:, n0:], r)
+
+    rng = np.random.default_rng(6)
+    a = rng.standard_normal((13, 21)).astype(np.float32)
+    b = rng.standard_normal((21, 10)).astype(np.float32)
+    (p,) = dot.plan(FakeDev(a.shape, "float32"), FakeDev(b.shape, "float32"),
+                    FakeDev((13, 10), "float32"), (8, 4), ctx=ctx)
+    assert p.fn is rt.hcamdGatherGemmLaunchF32
+    t = TablesOnly.last
+    assert (t.n_groups, t.tm, t.tn, t.k) == (2 * 3, 8, 4, 24)
+    got = np.full((13, 10), np.nan, np.float32)
+    t.run(a, b, got)
+    np.testing.assert_allclose(got, a.astype(np.float64) @ b.astype(np.float64), rtol=1e-5, atol=1e-5)
+
+
+def test_mappings_that_no_table_can_express_are_refused(ctx, monkeypatch):
+    from hc_amd.kernel import create_mapping
+    monkeypatch.setattr(rt, "GatherGemm", TablesOnly)
+    M, N, K = sym.M, sym.N, sym.K
+
+    def make(a_func, dtype="float32", store_func=None):
+        a_map = create_mapping(a_func)
+        o_map = create_mapping(store_func) if store_func else None
+
+        @kernel(work_shape=(M, N), group_shape=(4, 4))
+        def body(gr: CurrentGroup, a: Buffer[M, K, DT], b: Buffer[K, N, DT], out: Buffer[M, N, DT]):
+            m0, n0 = gr.work_offset
+            av = gr.load(a[m0:, :], shape=(4, K), mapping=a_map)
+            bv = gr.load(b[:, n0:], shape=(K, 4))
+            gr.store(out[m0:, n0:], np.dot(av, bv), mapping=o_map)
+        return body.plan(FakeDev((8, 6), dtype), FakeDev((6, 8), dtype), FakeDev((8, 8), dtype),
+                         ctx=ctx)
+
+    (p,) = make(lambda i, j: (i, j))
+    assert p.fn is rt.hcamdGatherGemmLaunchF32
+    (p,) = make(lambda i, j: (i, 5 - j), store_func=lambda i, j: (3 - i, j))   # reversed K, flipped rows
+    assert p.fn is rt.hcamdGatherGemmLaunchF32
+    with pytest.raises(NoNativeKernel, match="both tile coordinates"):
+        make(lambda i, j: (i + j, j))
+    with pytest.raises(NoNativeKernel, match="one destination"):
+        make(lambda i, j: (i, j), store_func=lambda i, j: (i // 2, j))
+    with pytest.raises(NoNativeKernel, match="float32"):
+        make(lambda i, j: (i, j), dtype="float16", store_func=lambda i, j: (i, j))
+    with pytest.raises(NoNativeKernel, match="must return 2 indices"):
+        make(lambda i, j: (i, j, 0))
+    with pytest.raises(NoNativeKernel, match="cannot be evaluated"):
+        make(lambda i, j: (i, j if j < 3 else 0))
+
+
+def test_offsets_with_division_are_for_mapped_accesses_only(ctx):
+    W, H = sym.W, sym.H
+
+    @kernel(work_shape=(W, H), group_shape=(4, 4))
+    def body(gr: CurrentGroup, src: Buffer[W, H, DT], dst: Buffer[W, H, DT]):
+        x, y = gr.work_offset
+        gr.store(dst[x:, y:], gr.load(src[x // 2:, y:], shape=gr.shape))
+
+    with pytest.raises(NoNativeKernel, match="mapped loads and stores only"):
+        body.plan(FakeDev((8, 8), "float32"), FakeDev((8, 8), "float32"), ctx=ctx)
