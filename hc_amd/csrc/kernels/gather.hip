@@ -19,20 +19,21 @@
 //   *_rows[r], *_cols[c]  8 ints: {offset, index[4], unused[3]} (offset = sum
 //              of index * stride; dimensions the other coordinate drives hold 0)
 //
-// One workgroup of 256 lanes per group; the TM x TN tile is walked in 64 x 64
-// blocks, 4 x 4 outputs per lane, K in steps of 32 through LDS panels stored
-// k-major so that a lane's four operands are one 16-byte LDS read.  The gathers
-// of the next K step are issued before the multiply-adds of the current one.
-// Consecutive groups (which usually share operand data) go to the same XCD so
-// that they share its L2.
+// One workgroup per group; the TM x TN tile is walked in T x T blocks, R x R
+// outputs per lane, K in steps of 32 through LDS panels stored k-major so that
+// a lane's R operands are one LDS read.  Four shapes are built: T = 64 (R = 4,
+// 256 lanes) for large tiles and T = 32, 16, 8 (R = 4, 2, 1, one wave) so that
+// small tiles do not pay for a 64 x 64 block of mostly inactive lanes.  The
+// gathers of the next K step are issued before the multiply-adds of the current
+// one.  The host lays the group records out by window address, and consecutive
+// records go to the same XCD, so that groups that run together share cache lines
+// in that XCD's L2.
 #include "common.h"
 
 using namespace hcamd;
 
 namespace {
-constexpr int kTile = 64;
 constexpr int kStep = 32;
-constexpr int kPitch = kTile + 4;
 constexpr int kXcds = 8;
 
 struct GatherGemmArgs {
@@ -66,13 +67,17 @@ __device__ __forceinline__ Window window_of(const int32_t *rec) {
     w.ext[d] = static_cast<uint32_t>(rec[1 + d]);
   return w;
 }
-} // namespace
-
-extern "C" __global__ __launch_bounds__(256) void hcamd_gather_gemm_f32(
-    GatherGemmArgs p) {
+template <int T, int R>
+__device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
+  constexpr int kSide = T / R;            // lanes per block edge
+  constexpr int kThreads = kSide * kSide;
+  constexpr int kPitch = T + 4;
+  constexpr int kRowsPerPass = kThreads / kStep;
+  constexpr int kPasses = T / kRowsPerPass; // gathers per lane, operand and K step
+  static_assert(kThreads % kStep == 0 && T % kRowsPerPass == 0, "panel split");
   __shared__ __attribute__((aligned(16))) float as[kStep][kPitch];
   __shared__ __attribute__((aligned(16))) float bs[kStep][kPitch];
-  __shared__ int row_a[kTile], col_b[kTile], row_o[kTile], col_o[kTile];
+  __shared__ int row_a[T], col_b[T], row_o[T], col_o[T];
 
   const uint32_t g = (blockIdx.x % kXcds) * p.per_xcd + blockIdx.x / kXcds;
   if (g >= p.n_groups)
@@ -85,36 +90,38 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_gather_gemm_f32(
   float *out = p.out + wo.base;
 
   const int t = threadIdx.x;
-  const int tx = t % 16, ty = t / 16;
+  const int tx = t % kSide, ty = t / kSide;
   const int ld_k = t % kStep, ld_r = t / kStep;
 
-  for (uint32_t m0 = 0; m0 < p.tm; m0 += kTile)
-    for (uint32_t n0 = 0; n0 < p.tn; n0 += kTile) {
-      if (t < kTile) {
-        const uint32_t r = m0 + t;
-        row_a[t] = r < p.tm ? resolve(p.a_rows + 8 * (size_t)r, wa) : -1;
-        row_o[t] = r < p.tm ? resolve(p.o_rows + 8 * (size_t)r, wo) : -1;
-      } else if (t < 2 * kTile) {
-        const uint32_t c = n0 + t - kTile;
-        col_b[t - kTile] = c < p.tn ? resolve(p.b_cols + 8 * (size_t)c, wb) : -1;
-        col_o[t - kTile] = c < p.tn ? resolve(p.o_cols + 8 * (size_t)c, wo) : -1;
+  for (uint32_t m0 = 0; m0 < p.tm; m0 += T)
+    for (uint32_t n0 = 0; n0 < p.tn; n0 += T) {
+      for (int e = t; e < 2 * T; e += kThreads) {
+        if (e < T) {
+          const uint32_t r = m0 + e;
+          row_a[e] = r < p.tm ? resolve(p.a_rows + 8 * (size_t)r, wa) : -1;
+          row_o[e] = r < p.tm ? resolve(p.o_rows + 8 * (size_t)r, wo) : -1;
+        } else {
+          const uint32_t c = n0 + e - T;
+          col_b[e - T] = c < p.tn ? resolve(p.b_cols + 8 * (size_t)c, wb) : -1;
+          col_o[e - T] = c < p.tn ? resolve(p.o_cols + 8 * (size_t)c, wo) : -1;
+        }
       }
       __syncthreads();
 
-      int ra[8], cb[8];
+      int ra[kPasses], cb[kPasses];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        ra[i] = row_a[ld_r + 8 * i];
-        cb[i] = col_b[ld_r + 8 * i];
+      for (int i = 0; i < kPasses; ++i) {
+        ra[i] = row_a[ld_r + kRowsPerPass * i];
+        cb[i] = col_b[ld_r + kRowsPerPass * i];
       }
-      float acc[4][4];
+      float acc[R][R];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < R; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < R; ++j)
           acc[i][j] = 0.0f;
 
-      float va[8], vb[8];
+      float va[kPasses], vb[kPasses];
       auto gather = [&](uint32_t k0) {
         const uint32_t kk = k0 + ld_k;
         int oa = -1, ob = -1;
@@ -123,7 +130,7 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_gather_gemm_f32(
           ob = resolve(p.b_rows + 8 * (size_t)kk, wb);
         }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < kPasses; ++i) {
           // both offsets are non-negative when valid: the sign of the OR says
           // whether either is the -1 marker
           va[i] = (oa | ra[i]) >= 0 ? a[oa + ra[i]] : 0.0f;
@@ -135,32 +142,46 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_gather_gemm_f32(
         gather(0);
       for (uint32_t k0 = 0; k0 < p.k; k0 += kStep) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          as[ld_k][ld_r + 8 * i] = va[i];
-          bs[ld_k][ld_r + 8 * i] = vb[i];
+        for (int i = 0; i < kPasses; ++i) {
+          as[ld_k][ld_r + kRowsPerPass * i] = va[i];
+          bs[ld_k][ld_r + kRowsPerPass * i] = vb[i];
         }
         __syncthreads();
         if (k0 + kStep < p.k)
           gather(k0 + kStep);
 #pragma unroll 8
         for (int kk = 0; kk < kStep; ++kk) {
-          const f32x4 av = *reinterpret_cast<const f32x4 *>(&as[kk][4 * ty]);
-          const f32x4 bv = *reinterpret_cast<const f32x4 *>(&bs[kk][4 * tx]);
+          float av[R], bv[R];
+          if constexpr (R == 4) {
+            const f32x4 x = *reinterpret_cast<const f32x4 *>(&as[kk][R * ty]);
+            const f32x4 y = *reinterpret_cast<const f32x4 *>(&bs[kk][R * tx]);
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < R; ++i) {
+              av[i] = x[i];
+              bv[i] = y[i];
+            }
+          } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int i = 0; i < R; ++i) {
+              av[i] = as[kk][R * ty + i];
+              bv[i] = bs[kk][R * tx + i];
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < R; ++i)
+#pragma unroll
+            for (int j = 0; j < R; ++j)
               acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
         }
         __syncthreads();
       }
 
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int ro = row_o[4 * ty + i];
+      for (int i = 0; i < R; ++i) {
+        const int ro = row_o[R * ty + i];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int co = col_o[4 * tx + j];
+        for (int j = 0; j < R; ++j) {
+          const int co = col_o[R * tx + j];
           if ((ro | co) >= 0)
             out[ro + co] = acc[i][j];
         }
@@ -168,3 +189,14 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_gather_gemm_f32(
       __syncthreads();
     }
 }
+} // namespace
+
+#define HCAMD_GATHER_GEMM(T, R)                                                \
+  extern "C" __global__ __launch_bounds__((T / R) * (T / R)) void              \
+      hcamd_gather_gemm_f32_t##T(GatherGemmArgs p) {                           \
+    gather_gemm<T, R>(p);                                                      \
+  }
+HCAMD_GATHER_GEMM(64, 4)
+HCAMD_GATHER_GEMM(32, 4)
+HCAMD_GATHER_GEMM(16, 2)
+HCAMD_GATHER_GEMM(8, 1)

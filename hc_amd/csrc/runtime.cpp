@@ -262,7 +262,8 @@ uint32_t upPow2(uint32_t x) {
 std::unordered_map<std::string, int> &variants() {
   static std::unordered_map<std::string, int> v{
       {"add", 0},     {"fma", 0},  {"softmax", 0},
-      {"quantize", 0}, {"gemm", 0}, {"copy", 0}, {"map", 0}};
+      {"quantize", 0}, {"gemm", 0}, {"copy", 0}, {"map", 0},
+      {"gather", 0}};
   return v;
 }
 int variantOf(const char *family) { return variants()[family]; }
@@ -1258,8 +1259,28 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
     delete plan;
     return nullptr;
   }
+  // Groups may run in any order.  They are laid out by the address of their a
+  // window (then b), so that workgroups that are resident together, and the
+  // run of groups each XCD receives, touch neighbouring memory: windows that
+  // overlap or share cache lines are then served by one L2 fill.
+  std::vector<uint32_t> order(nGroups);
+  std::vector<int64_t> key(nGroups * 2, 0);
   for (size_t g = 0; g < nGroups; ++g) {
-    int32_t *rec = host.data() + plan->offGroups + g * kGatherRecord;
+    order[g] = (uint32_t)g;
+    for (int o = 0; o < 2; ++o) {
+      const HcamdGatherOperand &op = *ops[o];
+      for (int d = 0; d < op.ndim; ++d)
+        key[g * 2 + o] += (int64_t)op.starts[g * op.ndim + d] * (int64_t)op.strides[d];
+    }
+  }
+  std::stable_sort(order.begin(), order.end(), [&](uint32_t x, uint32_t y) {
+    if (key[2 * (size_t)x] != key[2 * (size_t)y])
+      return key[2 * (size_t)x] < key[2 * (size_t)y];
+    return key[2 * (size_t)x + 1] < key[2 * (size_t)y + 1];
+  });
+  for (size_t slot = 0; slot < nGroups; ++slot) {
+    const size_t g = order[slot];
+    int32_t *rec = host.data() + plan->offGroups + slot * kGatherRecord;
     for (int o = 0; o < 3; ++o) {
       const HcamdGatherOperand &op = *ops[o];
       int32_t *w = rec + 5 * o;
@@ -1315,7 +1336,23 @@ int hcamdGatherGemmLaunchF32(OlQueue q, HcamdGatherGemm plan, const float *a,
     dev->report("hcamdGatherGemmLaunchF32: null pointer");
     return 1;
   }
-  Kernel *kern = builtinKernel(dev, "gather", "hcamd_gather_gemm_f32");
+  // block edge of the kernel: the smallest of 8, 16, 32, 64 that holds the
+  // tile (64 for larger tiles, which are walked block by block)
+  const uint32_t side = std::max(plan->tm, plan->tn);
+  const int variant = variantOf("gather");
+  const char *name = "hcamd_gather_gemm_f32_t64";
+  size_t threads = 256;
+  if (variant == 0 ? side <= 8 : variant == 4) {
+    name = "hcamd_gather_gemm_f32_t8";
+    threads = 64;
+  } else if (variant == 0 ? side <= 16 : variant == 3) {
+    name = "hcamd_gather_gemm_f32_t16";
+    threads = 64;
+  } else if (variant == 0 ? side <= 32 : variant == 2) {
+    name = "hcamd_gather_gemm_f32_t32";
+    threads = 64;
+  }
+  Kernel *kern = builtinKernel(dev, "gather", name);
   if (!kern)
     return 1;
   GatherGemmArgs args;
@@ -1337,7 +1374,7 @@ int hcamdGatherGemmLaunchF32(OlQueue q, HcamdGatherGemm plan, const float *a,
   args.per_xcd = (plan->nGroups + 7) / 8;
   void *params[] = {&args};
   const size_t grid[3] = {(size_t)args.per_xcd * 8, 1, 1};
-  const size_t block[3] = {256, 1, 1};
+  const size_t block[3] = {threads, 1, 1};
   return launch(queue, kern, grid, block, params, 0);
 }
 

@@ -399,8 +399,8 @@ int hcamdLaunchGemmF16(OlQueue q, const void *a, size_t lda, const void *bt,
 
 /* Chooses between kernel variants of one family by number (0 = default
  * choice by shape).  For tuning and measurement; family names are "add",
- * "fma", "softmax", "quantize", "gemm", "copy". Returns 1 for an unknown
- * family. */
+ * "fma", "softmax", "quantize", "gemm", "copy", "map", "gather". Returns 1
+ * for an unknown family. */
 int hcamdSetVariant(const char *family, int variant) HCAMD_NOEXCEPT;
 
 /* Name and launch geometry of the kernel the most recent typed launcher
