@@ -287,6 +287,49 @@ def make_workloads(rt, wl):
             t = _best_of(lambda: np.linalg.norm(a[:, None, :] - b[None, :, :], axis=2), 2)
             return t * (self.M / 512) * (self.N / 512), "512 x 512 block scaled to full size", 1
 
+    class X4(Workload):
+        """3 x 3 convolution, NCHW fp32, written as the implicit-GEMM body of the
+        reference's examples (one group = 64 images x 64 filters at one output
+        position, operands gathered through index mappings) and launched
+        through the @kernel front-end."""
+        N, C, HW, NF, F = 64, 64, 58, 64, 3
+
+        def setup(self, rt):
+            from hc_amd.examples import convolution
+            self.kernel = convolution(stride=1, tile=64, k_block=64)
+            rng = np.random.default_rng(7)
+            self.x = rng.standard_normal((self.N, self.C, self.HW, self.HW)).astype(np.float32)
+            self.f = rng.standard_normal((self.NF, self.C, self.F, self.F)).astype(np.float32)
+            ho = self.HW - self.F + 1
+            return [(rt.to_device(self.x), rt.to_device(self.f),
+                     rt.DeviceArray((self.N, self.NF, ho, ho), np.float32)) for _ in range(ROTATE)]
+
+        def plan(self, rt, s):
+            (p,) = self.kernel.plan(*s)
+            return p
+
+        def _direct(self, x, f):
+            ho = self.HW - self.F + 1
+            out = np.zeros((x.shape[0], f.shape[0], ho, ho), np.float64)
+            for p in range(ho):
+                for q in range(ho):
+                    out[:, :, p, q] = np.einsum("nchw,fchw->nf", x[:, :, p:p + self.F, q:q + self.F],
+                                                f, optimize=True)
+            return out
+
+        def check(self, rt, s):
+            got = s[2].to_host()[:2, :8]
+            want = self._direct(self.x[:2].astype(np.float64), self.f[:8].astype(np.float64))
+            k = self.C * self.F * self.F
+            ok = np.allclose(got, want, rtol=1e-4, atol=(k + 2) * 2.0 ** -22)
+            return {"parity": "rtol 1e-4, atol (k+2) * 2^-22 vs fp64 (2 images x 8 filters)"
+                    if ok else "MISMATCH", "ok": bool(ok)}
+
+        def cpu(self):
+            x, f = self.x[:4], self.f
+            t = _best_of(lambda: self._direct(x, f), 1)
+            return t * (self.N / 4), "4 of 64 images (einsum per output position), scaled", 1
+
     table = {
         "c0": C0("c0", "copy 256 MiB int32 (calibration)", "u32", "hbm", 2 * 4 * 64 * 1024 * 1024,
                  "GB/s"),
@@ -301,11 +344,13 @@ def make_workloads(rt, wl):
         "x2": X2("x2", "map-sum kernel: dot fp32 N=16777259", "f32", "hbm", 8 * W.C1_N, "GB/s"),
         "x3": X3("x3", "pairwise distance fp32 8192x8192x128 (sub + fma per term)", "f32", "valu",
                  3 * 8192 * 8192 * 128, "TFLOP/s"),
+        "x4": X4("x4", "implicit-GEMM convolution fp32 64x64x58x58 * 64x64x3x3 (gathered tiles)",
+                 "f32", "valu", 2 * 64 * 64 * 64 * 9 * 56 * 56, "TFLOP/s"),
     }
     if wl == "all":
         keys = ["c1", "c2", "c3", "c4", "c5"]
     elif wl == "extra":
-        keys = ["x1", "x2", "x3"]
+        keys = ["x1", "x2", "x3", "x4"]
     else:
         keys = [wl]
     return [table[k] for k in keys]
@@ -372,7 +417,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="all", choices=["all", "c0", "c1", "c2", "c3", "c4", "c5", "extra", "x1", "x2", "x3"])
+    ap.add_argument("--workload", default="all", choices=["all", "c0", "c1", "c2", "c3", "c4", "c5", "extra", "x1", "x2", "x3", "x4"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy CPU baseline")
     ap.add_argument("--prewarm", type=float, default=PREWARM_SECONDS,
                     help="seconds of untimed device warm-up per workload")

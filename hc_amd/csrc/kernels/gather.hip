@@ -67,10 +67,18 @@ __device__ __forceinline__ Window window_of(const int32_t *rec) {
     w.ext[d] = static_cast<uint32_t>(rec[1 + d]);
   return w;
 }
-template <int T, int R>
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// MFMA = false: R x R outputs per lane, fp32 FMAs on the vector ALUs.
+// MFMA = true (T = 32 or 64, R = 4): every wave owns a 32 x 32 sub-block and
+// accumulates it with v_mfma_f32_32x32x2_f32, two K values per instruction:
+// lane l supplies a[l % 32][l / 32] and b[l / 32][l % 32] and holds
+// c[8*g + 4*(l/32) + e][l % 32] in accumulator element 4*g + e.
+template <int T, int R, bool MFMA>
 __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
   constexpr int kSide = T / R;            // lanes per block edge
   constexpr int kThreads = kSide * kSide;
+  static_assert(!MFMA || (R == 4 && (T == 32 || T == 64)), "MFMA block shapes");
   constexpr int kPitch = T + 4;
   constexpr int kRowsPerPass = kThreads / kStep;
   constexpr int kPasses = T / kRowsPerPass; // gathers per lane, operand and K step
@@ -92,6 +100,11 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
   const int t = threadIdx.x;
   const int tx = t % kSide, ty = t / kSide;
   const int ld_k = t % kStep, ld_r = t / kStep;
+  // MFMA: sub-block of this wave and the lane's place in it
+  const int lane = t % kWave, wave = t / kWave;
+  constexpr int kSubs = T >= 32 ? T / 32 : 1; // 32 x 32 sub-blocks per edge
+  const int sub_m = 32 * (wave / kSubs), sub_n = 32 * (wave % kSubs);
+  const int l_lo = lane % 32, l_hi = lane / 32;
 
   for (uint32_t m0 = 0; m0 < p.tm; m0 += T)
     for (uint32_t n0 = 0; n0 < p.tn; n0 += T) {
@@ -120,6 +133,10 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
 #pragma unroll
         for (int j = 0; j < R; ++j)
           acc[i][j] = 0.0f;
+      f32x16 macc;
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        macc[i] = 0.0f;
 
       float va[kPasses], vb[kPasses];
       auto gather = [&](uint32_t k0) {
@@ -149,41 +166,59 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
         __syncthreads();
         if (k0 + kStep < p.k)
           gather(k0 + kStep);
+        if constexpr (MFMA) {
+#pragma unroll
+          for (int kk = 0; kk < kStep; kk += 2)
+            macc = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                as[kk + l_hi][sub_m + l_lo], bs[kk + l_hi][sub_n + l_lo], macc,
+                0, 0, 0);
+        } else {
 #pragma unroll 8
-        for (int kk = 0; kk < kStep; ++kk) {
-          float av[R], bv[R];
-          if constexpr (R == 4) {
-            const f32x4 x = *reinterpret_cast<const f32x4 *>(&as[kk][R * ty]);
-            const f32x4 y = *reinterpret_cast<const f32x4 *>(&bs[kk][R * tx]);
+          for (int kk = 0; kk < kStep; ++kk) {
+            float av[R], bv[R];
+            if constexpr (R == 4) {
+              const f32x4 x = *reinterpret_cast<const f32x4 *>(&as[kk][R * ty]);
+              const f32x4 y = *reinterpret_cast<const f32x4 *>(&bs[kk][R * tx]);
 #pragma unroll
-            for (int i = 0; i < R; ++i) {
-              av[i] = x[i];
-              bv[i] = y[i];
-            }
-          } else {
+              for (int i = 0; i < R; ++i) {
+                av[i] = x[i];
+                bv[i] = y[i];
+              }
+            } else {
 #pragma unroll
-            for (int i = 0; i < R; ++i) {
-              av[i] = as[kk][R * ty + i];
-              bv[i] = bs[kk][R * tx + i];
+              for (int i = 0; i < R; ++i) {
+                av[i] = as[kk][R * ty + i];
+                bv[i] = bs[kk][R * tx + i];
+              }
             }
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+              for (int j = 0; j < R; ++j)
+                acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
           }
-#pragma unroll
-          for (int i = 0; i < R; ++i)
-#pragma unroll
-            for (int j = 0; j < R; ++j)
-              acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
         }
         __syncthreads();
       }
 
+      if constexpr (MFMA) {
+        const int co = col_o[sub_n + l_lo];
 #pragma unroll
-      for (int i = 0; i < R; ++i) {
-        const int ro = row_o[R * ty + i];
-#pragma unroll
-        for (int j = 0; j < R; ++j) {
-          const int co = col_o[R * tx + j];
+        for (int r = 0; r < 16; ++r) {
+          const int ro = row_o[sub_m + 8 * (r / 4) + 4 * l_hi + r % 4];
           if ((ro | co) >= 0)
-            out[ro + co] = acc[i][j];
+            out[ro + co] = macc[r];
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+          const int ro = row_o[R * ty + i];
+#pragma unroll
+          for (int j = 0; j < R; ++j) {
+            const int co = col_o[R * tx + j];
+            if ((ro | co) >= 0)
+              out[ro + co] = acc[i][j];
+          }
         }
       }
       __syncthreads();
@@ -191,12 +226,14 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
 }
 } // namespace
 
-#define HCAMD_GATHER_GEMM(T, R)                                                \
-  extern "C" __global__ __launch_bounds__((T / R) * (T / R)) void              \
-      hcamd_gather_gemm_f32_t##T(GatherGemmArgs p) {                           \
-    gather_gemm<T, R>(p);                                                      \
+#define HCAMD_GATHER_GEMM(NAME, T, R, MFMA)                                    \
+  extern "C" __global__ __launch_bounds__((T / R) * (T / R)) void NAME(        \
+      GatherGemmArgs p) {                                                      \
+    gather_gemm<T, R, MFMA>(p);                                                \
   }
-HCAMD_GATHER_GEMM(64, 4)
-HCAMD_GATHER_GEMM(32, 4)
-HCAMD_GATHER_GEMM(16, 2)
-HCAMD_GATHER_GEMM(8, 1)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_m64, 64, 4, true)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_m32, 32, 4, true)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t64, 64, 4, false)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t32, 32, 4, false)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t16, 16, 2, false)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t8, 8, 1, false)

@@ -1336,22 +1336,20 @@ int hcamdGatherGemmLaunchF32(OlQueue q, HcamdGatherGemm plan, const float *a,
     dev->report("hcamdGatherGemmLaunchF32: null pointer");
     return 1;
   }
-  // block edge of the kernel: the smallest of 8, 16, 32, 64 that holds the
-  // tile (64 for larger tiles, which are walked block by block)
+  // Block edge of the kernel: the smallest of 8, 16, 32, 64 that holds the
+  // tile (64 for larger tiles, which are walked block by block).  Blocks of 32
+  // and 64 multiply on the matrix cores, the small ones on the vector ALUs.
+  // Variants: 1 m64, 2 m32, 3 t16, 4 t8, 5 t64, 6 t32 (t = vector ALUs).
   const uint32_t side = std::max(plan->tm, plan->tn);
-  const int variant = variantOf("gather");
-  const char *name = "hcamd_gather_gemm_f32_t64";
-  size_t threads = 256;
-  if (variant == 0 ? side <= 8 : variant == 4) {
-    name = "hcamd_gather_gemm_f32_t8";
-    threads = 64;
-  } else if (variant == 0 ? side <= 16 : variant == 3) {
-    name = "hcamd_gather_gemm_f32_t16";
-    threads = 64;
-  } else if (variant == 0 ? side <= 32 : variant == 2) {
-    name = "hcamd_gather_gemm_f32_t32";
-    threads = 64;
-  }
+  int variant = variantOf("gather");
+  if (variant < 1 || variant > 6)
+    variant = side <= 8 ? 4 : side <= 16 ? 3 : side <= 32 ? 2 : 1;
+  static const char *const kNames[] = {
+      "hcamd_gather_gemm_f32_m64", "hcamd_gather_gemm_f32_m32",
+      "hcamd_gather_gemm_f32_t16", "hcamd_gather_gemm_f32_t8",
+      "hcamd_gather_gemm_f32_t64", "hcamd_gather_gemm_f32_t32"};
+  const char *name = kNames[variant - 1];
+  const size_t threads = (variant == 1 || variant == 5) ? 256 : 64;
   Kernel *kern = builtinKernel(dev, "gather", name);
   if (!kern)
     return 1;

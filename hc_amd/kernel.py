@@ -76,6 +76,11 @@ def _binders(func):
     for i, name in enumerate(inspect.signature(func).parameters):
         a = ann.get(name)
         pos = i - 1                      # the first parameter is the group
+        if isinstance(a, str):
+            raise RuntimeError(
+                f"parameter {name!r} of {func.__name__}: the annotation is the string {a!r}; "
+                "kernel bodies need evaluated annotations (define them in a module without "
+                "`from __future__ import annotations`)")
         if a is None or a in (CurrentGroup, CurrentGroup1, CurrentGroup2, CurrentGroup3,
                               CurrentSubGroup, CurrentWorkitem):
             continue

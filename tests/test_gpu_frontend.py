@@ -598,7 +598,7 @@ def test_implicit_gemm_convolution_of_the_reference_examples(n, c, nf, stride, t
     out = rt.to_device(np.zeros((n, nf, ho, wo), np.float32))
     k = _conv_kernel(kernel, create_mapping, stride).parametrize(tiles)
     k(rt.to_device(x), rt.to_device(f), out)
-    assert rt.last_kernel_name().startswith("hcamd_gather_gemm_f32_t")
+    assert rt.last_kernel_name().startswith("hcamd_gather_gemm_f32_")
     want = np.zeros((n, nf, ho, wo), np.float32)
     _conv_kernel(sim_kernel, hcsim.create_mapping, stride).parametrize(tiles)(x, f, want)
     # K = c * hf * wf <= 12 products per output, summed in fp32 in another order
@@ -648,7 +648,7 @@ def test_float32_dot_with_row_major_b():
     b = rng.standard_normal((77, 95)).astype(np.float32)
     out = rt.to_device(np.zeros((130, 95), np.float32))
     make(kernel)(rt.to_device(a), rt.to_device(b), out, (64, 64))
-    assert rt.last_kernel_name().startswith("hcamd_gather_gemm_f32_t")
+    assert rt.last_kernel_name().startswith("hcamd_gather_gemm_f32_")
     want = np.zeros((130, 95), np.float32)
     make(sim_kernel)(a, b, want, (64, 64))
     assert_allclose(out.to_host(), want, rtol=1e-4, atol=79 * 2.0 ** -22)

@@ -352,8 +352,12 @@ def _gather_reference(ops, n_groups, tm, tn, k, a, b, out):
     return out
 
 
+@pytest.mark.parametrize("variant", range(7))
 @pytest.mark.parametrize("case", ["plain", "tails", "blocks", "transposed", "k0"])
-def test_gathered_product_against_the_table_semantics(ctx, case):
+def test_gathered_product_against_the_table_semantics(ctx, case, variant):
+    """variant 0: block shape chosen by tile size; 1-6: every block shape
+    (matrix-core and vector-ALU kernels) on every tile size."""
+    rt.set_variant("gather", variant)
     rng = np.random.default_rng(len(case))
     # a[M, K] x b[K, N] walked by gm x gn groups of tm x tn tiles, written as tables
     M, N, K, tm, tn = {"plain": (64, 64, 32, 64, 64), "tails": (70, 45, 37, 16, 24),
@@ -382,7 +386,7 @@ def test_gathered_product_against_the_table_semantics(ctx, case):
     ops = (a_op, b_op, o_op)
     tables = rt.GatherGemm(ctx, *ops, gm * gn, tm, tn, K)
     out = poisoned(out_shape, np.float32)
-    say("gather", case, M, N, K, tm, tn)
+    say("gather", case, variant, M, N, K, tm, tn)
     rt.plan_gather_gemm_f32(tables, dev(a), dev(b), out).launch(sync=True)
     got = out.to_host()
     want = _gather_reference(ops, gm * gn, tm, tn, K, a, b, np.full(out_shape, np.nan, np.float32))
