@@ -28,12 +28,18 @@
 // one.  The host lays the group records out by window address, and consecutive
 // records go to the same XCD, so that groups that run together share cache lines
 // in that XCD's L2.
+//
+// Fusion (G = 2 or 4): a workgroup takes G consecutive records that read the
+// same b window and treats them as one tile of G * TM rows, row v belonging to
+// record v % G and tile row v / G.  The b panel is then gathered once for G
+// groups, and because neighbouring records are neighbouring windows of a (the
+// next output position of a convolution), the G lanes that gather one tile row
+// for the G groups read adjacent addresses: one cache line serves them all.
 #include "common.h"
 
 using namespace hcamd;
 
 namespace {
-constexpr int kStep = 32;
 constexpr int kXcds = 8;
 
 struct GatherGemmArgs {
@@ -69,12 +75,16 @@ __device__ __forceinline__ Window window_of(const int32_t *rec) {
 }
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
+__device__ __forceinline__ bool inside(u32x4 lo, uint32_t i3, const Window &w) {
+  return lo.y < w.ext[0] && lo.z < w.ext[1] && lo.w < w.ext[2] && i3 < w.ext[3];
+}
+
 // MFMA = false: R x R outputs per lane, fp32 FMAs on the vector ALUs.
 // MFMA = true (T = 32 or 64, R = 4): every wave owns a 32 x 32 sub-block and
 // accumulates it with v_mfma_f32_32x32x2_f32, two K values per instruction:
 // lane l supplies a[l % 32][l / 32] and b[l / 32][l % 32] and holds
 // c[8*g + 4*(l/32) + e][l % 32] in accumulator element 4*g + e.
-template <int T, int R, bool MFMA>
+template <int T, int R, bool MFMA, int G, int kStep>
 __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
   constexpr int kSide = T / R;            // lanes per block edge
   constexpr int kThreads = kSide * kSide;
@@ -83,40 +93,87 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
   constexpr int kRowsPerPass = kThreads / kStep;
   constexpr int kPasses = T / kRowsPerPass; // gathers per lane, operand and K step
   static_assert(kThreads % kStep == 0 && T % kRowsPerPass == 0, "panel split");
+  static_assert(kRowsPerPass % G == 0, "a pass gathers whole sets of G rows");
   __shared__ __attribute__((aligned(16))) float as[kStep][kPitch];
   __shared__ __attribute__((aligned(16))) float bs[kStep][kPitch];
-  __shared__ int row_a[T], col_b[T], row_o[T], col_o[T];
+  // row_a / row_o: absolute element offset of the row's first element, or -1;
+  // col_o: offset inside the window; col_ok: bit g set if the column is inside
+  // the out window of record g
+  __shared__ int row_a[T], col_b[T], row_o[T], col_o[T], col_ok[T];
 
-  const uint32_t g = (blockIdx.x % kXcds) * p.per_xcd + blockIdx.x / kXcds;
-  if (g >= p.n_groups)
+  // n_groups counts sets of G records here
+  const uint32_t set = (blockIdx.x % kXcds) * p.per_xcd + blockIdx.x / kXcds;
+  if (set >= p.n_groups)
     return;
-  const int32_t *rec = p.groups + static_cast<size_t>(g) * 16;
-  const Window wa = window_of(rec), wb = window_of(rec + 5),
-               wo = window_of(rec + 10);
-  const float *a = p.a + wa.base;
+  const int32_t *rec = p.groups + static_cast<size_t>(set) * 16 * G;
+  Window wa[G], wo[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    wa[g] = window_of(rec + 16 * g);
+    wo[g] = window_of(rec + 16 * g + 10);
+  }
+  const Window wb = window_of(rec + 5);
+  const float *a = p.a;
   const float *b = p.b + wb.base;
-  float *out = p.out + wo.base;
+  float *out = p.out;
+  const uint32_t rows = p.tm * G;
 
   const int t = threadIdx.x;
   const int tx = t % kSide, ty = t / kSide;
-  const int ld_k = t % kStep, ld_r = t / kStep;
+  // gathers: G adjacent lanes take the G records of one tile row (or, for b,
+  // G adjacent columns), the next 32 lanes step through K
+  const int ld_g = t % G, ld_k = (t / G) % kStep, ld_r = t / (G * kStep);
+  Window my_wa = wa[0];
+#pragma unroll
+  for (int g = 1; g < G; ++g)
+    if (ld_g == g)
+      my_wa = wa[g];
   // MFMA: sub-block of this wave and the lane's place in it
   const int lane = t % kWave, wave = t / kWave;
   constexpr int kSubs = T >= 32 ? T / 32 : 1; // 32 x 32 sub-blocks per edge
   const int sub_m = 32 * (wave / kSubs), sub_n = 32 * (wave % kSubs);
   const int l_lo = lane % 32, l_hi = lane / 32;
 
-  for (uint32_t m0 = 0; m0 < p.tm; m0 += T)
+  for (uint32_t m0 = 0; m0 < rows; m0 += T)
     for (uint32_t n0 = 0; n0 < p.tn; n0 += T) {
       for (int e = t; e < 2 * T; e += kThreads) {
         if (e < T) {
-          const uint32_t r = m0 + e;
-          row_a[e] = r < p.tm ? resolve(p.a_rows + 8 * (size_t)r, wa) : -1;
-          row_o[e] = r < p.tm ? resolve(p.o_rows + 8 * (size_t)r, wo) : -1;
+          const uint32_t v = m0 + e, i = v / G;
+          const int g = v % G;
+          int oa = -1, oo = -1;
+          if (i < p.tm) {
+            const int32_t *ea = p.a_rows + 8 * (size_t)i;
+            const int32_t *eo = p.o_rows + 8 * (size_t)i;
+            const u32x4 la = *reinterpret_cast<const u32x4 *>(ea);
+            const u32x4 lo = *reinterpret_cast<const u32x4 *>(eo);
+            const uint32_t a3 = ea[4], o3 = eo[4];
+#pragma unroll
+            for (int h = 0; h < G; ++h)
+              if (g == h) {
+                if (inside(la, a3, wa[h]))
+                  oa = (int)(wa[h].base + la.x);
+                if (inside(lo, o3, wo[h]))
+                  oo = (int)(wo[h].base + lo.x);
+              }
+          }
+          row_a[e] = oa;
+          row_o[e] = oo;
         } else {
           const uint32_t c = n0 + e - T;
-          col_b[e - T] = c < p.tn ? resolve(p.b_cols + 8 * (size_t)c, wb) : -1;
-          col_o[e - T] = c < p.tn ? resolve(p.o_cols + 8 * (size_t)c, wo) : -1;
+          int ob = -1, oo = 0, ok = 0;
+          if (c < p.tn) {
+            ob = resolve(p.b_cols + 8 * (size_t)c, wb);
+            const int32_t *eo = p.o_cols + 8 * (size_t)c;
+            const u32x4 lo = *reinterpret_cast<const u32x4 *>(eo);
+            const uint32_t o3 = eo[4];
+            oo = (int)lo.x;
+#pragma unroll
+            for (int h = 0; h < G; ++h)
+              ok |= inside(lo, o3, wo[h]) ? 1 << h : 0;
+          }
+          col_b[e - T] = ob;
+          col_o[e - T] = oo;
+          col_ok[e - T] = ok;
         }
       }
       __syncthreads();
@@ -124,8 +181,9 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
       int ra[kPasses], cb[kPasses];
 #pragma unroll
       for (int i = 0; i < kPasses; ++i) {
-        ra[i] = row_a[ld_r + kRowsPerPass * i];
-        cb[i] = col_b[ld_r + kRowsPerPass * i];
+        const int v = (ld_r + kRowsPerPass / G * i) * G + ld_g;
+        ra[i] = row_a[v];
+        cb[i] = col_b[v];
       }
       float acc[R][R];
 #pragma unroll
@@ -143,7 +201,7 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
         const uint32_t kk = k0 + ld_k;
         int oa = -1, ob = -1;
         if (kk < p.k) {
-          oa = resolve(p.a_cols + 8 * (size_t)kk, wa);
+          oa = resolve(p.a_cols + 8 * (size_t)kk, my_wa);
           ob = resolve(p.b_rows + 8 * (size_t)kk, wb);
         }
 #pragma unroll
@@ -160,8 +218,9 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
       for (uint32_t k0 = 0; k0 < p.k; k0 += kStep) {
 #pragma unroll
         for (int i = 0; i < kPasses; ++i) {
-          as[ld_k][ld_r + kRowsPerPass * i] = va[i];
-          bs[ld_k][ld_r + kRowsPerPass * i] = vb[i];
+          const int v = (ld_r + kRowsPerPass / G * i) * G + ld_g;
+          as[ld_k][v] = va[i];
+          bs[ld_k][v] = vb[i];
         }
         __syncthreads();
         if (k0 + kStep < p.k)
@@ -201,22 +260,25 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
         __syncthreads();
       }
 
+      // block row v belongs to record v % G (m0 is a multiple of G)
       if constexpr (MFMA) {
-        const int co = col_o[sub_n + l_lo];
+        const int co = col_o[sub_n + l_lo], ok = col_ok[sub_n + l_lo];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int ro = row_o[sub_m + 8 * (r / 4) + 4 * l_hi + r % 4];
-          if ((ro | co) >= 0)
+          const int v = sub_m + 8 * (r / 4) + 4 * l_hi + r % 4;
+          const int ro = row_o[v];
+          if (ro >= 0 && ((ok >> (v % G)) & 1))
             out[ro + co] = macc[r];
         }
       } else {
 #pragma unroll
         for (int i = 0; i < R; ++i) {
-          const int ro = row_o[R * ty + i];
+          const int v = R * ty + i;
+          const int ro = row_o[v];
 #pragma unroll
           for (int j = 0; j < R; ++j) {
-            const int co = col_o[R * tx + j];
-            if ((ro | co) >= 0)
+            const int co = col_o[R * tx + j], ok = col_ok[R * tx + j];
+            if (ro >= 0 && ((ok >> (v % G)) & 1))
               out[ro + co] = acc[i][j];
           }
         }
@@ -226,14 +288,19 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
 }
 } // namespace
 
-#define HCAMD_GATHER_GEMM(NAME, T, R, MFMA)                                    \
+#define HCAMD_GATHER_GEMM(NAME, T, R, MFMA, G, KS)                             \
   extern "C" __global__ __launch_bounds__((T / R) * (T / R)) void NAME(        \
       GatherGemmArgs p) {                                                      \
-    gather_gemm<T, R, MFMA>(p);                                                \
+    gather_gemm<T, R, MFMA, G, KS>(p);                                         \
   }
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_m64, 64, 4, true)
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_m32, 32, 4, true)
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t64, 64, 4, false)
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t32, 32, 4, false)
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t16, 16, 2, false)
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t8, 8, 1, false)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_m64_g1, 64, 4, true, 1, 32)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_m64_g2, 64, 4, true, 2, 32)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_m64_g4, 64, 4, true, 4, 32)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_m32_g1, 32, 4, true, 1, 32)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_m32_g2, 32, 4, true, 2, 32)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t16_g1, 16, 2, false, 1, 32)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t16_g2, 16, 2, false, 2, 32)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t8_g1, 8, 1, false, 1, 32)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t8_g2, 8, 1, false, 2, 32)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t64_g1, 64, 4, false, 1, 32)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t32_g1, 32, 4, false, 1, 32)

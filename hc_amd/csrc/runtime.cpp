@@ -263,7 +263,7 @@ std::unordered_map<std::string, int> &variants() {
   static std::unordered_map<std::string, int> v{
       {"add", 0},     {"fma", 0},  {"softmax", 0},
       {"quantize", 0}, {"gemm", 0}, {"copy", 0}, {"map", 0},
-      {"gather", 0}};
+      {"gather", 0}, {"gather_fuse", 0}};
   return v;
 }
 int variantOf(const char *family) { return variants()[family]; }
@@ -1120,6 +1120,7 @@ struct HcamdGatherGemm_ {
   size_t offGroups = 0, offRows[3] = {0, 0, 0}, offCols[3] = {0, 0, 0};
   size_t elems[3] = {0, 0, 0}; // span of each buffer in elements
   uint32_t tm = 0, tn = 0, k = 0, nGroups = 0;
+  uint32_t fuse = 1, nSets = 0; // records per workgroup, number of workgroups
 };
 
 namespace {
@@ -1232,6 +1233,80 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
         }
   }
 
+  // Groups may run in any order.  They are laid out by the address of their
+  // windows, so that workgroups that are resident together, and the run of
+  // groups each XCD receives, touch neighbouring memory: windows that overlap or
+  // share cache lines are then served by one L2 fill.  Sorted by (b, a), runs
+  // of records that read the same b window can be fused, G to a workgroup
+  // (kernels/gather.hip); unfused, the order is (a, b).
+  std::vector<uint32_t> order;
+  std::vector<int64_t> key;
+  try {
+    order.resize(nGroups);
+    key.assign(nGroups * 2, 0);
+  } catch (...) {
+    dev->report("hcamdGatherGemmCreate: out of host memory");
+    return nullptr;
+  }
+  for (size_t g = 0; g < nGroups; ++g) {
+    order[g] = (uint32_t)g;
+    for (int o = 0; o < 2; ++o) {
+      const HcamdGatherOperand &op = *ops[o];
+      for (int d = 0; d < op.ndim; ++d)
+        key[g * 2 + o] += (int64_t)op.starts[g * op.ndim + d] * (int64_t)op.strides[d];
+    }
+  }
+  auto sortBy = [&](int first) {
+    std::stable_sort(order.begin(), order.end(), [&](uint32_t x, uint32_t y) {
+      const int64_t x0 = key[2 * (size_t)x + first], y0 = key[2 * (size_t)y + first];
+      if (x0 != y0)
+        return x0 < y0;
+      return key[2 * (size_t)x + 1 - first] < key[2 * (size_t)y + 1 - first];
+    });
+  };
+  sortBy(1);
+  auto sameB = [&](size_t x, size_t y) {
+    for (int d = 0; d < b->ndim; ++d)
+      if (b->starts[x * b->ndim + d] != b->starts[y * b->ndim + d])
+        return false;
+    return true;
+  };
+  // G = 4 needs the 64-row block; small tiles fuse in pairs.  Fusion must leave
+  // enough workgroups to fill the device.  A run of records with one b window
+  // is padded with empty records (extent 0) to a multiple of G, so that no set
+  // mixes two b windows.
+  const int wanted = variantOf("gather_fuse");
+  const size_t cus = (size_t)std::max(computeUnitsOf(dev), 1);
+  size_t fuse = wanted == 0 ? (tm < 16 ? 2 : 4) : wanted >= 4 ? 4 : wanted >= 2 ? 2 : 1;
+  if (wanted == 0 && nGroups / fuse < 2 * cus)
+    fuse = 1;
+  std::vector<int64_t> slots; // record in each slot, -1 = empty
+  try {
+    slots.reserve(nGroups + fuse);
+    if (fuse == 1) {
+      sortBy(0);
+      for (size_t i = 0; i < nGroups; ++i)
+        slots.push_back(order[i]);
+    } else {
+      for (size_t i = 0; i < nGroups; ++i) {
+        if (i > 0 && !sameB(order[i - 1], order[i]))
+          while (slots.size() % fuse)
+            slots.push_back(-1);
+        slots.push_back(order[i]);
+      }
+      while (slots.size() % fuse)
+        slots.push_back(-1);
+    }
+  } catch (...) {
+    dev->report("hcamdGatherGemmCreate: out of host memory");
+    return nullptr;
+  }
+  const size_t nSets = slots.size() / fuse;
+  if (nSets > 0x7ffffff0ull) {
+    dev->report("hcamdGatherGemmCreate: too many groups");
+    return nullptr;
+  }
+
   auto plan = new (std::nothrow) HcamdGatherGemm_;
   if (!plan)
     return nullptr;
@@ -1240,9 +1315,11 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
   plan->tn = (uint32_t)tn;
   plan->k = (uint32_t)k;
   plan->nGroups = (uint32_t)nGroups;
+  plan->fuse = (uint32_t)fuse;
+  plan->nSets = (uint32_t)nSets;
   size_t total = 0;
   plan->offGroups = total;
-  total += nGroups * kGatherRecord;
+  total += nSets * fuse * kGatherRecord; // records past nGroups stay empty (extent 0)
   for (int o = 0; o < 3; ++o) {
     plan->elems[o] = span[o];
     plan->offRows[o] = total;
@@ -1259,27 +1336,10 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
     delete plan;
     return nullptr;
   }
-  // Groups may run in any order.  They are laid out by the address of their a
-  // window (then b), so that workgroups that are resident together, and the
-  // run of groups each XCD receives, touch neighbouring memory: windows that
-  // overlap or share cache lines are then served by one L2 fill.
-  std::vector<uint32_t> order(nGroups);
-  std::vector<int64_t> key(nGroups * 2, 0);
-  for (size_t g = 0; g < nGroups; ++g) {
-    order[g] = (uint32_t)g;
-    for (int o = 0; o < 2; ++o) {
-      const HcamdGatherOperand &op = *ops[o];
-      for (int d = 0; d < op.ndim; ++d)
-        key[g * 2 + o] += (int64_t)op.starts[g * op.ndim + d] * (int64_t)op.strides[d];
-    }
-  }
-  std::stable_sort(order.begin(), order.end(), [&](uint32_t x, uint32_t y) {
-    if (key[2 * (size_t)x] != key[2 * (size_t)y])
-      return key[2 * (size_t)x] < key[2 * (size_t)y];
-    return key[2 * (size_t)x + 1] < key[2 * (size_t)y + 1];
-  });
-  for (size_t slot = 0; slot < nGroups; ++slot) {
-    const size_t g = order[slot];
+  for (size_t slot = 0; slot < slots.size(); ++slot) {
+    if (slots[slot] < 0)
+      continue; // stays all zero: nothing is inside an empty window
+    const size_t g = (size_t)slots[slot];
     int32_t *rec = host.data() + plan->offGroups + slot * kGatherRecord;
     for (int o = 0; o < 3; ++o) {
       const HcamdGatherOperand &op = *ops[o];
@@ -1337,18 +1397,28 @@ int hcamdGatherGemmLaunchF32(OlQueue q, HcamdGatherGemm plan, const float *a,
     return 1;
   }
   // Block edge of the kernel: the smallest of 8, 16, 32, 64 that holds the
-  // tile (64 for larger tiles, which are walked block by block).  Blocks of 32
-  // and 64 multiply on the matrix cores, the small ones on the vector ALUs.
-  // Variants: 1 m64, 2 m32, 3 t16, 4 t8, 5 t64, 6 t32 (t = vector ALUs).
-  const uint32_t side = std::max(plan->tm, plan->tn);
+  // tile of fuse * tm rows (64 for larger tiles, which are walked block by
+  // block).  Blocks of 32 and 64 multiply on the matrix cores, the small ones
+  // on the vector ALUs.  Variants: 1 m64, 2 m32, 3 t16, 4 t8, 5 t64, 6 t32
+  // (t = vector ALUs); fusing four records needs m64, fusing two any but the
+  // last two.
+  const uint32_t side = std::max(plan->tm * plan->fuse, plan->tn);
   int variant = variantOf("gather");
   if (variant < 1 || variant > 6)
-    variant = side <= 8 ? 4 : side <= 16 ? 3 : side <= 32 ? 2 : 1;
-  static const char *const kNames[] = {
-      "hcamd_gather_gemm_f32_m64", "hcamd_gather_gemm_f32_m32",
-      "hcamd_gather_gemm_f32_t16", "hcamd_gather_gemm_f32_t8",
-      "hcamd_gather_gemm_f32_t64", "hcamd_gather_gemm_f32_t32"};
-  const char *name = kNames[variant - 1];
+    variant = plan->fuse == 4 ? 1
+              : side <= 8     ? 4
+              : side <= 16    ? 3
+              : side <= 32    ? 2
+                              : 1;
+  if ((plan->fuse == 4 && variant != 1) || (plan->fuse == 2 && variant > 4)) {
+    dev->report("hcamdGatherGemmLaunchF32: block shape %d is not built for %u "
+                "fused records", variant, plan->fuse);
+    return 1;
+  }
+  static const char *const kShapes[] = {"m64", "m32", "t16", "t8", "t64", "t32"};
+  char name[64];
+  std::snprintf(name, sizeof(name), "hcamd_gather_gemm_f32_%s_g%u",
+                kShapes[variant - 1], plan->fuse);
   const size_t threads = (variant == 1 || variant == 5) ? 256 : 64;
   Kernel *kern = builtinKernel(dev, "gather", name);
   if (!kern)
@@ -1368,8 +1438,8 @@ int hcamdGatherGemmLaunchF32(OlQueue q, HcamdGatherGemm plan, const float *a,
   args.tm = plan->tm;
   args.tn = plan->tn;
   args.k = plan->k;
-  args.n_groups = plan->nGroups;
-  args.per_xcd = (plan->nGroups + 7) / 8;
+  args.n_groups = plan->nSets;
+  args.per_xcd = (plan->nSets + 7) / 8;
   void *params[] = {&args};
   const size_t grid[3] = {(size_t)args.per_xcd * 8, 1, 1};
   const size_t block[3] = {threads, 1, 1};

@@ -606,7 +606,8 @@ def test_implicit_gemm_convolution_of_the_reference_examples(n, c, nf, stride, t
     assert_allclose(out.to_host(), conv_direct(x, f, stride), rtol=1e-5, atol=1e-5)
 
 
-def test_convolution_at_a_larger_size_with_full_tiles():
+@pytest.mark.parametrize("fuse", [0, 1, 2, 4])
+def test_convolution_at_a_larger_size_with_full_tiles(fuse):
     from hc_amd.kernel import create_mapping
     from test_kernel_frontend import _conv_kernel, conv_direct
     rng = np.random.default_rng(2024)
@@ -618,8 +619,14 @@ def test_convolution_at_a_larger_size_with_full_tiles():
     for stride, tiles in ((1, {sym.TN: 63, sym.TNF: 63, sym.KB: 16}), (2, {sym.TN: 32, sym.TNF: 40})):
         ho = (hw - hf) // stride + 1
         out = rt.to_device(np.full((n, nf, ho, ho), np.nan, np.float32))
-        _conv_kernel(kernel, create_mapping, stride).parametrize(tiles)(
-            rt.to_device(x), rt.to_device(f), out)
+        rt.set_variant("gather_fuse", fuse)
+        try:
+            _conv_kernel(kernel, create_mapping, stride).parametrize(tiles)(
+                rt.to_device(x), rt.to_device(f), out)
+        finally:
+            rt.set_variant("gather_fuse", 0)
+        if fuse:
+            assert rt.last_kernel_name().endswith(f"_g{fuse}")
         got = out.to_host()
         assert not np.isnan(got).any()
         assert_allclose(got, conv_direct(x, f, stride), rtol=1e-4, atol=(c * hf * hf + 2) * 2.0 ** -22)

@@ -34,10 +34,10 @@ def ctx():
 
 @pytest.fixture(autouse=True)
 def default_variants():
-    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy", "map", "gather"):
+    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy", "map", "gather", "gather_fuse"):
         rt.set_variant(fam, 0)
     yield
-    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy", "map", "gather"):
+    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy", "map", "gather", "gather_fuse"):
         rt.set_variant(fam, 0)
 
 
@@ -352,12 +352,17 @@ def _gather_reference(ops, n_groups, tm, tn, k, a, b, out):
     return out
 
 
-@pytest.mark.parametrize("variant", range(7))
+_GATHER_KERNELS = ([(v, 1) for v in range(7)] + [(v, 2) for v in range(5)] + [(0, 4), (1, 4)])
+
+
+@pytest.mark.parametrize("variant,fuse", _GATHER_KERNELS)
 @pytest.mark.parametrize("case", ["plain", "tails", "blocks", "transposed", "k0"])
-def test_gathered_product_against_the_table_semantics(ctx, case, variant):
+def test_gathered_product_against_the_table_semantics(ctx, case, variant, fuse):
     """variant 0: block shape chosen by tile size; 1-6: every block shape
-    (matrix-core and vector-ALU kernels) on every tile size."""
+    (matrix-core and vector-ALU kernels) on every tile size; fuse: records per
+    workgroup (runs of groups that read one b window, padded to a multiple)."""
     rt.set_variant("gather", variant)
+    rt.set_variant("gather_fuse", fuse)
     rng = np.random.default_rng(len(case))
     # a[M, K] x b[K, N] walked by gm x gn groups of tm x tn tiles, written as tables
     M, N, K, tm, tn = {"plain": (64, 64, 32, 64, 64), "tails": (70, 45, 37, 16, 24),
@@ -386,8 +391,9 @@ def test_gathered_product_against_the_table_semantics(ctx, case, variant):
     ops = (a_op, b_op, o_op)
     tables = rt.GatherGemm(ctx, *ops, gm * gn, tm, tn, K)
     out = poisoned(out_shape, np.float32)
-    say("gather", case, variant, M, N, K, tm, tn)
+    say("gather", case, variant, fuse, M, N, K, tm, tn)
     rt.plan_gather_gemm_f32(tables, dev(a), dev(b), out).launch(sync=True)
+    assert rt.last_kernel_name().endswith(f"_g{fuse}")
     got = out.to_host()
     want = _gather_reference(ops, gm * gn, tm, tn, K, a, b, np.full(out_shape, np.nan, np.float32))
     assert not np.isnan(want).any()
@@ -396,7 +402,8 @@ def test_gathered_product_against_the_table_semantics(ctx, case, variant):
     assert_allclose(got, want, rtol=1e-5, atol=(K + 2) * 2.0 ** -22)
 
 
-def test_gathered_product_inactive_elements_and_untouched_memory(ctx):
+@pytest.mark.parametrize("fuse", [1, 2, 4])
+def test_gathered_product_inactive_elements_and_untouched_memory(ctx, fuse):
     """Windows that leave the buffer, negative and too-large indices, a start
     beyond the end: inactive operands count as zero, inactive outputs keep
     their bytes."""
@@ -405,6 +412,7 @@ def test_gathered_product_inactive_elements_and_untouched_memory(ctx):
     b = rng.standard_normal((7, 12)).astype(np.float32)
     out_shape = (3, 12, 11)                                         # [batch, cols, rows + 1]
     tm, tn, k = 6, 8, 9
+    rt.set_variant("gather_fuse", fuse)
     groups = [(g0, g1) for g0 in range(4) for g1 in range(2)]       # batch 3 does not exist
     a_op = _operand(a.shape, [[g0, 5 * g1, 0] for g0, g1 in groups],
                     [[0, r - 1, 0] for r in range(tm)],             # row -1 is inactive
