@@ -15,7 +15,8 @@
 //
 // Tables (built and bounds-checked on the host):
 //   groups[g]  16 ints: {base, extent[4]} for a, b and out (base = element
-//              offset of the window, extent = buffer size - start per dim)
+//              offset of the window, extent = buffer size - start per dim),
+//              then one word of flags
 //   *_rows[r], *_cols[c]  8 ints: {offset, index[4], unused[3]} (offset = sum
 //              of index * stride; dimensions the other coordinate drives hold 0)
 //
@@ -74,6 +75,8 @@ __device__ __forceinline__ Window window_of(const int32_t *rec) {
   return w;
 }
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+// four floats that are only 4-byte aligned
+typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));
 
 __device__ __forceinline__ bool inside(u32x4 lo, uint32_t i3, const Window &w) {
   return lo.y < w.ext[0] && lo.z < w.ext[1] && lo.w < w.ext[2] && i3 < w.ext[3];
@@ -94,12 +97,13 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
   constexpr int kPasses = T / kRowsPerPass; // gathers per lane, operand and K step
   static_assert(kThreads % kStep == 0 && T % kRowsPerPass == 0, "panel split");
   static_assert(kRowsPerPass % G == 0, "a pass gathers whole sets of G rows");
+  constexpr bool kPackA = G == 4 && T == 64 && kThreads == 256 && kStep == 32;
   __shared__ __attribute__((aligned(16))) float as[kStep][kPitch];
   __shared__ __attribute__((aligned(16))) float bs[kStep][kPitch];
   // row_a / row_o: absolute element offset of the row's first element, or -1;
   // col_o: offset inside the window; col_ok: bit g set if the column is inside
   // the out window of record g
-  __shared__ int row_a[T], col_b[T], row_o[T], col_o[T], col_ok[T];
+  __shared__ __attribute__((aligned(16))) int row_a[T], col_b[T], row_o[T], col_o[T], col_ok[T];
 
   // n_groups counts sets of G records here
   const uint32_t set = (blockIdx.x % kXcds) * p.per_xcd + blockIdx.x / kXcds;
@@ -113,6 +117,9 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
     wo[g] = window_of(rec + 16 * g + 10);
   }
   const Window wb = window_of(rec + 5);
+  // set by the host in the first record of a set: the out windows of its
+  // records are one element apart, in record order
+  const bool run_o = G == 4 && (rec[15] & 1);
   const float *a = p.a;
   const float *b = p.b + wb.base;
   float *out = p.out;
@@ -196,20 +203,71 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
       for (int i = 0; i < 16; ++i)
         macc[i] = 0.0f;
 
+      // Four fused records (kPackA): a lane gathers one tile row of a for all
+      // four records at once.  When their windows follow each other element by
+      // element the four values are one 16-byte load; they land next to each
+      // other in the panel either way.
+      [[maybe_unused]] int ra4[2][4];
+      [[maybe_unused]] bool run4[2];
+      [[maybe_unused]] f32x4 va4[2];
+      const int pk = t % kStep, pi = t / kStep; // kPackA: K value and tile row
+      if constexpr (kPackA) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int v0 = 4 * (pi + 8 * j);
+          bool run = true;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            ra4[j][e] = row_a[v0 + e];
+            run = run && ra4[j][e] >= 0 && ra4[j][e] == ra4[j][0] + e;
+          }
+          run4[j] = run;
+        }
+      }
       float va[kPasses], vb[kPasses];
       auto gather = [&](uint32_t k0) {
         const uint32_t kk = k0 + ld_k;
         int oa = -1, ob = -1;
         if (kk < p.k) {
-          oa = resolve(p.a_cols + 8 * (size_t)kk, my_wa);
+          if constexpr (!kPackA)
+            oa = resolve(p.a_cols + 8 * (size_t)kk, my_wa);
           ob = resolve(p.b_rows + 8 * (size_t)kk, wb);
         }
 #pragma unroll
         for (int i = 0; i < kPasses; ++i) {
           // both offsets are non-negative when valid: the sign of the OR says
           // whether either is the -1 marker
-          va[i] = (oa | ra[i]) >= 0 ? a[oa + ra[i]] : 0.0f;
+          if constexpr (!kPackA)
+            va[i] = (oa | ra[i]) >= 0 ? a[oa + ra[i]] : 0.0f;
           vb[i] = (ob | cb[i]) >= 0 ? b[ob + cb[i]] : 0.0f;
+        }
+        if constexpr (kPackA) {
+          const uint32_t ka = k0 + pk;
+          u32x4 ea = {0, ~0u, ~0u, ~0u};           // outside every window
+          uint32_t ea3 = ~0u;
+          if (ka < p.k) {
+            const int32_t *pa = p.a_cols + 8 * (size_t)ka;
+            ea = *reinterpret_cast<const u32x4 *>(pa);
+            ea3 = pa[4];
+          }
+          bool in[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            in[e] = inside(ea, ea3, wa[e]);
+          const int off = (int)ea.x;
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            if (run4[j] && in[0] && in[1] && in[2] && in[3]) {
+              const f32x4u x = *reinterpret_cast<const f32x4u *>(a + off + ra4[j][0]);
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                va4[j][e] = x[e];
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                va4[j][e] = (in[e] && ra4[j][e] >= 0) ? a[off + ra4[j][e]] : 0.0f;
+            }
+          }
         }
       };
 
@@ -219,8 +277,14 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
 #pragma unroll
         for (int i = 0; i < kPasses; ++i) {
           const int v = (ld_r + kRowsPerPass / G * i) * G + ld_g;
-          as[ld_k][v] = va[i];
+          if constexpr (!kPackA)
+            as[ld_k][v] = va[i];
           bs[ld_k][v] = vb[i];
+        }
+        if constexpr (kPackA) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            *reinterpret_cast<f32x4 *>(&as[pk][4 * (pi + 8 * j)]) = va4[j];
         }
         __syncthreads();
         if (k0 + kStep < p.k)
@@ -264,11 +328,31 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
       if constexpr (MFMA) {
         const int co = col_o[sub_n + l_lo], ok = col_ok[sub_n + l_lo];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int v = sub_m + 8 * (r / 4) + 4 * l_hi + r % 4;
-          const int ro = row_o[v];
-          if (ro >= 0 && ((ok >> (v % G)) & 1))
-            out[ro + co] = macc[r];
+        for (int q = 0; q < 4; ++q) {
+          // accumulator elements 4q .. 4q+3 are four consecutive block rows:
+          // with G = 4 one tile row for the four records of the set.  When
+          // their out windows follow each other element by element
+          // (run_o) the four values are one 16-byte store.
+          const int v0 = sub_m + 8 * q + 4 * l_hi;
+          int ro[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            ro[e] = row_o[v0 + e];
+          bool packed = false;
+          if constexpr (G == 4)
+            packed = run_o && ok == 0xF && (ro[0] | ro[1] | ro[2] | ro[3]) >= 0;
+          if (packed) {
+            f32x4u val;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              val[e] = macc[4 * q + e];
+            *reinterpret_cast<f32x4u *>(out + ro[0] + co) = val;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (ro[e] >= 0 && ((ok >> ((v0 + e) % G)) & 1))
+                out[ro[e] + co] = macc[4 * q + e];
+          }
         }
       } else {
 #pragma unroll

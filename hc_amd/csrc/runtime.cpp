@@ -1362,6 +1362,22 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
       w[0] = empty ? 0 : (int32_t)base;
     }
   }
+  // Flag (word 15 of a set's first record): the out windows of the set's records
+  // follow each other element by element and have equal extents along the
+  // dimensions the tile column drives, so that the values one tile element has
+  // for the records of the set are adjacent in memory.
+  if (fuse == 4)
+    for (size_t s0 = 0; s0 < slots.size(); s0 += fuse) {
+      int32_t *rec0 = host.data() + plan->offGroups + s0 * kGatherRecord;
+      bool run = true;
+      for (size_t i = 1; i < fuse && run; ++i) {
+        const int32_t *ri = rec0 + i * kGatherRecord, *rp = ri - kGatherRecord;
+        run = slots[s0 + i] >= 0 && slots[s0 + i - 1] >= 0 && ri[10] == rp[10] + 1;
+        for (int d = 0; d < 4 && run; ++d)
+          run = ri[11 + d] > 0 && rp[11 + d] > 0;
+      }
+      rec0[15] = run ? 1 : 0;
+    }
   for (int o = 0; o < 3; ++o) {
     gatherEntries(*ops[o], ops[o]->rowIndex, rows[o], rowDim[o],
                   host.data() + plan->offRows[o]);
