@@ -16,9 +16,16 @@
 // Tables (built and bounds-checked on the host):
 //   groups[g]  16 ints: {base, extent[4]} for a, b and out (base = element
 //              offset of the window, extent = buffer size - start per dim),
-//              then one word of flags
+//              then one word: bit 0 = the set's out windows are neighbours,
+//              bits 1.. = index of the packed b tile
 //   *_rows[r], *_cols[c]  8 ints: {offset, index[4], unused[3]} (offset = sum
 //              of index * stride; dimensions the other coordinate drives hold 0)
+//
+// The b tile of a group depends only on its b window, and many groups share one
+// (every output position of a convolution reads the same filters).  A first
+// kernel gathers each distinct b tile once into a dense K_pad x TN_pad array
+// (inactive elements and padding are zero); the product kernel then reads its b
+// panels with plain 16-byte loads and spends its gathers on a alone.
 //
 // One workgroup per group; the TM x TN tile is walked in T x T blocks, R x R
 // outputs per lane, K in steps of 32 through LDS panels stored k-major so that
@@ -45,11 +52,20 @@ constexpr int kXcds = 8;
 
 struct GatherGemmArgs {
   const float *a;
-  const float *b;
+  const float *bpack; // b tiles packed by hcamd_gather_pack_b
   float *out;
   const int32_t *groups;
-  const int32_t *a_rows, *a_cols, *b_rows, *b_cols, *o_rows, *o_cols;
+  const int32_t *a_rows, *a_cols, *o_rows, *o_cols;
   uint32_t tm, tn, k, n_groups, per_xcd;
+  uint32_t k_pad, tn_pad; // rows / row length of a packed b tile
+};
+
+struct PackBArgs {
+  const float *b;
+  float *bpack;
+  const int32_t *windows; // [n_windows][8]: base, extent[4]
+  const int32_t *b_rows, *b_cols;
+  uint32_t k, tn, k_pad, tn_pad, n_windows;
 };
 
 struct Window {
@@ -98,12 +114,14 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
   static_assert(kThreads % kStep == 0 && T % kRowsPerPass == 0, "panel split");
   static_assert(kRowsPerPass % G == 0, "a pass gathers whole sets of G rows");
   constexpr bool kPackA = G == 4 && T == 64 && kThreads == 256 && kStep == 32;
+  constexpr int kBLoads = kStep * (T / 4) / kThreads; // 16-byte b loads per lane and K step
+  static_assert(kStep * (T / 4) % kThreads == 0, "b panel split");
   __shared__ __attribute__((aligned(16))) float as[kStep][kPitch];
   __shared__ __attribute__((aligned(16))) float bs[kStep][kPitch];
   // row_a / row_o: absolute element offset of the row's first element, or -1;
   // col_o: offset inside the window; col_ok: bit g set if the column is inside
   // the out window of record g
-  __shared__ __attribute__((aligned(16))) int row_a[T], col_b[T], row_o[T], col_o[T], col_ok[T];
+  __shared__ __attribute__((aligned(16))) int row_a[T], row_o[T], col_o[T], col_ok[T];
 
   // n_groups counts sets of G records here
   const uint32_t set = (blockIdx.x % kXcds) * p.per_xcd + blockIdx.x / kXcds;
@@ -116,12 +134,13 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
     wa[g] = window_of(rec + 16 * g);
     wo[g] = window_of(rec + 16 * g + 10);
   }
-  const Window wb = window_of(rec + 5);
   // set by the host in the first record of a set: the out windows of its
   // records are one element apart, in record order
   const bool run_o = G == 4 && (rec[15] & 1);
   const float *a = p.a;
-  const float *b = p.b + wb.base;
+  // word 15 of the set's first record: bit 0 flags neighbouring out windows,
+  // the rest says which packed b tile the set reads
+  const float *bp = p.bpack + (size_t)((uint32_t)rec[15] >> 1) * p.k_pad * p.tn_pad;
   float *out = p.out;
   const uint32_t rows = p.tm * G;
 
@@ -167,9 +186,8 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
           row_o[e] = oo;
         } else {
           const uint32_t c = n0 + e - T;
-          int ob = -1, oo = 0, ok = 0;
+          int oo = 0, ok = 0;
           if (c < p.tn) {
-            ob = resolve(p.b_cols + 8 * (size_t)c, wb);
             const int32_t *eo = p.o_cols + 8 * (size_t)c;
             const u32x4 lo = *reinterpret_cast<const u32x4 *>(eo);
             const uint32_t o3 = eo[4];
@@ -178,20 +196,16 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
             for (int h = 0; h < G; ++h)
               ok |= inside(lo, o3, wo[h]) ? 1 << h : 0;
           }
-          col_b[e - T] = ob;
           col_o[e - T] = oo;
           col_ok[e - T] = ok;
         }
       }
       __syncthreads();
 
-      int ra[kPasses], cb[kPasses];
+      int ra[kPasses];
 #pragma unroll
-      for (int i = 0; i < kPasses; ++i) {
-        const int v = (ld_r + kRowsPerPass / G * i) * G + ld_g;
-        ra[i] = row_a[v];
-        cb[i] = col_b[v];
-      }
+      for (int i = 0; i < kPasses; ++i)
+        ra[i] = row_a[(ld_r + kRowsPerPass / G * i) * G + ld_g];
       float acc[R][R];
 #pragma unroll
       for (int i = 0; i < R; ++i)
@@ -224,22 +238,25 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
           run4[j] = run;
         }
       }
-      float va[kPasses], vb[kPasses];
+      float va[kPasses];
+      f32x4 vb[kBLoads];
       auto gather = [&](uint32_t k0) {
-        const uint32_t kk = k0 + ld_k;
-        int oa = -1, ob = -1;
-        if (kk < p.k) {
-          if constexpr (!kPackA)
-            oa = resolve(p.a_cols + 8 * (size_t)kk, my_wa);
-          ob = resolve(p.b_rows + 8 * (size_t)kk, wb);
-        }
+        // b: the next kStep rows of the packed tile, columns n0 .. n0 + T
 #pragma unroll
-        for (int i = 0; i < kPasses; ++i) {
+        for (int j = 0; j < kBLoads; ++j) {
+          const int id = t + j * kThreads, kr = id / (T / 4), c = n0 + 4 * (id % (T / 4));
+          vb[j] = c < p.tn_pad
+                      ? *reinterpret_cast<const f32x4 *>(bp + (size_t)(k0 + kr) * p.tn_pad + c)
+                      : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+        if constexpr (!kPackA) {
+          const uint32_t kk = k0 + ld_k;
+          const int oa = kk < p.k ? resolve(p.a_cols + 8 * (size_t)kk, my_wa) : -1;
           // both offsets are non-negative when valid: the sign of the OR says
           // whether either is the -1 marker
-          if constexpr (!kPackA)
+#pragma unroll
+          for (int i = 0; i < kPasses; ++i)
             va[i] = (oa | ra[i]) >= 0 ? a[oa + ra[i]] : 0.0f;
-          vb[i] = (ob | cb[i]) >= 0 ? b[ob + cb[i]] : 0.0f;
         }
         if constexpr (kPackA) {
           const uint32_t ka = k0 + pk;
@@ -275,11 +292,14 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
         gather(0);
       for (uint32_t k0 = 0; k0 < p.k; k0 += kStep) {
 #pragma unroll
-        for (int i = 0; i < kPasses; ++i) {
-          const int v = (ld_r + kRowsPerPass / G * i) * G + ld_g;
-          if constexpr (!kPackA)
-            as[ld_k][v] = va[i];
-          bs[ld_k][v] = vb[i];
+        for (int j = 0; j < kBLoads; ++j) {
+          const int id = t + j * kThreads;
+          *reinterpret_cast<f32x4 *>(&bs[id / (T / 4)][4 * (id % (T / 4))]) = vb[j];
+        }
+        if constexpr (!kPackA) {
+#pragma unroll
+          for (int i = 0; i < kPasses; ++i)
+            as[ld_k][(ld_r + kRowsPerPass / G * i) * G + ld_g] = va[i];
         }
         if constexpr (kPackA) {
 #pragma unroll
@@ -371,6 +391,26 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
     }
 }
 } // namespace
+
+// bpack[w][k][c] = b element (k, c) of window w, zero where inactive or padding
+extern "C" __global__ __launch_bounds__(256) void hcamd_gather_pack_b(PackBArgs p) {
+  const uint32_t w = blockIdx.y;
+  const int32_t *rec = p.windows + 8 * (size_t)w;
+  const Window wb = window_of(rec);
+  const size_t per = (size_t)p.k_pad * p.tn_pad;
+  for (size_t id = (size_t)blockIdx.x * 256 + threadIdx.x; id < per;
+       id += (size_t)gridDim.x * 256) {
+    const uint32_t k = (uint32_t)(id / p.tn_pad), c = (uint32_t)(id % p.tn_pad);
+    float v = 0.0f;
+    if (k < p.k && c < p.tn) {
+      const int ok = resolve(p.b_rows + 8 * (size_t)k, wb);
+      const int oc = resolve(p.b_cols + 8 * (size_t)c, wb);
+      if ((ok | oc) >= 0)
+        v = p.b[wb.base + ok + oc];
+    }
+    p.bpack[(size_t)w * per + id] = v;
+  }
+}
 
 #define HCAMD_GATHER_GEMM(NAME, T, R, MFMA, G, KS)                             \
   extern "C" __global__ __launch_bounds__((T / R) * (T / R)) void NAME(        \

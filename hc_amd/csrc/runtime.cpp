@@ -1121,17 +1121,29 @@ struct HcamdGatherGemm_ {
   size_t elems[3] = {0, 0, 0}; // span of each buffer in elements
   uint32_t tm = 0, tn = 0, k = 0, nGroups = 0;
   uint32_t fuse = 1, nSets = 0; // records per workgroup, number of workgroups
+  // distinct b windows, their table, and the scratch their packed tiles live in
+  uint32_t nWindows = 0, kPad = 0, tnPad = 0;
+  size_t offWindows = 0;
+  float *bpack = nullptr;
 };
 
 namespace {
-// must match GatherGemmArgs in kernels/gather.hip
+// must match GatherGemmArgs and PackBArgs in kernels/gather.hip
 struct GatherGemmArgs {
   const float *a;
-  const float *b;
+  const float *bpack;
   float *out;
   const int32_t *groups;
-  const int32_t *a_rows, *a_cols, *b_rows, *b_cols, *o_rows, *o_cols;
+  const int32_t *a_rows, *a_cols, *o_rows, *o_cols;
   uint32_t tm, tn, k, n_groups, per_xcd;
+  uint32_t k_pad, tn_pad;
+};
+struct PackBArgs {
+  const float *b;
+  float *bpack;
+  const int32_t *windows;
+  const int32_t *b_rows, *b_cols;
+  uint32_t k, tn, k_pad, tn_pad, n_windows;
 };
 
 constexpr int kGatherEntry = 8;   // ints per row / column entry
@@ -1317,9 +1329,43 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
   plan->nGroups = (uint32_t)nGroups;
   plan->fuse = (uint32_t)fuse;
   plan->nSets = (uint32_t)nSets;
+  // distinct b windows in slot order: index per group, representative group
+  std::vector<uint32_t> windowOf, windowRep;
+  try {
+    windowOf.assign(nGroups, 0);
+    std::vector<uint32_t> byB(order); // groups with equal b windows adjacent
+    std::stable_sort(byB.begin(), byB.end(), [&](uint32_t x, uint32_t y) {
+      for (int d = 0; d < b->ndim; ++d) {
+        const int32_t sx = b->starts[(size_t)x * b->ndim + d],
+                      sy = b->starts[(size_t)y * b->ndim + d];
+        if (sx != sy)
+          return sx < sy;
+      }
+      return false;
+    });
+    for (size_t i = 0; i < nGroups; ++i) {
+      if (i == 0 || !sameB(byB[i - 1], byB[i]))
+        windowRep.push_back(byB[i]);
+      windowOf[byB[i]] = (uint32_t)windowRep.size() - 1;
+    }
+  } catch (...) {
+    dev->report("hcamdGatherGemmCreate: out of host memory");
+    delete plan;
+    return nullptr;
+  }
+  plan->nWindows = (uint32_t)windowRep.size();
+  plan->kPad = (uint32_t)(ceilDiv(k, 32) * 32);
+  plan->tnPad = (uint32_t)(ceilDiv(tn, 4) * 4);
+  if (windowRep.size() > 65535) {
+    dev->report("hcamdGatherGemmCreate: more than 65535 distinct b windows");
+    delete plan;
+    return nullptr;
+  }
   size_t total = 0;
   plan->offGroups = total;
   total += nSets * fuse * kGatherRecord; // records past nGroups stay empty (extent 0)
+  plan->offWindows = total;
+  total += windowRep.size() * 8;
   for (int o = 0; o < 3; ++o) {
     plan->elems[o] = span[o];
     plan->offRows[o] = total;
@@ -1361,6 +1407,17 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
       }
       w[0] = empty ? 0 : (int32_t)base;
     }
+    rec[15] = (int32_t)(windowOf[g] << 1); // bit 0 is the flag set below
+  }
+  for (size_t w = 0; w < windowRep.size(); ++w) {
+    // the b window of any record that has it (records hold it at words 5..9)
+    int32_t *dst = host.data() + plan->offWindows + w * 8;
+    for (size_t slot = 0; slot < slots.size(); ++slot)
+      if (slots[slot] >= 0 && windowOf[(size_t)slots[slot]] == w) {
+        std::memcpy(dst, host.data() + plan->offGroups + slot * kGatherRecord + 5,
+                    5 * sizeof(int32_t));
+        break;
+      }
   }
   // Flag (word 15 of a set's first record): the out windows of the set's records
   // follow each other element by element and have equal extents along the
@@ -1376,7 +1433,7 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
         for (int d = 0; d < 4 && run; ++d)
           run = ri[11 + d] > 0 && rp[11 + d] > 0;
       }
-      rec0[15] = run ? 1 : 0;
+      rec0[15] |= run ? 1 : 0;
     }
   for (int o = 0; o < 3; ++o) {
     gatherEntries(*ops[o], ops[o]->rowIndex, rows[o], rowDim[o],
@@ -1389,8 +1446,11 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
     delete plan;
     return nullptr;
   }
+  const size_t packed = std::max<size_t>(
+      (size_t)plan->nWindows * plan->kPad * plan->tnPad, 4);
   if (HIP_CHECK(dev, hipMemcpy(plan->tables, host.data(),
-                               total * sizeof(int32_t), hipMemcpyHostToDevice))) {
+                               total * sizeof(int32_t), hipMemcpyHostToDevice)) ||
+      HIP_CHECK(dev, hipMalloc((void **)&plan->bpack, packed * sizeof(float)))) {
     (void)hipFree(plan->tables);
     delete plan;
     return nullptr;
@@ -1439,16 +1499,38 @@ int hcamdGatherGemmLaunchF32(OlQueue q, HcamdGatherGemm plan, const float *a,
   Kernel *kern = builtinKernel(dev, "gather", name);
   if (!kern)
     return 1;
+  const int32_t *t = plan->tables;
+  if (plan->k > 0) {
+    // every distinct b tile once, then the products
+    Kernel *pack = builtinKernel(dev, "gather", "hcamd_gather_pack_b");
+    if (!pack)
+      return 1;
+    PackBArgs pb;
+    pb.b = b;
+    pb.bpack = plan->bpack;
+    pb.windows = t + plan->offWindows;
+    pb.b_rows = t + plan->offRows[1];
+    pb.b_cols = t + plan->offCols[1];
+    pb.k = plan->k;
+    pb.tn = plan->tn;
+    pb.k_pad = plan->kPad;
+    pb.tn_pad = plan->tnPad;
+    pb.n_windows = plan->nWindows;
+    void *pparams[] = {&pb};
+    const size_t per = (size_t)plan->kPad * plan->tnPad;
+    const size_t pgrid[3] = {std::min<size_t>(ceilDiv(per, 256), 4096),
+                             plan->nWindows, 1};
+    const size_t pblock[3] = {256, 1, 1};
+    if (launch(queue, pack, pgrid, pblock, pparams, 0))
+      return 1;
+  }
   GatherGemmArgs args;
   args.a = a;
-  args.b = b;
+  args.bpack = plan->bpack;
   args.out = out;
-  const int32_t *t = plan->tables;
   args.groups = t + plan->offGroups;
   args.a_rows = t + plan->offRows[0];
   args.a_cols = t + plan->offCols[0];
-  args.b_rows = t + plan->offRows[1];
-  args.b_cols = t + plan->offCols[1];
   args.o_rows = t + plan->offRows[2];
   args.o_cols = t + plan->offCols[2];
   args.tm = plan->tm;
@@ -1456,6 +1538,8 @@ int hcamdGatherGemmLaunchF32(OlQueue q, HcamdGatherGemm plan, const float *a,
   args.k = plan->k;
   args.n_groups = plan->nSets;
   args.per_xcd = (plan->nSets + 7) / 8;
+  args.k_pad = plan->kPad;
+  args.tn_pad = plan->tnPad;
   void *params[] = {&args};
   const size_t grid[3] = {(size_t)args.per_xcd * 8, 1, 1};
   const size_t block[3] = {threads, 1, 1};
@@ -1465,8 +1549,12 @@ int hcamdGatherGemmLaunchF32(OlQueue q, HcamdGatherGemm plan, const float *a,
 void hcamdGatherGemmRelease(HcamdGatherGemm plan) noexcept {
   if (!plan)
     return;
-  if (plan->tables && !plan->device->makeCurrent())
-    (void)hipFree(plan->tables);
+  if (!plan->device->makeCurrent()) {
+    if (plan->tables)
+      (void)hipFree(plan->tables);
+    if (plan->bpack)
+      (void)hipFree(plan->bpack);
+  }
   delete plan;
 }
 
