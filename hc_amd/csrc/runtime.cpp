@@ -1289,9 +1289,13 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
   // mixes two b windows.
   const int wanted = variantOf("gather_fuse");
   const size_t cus = (size_t)std::max(computeUnitsOf(dev), 1);
-  size_t fuse = wanted == 0 ? (tm < 16 ? 2 : 4) : wanted >= 4 ? 4 : wanted >= 2 ? 2 : 1;
-  if (wanted == 0 && nGroups / fuse < 2 * cus)
-    fuse = 1;
+  size_t fuse = wanted >= 4 ? 4 : wanted >= 2 ? 2 : 1;
+  if (wanted == 0) {
+    if (tm >= 16 && nGroups / 4 >= 2 * cus)
+      fuse = 4;
+    else if (nGroups / 2 >= cus)
+      fuse = 2;
+  }
   std::vector<int64_t> slots; // record in each slot, -1 = empty
   try {
     slots.reserve(nGroups + fuse);

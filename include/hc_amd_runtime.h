@@ -341,11 +341,15 @@ int hcamdLaunchPairwiseDistF32(OlQueue q, const float *a, size_t lda,
  * destination (their order is not defined).
  *
  * hcamdGatherGemmCreate checks the description, builds the device tables and
- * returns a plan (NULL after reporting an error); it allocates device memory and
- * synchronises.  hcamdGatherGemmLaunchF32 enqueues one launch of the plan on
- * buffers that have the shapes and strides given at creation; it neither
- * allocates nor synchronises.  All pointers in HcamdGatherOperand are host
- * memory and are not kept. */
+ * returns a plan (NULL after reporting an error); it allocates device memory
+ * (the tables and a scratch array of one packed k x tn tile per distinct b
+ * window, about the size of b) and synchronises.  hcamdGatherGemmLaunchF32
+ * enqueues one launch of the plan (two kernels: the b tiles are packed, then
+ * multiplied) on buffers that have the shapes and strides given at creation;
+ * it neither allocates nor synchronises.  Launches of one plan share its
+ * scratch array: enqueue them on one queue, or wait between them.  Groups run in
+ * an order the plan chooses (by window address).  All pointers in
+ * HcamdGatherOperand are host memory and are not kept. */
 typedef struct HcamdGatherOperand {
   int ndim;               /* 1..4 */
   size_t shape[4];        /* elements per dimension of the whole buffer */
@@ -399,8 +403,9 @@ int hcamdLaunchGemmF16(OlQueue q, const void *a, size_t lda, const void *bt,
 
 /* Chooses between kernel variants of one family by number (0 = default
  * choice by shape).  For tuning and measurement; family names are "add",
- * "fma", "softmax", "quantize", "gemm", "copy", "map", "gather". Returns 1
- * for an unknown family. */
+ * "fma", "softmax", "quantize", "gemm", "copy", "map", "gather" (block
+ * shape), "gather_fuse" (groups per workgroup; read by hcamdGatherGemmCreate).
+ * Returns 1 for an unknown family. */
 int hcamdSetVariant(const char *family, int variant) HCAMD_NOEXCEPT;
 
 /* Name and launch geometry of the kernel the most recent typed launcher
