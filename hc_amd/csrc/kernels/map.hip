@@ -520,6 +520,56 @@ HCAMD_MAP_FLAT(hcamd_map_sum_flat_n1u4, 1, 4, false, true)
 HCAMD_MAP_FLAT(hcamd_map_sum_flat_n4u2h, 4, 2, true, true)
 HCAMD_MAP_FLAT(hcamd_map_sum_flat_n2u4h, 2, 4, true, true)
 
+// The two commonest reductions without the interpreter: sum(x) and sum(x * y)
+// over flat fp32 arrays (a dot product; y = x gives a sum of squares).  One
+// 1024-lane workgroup per CU strides over the data with four independent 16-byte
+// loads per operand in flight and four partial sums per lane; the end is the
+// same as above, one atomic addition per workgroup.
+template <bool DOT>
+__device__ __forceinline__ void reduce_f32(const float *__restrict__ x,
+                                           const float *__restrict__ y,
+                                           float *cell, size_t n) {
+  const size_t n4 = n / 4;
+  const size_t stride = (size_t)gridDim.x * 1024;
+  const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x);
+  const f32x4 *y4 = reinterpret_cast<const f32x4 *>(y);
+  f32x4 part[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+    part[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  size_t c = (size_t)blockIdx.x * 1024 + threadIdx.x;
+  for (; c + 3 * stride < n4; c += 4 * stride) {
+    f32x4 a[4], b[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      a[u] = ldg<true>(x4 + c + u * stride);
+      if constexpr (DOT)
+        b[u] = ldg<true>(y4 + c + u * stride);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      part[u] = DOT ? part[u] + a[u] * b[u] : part[u] + a[u];
+  }
+  for (; c < n4; c += stride) {
+    const f32x4 a = ldg<true>(x4 + c);
+    part[0] = DOT ? part[0] + a * ldg<true>(y4 + c) : part[0] + a;
+  }
+  const f32x4 s = (part[0] + part[1]) + (part[2] + part[3]);
+  float acc = (s.x + s.y) + (s.z + s.w);
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 1023)
+    for (size_t i = n4 * 4; i < n; ++i)
+      acc += DOT ? x[i] * y[i] : x[i];
+  finish_sum<1024>(acc, cell);
+}
+extern "C" __global__ __launch_bounds__(1024) void hcamd_sum_f32(
+    const float *x, float *cell, size_t n) {
+  reduce_f32<false>(x, x, cell, n);
+}
+extern "C" __global__ __launch_bounds__(1024) void hcamd_dot_f32(
+    const float *x, const float *y, float *cell, size_t n) {
+  reduce_f32<true>(x, y, cell, n);
+}
+
 // The map itself: one chunk per lane, one pass, no loop around the interpreter
 // (several chunks per pass, or a persistent grid, measured slower here: the
 // stores of one workgroup already overlap the loads of the next).

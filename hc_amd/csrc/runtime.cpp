@@ -1018,6 +1018,29 @@ int launchMap(OlQueue q, bool sum, const HcamdMapInstr *prog, size_t nInstr,
     // The reduction picks its kernel by operand count and storage type: fewer
     // or narrower operands leave registers for more chunks in flight per lane.
     const bool half = nInputs > 0 && (a.f16_mask & 0xffu) == (1u << nInputs) - 1u;
+    // sum(x) and sum(x * y) over fp32 have kernels of their own (variant 2 of
+    // "map" keeps them on the interpreter)
+    if (sum && (a.f16_mask & 0xffu) == 0 && variantOf("map") != 2) {
+      const bool isSum = nInstr == 1 && prog[0].op == HCAMD_MAP_IN;
+      const bool isDot = nInstr == 2 && prog[0].op == HCAMD_MAP_IN &&
+                         prog[1].op == HCAMD_MAP_MUL_IN;
+      if (isSum || isDot) {
+        const void *x = inputs[prog[0].arg];
+        const void *y = isDot ? inputs[prog[1].arg] : x;
+        size_t n = a.cols;
+        void *rargs[4];
+        int na = 0;
+        rargs[na++] = &x;
+        if (isDot)
+          rargs[na++] = &y;
+        rargs[na++] = &out;
+        rargs[na++] = &n;
+        const size_t groups = std::min(std::max(ceilDiv(n, (size_t)1024 * 16), (size_t)1),
+                                       (size_t)computeUnitsOf(dev));
+        return launch1d(queue, "map", isDot ? "hcamd_dot_f32" : "hcamd_sum_f32",
+                        groups, 1024, rargs);
+      }
+    }
     const char *name = "hcamd_map_flat";
     size_t u = 1;
     if (sum && half) {

@@ -646,6 +646,36 @@ def test_map_sum_flat_strided_and_accumulation(ctx):
         rt.plan_map_sum([I("add")], [da], cell).launch(sync=True)
 
 
+@pytest.mark.parametrize("n", [1, 3, 4, 1023, 4096 * 4, 1_000_003, cf.C1_N])
+def test_sum_and_dot_of_fp32_vectors_have_their_own_kernels(ctx, n):
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal(n).astype(np.float32)
+    y = rng.standard_normal(n).astype(np.float32)
+    dx, dy = dev(x), dev(y)
+    cases = {"hcamd_sum_f32": ([I("in", 0)], [dx], x.astype(np.float64)),
+             "hcamd_dot_f32": ([I("in", 1), I("mul_in", 0)], [dx, dy], (x * y).astype(np.float64)),
+             "hcamd_dot_f32 ": ([I("in", 0), I("mul_in", 0)], [dx], (x * x).astype(np.float64))}
+    for kernel, (prog, ins, terms) in cases.items():
+        bound = 64 * 2.0 ** -24 * np.abs(terms).sum()
+        for variant, name in ((0, kernel.strip()), (2, None)):     # 2: the interpreter
+            rt.set_variant("map", variant)
+            cell = dev(np.array([7.0], np.float32))
+            rt.plan_map_sum(prog, ins, cell).launch(sync=True)
+            if name:
+                assert rt.last_kernel_name() == name
+            else:
+                assert rt.last_kernel_name().startswith("hcamd_map_sum_flat")
+            assert abs(float(cell.to_host()[0]) - 7.0 - terms.sum()) <= bound + 7.0 * 2.0 ** -23
+    # a misaligned operand keeps the general kernel
+    rt.set_variant("map", 0)
+    if n > 8:
+        cell = dev(np.zeros(1, np.float32))
+        rt.plan_map_sum([I("in", 0)], [_view(dx, n - 1, 1)], cell).launch(sync=True)
+        assert rt.last_kernel_name() == "hcamd_map_sum_strided"
+        assert abs(float(cell.to_host()[0]) - x[1:].astype(np.float64).sum()) <= \
+            64 * 2.0 ** -24 * np.abs(x).sum()
+
+
 def test_map_full_benchmark_size_fma(ctx):
     a, b, c = cf.inputs_c2()
     d = rt.DeviceArray(a.shape, np.float16)
