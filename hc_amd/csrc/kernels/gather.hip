@@ -160,8 +160,12 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
   const int sub_m = 32 * (wave / kSubs), sub_n = 32 * (wave % kSubs);
   const int l_lo = lane % 32, l_hi = lane / 32;
 
-  for (uint32_t m0 = 0; m0 < rows; m0 += T)
-    for (uint32_t n0 = 0; n0 < p.tn; n0 += T) {
+  // the T x T blocks of the tile are spread over blockIdx.y
+  const uint32_t n_blocks = (p.tn + T - 1) / T;
+  const uint32_t blocks = ((rows + T - 1) / T) * n_blocks;
+  for (uint32_t block = blockIdx.y; block < blocks; block += gridDim.y) {
+    const uint32_t m0 = block / n_blocks * T, n0 = block % n_blocks * T;
+    {
       for (int e = t; e < 2 * T; e += kThreads) {
         if (e < T) {
           const uint32_t v = m0 + e, i = v / G;
@@ -389,6 +393,7 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
       }
       __syncthreads();
     }
+  }
 }
 } // namespace
 

@@ -1314,7 +1314,7 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
   const size_t cus = (size_t)std::max(computeUnitsOf(dev), 1);
   size_t fuse = wanted >= 4 ? 4 : wanted >= 2 ? 2 : 1;
   if (wanted == 0) {
-    if (tm >= 16 && nGroups / 4 >= 2 * cus)
+    if (tm >= 16 && nGroups / 4 * ceilDiv(4 * tm, (size_t)64) * ceilDiv(tn, (size_t)64) >= cus)
       fuse = 4;
     else if (nGroups / 2 >= cus)
       fuse = 2;
@@ -1568,7 +1568,15 @@ int hcamdGatherGemmLaunchF32(OlQueue q, HcamdGatherGemm plan, const float *a,
   args.k_pad = plan->kPad;
   args.tn_pad = plan->tnPad;
   void *params[] = {&args};
-  const size_t grid[3] = {(size_t)args.per_xcd * 8, 1, 1};
+  // y: the blocks of a tile (the kernel strides over them if there are more)
+  const size_t edge = (variant == 1 || variant == 5)   ? 64
+                      : (variant == 2 || variant == 6) ? 32
+                      : variant == 3                   ? 16
+                                                       : 8;
+  const size_t tileBlocks = ceilDiv((size_t)plan->tm * plan->fuse, edge) *
+                            ceilDiv((size_t)plan->tn, edge);
+  const size_t grid[3] = {(size_t)args.per_xcd * 8,
+                          std::min<size_t>(tileBlocks, 65535), 1};
   const size_t block[3] = {threads, 1, 1};
   return launch(queue, kern, grid, block, params, 0);
 }
