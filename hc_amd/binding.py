@@ -528,6 +528,63 @@ def _group_starts(view, n_groups):
     return out
 
 
+_MERGED_EDGE = 64         # merged tiles grow up to the kernel's largest block
+
+
+def _merge_groups(tables, grid, tm, tn):
+    """Joins neighbouring groups into larger tiles where that changes nothing
+    but the tiling: along a group axis on which the b window stays put and the a
+    and out windows advance by a fixed step in dimensions their tile rows drive,
+    m groups are one group with m times the rows (row tables repeated with the
+    step added).  The same with a and b exchanged grows the columns.  A user's
+    8 x 8 tiles thus reach the kernel as 64 x 64 ones.  Exactness: a row that was
+    active in its own group is active in the merged one and the other way round,
+    because window start plus index is unchanged; that needs indices >= 0 (a
+    negative index could become a valid element of the neighbouring window), so
+    tables with negative entries are left alone.  tables: [(shape, strides,
+    starts, rows, cols)] for a, b, out.  Returns (tables, grid, tm, tn)."""
+    import numpy as np
+    grid = list(grid)
+    ops = [list(t) for t in tables]
+    # (operands whose tile rows / columns grow, table slot, the operand that must not move)
+    plans = (("rows", (0, 2), 3, 1), ("cols", (1, 2), 4, 0))
+    for axis in range(len(grid)):
+        for kind, moving, slot, fixed in plans:
+            extent = tm if kind == "rows" else tn
+            if grid[axis] < 2 or extent >= _MERGED_EDGE:
+                continue
+            m = max((d for d in range(1, grid[axis] + 1)
+                     if grid[axis] % d == 0 and d * extent <= _MERGED_EDGE), default=1)
+            if m < 2:
+                continue
+            starts = [np.asarray(o[2]).reshape(*grid, -1) for o in ops]
+            if np.diff(starts[fixed], axis=axis).any():
+                continue
+            deltas, ok = {}, True
+            for o in moving:
+                d = np.diff(starts[o], axis=axis).reshape(-1, starts[o].shape[-1])
+                step = d[0]
+                other = ops[o][4] if slot == 3 else ops[o][3]     # the other coordinate's table
+                ok = ok and not (d != step).any() and (step >= 0).all() \
+                    and not (other[:, step != 0] != 0).any() \
+                    and (ops[o][slot] >= 0).all()
+                deltas[o] = step
+            if not ok:
+                continue
+            for o in moving:
+                table = ops[o][slot]
+                ops[o][slot] = np.concatenate([table + j * deltas[o] for j in range(m)], axis=0)
+            for o in range(3):
+                ops[o][2] = np.take(starts[o], np.arange(0, grid[axis], m), axis=axis) \
+                    .reshape(-1, starts[o].shape[-1])
+            grid[axis] //= m
+            if kind == "rows":
+                tm *= m
+            else:
+                tn *= m
+    return [tuple(o) for o in ops], tuple(grid), tm, tn
+
+
 def match_gather_gemm(dst_view, value, n_groups, out_func=None, plain=True):
     """store(sum_k dot(A chunk, B chunk)) where the chunks are slices of one A
     tile and one B tile, any of them loaded or stored through a mapping."""
@@ -600,6 +657,7 @@ def match_gather_gemm(dst_view, value, n_groups, out_func=None, plain=True):
     if len(np.unique(dest)) != dest.size:
         raise NoNativeKernel(f"{names[2]}: the store mapping sends two tile elements to one "
                              "destination")
+    tables, n_groups, tm, tn = _merge_groups(tables, n_groups, tm, tn)
     total = 1
     for n in n_groups:
         total *= n

@@ -576,7 +576,12 @@ def test_convolution_example_binds_to_the_gathered_product(ctx, monkeypatch, n, 
     t = TablesOnly.last
     assert p.args == (ctx.queue, t.handle, dx.ptr, df.ptr, do.ptr)
     tn, tnf = tiles.get(sym.TN, 8), tiles.get(sym.TNF, 8)
-    assert (t.tm, t.tn, t.k) == (tn, tnf, c * hf * wf)
+
+    def merged(extent, count):
+        # neighbouring groups are joined while the tile stays within 64 and the count divides
+        return extent * max(d for d in range(1, count + 1) if count % d == 0 and d * extent <= 64)
+    assert (t.tm, t.tn, t.k) == (merged(tn, cdiv(n, tn)), merged(tnf, cdiv(nf, tnf)), c * hf * wf)
+    assert t.n_groups == cdiv(n, t.tm) * cdiv(nf, t.tn) * ho * wo if stride < 3 else True
     got = np.full((n, nf, ho, wo), np.nan, np.float32)
     t.run(x, f, got)
 
@@ -610,7 +615,8 @@ def test_plain_float32_dot_binds_to_the_gathered_product(ctx, monkeypatch):
                     FakeDev((13, 10), "float32"), (8, 4), ctx=ctx)
     assert p.fn is rt.hcamdGatherGemmLaunchF32
     t = TablesOnly.last
-    assert (t.n_groups, t.tm, t.tn, t.k) == (2 * 3, 8, 4, 24)
+    # 2 x 3 groups of 8 x 4 are joined into one 16 x 12 tile
+    assert (t.n_groups, t.tm, t.tn, t.k) == (1, 16, 12, 24)
     got = np.full((13, 10), np.nan, np.float32)
     t.run(a, b, got)
     np.testing.assert_allclose(got, a.astype(np.float64) @ b.astype(np.float64), rtol=1e-5, atol=1e-5)
@@ -660,3 +666,32 @@ def test_offsets_with_division_are_for_mapped_accesses_only(ctx):
 
     with pytest.raises(NoNativeKernel, match="mapped loads and stores only"):
         body.plan(FakeDev((8, 8), "float32"), FakeDev((8, 8), "float32"), ctx=ctx)
+
+
+def test_groups_are_joined_only_when_that_is_exact(ctx, monkeypatch):
+    """Row index -1 of a tile is inactive in its own window but would be the last
+    row of the window before it: such tables keep the user's tiling."""
+    from hc_amd.kernel import create_mapping
+    monkeypatch.setattr(rt, "GatherGemm", TablesOnly)
+    M, N, K = sym.M, sym.N, sym.K
+    shifted = create_mapping(lambda i, j: (i - 1, j))
+
+    @kernel(work_shape=(M, N), group_shape=(4, 4))
+    def body(gr: CurrentGroup, a: Buffer[M, K, DT], b: Buffer[K, N, DT], out: Buffer[M, N, DT]):
+        m0, n0 = gr.work_offset
+        av = gr.load(a[m0:, :], shape=(4, K), mapping=shifted)
+        bv = gr.load(b[:, n0:], shape=(K, 4))
+        gr.store(out[m0:, n0:], np.dot(av, bv))
+
+    rng = np.random.default_rng(3)
+    a = rng.standard_normal((8, 6)).astype(np.float32)
+    b = rng.standard_normal((6, 8)).astype(np.float32)
+    body.plan(FakeDev((8, 6), "float32"), FakeDev((6, 8), "float32"), FakeDev((8, 8), "float32"),
+              ctx=ctx)
+    t = TablesOnly.last
+    assert (t.tm, t.tn, t.n_groups) == (4, 8, 2)      # columns joined, rows not
+    got = np.full((8, 8), np.nan, np.float32)
+    t.run(a, b, got)
+    want = np.zeros((8, 8))
+    want[1:4], want[5:8] = a[0:3] @ b, a[4:7] @ b     # row 0 of each group reads nothing
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
