@@ -35,6 +35,7 @@ _FAMILIES = {
     "hcamdLaunchQuantizeF16I8": ("quantize", (0, 2, 3, 4, 7, 8, 9, 10, 11)),
     "hcamdLaunchGemmBF16": ("gemm", (1, 2, 3, 4, 5, 7, 8, 9, 10, 11, 12)),
     "hcamdGatherGemmLaunchF32": ("gather", (1, 2, 3, 4, 5, 6)),
+    "hcamdGatherGemmLaunch": ("gather", (1, 2, 3, 4)),
 }
 
 

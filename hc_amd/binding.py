@@ -637,8 +637,11 @@ def match_gather_gemm(dst_view, value, n_groups, out_func=None, plain=True):
     o_op = _Operand(dst_view, out_func, (tm, tn))
     ops = (a_op, b_op, o_op)
     names = tuple(o.view.base.name for o in ops)
-    if any(o.view.base.dtype_name != "float32" for o in ops):
-        raise NoNativeKernel("products of gathered tiles are bound for float32 buffers "
+    elem = ops[0].view.base.dtype_name
+    if elem not in ("float32", "float16", "bfloat16") or \
+            any(o.view.base.dtype_name != elem for o in ops):
+        raise NoNativeKernel("products of gathered tiles are bound for three float32, float16 or "
+                             f"bfloat16 buffers of one type "
                              f"({', '.join(o.view.base.dtype_name for o in ops)} given)")
     dims = ((tm, k_total), (k_total, tn), (tm, tn))
     tables = []
@@ -668,7 +671,7 @@ def match_gather_gemm(dst_view, value, n_groups, out_func=None, plain=True):
         g = cache.get(id(ctx))
         if g is None:
             g = cache[id(ctx)] = rt.GatherGemm(ctx, *tables, total, tm, tn, k_total)
-        return [rt.plan_gather_gemm_f32(g, *[_Arr(mem[i], ctx) for i in idx])]
+        return [rt.plan_gather_gemm(g, *[_Arr(mem[i], ctx) for i in idx], elem)]
     return make
 
 

@@ -1,4 +1,5 @@
-// Matrix product of gathered tiles, fp32:
+// Matrix product of gathered tiles (fp32, fp16 or bf16 storage; products and sums
+// in fp32, one rounding on the way out):
 //
 //   out[map_o(i, j)] = sum_k a[map_a(i, k)] * b[map_b(k, j)]      per group
 //
@@ -51,9 +52,9 @@ namespace {
 constexpr int kXcds = 8;
 
 struct GatherGemmArgs {
-  const float *a;
-  const float *bpack; // b tiles packed by hcamd_gather_pack_b
-  float *out;
+  const void *a;
+  const float *bpack; // b tiles packed by hcamd_gather_pack_b (always fp32)
+  void *out;
   const int32_t *groups;
   const int32_t *a_rows, *a_cols, *o_rows, *o_cols;
   uint32_t tm, tn, k, n_groups, per_xcd;
@@ -61,7 +62,7 @@ struct GatherGemmArgs {
 };
 
 struct PackBArgs {
-  const float *b;
+  const void *b;
   float *bpack;
   const int32_t *windows; // [n_windows][8]: base, extent[4]
   const int32_t *b_rows, *b_cols;
@@ -91,8 +92,6 @@ __device__ __forceinline__ Window window_of(const int32_t *rec) {
   return w;
 }
 typedef float f32x16 __attribute__((ext_vector_type(16)));
-// four floats that are only 4-byte aligned
-typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));
 
 __device__ __forceinline__ bool inside(u32x4 lo, uint32_t i3, const Window &w) {
   return lo.y < w.ext[0] && lo.z < w.ext[1] && lo.w < w.ext[2] && i3 < w.ext[3];
@@ -103,8 +102,10 @@ __device__ __forceinline__ bool inside(u32x4 lo, uint32_t i3, const Window &w) {
 // accumulates it with v_mfma_f32_32x32x2_f32, two K values per instruction:
 // lane l supplies a[l % 32][l / 32] and b[l / 32][l % 32] and holds
 // c[8*g + 4*(l/32) + e][l % 32] in accumulator element 4*g + e.
-template <int T, int R, bool MFMA, int G, int kStep>
+template <class E, int T, int R, bool MFMA, int G, int kStep>
 __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
+  // four elements that are only aligned like one
+  typedef E ex4u __attribute__((ext_vector_type(4), aligned(sizeof(E))));
   constexpr int kSide = T / R;            // lanes per block edge
   constexpr int kThreads = kSide * kSide;
   static_assert(!MFMA || (R == 4 && (T == 32 || T == 64)), "MFMA block shapes");
@@ -137,11 +138,11 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
   // set by the host in the first record of a set: the out windows of its
   // records are one element apart, in record order
   const bool run_o = G == 4 && (rec[15] & 1);
-  const float *a = p.a;
+  const E *a = static_cast<const E *>(p.a);
   // word 15 of the set's first record: bit 0 flags neighbouring out windows,
   // the rest says which packed b tile the set reads
   const float *bp = p.bpack + (size_t)((uint32_t)rec[15] >> 1) * p.k_pad * p.tn_pad;
-  float *out = p.out;
+  E *out = static_cast<E *>(p.out);
   const uint32_t rows = p.tm * G;
 
   const int t = threadIdx.x;
@@ -260,7 +261,7 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
           // whether either is the -1 marker
 #pragma unroll
           for (int i = 0; i < kPasses; ++i)
-            va[i] = (oa | ra[i]) >= 0 ? a[oa + ra[i]] : 0.0f;
+            va[i] = (oa | ra[i]) >= 0 ? (float)a[oa + ra[i]] : 0.0f;
         }
         if constexpr (kPackA) {
           const uint32_t ka = k0 + pk;
@@ -279,14 +280,14 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
             if (run4[j] && in[0] && in[1] && in[2] && in[3]) {
-              const f32x4u x = *reinterpret_cast<const f32x4u *>(a + off + ra4[j][0]);
+              const ex4u x = *reinterpret_cast<const ex4u *>(a + off + ra4[j][0]);
 #pragma unroll
               for (int e = 0; e < 4; ++e)
-                va4[j][e] = x[e];
+                va4[j][e] = (float)x[e];
             } else {
 #pragma unroll
               for (int e = 0; e < 4; ++e)
-                va4[j][e] = (in[e] && ra4[j][e] >= 0) ? a[off + ra4[j][e]] : 0.0f;
+                va4[j][e] = (in[e] && ra4[j][e] >= 0) ? (float)a[off + ra4[j][e]] : 0.0f;
             }
           }
         }
@@ -366,16 +367,16 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
           if constexpr (G == 4)
             packed = run_o && ok == 0xF && (ro[0] | ro[1] | ro[2] | ro[3]) >= 0;
           if (packed) {
-            f32x4u val;
+            ex4u val;
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-              val[e] = macc[4 * q + e];
-            *reinterpret_cast<f32x4u *>(out + ro[0] + co) = val;
+              val[e] = (E)macc[4 * q + e];
+            *reinterpret_cast<ex4u *>(out + ro[0] + co) = val;
           } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
               if (ro[e] >= 0 && ((ok >> ((v0 + e) % G)) & 1))
-                out[ro[e] + co] = macc[4 * q + e];
+                out[ro[e] + co] = (E)macc[4 * q + e];
           }
         }
       } else {
@@ -387,7 +388,7 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
           for (int j = 0; j < R; ++j) {
             const int co = col_o[R * tx + j], ok = col_ok[R * tx + j];
             if (ro >= 0 && ((ok >> (v % G)) & 1))
-              out[ro + co] = acc[i][j];
+              out[ro + co] = (E)acc[i][j];
           }
         }
       }
@@ -398,10 +399,11 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
 } // namespace
 
 // bpack[w][k][c] = b element (k, c) of window w, zero where inactive or padding
-extern "C" __global__ __launch_bounds__(256) void hcamd_gather_pack_b(PackBArgs p) {
+template <class E> __device__ __forceinline__ void pack_b(const PackBArgs &p) {
   const uint32_t w = blockIdx.y;
   const int32_t *rec = p.windows + 8 * (size_t)w;
   const Window wb = window_of(rec);
+  const E *b = static_cast<const E *>(p.b);
   const size_t per = (size_t)p.k_pad * p.tn_pad;
   for (size_t id = (size_t)blockIdx.x * 256 + threadIdx.x; id < per;
        id += (size_t)gridDim.x * 256) {
@@ -411,25 +413,40 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_gather_pack_b(PackBArgs 
       const int ok = resolve(p.b_rows + 8 * (size_t)k, wb);
       const int oc = resolve(p.b_cols + 8 * (size_t)c, wb);
       if ((ok | oc) >= 0)
-        v = p.b[wb.base + ok + oc];
+        v = (float)b[wb.base + ok + oc];
     }
     p.bpack[(size_t)w * per + id] = v;
   }
 }
+extern "C" __global__ __launch_bounds__(256) void hcamd_gather_pack_b_f32(PackBArgs p) {
+  pack_b<float>(p);
+}
+extern "C" __global__ __launch_bounds__(256) void hcamd_gather_pack_b_f16(PackBArgs p) {
+  pack_b<_Float16>(p);
+}
+extern "C" __global__ __launch_bounds__(256) void hcamd_gather_pack_b_bf16(PackBArgs p) {
+  pack_b<__bf16>(p);
+}
 
-#define HCAMD_GATHER_GEMM(NAME, T, R, MFMA, G, KS)                             \
+#define HCAMD_GATHER_GEMM(NAME, E, T, R, MFMA, G, KS)                          \
   extern "C" __global__ __launch_bounds__((T / R) * (T / R)) void NAME(        \
       GatherGemmArgs p) {                                                      \
-    gather_gemm<T, R, MFMA, G, KS>(p);                                         \
+    gather_gemm<E, T, R, MFMA, G, KS>(p);                                      \
   }
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_m64_g1, 64, 4, true, 1, 32)
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_m64_g2, 64, 4, true, 2, 32)
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_m64_g4, 64, 4, true, 4, 32)
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_m32_g1, 32, 4, true, 1, 32)
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_m32_g2, 32, 4, true, 2, 32)
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t16_g1, 16, 2, false, 1, 32)
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t16_g2, 16, 2, false, 2, 32)
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t8_g1, 8, 1, false, 1, 32)
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t8_g2, 8, 1, false, 2, 32)
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t64_g1, 64, 4, false, 1, 32)
-HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t32_g1, 32, 4, false, 1, 32)
+// block shape (m = matrix cores, t = vector ALUs) and records per workgroup
+#define HCAMD_GATHER_SET(TY, E)                                                \
+  HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_m64_g1, E, 64, 4, true, 1, 32)    \
+  HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_m64_g2, E, 64, 4, true, 2, 32)    \
+  HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_m64_g4, E, 64, 4, true, 4, 32)    \
+  HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_m32_g1, E, 32, 4, true, 1, 32)    \
+  HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_m32_g2, E, 32, 4, true, 2, 32)    \
+  HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_t16_g1, E, 16, 2, false, 1, 32)   \
+  HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_t16_g2, E, 16, 2, false, 2, 32)   \
+  HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_t8_g1, E, 8, 1, false, 1, 32)     \
+  HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_t8_g2, E, 8, 1, false, 2, 32)
+HCAMD_GATHER_SET(f32, float)
+HCAMD_GATHER_SET(f16, _Float16)
+HCAMD_GATHER_SET(bf16, __bf16)
+// the 64- and 32-wide blocks on the vector ALUs, kept for comparison (fp32 only)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t64_g1, float, 64, 4, false, 1, 32)
+HCAMD_GATHER_GEMM(hcamd_gather_gemm_f32_t32_g1, float, 32, 4, false, 1, 32)

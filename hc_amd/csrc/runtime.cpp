@@ -1153,16 +1153,16 @@ struct HcamdGatherGemm_ {
 namespace {
 // must match GatherGemmArgs and PackBArgs in kernels/gather.hip
 struct GatherGemmArgs {
-  const float *a;
+  const void *a;
   const float *bpack;
-  float *out;
+  void *out;
   const int32_t *groups;
   const int32_t *a_rows, *a_cols, *o_rows, *o_cols;
   uint32_t tm, tn, k, n_groups, per_xcd;
   uint32_t k_pad, tn_pad;
 };
 struct PackBArgs {
-  const float *b;
+  const void *b;
   float *bpack;
   const int32_t *windows;
   const int32_t *b_rows, *b_cols;
@@ -1487,16 +1487,27 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
 
 int hcamdGatherGemmLaunchF32(OlQueue q, HcamdGatherGemm plan, const float *a,
                              const float *b, float *out) noexcept {
+  return hcamdGatherGemmLaunch(q, plan, HCAMD_F32, a, b, out);
+}
+
+int hcamdGatherGemmLaunch(OlQueue q, HcamdGatherGemm plan, int elemType,
+                          const void *a, const void *b, void *out) noexcept {
   auto *queue = static_cast<Queue *>(q);
   if (!queue)
     return 1;
   Device *dev = queue->device;
+  if (elemType != HCAMD_F32 && elemType != HCAMD_F16 && elemType != HCAMD_BF16) {
+    dev->report("hcamdGatherGemmLaunch: unknown element type %d", elemType);
+    return 1;
+  }
+  static const char *const kTypes[] = {"f32", "f16", "bf16"};
+  const char *ty = kTypes[elemType];
   if (!plan || plan->device != dev) {
-    dev->report("hcamdGatherGemmLaunchF32: the plan belongs to another device");
+    dev->report("hcamdGatherGemmLaunch: the plan belongs to another device");
     return 1;
   }
   if (!a || !b || !out) {
-    dev->report("hcamdGatherGemmLaunchF32: null pointer");
+    dev->report("hcamdGatherGemmLaunch: null pointer");
     return 1;
   }
   // Block edge of the kernel: the smallest of 8, 16, 32, 64 that holds the
@@ -1513,14 +1524,15 @@ int hcamdGatherGemmLaunchF32(OlQueue q, HcamdGatherGemm plan, const float *a,
               : side <= 16    ? 3
               : side <= 32    ? 2
                               : 1;
-  if ((plan->fuse == 4 && variant != 1) || (plan->fuse == 2 && variant > 4)) {
-    dev->report("hcamdGatherGemmLaunchF32: block shape %d is not built for %u "
-                "fused records", variant, plan->fuse);
+  if ((plan->fuse == 4 && variant != 1) || (plan->fuse == 2 && variant > 4) ||
+      (elemType != HCAMD_F32 && variant > 4)) {
+    dev->report("hcamdGatherGemmLaunch: block shape %d is not built for %u "
+                "fused records of type %s", variant, plan->fuse, ty);
     return 1;
   }
   static const char *const kShapes[] = {"m64", "m32", "t16", "t8", "t64", "t32"};
   char name[64];
-  std::snprintf(name, sizeof(name), "hcamd_gather_gemm_f32_%s_g%u",
+  std::snprintf(name, sizeof(name), "hcamd_gather_gemm_%s_%s_g%u", ty,
                 kShapes[variant - 1], plan->fuse);
   const size_t threads = (variant == 1 || variant == 5) ? 256 : 64;
   Kernel *kern = builtinKernel(dev, "gather", name);
@@ -1529,7 +1541,9 @@ int hcamdGatherGemmLaunchF32(OlQueue q, HcamdGatherGemm plan, const float *a,
   const int32_t *t = plan->tables;
   if (plan->k > 0) {
     // every distinct b tile once, then the products
-    Kernel *pack = builtinKernel(dev, "gather", "hcamd_gather_pack_b");
+    char packName[40];
+    std::snprintf(packName, sizeof(packName), "hcamd_gather_pack_b_%s", ty);
+    Kernel *pack = builtinKernel(dev, "gather", packName);
     if (!pack)
       return 1;
     PackBArgs pb;

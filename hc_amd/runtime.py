@@ -119,6 +119,7 @@ hcamdGatherGemmCreate = _sig(_rt, "hcamdGatherGemmCreate", _vp, _vp, C.POINTER(G
                              C.POINTER(GatherOperand), C.POINTER(GatherOperand), _sz, _sz,
                              _sz, _sz)
 hcamdGatherGemmLaunchF32 = _sig(_rt, "hcamdGatherGemmLaunchF32", _int, _vp, _vp, _vp, _vp, _vp)
+hcamdGatherGemmLaunch = _sig(_rt, "hcamdGatherGemmLaunch", _int, _vp, _vp, _int, _vp, _vp, _vp)
 hcamdGatherGemmRelease = _sig(_rt, "hcamdGatherGemmRelease", None, _vp)
 hcamdConvertPyArray = _sig(_py, "hcamdConvertPyArray", _int, C.py_object, _int, _vp,
                            _sz_p, C.c_char_p, _sz)
@@ -408,7 +409,7 @@ MAP_OPS = {"in": 1, "const": 2, "add": 3, "sub": 4, "mul": 5, "div": 6, "max": 7
            "mul_in": 29, "div_in": 30, "max_in": 31, "min_in": 32, "rsub_in": 33,
            "rdiv_in": 34}
 MAP_MAX_INPUTS, MAP_MAX_INSTRS, MAP_STACK_DEPTH = 4, 32, 4
-F32, F16 = 0, 1
+F32, F16, BF16 = 0, 1, 2
 
 
 def plan_map(program, inputs, out, types=None) -> Plan:
@@ -536,17 +537,26 @@ class GatherGemm:
             self.handle = None
 
 
-def plan_gather_gemm_f32(tables: GatherGemm, a, b, out) -> Plan:
-    """One launch of a GatherGemm on fp32 buffers of the shapes it was built for."""
+def plan_gather_gemm(tables: GatherGemm, a, b, out, dtype: str = "float32") -> Plan:
+    """One launch of a GatherGemm on buffers of the shapes it was built for;
+    dtype ('float32', 'float16' or 'bfloat16') is the storage type of all three."""
     ctx = _ctx_of(a, b, out)
     ma, mb, mo = as_memref(a), as_memref(b), as_memref(out)
+    code, size = {"float32": (F32, 4), "float16": (F16, 2), "bfloat16": (BF16, 2)}[dtype]
     for m, n, lay in zip((ma, mb, mo), ("a", "b", "out"), tables.layouts):
-        _expect(m, 4, n)
+        _expect(m, size, n)
         if (tuple(m.shape), tuple(m.strides)) != lay:
-            raise HcRuntimeError(f"gather_gemm_f32: {n} has shape {m.shape} strides {m.strides}, "
+            raise HcRuntimeError(f"gather_gemm: {n} has shape {m.shape} strides {m.strides}, "
                                  f"the tables were built for {lay[0]} {lay[1]}")
-    return Plan(ctx, hcamdGatherGemmLaunchF32, (ctx.queue, tables.handle, ma.ptr, mb.ptr, mo.ptr),
-                "hcamdGatherGemmLaunchF32", (tables, a, b, out))
+    if code == F32:
+        return Plan(ctx, hcamdGatherGemmLaunchF32, (ctx.queue, tables.handle, ma.ptr, mb.ptr, mo.ptr),
+                    "hcamdGatherGemmLaunchF32", (tables, a, b, out))
+    return Plan(ctx, hcamdGatherGemmLaunch, (ctx.queue, tables.handle, code, ma.ptr, mb.ptr, mo.ptr),
+                "hcamdGatherGemmLaunch", (tables, a, b, out))
+
+
+def plan_gather_gemm_f32(tables: GatherGemm, a, b, out) -> Plan:
+    return plan_gather_gemm(tables, a, b, out, "float32")
 
 
 def plan_softmax_f32(x, y) -> Plan:

@@ -249,7 +249,7 @@ int hcamdLaunchFmaF16(OlQueue q, const void *a, size_t lda, const void *b,
  * nearest even.  Operands are fp32 or fp16, each with its own leading
  * dimension in elements.  The program is validated on the host; a malformed
  * one is an error, not a launch. */
-enum HcamdElemType { HCAMD_F32 = 0, HCAMD_F16 = 1 };
+enum HcamdElemType { HCAMD_F32 = 0, HCAMD_F16 = 1, HCAMD_BF16 = 2 };
 enum HcamdMapOp {
   HCAMD_MAP_END = 0,
   HCAMD_MAP_IN = 1,    /* push operand `arg` */
@@ -366,6 +366,12 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
                                       size_t k) HCAMD_NOEXCEPT;
 int hcamdGatherGemmLaunchF32(OlQueue q, HcamdGatherGemm plan, const float *a,
                              const float *b, float *out) HCAMD_NOEXCEPT;
+/* The same for buffers of another storage type (HcamdElemType; a, b and out
+ * alike): elements are widened to fp32 when read, products and sums are fp32,
+ * the result is rounded to nearest even when stored. */
+int hcamdGatherGemmLaunch(OlQueue q, HcamdGatherGemm plan, int elemType,
+                          const void *a, const void *b,
+                          void *out) HCAMD_NOEXCEPT;
 void hcamdGatherGemmRelease(HcamdGatherGemm plan) HCAMD_NOEXCEPT;
 
 /* Row softmax, fp32: y[r,:] = exp(x[r,:]-max(x[r,:])) / sum(exp(...)).

@@ -660,3 +660,30 @@ def test_float32_dot_with_row_major_b():
     make(sim_kernel)(a, b, want, (64, 64))
     assert_allclose(out.to_host(), want, rtol=1e-4, atol=79 * 2.0 ** -22)
     assert_allclose(out.to_host(), a.astype(np.float64) @ b, rtol=1e-4, atol=79 * 2.0 ** -22)
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_convolution_on_16_bit_arrays(dtype):
+    from hc_amd.kernel import create_mapping
+    from test_kernel_frontend import _conv_kernel, conv_direct
+    rng = np.random.default_rng(99)
+    n, c, hw, nf, hf = 20, 5, 9, 12, 3
+    x32 = rng.standard_normal((n, c, hw, hw)).astype(np.float32)
+    f32 = rng.standard_normal((nf, c, hf, hf)).astype(np.float32)
+    ho = hw - hf + 1
+    if dtype == "float16":
+        x, f = x32.astype(np.float16), f32.astype(np.float16)
+        dx, df = rt.to_device(x), rt.to_device(f)
+        out = rt.to_device(np.zeros((n, nf, ho, ho), np.float16))
+        xv, fv = x.astype(np.float32), f.astype(np.float32)
+    else:
+        xb, fb = cf.f32_to_bf16_bits(x32), cf.f32_to_bf16_bits(f32)
+        dx, df = rt.to_device(xb, bf16=True), rt.to_device(fb, bf16=True)
+        out = rt.to_device(np.zeros((n, nf, ho, ho), np.uint16), bf16=True)
+        xv, fv = cf.bf16_bits_to_f32(xb), cf.bf16_bits_to_f32(fb)
+    _conv_kernel(kernel, create_mapping, 1)(dx, df, out)
+    assert "_f16_" in rt.last_kernel_name() or "_bf16_" in rt.last_kernel_name()
+    raw = out.to_host()
+    got = raw.astype(np.float32) if dtype == "float16" else cf.bf16_bits_to_f32(raw)
+    eps = 2.0 ** -11 if dtype == "float16" else 2.0 ** -8
+    assert_allclose(got, conv_direct(xv, fv, 1), rtol=1.01 * eps, atol=(c * hf * hf + 2) * 2.0 ** -22)

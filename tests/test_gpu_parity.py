@@ -434,6 +434,47 @@ def test_gathered_product_inactive_elements_and_untouched_memory(ctx, fuse):
     assert_allclose(got[written], want[written], rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("fuse", [1, 2, 4])
+def test_gathered_product_on_16_bit_storage(ctx, dtype, fuse):
+    """Elements are widened to fp32, multiplied and summed in fp32 and rounded
+    once when stored: the result is the rounding of an fp32-accurate product."""
+    rng = np.random.default_rng(fuse)
+    M, N, K, tm, tn = 150, 140, 70, 40, 70
+    gm, gn = -(-M // tm), -(-N // tn)
+
+    def store(x):                                   # device array + the values it holds
+        if dtype == "float16":
+            h = x.astype(np.float16)
+            return dev(h), h.astype(np.float32)
+        bits = cf.f32_to_bf16_bits(x)
+        return dev(bits, bf16=True), cf.bf16_bits_to_f32(bits)
+
+    da, a = store(rng.standard_normal((M, K)).astype(np.float32))
+    db, b = store(rng.standard_normal((K, N)).astype(np.float32))
+    groups = [(gi, gj) for gi in range(gm) for gj in range(gn)]
+    ops = (_operand(a.shape, [[gi * tm, 0] for gi, gj in groups], [[r, 0] for r in range(tm)],
+                    [[0, c] for c in range(K)]),
+           _operand(b.shape, [[0, gj * tn] for gi, gj in groups], [[r, 0] for r in range(K)],
+                    [[0, c] for c in range(tn)]),
+           _operand((M, N), [[gi * tm, gj * tn] for gi, gj in groups], [[r, 0] for r in range(tm)],
+                    [[0, c] for c in range(tn)]))
+    rt.set_variant("gather_fuse", fuse)
+    tables = rt.GatherGemm(ctx, *ops, len(groups), tm, tn, K)
+    out = rt.DeviceArray((M, N), np.float16 if dtype == "float16" else np.uint16, ctx,
+                         dtype == "bfloat16").fill_bytes32(POISON32)
+    rt.plan_gather_gemm(tables, da, db, out, dtype).launch(sync=True)
+    assert rt.last_kernel_name().startswith(f"hcamd_gather_gemm_{'f16' if dtype == 'float16' else 'bf16'}_")
+    raw = out.to_host()
+    got = raw.astype(np.float32) if dtype == "float16" else cf.bf16_bits_to_f32(raw)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    # one rounding to 11 (fp16) or 8 (bf16) significant bits on top of the fp32 sum
+    eps = 2.0 ** -11 if dtype == "float16" else 2.0 ** -8
+    assert_allclose(got, want, rtol=1.01 * eps, atol=(K + 2) * 2.0 ** -22)
+    with pytest.raises(rt.HcRuntimeError, match="element size"):
+        rt.plan_gather_gemm(tables, da, db, out, "float32")
+
+
 def test_gathered_product_rejects_bad_descriptions(ctx):
     ok = _operand((8, 8), [[0, 0]], [[r, 0] for r in range(4)], [[0, c] for c in range(4)])
     both = _operand((8, 8), [[0, 0]], [[r, r] for r in range(4)], [[0, c] for c in range(4)])

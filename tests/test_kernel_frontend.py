@@ -648,8 +648,11 @@ def test_mappings_that_no_table_can_express_are_refused(ctx, monkeypatch):
         make(lambda i, j: (i + j, j))
     with pytest.raises(NoNativeKernel, match="one destination"):
         make(lambda i, j: (i, j), store_func=lambda i, j: (i // 2, j))
-    with pytest.raises(NoNativeKernel, match="float32"):
-        make(lambda i, j: (i, j), dtype="float16", store_func=lambda i, j: (i, j))
+    with pytest.raises(NoNativeKernel, match="float32, float16 or bfloat16"):
+        make(lambda i, j: (i, j), dtype="int32", store_func=lambda i, j: (i, j))
+    for dtype, code in (("float16", rt.F16), ("bfloat16", rt.BF16)):
+        (p,) = make(lambda i, j: (i, j), dtype=dtype, store_func=lambda i, j: (i, j))
+        assert p.fn is rt.hcamdGatherGemmLaunch and p.args[2] == code
     with pytest.raises(NoNativeKernel, match="must return 2 indices"):
         make(lambda i, j: (i, j, 0))
     with pytest.raises(NoNativeKernel, match="cannot be evaluated"):
