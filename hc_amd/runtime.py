@@ -532,9 +532,12 @@ class GatherGemm:
         self.handle = h
 
     def __del__(self):
-        if getattr(self, "handle", None):
-            hcamdGatherGemmRelease(self.handle)
-            self.handle = None
+        handle, self.handle = getattr(self, "handle", None), None
+        if handle:
+            try:
+                hcamdGatherGemmRelease(handle)
+            except Exception:       # interpreter shutdown: the library may be gone
+                pass
 
 
 def plan_gather_gemm(tables: GatherGemm, a, b, out, dtype: str = "float32") -> Plan:
