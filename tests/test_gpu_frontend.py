@@ -687,3 +687,26 @@ def test_convolution_on_16_bit_arrays(dtype):
     got = raw.astype(np.float32) if dtype == "float16" else cf.bf16_bits_to_f32(raw)
     eps = 2.0 ** -11 if dtype == "float16" else 2.0 ** -8
     assert_allclose(got, conv_direct(xv, fv, 1), rtol=1.01 * eps, atol=(c * hf * hf + 2) * 2.0 ** -22)
+
+
+def test_autotune_of_the_convolution_example():
+    """The tunables of python/hckernel/tests/test_examples.py:216-218 (tile sizes
+    and K block) and the block shapes of the kernel it binds to are timed; the
+    tuned kernel computes the same convolution."""
+    from hc_amd.kernel import autotune, create_mapping
+    from test_kernel_frontend import _conv_kernel, conv_direct
+    rng = np.random.default_rng(5)
+    n, c, hw, nf, hf = 24, 4, 10, 16, 3
+    x = rng.standard_normal((n, c, hw, hw)).astype(np.float32)
+    f = rng.standard_normal((nf, c, hf, hf)).astype(np.float32)
+    ho = hw - hf + 1
+    dx, df = rt.to_device(x), rt.to_device(f)
+    out = rt.to_device(np.zeros((n, nf, ho, ho), np.float32))
+    conv = _conv_kernel(kernel, create_mapping, 1)
+    tp = autotune(conv, dx, df, out, max_trials=6, iters=3, warmup=1)
+    assert 1 <= tp[sym.TN] < 64 and 1 <= tp[sym.TNF] < 64 and 8 <= tp[sym.KB] < 128
+    assert set(tp.variants) <= {"gather"}
+    out2 = rt.to_device(np.full((n, nf, ho, ho), np.nan, np.float32))
+    conv.parametrize(tp)(dx, df, out2)
+    rt.set_variant("gather", 0)
+    assert_allclose(out2.to_host(), conv_direct(x, f, 1), rtol=1e-4, atol=(c * hf * hf + 2) * 2.0 ** -22)
