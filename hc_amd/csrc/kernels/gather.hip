@@ -45,6 +45,7 @@
 // next output position of a convolution), the G lanes that gather one tile row
 // for the G groups read adjacent addresses: one cache line serves them all.
 #include "common.h"
+#include <type_traits>
 
 using namespace hcamd;
 
@@ -117,8 +118,21 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
   constexpr bool kPackA = G == 4 && T == 64 && kThreads == 256 && kStep == 32;
   constexpr int kBLoads = kStep * (T / 4) / kThreads; // 16-byte b loads per lane and K step
   static_assert(kStep * (T / 4) % kThreads == 0, "b panel split");
-  __shared__ __attribute__((aligned(16))) float as[kStep][kPitch];
-  __shared__ __attribute__((aligned(16))) float bs[kStep][kPitch];
+  // 16-bit storage on the matrix cores: the panels hold the stored type, row by
+  // row (32 K values + 8 of padding, so that the 16-byte operand reads of eight
+  // consecutive rows cover all banks), and feed v_mfma_f32_32x32x16 directly;
+  // lane l supplies K values 16*s + 8*(l/32) .. +8 of row l % 32 in sub-step s.
+  constexpr bool kLow = MFMA && sizeof(E) == 2;
+  static_assert(!kLow || kStep == 32, "16-bit panels are 32 K values wide");
+  constexpr int kLowPitch = kStep + 8;
+  typedef E ex8 __attribute__((ext_vector_type(8)));
+  __shared__ __attribute__((aligned(16))) float as[kLow ? 1 : kStep][kLow ? 4 : kPitch];
+  __shared__ __attribute__((aligned(16))) float bs[kLow ? 1 : kStep][kLow ? 4 : kPitch];
+  __shared__ __attribute__((aligned(16))) E as16[kLow ? T : 1][kLow ? kLowPitch : 8];
+  __shared__ __attribute__((aligned(16))) E bs16[kLow ? T : 1][kLow ? kLowPitch : 8];
+  // 16-byte b loads per lane and K step: rows of the packed tile are K-major
+  // [k][column] fp32, or, for kLow, column-major [column][k] in the stored type
+  constexpr int kBLoads16 = kLow ? T * (kStep / 8) / kThreads : 1;
   // row_a / row_o: absolute element offset of the row's first element, or -1;
   // col_o: offset inside the window; col_ok: bit g set if the column is inside
   // the out window of record g
@@ -245,14 +259,31 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
       }
       float va[kPasses];
       f32x4 vb[kBLoads];
+      [[maybe_unused]] ex8 vb16[kBLoads16];
       auto gather = [&](uint32_t k0) {
         // b: the next kStep rows of the packed tile, columns n0 .. n0 + T
+        if constexpr (kLow) {
+          const E *bp16 = reinterpret_cast<const E *>(p.bpack) +
+                          (size_t)((uint32_t)rec[15] >> 1) * p.k_pad * p.tn_pad;
 #pragma unroll
-        for (int j = 0; j < kBLoads; ++j) {
-          const int id = t + j * kThreads, kr = id / (T / 4), c = n0 + 4 * (id % (T / 4));
-          vb[j] = c < p.tn_pad
-                      ? *reinterpret_cast<const f32x4 *>(bp + (size_t)(k0 + kr) * p.tn_pad + c)
-                      : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+          for (int j = 0; j < kBLoads16; ++j) {
+            const int id = t + j * kThreads, c = n0 + id / (kStep / 8), part = id % (kStep / 8);
+            ex8 v;
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              v[e] = (E)0.0f;
+            if (c < p.tn_pad)
+              v = *reinterpret_cast<const ex8 *>(bp16 + (size_t)c * p.k_pad + k0 + 8 * part);
+            vb16[j] = v;
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < kBLoads; ++j) {
+            const int id = t + j * kThreads, kr = id / (T / 4), c = n0 + 4 * (id % (T / 4));
+            vb[j] = c < p.tn_pad
+                        ? *reinterpret_cast<const f32x4 *>(bp + (size_t)(k0 + kr) * p.tn_pad + c)
+                        : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+          }
         }
         if constexpr (!kPackA) {
           const uint32_t kk = k0 + ld_k;
@@ -296,25 +327,55 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
       if (p.k > 0)
         gather(0);
       for (uint32_t k0 = 0; k0 < p.k; k0 += kStep) {
+        if constexpr (kLow) {
+          // the values went through fp32 unchanged: narrowing them again is exact
 #pragma unroll
-        for (int j = 0; j < kBLoads; ++j) {
-          const int id = t + j * kThreads;
-          *reinterpret_cast<f32x4 *>(&bs[id / (T / 4)][4 * (id % (T / 4))]) = vb[j];
-        }
-        if constexpr (!kPackA) {
+          for (int j = 0; j < kBLoads16; ++j) {
+            const int id = t + j * kThreads;
+            *reinterpret_cast<ex8 *>(&bs16[id / (kStep / 8)][8 * (id % (kStep / 8))]) = vb16[j];
+          }
+          if constexpr (!kPackA) {
 #pragma unroll
-          for (int i = 0; i < kPasses; ++i)
-            as[ld_k][(ld_r + kRowsPerPass / G * i) * G + ld_g] = va[i];
-        }
-        if constexpr (kPackA) {
+            for (int i = 0; i < kPasses; ++i)
+              as16[(ld_r + kRowsPerPass / G * i) * G + ld_g][ld_k] = (E)va[i];
+          } else {
 #pragma unroll
-          for (int j = 0; j < 2; ++j)
-            *reinterpret_cast<f32x4 *>(&as[pk][4 * (pi + 8 * j)]) = va4[j];
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                as16[4 * (pi + 8 * j) + e][pk] = (E)va4[j][e];
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < kBLoads; ++j) {
+            const int id = t + j * kThreads;
+            *reinterpret_cast<f32x4 *>(&bs[id / (T / 4)][4 * (id % (T / 4))]) = vb[j];
+          }
+          if constexpr (!kPackA) {
+#pragma unroll
+            for (int i = 0; i < kPasses; ++i)
+              as[ld_k][(ld_r + kRowsPerPass / G * i) * G + ld_g] = va[i];
+          }
+          if constexpr (kPackA) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+              *reinterpret_cast<f32x4 *>(&as[pk][4 * (pi + 8 * j)]) = va4[j];
+          }
         }
         __syncthreads();
         if (k0 + kStep < p.k)
           gather(k0 + kStep);
-        if constexpr (MFMA) {
+        if constexpr (kLow) {
+#pragma unroll
+          for (int sub = 0; sub < kStep / 16; ++sub) {
+            const ex8 x = *reinterpret_cast<const ex8 *>(&as16[sub_m + l_lo][16 * sub + 8 * l_hi]);
+            const ex8 y = *reinterpret_cast<const ex8 *>(&bs16[sub_n + l_lo][16 * sub + 8 * l_hi]);
+            if constexpr (std::is_same<E, __bf16>::value)
+              macc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x, y, macc, 0, 0, 0);
+            else
+              macc = __builtin_amdgcn_mfma_f32_32x32x16_f16(x, y, macc, 0, 0, 0);
+          }
+        } else if constexpr (MFMA) {
 #pragma unroll
           for (int kk = 0; kk < kStep; kk += 2)
             macc = __builtin_amdgcn_mfma_f32_32x32x2f32(
@@ -417,6 +478,32 @@ template <class E> __device__ __forceinline__ void pack_b(const PackBArgs &p) {
     }
     p.bpack[(size_t)w * per + id] = v;
   }
+}
+// the same in the stored 16-bit type and column by column: bpack[w][c][k]
+template <class E> __device__ __forceinline__ void pack_b_low(const PackBArgs &p) {
+  const uint32_t w = blockIdx.y;
+  const Window wb = window_of(p.windows + 8 * (size_t)w);
+  const E *b = static_cast<const E *>(p.b);
+  E *dst = reinterpret_cast<E *>(p.bpack);
+  const size_t per = (size_t)p.k_pad * p.tn_pad;
+  for (size_t id = (size_t)blockIdx.x * 256 + threadIdx.x; id < per;
+       id += (size_t)gridDim.x * 256) {
+    const uint32_t c = (uint32_t)(id / p.k_pad), k = (uint32_t)(id % p.k_pad);
+    E v = (E)0.0f;
+    if (k < p.k && c < p.tn) {
+      const int ok = resolve(p.b_rows + 8 * (size_t)k, wb);
+      const int oc = resolve(p.b_cols + 8 * (size_t)c, wb);
+      if ((ok | oc) >= 0)
+        v = b[wb.base + ok + oc];
+    }
+    dst[(size_t)w * per + id] = v;
+  }
+}
+extern "C" __global__ __launch_bounds__(256) void hcamd_gather_pack_b_low_f16(PackBArgs p) {
+  pack_b_low<_Float16>(p);
+}
+extern "C" __global__ __launch_bounds__(256) void hcamd_gather_pack_b_low_bf16(PackBArgs p) {
+  pack_b_low<__bf16>(p);
 }
 extern "C" __global__ __launch_bounds__(256) void hcamd_gather_pack_b_f32(PackBArgs p) {
   pack_b<float>(p);

@@ -1541,8 +1541,12 @@ int hcamdGatherGemmLaunch(OlQueue q, HcamdGatherGemm plan, int elemType,
   const int32_t *t = plan->tables;
   if (plan->k > 0) {
     // every distinct b tile once, then the products
-    char packName[40];
-    std::snprintf(packName, sizeof(packName), "hcamd_gather_pack_b_%s", ty);
+    // 16-bit storage on the matrix-core blocks reads its b tiles in the
+    // stored type, column by column
+    const bool low = elemType != HCAMD_F32 && (variant == 1 || variant == 2);
+    char packName[48];
+    std::snprintf(packName, sizeof(packName), "hcamd_gather_pack_b_%s%s",
+                  low ? "low_" : "", ty);
     Kernel *pack = builtinKernel(dev, "gather", packName);
     if (!pack)
       return 1;
