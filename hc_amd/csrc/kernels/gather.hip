@@ -18,7 +18,8 @@
 //   groups[g]  16 ints: {base, extent[4]} for a, b and out (base = element
 //              offset of the window, extent = buffer size - start per dim),
 //              then one word: bit 0 = the set's out windows are neighbours,
-//              bits 1.. = index of the packed b tile
+//              bit 1 = its a windows are neighbours and every a element is
+//              active, bits 2.. = index of the packed b tile
 //   *_rows[r], *_cols[c]  8 ints: {offset, index[4], unused[3]} (offset = sum
 //              of index * stride; dimensions the other coordinate drives hold 0)
 //
@@ -38,7 +39,7 @@
 // records go to the same XCD, so that groups that run together share cache lines
 // in that XCD's L2.
 //
-// Fusion (G = 2 or 4): a workgroup takes G consecutive records that read the
+// Fusion (G = 2, 4 or 16): a workgroup takes G consecutive records that read the
 // same b window and treats them as one tile of G * TM rows, row v belonging to
 // record v % G and tile row v / G.  The b panel is then gathered once for G
 // groups, and because neighbouring records are neighbouring windows of a (the
@@ -114,8 +115,9 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
   constexpr int kRowsPerPass = kThreads / kStep;
   constexpr int kPasses = T / kRowsPerPass; // gathers per lane, operand and K step
   static_assert(kThreads % kStep == 0 && T % kRowsPerPass == 0, "panel split");
-  static_assert(kRowsPerPass % G == 0, "a pass gathers whole sets of G rows");
-  constexpr bool kPackA = G == 4 && T == 64 && kThreads == 256 && kStep == 32;
+  constexpr bool kPackA = G >= 4 && G % 4 == 0 && 8 % (G / 4) == 0 && T == 64 &&
+                          kThreads == 256 && kStep == 32;
+  static_assert(kPackA || kRowsPerPass % G == 0, "a pass gathers whole sets of G rows");
   constexpr int kBLoads = kStep * (T / 4) / kThreads; // 16-byte b loads per lane and K step
   static_assert(kStep * (T / 4) % kThreads == 0, "b panel split");
   // 16-bit storage on the matrix cores: the panels hold the stored type, row by
@@ -143,19 +145,18 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
   if (set >= p.n_groups)
     return;
   const int32_t *rec = p.groups + static_cast<size_t>(set) * 16 * G;
-  Window wa[G], wo[G];
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    wa[g] = window_of(rec + 16 * g);
-    wo[g] = window_of(rec + 16 * g + 10);
-  }
+  // the a / out window of record g of the set (the records are read where
+  // they are needed: a few cached loads per block)
+  auto win_a = [&](int g) { return window_of(rec + 16 * g); };
+  auto win_o = [&](int g) { return window_of(rec + 16 * g + 10); };
   // set by the host in the first record of a set: the out windows of its
   // records are one element apart, in record order
-  const bool run_o = G == 4 && (rec[15] & 1);
+  const bool run_o = kPackA && (rec[15] & 1);
   const E *a = static_cast<const E *>(p.a);
   // word 15 of the set's first record: bit 0 flags neighbouring out windows,
-  // the rest says which packed b tile the set reads
-  const float *bp = p.bpack + (size_t)((uint32_t)rec[15] >> 1) * p.k_pad * p.tn_pad;
+  // bit 1 a windows that are neighbours and fully active, the rest says which
+  // packed b tile the set reads
+  const float *bp = p.bpack + (size_t)((uint32_t)rec[15] >> 2) * p.k_pad * p.tn_pad;
   E *out = static_cast<E *>(p.out);
   const uint32_t rows = p.tm * G;
 
@@ -164,11 +165,7 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
   // gathers: G adjacent lanes take the G records of one tile row (or, for b,
   // G adjacent columns), the next 32 lanes step through K
   const int ld_g = t % G, ld_k = (t / G) % kStep, ld_r = t / (G * kStep);
-  Window my_wa = wa[0];
-#pragma unroll
-  for (int g = 1; g < G; ++g)
-    if (ld_g == g)
-      my_wa = wa[g];
+  const Window my_wa = win_a(kPackA ? 0 : ld_g);
   // MFMA: sub-block of this wave and the lane's place in it
   const int lane = t % kWave, wave = t / kWave;
   constexpr int kSubs = T >= 32 ? T / 32 : 1; // 32 x 32 sub-blocks per edge
@@ -192,14 +189,11 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
             const u32x4 la = *reinterpret_cast<const u32x4 *>(ea);
             const u32x4 lo = *reinterpret_cast<const u32x4 *>(eo);
             const uint32_t a3 = ea[4], o3 = eo[4];
-#pragma unroll
-            for (int h = 0; h < G; ++h)
-              if (g == h) {
-                if (inside(la, a3, wa[h]))
-                  oa = (int)(wa[h].base + la.x);
-                if (inside(lo, o3, wo[h]))
-                  oo = (int)(wo[h].base + lo.x);
-              }
+            const Window wa = win_a(g), wo = win_o(g);
+            if (inside(la, a3, wa))
+              oa = (int)(wa.base + la.x);
+            if (inside(lo, o3, wo))
+              oo = (int)(wo.base + lo.x);
           }
           row_a[e] = oa;
           row_o[e] = oo;
@@ -211,9 +205,8 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
             const u32x4 lo = *reinterpret_cast<const u32x4 *>(eo);
             const uint32_t o3 = eo[4];
             oo = (int)lo.x;
-#pragma unroll
             for (int h = 0; h < G; ++h)
-              ok |= inside(lo, o3, wo[h]) ? 1 << h : 0;
+              ok |= inside(lo, o3, win_o(h)) ? 1 << h : 0;
           }
           col_o[e - T] = oo;
           col_ok[e - T] = ok;
@@ -242,9 +235,14 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
       // other in the panel either way.
       [[maybe_unused]] int ra4[2][4];
       [[maybe_unused]] bool run4[2];
-      [[maybe_unused]] f32x4 va4[2];
-      const int pk = t % kStep, pi = t / kStep; // kPackA: K value and tile row
+      // kPackA: K value and row quad of the lane; quads pi and pi + 8 hold the
+      // same four records, 4 * (pi % (G / 4)) .. + 3
+      const int pk = t % kStep, pi = t / kStep;
+      [[maybe_unused]] Window wa4[4];
       if constexpr (kPackA) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          wa4[e] = win_a(4 * (pi % (G / 4)) + e);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           const int v0 = 4 * (pi + 8 * j);
@@ -257,114 +255,142 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
           run4[j] = run;
         }
       }
-      float va[kPasses];
-      f32x4 vb[kBLoads];
+      // Staging registers of one K step.  Every load below is unconditional: an
+      // inactive element is read from element 0 of its buffer (always there) and
+      // replaced by zero when the step is stored to LDS, so nothing between the
+      // loads and that store waits on memory and the loads of a step overlap
+      // each other and the multiply-adds of the step before.
+      [[maybe_unused]] E raw[kPackA ? 1 : kPasses];      // a, one element per pass
+      [[maybe_unused]] uint32_t raw_ok = 0;               // bit i: raw[i] is active
+      [[maybe_unused]] ex4u raw4[2];                      // a, kPackA with neighbouring windows
+      [[maybe_unused]] E raw1[2][4];                      // a, kPackA in general
+      f32x4 vb[kLow ? 1 : kBLoads];
       [[maybe_unused]] ex8 vb16[kBLoads16];
-      auto gather = [&](uint32_t k0) {
+      uint32_t vb_ok = 0;                                 // bit j: b load j is inside the tile
+      [[maybe_unused]] int next_off = 0;                  // kFast: a column offset of the next step
+      const E *bp16 = reinterpret_cast<const E *>(p.bpack) +
+                      (size_t)((uint32_t)rec[15] >> 2) * p.k_pad * p.tn_pad;
+      auto gather = [&](uint32_t k0, auto fast) {
+        constexpr bool kFast = decltype(fast)::value;
         // b: the next kStep rows of the packed tile, columns n0 .. n0 + T
+        vb_ok = 0;
         if constexpr (kLow) {
-          const E *bp16 = reinterpret_cast<const E *>(p.bpack) +
-                          (size_t)((uint32_t)rec[15] >> 1) * p.k_pad * p.tn_pad;
 #pragma unroll
           for (int j = 0; j < kBLoads16; ++j) {
-            const int id = t + j * kThreads, c = n0 + id / (kStep / 8), part = id % (kStep / 8);
-            ex8 v;
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-              v[e] = (E)0.0f;
-            if (c < p.tn_pad)
-              v = *reinterpret_cast<const ex8 *>(bp16 + (size_t)c * p.k_pad + k0 + 8 * part);
-            vb16[j] = v;
+            const int id = t + j * kThreads, part = id % (kStep / 8);
+            const uint32_t c = n0 + id / (kStep / 8);
+            const bool ok = c < p.tn_pad;
+            vb_ok |= ok ? 1u << j : 0u;
+            vb16[j] = *reinterpret_cast<const ex8 *>(bp16 + (size_t)(ok ? c : 0) * p.k_pad + k0 +
+                                                     8 * part);
           }
         } else {
 #pragma unroll
           for (int j = 0; j < kBLoads; ++j) {
-            const int id = t + j * kThreads, kr = id / (T / 4), c = n0 + 4 * (id % (T / 4));
-            vb[j] = c < p.tn_pad
-                        ? *reinterpret_cast<const f32x4 *>(bp + (size_t)(k0 + kr) * p.tn_pad + c)
-                        : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            const int id = t + j * kThreads, kr = id / (T / 4);
+            const uint32_t c = n0 + 4 * (id % (T / 4));
+            const bool ok = c < p.tn_pad;
+            vb_ok |= ok ? 1u << j : 0u;
+            vb[j] = *reinterpret_cast<const f32x4 *>(bp + (size_t)(k0 + kr) * p.tn_pad +
+                                                     (ok ? c : 0));
           }
         }
         if constexpr (!kPackA) {
           const uint32_t kk = k0 + ld_k;
-          const int oa = kk < p.k ? resolve(p.a_cols + 8 * (size_t)kk, my_wa) : -1;
-          // both offsets are non-negative when valid: the sign of the OR says
-          // whether either is the -1 marker
+          const int oa = resolve(p.a_cols + 8 * (size_t)(kk < p.k ? kk : 0), my_wa);
+          raw_ok = 0;
 #pragma unroll
-          for (int i = 0; i < kPasses; ++i)
-            va[i] = (oa | ra[i]) >= 0 ? (float)a[oa + ra[i]] : 0.0f;
-        }
-        if constexpr (kPackA) {
+          for (int i = 0; i < kPasses; ++i) {
+            // both offsets are non-negative when valid: the sign of the OR says
+            // whether either is the -1 marker
+            const bool ok = kk < p.k && (oa | ra[i]) >= 0;
+            raw_ok |= ok ? 1u << i : 0u;
+            raw[i] = a[ok ? oa + ra[i] : 0];
+          }
+        } else {
           const uint32_t ka = k0 + pk;
-          u32x4 ea = {0, ~0u, ~0u, ~0u};           // outside every window
-          uint32_t ea3 = ~0u;
-          if (ka < p.k) {
-            const int32_t *pa = p.a_cols + 8 * (size_t)ka;
-            ea = *reinterpret_cast<const u32x4 *>(pa);
-            ea3 = pa[4];
-          }
-          bool in[4];
+          const int32_t *pa = p.a_cols + 8 * (size_t)(ka < p.k ? ka : 0);
+          if constexpr (kFast) {
+            // every element of the set is active and the four windows of a quad
+            // are neighbours: one 16-byte (8-byte) load per quad.  The column
+            // offset was requested one step ago; the next one is requested now.
+            const int off = next_off;
+            const uint32_t kn = ka + kStep;
+            next_off = p.a_cols[8 * (size_t)(kn < p.k ? kn : 0)];
+            raw_ok = ka < p.k ? 1u : 0u;
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            in[e] = inside(ea, ea3, wa[e]);
-          const int off = (int)ea.x;
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            if (run4[j] && in[0] && in[1] && in[2] && in[3]) {
-              const ex4u x = *reinterpret_cast<const ex4u *>(a + off + ra4[j][0]);
-#pragma unroll
-              for (int e = 0; e < 4; ++e)
-                va4[j][e] = (float)x[e];
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; ++e)
-                va4[j][e] = (in[e] && ra4[j][e] >= 0) ? (float)a[off + ra4[j][e]] : 0.0f;
-            }
-          }
-        }
-      };
-
-      if (p.k > 0)
-        gather(0);
-      for (uint32_t k0 = 0; k0 < p.k; k0 += kStep) {
-        if constexpr (kLow) {
-          // the values went through fp32 unchanged: narrowing them again is exact
-#pragma unroll
-          for (int j = 0; j < kBLoads16; ++j) {
-            const int id = t + j * kThreads;
-            *reinterpret_cast<ex8 *>(&bs16[id / (kStep / 8)][8 * (id % (kStep / 8))]) = vb16[j];
-          }
-          if constexpr (!kPackA) {
-#pragma unroll
-            for (int i = 0; i < kPasses; ++i)
-              as16[(ld_r + kRowsPerPass / G * i) * G + ld_g][ld_k] = (E)va[i];
+            for (int j = 0; j < 2; ++j)
+              raw4[j] = *reinterpret_cast<const ex4u *>(a + off + ra4[j][0]);
           } else {
+            const u32x4 ea = *reinterpret_cast<const u32x4 *>(pa);
+            const uint32_t ea3 = pa[4];
+            const int off = (int)ea.x;
+            raw_ok = 0;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
-              for (int e = 0; e < 4; ++e)
-                as16[4 * (pi + 8 * j) + e][pk] = (E)va4[j][e];
+              for (int e = 0; e < 4; ++e) {
+                const bool ok = ka < p.k && inside(ea, ea3, wa4[e]) && ra4[j][e] >= 0;
+                raw_ok |= ok ? 1u << (4 * j + e) : 0u;
+                raw1[j][e] = a[ok ? off + ra4[j][e] : 0];
+              }
+          }
+        }
+      };
+      auto commit = [&](auto fast) {
+        constexpr bool kFast = decltype(fast)::value;
+        if constexpr (kLow) {
+#pragma unroll
+          for (int j = 0; j < kBLoads16; ++j) {
+            const int id = t + j * kThreads;
+            ex8 v = vb16[j];
+            if (!((vb_ok >> j) & 1))
+#pragma unroll
+              for (int e = 0; e < 8; ++e)
+                v[e] = (E)0.0f;
+            *reinterpret_cast<ex8 *>(&bs16[id / (kStep / 8)][8 * (id % (kStep / 8))]) = v;
           }
         } else {
 #pragma unroll
           for (int j = 0; j < kBLoads; ++j) {
             const int id = t + j * kThreads;
-            *reinterpret_cast<f32x4 *>(&bs[id / (T / 4)][4 * (id % (T / 4))]) = vb[j];
-          }
-          if constexpr (!kPackA) {
-#pragma unroll
-            for (int i = 0; i < kPasses; ++i)
-              as[ld_k][(ld_r + kRowsPerPass / G * i) * G + ld_g] = va[i];
-          }
-          if constexpr (kPackA) {
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-              *reinterpret_cast<f32x4 *>(&as[pk][4 * (pi + 8 * j)]) = va4[j];
+            const f32x4 v = ((vb_ok >> j) & 1) ? vb[j] : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            *reinterpret_cast<f32x4 *>(&bs[id / (T / 4)][4 * (id % (T / 4))]) = v;
           }
         }
-        __syncthreads();
-        if (k0 + kStep < p.k)
-          gather(k0 + kStep);
+        if constexpr (!kPackA) {
+#pragma unroll
+          for (int i = 0; i < kPasses; ++i) {
+            const int v = (ld_r + kRowsPerPass / G * i) * G + ld_g;
+            const E x = ((raw_ok >> i) & 1) ? raw[i] : (E)0.0f;
+            if constexpr (kLow)
+              as16[v][ld_k] = x;
+            else
+              as[ld_k][v] = (float)x;
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            E x[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if constexpr (kFast)
+                x[e] = (raw_ok & 1) ? (E)raw4[j][e] : (E)0.0f;
+              else
+                x[e] = ((raw_ok >> (4 * j + e)) & 1) ? raw1[j][e] : (E)0.0f;
+            }
+            if constexpr (kLow) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                as16[4 * (pi + 8 * j) + e][pk] = x[e];
+            } else {
+              *reinterpret_cast<f32x4 *>(&as[pk][4 * (pi + 8 * j)]) =
+                  f32x4{(float)x[0], (float)x[1], (float)x[2], (float)x[3]};
+            }
+          }
+        }
+      };
+      auto multiply = [&]() {
         if constexpr (kLow) {
 #pragma unroll
           for (int sub = 0; sub < kStep / 16; ++sub) {
@@ -407,8 +433,32 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
                 acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
           }
         }
-        __syncthreads();
-      }
+      };
+      auto k_loop = [&](auto fast) {
+        if constexpr (decltype(fast)::value)
+          next_off = p.a_cols[8 * (size_t)((uint32_t)pk < p.k ? pk : 0)];
+        if (p.k > 0)
+          gather(0, fast);
+        for (uint32_t k0 = 0; k0 < p.k; k0 += kStep) {
+          commit(fast);
+          __syncthreads();
+          if (k0 + kStep < p.k)
+            gather(k0 + kStep, fast);
+          multiply();
+          __syncthreads();
+        }
+      };
+      // bit 1 of the flag word: every a element of the set is active and its a
+      // windows are neighbours (host-checked), so the quads of this block can be
+      // read as vectors if their rows are neighbours too.  The choice is made per
+      // wave: both loops store the same panels and pass the same barriers.
+      bool fast_a = false;
+      if constexpr (kPackA)
+        fast_a = (rec[15] & 2) && __builtin_amdgcn_ballot_w64(!(run4[0] && run4[1])) == 0;
+      if (fast_a)
+        k_loop(std::true_type{});
+      else
+        k_loop(std::false_type{});
 
       // block row v belongs to record v % G (m0 is a multiple of G)
       if constexpr (MFMA) {
@@ -416,7 +466,7 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           // accumulator elements 4q .. 4q+3 are four consecutive block rows:
-          // with G = 4 one tile row for the four records of the set.  When
+          // with fused records one tile row for four records of the set.  When
           // their out windows follow each other element by element
           // (run_o) the four values are one 16-byte store.
           const int v0 = sub_m + 8 * q + 4 * l_hi;
@@ -425,8 +475,9 @@ __device__ __forceinline__ void gather_gemm(const GatherGemmArgs &p) {
           for (int e = 0; e < 4; ++e)
             ro[e] = row_o[v0 + e];
           bool packed = false;
-          if constexpr (G == 4)
-            packed = run_o && ok == 0xF && (ro[0] | ro[1] | ro[2] | ro[3]) >= 0;
+          if constexpr (kPackA)
+            packed = run_o && ((ok >> (v0 % G)) & 0xF) == 0xF &&
+                     (ro[0] | ro[1] | ro[2] | ro[3]) >= 0;
           if (packed) {
             ex4u val;
 #pragma unroll
@@ -525,6 +576,7 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_gather_pack_b_bf16(PackB
   HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_m64_g1, E, 64, 4, true, 1, 32)    \
   HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_m64_g2, E, 64, 4, true, 2, 32)    \
   HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_m64_g4, E, 64, 4, true, 4, 32)    \
+  HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_m64_g16, E, 64, 4, true, 16, 32)  \
   HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_m32_g1, E, 32, 4, true, 1, 32)    \
   HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_m32_g2, E, 32, 4, true, 2, 32)    \
   HCAMD_GATHER_GEMM(hcamd_gather_gemm_##TY##_t16_g1, E, 16, 2, false, 1, 32)   \

@@ -1312,9 +1312,15 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
   // mixes two b windows.
   const int wanted = variantOf("gather_fuse");
   const size_t cus = (size_t)std::max(computeUnitsOf(dev), 1);
-  size_t fuse = wanted >= 4 ? 4 : wanted >= 2 ? 2 : 1;
+  size_t fuse = wanted >= 16 ? 16 : wanted >= 4 ? 4 : wanted >= 2 ? 2 : 1;
   if (wanted == 0) {
-    if (tm >= 16 && nGroups / 4 * ceilDiv(4 * tm, (size_t)64) * ceilDiv(tn, (size_t)64) >= cus)
+    // workgroups a launch would have with G records fused (64-row blocks)
+    auto groupsOf = [&](size_t G) {
+      return nGroups / G * ceilDiv(G * tm, (size_t)64) * ceilDiv(tn, (size_t)64);
+    };
+    // (16 records per workgroup measured slower than 4 on the shapes tried:
+    // more registers, fewer resident waves; it stays selectable)
+    if (tm >= 16 && groupsOf(4) >= cus)
       fuse = 4;
     else if (nGroups / 2 >= cus)
       fuse = 2;
@@ -1434,7 +1440,7 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
       }
       w[0] = empty ? 0 : (int32_t)base;
     }
-    rec[15] = (int32_t)(windowOf[g] << 1); // bit 0 is the flag set below
+    rec[15] = (int32_t)(windowOf[g] << 2); // bits 0 and 1 are the flags set below
   }
   for (size_t w = 0; w < windowRep.size(); ++w) {
     // the b window of any record that has it (records hold it at words 5..9)
@@ -1446,27 +1452,52 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
         break;
       }
   }
-  // Flag (word 15 of a set's first record): the out windows of the set's records
-  // follow each other element by element and have equal extents along the
-  // dimensions the tile column drives, so that the values one tile element has
-  // for the records of the set are adjacent in memory.
-  if (fuse == 4)
-    for (size_t s0 = 0; s0 < slots.size(); s0 += fuse) {
-      int32_t *rec0 = host.data() + plan->offGroups + s0 * kGatherRecord;
-      bool run = true;
-      for (size_t i = 1; i < fuse && run; ++i) {
-        const int32_t *ri = rec0 + i * kGatherRecord, *rp = ri - kGatherRecord;
-        run = slots[s0 + i] >= 0 && slots[s0 + i - 1] >= 0 && ri[10] == rp[10] + 1;
-        for (int d = 0; d < 4 && run; ++d)
-          run = ri[11 + d] > 0 && rp[11 + d] > 0;
-      }
-      rec0[15] |= run ? 1 : 0;
-    }
   for (int o = 0; o < 3; ++o) {
     gatherEntries(*ops[o], ops[o]->rowIndex, rows[o], rowDim[o],
                   host.data() + plan->offRows[o]);
     gatherEntries(*ops[o], ops[o]->colIndex, cols[o], colDim[o],
                   host.data() + plan->offCols[o]);
+  }
+  // Flags in word 15 of a set's first record.  Bit 0: the out windows of the
+  // set's records follow each other element by element (and are not empty), so
+  // the values one tile element has for neighbouring records are adjacent in
+  // memory.  Bit 1: the same for the a windows, and every a element (all tile
+  // rows, all of K) of every record is active, so the kernel may read them
+  // without looking at the tables' indices.
+  if (fuse >= 4) {
+    // largest index each a entry needs along each dimension
+    int32_t need[4] = {0, 0, 0, 0};
+    bool nonneg = true;
+    for (int axis = 0; axis < 2; ++axis) {
+      const size_t n = axis ? cols[0] : rows[0];
+      const int32_t *tab = host.data() + (axis ? plan->offCols[0] : plan->offRows[0]);
+      for (size_t i = 0; i < n; ++i)
+        for (int d = 0; d < 4; ++d) {
+          const int32_t idx = tab[i * kGatherEntry + 1 + d];
+          nonneg = nonneg && idx >= 0;
+          need[d] = std::max(need[d], idx);
+        }
+    }
+    for (size_t s0 = 0; s0 < slots.size(); s0 += fuse) {
+      int32_t *rec0 = host.data() + plan->offGroups + s0 * kGatherRecord;
+      bool runO = true, runA = nonneg;
+      for (size_t i = 0; i < fuse; ++i) {
+        const int32_t *ri = rec0 + i * kGatherRecord;
+        if (slots[s0 + i] < 0) {
+          runO = runA = false;
+          break;
+        }
+        for (int d = 0; d < 4; ++d) {
+          runO = runO && ri[11 + d] > 0;
+          runA = runA && ri[1 + d] > need[d];
+        }
+        if (i > 0) {
+          runO = runO && ri[10] == ri[10 - kGatherRecord] + 1;
+          runA = runA && ri[0] == ri[0 - kGatherRecord] + 1;
+        }
+      }
+      rec0[15] |= (runO ? 1 : 0) | (runA ? 2 : 0);
+    }
   }
   if (dev->makeCurrent() ||
       HIP_CHECK(dev, hipMalloc((void **)&plan->tables, total * sizeof(int32_t)))) {
@@ -1519,12 +1550,12 @@ int hcamdGatherGemmLaunch(OlQueue q, HcamdGatherGemm plan, int elemType,
   const uint32_t side = std::max(plan->tm * plan->fuse, plan->tn);
   int variant = variantOf("gather");
   if (variant < 1 || variant > 6)
-    variant = plan->fuse == 4 ? 1
+    variant = plan->fuse >= 4 ? 1
               : side <= 8     ? 4
               : side <= 16    ? 3
               : side <= 32    ? 2
                               : 1;
-  if ((plan->fuse == 4 && variant != 1) || (plan->fuse == 2 && variant > 4) ||
+  if ((plan->fuse >= 4 && variant != 1) || (plan->fuse == 2 && variant > 4) ||
       (elemType != HCAMD_F32 && variant > 4)) {
     dev->report("hcamdGatherGemmLaunch: block shape %d is not built for %u "
                 "fused records of type %s", variant, plan->fuse, ty);

@@ -606,7 +606,7 @@ def test_implicit_gemm_convolution_of_the_reference_examples(n, c, nf, stride, t
     assert_allclose(out.to_host(), conv_direct(x, f, stride), rtol=1e-5, atol=1e-5)
 
 
-@pytest.mark.parametrize("fuse", [0, 1, 2, 4])
+@pytest.mark.parametrize("fuse", [0, 1, 2, 4, 16])
 def test_convolution_at_a_larger_size_with_full_tiles(fuse):
     from hc_amd.kernel import create_mapping
     from test_kernel_frontend import _conv_kernel, conv_direct

@@ -352,7 +352,7 @@ def _gather_reference(ops, n_groups, tm, tn, k, a, b, out):
     return out
 
 
-_GATHER_KERNELS = ([(v, 1) for v in range(7)] + [(v, 2) for v in range(5)] + [(0, 4), (1, 4)])
+_GATHER_KERNELS = ([(v, 1) for v in range(7)] + [(v, 2) for v in range(5)] + [(0, 4), (1, 4), (0, 16), (1, 16)])
 
 
 @pytest.mark.parametrize("variant,fuse", _GATHER_KERNELS)
@@ -402,7 +402,7 @@ def test_gathered_product_against_the_table_semantics(ctx, case, variant, fuse):
     assert_allclose(got, want, rtol=1e-5, atol=(K + 2) * 2.0 ** -22)
 
 
-@pytest.mark.parametrize("fuse", [1, 2, 4])
+@pytest.mark.parametrize("fuse", [1, 2, 4, 16])
 def test_gathered_product_inactive_elements_and_untouched_memory(ctx, fuse):
     """Windows that leave the buffer, negative and too-large indices, a start
     beyond the end: inactive operands count as zero, inactive outputs keep
@@ -435,7 +435,7 @@ def test_gathered_product_inactive_elements_and_untouched_memory(ctx, fuse):
 
 
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
-@pytest.mark.parametrize("fuse", [1, 2, 4])
+@pytest.mark.parametrize("fuse", [1, 2, 4, 16])
 def test_gathered_product_on_16_bit_storage(ctx, dtype, fuse):
     """Elements are widened to fp32, multiplied and summed in fp32 and rounded
     once when stored: the result is the rounding of an fp32-accurate product."""
