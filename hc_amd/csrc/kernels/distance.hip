@@ -43,12 +43,22 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_pairwise_dist_f32(
   const int ld_d = t % kStep, ld_r = t / kStep;
   for (size_t d0 = 0; d0 < D; d0 += kStep) {
     const size_t d = d0 + ld_d;
+    // all sixteen loads are issued before any is used: an element outside the
+    // matrices is read from element 0 instead and replaced by zero afterwards
+    // (a load inside a per-lane branch would be waited for on the spot)
+    float va[kTile / 8], vb[kTile / 8];
 #pragma unroll
     for (int k = 0; k < kTile / 8; ++k) {
       const int r = ld_r + 8 * k;
       const size_t ma = m0 + r, nb = n0 + r;
-      as[ld_d][r] = (d < D && ma < M) ? a[ma * lda + d] : 0.0f;
-      bs[ld_d][r] = (d < D && nb < N) ? b[nb * ldb + d] : 0.0f;
+      va[k] = a[(d < D && ma < M) ? ma * lda + d : 0];
+      vb[k] = b[(d < D && nb < N) ? nb * ldb + d : 0];
+    }
+#pragma unroll
+    for (int k = 0; k < kTile / 8; ++k) {
+      const int r = ld_r + 8 * k;
+      as[ld_d][r] = (d < D && m0 + r < M) ? va[k] : 0.0f;
+      bs[ld_d][r] = (d < D && n0 + r < N) ? vb[k] : 0.0f;
     }
     __syncthreads();
 #pragma unroll 8
