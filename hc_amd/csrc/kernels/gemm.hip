@@ -242,7 +242,13 @@ __device__ __forceinline__ Acc mfma_block(V b, V a, Acc c) {
   }
 }
 
-template <class E, int BM, int BN, int WM, int WN, int MF>
+// EDGE = true: M and N need not be multiples of the tile and K only a multiple
+// of 8.  Panel rows past the last row are read from the last row (their results
+// are never stored); in the last K tile the 16-byte chunks past K are read from
+// the start of their row instead and overwritten with zeros in LDS by the lane
+// that fetched them, before the barrier that releases the tile; stores are
+// masked.  Everything else, and the speed on whole tiles, is the same.
+template <class E, int BM, int BN, int WM, int WN, int MF, bool EDGE = false>
 __device__ __forceinline__ void gemm_tile_pipelined(
     const E *__restrict__ A, size_t lda, const E *__restrict__ Bt, size_t ldb,
     E *__restrict__ C, size_t ldc, int M, int N, int K) {
@@ -268,11 +274,17 @@ __device__ __forceinline__ void gemm_tile_pipelined(
   __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kStageBytes];
 
   int tm, tn;
-  tile_of_workgroup(M / BM, N / BN, tm, tn);
+  if constexpr (EDGE)
+    tile_of_workgroup((M + BM - 1) / BM, (N + BN - 1) / BN, tm, tn);
+  else
+    tile_of_workgroup(M / BM, N / BN, tm, tn);
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int wave_m = (wave / WN) * kWaveM;
   const int wave_n = (wave % WN) * kWaveN;
+  const int KT = EDGE ? (K + kBK - 1) / kBK : K / kBK; // host guarantees KT >= 2
+  // EDGE: whole 16-byte chunks of the last K tile that hold data (8 = all)
+  const int tail_chunks = EDGE && K % kBK ? (K % kBK) / 8 : 8;
 
   // ---- global -> LDS ---------------------------------------------------------
   // load i of this wave fills panel rows (i*kWaves + wave)*8 .. +8
@@ -282,26 +294,54 @@ __device__ __forceinline__ void gemm_tile_pipelined(
 #pragma unroll
   for (int i = 0; i < kALoads; ++i) {
     const int r = (i * kWaves + wave) * 8 + ld_row;
-    a_src[i] = A + (size_t)(tm * BM + r) * lda + ((ld_pchunk ^ swz<SH>(r)) * 8);
+    const int row = EDGE ? min(tm * BM + r, M - 1) : tm * BM + r;
+    a_src[i] = A + (size_t)row * lda + ((ld_pchunk ^ swz<SH>(r)) * 8);
   }
 #pragma unroll
   for (int i = 0; i < kBLoads; ++i) {
     const int r = (i * kWaves + wave) * 8 + ld_row;
-    b_src[i] = Bt + (size_t)(tn * BN + r) * ldb + ((ld_pchunk ^ swz<SH>(r)) * 8);
+    const int row = EDGE ? min(tn * BN + r, N - 1) : tn * BN + r;
+    b_src[i] = Bt + (size_t)row * ldb + ((ld_pchunk ^ swz<SH>(r)) * 8);
   }
+  // logical chunk the lane fetches in load i (the swizzle depends on the row)
+  auto chunk_of = [&](int i) { return ld_pchunk ^ swz<SH>((i * kWaves + wave) * 8 + ld_row); };
   auto issue_loads = [&](int kt, int buf) {
     const size_t k0 = (size_t)kt * kBK;
     unsigned char *base = lds + buf * kStageBytes + wave * 1024;
+    const bool tail = EDGE && kt == KT - 1 && tail_chunks < 8;
 #pragma unroll
-    for (int i = 0; i < kALoads; ++i)
-      __builtin_amdgcn_global_load_lds((global_cptr)(a_src[i] + k0),
+    for (int i = 0; i < kALoads; ++i) {
+      const E *src = a_src[i] + k0;
+      if (tail && chunk_of(i) >= tail_chunks)
+        src -= chunk_of(i) * 8;          // chunk 0 of the row: valid, zeroed later
+      __builtin_amdgcn_global_load_lds((global_cptr)src,
                                        (lds_ptr)(base + i * kWaves * 1024), 16,
                                        0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < kBLoads; ++i) {
+      const E *src = b_src[i] + k0;
+      if (tail && chunk_of(i) >= tail_chunks)
+        src -= chunk_of(i) * 8;
+      __builtin_amdgcn_global_load_lds(
+          (global_cptr)src, (lds_ptr)(base + kABytes + i * kWaves * 1024), 16, 0,
+          0);
+    }
+  };
+  // EDGE: after the last K tile has landed, the chunks past K become zeros
+  auto zero_tail = [&](int buf) {
+    if (!(EDGE && tail_chunks < 8))
+      return;
+    unsigned char *base = lds + buf * kStageBytes + wave * 1024 + lane * 16;
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < kALoads; ++i)
+      if (chunk_of(i) >= tail_chunks)
+        *reinterpret_cast<u32x4 *>(base + i * kWaves * 1024) = zero;
 #pragma unroll
     for (int i = 0; i < kBLoads; ++i)
-      __builtin_amdgcn_global_load_lds(
-          (global_cptr)(b_src[i] + k0),
-          (lds_ptr)(base + kABytes + i * kWaves * 1024), 16, 0, 0);
+      if (chunk_of(i) >= tail_chunks)
+        *reinterpret_cast<u32x4 *>(base + kABytes + i * kWaves * 1024) = zero;
   };
 
   // ---- LDS -> operand registers ------------------------------------------------
@@ -378,7 +418,6 @@ __device__ __forceinline__ void gemm_tile_pipelined(
   using NoVmem = std::integral_constant<int, 0>;
   using WithVmem = std::integral_constant<int, kALoads + kBLoads>;
 
-  const int KT = K / kBK; // host guarantees KT >= 2
   issue_loads(0, 0);
   issue_loads(1, 1);
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(kALoads + kBLoads, kNoLgkm));
@@ -388,6 +427,8 @@ __device__ __forceinline__ void gemm_tile_pipelined(
   auto tile_step = [&](int t, auto load_next2, auto read_next) {
     constexpr bool LOAD = decltype(load_next2)::value;
     constexpr bool READ = decltype(read_next)::value;
+    // the step before the last: the last tile has landed at its barrier
+    constexpr bool ZERO = EDGE && !LOAD && READ;
     const int buf = t & 1;
     // even half-step: consume slot 0 (requested a whole half-step ago, so the
     // wait is free and makes the later waits exact), fetch slot 1
@@ -399,6 +440,10 @@ __device__ __forceinline__ void gemm_tile_pipelined(
     // odd half-step; the fences keep the MFMAs above on this side of the wait
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+    if constexpr (ZERO) {
+      zero_tail(buf ^ 1);
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoVm, 0));
+    }
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (LOAD)
@@ -421,9 +466,12 @@ __device__ __forceinline__ void gemm_tile_pipelined(
   // ---- epilogue ------------------------------------------------------------------
   const int m_base = tm * BM + wave_m + lrow;
   const int n_base = tn * BN + wave_n + lchunk * 4;
+  const bool vec_c = !EDGE || (ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(C) & 7) == 0);
 #pragma unroll
   for (int i = 0; i < kMI; ++i) {
     E *crow = C + (size_t)(m_base + i * MF) * ldc + n_base;
+    if (EDGE && m_base + i * MF >= M)
+      continue;
 #pragma unroll
     for (int j = 0; j < kNI; ++j) {
 #pragma unroll
@@ -432,7 +480,15 @@ __device__ __forceinline__ void gemm_tile_pipelined(
 #pragma unroll
         for (int e = 0; e < 4; ++e)
           o[e] = (E)acc[i][j][4 * g + e];
-        *reinterpret_cast<ex4 *>(crow + j * MF + g * 8) = o;
+        const int n = n_base + j * MF + g * 8;
+        if (!EDGE || (vec_c && n + 3 < N)) {
+          *reinterpret_cast<ex4 *>(crow + j * MF + g * 8) = o;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < N)
+              crow[j * MF + g * 8 + e] = o[e];
+        }
       }
     }
   }
@@ -446,6 +502,17 @@ __device__ __forceinline__ void gemm_tile_pipelined(
     gemm_tile_pipelined<E, BM, BN, WM, WN, MF>(A, lda, Bt, ldb, C, ldc, M, N,  \
                                                K);                             \
   }
+#define HCAMD_GEMM_PE(NAME, E, BM, BN, WM, WN, MF)                             \
+  extern "C" __global__ __launch_bounds__(WM *WN * 64) void NAME(              \
+      const E *A, size_t lda, const E *Bt, size_t ldb, E *C, size_t ldc,       \
+      int M, int N, int K) {                                                   \
+    gemm_tile_pipelined<E, BM, BN, WM, WN, MF, true>(A, lda, Bt, ldb, C, ldc,  \
+                                                     M, N, K);                 \
+  }
+HCAMD_GEMM_PE(hcamd_gemm_bf16_p256x256_w2x4_edge, __bf16, 256, 256, 2, 4, 16)
+HCAMD_GEMM_PE(hcamd_gemm_f16_p256x256_w2x4_edge, _Float16, 256, 256, 2, 4, 16)
+HCAMD_GEMM_PE(hcamd_gemm_bf16_p128x128_w2x2_edge, __bf16, 128, 128, 2, 2, 16)
+HCAMD_GEMM_PE(hcamd_gemm_f16_p128x128_w2x2_edge, _Float16, 128, 128, 2, 2, 16)
 HCAMD_GEMM_P(hcamd_gemm_bf16_p256x256_w2x4, __bf16, 256, 256, 2, 4, 16)
 HCAMD_GEMM_P(hcamd_gemm_bf16_p256x256_w4x2, __bf16, 256, 256, 4, 2, 16)
 HCAMD_GEMM_P(hcamd_gemm_bf16_p128x128_w2x2, __bf16, 128, 128, 2, 2, 16)

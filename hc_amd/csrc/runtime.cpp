@@ -1862,11 +1862,33 @@ int launchGemm(OlQueue q, bool half, const void *a, size_t lda, const void *bt,
         pick = &tiled[3];
     }
   }
+  // Shapes the whole-tile kernels cannot take (M or N not a multiple of the
+  // tile, K not a multiple of 64) go to the edge-capable build of the pipelined
+  // kernel as long as the panels can be fetched in 16-byte pieces; only what
+  // is left (odd K or leading dimensions, K <= 64, misaligned A / Bt) takes the
+  // general kernel.  Variant 13 forces the edge kernel, 6 the general one.
+  static const Tiled edge[2][2] = {
+      {{"hcamd_gemm_bf16_p256x256_w2x4_edge", 256, 256, 512},
+       {"hcamd_gemm_bf16_p128x128_w2x2_edge", 128, 128, 256}},
+      {{"hcamd_gemm_f16_p256x256_w2x4_edge", 256, 256, 512},
+       {"hcamd_gemm_f16_p128x128_w2x2_edge", 128, 128, 256}}};
+  const bool edge_ok = aligned16(a) && aligned16(bt) && lda % 8 == 0 &&
+                       ldb % 8 == 0 && k % 8 == 0 && k > 64 &&
+                       (reinterpret_cast<uintptr_t>(c) & 1) == 0;
+  bool ragged = false;
+  if (edge_ok && variant != kGeneral && (!pick || variant == 13)) {
+    // the smaller tile when the larger one would leave most CUs idle
+    const size_t big = ceilDiv(m, (size_t)256) * ceilDiv(n, (size_t)256);
+    pick = &edge[half ? 1 : 0][big >= (size_t)computeUnitsOf(dev) / 2 ? 0 : 1];
+    ragged = true;
+  }
   if (pick) {
     Kernel *kn = builtinKernel(dev, "gemm", pick->name);
     if (!kn)
       return 1;
-    const size_t grid[3] = {(m / pick->bm) * (n / pick->bn), 1, 1};
+    const size_t grid[3] = {ragged ? ceilDiv(m, (size_t)pick->bm) * ceilDiv(n, (size_t)pick->bn)
+                                   : (m / pick->bm) * (n / pick->bn),
+                            1, 1};
     const size_t block[3] = {(size_t)pick->threads, 1, 1};
     return launch(queue, kn, grid, block, args, 0);
   }

@@ -392,9 +392,12 @@ int hcamdLaunchQuantizeF16I8(OlQueue q, const void *x, size_t ldx, int8_t *qout,
 
 /* C[M,N] = A[M,K] * B[K,N]; A row-major bf16 (lda), B column-major bf16 given
  * as Bt[N,K] row-major (ldb), fp32 accumulation on MFMA, C row-major bf16
- * (ldc), round to nearest even.  Any M, N, K >= 1; K-contiguous rows must be
- * 16-byte aligned for the fast path (ld % 8 == 0 and aligned base), otherwise
- * a slower general kernel runs. */
+ * (ldc), round to nearest even.  Any M, N, K >= 1.  The matrix-core kernels
+ * take every shape whose K-contiguous rows can be fetched in 16-byte pieces
+ * (A and Bt 16-byte aligned, lda, ldb and K multiples of 8, K > 64): M and N
+ * need not be multiples of the tile, C may have any leading dimension.  Other
+ * shapes (odd K or leading dimensions, K <= 64) run a much slower general
+ * kernel. */
 int hcamdLaunchGemmBF16(OlQueue q, const void *a, size_t lda, const void *bt,
                         size_t ldb, void *c, size_t ldc, size_t m, size_t n,
                         size_t k) HCAMD_NOEXCEPT;

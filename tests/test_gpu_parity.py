@@ -1005,11 +1005,57 @@ def test_gemm_fp16_against_fp32_accumulation(ctx, mnk):
     assert_array_equal(c2.to_host().astype(np.float32), ai.astype(np.float32) @ bi.astype(np.float32).T)
 
 
+@pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("mnk", [(300, 200, 136), (257, 255, 72), (1000, 1000, 1000), (129, 640, 192),
+                                 (1, 1, 128), (513, 7, 4096 + 8)])
+def test_gemm_ragged_shapes_take_the_edge_kernel(ctx, mnk, half):
+    """M and N off the tile, K a multiple of 8 only: rows past the end are never
+    stored, the K chunks past the end are zeros, and the result equals the
+    whole-tile kernel's arithmetic (fp32 accumulation, one rounding)."""
+    m, n, k = mnk
+    rng = np.random.default_rng(sum(mnk))
+    a32 = (0.5 * rng.standard_normal((m, k))).astype(np.float32)
+    b32 = (0.5 * rng.standard_normal((n, k))).astype(np.float32)
+    pad = 3                                       # odd leading dimension of C: scalar stores
+    if half:
+        a, bt = a32.astype(np.float16), b32.astype(np.float16)
+        c = poisoned((m + 2, n + pad), np.float16)
+        rt.plan_gemm_f16(dev(a), dev(bt), _View(c, (m, n), 0, (n + pad, 1))).launch(sync=True)
+        got = c.to_host().astype(np.float32)
+        av, bv, eps = a.astype(np.float32), bt.astype(np.float32), 2.0 ** -10
+    else:
+        a, bt = cf.f32_to_bf16_bits(a32), cf.f32_to_bf16_bits(b32)
+        c = rt.DeviceArray((m + 2, n + pad), np.uint16, ctx, True).fill_bytes32(POISON32)
+        rt.plan_gemm_bf16(dev(a, bf16=True), dev(bt, bf16=True),
+                          _View(c, (m, n), 0, (n + pad, 1))).launch(sync=True)
+        got = cf.bf16_bits_to_f32(c.to_host())
+        av, bv, eps = cf.bf16_bits_to_f32(a), cf.bf16_bits_to_f32(bt), 2.0 ** -7
+    say("gemm ragged", mnk, half, rt.last_kernel_name())
+    assert rt.last_kernel_name().endswith("_edge")
+    want = av.astype(np.float64) @ bv.astype(np.float64).T
+    assert_allclose(got[:m, :n], want, rtol=eps, atol=eps * np.sqrt(k) * 0.25)
+    raw = c.to_host().view(np.uint16)
+    assert (raw[m:] == (POISON32 & 0xFFFF)).all() and (raw[:, n:] == (POISON32 & 0xFFFF)).all()
+    # the general kernel (variant 6) agrees to the last bit: same products, fp32 sums in
+    # another order would differ, so compare within one rounding instead
+    rt.set_variant("gemm", 6)
+    if half:
+        c2 = rt.DeviceArray((m, n), np.float16)
+        rt.plan_gemm_f16(dev(a), dev(bt), c2).launch(sync=True)
+        got2 = c2.to_host().astype(np.float32)
+    else:
+        c2 = rt.DeviceArray((m, n), np.uint16, ctx, True)
+        rt.plan_gemm_bf16(dev(a, bf16=True), dev(bt, bf16=True), c2).launch(sync=True)
+        got2 = cf.bf16_bits_to_f32(c2.to_host())
+    assert rt.last_kernel_name().endswith("_general")
+    assert_allclose(got[:m, :n], got2, rtol=2 * eps, atol=eps * np.sqrt(k) * 0.25)
+
+
 def test_gemm_all_variants_and_padded_output(ctx):
     ab, bb = cf.inputs_c5((512, 512, 256))
     want = cf.np_gemm_bf16(ab, bb, np.float32)
     sigma = 0.02 * 0.02 * 16
-    for v in range(0, 13):
+    for v in range(0, 14):
         rt.set_variant("gemm", v)
         got = cf.bf16_bits_to_f32(run_gemm(ab, bb, ldc_pad=8))
         say("gemm variant", v, rt.last_kernel_name())
