@@ -7,7 +7,10 @@
 // workgroup per row (rows up to 1024*VPT columns); TPR = 64 gives one wave per
 // row and four rows per workgroup for short rows, with no barrier at all.
 //
-// A streaming kernel covers rows that do not fit or are not 16-byte aligned.
+// Rows that are not 16-byte aligned stay register-resident with 4-byte
+// accesses (256 or 1024 lanes per row, up to 32,768 columns); longer rows take
+// two sweeps with an online maximum and sum.  The three-sweep streaming kernel
+// is kept as the plainest statement of the operation (variant 1).
 #include "common.h"
 
 using namespace hcamd;
@@ -244,6 +247,161 @@ __device__ __forceinline__ void softmax_persistent(const float *x, size_t ldx,
 HCAMD_SOFTMAX_PERSIST(hcamd_softmax_f32_p256_v8_nt, 8, true)
 HCAMD_SOFTMAX_PERSIST(hcamd_softmax_f32_p256_v8, 8, false)
 HCAMD_SOFTMAX_PERSIST(hcamd_softmax_f32_p256_v4_nt, 4, true)
+
+// Rows that are not 16-byte aligned (a column count or leading dimension that
+// is not a multiple of 4) but still fit in registers: one workgroup per row,
+// lane t holds elements t, t + 256, ... (EPL of them), read and written with
+// 4-byte accesses that a wave coalesces into 256-byte requests.  The row still
+// crosses HBM once each way.  All loads are issued before the first is used;
+// elements past the end are read from element 0 and replaced by -inf.
+template <int EPL, int kThreads = 256>
+__device__ __forceinline__ void softmax_scalar_regs(const float *x, size_t ldx, float *y,
+                                                    size_t ldy, size_t cols) {
+  __shared__ float smax[kThreads / kWave];
+  __shared__ float ssum[kThreads / kWave];
+  const size_t row = blockIdx.x;
+  const float *xr = x + row * ldx;
+  float *yr = y + row * ldy;
+  const int t = threadIdx.x;
+  float v[EPL];
+  // 32-bit element offsets from the row start (rows are shorter than 2^31)
+  const uint32_t n = (uint32_t)cols;
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    const uint32_t c = (uint32_t)j * kThreads + t;
+    v[j] = __builtin_nontemporal_load(xr + (c < n ? c : 0u));
+    if (j % 16 == 15) // keeps the address arithmetic of later loads from piling up
+      __builtin_amdgcn_sched_barrier(0);
+  }
+  float m = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    v[j] = (size_t)j * kThreads + t < cols ? v[j] : -INFINITY;
+    m = fmaxf(m, v[j]);
+  }
+  m = group_reduce<MaxOp, kThreads / kWave>(m, smax);
+  float s = 0.0f;
+  if (__builtin_fabsf(m) < kFusedMaxAbs) { // uniform over the row
+    const float m_log2e = m * 1.44269502162933349609375f;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) {
+      v[j] = exp_scaled(v[j], m_log2e);
+      s += v[j];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) {
+      v[j] = exp_shifted(v[j], m);
+      s += v[j];
+    }
+  }
+  s = group_reduce<SumOp, kThreads / kWave>(s, ssum);
+  const float inv = 1.0f / s;
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    const size_t c = (size_t)j * kThreads + t;
+    if (c < cols)
+      __builtin_nontemporal_store(v[j] * inv, yr + c);
+  }
+}
+#define HCAMD_SOFTMAX_SCALAR(NAME, EPL)                                        \
+  extern "C" __global__ __launch_bounds__(256) void NAME(                      \
+      const float *x, size_t ldx, float *y, size_t ldy, size_t rows,           \
+      size_t cols) {                                                           \
+    softmax_scalar_regs<EPL>(x, ldx, y, ldy, cols);                            \
+  }
+HCAMD_SOFTMAX_SCALAR(hcamd_softmax_f32_s256_e4, 4)
+HCAMD_SOFTMAX_SCALAR(hcamd_softmax_f32_s256_e8, 8)
+HCAMD_SOFTMAX_SCALAR(hcamd_softmax_f32_s256_e16, 16)
+HCAMD_SOFTMAX_SCALAR(hcamd_softmax_f32_s256_e32, 32)
+HCAMD_SOFTMAX_SCALAR(hcamd_softmax_f32_s256_e64, 64)
+// the same with 1024 lanes per row: rows of up to 32,768 elements stay in
+// registers (32 per lane, four waves per SIMD)
+#define HCAMD_SOFTMAX_SCALAR_1024(NAME, EPL)                                   \
+  extern "C" __global__ __launch_bounds__(1024) void NAME(                     \
+      const float *x, size_t ldx, float *y, size_t ldy, size_t rows,           \
+      size_t cols) {                                                           \
+    softmax_scalar_regs<EPL, 1024>(x, ldx, y, ldy, cols);                      \
+  }
+HCAMD_SOFTMAX_SCALAR_1024(hcamd_softmax_f32_s1024_e32, 32)
+
+// Rows too long for registers: two sweeps instead of three.  The first keeps a
+// running maximum and a sum that is rescaled whenever the maximum grows (the
+// online form: s <- s * exp(m_old - m_new) + exp(x - m_new)), per lane, and
+// lanes are merged the same way at the end; the second sweep writes.  A
+// workgroup of 1024 lanes per row, so that a row of 50,000 elements is ~49
+// elements per lane and the second sweep finds the row in L2.
+__device__ __forceinline__ void online_merge(float &m, float &s, float m2, float s2) {
+  const float mm = fmaxf(m, m2);
+  // exp(-inf - -inf) would be NaN: a side that has seen nothing contributes 0
+  const float a = m == -INFINITY ? 0.0f : s * exp_nonpos(m - mm);
+  const float b = m2 == -INFINITY ? 0.0f : s2 * exp_nonpos(m2 - mm);
+  m = mm;
+  s = a + b;
+}
+extern "C" __global__ __launch_bounds__(1024) void hcamd_softmax_f32_online(
+    const float *x, size_t ldx, float *y, size_t ldy, size_t rows,
+    size_t cols) {
+  constexpr int kT = 1024;
+  __shared__ float sm[kT / kWave], ss[kT / kWave];
+  const size_t row = blockIdx.x;
+  const float *xr = x + row * ldx;
+  float *yr = y + row * ldy;
+  const int t = threadIdx.x;
+  float m = -INFINITY, s = 0.0f;
+  bool nan = false;
+  size_t c = t;
+  // four independent loads in flight per lane
+  for (; c + 3 * kT < cols; c += 4 * kT) {
+    float v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      v[u] = xr[c + u * kT];
+    const float vm = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
+    nan = nan || v[0] != v[0] || v[1] != v[1] || v[2] != v[2] || v[3] != v[3];
+    if (vm > m) {
+      s = m == -INFINITY ? 0.0f : s * exp_nonpos(m - vm);
+      m = vm;
+    }
+    // while the maximum is still -inf every element so far was -inf (or NaN,
+    // which the flag remembers) and adds nothing; -inf - -inf would be NaN
+    if (m != -INFINITY) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        s += exp_nonpos(v[u] - m);
+    }
+  }
+  for (; c < cols; c += kT) {
+    const float v = xr[c];
+    nan = nan || v != v;
+    if (v > m) {
+      s = m == -INFINITY ? 0.0f : s * exp_nonpos(m - v);
+      m = v;
+    }
+    if (m != -INFINITY)
+      s += exp_nonpos(v - m);
+  }
+  // lanes -> wave (DPP shuffles through readlane-free butterfly) -> workgroup
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float m2 = __shfl_xor(m, off, kWave), s2 = __shfl_xor(s, off, kWave);
+    online_merge(m, s, m2, s2);
+  }
+  if (t % kWave == 0) {
+    sm[t / kWave] = m;
+    ss[t / kWave] = s;
+  }
+  const bool any_nan = __syncthreads_or(nan);
+  m = sm[0];
+  s = ss[0];
+#pragma unroll
+  for (int w = 1; w < kT / kWave; ++w)
+    online_merge(m, s, sm[w], ss[w]);
+  // a NaN anywhere makes the whole row NaN, as the whole-array expression does
+  const float inv = any_nan ? __builtin_nanf("") : 1.0f / s;
+  for (c = t; c < cols; c += kT)
+    yr[c] = exp_nonpos(xr[c] - m) * inv;
+}
 
 // Streaming kernel: one workgroup per row, three sweeps over the row (max,
 // sum, write) with scalar accesses; the second and third sweeps hit L2.  Any

@@ -1666,9 +1666,29 @@ int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,
   const int variant = variantOf("softmax");
   const bool vec_ok = aligned16(x) && aligned16(y) &&
                       (rows == 1 || (ldx % 4 == 0 && ldy % 4 == 0));
-  if (!vec_ok || cols > 16384 || variant == 1)
+  if (variant == 1)
     return launch1d(queue, "softmax", "hcamd_softmax_f32_stream", rows, 256,
                     args);
+  if (cols > 32768 || (cols > 16384 && variant == 2))
+    // longer than the registers of a workgroup: two sweeps, online maximum / sum
+    // (parking the tail of such a row in LDS, one 1024-lane workgroup per CU,
+    // measured no faster)
+    return launch1d(queue, "softmax", "hcamd_softmax_f32_online", rows, 1024,
+                    args);
+  if (cols > 16384)
+    // 1024 lanes per row, 32 elements per lane in registers
+    return launch1d(queue, "softmax", "hcamd_softmax_f32_s1024_e32", rows, 1024,
+                    args);
+  if (!vec_ok) {
+    // rows that do not start on 16-byte boundaries: register-resident with
+    // 4-byte accesses
+    const char *scalar = cols <= 1024   ? "hcamd_softmax_f32_s256_e4"
+                         : cols <= 2048 ? "hcamd_softmax_f32_s256_e8"
+                         : cols <= 4096 ? "hcamd_softmax_f32_s256_e16"
+                         : cols <= 8192 ? "hcamd_softmax_f32_s256_e32"
+                                        : "hcamd_softmax_f32_s256_e64";
+    return launch1d(queue, "softmax", scalar, rows, 256, args);
+  }
   const char *name;
   size_t groups = rows;
   if (cols <= 1024) {

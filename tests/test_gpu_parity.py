@@ -734,7 +734,8 @@ SOFTMAX_ATOL = 1e-9
 
 @pytest.mark.parametrize("shape", [(1, 1), (5, 7), (33, 256), (7, 257), (64, 1000), (16, 1024),
                                    (8, 2048), (9, 4097), (12, 8192), (5, 8190), (3, 16384),
-                                   (3, 12345), (2, 20000), (1030, 512)])
+                                   (3, 12345), (2, 20000), (1030, 512), (4, 1001), (3, 2047),
+                                   (2, 16383), (2, 16385), (3, 50257), (2, 131072)])
 def test_softmax_against_both_oracles(ctx, shape):
     (x,) = cf.inputs_c3(shape)
     dy = poisoned(shape, np.float32)
@@ -759,16 +760,21 @@ def test_softmax_variants_and_strided_rows(ctx):
         out = dy.to_host()
         assert_allclose(out[:, :cols], want, rtol=SOFTMAX_RTOL, atol=SOFTMAX_ATOL)
         assert (out[:, cols:].view(np.uint32) == POISON32).all()
-    # unaligned base pointer -> streaming kernel
+    # unaligned base pointer -> register-resident kernel with 4-byte accesses
     rt.set_variant("softmax", 0)
-    dy = poisoned((rows, ld), np.float32)
-    rt.softmax_f32(_View(dx, (rows, 1000), 1, (ld, 1)), _View(dy, (rows, 1000), 1, (ld, 1)))
-    assert rt.last_kernel_name() == "hcamd_softmax_f32_stream"
-    assert_allclose(dy.to_host()[:, 1:1001], cf.np_softmax(x[:, 1:1001]), rtol=SOFTMAX_RTOL,
-                    atol=SOFTMAX_ATOL)
+    for width, kernel in ((1000, "hcamd_softmax_f32_s256_e4"), (8190, "hcamd_softmax_f32_s256_e32")):
+        dy = poisoned((rows, ld), np.float32)
+        rt.softmax_f32(_View(dx, (rows, width), 1, (ld, 1)), _View(dy, (rows, width), 1, (ld, 1)))
+        assert rt.last_kernel_name() == kernel
+        out = dy.to_host()
+        assert_allclose(out[:, 1:1 + width], cf.np_softmax(x[:, 1:1 + width]), rtol=SOFTMAX_RTOL,
+                        atol=SOFTMAX_ATOL)
+        assert (out[:, 0].view(np.uint32) == POISON32).all()
+        assert (out[:, 1 + width:].view(np.uint32) == POISON32).all()
 
 
-@pytest.mark.parametrize("cols,variant", [(1024, 0), (8192, 0), (8192, 5)])
+@pytest.mark.parametrize("cols,variant", [(1024, 0), (8192, 0), (8192, 5), (1023, 0), (8191, 0),
+                                          (12345, 0), (20000, 0), (50257, 0), (70001, 0), (20000, 2), (8192, 1)])
 def test_softmax_extreme_and_special_rows(ctx, cols, variant):
     f = np.float32
     x = np.zeros((6, cols), f)
@@ -793,7 +799,8 @@ def test_softmax_extreme_and_special_rows(ctx, cols, variant):
     assert y[5, 3] == 1.0 and y[5].sum() == 1.0
 
 
-@pytest.mark.parametrize("cols,variant", [(1000, 0), (4096, 0), (8192, 0), (8192, 5)])
+@pytest.mark.parametrize("cols,variant", [(1000, 0), (4096, 0), (8192, 0), (8192, 5), (4095, 0),
+                                          (20001, 0), (40000, 0), (66000, 0)])
 def test_softmax_rows_of_huge_magnitude(ctx, cols, variant):
     # a row's maximum may be far from 0: only differences matter
     f = np.float32
