@@ -246,6 +246,112 @@ __device__ __forceinline__ void quantize_persistent(const _Float16 *x, size_t ld
     cur[1] = nxt[1];
   }
 }
+// Rows that are not 16-byte aligned but still fit in registers: one workgroup
+// per row, lane t holds groups t, t + 256, ... of V consecutive elements (V = 4,
+// 2 or 1 as the leading dimensions allow: 8-, 4- or 2-byte loads and 4-, 2- or
+// 1-byte stores).  The row crosses HBM once each way; every load is
+// unconditional (a group past the end is read from group 0 and ignored) and
+// issued before the first use.  The cols % V elements after the last whole group
+// are handled one per lane.
+template <int V, int EPL>
+__device__ __forceinline__ void quantize_small(const _Float16 *x, size_t ldx, int8_t *q,
+                                               size_t ldq, float *scale_out, size_t cols) {
+  typedef unsigned short hx __attribute__((ext_vector_type(V)));
+  typedef signed char qx __attribute__((ext_vector_type(V)));
+  __shared__ uint32_t smax[kThreads / kWave];
+  const size_t row = blockIdx.x;
+  const unsigned short *xr = reinterpret_cast<const unsigned short *>(x) + row * ldx;
+  int8_t *qr = q + row * ldq;
+  const int t = threadIdx.x;
+  const uint32_t n = (uint32_t)cols, whole = n / V, tail = n % V;
+
+  // groups per lane that exist at all (uniform): the rest are skipped whole
+  const uint32_t used = (whole + kThreads - 1) / kThreads;
+  unsigned short v[EPL][V];
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    if ((uint32_t)j >= used) {
+#pragma unroll
+      for (int e = 0; e < V; ++e)
+        v[j][e] = 0;
+      continue;
+    }
+    const uint32_t g = (uint32_t)j * kThreads + t;
+    const uint32_t gs = (g < whole) ? g : 0u;
+    if constexpr (V == 1) {
+      v[j][0] = __builtin_nontemporal_load(xr + (whole ? gs : 0u));
+    } else {
+      // whole == 0 only if cols < V: then nothing of this load is used, and
+      // element 0 .. V-1 of the row may not all exist, so read one element
+      hx w;
+      if (whole) {
+        w = __builtin_nontemporal_load(reinterpret_cast<const hx *>(xr) + gs);
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; ++e)
+          w[e] = 0;
+      }
+#pragma unroll
+      for (int e = 0; e < V; ++e)
+        v[j][e] = w[e];
+    }
+  }
+  unsigned short tv = 0;
+  if (V > 1 && (uint32_t)t < tail)
+    tv = xr[whole * V + t];
+
+  uint32_t m = tv & 0x7fffu;
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    const bool in = (uint32_t)j * kThreads + t < whole;
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      v[j][e] = in ? v[j][e] : (unsigned short)0;
+      const uint32_t b = v[j][e] & 0x7fffu;
+      m = b > m ? b : m;
+    }
+  }
+  m = group_reduce<UMaxOp, kThreads / kWave>(m, smax);
+  const float amax = half_bits_to_float(m);
+  const float scale = amax / 127.0f;
+  if (t == 0)
+    scale_out[row] = scale;
+  const bool special = !(amax < INFINITY); // inf or NaN, uniform per row
+  const float div = (amax == 0.0f) ? 1.0f : scale;
+  const float rcp = 1.0f / div;
+  auto one = [&](unsigned short bits) -> int8_t {
+    const float f = half_bits_to_float(bits);
+    if (special)
+      return quant_special(f, scale);
+    return (int8_t)(pack4(quotient<false>(f, div, rcp), 0.0f, 0.0f, 0.0f) & 0xff);
+  };
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    const uint32_t g = (uint32_t)j * kThreads + t;
+    if (g >= whole)
+      continue;
+    if constexpr (V == 4) {
+      if (!special) {
+        const uint32_t o = pack4(quotient<false>(half_bits_to_float(v[j][0]), div, rcp),
+                                 quotient<false>(half_bits_to_float(v[j][1]), div, rcp),
+                                 quotient<false>(half_bits_to_float(v[j][2]), div, rcp),
+                                 quotient<false>(half_bits_to_float(v[j][3]), div, rcp));
+        __builtin_nontemporal_store(o, reinterpret_cast<uint32_t *>(qr) + g);
+        continue;
+      }
+    }
+    qx o;
+#pragma unroll
+    for (int e = 0; e < V; ++e)
+      o[e] = one(v[j][e]);
+    if constexpr (V == 1)
+      qr[g] = o[0];
+    else
+      *(reinterpret_cast<qx *>(qr) + g) = o;
+  }
+  if (V > 1 && (uint32_t)t < tail)
+    qr[whole * V + t] = one(tv);
+}
 } // namespace
 
 extern "C" __global__ __launch_bounds__(256) void hcamd_quant_f16_i8_p256_v1_nt(
@@ -273,6 +379,24 @@ HCAMD_QUANT(hcamd_quant_f16_i8_g128_v2_nt, 128, 2, false, true)
 HCAMD_QUANT(hcamd_quant_f16_i8_g256_v2, 256, 2, false, false)
 HCAMD_QUANT(hcamd_quant_f16_i8_g256_v4, 256, 4, false, false)
 HCAMD_QUANT(hcamd_quant_f16_i8_g256_v8, 256, 8, false, false)
+
+#define HCAMD_QUANT_SMALL(NAME, V, EPL)                                        \
+  extern "C" __global__ __launch_bounds__(256) void NAME(                      \
+      const _Float16 *x, size_t ldx, int8_t *q, size_t ldq, float *scale,      \
+      size_t rows, size_t cols) {                                              \
+    quantize_small<V, EPL>(x, ldx, q, ldq, scale, cols);                       \
+  }
+HCAMD_QUANT_SMALL(hcamd_quant_f16_i8_s4_e4, 4, 4)
+HCAMD_QUANT_SMALL(hcamd_quant_f16_i8_s4_e8, 4, 8)
+HCAMD_QUANT_SMALL(hcamd_quant_f16_i8_s4_e16, 4, 16)
+HCAMD_QUANT_SMALL(hcamd_quant_f16_i8_s4_e32, 4, 32)
+HCAMD_QUANT_SMALL(hcamd_quant_f16_i8_s2_e8, 2, 8)
+HCAMD_QUANT_SMALL(hcamd_quant_f16_i8_s2_e16, 2, 16)
+HCAMD_QUANT_SMALL(hcamd_quant_f16_i8_s2_e32, 2, 32)
+HCAMD_QUANT_SMALL(hcamd_quant_f16_i8_s2_e64, 2, 64)
+HCAMD_QUANT_SMALL(hcamd_quant_f16_i8_s1_e16, 1, 16)
+HCAMD_QUANT_SMALL(hcamd_quant_f16_i8_s1_e32, 1, 32)
+HCAMD_QUANT_SMALL(hcamd_quant_f16_i8_s1_e64, 1, 64)
 
 // Streaming kernel: one workgroup per row, two sweeps (absmax, quantise) with
 // element accesses and the compiler's IEEE division.  Any alignment, any

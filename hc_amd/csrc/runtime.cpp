@@ -1755,6 +1755,29 @@ int hcamdLaunchQuantizeF16I8(OlQueue q, const void *x, size_t ldx, int8_t *qout,
   const int variant = variantOf("quantize");
   const bool vec_ok = aligned16(x) && aligned16(qout) &&
                       (rows == 1 || (ldx % 8 == 0 && ldq % 16 == 0));
+  if (!vec_ok && variant != 1 && cols <= 32768) {
+    // rows that cannot be walked in 16-byte pieces: register-resident with the
+    // widest access the leading dimensions and base addresses allow
+    const uintptr_t ax = reinterpret_cast<uintptr_t>(x), aq = reinterpret_cast<uintptr_t>(qout);
+    const bool one_row = rows == 1;
+    const char *small = nullptr;
+    if (ax % 8 == 0 && aq % 4 == 0 && (one_row || (ldx % 4 == 0 && ldq % 4 == 0)))
+      small = cols <= 4096    ? "hcamd_quant_f16_i8_s4_e4"
+              : cols <= 8192  ? "hcamd_quant_f16_i8_s4_e8"
+              : cols <= 16384 ? "hcamd_quant_f16_i8_s4_e16"
+                              : "hcamd_quant_f16_i8_s4_e32";
+    else if (ax % 4 == 0 && aq % 2 == 0 && (one_row || (ldx % 2 == 0 && ldq % 2 == 0)))
+      small = cols <= 4096    ? "hcamd_quant_f16_i8_s2_e8"
+              : cols <= 8192  ? "hcamd_quant_f16_i8_s2_e16"
+              : cols <= 16384 ? "hcamd_quant_f16_i8_s2_e32"
+                              : "hcamd_quant_f16_i8_s2_e64";
+    else if (cols <= 16384)
+      small = cols <= 4096   ? "hcamd_quant_f16_i8_s1_e16"
+              : cols <= 8192 ? "hcamd_quant_f16_i8_s1_e32"
+                             : "hcamd_quant_f16_i8_s1_e64";
+    if (small)
+      return launch1d(queue, "quantize", small, rows, 256, args);
+  }
   if (!vec_ok || cols > 32768 || variant == 1)
     return launch1d(queue, "quantize", "hcamd_quant_f16_i8_stream", rows, 256,
                     args);

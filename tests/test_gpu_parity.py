@@ -877,6 +877,43 @@ def test_quantize_bit_exact(ctx, shape):
         assert_array_equal(q, q_c)
 
 
+@pytest.mark.parametrize("shape,ld,off,kernel", [
+    ((37, 4100), None, 0, "s4_e8"), ((19, 1000), None, 0, "s4_e4"), ((7, 4088), None, 0, "s4_e4"),
+    ((5, 20004), None, 0, "s4_e32"), ((9, 4094), None, 0, "s2_e8"), ((6, 10002), None, 0, "s2_e32"), ((6, 6002), None, 0, "s2_e16"), ((6, 6001), None, 0, "s1_e32"),
+    ((3, 30002), None, 0, "s2_e64"), ((11, 4095), None, 0, "s1_e16"), ((5, 15001), None, 0, "s1_e64"),
+    ((4, 1), None, 0, "s1_e16"), ((4, 2), None, 0, "s2_e8"), ((4, 3), None, 0, "s1_e16"),
+    ((8, 1003), 1004, 0, "s4_e4"), ((8, 1001), 1002, 0, "s2_e8"), ((8, 512), 520, 1, "s1_e16"),
+    ((8, 512), 520, 2, "s2_e8"), ((8, 512), 520, 4, "s4_e4"), ((3, 20001), None, 0, "stream")])
+def test_quantize_rows_that_are_not_16_byte_aligned(ctx, shape, ld, off, kernel):
+    """Column counts, leading dimensions and base addresses that rule out 16-byte
+    accesses: register-resident kernels with 8-, 4- or 2-byte loads, bit for bit
+    like the aligned ones, nothing written outside the rows."""
+    rows, cols = shape
+    ld = ld or cols
+    (x,) = cf.inputs_c4(shape)
+    x[0, ::7] = 0                                        # some exact zeros
+    if rows > 2:
+        x[1] = 0                                         # an all-zero row
+        x[2, cols // 2] = np.float16(np.inf) if cols > 1 else x[2, 0]
+    xp = np.full((rows * ld + off + 8,), 7, np.float16)
+    xv = xp[off:off + rows * ld].reshape(rows, ld)
+    xv[:, :cols] = x
+    dx = dev(xp)
+    dq = poisoned((rows * ld + off + 8,), np.int8)
+    ds = poisoned((rows,), np.float32)
+    rt.quantize_f16_i8(_View(dx, (rows, cols), off, (ld, 1)), _View(dq, (rows, cols), off, (ld, 1)), ds)
+    say("quantize unaligned", shape, ld, off, rt.last_kernel_name())
+    assert rt.last_kernel_name().endswith(kernel)
+    with np.errstate(all="ignore"):
+        q_np, s_np = cf.np_quantize(x)
+    raw = dq.to_host()
+    got = raw[off:off + rows * ld].reshape(rows, ld)
+    assert_array_equal(got[:, :cols], q_np)
+    assert (got[:, cols:].view(np.uint8) == 0xA5).all()
+    assert (raw[:off].view(np.uint8) == 0xA5).all() and (raw[off + rows * ld:].view(np.uint8) == 0xA5).all()
+    assert_array_equal(ds.to_host().view(np.uint32), s_np.view(np.uint32))
+
+
 def test_quantize_variants_and_strides(ctx):
     (x,) = cf.inputs_c4((301, 4096))
     q_np, s_np = cf.np_quantize(x)
