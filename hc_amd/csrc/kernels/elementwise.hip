@@ -150,6 +150,48 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_add_f32_scalar(
     c[i] = a[i] + b[i];
 }
 
+// Windows of larger arrays (leading dimension != columns): a row is walked in
+// groups of V elements, V = 8, 4 or 2 as the common alignment of the four
+// arrays' rows allows (16-, 8- or 4-byte accesses), the cols % V elements at
+// the end of the row one by one.  blockIdx.y walks rows, x the groups of a row.
+template <int V>
+__device__ __forceinline__ void fma_rows(const _Float16 *a, size_t lda, const _Float16 *b,
+                                         size_t ldb, const _Float16 *c, size_t ldc,
+                                         _Float16 *d, size_t ldd, size_t cols) {
+  typedef _Float16 hv __attribute__((ext_vector_type(V)));
+  const size_t row = blockIdx.y;
+  const size_t g = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t whole = cols / V;
+  const _Float16 *ar = a + row * lda, *br = b + row * ldb, *cr = c + row * ldc;
+  _Float16 *dr = d + row * ldd;
+  if (g < whole) {
+    const hv x = __builtin_nontemporal_load(reinterpret_cast<const hv *>(ar) + g);
+    const hv y = __builtin_nontemporal_load(reinterpret_cast<const hv *>(br) + g);
+    const hv z = __builtin_nontemporal_load(reinterpret_cast<const hv *>(cr) + g);
+    hv r;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      _Float16 e[3] = {x[i], y[i], z[i]};
+      r[i] = FmaF16::apply1(e);
+    }
+    __builtin_nontemporal_store(r, reinterpret_cast<hv *>(dr) + g);
+  } else if (g - whole < cols % V) {
+    const size_t col = whole * V + (g - whole);
+    _Float16 e[3] = {ar[col], br[col], cr[col]};
+    dr[col] = FmaF16::apply1(e);
+  }
+}
+#define HCAMD_FMA_ROWS(NAME, V)                                                \
+  extern "C" __global__ __launch_bounds__(256) void NAME(                      \
+      const _Float16 *a, size_t lda, const _Float16 *b, size_t ldb,            \
+      const _Float16 *c, size_t ldc, _Float16 *d, size_t ldd, size_t rows,     \
+      size_t cols) {                                                           \
+    fma_rows<V>(a, lda, b, ldb, c, ldc, d, ldd, cols);                         \
+  }
+HCAMD_FMA_ROWS(hcamd_fma_f16_rows_v8, 8)
+HCAMD_FMA_ROWS(hcamd_fma_f16_rows_v4, 4)
+HCAMD_FMA_ROWS(hcamd_fma_f16_rows_v2, 2)
+
 extern "C" __global__ __launch_bounds__(256) void hcamd_fma_f16_2d(
     const _Float16 *a, size_t lda, const _Float16 *b, size_t ldb,
     const _Float16 *c, size_t ldc, _Float16 *d, size_t ldd, size_t rows,

@@ -739,6 +739,25 @@ int hcamdLaunchCopy2D(OlQueue q, size_t elemSize, const void *src,
     return launch1d(queue, "copy", names[v], ceilDiv(words, 256 * (size_t)vpt[v]),
                     256, args);
   }
+  // A window of rows that are contiguous inside: use the widest element both
+  // arrays' rows are aligned for (an int32 window with even extents and strides
+  // is an int64 window of half the width, and so on up to 16 bytes).
+  if (ss1 == 1 && ds1 == 1 && variant != 9) {
+    while (elemSize < 16 && cols % 2 == 0 &&
+           (rows == 1 || (ss0 % 2 == 0 && ds0 % 2 == 0)) &&
+           (reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) %
+                   (2 * elemSize) == 0) {
+      elemSize *= 2;
+      cols /= 2;
+      ss0 /= 2;
+      ds0 /= 2;
+    }
+    suffix = elemSize == 1   ? "b1"
+             : elemSize == 2 ? "b2"
+             : elemSize == 4 ? "b4"
+             : elemSize == 8 ? "b8"
+                             : "b16";
+  }
   const std::string name = std::string("hcamd_copy2d_") + suffix;
   Kernel *k = builtinKernel(dev, "copy", name.c_str());
   if (!k)
@@ -860,9 +879,23 @@ int hcamdLaunchFmaF16(OlQueue q, const void *a, size_t lda, const void *b,
     return launch1d(queue, "elementwise", names[v],
                     ceilDiv(words, 256 * (size_t)vpt[v]), 256, args);
   }
-  Kernel *k = builtinKernel(dev, "elementwise", "hcamd_fma_f16_2d");
+  // windows: the widest access all four arrays' rows are aligned for
+  size_t width = 1; // elements per access
+  if (variant != 7) {
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) |
+                           reinterpret_cast<uintptr_t>(c) | reinterpret_cast<uintptr_t>(d) |
+                           (rows > 1 ? (lda | ldb | ldc | ldd) * 2 : 0);
+    width = bits % 16 == 0 ? 8 : bits % 8 == 0 ? 4 : bits % 4 == 0 ? 2 : 1;
+  }
+  Kernel *k = builtinKernel(dev, "elementwise",
+                            width == 8   ? "hcamd_fma_f16_rows_v8"
+                            : width == 4 ? "hcamd_fma_f16_rows_v4"
+                            : width == 2 ? "hcamd_fma_f16_rows_v2"
+                                         : "hcamd_fma_f16_2d");
   if (!k)
     return 1;
+  // lanes per row: one per group of `width` elements plus one per leftover
+  const size_t lanes = cols / width + cols % width;
   for (size_t r0 = 0; r0 < rows; r0 += 65535) {
     size_t nr = std::min(rows - r0, (size_t)65535);
     const char *pa = static_cast<const char *>(a) + r0 * lda * 2;
@@ -870,7 +903,7 @@ int hcamdLaunchFmaF16(OlQueue q, const void *a, size_t lda, const void *b,
     const char *pc = static_cast<const char *>(c) + r0 * ldc * 2;
     char *pd = static_cast<char *>(d) + r0 * ldd * 2;
     void *args[] = {&pa, &lda, &pb, &ldb, &pc, &ldc, &pd, &ldd, &nr, &cols};
-    const size_t grid[3] = {ceilDiv(cols, 256), nr, 1};
+    const size_t grid[3] = {ceilDiv(lanes, 256), nr, 1};
     const size_t block[3] = {256, 1, 1};
     if (launch(queue, k, grid, block, args, 0))
       return 1;

@@ -193,6 +193,23 @@ def test_copy_window_smaller_than_destination_leaves_rest_untouched(ctx, itemsiz
     assert_array_equal(small.to_host(), big.to_host()[:5, :9])
 
 
+@pytest.mark.parametrize("cols,lds,ldd,off,kernel", [
+    (100, 132, 136, 0, "b16"), (100, 132, 136, 2, "b8"), (100, 132, 136, 1, "b4"),
+    (102, 132, 136, 0, "b8"), (100, 130, 136, 0, "b8"), (101, 132, 136, 0, "b4"),
+    (128, 129, 128, 0, "b4")])
+def test_copy_windows_use_the_widest_element_their_rows_allow(ctx, cols, lds, ldd, off, kernel):
+    rows = 37
+    rng = np.random.default_rng(cols + off)
+    a = rng.integers(0, 1 << 30, (rows * lds + 8,)).astype(np.int32)
+    src, dst = dev(a), poisoned((rows * ldd + 8,), np.int32)
+    rt.copy2d(_View(src, (rows, cols), off, (lds, 1)), _View(dst, (rows, cols), off, (ldd, 1)))
+    assert rt.last_kernel_name() == "hcamd_copy2d_" + kernel
+    want = np.full((rows * ldd + 8,), poison_value(np.int32), np.int32)
+    want[off:off + rows * ldd].reshape(rows, ldd)[:, :cols] = \
+        a[off:off + rows * lds].reshape(rows, lds)[:, :cols]
+    assert_array_equal(dst.to_host(), want)
+
+
 def test_copy_large_flat_all_variants(ctx):
     a = np.random.default_rng(1).integers(0, 2 ** 31, 4_000_037, dtype=np.int32)[None, :]
     src = dev(a)
@@ -275,18 +292,28 @@ def test_fma_bit_exact_all_variants(ctx, shape):
         assert (out[want.size:].view(np.uint16) == 0xA5A5).all(), (v, rt.last_kernel_name())
 
 
-def test_fma_strided_rows(ctx):
-    rows, cols, ld = 33, 1000, 1024
-    a, b, c = cf.inputs_c2((rows, ld))
-    da, db, dc = dev(a), dev(b), dev(c)
-    dd = poisoned((rows, ld), np.float16)
-    views = [_View(x, (rows, cols), 0, (ld, 1)) for x in (da, db, dc, dd)]
+@pytest.mark.parametrize("cols,ld,off,kernel", [
+    (1000, 1024, 0, "rows_v8"), (1003, 1024, 0, "rows_v8"), (1003, 1024, 8, "rows_v8"),
+    (1001, 1028, 0, "rows_v4"), (1001, 1028, 4, "rows_v4"), (999, 1002, 0, "rows_v2"),
+    (999, 1002, 2, "rows_v2"), (1000, 1001, 0, "2d"), (1000, 1024, 1, "2d"), (5, 1024, 0, "rows_v8")])
+def test_fma_strided_rows(ctx, cols, ld, off, kernel):
+    """Windows of larger arrays: the widest access the rows are aligned for, the
+    leftover elements of a row one by one, nothing written outside the window."""
+    rows = 33
+    a, b, c = cf.inputs_c2((rows, ld + 1))
+    flat = [x.ravel()[:rows * ld + 16].copy() for x in (a, b, c)]
+    da, db, dc = (dev(x) for x in flat)
+    dd = poisoned((rows * ld + 16,), np.float16)
+    views = [_View(x, (rows, cols), off, (ld, 1)) for x in (da, db, dc, dd)]
     rt.fma_f16(*views)
-    assert rt.last_kernel_name() == "hcamd_fma_f16_2d"
-    out = dd.to_host()
-    assert_array_equal(out[:, :cols].view(np.uint16),
-                       cf.np_fma_f16(a[:, :cols], b[:, :cols], c[:, :cols]).view(np.uint16))
-    assert (out[:, cols:].view(np.uint16) == 0xA5A5).all()
+    assert rt.last_kernel_name() == "hcamd_fma_f16_" + kernel
+    win = [x[off:off + rows * ld].reshape(rows, ld)[:, :cols] for x in flat]
+    raw = dd.to_host()
+    out = raw[off:off + rows * ld].reshape(rows, ld)
+    assert_array_equal(out[:, :cols].view(np.uint16), cf.np_fma_f16(*win).view(np.uint16))
+    assert (out[:-1, cols:].view(np.uint16) == 0xA5A5).all()
+    assert (raw[:off].view(np.uint16) == 0xA5A5).all()
+    assert (raw[off + (rows - 1) * ld + cols:].view(np.uint16) == 0xA5A5).all()
 
 
 def test_fma_special_values(ctx):
