@@ -470,34 +470,147 @@ __device__ __forceinline__ void map_flat(const MapArgs &a, const uint32_t n_in) 
     finish_sum<kThreads>(acc, static_cast<float *>(a.out));
 }
 
-// Strided form: blockIdx.y walks rows, x walks the columns of a row in runs of
-// 256 * 8; lane t takes columns t, t + 256, ... so a wave reads consecutive
-// elements.
+// Strided form: a work item is a run of 256 * 8 columns of one row; lane t takes
+// columns t, t + 256, ... of the run, so a wave reads consecutive elements.  The
+// map launches one workgroup per item (blockIdx.y = row, x = run); the reduction
+// launches a grid capped by the host whose workgroups stride over the items, row
+// after row, and ends in one atomic addition per workgroup.
 template <bool SUM>
 __device__ __forceinline__ void map_strided(const MapArgs &a, const uint32_t n_in) {
-  const size_t row = blockIdx.y;
-  const size_t col0 = (size_t)blockIdx.x * (kThreads * kN) + threadIdx.x;
-  Raw raw;
-  gather(a, n_in, raw, [&](int i, int e, size_t &off) {
-    const size_t col = col0 + (size_t)e * kThreads;
-    off = row * a.ld[i] + col;
-    return col < a.cols;
-  });
-  Stack r;
-  run_program(a, raw, 0, r);
   float acc = 0.0f;
+  auto item = [&](const size_t row, const size_t run) {
+    const size_t col0 = run * (kThreads * kN) + threadIdx.x;
+    Raw raw;
+    gather(a, n_in, raw, [&](int i, int e, size_t &off) {
+      const size_t col = col0 + (size_t)e * kThreads;
+      off = row * a.ld[i] + col;
+      return col < a.cols;
+    });
+    Stack r;
+    run_program(a, raw, 0, r);
 #pragma unroll
-  for (int e = 0; e < kN; ++e) {
-    const size_t col = col0 + (size_t)e * kThreads;
-    if (col < a.cols) {
-      if constexpr (SUM)
-        acc += r.st[0][e];
-      else
-        store_elem(a.out, (a.f16_mask >> 8) & 1, row * a.ldo + col, r.st[0][e]);
+    for (int e = 0; e < kN; ++e) {
+      const size_t col = col0 + (size_t)e * kThreads;
+      if (col < a.cols) {
+        if constexpr (SUM)
+          acc += r.st[0][e];
+        else
+          store_elem(a.out, (a.f16_mask >> 8) & 1, row * a.ldo + col, r.st[0][e]);
+      }
     }
-  }
-  if constexpr (SUM)
+  };
+  if constexpr (SUM) {
+    const size_t runs = (a.cols + kThreads * kN - 1) / (kThreads * kN);
+    const size_t items = a.rows * runs;
+    for (size_t i = blockIdx.x; i < items; i += gridDim.x)
+      item(i / runs, i % runs);
     finish_sum<kThreads>(acc, static_cast<float *>(a.out));
+  } else {
+    item(blockIdx.y, blockIdx.x);
+  }
+}
+
+// Row form for windows whose rows start on 16-byte boundaries: the work items
+// are the chunks of all rows, numbered row after row (a row has cols / 8 whole
+// chunks and, when cols is not a multiple of 8, one short chunk at its end), and
+// lane t of workgroup g takes item g * T + t, then strides by the grid.  Whole
+// chunks move with 16-byte accesses like the flat form; a short chunk is read
+// element by element (every load issued, from the row's first element where the
+// column is past the end, and zeroed afterwards) and packed the way a whole
+// chunk arrives, so one run of the interpreter serves both.  The reduction runs
+// 1024-lane workgroups on a grid capped by the host, so that it ends in a few
+// hundred atomic additions however many rows there are.
+template <bool SUM>
+__device__ __forceinline__ void map_rows(const MapArgs &a, const uint32_t n_in) {
+  constexpr int T = SUM ? 1024 : 256;
+  const uint32_t whole = (uint32_t)(a.cols / 8);
+  const uint32_t rem = (uint32_t)(a.cols % 8);
+  const uint32_t per_row = whole + (rem ? 1u : 0u);
+  const uint32_t items = (uint32_t)a.rows * per_row;
+  const bool out_f16 = (a.f16_mask >> 8) & 1;
+  float acc = 0.0f;
+  // every lane makes the same number of passes: the interpreter's control flow
+  // stays uniform, passes past the end are predicated off
+  auto pass = [&](const uint32_t item) {
+    Raw raw;
+    Stack r;
+    const bool live = item < items;
+    const uint32_t row = live ? item / per_row : 0;
+    const uint32_t c = live ? item - row * per_row : 0;
+    const bool shortc = live && c == whole; // only with rem != 0
+    // whole chunks: every lane loads (idle and short-chunk lanes the row's
+    // first chunk), so that no load sits in a divergent branch
+    const uint32_t cv = (live && !shortc) ? c : 0;
+    if (whole) {
+#pragma unroll
+      for (int i = 0; i < kMaxIn; ++i)
+        if (i < (int)n_in) {
+          const bool f16 = (a.f16_mask >> i) & 1;
+          const char *base = static_cast<const char *>(a.in[i]) +
+                             (size_t)row * a.ld[i] * (f16 ? 2 : 4);
+          const u32x4 *q = reinterpret_cast<const u32x4 *>(base) + (f16 ? cv : 2 * cv);
+          raw.w[i][0] = ldg<true>(q);
+          if (!f16)
+            raw.w[i][1] = ldg<true>(q + 1);
+        }
+    }
+    if (shortc) {
+#pragma unroll
+      for (int i = 0; i < kMaxIn; ++i)
+        if (i < (int)n_in) {
+          const bool f16 = (a.f16_mask >> i) & 1;
+          const char *base = static_cast<const char *>(a.in[i]) +
+                             (size_t)row * a.ld[i] * (f16 ? 2 : 4);
+          uint32_t v[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const size_t at = (uint32_t)e < rem ? (size_t)whole * 8 + e : 0;
+            v[e] = f16 ? (uint32_t) reinterpret_cast<const uint16_t *>(base)[at]
+                       : reinterpret_cast<const uint32_t *>(base)[at];
+          }
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            v[e] = (uint32_t)e < rem ? v[e] : 0u;
+          if (f16) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              raw.w[i][0][e] = v[2 * e] | (v[2 * e + 1] << 16);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              raw.w[i][e / 4][e % 4] = v[e];
+          }
+        }
+    }
+    run_program(a, raw, a.f16_mask, r);
+    if (live) {
+      if constexpr (SUM) {
+#pragma unroll
+        for (int e = 0; e < kN; ++e)
+          acc += (!shortc || (uint32_t)e < rem) ? r.st[0][e] : 0.0f;
+      } else {
+        char *orow = static_cast<char *>(a.out) + (size_t)row * a.ldo * (out_f16 ? 2 : 4);
+        if (!shortc) {
+          store_chunk(orow, out_f16, c, r.st[0]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if ((uint32_t)e < rem)
+              store_elem(orow, out_f16, (size_t)whole * 8 + e, r.st[0][e]);
+        }
+      }
+    }
+  };
+  if constexpr (SUM) {
+    const uint32_t stride = gridDim.x * T;
+    const uint32_t passes = (items + stride - 1) / stride;
+    uint32_t item = blockIdx.x * T + threadIdx.x;
+    for (uint32_t p = 0; p < passes; ++p, item += stride)
+      pass(item);
+    finish_sum<T>(acc, static_cast<float *>(a.out));
+  } else {
+    pass(blockIdx.x * T + threadIdx.x); // the host launches one lane per item
+  }
 }
 } // namespace
 
@@ -611,11 +724,23 @@ __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcam
   }
 }
 
-extern "C" __global__ __launch_bounds__(256) void hcamd_map_strided(
+extern "C" __global__ __launch_bounds__(256)
+__attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcamd_map_strided(
     const MapArgs a, const uint32_t n_in) {
   map_strided<false>(a, n_in);
 }
-extern "C" __global__ __launch_bounds__(256) void hcamd_map_sum_strided(
+extern "C" __global__ __launch_bounds__(256)
+__attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcamd_map_sum_strided(
     const MapArgs a, const uint32_t n_in) {
   map_strided<true>(a, n_in);
+}
+extern "C" __global__ __launch_bounds__(256)
+__attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcamd_map_rows(
+    const MapArgs a, const uint32_t n_in) {
+  map_rows<false>(a, n_in);
+}
+extern "C" __global__ __launch_bounds__(1024)
+__attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcamd_map_sum_rows(
+    const MapArgs a, const uint32_t n_in) {
+  map_rows<true>(a, n_in);
 }

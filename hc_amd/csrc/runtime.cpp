@@ -1096,12 +1096,37 @@ int launchMap(OlQueue q, bool sum, const HcamdMapInstr *prog, size_t nInstr,
       groups = std::min(groups, (size_t)computeUnitsOf(dev));
     return launch1d(queue, "map", name, groups, threads, args);
   }
+  a.cols = cols;
+  // Windows whose rows all start on 16-byte boundaries: 16-byte accesses along
+  // the rows (variant 1 of "map" keeps the element-wise kernel below).
+  bool rowsAligned = variantOf("map") != 1 &&
+                     (sum || (aligned16(out) && (ldo * (outType == HCAMD_F16 ? 2 : 4)) % 16 == 0));
+  for (size_t i = 0; i < nInputs && rowsAligned; ++i)
+    rowsAligned = aligned16(inputs[i]) &&
+                  (inputLd[i] * (inputTypes[i] == HCAMD_F16 ? 2 : 4)) % 16 == 0;
+  const size_t perRow = cols / 8 + (cols % 8 ? 1 : 0);
+  if (rowsAligned && rows <= ((size_t)1 << 30) / perRow) {
+    a.rows = rows;
+    const size_t items = rows * perRow;
+    const size_t threads = sum ? 1024 : 256;
+    size_t groups = ceilDiv(items, threads);
+    if (sum)
+      groups = std::min(groups, (size_t)computeUnitsOf(dev));
+    return launch1d(queue, "map", sum ? "hcamd_map_sum_rows" : "hcamd_map_rows", groups,
+                    threads, args);
+  }
   Kernel *k = builtinKernel(dev, "map",
                             sum ? "hcamd_map_sum_strided" : "hcamd_map_strided");
   if (!k)
     return 1;
-  a.cols = cols;
   const size_t esz_out = outType == HCAMD_F16 ? 2 : 4;
+  if (sum) {
+    a.rows = rows;
+    const size_t groups = std::min(rows * ceilDiv(cols, kPerGroup),
+                                   (size_t)computeUnitsOf(dev) * 4);
+    const size_t grid[3] = {groups, 1, 1}, block[3] = {256, 1, 1};
+    return launch(queue, k, grid, block, args, 0);
+  }
   for (size_t r0 = 0; r0 < rows; r0 += 65535) {
     const size_t nr = std::min(rows - r0, (size_t)65535);
     a.rows = nr;

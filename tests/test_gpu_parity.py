@@ -574,6 +574,63 @@ def test_map_window_of_larger_arrays_leaves_the_rest_untouched(ctx):
     assert (got[:, cols:].view(np.uint16) == p.view(np.uint16)).all()
 
 
+@pytest.mark.parametrize("cols", [1, 5, 8, 9, 1031, 1032, 2049])
+@pytest.mark.parametrize("types", [(np.float16,) * 4, (np.float32,) * 4,
+                                   (np.float16, np.float32, np.float16, np.float32)])
+def test_map_windows_with_aligned_rows_take_16_byte_accesses(ctx, cols, types):
+    """Rows that start on 16-byte boundaries: the row kernel, bit for bit the
+    element-wise kernel's results, nothing written outside the window, nothing
+    read from outside it (the surroundings hold NaN)."""
+    rows, ld = 37, 2064
+    rng = np.random.default_rng(cols)
+    ins = [rng.standard_normal((rows, cols)).astype(t) for t in types[:3]]
+    big = [np.full((rows + 2, ld), np.nan, t) for t in types[:3]]
+    for dst, src in zip(big, ins):
+        dst[1:rows + 1, 8:8 + cols] = src
+    dbig = [dev(x) for x in big]
+    views = [_View(x, (rows, cols), ld + 8, (ld, 1)) for x in dbig]
+    got = {}
+    for variant in (0, 1):
+        rt.set_variant("map", variant)
+        out = poisoned((rows + 2, ld), types[3])
+        rt.plan_map(FMA_PROGRAM, views, _View(out, (rows, cols), ld + 8, (ld, 1))).launch(sync=True)
+        say("map window", cols, [np.dtype(t).name for t in types], rt.last_kernel_name())
+        assert rt.last_kernel_name() == ("hcamd_map_rows" if variant == 0 else "hcamd_map_strided")
+        got[variant] = out.to_host()
+    rt.set_variant("map", 0)
+    assert_array_equal(got[0].view(np.uint8), got[1].view(np.uint8))
+    want = (ins[0].astype(np.float32) * ins[1].astype(np.float32)
+            + ins[2].astype(np.float32)).astype(types[3])
+    assert_same_floats(np.ascontiguousarray(got[0][1:rows + 1, 8:8 + cols]), want)
+    mask = np.ones((rows + 2, ld), bool)
+    mask[1:rows + 1, 8:8 + cols] = False
+    p = poison_value(types[3])
+    u = {2: np.uint16, 4: np.uint32}[np.dtype(types[3]).itemsize]
+    assert (got[0].view(u)[mask] == p.view(u)).all()
+
+
+@pytest.mark.parametrize("rows,cols", [(2, 3), (37, 1031), (5000, 40), (3, 70_001)])
+def test_map_sum_over_windows_with_aligned_rows(ctx, rows, cols):
+    ld = (cols + 8 + 7) // 8 * 8
+    rng = np.random.default_rng(rows)
+    a = rng.standard_normal((rows, cols)).astype(np.float16)
+    b = rng.standard_normal((rows, cols)).astype(np.float32)
+    big_a, big_b = np.full((rows, ld), np.nan, np.float16), np.full((rows, ld), np.nan, np.float32)
+    big_a[:, 8:8 + cols], big_b[:, 4:4 + cols] = a, b
+    terms = (a.astype(np.float32) * b).astype(np.float64)
+    bound = 64 * 2.0 ** -24 * np.abs(terms).sum()
+    da, db = dev(big_a), dev(big_b)
+    views = [_View(da, (rows, cols), 8, (ld, 1)), _View(db, (rows, cols), 4, (ld, 1))]
+    for variant, name in ((0, "hcamd_map_sum_rows"), (1, "hcamd_map_sum_strided")):
+        rt.set_variant("map", variant)
+        cell = dev(np.array([3.0, 0.0], np.float32))
+        rt.plan_map_sum([I("in", 0), I("mul_in", 1)], views, cell).launch(sync=True)
+        assert rt.last_kernel_name() == name
+        got = cell.to_host()
+        assert got[1] == 0.0 and abs(float(got[0]) - 3.0 - terms.sum()) <= bound + 3.0 * 2.0 ** -23
+    rt.set_variant("map", 0)
+
+
 def test_map_every_operation_against_numpy(ctx):
     rng = np.random.default_rng(11)
     n = 50_001
