@@ -744,3 +744,265 @@ __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcam
     const MapArgs a, const uint32_t n_in) {
   map_rows<true>(a, n_in);
 }
+
+// ---- row programs ---------------------------------------------------------------
+// Bodies that mix elementwise arithmetic with reductions along the rows of a
+// tile (normalisations, softmax-like expressions, row sums): a list of stages,
+// each a postfix program of the interpreter above, run row by row.
+//
+//   SUM / MAX / MIN  the program's value at every element of the row is folded
+//                    into row scalar `dst`
+//   SCALAR           the program reads row scalars only; its value becomes row
+//                    scalar `dst`
+//   STORE            the program's value at every element is stored to the
+//                    output tile
+//   STORE_COL        as SCALAR, stored to out[row * ldo]
+//
+// Row scalars live in scalar registers (a row belongs to one wave or to the
+// four waves of one workgroup).  A program reaches them through the RED
+// opcodes, which are rewritten on the fly into the immediate forms of the
+// interpreter with the scalar as the immediate, so the interpreter itself does
+// not know about them.  Column operands (one value per row) are row scalars
+// that are loaded instead of computed.
+//
+// LPR lanes share a row (256: one row per workgroup; 64: one row per wave,
+// four rows per workgroup).  A lane's chunks of the row are LPR chunks apart.
+// Operands that later stages read again can be kept in LDS as they were
+// loaded; every lane reads back only what it wrote itself, so the copy needs no
+// barrier.  Reductions add in a fixed order for a given shape: results are
+// reproducible from run to run.
+namespace {
+constexpr int kMaxRed = 8;
+constexpr int kMaxStages = 8;
+constexpr int kRowProg = 64;
+enum : uint32_t {
+  OP_RED = 35,     // push row scalar `arg`
+  OP_ADD_RED = 36, // top = top op row scalar `arg`, in the order of OP_ADD_IN..
+  OP_RDIV_RED = 43,
+};
+enum : uint32_t { ST_SUM = 0, ST_MAX = 1, ST_MIN = 2, ST_SCALAR = 3, ST_STORE = 4, ST_STORE_COL = 5 };
+
+struct Stage {
+  uint16_t begin, end; // instructions [begin, end)
+  uint8_t kind, dst;
+  uint8_t load_mask; // operands read from memory in this stage
+  uint8_t lds_mask;  // operands read from their LDS copy
+  uint8_t keep_mask; // operands copied to LDS after loading
+  uint8_t pad[3];
+};
+
+struct RowArgs {
+  const void *in[kMaxIn];
+  const void *col[kMaxIn]; // column operands: row scalars 0 .. n_col-1
+  void *out;
+  size_t ld[kMaxIn]; // row stride in elements (0: the same vector for every row)
+  size_t ldo;
+  size_t rows, cols;
+  uint32_t f16_mask; // bit i: operand i is fp16; bit 8: the output; bit 16+k: column k
+  uint32_t vec_mask; // bit i: rows of operand i start on 16-byte boundaries; bit 8: the output
+  uint32_t keep_l2;  // bit i: operand i is read again from memory by a later stage
+  uint32_t n_col, n_stages, passes;
+  uint8_t cache_slot[kMaxIn];
+  Stage stage[kMaxStages];
+  Instr prog[kRowProg];
+};
+
+struct NanMaxOp {
+  using T = float;
+  static __device__ __forceinline__ float identity() { return -INFINITY; }
+  static __device__ __forceinline__ float apply(float a, float b) { return nan_max(a, b); }
+};
+struct NanMinOp {
+  using T = float;
+  static __device__ __forceinline__ float identity() { return INFINITY; }
+  static __device__ __forceinline__ float apply(float a, float b) { return nan_min(a, b); }
+};
+
+// Row scalars are kept in LDS, one copy per wave (indexed registers would end up
+// in scratch memory); every lane of a wave writes the same value and reads it
+// back through readfirstlane, so no barrier is involved.
+struct Reds {
+  float *v; // this wave's kMaxRed cells
+};
+__device__ __forceinline__ float uniform(float x) {
+  return __builtin_bit_cast(float,
+                            __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
+}
+
+__device__ __forceinline__ float red_get(const Reds &r, uint32_t k) {
+  return uniform(r.v[k & (kMaxRed - 1)]);
+}
+__device__ __forceinline__ void red_set(Reds &r, uint32_t k, float x) {
+  r.v[k & (kMaxRed - 1)] = x;
+}
+
+__device__ __forceinline__ void run_stage(const RowArgs &a, uint32_t begin, uint32_t end,
+                                          const Raw &raw, const Reds &red, Stack &r) {
+  int sp = 0;
+  Instr next = a.prog[begin & (kRowProg - 1)];
+  for (uint32_t pc = begin; pc < end; ++pc) {
+    const Instr cur = next;
+    next = a.prog[(pc + 1) & (kRowProg - 1)];
+    uint32_t op = cur.op;
+    const uint32_t arg = cur.arg;
+    float imm = cur.imm;
+    if (op >= OP_RED) {
+      imm = red_get(red, arg);
+      op = op == OP_RED ? (uint32_t)OP_CONST : op - OP_ADD_RED + OP_ADDI;
+    }
+    switch (sp) {
+    case 0: sp = step<0>(r, raw, a.f16_mask, op, arg, imm); break;
+    case 1: sp = step<1>(r, raw, a.f16_mask, op, arg, imm); break;
+    case 2: sp = step<2>(r, raw, a.f16_mask, op, arg, imm); break;
+    case 3: sp = step<3>(r, raw, a.f16_mask, op, arg, imm); break;
+    default: sp = step<4>(r, raw, a.f16_mask, op, arg, imm); break;
+    }
+  }
+}
+
+template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a) {
+  extern __shared__ u32x4 row_cache[];
+  __shared__ float slots[2][kThreads / kWave];
+  const uint32_t t = threadIdx.x, lane = t % LPR;
+  const size_t row_at = (size_t)blockIdx.x * (kThreads / LPR) + t / LPR;
+  const bool row_live = row_at < a.rows;
+  const size_t row = row_live ? row_at : 0; // idle lanes compute on row 0 and store nothing
+  const uint32_t whole = (uint32_t)(a.cols / 8), rem = (uint32_t)(a.cols % 8);
+  const uint32_t per_row = whole + (rem ? 1u : 0u);
+  const bool out_f16 = (a.f16_mask >> 8) & 1;
+  __shared__ float red_cells[kThreads / kWave][kMaxRed];
+  Reds red{red_cells[t / kWave]};
+#pragma unroll
+  for (int k = 0; k < kMaxIn; ++k)
+    if (k < (int)a.n_col)
+      red_set(red, k, uniform(load_elem(a.col[k], (a.f16_mask >> (16 + k)) & 1, row)));
+  uint32_t parity = 0;
+#pragma nounroll
+  for (uint32_t s = 0; s < a.n_stages; ++s) {
+    const Stage st = a.stage[s];
+    const uint32_t kind = st.kind;
+    const bool per_element = kind <= ST_MIN || kind == ST_STORE;
+    const uint32_t n_pass = per_element ? a.passes : 1;
+    float acc = kind == ST_MAX ? -INFINITY : kind == ST_MIN ? INFINITY : 0.0f;
+    Raw raw;
+    Stack r;
+#pragma nounroll
+    for (uint32_t p = 0; p < n_pass; ++p) {
+      const uint32_t c_at = p * LPR + lane;
+      const bool live = per_element && row_live && c_at < per_row;
+      const uint32_t c = live ? c_at : 0;
+      const bool shortc = live && c == whole;
+      const uint32_t n_valid = !live ? 0u : shortc ? rem : 8u;
+      if (per_element) {
+#pragma unroll
+        for (int i = 0; i < kMaxIn; ++i) {
+          const bool f16 = (a.f16_mask >> i) & 1;
+          const uint32_t slot = ((a.cache_slot[i] * a.passes + p) * 2) * kThreads + t;
+          if ((st.lds_mask >> i) & 1) {
+            raw.w[i][0] = row_cache[slot];
+            if (!f16)
+              raw.w[i][1] = row_cache[slot + kThreads];
+          } else if ((st.load_mask >> i) & 1) {
+            const char *base = static_cast<const char *>(a.in[i]) +
+                               row * a.ld[i] * (f16 ? 2 : 4);
+            const bool vec = (a.vec_mask >> i) & 1; // implies whole >= 1
+            if (vec) {
+              const uint32_t cv = shortc ? 0 : c;
+              const u32x4 *q = reinterpret_cast<const u32x4 *>(base) + (f16 ? cv : 2 * cv);
+              if ((a.keep_l2 >> i) & 1) {
+                raw.w[i][0] = ldg<false>(q);
+                if (!f16)
+                  raw.w[i][1] = ldg<false>(q + 1);
+              } else {
+                raw.w[i][0] = ldg<true>(q);
+                if (!f16)
+                  raw.w[i][1] = ldg<true>(q + 1);
+              }
+            }
+            if (!vec || shortc) {
+              // element by element; every load is issued (from the row's first
+              // element where the column is past the end) and zeroed afterwards
+              uint32_t v[8];
+#pragma unroll
+              for (int e = 0; e < 8; ++e) {
+                const size_t at = (uint32_t)e < n_valid ? (size_t)c * 8 + e : 0;
+                v[e] = f16 ? (uint32_t) reinterpret_cast<const uint16_t *>(base)[at]
+                           : reinterpret_cast<const uint32_t *>(base)[at];
+              }
+#pragma unroll
+              for (int e = 0; e < 8; ++e)
+                v[e] = (uint32_t)e < n_valid ? v[e] : 0u;
+              if (f16) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                  raw.w[i][0][e] = v[2 * e] | (v[2 * e + 1] << 16);
+              } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                  raw.w[i][e / 4][e % 4] = v[e];
+              }
+            }
+            if ((st.keep_mask >> i) & 1) {
+              row_cache[slot] = raw.w[i][0];
+              if (!f16)
+                row_cache[slot + kThreads] = raw.w[i][1];
+            }
+          }
+        }
+      }
+      run_stage(a, st.begin, st.end, raw, red, r);
+      if (kind == ST_STORE) {
+        char *orow = static_cast<char *>(a.out) + row * a.ldo * (out_f16 ? 2 : 4);
+        if (((a.vec_mask >> 8) & 1) && n_valid == 8) {
+          store_chunk(orow, out_f16, c, r.st[0]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if ((uint32_t)e < n_valid)
+              store_elem(orow, out_f16, (size_t)c * 8 + e, r.st[0][e]);
+        }
+      } else if (kind == ST_SUM) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          acc += (uint32_t)e < n_valid ? r.st[0][e] : 0.0f;
+      } else if (kind == ST_MAX) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          acc = (uint32_t)e < n_valid ? nan_max(acc, r.st[0][e]) : acc;
+      } else if (kind == ST_MIN) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          acc = (uint32_t)e < n_valid ? nan_min(acc, r.st[0][e]) : acc;
+      }
+    }
+    if (kind <= ST_MIN) {
+      constexpr int W = LPR / kWave;
+      float total;
+      if (kind == ST_SUM)
+        total = group_reduce<SumOp, W>(acc, slots[parity]);
+      else if (kind == ST_MAX)
+        total = group_reduce<NanMaxOp, W>(acc, slots[parity]);
+      else
+        total = group_reduce<NanMinOp, W>(acc, slots[parity]);
+      parity ^= 1;
+      red_set(red, st.dst, uniform(total));
+    } else if (kind == ST_SCALAR) {
+      red_set(red, st.dst, uniform(r.st[0][0]));
+    } else if (kind == ST_STORE_COL) {
+      if (row_live && lane == 0)
+        store_elem(a.out, out_f16, row * a.ldo, r.st[0][0]);
+    }
+  }
+}
+} // namespace
+
+extern "C" __global__ __launch_bounds__(256)
+__attribute__((amdgpu_waves_per_eu(3, 4))) void hcamd_row_program_w256(
+    const RowArgs a) {
+  row_program<256>(a);
+}
+extern "C" __global__ __launch_bounds__(256)
+__attribute__((amdgpu_waves_per_eu(3, 4))) void hcamd_row_program_w64(
+    const RowArgs a) {
+  row_program<64>(a);
+}

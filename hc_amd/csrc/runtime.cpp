@@ -263,7 +263,7 @@ std::unordered_map<std::string, int> &variants() {
   static std::unordered_map<std::string, int> v{
       {"add", 0},     {"fma", 0},  {"softmax", 0},
       {"quantize", 0}, {"gemm", 0}, {"copy", 0}, {"map", 0},
-      {"gather", 0}, {"gather_fuse", 0}};
+      {"gather", 0}, {"gather_fuse", 0}, {"rowprog", 0}};
   return v;
 }
 int variantOf(const char *family) { return variants()[family]; }
@@ -1158,6 +1158,227 @@ int hcamdLaunchMapSum(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
                       size_t rows, size_t cols) noexcept {
   return launchMap(q, true, prog, nInstr, inputs, inputTypes, inputLd, nInputs,
                    cell, HCAMD_F32, cols, rows, cols);
+}
+
+namespace {
+// Argument block of the row-program kernels (the same layout as in the device code).
+struct RowStageDev {
+  uint16_t begin, end;
+  uint8_t kind, dst, loadMask, ldsMask, keepMask, pad[3];
+};
+struct RowArgs {
+  const void *in[kMapMaxIn];
+  const void *col[kMapMaxIn];
+  void *out;
+  size_t ld[kMapMaxIn];
+  size_t ldo;
+  size_t rows, cols;
+  uint32_t f16Mask, vecMask, keepL2;
+  uint32_t nCol, nStages, passes;
+  uint8_t cacheSlot[kMapMaxIn];
+  RowStageDev stage[HCAMD_ROW_MAX_STAGES];
+  HcamdMapInstr prog[HCAMD_ROW_MAX_INSTRS];
+};
+} // namespace
+
+int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
+                          const HcamdRowStage *stages, size_t nStages,
+                          const void *const *inputs, const int *inputTypes,
+                          const size_t *inputLd, size_t nInputs,
+                          const void *const *columns, const int *columnTypes,
+                          size_t nColumns, void *out, int outType, size_t ldo,
+                          size_t rows, size_t cols) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  const char *who = "hcamdLaunchRowProgram";
+  auto typeOk = [](int t) { return t == HCAMD_F32 || t == HCAMD_F16; };
+  if (!prog || !stages || nStages == 0 || nStages > HCAMD_ROW_MAX_STAGES) {
+    dev->report("%s: %zu stages (1..%d allowed)", who, nStages, HCAMD_ROW_MAX_STAGES);
+    return 1;
+  }
+  if (nInputs > kMapMaxIn || (nInputs && (!inputs || !inputTypes || !inputLd)) ||
+      nColumns > kMapMaxIn || (nColumns && (!columns || !columnTypes))) {
+    dev->report("%s: %zu operands and %zu columns (at most %zu each)", who, nInputs,
+                nColumns, kMapMaxIn);
+    return 1;
+  }
+  if (!typeOk(outType)) {
+    dev->report("%s: unsupported output type %d", who, outType);
+    return 1;
+  }
+  RowArgs a{};
+  // Every stage must keep the stack within bounds, leave one value, and read
+  // only operands that exist and row scalars that have been written.
+  uint32_t written = (1u << nColumns) - 1u;
+  uint32_t usedIn[HCAMD_ROW_MAX_STAGES] = {};
+  size_t pc = 0;
+  for (size_t s = 0; s < nStages; ++s) {
+    const HcamdRowStage &st = stages[s];
+    if (st.kind > HCAMD_ROW_STORE_COL || st.nInstr == 0 ||
+        pc + st.nInstr > HCAMD_ROW_MAX_INSTRS) {
+      dev->report("%s: stage %zu: kind %u with %u instructions (%d in all allowed)", who,
+                  s, st.kind, st.nInstr, HCAMD_ROW_MAX_INSTRS);
+      return 1;
+    }
+    const bool stores = st.kind == HCAMD_ROW_STORE || st.kind == HCAMD_ROW_STORE_COL;
+    if (stores != (s + 1 == nStages)) {
+      dev->report("%s: the last stage, and only the last, must store", who);
+      return 1;
+    }
+    const bool perElement = st.kind <= HCAMD_ROW_MIN || st.kind == HCAMD_ROW_STORE;
+    if (!stores && st.dst >= HCAMD_ROW_MAX_SCALARS) {
+      dev->report("%s: stage %zu writes row scalar %u (%d exist)", who, s, st.dst,
+                  HCAMD_ROW_MAX_SCALARS);
+      return 1;
+    }
+    int sp = 0;
+    for (size_t i = pc; i < pc + st.nInstr; ++i) {
+      const unsigned op = prog[i].op;
+      int pops, pushes;
+      const bool red = op >= HCAMD_MAP_RED && op <= HCAMD_MAP_RDIV_RED;
+      if (red)
+        pops = op == HCAMD_MAP_RED ? 0 : 1, pushes = 1;
+      else
+        mapStackEffect(op, pops, pushes);
+      if (pops < 0) {
+        dev->report("%s: unknown opcode %u at %zu", who, op, i);
+        return 1;
+      }
+      const bool readsOperand =
+          op == HCAMD_MAP_IN || (op >= HCAMD_MAP_ADD_IN && op <= HCAMD_MAP_RDIV_IN);
+      if (readsOperand) {
+        if (!perElement || prog[i].arg >= nInputs) {
+          dev->report("%s: operand %u at %zu (%zu given; scalar stages read none)", who,
+                      prog[i].arg, i, nInputs);
+          return 1;
+        }
+        usedIn[s] |= 1u << prog[i].arg;
+      }
+      if (red && (prog[i].arg >= HCAMD_ROW_MAX_SCALARS || !((written >> prog[i].arg) & 1))) {
+        dev->report("%s: row scalar %u read at %zu before it is written", who,
+                    prog[i].arg, i);
+        return 1;
+      }
+      if (sp < pops) {
+        dev->report("%s: stack underflow at %zu", who, i);
+        return 1;
+      }
+      sp += pushes - pops;
+      if (sp > kMapDepth) {
+        dev->report("%s: stack deeper than %d at %zu", who, kMapDepth, i);
+        return 1;
+      }
+    }
+    if (sp != 1) {
+      dev->report("%s: stage %zu leaves %d values, expected 1", who, s, sp);
+      return 1;
+    }
+    a.stage[s].begin = static_cast<uint16_t>(pc);
+    a.stage[s].end = static_cast<uint16_t>(pc + st.nInstr);
+    a.stage[s].kind = static_cast<uint8_t>(st.kind);
+    a.stage[s].dst = static_cast<uint8_t>(st.dst);
+    if (!stores)
+      written |= 1u << st.dst;
+    pc += st.nInstr;
+  }
+  std::memcpy(a.prog, prog, pc * sizeof(HcamdMapInstr));
+  if (rows == 0 || cols == 0)
+    return 0;
+  if (!out) {
+    dev->report("%s: null pointer", who);
+    return 1;
+  }
+  const bool storesTile = stages[nStages - 1].kind == HCAMD_ROW_STORE;
+  if (storesTile && rows > 1 && ldo < cols) {
+    dev->report("%s: leading dimension smaller than cols", who);
+    return 1;
+  }
+  if (cols / 8 + 1 > ((size_t)1 << 31) || rows > ((size_t)1 << 31)) {
+    dev->report("%s: more than 2^31 rows or 2^34 columns", who);
+    return 1;
+  }
+  const size_t perRow = cols / 8 + (cols % 8 ? 1 : 0);
+  const size_t lanesPerRow = perRow <= 64 ? 64 : 256;
+  const size_t passes = ceilDiv(perRow, lanesPerRow);
+  for (size_t i = 0; i < nInputs; ++i) {
+    if (!inputs[i]) {
+      dev->report("%s: null pointer", who);
+      return 1;
+    }
+    if (!typeOk(inputTypes[i])) {
+      dev->report("%s: unsupported operand type %d", who, inputTypes[i]);
+      return 1;
+    }
+    if (inputLd[i] != 0 && rows > 1 && inputLd[i] < cols) {
+      dev->report("%s: leading dimension smaller than cols", who);
+      return 1;
+    }
+    const size_t esz = inputTypes[i] == HCAMD_F16 ? 2 : 4;
+    a.in[i] = inputs[i];
+    a.ld[i] = inputLd[i];
+    if (inputTypes[i] == HCAMD_F16)
+      a.f16Mask |= 1u << i;
+    if (cols >= 8 && aligned16(inputs[i]) && (rows == 1 || (inputLd[i] * esz) % 16 == 0))
+      a.vecMask |= 1u << i;
+  }
+  for (size_t k = 0; k < nColumns; ++k) {
+    if (!columns[k] || !typeOk(columnTypes[k])) {
+      dev->report("%s: column %zu: null pointer or unsupported type", who, k);
+      return 1;
+    }
+    a.col[k] = columns[k];
+    if (columnTypes[k] == HCAMD_F16)
+      a.f16Mask |= 1u << (16 + k);
+  }
+  if (outType == HCAMD_F16)
+    a.f16Mask |= 1u << 8;
+  if (storesTile && cols >= 8 && aligned16(out) &&
+      (rows == 1 || (ldo * (outType == HCAMD_F16 ? 2 : 4)) % 16 == 0))
+    a.vecMask |= 1u << 8;
+  a.out = out;
+  a.ldo = ldo;
+  a.rows = rows;
+  a.cols = cols;
+  a.nCol = static_cast<uint32_t>(nColumns);
+  a.nStages = static_cast<uint32_t>(nStages);
+  a.passes = static_cast<uint32_t>(passes);
+  // Operands that several stages read stay in LDS after the first read while
+  // they fit (passes x 8 KiB each, 64 KiB per workgroup); the others are read
+  // again and therefore loaded without the streaming hint.
+  const size_t bytesPerOperand = passes * 2 * 256 * 16;
+  size_t cached = 0;
+  uint32_t cachedMask = 0;
+  for (size_t i = 0; i < nInputs; ++i) {
+    int uses = 0;
+    for (size_t s = 0; s < nStages; ++s)
+      uses += (usedIn[s] >> i) & 1;
+    if (uses < 2)
+      continue;
+    if (variantOf("rowprog") != 1 && (cached + 1) * bytesPerOperand <= 64 * 1024) {
+      a.cacheSlot[i] = static_cast<uint8_t>(cached++);
+      cachedMask |= 1u << i;
+    } else {
+      a.keepL2 |= 1u << i;
+    }
+  }
+  uint32_t seen = 0;
+  for (size_t s = 0; s < nStages; ++s) {
+    const uint32_t first = usedIn[s] & ~seen;
+    a.stage[s].loadMask = static_cast<uint8_t>((usedIn[s] & ~cachedMask) | first);
+    a.stage[s].ldsMask = static_cast<uint8_t>(usedIn[s] & cachedMask & seen);
+    a.stage[s].keepMask = static_cast<uint8_t>(first & cachedMask);
+    seen |= usedIn[s];
+  }
+  Kernel *k = builtinKernel(dev, "map", lanesPerRow == 64 ? "hcamd_row_program_w64"
+                                                         : "hcamd_row_program_w256");
+  if (!k)
+    return 1;
+  void *args[] = {&a};
+  const size_t grid[3] = {ceilDiv(rows, 256 / lanesPerRow), 1, 1};
+  const size_t block[3] = {256, 1, 1};
+  return launch(queue, k, grid, block, args, cached * bytesPerOperand);
 }
 
 int hcamdLaunchPairwiseDistF32(OlQueue q, const float *a, size_t lda,

@@ -108,6 +108,19 @@ hcamdLaunchPairwiseDistF32 = _sig(_rt, "hcamdLaunchPairwiseDistF32", _int, _vp, 
                                   _sz, _vp, _sz, _sz, _sz, _sz)
 hcamdLaunchMapSum = _sig(_rt, "hcamdLaunchMapSum", _int, _vp, C.POINTER(MapInstr), _sz,
                          C.POINTER(_vp), C.POINTER(_int), _sz_p, _sz, _vp, _sz, _sz)
+
+
+
+class RowStage(C.Structure):
+    """HcamdRowStage of include/hc_amd_runtime.h."""
+    _fields_ = [("kind", C.c_uint32), ("nInstr", C.c_uint32), ("dst", C.c_uint32)]
+
+
+hcamdLaunchRowProgram = _sig(_rt, "hcamdLaunchRowProgram", _int, _vp, C.POINTER(MapInstr),
+                             C.POINTER(RowStage), _sz, C.POINTER(_vp), C.POINTER(_int), _sz_p,
+                             _sz, C.POINTER(_vp), C.POINTER(_int), _sz, _vp, _int, _sz, _sz, _sz)
+
+
 class GatherOperand(C.Structure):
     """HcamdGatherOperand of include/hc_amd_runtime.h."""
     _fields_ = [("ndim", _int), ("shape", _sz * 4), ("strides", _sz * 4),
@@ -409,6 +422,11 @@ MAP_OPS = {"in": 1, "const": 2, "add": 3, "sub": 4, "mul": 5, "div": 6, "max": 7
            "mul_in": 29, "div_in": 30, "max_in": 31, "min_in": 32, "rsub_in": 33,
            "rdiv_in": 34}
 MAP_MAX_INPUTS, MAP_MAX_INSTRS, MAP_STACK_DEPTH = 4, 32, 4
+# Row programs (hcamdLaunchRowProgram): opcodes that read row scalars, stage kinds, limits
+MAP_OPS.update({"red": 35, "add_red": 36, "sub_red": 37, "mul_red": 38, "div_red": 39,
+                "max_red": 40, "min_red": 41, "rsub_red": 42, "rdiv_red": 43})
+ROW_KINDS = {"sum": 0, "max": 1, "min": 2, "scalar": 3, "store": 4, "store_col": 5}
+ROW_MAX_STAGES, ROW_MAX_SCALARS, ROW_MAX_INSTRS = 8, 8, 64
 F32, F16, BF16 = 0, 1, 2
 
 
@@ -477,6 +495,82 @@ def plan_map_sum(program, inputs, cell, index: int = 0, types=None) -> Plan:
     return Plan(ctx, hcamdLaunchMapSum,
                 (ctx.queue, prog, len(program), ptrs, tys, lds, n_in, mc.ptr + 4 * index,
                  rows, cols), "hcamdLaunchMapSum", (arrays, cell, prog, ptrs, tys, lds))
+
+
+def plan_row_program(stages, inputs, out, columns=(), types=None) -> Plan:
+    """Runs a row program (see hcamdLaunchRowProgram) over a rows x cols tile.
+
+    `stages` is a list of (kind, dst, program) with kind one of ROW_KINDS and
+    program a list of (opname, arg, imm).  `inputs` are rows x cols arrays, or
+    1-D arrays of cols elements that every row uses; `columns` are 1-D arrays
+    of rows elements that fill row scalars 0, 1, ...; `out` is rows x cols for a
+    final "store" stage, or holds one value per row (1-D, or rows x 1) for
+    "store_col".  `types` = F32/F16 per input, then per column, then the
+    output's (default: by element size)."""
+    inputs, columns = list(inputs), list(columns)
+    ctx = _ctx_of(*inputs, *columns, out)
+    mo = as_memref(out)
+    col_out = stages[-1][0] == "store_col"
+    if col_out:
+        if len(mo.shape) == 2 and mo.shape[1] == 1:
+            rows, ldo = mo.shape[0], (mo.strides[0] if mo.shape[0] > 1 else 1)
+        elif len(mo.shape) == 1:
+            rows, ldo = mo.shape[0], (mo.strides[0] if mo.shape[0] > 1 else 1)
+        else:
+            raise HcRuntimeError("row_program: a per-row result needs a 1-D or rows x 1 output")
+        cols = None
+    else:
+        rows, cols, ldo = _rows_cols(mo)
+        if len(mo.shape) == 1:
+            rows, cols, ldo = 1, mo.shape[0], mo.shape[0]
+    ms, lds = [], []
+    for x in inputs:
+        m = as_memref(x)
+        if len(m.shape) == 1 and (rows != 1 or col_out):    # one vector for every row
+            if m.shape[0] > 1 and m.strides[0] != 1:
+                raise HcRuntimeError("row_program: row vectors must be contiguous")
+            r, c, ld = None, m.shape[0], 0
+        else:
+            r, c, ld = _rows_cols(m)
+        if cols is None:
+            cols = c
+        if c != cols or (r is not None and r != rows):
+            raise HcRuntimeError("row_program: shape mismatch")
+        ms.append(m)
+        lds.append(ld)
+    if cols is None:
+        raise HcRuntimeError("row_program: no operand gives the row length")
+    mc = [as_memref(x) for x in columns]
+    for m in mc:
+        n = 1
+        for d in m.shape:
+            n *= d
+        if n != rows or not m.is_contiguous():
+            raise HcRuntimeError("row_program: a column operand needs one contiguous value per row")
+    everything = ms + mc + [mo]
+    if types is None:
+        types = []
+        for m in everything:
+            if m.itemsize not in (2, 4):
+                raise HcRuntimeError(f"row_program: element size {m.itemsize} (fp32 and fp16 only)")
+            types.append(F16 if m.itemsize == 2 else F32)
+    n_in, n_col = len(ms), len(mc)
+    flat = [ins for _, _, program in stages for ins in program]
+    prog = (MapInstr * max(len(flat), 1))()
+    for i, (name, arg, imm) in enumerate(flat):
+        prog[i].op, prog[i].arg, prog[i].imm = MAP_OPS[name], int(arg), float(imm)
+    st = (RowStage * max(len(stages), 1))()
+    for i, (kind, dst, program) in enumerate(stages):
+        st[i].kind, st[i].nInstr, st[i].dst = ROW_KINDS[kind], len(program), int(dst)
+    ptrs = (_vp * max(n_in, 1))(*[m.ptr for m in ms])
+    tys = (_int * max(n_in, 1))(*types[:n_in])
+    ldv = (_sz * max(n_in, 1))(*lds)
+    cptrs = (_vp * max(n_col, 1))(*[m.ptr for m in mc])
+    ctys = (_int * max(n_col, 1))(*types[n_in:n_in + n_col])
+    return Plan(ctx, hcamdLaunchRowProgram,
+                (ctx.queue, prog, st, len(stages), ptrs, tys, ldv, n_in, cptrs, ctys, n_col,
+                 mo.ptr, types[-1], ldo, rows, cols), "hcamdLaunchRowProgram",
+                (inputs, columns, out, prog, st, ptrs, tys, ldv, cptrs, ctys))
 
 
 def plan_pairwise_dist_f32(a, b, out) -> Plan:

@@ -312,6 +312,65 @@ int hcamdLaunchMapSum(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
                       const size_t *inputLd, size_t nInputs, float *cell,
                       size_t rows, size_t cols) HCAMD_NOEXCEPT;
 
+/* Row programs: bodies that mix elementwise arithmetic with reductions along
+ * the rows of a 2-D tile, e.g. the reference's row softmax
+ * (python/hckernel/tests/test_examples.py:304-336:
+ * exp = np.exp(x - x.max(axis=1, keepdims=True)); exp / exp.sum(axis=1, keepdims=True)),
+ * normalisations, row sums.  The expression is a list of stages; each stage is
+ * a postfix program in the instruction set of hcamdLaunchMap (its instructions
+ * follow the previous stage's in `prog`) and ends in one of:
+ *   SUM, MAX, MIN  the value at every element of a row is folded into row
+ *                  scalar `dst` of that row (fp32; MAX/MIN propagate NaN)
+ *   SCALAR         the program reads row scalars only; its value becomes row
+ *                  scalar `dst`
+ *   STORE          the value at every element is stored to out[row, col]
+ *   STORE_COL      as SCALAR, stored to out[row * ldo]
+ * Exactly one stage stores, and it is the last.  Programs read row scalars with
+ * HCAMD_MAP_RED (push) and the *_RED forms (top = top op scalar), only scalars
+ * that an earlier stage or a column operand has written.
+ * Operands: `inputs` are rows x cols tiles with a leading dimension in elements,
+ * or, with leading dimension 0, one vector of cols elements used for every row;
+ * `columns` hold one value per row and fill row scalars 0 .. nColumns-1.
+ * A row is handled by one wave (cols <= 512) or one workgroup; operands that
+ * several stages read are kept on chip between the stages when they fit (64 KiB
+ * per row group), otherwise they are read again.  Sums add in an order that
+ * depends on the shape only: results are reproducible, and agree with a
+ * sequential fp32 sum to within the usual n * 2^-24 bound. */
+enum HcamdRowStageKind {
+  HCAMD_ROW_SUM = 0,
+  HCAMD_ROW_MAX = 1,
+  HCAMD_ROW_MIN = 2,
+  HCAMD_ROW_SCALAR = 3,
+  HCAMD_ROW_STORE = 4,
+  HCAMD_ROW_STORE_COL = 5
+};
+enum {
+  HCAMD_MAP_RED = 35,     /* push row scalar `arg` */
+  HCAMD_MAP_ADD_RED = 36, /* top = top + row scalar `arg` */
+  HCAMD_MAP_SUB_RED = 37,
+  HCAMD_MAP_MUL_RED = 38,
+  HCAMD_MAP_DIV_RED = 39,
+  HCAMD_MAP_MAX_RED = 40,
+  HCAMD_MAP_MIN_RED = 41,
+  HCAMD_MAP_RSUB_RED = 42, /* scalar - top */
+  HCAMD_MAP_RDIV_RED = 43  /* scalar / top */
+};
+#define HCAMD_ROW_MAX_STAGES 8
+#define HCAMD_ROW_MAX_SCALARS 8
+#define HCAMD_ROW_MAX_INSTRS 64
+typedef struct HcamdRowStage {
+  uint32_t kind;   /* HcamdRowStageKind */
+  uint32_t nInstr; /* instructions of this stage */
+  uint32_t dst;    /* row scalar written by SUM, MAX, MIN, SCALAR */
+} HcamdRowStage;
+int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
+                          const HcamdRowStage *stages, size_t nStages,
+                          const void *const *inputs, const int *inputTypes,
+                          const size_t *inputLd, size_t nInputs,
+                          const void *const *columns, const int *columnTypes,
+                          size_t nColumns, void *out, int outType, size_t ldo,
+                          size_t rows, size_t cols) HCAMD_NOEXCEPT;
+
 /* Pairwise Euclidean distances, fp32: out[i, j] = sqrt(sum_k (a[i,k] - b[j,k])^2)
  * for a[m, d], b[n, d] row-major, out[m, n].  The expression of
  * python/hckernel/tests/test_examples.py:270-301

@@ -1,0 +1,201 @@
+"""Row programs (hcamdLaunchRowProgram) on the GPU against NumPy formulas.
+
+Expected values are written as plain NumPy expressions in float64 (not as an
+emulation of the stage programs), so a wrong stage order, a reduction that
+misses elements, or a row scalar read from the wrong row fails them.  Sums are
+compared within the fp32 bound of a sum of n terms; max/min and everything
+after them within a few ulp of fp32.
+"""
+import sys
+
+import numpy as np
+import pytest
+from numpy.testing import assert_allclose, assert_array_equal
+
+from hc_amd import runtime as rt
+
+pytestmark = pytest.mark.gpu
+
+POISON32 = 0xA5A5A5A5
+
+
+def I(name, arg=0, imm=0.0):
+    return (name, arg, imm)
+
+
+def say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    return rt.default_context("hip:0")
+
+
+def poisoned(shape, dtype):
+    return rt.DeviceArray(shape, dtype).fill_bytes32(POISON32)
+
+
+class _View:
+    def __init__(self, base, shape, offset_elems=0, strides=None):
+        self.shape = tuple(shape)
+        self.ctx = base.ctx
+        item = base.dtype.itemsize
+        self.__cuda_array_interface__ = {
+            "shape": self.shape, "typestr": rt._TYPESTR[base.dtype.name],
+            "data": (int(base.ptr) + offset_elems * item, False),
+            "strides": None if strides is None else tuple(s * item for s in strides),
+            "version": 2}
+
+
+SOFTMAX = [("max", 0, [I("in", 0)]),
+           ("sum", 1, [I("in", 0), I("sub_red", 0), I("exp")]),
+           ("store", 0, [I("in", 0), I("sub_red", 0), I("exp"), I("div_red", 1)])]
+
+
+def np_softmax(x):
+    x = x.astype(np.float64)
+    e = np.exp(x - x.max(axis=1, keepdims=True))
+    return e / e.sum(axis=1, keepdims=True)
+
+
+# cols: one wave per row (<= 512), one workgroup per row, several passes, rows
+# kept in LDS (<= 16384 fp32) and rows read again from memory (above)
+@pytest.mark.parametrize("rows,cols", [(1, 1), (30, 25), (7, 8), (5, 512), (9, 513), (33, 2048),
+                                       (17, 4099), (64, 8192), (3, 16384), (2, 16392), (2, 40_001)])
+def test_softmax_as_a_row_program(ctx, rows, cols):
+    rng = np.random.default_rng(cols)
+    x = (rng.standard_normal((rows, cols)) * 3).astype(np.float32)
+    out = poisoned((rows, cols), np.float32)
+    say("row program softmax", rows, cols)
+    rt.plan_row_program(SOFTMAX, [rt.to_device(x)], out).launch(sync=True)
+    say("  ", rt.last_kernel_name())
+    assert rt.last_kernel_name() == ("hcamd_row_program_w64" if cols <= 512 else "hcamd_row_program_w256")
+    assert_allclose(out.to_host(), np_softmax(x), rtol=1e-5, atol=1e-30)
+
+
+def test_softmax_with_the_on_chip_copy_switched_off_gives_the_same_bits(ctx):
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((40, 3001)).astype(np.float32)
+    dx = rt.to_device(x)
+    got = []
+    for variant in (0, 1):
+        rt.set_variant("rowprog", variant)
+        out = poisoned(x.shape, np.float32)
+        rt.plan_row_program(SOFTMAX, [dx], out).launch(sync=True)
+        got.append(out.to_host())
+    rt.set_variant("rowprog", 0)
+    assert_array_equal(got[0].view(np.uint32), got[1].view(np.uint32))
+
+
+@pytest.mark.parametrize("cols,dtype", [(300, np.float32), (1000, np.float16), (8192, np.float32),
+                                        (4104, np.float16)])
+def test_layer_normalisation_with_weight_and_bias_vectors(ctx, cols, dtype):
+    rows = 50
+    rng = np.random.default_rng(cols)
+    x = (rng.standard_normal((rows, cols)) * 2 + 0.5).astype(dtype)
+    g = rng.standard_normal(cols).astype(np.float32)
+    b = rng.standard_normal(cols).astype(np.float32)
+    eps = 1e-5
+    n = float(cols)
+    stages = [
+        ("sum", 0, [I("in", 0)]),
+        ("scalar", 0, [I("red", 0), I("divi", 0, n)]),                                   # mean
+        ("sum", 1, [I("in", 0), I("sub_red", 0), I("in", 0), I("sub_red", 0), I("mul")]),
+        ("scalar", 1, [I("red", 1), I("divi", 0, n), I("addi", 0, eps), I("sqrt")]),     # std
+        ("store", 0, [I("in", 0), I("sub_red", 0), I("div_red", 1), I("mul_in", 1), I("add_in", 2)]),
+    ]
+    out = poisoned((rows, cols), np.float32)
+    rt.plan_row_program(stages, [rt.to_device(x), rt.to_device(g), rt.to_device(b)], out).launch(sync=True)
+    x64 = x.astype(np.float64)
+    want = (x64 - x64.mean(axis=1, keepdims=True)) / np.sqrt(x64.var(axis=1, keepdims=True) + eps) * g + b
+    assert_allclose(out.to_host(), want, rtol=2e-5, atol=2e-5)
+
+
+@pytest.mark.parametrize("rows,cols", [(1000, 7), (129, 1031), (4, 70_001)])
+def test_row_sums_maxima_and_minima_as_per_row_results(ctx, rows, cols):
+    rng = np.random.default_rng(rows)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    dx = rt.to_device(x)
+    x64 = x.astype(np.float64)
+    cases = {"sum": ((x64 * x64).sum(axis=1), [I("in", 0), I("mul_in", 0)]),
+             "max": (x64.max(axis=1), [I("in", 0)]),
+             "min": (np.abs(x64).min(axis=1), [I("in", 0), I("abs")])}
+    for kind, (want, program) in cases.items():
+        for shape in ((rows,), (rows, 1)):
+            out = poisoned(shape, np.float32)
+            rt.plan_row_program([(kind, 2, program), ("store_col", 0, [I("red", 2)])], [dx], out).launch(sync=True)
+            got = out.to_host().reshape(rows)
+            if kind == "sum":
+                assert_allclose(got, want, rtol=0, atol=cols * 2.0 ** -24 * np.abs(x64 * x64).sum(axis=1).max())
+            else:
+                assert_array_equal(got, want.astype(np.float32))
+
+
+def test_column_operands_fill_row_scalars_and_fp16_results_round_once(ctx):
+    rows, cols = 77, 1000
+    rng = np.random.default_rng(5)
+    q = rng.integers(-127, 128, (rows, cols)).astype(np.float16)
+    scale = rng.uniform(0.01, 2.0, rows).astype(np.float32)
+    shift = rng.standard_normal(rows).astype(np.float16)
+    out = poisoned((rows, cols), np.float16)
+    rt.plan_row_program([("store", 0, [I("in", 0), I("mul_red", 0), I("add_red", 1)])],
+                        [rt.to_device(q)], out,
+                        columns=[rt.to_device(scale), rt.to_device(shift)]).launch(sync=True)
+    want = ((q.astype(np.float32) * scale[:, None]) + shift.astype(np.float32)[:, None]).astype(np.float16)
+    assert_array_equal(out.to_host().view(np.uint16), want.view(np.uint16))
+
+
+def test_windows_of_larger_arrays_and_untouched_surroundings(ctx):
+    rows, cols = 19, 1003
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    for ld, off in ((1024, 4), (1011, 3)):            # 16-byte aligned rows, and not
+        big = np.full((rows + 2, ld), np.nan, np.float32)
+        big[1:rows + 1, off:off + cols] = x
+        dbig = rt.to_device(big)
+        out = poisoned((rows + 2, ld), np.float32)
+        rt.plan_row_program(SOFTMAX, [_View(dbig, (rows, cols), ld + off, (ld, 1))],
+                            _View(out, (rows, cols), ld + off, (ld, 1))).launch(sync=True)
+        got = out.to_host()
+        assert_allclose(got[1:rows + 1, off:off + cols], np_softmax(x), rtol=1e-5)
+        mask = np.ones(got.shape, bool)
+        mask[1:rows + 1, off:off + cols] = False
+        assert (got.view(np.uint32)[mask] == POISON32).all()
+
+
+def test_special_values_follow_numpy(ctx):
+    x = np.zeros((6, 600), np.float32)
+    x[0, 5] = np.nan                    # NaN reaches every result of its row only
+    x[1, :] = -np.inf                   # exp(-inf - -inf) = NaN in NumPy too
+    x[2, 7] = np.inf
+    x[3, :] = 1e30
+    x[4, 100] = -np.inf
+    out = poisoned(x.shape, np.float32)
+    rt.plan_row_program(SOFTMAX, [rt.to_device(x)], out).launch(sync=True)
+    with np.errstate(all="ignore"):
+        want = np_softmax(x)
+    got = out.to_host()
+    assert_array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert_allclose(got[ok], want[ok], rtol=1e-5)
+
+
+def test_malformed_programs_are_refused_before_anything_runs(ctx):
+    x = rt.to_device(np.ones((4, 16), np.float32))
+    out = poisoned((4, 16), np.float32)
+    bad = {
+        "before it is written": [("store", 0, [I("in", 0), I("sub_red", 3)])],
+        "must store": [("sum", 0, [I("in", 0)])],
+        "only the last": [("store", 0, [I("in", 0)]), ("store", 0, [I("in", 0)])],
+        "scalar stages read none": [("scalar", 0, [I("in", 0)]), ("store", 0, [I("in", 0)])],
+        "underflow": [("store", 0, [I("add")])],
+        "leaves 2 values": [("store", 0, [I("in", 0), I("in", 0)])],
+        "operand 1": [("store", 0, [I("in", 1)])],
+    }
+    for message, stages in bad.items():
+        with pytest.raises(rt.HcRuntimeError, match=message):
+            rt.plan_row_program(stages, [x], out).launch(sync=True)
+    assert (out.to_host().view(np.uint32) == POISON32).all()
+    with pytest.raises(rt.HcRuntimeError, match="shape mismatch"):
+        rt.plan_row_program(SOFTMAX, [rt.to_device(np.ones((4, 17), np.float32))], out)
