@@ -758,19 +758,22 @@ __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcam
 //                    output tile
 //   STORE_COL        as SCALAR, stored to out[row * ldo]
 //
-// Row scalars live in scalar registers (a row belongs to one wave or to the
-// four waves of one workgroup).  A program reaches them through the RED
-// opcodes, which are rewritten on the fly into the immediate forms of the
-// interpreter with the scalar as the immediate, so the interpreter itself does
-// not know about them.  Column operands (one value per row) are row scalars
-// that are loaded instead of computed.
+// A program reaches row scalars through the RED opcodes, which are rewritten on
+// the fly into the immediate forms of the interpreter with the scalar as the
+// immediate, so the interpreter itself does not know about them.  Column
+// operands (one value per row) are row scalars that are loaded instead of
+// computed.  Row scalars are wave-uniform: their home is a few LDS cells per
+// wave, and a stage starts by reading them into one vector register, scalar k
+// in lane k, from which a readlane fetches the one an instruction names.
 //
 // LPR lanes share a row (256: one row per workgroup; 64: one row per wave,
 // four rows per workgroup).  A lane's chunks of the row are LPR chunks apart.
-// Operands that later stages read again can be kept in LDS as they were
-// loaded; every lane reads back only what it wrote itself, so the copy needs no
-// barrier.  Reductions add in a fixed order for a given shape: results are
-// reproducible from run to run.
+// Every stage loads the operands it uses again; a row that a workgroup has just
+// read is still in L2, so only the first read goes to HBM.  (Keeping the rows
+// in LDS between the stages, each lane its own chunks, measured 10 to 70 %
+// slower: the kernel is bound by the interpreter's instruction issue, not by
+// the reads, and the LDS footprint costs occupancy.)  Reductions add in a fixed
+// order for a given shape: results are reproducible from run to run.
 namespace {
 constexpr int kMaxRed = 8;
 constexpr int kMaxStages = 8;
@@ -785,10 +788,8 @@ enum : uint32_t { ST_SUM = 0, ST_MAX = 1, ST_MIN = 2, ST_SCALAR = 3, ST_STORE = 
 struct Stage {
   uint16_t begin, end; // instructions [begin, end)
   uint8_t kind, dst;
-  uint8_t load_mask; // operands read from memory in this stage
-  uint8_t lds_mask;  // operands read from their LDS copy
-  uint8_t keep_mask; // operands copied to LDS after loading
-  uint8_t pad[3];
+  uint8_t load_mask; // operands this stage reads
+  uint8_t pad[5];
 };
 
 struct RowArgs {
@@ -800,9 +801,7 @@ struct RowArgs {
   size_t rows, cols;
   uint32_t f16_mask; // bit i: operand i is fp16; bit 8: the output; bit 16+k: column k
   uint32_t vec_mask; // bit i: rows of operand i start on 16-byte boundaries; bit 8: the output
-  uint32_t keep_l2;  // bit i: operand i is read again from memory by a later stage
   uint32_t n_col, n_stages, passes;
-  uint8_t cache_slot[kMaxIn];
   Stage stage[kMaxStages];
   Instr prog[kRowProg];
 };
@@ -818,64 +817,115 @@ struct NanMinOp {
   static __device__ __forceinline__ float apply(float a, float b) { return nan_min(a, b); }
 };
 
-// Row scalars are kept in LDS, one copy per wave (indexed registers would end up
-// in scratch memory); every lane of a wave writes the same value and reads it
-// back through readfirstlane, so no barrier is involved.
-struct Reds {
-  float *v; // this wave's kMaxRed cells
-};
 __device__ __forceinline__ float uniform(float x) {
   return __builtin_bit_cast(float,
                             __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
 }
-
-__device__ __forceinline__ float red_get(const Reds &r, uint32_t k) {
-  return uniform(r.v[k & (kMaxRed - 1)]);
-}
-__device__ __forceinline__ void red_set(Reds &r, uint32_t k, float x) {
-  r.v[k & (kMaxRed - 1)] = x;
-}
-
+// The row scalars come in as one vector register, scalar k in lane k (the same
+// in every wave of a row): reading one is a single readlane with the index in
+// a scalar register.
 __device__ __forceinline__ void run_stage(const RowArgs &a, uint32_t begin, uint32_t end,
-                                          const Raw &raw, const Reds &red, Stack &r) {
+                                          const Raw &raw, Stack &r, uint32_t reds) {
   int sp = 0;
   Instr next = a.prog[begin & (kRowProg - 1)];
   for (uint32_t pc = begin; pc < end; ++pc) {
     const Instr cur = next;
     next = a.prog[(pc + 1) & (kRowProg - 1)];
-    uint32_t op = cur.op;
     const uint32_t arg = cur.arg;
-    float imm = cur.imm;
+    // RED forms become the immediate forms with the row scalar as the immediate.
+    // The rewritten opcode is hidden from the optimiser behind an empty asm
+    // statement: an opcode whose value is known on some path would be threaded
+    // into the dispatch below and tear its arms apart.
+    uint32_t op = cur.op;
+    uint32_t imm_bits = __builtin_bit_cast(uint32_t, cur.imm);
     if (op >= OP_RED) {
-      imm = red_get(red, arg);
+      imm_bits = __builtin_amdgcn_readlane(reds, arg & (kMaxRed - 1));
       op = op == OP_RED ? (uint32_t)OP_CONST : op - OP_ADD_RED + OP_ADDI;
     }
+    asm volatile("" : "+s"(op), "+s"(imm_bits));
+    const float imm = __builtin_bit_cast(float, imm_bits);
+    // The arms differ only in the stack entries they touch.  The marker
+    // comments keep them apart: merged into one arm, every operation would
+    // pick its entries with per-element selects, eight times the vector work.
     switch (sp) {
-    case 0: sp = step<0>(r, raw, a.f16_mask, op, arg, imm); break;
-    case 1: sp = step<1>(r, raw, a.f16_mask, op, arg, imm); break;
-    case 2: sp = step<2>(r, raw, a.f16_mask, op, arg, imm); break;
-    case 3: sp = step<3>(r, raw, a.f16_mask, op, arg, imm); break;
-    default: sp = step<4>(r, raw, a.f16_mask, op, arg, imm); break;
+    case 0: asm volatile("; stack depth 0"); sp = step<0>(r, raw, a.f16_mask, op, arg, imm); break;
+    case 1: asm volatile("; stack depth 1"); sp = step<1>(r, raw, a.f16_mask, op, arg, imm); break;
+    case 2: asm volatile("; stack depth 2"); sp = step<2>(r, raw, a.f16_mask, op, arg, imm); break;
+    case 3: asm volatile("; stack depth 3"); sp = step<3>(r, raw, a.f16_mask, op, arg, imm); break;
+    default: asm volatile("; stack depth 4"); sp = step<4>(r, raw, a.f16_mask, op, arg, imm); break;
+    }
+  }
+}
+
+// Where a lane stands in its row during pass p.
+struct Place {
+  uint32_t c;       // chunk of the row (0 when the lane has none in this pass)
+  uint32_t n_valid; // elements of the chunk inside the row: 8, cols % 8, or 0
+};
+
+// The chunk `at` of operand i's row, as loaded: w0 (and w1 for fp32).  A wave
+// whose lanes all stand on whole chunks of 16-byte aligned rows (or on nothing)
+// uses 16-byte loads.  Any other wave reads element by element in all its
+// lanes, every load issued (from the row's first element where the column is
+// past the end) and zeroed afterwards.  The choice is per wave, not per lane: a
+// load in a branch that only some lanes take would be waited for on the spot,
+// together with every load issued before it.
+__device__ __forceinline__ void load_chunk(const RowArgs &a, int i, size_t row, Place at,
+                                           u32x4 &w0, u32x4 &w1) {
+  const bool f16 = (a.f16_mask >> i) & 1;
+  const char *base = static_cast<const char *>(a.in[i]) + row * a.ld[i] * (f16 ? 2 : 4);
+  const bool vec = (a.vec_mask >> i) & 1; // implies at least one whole chunk per row
+  const bool partial = at.n_valid != 8 && at.n_valid != 0;
+  w1 = u32x4{0u, 0u, 0u, 0u}; // fp16: unused, but never a value left over from another chunk
+  if (vec && __builtin_amdgcn_ballot_w64(partial) == 0) {
+    const u32x4 *q = reinterpret_cast<const u32x4 *>(base) + (f16 ? at.c : 2 * at.c);
+    w0 = ldg<false>(q);
+    if (!f16)
+      w1 = ldg<false>(q + 1);
+  } else {
+    uint32_t v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const size_t el = (uint32_t)e < at.n_valid ? (size_t)at.c * 8 + e : 0;
+      v[e] = f16 ? (uint32_t) reinterpret_cast<const uint16_t *>(base)[el]
+                 : reinterpret_cast<const uint32_t *>(base)[el];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      v[e] = (uint32_t)e < at.n_valid ? v[e] : 0u;
+    if (f16) {
+      w0 = u32x4{v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16),
+                 v[6] | (v[7] << 16)};
+    } else {
+      w0 = u32x4{v[0], v[1], v[2], v[3]};
+      w1 = u32x4{v[4], v[5], v[6], v[7]};
     }
   }
 }
 
 template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a) {
-  extern __shared__ u32x4 row_cache[];
   __shared__ float slots[2][kThreads / kWave];
+  __shared__ float red_cells[kThreads / kWave][kMaxRed];
   const uint32_t t = threadIdx.x, lane = t % LPR;
+  float *cells = red_cells[t / kWave];
   const size_t row_at = (size_t)blockIdx.x * (kThreads / LPR) + t / LPR;
   const bool row_live = row_at < a.rows;
   const size_t row = row_live ? row_at : 0; // idle lanes compute on row 0 and store nothing
   const uint32_t whole = (uint32_t)(a.cols / 8), rem = (uint32_t)(a.cols % 8);
   const uint32_t per_row = whole + (rem ? 1u : 0u);
   const bool out_f16 = (a.f16_mask >> 8) & 1;
-  __shared__ float red_cells[kThreads / kWave][kMaxRed];
-  Reds red{red_cells[t / kWave]};
+  auto place = [&](uint32_t p) {
+    const uint32_t c = p * LPR + lane;
+    const bool live = row_live && p < a.passes && c < per_row;
+    return Place{live ? c : 0u, !live ? 0u : c == whole ? rem : 8u};
+  };
+  if (t % kWave < kMaxRed)
+    cells[t % kWave] = 0.0f;
 #pragma unroll
   for (int k = 0; k < kMaxIn; ++k)
     if (k < (int)a.n_col)
-      red_set(red, k, uniform(load_elem(a.col[k], (a.f16_mask >> (16 + k)) & 1, row)));
+      cells[k] = uniform(load_elem(a.col[k], (a.f16_mask >> (16 + k)) & 1, row));
+
   uint32_t parity = 0;
 #pragma nounroll
   for (uint32_t s = 0; s < a.n_stages; ++s) {
@@ -883,96 +933,45 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
     const uint32_t kind = st.kind;
     const bool per_element = kind <= ST_MIN || kind == ST_STORE;
     const uint32_t n_pass = per_element ? a.passes : 1;
+    // the row scalars, scalar k in lane k
+    const uint32_t reds = __builtin_bit_cast(uint32_t, cells[t & (kMaxRed - 1)]);
     float acc = kind == ST_MAX ? -INFINITY : kind == ST_MIN ? INFINITY : 0.0f;
-    Raw raw;
     Stack r;
 #pragma nounroll
     for (uint32_t p = 0; p < n_pass; ++p) {
-      const uint32_t c_at = p * LPR + lane;
-      const bool live = per_element && row_live && c_at < per_row;
-      const uint32_t c = live ? c_at : 0;
-      const bool shortc = live && c == whole;
-      const uint32_t n_valid = !live ? 0u : shortc ? rem : 8u;
+      const Place at = per_element ? place(p) : Place{0u, 0u};
+      Raw raw;
       if (per_element) {
 #pragma unroll
         for (int i = 0; i < kMaxIn; ++i) {
-          const bool f16 = (a.f16_mask >> i) & 1;
-          const uint32_t slot = ((a.cache_slot[i] * a.passes + p) * 2) * kThreads + t;
-          if ((st.lds_mask >> i) & 1) {
-            raw.w[i][0] = row_cache[slot];
-            if (!f16)
-              raw.w[i][1] = row_cache[slot + kThreads];
-          } else if ((st.load_mask >> i) & 1) {
-            const char *base = static_cast<const char *>(a.in[i]) +
-                               row * a.ld[i] * (f16 ? 2 : 4);
-            const bool vec = (a.vec_mask >> i) & 1; // implies whole >= 1
-            if (vec) {
-              const uint32_t cv = shortc ? 0 : c;
-              const u32x4 *q = reinterpret_cast<const u32x4 *>(base) + (f16 ? cv : 2 * cv);
-              if ((a.keep_l2 >> i) & 1) {
-                raw.w[i][0] = ldg<false>(q);
-                if (!f16)
-                  raw.w[i][1] = ldg<false>(q + 1);
-              } else {
-                raw.w[i][0] = ldg<true>(q);
-                if (!f16)
-                  raw.w[i][1] = ldg<true>(q + 1);
-              }
-            }
-            if (!vec || shortc) {
-              // element by element; every load is issued (from the row's first
-              // element where the column is past the end) and zeroed afterwards
-              uint32_t v[8];
-#pragma unroll
-              for (int e = 0; e < 8; ++e) {
-                const size_t at = (uint32_t)e < n_valid ? (size_t)c * 8 + e : 0;
-                v[e] = f16 ? (uint32_t) reinterpret_cast<const uint16_t *>(base)[at]
-                           : reinterpret_cast<const uint32_t *>(base)[at];
-              }
-#pragma unroll
-              for (int e = 0; e < 8; ++e)
-                v[e] = (uint32_t)e < n_valid ? v[e] : 0u;
-              if (f16) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                  raw.w[i][0][e] = v[2 * e] | (v[2 * e + 1] << 16);
-              } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                  raw.w[i][e / 4][e % 4] = v[e];
-              }
-            }
-            if ((st.keep_mask >> i) & 1) {
-              row_cache[slot] = raw.w[i][0];
-              if (!f16)
-                row_cache[slot + kThreads] = raw.w[i][1];
-            }
+          if ((st.load_mask >> i) & 1) {
+            load_chunk(a, i, row, at, raw.w[i][0], raw.w[i][1]);
           }
         }
       }
-      run_stage(a, st.begin, st.end, raw, red, r);
+      run_stage(a, st.begin, st.end, raw, r, reds);
       if (kind == ST_STORE) {
         char *orow = static_cast<char *>(a.out) + row * a.ldo * (out_f16 ? 2 : 4);
-        if (((a.vec_mask >> 8) & 1) && n_valid == 8) {
-          store_chunk(orow, out_f16, c, r.st[0]);
+        if (((a.vec_mask >> 8) & 1) && at.n_valid == 8) {
+          store_chunk(orow, out_f16, at.c, r.st[0]);
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if ((uint32_t)e < n_valid)
-              store_elem(orow, out_f16, (size_t)c * 8 + e, r.st[0][e]);
+            if ((uint32_t)e < at.n_valid)
+              store_elem(orow, out_f16, (size_t)at.c * 8 + e, r.st[0][e]);
         }
       } else if (kind == ST_SUM) {
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-          acc += (uint32_t)e < n_valid ? r.st[0][e] : 0.0f;
+          acc += (uint32_t)e < at.n_valid ? r.st[0][e] : 0.0f;
       } else if (kind == ST_MAX) {
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-          acc = (uint32_t)e < n_valid ? nan_max(acc, r.st[0][e]) : acc;
+          acc = (uint32_t)e < at.n_valid ? nan_max(acc, r.st[0][e]) : acc;
       } else if (kind == ST_MIN) {
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-          acc = (uint32_t)e < n_valid ? nan_min(acc, r.st[0][e]) : acc;
+          acc = (uint32_t)e < at.n_valid ? nan_min(acc, r.st[0][e]) : acc;
       }
     }
     if (kind <= ST_MIN) {
@@ -985,9 +984,9 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
       else
         total = group_reduce<NanMinOp, W>(acc, slots[parity]);
       parity ^= 1;
-      red_set(red, st.dst, uniform(total));
+      cells[st.dst & (kMaxRed - 1)] = total;
     } else if (kind == ST_SCALAR) {
-      red_set(red, st.dst, uniform(r.st[0][0]));
+      cells[st.dst & (kMaxRed - 1)] = uniform(r.st[0][0]);
     } else if (kind == ST_STORE_COL) {
       if (row_live && lane == 0)
         store_elem(a.out, out_f16, row * a.ldo, r.st[0][0]);
@@ -997,12 +996,10 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
 } // namespace
 
 extern "C" __global__ __launch_bounds__(256)
-__attribute__((amdgpu_waves_per_eu(3, 4))) void hcamd_row_program_w256(
-    const RowArgs a) {
+__attribute__((amdgpu_waves_per_eu(2, 4))) void hcamd_row_program_w256(const RowArgs a) {
   row_program<256>(a);
 }
 extern "C" __global__ __launch_bounds__(256)
-__attribute__((amdgpu_waves_per_eu(3, 4))) void hcamd_row_program_w64(
-    const RowArgs a) {
+__attribute__((amdgpu_waves_per_eu(2, 4))) void hcamd_row_program_w64(const RowArgs a) {
   row_program<64>(a);
 }

@@ -263,7 +263,7 @@ std::unordered_map<std::string, int> &variants() {
   static std::unordered_map<std::string, int> v{
       {"add", 0},     {"fma", 0},  {"softmax", 0},
       {"quantize", 0}, {"gemm", 0}, {"copy", 0}, {"map", 0},
-      {"gather", 0}, {"gather_fuse", 0}, {"rowprog", 0}};
+      {"gather", 0}, {"gather_fuse", 0}};
   return v;
 }
 int variantOf(const char *family) { return variants()[family]; }
@@ -1164,7 +1164,7 @@ namespace {
 // Argument block of the row-program kernels (the same layout as in the device code).
 struct RowStageDev {
   uint16_t begin, end;
-  uint8_t kind, dst, loadMask, ldsMask, keepMask, pad[3];
+  uint8_t kind, dst, loadMask, pad[5];
 };
 struct RowArgs {
   const void *in[kMapMaxIn];
@@ -1173,9 +1173,8 @@ struct RowArgs {
   size_t ld[kMapMaxIn];
   size_t ldo;
   size_t rows, cols;
-  uint32_t f16Mask, vecMask, keepL2;
+  uint32_t f16Mask, vecMask;
   uint32_t nCol, nStages, passes;
-  uint8_t cacheSlot[kMapMaxIn];
   RowStageDev stage[HCAMD_ROW_MAX_STAGES];
   HcamdMapInstr prog[HCAMD_ROW_MAX_INSTRS];
 };
@@ -1300,7 +1299,8 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
     return 1;
   }
   const size_t perRow = cols / 8 + (cols % 8 ? 1 : 0);
-  const size_t lanesPerRow = perRow <= 64 ? 64 : 256;
+  // a wave per row up to 4096 columns (at most 8 chunks per lane), else a workgroup
+  const size_t lanesPerRow = perRow <= 512 ? 64 : 256;
   const size_t passes = ceilDiv(perRow, lanesPerRow);
   for (size_t i = 0; i < nInputs; ++i) {
     if (!inputs[i]) {
@@ -1344,33 +1344,8 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
   a.nCol = static_cast<uint32_t>(nColumns);
   a.nStages = static_cast<uint32_t>(nStages);
   a.passes = static_cast<uint32_t>(passes);
-  // Operands that several stages read stay in LDS after the first read while
-  // they fit (passes x 8 KiB each, 64 KiB per workgroup); the others are read
-  // again and therefore loaded without the streaming hint.
-  const size_t bytesPerOperand = passes * 2 * 256 * 16;
-  size_t cached = 0;
-  uint32_t cachedMask = 0;
-  for (size_t i = 0; i < nInputs; ++i) {
-    int uses = 0;
-    for (size_t s = 0; s < nStages; ++s)
-      uses += (usedIn[s] >> i) & 1;
-    if (uses < 2)
-      continue;
-    if (variantOf("rowprog") != 1 && (cached + 1) * bytesPerOperand <= 64 * 1024) {
-      a.cacheSlot[i] = static_cast<uint8_t>(cached++);
-      cachedMask |= 1u << i;
-    } else {
-      a.keepL2 |= 1u << i;
-    }
-  }
-  uint32_t seen = 0;
-  for (size_t s = 0; s < nStages; ++s) {
-    const uint32_t first = usedIn[s] & ~seen;
-    a.stage[s].loadMask = static_cast<uint8_t>((usedIn[s] & ~cachedMask) | first);
-    a.stage[s].ldsMask = static_cast<uint8_t>(usedIn[s] & cachedMask & seen);
-    a.stage[s].keepMask = static_cast<uint8_t>(first & cachedMask);
-    seen |= usedIn[s];
-  }
+  for (size_t s = 0; s < nStages; ++s)
+    a.stage[s].loadMask = static_cast<uint8_t>(usedIn[s]);
   Kernel *k = builtinKernel(dev, "map", lanesPerRow == 64 ? "hcamd_row_program_w64"
                                                          : "hcamd_row_program_w256");
   if (!k)
@@ -1378,7 +1353,7 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
   void *args[] = {&a};
   const size_t grid[3] = {ceilDiv(rows, 256 / lanesPerRow), 1, 1};
   const size_t block[3] = {256, 1, 1};
-  return launch(queue, k, grid, block, args, cached * bytesPerOperand);
+  return launch(queue, k, grid, block, args, 0);
 }
 
 int hcamdLaunchPairwiseDistF32(OlQueue q, const float *a, size_t lda,

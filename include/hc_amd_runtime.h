@@ -331,9 +331,8 @@ int hcamdLaunchMapSum(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
  * Operands: `inputs` are rows x cols tiles with a leading dimension in elements,
  * or, with leading dimension 0, one vector of cols elements used for every row;
  * `columns` hold one value per row and fill row scalars 0 .. nColumns-1.
- * A row is handled by one wave (cols <= 512) or one workgroup; operands that
- * several stages read are kept on chip between the stages when they fit (64 KiB
- * per row group), otherwise they are read again.  Sums add in an order that
+ * A row is handled by one wave (cols <= 4096) or one workgroup; every stage
+ * reads the operands it uses again (a row just read is still in L2).  Sums add in an order that
  * depends on the shape only: results are reproducible, and agree with a
  * sequential fp32 sum to within the usual n * 2^-24 bound. */
 enum HcamdRowStageKind {

@@ -59,8 +59,7 @@ def np_softmax(x):
     return e / e.sum(axis=1, keepdims=True)
 
 
-# cols: one wave per row (<= 512), one workgroup per row, several passes, rows
-# kept in LDS (<= 16384 fp32) and rows read again from memory (above)
+# cols: one wave per row (<= 4096), one workgroup per row, one and several chunks per lane
 @pytest.mark.parametrize("rows,cols", [(1, 1), (30, 25), (7, 8), (5, 512), (9, 513), (33, 2048),
                                        (17, 4099), (64, 8192), (3, 16384), (2, 16392), (2, 40_001)])
 def test_softmax_as_a_row_program(ctx, rows, cols):
@@ -70,22 +69,8 @@ def test_softmax_as_a_row_program(ctx, rows, cols):
     say("row program softmax", rows, cols)
     rt.plan_row_program(SOFTMAX, [rt.to_device(x)], out).launch(sync=True)
     say("  ", rt.last_kernel_name())
-    assert rt.last_kernel_name() == ("hcamd_row_program_w64" if cols <= 512 else "hcamd_row_program_w256")
+    assert rt.last_kernel_name() == ("hcamd_row_program_w64" if cols <= 4096 else "hcamd_row_program_w256")
     assert_allclose(out.to_host(), np_softmax(x), rtol=1e-5, atol=1e-30)
-
-
-def test_softmax_with_the_on_chip_copy_switched_off_gives_the_same_bits(ctx):
-    rng = np.random.default_rng(1)
-    x = rng.standard_normal((40, 3001)).astype(np.float32)
-    dx = rt.to_device(x)
-    got = []
-    for variant in (0, 1):
-        rt.set_variant("rowprog", variant)
-        out = poisoned(x.shape, np.float32)
-        rt.plan_row_program(SOFTMAX, [dx], out).launch(sync=True)
-        got.append(out.to_host())
-    rt.set_variant("rowprog", 0)
-    assert_array_equal(got[0].view(np.uint32), got[1].view(np.uint32))
 
 
 @pytest.mark.parametrize("cols,dtype", [(300, np.float32), (1000, np.float16), (8192, np.float32),
