@@ -28,6 +28,7 @@ there is no interpreter or CPU path behind it.
 
 from __future__ import annotations
 
+import math
 from dataclasses import dataclass
 
 from . import runtime as rt
@@ -836,6 +837,380 @@ def match_map(dst_view, value, n_groups):
     return make
 
 
+# ---------------------------------------------------------------------------
+# Row programs: elementwise arithmetic mixed with reductions along rows
+# ---------------------------------------------------------------------------
+_ROW_REDUCE = {"sum": "sum", "max": "max", "min": "min"}
+
+
+class _RowCompiler(_MapCompiler):
+    """Splits an expression over (rows, N) tiles that contains reductions along
+    axis 1 into the stages of hcamdLaunchRowProgram.
+
+    Every node is one of: E, an elementwise value of shape (rows, N); S, a row
+    scalar of shape (rows, 1) or (rows,); V, a vector of shape (N,) or (1, N)
+    that every row uses (loads only); or a constant.  A reduction of an E
+    expression, a column load and an arithmetic expression of S nodes each get
+    a row scalar slot; E programs read slots through the RED instructions."""
+
+    def __init__(self, n_groups, rows, n):
+        super().__init__(n_groups)
+        self.rows, self.n = rows, n
+        self.kinds = {}            # operand index -> "tile" | "vector"
+        self.columns = []          # (buffer index, starts, load Tile)
+        self.stages = []           # (kind, slot, program)
+        self.slots = {}            # uid of an S node -> slot
+        self.n_slots = 0
+
+    # -- classification ----------------------------------------------------------
+    def klass(self, t: Tile) -> str:
+        if _const(t):
+            return "C"
+        if t.shape == (self.rows, self.n) and len(t.shape) == 2 and not self._is_scalar_node(t):
+            return "E"
+        if self._is_scalar_node(t):
+            return "S"
+        if t.shape in ((self.n,), (1, self.n)):
+            return "V"
+        return "?"
+
+    def _is_scalar_node(self, t: Tile) -> bool:
+        """Shape (rows, 1) or (rows,), and made of reductions along axis 1,
+        1-D loads of `rows` elements, constants and arithmetic on those."""
+        if t.shape not in ((self.rows, 1), (self.rows,)):
+            return False
+        if t.op in _ROW_REDUCE and t.attrs.get("axes") == (1,):
+            return True
+        if _is(t, "load") or _is(t, "slice", 1) or _is(t, "reshape", 1):
+            if self.column_load(t) is not None:
+                return True
+            return not _is(t, "load") and self._is_scalar_node(t.args[0])
+        if _is(t, "astype", 1) or t.op in _MAP_UNARY or _is(t, "clip", 1):
+            return self._is_scalar_node(t.args[0])
+        if t.op in _MAP_BINARY and len(t.args) == 2:
+            return all(_const(a) or self._is_scalar_node(a) for a in t.args) and \
+                not all(_const(a) for a in t.args)
+        return False
+
+    def column_load(self, t: Tile):
+        """The load behind t if t is a per-row operand: a 1-D load of `rows`
+        elements, as it is (when that cannot be mistaken for a vector of N
+        elements) or viewed as (rows, 1)."""
+        base = self._strip_views(t)
+        if not _is(base, "load") or base.shape not in ((self.rows,), (self.rows, 1)):
+            return None
+        if base.shape == (self.rows, 1) and self.n == 1:
+            return None                                    # a one-column tile is still a tile
+        if t.shape == (self.rows, 1):
+            return base
+        if t.shape == (self.rows,) and self.rows != self.n:
+            return base
+        return None
+
+    @staticmethod
+    def _strip_views(t: Tile) -> Tile:
+        while _is(t, "slice", 1) or _is(t, "reshape", 1):
+            t = t.args[0]
+        return t
+
+    # -- row scalars --------------------------------------------------------------
+    def _new_slot(self, t: Tile) -> int:
+        if self.n_slots >= rt.ROW_MAX_SCALARS:
+            raise NoNativeKernel(f"the expression needs more than {rt.ROW_MAX_SCALARS} row "
+                                 "scalars (reductions, per-row operands and expressions of them)")
+        self.slots[t.uid] = self.n_slots
+        self.n_slots += 1
+        return self.slots[t.uid]
+
+    def find_columns(self, t: Tile, seen=None):
+        """Per-row operands take the first slots, in the order they are met."""
+        seen = set() if seen is None else seen
+        if t.uid in seen:
+            return
+        seen.add(t.uid)
+        if self.column_load(t) is not None:
+            t = self.column_load(t)
+            v = t.attrs["view"]
+            if t.dtype_name not in _MAP_FLOATS:
+                raise NoNativeKernel(f"{v.base.name}: per-row operands must be float32 or float16")
+            for i, (b, st, _) in enumerate(self.columns):
+                if b == v.base.index and st == v.starts:
+                    self.slots[t.uid] = i
+                    return
+            if len(self.columns) >= rt.MAP_MAX_INPUTS:
+                raise NoNativeKernel(f"more than {rt.MAP_MAX_INPUTS} per-row operands")
+            self.columns.append((v.base.index, v.starts, t))
+            self._new_slot(t)
+            return
+        for a in t.args:
+            self.find_columns(a, seen)
+
+    def scalar(self, t: Tile) -> int:
+        """The slot that holds S node t, adding the stages that compute it."""
+        t = self._strip_views(t)
+        if t.uid in self.slots:
+            return self.slots[t.uid]
+        for uid_t, slot in self._same_reductions:
+            if _same(uid_t, t):
+                self.slots[t.uid] = slot
+                return slot
+        if t.op in _ROW_REDUCE and t.attrs.get("axes") == (1,):
+            body = t.args[0]
+            if self.klass(body) != "E":
+                raise NoNativeKernel(f"{t!r}: only reductions of (rows, N) tiles along axis 1 "
+                                     "have native code")
+            if t.op == "sum" and body.dtype_name != "float32":
+                raise NoNativeKernel("row sums are computed in float32: cast the tile with "
+                                     ".astype(np.float32) before adding it up")
+            program = self.program(body)
+            slot = self._new_slot(t)
+            self.stages.append((_ROW_REDUCE[t.op], slot, program))
+            self._same_reductions.append((t, slot))
+            return slot
+        if _is(t, "astype", 1) and t.dtype_name == "float32" and self._is_scalar_node(t.args[0]) \
+                and self._strip_views(t.args[0]).uid in self.slots:
+            return self.slots[self._strip_views(t.args[0]).uid]     # widening changes nothing
+        program = self.program(t, scalar=True)
+        slot = self._new_slot(t)
+        self.stages.append(("scalar", slot, program))
+        self._same_reductions.append((t, slot))
+        return slot
+
+    _same_reductions: list
+
+    # -- programs -------------------------------------------------------------------
+    def prepare(self, t: Tile, scalar: bool):
+        """Makes sure every row scalar an expression reads has its slot (and
+        the stages that fill it come first)."""
+        if _const(t) or _is(t, "load") and not self._is_scalar_node(t):
+            return
+        k = self.klass(t)
+        if not scalar and k == "S":
+            self.scalar(t)
+            return
+        if scalar:
+            base = self._strip_views(t)
+            if base.uid in self.slots:
+                return
+            if base.op in _ROW_REDUCE and base.attrs.get("axes") == (1,) or _is(base, "load"):
+                self.scalar(base)
+                return
+            t = base
+        for a in t.args:
+            self.prepare(a, scalar)
+
+    def program(self, t: Tile, scalar: bool = False) -> list:
+        self.prepare(t, scalar)
+        self._scalar_mode = scalar
+        self.need_cache = {}
+        if not self.supported(t):
+            raise NoNativeKernel(f"{t!r} is not an expression of float32 / float16 tiles, row "
+                                 "reductions, per-row operands and constants")
+        if self.need(t) > rt.MAP_STACK_DEPTH:
+            raise NoNativeKernel("expression needs an evaluation stack deeper than "
+                                 f"{rt.MAP_STACK_DEPTH}")
+        out: list = []
+        self.emit(t, out)
+        return out
+
+    def slot_of(self, t: Tile):
+        """Slot of t if pushing t means reading a row scalar."""
+        if not isinstance(t, Tile) or _const(t):
+            return None
+        base = self._strip_views(t)
+        if base.uid in self.slots:
+            return self.slots[base.uid]
+        if _is(base, "astype", 1) and base.dtype_name == "float32":
+            inner = self._strip_views(base.args[0])
+            if inner.uid in self.slots:
+                return self.slots[inner.uid]
+        return None
+
+    def operand(self, t: Tile) -> int:
+        i = super().operand(t)
+        kind = "vector" if self.klass(t) == "V" else "tile"
+        if self.kinds.setdefault(i, kind) != kind:
+            raise NoNativeKernel("one window is used both as a tile and as a vector")
+        return i
+
+    def supported(self, t: Tile) -> bool:
+        if _const(t) or self.slot_of(t) is not None:
+            return True
+        if t.dtype_name not in _MAP_FLOATS:
+            return False
+        if _is(t, "slice", 1) or _is(t, "reshape", 1):
+            # views are transparent on row scalars and on (N,) -> (1, N) vectors
+            inner = t.args[0]
+            ok_shape = self.klass(t) in ("S", "V") and self.klass(inner) == self.klass(t)
+            return ok_shape and self.supported(inner)
+        if _is(t, "load"):
+            return self.klass(t) in ("E", "V") and not self._scalar_mode
+        if _is(t, "astype", 1) or t.op in _MAP_UNARY or _is(t, "clip", 1):
+            return len(t.args) == 1 and self.supported(t.args[0])
+        if t.op in _MAP_BINARY and len(t.args) == 2:
+            if all(_const(a) for a in t.args):
+                return False
+            return all(self.supported(a) for a in t.args)
+        return False
+
+    def need(self, t: Tile) -> int:
+        if self.slot_of(t) is not None:
+            return 1
+        if _is(t, "slice", 1) or _is(t, "reshape", 1):
+            return self.need(t.args[0])
+        if t.uid in self.need_cache:
+            return self.need_cache[t.uid]
+        if t.op in _MAP_BINARY and len(t.args) == 2:
+            a, b = t.args
+            if not (_const(a) or _const(b)):
+                # a row scalar on one side is read by the operation itself
+                if self.slot_of(b) is not None or self.slot_of(a) is not None:
+                    n = self.need(a if self.slot_of(b) is not None else b)
+                    self.need_cache[t.uid] = n
+                    return n
+        return super().need(t)
+
+    def emit(self, t: Tile, out: list):
+        slot = self.slot_of(t)
+        if slot is not None:
+            out.append(("red", slot, 0.0))
+            return
+        if _is(t, "slice", 1) or _is(t, "reshape", 1):
+            self.emit(t.args[0], out)
+            return
+        if t.op in _MAP_BINARY and len(t.args) == 2 and not (_const(t.args[0]) or _const(t.args[1])):
+            fwd, rev, _ = _MAP_BINARY[t.op]
+            a, b = t.args
+            sa, sb = self.slot_of(a), self.slot_of(b)
+            if sb is not None or sa is not None:
+                if sb is not None:
+                    self.emit(a, out)
+                    out.append((fwd + "_red", sb, 0.0))
+                else:
+                    self.emit(b, out)
+                    out.append((rev + "_red", sa, 0.0))
+                if t.dtype_name == "float16" and t.op not in _MAP_EXACT:
+                    out.append(("r16", 0, 0.0))
+                return
+        super().emit(t, out)
+
+
+def match_rows(dst_view, value, n_groups):
+    """Elementwise expressions with reductions along the rows, e.g.
+    (x - x.mean(axis=1, keepdims=True)) / x.std(axis=1, keepdims=True) or
+    x.sum(axis=1): python/hckernel/tests/test_examples.py:304-336 is the
+    softmax instance of the pattern.  Tiles must hold whole rows."""
+    if dst_view.base.dtype_name not in _MAP_FLOATS:
+        return None
+
+    def has_row_reduce(t, seen):
+        if t.uid in seen:
+            return False
+        seen.add(t.uid)
+        if t.op in _ROW_REDUCE and t.attrs.get("axes") == (1,) and len(t.args[0].shape) == 2:
+            return True
+        return any(has_row_reduce(a, seen) for a in t.args)
+
+    def first_tile(t):
+        if _is(t, "load") and len(t.shape) == 2:
+            return t
+        for a in t.args:
+            r = first_tile(a)
+            if r is not None:
+                return r
+        return None
+
+    if not has_row_reduce(value, set()):
+        return None
+    x = first_tile(value)
+    if x is None:
+        return None
+    rows, n = x.shape
+    comp = _RowCompiler(n_groups, rows, n)
+    comp._same_reductions = []
+    comp.find_columns(value)
+    per_row = comp._is_scalar_node(value)
+    if not per_row and value.shape != (rows, n):
+        return None
+    if per_row:
+        comp.prepare(value, True)
+        slot = comp.slot_of(value)
+        program = [("red", slot, 0.0)] if slot is not None else comp.program(value, scalar=True)
+        comp.stages.append(("store_col", 0, program))
+    else:
+        program = comp.program(value)
+        comp.stages.append(("store", 0, program))
+    if len(comp.stages) > rt.ROW_MAX_STAGES:
+        raise NoNativeKernel(f"the expression needs {len(comp.stages)} passes over the rows "
+                             f"(at most {rt.ROW_MAX_STAGES})")
+    if sum(len(p) for _, _, p in comp.stages) > rt.ROW_MAX_INSTRS:
+        raise NoNativeKernel(f"the expression compiles to more than {rt.ROW_MAX_INSTRS} operations")
+    if len(comp.inputs) > rt.MAP_MAX_INPUTS:
+        raise NoNativeKernel(f"the expression reads {len(comp.inputs)} arrays "
+                             f"(at most {rt.MAP_MAX_INPUTS})")
+    # windows: tiles and the output walk the same whole rows; vectors are read
+    # whole by every group; per-row operands walk the same rows
+    wins, tile_win = [], None
+    for i, (_, _, t) in enumerate(comp.inputs):
+        w = window_of(t.attrs["view"], t.shape, n_groups)
+        if comp.kinds[i] == "tile":
+            if len(w.extent) != 2 or w.driver[1] is not None or \
+                    w.extent[1] != t.attrs["view"].base.shape[1] or w.extent[1] != n:
+                raise NoNativeKernel("row reductions need tiles that hold whole rows")
+            if tile_win is not None and (w.extent != tile_win.extent or w.driver != tile_win.driver):
+                raise NoNativeKernel("the tiles of a row expression must walk the same rows")
+            tile_win = tile_win or w
+        else:
+            if any(d is not None for d in w.driver) or math.prod(w.extent) != n:
+                raise NoNativeKernel("a vector used by every row must be loaded whole by every group")
+        wins.append(w)
+    if tile_win is None:
+        return None
+    col_wins = []
+    for _, _, t in comp.columns:
+        w = window_of(t.attrs["view"], t.shape, n_groups)
+        if w.extent[0] != tile_win.extent[0] or w.driver[0] != tile_win.driver[0] or \
+                math.prod(w.extent) != w.extent[0]:
+            raise NoNativeKernel("per-row operands and tiles walk different rows")
+        col_wins.append(w)
+    if per_row:
+        out_shape = (rows,) + (1,) * (dst_view.base.ndim - 1)
+        wo = window_of(dst_view, out_shape, n_groups)
+        if wo.extent[0] != tile_win.extent[0] or wo.driver[0] != tile_win.driver[0] or \
+                math.prod(wo.extent) != wo.extent[0]:
+            raise NoNativeKernel("the per-row result and the tiles walk different rows")
+    else:
+        wo = window_of(dst_view, value.shape, n_groups)
+        if wo.extent != tile_win.extent or wo.driver != tile_win.driver:
+            raise NoNativeKernel("loads and the store walk different windows")
+    ftype = lambda name: rt.F16 if name == "float16" else rt.F32
+    types = [ftype(t.dtype_name) for _, _, t in comp.inputs] + \
+            [ftype(t.dtype_name) for _, _, t in comp.columns] + [ftype(dst_view.base.dtype_name)]
+    stages = list(comp.stages)
+    n_rows = tile_win.extent[0]
+
+    def make(mem, ctx):
+        ins = []
+        for i, w in enumerate(wins):
+            m = mem[w.buffer]
+            if comp.kinds[i] == "tile":
+                ins.append(_Arr(_sub(m, w.extent), ctx))
+            else:
+                ins.append(_Arr(rt.Memref(m.ptr, (n,), (m.strides[-1],), m.itemsize), ctx))
+        cols = []
+        for w in col_wins:
+            m = mem[w.buffer]
+            cols.append(_Arr(rt.Memref(m.ptr, (n_rows,), (m.strides[0],), m.itemsize), ctx))
+        mo = mem[wo.buffer]
+        if per_row:
+            out = _Arr(rt.Memref(mo.ptr, (n_rows,), (mo.strides[0],), mo.itemsize), ctx)
+        else:
+            out = _Arr(_sub(mo, wo.extent), ctx)
+        return [rt.plan_row_program(stages, ins, out, cols, types)]
+    make.stages = stages
+    return make
+
+
 def match_pairwise(dst_view, value, n_groups):
     """out[m, n] = ||a[m, :] - b[n, :]||: the body of
     python/hckernel/tests/test_examples.py:270-301."""
@@ -970,7 +1345,7 @@ def bind(stores, n_groups, atomics=(), mapped_stores=()):
             return makers + [q]
         for view, value in stores:
             for matcher in (match_copy, match_add, match_fma, match_softmax, match_gemm,
-                            match_gather_gemm, match_pairwise, match_map):
+                            match_gather_gemm, match_pairwise, match_rows, match_map):
                 mk = matcher(view, value, n_groups)
                 if mk is not None:
                     makers.append(mk)
@@ -980,7 +1355,7 @@ def bind(stores, n_groups, atomics=(), mapped_stores=()):
                     f"no hand-written kernel matches the value stored to {view.base.name} "
                     f"({value!r}); bound patterns: copy, a+b (fp32), a*b+c (fp16 storage, fp32 "
                     "math), row softmax (fp32), row absmax int8 quantisation, bf16 GEMM, elementwise "
-                    "expressions over fp32 / fp16 arrays")
+                    "expressions over fp32 / fp16 arrays, with reductions along whole rows")
         return makers
     except TraceError as exc:
         raise NoNativeKernel(str(exc)) from exc

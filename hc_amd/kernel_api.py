@@ -437,7 +437,7 @@ def _as_view(x) -> BufferView:
 _UFUNC_OPS = {"add": "add", "subtract": "sub", "multiply": "mul", "true_divide": "div",
               "divide": "div", "exp": "exp", "absolute": "abs", "fabs": "abs", "rint": "rint",
               "negative": "neg", "maximum": "maximum", "minimum": "minimum", "sqrt": "sqrt",
-              "log": "log", "tanh": "tanh"}
+              "log": "log", "tanh": "tanh", "square": "square", "power": "power"}
 
 
 def _result_dtype(a: "Tile", b: "Tile") -> str:
@@ -515,8 +515,12 @@ class Tile:
             raise TraceError(f"numpy.{ufunc.__name__} ({method}) is not supported in a GPU kernel")
         if len(inputs) == 1:
             x = Tile.wrap(inputs[0])
+            if op == "square":
+                return x * x
             return Tile(op, (x,), x.shape, x.dtype_name)
         a, b = inputs
+        if op == "power":
+            return Tile.wrap(a) ** b
         if isinstance(a, Tile):
             return a._binary(b, op)
         return Tile.wrap(b)._binary(a, op, reflected=True)
@@ -535,6 +539,16 @@ class Tile:
             return x._reduce({"amax": "max", "amin": "min"}.get(name, name),
                              kwargs.get("axis", args[1] if len(args) > 1 else None),
                              kwargs.get("keepdims", False))
+        if name in ("mean", "var", "std"):
+            extra = set(kwargs) - {"axis", "keepdims", "ddof"}
+            if extra or len(args) > 2:
+                raise TraceError(f"numpy.{name}: only axis, keepdims and ddof are supported")
+            if name == "mean" and "ddof" in kwargs:
+                raise TraceError("numpy.mean takes no ddof")
+            kw = dict(kwargs)
+            if len(args) > 1:
+                kw["axis"] = args[1]
+            return getattr(Tile.wrap(args[0]), name)(**kw)
         if name == "transpose" and len(args) == 1:
             return Tile.wrap(args[0]).T
         if name == "norm" and kwargs.get("ord", args[1] if len(args) > 1 else None) is None:
@@ -557,6 +571,40 @@ class Tile:
     def max(self, axis=None, keepdims=False): return self._reduce("max", axis, keepdims)
     def min(self, axis=None, keepdims=False): return self._reduce("min", axis, keepdims)
     def sum(self, axis=None, keepdims=False): return self._reduce("sum", axis, keepdims)
+
+    # mean, var and std are spelled out the way NumPy computes them
+    # (numpy/_core/_methods.py: _mean, _var), so that the host executor and the
+    # traced program round at the same places.
+    def _count(self, axis):
+        axes = range(len(self.shape)) if axis is None else \
+            ((axis,) if isinstance(axis, int) else axis)
+        return math.prod(self.shape[a % len(self.shape)] for a in axes)
+
+    def mean(self, axis=None, keepdims=False):
+        if self.dtype_name == "float16":        # NumPy adds up fp16 data in fp32
+            total = self.astype("float32")._reduce("sum", axis, keepdims)
+            return (total / self._count(axis)).astype("float16")
+        return self._reduce("sum", axis, keepdims) / self._count(axis)
+
+    def var(self, axis=None, keepdims=False, ddof=0):
+        if self.dtype_name != "float32":
+            raise TraceError("var/std of a tile: float32 tiles only (cast first)")
+        centred = self - self._reduce("sum", axis, True) / self._count(axis)
+        return (centred * centred)._reduce("sum", axis, keepdims) / max(self._count(axis) - ddof, 0)
+
+    def std(self, axis=None, keepdims=False, ddof=0):
+        v = self.var(axis, keepdims, ddof)
+        return Tile("sqrt", (v,), v.shape, v.dtype_name)
+
+    def __pow__(self, e):
+        if isinstance(e, (int, float, np.generic)) and not isinstance(e, bool):
+            if float(e) == 2.0:
+                return self * self              # what numpy.power does for this exponent
+            if float(e) == 0.5:
+                return Tile("sqrt", (self,), self.shape, self.dtype_name)
+            if float(e) == 1.0:
+                return self
+        raise TraceError("tile ** e: only the exponents 2, 1 and 0.5 have native code")
 
     def astype(self, dt):
         name = dtype_name(dt)

@@ -710,3 +710,53 @@ def test_autotune_of_the_convolution_example():
     conv.parametrize(tp)(dx, df, out2)
     rt.set_variant("gather", 0)
     assert_allclose(out2.to_host(), conv_direct(x, f, 1), rtol=1e-4, atol=(c * hf * hf + 2) * 2.0 ** -22)
+
+
+# ---------------------------------------------------------------------------
+# bodies with reductions along rows -> hcamdLaunchRowProgram
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("rows,n", [(37, 200), (64, 4096), (9, 4104), (5, 20_003)])
+@pytest.mark.parametrize("name", ["layernorm", "rmsnorm_half", "log_softmax_t", "row_norms", "spread"])
+def test_row_reduction_bodies_match_the_simulator(name, rows, n):
+    """The same body on the GPU and on the CPU simulator.  fp32 results agree
+    to rtol 2e-5 (sums run in a different order, exp/log differ in the last
+    bit); the fp16 output of rmsnorm_half to one fp16 ulp."""
+    from test_kernel_frontend import _row_bodies, _row_case
+    host = _row_case(name, rows, n, seed=rows)
+    want = host[-1].copy()
+    with np.errstate(all="ignore"):                     # masked rows of the last group
+        _row_bodies(sim_kernel)[name](*host[:-1], want, 8)
+    out = rt.DeviceArray(host[-1].shape, host[-1].dtype).fill_bytes32(0xA5A5A5A5)
+    _row_bodies(kernel)[name](*[rt.to_device(a) for a in host[:-1]], out, 8)
+    assert rt.last_kernel_name().startswith("hcamd_row_program")
+    got = out.to_host()
+    if got.dtype == np.float16:
+        assert_allclose(got.astype(np.float32), want.astype(np.float32), rtol=1.1e-3)
+    else:
+        assert_allclose(got, want, rtol=2e-5, atol=2e-6)
+
+
+def test_softmax_with_a_temperature_is_a_row_program_and_plain_softmax_keeps_its_kernel():
+    M, N, GM = sym.M, sym.N, sym.GM
+
+    def make(deco, temperature):
+        @deco(work_shape=M, group_shape=GM)
+        def softmax(gr: CurrentGroup, a: Buffer[M, N, DT], out: Buffer[M, N, DT], gshape: GM):
+            m0, mb = gr.work_offset[0], gr.shape[0]
+            t = gr.load(a[m0:, :], shape=(mb, N))
+            if temperature != 1.0:
+                t = t / np.float32(temperature)
+            e = np.exp(t - t.max(axis=1, keepdims=True))
+            gr.store(out[m0:, :], e / e.sum(axis=1, keepdims=True))
+        return softmax
+
+    x = (np.random.default_rng(3).standard_normal((100, 1000)) * 4).astype(np.float32)
+    dx = rt.to_device(x)
+    for temperature, name in ((1.0, "hcamd_softmax"), (0.7, "hcamd_row_program")):
+        want = np.zeros_like(x)
+        with np.errstate(all="ignore"):
+            make(sim_kernel, temperature)(x, want, 8)
+        out = rt.DeviceArray(x.shape, np.float32)
+        make(kernel, temperature)(dx, out, 8)
+        assert rt.last_kernel_name().startswith(name), rt.last_kernel_name()
+        assert_allclose(out.to_host(), want, rtol=1e-5, atol=1e-30)

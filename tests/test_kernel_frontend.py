@@ -698,3 +698,209 @@ def test_groups_are_joined_only_when_that_is_exact(ctx, monkeypatch):
     want = np.zeros((8, 8))
     want[1:4], want[5:8] = a[0:3] @ b, a[4:7] @ b     # row 0 of each group reads nothing
     np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
+
+
+# ---------------------------------------------------------------------------
+# Row programs: elementwise arithmetic mixed with reductions along the rows
+# ---------------------------------------------------------------------------
+def row_stages(plan):
+    """[(kind, slot, [(opname, arg, imm)])] of a hcamdLaunchRowProgram plan."""
+    assert plan.fn is rt.hcamdLaunchRowProgram
+    names = {v: k for k, v in rt.MAP_OPS.items()}
+    kinds = {v: k for k, v in rt.ROW_KINDS.items()}
+    prog, st, n = plan.args[1], plan.args[2], plan.args[3]
+    out, pc = [], 0
+    for i in range(n):
+        out.append((kinds[st[i].kind], st[i].dst,
+                    [(names[prog[j].op], prog[j].arg, prog[j].imm)
+                     for j in range(pc, pc + st[i].nInstr)]))
+        pc += st[i].nInstr
+    return out
+
+
+def run_row_stages(stages, inputs, columns=(), out_dtype=np.float32):
+    """What hcamdLaunchRowProgram computes, in NumPy fp32 (reductions with
+    NumPy's own summation order): enough to check on the CPU that the stages
+    the front-end emits mean what the kernel body says."""
+    f = np.float32
+    rows = next(x.shape[0] for x in inputs if x.ndim == 2)
+    red = {k: c.astype(f).reshape(rows, 1) for k, c in enumerate(columns)}
+    binary = {"add": lambda a, b: a + b, "sub": lambda a, b: a - b, "mul": lambda a, b: a * b,
+              "div": lambda a, b: a / b, "max": np.maximum, "min": np.minimum,
+              "rsub": lambda a, b: b - a, "rdiv": lambda a, b: b / a}
+    unary = {"neg": np.negative, "abs": np.abs, "sqrt": np.sqrt, "rint": np.rint, "exp": np.exp,
+             "log": np.log, "tanh": np.tanh, "r16": lambda a: a.astype(np.float16).astype(f)}
+    result = None
+    with np.errstate(all="ignore"):
+        for kind, dst, program in stages:
+            stack = []
+            for name, arg, imm in program:
+                if name == "in":
+                    stack.append(inputs[arg].astype(f))
+                elif name == "red":
+                    stack.append(red[arg])
+                elif name == "const":
+                    stack.append(f(imm))
+                elif name in unary:
+                    stack.append(unary[name](stack.pop()))
+                elif name in binary:
+                    b = stack.pop()
+                    stack.append(binary[name](stack.pop(), b))
+                else:
+                    op, form = name[:-1] if name.endswith("i") else name.rsplit("_", 1)[0], name
+                    other = f(imm) if form.endswith("i") else \
+                        red[arg] if form.endswith("_red") else inputs[arg].astype(f)
+                    stack.append(binary[op](stack.pop(), other))
+            (top,) = stack
+            top = np.asarray(top, f)
+            if kind in ("sum", "max", "min"):
+                full = np.broadcast_to(top, (rows, top.shape[-1] if top.ndim == 2 else 1))
+                red[dst] = getattr(full, kind)(axis=1, keepdims=True).astype(f)
+            elif kind == "scalar":
+                red[dst] = np.broadcast_to(top, (rows, 1)).astype(f)
+            elif kind == "store":
+                result = top.astype(out_dtype)
+            else:
+                result = np.broadcast_to(top, (rows, 1)).reshape(rows).astype(out_dtype)
+    return result
+
+
+def _row_bodies(deco):
+    """Kernel bodies with reductions along rows, written against the reference's
+    API; `deco` is hc_amd's kernel or the CPU simulator's."""
+    M, N, GM = sym.M, sym.N, sym.GM
+    f = np.float32
+
+    @deco(work_shape=M, group_shape=GM)
+    def layernorm(gr: CurrentGroup, x: Buffer[M, N, DT], g: Buffer[N, DT], b: Buffer[N, DT],
+                  out: Buffer[M, N, DT], gshape: GM):
+        m0, mb = gr.work_offset[0], gr.shape[0]
+        t = gr.load(x[m0:, :], shape=(mb, N))
+        w, bias = gr.load(g[:], shape=(N,)), gr.load(b[:], shape=(N,))
+        mean = t.mean(axis=1, keepdims=True)
+        var = t.var(axis=1, keepdims=True)
+        gr.store(out[m0:, :], (t - mean) / np.sqrt(var + f(1e-5)) * w + bias)
+
+    @deco(work_shape=M, group_shape=GM)
+    def rmsnorm_half(gr: CurrentGroup, x: Buffer[M, N, DT], g: Buffer[N, DT],
+                     out: Buffer[M, N, DT], gshape: GM):
+        m0, mb = gr.work_offset[0], gr.shape[0]
+        t = gr.load(x[m0:, :], shape=(mb, N)).astype(f)
+        ms = np.mean(np.square(t), axis=1, keepdims=True)
+        gr.store(out[m0:, :], (t / np.sqrt(ms + f(1e-6)) * gr.load(g[:], shape=(N,))).astype(np.float16))
+
+    @deco(work_shape=M, group_shape=GM)
+    def log_softmax_t(gr: CurrentGroup, x: Buffer[M, N, DT], temp: Buffer[M, DT],
+                      out: Buffer[M, N, DT], gshape: GM):
+        m0, mb = gr.work_offset[0], gr.shape[0]
+        t = gr.load(x[m0:, :], shape=(mb, N))
+        s = gr.load(temp[m0:], shape=(mb,))
+        z = (t - t.max(axis=1, keepdims=True)) * s[:, None]
+        gr.store(out[m0:, :], z - np.log(np.exp(z).sum(axis=1, keepdims=True)))
+
+    @deco(work_shape=M, group_shape=GM)
+    def row_norms(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[M, DT], gshape: GM):
+        m0, mb = gr.work_offset[0], gr.shape[0]
+        t = gr.load(x[m0:, :], shape=(mb, N))
+        gr.store(out[m0:], np.sqrt((t * t).sum(axis=1)))
+
+    @deco(work_shape=M, group_shape=GM)
+    def spread(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[M, N, DT], gshape: GM):
+        m0, mb = gr.work_offset[0], gr.shape[0]
+        t = gr.load(x[m0:, :], shape=(mb, N))
+        lo, hi = t.min(axis=1), np.max(t, axis=1)
+        gr.store(out[m0:, :], (t - lo[:, None]) / (hi - lo)[:, None])
+
+    return {"layernorm": layernorm, "rmsnorm_half": rmsnorm_half, "log_softmax_t": log_softmax_t,
+            "row_norms": row_norms, "spread": spread}
+
+
+def _row_case(name, rows, n, seed=0):
+    """Host operands of a body, in argument order, the last one the output."""
+    rng = np.random.default_rng(seed)
+    f = np.float32
+    x = (rng.standard_normal((rows, n)) * 2 + 0.25).astype(f)
+    if name == "layernorm":
+        return [x, rng.standard_normal(n).astype(f), rng.standard_normal(n).astype(f),
+                np.zeros((rows, n), f)]
+    if name == "rmsnorm_half":
+        return [x.astype(np.float16), rng.standard_normal(n).astype(f), np.zeros((rows, n), np.float16)]
+    if name == "log_softmax_t":
+        return [x, rng.uniform(0.5, 2.0, rows).astype(f), np.zeros((rows, n), f)]
+    if name == "row_norms":
+        return [x, np.zeros(rows, f)]
+    return [x, np.zeros((rows, n), f)]
+
+
+def test_bodies_with_row_reductions_compile_to_row_programs(ctx):
+    from oracle.hcsim import kernel as sim_kernel
+    rows, n = 37, 200
+    gpu, sim = _row_bodies(kernel), _row_bodies(sim_kernel)
+    want_stages = {
+        # sum(x) is computed once for the mean and the variance
+        "layernorm": ["sum", "scalar", "sum", "scalar", "store"],
+        "rmsnorm_half": ["sum", "scalar", "store"],
+        "log_softmax_t": ["max", "sum", "scalar", "store"],
+        "row_norms": ["sum", "store_col"],
+        "spread": ["min", "max", "scalar", "store"],
+    }
+    for name, body in gpu.items():
+        host = _row_case(name, rows, n)
+        fake = [FakeDev(a.shape, a.dtype.name) for a in host]
+        (p,) = body.plan(*fake, 8, ctx=ctx)
+        stages = row_stages(p)
+        assert [k for k, _, _ in stages] == want_stages[name], (name, stages)
+        assert p.args[-2:] == (rows, n)
+        n_in, n_col = p.args[7], p.args[10]
+        # the stages mean what the body says: run them in NumPy, run the body
+        # on the simulator
+        tiles = [a for a in host[:-1] if not (a.ndim == 1 and a.shape[0] == rows)]
+        cols = [a for a in host[:-1] if a.ndim == 1 and a.shape[0] == rows]
+        assert (n_in, n_col) == (len(tiles), len(cols)), name
+        got = run_row_stages(stages, tiles, cols, host[-1].dtype)
+        want = host[-1].copy()
+        sim[name](*host[:-1], want, 8)
+        if host[-1].dtype == np.float16:
+            np.testing.assert_allclose(got.astype(np.float32), want.astype(np.float32), rtol=2e-3)
+        else:
+            np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-6, err_msg=name)
+    # details of one program: the row scalars are read by the operations themselves
+    (p,) = gpu["layernorm"].plan(*[FakeDev(a.shape, a.dtype.name)
+                                   for a in _row_case("layernorm", rows, n)], 8, ctx=ctx)
+    st = row_stages(p)
+    assert [i[0] for i in st[-1][2]] == ["in", "sub_red", "div_red", "mul_in", "add_in"]
+    assert st[1][2] == [("red", 0, 0.0), ("divi", 0, float(n))]
+    assert list(p.args[6][:3]) == [n, 0, 0]                 # tile, then two vectors (stride 0)
+
+
+def test_row_bodies_without_native_code_say_why(ctx):
+    M, N, GM = sym.M, sym.N, sym.GM
+
+    def body(fn, out_shape=None):
+        @kernel(work_shape=M, group_shape=GM)
+        def k(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[M, N, DT], gshape: GM):
+            m0, mb = gr.work_offset[0], gr.shape[0]
+            gr.store(out[m0:, :], fn(gr.load(x[m0:, :], shape=(mb, N))))
+        return k
+
+    x16, x32 = FakeDev((64, 128), "float16"), FakeDev((64, 128), "float32")
+    with pytest.raises(NoNativeKernel, match="cast the tile"):
+        body(lambda t: t / t.sum(axis=1, keepdims=True)).plan(x16, FakeDev((64, 128), "float16"), 8, ctx=ctx)
+    with pytest.raises(NoNativeKernel):                        # reductions down the columns
+        body(lambda t: t - t.max(axis=0, keepdims=True)).plan(x32, FakeDev((64, 128), "float32"), 8, ctx=ctx)
+    with pytest.raises(NoNativeKernel, match="row scalars"):
+        def many(t):
+            acc = t
+            for k in range(9):
+                acc = acc - (t * float(k + 1)).max(axis=1, keepdims=True)
+            return acc
+        body(many).plan(x32, FakeDev((64, 128), "float32"), 8, ctx=ctx)
+
+    # tiles that hold parts of rows
+    @kernel(work_shape=(M, N), group_shape=(8, 32))
+    def partial(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[M, N, DT]):
+        m0, n0 = gr.work_offset
+        t = gr.load(x[m0:, n0:], shape=gr.shape)
+        gr.store(out[m0:, n0:], t - t.max(axis=1, keepdims=True))
+    with pytest.raises(NoNativeKernel, match="whole rows"):
+        partial.plan(x32, FakeDev((64, 128), "float32"), ctx=ctx)
