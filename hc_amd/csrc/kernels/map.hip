@@ -893,10 +893,9 @@ struct Place {
 // past the end) and zeroed afterwards.  The choice is per wave, not per lane: a
 // load in a branch that only some lanes take would be waited for on the spot,
 // together with every load issued before it.
-__device__ __forceinline__ void load_chunk(const RowArgs &a, int i, size_t row, Place at,
+__device__ __forceinline__ void load_chunk(const RowArgs &a, int i, const char *base, Place at,
                                            u32x4 &w0, u32x4 &w1) {
   const bool f16 = (a.f16_mask >> i) & 1;
-  const char *base = static_cast<const char *>(a.in[i]) + row * a.ld[i] * (f16 ? 2 : 4);
   const bool vec = (a.vec_mask >> i) & 1; // implies at least one whole chunk per row
   const bool partial = at.n_valid != 8 && at.n_valid != 0;
   w1 = u32x4{0u, 0u, 0u, 0u}; // fp16: unused, but never a value left over from another chunk
@@ -949,6 +948,14 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
     if (k < (int)a.n_col)
       cells[k] = uniform(load_elem(a.col[k], (a.f16_mask >> (16 + k)) & 1, row));
 
+  // where this lane's row starts in every operand and in the output
+  const char *bases[kMaxIn];
+#pragma unroll
+  for (int i = 0; i < kMaxIn; ++i)
+    bases[i] = static_cast<const char *>(a.in[i]) +
+               row * a.ld[i] * (((a.f16_mask >> i) & 1) ? 2 : 4);
+  char *const orow = static_cast<char *>(a.out) + row * a.ldo * (out_f16 ? 2 : 4);
+
   uint32_t parity = 0;
 #pragma nounroll
   for (uint32_t s = 0; s < a.n_stages; ++s) {
@@ -968,13 +975,14 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
 #pragma unroll
         for (int i = 0; i < kMaxIn; ++i) {
           if ((st.load_mask >> i) & 1) {
-            load_chunk(a, i, row, at, raw.w[i][0], raw.w[i][1]);
+            load_chunk(a, i, bases[i], at, raw.w[i][0], raw.w[i][1]);
           }
         }
       }
       run_stage(a, st.begin, st.end, raw, r, reds);
+      // a wave whose lanes all hold whole chunks folds them without masks
+      const bool all_whole = __builtin_amdgcn_ballot_w64(at.n_valid != 8) == 0;
       if (kind == ST_STORE) {
-        char *orow = static_cast<char *>(a.out) + row * a.ldo * (out_f16 ? 2 : 4);
         if (((a.vec_mask >> 8) & 1) && at.n_valid == 8) {
           store_chunk(orow, out_f16, at.c, r.st[0]);
         } else {
@@ -984,17 +992,35 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
               store_elem(orow, out_f16, (size_t)at.c * 8 + e, r.st[0][e]);
         }
       } else if (kind == ST_SUM) {
+        if (all_whole) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          acc += (uint32_t)e < at.n_valid ? r.st[0][e] : 0.0f;
+          for (int e = 0; e < 8; ++e)
+            acc += r.st[0][e];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            acc += (uint32_t)e < at.n_valid ? r.st[0][e] : 0.0f;
+        }
       } else if (kind == ST_MAX) {
+        if (all_whole) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          acc = (uint32_t)e < at.n_valid ? nan_max(acc, r.st[0][e]) : acc;
+          for (int e = 0; e < 8; ++e)
+            acc = nan_max(acc, r.st[0][e]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            acc = (uint32_t)e < at.n_valid ? nan_max(acc, r.st[0][e]) : acc;
+        }
       } else if (kind == ST_MIN) {
+        if (all_whole) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          acc = (uint32_t)e < at.n_valid ? nan_min(acc, r.st[0][e]) : acc;
+          for (int e = 0; e < 8; ++e)
+            acc = nan_min(acc, r.st[0][e]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            acc = (uint32_t)e < at.n_valid ? nan_min(acc, r.st[0][e]) : acc;
+        }
       }
     }
     if (kind <= ST_MIN) {
