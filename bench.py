@@ -330,6 +330,37 @@ def make_workloads(rt, wl):
             t = _best_of(lambda: self._direct(x, f), 1)
             return t * (self.N / 4), "4 of 64 images (einsum per output position), scaled", 1
 
+    class X5(Workload):
+        """Layer normalisation with weight and bias over the rows of the C3 matrix,
+        written as a kernel body with mean and var along axis 1 and launched
+        through the @kernel front-end (a five-stage row program)."""
+
+        def setup(self, rt):
+            from hc_amd.examples import layer_norm
+            self.kernel = layer_norm()
+            (self.x,) = W.inputs_c3()
+            rng = np.random.default_rng(8)
+            self.g = rng.standard_normal(self.x.shape[1]).astype(np.float32)
+            self.b = rng.standard_normal(self.x.shape[1]).astype(np.float32)
+            return [(rt.to_device(self.x), rt.to_device(self.g), rt.to_device(self.b),
+                     rt.DeviceArray(self.x.shape, np.float32)) for _ in range(ROTATE)]
+
+        def plan(self, rt, s):
+            (p,) = self.kernel.plan_rows(*s)
+            return p
+
+        def _numpy(self, x):
+            m = x.mean(axis=1, keepdims=True)
+            return (x - m) / np.sqrt(x.var(axis=1, keepdims=True) + x.dtype.type(1e-5)) * self.g + self.b
+
+        def check(self, rt, s):
+            got, want = s[3].to_host(), self._numpy(self.x.astype(np.float64))
+            ok = np.allclose(got, want, rtol=2e-5, atol=2e-5)
+            return {"parity": "rtol 2e-5, atol 2e-5 vs fp64" if ok else "MISMATCH", "ok": bool(ok)}
+
+        def cpu(self):
+            return _best_of(lambda: self._numpy(self.x), 2), "full size, NumPy fp32", 1
+
     table = {
         "c0": C0("c0", "copy 256 MiB int32 (calibration)", "u32", "hbm", 2 * 4 * 64 * 1024 * 1024,
                  "GB/s"),
@@ -346,11 +377,13 @@ def make_workloads(rt, wl):
                  3 * 8192 * 8192 * 128, "TFLOP/s"),
         "x4": X4("x4", "implicit-GEMM convolution fp32 64x64x58x58 * 64x64x3x3 (gathered tiles)",
                  "f32", "valu", 2 * 64 * 64 * 64 * 9 * 56 * 56, "TFLOP/s"),
+        "x5": X5("x5", "row program: layer norm fp32 4096x8192 with weight and bias", "f32", "hbm",
+                 W.work_c3(), "GB/s"),
     }
     if wl == "all":
         keys = ["c1", "c2", "c3", "c4", "c5"]
     elif wl == "extra":
-        keys = ["x1", "x2", "x3", "x4"]
+        keys = ["x1", "x2", "x3", "x4", "x5"]
     else:
         keys = [wl]
     return [table[k] for k in keys]
@@ -417,7 +450,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="all", choices=["all", "c0", "c1", "c2", "c3", "c4", "c5", "extra", "x1", "x2", "x3", "x4"])
+    ap.add_argument("--workload", default="all", choices=["all", "c0", "c1", "c2", "c3", "c4", "c5", "extra", "x1", "x2", "x3", "x4", "x5"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy CPU baseline")
     ap.add_argument("--prewarm", type=float, default=PREWARM_SECONDS,
                     help="seconds of untimed device warm-up per workload")

@@ -37,7 +37,7 @@ constexpr int kDepth = 4;    // evaluation stack entries
 constexpr int kMaxIn = 4;    // operands
 constexpr int kMaxProg = 32; // instructions
 #ifndef HCAMD_MAP_WAVES
-#define HCAMD_MAP_WAVES 4 // resident waves per SIMD the flat kernel is compiled for
+#define HCAMD_MAP_WAVES 5 // resident waves per SIMD the flat kernel is compiled for
 #endif
 constexpr int kN = 8; // elements per lane per run of the program (one chunk)
 

@@ -44,3 +44,26 @@ def convolution(stride: int = 1, tile: int = 64, k_block: int = 64):
         gr.store(out[i0:, o0:, p:, q:], r, mapping=o_map)
 
     return conv
+
+
+def layer_norm(eps: float = 1e-5, rows_per_group: int = 8):
+    """out = (x - mean(x)) / sqrt(var(x) + eps) * weight + bias along the rows of
+    a float32 matrix: a body that mixes elementwise arithmetic with reductions
+    along axis 1 (the shape of python/hckernel/tests/test_examples.py:304-336,
+    the reference's softmax example).  A group owns `rows_per_group` whole rows."""
+    M, N, GM = sym.M, sym.N, sym.GM
+
+    @kernel(work_shape=M, group_shape=GM)
+    def body(gr: CurrentGroup, x: Buffer[M, N, DT], weight: Buffer[N, DT], bias: Buffer[N, DT],
+             out: Buffer[M, N, DT], gshape: GM):
+        m0, mb = gr.work_offset[0], gr.shape[0]
+        t = gr.load(x[m0:, :], shape=(mb, N))
+        w, b = gr.load(weight[:], shape=(N,)), gr.load(bias[:], shape=(N,))
+        mean = t.mean(axis=1, keepdims=True)
+        var = t.var(axis=1, keepdims=True)
+        gr.store(out[m0:, :], (t - mean) / np.sqrt(var + np.float32(eps)) * w + b)
+
+    def plan(x, weight, bias, out, **kw):
+        return body.plan(x, weight, bias, out, rows_per_group, **kw)
+    body.plan_rows = plan
+    return body
