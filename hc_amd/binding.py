@@ -879,7 +879,7 @@ class _RowCompiler(_MapCompiler):
         1-D loads of `rows` elements, constants and arithmetic on those."""
         if t.shape not in ((self.rows, 1), (self.rows,)):
             return False
-        if t.op in _ROW_REDUCE and t.attrs.get("axes") == (1,):
+        if (t.op in _ROW_REDUCE or t.op == "norm") and t.attrs.get("axes") == (1,):
             return True
         if _is(t, "load") or _is(t, "slice", 1) or _is(t, "reshape", 1):
             if self.column_load(t) is not None:
@@ -954,6 +954,13 @@ class _RowCompiler(_MapCompiler):
             if _same(uid_t, t):
                 self.slots[t.uid] = slot
                 return slot
+        if t.op == "norm" and t.attrs.get("axes") == (1,):
+            # numpy.linalg.norm along an axis is sqrt(add.reduce(x * x))
+            body = t.args[0]
+            total = (body * body)._reduce("sum", 1, t.attrs.get("keepdims", False))
+            slot = self.scalar(Tile("sqrt", (total,), total.shape, total.dtype_name))
+            self.slots[t.uid] = slot
+            return slot
         if t.op in _ROW_REDUCE and t.attrs.get("axes") == (1,):
             body = t.args[0]
             if self.klass(body) != "E":
@@ -992,7 +999,8 @@ class _RowCompiler(_MapCompiler):
             base = self._strip_views(t)
             if base.uid in self.slots:
                 return
-            if base.op in _ROW_REDUCE and base.attrs.get("axes") == (1,) or _is(base, "load"):
+            if base.op in (*_ROW_REDUCE, "norm") and base.attrs.get("axes") == (1,) or \
+                    _is(base, "load"):
                 self.scalar(base)
                 return
             t = base
@@ -1107,7 +1115,8 @@ def match_rows(dst_view, value, n_groups):
         if t.uid in seen:
             return False
         seen.add(t.uid)
-        if t.op in _ROW_REDUCE and t.attrs.get("axes") == (1,) and len(t.args[0].shape) == 2:
+        if (t.op in _ROW_REDUCE or t.op == "norm") and t.attrs.get("axes") == (1,) \
+                and len(t.args[0].shape) == 2:
             return True
         return any(has_row_reduce(a, seen) for a in t.args)
 

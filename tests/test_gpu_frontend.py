@@ -716,7 +716,8 @@ def test_autotune_of_the_convolution_example():
 # bodies with reductions along rows -> hcamdLaunchRowProgram
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("rows,n", [(37, 200), (64, 4096), (9, 4104), (5, 20_003)])
-@pytest.mark.parametrize("name", ["layernorm", "rmsnorm_half", "log_softmax_t", "row_norms", "spread"])
+@pytest.mark.parametrize("name", ["layernorm", "rmsnorm_half", "log_softmax_t", "row_norms", "spread",
+                                  "unit_rows", "log_sum_exp"])
 def test_row_reduction_bodies_match_the_simulator(name, rows, n):
     """The same body on the GPU and on the CPU simulator.  fp32 results agree
     to rtol 2e-5 (sums run in a different order, exp/log differ in the last

@@ -811,8 +811,22 @@ def _row_bodies(deco):
         lo, hi = t.min(axis=1), np.max(t, axis=1)
         gr.store(out[m0:, :], (t - lo[:, None]) / (hi - lo)[:, None])
 
+    @deco(work_shape=M, group_shape=GM)
+    def unit_rows(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[M, N, DT], gshape: GM):
+        m0, mb = gr.work_offset[0], gr.shape[0]
+        t = gr.load(x[m0:, :], shape=(mb, N))
+        gr.store(out[m0:, :], t / np.linalg.norm(t, axis=1, keepdims=True))
+
+    @deco(work_shape=M, group_shape=GM)
+    def log_sum_exp(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[M, DT], gshape: GM):
+        m0, mb = gr.work_offset[0], gr.shape[0]
+        t = gr.load(x[m0:, :], shape=(mb, N))
+        top = t.max(axis=1)
+        gr.store(out[m0:], top + np.log(np.exp(t - top[:, None]).sum(axis=-1)))
+
     return {"layernorm": layernorm, "rmsnorm_half": rmsnorm_half, "log_softmax_t": log_softmax_t,
-            "row_norms": row_norms, "spread": spread}
+            "row_norms": row_norms, "spread": spread, "unit_rows": unit_rows,
+            "log_sum_exp": log_sum_exp}
 
 
 def _row_case(name, rows, n, seed=0):
@@ -827,7 +841,7 @@ def _row_case(name, rows, n, seed=0):
         return [x.astype(np.float16), rng.standard_normal(n).astype(f), np.zeros((rows, n), np.float16)]
     if name == "log_softmax_t":
         return [x, rng.uniform(0.5, 2.0, rows).astype(f), np.zeros((rows, n), f)]
-    if name == "row_norms":
+    if name in ("row_norms", "log_sum_exp"):
         return [x, np.zeros(rows, f)]
     return [x, np.zeros((rows, n), f)]
 
@@ -843,6 +857,8 @@ def test_bodies_with_row_reductions_compile_to_row_programs(ctx):
         "log_softmax_t": ["max", "sum", "scalar", "store"],
         "row_norms": ["sum", "store_col"],
         "spread": ["min", "max", "scalar", "store"],
+        "unit_rows": ["sum", "scalar", "store"],
+        "log_sum_exp": ["max", "sum", "store_col"],
     }
     for name, body in gpu.items():
         host = _row_case(name, rows, n)
