@@ -163,47 +163,56 @@ template <int OP> __device__ __forceinline__ float unary(float a) {
   return a;
 }
 
-// Operands of one chunk, as loaded: eight fp16 in w[..][0], or eight fp32 in
-// w[..][0..1].
-struct Raw {
-  u32x4 w[kMaxIn][2];
+// Operands of one chunk of N elements, as loaded: N fp16 in w[..][0 .. N/8-1],
+// or N fp32 in w[..][0 .. N/4-1].  The kernels below work on chunks of eight;
+// so do the row programs (the chunk size is a parameter because sixteen was tried there).
+template <int N> struct RawT {
+  u32x4 w[kMaxIn][N / 4];
 };
-
-struct Stack {
-  float st[kDepth][kN];
+template <int N> struct StackT {
+  float st[kDepth][N];
 };
+using Raw = RawT<kN>;
+using Stack = StackT<kN>;
 
-__device__ __forceinline__ void unpack(const Raw &raw, int i, bool f16, float *dst) {
+template <int N>
+__device__ __forceinline__ void unpack(const RawT<N> &raw, int i, bool f16, float *dst) {
   // The empty asm statements pin the conversion to the arm that pushes the
-  // operand: hoisted out of the interpreter loop it would hold eight more
+  // operand: hoisted out of the interpreter loop it would hold N more
   // registers per operand for the whole pass.
   if (f16) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      uint32_t w = raw.w[i][0][e];
-      asm volatile("" : "+v"(w));
-      dst[2 * e] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
-      dst[2 * e + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+    for (int j = 0; j < N / 8; ++j) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        uint32_t w = raw.w[i][j][e];
+        asm volatile("" : "+v"(w));
+        dst[8 * j + 2 * e] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
+        dst[8 * j + 2 * e + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+      }
     }
   } else {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      uint32_t lo = raw.w[i][0][e], hi = raw.w[i][1][e];
-      asm volatile("" : "+v"(lo), "+v"(hi));
-      dst[e] = __builtin_bit_cast(float, lo);
-      dst[4 + e] = __builtin_bit_cast(float, hi);
+    for (int j = 0; j < N / 4; ++j) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        uint32_t w = raw.w[i][j][e];
+        asm volatile("" : "+v"(w));
+        dst[4 * j + e] = __builtin_bit_cast(float, w);
+      }
     }
   }
 }
 
-template <int SP, int OP> __device__ __forceinline__ void do_binary(Stack &r) {
+template <int SP, int OP, int N> __device__ __forceinline__ void do_binary(StackT<N> &r) {
   if constexpr (SP >= 2) {
 #pragma unroll
-    for (int e = 0; e < kN; ++e)
+    for (int e = 0; e < N; ++e)
       r.st[SP - 2][e] = binary<OP>(r.st[SP - 2][e], r.st[SP - 1][e]);
   }
 }
-template <int SP, int OP> __device__ __forceinline__ void do_imm(Stack &r, float imm) {
+template <int SP, int OP, int N>
+__device__ __forceinline__ void do_imm(StackT<N> &r, float imm) {
   if constexpr (SP >= 1) {
     // the same operation with the immediate as the second operand
     constexpr int B = OP == OP_ADDI   ? OP_ADD
@@ -215,16 +224,16 @@ template <int SP, int OP> __device__ __forceinline__ void do_imm(Stack &r, float
                       : OP == OP_RSUBI ? OP_RSUB
                                        : OP_RDIV;
 #pragma unroll
-    for (int e = 0; e < kN; ++e)
+    for (int e = 0; e < N; ++e)
       r.st[SP - 1][e] = binary<B>(r.st[SP - 1][e], imm);
   }
 }
-template <int SP, int OP>
-__device__ __forceinline__ void do_operand(Stack &r, const Raw &raw, uint32_t f16_mask,
+template <int SP, int OP, int N>
+__device__ __forceinline__ void do_operand(StackT<N> &r, const RawT<N> &raw, uint32_t f16_mask,
                                            uint32_t arg) {
   if constexpr (SP >= 1) {
     constexpr int B = OP - OP_ADD_IN + OP_ADD; // the plain binary operation
-    float t[kN];
+    float t[N];
     switch (arg) {
     case 0: unpack(raw, 0, f16_mask & 1, t); break;
     case 1: unpack(raw, 1, f16_mask & 2, t); break;
@@ -232,14 +241,14 @@ __device__ __forceinline__ void do_operand(Stack &r, const Raw &raw, uint32_t f1
     default: unpack(raw, 3, f16_mask & 8, t); break;
     }
 #pragma unroll
-    for (int e = 0; e < kN; ++e)
+    for (int e = 0; e < N; ++e)
       r.st[SP - 1][e] = binary<B>(r.st[SP - 1][e], t[e]);
   }
 }
-template <int SP, int OP> __device__ __forceinline__ void do_unary(Stack &r) {
+template <int SP, int OP, int N> __device__ __forceinline__ void do_unary(StackT<N> &r) {
   if constexpr (SP >= 1) {
 #pragma unroll
-    for (int e = 0; e < kN; ++e)
+    for (int e = 0; e < N; ++e)
       r.st[SP - 1][e] = unary<OP>(r.st[SP - 1][e]);
   }
 }
@@ -247,8 +256,8 @@ template <int SP, int OP> __device__ __forceinline__ void do_unary(Stack &r) {
 // One instruction with SP entries on the stack; returns the new stack pointer.
 // The host has verified the program, so pushes never overflow and pops never
 // underflow; the guards only keep impossible arms out of the code.
-template <int SP>
-__device__ __forceinline__ int step(Stack &r, const Raw &raw, uint32_t f16_mask,
+template <int SP, int N>
+__device__ __forceinline__ int step(StackT<N> &r, const RawT<N> &raw, uint32_t f16_mask,
                                     uint32_t op, uint32_t arg, float imm) {
   switch (op) {
   case OP_IN:
@@ -264,7 +273,7 @@ __device__ __forceinline__ int step(Stack &r, const Raw &raw, uint32_t f16_mask,
   case OP_CONST:
     if constexpr (SP < kDepth) {
 #pragma unroll
-      for (int e = 0; e < kN; ++e) r.st[SP][e] = imm;
+      for (int e = 0; e < N; ++e) r.st[SP][e] = imm;
     }
     return SP + 1;
 #define HCAMD_BIN(OP)                                                          \
@@ -801,6 +810,7 @@ namespace {
 constexpr int kMaxRed = 8;
 constexpr int kMaxStages = 8;
 constexpr int kRowProg = 64;
+constexpr int kRowN = 8; // elements per lane per run of a stage's program (16: registers cost more than the halved dispatch gains)
 enum : uint32_t {
   OP_RED = 35,     // push row scalar `arg`
   OP_ADD_RED = 36, // top = top op row scalar `arg`, in the order of OP_ADD_IN..
@@ -848,7 +858,8 @@ __device__ __forceinline__ float uniform(float x) {
 // in every wave of a row): reading one is a single readlane with the index in
 // a scalar register.
 __device__ __forceinline__ void run_stage(const RowArgs &a, uint32_t begin, uint32_t end,
-                                          const Raw &raw, Stack &r, uint32_t reds) {
+                                          const RawT<kRowN> &raw, StackT<kRowN> &r,
+                                          uint32_t reds) {
   int sp = 0;
   Instr next = a.prog[begin & (kRowProg - 1)];
   for (uint32_t pc = begin; pc < end; ++pc) {
@@ -883,44 +894,56 @@ __device__ __forceinline__ void run_stage(const RowArgs &a, uint32_t begin, uint
 // Where a lane stands in its row during pass p.
 struct Place {
   uint32_t c;       // chunk of the row (0 when the lane has none in this pass)
-  uint32_t n_valid; // elements of the chunk inside the row: 8, cols % 8, or 0
+  uint32_t n_valid; // elements of the chunk inside the row: kRowN, cols % kRowN, or 0
 };
 
-// The chunk `at` of operand i's row, as loaded: w0 (and w1 for fp32).  A wave
-// whose lanes all stand on whole chunks of 16-byte aligned rows (or on nothing)
-// uses 16-byte loads.  Any other wave reads element by element in all its
-// lanes, every load issued (from the row's first element where the column is
-// past the end) and zeroed afterwards.  The choice is per wave, not per lane: a
-// load in a branch that only some lanes take would be waited for on the spot,
-// together with every load issued before it.
+// The chunk `at` of operand i's row, as loaded.  A wave whose lanes all stand
+// on whole chunks of 16-byte aligned rows (or on nothing) uses 16-byte loads.
+// Any other wave reads element by element in all its lanes, every load issued
+// (from the row's first element where the column is past the end) and zeroed
+// afterwards.  The choice is per wave, not per lane: a load in a branch that
+// only some lanes take would be waited for on the spot, together with every
+// load issued before it.
 __device__ __forceinline__ void load_chunk(const RowArgs &a, int i, const char *base, Place at,
-                                           u32x4 &w0, u32x4 &w1) {
+                                           u32x4 (&w)[kRowN / 4]) {
   const bool f16 = (a.f16_mask >> i) & 1;
   const bool vec = (a.vec_mask >> i) & 1; // implies at least one whole chunk per row
-  const bool partial = at.n_valid != 8 && at.n_valid != 0;
-  w1 = u32x4{0u, 0u, 0u, 0u}; // fp16: unused, but never a value left over from another chunk
-  if (vec && __builtin_amdgcn_ballot_w64(partial) == 0) {
-    const u32x4 *q = reinterpret_cast<const u32x4 *>(base) + (f16 ? at.c : 2 * at.c);
-    w0 = ldg<false>(q);
-    if (!f16)
-      w1 = ldg<false>(q + 1);
-  } else {
-    uint32_t v[8];
+  const bool partial = at.n_valid != kRowN && at.n_valid != 0;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const size_t el = (uint32_t)e < at.n_valid ? (size_t)at.c * 8 + e : 0;
+  for (int j = 0; j < kRowN / 4; ++j) // never a value left over from another chunk
+    w[j] = u32x4{0u, 0u, 0u, 0u};
+  if (vec && __builtin_amdgcn_ballot_w64(partial) == 0) {
+    if (f16) {
+      const u32x4 *q = reinterpret_cast<const u32x4 *>(base) + (size_t)at.c * (kRowN / 8);
+#pragma unroll
+      for (int j = 0; j < kRowN / 8; ++j)
+        w[j] = ldg<false>(q + j);
+    } else {
+      const u32x4 *q = reinterpret_cast<const u32x4 *>(base) + (size_t)at.c * (kRowN / 4);
+#pragma unroll
+      for (int j = 0; j < kRowN / 4; ++j)
+        w[j] = ldg<false>(q + j);
+    }
+  } else {
+    uint32_t v[kRowN];
+#pragma unroll
+    for (int e = 0; e < kRowN; ++e) {
+      const size_t el = (uint32_t)e < at.n_valid ? (size_t)at.c * kRowN + e : 0;
       v[e] = f16 ? (uint32_t) reinterpret_cast<const uint16_t *>(base)[el]
                  : reinterpret_cast<const uint32_t *>(base)[el];
     }
 #pragma unroll
-    for (int e = 0; e < 8; ++e)
+    for (int e = 0; e < kRowN; ++e)
       v[e] = (uint32_t)e < at.n_valid ? v[e] : 0u;
     if (f16) {
-      w0 = u32x4{v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16),
-                 v[6] | (v[7] << 16)};
+#pragma unroll
+      for (int j = 0; j < kRowN / 8; ++j)
+        w[j] = u32x4{v[8 * j] | (v[8 * j + 1] << 16), v[8 * j + 2] | (v[8 * j + 3] << 16),
+                     v[8 * j + 4] | (v[8 * j + 5] << 16), v[8 * j + 6] | (v[8 * j + 7] << 16)};
     } else {
-      w0 = u32x4{v[0], v[1], v[2], v[3]};
-      w1 = u32x4{v[4], v[5], v[6], v[7]};
+#pragma unroll
+      for (int j = 0; j < kRowN / 4; ++j)
+        w[j] = u32x4{v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]};
     }
   }
 }
@@ -933,13 +956,13 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
   const size_t row_at = (size_t)blockIdx.x * (kThreads / LPR) + t / LPR;
   const bool row_live = row_at < a.rows;
   const size_t row = row_live ? row_at : 0; // idle lanes compute on row 0 and store nothing
-  const uint32_t whole = (uint32_t)(a.cols / 8), rem = (uint32_t)(a.cols % 8);
+  const uint32_t whole = (uint32_t)(a.cols / kRowN), rem = (uint32_t)(a.cols % kRowN);
   const uint32_t per_row = whole + (rem ? 1u : 0u);
   const bool out_f16 = (a.f16_mask >> 8) & 1;
   auto place = [&](uint32_t p) {
     const uint32_t c = p * LPR + lane;
     const bool live = row_live && p < a.passes && c < per_row;
-    return Place{live ? c : 0u, !live ? 0u : c == whole ? rem : 8u};
+    return Place{live ? c : 0u, !live ? 0u : c == whole ? rem : (uint32_t)kRowN};
   };
   if (t % kWave < kMaxRed)
     cells[t % kWave] = 0.0f;
@@ -966,59 +989,61 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
     // the row scalars, scalar k in lane k
     const uint32_t reds = __builtin_bit_cast(uint32_t, cells[t & (kMaxRed - 1)]);
     float acc = kind == ST_MAX ? -INFINITY : kind == ST_MIN ? INFINITY : 0.0f;
-    Stack r;
+    StackT<kRowN> r;
 #pragma nounroll
     for (uint32_t p = 0; p < n_pass; ++p) {
       const Place at = per_element ? place(p) : Place{0u, 0u};
-      Raw raw;
+      RawT<kRowN> raw;
       if (per_element) {
 #pragma unroll
         for (int i = 0; i < kMaxIn; ++i) {
           if ((st.load_mask >> i) & 1) {
-            load_chunk(a, i, bases[i], at, raw.w[i][0], raw.w[i][1]);
+            load_chunk(a, i, bases[i], at, raw.w[i]);
           }
         }
       }
       run_stage(a, st.begin, st.end, raw, r, reds);
       // a wave whose lanes all hold whole chunks folds them without masks
-      const bool all_whole = __builtin_amdgcn_ballot_w64(at.n_valid != 8) == 0;
+      const bool all_whole = __builtin_amdgcn_ballot_w64(at.n_valid != kRowN) == 0;
       if (kind == ST_STORE) {
-        if (((a.vec_mask >> 8) & 1) && at.n_valid == 8) {
-          store_chunk(orow, out_f16, at.c, r.st[0]);
+        if (((a.vec_mask >> 8) & 1) && at.n_valid == kRowN) {
+#pragma unroll
+          for (int j = 0; j < kRowN / 8; ++j)
+            store_chunk(orow, out_f16, (size_t)at.c * (kRowN / 8) + j, r.st[0] + 8 * j);
         } else {
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
+          for (int e = 0; e < kRowN; ++e)
             if ((uint32_t)e < at.n_valid)
-              store_elem(orow, out_f16, (size_t)at.c * 8 + e, r.st[0][e]);
+              store_elem(orow, out_f16, (size_t)at.c * kRowN + e, r.st[0][e]);
         }
       } else if (kind == ST_SUM) {
         if (all_whole) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
+          for (int e = 0; e < kRowN; ++e)
             acc += r.st[0][e];
         } else {
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
+          for (int e = 0; e < kRowN; ++e)
             acc += (uint32_t)e < at.n_valid ? r.st[0][e] : 0.0f;
         }
       } else if (kind == ST_MAX) {
         if (all_whole) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
+          for (int e = 0; e < kRowN; ++e)
             acc = nan_max(acc, r.st[0][e]);
         } else {
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
+          for (int e = 0; e < kRowN; ++e)
             acc = (uint32_t)e < at.n_valid ? nan_max(acc, r.st[0][e]) : acc;
         }
       } else if (kind == ST_MIN) {
         if (all_whole) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
+          for (int e = 0; e < kRowN; ++e)
             acc = nan_min(acc, r.st[0][e]);
         } else {
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
+          for (int e = 0; e < kRowN; ++e)
             acc = (uint32_t)e < at.n_valid ? nan_min(acc, r.st[0][e]) : acc;
         }
       }
