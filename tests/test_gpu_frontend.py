@@ -761,3 +761,34 @@ def test_softmax_with_a_temperature_is_a_row_program_and_plain_softmax_keeps_its
         make(kernel, temperature)(dx, out, 8)
         assert rt.last_kernel_name().startswith(name), rt.last_kernel_name()
         assert_allclose(out.to_host(), want, rtol=1e-5, atol=1e-30)
+
+
+def test_random_row_expressions_match_the_simulator():
+    """Random bodies mixing elementwise arithmetic and reductions along rows,
+    on the GPU and on the CPU simulator (rtol 1e-4: sums in a different order,
+    exp in the last bit, and cancellation in expressions like x - mean(x))."""
+    from test_kernel_frontend import random_row_body, random_row_expression, random_row_operands
+    rng = np.random.default_rng(77)
+    shapes = [(1, 1), (3, 7), (21, 96), (40, 513), (17, 2048), (5, 4099), (3, 9001)]
+    bound = tried = 0
+    while bound < 28:
+        expr, text, per_row = random_row_expression(rng, 3)
+        tried += 1
+        rows, n = shapes[tried % len(shapes)]
+        host = random_row_operands(rng, rows, n, per_row)
+        out = rt.DeviceArray(host[-1].shape, np.float32).fill_bytes32(0xA5A5A5A5)
+        try:
+            random_row_body(kernel, expr, per_row)(*[rt.to_device(a) for a in host[:-1]], out, 8)
+        except NoNativeKernel as exc:
+            assert any(w in str(exc) for w in ("stack", "row scalars", "operations", "passes",
+                                               "arrays")), (text, str(exc))
+            continue
+        assert rt.last_kernel_name().startswith("hcamd_row_program"), text
+        bound += 1
+        want = host[-1].copy()
+        with np.errstate(all="ignore"):
+            random_row_body(sim_kernel, expr, per_row)(*host[:-1], want, 8)
+        scale = 1.0 + float(np.abs(want).max())
+        assert_allclose(out.to_host(), want, rtol=1e-4, atol=1e-5 * scale,
+                        err_msg=f"{text} on {rows} x {n}")
+    assert tried < 90

@@ -920,3 +920,115 @@ def test_row_bodies_without_native_code_say_why(ctx):
         gr.store(out[m0:, n0:], t - t.max(axis=1, keepdims=True))
     with pytest.raises(NoNativeKernel, match="whole rows"):
         partial.plan(x32, FakeDev((64, 128), "float32"), ctx=ctx)
+
+
+def random_row_expression(rng, depth):
+    """A function of two (rows, N) tiles T, U and a vector W of N elements that
+    mixes elementwise arithmetic with reductions along axis 1, and its source
+    text.  Returns (function, text, per_row): per_row says the value has one
+    element per row.  Everything is float32 (K = numpy.float32 keeps Python
+    scalars from promoting the simulator's masked arithmetic to float64);
+    denominators are kept away from zero and exponents bounded."""
+    ops = ["+", "-", "*"]
+
+    def elem(d):
+        if d == 0 or rng.random() < 0.2:
+            return rng.choice(["T", "T", "U", "W"])
+        kind = rng.integers(0, 9)
+        x = elem(d - 1)
+        if kind <= 1:
+            return f"({x} {rng.choice(ops)} {elem(d - 1)})"
+        if kind <= 3:
+            return f"({x} {rng.choice(ops)} {scal(d - 1)})"
+        if kind == 4:
+            return f"({x} / (np.abs({scal(d - 1)}) + K(1.0)))"
+        if kind == 5:
+            return f"np.exp(-np.abs({x}))"
+        if kind == 6:
+            return f"np.sqrt(np.abs({x}))"
+        if kind == 7:
+            return f"np.maximum({x}, {scal(d - 1)})"
+        return f"({x} {rng.choice(ops + ['/'])} K({rng.choice(['0.5', '3.0', '-1.25'])}))"
+
+    def scal(d, keep="True"):
+        kind = rng.integers(0, 7) if d > 0 else 0
+        if kind <= 2:
+            inner = elem(max(d - 1, 0))
+            if "T" not in inner and "U" not in inner:
+                inner = f"(T + {inner})"                  # a reduction needs a tile under it
+            fn = rng.choice(["sum", "max", "min", "mean"])
+            return f"({inner}).{fn}(axis=1, keepdims={keep})"
+        x = scal(d - 1, keep)
+        if kind == 3:
+            return f"({x} {rng.choice(ops)} {scal(d - 1, keep)})"
+        if kind == 4:
+            return f"np.sqrt(np.abs({x}))"
+        if kind == 5:
+            return f"({x} / (np.abs({scal(d - 1, keep)}) + K(1.0)))"
+        return f"({x} {rng.choice(ops)} K({rng.choice(['0.25', '2.0'])}))"
+
+    per_row = rng.random() < 0.3
+    if per_row:
+        text = scal(depth, keep="False")
+    else:
+        text = f"({elem(depth)} {rng.choice(ops)} {scal(depth - 1)})"
+    return eval(f"lambda T, U, W: {text}", {"np": np, "K": np.float32}), text, per_row
+
+
+def random_row_body(deco, expr, per_row):
+    M, N, GM = sym.M, sym.N, sym.GM
+    if per_row:
+        @deco(work_shape=M, group_shape=GM)
+        def body(gr: CurrentGroup, x: Buffer[M, N, DT], y: Buffer[M, N, DT], v: Buffer[N, DT],
+                 out: Buffer[M, DT], gshape: GM):
+            m0, mb = gr.work_offset[0], gr.shape[0]
+            gr.store(out[m0:], expr(gr.load(x[m0:, :], shape=(mb, N)),
+                                    gr.load(y[m0:, :], shape=(mb, N)), gr.load(v[:], shape=(N,))))
+    else:
+        @deco(work_shape=M, group_shape=GM)
+        def body(gr: CurrentGroup, x: Buffer[M, N, DT], y: Buffer[M, N, DT], v: Buffer[N, DT],
+                 out: Buffer[M, N, DT], gshape: GM):
+            m0, mb = gr.work_offset[0], gr.shape[0]
+            gr.store(out[m0:, :], expr(gr.load(x[m0:, :], shape=(mb, N)),
+                                       gr.load(y[m0:, :], shape=(mb, N)), gr.load(v[:], shape=(N,))))
+    return body
+
+
+def random_row_operands(rng, rows, n, per_row):
+    f = np.float32
+    return [(rng.uniform(0.5, 2.0, (rows, n)) * rng.choice([-1.0, 1.0], (rows, n))).astype(f),
+            rng.standard_normal((rows, n)).astype(f), rng.uniform(-1.0, 1.0, n).astype(f),
+            np.zeros(rows if per_row else (rows, n), f)]
+
+
+def test_random_row_expressions_compile_to_stages_that_mean_the_same(ctx):
+    """Random bodies with reductions along rows: the stages the front-end emits,
+    run in NumPy, against the simulator running the body itself."""
+    from oracle.hcsim import kernel as sim_kernel
+    rng = np.random.default_rng(2024)
+    rows, n = 21, 96
+    bound = tried = 0
+    while bound < 40:
+        expr, text, per_row = random_row_expression(rng, 3)
+        tried += 1
+        host = random_row_operands(rng, rows, n, per_row)
+        fake = [FakeDev(a.shape, a.dtype.name) for a in host]
+        try:
+            (p,) = random_row_body(kernel, expr, per_row).plan(*fake, 8, ctx=ctx)
+        except NoNativeKernel as exc:
+            assert any(w in str(exc) for w in ("stack", "row scalars", "operations", "passes",
+                                               "arrays")), (text, str(exc))
+            continue
+        assert p.fn is rt.hcamdLaunchRowProgram, text
+        bound += 1
+        stages = row_stages(p)
+        by_ptr = {f.ptr: a for f, a in zip(fake, host)}
+        inputs = [by_ptr[p.args[4][i]] for i in range(p.args[7])]
+        assert p.args[10] == 0, text
+        got = run_row_stages(stages, inputs, (), np.float32)
+        want = host[-1].copy()
+        with np.errstate(all="ignore"):
+            random_row_body(sim_kernel, expr, per_row)(*host[:-1], want, 8)
+        scale = 1.0 + float(np.abs(want).max())
+        np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-5 * scale, err_msg=text)
+    assert tried < 120
