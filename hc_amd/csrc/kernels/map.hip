@@ -925,12 +925,19 @@ __device__ __forceinline__ void load_chunk(const RowArgs &a, int i, const char *
         w[j] = ldg<false>(q + j);
     }
   } else {
+    // The empty asm statement keeps the index arithmetic of this seldom-taken
+    // path in this path (the compiler would hoist it into every pass).
+    uint32_t first = at.c * kRowN;
+    asm volatile("" : "+v"(first));
     uint32_t v[kRowN];
+    if (f16) {
 #pragma unroll
-    for (int e = 0; e < kRowN; ++e) {
-      const size_t el = (uint32_t)e < at.n_valid ? (size_t)at.c * kRowN + e : 0;
-      v[e] = f16 ? (uint32_t) reinterpret_cast<const uint16_t *>(base)[el]
-                 : reinterpret_cast<const uint32_t *>(base)[el];
+      for (int e = 0; e < kRowN; ++e)
+        v[e] = reinterpret_cast<const uint16_t *>(base)[(uint32_t)e < at.n_valid ? first + e : 0u];
+    } else {
+#pragma unroll
+      for (int e = 0; e < kRowN; ++e)
+        v[e] = reinterpret_cast<const uint32_t *>(base)[(uint32_t)e < at.n_valid ? first + e : 0u];
     }
 #pragma unroll
     for (int e = 0; e < kRowN; ++e)

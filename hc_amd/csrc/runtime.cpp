@@ -1294,8 +1294,8 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
     dev->report("%s: leading dimension smaller than cols", who);
     return 1;
   }
-  if (cols / 8 + 1 > ((size_t)1 << 31) || rows > ((size_t)1 << 31)) {
-    dev->report("%s: more than 2^31 rows or 2^34 columns", who);
+  if (cols >= ((size_t)1 << 32) || rows > ((size_t)1 << 31)) {
+    dev->report("%s: more than 2^31 rows or 2^32 - 1 columns", who);
     return 1;
   }
   const size_t perRow = cols / 8 + (cols % 8 ? 1 : 0);
