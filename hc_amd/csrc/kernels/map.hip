@@ -807,9 +807,9 @@ __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcam
 // the reads, and the LDS footprint costs occupancy.)  Reductions add in a fixed
 // order for a given shape: results are reproducible from run to run.
 namespace {
-constexpr int kMaxRed = 8;
-constexpr int kMaxStages = 8;
-constexpr int kRowProg = 64;
+constexpr int kMaxRed = 16;
+constexpr int kMaxStages = 16;
+constexpr int kRowProg = 128;
 constexpr int kRowN = 8; // elements per lane per run of a stage's program (16: registers cost more than the halved dispatch gains)
 enum : uint32_t {
   OP_RED = 35,     // push row scalar `arg`

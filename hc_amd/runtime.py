@@ -426,7 +426,7 @@ MAP_MAX_INPUTS, MAP_MAX_INSTRS, MAP_STACK_DEPTH = 4, 32, 4
 MAP_OPS.update({"red": 35, "add_red": 36, "sub_red": 37, "mul_red": 38, "div_red": 39,
                 "max_red": 40, "min_red": 41, "rsub_red": 42, "rdiv_red": 43})
 ROW_KINDS = {"sum": 0, "max": 1, "min": 2, "scalar": 3, "store": 4, "store_col": 5}
-ROW_MAX_STAGES, ROW_MAX_SCALARS, ROW_MAX_INSTRS = 8, 8, 64
+ROW_MAX_STAGES, ROW_MAX_SCALARS, ROW_MAX_INSTRS = 16, 16, 128
 F32, F16, BF16 = 0, 1, 2
 
 

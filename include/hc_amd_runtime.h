@@ -354,9 +354,9 @@ enum {
   HCAMD_MAP_RSUB_RED = 42, /* scalar - top */
   HCAMD_MAP_RDIV_RED = 43  /* scalar / top */
 };
-#define HCAMD_ROW_MAX_STAGES 8
-#define HCAMD_ROW_MAX_SCALARS 8
-#define HCAMD_ROW_MAX_INSTRS 64
+#define HCAMD_ROW_MAX_STAGES 16
+#define HCAMD_ROW_MAX_SCALARS 16
+#define HCAMD_ROW_MAX_INSTRS 128
 typedef struct HcamdRowStage {
   uint32_t kind;   /* HcamdRowStageKind */
   uint32_t nInstr; /* instructions of this stage */

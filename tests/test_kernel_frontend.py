@@ -907,7 +907,7 @@ def test_row_bodies_without_native_code_say_why(ctx):
     with pytest.raises(NoNativeKernel, match="row scalars"):
         def many(t):
             acc = t
-            for k in range(9):
+            for k in range(17):
                 acc = acc - (t * float(k + 1)).max(axis=1, keepdims=True)
             return acc
         body(many).plan(x32, FakeDev((64, 128), "float32"), 8, ctx=ctx)
