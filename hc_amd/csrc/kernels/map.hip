@@ -834,6 +834,7 @@ struct RowArgs {
   size_t rows, cols;
   uint32_t f16_mask; // bit i: operand i is fp16; bit 8: the output; bit 16+k: column k
   uint32_t vec_mask; // bit i: rows of operand i start on 16-byte boundaries; bit 8: the output
+  uint32_t interleaved; // columns are dealt to lanes one by one (then vec_mask is 0)
   uint32_t n_col, n_stages, passes;
   Stage stage[kMaxStages];
   Instr prog[kRowProg];
@@ -892,9 +893,17 @@ __device__ __forceinline__ void run_stage(const RowArgs &a, uint32_t begin, uint
 }
 
 // Where a lane stands in its row during pass p.
+// Element e of the lane's chunk is column first + e * step of the row, inside
+// the row for e < n_valid.  Two assignments of columns to lanes exist.  With
+// step 1 a lane holds kRowN consecutive columns: the form for rows that start
+// on 16-byte boundaries in every operand, moved with 16-byte accesses.  With
+// step = the number of lanes that share the row, the lanes interleave, so that
+// the element-wise accesses that unaligned rows need are coalesced (a wave
+// reads consecutive elements); a program does not care which columns share a
+// lane as long as all operands and the output agree.
 struct Place {
-  uint32_t c;       // chunk of the row (0 when the lane has none in this pass)
-  uint32_t n_valid; // elements of the chunk inside the row: kRowN, cols % kRowN, or 0
+  uint32_t first, step;
+  uint32_t n_valid;
 };
 
 // The chunk `at` of operand i's row, as loaded.  A wave whose lanes all stand
@@ -908,18 +917,18 @@ __device__ __forceinline__ void load_chunk(const RowArgs &a, int i, const char *
                                            u32x4 (&w)[kRowN / 4]) {
   const bool f16 = (a.f16_mask >> i) & 1;
   const bool vec = (a.vec_mask >> i) & 1; // implies at least one whole chunk per row
-  const bool partial = at.n_valid != kRowN && at.n_valid != 0;
+  const bool partial = at.n_valid != kRowN && at.n_valid != 0; // never with step != 1: no vec bits
 #pragma unroll
   for (int j = 0; j < kRowN / 4; ++j) // never a value left over from another chunk
     w[j] = u32x4{0u, 0u, 0u, 0u};
   if (vec && __builtin_amdgcn_ballot_w64(partial) == 0) {
     if (f16) {
-      const u32x4 *q = reinterpret_cast<const u32x4 *>(base) + (size_t)at.c * (kRowN / 8);
+      const u32x4 *q = reinterpret_cast<const u32x4 *>(base) + at.first / 8;
 #pragma unroll
       for (int j = 0; j < kRowN / 8; ++j)
         w[j] = ldg<false>(q + j);
     } else {
-      const u32x4 *q = reinterpret_cast<const u32x4 *>(base) + (size_t)at.c * (kRowN / 4);
+      const u32x4 *q = reinterpret_cast<const u32x4 *>(base) + at.first / 4;
 #pragma unroll
       for (int j = 0; j < kRowN / 4; ++j)
         w[j] = ldg<false>(q + j);
@@ -927,17 +936,19 @@ __device__ __forceinline__ void load_chunk(const RowArgs &a, int i, const char *
   } else {
     // The empty asm statement keeps the index arithmetic of this seldom-taken
     // path in this path (the compiler would hoist it into every pass).
-    uint32_t first = at.c * kRowN;
+    uint32_t first = at.first;
     asm volatile("" : "+v"(first));
     uint32_t v[kRowN];
     if (f16) {
 #pragma unroll
       for (int e = 0; e < kRowN; ++e)
-        v[e] = reinterpret_cast<const uint16_t *>(base)[(uint32_t)e < at.n_valid ? first + e : 0u];
+        v[e] = reinterpret_cast<const uint16_t *>(
+            base)[(uint32_t)e < at.n_valid ? first + e * at.step : 0u];
     } else {
 #pragma unroll
       for (int e = 0; e < kRowN; ++e)
-        v[e] = reinterpret_cast<const uint32_t *>(base)[(uint32_t)e < at.n_valid ? first + e : 0u];
+        v[e] = reinterpret_cast<const uint32_t *>(
+            base)[(uint32_t)e < at.n_valid ? first + e * at.step : 0u];
     }
 #pragma unroll
     for (int e = 0; e < kRowN; ++e)
@@ -966,10 +977,18 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
   const uint32_t whole = (uint32_t)(a.cols / kRowN), rem = (uint32_t)(a.cols % kRowN);
   const uint32_t per_row = whole + (rem ? 1u : 0u);
   const bool out_f16 = (a.f16_mask >> 8) & 1;
+  const uint32_t cols = (uint32_t)a.cols;
   auto place = [&](uint32_t p) {
+    if (a.interleaved) {
+      const uint32_t first = p * (LPR * kRowN) + lane;
+      const bool live = row_live && first < cols;
+      const uint32_t n = (cols - first + LPR - 1) / LPR;
+      return Place{live ? first : 0u, (uint32_t)LPR,
+                   !live ? 0u : n < (uint32_t)kRowN ? n : (uint32_t)kRowN};
+    }
     const uint32_t c = p * LPR + lane;
-    const bool live = row_live && p < a.passes && c < per_row;
-    return Place{live ? c : 0u, !live ? 0u : c == whole ? rem : (uint32_t)kRowN};
+    const bool live = row_live && c < per_row;
+    return Place{live ? c * kRowN : 0u, 1u, !live ? 0u : c == whole ? rem : (uint32_t)kRowN};
   };
   if (t % kWave < kMaxRed)
     cells[t % kWave] = 0.0f;
@@ -999,7 +1018,7 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
     StackT<kRowN> r;
 #pragma nounroll
     for (uint32_t p = 0; p < n_pass; ++p) {
-      const Place at = per_element ? place(p) : Place{0u, 0u};
+      const Place at = per_element ? place(p) : Place{0u, 1u, 0u};
       RawT<kRowN> raw;
       if (per_element) {
 #pragma unroll
@@ -1016,12 +1035,12 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
         if (((a.vec_mask >> 8) & 1) && at.n_valid == kRowN) {
 #pragma unroll
           for (int j = 0; j < kRowN / 8; ++j)
-            store_chunk(orow, out_f16, (size_t)at.c * (kRowN / 8) + j, r.st[0] + 8 * j);
+            store_chunk(orow, out_f16, at.first / 8 + j, r.st[0] + 8 * j);
         } else {
 #pragma unroll
           for (int e = 0; e < kRowN; ++e)
             if ((uint32_t)e < at.n_valid)
-              store_elem(orow, out_f16, (size_t)at.c * kRowN + e, r.st[0][e]);
+              store_elem(orow, out_f16, at.first + e * at.step, r.st[0][e]);
         }
       } else if (kind == ST_SUM) {
         if (all_whole) {

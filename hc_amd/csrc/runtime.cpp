@@ -1115,6 +1115,15 @@ int launchMap(OlQueue q, bool sum, const HcamdMapInstr *prog, size_t nInstr,
     return launch1d(queue, "map", sum ? "hcamd_map_sum_rows" : "hcamd_map_rows", groups,
                     threads, args);
   }
+  // Windows with fp16 operands whose rows are not 16-byte aligned: the row-program
+  // kernel run as a single store stage reads them coalesced with 32-bit index
+  // arithmetic, about twice as fast as the element-wise kernel below, which
+  // stays for fp32 (where it is the faster one) and under variant 1 of "map".
+  if (!sum && a.f16_mask != 0 && variantOf("map") != 1) {
+    const HcamdRowStage whole = {HCAMD_ROW_STORE, static_cast<uint32_t>(nInstr), 0};
+    return hcamdLaunchRowProgram(q, prog, &whole, 1, inputs, inputTypes, inputLd, nInputs,
+                                 nullptr, nullptr, 0, out, outType, ldo, rows, cols);
+  }
   Kernel *k = builtinKernel(dev, "map",
                             sum ? "hcamd_map_sum_strided" : "hcamd_map_strided");
   if (!k)
@@ -1173,7 +1182,7 @@ struct RowArgs {
   size_t ld[kMapMaxIn];
   size_t ldo;
   size_t rows, cols;
-  uint32_t f16Mask, vecMask;
+  uint32_t f16Mask, vecMask, interleaved;
   uint32_t nCol, nStages, passes;
   RowStageDev stage[HCAMD_ROW_MAX_STAGES];
   HcamdMapInstr prog[HCAMD_ROW_MAX_INSTRS];
@@ -1344,8 +1353,18 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
   a.nCol = static_cast<uint32_t>(nColumns);
   a.nStages = static_cast<uint32_t>(nStages);
   a.passes = static_cast<uint32_t>(passes);
-  for (size_t s = 0; s < nStages; ++s)
+  uint32_t used = 0;
+  for (size_t s = 0; s < nStages; ++s) {
     a.stage[s].loadMask = static_cast<uint8_t>(usedIn[s]);
+    used |= usedIn[s];
+  }
+  // 16-byte accesses need every operand in use and a stored tile to allow them;
+  // otherwise the columns are dealt to the lanes one by one and every access
+  // is element-wise but coalesced.
+  if ((used & ~a.vecMask & 0xffu) || (storesTile && !((a.vecMask >> 8) & 1))) {
+    a.vecMask = 0;
+    a.interleaved = 1;
+  }
   Kernel *k = builtinKernel(dev, "map", lanesPerRow == 64 ? "hcamd_row_program_w64"
                                                          : "hcamd_row_program_w256");
   if (!k)

@@ -565,13 +565,21 @@ def test_map_window_of_larger_arrays_leaves_the_rest_untouched(ctx):
     dbig = [dev(x) for x in big]
     out = poisoned((40, 1040), np.float16)
     views = [_View(x, (rows, cols), 0, (1100, 1)) for x in dbig]
-    rt.plan_map(FMA_PROGRAM, views, _View(out, (rows, cols), 0, (1040, 1))).launch(sync=True)
-    assert rt.last_kernel_name() == "hcamd_map_strided"
-    got = out.to_host()
-    assert_array_equal(got[:rows, :cols].view(np.uint16), cf.np_fma_f16(a, b, c).view(np.uint16))
-    p = poison_value(np.float16)
-    assert (got[rows:].view(np.uint16) == p.view(np.uint16)).all()
-    assert (got[:, cols:].view(np.uint16) == p.view(np.uint16)).all()
+    # fp16 rows that do not start on 16-byte boundaries: the row-program kernel
+    # with interleaved lanes by default, the element-wise kernel as variant 1
+    for variant, name in ((0, "hcamd_row_program_w64"), (1, "hcamd_map_strided")):
+        rt.set_variant("map", variant)
+        out = poisoned((40, 1040), np.float16)
+        try:
+            rt.plan_map(FMA_PROGRAM, views, _View(out, (rows, cols), 0, (1040, 1))).launch(sync=True)
+        finally:
+            rt.set_variant("map", 0)
+        assert rt.last_kernel_name() == name
+        got = out.to_host()
+        assert_array_equal(got[:rows, :cols].view(np.uint16), cf.np_fma_f16(a, b, c).view(np.uint16))
+        p = poison_value(np.float16)
+        assert (got[rows:].view(np.uint16) == p.view(np.uint16)).all()
+        assert (got[:, cols:].view(np.uint16) == p.view(np.uint16)).all()
 
 
 @pytest.mark.parametrize("cols", [1, 5, 8, 9, 1031, 1032, 2049])

@@ -149,6 +149,46 @@ def test_windows_of_larger_arrays_and_untouched_surroundings(ctx):
         assert (got.view(np.uint32)[mask] == POISON32).all()
 
 
+@pytest.mark.parametrize("cols,ld", [(7, 9), (513, 515), (1003, 1011), (5001, 5003), (70_001, 70_003)])
+def test_fp16_rows_off_16_byte_boundaries_interleave_the_lanes(ctx, cols, ld):
+    """Rows of fp16 that start on odd multiples of 2 bytes: columns are dealt to
+    the lanes one by one (one pass and several, one wave per row and four).  A
+    stored tile and a per-row sum, bit for bit / within the fp32 sum bound, and
+    nothing touched outside the window."""
+    rows = 11
+    rng = np.random.default_rng(cols)
+    x = rng.standard_normal((rows, cols)).astype(np.float16)
+    y = rng.standard_normal((rows, cols)).astype(np.float16)
+    bigs = []
+    for src in (x, y):
+        big = np.full((rows + 2, ld), np.nan, np.float16)
+        big[1:rows + 1, 1:1 + cols] = src
+        bigs.append(rt.to_device(big))
+    views = [_View(b, (rows, cols), ld + 1, (ld, 1)) for b in bigs]
+    out = poisoned((rows + 2, ld + 1), np.float16)
+    tile = [I("in", 0), I("mul_in", 1), I("add_in", 0)]
+    rt.plan_row_program([("store", 0, tile)], views,
+                        _View(out, (rows, cols), ld + 2, (ld + 1, 1))).launch(sync=True)
+    say("fp16 interleaved", cols, rt.last_kernel_name())
+    x32, y32 = x.astype(np.float32), y.astype(np.float32)
+    prod = x32 * y32                                   # fp32 arithmetic, one rounding at the store
+    want = (prod + x32).astype(np.float16)
+    flat = out.to_host().reshape(-1)
+    starts = [(r + 1) * (ld + 1) + 1 for r in range(rows)]
+    got = np.stack([flat[s0:s0 + cols] for s0 in starts])
+    assert_array_equal(got.view(np.uint16), want.view(np.uint16))
+    mask = np.ones(flat.shape, bool)
+    for s0 in starts:
+        mask[s0:s0 + cols] = False
+    assert (flat.view(np.uint16)[mask] == (POISON32 & 0xFFFF)).all()
+    sums = poisoned((rows,), np.float32)
+    rt.plan_row_program([("sum", 0, [I("in", 0), I("mul_in", 1)]), ("store_col", 0, [I("red", 0)])],
+                        views, sums).launch(sync=True)
+    p64 = prod.astype(np.float64)
+    assert_allclose(sums.to_host(), p64.sum(axis=1), rtol=0,
+                    atol=cols * 2.0 ** -24 * np.abs(p64).sum(axis=1).max() + 1e-30)
+
+
 def test_special_values_follow_numpy(ctx):
     x = np.zeros((6, 600), np.float32)
     x[0, 5] = np.nan                    # NaN reaches every result of its row only
