@@ -777,6 +777,205 @@ __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcam
   map_rows<true>(a, n_in);
 }
 
+// ---- reductions along columns -------------------------------------------------------
+// out[c] = post(fold over the rows r of f(in0[r][c], ...)) for a rows x cols
+// window: f is the map program, the fold is a sum, a NaN-propagating maximum or
+// minimum, and post is a second short program whose operand 0 is the folded
+// value (the division of a mean, the square root of a norm).
+//
+// A lane owns one chunk of eight consecutive columns and walks down the rows, so
+// a wave reads 64 neighbouring chunks of one row at a time (16-byte accesses
+// where every row of an operand starts on a 16-byte boundary, element accesses
+// otherwise; an operand with leading dimension 0 is a vector that every row
+// uses).  The four waves of a workgroup take every fourth row of the
+// workgroup's band of rows and meet in LDS.  blockIdx.x numbers blocks of 64
+// chunks, blockIdx.y bands of rows: with more than one band the folded values go
+// to partial[band][column] (fp32, `cols_pad` per band) and a second launch of
+// this kernel folds the bands, as the rows of an fp32 operand, in the same
+// fixed order; the launch with one band runs `post` and stores.  Nothing is
+// atomic: results are the same from run to run.
+namespace {
+constexpr int kPostProg = 8;
+enum : uint32_t { COL_SUM = 0, COL_MAX = 1, COL_MIN = 2 };
+struct ColArgs {
+  float *partial;       // bands x cols_pad, used when gridDim.y > 1
+  uint32_t cols_pad;    // multiple of 8, at least cols
+  uint32_t band;        // rows per band
+  uint32_t kind;
+  uint32_t vec_mask;    // bit i: operand i may be read 16 bytes at a time; bit 8: out written so
+  uint32_t n_post;
+  Instr post[kPostProg];
+};
+
+__device__ __forceinline__ void run_post(const ColArgs &c, const Raw &raw, Stack &r) {
+  int sp = 0;
+  Instr next = c.post[0];
+  for (uint32_t pc = 0; pc < c.n_post; ++pc) {
+    const Instr cur = next;
+    next = c.post[(pc + 1) & (kPostProg - 1)];
+    const uint32_t op = cur.op, arg = cur.arg;
+    const float imm = cur.imm;
+    switch (sp) {
+    case 0: sp = step<0>(r, raw, 0u, op, arg, imm); break;
+    case 1: sp = step<1>(r, raw, 0u, op, arg, imm); break;
+    case 2: sp = step<2>(r, raw, 0u, op, arg, imm); break;
+    case 3: sp = step<3>(r, raw, 0u, op, arg, imm); break;
+    default: sp = step<4>(r, raw, 0u, op, arg, imm); break;
+    }
+  }
+}
+
+__device__ __forceinline__ float col_fold(uint32_t kind, float a, float b) {
+  return kind == COL_SUM ? a + b : kind == COL_MAX ? nan_max(a, b) : nan_min(a, b);
+}
+
+// NIN: operands the kernel is compiled for; U: rows a wave has in flight (their
+// loads are issued together, then the program runs on one row after the other:
+// fewer operands leave registers for more rows).
+template <int NIN, int U>
+__device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, const uint32_t n_in) {
+  constexpr int kWaves = kThreads / kWave;
+  __shared__ float slots[kWaves - 1][kWave][kN + 1];
+  const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const uint32_t cols = (uint32_t)a.cols, rows = (uint32_t)a.rows;
+  const uint32_t chunk = blockIdx.x * kWave + lane;
+  const uint32_t first = chunk * kN;
+  const uint32_t n_valid =
+      first >= cols ? 0u : cols - first < (uint32_t)kN ? cols - first : (uint32_t)kN;
+  const uint32_t row_begin = blockIdx.y * c.band;
+  const uint32_t row_end = row_begin + c.band < rows ? row_begin + c.band : rows;
+  const float identity =
+      c.kind == COL_SUM ? 0.0f : c.kind == COL_MAX ? -__builtin_inff() : __builtin_inff();
+  float acc[kN];
+#pragma unroll
+  for (int e = 0; e < kN; ++e)
+    acc[e] = identity;
+  // a wave whose lanes all hold whole chunks takes the 16-byte path for the
+  // operands that allow it
+  const bool all_whole = __builtin_amdgcn_ballot_w64(n_valid != (uint32_t)kN) == 0;
+  Raw raw;
+  Stack r;
+#pragma nounroll
+  for (uint32_t row0 = row_begin + wave; row0 < row_end; row0 += kWaves * U) {
+    u32x4 staged[NIN][U][2];
+#pragma unroll
+    for (int i = 0; i < NIN; ++i)
+      if (i < (int)n_in) {
+        const bool f16 = (a.f16_mask >> i) & 1;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t row = row0 + u * kWaves;
+          if (row < row_end) {
+            const char *base =
+                static_cast<const char *>(a.in[i]) + (size_t)row * a.ld[i] * (f16 ? 2 : 4);
+            if (((c.vec_mask >> i) & 1) && all_whole) {
+              const u32x4 *q = reinterpret_cast<const u32x4 *>(base) + (f16 ? chunk : 2 * chunk);
+              staged[i][u][0] = ldg<true>(q);
+              if (!f16)
+                staged[i][u][1] = ldg<true>(q + 1);
+            } else {
+              uint32_t v[kN];
+#pragma unroll
+              for (int e = 0; e < kN; ++e) {
+                const uint32_t at = (uint32_t)e < n_valid ? first + e : 0u;
+                v[e] = f16 ? (uint32_t) reinterpret_cast<const uint16_t *>(base)[at]
+                           : reinterpret_cast<const uint32_t *>(base)[at];
+              }
+              if (f16) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                  staged[i][u][0][e] = v[2 * e] | (v[2 * e + 1] << 16);
+              } else {
+#pragma unroll
+                for (int e = 0; e < kN; ++e)
+                  staged[i][u][e / 4][e % 4] = v[e];
+              }
+            }
+          }
+        }
+      }
+#pragma nounroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int i = 0; i < NIN; ++i) {
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          raw.w[i][w] = staged[i][0][w];
+#pragma unroll
+          for (int k = 0; k + 1 < U; ++k)
+            staged[i][k][w] = staged[i][k + 1][w];
+        }
+      }
+      run_program(a, raw, a.f16_mask, r);
+      if (row0 + u * kWaves < row_end) {
+#pragma unroll
+        for (int e = 0; e < kN; ++e)
+          acc[e] = col_fold(c.kind, acc[e], r.st[0][e]);
+      }
+    }
+  }
+  // waves 1.. park their values, wave 0 folds them in wave order
+  if (wave != 0) {
+#pragma unroll
+    for (int e = 0; e < kN; ++e)
+      slots[wave - 1][lane][e] = acc[e];
+  }
+  __syncthreads();
+  if (wave != 0)
+    return;
+#pragma unroll
+  for (int w = 0; w < kWaves - 1; ++w)
+#pragma unroll
+    for (int e = 0; e < kN; ++e)
+      acc[e] = col_fold(c.kind, acc[e], slots[w][lane][e]);
+  if (gridDim.y > 1) {
+    if (n_valid) {
+      float *dst = c.partial + (size_t)blockIdx.y * c.cols_pad + first;
+      f32x4 lo, hi;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        lo[e] = acc[e];
+        hi[e] = acc[4 + e];
+      }
+      *reinterpret_cast<f32x4 *>(dst) = lo;
+      *reinterpret_cast<f32x4 *>(dst + 4) = hi;
+    }
+    return;
+  }
+  if (c.n_post) {
+#pragma unroll
+    for (int e = 0; e < kN; ++e)
+      raw.w[0][e / 4][e % 4] = __builtin_bit_cast(uint32_t, acc[e]);
+    run_post(c, raw, r);
+  } else {
+#pragma unroll
+    for (int e = 0; e < kN; ++e)
+      r.st[0][e] = acc[e];
+  }
+  const bool out_f16 = (a.f16_mask >> 8) & 1;
+  if (((c.vec_mask >> 8) & 1) && n_valid == (uint32_t)kN) {
+    store_chunk(a.out, out_f16, chunk, r.st[0]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < kN; ++e)
+      if ((uint32_t)e < n_valid)
+        store_elem(a.out, out_f16, (size_t)first + e, r.st[0][e]);
+  }
+}
+} // namespace
+
+// Four waves per SIMD: the eight running values per lane on top of the
+// interpreter's registers spill at five.
+#define HCAMD_REDUCE_COLS(NAME, NIN, U)                                        \
+  extern "C" __global__ __launch_bounds__(256) __attribute__((                 \
+      amdgpu_waves_per_eu(4, 4))) void                                         \
+  NAME(const MapArgs a, const ColArgs c, const uint32_t n_in) {                \
+    reduce_cols<NIN, U>(a, c, n_in);                                           \
+  }
+HCAMD_REDUCE_COLS(hcamd_map_reduce_cols_n4u1, 4, 1)
+HCAMD_REDUCE_COLS(hcamd_map_reduce_cols_n2u2, 2, 2)
+HCAMD_REDUCE_COLS(hcamd_map_reduce_cols_n1u4, 1, 4)
+
 // ---- row programs ---------------------------------------------------------------
 // Bodies that mix elementwise arithmetic with reductions along the rows of a
 // tile (normalisations, softmax-like expressions, row sums): a list of stages,

@@ -1170,6 +1170,204 @@ int hcamdLaunchMapSum(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
 }
 
 namespace {
+// Second argument block of the column-reduction kernels (device layout).
+struct ColArgs {
+  float *partial;
+  uint32_t colsPad, band, kind, vecMask, nPost;
+  HcamdMapInstr post[HCAMD_COLS_MAX_POST];
+};
+
+// Stack discipline of a map program: within bounds, one value left, operands
+// below nInputs.
+bool mapProgramOk(Device *dev, const char *who, const HcamdMapInstr *prog, size_t nInstr,
+                  size_t nInputs) {
+  int sp = 0;
+  for (size_t i = 0; i < nInstr; ++i) {
+    int pops, pushes;
+    mapStackEffect(prog[i].op, pops, pushes);
+    if (pops < 0) {
+      dev->report("%s: unknown opcode %u at %zu", who, prog[i].op, i);
+      return false;
+    }
+    const bool readsOperand =
+        prog[i].op == HCAMD_MAP_IN ||
+        (prog[i].op >= HCAMD_MAP_ADD_IN && prog[i].op <= HCAMD_MAP_RDIV_IN);
+    if (readsOperand && prog[i].arg >= nInputs) {
+      dev->report("%s: operand %u at %zu (only %zu given)", who, prog[i].arg, i, nInputs);
+      return false;
+    }
+    if (sp < pops) {
+      dev->report("%s: stack underflow at %zu", who, i);
+      return false;
+    }
+    sp += pushes - pops;
+    if (sp > kMapDepth) {
+      dev->report("%s: stack deeper than %d at %zu", who, kMapDepth, i);
+      return false;
+    }
+  }
+  if (sp != 1) {
+    dev->report("%s: program leaves %d values, expected 1", who, sp);
+    return false;
+  }
+  return true;
+}
+
+// Bands of rows a column reduction is cut into, so that the launch has a few
+// workgroups per compute unit however narrow the window is; 1 = one launch.
+void colBands(Device *dev, size_t rows, size_t cols, size_t &bands, size_t &band) {
+  const size_t blocks = ceilDiv(ceilDiv(cols, (size_t)8), (size_t)64);
+  const size_t wanted = ceilDiv((size_t)computeUnitsOf(dev) * 6, blocks);
+  bands = std::max(std::min(wanted, rows / 64), (size_t)1);
+  band = ceilDiv(ceilDiv(rows, bands), (size_t)16) * 16; // whole turns of 4 waves x 4 rows
+  bands = ceilDiv(rows, band);
+}
+} // namespace
+
+size_t hcamdMapReduceColsWorkspace(OlQueue q, size_t rows, size_t cols) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue || rows == 0 || cols == 0)
+    return 0;
+  size_t bands, band;
+  colBands(queue->device, rows, cols, bands, band);
+  return bands > 1 ? bands * ceilDiv(cols, (size_t)8) * 8 * sizeof(float) : 0;
+}
+
+int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, size_t nInstr,
+                             const HcamdMapInstr *post, size_t nPost,
+                             const void *const *inputs, const int *inputTypes,
+                             const size_t *inputLd, size_t nInputs, void *out, int outType,
+                             size_t rows, size_t cols, void *workspace,
+                             size_t workspaceBytes) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  const char *who = "hcamdLaunchMapReduceCols";
+  if (kind != HCAMD_COLS_SUM && kind != HCAMD_COLS_MAX && kind != HCAMD_COLS_MIN) {
+    dev->report("%s: unknown reduction %d", who, kind);
+    return 1;
+  }
+  if (!prog || nInstr == 0 || nInstr > kMapMaxProg || nPost > HCAMD_COLS_MAX_POST ||
+      (nPost && !post)) {
+    dev->report("%s: programs of %zu and %zu instructions (1..%zu and 0..%d allowed)", who,
+                nInstr, nPost, kMapMaxProg, HCAMD_COLS_MAX_POST);
+    return 1;
+  }
+  if (nInputs == 0 || nInputs > kMapMaxIn || !inputs || !inputTypes || !inputLd) {
+    dev->report("%s: %zu operands (1..%zu)", who, nInputs, kMapMaxIn);
+    return 1;
+  }
+  auto typeOk = [](int t) { return t == HCAMD_F32 || t == HCAMD_F16; };
+  if (!typeOk(outType)) {
+    dev->report("%s: unsupported output type %d", who, outType);
+    return 1;
+  }
+  if (!mapProgramOk(dev, who, prog, nInstr, nInputs) ||
+      (nPost && !mapProgramOk(dev, who, post, nPost, 1)))
+    return 1;
+  if (cols == 0)
+    return 0;
+  if (rows == 0) {
+    dev->report("%s: no rows to reduce", who);
+    return 1;
+  }
+  if (rows >= ((size_t)1 << 32) || cols > ((size_t)1 << 32) - 8) {
+    dev->report("%s: window of %zu x %zu (below 2^32 each)", who, rows, cols);
+    return 1;
+  }
+  if (!out) {
+    dev->report("%s: null pointer", who);
+    return 1;
+  }
+  MapArgs a{};
+  ColArgs c{};
+  for (size_t i = 0; i < nInputs; ++i) {
+    if (!inputs[i]) {
+      dev->report("%s: null pointer", who);
+      return 1;
+    }
+    if (!typeOk(inputTypes[i])) {
+      dev->report("%s: unsupported operand type %d", who, inputTypes[i]);
+      return 1;
+    }
+    // leading dimension 0: a vector of cols elements that every row uses
+    if (inputLd[i] != 0 && rows > 1 && inputLd[i] < cols) {
+      dev->report("%s: leading dimension smaller than cols", who);
+      return 1;
+    }
+    a.in[i] = inputs[i];
+    a.ld[i] = inputLd[i];
+    const size_t size = inputTypes[i] == HCAMD_F16 ? 2 : 4;
+    if (inputTypes[i] == HCAMD_F16)
+      a.f16_mask |= 1u << i;
+    if (aligned16(inputs[i]) && (inputLd[i] * size) % 16 == 0)
+      c.vecMask |= 1u << i;
+  }
+  size_t bands, band;
+  colBands(dev, rows, cols, bands, band);
+  const size_t colsPad = ceilDiv(cols, (size_t)8) * 8;
+  if (bands > 1 && (!workspace || !aligned16(workspace) ||
+                    workspaceBytes < bands * colsPad * sizeof(float))) {
+    dev->report("%s: workspace of %zu bytes, 16-byte aligned, needed (%zu given)", who,
+                bands * colsPad * sizeof(float), workspaceBytes);
+    return 1;
+  }
+  const size_t blocks = ceilDiv(colsPad / 8, (size_t)64);
+  auto launchOne = [&](MapArgs &ma, ColArgs &ca, size_t nIn, size_t nBands) {
+    const char *name = nIn <= 1   ? "hcamd_map_reduce_cols_n1u4"
+                       : nIn <= 2 ? "hcamd_map_reduce_cols_n2u2"
+                                  : "hcamd_map_reduce_cols_n4u1";
+    Kernel *k = builtinKernel(dev, "map", name);
+    if (!k)
+      return 1;
+    uint32_t n = static_cast<uint32_t>(nIn);
+    void *args[] = {&ma, &ca, &n};
+    const size_t grid[3] = {blocks, nBands, 1}, block[3] = {256, 1, 1};
+    return launch(queue, k, grid, block, args, 0);
+  };
+  auto finish = [&](MapArgs &ma, ColArgs &ca) {
+    ma.out = out;
+    if (outType == HCAMD_F16)
+      ma.f16_mask |= 1u << 8;
+    if (aligned16(out))
+      ca.vecMask |= 1u << 8;
+    ca.nPost = static_cast<uint32_t>(nPost);
+    if (nPost)
+      std::memcpy(ca.post, post, nPost * sizeof(HcamdMapInstr));
+  };
+  a.rows = rows;
+  a.cols = cols;
+  a.n_instr = static_cast<uint32_t>(nInstr);
+  std::memcpy(a.prog, prog, nInstr * sizeof(HcamdMapInstr));
+  c.kind = static_cast<uint32_t>(kind);
+  c.colsPad = static_cast<uint32_t>(colsPad);
+  c.band = static_cast<uint32_t>(band);
+  if (bands == 1) {
+    finish(a, c);
+    return launchOne(a, c, nInputs, 1);
+  }
+  c.partial = static_cast<float *>(workspace);
+  if (int rc = launchOne(a, c, nInputs, bands))
+    return rc;
+  // the bands are the rows of an fp32 operand, folded the same way
+  MapArgs a2{};
+  ColArgs c2{};
+  a2.in[0] = workspace;
+  a2.ld[0] = colsPad;
+  a2.rows = bands;
+  a2.cols = cols;
+  a2.n_instr = 1;
+  a2.prog[0].op = HCAMD_MAP_IN;
+  c2.kind = c.kind;
+  c2.colsPad = c.colsPad;
+  c2.band = static_cast<uint32_t>(bands);
+  c2.vecMask = 1u;
+  finish(a2, c2);
+  return launchOne(a2, c2, 1, 1);
+}
+
+namespace {
 // Argument block of the row-program kernels (the same layout as in the device code).
 struct RowStageDev {
   uint16_t begin, end;

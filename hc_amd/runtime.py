@@ -109,6 +109,11 @@ hcamdLaunchPairwiseDistF32 = _sig(_rt, "hcamdLaunchPairwiseDistF32", _int, _vp, 
 hcamdLaunchMapSum = _sig(_rt, "hcamdLaunchMapSum", _int, _vp, C.POINTER(MapInstr), _sz,
                          C.POINTER(_vp), C.POINTER(_int), _sz_p, _sz, _vp, _sz, _sz)
 
+hcamdMapReduceColsWorkspace = _sig(_rt, "hcamdMapReduceColsWorkspace", _sz, _vp, _sz, _sz)
+hcamdLaunchMapReduceCols = _sig(_rt, "hcamdLaunchMapReduceCols", _int, _vp, _int,
+                                C.POINTER(MapInstr), _sz, C.POINTER(MapInstr), _sz,
+                                C.POINTER(_vp), C.POINTER(_int), _sz_p, _sz, _vp, _int, _sz, _sz,
+                                _vp, _sz)
 
 
 class RowStage(C.Structure):
@@ -495,6 +500,67 @@ def plan_map_sum(program, inputs, cell, index: int = 0, types=None) -> Plan:
     return Plan(ctx, hcamdLaunchMapSum,
                 (ctx.queue, prog, len(program), ptrs, tys, lds, n_in, mc.ptr + 4 * index,
                  rows, cols), "hcamdLaunchMapSum", (arrays, cell, prog, ptrs, tys, lds))
+
+
+COLS_KINDS = {"sum": 0, "max": 1, "min": 2}
+COLS_MAX_POST = 8
+
+
+def plan_map_reduce_cols(kind, program, inputs, out, post=(), types=None) -> Plan:
+    """out[c] = post(fold over the rows of f(inputs...)) (see
+    hcamdLaunchMapReduceCols).  `kind` is "sum", "max" or "min"; `program` and
+    `post` are map programs ((opname, arg, imm) triples; `post` reads the folded
+    value as operand 0).  `inputs` are rows x cols arrays, or 1-D arrays of
+    cols elements that every row uses; `out` holds cols contiguous elements.
+    The workspace the launch needs is allocated here, once, with the plan."""
+    inputs = list(inputs)
+    ctx = _ctx_of(*inputs, out)
+    mo = as_memref(out)
+    cols = 1
+    for n in mo.shape:
+        cols *= n
+    if not mo.is_contiguous():
+        raise HcRuntimeError("map_reduce_cols: the result must be contiguous")
+    ms, lds, rows = [], [], None
+    for x in inputs:
+        m = as_memref(x)
+        if len(m.shape) == 1:
+            if m.shape[0] > 1 and m.strides[0] != 1:
+                raise HcRuntimeError("map_reduce_cols: row vectors must be contiguous")
+            r, c, ld = None, m.shape[0], 0
+        else:
+            r, c, ld = _rows_cols(m)
+        if c != cols or (r is not None and rows is not None and r != rows):
+            raise HcRuntimeError("map_reduce_cols: shape mismatch")
+        rows = r if r is not None else rows
+        ms.append(m)
+        lds.append(ld)
+    if rows is None:
+        raise HcRuntimeError("map_reduce_cols: at least one rows x cols operand is needed")
+    if types is None:
+        types = []
+        for m in ms + [mo]:
+            if m.itemsize not in (2, 4):
+                raise HcRuntimeError(f"map_reduce_cols: element size {m.itemsize} "
+                                     "(fp32 and fp16 only)")
+            types.append(F16 if m.itemsize == 2 else F32)
+    n_in = len(inputs)
+
+    def instrs(p):
+        arr = (MapInstr * max(len(p), 1))()
+        for i, (name, arg, imm) in enumerate(p):
+            arr[i].op, arr[i].arg, arr[i].imm = MAP_OPS[name], int(arg), float(imm)
+        return arr
+    prog, post_prog = instrs(program), instrs(post)
+    ptrs = (_vp * max(n_in, 1))(*[m.ptr for m in ms])
+    tys = (_int * max(n_in, 1))(*types[:n_in])
+    ldv = (_sz * max(n_in, 1))(*lds)
+    need = hcamdMapReduceColsWorkspace(ctx.queue, rows, cols)
+    work = DeviceArray((need // 4,), np.float32, ctx) if need else None
+    return Plan(ctx, hcamdLaunchMapReduceCols,
+                (ctx.queue, COLS_KINDS[kind], prog, len(program), post_prog, len(post), ptrs, tys,
+                 ldv, n_in, mo.ptr, types[-1], rows, cols, work.ptr if work else None, need),
+                "hcamdLaunchMapReduceCols", (inputs, out, prog, post_prog, ptrs, tys, ldv, work))
 
 
 def plan_row_program(stages, inputs, out, columns=(), types=None) -> Plan:

@@ -312,6 +312,31 @@ int hcamdLaunchMapSum(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
                       const size_t *inputLd, size_t nInputs, float *cell,
                       size_t rows, size_t cols) HCAMD_NOEXCEPT;
 
+/* Reductions along columns: out[c] = post(fold over the rows r of
+ * f(in_0[r][c] .. in_{n-1}[r][c])) for a rows x cols window, i.e. the tile
+ * methods the reference's simulator forwards to NumPy (`tile.sum(axis=0)`,
+ * `max`, `min`, `mean`: python/hckernel/kernel_api.py:150-151) applied to an
+ * elementwise expression of loads.  `prog` is a map program as for
+ * hcamdLaunchMap; `kind` selects the fold (fp32 sum; maximum and minimum
+ * propagate NaN like numpy.maximum / numpy.minimum); `post` (nPost may be 0)
+ * is a map program with the folded value as its operand 0, e.g. the division
+ * of a mean.  An operand with leading dimension 0 is a vector of cols elements
+ * that every row uses.  `out` holds cols contiguous elements.  Rows are folded
+ * in a fixed order: results do not change from run to run.  Windows with many
+ * rows and few columns are cut into bands of rows whose results meet in
+ * `workspace` (device memory, 16-byte aligned, at least
+ * hcamdMapReduceColsWorkspace(q, rows, cols) bytes; that is 0 when one launch
+ * does it all and workspace may then be null).  The launch allocates nothing. */
+enum HcamdColsKind { HCAMD_COLS_SUM = 0, HCAMD_COLS_MAX = 1, HCAMD_COLS_MIN = 2 };
+#define HCAMD_COLS_MAX_POST 8
+size_t hcamdMapReduceColsWorkspace(OlQueue q, size_t rows, size_t cols) HCAMD_NOEXCEPT;
+int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, size_t nInstr,
+                             const HcamdMapInstr *post, size_t nPost,
+                             const void *const *inputs, const int *inputTypes,
+                             const size_t *inputLd, size_t nInputs, void *out,
+                             int outType, size_t rows, size_t cols, void *workspace,
+                             size_t workspaceBytes) HCAMD_NOEXCEPT;
+
 /* Row programs: bodies that mix elementwise arithmetic with reductions along
  * the rows of a 2-D tile, e.g. the reference's row softmax
  * (python/hckernel/tests/test_examples.py:304-336:

@@ -1,0 +1,157 @@
+"""Reductions along columns (hcamdLaunchMapReduceCols) on the GPU against NumPy.
+
+Expected values are plain NumPy expressions in float64: sums are held to the
+fp32 bound of a sum of `rows` terms, maxima and minima are exact, and what a
+`post` program computes from them is held to a few ulp of fp32.
+"""
+import sys
+
+import numpy as np
+import pytest
+from numpy.testing import assert_allclose, assert_array_equal
+
+from hc_amd import runtime as rt
+
+pytestmark = pytest.mark.gpu
+
+POISON32 = 0xA5A5A5A5
+
+
+def I(name, arg=0, imm=0.0):
+    return (name, arg, imm)
+
+
+def say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    return rt.default_context("hip:0")
+
+
+def poisoned(shape, dtype):
+    return rt.DeviceArray(shape, dtype).fill_bytes32(POISON32)
+
+
+class _View:
+    def __init__(self, base, shape, offset_elems=0, strides=None):
+        self.shape = tuple(shape)
+        self.ctx = base.ctx
+        item = base.dtype.itemsize
+        self.__cuda_array_interface__ = {
+            "shape": self.shape, "typestr": rt._TYPESTR[base.dtype.name],
+            "data": (int(base.ptr) + offset_elems * item, False),
+            "strides": None if strides is None else tuple(s * item for s in strides),
+            "version": 2}
+
+
+def sum_bound(terms64):
+    """fp32 error bound of rounding the rows of `terms64` and adding them up in
+    any order."""
+    return (terms64.shape[0] + 1) * 2.0 ** -24 * np.abs(terms64).sum(axis=0) + 1e-30
+
+
+def within(got, want, bound):
+    err = np.abs(got.astype(np.float64) - want)
+    worst = int(np.argmax(err - bound))
+    assert (err <= bound).all(), (worst, got[worst], want[worst], err[worst], np.broadcast_to(bound, err.shape)[worst])
+
+
+# one launch and several bands of rows, whole and ragged chunks of columns
+SHAPES = [(1, 1), (5, 7), (100, 513), (4097, 1031), (8192, 64), (20_000, 24), (64, 70_001),
+          (3000, 4096)]
+
+
+@pytest.mark.parametrize("rows,cols", SHAPES)
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_sums_maxima_and_minima_of_expressions_down_the_columns(ctx, rows, cols, dtype):
+    rng = np.random.default_rng(rows * 31 + cols)
+    x = rng.standard_normal((rows, cols)).astype(dtype)
+    y = rng.standard_normal((rows, cols)).astype(dtype)
+    dx, dy = rt.to_device(x), rt.to_device(y)
+    x64, y64 = x.astype(np.float64), y.astype(np.float64)
+    say("reduce_cols", rows, cols, np.dtype(dtype).name)
+    out = poisoned((cols + 8,), np.float32)
+    res = _View(out, (cols,), 0)
+
+    rt.plan_map_reduce_cols("sum", [I("in", 0), I("mul_in", 1)], [dx, dy], res).launch(sync=True)
+    got = out.to_host()
+    within(got[:cols], (x64 * y64).sum(axis=0), sum_bound(x64 * y64))
+    assert (got[cols:].view(np.uint32) == POISON32).all()
+    again = poisoned((cols + 8,), np.float32)
+    rt.plan_map_reduce_cols("sum", [I("in", 0), I("mul_in", 1)], [dx, dy],
+                            _View(again, (cols,), 0)).launch(sync=True)
+    assert_array_equal(again.to_host()[:cols].view(np.uint32), got[:cols].view(np.uint32))
+
+    rt.plan_map_reduce_cols("max", [I("in", 0), I("abs")], [dx], res).launch(sync=True)
+    assert_array_equal(out.to_host()[:cols], np.abs(x).max(axis=0).astype(np.float32))
+    rt.plan_map_reduce_cols("min", [I("in", 0), I("sub_in", 1)], [dx, dy], res).launch(sync=True)
+    want = (x.astype(np.float32) - y.astype(np.float32)).min(axis=0)
+    assert_array_equal(out.to_host()[:cols], want)
+
+    # the mean: the division runs on the folded value
+    rt.plan_map_reduce_cols("sum", [I("in", 0)], [dx], res, post=[I("in", 0), I("divi", 0, rows)]
+                            ).launch(sync=True)
+    within(out.to_host()[:cols], x64.mean(axis=0), sum_bound(x64) / rows + 1e-6 * np.abs(x64.mean(axis=0)))
+
+
+@pytest.mark.parametrize("ld,off", [(1040, 8), (1037, 3)])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_windows_of_larger_arrays_vectors_and_fp16_results(ctx, ld, off, dtype):
+    """Rows on and off 16-byte boundaries, NaN around the window, a vector that
+    every row uses, a square root of the folded value as an fp16 result."""
+    rows, cols = 777, 1001
+    rng = np.random.default_rng(ld)
+    x = rng.standard_normal((rows, cols)).astype(dtype)
+    v = rng.standard_normal(cols).astype(np.float32)
+    big = np.full((rows + 2, ld), np.nan, dtype)
+    big[1:rows + 1, off:off + cols] = x
+    dbig, dv = rt.to_device(big), rt.to_device(v)
+    out = poisoned((cols + 9,), np.float16)
+    rt.plan_map_reduce_cols("sum", [I("in", 0), I("sub_in", 1), I("abs")],
+                            [_View(dbig, (rows, cols), ld + off, (ld, 1)), dv],
+                            _View(out, (cols,), 1), post=[I("in", 0), I("sqrt")]).launch(sync=True)
+    got = out.to_host()
+    d = x.astype(np.float32) - v
+    want = np.sqrt(np.abs(d.astype(np.float64)).sum(axis=0))
+    assert_allclose(got[1:cols + 1].astype(np.float64), want, rtol=2.0 ** -11 + 1e-5)
+    assert (got[:1].view(np.uint16) == POISON32 & 0xFFFF).all()
+    assert (got[cols + 1:].view(np.uint16) == POISON32 & 0xFFFF).all()
+
+
+def test_nan_and_infinities_follow_numpy(ctx):
+    rows, cols = 300, 40
+    x = np.random.default_rng(1).standard_normal((rows, cols)).astype(np.float32)
+    x[17, 3] = np.nan
+    x[250, 5] = np.inf
+    x[0, 6] = -np.inf
+    dx = rt.to_device(x)
+    out = rt.DeviceArray((cols,), np.float32)
+    with np.errstate(invalid="ignore"):
+        for kind, want in (("max", x.max(axis=0)), ("min", x.min(axis=0)), ("sum", x.sum(axis=0))):
+            rt.plan_map_reduce_cols(kind, [I("in", 0)], [dx], out).launch(sync=True)
+            got = out.to_host()
+            assert_array_equal(np.isnan(got), np.isnan(want))
+            assert_array_equal(np.isinf(got), np.isinf(want))
+            if kind != "sum":
+                assert_array_equal(got[~np.isnan(want)], want[~np.isnan(want)])
+
+
+def test_malformed_requests_are_refused_before_anything_runs(ctx):
+    x = rt.to_device(np.ones((8, 8), np.float32))
+    out = rt.DeviceArray((8,), np.float32)
+    with pytest.raises(rt.HcRuntimeError, match="leaves 2 values"):
+        rt.plan_map_reduce_cols("sum", [I("in", 0), I("in", 0)], [x], out).launch(sync=True)
+    with pytest.raises(rt.HcRuntimeError, match="operand 1"):
+        rt.plan_map_reduce_cols("sum", [I("in", 0)], [x], out,
+                                post=[I("in", 1)]).launch(sync=True)
+    # a window that needs bands of rows, launched without its workspace
+    rows, cols = 100_000, 16
+    big = rt.to_device(np.ones((rows, cols), np.float32))
+    assert rt.hcamdMapReduceColsWorkspace(ctx.queue, rows, cols) > 0
+    p = rt.plan_map_reduce_cols("sum", [I("in", 0)], [big], rt.DeviceArray((cols,), np.float32))
+    args = list(p.args)
+    args[-2], args[-1] = None, 0
+    with pytest.raises(rt.HcRuntimeError, match="workspace"):
+        rt.Plan(ctx, p.fn, tuple(args), "hcamdLaunchMapReduceCols", p.keep).launch(sync=True)
