@@ -783,17 +783,22 @@ __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcam
 // minimum, and post is a second short program whose operand 0 is the folded
 // value (the division of a mean, the square root of a norm).
 //
-// A lane owns one chunk of eight consecutive columns and walks down the rows, so
-// a wave reads 64 neighbouring chunks of one row at a time (16-byte accesses
-// where every row of an operand starts on a 16-byte boundary, element accesses
-// otherwise; an operand with leading dimension 0 is a vector that every row
-// uses).  The four waves of a workgroup take every fourth row of the
-// workgroup's band of rows and meet in LDS.  blockIdx.x numbers blocks of 64
-// chunks, blockIdx.y bands of rows: with more than one band the folded values go
-// to partial[band][column] (fp32, `cols_pad` per band) and a second launch of
-// this kernel folds the bands, as the rows of an fp32 operand, in the same
-// fixed order; the launch with one band runs `post` and stores.  Nothing is
-// atomic: results are the same from run to run.
+// A lane owns eight columns and walks down the rows.  L lanes share a row (64,
+// or the next power of two above the chunks of a narrow row, so that a wave
+// covers 64 / L rows at a time and no lane idles); blockIdx.x numbers blocks of
+// 8 * L columns.  Where every row of every operand starts on a 16-byte boundary
+// a lane's columns are consecutive and move with 16-byte accesses; otherwise the
+// columns of a block are dealt to its lanes one by one, so that the element
+// accesses of a wave are coalesced (columns are independent: any assignment
+// works as long as operands and result agree).  An operand with leading
+// dimension 0 is a vector that every row uses.  The waves of a workgroup take
+// turns down the workgroup's band of rows; at the end the lanes that share
+// columns fold through cross-lane exchanges and the waves meet in LDS.
+// blockIdx.y numbers the bands: with more than one, the folded values go to
+// partial[band][column] (fp32, `cols_pad` per band) and the host launches the
+// kernel again on the bands as the rows of an fp32 operand; the launch with one
+// band runs `post` and stores.  Nothing is atomic and every order is fixed:
+// results are the same from run to run.
 namespace {
 constexpr int kPostProg = 8;
 enum : uint32_t { COL_SUM = 0, COL_MAX = 1, COL_MIN = 2 };
@@ -802,7 +807,9 @@ struct ColArgs {
   uint32_t cols_pad;    // multiple of 8, at least cols
   uint32_t band;        // rows per band
   uint32_t kind;
-  uint32_t vec_mask;    // bit i: operand i may be read 16 bytes at a time; bit 8: out written so
+  uint32_t lanes;       // L
+  uint32_t interleaved; // columns of a block dealt to the lanes one by one
+  uint32_t out_vec;     // the result may be written 16 bytes at a time
   uint32_t n_post;
   Instr post[kPostProg];
 };
@@ -829,8 +836,8 @@ __device__ __forceinline__ float col_fold(uint32_t kind, float a, float b) {
   return kind == COL_SUM ? a + b : kind == COL_MAX ? nan_max(a, b) : nan_min(a, b);
 }
 
-// NIN: operands the kernel is compiled for; U: rows a wave has in flight (their
-// loads are issued together, then the program runs on one row after the other:
+// NIN: operands the kernel is compiled for; U: turns a wave has in flight (their
+// loads are issued together, then the program runs on one after the other:
 // fewer operands leave registers for more rows).
 template <int NIN, int U>
 __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, const uint32_t n_in) {
@@ -838,25 +845,31 @@ __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, 
   __shared__ float slots[kWaves - 1][kWave][kN + 1];
   const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const uint32_t cols = (uint32_t)a.cols, rows = (uint32_t)a.rows;
-  const uint32_t chunk = blockIdx.x * kWave + lane;
-  const uint32_t first = chunk * kN;
-  const uint32_t n_valid =
-      first >= cols ? 0u : cols - first < (uint32_t)kN ? cols - first : (uint32_t)kN;
+  const uint32_t L = c.lanes, R = kWave / L;
+  const uint32_t cl = lane & (L - 1), sub = lane / L;
+  // column of element e: first + e * step
+  const uint32_t chunk = blockIdx.x * L + cl;
+  const uint32_t first = c.interleaved ? blockIdx.x * L * kN + cl : chunk * kN;
+  const uint32_t step = c.interleaved ? L : 1u;
+  const uint32_t n_valid = first >= cols ? 0u
+                           : (cols - first + step - 1) / step < (uint32_t)kN
+                               ? (cols - first + step - 1) / step
+                               : (uint32_t)kN;
   const uint32_t row_begin = blockIdx.y * c.band;
   const uint32_t row_end = row_begin + c.band < rows ? row_begin + c.band : rows;
+  // -0 is the identity of IEEE addition (0 would turn a column of -0 into +0)
   const float identity =
-      c.kind == COL_SUM ? 0.0f : c.kind == COL_MAX ? -__builtin_inff() : __builtin_inff();
+      c.kind == COL_SUM ? -0.0f : c.kind == COL_MAX ? -__builtin_inff() : __builtin_inff();
   float acc[kN];
 #pragma unroll
   for (int e = 0; e < kN; ++e)
     acc[e] = identity;
-  // a wave whose lanes all hold whole chunks takes the 16-byte path for the
-  // operands that allow it
-  const bool all_whole = __builtin_amdgcn_ballot_w64(n_valid != (uint32_t)kN) == 0;
+  // 16-byte accesses: consecutive columns and a wave of whole chunks
+  const bool vec = !c.interleaved && __builtin_amdgcn_ballot_w64(n_valid != (uint32_t)kN) == 0;
   Raw raw;
   Stack r;
 #pragma nounroll
-  for (uint32_t row0 = row_begin + wave; row0 < row_end; row0 += kWaves * U) {
+  for (uint32_t row0 = row_begin + wave * R; row0 < row_end; row0 += kWaves * R * U) {
     u32x4 staged[NIN][U][2];
 #pragma unroll
     for (int i = 0; i < NIN; ++i)
@@ -864,11 +877,11 @@ __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, 
         const bool f16 = (a.f16_mask >> i) & 1;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-          const uint32_t row = row0 + u * kWaves;
+          const uint32_t row = row0 + u * kWaves * R + sub;
           if (row < row_end) {
             const char *base =
                 static_cast<const char *>(a.in[i]) + (size_t)row * a.ld[i] * (f16 ? 2 : 4);
-            if (((c.vec_mask >> i) & 1) && all_whole) {
+            if (vec) {
               const u32x4 *q = reinterpret_cast<const u32x4 *>(base) + (f16 ? chunk : 2 * chunk);
               staged[i][u][0] = ldg<true>(q);
               if (!f16)
@@ -877,7 +890,7 @@ __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, 
               uint32_t v[kN];
 #pragma unroll
               for (int e = 0; e < kN; ++e) {
-                const uint32_t at = (uint32_t)e < n_valid ? first + e : 0u;
+                const uint32_t at = (uint32_t)e < n_valid ? first + e * step : 0u;
                 v[e] = f16 ? (uint32_t) reinterpret_cast<const uint16_t *>(base)[at]
                            : reinterpret_cast<const uint32_t *>(base)[at];
               }
@@ -907,21 +920,26 @@ __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, 
         }
       }
       run_program(a, raw, a.f16_mask, r);
-      if (row0 + u * kWaves < row_end) {
+      if (row0 + u * kWaves * R + sub < row_end) {
 #pragma unroll
         for (int e = 0; e < kN; ++e)
           acc[e] = col_fold(c.kind, acc[e], r.st[0][e]);
       }
     }
   }
-  // waves 1.. park their values, wave 0 folds them in wave order
+  // lanes that share columns (the rows of one turn), then the waves in order
+  for (uint32_t s = L; s < (uint32_t)kWave; s <<= 1) {
+#pragma unroll
+    for (int e = 0; e < kN; ++e)
+      acc[e] = col_fold(c.kind, acc[e], __shfl_xor(acc[e], (int)s, kWave));
+  }
   if (wave != 0) {
 #pragma unroll
     for (int e = 0; e < kN; ++e)
       slots[wave - 1][lane][e] = acc[e];
   }
   __syncthreads();
-  if (wave != 0)
+  if (wave != 0 || sub != 0)
     return;
 #pragma unroll
   for (int w = 0; w < kWaves - 1; ++w)
@@ -929,16 +947,21 @@ __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, 
     for (int e = 0; e < kN; ++e)
       acc[e] = col_fold(c.kind, acc[e], slots[w][lane][e]);
   if (gridDim.y > 1) {
-    if (n_valid) {
-      float *dst = c.partial + (size_t)blockIdx.y * c.cols_pad + first;
+    float *dst = c.partial + (size_t)blockIdx.y * c.cols_pad;
+    if (!c.interleaved && n_valid) { // cols_pad covers whole chunks
       f32x4 lo, hi;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         lo[e] = acc[e];
         hi[e] = acc[4 + e];
       }
-      *reinterpret_cast<f32x4 *>(dst) = lo;
-      *reinterpret_cast<f32x4 *>(dst + 4) = hi;
+      *reinterpret_cast<f32x4 *>(dst + first) = lo;
+      *reinterpret_cast<f32x4 *>(dst + first + 4) = hi;
+    } else {
+#pragma unroll
+      for (int e = 0; e < kN; ++e)
+        if ((uint32_t)e < n_valid)
+          dst[first + e * step] = acc[e];
     }
     return;
   }
@@ -953,13 +976,13 @@ __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, 
       r.st[0][e] = acc[e];
   }
   const bool out_f16 = (a.f16_mask >> 8) & 1;
-  if (((c.vec_mask >> 8) & 1) && n_valid == (uint32_t)kN) {
+  if (c.out_vec && !c.interleaved && n_valid == (uint32_t)kN) {
     store_chunk(a.out, out_f16, chunk, r.st[0]);
   } else {
 #pragma unroll
     for (int e = 0; e < kN; ++e)
       if ((uint32_t)e < n_valid)
-        store_elem(a.out, out_f16, (size_t)first + e, r.st[0][e]);
+        store_elem(a.out, out_f16, (size_t)first + e * step, r.st[0][e]);
   }
 }
 } // namespace

@@ -1173,7 +1173,7 @@ namespace {
 // Second argument block of the column-reduction kernels (device layout).
 struct ColArgs {
   float *partial;
-  uint32_t colsPad, band, kind, vecMask, nPost;
+  uint32_t colsPad, band, kind, lanes, interleaved, outVec, nPost;
   HcamdMapInstr post[HCAMD_COLS_MAX_POST];
 };
 
@@ -1213,14 +1213,43 @@ bool mapProgramOk(Device *dev, const char *who, const HcamdMapInstr *prog, size_
   return true;
 }
 
+// Lanes that share a row: 64, or the next power of two above the chunks of a
+// narrow row.
+size_t colLanes(size_t cols) {
+  const size_t perRow = ceilDiv(cols, (size_t)8);
+  size_t lanes = 1;
+  while (lanes < 64 && lanes < perRow)
+    lanes *= 2;
+  return lanes;
+}
+
 // Bands of rows a column reduction is cut into, so that the launch has a few
 // workgroups per compute unit however narrow the window is; 1 = one launch.
 void colBands(Device *dev, size_t rows, size_t cols, size_t &bands, size_t &band) {
-  const size_t blocks = ceilDiv(ceilDiv(cols, (size_t)8), (size_t)64);
+  const size_t lanes = colLanes(cols);
+  const size_t blocks = ceilDiv(ceilDiv(cols, (size_t)8), lanes);
+  const size_t turn = 16 * (64 / lanes); // rows of one turn of 4 waves x 4 rows in flight
   const size_t wanted = ceilDiv((size_t)computeUnitsOf(dev) * 6, blocks);
-  bands = std::max(std::min(wanted, rows / 64), (size_t)1);
-  band = ceilDiv(ceilDiv(rows, bands), (size_t)16) * 16; // whole turns of 4 waves x 4 rows
+  bands = std::max(std::min(wanted, rows / (4 * turn)), (size_t)1);
+  band = ceilDiv(ceilDiv(rows, bands), turn) * turn;
   bands = ceilDiv(rows, band);
+}
+
+// Levels of a reduction: the bands of one level are the rows of the next.
+// Returns the floats of workspace all levels need together.
+size_t colLevels(Device *dev, size_t rows, size_t cols, std::vector<std::pair<size_t, size_t>> *levels) {
+  const size_t colsPad = ceilDiv(cols, (size_t)8) * 8;
+  size_t floats = 0;
+  for (;;) {
+    size_t bands, band;
+    colBands(dev, rows, cols, bands, band);
+    if (levels)
+      levels->push_back({bands, band});
+    if (bands == 1)
+      return floats;
+    floats += bands * colsPad;
+    rows = bands;
+  }
 }
 } // namespace
 
@@ -1228,9 +1257,7 @@ size_t hcamdMapReduceColsWorkspace(OlQueue q, size_t rows, size_t cols) noexcept
   auto *queue = static_cast<Queue *>(q);
   if (!queue || rows == 0 || cols == 0)
     return 0;
-  size_t bands, band;
-  colBands(queue->device, rows, cols, bands, band);
-  return bands > 1 ? bands * ceilDiv(cols, (size_t)8) * 8 * sizeof(float) : 0;
+  return colLevels(queue->device, rows, cols, nullptr) * sizeof(float);
 }
 
 int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, size_t nInstr,
@@ -1272,7 +1299,7 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
     dev->report("%s: no rows to reduce", who);
     return 1;
   }
-  if (rows >= ((size_t)1 << 32) || cols > ((size_t)1 << 32) - 8) {
+  if (rows >= ((size_t)1 << 32) || cols > ((size_t)1 << 32) - 1024) {
     dev->report("%s: window of %zu x %zu (below 2^32 each)", who, rows, cols);
     return 1;
   }
@@ -1282,6 +1309,7 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
   }
   MapArgs a{};
   ColArgs c{};
+  bool allVec = true;
   for (size_t i = 0; i < nInputs; ++i) {
     if (!inputs[i]) {
       dev->report("%s: null pointer", who);
@@ -1301,20 +1329,41 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
     const size_t size = inputTypes[i] == HCAMD_F16 ? 2 : 4;
     if (inputTypes[i] == HCAMD_F16)
       a.f16_mask |= 1u << i;
-    if (aligned16(inputs[i]) && (inputLd[i] * size) % 16 == 0)
-      c.vecMask |= 1u << i;
+    allVec = allVec && aligned16(inputs[i]) && (inputLd[i] * size) % 16 == 0;
   }
-  size_t bands, band;
-  colBands(dev, rows, cols, bands, band);
+  std::vector<std::pair<size_t, size_t>> levels;
   const size_t colsPad = ceilDiv(cols, (size_t)8) * 8;
-  if (bands > 1 && (!workspace || !aligned16(workspace) ||
-                    workspaceBytes < bands * colsPad * sizeof(float))) {
+  const size_t floats = colLevels(dev, rows, cols, &levels);
+  if (floats && (!workspace || !aligned16(workspace) || workspaceBytes < floats * sizeof(float))) {
     dev->report("%s: workspace of %zu bytes, 16-byte aligned, needed (%zu given)", who,
-                bands * colsPad * sizeof(float), workspaceBytes);
+                floats * sizeof(float), workspaceBytes);
     return 1;
   }
-  const size_t blocks = ceilDiv(colsPad / 8, (size_t)64);
-  auto launchOne = [&](MapArgs &ma, ColArgs &ca, size_t nIn, size_t nBands) {
+  const size_t lanes = colLanes(cols);
+  const size_t blocks = ceilDiv(colsPad / 8, lanes);
+  a.cols = cols;
+  a.n_instr = static_cast<uint32_t>(nInstr);
+  std::memcpy(a.prog, prog, nInstr * sizeof(HcamdMapInstr));
+  c.kind = static_cast<uint32_t>(kind);
+  c.colsPad = static_cast<uint32_t>(colsPad);
+  c.lanes = static_cast<uint32_t>(lanes);
+  c.interleaved = allVec ? 0u : 1u;
+  float *level = static_cast<float *>(workspace);
+  size_t nIn = nInputs, levelRows = rows;
+  for (size_t l = 0; l < levels.size(); ++l) {
+    const size_t bands = levels[l].first;
+    a.rows = levelRows;
+    c.band = static_cast<uint32_t>(levels[l].second);
+    c.partial = level;
+    if (bands == 1) { // the last launch runs `post` and stores
+      a.out = out;
+      if (outType == HCAMD_F16)
+        a.f16_mask |= 1u << 8;
+      c.outVec = aligned16(out) ? 1u : 0u;
+      c.nPost = static_cast<uint32_t>(nPost);
+      if (nPost)
+        std::memcpy(c.post, post, nPost * sizeof(HcamdMapInstr));
+    }
     const char *name = nIn <= 1   ? "hcamd_map_reduce_cols_n1u4"
                        : nIn <= 2 ? "hcamd_map_reduce_cols_n2u2"
                                   : "hcamd_map_reduce_cols_n4u1";
@@ -1322,49 +1371,26 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
     if (!k)
       return 1;
     uint32_t n = static_cast<uint32_t>(nIn);
-    void *args[] = {&ma, &ca, &n};
-    const size_t grid[3] = {blocks, nBands, 1}, block[3] = {256, 1, 1};
-    return launch(queue, k, grid, block, args, 0);
-  };
-  auto finish = [&](MapArgs &ma, ColArgs &ca) {
-    ma.out = out;
-    if (outType == HCAMD_F16)
-      ma.f16_mask |= 1u << 8;
-    if (aligned16(out))
-      ca.vecMask |= 1u << 8;
-    ca.nPost = static_cast<uint32_t>(nPost);
-    if (nPost)
-      std::memcpy(ca.post, post, nPost * sizeof(HcamdMapInstr));
-  };
-  a.rows = rows;
-  a.cols = cols;
-  a.n_instr = static_cast<uint32_t>(nInstr);
-  std::memcpy(a.prog, prog, nInstr * sizeof(HcamdMapInstr));
-  c.kind = static_cast<uint32_t>(kind);
-  c.colsPad = static_cast<uint32_t>(colsPad);
-  c.band = static_cast<uint32_t>(band);
-  if (bands == 1) {
-    finish(a, c);
-    return launchOne(a, c, nInputs, 1);
+    void *args[] = {&a, &c, &n};
+    const size_t grid[3] = {blocks, bands, 1}, block[3] = {256, 1, 1};
+    if (int rc = launch(queue, k, grid, block, args, 0))
+      return rc;
+    if (bands == 1)
+      break;
+    // the bands just written are the rows of an fp32 operand of the next level
+    std::memset(a.in, 0, sizeof a.in);
+    std::memset(a.ld, 0, sizeof a.ld);
+    a.in[0] = level;
+    a.ld[0] = colsPad;
+    a.f16_mask = 0;
+    a.n_instr = 1;
+    a.prog[0] = HcamdMapInstr{HCAMD_MAP_IN, 0, 0.0f};
+    c.interleaved = 0;
+    nIn = 1;
+    levelRows = bands;
+    level += bands * colsPad;
   }
-  c.partial = static_cast<float *>(workspace);
-  if (int rc = launchOne(a, c, nInputs, bands))
-    return rc;
-  // the bands are the rows of an fp32 operand, folded the same way
-  MapArgs a2{};
-  ColArgs c2{};
-  a2.in[0] = workspace;
-  a2.ld[0] = colsPad;
-  a2.rows = bands;
-  a2.cols = cols;
-  a2.n_instr = 1;
-  a2.prog[0].op = HCAMD_MAP_IN;
-  c2.kind = c.kind;
-  c2.colsPad = c.colsPad;
-  c2.band = static_cast<uint32_t>(bands);
-  c2.vecMask = 1u;
-  finish(a2, c2);
-  return launchOne(a2, c2, 1, 1);
+  return 0;
 }
 
 namespace {
