@@ -1220,6 +1220,112 @@ def match_rows(dst_view, value, n_groups):
     return make
 
 
+# ---------------------------------------------------------------------------
+# Reductions along columns: x.sum(axis=0) and friends of an elementwise expression
+# ---------------------------------------------------------------------------
+class _PostCompiler(_MapCompiler):
+    """Compiles what is done to a reduction's result (a chain of unary
+    operations, casts and operations with constants) with that result as
+    operand 0."""
+
+    def __init__(self, n_groups, root: Tile):
+        super().__init__(n_groups)
+        self.root = root
+
+    def supported(self, t: Tile) -> bool:
+        return t is self.root or super().supported(t)
+
+    def need(self, t: Tile) -> int:
+        return 1 if t is self.root else super().need(t)
+
+    def emit(self, t: Tile, out: list):
+        if t is self.root:
+            out.append(("in", 0, 0.0))
+        else:
+            super().emit(t, out)
+
+
+def match_cols(dst_view, value, n_groups):
+    """value = post(reduce(f(tiles...), axis=0)): sums, maxima, minima, means
+    and 2-norms down the columns of (rows, N) tiles that hold whole columns of
+    their arrays, one group per block of columns.  The tile methods are the ones
+    the simulator forwards to NumPy (python/hckernel/kernel_api.py:150-151)."""
+    if dst_view.base.dtype_name not in _MAP_FLOATS:
+        return None
+    # walk down from the stored value to the reduction
+    t = value
+    while True:
+        if (t.op in _ROW_REDUCE or t.op == "norm") and t.attrs.get("axes") == (0,) \
+                and len(t.args) == 1 and len(t.args[0].shape) == 2:
+            break
+        if len(t.args) == 1 and (_is(t, "astype", 1) or t.op in _MAP_UNARY or _is(t, "clip", 1)):
+            t = t.args[0]
+        elif t.op in _MAP_BINARY and len(t.args) == 2 and _const(t.args[0]) != _const(t.args[1]):
+            t = t.args[0] if _const(t.args[1]) else t.args[1]
+        else:
+            return None
+    red, body = t, t.args[0]
+    rows, n = body.shape
+    if red.op == "norm":          # numpy.linalg.norm along an axis is sqrt(add.reduce(x * x))
+        body = body * body
+    if red.op in ("sum", "norm") and body.dtype_name != "float32":
+        raise NoNativeKernel("column sums are computed in float32: cast the tile with "
+                             ".astype(np.float32) before adding it up")
+    comp = _MapCompiler(n_groups)
+    if _const(body) or not comp.supported(body):
+        raise NoNativeKernel(f"{body!r} is not an elementwise expression of float32 / float16 "
+                             "tiles and constants")
+    if comp.need(body) > rt.MAP_STACK_DEPTH:
+        raise NoNativeKernel("expression needs an evaluation stack deeper than "
+                             f"{rt.MAP_STACK_DEPTH}")
+    program: list = []
+    comp.emit(body, program)
+    if len(program) > rt.MAP_MAX_INSTRS or not 1 <= len(comp.inputs) <= rt.MAP_MAX_INPUTS:
+        raise NoNativeKernel(f"the reduced expression compiles to {len(program)} operations on "
+                             f"{len(comp.inputs)} arrays (at most {rt.MAP_MAX_INSTRS} on "
+                             f"{rt.MAP_MAX_INPUTS})")
+    post: list = []
+    if red.op == "norm":
+        post = [("in", 0, 0.0), ("sqrt", 0, 0.0)]
+    if value is not red:
+        pc = _PostCompiler(n_groups, red)
+        if not pc.supported(value):
+            raise NoNativeKernel(f"{value!r}: what follows a column reduction must be float32 / "
+                                 "float16 arithmetic with constants")
+        tail: list = []
+        pc.emit(value, tail)
+        post = post + tail[1:] if post else tail
+    if len(post) > rt.COLS_MAX_POST:
+        raise NoNativeKernel(f"{len(post)} operations follow the column reduction "
+                             f"(at most {rt.COLS_MAX_POST})")
+    wins = [window_of(tl.attrs["view"], tl.shape, n_groups) for _, _, tl in comp.inputs]
+    w = wins[0]
+    for x, (_, _, tl) in zip(wins, comp.inputs):
+        if len(x.extent) != 2 or x.extent != w.extent or x.driver != w.driver:
+            raise NoNativeKernel("the tiles of a column reduction must walk the same columns")
+        if x.driver[0] is not None or tl.shape[0] != tl.attrs["view"].base.shape[0]:
+            raise NoNativeKernel("column reductions need tiles that hold whole columns "
+                                 "(as many rows as the array has)")
+    wo = window_of(dst_view, value.shape, n_groups)
+    if wo.extent[-1] != w.extent[1] or wo.driver[-1] != w.driver[1] or \
+            math.prod(wo.extent) != wo.extent[-1]:
+        raise NoNativeKernel("the per-column result and the tiles walk different columns")
+    ftype = lambda name: rt.F16 if name == "float16" else rt.F32
+    types = [ftype(tl.dtype_name) for _, _, tl in comp.inputs] + [ftype(dst_view.base.dtype_name)]
+    kind = "sum" if red.op == "norm" else _ROW_REDUCE[red.op]
+    n_cols = w.extent[1]
+
+    def make(mem, ctx):
+        ins = [_Arr(_sub(mem[x.buffer], x.extent), ctx) for x in wins]
+        mo = mem[wo.buffer]
+        if n_cols > 1 and mo.strides[-1] != 1:
+            raise NoNativeKernel("the per-column result must be contiguous")
+        out = _Arr(rt.Memref(mo.ptr, (n_cols,), (1,), mo.itemsize), ctx)
+        return [rt.plan_map_reduce_cols(kind, program, ins, out, post, types)]
+    make.program, make.post, make.kind = program, post, kind
+    return make
+
+
 def match_pairwise(dst_view, value, n_groups):
     """out[m, n] = ||a[m, :] - b[n, :]||: the body of
     python/hckernel/tests/test_examples.py:270-301."""
@@ -1354,7 +1460,7 @@ def bind(stores, n_groups, atomics=(), mapped_stores=()):
             return makers + [q]
         for view, value in stores:
             for matcher in (match_copy, match_add, match_fma, match_softmax, match_gemm,
-                            match_gather_gemm, match_pairwise, match_rows, match_map):
+                            match_gather_gemm, match_pairwise, match_cols, match_rows, match_map):
                 mk = matcher(view, value, n_groups)
                 if mk is not None:
                     makers.append(mk)
@@ -1364,7 +1470,8 @@ def bind(stores, n_groups, atomics=(), mapped_stores=()):
                     f"no hand-written kernel matches the value stored to {view.base.name} "
                     f"({value!r}); bound patterns: copy, a+b (fp32), a*b+c (fp16 storage, fp32 "
                     "math), row softmax (fp32), row absmax int8 quantisation, bf16 GEMM, elementwise "
-                    "expressions over fp32 / fp16 arrays, with reductions along whole rows")
+                    "expressions over fp32 / fp16 arrays, with reductions along whole rows or down "
+                    "whole columns")
         return makers
     except TraceError as exc:
         raise NoNativeKernel(str(exc)) from exc

@@ -1225,11 +1225,11 @@ size_t colLanes(size_t cols) {
 
 // Bands of rows a column reduction is cut into, so that the launch has a few
 // workgroups per compute unit however narrow the window is; 1 = one launch.
-void colBands(Device *dev, size_t rows, size_t cols, size_t &bands, size_t &band) {
+void colBands(size_t rows, size_t cols, size_t &bands, size_t &band) {
   const size_t lanes = colLanes(cols);
   const size_t blocks = ceilDiv(ceilDiv(cols, (size_t)8), lanes);
   const size_t turn = 16 * (64 / lanes); // rows of one turn of 4 waves x 4 rows in flight
-  const size_t wanted = ceilDiv((size_t)computeUnitsOf(dev) * 6, blocks);
+  const size_t wanted = ceilDiv((size_t)1536, blocks); // six workgroups for each of 256 compute units
   bands = std::max(std::min(wanted, rows / (4 * turn)), (size_t)1);
   band = ceilDiv(ceilDiv(rows, bands), turn) * turn;
   bands = ceilDiv(rows, band);
@@ -1237,12 +1237,12 @@ void colBands(Device *dev, size_t rows, size_t cols, size_t &bands, size_t &band
 
 // Levels of a reduction: the bands of one level are the rows of the next.
 // Returns the floats of workspace all levels need together.
-size_t colLevels(Device *dev, size_t rows, size_t cols, std::vector<std::pair<size_t, size_t>> *levels) {
+size_t colLevels(size_t rows, size_t cols, std::vector<std::pair<size_t, size_t>> *levels) {
   const size_t colsPad = ceilDiv(cols, (size_t)8) * 8;
   size_t floats = 0;
   for (;;) {
     size_t bands, band;
-    colBands(dev, rows, cols, bands, band);
+    colBands(rows, cols, bands, band);
     if (levels)
       levels->push_back({bands, band});
     if (bands == 1)
@@ -1253,11 +1253,10 @@ size_t colLevels(Device *dev, size_t rows, size_t cols, std::vector<std::pair<si
 }
 } // namespace
 
-size_t hcamdMapReduceColsWorkspace(OlQueue q, size_t rows, size_t cols) noexcept {
-  auto *queue = static_cast<Queue *>(q);
-  if (!queue || rows == 0 || cols == 0)
+size_t hcamdMapReduceColsWorkspace(size_t rows, size_t cols) noexcept {
+  if (rows == 0 || cols == 0)
     return 0;
-  return colLevels(queue->device, rows, cols, nullptr) * sizeof(float);
+  return colLevels(rows, cols, nullptr) * sizeof(float);
 }
 
 int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, size_t nInstr,
@@ -1333,7 +1332,7 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
   }
   std::vector<std::pair<size_t, size_t>> levels;
   const size_t colsPad = ceilDiv(cols, (size_t)8) * 8;
-  const size_t floats = colLevels(dev, rows, cols, &levels);
+  const size_t floats = colLevels(rows, cols, &levels);
   if (floats && (!workspace || !aligned16(workspace) || workspaceBytes < floats * sizeof(float))) {
     dev->report("%s: workspace of %zu bytes, 16-byte aligned, needed (%zu given)", who,
                 floats * sizeof(float), workspaceBytes);

@@ -109,7 +109,7 @@ hcamdLaunchPairwiseDistF32 = _sig(_rt, "hcamdLaunchPairwiseDistF32", _int, _vp, 
 hcamdLaunchMapSum = _sig(_rt, "hcamdLaunchMapSum", _int, _vp, C.POINTER(MapInstr), _sz,
                          C.POINTER(_vp), C.POINTER(_int), _sz_p, _sz, _vp, _sz, _sz)
 
-hcamdMapReduceColsWorkspace = _sig(_rt, "hcamdMapReduceColsWorkspace", _sz, _vp, _sz, _sz)
+hcamdMapReduceColsWorkspace = _sig(_rt, "hcamdMapReduceColsWorkspace", _sz, _sz, _sz)
 hcamdLaunchMapReduceCols = _sig(_rt, "hcamdLaunchMapReduceCols", _int, _vp, _int,
                                 C.POINTER(MapInstr), _sz, C.POINTER(MapInstr), _sz,
                                 C.POINTER(_vp), C.POINTER(_int), _sz_p, _sz, _vp, _int, _sz, _sz,
@@ -555,7 +555,7 @@ def plan_map_reduce_cols(kind, program, inputs, out, post=(), types=None) -> Pla
     ptrs = (_vp * max(n_in, 1))(*[m.ptr for m in ms])
     tys = (_int * max(n_in, 1))(*types[:n_in])
     ldv = (_sz * max(n_in, 1))(*lds)
-    need = hcamdMapReduceColsWorkspace(ctx.queue, rows, cols)
+    need = hcamdMapReduceColsWorkspace(rows, cols)
     work = DeviceArray((need // 4,), np.float32, ctx) if need else None
     return Plan(ctx, hcamdLaunchMapReduceCols,
                 (ctx.queue, COLS_KINDS[kind], prog, len(program), post_prog, len(post), ptrs, tys,

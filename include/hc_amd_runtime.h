@@ -325,11 +325,12 @@ int hcamdLaunchMapSum(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
  * in a fixed order: results do not change from run to run.  Windows with many
  * rows and few columns are cut into bands of rows whose results meet in
  * `workspace` (device memory, 16-byte aligned, at least
- * hcamdMapReduceColsWorkspace(q, rows, cols) bytes; that is 0 when one launch
- * does it all and workspace may then be null).  The launch allocates nothing. */
+ * hcamdMapReduceColsWorkspace(rows, cols) bytes, a function of the shape alone;
+ * that is 0 when one launch does it all and workspace may then be null).  The
+ * launch allocates nothing. */
 enum HcamdColsKind { HCAMD_COLS_SUM = 0, HCAMD_COLS_MAX = 1, HCAMD_COLS_MIN = 2 };
 #define HCAMD_COLS_MAX_POST 8
-size_t hcamdMapReduceColsWorkspace(OlQueue q, size_t rows, size_t cols) HCAMD_NOEXCEPT;
+size_t hcamdMapReduceColsWorkspace(size_t rows, size_t cols) HCAMD_NOEXCEPT;
 int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, size_t nInstr,
                              const HcamdMapInstr *post, size_t nPost,
                              const void *const *inputs, const int *inputTypes,

@@ -737,6 +737,34 @@ def test_row_reduction_bodies_match_the_simulator(name, rows, n):
         assert_allclose(got, want, rtol=2e-5, atol=2e-6)
 
 
+@pytest.mark.parametrize("rows,n,gn", [(37, 200, 64), (3000, 4096, 512), (70_000, 24, 24),
+                                       (513, 1031, 1031)])
+@pytest.mark.parametrize("name", ["col_sums", "col_max_abs", "col_min", "col_means", "col_norms",
+                                  "col_rms"])
+def test_column_reduction_bodies_match_the_simulator(name, rows, n, gn):
+    """The same body on the GPU and on the CPU simulator: maxima and minima bit
+    for bit, sums within the fp32 bound of adding `rows` terms in another
+    order, what is computed from a sum to the same relative bound."""
+    from test_kernel_frontend import _col_bodies
+    rng = np.random.default_rng(rows + n)
+    x = rng.standard_normal((rows, n)).astype(np.float32)
+    y = rng.standard_normal((rows, n)).astype(np.float32)
+    want = np.zeros(n, np.float32)
+    _col_bodies(sim_kernel)[name](x, y, want, gn)
+    out = rt.DeviceArray((n,), np.float32).fill_bytes32(0xA5A5A5A5)
+    _col_bodies(kernel)[name](rt.to_device(x), rt.to_device(y), out, gn)
+    assert rt.last_kernel_name().startswith("hcamd_map_reduce_cols")
+    got = out.to_host()
+    if name in ("col_max_abs", "col_min"):
+        assert_array_equal(got, want)
+    else:
+        x64, y64 = x.astype(np.float64), y.astype(np.float64)
+        terms = {"col_sums": x64 * y64, "col_means": x64 + y64, "col_norms": (x64 - y64) ** 2,
+                 "col_rms": x64 * x64}[name]
+        rel = (rows + 2) * 2.0 ** -23 * np.abs(terms).sum(axis=0) / np.maximum(np.abs(terms.sum(axis=0)), 1e-30)
+        assert (np.abs(got - want) <= (rel + 4e-7) * np.abs(want) + 1e-30).all()
+
+
 def test_softmax_with_a_temperature_is_a_row_program_and_plain_softmax_keeps_its_kernel():
     M, N, GM = sym.M, sym.N, sym.GM
 

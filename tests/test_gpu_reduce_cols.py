@@ -149,7 +149,7 @@ def test_malformed_requests_are_refused_before_anything_runs(ctx):
     # a window that needs bands of rows, launched without its workspace
     rows, cols = 100_000, 16
     big = rt.to_device(np.ones((rows, cols), np.float32))
-    assert rt.hcamdMapReduceColsWorkspace(ctx.queue, rows, cols) > 0
+    assert rt.hcamdMapReduceColsWorkspace(rows, cols) > 0
     p = rt.plan_map_reduce_cols("sum", [I("in", 0)], [big], rt.DeviceArray((cols,), np.float32))
     args = list(p.args)
     args[-2], args[-1] = None, 0

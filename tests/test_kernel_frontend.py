@@ -922,6 +922,73 @@ def test_row_bodies_without_native_code_say_why(ctx):
         partial.plan(x32, FakeDev((64, 128), "float32"), ctx=ctx)
 
 
+# ---------------------------------------------------------------------------
+# Reductions down the columns -> hcamdLaunchMapReduceCols
+# ---------------------------------------------------------------------------
+def _col_bodies(deco):
+    """Kernel bodies that reduce (M, GN) tiles holding whole columns along axis
+    0, one group per block of GN columns; `deco` is hc_amd's kernel or the CPU
+    simulator's."""
+    M, N, GN = sym.M, sym.N, sym.GN
+
+    def body(fn):
+        @deco(work_shape=cdiv(N, GN), group_shape=1, literals={GN})
+        def k(gr: CurrentGroup, x: Buffer[M, N, DT], y: Buffer[M, N, DT], out: Buffer[N, DT],
+              gn: GN):
+            n0 = gr.id[0] * GN
+            tx = gr.load(x[:, n0:], shape=(M, GN))
+            ty = gr.load(y[:, n0:], shape=(M, GN))
+            gr.store(out[n0:], fn(tx, ty))
+        return k
+
+    f32 = np.float32
+    return {
+        "col_sums": body(lambda a, b: (a * b).sum(axis=0)),
+        "col_max_abs": body(lambda a, b: np.abs(a - b).max(axis=0)),
+        "col_min": body(lambda a, b: np.minimum(a, b).min(axis=0)),
+        "col_means": body(lambda a, b: (a + b).mean(axis=0) * f32(0.5)),
+        "col_norms": body(lambda a, b: np.linalg.norm(a - b, axis=0)),
+        "col_rms": body(lambda a, b: np.sqrt((a * a).sum(axis=0) / f32(a.shape[0]) + f32(1e-6))),
+    }
+
+
+def test_column_reductions_compile_to_a_program_a_fold_and_a_post_program(ctx):
+    gpu = _col_bodies(kernel)
+    x, y, out = FakeDev((40, 100), "float32"), FakeDev((40, 100), "float32"), FakeDev((100,), "float32")
+    want = {
+        "col_sums": ("sum", [("in", 0, 0.0), ("mul_in", 1, 0.0)], []),
+        "col_max_abs": ("max", [("in", 0, 0.0), ("sub_in", 1, 0.0), ("abs", 0, 0.0)], []),
+        "col_means": ("sum", [("in", 0, 0.0), ("add_in", 1, 0.0)],
+                      [("in", 0, 0.0), ("divi", 0, 40.0), ("muli", 0, 0.5)]),
+        "col_norms": ("sum", None, [("in", 0, 0.0), ("sqrt", 0, 0.0)]),
+    }
+    names = {code: op for op, code in rt.MAP_OPS.items()}
+    for name, (kind, program, post) in want.items():
+        (p,) = gpu[name].plan(x, y, out, 32, ctx=ctx)
+        assert p.fn is rt.hcamdLaunchMapReduceCols
+        assert p.args[1] == rt.COLS_KINDS[kind] and p.args[12:14] == (40, 100)
+        got = [(names[p.args[2][i].op], p.args[2][i].arg, p.args[2][i].imm)
+               for i in range(p.args[3])]
+        if program is not None:
+            assert got == program
+        got_post = [(names[p.args[4][i].op], p.args[4][i].arg, p.args[4][i].imm)
+                    for i in range(p.args[5])]
+        assert got_post == post
+    # fp16 sums are refused with the advice to cast, as for rows
+    x16 = FakeDev((40, 100), "float16")
+    with pytest.raises(NoNativeKernel, match="cast the tile"):
+        gpu["col_sums"].plan(x16, x16, FakeDev((100,), "float16"), 32, ctx=ctx)
+    # tiles that do not hold whole columns
+    M, N = sym.M, sym.N
+
+    @kernel(work_shape=(cdiv(M, 8), cdiv(N, 32)), group_shape=(1, 1))
+    def partial(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[N, DT]):
+        t = gr.load(x[gr.id[0] * 8:, gr.id[1] * 32:], shape=(8, 32))
+        gr.store(out[gr.id[1] * 32:], t.sum(axis=0))
+    with pytest.raises(NoNativeKernel, match="whole columns"):
+        partial.plan(x, out, ctx=ctx)
+
+
 def random_row_expression(rng, depth):
     """A function of two (rows, N) tiles T, U and a vector W of N elements that
     mixes elementwise arithmetic with reductions along axis 1, and its source
