@@ -361,6 +361,33 @@ def make_workloads(rt, wl):
         def cpu(self):
             return _best_of(lambda: self._numpy(self.x), 2), "full size, NumPy fp32", 1
 
+    class X6(Workload):
+        """Root mean square down the columns of the C3 matrix, written as a kernel
+        body with a mean along axis 0 of whole-column tiles and launched through
+        the @kernel front-end (the column-reduction kernel, three levels)."""
+
+        def setup(self, rt):
+            from hc_amd.examples import column_rms
+            self.kernel = column_rms()
+            (self.x,) = W.inputs_c3()
+            return [(rt.to_device(self.x), rt.DeviceArray((self.x.shape[1],), np.float32))
+                    for _ in range(ROTATE)]
+
+        def plan(self, rt, s):
+            (p,) = self.kernel.plan_cols(*s)
+            return p
+
+        def _numpy(self, x):
+            return np.sqrt((x * x).mean(axis=0) + x.dtype.type(1e-6))
+
+        def check(self, rt, s):
+            got, want = s[1].to_host(), self._numpy(self.x.astype(np.float64))
+            ok = np.allclose(got, want, rtol=1e-5)
+            return {"parity": "rtol 1e-5 vs fp64" if ok else "MISMATCH", "ok": bool(ok)}
+
+        def cpu(self):
+            return _best_of(lambda: self._numpy(self.x), 2), "full size, NumPy fp32", 1
+
     table = {
         "c0": C0("c0", "copy 256 MiB int32 (calibration)", "u32", "hbm", 2 * 4 * 64 * 1024 * 1024,
                  "GB/s"),
@@ -379,11 +406,13 @@ def make_workloads(rt, wl):
                  "f32", "valu", 2 * 64 * 64 * 64 * 9 * 56 * 56, "TFLOP/s"),
         "x5": X5("x5", "row program: layer norm fp32 4096x8192 with weight and bias", "f32", "hbm",
                  W.work_c3(), "GB/s"),
+        "x6": X6("x6", "column reduction: root mean square down the columns, fp32 4096x8192", "f32",
+                 "hbm", W.work_c3() // 2 + 4 * 8192, "GB/s"),
     }
     if wl == "all":
         keys = ["c1", "c2", "c3", "c4", "c5"]
     elif wl == "extra":
-        keys = ["x1", "x2", "x3", "x4", "x5"]
+        keys = ["x1", "x2", "x3", "x4", "x5", "x6"]
     else:
         keys = [wl]
     return [table[k] for k in keys]
@@ -450,7 +479,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="all", choices=["all", "c0", "c1", "c2", "c3", "c4", "c5", "extra", "x1", "x2", "x3", "x4", "x5"])
+    ap.add_argument("--workload", default="all", choices=["all", "c0", "c1", "c2", "c3", "c4", "c5", "extra", "x1", "x2", "x3", "x4", "x5", "x6"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy CPU baseline")
     ap.add_argument("--prewarm", type=float, default=PREWARM_SECONDS,
                     help="seconds of untimed device warm-up per workload")

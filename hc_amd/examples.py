@@ -67,3 +67,23 @@ def layer_norm(eps: float = 1e-5, rows_per_group: int = 8):
         return body.plan(x, weight, bias, out, rows_per_group, **kw)
     body.plan_rows = plan
     return body
+
+
+def column_rms(eps: float = 1e-6, cols_per_group: int = 512):
+    """out[c] = sqrt(mean(x[:, c] ** 2) + eps) down the columns of a float32
+    matrix: a body that reduces tiles holding whole columns along axis 0 (the
+    tile methods the simulator forwards to NumPy,
+    python/hckernel/kernel_api.py:150-151).  A group owns `cols_per_group`
+    columns."""
+    M, N, GN = sym.M, sym.N, sym.GN
+
+    @kernel(work_shape=(N + GN - 1) // GN, group_shape=1, literals={GN})
+    def body(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[N, DT], gn: GN):
+        n0 = gr.id[0] * GN
+        t = gr.load(x[:, n0:], shape=(M, GN))
+        gr.store(out[n0:], np.sqrt((t * t).mean(axis=0) + np.float32(eps)))
+
+    def plan(x, out, **kw):
+        return body.plan(x, out, cols_per_group, **kw)
+    body.plan_cols = plan
+    return body
