@@ -1235,28 +1235,22 @@ void colBands(size_t rows, size_t cols, size_t &bands, size_t &band) {
   bands = ceilDiv(rows, band);
 }
 
-// Levels of a reduction: the bands of one level are the rows of the next.
-// Returns the floats of workspace all levels need together.
-size_t colLevels(size_t rows, size_t cols, std::vector<std::pair<size_t, size_t>> *levels) {
-  const size_t colsPad = ceilDiv(cols, (size_t)8) * 8;
-  size_t floats = 0;
-  for (;;) {
-    size_t bands, band;
-    colBands(rows, cols, bands, band);
-    if (levels)
-      levels->push_back({bands, band});
-    if (bands == 1)
-      return floats;
-    floats += bands * colsPad;
-    rows = bands;
-  }
+// The bands of the first launch are the rows of the second, which always
+// finishes: it spreads its few rows over the lanes of a wave (fewer lanes per
+// row), so that a wave has them all in flight in one or two turns.
+size_t colSecondLanes(size_t bands, size_t lanes) {
+  while (lanes > 1 && ceilDiv(bands, 16 * (64 / lanes)) > 1)
+    lanes /= 2;
+  return lanes;
 }
 } // namespace
 
 size_t hcamdMapReduceColsWorkspace(size_t rows, size_t cols) noexcept {
   if (rows == 0 || cols == 0)
     return 0;
-  return colLevels(rows, cols, nullptr) * sizeof(float);
+  size_t bands, band;
+  colBands(rows, cols, bands, band);
+  return bands > 1 ? bands * ceilDiv(cols, (size_t)8) * 8 * sizeof(float) : 0;
 }
 
 int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, size_t nInstr,
@@ -1330,39 +1324,16 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
       a.f16_mask |= 1u << i;
     allVec = allVec && aligned16(inputs[i]) && (inputLd[i] * size) % 16 == 0;
   }
-  std::vector<std::pair<size_t, size_t>> levels;
   const size_t colsPad = ceilDiv(cols, (size_t)8) * 8;
-  const size_t floats = colLevels(rows, cols, &levels);
+  size_t bands, band;
+  colBands(rows, cols, bands, band);
+  const size_t floats = bands > 1 ? bands * colsPad : 0;
   if (floats && (!workspace || !aligned16(workspace) || workspaceBytes < floats * sizeof(float))) {
     dev->report("%s: workspace of %zu bytes, 16-byte aligned, needed (%zu given)", who,
                 floats * sizeof(float), workspaceBytes);
     return 1;
   }
-  const size_t lanes = colLanes(cols);
-  const size_t blocks = ceilDiv(colsPad / 8, lanes);
-  a.cols = cols;
-  a.n_instr = static_cast<uint32_t>(nInstr);
-  std::memcpy(a.prog, prog, nInstr * sizeof(HcamdMapInstr));
-  c.kind = static_cast<uint32_t>(kind);
-  c.colsPad = static_cast<uint32_t>(colsPad);
-  c.lanes = static_cast<uint32_t>(lanes);
-  c.interleaved = allVec ? 0u : 1u;
-  float *level = static_cast<float *>(workspace);
-  size_t nIn = nInputs, levelRows = rows;
-  for (size_t l = 0; l < levels.size(); ++l) {
-    const size_t bands = levels[l].first;
-    a.rows = levelRows;
-    c.band = static_cast<uint32_t>(levels[l].second);
-    c.partial = level;
-    if (bands == 1) { // the last launch runs `post` and stores
-      a.out = out;
-      if (outType == HCAMD_F16)
-        a.f16_mask |= 1u << 8;
-      c.outVec = aligned16(out) ? 1u : 0u;
-      c.nPost = static_cast<uint32_t>(nPost);
-      if (nPost)
-        std::memcpy(c.post, post, nPost * sizeof(HcamdMapInstr));
-    }
+  auto launchOne = [&](MapArgs &ma, ColArgs &ca, size_t nIn, size_t nBands) {
     const char *name = nIn <= 1   ? "hcamd_map_reduce_cols_n1u4"
                        : nIn <= 2 ? "hcamd_map_reduce_cols_n2u2"
                                   : "hcamd_map_reduce_cols_n4u1";
@@ -1370,26 +1341,52 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
     if (!k)
       return 1;
     uint32_t n = static_cast<uint32_t>(nIn);
-    void *args[] = {&a, &c, &n};
-    const size_t grid[3] = {blocks, bands, 1}, block[3] = {256, 1, 1};
-    if (int rc = launch(queue, k, grid, block, args, 0))
-      return rc;
-    if (bands == 1)
-      break;
-    // the bands just written are the rows of an fp32 operand of the next level
-    std::memset(a.in, 0, sizeof a.in);
-    std::memset(a.ld, 0, sizeof a.ld);
-    a.in[0] = level;
-    a.ld[0] = colsPad;
-    a.f16_mask = 0;
-    a.n_instr = 1;
-    a.prog[0] = HcamdMapInstr{HCAMD_MAP_IN, 0, 0.0f};
-    c.interleaved = 0;
-    nIn = 1;
-    levelRows = bands;
-    level += bands * colsPad;
+    void *args[] = {&ma, &ca, &n};
+    const size_t grid[3] = {ceilDiv(colsPad / 8, (size_t)ca.lanes), nBands, 1};
+    const size_t block[3] = {256, 1, 1};
+    return launch(queue, k, grid, block, args, 0);
+  };
+  // the launch that runs `post` and stores
+  auto finishing = [&](MapArgs &ma, ColArgs &ca) {
+    ma.out = out;
+    if (outType == HCAMD_F16)
+      ma.f16_mask |= 1u << 8;
+    ca.outVec = aligned16(out) ? 1u : 0u;
+    ca.nPost = static_cast<uint32_t>(nPost);
+    if (nPost)
+      std::memcpy(ca.post, post, nPost * sizeof(HcamdMapInstr));
+  };
+  a.rows = rows;
+  a.cols = cols;
+  a.n_instr = static_cast<uint32_t>(nInstr);
+  std::memcpy(a.prog, prog, nInstr * sizeof(HcamdMapInstr));
+  c.kind = static_cast<uint32_t>(kind);
+  c.colsPad = static_cast<uint32_t>(colsPad);
+  c.band = static_cast<uint32_t>(band);
+  c.lanes = static_cast<uint32_t>(colLanes(cols));
+  c.interleaved = allVec ? 0u : 1u;
+  if (bands == 1) {
+    finishing(a, c);
+    return launchOne(a, c, nInputs, 1);
   }
-  return 0;
+  c.partial = static_cast<float *>(workspace);
+  if (int rc = launchOne(a, c, nInputs, bands))
+    return rc;
+  // the bands just written are the rows of an fp32 operand
+  MapArgs a2{};
+  ColArgs c2{};
+  a2.in[0] = workspace;
+  a2.ld[0] = colsPad;
+  a2.rows = bands;
+  a2.cols = cols;
+  a2.n_instr = 1;
+  a2.prog[0] = HcamdMapInstr{HCAMD_MAP_IN, 0, 0.0f};
+  c2.kind = c.kind;
+  c2.colsPad = c.colsPad;
+  c2.band = static_cast<uint32_t>(bands);
+  c2.lanes = static_cast<uint32_t>(colSecondLanes(bands, c.lanes));
+  finishing(a2, c2);
+  return launchOne(a2, c2, 1, 1);
 }
 
 namespace {
