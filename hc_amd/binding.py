@@ -1245,36 +1245,58 @@ class _PostCompiler(_MapCompiler):
             super().emit(t, out)
 
 
-def match_cols(dst_view, value, n_groups):
-    """value = post(reduce(f(tiles...), axis=0)): sums, maxima, minima, means
-    and 2-norms down the columns of (rows, N) tiles that hold whole columns of
-    their arrays, one group per block of columns.  The tile methods are the ones
-    the simulator forwards to NumPy (python/hckernel/kernel_api.py:150-151)."""
-    if dst_view.base.dtype_name not in _MAP_FLOATS:
-        return None
-    # walk down from the stored value to the reduction
-    t = value
-    while True:
-        if (t.op in _ROW_REDUCE or t.op == "norm") and t.attrs.get("axes") == (0,) \
-                and len(t.args) == 1 and len(t.args[0].shape) == 2:
-            break
-        if len(t.args) == 1 and (_is(t, "astype", 1) or t.op in _MAP_UNARY or _is(t, "clip", 1)):
-            t = t.args[0]
-        elif t.op in _MAP_BINARY and len(t.args) == 2 and _const(t.args[0]) != _const(t.args[1]):
-            t = t.args[0] if _const(t.args[1]) else t.args[1]
+def _is_col_reduce(t: Tile) -> bool:
+    return (t.op in _ROW_REDUCE or t.op == "norm") and t.attrs.get("axes") == (0,) \
+        and len(t.args) == 1 and len(t.args[0].shape) == 2
+
+
+class _ColBodyCompiler(_MapCompiler):
+    """The expression under a column reduction.  Besides (rows, N) tiles it may
+    read per-column vectors of shape (1, N): the results of earlier column
+    reductions (`temps`: uid of the reduction -> operand slot), which every row
+    uses."""
+
+    def __init__(self, n_groups, temps):
+        super().__init__(n_groups)
+        self.temps = temps            # uid -> index into the list of temporaries
+        self.temp_operand = {}        # index of a temporary -> operand number
+
+    def supported(self, t: Tile) -> bool:
+        if t.uid in self.temps:
+            return True
+        if t.op in _MAP_BINARY and len(t.args) == 2 and not all(_const(a) for a in t.args) \
+                and t.dtype_name in _MAP_FLOATS and len(t.shape) == 2:
+            return all(self.supported(a) and (_const(a) or a.shape in (t.shape, (1, t.shape[1])))
+                       for a in t.args)
+        return super().supported(t)
+
+    def need(self, t: Tile) -> int:
+        return 1 if t.uid in self.temps else super().need(t)
+
+    def emit(self, t: Tile, out: list):
+        if t.uid in self.temps:
+            k = self.temps[t.uid]
+            if k not in self.temp_operand:
+                self.inputs.append((None, k, t))
+                self.temp_operand[k] = len(self.inputs) - 1
+            out.append(("in", self.temp_operand[k], 0.0))
         else:
-            return None
-    red, body = t, t.args[0]
-    rows, n = body.shape
+            super().emit(t, out)
+
+
+def _compile_col_reduce(red: Tile, root: Tile, n_groups, temps):
+    """(kind, program, post, compiler) of root = post(red), red a reduction
+    along axis 0."""
+    body = red.args[0]
     if red.op == "norm":          # numpy.linalg.norm along an axis is sqrt(add.reduce(x * x))
         body = body * body
     if red.op in ("sum", "norm") and body.dtype_name != "float32":
         raise NoNativeKernel("column sums are computed in float32: cast the tile with "
                              ".astype(np.float32) before adding it up")
-    comp = _MapCompiler(n_groups)
+    comp = _ColBodyCompiler(n_groups, temps)
     if _const(body) or not comp.supported(body):
         raise NoNativeKernel(f"{body!r} is not an elementwise expression of float32 / float16 "
-                             "tiles and constants")
+                             "tiles, earlier column reductions and constants")
     if comp.need(body) > rt.MAP_STACK_DEPTH:
         raise NoNativeKernel("expression needs an evaluation stack deeper than "
                              f"{rt.MAP_STACK_DEPTH}")
@@ -1287,42 +1309,112 @@ def match_cols(dst_view, value, n_groups):
     post: list = []
     if red.op == "norm":
         post = [("in", 0, 0.0), ("sqrt", 0, 0.0)]
-    if value is not red:
+    if root is not red:
         pc = _PostCompiler(n_groups, red)
-        if not pc.supported(value):
-            raise NoNativeKernel(f"{value!r}: what follows a column reduction must be float32 / "
+        if not pc.supported(root):
+            raise NoNativeKernel(f"{root!r}: what follows a column reduction must be float32 / "
                                  "float16 arithmetic with constants")
         tail: list = []
-        pc.emit(value, tail)
+        pc.emit(root, tail)
         post = post + tail[1:] if post else tail
     if len(post) > rt.COLS_MAX_POST:
         raise NoNativeKernel(f"{len(post)} operations follow the column reduction "
                              f"(at most {rt.COLS_MAX_POST})")
-    wins = [window_of(tl.attrs["view"], tl.shape, n_groups) for _, _, tl in comp.inputs]
-    w = wins[0]
-    for x, (_, _, tl) in zip(wins, comp.inputs):
-        if len(x.extent) != 2 or x.extent != w.extent or x.driver != w.driver:
-            raise NoNativeKernel("the tiles of a column reduction must walk the same columns")
-        if x.driver[0] is not None or tl.shape[0] != tl.attrs["view"].base.shape[0]:
-            raise NoNativeKernel("column reductions need tiles that hold whole columns "
-                                 "(as many rows as the array has)")
+    kind = "sum" if red.op == "norm" else _ROW_REDUCE[red.op]
+    return kind, program, post, comp
+
+
+def match_cols(dst_view, value, n_groups):
+    """value = post(reduce(f(tiles...), axis=0)): sums, maxima, minima, means,
+    variances, standard deviations and 2-norms down the columns of (rows, N)
+    tiles that hold whole columns of their arrays, one group per block of
+    columns.  The tile methods are the ones the simulator forwards to NumPy
+    (python/hckernel/kernel_api.py:150-151).  A reduction whose expression
+    reads an earlier one (the centred squares of a variance read the mean) runs
+    after it, the earlier result in a temporary vector that every row uses."""
+    if dst_view.base.dtype_name not in _MAP_FLOATS:
+        return None
+    # walk down from the stored value to the reduction
+    t = value
+    while not _is_col_reduce(t):
+        if len(t.args) == 1 and (_is(t, "astype", 1) or t.op in _MAP_UNARY or _is(t, "clip", 1)):
+            t = t.args[0]
+        elif t.op in _MAP_BINARY and len(t.args) == 2 and _const(t.args[0]) != _const(t.args[1]):
+            t = t.args[0] if _const(t.args[1]) else t.args[1]
+        else:
+            return None
+    outer = t
+    # reductions inside the reduced expression, innermost first
+    order, seen = [], set()
+
+    def inner(t):
+        if t.uid in seen:
+            return
+        seen.add(t.uid)
+        for a in t.args:
+            inner(a)
+        if _is_col_reduce(t) and t is not outer:
+            if not t.attrs.get("keepdims"):
+                raise NoNativeKernel("a column reduction that an expression reads back needs "
+                                     "keepdims=True")
+            order.append(t)
+    inner(outer.args[0])
+    temps, steps = {}, []
+    for red in order:
+        steps.append(_compile_col_reduce(red, red, n_groups, dict(temps)))
+        temps[red.uid] = len(temps)
+    steps.append(_compile_col_reduce(outer, value, n_groups, dict(temps)))
+    # windows: every tile of every step walks the same whole columns
+    w, step_wins = None, []
+    for _, _, _, comp in steps:
+        wins = []
+        for b, _, tl in comp.inputs:
+            if b is None:
+                wins.append(None)
+                continue
+            x = window_of(tl.attrs["view"], tl.shape, n_groups)
+            w = w or x
+            if len(x.extent) != 2 or x.extent != w.extent or x.driver != w.driver:
+                raise NoNativeKernel("the tiles of a column reduction must walk the same columns")
+            if x.driver[0] is not None or tl.shape[0] != tl.attrs["view"].base.shape[0]:
+                raise NoNativeKernel("column reductions need tiles that hold whole columns "
+                                     "(as many rows as the array has)")
+            wins.append(x)
+        step_wins.append(wins)
+    if w is None:
+        return None
     wo = window_of(dst_view, value.shape, n_groups)
     if wo.extent[-1] != w.extent[1] or wo.driver[-1] != w.driver[1] or \
             math.prod(wo.extent) != wo.extent[-1]:
         raise NoNativeKernel("the per-column result and the tiles walk different columns")
     ftype = lambda name: rt.F16 if name == "float16" else rt.F32
-    types = [ftype(tl.dtype_name) for _, _, tl in comp.inputs] + [ftype(dst_view.base.dtype_name)]
-    kind = "sum" if red.op == "norm" else _ROW_REDUCE[red.op]
     n_cols = w.extent[1]
 
     def make(mem, ctx):
-        ins = [_Arr(_sub(mem[x.buffer], x.extent), ctx) for x in wins]
+        import numpy as np
         mo = mem[wo.buffer]
         if n_cols > 1 and mo.strides[-1] != 1:
             raise NoNativeKernel("the per-column result must be contiguous")
-        out = _Arr(rt.Memref(mo.ptr, (n_cols,), (1,), mo.itemsize), ctx)
-        return [rt.plan_map_reduce_cols(kind, program, ins, out, post, types)]
-    make.program, make.post, make.kind = program, post, kind
+        vectors = [rt.DeviceArray((n_cols,), np.float32, ctx) for _ in order]
+        plans = []
+        for i, ((kind, program, post, comp), wins) in enumerate(zip(steps, step_wins)):
+            ins, types = [], []
+            for (b, k, tl), x in zip(comp.inputs, wins):
+                if b is None:
+                    ins.append(vectors[k])
+                    types.append(rt.F32)
+                else:
+                    ins.append(_Arr(_sub(mem[x.buffer], x.extent), ctx))
+                    types.append(ftype(tl.dtype_name))
+            if i < len(order):
+                out, out_type = vectors[i], rt.F32
+            else:
+                out = _Arr(rt.Memref(mo.ptr, (n_cols,), (1,), mo.itemsize), ctx)
+                out_type = ftype(dst_view.base.dtype_name)
+            plans.append(rt.plan_map_reduce_cols(kind, program, ins, out, post, types + [out_type]))
+        return plans
+    make.program, make.post, make.kind = steps[-1][1], steps[-1][2], steps[-1][0]
+    make.steps = [(k, pr, po) for k, pr, po, _ in steps]
     return make
 
 

@@ -740,11 +740,13 @@ def test_row_reduction_bodies_match_the_simulator(name, rows, n):
 @pytest.mark.parametrize("rows,n,gn", [(37, 200, 64), (3000, 4096, 512), (70_000, 24, 24),
                                        (513, 1031, 1031)])
 @pytest.mark.parametrize("name", ["col_sums", "col_max_abs", "col_min", "col_means", "col_norms",
-                                  "col_rms"])
+                                  "col_rms", "col_var", "col_std"])
 def test_column_reduction_bodies_match_the_simulator(name, rows, n, gn):
     """The same body on the GPU and on the CPU simulator: maxima and minima bit
     for bit, sums within the fp32 bound of adding `rows` terms in another
-    order, what is computed from a sum to the same relative bound."""
+    order, what is computed from a sum to the same relative bound.  The
+    variance and the standard deviation are two reductions, the second reading
+    the first one's result from a temporary vector."""
     from test_kernel_frontend import _col_bodies
     rng = np.random.default_rng(rows + n)
     x = rng.standard_normal((rows, n)).astype(np.float32)
@@ -759,8 +761,10 @@ def test_column_reduction_bodies_match_the_simulator(name, rows, n, gn):
         assert_array_equal(got, want)
     else:
         x64, y64 = x.astype(np.float64), y.astype(np.float64)
-        terms = {"col_sums": x64 * y64, "col_means": x64 + y64, "col_norms": (x64 - y64) ** 2,
-                 "col_rms": x64 * x64}[name]
+        d64 = x64 - y64
+        terms = {"col_sums": x64 * y64, "col_means": x64 + y64, "col_norms": d64 ** 2,
+                 "col_rms": x64 * x64, "col_var": (x64 - x64.mean(axis=0)) ** 2,
+                 "col_std": (d64 - d64.mean(axis=0)) ** 2}[name]
         rel = (rows + 2) * 2.0 ** -23 * np.abs(terms).sum(axis=0) / np.maximum(np.abs(terms.sum(axis=0)), 1e-30)
         assert (np.abs(got - want) <= (rel + 4e-7) * np.abs(want) + 1e-30).all()
 

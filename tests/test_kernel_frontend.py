@@ -949,6 +949,8 @@ def _col_bodies(deco):
         "col_means": body(lambda a, b: (a + b).mean(axis=0) * f32(0.5)),
         "col_norms": body(lambda a, b: np.linalg.norm(a - b, axis=0)),
         "col_rms": body(lambda a, b: np.sqrt((a * a).sum(axis=0) / f32(a.shape[0]) + f32(1e-6))),
+        "col_var": body(lambda a, b: a.var(axis=0)),
+        "col_std": body(lambda a, b: (a - b).std(axis=0, ddof=1)),
     }
 
 
