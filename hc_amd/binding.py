@@ -1418,6 +1418,100 @@ def match_cols(dst_view, value, n_groups):
     return make
 
 
+def match_cols_tile(dst_view, value, n_groups):
+    """A stored (rows, N) tile expression that reads reductions down its own
+    columns, e.g. (x - x.mean(axis=0, keepdims=True)) / x.std(axis=0,
+    keepdims=True): the reductions run first, each into a temporary vector, and
+    the tile is then one elementwise pass in which every row uses those
+    vectors."""
+    if dst_view.base.dtype_name not in _MAP_FLOATS or len(value.shape) != 2:
+        return None
+    order, seen = [], set()
+
+    def inner(t):
+        if t.uid in seen:
+            return
+        seen.add(t.uid)
+        for a in t.args:
+            inner(a)
+        if _is_col_reduce(t):
+            if not t.attrs.get("keepdims"):
+                raise NoNativeKernel("a column reduction that an expression reads back needs "
+                                     "keepdims=True")
+            order.append(t)
+    inner(value)
+    if not order:
+        return None
+    temps, steps = {}, []
+    for red in order:
+        steps.append(_compile_col_reduce(red, red, n_groups, dict(temps)))
+        temps[red.uid] = len(temps)
+    final = _ColBodyCompiler(n_groups, dict(temps))
+    if not final.supported(value):
+        raise NoNativeKernel(f"{value!r} is not an elementwise expression of float32 / float16 "
+                             "tiles, column reductions and constants")
+    if final.need(value) > rt.MAP_STACK_DEPTH:
+        raise NoNativeKernel("expression needs an evaluation stack deeper than "
+                             f"{rt.MAP_STACK_DEPTH}")
+    program: list = []
+    final.emit(value, program)
+    if len(program) > rt.MAP_MAX_INSTRS or len(final.inputs) > rt.MAP_MAX_INPUTS:
+        raise NoNativeKernel(f"the stored expression compiles to {len(program)} operations on "
+                             f"{len(final.inputs)} arrays (at most {rt.MAP_MAX_INSTRS} on "
+                             f"{rt.MAP_MAX_INPUTS})")
+    w, step_wins = None, []
+    for comp in [st[3] for st in steps] + [final]:
+        wins = []
+        for b, _, tl in comp.inputs:
+            if b is None:
+                wins.append(None)
+                continue
+            x = window_of(tl.attrs["view"], tl.shape, n_groups)
+            w = w or x
+            if len(x.extent) != 2 or x.extent != w.extent or x.driver != w.driver:
+                raise NoNativeKernel("the tiles of a column reduction must walk the same columns")
+            if x.driver[0] is not None or tl.shape[0] != tl.attrs["view"].base.shape[0]:
+                raise NoNativeKernel("column reductions need tiles that hold whole columns "
+                                     "(as many rows as the array has)")
+            wins.append(x)
+        step_wins.append(wins)
+    if w is None or all(x is None for x in step_wins[-1]):
+        return None
+    wo = window_of(dst_view, value.shape, n_groups)
+    if wo.extent != w.extent or wo.driver != w.driver:
+        raise NoNativeKernel("loads and the store walk different windows")
+    ftype = lambda name: rt.F16 if name == "float16" else rt.F32
+    n_cols = w.extent[1]
+
+    def make(mem, ctx):
+        import numpy as np
+        vectors = [rt.DeviceArray((n_cols,), np.float32, ctx) for _ in order]
+
+        def operands(comp, wins):
+            ins, types = [], []
+            for (b, k, tl), x in zip(comp.inputs, wins):
+                if b is None:
+                    ins.append(vectors[k])
+                    types.append(rt.F32)
+                else:
+                    ins.append(_Arr(_sub(mem[x.buffer], x.extent), ctx))
+                    types.append(ftype(tl.dtype_name))
+            return ins, types
+        plans = []
+        for i, (kind, prog, post, comp) in enumerate(steps):
+            ins, types = operands(comp, step_wins[i])
+            plans.append(rt.plan_map_reduce_cols(kind, prog, ins, vectors[i], post,
+                                                 types + [rt.F32]))
+        ins, types = operands(final, step_wins[-1])
+        out = _Arr(_sub(mem[wo.buffer], wo.extent), ctx)
+        plans.append(rt.plan_row_program([("store", 0, program)], ins, out, (),
+                                         types + [ftype(dst_view.base.dtype_name)]))
+        return plans
+    make.program = program
+    make.steps = [(k, pr, po) for k, pr, po, _ in steps]
+    return make
+
+
 def match_pairwise(dst_view, value, n_groups):
     """out[m, n] = ||a[m, :] - b[n, :]||: the body of
     python/hckernel/tests/test_examples.py:270-301."""
@@ -1552,7 +1646,8 @@ def bind(stores, n_groups, atomics=(), mapped_stores=()):
             return makers + [q]
         for view, value in stores:
             for matcher in (match_copy, match_add, match_fma, match_softmax, match_gemm,
-                            match_gather_gemm, match_pairwise, match_cols, match_rows, match_map):
+                            match_gather_gemm, match_pairwise, match_cols, match_cols_tile, match_rows,
+                            match_map):
                 mk = matcher(view, value, n_groups)
                 if mk is not None:
                     makers.append(mk)

@@ -769,6 +769,25 @@ def test_column_reduction_bodies_match_the_simulator(name, rows, n, gn):
         assert (np.abs(got - want) <= (rel + 4e-7) * np.abs(want) + 1e-30).all()
 
 
+@pytest.mark.parametrize("rows,n,gn", [(37, 200, 64), (2000, 1031, 256), (5000, 24, 24)])
+@pytest.mark.parametrize("name", ["batch_norm", "col_softmax", "centre"])
+def test_tiles_computed_from_their_own_column_reductions_match_the_simulator(name, rows, n, gn):
+    """The reductions run first, each into a temporary vector; the tile is then
+    one elementwise pass.  fp32 results agree with the simulator to the bound
+    of sums added in another order."""
+    from test_kernel_frontend import _col_tile_bodies
+    rng = np.random.default_rng(rows + n)
+    x = rng.standard_normal((rows, n)).astype(np.float32)
+    w = rng.standard_normal((rows, n)).astype(np.float32)
+    want = np.zeros((rows, n), np.float32)
+    _col_tile_bodies(sim_kernel)[name](x, w, want, gn)
+    out = rt.DeviceArray((rows, n), np.float32).fill_bytes32(0xA5A5A5A5)
+    _col_tile_bodies(kernel)[name](rt.to_device(x), rt.to_device(w), out, gn)
+    assert rt.last_kernel_name().startswith(("hcamd_row_program", "hcamd_map"))
+    got = out.to_host()
+    assert_allclose(got, want, rtol=(rows + 8) * 2.0 ** -23, atol=(rows + 8) * 2.0 ** -23)
+
+
 def test_softmax_with_a_temperature_is_a_row_program_and_plain_softmax_keeps_its_kernel():
     M, N, GM = sym.M, sym.N, sym.GM
 

@@ -954,6 +954,35 @@ def _col_bodies(deco):
     }
 
 
+def _col_tile_bodies(deco):
+    """Bodies that store a (M, GN) tile computed from reductions down its own
+    columns (a batch normalisation, a column softmax)."""
+    M, N, GN = sym.M, sym.N, sym.GN
+
+    def body(fn):
+        @deco(work_shape=cdiv(N, GN), group_shape=1, literals={GN})
+        def k(gr: CurrentGroup, x: Buffer[M, N, DT], w: Buffer[M, N, DT], out: Buffer[M, N, DT],
+              gn: GN):
+            n0 = gr.id[0] * GN
+            tx = gr.load(x[:, n0:], shape=(M, GN))
+            tw = gr.load(w[:, n0:], shape=(M, GN))
+            gr.store(out[:, n0:], fn(tx, tw))
+        return k
+
+    f32 = np.float32
+
+    def batch_norm(a, b):
+        mean = a.mean(axis=0, keepdims=True)
+        return (a - mean) / np.sqrt(a.var(axis=0, keepdims=True) + f32(1e-5)) * b
+
+    def col_softmax(a, b):
+        e = np.exp(a - a.max(axis=0, keepdims=True))
+        return e / e.sum(axis=0, keepdims=True)
+
+    return {"batch_norm": body(batch_norm), "col_softmax": body(col_softmax),
+            "centre": body(lambda a, b: a - (a * b).sum(axis=0, keepdims=True) / f32(a.shape[0]))}
+
+
 def test_column_reductions_compile_to_a_program_a_fold_and_a_post_program(ctx):
     gpu = _col_bodies(kernel)
     x, y, out = FakeDev((40, 100), "float32"), FakeDev((40, 100), "float32"), FakeDev((100,), "float32")
