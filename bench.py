@@ -54,6 +54,8 @@ MEASURED_TRAFFIC = {
     "c3": int((65566.9 * 2.0 + 131125.1) * _KIB),    # algorithmic 268,435,456
     "c4": int((65869.6 * 2.0 + 66048.0) * _KIB),     # algorithmic 201,392,128
     "c5": int((98362.2 * 2.0 + 32768.0) * _KIB),     # 2.3 x the algorithmic 100,663,296 (L2 refetch)
+    # both launches of the step: the bands (67,221.4 / 2,048.0) and their fold (1,177.5 / 32.0)
+    "x6": int(((67221.4 + 1177.5) * 2.0 + 2048.0 + 32.0) * _KIB),   # algorithmic 134,250,496
 }
 
 
