@@ -28,16 +28,20 @@ Pinning status (what each part is checked against, see tests/test_oracle_*.py):
     statement, rows-sum-to-one and shift invariance.
   * W5 GEMM: exact small-integer matrices, the reference's 16x32x64 dot
     input recipe (test_examples.py:113-121), fp64 accumulation.
-  * parity unpinned: behaviour that follows only from numpy.ma internals
-    (in-place operators on partially active tiles, loads from already masked
-    tiles, domain masking of divide/sqrt/log, np.dot on masked tiles,
-    compressed()/repr).  hcsim follows the documented numpy.ma rules for
-    these, but no reference test or fixture fixes them.
-  * parity unpinned: a bare Python scalar next to a tile (`tile * 0.5`).
-    numpy.ma turns the scalar into a 0-d float64 array, so under NumPy >= 2
-    the simulator computes such an expression in float64, under NumPy 1.x in
-    the tile's type; the reference pins no NumPy version and no test covers
-    it.  The GPU front-end gives the scalar the tile's type (what a plain
-    ndarray does); tests that compare the two write scalars as np.float32(..)
-    / np.float16(..), which both sides treat alike.
+  * hcsim behaviour that follows from numpy.ma internals (in-place operators
+    on partially active tiles, loads from already masked tiles, domain
+    masking of / // % **, NumPy functions and reductions on tiles,
+    compressed()/repr, every installed operator on int32 / float32 / bool
+    tiles, stores of numpy.ma results, Python and NumPy scalars next to a
+    tile): tests/golden/sim_golden.json, written by
+    tests/golden/make_sim_golden.py from the reference's own simulator running
+    the bodies of tests/golden/sim_cases.py; tests/test_oracle_sim_golden.py
+    demands equal bytes wherever the reference returns a value.  The vectors
+    are numpy.ma's behaviour at the NumPy version recorded in the file (the
+    reference pins none): under NumPy >= 2 a bare Python scalar promotes a
+    float32 tile to float64 (`tile * 0.5`), a NumPy scalar of the tile's type
+    does not.
+  * W0 copy (np_copy_window, oracle_copy2d): the reference's arange(12) / -1
+    known answer (python/hckernel/tests/test_kernel_sim.py:91-104), a ragged
+    2-D window written out by hand, strided poison-filled views.
 """

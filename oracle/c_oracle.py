@@ -90,6 +90,18 @@ def float_to_bf16(x: np.ndarray) -> np.ndarray:
     return b
 
 
+def copy2d(src: np.ndarray, dst: np.ndarray) -> None:
+    """Masked window copy in place: dst[:r, :c] = src[:r, :c] over the common
+    window; both may be strided 2-D views.  Nothing else of dst is written."""
+    assert src.ndim == 2 and dst.ndim == 2 and src.dtype == dst.dtype
+    e = src.itemsize
+    assert all(s % e == 0 for s in src.strides + dst.strides)
+    lib().oracle_copy2d(e, src.ctypes.data, src.shape[0], src.shape[1],
+                        src.strides[0] // e, src.strides[1] // e,
+                        dst.ctypes.data, dst.shape[0], dst.shape[1],
+                        dst.strides[0] // e, dst.strides[1] // e)
+
+
 def add_f32(a: np.ndarray, b: np.ndarray) -> np.ndarray:
     a = np.ascontiguousarray(a, np.float32)
     b = np.ascontiguousarray(b, np.float32)

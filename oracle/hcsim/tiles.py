@@ -117,8 +117,10 @@ def _install_operators():
             setattr(Tile, f"__r{stem}__", ref)
     for name in unary:
         fn = getattr(operator, name)
-        stem = {"not_": "not", "inv": "invert"}.get(name, name)
-        setattr(Tile, f"__{stem}__", lambda self, _fn=fn: Tile(_fn(self._m)))
+        # kernel_api.py:180-201 names the methods __abs__, __neg__, __not__ and
+        # __inv__; the last two are reachable by name only (`~tile` and
+        # `not tile` never look them up), and so they are here.
+        setattr(Tile, f"__{name.rstrip('_')}__", lambda self, _fn=fn: Tile(_fn(self._m)))
     Tile.__hash__ = None
 
 

@@ -1,0 +1,403 @@
+"""Small kernel bodies whose results follow from numpy.ma internals rather than
+from any test or document of the reference simulator: in-place operators on
+partially active tiles, loads from tiles that are already masked, domain
+masking of divide / floordiv / mod / pow, NumPy functions applied to tiles,
+compressed() / repr, Python scalars next to a tile, and the 19 binary + 4 unary
+operators the simulator installs (python/hckernel/kernel_api.py:106-211).
+
+Every case takes `api`, a namespace with the simulator's public names (`kernel`,
+`sym`, `CurrentGroup`, ...), runs one or more kernels through it and returns a
+flat dict name -> ndarray.  tests/golden/make_sim_golden.py runs them with the
+reference's simulator and writes the results; tests/test_oracle_sim_golden.py
+runs them with oracle.hcsim and compares.  This file holds inputs and recording
+code only, no expected values.
+"""
+
+import operator
+import warnings
+
+import numpy as np
+
+POISON = -77
+
+
+def _text(s):
+    return np.frombuffer(s.encode(), dtype=np.uint8).copy()
+
+
+class Recorder:
+    def __init__(self):
+        self.out = {}
+
+    def tile(self, name, t):
+        """A tile: type tag, dtype, active flags, data where active."""
+        try:
+            has_mask = hasattr(t, "mask") and hasattr(t, "data") and not isinstance(t, np.ndarray)
+        except AssertionError:
+            # the reference's mask property cannot invert numpy.ma's scalar
+            # "no mask" (kernel_api.py:93-103,117-119): such a tile cannot be
+            # stored either, so there is no result to record
+            self.out[name + ".raises"] = _text("AssertionError:mask")
+            return
+        if has_mask:
+            m = np.asarray(t.mask)
+            d = np.asarray(t.data)
+            if m.shape != d.shape:              # numpy.ma's scalar "nomask"
+                m = np.broadcast_to(m, d.shape)
+            kind = "masked_array" if isinstance(t, np.ma.MaskedArray) else "tile"
+            self.out[name + ".kind"] = _text(kind)
+            self.out[name + ".active"] = m.astype(np.uint8)
+            if kind == "masked_array":          # numpy.ma's own polarity: True = masked
+                act = ~m
+            else:
+                act = m
+            self.out[name + ".dtype"] = _text(str(d.dtype))
+            self.out[name + ".value"] = np.where(act, d, np.zeros((), d.dtype))
+        else:
+            a = np.asarray(t)
+            self.out[name + ".kind"] = _text("ndarray" if isinstance(t, np.ndarray) else type(t).__name__)
+            self.out[name + ".dtype"] = _text(str(a.dtype))
+            self.out[name + ".value"] = a
+
+    def array(self, name, a):
+        self.out[name] = np.asarray(a).copy()
+
+    def attempt(self, name, fn):
+        """Records fn()'s tile, or the name of the exception it raises."""
+        try:
+            t = fn()
+        except Exception as e:                  # noqa: BLE001  the type is the datum
+            self.out[name + ".raises"] = _text(type(e).__name__)
+            return None
+        self.tile(name, t)
+        return None if name + ".raises" in self.out else t
+
+
+def _one_group(api, body, *args, group=8):
+    # The symbol parameter is there because the reference's launcher needs at
+    # least one annotated parameter (kernel_sim.py:144-157).
+    def entry(gr, n: api.sym.N, *rest):
+        body(gr, *rest)
+
+    api.kernel(work_shape=api.sym.N, group_shape=group)(entry)(group, *args)
+
+
+def case_inplace_partial(api):
+    rec = Recorder()
+    x = np.arange(1, 9, dtype=np.float32)
+    y = np.array([2, 0, 4, 0.5, -1, 3, 7, 9], dtype=np.float32)
+    dst = np.full((4, 8), POISON, np.float32)
+
+    def body(gr, x, y, dst):
+        a = gr.load(x[:5], shape=8)             # 5 active
+        b = gr.load(y[:3], shape=8)             # 3 active
+        acc = gr.zeros(8, np.float32)           # all active
+        acc += a
+        rec.tile("full_plus_partial", acc)
+        gr.store(dst[0], acc)
+        acc2 = gr.load(x[:5], shape=8)
+        acc2 += b
+        rec.tile("partial_plus_narrower", acc2)
+        acc2 *= b
+        acc2 -= 1.5
+        rec.tile("after_mul_sub", acc2)
+        gr.store(dst[1], acc2)
+        acc3 = gr.load(y[:3], shape=8)
+        acc3 += a                               # wider operand: does activity grow?
+        rec.tile("narrow_plus_wider", acc3)
+        gr.store(dst[2], acc3)
+        acc4 = gr.load(x[:6], shape=8)
+        acc4 /= gr.load(y[:8], shape=8)         # y[1] == 0
+        rec.tile("inplace_div_by_zero", acc4)
+        gr.store(dst[3], acc4)
+
+    with np.errstate(all="ignore"):
+        _one_group(api, body, x, y, dst)
+    rec.array("dst", dst)
+    return rec.out
+
+
+def case_load_from_masked(api):
+    rec = Recorder()
+    x = np.arange(18, dtype=np.int32).reshape(3, 6) + 1
+    dst = np.full((2, 4, 4), POISON, np.int32)
+
+    def body(gr, x, dst):
+        t = gr.load(x, shape=(4, 8))            # 3 x 6 active
+        rec.tile("outer", t)
+        u = gr.load(t[:, 2:], shape=(4, 4))     # window of a masked tile
+        rec.tile("load_window", u)
+        gr.store(dst[0], u)
+        v = gr.vload(t[1:, 4:], shape=(4, 4))   # source smaller than the request
+        rec.tile("vload_window", v)
+        gr.store(dst[1], v)
+        rec.attempt("vec_of_tile", lambda: gr.vec(t, (2, 3)))
+        rec.attempt("vec_whole", lambda: gr.vec(u))
+
+    _one_group(api, body, x, dst)
+    rec.array("dst", dst)
+    return rec.out
+
+
+def case_domain_masking(api):
+    rec = Recorder()
+    num = np.array([4, -9, 0, 7, 5, -3, 8, 1], dtype=np.float32)
+    den = np.array([2, 0, 0, -2, 0.5, 3, 0, 4], dtype=np.float32)
+    inum = np.array([7, -7, 0, 9, 5, -3, 8, 1], dtype=np.int32)
+    iden = np.array([2, 0, 0, -2, 3, 3, 0, 4], dtype=np.int32)
+    dst = np.full((8, 8), POISON, np.float32)
+    idst = np.full((2, 8), POISON, np.int32)
+    pdst = np.full(8, POISON, np.int32)
+
+    def body(gr, num, den, inum, iden, dst, idst, pdst):
+        a, b = gr.load(num, shape=8), gr.load(den[:7], shape=8)
+        ia, ib = gr.load(inum, shape=8), gr.load(iden[:7], shape=8)
+        for row, (name, fn) in enumerate([
+                ("truediv", lambda: a / b),
+                ("floordiv", lambda: a // b),
+                ("mod", lambda: a % b),
+                ("pow_half", lambda: a ** 0.5),
+                ("pow_tile", lambda: a ** b),
+                ("int_truediv", lambda: ia / ib)]):
+            t = rec.attempt(name, fn)
+            if t is not None:
+                gr.store(dst[row], t)
+        for row, (name, fn) in enumerate([
+                ("int_floordiv", lambda: ia // ib),
+                ("int_mod", lambda: ia % ib)]):
+            t = rec.attempt(name, fn)
+            if t is not None:
+                gr.store(idst[row], t)
+        t = rec.attempt("int_pow", lambda: ia ** 2)
+        if t is not None:
+            gr.store(pdst, t)
+            rec.array("int_pow.dst", pdst)
+        # NumPy functions see a tile through __array__
+        for row, (name, fn) in enumerate([("np_sqrt", lambda: np.sqrt(a)),
+                                           ("np_log", lambda: np.log(b))]):
+            t = rec.attempt(name, fn)
+            if t is not None:
+                gr.store(dst[6 + row], t)
+
+    with np.errstate(all="ignore"), warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        _one_group(api, body, num, den, inum, iden, dst, idst, pdst)
+    rec.array("dst", dst)
+    rec.array("idst", idst)
+    return rec.out
+
+
+def case_numpy_functions(api):
+    rec = Recorder()
+    rng = np.random.default_rng(7)
+    x = rng.integers(-4, 5, (3, 5)).astype(np.float64)
+    y = rng.integers(-4, 5, (5, 2)).astype(np.float64)
+    dst = np.full((4, 4), POISON, np.float64)
+    dsum = np.full((3, 4), POISON, np.float64)
+
+    def body(gr, x, y, dst, dsum):
+        a = gr.load(x, shape=(4, 6))            # 3 x 5 active of 4 x 6
+        b = gr.load(y, shape=(6, 4))            # 5 x 2 active of 6 x 4
+        rec.attempt("np_dot", lambda: np.dot(a, b))
+        rec.attempt("matmul", lambda: a @ b)
+        rec.attempt("norm_rows", lambda: np.linalg.norm(a, axis=-1))
+        rec.attempt("np_exp", lambda: np.exp(a))
+        rec.attempt("sum_all", lambda: a.sum())
+        rec.attempt("max_all", lambda: a.max())
+        rec.attempt("sum_rows", lambda: a.sum(axis=1))
+        rec.attempt("max_cols", lambda: a.max(axis=0))
+        rec.attempt("mean_cols", lambda: a.mean(axis=0))
+        rec.attempt("astype", lambda: a.astype(np.float32))
+        rec.attempt("reshape", lambda: a.reshape(6, 4))
+        rec.attempt("transpose", lambda: a.T)
+        rec.attempt("np_sum_function", lambda: np.sum(a))
+        t = rec.attempt("acc_dot", lambda: _acc_dot(gr, a, b))
+        if t is not None:
+            gr.store(dst, t)
+        for row, fn in enumerate([lambda: a.sum(axis=1), lambda: a.max(axis=1),
+                                  lambda: a.min(axis=1)]):
+            gr.store(dsum[row], fn())
+
+    def _acc_dot(gr, a, b):
+        r = gr.zeros((4, 4), np.float64)
+        r += np.dot(a, b)
+        return r
+
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        _one_group(api, body, x, y, dst, dsum)
+    rec.array("dst", dst)
+    rec.array("dsum", dsum)
+    return rec.out
+
+
+def case_compressed_repr(api):
+    rec = Recorder()
+    x = np.arange(10, dtype=np.int64) * 3
+
+    def body(gr, x):
+        t = gr.load(x[2:7], shape=8)
+        rec.array("compressed", t.compressed())
+        rec.array("repr", _text(repr(t)))
+        rec.array("str", _text(str(t)))
+        e = gr.load(x[:0], shape=4)
+        rec.array("compressed_empty", e.compressed())
+        rec.array("repr_all_inactive", _text(repr(e)))
+        z = gr.ones((2, 3), np.float32)
+        rec.array("repr_all_active", _text(repr(z)))
+        rec.array("shape", np.array(t.shape))
+        rec.attempt("len", lambda: np.array(len(z)))
+
+    _one_group(api, body, x)
+    return rec.out
+
+
+def case_scalar_promotion(api):
+    rec = Recorder()
+    xs = {"f32": np.array([1.5, -2.25, 3, 0.1, 7, 8, 9, 10], np.float32),
+          "f16": np.array([1.5, -2.25, 3, 0.1, 7, 8, 9, 10], np.float16),
+          "i32": np.array([1, -2, 3, 4, 7, 8, 9, 10], np.int32)}
+    dst = {k: np.full((4, 8), POISON, v.dtype) for k, v in xs.items()}
+
+    def body(gr, x, dst, tag):
+        t = gr.load(x[:6], shape=8)
+        for row, (name, fn) in enumerate([
+                ("mul_pyfloat", lambda: t * 0.5),
+                ("add_pyint", lambda: t + 1),
+                ("mul_npf32", lambda: t * np.float32(0.5)),
+                ("div_pyint", lambda: t / 2)]):
+            r = rec.attempt(f"{tag}.{name}", fn)
+            if r is not None:
+                gr.store(dst[row], r)
+
+    with np.errstate(all="ignore"):
+        for tag, x in xs.items():
+            _one_group(api, lambda gr, x, d, _t=tag: body(gr, x, d, _t), x, dst[tag])
+    for tag in xs:
+        rec.array(f"dst.{tag}", dst[tag])
+    return rec.out
+
+
+BINARY = ["add", "sub", "mul", "matmul", "truediv", "floordiv", "pow", "mod", "lt", "le",
+          "eq", "ne", "ge", "gt", "and_", "or_", "xor", "rshift", "lshift"]
+UNARY = ["abs", "neg", "not_", "inv"]
+
+
+def case_operators(api):
+    rec = Recorder()
+    xs = {"i32": (np.array([5, -3, 12, 0, 7, -8, 9, 2], np.int32),
+                  np.array([2, 3, 1, 4, 0, 2, 3, 1], np.int32)),
+          "f32": (np.array([5.5, -3, 12, 0, 7, -8.25, 9, 2], np.float32),
+                  np.array([2, 3, 0.5, 4, 0, 2, 3, 1], np.float32)),
+          "bool": (np.array([1, 0, 1, 1, 0, 0, 1, 0], np.bool_),
+                   np.array([1, 1, 0, 1, 0, 1, 0, 0], np.bool_))}
+
+    def body(gr, x, y, tag):
+        a = gr.load(x[:7], shape=8)
+        b = gr.load(y[1:], shape=8)             # 7 elements, shifted by one
+        for name in BINARY:
+            op = getattr(operator, name)
+            rec.attempt(f"{tag}.{name}", lambda: op(a, b))
+            stem = name.rstrip("_")
+
+            def inplace():
+                c = gr.load(x[:7], shape=8)
+                c = getattr(c, f"__i{stem}__")(b)
+                return c
+
+            rec.attempt(f"{tag}.i{stem}", inplace)
+        for name in UNARY:
+            # the simulator installs __not__ and __inv__ (kernel_api.py:180-201),
+            # names the interpreter never looks up: the operator form and the
+            # method called by name are different things
+            stem = name.rstrip("_")
+            rec.attempt(f"{tag}.{stem}.operator", lambda: getattr(operator, name)(a))
+            rec.attempt(f"{tag}.{stem}.dunder", lambda: getattr(a, f"__{stem}__")())
+        one = gr.load(x[2:3], shape=1)
+        rec.attempt(f"{tag}.not_single.dunder", lambda: one.__not__())
+        # operands on the left that are not tiles
+        rec.attempt(f"{tag}.pyscalar_left_mul", lambda: 2 * a)
+        rec.attempt(f"{tag}.pyscalar_left_sub", lambda: 2 - a)
+        rec.attempt(f"{tag}.npscalar_left_mul", lambda: x.dtype.type(2) * a)
+        rec.attempt(f"{tag}.ndarray_left_add", lambda: x + a)
+        rec.attempt(f"{tag}.ndarray_right_add", lambda: a + x)
+
+    with np.errstate(all="ignore"), warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        for tag, (x, y) in xs.items():
+            _one_group(api, lambda gr, x, y, _t=tag: body(gr, x, y, _t), x, y)
+    return rec.out
+
+
+def case_store_forms(api):
+    """Stores whose source is not a tile of the simulator: numpy.ma arrays that
+    reductions return, plain arrays, scalars broadcast by a window."""
+    rec = Recorder()
+    x = (np.arange(24, dtype=np.float32).reshape(4, 6) - 7)
+    dst = np.full((5, 4), POISON, np.float32)
+    wide = np.full((2, 4, 8), POISON, np.float32)
+
+    def body(gr, x, dst, wide):
+        t = gr.load(x[:3, :5], shape=(4, 8))
+        gr.store(dst[0], t.sum(axis=1))          # numpy.ma result, last row fully inactive
+        gr.store(dst[1], t.max(axis=1))
+        gr.store(dst[2], np.exp(t).sum(axis=1))  # plain ndarray: unconditional
+        s = t - t.max(axis=1, keepdims=True)
+        rec.tile("centred", s)
+        gr.store(wide[0], s)
+        e = np.exp(s)
+        rec.tile("exp_of_centred", e)
+        q = e / e.sum(axis=1, keepdims=True)
+        rec.tile("normalised", q)
+        gr.store(wide[1], q)
+        gr.store(dst[3], gr.load(x[0, :2], shape=4) * 2)
+        gr.store(dst[4, 1:], gr.load(x[1], shape=8))   # destination narrower than the tile
+
+    with np.errstate(all="ignore"), warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        _one_group(api, body, x, dst, wide)
+    rec.array("dst", dst)
+    rec.array("wide", wide)
+    return rec.out
+
+
+CASES = {
+    "inplace_partial": case_inplace_partial,
+    "load_from_masked": case_load_from_masked,
+    "domain_masking": case_domain_masking,
+    "numpy_functions": case_numpy_functions,
+    "compressed_repr": case_compressed_repr,
+    "scalar_promotion": case_scalar_promotion,
+    "operators": case_operators,
+    "store_forms": case_store_forms,
+}
+
+
+def run_all(api):
+    out = {}
+    for cname, fn in CASES.items():
+        for k, v in fn(api).items():
+            out[f"{cname}/{k}"] = v
+    return out
+
+
+def dump(entries, path):
+    """One entry per line: name -> [dtype, shape, bytes as hex] (exact for NaN,
+    inf and signed zeros, and readable in a diff)."""
+    import json
+    with open(path, "w") as f:
+        f.write("{\n")
+        rows = []
+        for k in sorted(entries):
+            a = np.asarray(entries[k])
+            rows.append(f"{json.dumps(k)}: {json.dumps([str(a.dtype), list(a.shape), a.tobytes().hex()])}")
+        f.write(",\n".join(rows))
+        f.write("\n}\n")
+
+
+def load(path):
+    import json
+    with open(path) as f:
+        raw = json.load(f)
+    return {k: np.frombuffer(bytes.fromhex(h), dtype=np.dtype(dt)).reshape(shape)
+            for k, (dt, shape, h) in raw.items()}

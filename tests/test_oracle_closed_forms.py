@@ -76,6 +76,52 @@ def test_bf16_rounding_two_statements_and_ties():
 # ---------------------------------------------------------------------------
 # W1 / W2
 # ---------------------------------------------------------------------------
+# --- W0 masked window copy ------------------------------------------------------
+def test_copy_window_known_answers():
+    # python/hckernel/tests/test_kernel_sim.py:91-104: twelve values stored into
+    # sixteen cells of -1 leave the last four cells alone
+    src, dst = np.arange(12), np.full(16, -1)
+    want = np.array(list(range(12)) + [-1] * 4)
+    assert np.array_equal(cf.np_copy_window(src, dst), want)
+    assert np.array_equal(dst, np.full(16, -1)), "np_copy_window must not write its argument"
+    d2 = dst.reshape(1, 16).copy()
+    co.copy2d(src.reshape(1, 12), d2)
+    assert np.array_equal(d2[0], want)
+    # a source wider than the destination is cut, not wrapped
+    assert np.array_equal(cf.np_copy_window(np.arange(20), np.full(16, -1)), np.arange(16))
+
+    # 2-D, ragged both ways, written out by hand: 3 x 5 source into a 4 x 3
+    # destination of -7 copies a 3 x 3 window
+    src = np.array([[0, 1, 2, 3, 4], [10, 11, 12, 13, 14], [20, 21, 22, 23, 24]], np.int32)
+    want = np.array([[0, 1, 2], [10, 11, 12], [20, 21, 22], [-7, -7, -7]], np.int32)
+    dst = np.full((4, 3), -7, np.int32)
+    assert np.array_equal(cf.np_copy_window(src, dst), want)
+    co.copy2d(src, dst)
+    assert np.array_equal(dst, want)
+
+
+@pytest.mark.parametrize("itemsize_dtype", [np.int8, np.float16, np.int32, np.float64])
+def test_copy2d_strided_views_leave_poison_alone(itemsize_dtype):
+    # windows of larger poison-filled arrays, strided in both dimensions: every
+    # byte outside the common window keeps its poison, inside it equals the source
+    rng = np.random.default_rng(11)
+    big_s = rng.integers(1, 100, (9, 14)).astype(itemsize_dtype)
+    big_d = np.full((11, 17), 101, itemsize_dtype)
+    src = big_s[1:8:2, 2:13:3]            # 4 x 4, strides (2 rows, 3 elements)
+    dst = big_d[2:11:3, 1:16:2]           # 3 x 8, strides (3 rows, 2 elements)
+    expect = big_d.copy()
+    for r in range(3):
+        for c in range(4):
+            expect[2 + 3 * r, 1 + 2 * c] = big_s[1 + 2 * r, 2 + 3 * c]
+    assert np.array_equal(cf.np_copy_window(src, dst), expect[2:11:3, 1:16:2])
+    co.copy2d(src, dst)
+    assert np.array_equal(big_d, expect)
+    # transposed source (column-major walk)
+    d2 = np.full((5, 5), 101, itemsize_dtype)
+    co.copy2d(big_s.T[:3, :2], d2)
+    assert np.array_equal(d2[:3, :2], big_s[:2, :3].T) and (d2[3:] == 101).all() and (d2[:, 2:] == 101).all()
+
+
 def test_add_two_statements_bit_equal():
     a, b = cf.inputs_c1(100_003)
     assert_array_equal(co.add_f32(a, b).view(np.uint32), cf.np_add(a, b).view(np.uint32))
