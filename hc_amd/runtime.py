@@ -114,8 +114,6 @@ hcamdLaunchMapReduceCols = _sig(_rt, "hcamdLaunchMapReduceCols", _int, _vp, _int
                                 C.POINTER(MapInstr), _sz, C.POINTER(MapInstr), _sz,
                                 C.POINTER(_vp), C.POINTER(_int), _sz_p, _sz, _vp, _int, _sz, _sz,
                                 _vp, _sz)
-
-
 class RowStage(C.Structure):
     """HcamdRowStage of include/hc_amd_runtime.h."""
     _fields_ = [("kind", C.c_uint32), ("nInstr", C.c_uint32), ("dst", C.c_uint32)]
@@ -353,6 +351,8 @@ class Plan:
 
 def _rows_cols(m: Memref):
     if len(m.shape) == 1:
+        if m.shape[0] > 1 and m.strides[0] != 1:
+            raise HcRuntimeError("a 1-D operand must be contiguous (stride 1)")
         return 1, m.shape[0], m.shape[0]
     if len(m.shape) == 2:
         if m.strides[1] != 1 and m.shape[1] > 1:

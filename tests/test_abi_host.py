@@ -160,6 +160,23 @@ def test_convert_cuda_array_interface_objects():
         rt.as_memref(Fake((15, 2)))
 
 
+def test_strided_1d_operands_are_not_taken_for_dense():
+    # a view like x[::2], or a column passed as a vector: the dense kernels would
+    # read and write the wrong elements
+    class Fake:
+        def __init__(self, n, stride_bytes):
+            self.shape = (n,)
+            self.__cuda_array_interface__ = {
+                "shape": (n,), "typestr": "<f4", "data": (0x7F0000001000, False),
+                "strides": (stride_bytes,), "version": 2}
+
+    assert rt._rows_cols(rt.as_memref(Fake(8, 4))) == (1, 8, 8)
+    assert rt._rows_cols(rt.Memref(0x1000, (1,), (7,), 4)) == (1, 1, 1)
+    for m in (rt.as_memref(Fake(8, 8)), rt.Memref(0x1000, (8,), (2,), 4)):
+        with pytest.raises(rt.HcRuntimeError, match="contiguous"):
+            rt._rows_cols(m)
+
+
 def test_convert_torch_cpu_tensor_via_dlpack():
     torch = pytest.importorskip("torch")
     t = torch.arange(12, dtype=torch.float32).reshape(3, 4)
