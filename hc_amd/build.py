@@ -83,16 +83,27 @@ def _rocm_root() -> Path:
     return Path(os.environ.get("ROCM_PATH") or Path(_hipcc()).resolve().parents[1])
 
 
+def build_scratch() -> Path:
+    # The one source with both host and device code: the static device scratch
+    # array of the entry point that allocates nothing has to be a registered
+    # device symbol, so hipcc compiles it into an ordinary object.
+    out = BUILD / "scratch.o"
+    _run([_hipcc(), "-c", "-fPIC", *DEVICE_FLAGS, "-I", str(INCLUDE), "-I", str(CSRC),
+          "-o", str(out), str(CSRC / "scratch.hip")])
+    return out
+
+
 def build_runtime() -> Path:
     # Host-only C++ on the HIP runtime API: the host compiler builds it and
     # links libamdhip64; blobs.S pulls the code objects in with .incbin.
     out = NATIVE / "libhc_amd_runtime.so"
     rocm = _rocm_root()
     cxx = shutil.which("g++") or "g++"
+    scratch = build_scratch()
     _run([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall",
           "-D__HIP_PLATFORM_AMD__", "-I", str(rocm / "include"),
-          "-I", str(INCLUDE), f"-Wa,-I{BUILD}",
-          str(CSRC / "runtime.cpp"), str(CSRC / "blobs.S"),
+          "-I", str(INCLUDE), "-I", str(CSRC), f"-Wa,-I{BUILD}",
+          str(CSRC / "runtime.cpp"), str(CSRC / "blobs.S"), str(scratch),
           "-o", str(out),
           f"-L{rocm / 'lib'}", f"-Wl,-rpath,{rocm / 'lib'}", "-lamdhip64"])
     return out

@@ -5,6 +5,7 @@
 // the reference interfaces they replace are documented in
 // include/hc_amd_runtime.h.
 #include "hc_amd_runtime.h"
+#include "internal.h"
 
 #include <hip/hip_runtime_api.h>
 
@@ -71,6 +72,7 @@ struct Device {
   void *ctx = nullptr;
   int index = 0;
   int computeUnits = 0; // filled in on first use
+  bool colsKernelsReady = false; // the column-reduction kernels were resolved at creation
   // built-in modules and kernels, loaded on first use
   std::unordered_map<std::string, hipModule_t> modules;
   std::unordered_map<std::string, struct Kernel *> kernels;
@@ -349,6 +351,19 @@ OlDevice olCreateDevice(const char *desc, OlErrorCallback errCallback,
   dev->index = std::atoi(id.c_str());
   if (dev->makeCurrent())
     return nullptr;
+  // Set-up for the entry point that allocates nothing: this GPU's address of the
+  // static scratch array, and the kernels it launches.  A failure here only
+  // makes that entry point refuse; every other one works without either.
+  char why[200] = {0};
+  if (hcamdInternalScratchSetup(dev->index, why, sizeof(why))) {
+    dev->report("%s", why);
+  } else {
+    dev->colsKernelsReady = true;
+    for (const char *name : {"hcamd_map_reduce_cols_n1u4", "hcamd_map_reduce_cols_n2u2",
+                             "hcamd_map_reduce_cols_n4u1"})
+      if (!builtinKernel(dev.get(), "map", name))
+        dev->colsKernelsReady = false;
+  }
   return dev.release();
 }
 
@@ -549,6 +564,25 @@ OlQueue hcamdGetDefaultQueue(const char *deviceDesc) noexcept {
 
 OlDevice hcamdGetDefaultDevice(const char *deviceDesc) noexcept {
   return hcamdGetDefaultQueue(deviceDesc) ? g_device : nullptr;
+}
+
+int hcamdInternalQueueDeviceIndex(OlQueue q) noexcept {
+  return q ? static_cast<Queue *>(q)->device->index : -1;
+}
+
+void hcamdInternalReport(OlQueue q, const char *fmt, ...) noexcept {
+  if (!q)
+    return;
+  char buf[256] = {0};
+  va_list ap;
+  va_start(ap, fmt);
+  std::vsnprintf(buf, sizeof(buf) - 1, fmt, ap);
+  va_end(ap);
+  static_cast<Queue *>(q)->device->report("%s", buf);
+}
+
+int hcamdInternalColsKernelsReady(OlQueue q) noexcept {
+  return q && static_cast<Queue *>(q)->device->colsKernelsReady ? 1 : 0;
 }
 
 OlDevice hcamdQueueDevice(OlQueue q) noexcept {

@@ -114,6 +114,15 @@ hcamdLaunchMapReduceCols = _sig(_rt, "hcamdLaunchMapReduceCols", _int, _vp, _int
                                 C.POINTER(MapInstr), _sz, C.POINTER(MapInstr), _sz,
                                 C.POINTER(_vp), C.POINTER(_int), _sz_p, _sz, _vp, _int, _sz, _sz,
                                 _vp, _sz)
+# The same launch without a workspace: the bands meet in the library's static
+# device scratch array (for callers that cannot allocate device memory).
+NOALLOC_SCRATCH_BYTES = 4 << 20
+hcamdLaunchMapReduceColsNoAlloc = _sig(_rt, "hcamdLaunchMapReduceColsNoAlloc", _int, _vp, _int,
+                                       C.POINTER(MapInstr), _sz, C.POINTER(MapInstr), _sz,
+                                       C.POINTER(_vp), C.POINTER(_int), _sz_p, _sz, _vp, _int,
+                                       _sz, _sz)
+
+
 class RowStage(C.Structure):
     """HcamdRowStage of include/hc_amd_runtime.h."""
     _fields_ = [("kind", C.c_uint32), ("nInstr", C.c_uint32), ("dst", C.c_uint32)]

@@ -338,6 +338,26 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
                              int outType, size_t rows, size_t cols, void *workspace,
                              size_t workspaceBytes) HCAMD_NOEXCEPT;
 
+/* hcamdLaunchMapReduceCols for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  Same arguments and results
+ * (bit for bit) without the workspace: the bands meet in a static device array
+ * of HCAMD_NOALLOC_SCRATCH_BYTES that each GPU the library runs on holds until
+ * the process ends; its address is looked up when the device is created
+ * (olCreateDevice), where the kernels are resolved too, so the call itself
+ * allocates and loads nothing.  A window whose
+ * hcamdMapReduceColsWorkspace(rows, cols) exceeds the limit is refused with a
+ * message (the workspace never exceeds about 3.1 MiB for any window the
+ * kernel accepts today; the limit is what protects a change of that).  All
+ * calls on one GPU share the array: calls that overlap on one GPU (two
+ * queues, two threads) race; calls on one queue are ordered and safe. */
+#define HCAMD_NOALLOC_SCRATCH_BYTES ((size_t)4 << 20)
+int hcamdLaunchMapReduceColsNoAlloc(OlQueue q, int kind, const HcamdMapInstr *prog,
+                                    size_t nInstr, const HcamdMapInstr *post, size_t nPost,
+                                    const void *const *inputs, const int *inputTypes,
+                                    const size_t *inputLd, size_t nInputs, void *out,
+                                    int outType, size_t rows, size_t cols) HCAMD_NOEXCEPT;
+
 /* Row programs: bodies that mix elementwise arithmetic with reductions along
  * the rows of a 2-D tile, e.g. the reference's row softmax
  * (python/hckernel/tests/test_examples.py:304-336:
