@@ -182,6 +182,83 @@ __device__ __forceinline__ void quantize_regs(const _Float16 *x, size_t ldx,
     }
   }
 }
+// Word layout: a row is walked in 16-byte words of 8 fp16 values; lane t of the
+// TPR lanes that share a row takes words t, t + TPR, ..., so every wave-level
+// load covers 1 KiB of consecutive bytes and every wave-level store (8 int8
+// values per lane) 512 consecutive bytes, exactly the access pattern of a plain
+// copy.  (quantize_regs gives a lane 16 consecutive values so that it can
+// store 16 bytes; its loads then touch every cache line twice, which costs
+// about 6 % at 16384 x 4096.)  T / TPR rows share a workgroup.  Needs
+// cols % 8 == 0, rows of x on 16-byte and rows of q on 8-byte boundaries, and
+// cols <= 8 * TPR * VPT; FULL: cols == 8 * TPR * VPT and rows % (T / TPR) == 0,
+// no predicates at all.
+template <int TPR, int T, int VPT, bool FULL, bool NT>
+__device__ __forceinline__ void quantize_words(const _Float16 *x, size_t ldx, int8_t *q,
+                                               size_t ldq, float *scale_out, size_t rows,
+                                               size_t cols) {
+  constexpr int kRowsPerGroup = T / TPR;
+  constexpr int kWaves = TPR / kWave;
+  __shared__ uint32_t smax[kRowsPerGroup * kWaves];
+  const int t = threadIdx.x % TPR;
+  const int rg = threadIdx.x / TPR;
+  const size_t row = (size_t)blockIdx.x * kRowsPerGroup + rg;
+  const bool row_ok = FULL || row < rows; // uniform per wave
+  const uint32_t words = (uint32_t)(cols / 8);
+  const u32x4 *xr = reinterpret_cast<const u32x4 *>(x + (row_ok ? row : 0) * ldx);
+  u32x4 v[VPT];
+  uint32_t m = 0;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const uint32_t w = (uint32_t)j * TPR + t;
+    if (FULL || (row_ok && w < words))
+      v[j] = ldg<NT>(xr + w);
+    else
+      v[j] = u32x4{0, 0, 0, 0};
+  }
+#pragma unroll
+  for (int j = 0; j < VPT; ++j)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      m = absmax_bits(m, v[j][i]);
+  m = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
+  m = group_reduce<UMaxOp, kWaves>(m, smax + rg * kWaves);
+
+  const float amax = half_bits_to_float(m);
+  const float scale = amax / 127.0f;
+  if (row_ok && t == 0)
+    scale_out[row] = scale;
+  if (!row_ok)
+    return;
+  const bool special = !(amax < INFINITY); // inf or NaN, uniform per row
+  const float div = (amax == 0.0f) ? 1.0f : scale;
+  const float rcp = 1.0f / div;
+  int8_t *qr = q + row * ldq;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const uint32_t w = (uint32_t)j * TPR + t;
+    if (!FULL && w >= words)
+      continue;
+    if (special) {
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t pair = v[j][i / 2];
+        const uint32_t bits = (i & 1) ? (pair >> 16) : (pair & 0xffffu);
+        qr[(size_t)w * 8 + i] = quant_special(half_bits_to_float(bits), scale);
+      }
+      continue;
+    }
+    u32x2 o;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const uint32_t w0 = v[j][2 * k], w1 = v[j][2 * k + 1];
+      o[k] = pack4(quotient<false>(half_bits_to_float(w0 & 0xffffu), div, rcp),
+                   quotient<false>(half_bits_to_float(w0 >> 16), div, rcp),
+                   quotient<false>(half_bits_to_float(w1 & 0xffffu), div, rcp),
+                   quotient<false>(half_bits_to_float(w1 >> 16), div, rcp));
+    }
+    stg<NT>(reinterpret_cast<u32x2 *>(qr) + w, o);
+  }
+}
+
 // Persistent form for rows of exactly 256 * 16 columns, 16-byte aligned: a
 // workgroup strides over the rows, and the loads of its next row are issued
 // before the absmax reduction of the current one, so requests stay in flight
@@ -379,6 +456,16 @@ HCAMD_QUANT(hcamd_quant_f16_i8_g128_v2_nt, 128, 2, false, true)
 HCAMD_QUANT(hcamd_quant_f16_i8_g256_v2, 256, 2, false, false)
 HCAMD_QUANT(hcamd_quant_f16_i8_g256_v4, 256, 4, false, false)
 HCAMD_QUANT(hcamd_quant_f16_i8_g256_v8, 256, 8, false, false)
+
+// two rows per workgroup of 512 lanes, 256 lanes and two words per lane per row
+#define HCAMD_QUANT_WORDS(NAME, FULL)                                          \
+  extern "C" __global__ __launch_bounds__(512) void NAME(                      \
+      const _Float16 *x, size_t ldx, int8_t *q, size_t ldq, float *scale,      \
+      size_t rows, size_t cols) {                                              \
+    quantize_words<256, 512, 2, FULL, true>(x, ldx, q, ldq, scale, rows, cols);\
+  }
+HCAMD_QUANT_WORDS(hcamd_quant_f16_i8_c256x2_w2_nt, false)
+HCAMD_QUANT_WORDS(hcamd_quant_f16_i8_c256x2_w2_full_nt, true)
 
 #define HCAMD_QUANT_SMALL(NAME, V, EPL)                                        \
   extern "C" __global__ __launch_bounds__(256) void NAME(                      \

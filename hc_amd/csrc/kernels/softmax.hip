@@ -175,6 +175,61 @@ HCAMD_SOFTMAX(hcamd_softmax_f32_g256_v2_full, 256, 2, true, false)
 HCAMD_SOFTMAX_ACC(hcamd_softmax_f32_g256_v8_full_nt_acc, 256, 8, true, true)
 HCAMD_SOFTMAX_ACC(hcamd_softmax_f32_g256_v8_acc, 256, 8, false, false)
 
+// Full rows of 8192 columns on 1024 lanes, two words per lane, one row per
+// workgroup.  Same arithmetic as softmax_regs; what differs is how much of the
+// matrix is in flight: two workgroups of this size fit a compute unit, so the
+// chip holds 512 rows (16 MiB) at a time instead of 2048, and HBM sees a
+// narrower window of addresses (measured 44.0 us against 44.9 for the
+// persistent kernel and 46.4 for 256 lanes per row at 4096 x 8192).
+template <int T, int VPT, bool NT>
+__device__ __forceinline__ void softmax_wide(const float *x, size_t ldx, float *y,
+                                             size_t ldy) {
+  constexpr int kWaves = T / kWave;
+  __shared__ float smax[kWaves];
+  __shared__ float ssum[kWaves];
+  const int t = threadIdx.x;
+  const size_t row = blockIdx.x;
+  const f32x4 *xr = reinterpret_cast<const f32x4 *>(x + row * ldx);
+  f32x4 *yr = reinterpret_cast<f32x4 *>(y + row * ldy);
+  f32x4 v[VPT];
+#pragma unroll
+  for (int j = 0; j < VPT; ++j)
+    v[j] = ldg<NT>(xr + j * T + t);
+  float m = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j)
+    m = fmaxf(fmaxf(fmaxf(m, v[j][0]), fmaxf(v[j][1], v[j][2])), v[j][3]);
+  m = group_reduce<MaxOp, kWaves>(m, smax);
+  const float m_log2e = m * 1.44269502162933349609375f;
+  float s = 0.0f;
+  if (__builtin_fabsf(m) < kFusedMaxAbs) { // uniform over the row
+#pragma unroll
+    for (int j = 0; j < VPT; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[j][i] = exp_scaled(v[j][i], m_log2e);
+        s += v[j][i];
+      }
+  } else {
+#pragma unroll
+    for (int j = 0; j < VPT; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[j][i] = exp_shifted(v[j][i], m);
+        s += v[j][i];
+      }
+  }
+  s = group_reduce<SumOp, kWaves>(s, ssum);
+  const float inv = 1.0f / s;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j)
+    stg<NT>(yr + j * T + t, v[j] * inv);
+}
+extern "C" __global__ __launch_bounds__(1024) void hcamd_softmax_f32_g1024_v2_full_nt(
+    const float *x, size_t ldx, float *y, size_t ldy, size_t rows, size_t cols) {
+  softmax_wide<1024, 2, true>(x, ldx, y, ldy);
+}
+
 // Persistent form of the full-row kernel: a workgroup walks rows blockIdx.x,
 // blockIdx.x + gridDim.x, ... and requests the next row before it reduces the
 // current one, so that loads stay in flight during the reductions, the

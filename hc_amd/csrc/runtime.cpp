@@ -2231,7 +2231,11 @@ int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,
                                           : "hcamd_softmax_f32_g256_v4";
   } else if (cols <= 8192) {
     const size_t cus = (size_t)computeUnitsOf(dev);
-    if (cols == 8192 && ((variant == 0 && rows >= 8 * cus) ||
+    if (cols == 8192 && variant == 0)
+      // full rows: 1024 lanes per row, two 16-byte words per lane
+      return launch1d(queue, "softmax", "hcamd_softmax_f32_g1024_v2_full_nt", rows, 1024,
+                      args);
+    if (cols == 8192 && ((variant == 10 && rows >= 8 * cus) ||
                          (variant >= 5 && variant <= 9))) {
       // Full rows and enough of them: the persistent kernel, a fixed number of
       // workgroups per compute unit, each prefetching its next row.
@@ -2282,6 +2286,16 @@ int hcamdLaunchQuantizeF16I8(OlQueue q, const void *x, size_t ldx, int8_t *qout,
   const int variant = variantOf("quantize");
   const bool vec_ok = aligned16(x) && aligned16(qout) &&
                       (rows == 1 || (ldx % 8 == 0 && ldq % 16 == 0));
+  if (variant == 0 && cols > 2048 && cols <= 4096 && cols % 8 == 0 && aligned16(x) &&
+      reinterpret_cast<uintptr_t>(qout) % 8 == 0 && (rows == 1 || (ldx % 8 == 0 && ldq % 8 == 0))) {
+    // 16-byte words dealt to the lanes one by one (the accesses of a plain copy:
+    // 16-byte loads, 8-byte stores), two rows per workgroup of 512 lanes
+    const bool full = cols == 4096 && rows % 2 == 0;
+    return launch1d(queue, "quantize",
+                    full ? "hcamd_quant_f16_i8_c256x2_w2_full_nt"
+                         : "hcamd_quant_f16_i8_c256x2_w2_nt",
+                    ceilDiv(rows, (size_t)2), 512, args);
+  }
   if (!vec_ok && variant != 1 && cols <= 32768) {
     // rows that cannot be walked in 16-byte pieces: register-resident with the
     // widest access the leading dimensions and base addresses allow

@@ -844,7 +844,7 @@ def test_softmax_variants_and_strided_rows(ctx):
     (x,) = cf.inputs_c3((rows, ld))
     want = cf.np_softmax(x[:, :cols])
     dx = dev(x)
-    for v in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9):
+    for v in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10):
         rt.set_variant("softmax", v)
         dy = poisoned((rows, ld), np.float32)
         rt.softmax_f32(_View(dx, (rows, cols), 0, (ld, 1)), _View(dy, (rows, cols), 0, (ld, 1)))
@@ -929,7 +929,7 @@ def test_softmax_full_benchmark_size(ctx):
     assert x.shape == (4096, 8192)
     dy = rt.DeviceArray(x.shape, np.float32)
     rt.softmax_f32(dev(x), dy)
-    assert rt.last_kernel_name() == "hcamd_softmax_f32_p256_v8_nt"
+    assert rt.last_kernel_name() == "hcamd_softmax_f32_g1024_v2_full_nt"
     y = dy.to_host()
     assert_allclose(y, cf.np_softmax(x), rtol=SOFTMAX_RTOL, atol=SOFTMAX_ATOL)
     assert_allclose(y.astype(np.float64).sum(1), 1.0, atol=2e-6)
@@ -969,8 +969,36 @@ def test_quantize_bit_exact(ctx, shape):
         assert_array_equal(q, q_c)
 
 
+@pytest.mark.parametrize("shape,ld,kernel", [
+    ((64, 4096), None, "c256x2_w2_full_nt"), ((63, 4096), None, "c256x2_w2_nt"),
+    ((7, 2056), None, "c256x2_w2_nt"), ((5, 3000), 3008, "c256x2_w2_nt"),
+    ((1, 4096), None, "c256x2_w2_nt"), ((2, 4096), 4160, "c256x2_w2_full_nt"),
+    ((9, 4088), 4096, "c256x2_w2_nt")])
+def test_quantize_word_layout_kernel(ctx, shape, ld, kernel):
+    """Rows of 2049..4096 columns (a multiple of 8) take the kernel that deals
+    16-byte words to the lanes: whole and ragged widths, odd row counts, padded
+    leading dimensions, zero / inf / NaN rows through its per-element path."""
+    rows, cols = shape
+    (x,) = cf.inputs_c4(shape)
+    x[0, ::5] = 0
+    if rows > 3:
+        x[1] = 0
+        x[2, cols - 1] = np.float16(np.inf)
+        x[3, 17] = np.float16(np.nan)
+    with np.errstate(all="ignore"):
+        q_np, s_np = cf.np_quantize(x)
+    q, s = run_quantize(x, ld)
+    say("quantize words", shape, ld, rt.last_kernel_name())
+    assert rt.last_kernel_name().endswith(kernel)
+    assert_array_equal(q, q_np)
+    assert_array_equal(s.view(np.uint32), s_np.view(np.uint32))
+    if rows > 3:
+        q_c, s_c = co.quantize(x)
+        assert_array_equal(q, q_c)
+
+
 @pytest.mark.parametrize("shape,ld,off,kernel", [
-    ((37, 4100), None, 0, "s4_e8"), ((19, 1000), None, 0, "s4_e4"), ((7, 4088), None, 0, "s4_e4"),
+    ((37, 4100), None, 0, "s4_e8"), ((19, 1000), None, 0, "s4_e4"), ((7, 4088), None, 0, "c256x2_w2_nt"),
     ((5, 20004), None, 0, "s4_e32"), ((9, 4094), None, 0, "s2_e8"), ((6, 10002), None, 0, "s2_e32"), ((6, 6002), None, 0, "s2_e16"), ((6, 6001), None, 0, "s1_e32"),
     ((3, 30002), None, 0, "s2_e64"), ((11, 4095), None, 0, "s1_e16"), ((5, 15001), None, 0, "s1_e64"),
     ((4, 1), None, 0, "s1_e16"), ((4, 2), None, 0, "s2_e8"), ((4, 3), None, 0, "s1_e16"),
@@ -1033,7 +1061,7 @@ def test_quantize_every_fp16_value_against_many_scales(ctx):
     bits |= (rng.integers(0, 2, (rows, cols)).astype(np.uint16) << 15)
     x = bits.view(np.float16)
     q_np, s_np = cf.np_quantize(x)
-    for v in (0, 2):
+    for v in (0, 2, 3):
         rt.set_variant("quantize", v)
         q, s = run_quantize(x)
         assert_array_equal(q, q_np)
