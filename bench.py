@@ -59,6 +59,21 @@ MEASURED_TRAFFIC = {
 }
 
 
+# Stream calibrations: (key, read streams, what is written, MiB per read stream).
+# The first four have the read:write mix and size of c1..c4 and are timed next
+# to them in the default run.
+STREAMS = [
+    ("s1", 2, "full", 64),     # c1: two reads, one write of 64 MiB
+    ("s2", 3, "full", 128),    # c2: three reads, one write of 128 MiB
+    ("s3", 1, "full", 128),    # c3: 128 MiB each way
+    ("s4", 1, "half", 128),    # c4: 128 MiB in, 64 MiB out
+    ("s5", 1, "none", 256), ("s6", 0, "full", 256), ("s7", 1, "full", 256),
+    ("s8", 2, "full", 128), ("s9", 2, "full", 256), ("s10", 3, "full", 256),
+    ("s11", 1, "half", 256), ("s12", 1, "none", 128), ("s13", 0, "full", 128),
+]
+STREAM_OF = {"c1": "s1", "c2": "s2", "c3": "s3", "c4": "s4"}
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -228,6 +243,50 @@ def make_workloads(rt, wl):
             dst = np.empty_like(self.src)
             return _best_of(lambda: np.copyto(dst, self.src)), "full size, numpy.copyto", 1
 
+
+    class Stream(Workload):
+        """Stream calibration: n_reads vectors of `mib` MiB added word by word and
+        written whole ("full"), folded to half the bytes ("half") or only summed
+        ("none"): what HBM delivers for that mix of reads and writes."""
+
+        def __init__(self, key, n_reads, write, mib):
+            self.n_reads, self.write, self.nbytes = n_reads, write, mib << 20
+            out = {"full": self.nbytes, "half": self.nbytes // 2, "none": self.nbytes // 4096}[write]
+            self.out_bytes = out
+            mix = f"r{n_reads}w{0 if write == 'none' else 1}{'h' if write == 'half' else ''}"
+            moved = n_reads * self.nbytes + (0 if write == "none" else out)
+            super().__init__(key, f"stream {mix}: {n_reads} read stream(s) of {mib} MiB, "
+                             f"{out >> 20} MiB written (calibration)", "u32", "hbm", moved, "GB/s")
+            self.mix = mix
+
+        def setup(self, rt):
+            rng = np.random.default_rng(9)
+            self.ins = [rng.integers(0, 2 ** 32, self.nbytes // 4, dtype=np.uint32)
+                        for _ in range(self.n_reads)]
+            return [tuple(rt.to_device(x) for x in self.ins) +
+                    (rt.DeviceArray((self.out_bytes // 4,), np.uint32),) for _ in range(ROTATE)]
+
+        def plan(self, rt, s):
+            return rt.plan_stream(s[:-1], s[-1], self.write)
+
+        def _numpy(self):
+            if not self.ins:
+                return np.repeat(np.arange(self.nbytes // 16, dtype=np.uint32), 4)
+            total = self.ins[0].copy()
+            for x in self.ins[1:]:
+                total += x
+            if self.write == "full":
+                return total
+            if self.write == "half":
+                return total[0::2] ^ total[1::2]
+            return total.reshape(-1, 4096).sum(axis=1, dtype=np.uint32)
+
+        def check(self, rt, s):
+            ok = np.array_equal(s[-1].to_host(), self._numpy())
+            return {"parity": "bit-exact" if ok else "MISMATCH", "ok": bool(ok)}
+
+        def cpu(self):
+            return _best_of(self._numpy, 1), "full size, NumPy uint32 arithmetic", 1
 
     # ---- beyond the five configurations: the generic paths, on request only ------
     I = lambda name, arg=0, imm=0.0: (name, arg, imm)      # noqa: E731
@@ -411,8 +470,13 @@ def make_workloads(rt, wl):
         "x6": X6("x6", "column reduction: root mean square down the columns, fp32 4096x8192", "f32",
                  "hbm", W.work_c3() // 2 + 4 * 8192, "GB/s"),
     }
+    # the mix and size of each memory-bound configuration, then the plain streams
+    for key, n_reads, write, mib in STREAMS:
+        table[key] = Stream(key, n_reads, write, mib)
     if wl == "all":
         keys = ["c1", "c2", "c3", "c4", "c5"]
+    elif wl == "streams":
+        keys = [k for k, *_ in STREAMS]
     elif wl == "extra":
         keys = ["x1", "x2", "x3", "x4", "x5", "x6"]
     else:
@@ -481,7 +545,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="all", choices=["all", "c0", "c1", "c2", "c3", "c4", "c5", "extra", "x1", "x2", "x3", "x4", "x5", "x6"])
+    ap.add_argument("--workload", default="all", choices=["all", "streams", "c0", "c1", "c2", "c3", "c4", "c5", "extra", "x1", "x2", "x3",
+                             "x4", "x5", "x6"] + [k for k, *_ in STREAMS])
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy CPU baseline")
     ap.add_argument("--prewarm", type=float, default=PREWARM_SECONDS,
                     help="seconds of untimed device warm-up per workload")
@@ -501,6 +566,18 @@ def main():
     for w in make_workloads(rt, args.workload):
         results[w.key] = run_one(rt, ctx, w, args.steps, args.warmup, not args.no_cpu,
                                  args.prewarm)
+        if args.workload == "all" and w.key in STREAM_OF:
+            # the plain stream of the same read:write mix and size, timed the same
+            # way: the ceiling this kernel is held to
+            (sw,) = make_workloads(rt, STREAM_OF[w.key])
+            sr = run_one(rt, ctx, sw, args.steps, args.warmup, False, args.prewarm)
+            kern = results[w.key]["roofline"]
+            results[w.key]["stream_ceiling"] = {
+                "workload": sr["workload"], "kernel": sr["kernel"],
+                "kernel_avg_us": sr["roofline"]["kernel_avg_us"],
+                "achieved": sr["roofline"]["achieved"], "unit": "GB/s",
+                "frac_of_peak": sr["roofline"]["frac"], "parity_ok": sr["parity"]["ok"],
+                "workload_vs_stream": round(kern["achieved"] / sr["roofline"]["achieved"], 4)}
 
     head_key = "c2" if "c2" in results else next(iter(results))
     head = results[head_key]

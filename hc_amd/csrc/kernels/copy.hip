@@ -111,6 +111,72 @@ HCAMD_COPY_TILED(hcamd_copy2d_tiled_b4, uint32_t)
 HCAMD_COPY_TILED(hcamd_copy2d_tiled_b8, uint64_t)
 HCAMD_COPY_TILED(hcamd_copy2d_tiled_b16, u32x4)
 
+// ---------------------------------------------------------------------------
+// Stream calibration: what HBM delivers for a given mix of read and write
+// streams when nothing else is in the way.  R input vectors of 16-byte words
+// are added lane by lane (32-bit wrap-around) and
+//   W = 1: the sum word is written (16 bytes out per 16 bytes of each input),
+//   W = 2: its halves are xor-ed and 8 bytes written (the 2:1 byte ratio of the
+//          int8 quantiser),
+//   W = 0: nothing is written but one 32-bit sum per workgroup (a read-only
+//          stream with a checkable result).
+// With R = 0 the kernel writes the word index (a fill).  A workgroup of 512
+// lanes owns 1024 consecutive words, two per lane, non-temporal both ways: the
+// structure that measured fastest for every mix.  The launcher passes whole
+// workgroups only (bytes a multiple of 16 KiB).
+template <int R, int W>
+__device__ __forceinline__ void stream_mix(const u32x4 *a, const u32x4 *b, const u32x4 *c,
+                                           void *out) {
+  constexpr int kT = 512, kVpt = 2;
+  const u32x4 *in[3] = {a, b, c};
+  const size_t first = (size_t)blockIdx.x * (kT * kVpt) + threadIdx.x;
+  u32x4 v[kVpt][R > 0 ? R : 1];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int j = 0; j < kVpt; ++j)
+      v[j][r] = ldg<true>(in[r] + first + (size_t)j * kT);
+  uint32_t total = 0;
+#pragma unroll
+  for (int j = 0; j < kVpt; ++j) {
+    const uint32_t w = (uint32_t)(first + (size_t)j * kT);
+    u32x4 s = R ? v[j][0] : u32x4{w, w, w, w};
+#pragma unroll
+    for (int r = 1; r < R; ++r)
+      s += v[j][r];
+    if constexpr (W == 1) {
+      stg<true>(static_cast<u32x4 *>(out) + first + (size_t)j * kT, s);
+    } else if constexpr (W == 2) {
+      const u32x2 h = {s[0] ^ s[1], s[2] ^ s[3]};
+      stg<true>(static_cast<u32x2 *>(out) + first + (size_t)j * kT, h);
+    } else {
+      total += s[0] + s[1] + s[2] + s[3];
+    }
+  }
+  if constexpr (W == 0) {
+    __shared__ uint32_t slots[kT / kWave];
+    struct USum {
+      using T = uint32_t;
+      static __device__ __forceinline__ uint32_t identity() { return 0u; }
+      static __device__ __forceinline__ uint32_t apply(uint32_t x, uint32_t y) { return x + y; }
+    };
+    total = group_reduce<USum, kT / kWave>(total, slots);
+    if (threadIdx.x == 0)
+      static_cast<uint32_t *>(out)[blockIdx.x] = total;
+  }
+}
+#define HCAMD_STREAM(NAME, R, W)                                               \
+  extern "C" __global__ __launch_bounds__(512) void NAME(                      \
+      const u32x4 *a, const u32x4 *b, const u32x4 *c, void *out) {             \
+    stream_mix<R, W>(a, b, c, out);                                            \
+  }
+HCAMD_STREAM(hcamd_stream_r1w0, 1, 0)
+HCAMD_STREAM(hcamd_stream_r0w1, 0, 1)
+HCAMD_STREAM(hcamd_stream_r1w1, 1, 1)
+HCAMD_STREAM(hcamd_stream_r2w1, 2, 1)
+HCAMD_STREAM(hcamd_stream_r3w1, 3, 1)
+HCAMD_STREAM(hcamd_stream_r1w1h, 1, 2)
+
 extern "C" __global__ __launch_bounds__(256) void hcamd_fill32(uint32_t *dst,
                                                                uint32_t value,
                                                                size_t count) {

@@ -812,6 +812,49 @@ int hcamdLaunchCopy2D(OlQueue q, size_t elemSize, const void *src,
   return 0;
 }
 
+int hcamdLaunchStream(OlQueue q, int nReads, int writeMode, const void *const *inputs,
+                      void *out, size_t bytes) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  const char *name = nullptr;
+  if (writeMode == HCAMD_STREAM_NONE && nReads == 1)
+    name = "hcamd_stream_r1w0";
+  else if (writeMode == HCAMD_STREAM_HALF && nReads == 1)
+    name = "hcamd_stream_r1w1h";
+  else if (writeMode == HCAMD_STREAM_FULL && nReads >= 0 && nReads <= 3) {
+    static const char *const full[] = {"hcamd_stream_r0w1", "hcamd_stream_r1w1",
+                                       "hcamd_stream_r2w1", "hcamd_stream_r3w1"};
+    name = full[nReads];
+  }
+  if (!name) {
+    dev->report("hcamdLaunchStream: no kernel for %d read stream(s) and write mode %d", nReads,
+                writeMode);
+    return 1;
+  }
+  if (bytes == 0)
+    return 0;
+  if (bytes % 16384 != 0 || bytes / 16384 > 0x7fffffffull) {
+    dev->report("hcamdLaunchStream: %zu bytes (a multiple of 16 KiB, below 2^45)", bytes);
+    return 1;
+  }
+  const void *in[3] = {nullptr, nullptr, nullptr};
+  for (int i = 0; i < nReads; ++i) {
+    if (!inputs || !inputs[i] || !aligned16(inputs[i])) {
+      dev->report("hcamdLaunchStream: null or unaligned input %d", i);
+      return 1;
+    }
+    in[i] = inputs[i];
+  }
+  if (!out || !aligned16(out)) {
+    dev->report("hcamdLaunchStream: null or unaligned output");
+    return 1;
+  }
+  void *args[] = {&in[0], &in[1], &in[2], &out};
+  return launch1d(queue, "copy", name, bytes / 16384, 512, args);
+}
+
 int hcamdLaunchCopy2DTiled(OlQueue q, size_t elemSize, const void *src,
                            void *dst, size_t rows, size_t cols, ptrdiff_t ss0,
                            ptrdiff_t ds0, size_t blockX, size_t blockY,

@@ -84,6 +84,7 @@ hcamdLaunchCopy2D = _sig(_rt, "hcamdLaunchCopy2D", _int, _vp, _sz, _vp, _sz, _sz
                          _ssz, _ssz, _vp, _sz, _sz, _ssz, _ssz)
 hcamdLaunchCopy2DTiled = _sig(_rt, "hcamdLaunchCopy2DTiled", _int, _vp, _sz, _vp, _vp,
                               _sz, _sz, _ssz, _ssz, _sz, _sz, _sz)
+hcamdLaunchStream = _sig(_rt, "hcamdLaunchStream", _int, _vp, _int, _int, C.POINTER(_vp), _vp, _sz)
 hcamdLaunchAddF32 = _sig(_rt, "hcamdLaunchAddF32", _int, _vp, _vp, _vp, _vp, _sz)
 hcamdLaunchFmaF16 = _sig(_rt, "hcamdLaunchFmaF16", _int, _vp, _vp, _sz, _vp, _sz, _vp,
                          _sz, _vp, _sz, _sz, _sz)
@@ -398,6 +399,33 @@ def plan_copy2d_tiled(src, dst, block_x: int, block_y: int, unroll: int = 1) -> 
     return Plan(ctx, hcamdLaunchCopy2DTiled,
                 (ctx.queue, s.itemsize, s.ptr, d.ptr, rows, cols, s.strides[0], d.strides[0],
                  block_x, block_y, unroll), "hcamdLaunchCopy2DTiled", (src, dst))
+
+
+STREAM_WRITE = {"none": 0, "full": 1, "half": 2}
+
+
+def plan_stream(inputs, out, write="full") -> Plan:
+    """Stream calibration (see hcamdLaunchStream): the inputs (0..3 contiguous
+    arrays of equal byte size, a multiple of 16 KiB) are added in 32-bit lanes;
+    `write` is "full" (the sum), "half" (xor of each sum word's halves, half the
+    bytes) or "none" (one 32-bit total per 16 KiB)."""
+    inputs = list(inputs)
+    ctx = _ctx_of(*inputs, out)
+    ms = [as_memref(x) for x in inputs]
+    mo = as_memref(out)
+    if any(not m.is_contiguous() for m in ms + [mo]):
+        raise HcRuntimeError("stream: contiguous arrays only")
+    sizes = {m.size * m.itemsize for m in ms}
+    if len(sizes) > 1:
+        raise HcRuntimeError("stream: inputs of different sizes")
+    out_bytes = mo.size * mo.itemsize
+    nbytes = sizes.pop() if sizes else out_bytes
+    need = {"full": nbytes, "half": nbytes // 2, "none": nbytes // 4096}[write]
+    if out_bytes < need:
+        raise HcRuntimeError(f"stream: the output holds {out_bytes} bytes, {need} needed")
+    ptrs = (_vp * 3)(*[m.ptr for m in ms])
+    return Plan(ctx, hcamdLaunchStream, (ctx.queue, len(ms), STREAM_WRITE[write], ptrs, mo.ptr,
+                                         nbytes), "hcamdLaunchStream", (inputs, out, ptrs))
 
 
 def plan_add_f32(a, b, c) -> Plan:

@@ -214,6 +214,20 @@ int hcamdLaunchCopy2D(OlQueue q, size_t elemSize, const void *src,
                       size_t dstCols, ptrdiff_t dstStride0,
                       ptrdiff_t dstStride1) HCAMD_NOEXCEPT;
 
+/* Stream calibration (no counterpart in the reference): what HBM delivers for
+ * a mix of read and write streams with nothing else in the way, the yardstick
+ * the memory-bound kernels are held to.  nReads (0..3) vectors of `bytes` bytes
+ * are added in 32-bit lanes, word by word; writeMode selects what leaves:
+ * HCAMD_STREAM_FULL the sum (bytes out), HCAMD_STREAM_HALF the xor of each sum
+ * word's halves (bytes / 2 out: the 2:1 ratio of the int8 quantiser),
+ * HCAMD_STREAM_NONE one 32-bit total per 16 KiB of input (bytes / 4096 out: a
+ * read-only stream with a checkable result).  nReads == 0 writes the word
+ * index (a fill; HCAMD_STREAM_FULL only).  bytes must be a multiple of 16 KiB,
+ * pointers 16-byte aligned. */
+enum HcamdStreamWrite { HCAMD_STREAM_NONE = 0, HCAMD_STREAM_FULL = 1, HCAMD_STREAM_HALF = 2 };
+int hcamdLaunchStream(OlQueue q, int nReads, int writeMode, const void *const *inputs,
+                      void *out, size_t bytes) HCAMD_NOEXCEPT;
+
 /* The same copy launched with the reference's own geometry and kernel argument
  * list (tests/Transforms/gpu-to-gpu-runtime.mlir:34-37): grid =
  * (ceil(cols/(bx*unroll)), ceil(rows/by), 1), block = (bx, by, 1), one element

@@ -223,6 +223,43 @@ def test_copy_large_flat_all_variants(ctx):
 
 
 # ---------------------------------------------------------------------------
+# stream calibration kernels (the yardstick of the memory-bound kernels)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("n_reads,write", [(1, "full"), (2, "full"), (3, "full"), (0, "full"),
+                                            (1, "half"), (1, "none")])
+def test_stream_mixes_compute_what_they_say(ctx, n_reads, write):
+    nbytes = 5 * 16384
+    rng = np.random.default_rng(60 + n_reads)
+    ins = [rng.integers(0, 2 ** 32, nbytes // 4, dtype=np.uint32) for _ in range(n_reads)]
+    words = {"full": nbytes // 4, "half": nbytes // 8, "none": nbytes // 16384}[write]
+    pad = 8
+    out = poisoned((words + pad,), np.uint32)
+    rt.plan_stream([dev(x) for x in ins], _View(out, (words,), 0), write).launch(sync=True)
+    say("stream", n_reads, write, rt.last_kernel_name())
+    total = np.zeros(nbytes // 4, np.uint32)
+    for x in ins:
+        total += x
+    if n_reads == 0:
+        total = np.repeat(np.arange(nbytes // 16, dtype=np.uint32), 4)
+    want = {"full": total, "half": total[0::2] ^ total[1::2],
+            "none": total.reshape(-1, 4096).sum(axis=1, dtype=np.uint32)}[write]
+    got = out.to_host()
+    assert_array_equal(got[:words], want)
+    assert (got[words:] == POISON32).all()
+
+
+def test_stream_refusals(ctx):
+    x = dev(np.zeros(16384 // 4, np.uint32))
+    y = rt.DeviceArray((16384 // 4,), np.uint32)
+    with pytest.raises(rt.HcRuntimeError, match="multiple of 16 KiB"):
+        rt.plan_stream([_View(x, (1000,), 0)], _View(y, (1000,), 0)).launch(sync=True)
+    with pytest.raises(rt.HcRuntimeError, match="no kernel"):
+        rt.plan_stream([x, x], y, "half").launch(sync=True)
+    with pytest.raises(rt.HcRuntimeError, match="needed"):
+        rt.plan_stream([x], _View(y, (100,), 0), "full")
+
+
+# ---------------------------------------------------------------------------
 # W1 c = a + b
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("n", [1, 3, 4, 255, 1024, 4099, 262_144, 1_000_003])
