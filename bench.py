@@ -41,22 +41,66 @@ FP32_VECTOR_PEAK_TFLOPS = 157.3
 ROTATE = 4
 PREWARM_SECONDS = 0.4        # untimed, per workload, before the W warm-up steps
 
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
-# scaled by a copy kernel of known size; filled in from profiles/*.txt.
-# FETCH_SIZE reads half the true value on this device (a 256 MiB copy reads
-# 131,082 KiB), WRITE_SIZE reads true (262,215 KiB), so fetches are scaled by
-# 2.0 and writes by 1.0.  Source: profiles/hbm_traffic_pmc.txt.
-_KIB = 1024
-MEASURED_TRAFFIC = {
-    "c0": int((131085.1 * 2.0 + 262156.5) * _KIB),
-    "c1": int((65556.6 * 2.0 + 65536.2) * _KIB),     # algorithmic 201,327,108
-    "c2": int((196637.6 * 2.0 + 131072.0) * _KIB),   # algorithmic 536,870,904
-    "c3": int((65566.9 * 2.0 + 131125.1) * _KIB),    # algorithmic 268,435,456
-    "c4": int((65869.6 * 2.0 + 66048.0) * _KIB),     # algorithmic 201,392,128
-    "c5": int((98362.2 * 2.0 + 32768.0) * _KIB),     # 2.3 x the algorithmic 100,663,296 (L2 refetch)
-    # both launches of the step: the bands (67,221.4 / 2,048.0) and their fold (1,177.5 / 32.0)
-    "x6": int(((67221.4 + 1177.5) * 2.0 + 2048.0 + 32.0) * _KIB),   # algorithmic 134,250,496
-}
+# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE in
+# KiB per dispatch), scaled by what the same counters read for the plain copy
+# of known size (workload c0).  The figures live in profiles/hbm_traffic.json,
+# which `bench.py --traffic-from DIR` writes from the counter files of the
+# commands listed in profiles/hbm_traffic_pmc.txt; a figure is reported only
+# while the kernel that ran is the kernel that was measured.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+TRAFFIC_WORKLOADS = ("c0", "c1", "c2", "c3", "c4", "c5", "x6")
+C0_KIB = 256 * 1024          # c0 reads and writes 256 MiB
+
+
+def measured_traffic(key, kernel):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)["workloads"].get(key)
+    except (OSError, ValueError, KeyError):
+        return None
+    if not rec or rec["kernel"] != kernel:
+        return None
+    return rec["bytes"]
+
+
+def traffic_from(dirname, launches):
+    """Reads DIR/<workload>_<counter>_counter_collection.csv (rocprofv3 --pmc, one
+    counter and one workload per run, `launches` launches each) and writes
+    profiles/hbm_traffic.json."""
+    import collections
+    import csv
+
+    def per_launch(w, counter):
+        total = collections.defaultdict(float)
+        with open(os.path.join(dirname, f"{w}_{counter}_counter_collection.csv")) as f:
+            for r in csv.DictReader(f):
+                k = r["Kernel_Name"]
+                if k.startswith("hcamd_") and "fill" not in k:
+                    total[k] += float(r["Counter_Value"])
+        (kernel, value), = total.items()       # one kernel per workload
+        return kernel, value / launches
+
+    _, f0 = per_launch("c0", "FETCH_SIZE")
+    _, w0 = per_launch("c0", "WRITE_SIZE")
+    scale = {"FETCH_SIZE": C0_KIB / f0, "WRITE_SIZE": C0_KIB / w0}
+    out = {"unit": "KiB per launch as the counters report them; bytes = scaled sum",
+           "calibration": {"workload": "c0", "true_KiB_each_way": C0_KIB,
+                           "FETCH_SIZE_KiB": round(f0, 1), "WRITE_SIZE_KiB": round(w0, 1),
+                           "scale": {k: round(v, 4) for k, v in scale.items()}},
+           "launches_per_run": launches, "workloads": {}}
+    for w in TRAFFIC_WORKLOADS:
+        try:
+            kernel, fetch = per_launch(w, "FETCH_SIZE")
+            _, write = per_launch(w, "WRITE_SIZE")
+        except OSError:
+            continue
+        out["workloads"][w] = {
+            "kernel": kernel, "FETCH_SIZE_KiB": round(fetch, 1), "WRITE_SIZE_KiB": round(write, 1),
+            "bytes": int((fetch * scale["FETCH_SIZE"] + write * scale["WRITE_SIZE"]) * 1024)}
+    with open(TRAFFIC_FILE, "w") as f:
+        json.dump(out, f, indent=1, sort_keys=True)
+        f.write("\n")
+    print(json.dumps(out, indent=1, sort_keys=True))
 
 
 # Stream calibrations: (key, read streams, what is written, MiB per read stream).
@@ -243,6 +287,60 @@ def make_workloads(rt, wl):
             dst = np.empty_like(self.src)
             return _best_of(lambda: np.copyto(dst, self.src)), "full size, numpy.copyto", 1
 
+
+    class V5(C5):
+        """The vendor library's GEMM on the same operands (hipBLASLt, reached through
+        torch.matmul with B given as the transposed view of Bt): the yardstick for
+        c5 that is not this library.  PyTorch launches on its own stream, so this
+        workload brings its own events."""
+
+        def setup(self, rt):
+            import torch
+            self.torch = torch
+            self.a, self.bt = W.inputs_c5()
+            dev = torch.device("cuda:0")
+
+            def bf16(bits):
+                return torch.from_numpy(bits.view(np.int16)).to(dev).view(torch.bfloat16)
+            return [(bf16(self.a), bf16(self.bt),
+                     torch.empty((self.a.shape[0], self.bt.shape[0]), dtype=torch.bfloat16,
+                                 device=dev)) for _ in range(ROTATE)]
+
+        def plan(self, rt, s):
+            torch = self.torch
+
+            class TorchPlan:
+                def launch(self_inner):
+                    torch.matmul(s[0], s[1].T, out=s[2])
+            return TorchPlan()
+
+        def make_events(self):
+            torch = self.torch
+
+            class Ev:
+                def __init__(self):
+                    self.e = torch.cuda.Event(enable_timing=True)
+
+                def record(self):
+                    self.e.record()
+
+                def elapsed_ms(self, other):
+                    return self.e.elapsed_time(other.e)
+            return Ev(), Ev()
+
+        def synchronize(self):
+            self.torch.cuda.synchronize()
+
+        def kernel_name(self):
+            return "hipBLASLt via torch.matmul (torch %s)" % self.torch.__version__
+
+        def check(self, rt, s):
+            from oracle import closed_forms as cf
+            got = W.bf16_bits_to_f32(s[2].view(self.torch.int16).cpu().numpy().view(np.uint16))
+            want = cf.np_gemm_bf16(self.a, self.bt, np.float32)
+            ok = np.allclose(got, want, rtol=1e-2, atol=2.6e-4)
+            return {"parity": "rtol 1e-2 vs fp32 accumulation" if ok else "MISMATCH",
+                    "ok": bool(ok), "max_abs_err": float(np.max(np.abs(got - want)))}
 
     class Stream(Workload):
         """Stream calibration: n_reads vectors of `mib` MiB added word by word and
@@ -458,6 +556,8 @@ def make_workloads(rt, wl):
         "c4": C4("c4", "row absmax int8 quantize fp16 16384x4096", "f16->i8", "hbm",
                  W.work_c4(), "GB/s"),
         "c5": C5("c5", "GEMM bf16 4096^3 (fp32 acc)", "bf16", "mfma", W.work_c5(), "TFLOP/s"),
+        "v5": V5("v5", "vendor library GEMM bf16 4096^3 on the c5 operands (yardstick)", "bf16",
+                 "mfma", W.work_c5(), "TFLOP/s"),
         "x1": X1("x1", "map kernel: fma fp16 8191x8193 as a 3-instruction program", "f16", "hbm",
                  W.work_c2(), "GB/s"),
         "x2": X2("x2", "map-sum kernel: dot fp32 N=16777259", "f32", "hbm", 8 * W.C1_N, "GB/s"),
@@ -484,30 +584,33 @@ def make_workloads(rt, wl):
     return [table[k] for k in keys]
 
 
-def run_one(rt, ctx, w, steps, warmup, want_cpu, prewarm):
+def run_one(rt, ctx, w, steps, warmup, want_cpu, prewarm, check=True):
     log(f"[bench] {w.key}: {w.title}: building inputs")
     sets = w.setup(rt)
     plans = [w.plan(rt, s) for s in sets]
     launches = [p.launch for p in plans]
-    ctx.synchronize()
+    # a workload that does not launch on this library's queue brings its own
+    # synchronisation and events (the vendor-library yardstick)
+    sync = getattr(w, "synchronize", ctx.synchronize)
+    sync()
     # Untimed device warm-up: the GPU raises its clocks only under sustained
     # load, so a short burst would time the ramp instead of the kernel.
     t_end = time.perf_counter() + prewarm
     while time.perf_counter() < t_end:
         for i in range(50):
             launches[i % ROTATE]()
-        ctx.synchronize()
+        sync()
     for i in range(warmup):
         launches[i % ROTATE]()
-    ctx.synchronize()
-    kernel = rt.last_kernel_name()
-    start, stop = rt.Event(ctx), rt.Event(ctx)
+    sync()
+    kernel = w.kernel_name() if hasattr(w, "kernel_name") else rt.last_kernel_name()
+    start, stop = w.make_events() if hasattr(w, "make_events") else (rt.Event(ctx), rt.Event(ctx))
     t0 = time.perf_counter()
     start.record()
     for i in range(steps):
         launches[i % ROTATE]()
     stop.record()
-    ctx.synchronize()
+    sync()
     wall = time.perf_counter() - t0
     ev_ms = start.elapsed_ms(stop)
     ms_step = wall * 1e3 / steps
@@ -521,13 +624,16 @@ def run_one(rt, ctx, w, steps, warmup, want_cpu, prewarm):
         "value": round(value, 2), "unit": w.unit, "ms_per_step": round(ms_step, 5),
         "roofline": {"bound": w.bound, "achieved": round(achieved, 2), "peak": peak,
                      "unit": w.unit, "frac": round(achieved / peak, 4),
-                     "traffic": MEASURED_TRAFFIC.get(w.key),
+                     "traffic": measured_traffic(w.key, kernel),
                      "kernel_avg_us": round(kern_ms * 1e3, 3),
                      "algorithmic_work": w.work},
     }
+    if res["roofline"]["traffic"] and w.bound == "hbm":
+        res["roofline"]["traffic_vs_algorithmic"] = round(res["roofline"]["traffic"] / w.work, 4)
     log(f"[bench] {w.key}: {kernel}: {kern_ms * 1e3:.2f} us/launch, "
         f"{achieved:.1f} {w.unit} = {100 * achieved / peak:.1f}% of peak; checking parity")
-    res["parity"] = w.check(rt, sets[(steps - 1) % ROTATE])
+    res["parity"] = (w.check(rt, sets[(steps - 1) % ROTATE]) if check
+                     else {"parity": "not checked", "ok": True, "checked": False})
     if want_cpu:
         sec, sample, cores = w.cpu()
         res["cpu_baseline"] = {"value": round(w.work * scale / sec, 3), "unit": w.unit,
@@ -536,7 +642,8 @@ def run_one(rt, ctx, w, steps, warmup, want_cpu, prewarm):
         log(f"[bench] {w.key}: cpu {res['cpu_baseline']['value']} {w.unit} on {cores} core(s)")
     for s in sets:
         for a in s:
-            a.free()
+            if hasattr(a, "free"):
+                a.free()
     return res
 
 
@@ -545,12 +652,26 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="all", choices=["all", "streams", "c0", "c1", "c2", "c3", "c4", "c5", "extra", "x1", "x2", "x3",
+    ap.add_argument("--workload", default="all", choices=["all", "streams", "c0", "c1", "c2", "c3", "c4", "c5", "v5", "extra", "x1", "x2", "x3",
                              "x4", "x5", "x6"] + [k for k, *_ in STREAMS])
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy CPU baseline")
+    ap.add_argument("--variant", action="append", default=[], metavar="FAMILY=N",
+                    help="measure kernel variant N of a family (hcamdSetVariant), e.g. gemm=14; "
+                         "for profiling alternatives, never part of the default run")
+    ap.add_argument("--no-check", action="store_true",
+                    help="skip the parity check (only for measurement probes whose output "
+                         "is not the product, such as gemm=17)")
     ap.add_argument("--prewarm", type=float, default=PREWARM_SECONDS,
                     help="seconds of untimed device warm-up per workload")
+    ap.add_argument("--traffic-from", metavar="DIR",
+                    help="no benchmark: read rocprofv3 --pmc counter files from DIR and write "
+                         "profiles/hbm_traffic.json (see profiles/hbm_traffic_pmc.txt)")
+    ap.add_argument("--traffic-launches", type=int, default=6,
+                    help="launches per counter run (warm-up + steps) for --traffic-from")
     args = ap.parse_args()
+    if args.traffic_from:
+        traffic_from(args.traffic_from, args.traffic_launches)
+        return
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no "
                  "sharding); run with --gpus 1")
@@ -562,10 +683,13 @@ def main():
     info = ctx.info()
     log(f"[bench] device {info}")
 
+    for spec in args.variant:
+        family, _, number = spec.partition("=")
+        rt.set_variant(family, int(number))
     results = {}
     for w in make_workloads(rt, args.workload):
         results[w.key] = run_one(rt, ctx, w, args.steps, args.warmup, not args.no_cpu,
-                                 args.prewarm)
+                                 args.prewarm, not args.no_check)
         if args.workload == "all" and w.key in STREAM_OF:
             # the plain stream of the same read:write mix and size, timed the same
             # way: the ceiling this kernel is held to

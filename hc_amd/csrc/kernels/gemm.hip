@@ -248,7 +248,18 @@ __device__ __forceinline__ Acc mfma_block(V b, V a, Acc c) {
 // the start of their row instead and overwritten with zeros in LDS by the lane
 // that fetched them, before the barrier that releases the tile; stores are
 // masked.  Everything else, and the speed on whole tiles, is the same.
-template <class E, int BM, int BN, int WM, int WN, int MF, bool EDGE = false>
+// EPI selects the epilogue of whole-tile builds: 0 stores each lane's four
+// consecutive columns as they lie in the accumulators (8-byte stores, 32 bytes
+// per row and instruction); 1 and 2 pass the tile through LDS, which the main
+// loop no longer needs, so that eight lanes write one whole 128-byte row
+// segment with 16-byte stores (2: non-temporal).  PRIO raises the wave's issue
+// priority for the duration of each MFMA burst.  PROBE is a measurement build,
+// not a product path: it fetches the first K tile only and then issues the
+// main loop's MFMAs on those fragments with no loads, LDS reads, waits or
+// barriers, which times the matrix cores alone on real operand data (its
+// output is not the product).
+template <class E, int BM, int BN, int WM, int WN, int MF, bool EDGE = false, int EPI = 0,
+          bool PRIO = false, int PROBE = 0>
 __device__ __forceinline__ void gemm_tile_pipelined(
     const E *__restrict__ A, size_t lda, const E *__restrict__ Bt, size_t ldb,
     E *__restrict__ C, size_t ldc, int M, int N, int K) {
@@ -434,36 +445,97 @@ __device__ __forceinline__ void gemm_tile_pipelined(
     // wait is free and makes the later waits exact), fetch slot 1
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoVm, 0));
     __builtin_amdgcn_sched_barrier(0);
-    read_frags(buf, 1, Slot1{});
+    if constexpr (PROBE != 4)
+      read_frags(buf, 1, Slot1{});
+    if constexpr (PRIO)
+      __builtin_amdgcn_s_setprio(1);
     mma(Slot0{});
     interleave(NoVmem{});
+    if constexpr (PRIO)
+      __builtin_amdgcn_s_setprio(0);
     // odd half-step; the fences keep the MFMAs above on this side of the wait
     __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+    if constexpr (PROBE == 2)
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoVm, 0));
+    else
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
     if constexpr (ZERO) {
       zero_tail(buf ^ 1);
       __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoVm, 0));
     }
-    __builtin_amdgcn_s_barrier();
+    if constexpr (PROBE != 3)
+      __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (LOAD)
+    if constexpr (LOAD && PROBE != 5)
       issue_loads(t + 2, buf);
-    if constexpr (READ)
+    if constexpr (READ && PROBE != 4)
       read_frags(buf ^ 1, 0, Slot0{});
+    if constexpr (PRIO)
+      __builtin_amdgcn_s_setprio(1);
     mma(Slot1{});
     if constexpr (LOAD && READ)
       interleave(WithVmem{});
     else if constexpr (READ)
       interleave(NoVmem{});
+    if constexpr (PRIO)
+      __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
   };
-  int t = 0;
-  for (; t < KT - 2; ++t)
-    tile_step(t, std::true_type{}, std::true_type{});
-  tile_step(t, std::false_type{}, std::true_type{});
-  tile_step(t + 1, std::false_type{}, std::false_type{});
+  if constexpr (PROBE == 1) {
+    read_frags(0, 1, Slot1{});
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+    for (int t = 0; t < KT; ++t) {
+      mma(Slot0{});
+      mma(Slot1{});
+    }
+  } else {
+    if constexpr (PROBE == 4)
+      read_frags(0, 1, Slot1{});
+    int t = 0;
+    for (; t < KT - 2; ++t)
+      tile_step(t, std::true_type{}, std::true_type{});
+    tile_step(t, std::false_type{}, std::true_type{});
+    tile_step(t + 1, std::false_type{}, std::false_type{});
+  }
 
   // ---- epilogue ------------------------------------------------------------------
+  if constexpr (EPI != 0 && !EDGE && MF == 16) {
+    // Through LDS: the wave's kWaveM x kWaveN tile as rows of kWaveN elements,
+    // 16-byte chunk c of row r kept at chunk c ^ (r & 7) (the writes of sixteen
+    // rows at one column then spread over the banks); read back eight lanes to
+    // a row.  Every wave uses a region of its own, but the stage buffers it
+    // lies in may still be read by slower waves: one barrier first.
+    static_assert(kWaveN * sizeof(E) == 128, "a wave row is eight 16-byte chunks");
+    static_assert(kWaves * kWaveM * 128 <= 2 * kStageBytes, "the tile fits the stage buffers");
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoVm, 0));
+    __builtin_amdgcn_s_barrier();
+    unsigned char *mine = lds + wave * (kWaveM * 128);
+#pragma unroll
+    for (int i = 0; i < kMI; ++i)
+#pragma unroll
+      for (int j = 0; j < kNI; ++j) {
+        ex4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          o[e] = (E)acc[i][j][e];
+        const int r = i * 16 + lrow;
+        const int chunk = 2 * j + lchunk / 2;
+        *reinterpret_cast<ex4 *>(mine + r * 128 + ((chunk ^ (r & 7)) * 16) + (lchunk % 2) * 8) = o;
+      }
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoVm, 0));
+    const int rr = lane / 8, pc = lane % 8;
+#pragma unroll
+    for (int r0 = 0; r0 < kWaveM; r0 += 8) {
+      const int r = r0 + rr;
+      const u32x4 v = *reinterpret_cast<const u32x4 *>(mine + r * 128 + pc * 16);
+      E *dst = C + (size_t)(tm * BM + wave_m + r) * ldc + tn * BN + wave_n + ((pc ^ (r & 7)) * 8);
+      if constexpr (EPI == 2)
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst));
+      else
+        *reinterpret_cast<u32x4 *>(dst) = v;
+    }
+    return;
+  }
   const int m_base = tm * BM + wave_m + lrow;
   const int n_base = tn * BN + wave_n + lchunk * 4;
   const bool vec_c = !EDGE || (ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(C) & 7) == 0);
@@ -509,18 +581,35 @@ __device__ __forceinline__ void gemm_tile_pipelined(
     gemm_tile_pipelined<E, BM, BN, WM, WN, MF, true>(A, lda, Bt, ldb, C, ldc,  \
                                                      M, N, K);                 \
   }
+#define HCAMD_GEMM_PX(NAME, E, BM, BN, WM, WN, MF, EPI, PRIO, PROBE)             \
+  extern "C" __global__ __launch_bounds__(WM *WN * 64) void NAME(              \
+      const E *A, size_t lda, const E *Bt, size_t ldb, E *C, size_t ldc,       \
+      int M, int N, int K) {                                                   \
+    gemm_tile_pipelined<E, BM, BN, WM, WN, MF, false, EPI, PRIO, PROBE>(       \
+        A, lda, Bt, ldb, C, ldc, M, N, K);                                     \
+  }
+// the default whole-tile kernels: LDS-staged epilogue with non-temporal stores
+HCAMD_GEMM_PX(hcamd_gemm_bf16_p256x256_w2x4, __bf16, 256, 256, 2, 4, 16, 2, false, 0)
+HCAMD_GEMM_PX(hcamd_gemm_bf16_p128x128_w2x2, __bf16, 128, 128, 2, 2, 16, 2, false, 0)
+HCAMD_GEMM_PX(hcamd_gemm_f16_p256x256_w2x4, _Float16, 256, 256, 2, 4, 16, 2, false, 0)
+HCAMD_GEMM_PX(hcamd_gemm_f16_p128x128_w2x2, _Float16, 128, 128, 2, 2, 16, 2, false, 0)
+// the same main loop with the other epilogues / wave priorities, for measurement
+HCAMD_GEMM_PX(hcamd_gemm_bf16_p256x256_w2x4_direct, __bf16, 256, 256, 2, 4, 16, 0, false, 0)
+HCAMD_GEMM_PX(hcamd_gemm_bf16_p256x256_w2x4_lds, __bf16, 256, 256, 2, 4, 16, 1, false, 0)
+HCAMD_GEMM_PX(hcamd_gemm_bf16_p256x256_w2x4_prio, __bf16, 256, 256, 2, 4, 16, 2, true, 0)
+HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_mfma_only, __bf16, 256, 256, 2, 4, 16, 2, false, 1)
+HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_no_vmwait, __bf16, 256, 256, 2, 4, 16, 2, false, 2)
+HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_no_barrier, __bf16, 256, 256, 2, 4, 16, 2, false, 3)
+HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_no_ldsread, __bf16, 256, 256, 2, 4, 16, 2, false, 4)
+HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_no_loads, __bf16, 256, 256, 2, 4, 16, 2, false, 5)
 HCAMD_GEMM_PE(hcamd_gemm_bf16_p256x256_w2x4_edge, __bf16, 256, 256, 2, 4, 16)
 HCAMD_GEMM_PE(hcamd_gemm_f16_p256x256_w2x4_edge, _Float16, 256, 256, 2, 4, 16)
 HCAMD_GEMM_PE(hcamd_gemm_bf16_p128x128_w2x2_edge, __bf16, 128, 128, 2, 2, 16)
 HCAMD_GEMM_PE(hcamd_gemm_f16_p128x128_w2x2_edge, _Float16, 128, 128, 2, 2, 16)
-HCAMD_GEMM_P(hcamd_gemm_bf16_p256x256_w2x4, __bf16, 256, 256, 2, 4, 16)
 HCAMD_GEMM_P(hcamd_gemm_bf16_p256x256_w4x2, __bf16, 256, 256, 4, 2, 16)
-HCAMD_GEMM_P(hcamd_gemm_bf16_p128x128_w2x2, __bf16, 128, 128, 2, 2, 16)
 HCAMD_GEMM_P(hcamd_gemm_bf16_p256x128_w2x2, __bf16, 256, 128, 2, 2, 16)
 HCAMD_GEMM_P(hcamd_gemm_bf16_p32_256x256_w2x4, __bf16, 256, 256, 2, 4, 32)
 HCAMD_GEMM_P(hcamd_gemm_bf16_p32_256x256_w4x2, __bf16, 256, 256, 4, 2, 32)
-HCAMD_GEMM_P(hcamd_gemm_f16_p256x256_w2x4, _Float16, 256, 256, 2, 4, 16)
-HCAMD_GEMM_P(hcamd_gemm_f16_p128x128_w2x2, _Float16, 128, 128, 2, 2, 16)
 
 #define HCAMD_GEMM(NAME, BM, BN, WM, WN, SH)                                   \
   extern "C" __global__ __launch_bounds__(WM * WN * 64) void NAME(             \

@@ -2452,6 +2452,15 @@ int launchGemm(OlQueue q, bool half, const void *a, size_t lda, const void *bt,
       {"hcamd_gemm_bf16_p256x128_w2x2", 256, 128, 256},
       {"hcamd_gemm_bf16_p32_256x256_w2x4", 256, 256, 512}, // 11
       {"hcamd_gemm_bf16_p32_256x256_w4x2", 256, 256, 512},
+      {nullptr, 0, 0, 0}, // 13: the edge-capable kernel (chosen below)
+      {"hcamd_gemm_bf16_p256x256_w2x4_direct", 256, 256, 512}, // 14: 8-byte stores from the accumulators
+      {"hcamd_gemm_bf16_p256x256_w2x4_lds", 256, 256, 512},    // 15: through LDS, plain stores
+      {"hcamd_gemm_bf16_p256x256_w2x4_prio", 256, 256, 512},   // 16: raised priority in the MFMA bursts
+      {"hcamd_gemm_bf16_probe_mfma_only", 256, 256, 512},      // 17: measurement only, output is not the product
+      {"hcamd_gemm_bf16_probe_no_vmwait", 256, 256, 512},      // 18..21: likewise
+      {"hcamd_gemm_bf16_probe_no_barrier", 256, 256, 512},
+      {"hcamd_gemm_bf16_probe_no_ldsread", 256, 256, 512},
+      {"hcamd_gemm_bf16_probe_no_loads", 256, 256, 512},
   };
   constexpr int kGeneral = 6;
   constexpr int kFirstPipelined = 7; // variants from here need K >= 128

@@ -1256,11 +1256,17 @@ def test_gemm_all_variants_and_padded_output(ctx):
     ab, bb = cf.inputs_c5((512, 512, 256))
     want = cf.np_gemm_bf16(ab, bb, np.float32)
     sigma = 0.02 * 0.02 * 16
-    for v in range(0, 14):
+    bits0 = None
+    for v in range(0, 17):             # 17 is a measurement probe whose output is not the product
         rt.set_variant("gemm", v)
-        got = cf.bf16_bits_to_f32(run_gemm(ab, bb, ldc_pad=8))
+        bits = run_gemm(ab, bb, ldc_pad=8)
+        got = cf.bf16_bits_to_f32(bits)
         say("gemm variant", v, rt.last_kernel_name())
         assert_allclose(got, want, rtol=GEMM_RTOL, atol=1e-2 * sigma)
+        if v == 0:
+            bits0 = bits
+        if v in (7, 14, 15, 16):       # the same main loop with other epilogues / priorities
+            assert_array_equal(bits, bits0)
 
 
 def test_gemm_full_benchmark_size_and_linearity(ctx):
