@@ -32,7 +32,8 @@ import math
 from dataclasses import dataclass
 
 from . import runtime as rt
-from .kernel_api import Affine, BufferView, Tile, TraceError
+from .kernel_api import (Affine, BufferView, ItemIndex, Tile, TraceError, same_index,
+                         same_starts)
 
 
 class NoNativeKernel(RuntimeError):
@@ -115,7 +116,7 @@ def _same(a: Tile, b: Tile) -> bool:
         return False
     if a.op == "load":
         va, vb = a.attrs["view"], b.attrs["view"]
-        return va.base.index == vb.base.index and va.starts == vb.starts
+        return va.base.index == vb.base.index and same_starts(va.starts, vb.starts)
     if {k: v for k, v in a.attrs.items()} != {k: v for k, v in b.attrs.items()}:
         return False
     return len(a.args) == len(b.args) and all(_same(x, y) for x, y in zip(a.args, b.args))
@@ -407,7 +408,7 @@ class _Operand:
 
 
 def _same_index(a, b):
-    return a is b or (isinstance(a, Affine) and isinstance(b, Affine) and a == b)
+    return same_index(a, b)
 
 
 def _region(t: Tile, axis_k: int):
@@ -716,7 +717,7 @@ class _MapCompiler:
     def operand(self, t: Tile) -> int:
         v = t.attrs["view"]
         for i, (b, st, _) in enumerate(self.inputs):
-            if b == v.base.index and st == v.starts:
+            if b == v.base.index and same_starts(st, v.starts):
                 return i
         self.inputs.append((v.base.index, v.starts, t))
         return len(self.inputs) - 1
@@ -934,7 +935,7 @@ class _RowCompiler(_MapCompiler):
             if t.dtype_name not in _MAP_FLOATS:
                 raise NoNativeKernel(f"{v.base.name}: per-row operands must be float32 or float16")
             for i, (b, st, _) in enumerate(self.columns):
-                if b == v.base.index and st == v.starts:
+                if b == v.base.index and same_starts(st, v.starts):
                     self.slots[t.uid] = i
                     return
             if len(self.columns) >= rt.MAP_MAX_INPUTS:
@@ -1625,13 +1626,147 @@ def match_sum(proxy, index, value, n_groups):
     return makers
 
 
-def bind(stores, n_groups, atomics=(), mapped_stores=()):
+# ---------------------------------------------------------------------------
+# Per-subgroup partial results folded back into whole-row reductions
+# ---------------------------------------------------------------------------
+_FOLDS = ("max", "min", "sum")
+
+
+def _slice_ranges(node: Tile):
+    """(T, per-dim index or (start, stop)) if node == T[key] with unit steps."""
+    if not _is(node, "slice", 1):
+        return None
+    src = node.args[0]
+    out = []
+    dims = iter(src.shape)
+    for k in node.attrs["key"]:
+        if k == "new":
+            return None
+        n = next(dims)
+        if isinstance(k, tuple):
+            start, stop, step = slice(*k).indices(n)
+            if step != 1:
+                return None
+            out.append((start, max(stop, start)))
+        else:
+            out.append(int(k) % n)
+    return src, tuple(out)
+
+
+def _assembled_reduce(t: Tile):
+    """t = fold(U) where the workgroup tile U was filled, element by element,
+    with the same fold of disjoint pieces of one tile T that together cover T's
+    rows (what subgroup-scope bodies leave behind: `partial[i, k] =
+    x[i, a_k:b_k].max()` per subgroup, then `partial.max(axis=1)` after the
+    barrier).  Returns the fold over T's rows, or None."""
+    if t.op not in _FOLDS or len(t.args) != 1 or not _is(t.args[0], "update"):
+        return None
+    u = t.args[0]
+    two_d = len(u.shape) == 2
+    if len(u.shape) not in (1, 2):
+        return None
+    axes = t.attrs.get("axes")
+    rows = u.shape[0] if two_d else 1
+    if two_d and not (axes == (1,) or (axes == (0, 1) and rows == 1)):
+        return None
+    if not two_d and axes != (0,):
+        return None
+    pieces = {}
+    node = u
+    while _is(node, "update"):
+        key, value = node.attrs["key"], node.args[1]
+        if any(isinstance(k, tuple) for k in key):
+            return None                          # a slice was assigned, not an element
+        pieces.setdefault(key, value)            # the newest assignment wins
+        node = node.args[0]
+    if len(pieces) != math.prod(u.shape):
+        return None                              # some element still holds the initial value
+    source = None
+    spans = {}
+    for key, value in pieces.items():
+        if not (_is(value, t.op, 1) and value.shape == ()):
+            return None
+        got = _slice_ranges(value.args[0])
+        if got is None:
+            return None
+        src, ranges = got
+        if source is None:
+            source = src
+        elif src is not source and not _same(src, source):
+            return None
+        if len(src.shape) != len(u.shape):
+            return None
+        if two_d:
+            if not (isinstance(ranges[0], int) and ranges[0] == key[0] and isinstance(ranges[1], tuple)):
+                return None
+            spans.setdefault(key[0], []).append(ranges[1])
+        else:
+            if not isinstance(ranges[0], tuple):
+                return None
+            spans.setdefault(0, []).append(ranges[0])
+    if source is None or (two_d and source.shape[0] != rows):
+        return None
+    n = source.shape[-1]
+    for row in range(rows):
+        at = 0
+        for a, b in sorted(spans.get(row, [])):
+            if a != at:
+                return None
+            at = b
+        if at != n:
+            return None
+    keep = bool(t.attrs.get("keepdims"))
+    if two_d and axes == (1,):
+        return source._reduce(t.op, 1, keep)
+    return source._reduce(t.op, None, keep)
+
+
+def simplify(t: Tile, memo=None) -> Tile:
+    """The traced expression with per-subgroup partial folds replaced by the
+    whole-row folds they add up to; everything else unchanged."""
+    memo = {} if memo is None else memo
+    if id(t) in memo:
+        return memo[id(t)]
+    args = tuple(simplify(a, memo) for a in t.args)
+    out = t
+    if any(a is not b for a, b in zip(args, t.args)):
+        out = Tile(t.op, args, t.shape, t.dtype_name, **t.attrs)
+    folded = _assembled_reduce(out)
+    if folded is not None:
+        out = folded
+    memo[id(t)] = out
+    return out
+
+
+def match_id_store(proxy, index, value, per_item, n_groups, group_shape):
+    if proxy.dtype_name not in ("int32", "int64", "float32"):
+        raise NoNativeKernel(f"ids can be stored to int32, int64 and float32 buffers, "
+                             f"{proxy.name} is {proxy.dtype_name}")
+    if math.prod(group_shape) > 1024:
+        raise NoNativeKernel("a scope whose ids are stored needs groups of at most 1024 work-items")
+    out_type = {"int32": rt.I32, "int64": rt.I64, "float32": rt.F32}[proxy.dtype_name]
+    idx = [(i.const, i.g, i.l) for i in index]
+    val = (value.const, value.g, value.l)
+
+    def make(mem, ctx):
+        return [rt.plan_id_scatter(_Arr(mem[proxy.index], ctx), idx, val, n_groups, group_shape,
+                                   per_item, out_type)]
+    return make
+
+
+def bind(stores, n_groups, atomics=(), mapped_stores=(), id_stores=(), group_shape=()):
     """stores: list of (BufferView, Tile) from one traced execution; atomics:
     list of (BufferProxy, index, Tile) atomic additions; mapped_stores: list of
-    (BufferView, Tile, index function).  Returns a list of plan makers; raises
-    NoNativeKernel when nothing matches."""
-    if not stores and not atomics and not mapped_stores:
+    (BufferView, Tile, index function); id_stores: (BufferProxy, index, value,
+    per work-item?) element stores of ids.  Returns a list of plan makers;
+    raises NoNativeKernel when nothing matches."""
+    if not stores and not atomics and not mapped_stores and not id_stores:
         raise NoNativeKernel("the kernel body stores nothing")
+    memo = {}
+    stores = [(view, simplify(value, memo)) for view, value in stores]
+    id_makers = [match_id_store(p, i, v, per, n_groups, group_shape) for p, i, v, per in id_stores]
+    if id_stores and not (stores or atomics or mapped_stores):
+        return id_makers
     try:
         if atomics:
             if stores or mapped_stores:
@@ -1639,8 +1774,8 @@ def bind(stores, n_groups, atomics=(), mapped_stores=()):
                                      "atomically has no native kernel")
             return [mk for proxy, index, value in atomics
                     for mk in match_sum(proxy, index, value, n_groups)]
-        makers = [match_gather_gemm(view, value, n_groups, func, plain=False)
-                  for view, value, func in mapped_stores]
+        makers = id_makers + [match_gather_gemm(view, value, n_groups, func, plain=False)
+                              for view, value, func in mapped_stores]
         q = match_quantize(stores, n_groups)
         if q is not None:
             return makers + [q]

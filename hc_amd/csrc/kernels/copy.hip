@@ -177,6 +177,55 @@ HCAMD_STREAM(hcamd_stream_r2w1, 2, 1)
 HCAMD_STREAM(hcamd_stream_r3w1, 3, 1)
 HCAMD_STREAM(hcamd_stream_r1w1h, 1, 2)
 
+// ---------------------------------------------------------------------------
+// Ids as data: out[index(g, l)] = value(g, l), both affine in the group id g and
+// the local id l, for every work-item (per_item) or once per group.  Launched
+// with the reference's own geometry (block = group shape, grid = group counts,
+// last Python dimension on x: mlir/lib/Transforms/LowerHKernel.cpp:284-367), so
+// the hardware ids ARE the ids of the programming model
+// (python/hckernel/kernel.py:97-131: work_offset = group_id * group_shape,
+// global id = work_offset + local_id).  An index outside the buffer stores
+// nothing.
+struct IdScatterArgs {
+  void *out;
+  int32_t out_type; // 0 int32, 1 int64, 2 float32
+  int32_t out_rank;
+  int32_t rank;     // of the work shape
+  int32_t per_item;
+  int64_t out_shape[3], out_stride[3];
+  int64_t idx_c[3], idx_g[3][3], idx_l[3][3];
+  int64_t val_c, val_g[3], val_l[3];
+};
+extern "C" __global__ __launch_bounds__(1024) void hcamd_id_scatter(IdScatterArgs a) {
+  const int64_t hw_g[3] = {blockIdx.x, blockIdx.y, blockIdx.z};
+  const int64_t hw_l[3] = {threadIdx.x, threadIdx.y, threadIdx.z};
+  int64_t g[3] = {0, 0, 0}, l[3] = {0, 0, 0};
+  for (int d = 0; d < a.rank; ++d) {
+    g[d] = hw_g[a.rank - 1 - d];
+    l[d] = hw_l[a.rank - 1 - d];
+  }
+  if (!a.per_item && (l[0] | l[1] | l[2]) != 0)
+    return;
+  int64_t at = 0;
+  for (int d = 0; d < a.out_rank; ++d) {
+    int64_t i = a.idx_c[d];
+    for (int k = 0; k < 3; ++k)
+      i += a.idx_g[d][k] * g[k] + a.idx_l[d][k] * l[k];
+    if (i < 0 || i >= a.out_shape[d])
+      return;
+    at += i * a.out_stride[d];
+  }
+  int64_t v = a.val_c;
+  for (int k = 0; k < 3; ++k)
+    v += a.val_g[k] * g[k] + a.val_l[k] * l[k];
+  if (a.out_type == 0)
+    static_cast<int32_t *>(a.out)[at] = (int32_t)v;
+  else if (a.out_type == 1)
+    static_cast<int64_t *>(a.out)[at] = v;
+  else
+    static_cast<float *>(a.out)[at] = (float)v;
+}
+
 extern "C" __global__ __launch_bounds__(256) void hcamd_fill32(uint32_t *dst,
                                                                uint32_t value,
                                                                size_t count) {

@@ -812,6 +812,81 @@ int hcamdLaunchCopy2D(OlQueue q, size_t elemSize, const void *src,
   return 0;
 }
 
+namespace {
+struct IdScatterArgs {
+  void *out;
+  int32_t out_type, out_rank, rank, per_item;
+  int64_t out_shape[3], out_stride[3];
+  int64_t idx_c[3], idx_g[3][3], idx_l[3][3];
+  int64_t val_c, val_g[3], val_l[3];
+};
+} // namespace
+
+int hcamdLaunchIdScatter(OlQueue q, void *out, int outType, size_t outRank,
+                         const size_t *outShape, const ptrdiff_t *outStrides,
+                         const HcamdAffineId *index, const HcamdAffineId *value, size_t rank,
+                         const size_t *groupCount, const size_t *groupShape,
+                         int perItem) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  const char *who = "hcamdLaunchIdScatter";
+  if (!out || !outShape || !outStrides || !index || !value || !groupCount || !groupShape) {
+    dev->report("%s: null pointer", who);
+    return 1;
+  }
+  if (rank < 1 || rank > 3 || outRank < 1 || outRank > 3) {
+    dev->report("%s: ranks %zu / %zu (1..3)", who, rank, outRank);
+    return 1;
+  }
+  IdScatterArgs a{};
+  a.out = out;
+  a.out_type = outType == HCAMD_I32 ? 0 : outType == HCAMD_I64 ? 1 : outType == HCAMD_F32 ? 2 : -1;
+  if (a.out_type < 0) {
+    dev->report("%s: unsupported output type %d", who, outType);
+    return 1;
+  }
+  a.out_rank = (int32_t)outRank;
+  a.rank = (int32_t)rank;
+  a.per_item = perItem ? 1 : 0;
+  size_t grid[3] = {1, 1, 1}, block[3] = {1, 1, 1}, threads = 1, groups = 1;
+  for (size_t d = 0; d < rank; ++d) {
+    // Python dimension d is hardware dimension rank - 1 - d
+    grid[rank - 1 - d] = groupCount[d];
+    block[rank - 1 - d] = groupShape[d];
+    threads *= groupShape[d];
+    groups *= groupCount[d];
+  }
+  if (groups == 0 || threads == 0)
+    return 0;
+  if (threads > 1024) {
+    dev->report("%s: a group of %zu work-items (at most 1024 fit one workgroup)", who, threads);
+    return 1;
+  }
+  for (size_t d = 0; d < outRank; ++d) {
+    if (outShape[d] == 0)
+      return 0;
+    a.out_shape[d] = (int64_t)outShape[d];
+    a.out_stride[d] = (int64_t)outStrides[d];
+    a.idx_c[d] = index[d].c;
+    for (int k = 0; k < 3; ++k) {
+      a.idx_g[d][k] = index[d].g[k];
+      a.idx_l[d][k] = index[d].l[k];
+    }
+  }
+  a.val_c = value->c;
+  for (int k = 0; k < 3; ++k) {
+    a.val_g[k] = value->g[k];
+    a.val_l[k] = value->l[k];
+  }
+  Kernel *k = builtinKernel(dev, "copy", "hcamd_id_scatter");
+  if (!k)
+    return 1;
+  void *args[] = {&a};
+  return launch(queue, k, grid, block, args, 0);
+}
+
 int hcamdLaunchStream(OlQueue q, int nReads, int writeMode, const void *const *inputs,
                       void *out, size_t bytes) noexcept {
   auto *queue = static_cast<Queue *>(q);

@@ -245,7 +245,8 @@ class GpuKernel:
             body(group_obj, *proxies)
         except TraceError as exc:
             raise NoNativeKernel(f"{self.func.__name__}: {exc}") from exc
-        return bind(group_obj.stores, n_groups, group_obj.atomics, group_obj.mapped_stores)
+        return bind(group_obj.stores, n_groups, group_obj.atomics, group_obj.mapped_stores,
+                    group_obj.id_stores, group)
 
     def plan(self, *args, ctx=None):
         """Everything a call does short of launching: returns the list of

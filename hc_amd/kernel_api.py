@@ -13,6 +13,8 @@ kernels.  Nothing in this module computes array values.
 
 from __future__ import annotations
 
+import functools
+import itertools
 import math
 import operator
 from collections.abc import Iterable
@@ -190,9 +192,36 @@ class IndexExpr:
 
     __truediv__ = __rtruediv__ = __lt__ = __le__ = __gt__ = __ge__ = _unsupported
 
+    def _no_test(self, *_):
+        raise TraceError("a group-id dependent index was compared or tested (`==`, `!=`, "
+                         "`if idx:`): the body is traced once for all groups, so control flow "
+                         "cannot depend on the group")
+
+    __eq__ = __ne__ = __bool__ = _no_test
+    __hash__ = object.__hash__
+
+    def same_as(self, o) -> bool:
+        return self is o or (isinstance(o, IndexExpr) and self.op == o.op and
+                             all(same_index(a, b) for a, b in zip(self.args, o.args)))
+
     def __repr__(self):
         sign = {"add": "+", "sub": "-", "mul": "*", "floordiv": "//", "mod": "%"}[self.op]
         return f"({self.args[0]!r} {sign} {self.args[1]!r})"
+
+
+def same_index(a, b) -> bool:
+    """Structural equality of two index values (numbers, Affine, IndexExpr)."""
+    if a is b:
+        return True
+    if isinstance(a, (Affine, IndexExpr)):
+        return a.same_as(b)
+    if isinstance(b, (Affine, IndexExpr)):
+        return False
+    return a == b
+
+
+def same_starts(a, b) -> bool:
+    return len(a) == len(b) and all(same_index(x, y) for x, y in zip(a, b))
 
 
 def evaluate_index(e, group_ids):
@@ -239,7 +268,7 @@ class Affine:
         return not any(self.coeffs)
 
     def __add__(self, o):
-        if isinstance(o, IndexExpr):
+        if isinstance(o, (IndexExpr, ItemIndex)):
             return NotImplemented
         o = Affine.lift(o, len(self.coeffs))
         return Affine(self.const + o.const, [a + b for a, b in zip(self.coeffs, o.coeffs)])
@@ -250,17 +279,17 @@ class Affine:
         return Affine(-self.const, [-c for c in self.coeffs])
 
     def __sub__(self, o):
-        if isinstance(o, IndexExpr):
+        if isinstance(o, (IndexExpr, ItemIndex)):
             return NotImplemented
         return self + (-Affine.lift(o, len(self.coeffs)))
 
     def __rsub__(self, o):
-        if isinstance(o, IndexExpr):
+        if isinstance(o, (IndexExpr, ItemIndex)):
             return NotImplemented
         return Affine.lift(o, len(self.coeffs)) - self
 
     def __mul__(self, o):
-        if isinstance(o, IndexExpr):
+        if isinstance(o, (IndexExpr, ItemIndex)):
             return NotImplemented
         if isinstance(_index_const(o), Fraction):
             return IndexExpr.make("mul", self, o)
@@ -297,15 +326,120 @@ class Affine:
 
     __truediv__ = __rtruediv__ = __lt__ = __le__ = __gt__ = __ge__ = _unsupported
 
+    # The body is traced once for all groups, so a comparison whose outcome
+    # differs from group to group (`if gr.id[0] == 0:`) cannot be answered; it
+    # raises instead of picking one branch for every group.  Structural
+    # equality of two expressions is same_as().
+    def same_as(self, o) -> bool:
+        if not isinstance(o, Affine) or self.const != o.const:
+            return False
+        n = max(len(self.coeffs), len(o.coeffs))
+        return self.coeffs + (0,) * (n - len(self.coeffs)) == o.coeffs + (0,) * (n - len(o.coeffs))
+
+    def _compare(self, o):
+        if isinstance(o, Affine):
+            if self.is_const and o.is_const:
+                return self.const, o.const
+        elif self.is_const and isinstance(_index_const(o), (int, Fraction)):
+            return self.const, _index_const(o)
+        raise TraceError("a group id was compared or tested (`==`, `!=`, `if id:`): the body is "
+                         "traced once for all groups, so control flow cannot depend on the group")
+
     def __eq__(self, o):
-        o = Affine.lift(o, len(self.coeffs)) if not isinstance(o, Affine) else o
-        return self.const == o.const and self.coeffs == o.coeffs
+        a, b = self._compare(o)
+        return a == b
+
+    def __ne__(self, o):
+        a, b = self._compare(o)
+        return a != b
+
+    def __bool__(self):
+        a, _ = self._compare(0)
+        return bool(a)
 
     def __hash__(self):
-        return hash((self.const, self.coeffs))
+        return hash(self.const) if self.is_const else hash((self.const, self.coeffs))
 
     def __repr__(self):
         terms = [f"{c}*g{i}" for i, c in enumerate(self.coeffs) if c]
+        return " + ".join(terms + ([str(self.const)] if self.const or not terms else []))
+
+
+class ItemIndex:
+    """const + sum(g[i] * group_id[i]) + sum(l[i] * local_id[i]): what a body sees
+    inside a work-item scope (python/hckernel/kernel_api.py:397-403: local_id,
+    and global_id = group_id * group_shape + local_id).  Integer sums, differences
+    and integer multiples stay in this form; it indexes buffer elements
+    (`a[i, j]`) and may be stored as a value."""
+
+    __slots__ = ("const", "g", "l")
+
+    def __init__(self, const, g, l):
+        self.const, self.g, self.l = int(const), tuple(int(c) for c in g), tuple(int(c) for c in l)
+
+    @staticmethod
+    def lift(v, rank):
+        if isinstance(v, ItemIndex):
+            return v
+        if isinstance(v, Affine):
+            return ItemIndex(v.const, tuple(v.coeffs) + (0,) * (rank - len(v.coeffs)), (0,) * rank)
+        c = _index_const(v)
+        if not isinstance(c, int):
+            raise TraceError(f"unsupported work-item index value {v!r}")
+        return ItemIndex(c, (0,) * rank, (0,) * rank)
+
+    def __add__(self, o):
+        o = ItemIndex.lift(o, len(self.g))
+        return ItemIndex(self.const + o.const, [a + b for a, b in zip(self.g, o.g)],
+                         [a + b for a, b in zip(self.l, o.l)])
+
+    __radd__ = __add__
+
+    def __neg__(self):
+        return ItemIndex(-self.const, [-c for c in self.g], [-c for c in self.l])
+
+    def __sub__(self, o):
+        return self + (-ItemIndex.lift(o, len(self.g)))
+
+    def __rsub__(self, o):
+        return ItemIndex.lift(o, len(self.g)) - self
+
+    def __mul__(self, o):
+        if isinstance(o, (Affine, ItemIndex)):
+            varies = any(o.coeffs) if isinstance(o, Affine) else any(o.g) or any(o.l)
+            if varies:
+                if any(self.g) or any(self.l):
+                    raise TraceError("product of two ids")
+                return ItemIndex.lift(o, len(self.g)) * self.const
+            o = o.const
+        k = _index_const(o)
+        if not isinstance(k, int):
+            raise TraceError("a work-item index may only be multiplied by an integer")
+        return ItemIndex(self.const * k, [c * k for c in self.g], [c * k for c in self.l])
+
+    __rmul__ = __mul__
+
+    def _unsupported(self, *_):
+        raise TraceError("only + - and * by an integer are supported on work-item ids; comparisons "
+                         "and data-dependent control flow inside a scope have no native form")
+
+    __truediv__ = __rtruediv__ = __floordiv__ = __rfloordiv__ = __mod__ = __rmod__ = _unsupported
+    __lt__ = __le__ = __gt__ = __ge__ = __eq__ = __ne__ = __bool__ = _unsupported
+    __hash__ = None
+
+    def __index__(self):
+        if not any(self.g) and not any(self.l):
+            return self.const
+        raise TraceError("a work-item id was used where a number is needed")
+
+    __int__ = __index__
+
+    def key(self):
+        return (self.const, self.g, self.l)
+
+    def __repr__(self):
+        terms = [f"{c}*g{i}" for i, c in enumerate(self.g) if c]
+        terms += [f"{c}*l{i}" for i, c in enumerate(self.l) if c]
         return " + ".join(terms + ([str(self.const)] if self.const or not terms else []))
 
 
@@ -372,11 +506,29 @@ class BufferProxy:
     def ndim(self):
         return len(self.shape)
 
+    def _element_index(self, key):
+        """key as a tuple of ItemIndex if it addresses one element, else None."""
+        if len(key) != self.ndim or any(isinstance(k, slice) or k is None for k in key):
+            return None
+        group = getattr(self, "group", None)
+        if group is None:
+            raise TraceError("element access to a buffer outside a kernel body")
+        rank = len(group.shape)
+        out = []
+        for k in key:
+            if isinstance(k, IndexExpr):
+                raise TraceError("element indices with // or % of the group id have no native form")
+            out.append(ItemIndex.lift(k, rank))
+        return tuple(out)
+
     def __getitem__(self, key):
         if not isinstance(key, tuple):
             key = (key,)
         if len(key) > self.ndim:
             raise TraceError(f"too many indices for {self.name}")
+        index = self._element_index(key)
+        if index is not None:
+            return self.group.element_load(self, index)
         starts = []
         for k in key:
             if not isinstance(k, slice):
@@ -390,8 +542,15 @@ class BufferProxy:
                                       for s in starts))
 
     def __setitem__(self, key, value):
-        raise TraceError("direct assignment to a buffer is not supported on the GPU path; "
-                         "use group.store")
+        if value is _ATOMIC_DONE:
+            return
+        if not isinstance(key, tuple):
+            key = (key,)
+        index = self._element_index(key)
+        if index is None:
+            raise TraceError("assignment to a window of a buffer is not supported on the GPU "
+                             "path; use group.store (single elements may be assigned)")
+        self.group.element_store(self, index, value)
 
     def __repr__(self):
         return f"<buffer {self.name} {self.shape} {self.dtype_name}>"
@@ -647,6 +806,33 @@ class Tile:
                      (k.start, k.stop, k.step) if isinstance(k, slice) else int(k) for k in key)
         return Tile("slice", (self,), shape, self.dtype_name, key=norm)
 
+    def __setitem__(self, key, value):
+        """`tile[key] = value` with a static key: the tile object becomes the
+        updated tile (python/hckernel/kernel_api.py:125-131 assigns in place and
+        marks the elements active).  The old contents stay reachable as the first
+        argument of the new node."""
+        if not isinstance(key, tuple):
+            key = (key,)
+        if any(k is None or k is Ellipsis for k in key) or len(key) > len(self.shape):
+            raise TraceError("tile assignment: plain integer / slice keys only")
+        norm = []
+        for k, n in zip(key + (slice(None),) * (len(self.shape) - len(key)), self.shape):
+            if isinstance(k, slice):
+                start, stop, step = k.indices(n)
+                if step != 1:
+                    raise TraceError("tile assignment: unit-step slices only")
+                norm.append((start, max(stop, start)))
+            else:
+                i = int(k)                       # raises for ids that are not numbers
+                if not -n <= i < n:
+                    raise TraceError(f"tile assignment: index {i} out of range for extent {n}")
+                norm.append(i % n)
+        old = Tile(self.op, self.args, self.shape, self.dtype_name, **self.attrs)
+        self.op, self.args = "update", (old, Tile.wrap(value))
+        self.attrs = {"key": tuple(norm)}
+        Tile._counter += 1
+        self.uid = Tile._counter
+
     def reshape(self, *shape):
         shape = shape[0] if len(shape) == 1 and isinstance(shape[0], Iterable) else shape
         shape = tuple(int(s) for s in shape)
@@ -690,6 +876,10 @@ class CurrentGroup:
         self.stores = []          # (BufferView, Tile) in program order
         self.atomics = []         # (BufferProxy, element index, Tile) atomic additions
         self.mapped_stores = []   # (BufferView, Tile, index function) scattered stores
+        self.id_stores = []       # (BufferProxy, ItemIndex per dim, value ItemIndex, per work-item?)
+        self._ring = []           # greenlets of the subgroup scope that is running
+        self._turn = 0
+        self._in_workitems = False
 
     @property
     def id(self):
@@ -770,16 +960,114 @@ class CurrentGroup:
         return src[tuple(slice(0, s) for s in shape)]
 
     # -- nested scopes -----------------------------------------------------------------
+    # A subgroup scope is run as the reference's simulator runs it
+    # (python/hckernel/kernel_api.py:378-395,420-431): the number of subgroups of
+    # a group is a number at trace time, so the body is executed once per
+    # subgroup id, in order, each as a greenlet, and barrier() hands over to the
+    # next one.  What the bodies do to tiles (slices, reductions, element
+    # assignment into workgroup tiles, stores) lands in the same traced program;
+    # hc_amd.binding then folds per-subgroup partial results back into whole-row
+    # operations where a hand-written kernel does the same work.
+    #
+    # A work-item scope is traced once with symbolic local ids: a per-work-item
+    # value is the element of a group-shaped tile that belongs to the work-item,
+    # `a[wi.global_id()]` is that element of the group's tile of `a`, and
+    # `out[wi.global_id()] = v` stores the tile.  Statements execute for the whole
+    # group in program order, which is what barrier() asks for.
+    MAX_SUBGROUPS = 4096
+
     def subgroups(self, func):
-        raise TraceError("explicit subgroup scopes have no native kernel: the hand-written "
-                         "kernels choose their own wave-level decomposition")
+        ranges = [range(v) for v in self._shape[:-1]]
+        ranges.append(range(-(-self._shape[-1] // self._subgroup_size)))
+
+        def run():
+            from greenlet import greenlet
+            if self._ring or self._in_workitems:
+                raise TraceError("nested scopes are not supported")
+            ids = list(itertools.product(*ranges))
+            if len(ids) > self.MAX_SUBGROUPS:
+                raise TraceError(f"{len(ids)} subgroups per group: too many to trace one by one")
+
+            def task(sgid):
+                func(CurrentSubGroup(self._subgroup_size, sgid))
+
+            self._ring = [greenlet(functools.partial(task, i)) for i in ids]
+            self._turn = 0
+            try:
+                for t in list(self._ring):
+                    t.switch()
+            finally:
+                self._ring, self._turn = [], 0
+
+        return run
 
     def workitems(self, func):
-        raise TraceError("explicit work-item scopes have no native kernel: the hand-written "
-                         "kernels choose their own per-lane decomposition")
+        rank = len(self._shape)
+
+        def unit(d):
+            return tuple(1 if j == d else 0 for j in range(rank))
+
+        def run():
+            if self._ring or self._in_workitems:
+                raise TraceError("nested scopes are not supported")
+            zero = (0,) * rank
+            lid = tuple(ItemIndex(0, zero, unit(d)) for d in range(rank))
+            gid = tuple(ItemIndex(0, tuple(self._shape[d] * c for c in unit(d)), unit(d))
+                        for d in range(rank))
+            self._in_workitems = True
+            try:
+                func(CurrentWorkitem(lid, gid))
+            finally:
+                self._in_workitems = False
+
+        return run
 
     def barrier(self):
+        n = len(self._ring)
+        if n <= 1:
+            return None
+        self._turn = (self._turn + 1) % n
+        self._ring[self._turn].switch()
         return None
+
+    # -- single elements of buffers ------------------------------------------------------
+    def _is_global_id(self, index, proxy):
+        """index addresses, per buffer dim d, global id d (buffer rank == work rank)."""
+        rank = len(self._shape)
+        if proxy.ndim != rank:
+            return False
+        for d, ix in enumerate(index):
+            want_g = tuple(self._shape[d] if j == d else 0 for j in range(rank))
+            want_l = tuple(1 if j == d else 0 for j in range(rank))
+            if ix.const != 0 or ix.g != want_g or ix.l != want_l:
+                return False
+        return True
+
+    def element_load(self, proxy, index):
+        if not self._in_workitems:
+            raise TraceError("reading single buffer elements is supported inside a work-item "
+                             "scope only (use group.load elsewhere)")
+        if not self._is_global_id(index, proxy):
+            raise TraceError(f"{proxy.name}[{', '.join(map(repr, index))}]: inside a work-item "
+                             "scope a buffer is read at wi.global_id() only")
+        return self.load(proxy[tuple(slice(o, None) for o in self.work_offset)], self._shape)
+
+    def element_store(self, proxy, index, value):
+        if isinstance(value, Tile) and value.shape == self._shape and self._in_workitems:
+            if not self._is_global_id(index, proxy):
+                raise TraceError(f"{proxy.name}[...] = value: inside a work-item scope a value "
+                                 "is stored at wi.global_id() only")
+            self.store(proxy[tuple(slice(o, None) for o in self.work_offset)], value)
+            return
+        if isinstance(value, Tile):
+            raise TraceError("only ids, numbers and per-work-item values may be assigned to a "
+                             "buffer element")
+        rank = len(self._shape)
+        if isinstance(value, (float, np.floating)) and float(value) != int(value):
+            raise TraceError("only integers and ids may be assigned to a buffer element")
+        if isinstance(value, (float, np.floating)):
+            value = int(value)
+        self.id_stores.append((proxy, index, ItemIndex.lift(value, rank), self._in_workitems))
 
 
 class CurrentGroup1(CurrentGroup):

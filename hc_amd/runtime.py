@@ -84,6 +84,14 @@ hcamdLaunchCopy2D = _sig(_rt, "hcamdLaunchCopy2D", _int, _vp, _sz, _vp, _sz, _sz
                          _ssz, _ssz, _vp, _sz, _sz, _ssz, _ssz)
 hcamdLaunchCopy2DTiled = _sig(_rt, "hcamdLaunchCopy2DTiled", _int, _vp, _sz, _vp, _vp,
                               _sz, _sz, _ssz, _ssz, _sz, _sz, _sz)
+class AffineId(C.Structure):
+    """HcamdAffineId of include/hc_amd_runtime.h."""
+    _fields_ = [("c", C.c_int64), ("g", C.c_int64 * 3), ("l", C.c_int64 * 3)]
+
+
+hcamdLaunchIdScatter = _sig(_rt, "hcamdLaunchIdScatter", _int, _vp, _vp, _int, _sz, _sz_p,
+                            C.POINTER(_ssz), C.POINTER(AffineId), C.POINTER(AffineId), _sz, _sz_p,
+                            _sz_p, _int)
 hcamdLaunchStream = _sig(_rt, "hcamdLaunchStream", _int, _vp, _int, _int, C.POINTER(_vp), _vp, _sz)
 hcamdLaunchAddF32 = _sig(_rt, "hcamdLaunchAddF32", _int, _vp, _vp, _vp, _vp, _sz)
 hcamdLaunchFmaF16 = _sig(_rt, "hcamdLaunchFmaF16", _int, _vp, _vp, _sz, _vp, _sz, _vp,
@@ -399,6 +407,45 @@ def plan_copy2d_tiled(src, dst, block_x: int, block_y: int, unroll: int = 1) -> 
     return Plan(ctx, hcamdLaunchCopy2DTiled,
                 (ctx.queue, s.itemsize, s.ptr, d.ptr, rows, cols, s.strides[0], d.strides[0],
                  block_x, block_y, unroll), "hcamdLaunchCopy2DTiled", (src, dst))
+
+
+I32, I64 = 3, 4
+
+
+def plan_id_scatter(out, index, value, group_count, group_shape, per_item=True, out_type=None) -> Plan:
+    """out[index] = value for every work-item (or once per group), index (one
+    (c, g, l) triple per dimension of out) and value affine in group id and
+    local id: c + sum(g[k] * group_id[k]) + sum(l[k] * local_id[k]) (see
+    hcamdLaunchIdScatter)."""
+    ctx = _ctx_of(out)
+    m = as_memref(out)
+    if out_type is None:
+        name = getattr(getattr(out, "dtype", None), "name", None) or str(getattr(out, "dtype", ""))
+        out_type = {"int32": I32, "int64": I64, "float32": F32}.get(name.replace("torch.", ""))
+        if out_type is None:
+            raise HcRuntimeError(f"id_scatter: output type {name!r} (int32, int64, float32 only)")
+    rank = len(group_shape)
+
+    def pack(t):
+        c, g, l = t
+        a = AffineId()
+        a.c = int(c)
+        for k in range(3):
+            a.g[k] = int(g[k]) if k < len(g) else 0
+            a.l[k] = int(l[k]) if k < len(l) else 0
+        return a
+    if len(index) != len(m.shape):
+        raise HcRuntimeError("id_scatter: one index per dimension of the output")
+    idx = (AffineId * len(index))(*[pack(t) for t in index])
+    val = pack(value)
+    shape = (_sz * len(m.shape))(*m.shape)
+    strides = (_ssz * len(m.shape))(*m.strides)
+    counts = (_sz * rank)(*group_count)
+    gshape = (_sz * rank)(*group_shape)
+    return Plan(ctx, hcamdLaunchIdScatter,
+                (ctx.queue, m.ptr, out_type, len(m.shape), shape, strides, idx, C.byref(val), rank,
+                 counts, gshape, 1 if per_item else 0), "hcamdLaunchIdScatter",
+                (out, idx, val, shape, strides, counts, gshape))
 
 
 STREAM_WRITE = {"none": 0, "full": 1, "half": 2}

@@ -214,6 +214,26 @@ int hcamdLaunchCopy2D(OlQueue q, size_t elemSize, const void *src,
                       size_t dstCols, ptrdiff_t dstStride0,
                       ptrdiff_t dstStride1) HCAMD_NOEXCEPT;
 
+/* Ids as data: out[index] = value for every work-item (perItem != 0) or once per
+ * group, with index (one per dimension of out) and value affine in the group id
+ * and the local id: x = c + sum_k g[k] * group_id[k] + sum_k l[k] * local_id[k],
+ * k over the `rank` dimensions of the work shape in the Python order.  This is
+ * what a body computes that stores `wi.local_id()`, `wi.global_id()`, group ids
+ * or subgroup ids into a buffer (python/hckernel/kernel_api.py:231-252,397-403;
+ * python/hckernel/kernel.py:97-131), and the launch uses the reference's own
+ * geometry: block = groupShape, grid = groupCount, last dimension on x
+ * (mlir/lib/Transforms/LowerHKernel.cpp:284-367), so hardware ids are the
+ * model's ids.  outType: HCAMD_I32, HCAMD_I64 or HCAMD_F32; strides in
+ * elements.  An index outside out stores nothing.  prod(groupShape) <= 1024. */
+typedef struct HcamdAffineId {
+  int64_t c, g[3], l[3];
+} HcamdAffineId;
+int hcamdLaunchIdScatter(OlQueue q, void *out, int outType, size_t outRank,
+                         const size_t *outShape, const ptrdiff_t *outStrides,
+                         const HcamdAffineId *index, const HcamdAffineId *value, size_t rank,
+                         const size_t *groupCount, const size_t *groupShape,
+                         int perItem) HCAMD_NOEXCEPT;
+
 /* Stream calibration (no counterpart in the reference): what HBM delivers for
  * a mix of read and write streams with nothing else in the way, the yardstick
  * the memory-bound kernels are held to.  nReads (0..3) vectors of `bytes` bytes
@@ -263,7 +283,7 @@ int hcamdLaunchFmaF16(OlQueue q, const void *a, size_t lda, const void *b,
  * nearest even.  Operands are fp32 or fp16, each with its own leading
  * dimension in elements.  The program is validated on the host; a malformed
  * one is an error, not a launch. */
-enum HcamdElemType { HCAMD_F32 = 0, HCAMD_F16 = 1, HCAMD_BF16 = 2 };
+enum HcamdElemType { HCAMD_F32 = 0, HCAMD_F16 = 1, HCAMD_BF16 = 2, HCAMD_I32 = 3, HCAMD_I64 = 4 };
 enum HcamdMapOp {
   HCAMD_MAP_END = 0,
   HCAMD_MAP_IN = 1,    /* push operand `arg` */

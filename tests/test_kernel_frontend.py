@@ -1130,3 +1130,170 @@ def test_random_row_expressions_compile_to_stages_that_mean_the_same(ctx):
         scale = 1.0 + float(np.abs(want).max())
         np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-5 * scale, err_msg=text)
     assert tried < 120
+
+
+# ---------------------------------------------------------------------------
+# Control flow on group ids, subgroup and work-item scopes
+# ---------------------------------------------------------------------------
+def test_control_flow_on_the_group_id_is_refused_not_miscompiled(ctx):
+    N = sym.N
+    a, b = FakeDev((1024,), "float32"), FakeDev((1024,), "float32")
+    for test in (lambda gr: gr.work_offset[0] == 0, lambda gr: gr.id[0] != 0,
+                 lambda gr: bool(gr.id[0]), lambda gr: (gr.id[0] // 2) == 0,
+                 lambda gr: bool(gr.id[0] % 2)):
+        @kernel(work_shape=N, group_shape=256)
+        def k(gr: CurrentGroup, src: Buffer[N, DT], dst: Buffer[N, DT]):
+            o = gr.work_offset[0]
+            if test(gr):
+                gr.store(dst[o:], gr.load(src[o:], shape=gr.shape[0]))
+
+        with pytest.raises(NoNativeKernel, match="traced once for all groups"):
+            k.plan(a, b, ctx=ctx)
+
+    # the same tests on numbers that do not depend on the group are fine
+    @kernel(work_shape=N, group_shape=256)
+    def k2(gr: CurrentGroup, src: Buffer[N, DT], dst: Buffer[N, DT]):
+        o = gr.work_offset[0]
+        if (o - o) == 0 and gr.shape[0] == 256:
+            gr.store(dst[o:], gr.load(src[o:], shape=gr.shape[0]))
+
+    (p,) = k2.plan(a, b, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchCopy2D
+
+
+def _softmax_with_subgroup_partials(rows_per_group, lanes, sg):
+    from hc_amd.kernel import CurrentSubGroup
+    ROWS, N = sym.ROWS, sym.N
+
+    @kernel(work_shape=(ROWS, lanes), group_shape=(rows_per_group, lanes), subgroup_size=sg)
+    def softmax(gr: CurrentGroup, x: Buffer[ROWS, N, DT], y: Buffer[ROWS, N, DT]):
+        r0 = gr.work_offset[0]
+        n = x.shape[1]
+        nsub = gr.shape[1] // sg
+        seg = n // nsub
+        t = gr.load(x[r0:], shape=(gr.shape[0], n))
+        pmax = gr.zeros((gr.shape[0], nsub), np.float32)
+
+        @gr.subgroups
+        def part_max(s: CurrentSubGroup):
+            i, k = s.subgroup_id()
+            pmax[i, k] = t[i, k * seg:(k + 1) * seg].max()
+
+        part_max()
+        gr.barrier()
+        e = np.exp(t - pmax.max(axis=1, keepdims=True))
+        psum = gr.zeros((gr.shape[0], nsub), np.float32)
+
+        @gr.subgroups
+        def part_sum(s: CurrentSubGroup):
+            i, k = s.subgroup_id()
+            psum[i, k] = e[i, k * seg:(k + 1) * seg].sum()
+
+        part_sum()
+        gr.barrier()
+        gr.store(y[r0:], e / psum.sum(axis=1, keepdims=True))
+
+    return softmax
+
+
+def test_subgroup_partials_fold_back_into_the_row_softmax(ctx):
+    x, y = FakeDev((64, 8192), "float32"), FakeDev((64, 8192), "float32")
+    for rows, lanes, sg in ((1, 256, 64), (2, 256, 64), (1, 1024, 64), (1, 256, 16)):
+        (p,) = _softmax_with_subgroup_partials(rows, lanes, sg).plan(x, y, ctx=ctx)
+        assert p.fn is rt.hcamdLaunchSoftmaxF32
+        assert p.args[1] == x.ptr and p.args[3] == y.ptr and p.args[5:7] == (64, 8192)
+
+
+def test_subgroup_partials_that_do_not_cover_the_row_are_not_folded(ctx):
+    from hc_amd.kernel import CurrentSubGroup
+    ROWS, N = sym.ROWS, sym.N
+
+    @kernel(work_shape=(ROWS, 256), group_shape=(1, 256), subgroup_size=64)
+    def k(gr: CurrentGroup, x: Buffer[ROWS, N, DT], y: Buffer[ROWS, N, DT]):
+        r0 = gr.work_offset[0]
+        t = gr.load(x[r0:], shape=(1, x.shape[1]))
+        pmax = gr.zeros((1, 4), np.float32)
+
+        @gr.subgroups
+        def part(s: CurrentSubGroup):
+            i, k = s.subgroup_id()
+            pmax[i, k] = t[i, k * 100:(k + 1) * 100].max()      # 400 of 1024 columns
+
+        part()
+        gr.store(y[r0:], t - pmax.max(axis=1, keepdims=True))
+
+    with pytest.raises(NoNativeKernel):
+        k.plan(FakeDev((8, 1024), "float32"), FakeDev((8, 1024), "float32"), ctx=ctx)
+
+
+def test_subgroup_scope_runs_like_the_simulator(ctx):
+    """Ids, sizes and barrier phases of python/hckernel/tests/test_kernel_sim.py:229-320,
+    observed while the body is traced: one pass per subgroup id, in order."""
+    from hc_amd.kernel import CurrentSubGroup
+    G1, G2, G3, L1, L2, L3 = sym.G1, sym.G2, sym.G3, sym.L1, sym.L2, sym.L3
+    seen = []
+
+    @kernel(work_shape=(G1, G2, G3), group_shape=(L1, L2, L3), subgroup_size=4)
+    def k(gr: CurrentGroup, g: tuple[G1, G2, G3], l: tuple[L1, L2, L3], out):
+        @gr.subgroups
+        def inner(s: CurrentSubGroup):
+            seen.append((1, s.subgroup_id(), s.size()))
+            gr.barrier()
+            seen.append((2, s.subgroup_id(), s.size()))
+
+        inner()
+        out[gr.id[2]] = gr.id[2]
+
+    (p,) = k.plan((1, 1, 16), (1, 1, 8), FakeDev((2,), "int32"), ctx=ctx)
+    assert seen == [(1, (0, 0, 0), 4), (1, (0, 0, 1), 4), (2, (0, 0, 0), 4), (2, (0, 0, 1), 4)]
+    assert p.fn is rt.hcamdLaunchIdScatter
+
+
+def test_workitem_scope_binds_ids_and_elementwise_statements(ctx):
+    from hc_amd.kernel import CurrentWorkitem
+    N = sym.N
+
+    @kernel(work_shape=N, group_shape=64)
+    def ids(gr: CurrentGroup, lid: Buffer[N, DT], gid: Buffer[N, DT]):
+        @gr.workitems
+        def inner(wi: CurrentWorkitem):
+            (g,) = wi.global_id()
+            lid[g] = wi.local_id()[0]
+            gr.barrier()
+            gid[g] = 2 * g + 1
+
+        inner()
+
+    a, b = FakeDev((256,), "int32"), FakeDev((256,), "int32")
+    p1, p2 = ids.plan(a, b, ctx=ctx)
+    assert p1.fn is rt.hcamdLaunchIdScatter and p2.fn is rt.hcamdLaunchIdScatter
+    idx, val = p1.args[6][0], p1.args[7]._obj
+    assert (idx.c, idx.g[0], idx.l[0]) == (0, 64, 1) and (val.c, val.g[0], val.l[0]) == (0, 0, 1)
+    val2 = p2.args[7]._obj
+    assert (val2.c, val2.g[0], val2.l[0]) == (1, 128, 2)
+    assert tuple(p1.args[9]) == (4,) and tuple(p1.args[10]) == (64,) and p1.args[11] == 1
+
+    @kernel(work_shape=N, group_shape=256)
+    def vadd(gr: CurrentGroup, x: Buffer[N, DT], y: Buffer[N, DT], z: Buffer[N, DT]):
+        @gr.workitems
+        def inner(wi: CurrentWorkitem):
+            i = wi.global_id()
+            z[i] = x[i] + y[i]
+
+        inner()
+
+    x, y, z = (FakeDev((4096,), "float32") for _ in range(3))
+    (p,) = vadd.plan(x, y, z, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchAddF32 and p.args[1:4] == (x.ptr, y.ptr, z.ptr)
+
+    @kernel(work_shape=N, group_shape=256)
+    def shifted(gr: CurrentGroup, x: Buffer[N, DT], z: Buffer[N, DT]):
+        @gr.workitems
+        def inner(wi: CurrentWorkitem):
+            (i,) = wi.global_id()
+            z[i] = x[i + 1]
+
+        inner()
+
+    with pytest.raises(NoNativeKernel, match="wi.global_id"):
+        shifted.plan(x, z, ctx=ctx)
