@@ -268,7 +268,22 @@ std::unordered_map<std::string, int> &variants() {
       {"gather", 0}, {"gather_fuse", 0}};
   return v;
 }
-int variantOf(const char *family) { return variants()[family]; }
+std::mutex g_variantLock; // guards variants()
+// Per-thread overrides: a thread that launches with a variant of its own (a
+// tuned kernel object) neither disturbs nor sees what other threads selected.
+thread_local std::unordered_map<std::string, int> t_variants;
+
+int variantOf(const char *family) {
+  if (!t_variants.empty()) {
+    auto it = t_variants.find(family);
+    if (it != t_variants.end())
+      return it->second;
+  }
+  std::lock_guard<std::mutex> guard(g_variantLock);
+  auto &v = variants();
+  auto it = v.find(family);
+  return it == v.end() ? 0 : it->second;
+}
 
 // ---------------------------------------------------------------------------
 // Process-wide device and queue of the hcgpu* entry points
@@ -710,11 +725,31 @@ int hcamdDeviceInfo(OlDevice dev, int *computeUnits, int *clockKHz,
 int hcamdSetVariant(const char *family, int variant) noexcept {
   if (!family)
     return 1;
+  std::lock_guard<std::mutex> guard(g_variantLock);
   auto &v = variants();
   auto it = v.find(family);
   if (it == v.end())
     return 1;
   it->second = variant;
+  return 0;
+}
+
+int hcamdSetThreadVariant(const char *family, int variant) noexcept {
+  if (!family)
+    return 1;
+  {
+    std::lock_guard<std::mutex> guard(g_variantLock);
+    if (variants().find(family) == variants().end())
+      return 1;
+  }
+  try {
+    if (variant < 0)
+      t_variants.erase(family);
+    else
+      t_variants[family] = variant;
+  } catch (...) {
+    return 1;
+  }
   return 0;
 }
 
@@ -2087,15 +2122,20 @@ HcamdGatherGemm hcamdGatherGemmCreate(OlQueue q, const HcamdGatherOperand *a,
     }
     rec[15] = (int32_t)(windowOf[g] << 2); // bits 0 and 1 are the flags set below
   }
-  for (size_t w = 0; w < windowRep.size(); ++w) {
-    // the b window of any record that has it (records hold it at words 5..9)
-    int32_t *dst = host.data() + plan->offWindows + w * 8;
-    for (size_t slot = 0; slot < slots.size(); ++slot)
-      if (slots[slot] >= 0 && windowOf[(size_t)slots[slot]] == w) {
-        std::memcpy(dst, host.data() + plan->offGroups + slot * kGatherRecord + 5,
-                    5 * sizeof(int32_t));
-        break;
-      }
+  {
+    // the b window of each distinct window, from the first record that has it
+    // (records hold it at words 5..9): one pass over the slots
+    std::vector<char> have(windowRep.size(), 0);
+    for (size_t slot = 0; slot < slots.size(); ++slot) {
+      if (slots[slot] < 0)
+        continue;
+      const size_t w = windowOf[(size_t)slots[slot]];
+      if (have[w])
+        continue;
+      have[w] = 1;
+      std::memcpy(host.data() + plan->offWindows + w * 8,
+                  host.data() + plan->offGroups + slot * kGatherRecord + 5, 5 * sizeof(int32_t));
+    }
   }
   for (int o = 0; o < 3; ++o) {
     gatherEntries(*ops[o], ops[o]->rowIndex, rows[o], rowDim[o],

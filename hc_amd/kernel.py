@@ -36,7 +36,7 @@ from .autotune import TunedParams, autotune
 from .binding import NoNativeKernel, bind
 from .indexing import sym
 from .kernel_api import (Buffer, BufferProxy, CurrentGroup, CurrentGroup1, CurrentGroup2,
-                         CurrentGroup3, CurrentSubGroup, CurrentWorkitem, Mapping, TraceError,
+                         CurrentGroup3, CurrentSubGroup, CurrentWorkitem, DynInt, Mapping, TraceError,
                          TunableParam, atomic_ref, create_mapping, dtype_name)
 from .typename import Typename, typename
 
@@ -122,7 +122,7 @@ def _to_ints(expr, subs):
     return int(expr)
 
 
-def _resolve_symbols(func, subs, _memo=None):
+def _resolve_symbols(func, subs, _memo=None, dynamic=frozenset()):
     """Clone func with sympy symbols / expressions in its closure and globals
     replaced by their values (python/hckernel/kernel_api.py:43-90); index
     mappings found there are resolved the same way.  Each function is cloned
@@ -135,15 +135,19 @@ def _resolve_symbols(func, subs, _memo=None):
     memo[id(func)] = None                       # in progress
 
     def value_of(v):
+        # values of symbols in `dynamic` (known at launch only) are marked as such
         if isinstance(v, sympy.Symbol):
-            return subs.get(v)
+            r = subs.get(v)
+            return DynInt(r) if v in dynamic and type(r) is int else r
         if isinstance(v, sympy.Expr):
             r = v.subs(subs)
-            return int(r) if r.is_Integer else r
+            if not r.is_Integer:
+                return r
+            return DynInt(int(r)) if v.free_symbols & dynamic else int(r)
         if isinstance(v, Mapping):
             if memo.get(id(v.func), 0) is None:
                 return None
-            return Mapping(_resolve_symbols(v.func, subs, memo))
+            return Mapping(_resolve_symbols(v.func, subs, memo, dynamic))
         return None
 
     closure = None
@@ -229,22 +233,48 @@ class GpuKernel:
             raise RuntimeError("work_shape and group_shape have different ranks")
         n_groups = tuple(-(-w // g) for w, g in zip(work, group))
         names = list(inspect.signature(self.func).parameters)[1:]
+        # Symbols whose value is only known at launch: everything bound from the
+        # arguments except literals and tunables.
+        static_syms = set(self.literals) | set(self._defaults) | set(self.tuned)
+        dynamic = frozenset(k for k in subs if isinstance(k, sympy.Symbol) and k not in static_syms)
+        ann = inspect.get_annotations(self.func)
+
+        def dims_of(name, shape):
+            a = ann.get(name)
+            spec = getattr(a, "shape", None) if isinstance(a, type) and issubclass(a, Buffer) else None
+            out = []
+            for d, n in enumerate(shape):
+                s = spec[d] if spec is not None and d < len(spec) else None
+                static = isinstance(s, int) or (isinstance(s, sympy.Symbol) and s in static_syms)
+                out.append(int(n) if static else DynInt(n))
+            return tuple(out)
+
         proxies = []
         for i, (a, m) in enumerate(zip(args, memrefs)):
+            name = names[i] if i < len(names) else f"arg{i}"
             if m is None:
+                s = ann.get(name)
+                if type(a) is int and isinstance(s, sympy.Symbol) and s in dynamic:
+                    a = DynInt(a)
                 proxies.append(a)
             else:
-                proxies.append(BufferProxy(i, names[i] if i < len(names) else f"arg{i}",
-                                           m.shape, m.strides, _array_dtype(a), a))
+                proxies.append(BufferProxy(i, name, dims_of(name, m.shape), m.strides,
+                                           _array_dtype(a), a))
         group_obj = [CurrentGroup1, CurrentGroup2, CurrentGroup3][len(work) - 1](group, sg)
         for p in proxies:
             if isinstance(p, BufferProxy):
                 p.group = group_obj
-        body = _resolve_symbols(self.func, subs)
+        body = _resolve_symbols(self.func, subs, dynamic=dynamic)
         try:
             body(group_obj, *proxies)
         except TraceError as exc:
             raise NoNativeKernel(f"{self.func.__name__}: {exc}") from exc
+        finally:
+            # the plan makers take their arrays from the memrefs of each call; the
+            # arrays of the call that was traced must not live on in the cache
+            for p in proxies:
+                if isinstance(p, BufferProxy):
+                    p.obj = None
         return bind(group_obj.stores, n_groups, group_obj.atomics, group_obj.mapped_stores,
                     group_obj.id_stores, group)
 
@@ -279,14 +309,16 @@ class GpuKernel:
 
     def __call__(self, *args, sync: bool = True):
         plans = self.plan(*args)
+        # this kernel's tuned variants apply to this thread's launches only and
+        # leave a process-wide hcamdSetVariant choice untouched
         for family, v in self.variants.items():
-            rt.set_variant(family, v)
+            rt.set_thread_variant(family, v)
         try:
             for p in plans:
                 p.launch()
         finally:
             for family in self.variants:
-                rt.set_variant(family, 0)
+                rt.set_thread_variant(family, -1)
         self.last_plans = plans
         if sync and plans:
             plans[0].ctx.synchronize()

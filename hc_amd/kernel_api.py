@@ -27,6 +27,37 @@ class TraceError(RuntimeError):
     """The kernel body did something the tracer cannot express."""
 
 
+class DynInt(int):
+    """An integer that is only known at launch time: the value of a symbol bound
+    from a buffer dimension or from a scalar argument that is neither a literal
+    nor a tunable.  It behaves like the int it is; arithmetic on it stays
+    dynamic.  The one place that cares is vload, whose shape must be static
+    (docs/langref.md:226-243 of the reference: "Vector allocation shape must be
+    determinable at compile time")."""
+
+    __slots__ = ()
+
+
+def _dyn_method(name):
+    base = getattr(int, name)
+
+    def method(self, *args):
+        r = base(self, *args)
+        return DynInt(r) if type(r) is int else r
+    method.__name__ = name
+    return method
+
+
+for _name in ("__add__", "__radd__", "__sub__", "__rsub__", "__mul__", "__rmul__", "__floordiv__",
+              "__rfloordiv__", "__mod__", "__rmod__", "__neg__", "__pos__", "__abs__", "__pow__",
+              "__rpow__", "__lshift__", "__rshift__", "__and__", "__or__", "__xor__"):
+    setattr(DynInt, _name, _dyn_method(_name))
+
+
+def is_static(v) -> bool:
+    return not isinstance(v, DynInt)
+
+
 # ---------------------------------------------------------------------------
 # Small public types (kernel_api.py:35-40, 214-220, 231-252, 437-451)
 # ---------------------------------------------------------------------------
@@ -926,7 +957,18 @@ class CurrentGroup:
         return Tile("load", (), shape, view.base.dtype_name, view=view)
 
     def vload(self, array, shape, mapping=None):
-        return self.load(array, shape, mapping)
+        """A load into a vector: same result as load, but the shape has to be
+        static (numbers, group.shape, literal symbols and tunables), as the
+        reference specifies (docs/langref.md:226-243; a vector is register
+        resident, mlir/lib/Transforms/LowerHKernel.cpp:1056-1083)."""
+        dims = shape if isinstance(shape, Iterable) else (shape,)
+        if not all(is_static(d) for d in dims):
+            raise TraceError("vload needs a static shape: numbers, group.shape, literal symbols "
+                             "and tunables, not buffer dimensions or other values that are only "
+                             "known at launch (use load for those)")
+        t = self.load(array, shape, mapping)
+        t.attrs["vector"] = True
+        return t
 
     def store(self, dst, src, mapping=None):
         view = _as_view(dst)

@@ -79,6 +79,7 @@ hcamdDeviceInfo = _sig(_rt, "hcamdDeviceInfo", _int, _vp, C.POINTER(_int),
                        C.POINTER(_int), C.POINTER(_int), C.POINTER(_int), _sz_p,
                        C.c_char_p, _sz)
 hcamdSetVariant = _sig(_rt, "hcamdSetVariant", _int, C.c_char_p, _int)
+hcamdSetThreadVariant = _sig(_rt, "hcamdSetThreadVariant", _int, C.c_char_p, _int)
 hcamdLastKernelName = _sig(_rt, "hcamdLastKernelName", C.c_char_p)
 hcamdLaunchCopy2D = _sig(_rt, "hcamdLaunchCopy2D", _int, _vp, _sz, _vp, _sz, _sz,
                          _ssz, _ssz, _vp, _sz, _sz, _ssz, _ssz)
@@ -898,6 +899,12 @@ def gemm_bf16(a, bt, c, sync: bool = True) -> None:
 
 def set_variant(family: str, variant: int) -> None:
     if hcamdSetVariant(family.encode(), int(variant)):
+        raise HcRuntimeError(f"unknown kernel family {family!r}")
+
+
+def set_thread_variant(family: str, variant: int) -> None:
+    """The choice for this thread only (variant < 0 removes it)."""
+    if hcamdSetThreadVariant(family.encode(), int(variant)):
         raise HcRuntimeError(f"unknown kernel family {family!r}")
 
 

@@ -552,8 +552,14 @@ int hcamdLaunchGemmF16(OlQueue q, const void *a, size_t lda, const void *bt,
  * choice by shape).  For tuning and measurement; family names are "add",
  * "fma", "softmax", "quantize", "gemm", "copy", "map", "gather" (block
  * shape), "gather_fuse" (groups per workgroup; read by hcamdGatherGemmCreate).
- * Returns 1 for an unknown family. */
+ * Process-wide, guarded by a lock.  Returns 1 for an unknown family. */
 int hcamdSetVariant(const char *family, int variant) HCAMD_NOEXCEPT;
+/* The same choice for the calling thread only: it takes precedence over
+ * hcamdSetVariant for launches made by this thread and is invisible to others
+ * (variant < 0 removes it).  What a tuned kernel object uses around its own
+ * launches, so that threads launching differently tuned kernels do not race
+ * and a process-wide choice is left as it was. */
+int hcamdSetThreadVariant(const char *family, int variant) HCAMD_NOEXCEPT;
 
 /* Name and launch geometry of the kernel the most recent typed launcher
  * enqueued on this thread (for reports and profiles). */

@@ -843,3 +843,116 @@ def test_random_row_expressions_match_the_simulator():
         assert_allclose(out.to_host(), want, rtol=1e-4, atol=1e-5 * scale,
                         err_msg=f"{text} on {rows} x {n}")
     assert tried < 90
+
+
+# ---------------------------------------------------------------------------
+# Asynchronous launches, events, vload, per-thread variants
+# ---------------------------------------------------------------------------
+def test_dependent_launches_without_synchronisation_between_two_events():
+    """A chain of launches enqueued with sync=False on one queue, each reading
+    what the one before wrote (the reference synchronises after every launch,
+    python/cpp/py-runtime/src/GpuRuntime.cpp:60-69; here the queue keeps the
+    order).  The events bracket the chain on the queue; the host waits once."""
+    import time
+    N = sym.N
+    f = np.float32
+
+    @kernel(work_shape=N, group_shape=256)
+    def axpy(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], c: Buffer[N, DT]):
+        o = gr.work_offset[0]
+        gr.store(c[o:], gr.load(a[o:], shape=gr.shape[0]) * f(0.5) + gr.load(b[o:], shape=gr.shape[0]))
+
+    @kernel(work_shape=N, group_shape=256)
+    def total(gr: CurrentGroup, x: Buffer[N, DT], result: Buffer[1, DT]):
+        o = gr.work_offset[0]
+        atomic_ref(result)[0] += gr.load(x[o:], shape=gr.shape[0]).sum()
+
+    n = 8_000_003
+    x0, y0 = cf.inputs_c1(n)
+    ctx = rt.default_context("hip:0")
+    dx, dy = rt.to_device(x0), rt.to_device(y0)
+    t1, t2, t3 = (rt.DeviceArray((n,), np.float32) for _ in range(3))
+    cell = rt.to_device(np.zeros(1, np.float32))
+    axpy(dx, dy, t1)                                   # traced and built outside the timed part
+    total(t1, cell)
+    cell2 = rt.to_device(np.zeros(1, np.float32))
+    ctx.synchronize()
+    start, stop = rt.Event(ctx), rt.Event(ctx)
+    wall0 = time.perf_counter()
+    start.record()
+    axpy(dx, dy, t1, sync=False)                       # t1 = x/2 + y
+    axpy(t1, dx, t2, sync=False)                       # t2 = t1/2 + x
+    axpy(t2, t1, t3, sync=False)                       # t3 = t2/2 + t1
+    total(t3, cell2, sync=False)                       # sum of t3
+    stop.record()
+    enqueued = time.perf_counter() - wall0
+    stop.synchronize()
+    wall = time.perf_counter() - wall0
+    elapsed = start.elapsed_ms(stop) * 1e-3
+    h = f(0.5)
+    w1 = x0 * h + y0
+    w2 = w1 * h + x0
+    w3 = w2 * h + w1
+    assert_array_equal(t3.to_host().view(np.uint32), w3.view(np.uint32))
+    ref = w3.astype(np.float64)
+    assert abs(float(cell2.to_host()[0]) - ref.sum()) <= 64 * 2.0 ** -24 * np.abs(ref).sum()
+    assert 0.0 < elapsed < wall, (elapsed, wall)
+    # three 96 MB passes and a reduction cannot be done before they were enqueued
+    # unless the launches had blocked the host
+    assert elapsed > 30e-6 and enqueued < wall
+
+
+def test_vload_bodies_take_the_16_byte_per_lane_kernels():
+    W, H, V = sym.W, sym.H, sym.V
+
+    @kernel(work_shape=(W, sympy.ceiling(H / V)), literals=[V])
+    def vcopy(gr: CurrentGroup, src: Buffer[W, H, DT], dst: Buffer[W, H, DT], v: V):
+        x, y = gr.work_offset
+        gr.store(dst[x:, y * V:], gr.vload(src[x:, y * V:], shape=(gr.shape[0], gr.shape[1] * V)))
+
+    a = np.arange(256 * 1024, dtype=np.int32).reshape(256, 1024)
+    db = rt.to_device(np.zeros_like(a))
+    vcopy(rt.to_device(a), db, 4)
+    assert rt.last_kernel_name() == "hcamd_copy_flat_v4_nt"      # one 16-byte word per lane and step
+    assert_array_equal(db.to_host(), a)
+
+    N = sym.N
+
+    @kernel(work_shape=N, group_shape=256)
+    def vadd(gr: CurrentGroup, x: Buffer[N, DT], y: Buffer[N, DT], z: Buffer[N, DT]):
+        o = gr.work_offset[0]
+        gr.store(z[o:], gr.vload(x[o:], shape=256) + gr.vload(y[o:], shape=256))
+
+    x, y = cf.inputs_c1(100_003)
+    dz = rt.DeviceArray(x.shape, np.float32)
+    vadd(rt.to_device(x), rt.to_device(y), dz)
+    assert rt.last_kernel_name() == "hcamd_add_f32_v4_nt"
+    assert_array_equal(dz.to_host().view(np.uint32), cf.np_add(x, y).view(np.uint32))
+
+
+def test_thread_variant_selects_the_kernel_for_this_thread_only():
+    import threading
+    ab, bb = cf.inputs_c5((256, 256, 256))
+    da, dbt = rt.to_device(ab, bf16=True), rt.to_device(bb, bf16=True)
+    dc = rt.DeviceArray((256, 256), np.uint16, bf16=True)
+    plan = rt.plan_gemm_bf16(da, dbt, dc)
+    names = {}
+
+    def launch(tag, variant):
+        if variant is not None:
+            rt.set_thread_variant("gemm", variant)
+        plan.launch(sync=True)
+        names[tag] = rt.last_kernel_name()
+        if variant is not None:
+            rt.set_thread_variant("gemm", -1)
+
+    rt.set_thread_variant("gemm", 14)
+    t = threading.Thread(target=launch, args=("other", None))
+    t.start()
+    t.join()
+    launch("mine", None)                       # still under this thread's override
+    rt.set_thread_variant("gemm", -1)
+    launch("after", None)
+    assert names["other"] == "hcamd_gemm_bf16_p256x256_w2x4"
+    assert names["mine"] == "hcamd_gemm_bf16_p256x256_w2x4_direct"
+    assert names["after"] == "hcamd_gemm_bf16_p256x256_w2x4"

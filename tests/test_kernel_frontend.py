@@ -1297,3 +1297,93 @@ def test_workitem_scope_binds_ids_and_elementwise_statements(ctx):
 
     with pytest.raises(NoNativeKernel, match="wi.global_id"):
         shifted.plan(x, z, ctx=ctx)
+
+
+def test_vload_needs_a_static_shape(ctx):
+    """docs/langref.md:226-243 of the reference: a vector's shape must be known at
+    compile time.  Numbers, group.shape, literal symbols and tunables are;
+    buffer dimensions and ordinary scalar arguments are not."""
+    W, H, V, T, S = sym.W, sym.H, sym.V, sym.T, sym.S
+    a, b = FakeDev((64, 1024), "int32"), FakeDev((64, 1024), "int32")
+
+    @kernel(work_shape=(W, sympy.ceiling(H / V)), literals=[V])
+    def literal(gr: CurrentGroup, src: Buffer[W, H, DT], dst: Buffer[W, H, DT], v: V):
+        x, y = gr.work_offset
+        gr.store(dst[x:, y * V:], gr.vload(src[x:, y * V:], shape=(gr.shape[0], gr.shape[1] * V)))
+
+    (p,) = literal.plan(a, b, 4, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchCopy2D
+
+    @kernel(work_shape=W, group_shape=1, tunables=TunableParam(T, 1024, [512, 1024]))
+    def tunable(gr: CurrentGroup, src: Buffer[W, H, DT], dst: Buffer[W, H, DT]):
+        x = gr.work_offset[0]
+        gr.store(dst[x:, :], gr.vload(src[x:, :], shape=(1, T)))
+
+    (p,) = tunable.plan(a, b, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchCopy2D
+
+    @kernel(work_shape=W, group_shape=1)
+    def from_buffer_dim(gr: CurrentGroup, src: Buffer[W, H, DT], dst: Buffer[W, H, DT]):
+        x = gr.work_offset[0]
+        gr.store(dst[x:, :], gr.vload(src[x:, :], shape=(1, H)))
+
+    @kernel(work_shape=W, group_shape=1)
+    def from_shape_attr(gr: CurrentGroup, src: Buffer[W, H, DT], dst: Buffer[W, H, DT]):
+        x = gr.work_offset[0]
+        gr.store(dst[x:, :], gr.vload(src[x:, :], shape=(1, src.shape[1] // 2 * 2)))
+
+    @kernel(work_shape=W, group_shape=1)
+    def from_scalar(gr: CurrentGroup, src: Buffer[W, H, DT], dst: Buffer[W, H, DT], n: S):
+        x = gr.work_offset[0]
+        gr.store(dst[x:, :], gr.vload(src[x:, :], shape=(1, n)))
+
+    for k, extra in ((from_buffer_dim, ()), (from_shape_attr, ()), (from_scalar, (1024,))):
+        with pytest.raises(NoNativeKernel, match="static shape"):
+            k.plan(a, b, *extra, ctx=ctx)
+
+    # the same bodies with load are fine
+    @kernel(work_shape=W, group_shape=1)
+    def with_load(gr: CurrentGroup, src: Buffer[W, H, DT], dst: Buffer[W, H, DT]):
+        x = gr.work_offset[0]
+        gr.store(dst[x:, :], gr.load(src[x:, :], shape=(1, H)))
+
+    (p,) = with_load.plan(a, b, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchCopy2D
+
+
+def test_traced_arrays_are_not_kept_alive_by_the_cache(ctx):
+    import gc
+    import weakref
+    N = sym.N
+
+    @kernel(work_shape=N, group_shape=256)
+    def k(gr: CurrentGroup, src: Buffer[N, DT], dst: Buffer[N, DT]):
+        o = gr.work_offset[0]
+        gr.store(dst[o:], gr.load(src[o:], shape=gr.shape[0]))
+
+    a, b = FakeDev((1024,), "float32"), FakeDev((1024,), "float32")
+    k.plan(a, b, ctx=ctx)
+    ra = weakref.ref(a)
+    del a, b
+    gc.collect()
+    assert ra() is None, "the kernel's plan cache holds the arrays of the call that was traced"
+
+
+def test_thread_variants_are_private_to_the_thread():
+    import threading
+    with pytest.raises(rt.HcRuntimeError):
+        rt.set_thread_variant("no_such_family", 1)
+    rt.set_thread_variant("gemm", 14)
+    seen = {}
+
+    def other():
+        # another thread neither sees the override nor disturbs it
+        rt.set_thread_variant("gemm", 7)
+        rt.set_thread_variant("gemm", -1)
+        seen["ok"] = True
+
+    t = threading.Thread(target=other)
+    t.start()
+    t.join()
+    assert seen["ok"]
+    rt.set_thread_variant("gemm", -1)
