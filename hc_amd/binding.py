@@ -844,6 +844,116 @@ def match_map(dst_view, value, n_groups):
 _ROW_REDUCE = {"sum": "sum", "max": "max", "min": "min"}
 
 
+# ---------------------------------------------------------------------------
+# Integer tiles: elementwise expressions over int32 loads -> hcamdLaunchIMap
+# ---------------------------------------------------------------------------
+_IMAP_BINARY = {"add": "add", "sub": "sub", "mul": "mul", "floordiv": "floordiv", "mod": "mod",
+                "minimum": "min", "maximum": "max", "and": "and", "or": "or", "xor": "xor",
+                "shl": "shl", "shr": "shr", "lt": "lt", "le": "le", "eq": "eq", "ne": "ne",
+                "ge": "ge", "gt": "gt"}
+_IMAP_UNARY = {"neg": "neg", "abs": "abs"}
+
+
+def match_imap(dst_view, value, n_groups):
+    """An expression of int32 loads of one window, int32 constants and the
+    integer operators, stored to an int32 (or, for a comparison, bool) buffer."""
+    out_dt = dst_view.base.dtype_name
+    if out_dt not in ("int32", "bool"):
+        return None
+    loads, program = [], []
+
+    def const_of(t):
+        v = t.attrs.get("exact")
+        if v is None and t.op == "full":
+            v = t.args[0].attrs.get("exact")
+            if v is None and float(t.attrs["value"]).is_integer():
+                v = int(t.attrs["value"])
+        if v is None or not -2 ** 31 <= v < 2 ** 31:
+            raise NoNativeKernel(f"constant {t.attrs.get('value')} is not an int32")
+        return int(v)
+
+    mirrored = {"add": "add", "mul": "mul", "min": "min", "max": "max", "and": "and", "or": "or",
+                "xor": "xor", "eq": "eq", "ne": "ne", "lt": "gt", "gt": "lt", "le": "ge", "ge": "le"}
+    needs = {}
+
+    def need(t):
+        """Stack entries the evaluation of t takes (Sethi-Ullman numbers; an
+        operation whose operands may be exchanged evaluates the deeper one first)."""
+        if id(t) in needs:
+            return needs[id(t)]
+        if _is(t, "astype", 1) or (t.op in _IMAP_UNARY and len(t.args) == 1):
+            n = need(t.args[0])
+        elif t.op in _IMAP_BINARY and len(t.args) == 2:
+            a, b = need(t.args[0]), need(t.args[1])
+            if _IMAP_BINARY[t.op] in mirrored:
+                n = max(a, b) if a != b else a + 1
+            else:
+                n = max(a, b + 1)
+        else:
+            n = 1
+        needs[id(t)] = n
+        return n
+
+    def emit(t):
+        """Appends the code for t; returns False if t is not an int32 expression."""
+        if _is(t, "load"):
+            if t.dtype_name != "int32":
+                return False
+            for i, u in enumerate(loads):
+                if _same(u, t):
+                    program.append(("in", i, 0))
+                    return True
+            if len(loads) == 4:
+                raise NoNativeKernel("integer expressions read at most four arrays")
+            loads.append(t)
+            program.append(("in", len(loads) - 1, 0))
+            return True
+        if _const(t):
+            program.append(("const", 0, const_of(t)))
+            return True
+        if t.op in _IMAP_UNARY and len(t.args) == 1:
+            ok = emit(t.args[0])
+            program.append((_IMAP_UNARY[t.op], 0, 0))
+            return ok
+        if t.op in _IMAP_BINARY and len(t.args) == 2:
+            a, b = t.args
+            if t.attrs.get("operand_dtype", t.dtype_name) != "int32":
+                return False
+            op = _IMAP_BINARY[t.op]
+            if op in mirrored and need(b) > need(a):
+                a, b, op = b, a, mirrored[op]
+            ok = emit(a) and emit(b)
+            program.append((op, 0, 0))
+            return ok
+        if _is(t, "astype", 1) and t.dtype_name == "int32" and t.args[0].dtype_name == "bool":
+            return emit(t.args[0])                 # 0 / 1 as int32: the same bits
+        return False
+
+    is_cmp = value.dtype_name == "bool"
+    if value.dtype_name not in ("int32", "bool") or (out_dt == "bool") != is_cmp and out_dt == "bool":
+        return None
+    if not emit(value) or not loads:
+        return None
+    if need(value) > 4:
+        raise NoNativeKernel("integer expression too deep for the four-entry stack")
+    if len(program) > 32:
+        raise NoNativeKernel(f"integer expression too long ({len(program)} operations, at most 32)")
+    if _is(value, "load"):
+        return None                                # a plain copy
+    wins = [window_of(t.attrs["view"], t.shape, n_groups) for t in loads]
+    wins.append(window_of(dst_view, value.shape, n_groups))
+    w = _check_same_window(wins)
+    if len(w.extent) > 2:
+        raise NoNativeKernel("only 1-D and 2-D buffers have native kernels")
+    prog = list(program)
+
+    def make(mem, ctx):
+        arrays = [_Arr(_sub(mem[x.buffer], w.extent), ctx) for x in wins]
+        return [rt.plan_imap(prog, arrays[:-1], arrays[-1], out_bool=out_dt == "bool")]
+    make.program = prog
+    return make
+
+
 class _RowCompiler(_MapCompiler):
     """Splits an expression over (rows, N) tiles that contains reductions along
     axis 1 into the stages of hcamdLaunchRowProgram.
@@ -1780,7 +1890,7 @@ def bind(stores, n_groups, atomics=(), mapped_stores=(), id_stores=(), group_sha
         if q is not None:
             return makers + [q]
         for view, value in stores:
-            for matcher in (match_copy, match_add, match_fma, match_softmax, match_gemm,
+            for matcher in (match_copy, match_imap, match_add, match_fma, match_softmax, match_gemm,
                             match_gather_gemm, match_pairwise, match_cols, match_cols_tile, match_rows,
                             match_map):
                 mk = matcher(view, value, n_groups)

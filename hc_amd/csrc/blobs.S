@@ -18,6 +18,7 @@ hcamd_blob_\name\()_end:
         hcamd_blob copy
         hcamd_blob elementwise
         hcamd_blob map
+        hcamd_blob imap
         hcamd_blob distance
         hcamd_blob gather
         hcamd_blob softmax

@@ -140,6 +140,7 @@ Device::~Device() {
 HCAMD_BLOB(copy)
 HCAMD_BLOB(elementwise)
 HCAMD_BLOB(map)
+HCAMD_BLOB(imap)
 HCAMD_BLOB(distance)
 HCAMD_BLOB(gather)
 HCAMD_BLOB(softmax)
@@ -154,7 +155,7 @@ struct Blob {
 };
 #define HCAMD_BLOB(n) {#n, hcamd_blob_##n##_begin, hcamd_blob_##n##_end}
 const Blob kBlobs[] = {HCAMD_BLOB(copy), HCAMD_BLOB(elementwise),
-                       HCAMD_BLOB(map), HCAMD_BLOB(distance),
+                       HCAMD_BLOB(map), HCAMD_BLOB(imap), HCAMD_BLOB(distance),
                        HCAMD_BLOB(gather), HCAMD_BLOB(softmax),
                        HCAMD_BLOB(quantize), HCAMD_BLOB(gemm)};
 #undef HCAMD_BLOB
@@ -1346,6 +1347,123 @@ int hcamdLaunchMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
                    size_t cols) noexcept {
   return launchMap(q, false, prog, nInstr, inputs, inputTypes, inputLd, nInputs,
                    out, outType, ldo, rows, cols);
+}
+
+namespace {
+struct IMapInstr {
+  uint16_t op, arg;
+  int32_t imm;
+};
+struct IMapArgs {
+  const void *in[4];
+  void *out;
+  size_t ld[4];
+  size_t ldo, rows, cols;
+  uint32_t out_u8, vec, n_instr;
+  IMapInstr prog[32];
+};
+} // namespace
+
+int hcamdLaunchIMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
+                    const void *const *inputs, const size_t *inputLd, size_t nInputs,
+                    void *out, int outType, size_t ldo, size_t rows, size_t cols) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  const char *who = "hcamdLaunchIMap";
+  if (!prog || nInstr == 0 || nInstr > 32) {
+    dev->report("%s: program of %zu instructions (1..32)", who, nInstr);
+    return 1;
+  }
+  if (nInputs > 4 || (nInputs && (!inputs || !inputLd)) || !out) {
+    dev->report("%s: %zu operands (0..4) or a null pointer", who, nInputs);
+    return 1;
+  }
+  if (outType != HCAMD_I32 && outType != HCAMD_U8) {
+    dev->report("%s: unsupported output type %d", who, outType);
+    return 1;
+  }
+  IMapArgs a{};
+  int sp = 0;
+  for (size_t i = 0; i < nInstr; ++i) {
+    const unsigned op = prog[i].op;
+    if (op == HCAMD_IMAP_END || op >= HCAMD_IMAP_COUNT) {
+      dev->report("%s: bad opcode %u at %zu", who, op, i);
+      return 1;
+    }
+    if (op == HCAMD_IMAP_IN && prog[i].arg >= nInputs) {
+      dev->report("%s: operand %u at %zu (only %zu given)", who, prog[i].arg, i, nInputs);
+      return 1;
+    }
+    const bool push = op == HCAMD_IMAP_IN || op == HCAMD_IMAP_CONST;
+    const bool unary = op >= HCAMD_IMAP_NEG;
+    if (sp < (push ? 0 : unary ? 1 : 2)) {
+      dev->report("%s: stack underflow at %zu", who, i);
+      return 1;
+    }
+    sp += push ? 1 : unary ? 0 : -1;
+    if (sp > 4) {
+      dev->report("%s: stack deeper than 4 at %zu", who, i);
+      return 1;
+    }
+    a.prog[i].op = prog[i].op;
+    a.prog[i].arg = prog[i].arg;
+    std::memcpy(&a.prog[i].imm, &prog[i].imm, sizeof(int32_t));
+  }
+  if (sp != 1) {
+    dev->report("%s: program leaves %d values, expected 1", who, sp);
+    return 1;
+  }
+  if (rows == 0 || cols == 0)
+    return 0;
+  if (rows > 65535 && cols > 1) {
+    dev->report("%s: more than 65535 rows", who);
+    return 1;
+  }
+  if (rows > 65535) { // a column vector: walk it as one row when it is dense
+    bool dense = ldo == 1;
+    for (size_t i = 0; i < nInputs; ++i)
+      dense = dense && inputLd[i] == 1;
+    if (!dense) {
+      dev->report("%s: more than 65535 rows", who);
+      return 1;
+    }
+    cols = rows;
+    rows = 1;
+  }
+  bool vec = outType == HCAMD_I32 && aligned16(out) && (rows == 1 || ldo % 4 == 0);
+  for (size_t i = 0; i < nInputs; ++i) {
+    if (!inputs[i]) {
+      dev->report("%s: null pointer", who);
+      return 1;
+    }
+    if (rows > 1 && inputLd[i] < cols) {
+      dev->report("%s: leading dimension smaller than cols", who);
+      return 1;
+    }
+    a.in[i] = inputs[i];
+    a.ld[i] = inputLd[i];
+    vec = vec && aligned16(inputs[i]) && (rows == 1 || inputLd[i] % 4 == 0);
+  }
+  if (rows > 1 && ldo < cols) {
+    dev->report("%s: leading dimension smaller than cols", who);
+    return 1;
+  }
+  a.out = out;
+  a.ldo = ldo;
+  a.rows = rows;
+  a.cols = cols;
+  a.out_u8 = outType == HCAMD_U8 ? 1u : 0u;
+  a.vec = vec ? 1u : 0u;
+  a.n_instr = (uint32_t)nInstr;
+  Kernel *k = builtinKernel(dev, "imap", "hcamd_imap_i32");
+  if (!k)
+    return 1;
+  void *args[] = {&a};
+  const size_t grid[3] = {ceilDiv(ceilDiv(cols, (size_t)4), (size_t)256), rows, 1};
+  const size_t block[3] = {256, 1, 1};
+  return launch(queue, k, grid, block, args, 0);
 }
 
 int hcamdLaunchMapSum(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,

@@ -624,7 +624,11 @@ def _as_view(x) -> BufferView:
 # ---------------------------------------------------------------------------
 # Tiles: nodes of the traced expression DAG
 # ---------------------------------------------------------------------------
-_UFUNC_OPS = {"add": "add", "subtract": "sub", "multiply": "mul", "true_divide": "div",
+_UFUNC_OPS = {"floor_divide": "floordiv", "remainder": "mod", "mod": "mod", "bitwise_and": "and",
+              "bitwise_or": "or", "bitwise_xor": "xor", "left_shift": "shl", "right_shift": "shr",
+              "less": "lt", "less_equal": "le", "greater": "gt", "greater_equal": "ge",
+              "equal": "eq", "not_equal": "ne",
+              "add": "add", "subtract": "sub", "multiply": "mul", "true_divide": "div",
               "divide": "div", "exp": "exp", "absolute": "abs", "fabs": "abs", "rint": "rint",
               "negative": "neg", "maximum": "maximum", "minimum": "minimum", "sqrt": "sqrt",
               "log": "log", "tanh": "tanh", "square": "square", "power": "power"}
@@ -671,12 +675,15 @@ class Tile:
     def wrap(x, like: "Tile | None" = None) -> "Tile":
         if isinstance(x, Tile):
             return x
+        if isinstance(x, np.ndarray) and x.ndim == 0:
+            x = x[()]                       # a NumPy scalar that went through a ufunc call
         if isinstance(x, (bool, int, float, np.generic)):
             if isinstance(x, np.generic):
                 dt, weak = x.dtype.name, False
             else:
                 dt, weak = ("float64" if isinstance(x, float) else "int64"), True
-            return Tile("const", (), (), dt, value=float(x), weak=weak)
+            return Tile("const", (), (), dt, value=float(x), weak=weak,
+                        exact=int(x) if isinstance(x, (bool, int, np.integer)) else None)
         raise TraceError(f"cannot use {type(x).__name__} in a tile expression")
 
     def _binary(self, other, op, reflected=False):
@@ -695,6 +702,51 @@ class Tile:
     def __neg__(self): return Tile("neg", (self,), self.shape, self.dtype_name)
     def __abs__(self): return Tile("abs", (self,), self.shape, self.dtype_name)
 
+    # The rest of the operators the reference's wrapper forwards to NumPy
+    # (python/hckernel/kernel_api.py:157-180).  Comparisons give bool tiles;
+    # // % & | ^ << >> keep the operands' type.  Which of them have a native
+    # kernel is the binder's business (today: all of them on int32 tiles).
+    def __floordiv__(self, o): return self._binary(o, "floordiv")
+    def __rfloordiv__(self, o): return self._binary(o, "floordiv", True)
+    def __mod__(self, o): return self._binary(o, "mod")
+    def __rmod__(self, o): return self._binary(o, "mod", True)
+    def __and__(self, o): return self._binary(o, "and")
+    def __rand__(self, o): return self._binary(o, "and", True)
+    def __or__(self, o): return self._binary(o, "or")
+    def __ror__(self, o): return self._binary(o, "or", True)
+    def __xor__(self, o): return self._binary(o, "xor")
+    def __rxor__(self, o): return self._binary(o, "xor", True)
+    def __lshift__(self, o): return self._binary(o, "shl")
+    def __rlshift__(self, o): return self._binary(o, "shl", True)
+    def __rshift__(self, o): return self._binary(o, "shr")
+    def __rrshift__(self, o): return self._binary(o, "shr", True)
+
+    def _compare(self, other, op):
+        o = Tile.wrap(other)
+        return Tile(op, (self, o), _broadcast(self.shape, o.shape), "bool",
+                    operand_dtype=_result_dtype(self, o))
+
+    def __lt__(self, o): return self._compare(o, "lt")
+    def __le__(self, o): return self._compare(o, "le")
+    def __gt__(self, o): return self._compare(o, "gt")
+    def __ge__(self, o): return self._compare(o, "ge")
+    def __eq__(self, o): return self._compare(o, "eq")
+    def __ne__(self, o): return self._compare(o, "ne")
+    __hash__ = object.__hash__
+
+    def __invert__(self):
+        raise TraceError("~tile: the reference's tile type has no __invert__ either (its wrapper "
+                         "installs __inv__, which Python never calls)")
+
+    @property
+    def mask(self):
+        raise TraceError("tile.mask: which elements are active depends on the data (division by "
+                         "zero) and on the group; it is not available while the body is traced")
+
+    def compressed(self):
+        raise TraceError("tile.compressed(): the number of active elements is not known while the "
+                         "body is traced")
+
     def __matmul__(self, o):
         return _dot(self, Tile.wrap(o))
 
@@ -711,6 +763,9 @@ class Tile:
         a, b = inputs
         if op == "power":
             return Tile.wrap(a) ** b
+        if op in ("lt", "le", "gt", "ge", "eq", "ne"):
+            a, b = Tile.wrap(a), Tile.wrap(b)
+            return a._compare(b, op)
         if isinstance(a, Tile):
             return a._binary(b, op)
         return Tile.wrap(b)._binary(a, op, reflected=True)

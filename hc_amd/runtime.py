@@ -119,6 +119,8 @@ hcamdLaunchPairwiseDistF32 = _sig(_rt, "hcamdLaunchPairwiseDistF32", _int, _vp, 
 hcamdLaunchMapSum = _sig(_rt, "hcamdLaunchMapSum", _int, _vp, C.POINTER(MapInstr), _sz,
                          C.POINTER(_vp), C.POINTER(_int), _sz_p, _sz, _vp, _sz, _sz)
 
+hcamdLaunchIMap = _sig(_rt, "hcamdLaunchIMap", _int, _vp, C.POINTER(MapInstr), _sz, C.POINTER(_vp),
+                       _sz_p, _sz, _vp, _int, _sz, _sz, _sz)
 hcamdMapReduceColsWorkspace = _sig(_rt, "hcamdMapReduceColsWorkspace", _sz, _sz, _sz)
 hcamdLaunchMapReduceCols = _sig(_rt, "hcamdLaunchMapReduceCols", _int, _vp, _int,
                                 C.POINTER(MapInstr), _sz, C.POINTER(MapInstr), _sz,
@@ -264,7 +266,7 @@ def as_memref(obj, rank: int | None = None) -> Memref:
 
 _TYPESTR = {"float32": "<f4", "float16": "<f2", "int8": "|i1", "uint8": "|u1",
             "int16": "<i2", "uint16": "<u2", "int32": "<i4", "uint32": "<u4",
-            "int64": "<i8", "uint64": "<u8", "float64": "<f8"}
+            "int64": "<i8", "uint64": "<u8", "float64": "<f8", "bool": "|b1"}
 
 
 class DeviceArray:
@@ -585,6 +587,43 @@ def plan_map_sum(program, inputs, cell, index: int = 0, types=None) -> Plan:
     return Plan(ctx, hcamdLaunchMapSum,
                 (ctx.queue, prog, len(program), ptrs, tys, lds, n_in, mc.ptr + 4 * index,
                  rows, cols), "hcamdLaunchMapSum", (arrays, cell, prog, ptrs, tys, lds))
+
+
+U8 = 5
+IMAP_OPS = {"in": 1, "const": 2, "add": 3, "sub": 4, "mul": 5, "floordiv": 6, "mod": 7, "min": 8,
+            "max": 9, "and": 10, "or": 11, "xor": 12, "shl": 13, "shr": 14, "lt": 15, "le": 16,
+            "eq": 17, "ne": 18, "ge": 19, "gt": 20, "neg": 21, "abs": 22, "not": 23, "lnot": 24}
+
+
+def plan_imap(program, inputs, out, out_bool=False) -> Plan:
+    """out = f(inputs...) over int32 windows (see hcamdLaunchIMap).  `program` is
+    a postfix list of (opname, arg, int immediate); `out` is an int32 array, or
+    with out_bool a one-byte-per-element array that receives 0 / 1."""
+    inputs = list(inputs)
+    ctx = _ctx_of(*inputs, out)
+    mo = as_memref(out)
+    _expect(mo, 1 if out_bool else 4, "imap output")
+    rows, cols, ldo = _rows_cols(mo)
+    ms = []
+    for x in inputs:
+        m = as_memref(x)
+        _expect(m, 4, "imap operand")
+        r, c, _ = _rows_cols(m)
+        if (r, c) != (rows, cols):
+            raise HcRuntimeError("imap: shape mismatch")
+        ms.append(m)
+    n_in = len(ms)
+    prog = (MapInstr * max(len(program), 1))()
+    for i, (name, arg, imm) in enumerate(program):
+        prog[i].op, prog[i].arg = IMAP_OPS[name], int(arg)
+        # the float field carries the int32 bit pattern
+        C.memmove(C.addressof(prog[i]) + MapInstr.imm.offset,
+                  C.byref(C.c_int32(((int(imm) + 2 ** 31) % 2 ** 32) - 2 ** 31)), 4)
+    ptrs = (_vp * max(n_in, 1))(*[m.ptr for m in ms])
+    lds = (_sz * max(n_in, 1))(*[_rows_cols(m)[2] for m in ms])
+    return Plan(ctx, hcamdLaunchIMap,
+                (ctx.queue, prog, len(program), ptrs, lds, n_in, mo.ptr, U8 if out_bool else I32,
+                 ldo, rows, cols), "hcamdLaunchIMap", (inputs, out, prog, ptrs, lds))
 
 
 COLS_KINDS = {"sum": 0, "max": 1, "min": 2}

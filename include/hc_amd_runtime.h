@@ -283,7 +283,8 @@ int hcamdLaunchFmaF16(OlQueue q, const void *a, size_t lda, const void *b,
  * nearest even.  Operands are fp32 or fp16, each with its own leading
  * dimension in elements.  The program is validated on the host; a malformed
  * one is an error, not a launch. */
-enum HcamdElemType { HCAMD_F32 = 0, HCAMD_F16 = 1, HCAMD_BF16 = 2, HCAMD_I32 = 3, HCAMD_I64 = 4 };
+enum HcamdElemType { HCAMD_F32 = 0, HCAMD_F16 = 1, HCAMD_BF16 = 2, HCAMD_I32 = 3, HCAMD_I64 = 4,
+                     HCAMD_U8 = 5 };
 enum HcamdMapOp {
   HCAMD_MAP_END = 0,
   HCAMD_MAP_IN = 1,    /* push operand `arg` */
@@ -334,6 +335,31 @@ int hcamdLaunchMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
                    const size_t *inputLd, size_t nInputs, void *out,
                    int outType, size_t ldo, size_t rows,
                    size_t cols) HCAMD_NOEXCEPT;
+
+/* The integer sibling of hcamdLaunchMap: out = f(in_0 .. in_{n-1}) over a
+ * rows x cols window of int32 operands, f a postfix program of HCAMD_IMAP_*
+ * instructions on a four-entry stack (HcamdMapInstr with `imm` carrying the bit
+ * pattern of an int32 constant).  These are the integer operators the
+ * reference's tile wrapper forwards to NumPy
+ * (python/hckernel/kernel_api.py:157-211) with NumPy's int32 semantics: + - *
+ * wrap around, // and % are floor division and its remainder, << and >> with a
+ * count outside 0..31 give 0 (-1 for >> of a negative value), comparisons give
+ * 0 / 1.  An element that was divided by zero is inactive, as numpy.ma makes
+ * it: nothing is stored for it.  outType is HCAMD_I32, or HCAMD_U8 for a
+ * result of 0 / 1 stored as one byte (a bool buffer). */
+enum HcamdIMapOp {
+  HCAMD_IMAP_END = 0, HCAMD_IMAP_IN = 1, HCAMD_IMAP_CONST = 2,
+  HCAMD_IMAP_ADD = 3, HCAMD_IMAP_SUB = 4, HCAMD_IMAP_MUL = 5, HCAMD_IMAP_FLOORDIV = 6,
+  HCAMD_IMAP_MOD = 7, HCAMD_IMAP_MIN = 8, HCAMD_IMAP_MAX = 9, HCAMD_IMAP_AND = 10,
+  HCAMD_IMAP_OR = 11, HCAMD_IMAP_XOR = 12, HCAMD_IMAP_SHL = 13, HCAMD_IMAP_SHR = 14,
+  HCAMD_IMAP_LT = 15, HCAMD_IMAP_LE = 16, HCAMD_IMAP_EQ = 17, HCAMD_IMAP_NE = 18,
+  HCAMD_IMAP_GE = 19, HCAMD_IMAP_GT = 20,
+  HCAMD_IMAP_NEG = 21, HCAMD_IMAP_ABS = 22, HCAMD_IMAP_NOT = 23, HCAMD_IMAP_LNOT = 24,
+  HCAMD_IMAP_COUNT = 25
+};
+int hcamdLaunchIMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
+                    const void *const *inputs, const size_t *inputLd, size_t nInputs,
+                    void *out, int outType, size_t ldo, size_t rows, size_t cols) HCAMD_NOEXCEPT;
 
 /* Map-reduce: *cell += sum over the window of f(in_0 .. in_{n-1}), fp32, with
  * one hardware atomic add per workgroup.  This is the reference's reduction

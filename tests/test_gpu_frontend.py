@@ -956,3 +956,108 @@ def test_thread_variant_selects_the_kernel_for_this_thread_only():
     assert names["other"] == "hcamd_gemm_bf16_p256x256_w2x4"
     assert names["mine"] == "hcamd_gemm_bf16_p256x256_w2x4_direct"
     assert names["after"] == "hcamd_gemm_bf16_p256x256_w2x4"
+
+
+# ---------------------------------------------------------------------------
+# Integer tiles (python/hckernel/kernel_api.py:157-211 on int32 data)
+# ---------------------------------------------------------------------------
+_I32 = np.int32
+_INT_BIN = {
+    "add": lambda a, b: a + b, "sub": lambda a, b: a - b, "mul": lambda a, b: a * b,
+    "floordiv": lambda a, b: a // (b | _I32(1)), "mod": lambda a, b: a % (b | _I32(1)),
+    "min": lambda a, b: np.minimum(a, b), "max": lambda a, b: np.maximum(a, b),
+    "and": lambda a, b: a & b, "or": lambda a, b: a | b, "xor": lambda a, b: a ^ b,
+    "shl": lambda a, b: a << (b & _I32(31)), "shr": lambda a, b: a >> (b & _I32(31)),
+    "lt": lambda a, b: (a < b) * _I32(3), "ge": lambda a, b: (a >= b) * a, "ne": lambda a, b: (a != b) * b,
+}
+
+
+def _random_int_tree(rng, depth):
+    """A function tiles -> tile and its description."""
+    if depth == 0 or rng.random() < 0.2:
+        if rng.random() < 0.75:
+            i = int(rng.integers(0, 3))
+            return (lambda t, i=i: t[i]), f"t{i}"
+        c = _I32(rng.integers(-50, 51))
+        return (lambda t, c=c: c), str(int(c))
+    if rng.random() < 0.15:
+        f, d = _random_int_tree(rng, depth - 1)
+        if rng.random() < 0.5:
+            return (lambda t: -f(t)), f"-({d})"
+        return (lambda t: abs(f(t))), f"abs({d})"
+    name = list(_INT_BIN)[int(rng.integers(0, len(_INT_BIN)))]
+    fa, da = _random_int_tree(rng, depth - 1)
+    fb, db = _random_int_tree(rng, depth - 1)
+    op = _INT_BIN[name]
+    return (lambda t: op(fa(t), fb(t))), f"{name}({da}, {db})"
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_int32_expression_trees_equal_the_host_executor(seed):
+    rng = np.random.default_rng(1000 + seed)
+    R, Cc = sym.R, sym.C
+    while True:
+        f, desc = _random_int_tree(rng, 3)
+        if "t" in desc and desc not in ("t0", "t1", "t2"):
+            break
+
+    def body(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT], c: Buffer[R, Cc, DT],
+             out: Buffer[R, Cc, DT]):
+        x, y = gr.work_offset
+        tiles = [gr.load(v[x:, y:], shape=gr.shape) for v in (a, b, c)]
+        value = f(tiles)
+        if not hasattr(value, "shape") or value.shape == ():        # the tree folded to a constant
+            value = tiles[0] * _I32(0) + value
+        gr.store(out[x:, y:], value)
+
+    shape = [(37, 130), (64, 256), (5, 1031)][seed % 3]
+    big = seed % 4 == 0
+    ins = [rng.integers(-2 ** 31 if big else -1000, 2 ** 31 if big else 1000, shape).astype(np.int32)
+           for _ in range(3)]
+    host = np.full(shape, -777, np.int32)
+    dout = rt.to_device(host)
+    try:
+        kernel(work_shape=(R, Cc), group_shape=(4, 64))(body)(*[rt.to_device(v) for v in ins], dout)
+    except NoNativeKernel as e:
+        if "too deep" in str(e) or "too long" in str(e):
+            pytest.skip(f"{desc}: {e}")
+        raise
+    with np.errstate(all="ignore"):
+        sim_kernel(work_shape=(R, Cc), group_shape=(4, 64))(body)(*ins, host)
+    assert_array_equal(dout.to_host(), host, err_msg=desc)
+
+
+def test_int32_division_by_zero_deactivates_the_element_and_shift_counts():
+    """numpy.ma masks x // 0 and x % 0, and everything computed from them: the
+    store leaves those elements alone.  Shift counts outside 0..31 follow NumPy."""
+    N = sym.N
+
+    def body(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], q: Buffer[N, DT], r: Buffer[N, DT],
+             s: Buffer[N, DT], flag: Buffer[N, DT]):
+        o = gr.work_offset[0]
+        ta, tb = gr.load(a[o:], shape=gr.shape[0]), gr.load(b[o:], shape=gr.shape[0])
+        gr.store(q[o:], (ta // tb) * _I32(2) + _I32(1))
+        gr.store(r[o:], ta % tb)
+        gr.store(s[o:], (ta << tb) ^ (ta >> tb))
+        gr.store(flag[o:], ta % _I32(7) == tb % _I32(7))
+
+    rng = np.random.default_rng(77)
+    n = 5000
+    a = rng.integers(-10 ** 9, 10 ** 9, n).astype(np.int32)
+    b = rng.integers(-6, 41, n).astype(np.int32)              # zeros, negatives, counts past 31
+    a[:4] = [-2 ** 31, -2 ** 31, 2 ** 31 - 1, -7]
+    b[:4] = [-1, 0, -1, 2]
+    hosts = [np.full(n, -777, np.int32) for _ in range(3)] + [np.full(n, True)]
+    hosts[3][::2] = False
+    devs = [rt.to_device(h) for h in hosts]
+    kernel(work_shape=N, group_shape=256)(body)(rt.to_device(a), rt.to_device(b), *devs)
+    with np.errstate(all="ignore"):
+        sim_kernel(work_shape=N, group_shape=256)(body)(a, b, *hosts)
+    for d, h, name in zip(devs, hosts, "qrsf"):
+        assert_array_equal(d.to_host(), h, err_msg=name)
+    zero = (b == 0) & (a != -2 ** 31)
+    assert zero.sum() > 50 and (hosts[0][zero] == -777).all() and (hosts[1][zero] == -777).all()
+    assert (hosts[0][b != 0] != -777).any()
+    # numpy.ma's own corner: |INT_MIN| overflows in its divisor test, so INT_MIN // 0 stays
+    # active with NumPy's quotient 0 (element 1 of the inputs)
+    assert (a[1], b[1]) == (-2 ** 31, 0) and hosts[0][1] == 1 and hosts[1][1] == 0

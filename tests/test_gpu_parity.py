@@ -223,6 +223,82 @@ def test_copy_large_flat_all_variants(ctx):
 
 
 # ---------------------------------------------------------------------------
+# integer map (hcamdLaunchIMap)
+# ---------------------------------------------------------------------------
+def _np_floor_shift(op, a, b):
+    a64, b64 = a.astype(np.int64), b.astype(np.int64)
+    if op == "shl":
+        return np.where((b64 >= 0) & (b64 < 32), (a64 << np.clip(b64, 0, 31)), 0).astype(np.int64) \
+            .astype(np.uint64).astype(np.uint32).view(np.int32)
+    return np.where((b64 >= 0) & (b64 < 32), a64 >> np.clip(b64, 0, 31), np.where(a64 < 0, -1, 0)) \
+        .astype(np.int32)
+
+
+@pytest.mark.parametrize("shape,pad,off", [((1, 5000), 0, 0), ((37, 130), 6, 0), ((16, 256), 0, 0),
+                                           ((9, 33), 3, 1)])
+def test_imap_every_operation_against_numpy(ctx, shape, pad, off):
+    """One program per opcode, int32 wrap-around semantics, aligned (16-byte) and
+    unaligned / padded windows, poison outside the window."""
+    rng = np.random.default_rng(shape[1])
+    rows, cols = shape
+    ld = cols + pad
+    a = rng.integers(-2 ** 31, 2 ** 31, (rows, cols)).astype(np.int32)
+    b = rng.integers(-40, 41, (rows, cols)).astype(np.int32)
+    b[b == 0] = 7
+    a[0, :3] = [-2 ** 31, 2 ** 31 - 1, -1]
+
+    def padded(x):
+        buf = np.full(rows * ld + off + 4, 0x0BADBEEF, np.int32)
+        buf[off:off + rows * ld].reshape(rows, ld)[:, :cols] = x
+        return dev(buf)
+    da, dbb = padded(a), padded(b)
+    wrap = lambda v: (v & 0xFFFFFFFF).astype(np.uint32).view(np.int32)
+    a64, b64 = a.astype(np.int64), b.astype(np.int64)
+    cases = {"add": wrap(a64 + b64), "sub": wrap(a64 - b64), "mul": wrap(a64 * b64),
+             "floordiv": wrap(a64 // b64), "mod": (a64 % b64).astype(np.int32),
+             "min": np.minimum(a, b), "max": np.maximum(a, b), "and": a & b, "or": a | b, "xor": a ^ b,
+             "shl": _np_floor_shift("shl", a, b), "shr": _np_floor_shift("shr", a, b),
+             "lt": (a < b).astype(np.int32), "le": (a <= b).astype(np.int32),
+             "eq": (a == b).astype(np.int32), "ne": (a != b).astype(np.int32),
+             "ge": (a >= b).astype(np.int32), "gt": (a > b).astype(np.int32)}
+    view = lambda d: _View(d, (rows, cols), off, (ld, 1))
+    for name, want in cases.items():
+        out = poisoned((rows * ld + off + 4,), np.int32)
+        rt.plan_imap([I("in", 0), I("in", 1), I(name)], [view(da), view(dbb)], view(out)).launch(sync=True)
+        got = out.to_host()
+        win = got[off:off + rows * ld].reshape(rows, ld)
+        assert_array_equal(win[:, :cols], want, err_msg=name)
+        assert (win[:, cols:].view(np.uint32) == POISON32).all(), name
+        assert (got[:off].view(np.uint32) == POISON32).all() and (got[off + rows * ld:].view(np.uint32) == POISON32).all()
+    for name, want in {"neg": wrap(-a64), "abs": wrap(np.abs(a64)), "not": ~a,
+                       "lnot": (a == 0).astype(np.int32)}.items():
+        out = poisoned((rows * ld + off + 4,), np.int32)
+        rt.plan_imap([I("in", 0), I(name)], [view(da)], view(out)).launch(sync=True)
+        assert_array_equal(out.to_host()[off:off + rows * ld].reshape(rows, ld)[:, :cols], want, err_msg=name)
+    # a constant, and a 0 / 1 result into a one-byte buffer
+    flags = poisoned((rows, cols), np.uint8)
+    rt.plan_imap([I("in", 0), ("const", 0, -5), I("gt")], [view(da)], flags, out_bool=True).launch(sync=True)
+    assert_array_equal(flags.to_host(), (a > -5).astype(np.uint8))
+
+
+def test_imap_zero_divisors_are_left_alone_and_bad_programs_refused(ctx):
+    a = np.arange(-8, 8, dtype=np.int32)
+    b = np.array([0, 1, 2, 0] * 4, np.int32)
+    out = poisoned((16,), np.int32)
+    rt.plan_imap([I("in", 0), I("in", 1), I("floordiv"), ("const", 0, 100), I("add")],
+                 [dev(a), dev(b)], out).launch(sync=True)
+    got = out.to_host()
+    assert (got[b == 0].view(np.uint32) == POISON32).all()
+    assert_array_equal(got[b != 0], a[b != 0] // b[b != 0] + 100)
+    x = dev(a)
+    for prog, msg in (([I("in", 0), I("in", 0)], "leaves 2 values"), ([I("add")], "underflow"),
+                      ([I("in", 1)], "operand 1"),
+                      ([I("in", 0)] * 5 + [I("add")] * 4, "deeper than 4")):
+        with pytest.raises(rt.HcRuntimeError, match=msg):
+            rt.plan_imap(prog, [x], out).launch(sync=True)
+
+
+# ---------------------------------------------------------------------------
 # stream calibration kernels (the yardstick of the memory-bound kernels)
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("n_reads,write", [(1, "full"), (2, "full"), (3, "full"), (0, "full"),

@@ -15,7 +15,8 @@ from hc_amd.kernel import (Buffer, CurrentGroup, NoNativeKernel, TunableParam, a
 from oracle import closed_forms as cf
 
 DT = typename.DT
-CODES = {"float32": "<f4", "float16": "<f2", "int8": "|i1", "int32": "<i4", "bfloat16": "<u2"}
+CODES = {"float32": "<f4", "float16": "<f2", "int8": "|i1", "int32": "<i4", "bfloat16": "<u2",
+         "bool": "|b1"}
 
 
 class FakeDev:
@@ -121,8 +122,69 @@ def test_vector_add_binds_to_add_f32(ctx):
     (p3,) = vadd.plan(*(FakeDev((n,), "float16") for _ in range(3)), ctx=ctx)
     assert p3.fn is rt.hcamdLaunchMap
     assert map_program(p3) == [("in", 0, 0.0), ("add_in", 1, 0.0), ("r16", 0, 0.0)]
+    # int32 arrays: the integer map kernel
+    (p4,) = vadd.plan(*(FakeDev((n,), "int32") for _ in range(3)), ctx=ctx)
+    assert p4.fn is rt.hcamdLaunchIMap and imap_program(p4) == [("in", 0, 0), ("in", 1, 0), ("add", 0, 0)]
     with pytest.raises(NoNativeKernel):
-        vadd.plan(*(FakeDev((n,), "int32") for _ in range(3)), ctx=ctx)
+        vadd.plan(*(FakeDev((n,), "int8") for _ in range(3)), ctx=ctx)
+
+
+def imap_program(plan):
+    """(opname, arg, int immediate) triples of a hcamdLaunchIMap plan."""
+    import ctypes as C
+    names = {v: k for k, v in rt.IMAP_OPS.items()}
+    prog, n = plan.args[1], plan.args[2]
+    out = []
+    for i in range(n):
+        imm = C.c_int32.from_buffer_copy(bytes(C.string_at(C.addressof(prog[i]) + rt.MapInstr.imm.offset, 4)))
+        out.append((names[prog[i].op], prog[i].arg, imm.value))
+    return out
+
+
+def test_integer_tile_operators_bind_to_the_integer_map(ctx):
+    """The operators the reference's tile wrapper forwards for integer tiles
+    (python/hckernel/kernel_api.py:157-180): arithmetic, floor division and
+    remainder, bitwise, shifts, comparisons."""
+    R, Cc = sym.R, sym.C
+    i32 = np.int32
+
+    @kernel(work_shape=(R, Cc), group_shape=(4, 64))
+    def k(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT], out: Buffer[R, Cc, DT],
+          flag: Buffer[R, Cc, DT]):
+        x, y = gr.work_offset
+        ta, tb = gr.load(a[x:, y:], shape=gr.shape), gr.load(b[x:, y:], shape=gr.shape)
+        gr.store(out[x:, y:], ((ta * tb - i32(7)) // (tb | i32(1))) % i32(13) + (ta >> i32(2) ^ tb << i32(3)))
+        gr.store(flag[x:, y:], np.minimum(ta, tb) <= -abs(tb) & i32(255))
+
+    a, b, out = (FakeDev((37, 130), "int32") for _ in range(3))
+    flag = FakeDev((37, 130), "bool")
+    p1, p2 = k.plan(a, b, out, flag, ctx=ctx)
+    assert p1.fn is rt.hcamdLaunchIMap and p2.fn is rt.hcamdLaunchIMap
+    assert imap_program(p1) == [
+        ("in", 0, 0), ("in", 1, 0), ("mul", 0, 0), ("const", 0, 7), ("sub", 0, 0),
+        ("in", 1, 0), ("const", 0, 1), ("or", 0, 0), ("floordiv", 0, 0), ("const", 0, 13),
+        ("mod", 0, 0), ("in", 0, 0), ("const", 0, 2), ("shr", 0, 0), ("in", 1, 0), ("const", 0, 3),
+        ("shl", 0, 0), ("xor", 0, 0), ("add", 0, 0)]
+    assert p1.args[7] == rt.I32 and p1.args[9:11] == (37, 130)
+    assert imap_program(p2) == [("in", 0, 0), ("in", 1, 0), ("min", 0, 0), ("in", 1, 0), ("abs", 0, 0),
+                                ("neg", 0, 0), ("const", 0, 255), ("and", 0, 0), ("le", 0, 0)]
+    assert p2.args[7] == rt.U8
+
+    # what has no native form says so
+    @kernel(work_shape=(R, Cc), group_shape=(4, 64))
+    def truediv(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT], out: Buffer[R, Cc, DT]):
+        x, y = gr.work_offset
+        gr.store(out[x:, y:], gr.load(a[x:, y:], shape=gr.shape) / gr.load(b[x:, y:], shape=gr.shape))
+
+    @kernel(work_shape=(R, Cc), group_shape=(4, 64))
+    def uses_mask(gr: CurrentGroup, a: Buffer[R, Cc, DT], out: Buffer[R, Cc, DT]):
+        x, y = gr.work_offset
+        gr.store(out[x:, y:], gr.load(a[x:, y:], shape=gr.shape).mask)
+
+    with pytest.raises(NoNativeKernel):
+        truediv.plan(a, b, out, ctx=ctx)
+    with pytest.raises(NoNativeKernel, match="mask"):
+        uses_mask.plan(a, out, ctx=ctx)
 
 
 def map_program(plan):
