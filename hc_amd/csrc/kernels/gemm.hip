@@ -259,7 +259,7 @@ __device__ __forceinline__ Acc mfma_block(V b, V a, Acc c) {
 // barriers, which times the matrix cores alone on real operand data (its
 // output is not the product).
 template <class E, int BM, int BN, int WM, int WN, int MF, bool EDGE = false, int EPI = 0,
-          bool PRIO = false, int PROBE = 0>
+          bool PRIO = false, int PROBE = 0, int STAGE = 0, int RS = 0, int LF = 1, int LS = 2>
 __device__ __forceinline__ void gemm_tile_pipelined(
     const E *__restrict__ A, size_t lda, const E *__restrict__ Bt, size_t ldb,
     E *__restrict__ C, size_t ldc, int M, int N, int K) {
@@ -314,11 +314,124 @@ __device__ __forceinline__ void gemm_tile_pipelined(
     const int row = EDGE ? min(tn * BN + r, N - 1) : tn * BN + r;
     b_src[i] = Bt + (size_t)row * ldb + ((ld_pchunk ^ swz<SH>(r)) * 8);
   }
+  // Whole-tile builds address the panels through buffer descriptors: the lane's
+  // part of the address (its row among the eight of a wave-level load, its
+  // swizzled chunk) is one 32-bit register per panel for the whole kernel, and
+  // what changes from load to load and from K tile to K tile is a scalar
+  // offset, so the loop spends no vector instruction on addresses (the 64-bit
+  // pointer form needs two per load, sixteen per K tile, on the port the MFMAs
+  // issue through).  Offsets stay below 2^31: the host checks 256 * ld * 2.
+  constexpr bool BUF = !EDGE;
+  u32x4 probe_sink = {0u, 0u, 0u, 0u};
+  __amdgpu_buffer_rsrc_t a_rsrc, b_rsrc;
+  int a_voff = 0, b_voff = 0;
+  if constexpr (BUF) {
+    a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<E *>(A + (size_t)tm * BM * lda), 0, (int)(((size_t)(BM - 1) * lda + K) * sizeof(E)),
+        0x00020000);
+    b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<E *>(Bt + (size_t)tn * BN * ldb), 0, (int)(((size_t)(BN - 1) * ldb + K) * sizeof(E)),
+        0x00020000);
+    const int chunk = ld_pchunk ^ swz<SH>(ld_row); // rows advance in eights: the swizzle is the lane's
+    a_voff = (int)((ld_row * lda + chunk * 8) * sizeof(E));
+    b_voff = (int)((ld_row * ldb + chunk * 8) * sizeof(E));
+  }
+  const int a_step = (int)(kWaves * 8 * lda * sizeof(E)), b_step = (int)(kWaves * 8 * ldb * sizeof(E));
+  const int a_first = (int)(wave * 8 * lda * sizeof(E)), b_first = (int)(wave * 8 * ldb * sizeof(E));
   // logical chunk the lane fetches in load i (the swizzle depends on the row)
   auto chunk_of = [&](int i) { return ld_pchunk ^ swz<SH>((i * kWaves + wave) * 8 + ld_row); };
+  // STAGE: bit 0 sends the A panel, bit 1 the B panel through registers (a
+  // buffer load into a register quad, a 16-byte LDS write half a K tile later)
+  // instead of the load that writes LDS by itself.
+  constexpr bool kStageA = BUF && (STAGE & 1), kStageB = BUF && (STAGE & 2);
+  constexpr int kStaged = (kStageA ? kALoads : 0) + (kStageB ? kBLoads : 0);
+  constexpr int kDirect = kALoads + kBLoads - kStaged;
+  u32x4 stage_a[kALoads], stage_b[kBLoads];
+  auto write_staged = [&](int buf) {
+    unsigned char *base = lds + buf * kStageBytes + wave * 1024 + lane * 16;
+#pragma unroll
+    for (int i = 0; i < kALoads; ++i)
+      if constexpr (kStageA)
+        *reinterpret_cast<u32x4 *>(base + i * kWaves * 1024) = stage_a[i];
+#pragma unroll
+    for (int i = 0; i < kBLoads; ++i)
+      if constexpr (kStageB)
+        *reinterpret_cast<u32x4 *>(base + kABytes + i * kWaves * 1024) = stage_b[i];
+  };
+  bool in_loop = false;  // PROBE 7 only
   auto issue_loads = [&](int kt, int buf) {
     const size_t k0 = (size_t)kt * kBK;
     unsigned char *base = lds + buf * kStageBytes + wave * 1024;
+    if constexpr (BUF && PROBE == 7) {
+      // measurement build: inside the loop the A panel goes to LDS as always,
+      // the B operand blocks are fetched in the layout the MFMA takes them
+      // (sixteen rows of 64 bytes per load) into a register that nothing reads
+      if (in_loop) {
+        const int kbytes = (int)(k0 * sizeof(E));
+#pragma unroll
+        for (int i = 0; i < kALoads; ++i)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr)(base + i * kWaves * 1024), 16,
+                                                   a_voff, a_first + i * a_step + kbytes, 0, 0);
+        const uint64_t p = reinterpret_cast<uint64_t>(Bt + (size_t)tn * BN * ldb);
+        const u32x4 rb = {(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu,
+                          (uint32_t)(((size_t)(BN - 1) * ldb + K) * sizeof(E)), 0x00020000u};
+        const int voff = (int)(((lane % 16) * ldb + (lane / 16) * 8) * sizeof(E));
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int j = 0; j < kNI; ++j) {
+            const int so = (int)((wave_n + j * 16) * ldb * sizeof(E)) + h * 64 + kbytes;
+            asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(probe_sink) : "v"(voff), "s"(rb), "s"(so));
+          }
+        return;
+      }
+    }
+    if constexpr (BUF && PROBE == 6) {
+      // measurement build: the same fetches into a register instead of LDS
+      const int kbytes = (int)(k0 * sizeof(E));
+      auto desc = [](const void *base, size_t bytes) {
+        const uint64_t p = reinterpret_cast<uint64_t>(base);
+        return u32x4{(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, (uint32_t)bytes, 0x00020000u};
+      };
+      const u32x4 ra = desc(A + (size_t)tm * BM * lda, ((size_t)(BM - 1) * lda + K) * sizeof(E));
+      const u32x4 rb = desc(Bt + (size_t)tn * BN * ldb, ((size_t)(BN - 1) * ldb + K) * sizeof(E));
+#pragma unroll
+      for (int i = 0; i < kALoads; ++i) {
+        const int so = a_first + i * a_step + kbytes;
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(probe_sink) : "v"(a_voff), "s"(ra), "s"(so));
+      }
+#pragma unroll
+      for (int i = 0; i < kBLoads; ++i) {
+        const int so = b_first + i * b_step + kbytes;
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(probe_sink) : "v"(b_voff), "s"(rb), "s"(so));
+      }
+      return;
+    }
+    if constexpr (BUF) {
+      const int kbytes = (int)(k0 * sizeof(E));
+      // panels that pass through registers first: their loads are the oldest
+      // of the tile, so a wait that leaves the direct ones out covers them
+#pragma unroll
+      for (int i = 0; i < kALoads; ++i)
+        if constexpr (kStageA)
+          stage_a[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_voff, a_first + i * a_step + kbytes, 0);
+#pragma unroll
+      for (int i = 0; i < kBLoads; ++i)
+        if constexpr (kStageB)
+          stage_b[i] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_voff, b_first + i * b_step + kbytes, 0);
+#pragma unroll
+      for (int i = 0; i < kALoads; ++i)
+        if constexpr (!kStageA)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr)(base + i * kWaves * 1024), 16,
+                                                   a_voff, a_first + i * a_step + kbytes, 0, 0);
+#pragma unroll
+      for (int i = 0; i < kBLoads; ++i)
+        if constexpr (!kStageB)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc,
+                                                   (lds_ptr)(base + kABytes + i * kWaves * 1024), 16,
+                                                   b_voff, b_first + i * b_step + kbytes, 0, 0);
+      return;
+    }
     const bool tail = EDGE && kt == KT - 1 && tail_chunks < 8;
 #pragma unroll
     for (int i = 0; i < kALoads; ++i) {
@@ -337,6 +450,19 @@ __device__ __forceinline__ void gemm_tile_pipelined(
       __builtin_amdgcn_global_load_lds(
           (global_cptr)src, (lds_ptr)(base + kABytes + i * kWaves * 1024), 16, 0,
           0);
+    }
+  };
+  // one wave-level load of K tile kt (A panel first, then B), whole-tile builds
+  auto load_one = [&](int kt, int buf, int v) {
+    if constexpr (BUF) {
+      unsigned char *base = lds + buf * kStageBytes + wave * 1024;
+      const int kbytes = (int)((size_t)kt * kBK * sizeof(E));
+      if (v < kALoads)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr)(base + v * kWaves * 1024), 16, a_voff,
+                                                 a_first + v * a_step + kbytes, 0, 0);
+      else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (lds_ptr)(base + kABytes + (v - kALoads) * kWaves * 1024),
+                                                 16, b_voff, b_first + (v - kALoads) * b_step + kbytes, 0, 0);
     }
   };
   // EDGE: after the last K tile has landed, the chunks past K become zeros
@@ -382,7 +508,8 @@ __device__ __forceinline__ void gemm_tile_pipelined(
       const unsigned char *base = lds + buf * kStageBytes + (ks ? coff[1][u] : coff[0][u]);
 #pragma unroll
       for (int j = 0; j < kNI; ++j)
-        fb[S][u][j] = *reinterpret_cast<const ex8 *>(base + b_off[j]);
+        if (!(PROBE == 7 && in_loop))
+          fb[S][u][j] = *reinterpret_cast<const ex8 *>(base + b_off[j]);
 #pragma unroll
       for (int i = 0; i < kMI; ++i)
         fa[S][u][i] = *reinterpret_cast<const ex8 *>(base + a_off[i]);
@@ -410,47 +537,136 @@ __device__ __forceinline__ void gemm_tile_pipelined(
   };
   using Slot0 = std::integral_constant<int, 0>;
   using Slot1 = std::integral_constant<int, 1>;
+  // RS builds write the order of a half-step out by hand, one fenced slot per
+  // MFMA: LDS read r of the next half-step's operands goes before MFMA
+  // r * S / kReads (S = number of MFMAs the reads are spread over), the loads
+  // of K tile kt before the odd MFMAs from the second on.  Fragments are read
+  // in the order the MFMAs take them (Bt blocks, then A blocks), so the waits
+  // the compiler puts in front of each MFMA are for its own operands only.
+  auto half_step = [&](auto use, auto fill, auto spread, auto rfirst, auto lfirst, int rbuf, int rks, bool do_read,
+                       bool do_load, int kt, int lbuf) {
+    constexpr int U = decltype(use)::value;
+    constexpr int F = decltype(fill)::value;
+    constexpr int S = decltype(spread)::value;
+    constexpr int RF = decltype(rfirst)::value;
+    constexpr int LFv = decltype(lfirst)::value;
+    static_assert(kSub == 1, "written for the 16 x 16 x 32 blocks");
+    static_assert(LFv + (kALoads + kBLoads - 1) * LS < kMfma, "every load has its MFMA");
+    static_assert(RF + (kReads - 1) * S / kReads < kMfma, "every LDS read has its MFMA");
+    const unsigned char *rbase = lds + rbuf * kStageBytes + (rks ? coff[1][0] : coff[0][0]);
+#pragma unroll
+    for (int i = 0; i < kMI; ++i)
+#pragma unroll
+      for (int j = 0; j < kNI; ++j) {
+        const int slot = i * kNI + j;
+        if (do_read) {
+#pragma unroll
+          for (int r = 0; r < kReads; ++r)
+            if (RF + r * S / kReads == slot) {
+              if (r < kNI)
+                fb[F][0][r] = *reinterpret_cast<const ex8 *>(rbase + b_off[r]);
+              else
+                fa[F][0][r - kNI] = *reinterpret_cast<const ex8 *>(rbase + a_off[r - kNI]);
+            }
+        }
+        if (do_load && slot >= LFv && (slot - LFv) % LS == 0 && (slot - LFv) / LS < kALoads + kBLoads)
+          load_one(kt, lbuf, (slot - LFv) / LS);
+        acc[i][j] = mfma_block<E, MF>(fb[U][0][j], fa[U][0][i], acc[i][j]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+  };
 
   // Order inside a half-step: one LDS read per MFMA from the start, so the last
   // read is out after kReads MFMAs and has the rest of the sequence to land;
   // the global->LDS loads follow, one per MFMA.
-  auto interleave = [&](auto vmem) {
+  auto interleave = [&](auto vmem, auto dswrites, auto spread) {
     constexpr int V = decltype(vmem)::value;
+    constexpr int D = decltype(dswrites)::value;
+    constexpr int S = decltype(spread)::value;
 #pragma unroll
     for (int i = 0; i < kMfma; ++i) {
-      constexpr int kVFirst = kMfma >= kReads + V ? kReads : 0;
-      if (i < kReads)
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
-      if (i >= kVFirst && i - kVFirst < V)
-        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // VMEM read
+      if constexpr (S == 0) {
+        constexpr int kVFirst = kMfma >= kReads + V + D ? kReads : 0;
+        if (i < kReads)
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
+        if (i >= kVFirst && i - kVFirst < V)
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // VMEM read
+        if (i >= kVFirst + V && i - kVFirst - V < D)
+          __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // DS write
+      } else {
+        // LDS reads evenly over the first S MFMAs (read r before MFMA
+        // r * S / kReads), the loads before the odd MFMAs from the second on
+#pragma unroll
+        for (int r = 0; r < kReads; ++r)
+          if (r * S / kReads == i)
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if (i % 2 == 1 && i / 2 < V)
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        if (i % 2 == 0 && i / 2 < D)
+          __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+      }
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
     }
   };
   using NoVmem = std::integral_constant<int, 0>;
-  using WithVmem = std::integral_constant<int, kALoads + kBLoads>;
+  using WithVmem = std::integral_constant<int, PROBE == 7 ? kALoads + 2 * kNI : kALoads + kBLoads>;
+  using NoWrites = std::integral_constant<int, 0>;
+  using WithWrites = std::integral_constant<int, kStaged>;
+  // reads of the even half-step are the last of their buffer and have to be
+  // back before the barrier: they stop a quarter of the MFMAs earlier
+  using SpreadEven = std::integral_constant<int, RS == 0 ? 0 : (RS < kMfma * 3 / 4 ? RS : kMfma * 3 / 4)>;
+  using SpreadOdd = std::integral_constant<int, RS>;
 
   issue_loads(0, 0);
-  issue_loads(1, 1);
-  __builtin_amdgcn_s_waitcnt(waitcnt_imm(kALoads + kBLoads, kNoLgkm));
+  if constexpr (kStaged != 0) {
+    write_staged(0);  // the compiler waits for the registers
+    issue_loads(1, 1);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(kALoads + kBLoads, 0));
+  } else {
+    issue_loads(1, 1);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(kALoads + kBLoads, kNoLgkm));
+  }
   __builtin_amdgcn_s_barrier();
   read_frags(0, 0, Slot0{});
 
   auto tile_step = [&](int t, auto load_next2, auto read_next) {
     constexpr bool LOAD = decltype(load_next2)::value;
     constexpr bool READ = decltype(read_next)::value;
+    using RFirst = std::integral_constant<int, 0>;
+    using LFirst = std::integral_constant<int, LF>;
+    static_assert(RS == 0 || kStaged == 0, "the hand-ordered half-steps have no register-staged panels");
     // the step before the last: the last tile has landed at its barrier
     constexpr bool ZERO = EDGE && !LOAD && READ;
     const int buf = t & 1;
+    if constexpr (RS != 0) {
+      // every read was out a quarter of a half-step ago or earlier
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoVm, 0));
+      __builtin_amdgcn_sched_barrier(0);
+      half_step(Slot0{}, Slot1{}, SpreadEven{}, RFirst{}, LFirst{}, buf, 1, true, false, 0, 0);
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      half_step(Slot1{}, Slot0{}, SpreadOdd{}, RFirst{}, LFirst{}, buf ^ 1, 0, READ, LOAD, t + 2, buf);
+      return;
+    }
     // even half-step: consume slot 0 (requested a whole half-step ago, so the
     // wait is free and makes the later waits exact), fetch slot 1
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoVm, 0));
+    if constexpr (RS == 0)
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoVm, 0));
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (PROBE != 4)
       read_frags(buf, 1, Slot1{});
     if constexpr (PRIO)
       __builtin_amdgcn_s_setprio(1);
+    // staged panels of tile t + 1 (requested a K tile ago) go to the buffer
+    // that the barrier of the previous step released
+    if constexpr (READ && kStaged != 0)
+      write_staged(buf ^ 1);
     mma(Slot0{});
-    interleave(NoVmem{});
+    if constexpr (READ)
+      interleave(NoVmem{}, WithWrites{}, SpreadEven{});
+    else
+      interleave(NoVmem{}, NoWrites{}, SpreadEven{});
     if constexpr (PRIO)
       __builtin_amdgcn_s_setprio(0);
     // odd half-step; the fences keep the MFMAs above on this side of the wait
@@ -474,13 +690,17 @@ __device__ __forceinline__ void gemm_tile_pipelined(
       __builtin_amdgcn_s_setprio(1);
     mma(Slot1{});
     if constexpr (LOAD && READ)
-      interleave(WithVmem{});
+      interleave(WithVmem{}, NoWrites{}, SpreadOdd{});
     else if constexpr (READ)
-      interleave(NoVmem{});
+      interleave(NoVmem{}, NoWrites{}, SpreadOdd{});
     if constexpr (PRIO)
       __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
   };
+  if constexpr (PROBE == 7) {
+    read_frags(0, 1, Slot1{});
+    in_loop = true;
+  }
   if constexpr (PROBE == 1) {
     read_frags(0, 1, Slot1{});
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
@@ -498,6 +718,10 @@ __device__ __forceinline__ void gemm_tile_pipelined(
     tile_step(t + 1, std::false_type{}, std::false_type{});
   }
 
+  if constexpr (PROBE == 6 || PROBE == 7) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("" ::"v"(probe_sink));
+  }
   // ---- epilogue ------------------------------------------------------------------
   if constexpr (EPI != 0 && !EDGE && MF == 16) {
     // Through LDS: the wave's kWaveM x kWaveN tile as rows of kWaveN elements,
@@ -588,20 +812,38 @@ __device__ __forceinline__ void gemm_tile_pipelined(
     gemm_tile_pipelined<E, BM, BN, WM, WN, MF, false, EPI, PRIO, PROBE>(       \
         A, lda, Bt, ldb, C, ldc, M, N, K);                                     \
   }
-// the default whole-tile kernels: LDS-staged epilogue with non-temporal stores
-HCAMD_GEMM_PX(hcamd_gemm_bf16_p256x256_w2x4, __bf16, 256, 256, 2, 4, 16, 2, false, 0)
-HCAMD_GEMM_PX(hcamd_gemm_bf16_p128x128_w2x2, __bf16, 128, 128, 2, 2, 16, 2, false, 0)
-HCAMD_GEMM_PX(hcamd_gemm_f16_p256x256_w2x4, _Float16, 256, 256, 2, 4, 16, 2, false, 0)
-HCAMD_GEMM_PX(hcamd_gemm_f16_p128x128_w2x2, _Float16, 128, 128, 2, 2, 16, 2, false, 0)
-// the same main loop with the other epilogues / wave priorities, for measurement
+#define HCAMD_GEMM_PS(NAME, E, BM, BN, WM, WN, MF, STAGE, RS, LF, LS)          \
+  extern "C" __global__ __launch_bounds__(WM *WN * 64) void NAME(              \
+      const E *A, size_t lda, const E *Bt, size_t ldb, E *C, size_t ldc,       \
+      int M, int N, int K) {                                                   \
+    gemm_tile_pipelined<E, BM, BN, WM, WN, MF, false, 2, false, 0, STAGE, RS,  \
+                        LF, LS>(A, lda, Bt, ldb, C, ldc, M, N, K);             \
+  }
+// the default whole-tile kernels: LDS-staged epilogue with non-temporal stores,
+// hand-ordered half-steps (LDS reads over the first half of the MFMAs, the loads
+// evenly over all of them)
+HCAMD_GEMM_PS(hcamd_gemm_bf16_p256x256_w2x4, __bf16, 256, 256, 2, 4, 16, 0, 16, 1, 4)
+HCAMD_GEMM_PS(hcamd_gemm_bf16_p128x128_w2x2, __bf16, 128, 128, 2, 2, 16, 0, 8, 1, 2)
+HCAMD_GEMM_PS(hcamd_gemm_f16_p256x256_w2x4, _Float16, 256, 256, 2, 4, 16, 0, 16, 1, 4)
+HCAMD_GEMM_PS(hcamd_gemm_f16_p128x128_w2x2, _Float16, 128, 128, 2, 2, 16, 0, 8, 1, 2)
+// for measurement: the order of a half-step left to the compiler under
+// sched_group_barrier hints (one LDS read per MFMA from the start, the loads
+// bunched behind them), with each epilogue / with raised priority; the loads
+// early in hand-written order; the A panel staged through registers
+HCAMD_GEMM_PX(hcamd_gemm_bf16_p256x256_w2x4_hinted, __bf16, 256, 256, 2, 4, 16, 2, false, 0)
 HCAMD_GEMM_PX(hcamd_gemm_bf16_p256x256_w2x4_direct, __bf16, 256, 256, 2, 4, 16, 0, false, 0)
 HCAMD_GEMM_PX(hcamd_gemm_bf16_p256x256_w2x4_lds, __bf16, 256, 256, 2, 4, 16, 1, false, 0)
 HCAMD_GEMM_PX(hcamd_gemm_bf16_p256x256_w2x4_prio, __bf16, 256, 256, 2, 4, 16, 2, true, 0)
+HCAMD_GEMM_PS(hcamd_gemm_bf16_p256x256_w2x4_loads_early, __bf16, 256, 256, 2, 4, 16, 0, 16, 1, 2)
+HCAMD_GEMM_PS(hcamd_gemm_bf16_p256x256_w2x4_stage_a, __bf16, 256, 256, 2, 4, 16, 1, 0, 1, 2)
+// measurement builds whose output is not the product
 HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_mfma_only, __bf16, 256, 256, 2, 4, 16, 2, false, 1)
 HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_no_vmwait, __bf16, 256, 256, 2, 4, 16, 2, false, 2)
 HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_no_barrier, __bf16, 256, 256, 2, 4, 16, 2, false, 3)
 HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_no_ldsread, __bf16, 256, 256, 2, 4, 16, 2, false, 4)
 HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_no_loads, __bf16, 256, 256, 2, 4, 16, 2, false, 5)
+HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_loads_to_regs, __bf16, 256, 256, 2, 4, 16, 2, false, 6)
+HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_b_direct, __bf16, 256, 256, 2, 4, 16, 2, false, 7)
 HCAMD_GEMM_PE(hcamd_gemm_bf16_p256x256_w2x4_edge, __bf16, 256, 256, 2, 4, 16)
 HCAMD_GEMM_PE(hcamd_gemm_f16_p256x256_w2x4_edge, _Float16, 256, 256, 2, 4, 16)
 HCAMD_GEMM_PE(hcamd_gemm_bf16_p128x128_w2x2_edge, __bf16, 128, 128, 2, 2, 16)

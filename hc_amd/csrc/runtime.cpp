@@ -2694,6 +2694,11 @@ int launchGemm(OlQueue q, bool half, const void *a, size_t lda, const void *bt,
       {"hcamd_gemm_bf16_probe_no_barrier", 256, 256, 512},
       {"hcamd_gemm_bf16_probe_no_ldsread", 256, 256, 512},
       {"hcamd_gemm_bf16_probe_no_loads", 256, 256, 512},
+      {"hcamd_gemm_bf16_probe_loads_to_regs", 256, 256, 512}, // 22
+      {"hcamd_gemm_bf16_p256x256_w2x4_stage_a", 256, 256, 512},     // 23: A panel through registers
+      {"hcamd_gemm_bf16_p256x256_w2x4_hinted", 256, 256, 512},      // 24: half-step order left to the compiler
+      {"hcamd_gemm_bf16_p256x256_w2x4_loads_early", 256, 256, 512}, // 25: loads in the first half of the MFMAs
+      {"hcamd_gemm_bf16_probe_b_direct", 256, 256, 512},            // 26: measurement only
   };
   constexpr int kGeneral = 6;
   constexpr int kFirstPipelined = 7; // variants from here need K >= 128
@@ -2731,6 +2736,18 @@ int launchGemm(OlQueue q, bool half, const void *a, size_t lda, const void *bt,
         pick = &tiled[3];
     }
   }
+  // The whole-tile pipelined kernels address their panels with 32-bit byte
+  // offsets from the tile's first row (buffer loads): rows further apart than
+  // that go to the edge-capable build, which uses 64-bit pointers.
+  if (pick && pick - tiled >= kFirstPipelined - 1 &&
+      ((size_t)(pick->bm - 1) * lda + k) * 2 >= ((size_t)1 << 31))
+    pick = nullptr;
+  if (pick && (pick == &half256 || pick == &half128 || pick - tiled >= kFirstPipelined - 1) &&
+      ((size_t)(pick->bn - 1) * ldb + k) * 2 >= ((size_t)1 << 31))
+    pick = nullptr;
+  if (pick && (pick == &half256 || pick == &half128) &&
+      ((size_t)(pick->bm - 1) * lda + k) * 2 >= ((size_t)1 << 31))
+    pick = nullptr;
   // Shapes the whole-tile kernels cannot take (M or N not a multiple of the
   // tile, K not a multiple of 64) go to the edge-capable build of the pipelined
   // kernel as long as the panels can be fetched in 16-byte pieces; only what
