@@ -689,6 +689,53 @@ _MAP_EXACT = {"neg", "abs", "maximum", "minimum", "clip"}   # fp16 in -> fp16 ou
 _MAP_FLOATS = ("float16", "float32")
 
 
+def _masks(t: Tile) -> bool:
+    """t itself can deactivate elements at run time.  The tile operators / // %
+    and ** go through numpy.ma, which deactivates failed divisions and results
+    of ** that are not finite; NumPy functions with a domain (sqrt, log, divide)
+    called on tiles deactivate where the domain fails."""
+    if t.attrs.get("func"):
+        return t.op in ("sqrt", "log", "div", "floordiv", "mod")
+    return t.op in ("div", "floordiv", "mod") or bool(t.attrs.get("pow"))
+
+
+def _maybe_masked(t: Tile, memo=None) -> bool:
+    """Some element of t may be inactive for a reason only the data knows."""
+    memo = {} if memo is None else memo
+    if t.uid not in memo:
+        if _is(t, "load") or _const(t):
+            memo[t.uid] = False
+        else:
+            memo[t.uid] = _masks(t) or any(_maybe_masked(a, memo) for a in t.args if isinstance(a, Tile))
+    return memo[t.uid]
+
+
+# Operations that compute from their operands' values and change nothing about
+# which elements are active: NumPy functions without a domain, negation, abs,
+# conversions.  (The tile operators + - * are not: numpy.ma gives the first
+# operand's value where an operand is inactive.)
+_TRANSPARENT_FUNCS = ("exp", "rint", "tanh", "maximum", "minimum", "add", "sub", "mul", "clip", "neg", "abs")
+
+
+def _values_flow_plainly(t: Tile, clean: bool = True) -> bool:
+    """Every operation that can deactivate elements has only transparent
+    operations above it: then the value stored for a deactivated element is
+    what plain arithmetic on the value numpy.ma left there gives."""
+    if _is(t, "load") or _const(t):
+        return True
+    if _masks(t) and not clean:
+        return False
+    transparent = _is(t, "astype", 1) or t.op in ("neg", "abs") or \
+        (bool(t.attrs.get("func")) and t.op in _TRANSPARENT_FUNCS)
+    return all(_values_flow_plainly(a, clean and transparent) for a in t.args if isinstance(a, Tile))
+
+
+class _NeedsEntryMasks(Exception):
+    """The expression needs activity tracked per operand and numpy.ma's values
+    under deactivated elements: the general float map has both, the fast map
+    kernel one flag per element."""
+
+
 def _round_to(value: float, dtype: str) -> float:
     import numpy as np
     return float(np.float16(value)) if dtype == "float16" else float(np.float32(value))
@@ -708,6 +755,8 @@ class _MapCompiler:
     """Sethi-Ullman ordering: the operand that needs the deeper stack is
     evaluated first, constants become immediates, so an expression with up to
     eight distinct leaves in a balanced tree fits the four-entry stack."""
+
+    masked = False                # emit numpy.ma's division rule (element-wise map and its sum only)
 
     def __init__(self, n_groups):
         self.n_groups = n_groups
@@ -757,6 +806,11 @@ class _MapCompiler:
         return n
 
     def emit(self, t: Tile, out: list):
+        self._emit_node(t, out)
+        if self.masked and t.attrs.get("pow"):
+            out.append(("powchk", 0, 0.0))
+
+    def _emit_node(self, t: Tile, out: list):
         half = t.dtype_name == "float16"
         if _is(t, "load"):
             out.append(("in", self.operand(t), 0.0))
@@ -774,33 +828,44 @@ class _MapCompiler:
             out.append(("maxi", 0, _round_to(t.attrs["lo"], t.dtype_name)))
             out.append(("mini", 0, _round_to(t.attrs["hi"], t.dtype_name)))
             return
+        mdiv = self.masked and t.op == "div"
+        if mdiv and t.attrs.get("func"):
+            raise _NeedsEntryMasks()           # numpy.divide as a function: the general map has it
         if t.op in _MAP_UNARY:
             self.emit(t.args[0], out)
-            out.append((_MAP_UNARY[t.op], 0, 0.0))
+            name = _MAP_UNARY[t.op]
+            if self.masked and t.attrs.get("func") and name in ("sqrt", "log"):
+                name = "m" + name              # numpy.sqrt / numpy.log of a tile: domain fill
+            out.append((name, 0, 0.0))
+            if self.masked and t.op == "sqrt" and t.attrs.get("pow"):
+                out.append(("addi", 0, 0.0))   # x ** 0.5 of -0 is +0 (the square root's is -0)
         else:
             fwd, rev, _ = _MAP_BINARY[t.op]
+            if mdiv:
+                fwd, rev = "mdiv", "rmdiv"
+            flag = int(half) if mdiv else 0              # the quotient is tested as fp16
             a, b = t.args
             if _const(b):
                 self.emit(a, out)
-                out.append((fwd + "i", 0, _round_to(b.attrs["value"], t.dtype_name)))
+                out.append((fwd + "i", flag, _round_to(b.attrs["value"], t.dtype_name)))
             elif _const(a):
                 self.emit(b, out)
-                out.append((rev + "i", 0, _round_to(a.attrs["value"], t.dtype_name)))
+                out.append((rev + "i", flag, _round_to(a.attrs["value"], t.dtype_name)))
             elif _leaf(b) is not None:              # operand forms: one dispatch, no push
                 self.emit(a, out)
-                out.append((fwd + "_in", self.operand(_leaf(b)), 0.0))
+                out.append((fwd + "_in", self.operand(_leaf(b)) | (flag << 8), 0.0))
             elif _leaf(a) is not None:
                 self.emit(b, out)
-                out.append((rev + "_in", self.operand(_leaf(a)), 0.0))
+                out.append((rev + "_in", self.operand(_leaf(a)) | (flag << 8), 0.0))
             elif self.need(a) >= self.need(b):
                 self.emit(a, out)
                 self.emit(b, out)
-                out.append((fwd, 0, 0.0))
+                out.append((fwd, flag, 0.0))
             else:
                 self.emit(b, out)
                 self.emit(a, out)
-                out.append((rev, 0, 0.0))
-        if half and t.op not in _MAP_EXACT:
+                out.append((rev, flag, 0.0))
+        if half and t.op not in _MAP_EXACT and not mdiv:
             out.append(("r16", 0, 0.0))
 
 
@@ -808,13 +873,25 @@ def match_map(dst_view, value, n_groups):
     if dst_view.base.dtype_name not in _MAP_FLOATS:
         return None
     comp = _MapCompiler(n_groups)
+    comp.masked = True
     if _const(value) or not comp.supported(value):
         return None
     if comp.need(value) > rt.MAP_STACK_DEPTH:
+        if _maybe_masked(value):
+            return None                    # the general float map may still take it
         raise NoNativeKernel(f"elementwise expression stored to {dst_view.base.name} needs an "
                              f"evaluation stack deeper than {rt.MAP_STACK_DEPTH}")
+    masked = _maybe_masked(value)
+    stored_in_full = bool(value.attrs.get("plain"))    # a bare numpy.ma array: every value is written
+    if masked and stored_in_full and not _values_flow_plainly(value):
+        return None                        # the general float map keeps numpy.ma's values
     program: list = []
-    comp.emit(value, program)
+    try:
+        comp.emit(value, program)
+    except _NeedsEntryMasks:
+        return None
+    if masked and stored_in_full:
+        program.append(("clear", 0, 0.0))
     if len(program) > rt.MAP_MAX_INSTRS:
         raise NoNativeKernel(f"elementwise expression stored to {dst_view.base.name} compiles to "
                              f"{len(program)} operations (at most {rt.MAP_MAX_INSTRS})")
@@ -950,6 +1027,157 @@ def match_imap(dst_view, value, n_groups):
     def make(mem, ctx):
         arrays = [_Arr(_sub(mem[x.buffer], w.extent), ctx) for x in wins]
         return [rt.plan_imap(prog, arrays[:-1], arrays[-1], out_bool=out_dt == "bool")]
+    make.program = prog
+    return make
+
+
+# ---------------------------------------------------------------------------
+# General float expressions -> hcamdLaunchFMap (numpy.ma's activity rules, // %,
+# comparisons); what the fast map kernel does not take
+# ---------------------------------------------------------------------------
+_FMAP_BINARY = {"add": "add", "sub": "sub", "mul": "mul", "div": "div", "floordiv": "floordiv",
+                "mod": "mod", "maximum": "max", "minimum": "min", "lt": "lt", "le": "le", "eq": "eq",
+                "ne": "ne", "ge": "ge", "gt": "gt"}
+_FMAP_UNARY = {"neg": "neg", "abs": "abs", "sqrt": "sqrt", "rint": "rint", "exp": "exp", "log": "log"}
+_FMAP_MIRROR = {"add": "add", "mul": "mul", "max": "max", "min": "min", "eq": "eq", "ne": "ne",
+                "lt": "gt", "gt": "lt", "le": "ge", "ge": "le"}
+_FMAP_COMPARE = ("lt", "le", "eq", "ne", "ge", "gt")
+
+
+def match_fmap(dst_view, value, n_groups):
+    """An expression of fp32 / fp16 loads of one window, constants, the tile
+    operators and NumPy functions, stored to an fp32, fp16 or (for a
+    comparison) bool buffer, with activity tracked per operand."""
+    out_dt = dst_view.base.dtype_name
+    if out_dt not in _MAP_FLOATS + ("bool",):
+        return None
+    if (value.dtype_name == "bool") != (out_dt == "bool") or \
+            (value.dtype_name != "bool" and value.dtype_name not in _MAP_FLOATS):
+        return None
+    loads, program, needs, memo = [], [], {}, {}
+
+    def fdtype(t):
+        return t.attrs.get("operand_dtype", t.dtype_name) if t.op in _FMAP_COMPARE else t.dtype_name
+
+    def need(t):
+        if t.uid in needs:
+            return needs[t.uid]
+        if _is(t, "load") or _const(t):
+            n = 1
+        elif len(t.args) == 1:
+            n = need(t.args[0])
+        elif len(t.args) == 2:
+            a, b = need(t.args[0]), need(t.args[1])
+            if _FMAP_BINARY.get(t.op) in _FMAP_MIRROR and not _maybe_masked(t, memo):
+                n = max(a, b) if a != b else a + 1
+            else:
+                n = max(a, b + 1)
+        else:
+            n = 99
+        needs[t.uid] = n
+        return n
+
+    def emit(t):
+        """Appends the code for t; False if t is not a float expression this kernel takes."""
+        half = t.dtype_name == "float16"
+        func = bool(t.attrs.get("func"))
+        if _is(t, "load"):
+            if t.dtype_name not in _MAP_FLOATS:
+                return False
+            for i, u in enumerate(loads):
+                if _same(u, t):
+                    program.append(("in", i, 0.0))
+                    return True
+            if len(loads) == 4:
+                raise NoNativeKernel("float expressions read at most four arrays")
+            loads.append(t)
+            program.append(("in", len(loads) - 1, 0.0))
+            return True
+        if _const(t):
+            return False                       # constants are pushed by the operation that uses them
+        ok = True
+        if _is(t, "astype", 1):
+            src = t.args[0]
+            if t.dtype_name not in _MAP_FLOATS or src.dtype_name not in _MAP_FLOATS + ("bool",):
+                return False
+            ok = emit(src)
+            if half and src.dtype_name == "float32":
+                program.append(("r16", 0, 0.0))
+            return ok
+        if _is(t, "clip", 1):
+            ok = emit(t.args[0])
+            program.append(("const", 0, _round_to(t.attrs["lo"], t.dtype_name)))
+            program.append(("max", int(half), 0.0))
+            program.append(("const", 0, _round_to(t.attrs["hi"], t.dtype_name)))
+            program.append(("min", int(half), 0.0))
+        elif t.op in _FMAP_UNARY and len(t.args) == 1:
+            ok = emit(t.args[0])
+            name = _FMAP_UNARY[t.op]
+            if name == "sqrt" and t.attrs.get("pow"):
+                name = "psqrt"                 # x ** 0.5; numpy.sqrt(x) has a domain instead
+            elif name in ("sqrt", "log") and not func:
+                return False
+            program.append((name, 0, 0.0))
+            if half and t.op not in _MAP_EXACT:
+                program.append(("r16", 0, 0.0))
+        elif t.op in _FMAP_BINARY and len(t.args) == 2:
+            dt = fdtype(t)
+            if dt not in _MAP_FLOATS:
+                return False
+            op = _FMAP_BINARY[t.op]
+            if func and op == "floordiv":
+                raise NoNativeKernel("numpy.floor_divide called as a function has no native code "
+                                     "(the // operator has)")
+            a, b = t.args
+            if op in _FMAP_MIRROR and not _maybe_masked(t, memo) and need(b) > need(a):
+                a, b, op = b, a, _FMAP_MIRROR[op]
+            for x in (a, b):
+                if _const(x):
+                    program.append(("const", 0, _round_to(x.attrs["value"], dt)))
+                else:
+                    ok = emit(x) and ok
+            half_op = dt == "float16"
+            if op == "div" and func:
+                program.append(("udiv", 0, 0.0))
+            elif op in ("div", "floordiv"):
+                program.append((op, int(half_op), 0.0))
+            elif op in ("add", "sub", "mul"):
+                program.append((op, 2 if func else 0, 0.0))
+            elif op in ("min", "max"):
+                program.append((op, int(half_op), 0.0))
+            else:
+                program.append((op, 0, 0.0))
+            if half_op and t.op not in _MAP_EXACT and t.op not in _FMAP_COMPARE and \
+                    not (op in ("div", "floordiv") and not func):
+                program.append(("r16", 0, 0.0))
+        else:
+            return False
+        if t.attrs.get("pow"):
+            program.append(("powchk", 0, 0.0))
+        return ok
+
+    if _is(value, "load") or _const(value):
+        return None
+    if not emit(value) or not loads:
+        return None
+    if need(value) > 4:
+        raise NoNativeKernel("float expression too deep for the four-entry stack of the general map")
+    if len(program) > rt.FMAP_MAX_INSTRS:
+        raise NoNativeKernel(f"float expression too long ({len(program)} operations, at most "
+                             f"{rt.FMAP_MAX_INSTRS})")
+    wins = [window_of(t.attrs["view"], t.shape, n_groups) for t in loads]
+    wins.append(window_of(dst_view, value.shape, n_groups))
+    w = _check_same_window(wins)
+    if len(w.extent) > 2:
+        raise NoNativeKernel("only 1-D and 2-D buffers have native kernels")
+    types = [rt.F16 if t.dtype_name == "float16" else rt.F32 for t in loads]
+    types.append({"float32": rt.F32, "float16": rt.F16, "bool": rt.U8}[out_dt])
+    prog = list(program)
+    store_all = bool(value.attrs.get("plain"))     # a bare numpy.ma array is written in full
+
+    def make(mem, ctx):
+        arrays = [_Arr(_sub(mem[x.buffer], w.extent), ctx) for x in wins]
+        return [rt.plan_fmap(prog, arrays[:-1], arrays[-1], types, store_all)]
     make.program = prog
     return make
 
@@ -1703,7 +1931,11 @@ def match_sum(proxy, index, value, n_groups):
     # sum(x + y) = sum(x) + sum(y): every term of a top-level sum gets its own
     # pass, which also covers tiles that were added up one by one
     terms: list = []
-    _flatten_sum(value.args[0], terms)
+    if _maybe_masked(value.args[0]):
+        # an element that a division deactivated in one term is skipped as a whole
+        terms.append(value.args[0])
+    else:
+        _flatten_sum(value.args[0], terms)
     terms = [t for t in terms if not _const(t, 0)]
     terms = _merge_strided_loads(terms, n_groups)
     if not terms:
@@ -1711,6 +1943,7 @@ def match_sum(proxy, index, value, n_groups):
     makers = []
     for term in terms:
         comp = _MapCompiler(n_groups)
+        comp.masked = True
         if not comp.supported(term):
             raise NoNativeKernel(f"atomic accumulation into {proxy.name}: {term!r} is not an "
                                  "elementwise expression over fp32 / fp16 loads")
@@ -1718,7 +1951,11 @@ def match_sum(proxy, index, value, n_groups):
             raise NoNativeKernel("elementwise expression needs an evaluation stack deeper than "
                                  f"{rt.MAP_STACK_DEPTH}")
         program: list = []
-        comp.emit(term, program)
+        try:
+            comp.emit(term, program)
+        except _NeedsEntryMasks:
+            raise NoNativeKernel("numpy.divide called as a function inside a sum has no native "
+                                 "code (the / operator has)") from None
         if len(program) > rt.MAP_MAX_INSTRS or len(comp.inputs) > rt.MAP_MAX_INPUTS or \
                 not comp.inputs:
             raise NoNativeKernel("elementwise expression too large for the map kernel")
@@ -1892,7 +2129,7 @@ def bind(stores, n_groups, atomics=(), mapped_stores=(), id_stores=(), group_sha
         for view, value in stores:
             for matcher in (match_copy, match_imap, match_add, match_fma, match_softmax, match_gemm,
                             match_gather_gemm, match_pairwise, match_cols, match_cols_tile, match_rows,
-                            match_map):
+                            match_map, match_fmap):
                 mk = matcher(view, value, n_groups)
                 if mk is not None:
                     makers.append(mk)

@@ -29,7 +29,7 @@ NATIVE = PKG / "_native"
 BUILD = NATIVE / "build"
 INCLUDE = PKG.parent / "include"
 
-KERNEL_MODULES = ("copy", "elementwise", "map", "imap", "distance", "gather", "softmax", "quantize", "gemm")
+KERNEL_MODULES = ("copy", "elementwise", "map", "imap", "fmap", "distance", "gather", "softmax", "quantize", "gemm")
 ARCH = "gfx950"
 
 # Packed fp32 VALU forms are kept out of every kernel.

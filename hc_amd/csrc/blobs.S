@@ -19,6 +19,7 @@ hcamd_blob_\name\()_end:
         hcamd_blob elementwise
         hcamd_blob map
         hcamd_blob imap
+        hcamd_blob fmap
         hcamd_blob distance
         hcamd_blob gather
         hcamd_blob softmax

@@ -1,0 +1,321 @@
+// General elementwise map over fp32 / fp16 tiles with numpy.ma's activity rules:
+// out[i] = f(in0[i], ..., in3[i]) for a postfix program f, the float sibling of
+// the int32 map kernel.  It exists for what the fast fp32 map kernel leaves out
+// of the operators the reference's tile wrapper forwards to numpy.ma
+// (python/hckernel/kernel_api.py:157-211) -- // and %, the six comparisons --
+// and for expressions in which the value numpy.ma leaves under a deactivated
+// element is seen again.  Every stack entry carries, per element, whether the
+// element is still active in it.  The rules are numpy.ma's (NumPy 2, float32;
+// fp16 tiles: every operation in fp32 followed by FOP_R16, which is how
+// NumPy's half loops work):
+//   * the tile operators + - * give the first operand's value where an operand
+//     is inactive; called as NumPy functions (`arg` bit 1) they compute from the
+//     values whatever their activity.
+//   * the tile operators / and // : the element becomes inactive if the divisor
+//     is zero or the result is not finite (tested in the tile's type: `arg`
+//     bit 0 = fp16), and its value becomes 0 + dividend; an active quotient has
+//     0 * dividend added (numpy.ma's way of restoring the dividend), which
+//     turns -0 into +0 unless the dividend is negative.
+//   * % is ndarray's operator and reaches numpy.ma through __array_wrap__: the
+//     remainder is computed everywhere; where the divisor is zero or the
+//     dividend infinite (and neither is NaN) the element becomes inactive with
+//     the value 1.  FOP_UDIV is numpy.divide called as a function: the same
+//     test, value 1, otherwise the plain quotient.
+//   * // and % follow NumPy's divmod: fmod, then the Python sign convention,
+//     the quotient snapped to the nearest integer, signed zeros.
+//   * numpy.sqrt / numpy.log: where the operand is inactive or outside the
+//     domain (x < 0; x <= 0) the element is inactive with the value 0 / 1.
+//     Functions without a domain (exp, abs, rint, maximum, minimum, negation)
+//     compute from the values and keep the activity.
+//   * ** : FOP_PSQRT is the square root of x ** 0.5 (the operand's value where
+//     it is inactive), FOP_POWCHK what numpy.ma.power does afterwards: a result
+//     that is not finite becomes inactive with the value 1e20.
+//   * comparisons give 0 / 1 and are false for NaN except !=.
+// The store skips inactive elements, or with store_all writes every value: a
+// NumPy function returns a bare numpy.ma array, which the reference's store
+// copies in full.
+// Four stack entries in four fixed registers per element, four consecutive
+// elements per lane (one 16-byte fp32 or 8-byte fp16 access per operand where
+// rows allow it).  This is a correctness path for HBM-bound work, not tuned.
+#include "common.h"
+
+using namespace hcamd;
+
+namespace {
+constexpr int kMaxIn = 4;
+constexpr int kMaxProg = 48;
+constexpr int kV = 4;
+
+enum : uint32_t {
+  FOP_END = 0, FOP_IN = 1, FOP_CONST = 2,
+  FOP_ADD = 3, FOP_SUB = 4, FOP_MUL = 5, FOP_DIV = 6, FOP_FLOORDIV = 7, FOP_MOD = 8,
+  FOP_MIN = 9, FOP_MAX = 10, FOP_UDIV = 11,
+  FOP_LT = 12, FOP_LE = 13, FOP_EQ = 14, FOP_NE = 15, FOP_GE = 16, FOP_GT = 17,
+  FOP_NEG = 18, FOP_ABS = 19, FOP_SQRT = 20, FOP_RINT = 21, FOP_EXP = 22, FOP_LOG = 23,
+  FOP_R16 = 24, FOP_PSQRT = 25, FOP_POWCHK = 26,
+};
+
+struct Instr {
+  uint16_t op;
+  uint16_t arg;
+  float imm;
+};
+
+struct FMapArgs {
+  const void *in[kMaxIn];
+  void *out;
+  size_t ld[kMaxIn];
+  size_t ldo;
+  size_t rows, cols;
+  uint32_t f16_mask; // bit i: operand i is fp16
+  uint32_t out_type; // 0 fp32, 1 fp16, 2 one byte of 0 / 1
+  uint32_t vec;      // every row of every operand and of the output starts 16-byte aligned
+  uint32_t store_all; // write inactive elements too
+  uint32_t n_instr;
+  Instr prog[kMaxProg];
+};
+
+__device__ __forceinline__ bool finite(float x) { return __builtin_fabsf(x) < __builtin_inff(); }
+__device__ __forceinline__ float round16(float x) {
+  _Float16 h = (_Float16)x;
+  asm volatile("" : "+v"(h));
+  return (float)h;
+}
+// NumPy's maximum / minimum: a NaN wins, and of two equal values (+0 and -0) the second
+__device__ __forceinline__ float nan_max(float a, float b) { return (a > b || a != a) ? a : b; }
+__device__ __forceinline__ float nan_min(float a, float b) { return (a < b || a != a) ? a : b; }
+
+// NumPy's divmod for b != 0: the remainder takes the divisor's sign, the
+// quotient is (a - mod) / b snapped to the nearest integer
+__device__ __forceinline__ float np_divmod(float a, float b, float &mod) {
+  mod = fmodf(a, b);
+  float div = (a - mod) / b;
+  if (mod != 0.0f) {
+    if ((b < 0.0f) != (mod < 0.0f)) {
+      mod += b;
+      div -= 1.0f;
+    }
+  } else {
+    mod = __builtin_copysignf(0.0f, b);
+  }
+  float fl;
+  if (div != 0.0f) {
+    fl = __builtin_floorf(div);
+    if (div - fl > 0.5f)
+      fl += 1.0f;
+  } else {
+    fl = __builtin_copysignf(0.0f, a / b);
+  }
+  return fl;
+}
+__device__ __forceinline__ float np_floor_divide(float a, float b) {
+  if (b == 0.0f)
+    return a / b;
+  float mod;
+  return np_divmod(a, b, mod);
+}
+__device__ __forceinline__ float np_remainder(float a, float b) {
+  if (b == 0.0f)
+    return fmodf(a, b);
+  float mod;
+  (void)np_divmod(a, b, mod);
+  return mod;
+}
+
+// numpy.ma's test for a division: the divisor is zero or the dividend
+// infinite, and neither is NaN (|a| * tiny >= |b| in float64)
+__device__ __forceinline__ bool unsafe_divide(float a, float b) {
+  return a == a && b == b && (b == 0.0f || __builtin_fabsf(a) == __builtin_inff());
+}
+
+// one binary operation; ok comes in as "active in both operands"
+__device__ __forceinline__ float binary(uint32_t op, float a, float b, uint32_t arg, bool &ok) {
+  const bool half = arg & 1u, as_function = arg & 2u;
+  switch (op) {
+  case FOP_ADD: return (ok || as_function) ? a + b : a;
+  case FOP_SUB: return (ok || as_function) ? a - b : a;
+  case FOP_MUL: return (ok || as_function) ? a * b : a;
+  case FOP_DIV:
+  case FOP_FLOORDIV: {
+    float r = op == FOP_DIV ? a / b : np_floor_divide(a, b);
+    if (half)
+      r = round16(r);
+    if (!ok || b == 0.0f || !finite(r)) {
+      ok = false;
+      return 0.0f + a;
+    }
+    return r + 0.0f * a;
+  }
+  case FOP_MOD:
+  case FOP_UDIV:
+    if (unsafe_divide(a, b)) {
+      ok = false;
+      return 1.0f;
+    }
+    return op == FOP_MOD ? np_remainder(a, b) : a / b;
+  // NumPy's half loops keep the first of two equal values, its float loops the second
+  case FOP_MIN: return half ? ((a <= b || a != a) ? a : b) : nan_min(a, b);
+  case FOP_MAX: return half ? ((a >= b || a != a) ? a : b) : nan_max(a, b);
+  case FOP_LT: return a < b ? 1.0f : 0.0f;
+  case FOP_LE: return a <= b ? 1.0f : 0.0f;
+  case FOP_EQ: return a == b ? 1.0f : 0.0f;
+  case FOP_NE: return a != b ? 1.0f : 0.0f;
+  case FOP_GE: return a >= b ? 1.0f : 0.0f;
+  default: return a > b ? 1.0f : 0.0f; // FOP_GT
+  }
+}
+__device__ __forceinline__ float unary(uint32_t op, float a, bool &ok) {
+  switch (op) {
+  case FOP_NEG: return -a;
+  case FOP_ABS: return __builtin_fabsf(a);
+  case FOP_SQRT:
+    if (!ok || a < 0.0f) {
+      ok = false;
+      return 0.0f;
+    }
+    return __builtin_sqrtf(a);
+  case FOP_LOG:
+    if (!ok || a <= 0.0f) {
+      ok = false;
+      return 1.0f;
+    }
+    return logf(a);
+  case FOP_RINT: return __builtin_rintf(a);
+  case FOP_EXP: return expf(a);
+  case FOP_R16: return round16(a);
+  case FOP_PSQRT: return ok ? __builtin_sqrtf(a) + 0.0f : a; // pow(-0, 0.5) is +0
+  default: // FOP_POWCHK
+    if (!finite(a)) {
+      ok = false;
+      return 1e20f;
+    }
+    return a;
+  }
+}
+} // namespace
+
+extern "C" __global__ __launch_bounds__(256) void hcamd_fmap(FMapArgs a) {
+  const size_t row = blockIdx.y;
+  const size_t col0 = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * kV;
+  if (col0 >= a.cols)
+    return;
+  const bool whole = col0 + kV <= a.cols;
+  float v[kMaxIn][kV];
+#pragma unroll
+  for (int i = 0; i < kMaxIn; ++i) {
+    if (!a.in[i]) { // uniform: operands are packed from 0
+#pragma unroll
+      for (int e = 0; e < kV; ++e)
+        v[i][e] = 0.0f;
+      continue;
+    }
+    if ((a.f16_mask >> i) & 1) {
+      const _Float16 *p = static_cast<const _Float16 *>(a.in[i]) + row * a.ld[i] + col0;
+      if (a.vec && whole) {
+        const f16x4 w = *reinterpret_cast<const f16x4 *>(p);
+#pragma unroll
+        for (int e = 0; e < kV; ++e)
+          v[i][e] = (float)w[e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < kV; ++e)
+          v[i][e] = col0 + e < a.cols ? (float)p[e] : 0.0f;
+      }
+    } else {
+      const float *p = static_cast<const float *>(a.in[i]) + row * a.ld[i] + col0;
+      if (a.vec && whole) {
+        const f32x4 w = *reinterpret_cast<const f32x4 *>(p);
+#pragma unroll
+        for (int e = 0; e < kV; ++e)
+          v[i][e] = w[e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < kV; ++e)
+          v[i][e] = col0 + e < a.cols ? p[e] : 0.0f;
+      }
+    }
+  }
+  // the stack and, beside every entry, whether the element is still active in it
+  float t0[kV], t1[kV], t2[kV], t3[kV];
+  bool k0[kV], k1[kV], k2[kV], k3[kV];
+#pragma unroll
+  for (int e = 0; e < kV; ++e) {
+    t0[e] = t1[e] = t2[e] = t3[e] = 0.0f;
+    k0[e] = k1[e] = k2[e] = k3[e] = true;
+  }
+  for (uint32_t pc = 0; pc < a.n_instr; ++pc) {
+    const uint32_t op = a.prog[pc].op, arg = a.prog[pc].arg;
+    const float imm = a.prog[pc].imm;
+    if (op == FOP_IN || op == FOP_CONST) {
+#pragma unroll
+      for (int e = 0; e < kV; ++e) {
+        t3[e] = t2[e];
+        t2[e] = t1[e];
+        t1[e] = t0[e];
+        k3[e] = k2[e];
+        k2[e] = k1[e];
+        k1[e] = k0[e];
+        float x = imm;
+        if (op == FOP_IN)
+          x = arg == 0 ? v[0][e] : arg == 1 ? v[1][e] : arg == 2 ? v[2][e] : v[3][e];
+        t0[e] = x;
+        k0[e] = true;
+      }
+    } else if (op >= FOP_NEG) {
+#pragma unroll
+      for (int e = 0; e < kV; ++e)
+        t0[e] = unary(op, t0[e], k0[e]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < kV; ++e) {
+        bool ok = k1[e] && k0[e];
+        t0[e] = binary(op, t1[e], t0[e], arg, ok);
+        k0[e] = ok;
+        t1[e] = t2[e];
+        t2[e] = t3[e];
+        k1[e] = k2[e];
+        k2[e] = k3[e];
+      }
+    }
+  }
+  bool ok[kV];
+#pragma unroll
+  for (int e = 0; e < kV; ++e)
+    ok[e] = k0[e] || a.store_all != 0;
+  const bool all_ok = ok[0] && ok[1] && ok[2] && ok[3];
+  if (a.out_type == 2) {
+    uint8_t *o = static_cast<uint8_t *>(a.out) + row * a.ldo + col0;
+#pragma unroll
+    for (int e = 0; e < kV; ++e)
+      if (col0 + e < a.cols && ok[e])
+        o[e] = (uint8_t)(t0[e] != 0.0f);
+  } else if (a.out_type == 1) {
+    _Float16 *o = static_cast<_Float16 *>(a.out) + row * a.ldo + col0;
+    if (a.vec && whole && all_ok) {
+      f16x4 w;
+#pragma unroll
+      for (int e = 0; e < kV; ++e)
+        w[e] = (_Float16)t0[e];
+      *reinterpret_cast<f16x4 *>(o) = w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < kV; ++e)
+        if (col0 + e < a.cols && ok[e])
+          o[e] = (_Float16)t0[e];
+    }
+  } else {
+    float *o = static_cast<float *>(a.out) + row * a.ldo + col0;
+    if (a.vec && whole && all_ok) {
+      f32x4 w;
+#pragma unroll
+      for (int e = 0; e < kV; ++e)
+        w[e] = t0[e];
+      *reinterpret_cast<f32x4 *>(o) = w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < kV; ++e)
+        if (col0 + e < a.cols && ok[e])
+          o[e] = t0[e];
+    }
+  }
+}

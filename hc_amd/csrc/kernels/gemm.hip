@@ -253,11 +253,18 @@ __device__ __forceinline__ Acc mfma_block(V b, V a, Acc c) {
 // per row and instruction); 1 and 2 pass the tile through LDS, which the main
 // loop no longer needs, so that eight lanes write one whole 128-byte row
 // segment with 16-byte stores (2: non-temporal).  PRIO raises the wave's issue
-// priority for the duration of each MFMA burst.  PROBE is a measurement build,
-// not a product path: it fetches the first K tile only and then issues the
-// main loop's MFMAs on those fragments with no loads, LDS reads, waits or
-// barriers, which times the matrix cores alone on real operand data (its
-// output is not the product).
+// priority for the duration of each MFMA burst.  PROBE != 0 is a measurement
+// build whose output is not the product: the loop with one part taken out
+// (1: the MFMAs alone on the first K tile's fragments, no loads, LDS reads,
+// waits or barriers; 2: no wait for the loads at the barrier; 3: no barrier;
+// 4: no LDS operand reads; 5: no loads; 6: the loads fetch into a register
+// instead of LDS; 7: the Bt operand blocks are fetched in MFMA layout straight
+// into registers).  STAGE sends a panel through registers (buffer load, then
+// ds_write) instead of the load that writes LDS itself.  RS != 0 writes each
+// half-step out in hand order, one fenced slot per MFMA: the LDS reads of the
+// next half-step's operands over the first RS MFMAs, load v of the next tile
+// but one before MFMA LF + v * LS; RS == 0 leaves the order to the compiler
+// under sched_group_barrier hints.
 template <class E, int BM, int BN, int WM, int WN, int MF, bool EDGE = false, int EPI = 0,
           bool PRIO = false, int PROBE = 0, int STAGE = 0, int RS = 0, int LF = 1, int LS = 2>
 __device__ __forceinline__ void gemm_tile_pipelined(
@@ -386,27 +393,6 @@ __device__ __forceinline__ void gemm_tile_pipelined(
         return;
       }
     }
-    if constexpr (BUF && PROBE == 6) {
-      // measurement build: the same fetches into a register instead of LDS
-      const int kbytes = (int)(k0 * sizeof(E));
-      auto desc = [](const void *base, size_t bytes) {
-        const uint64_t p = reinterpret_cast<uint64_t>(base);
-        return u32x4{(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, (uint32_t)bytes, 0x00020000u};
-      };
-      const u32x4 ra = desc(A + (size_t)tm * BM * lda, ((size_t)(BM - 1) * lda + K) * sizeof(E));
-      const u32x4 rb = desc(Bt + (size_t)tn * BN * ldb, ((size_t)(BN - 1) * ldb + K) * sizeof(E));
-#pragma unroll
-      for (int i = 0; i < kALoads; ++i) {
-        const int so = a_first + i * a_step + kbytes;
-        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(probe_sink) : "v"(a_voff), "s"(ra), "s"(so));
-      }
-#pragma unroll
-      for (int i = 0; i < kBLoads; ++i) {
-        const int so = b_first + i * b_step + kbytes;
-        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(probe_sink) : "v"(b_voff), "s"(rb), "s"(so));
-      }
-      return;
-    }
     if constexpr (BUF) {
       const int kbytes = (int)(k0 * sizeof(E));
       // panels that pass through registers first: their loads are the oldest
@@ -457,6 +443,16 @@ __device__ __forceinline__ void gemm_tile_pipelined(
     if constexpr (BUF) {
       unsigned char *base = lds + buf * kStageBytes + wave * 1024;
       const int kbytes = (int)((size_t)kt * kBK * sizeof(E));
+      if constexpr (PROBE == 6) {
+        // measurement build: the same fetch into a register instead of LDS
+        const bool isa = v < kALoads;
+        const uint64_t p = reinterpret_cast<uint64_t>(isa ? A + (size_t)tm * BM * lda : Bt + (size_t)tn * BN * ldb);
+        const size_t bytes = ((size_t)((isa ? BM : BN) - 1) * (isa ? lda : ldb) + K) * sizeof(E);
+        const u32x4 r = {(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, (uint32_t)bytes, 0x00020000u};
+        const int so = isa ? a_first + v * a_step + kbytes : b_first + (v - kALoads) * b_step + kbytes;
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(probe_sink) : "v"(isa ? a_voff : b_voff), "s"(r), "s"(so));
+        return;
+      }
       if (v < kALoads)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr)(base + v * kWaves * 1024), 16, a_voff,
                                                  a_first + v * a_step + kbytes, 0, 0);
@@ -642,11 +638,13 @@ __device__ __forceinline__ void gemm_tile_pipelined(
       // every read was out a quarter of a half-step ago or earlier
       __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoVm, 0));
       __builtin_amdgcn_sched_barrier(0);
-      half_step(Slot0{}, Slot1{}, SpreadEven{}, RFirst{}, LFirst{}, buf, 1, true, false, 0, 0);
-      __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
-      __builtin_amdgcn_s_barrier();
+      half_step(Slot0{}, Slot1{}, SpreadEven{}, RFirst{}, LFirst{}, buf, 1, PROBE != 4, false, 0, 0);
+      __builtin_amdgcn_s_waitcnt(PROBE == 2 ? waitcnt_imm(kNoVm, 0) : waitcnt_imm(0, 0));
+      if constexpr (PROBE != 3)
+        __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
-      half_step(Slot1{}, Slot0{}, SpreadOdd{}, RFirst{}, LFirst{}, buf ^ 1, 0, READ, LOAD, t + 2, buf);
+      half_step(Slot1{}, Slot0{}, SpreadOdd{}, RFirst{}, LFirst{}, buf ^ 1, 0, READ && PROBE != 4,
+                LOAD && PROBE != 5, t + 2, buf);
       return;
     }
     // even half-step: consume slot 0 (requested a whole half-step ago, so the
@@ -819,6 +817,14 @@ __device__ __forceinline__ void gemm_tile_pipelined(
     gemm_tile_pipelined<E, BM, BN, WM, WN, MF, false, 2, false, 0, STAGE, RS,  \
                         LF, LS>(A, lda, Bt, ldb, C, ldc, M, N, K);             \
   }
+// the default 256 x 256 kernel's loop with one part taken out (PROBE)
+#define HCAMD_GEMM_PZ(NAME, PROBE)                                             \
+  extern "C" __global__ __launch_bounds__(512) void NAME(                      \
+      const __bf16 *A, size_t lda, const __bf16 *Bt, size_t ldb, __bf16 *C,    \
+      size_t ldc, int M, int N, int K) {                                       \
+    gemm_tile_pipelined<__bf16, 256, 256, 2, 4, 16, false, 2, false, PROBE, 0, \
+                        16, 1, 4>(A, lda, Bt, ldb, C, ldc, M, N, K);           \
+  }
 // the default whole-tile kernels: LDS-staged epilogue with non-temporal stores,
 // hand-ordered half-steps (LDS reads over the first half of the MFMAs, the loads
 // evenly over all of them)
@@ -837,12 +843,12 @@ HCAMD_GEMM_PX(hcamd_gemm_bf16_p256x256_w2x4_prio, __bf16, 256, 256, 2, 4, 16, 2,
 HCAMD_GEMM_PS(hcamd_gemm_bf16_p256x256_w2x4_loads_early, __bf16, 256, 256, 2, 4, 16, 0, 16, 1, 2)
 HCAMD_GEMM_PS(hcamd_gemm_bf16_p256x256_w2x4_stage_a, __bf16, 256, 256, 2, 4, 16, 1, 0, 1, 2)
 // measurement builds whose output is not the product
-HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_mfma_only, __bf16, 256, 256, 2, 4, 16, 2, false, 1)
-HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_no_vmwait, __bf16, 256, 256, 2, 4, 16, 2, false, 2)
-HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_no_barrier, __bf16, 256, 256, 2, 4, 16, 2, false, 3)
-HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_no_ldsread, __bf16, 256, 256, 2, 4, 16, 2, false, 4)
-HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_no_loads, __bf16, 256, 256, 2, 4, 16, 2, false, 5)
-HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_loads_to_regs, __bf16, 256, 256, 2, 4, 16, 2, false, 6)
+HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_mfma_only, 1)
+HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_no_vmwait, 2)
+HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_no_barrier, 3)
+HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_no_ldsread, 4)
+HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_no_loads, 5)
+HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_loads_to_regs, 6)
 HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_b_direct, __bf16, 256, 256, 2, 4, 16, 2, false, 7)
 HCAMD_GEMM_PE(hcamd_gemm_bf16_p256x256_w2x4_edge, __bf16, 256, 256, 2, 4, 16)
 HCAMD_GEMM_PE(hcamd_gemm_f16_p256x256_w2x4_edge, _Float16, 256, 256, 2, 4, 16)

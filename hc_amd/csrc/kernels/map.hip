@@ -84,6 +84,21 @@ enum : uint32_t {
   OP_RSUB_IN = 33, // operand - top
   OP_RDIV_IN = 34, // operand / top
   OP_COUNT = 35,
+  // 35 .. 43 are the row programs' scalar forms (below)
+  // The tile operator `/` as numpy.ma computes it: a quotient that is not finite
+  // (a zero divisor gives one) deactivates its element, whose value becomes the
+  // dividend.  `arg` bit 8 (MDIV_IN forms) or any `arg` (others): the tile is
+  // fp16 and the quotient is rounded to fp16 before the test.
+  OP_MDIV = 44,
+  OP_RMDIV = 45,
+  OP_MDIVI = 46,
+  OP_RMDIVI = 47,
+  OP_MDIV_IN = 48,
+  OP_RMDIV_IN = 49,
+  OP_CLEAR = 50,  // every element active again (a NumPy function returns a plain array)
+  OP_POWCHK = 51, // numpy.ma.power: a result that is not finite deactivates, value 1e20
+  OP_MSQRT = 52,  // numpy.sqrt of a tile: x < 0 deactivates, value 0
+  OP_MLOG = 53,   // numpy.log of a tile: x <= 0 deactivates, value 1
 };
 
 struct Instr {
@@ -103,14 +118,9 @@ struct MapArgs {
   Instr prog[kMaxProg];
 };
 
-__device__ __forceinline__ float nan_max(float a, float b) {
-  float r = __builtin_fmaxf(a, b);
-  return (a != a || b != b) ? a + b : r;
-}
-__device__ __forceinline__ float nan_min(float a, float b) {
-  float r = __builtin_fminf(a, b);
-  return (a != a || b != b) ? a + b : r;
-}
+// NumPy's maximum / minimum: a NaN wins, and of two equal values (+0 and -0) the second
+__device__ __forceinline__ float nan_max(float a, float b) { return (a > b || a != a) ? a : b; }
+__device__ __forceinline__ float nan_min(float a, float b) { return (a < b || a != a) ? a : b; }
 __device__ __forceinline__ float round16(float x) {
   _Float16 h = (_Float16)x;
   asm volatile("" : "+v"(h)); // keep the conversion pair from being folded
@@ -171,6 +181,7 @@ template <int N> struct RawT {
 };
 template <int N> struct StackT {
   float st[kDepth][N];
+  uint32_t bad; // bit e: element e of the chunk is inactive (masked operators only)
 };
 using Raw = RawT<kN>;
 using Stack = StackT<kN>;
@@ -253,6 +264,84 @@ template <int SP, int OP, int N> __device__ __forceinline__ void do_unary(StackT
   }
 }
 
+__device__ __forceinline__ bool is_finite(float x) { return __builtin_fabsf(x) < INFINITY; }
+// num / den under numpy.ma's rule, into `dst`
+template <int N>
+__device__ __forceinline__ void masked_div(StackT<N> &r, float *dst, const float *num, const float *den,
+                                           bool half) {
+  uint32_t bad = r.bad;
+#pragma unroll
+  for (int e = 0; e < N; ++e) {
+    const float n = num[e];
+    float q = n / den[e];
+    if (half)
+      q = round16(q);
+    const bool good = is_finite(q);
+    // numpy.ma adds 0 * dividend to the quotient (it restores the dividend under
+    // the mask that way): a quotient of -0 becomes +0 unless the dividend is negative
+    q += 0.0f * n;
+    dst[e] = good ? q : 0.0f + n;
+    bad |= good ? 0u : (1u << e);
+  }
+  r.bad = bad;
+}
+template <int SP, int OP, int N>
+__device__ __forceinline__ void do_masked(StackT<N> &r, const RawT<N> &raw, uint32_t f16_mask, uint32_t arg,
+                                          float imm) {
+  if constexpr (OP == OP_MDIV || OP == OP_RMDIV) {
+    if constexpr (SP >= 2) {
+      if constexpr (OP == OP_MDIV)
+        masked_div(r, r.st[SP - 2], r.st[SP - 2], r.st[SP - 1], arg != 0);
+      else
+        masked_div(r, r.st[SP - 2], r.st[SP - 1], r.st[SP - 2], arg != 0);
+    }
+  } else if constexpr (SP >= 1) {
+    float t[N];
+    if constexpr (OP == OP_MDIVI || OP == OP_RMDIVI) {
+#pragma unroll
+      for (int e = 0; e < N; ++e) t[e] = imm;
+    } else {
+      switch (arg & 3u) {
+      case 0: unpack(raw, 0, f16_mask & 1, t); break;
+      case 1: unpack(raw, 1, f16_mask & 2, t); break;
+      case 2: unpack(raw, 2, f16_mask & 4, t); break;
+      default: unpack(raw, 3, f16_mask & 8, t); break;
+      }
+    }
+    const bool half = (OP == OP_MDIVI || OP == OP_RMDIVI) ? arg != 0 : (arg & 0x100u) != 0;
+    if constexpr (OP == OP_MDIVI || OP == OP_MDIV_IN)
+      masked_div(r, r.st[SP - 1], r.st[SP - 1], t, half);
+    else
+      masked_div(r, r.st[SP - 1], t, r.st[SP - 1], half);
+  }
+}
+template <int SP, bool LOG, int N> __device__ __forceinline__ void do_domain(StackT<N> &r) {
+  if constexpr (SP >= 1) {
+    uint32_t bad = r.bad;
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+      const float x = r.st[SP - 1][e];
+      const bool out = LOG ? x <= 0.0f : x < 0.0f;
+      const float y = LOG ? logf(x) : __builtin_sqrtf(x);
+      r.st[SP - 1][e] = out ? (LOG ? 1.0f : 0.0f) : y;
+      bad |= out ? (1u << e) : 0u;
+    }
+    r.bad = bad;
+  }
+}
+template <int SP, int N> __device__ __forceinline__ void do_powchk(StackT<N> &r) {
+  if constexpr (SP >= 1) {
+    uint32_t bad = r.bad;
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+      const bool good = is_finite(r.st[SP - 1][e]);
+      r.st[SP - 1][e] = good ? r.st[SP - 1][e] : 1e20f;
+      bad |= good ? 0u : (1u << e);
+    }
+    r.bad = bad;
+  }
+}
+
 // One instruction with SP entries on the stack; returns the new stack pointer.
 // The host has verified the program, so pushes never overflow and pops never
 // underflow; the guards only keep impossible arms out of the code.
@@ -328,6 +417,33 @@ __device__ __forceinline__ int step(StackT<N> &r, const RawT<N> &raw, uint32_t f
     HCAMD_OPND(OP_RSUB_IN)
     HCAMD_OPND(OP_RDIV_IN)
 #undef HCAMD_OPND
+  case OP_MDIV:
+    do_masked<SP, OP_MDIV>(r, raw, f16_mask, arg, imm);
+    return SP - 1;
+  case OP_RMDIV:
+    do_masked<SP, OP_RMDIV>(r, raw, f16_mask, arg, imm);
+    return SP - 1;
+#define HCAMD_MASKED(OP)                                                       \
+  case OP:                                                                     \
+    do_masked<SP, OP>(r, raw, f16_mask, arg, imm);                             \
+    return SP;
+    HCAMD_MASKED(OP_MDIVI)
+    HCAMD_MASKED(OP_RMDIVI)
+    HCAMD_MASKED(OP_MDIV_IN)
+    HCAMD_MASKED(OP_RMDIV_IN)
+#undef HCAMD_MASKED
+  case OP_CLEAR:
+    r.bad = 0;
+    return SP;
+  case OP_POWCHK:
+    do_powchk<SP>(r);
+    return SP;
+  case OP_MSQRT:
+    do_domain<SP, false>(r);
+    return SP;
+  case OP_MLOG:
+    do_domain<SP, true>(r);
+    return SP;
   default:
     return SP;
   }
@@ -339,6 +455,7 @@ __device__ __forceinline__ int step(StackT<N> &r, const RawT<N> &raw, uint32_t f
 __device__ __forceinline__ void run_program(const MapArgs &a, const Raw &raw,
                                             uint32_t f16_mask, Stack &r) {
   int sp = 0;
+  r.bad = 0;
   Instr next = a.prog[0];
   for (uint32_t pc = 0; pc < a.n_instr; ++pc) {
     const Instr cur = next;
@@ -356,8 +473,17 @@ __device__ __forceinline__ void run_program(const MapArgs &a, const Raw &raw,
 }
 
 // ---- operand access -------------------------------------------------------------
+__device__ __forceinline__ void store_elem(void *p, bool f16, size_t i, float v);
+// bad: bit e set = element e is inactive and keeps what the output holds
 __device__ __forceinline__ void store_chunk(void *p, bool f16, size_t chunk,
-                                            const float *src) {
+                                            const float *src, uint32_t bad = 0) {
+  if (bad & 0xffu) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      if (!((bad >> e) & 1u))
+        store_elem(p, f16, chunk * 8 + e, src[e]);
+    return;
+  }
   if (f16) {
     f16x8 v;
 #pragma unroll
@@ -476,9 +602,9 @@ __device__ __forceinline__ void map_flat(const MapArgs &a, const uint32_t n_in) 
         if constexpr (SUM) {
 #pragma unroll
           for (int e = 0; e < kN; ++e)
-            acc += r.st[0][e];
+            acc += ((r.bad >> e) & 1u) ? 0.0f : r.st[0][e];
         } else {
-          store_chunk(a.out, out_f16, chunk, r.st[0]);
+          store_chunk(a.out, out_f16, chunk, r.st[0], r.bad);
         }
       }
     }
@@ -491,7 +617,7 @@ __device__ __forceinline__ void map_flat(const MapArgs &a, const uint32_t n_in) 
     run_program(a, raw, 0, r);
 #pragma unroll
     for (int e = 0; e < 8; ++e)
-      if (n_chunks * 8 + e < n) {
+      if (n_chunks * 8 + e < n && !((r.bad >> e) & 1u)) {
         if constexpr (SUM)
           acc += r.st[0][e];
         else
@@ -523,7 +649,7 @@ __device__ __forceinline__ void map_strided(const MapArgs &a, const uint32_t n_i
 #pragma unroll
     for (int e = 0; e < kN; ++e) {
       const size_t col = col0 + (size_t)e * kThreads;
-      if (col < a.cols) {
+      if (col < a.cols && !((r.bad >> e) & 1u)) {
         if constexpr (SUM)
           acc += r.st[0][e];
         else
@@ -619,15 +745,15 @@ __device__ __forceinline__ void map_rows(const MapArgs &a, const uint32_t n_in) 
       if constexpr (SUM) {
 #pragma unroll
         for (int e = 0; e < kN; ++e)
-          acc += (!shortc || (uint32_t)e < rem) ? r.st[0][e] : 0.0f;
+          acc += ((!shortc || (uint32_t)e < rem) && !((r.bad >> e) & 1u)) ? r.st[0][e] : 0.0f;
       } else {
         char *orow = static_cast<char *>(a.out) + (size_t)row * a.ldo * (out_f16 ? 2 : 4);
         if (!shortc) {
-          store_chunk(orow, out_f16, c, r.st[0]);
+          store_chunk(orow, out_f16, c, r.st[0], r.bad);
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if ((uint32_t)e < rem)
+            if ((uint32_t)e < rem && !((r.bad >> e) & 1u))
               store_elem(orow, out_f16, (size_t)whole * 8 + e, r.st[0][e]);
         }
       }
@@ -742,7 +868,7 @@ __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcam
   Stack r;
   run_program(a, raw, a.f16_mask, r);
   if (c < n_chunks)
-    store_chunk(a.out, out_f16, c, r.st[0]);
+    store_chunk(a.out, out_f16, c, r.st[0], r.bad);
   if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 255 && n_chunks * 8 < n) {
     gather(a, n_in, raw, [&](int, int e, size_t &off) {
       off = n_chunks * 8 + e;
@@ -751,7 +877,7 @@ __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcam
     run_program(a, raw, 0, r);
 #pragma unroll
     for (int e = 0; e < 8; ++e)
-      if (n_chunks * 8 + e < n)
+      if (n_chunks * 8 + e < n && !((r.bad >> e) & 1u))
         store_elem(a.out, out_f16, n_chunks * 8 + e, r.st[0][e]);
   }
 }

@@ -141,6 +141,7 @@ HCAMD_BLOB(copy)
 HCAMD_BLOB(elementwise)
 HCAMD_BLOB(map)
 HCAMD_BLOB(imap)
+HCAMD_BLOB(fmap)
 HCAMD_BLOB(distance)
 HCAMD_BLOB(gather)
 HCAMD_BLOB(softmax)
@@ -155,7 +156,7 @@ struct Blob {
 };
 #define HCAMD_BLOB(n) {#n, hcamd_blob_##n##_begin, hcamd_blob_##n##_end}
 const Blob kBlobs[] = {HCAMD_BLOB(copy), HCAMD_BLOB(elementwise),
-                       HCAMD_BLOB(map), HCAMD_BLOB(imap), HCAMD_BLOB(distance),
+                       HCAMD_BLOB(map), HCAMD_BLOB(imap), HCAMD_BLOB(fmap), HCAMD_BLOB(distance),
                        HCAMD_BLOB(gather), HCAMD_BLOB(softmax),
                        HCAMD_BLOB(quantize), HCAMD_BLOB(gemm)};
 #undef HCAMD_BLOB
@@ -1131,6 +1132,16 @@ void mapStackEffect(unsigned op, int &pops, int &pushes) {
     pops = -1, pushes = 0;
   }
 }
+// The same with the masked-division forms, which only the element-wise map and
+// its sum take.
+void mapStackEffectMasked(unsigned op, int &pops, int &pushes) {
+  if (op == HCAMD_MAP_MDIV || op == HCAMD_MAP_RMDIV)
+    pops = 2, pushes = 1;
+  else if (op >= HCAMD_MAP_MDIVI && op <= HCAMD_MAP_MLOG)
+    pops = 1, pushes = 1;
+  else
+    mapStackEffect(op, pops, pushes);
+}
 } // namespace
 
 namespace {
@@ -1162,17 +1173,20 @@ int launchMap(OlQueue q, bool sum, const HcamdMapInstr *prog, size_t nInstr,
   }
   // The program must keep the stack within bounds and leave one value.
   int sp = 0;
+  bool hasMasked = false; // numpy.ma's division forms: only the element-wise kernels have them
   for (size_t i = 0; i < nInstr; ++i) {
     int pops, pushes;
-    mapStackEffect(prog[i].op, pops, pushes);
+    mapStackEffectMasked(prog[i].op, pops, pushes);
     if (pops < 0) {
       dev->report("%s: unknown opcode %u at %zu", who, prog[i].op, i);
       return 1;
     }
+    const bool maskedOperand = prog[i].op == HCAMD_MAP_MDIV_IN || prog[i].op == HCAMD_MAP_RMDIV_IN;
+    hasMasked = hasMasked || prog[i].op >= HCAMD_MAP_MDIV;
     const bool readsOperand =
-        prog[i].op == HCAMD_MAP_IN ||
+        prog[i].op == HCAMD_MAP_IN || maskedOperand ||
         (prog[i].op >= HCAMD_MAP_ADD_IN && prog[i].op <= HCAMD_MAP_RDIV_IN);
-    if (readsOperand && prog[i].arg >= nInputs) {
+    if (readsOperand && (maskedOperand ? prog[i].arg & 0xffu : prog[i].arg) >= nInputs) {
       dev->report("%s: operand %u at %zu (only %zu given)", who,
                   prog[i].arg, i, nInputs);
       return 1;
@@ -1307,7 +1321,7 @@ int launchMap(OlQueue q, bool sum, const HcamdMapInstr *prog, size_t nInstr,
   // kernel run as a single store stage reads them coalesced with 32-bit index
   // arithmetic, about twice as fast as the element-wise kernel below, which
   // stays for fp32 (where it is the faster one) and under variant 1 of "map".
-  if (!sum && a.f16_mask != 0 && variantOf("map") != 1) {
+  if (!sum && a.f16_mask != 0 && variantOf("map") != 1 && !hasMasked) {
     const HcamdRowStage whole = {HCAMD_ROW_STORE, static_cast<uint32_t>(nInstr), 0};
     return hcamdLaunchRowProgram(q, prog, &whole, 1, inputs, inputTypes, inputLd, nInputs,
                                  nullptr, nullptr, 0, out, outType, ldo, rows, cols);
@@ -1458,6 +1472,127 @@ int hcamdLaunchIMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
   a.vec = vec ? 1u : 0u;
   a.n_instr = (uint32_t)nInstr;
   Kernel *k = builtinKernel(dev, "imap", "hcamd_imap_i32");
+  if (!k)
+    return 1;
+  void *args[] = {&a};
+  const size_t grid[3] = {ceilDiv(ceilDiv(cols, (size_t)4), (size_t)256), rows, 1};
+  const size_t block[3] = {256, 1, 1};
+  return launch(queue, k, grid, block, args, 0);
+}
+
+namespace {
+// Argument block of hcamd_fmap (device layout).
+struct FMapArgs {
+  const void *in[4];
+  void *out;
+  size_t ld[4];
+  size_t ldo, rows, cols;
+  uint32_t f16_mask, out_type, vec, store_all, n_instr;
+  HcamdMapInstr prog[48];
+};
+} // namespace
+
+int hcamdLaunchFMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
+                    const void *const *inputs, const int *inputTypes, const size_t *inputLd,
+                    size_t nInputs, void *out, int outType, size_t ldo, size_t rows,
+                    size_t cols, int storeAll) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  const char *who = "hcamdLaunchFMap";
+  if (!prog || nInstr == 0 || nInstr > 48) {
+    dev->report("%s: program of %zu instructions (1..48)", who, nInstr);
+    return 1;
+  }
+  if (nInputs > 4 || (nInputs && (!inputs || !inputLd || !inputTypes)) || !out) {
+    dev->report("%s: %zu operands (0..4) or a null pointer", who, nInputs);
+    return 1;
+  }
+  if (outType != HCAMD_F32 && outType != HCAMD_F16 && outType != HCAMD_U8) {
+    dev->report("%s: unsupported output type %d", who, outType);
+    return 1;
+  }
+  FMapArgs a{};
+  int sp = 0;
+  for (size_t i = 0; i < nInstr; ++i) {
+    const unsigned op = prog[i].op;
+    if (op == HCAMD_FMAP_END || op >= HCAMD_FMAP_COUNT) {
+      dev->report("%s: bad opcode %u at %zu", who, op, i);
+      return 1;
+    }
+    if (op == HCAMD_FMAP_IN && prog[i].arg >= nInputs) {
+      dev->report("%s: operand %u at %zu (only %zu given)", who, prog[i].arg, i, nInputs);
+      return 1;
+    }
+    const bool push = op == HCAMD_FMAP_IN || op == HCAMD_FMAP_CONST;
+    const bool unary = op >= HCAMD_FMAP_NEG;
+    if (sp < (push ? 0 : unary ? 1 : 2)) {
+      dev->report("%s: stack underflow at %zu", who, i);
+      return 1;
+    }
+    sp += push ? 1 : unary ? 0 : -1;
+    if (sp > 4) {
+      dev->report("%s: stack deeper than 4 at %zu", who, i);
+      return 1;
+    }
+    a.prog[i] = prog[i];
+  }
+  if (sp != 1) {
+    dev->report("%s: program leaves %d values, expected 1", who, sp);
+    return 1;
+  }
+  if (rows == 0 || cols == 0)
+    return 0;
+  if (rows > 65535) { // a column vector: walk it as one row when it is dense
+    bool dense = cols == 1 && ldo == 1;
+    for (size_t i = 0; i < nInputs; ++i)
+      dense = dense && inputLd[i] == 1;
+    if (!dense) {
+      dev->report("%s: more than 65535 rows", who);
+      return 1;
+    }
+    cols = rows;
+    rows = 1;
+  }
+  // a row of four-element pieces: fp32 pieces are 16 bytes, fp16 pieces 8
+  auto piece_ok = [&](const void *p, int type, size_t ld) {
+    const size_t bytes = type == HCAMD_F16 ? 8 : 16;
+    return reinterpret_cast<uintptr_t>(p) % bytes == 0 && (rows == 1 || ld % 4 == 0);
+  };
+  bool vec = outType == HCAMD_U8 || piece_ok(out, outType, ldo);
+  for (size_t i = 0; i < nInputs; ++i) {
+    if (!inputs[i]) {
+      dev->report("%s: null pointer", who);
+      return 1;
+    }
+    if (inputTypes[i] != HCAMD_F32 && inputTypes[i] != HCAMD_F16) {
+      dev->report("%s: unsupported operand type %d", who, inputTypes[i]);
+      return 1;
+    }
+    if (rows > 1 && inputLd[i] < cols) {
+      dev->report("%s: leading dimension smaller than cols", who);
+      return 1;
+    }
+    a.in[i] = inputs[i];
+    a.ld[i] = inputLd[i];
+    if (inputTypes[i] == HCAMD_F16)
+      a.f16_mask |= 1u << i;
+    vec = vec && piece_ok(inputs[i], inputTypes[i], inputLd[i]);
+  }
+  if (rows > 1 && ldo < cols) {
+    dev->report("%s: leading dimension smaller than cols", who);
+    return 1;
+  }
+  a.out = out;
+  a.ldo = ldo;
+  a.rows = rows;
+  a.cols = cols;
+  a.out_type = outType == HCAMD_F32 ? 0u : outType == HCAMD_F16 ? 1u : 2u;
+  a.vec = vec ? 1u : 0u;
+  a.store_all = storeAll ? 1u : 0u;
+  a.n_instr = (uint32_t)nInstr;
+  Kernel *k = builtinKernel(dev, "fmap", "hcamd_fmap");
   if (!k)
     return 1;
   void *args[] = {&a};

@@ -689,7 +689,12 @@ class Tile:
     def _binary(self, other, op, reflected=False):
         o = Tile.wrap(other)
         a, b = (o, self) if reflected else (self, o)
-        return Tile(op, (a, b), _broadcast(a.shape, b.shape), _result_dtype(a, b))
+        r = Tile(op, (a, b), _broadcast(a.shape, b.shape), _result_dtype(a, b))
+        if a.attrs.get("plain"):
+            # the left operand is what a NumPy function returned: in the reference a
+            # bare numpy.ma array, whose operator gives another one (stored in full)
+            r.attrs["plain"] = True
+        return r
 
     def __add__(self, o): return self._binary(o, "add")
     def __radd__(self, o): return self._binary(o, "add", True)
@@ -699,8 +704,11 @@ class Tile:
     def __rmul__(self, o): return self._binary(o, "mul", True)
     def __truediv__(self, o): return self._binary(o, "div")
     def __rtruediv__(self, o): return self._binary(o, "div", True)
-    def __neg__(self): return Tile("neg", (self,), self.shape, self.dtype_name)
-    def __abs__(self): return Tile("abs", (self,), self.shape, self.dtype_name)
+    def __neg__(self): return Tile("neg", (self,), self.shape, self.dtype_name, **self._plain_kw())
+    def __abs__(self): return Tile("abs", (self,), self.shape, self.dtype_name, **self._plain_kw())
+
+    def _plain_kw(self):
+        return {"plain": True} if self.attrs.get("plain") else {}
 
     # The rest of the operators the reference's wrapper forwards to NumPy
     # (python/hckernel/kernel_api.py:157-180).  Comparisons give bool tiles;
@@ -723,8 +731,11 @@ class Tile:
 
     def _compare(self, other, op):
         o = Tile.wrap(other)
-        return Tile(op, (self, o), _broadcast(self.shape, o.shape), "bool",
-                    operand_dtype=_result_dtype(self, o))
+        r = Tile(op, (self, o), _broadcast(self.shape, o.shape), "bool",
+                 operand_dtype=_result_dtype(self, o))
+        if self.attrs.get("plain"):
+            r.attrs["plain"] = True
+        return r
 
     def __lt__(self, o): return self._compare(o, "lt")
     def __le__(self, o): return self._compare(o, "le")
@@ -752,23 +763,49 @@ class Tile:
 
     # -- NumPy protocol -----------------------------------------------------------
     def __array_ufunc__(self, ufunc, method, *inputs, **kwargs):
+        """A NumPy function of tiles.  In the reference such a call reaches
+        numpy.ma through the tile wrapper's forwarded attributes
+        (python/hckernel/kernel_api.py:150-151): the function is applied to the
+        values, deactivated or not, numpy.ma's __array_wrap__ puts its fill
+        value where the function's domain fails (sqrt of a negative number: 0,
+        log of a non-positive one: 1, a division by zero: 1), and the result is
+        a bare numpy.ma array, which a store writes out in full.  The nodes made
+        here carry func=True (called as a function) and plain=True (not a tile:
+        stored in full)."""
         op = _UFUNC_OPS.get(ufunc.__name__)
         if method != "__call__" or op is None or kwargs:
             raise TraceError(f"numpy.{ufunc.__name__} ({method}) is not supported in a GPU kernel")
+
+        def plain(t: "Tile") -> "Tile":
+            t.attrs["plain"] = t.attrs["func"] = True
+            t.attrs.pop("pow", None)
+            return t
+
         if len(inputs) == 1:
             x = Tile.wrap(inputs[0])
             if op == "square":
-                return x * x
-            return Tile(op, (x,), x.shape, x.dtype_name)
+                return plain(x * x)
+            return plain(Tile(op, (x,), x.shape, x.dtype_name))
         a, b = inputs
+        if isinstance(a, np.generic) and isinstance(b, Tile):
+            # `np.float32(2) * tile`: the scalar's operator arrives here; it is the
+            # tile's reflected operator (which the reference's tile type lacks)
+            refl = {"add": "__radd__", "sub": "__rsub__", "mul": "__rmul__", "div": "__rtruediv__",
+                    "floordiv": "__rfloordiv__", "mod": "__rmod__", "lt": "__gt__", "le": "__ge__",
+                    "gt": "__lt__", "ge": "__le__", "eq": "__eq__", "ne": "__ne__"}.get(op)
+            if refl is not None:
+                return getattr(b, refl)(a)
         if op == "power":
-            return Tile.wrap(a) ** b
+            r = Tile.wrap(a) ** b
+            if r is a:                          # exponent 1: a new node, the same values
+                r = Tile.wrap(a) * Tile.wrap(np.dtype(r.dtype_name).type(1))
+            return plain(r)
         if op in ("lt", "le", "gt", "ge", "eq", "ne"):
             a, b = Tile.wrap(a), Tile.wrap(b)
-            return a._compare(b, op)
+            return plain(a._compare(b, op))
         if isinstance(a, Tile):
-            return a._binary(b, op)
-        return Tile.wrap(b)._binary(a, op, reflected=True)
+            return plain(a._binary(b, op))
+        return plain(Tile.wrap(b)._binary(a, op, reflected=True))
 
     def __array_function__(self, func, types, args, kwargs):
         name = func.__name__
@@ -778,7 +815,8 @@ class Tile:
             x = Tile.wrap(args[0])
             lo = kwargs.get("a_min", args[1] if len(args) > 1 else None)
             hi = kwargs.get("a_max", args[2] if len(args) > 2 else None)
-            return Tile("clip", (x,), x.shape, x.dtype_name, lo=float(lo), hi=float(hi))
+            return Tile("clip", (x,), x.shape, x.dtype_name, lo=float(lo), hi=float(hi), plain=True,
+                        func=True)
         if name in ("amax", "max", "sum", "amin", "min"):
             x = Tile.wrap(args[0])
             return x._reduce({"amax": "max", "amin": "min"}.get(name, name),
@@ -843,10 +881,13 @@ class Tile:
 
     def __pow__(self, e):
         if isinstance(e, (int, float, np.generic)) and not isinstance(e, bool):
+            # pow=True: numpy.ma.power deactivates results that are not finite
             if float(e) == 2.0:
-                return self * self              # what numpy.power does for this exponent
+                r = self * self                 # what numpy.power does for this exponent
+                r.attrs["pow"] = True
+                return r
             if float(e) == 0.5:
-                return Tile("sqrt", (self,), self.shape, self.dtype_name)
+                return Tile("sqrt", (self,), self.shape, self.dtype_name, pow=True, **self._plain_kw())
             if float(e) == 1.0:
                 return self
         raise TraceError("tile ** e: only the exponents 2, 1 and 0.5 have native code")

@@ -121,6 +121,8 @@ hcamdLaunchMapSum = _sig(_rt, "hcamdLaunchMapSum", _int, _vp, C.POINTER(MapInstr
 
 hcamdLaunchIMap = _sig(_rt, "hcamdLaunchIMap", _int, _vp, C.POINTER(MapInstr), _sz, C.POINTER(_vp),
                        _sz_p, _sz, _vp, _int, _sz, _sz, _sz)
+hcamdLaunchFMap = _sig(_rt, "hcamdLaunchFMap", _int, _vp, C.POINTER(MapInstr), _sz, C.POINTER(_vp),
+                       C.POINTER(_int), _sz_p, _sz, _vp, _int, _sz, _sz, _sz, _int)
 hcamdMapReduceColsWorkspace = _sig(_rt, "hcamdMapReduceColsWorkspace", _sz, _sz, _sz)
 hcamdLaunchMapReduceCols = _sig(_rt, "hcamdLaunchMapReduceCols", _int, _vp, _int,
                                 C.POINTER(MapInstr), _sz, C.POINTER(MapInstr), _sz,
@@ -512,7 +514,10 @@ MAP_OPS = {"in": 1, "const": 2, "add": 3, "sub": 4, "mul": 5, "div": 6, "max": 7
            "mini": 16, "rsubi": 17, "rdivi": 18, "neg": 19, "abs": 20, "sqrt": 21, "rint": 22,
            "exp": 23, "log": 24, "tanh": 25, "r16": 26, "add_in": 27, "sub_in": 28,
            "mul_in": 29, "div_in": 30, "max_in": 31, "min_in": 32, "rsub_in": 33,
-           "rdiv_in": 34}
+           "rdiv_in": 34,
+           # the tile operator `/` under numpy.ma's rule (element-wise map and its sum only)
+           "mdiv": 44, "rmdiv": 45, "mdivi": 46, "rmdivi": 47, "mdiv_in": 48, "rmdiv_in": 49,
+           "clear": 50, "powchk": 51, "msqrt": 52, "mlog": 53}
 MAP_MAX_INPUTS, MAP_MAX_INSTRS, MAP_STACK_DEPTH = 4, 32, 4
 # Row programs (hcamdLaunchRowProgram): opcodes that read row scalars, stage kinds, limits
 MAP_OPS.update({"red": 35, "add_red": 36, "sub_red": 37, "mul_red": 38, "div_red": 39,
@@ -624,6 +629,44 @@ def plan_imap(program, inputs, out, out_bool=False) -> Plan:
     return Plan(ctx, hcamdLaunchIMap,
                 (ctx.queue, prog, len(program), ptrs, lds, n_in, mo.ptr, U8 if out_bool else I32,
                  ldo, rows, cols), "hcamdLaunchIMap", (inputs, out, prog, ptrs, lds))
+
+
+FMAP_OPS = {"in": 1, "const": 2, "add": 3, "sub": 4, "mul": 5, "div": 6, "floordiv": 7, "mod": 8,
+            "min": 9, "max": 10, "udiv": 11, "lt": 12, "le": 13, "eq": 14, "ne": 15, "ge": 16,
+            "gt": 17, "neg": 18, "abs": 19, "sqrt": 20, "rint": 21, "exp": 22, "log": 23, "r16": 24,
+            "psqrt": 25, "powchk": 26}
+FMAP_MAX_INSTRS = 48
+
+
+def plan_fmap(program, inputs, out, types, store_all=False) -> Plan:
+    """out = f(inputs...) over fp32 / fp16 windows with numpy.ma's activity rules
+    (see hcamdLaunchFMap).  `program` is a postfix list of (opname, arg, float
+    immediate); `types` lists F32 / F16 for the inputs followed by F32, F16 or
+    U8 (a one-byte-per-element array that receives 0 / 1) for the output;
+    store_all writes inactive elements too."""
+    inputs = list(inputs)
+    ctx = _ctx_of(*inputs, out)
+    mo = as_memref(out)
+    _expect(mo, {F32: 4, F16: 2, U8: 1}[types[-1]], "fmap output")
+    rows, cols, ldo = _rows_cols(mo)
+    ms = []
+    for x, ty in zip(inputs, types):
+        m = as_memref(x)
+        _expect(m, {F32: 4, F16: 2}[ty], "fmap operand")
+        r, c, _ = _rows_cols(m)
+        if (r, c) != (rows, cols):
+            raise HcRuntimeError("fmap: shape mismatch")
+        ms.append(m)
+    n_in = len(ms)
+    prog = (MapInstr * max(len(program), 1))()
+    for i, (name, arg, imm) in enumerate(program):
+        prog[i].op, prog[i].arg, prog[i].imm = FMAP_OPS[name], int(arg), float(imm)
+    ptrs = (_vp * max(n_in, 1))(*[m.ptr for m in ms])
+    tys = (_int * max(n_in, 1))(*types[:n_in])
+    lds = (_sz * max(n_in, 1))(*[_rows_cols(m)[2] for m in ms])
+    return Plan(ctx, hcamdLaunchFMap,
+                (ctx.queue, prog, len(program), ptrs, tys, lds, n_in, mo.ptr, types[-1], ldo, rows,
+                 cols, int(bool(store_all))), "hcamdLaunchFMap", (inputs, out, prog, ptrs, tys, lds))
 
 
 COLS_KINDS = {"sum": 0, "max": 1, "min": 2}

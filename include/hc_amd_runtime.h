@@ -320,7 +320,27 @@ enum HcamdMapOp {
   HCAMD_MAP_MAX_IN = 31,
   HCAMD_MAP_MIN_IN = 32,
   HCAMD_MAP_RSUB_IN = 33, /* operand - top */
-  HCAMD_MAP_RDIV_IN = 34  /* operand / top */
+  HCAMD_MAP_RDIV_IN = 34, /* operand / top */
+  /* 35 .. 43: the row programs' scalar forms (enum HcamdRowOp) */
+  /* The tile OPERATOR `/`, as numpy.ma computes it
+   * (python/hckernel/kernel_api.py:157-180 forwards it to numpy.ma): a quotient
+   * that is not finite (a zero divisor gives one) makes its element inactive,
+   * nothing is stored or summed for it, and its value becomes 0 + dividend.
+   * The forms mirror DIV / RDIV; for an fp16 tile the quotient is rounded to
+   * fp16 before the test: `arg` != 0 says so (the *_IN forms: bit 8 of `arg`,
+   * whose low bits are the operand index).  HCAMD_MAP_DIV and its forms stay
+   * the plain quotient, which is numpy.divide called as a function.  hcamdLaunchMap
+   * and hcamdLaunchMapSum only. */
+  HCAMD_MAP_MDIV = 44,
+  HCAMD_MAP_RMDIV = 45,
+  HCAMD_MAP_MDIVI = 46,
+  HCAMD_MAP_RMDIVI = 47,
+  HCAMD_MAP_MDIV_IN = 48,
+  HCAMD_MAP_RMDIV_IN = 49,
+  HCAMD_MAP_CLEAR = 50,  /* every element active again (ends a program whose result is stored in full) */
+  HCAMD_MAP_POWCHK = 51, /* numpy.ma.power: top not finite -> inactive, value 1e20 */
+  HCAMD_MAP_MSQRT = 52,  /* numpy.sqrt of a tile: x < 0 -> inactive, value 0 */
+  HCAMD_MAP_MLOG = 53    /* numpy.log of a tile: x <= 0 -> inactive, value 1 */
 };
 #define HCAMD_MAP_MAX_INPUTS 4
 #define HCAMD_MAP_MAX_INSTRS 32
@@ -360,6 +380,52 @@ enum HcamdIMapOp {
 int hcamdLaunchIMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
                     const void *const *inputs, const size_t *inputLd, size_t nInputs,
                     void *out, int outType, size_t ldo, size_t rows, size_t cols) HCAMD_NOEXCEPT;
+
+/* The general float map: out = f(in_0 .. in_{n-1}) over a rows x cols window of
+ * fp32 / fp16 operands with numpy.ma's activity rules, for what hcamdLaunchMap
+ * leaves out of the operators the reference's tile wrapper forwards
+ * (python/hckernel/kernel_api.py:157-211): // and %, the six comparisons, and
+ * expressions in which the value numpy.ma leaves under a deactivated element
+ * is seen again.  Activity is tracked per stack entry:
+ *   ADD SUB MUL  tile operators: the first operand's value where an operand is
+ *                inactive; `arg` bit 1: called as a NumPy function (computed
+ *                from the values whatever their activity)
+ *   DIV FLOORDIV tile operators / and //: inactive if the divisor is zero or the
+ *                result is not finite (`arg` bit 0: tested as fp16), value
+ *                0 + dividend; an active quotient has 0 * dividend added
+ *   MOD, UDIV    % and numpy.divide as a function: inactive with the value 1
+ *                where the divisor is zero or the dividend infinite (neither
+ *                NaN), otherwise the remainder / the plain quotient
+ *   SQRT LOG     numpy.sqrt / numpy.log: inactive with the value 0 / 1 where the
+ *                operand is inactive or outside the domain
+ *   PSQRT POWCHK x ** 0.5 (the operand's value where it is inactive), and
+ *                numpy.ma.power's check: not finite -> inactive, value 1e20
+ *   MIN MAX      numpy.minimum / maximum: a NaN wins; of two equal values (+0, -0)
+ *                the second (`arg` bit 0, fp16 tiles: the first, as NumPy's half
+ *                loops do)
+ *   the rest     computed from the values, activity kept; comparisons give 0 / 1
+ * Every rounding to fp16 other than DIV / FLOORDIV's is an explicit
+ * HCAMD_FMAP_R16.  outType is HCAMD_F32, HCAMD_F16, or HCAMD_U8 (one byte of
+ * 0 / 1, a bool buffer).  Inactive elements are not stored, unless storeAll is
+ * set: a NumPy function returns a bare numpy.ma array, which the reference's
+ * store writes out in full.  Programs have at most 48 instructions on a
+ * four-entry stack. */
+enum HcamdFMapOp {
+  HCAMD_FMAP_END = 0, HCAMD_FMAP_IN = 1, HCAMD_FMAP_CONST = 2,
+  HCAMD_FMAP_ADD = 3, HCAMD_FMAP_SUB = 4, HCAMD_FMAP_MUL = 5, HCAMD_FMAP_DIV = 6,
+  HCAMD_FMAP_FLOORDIV = 7, HCAMD_FMAP_MOD = 8, HCAMD_FMAP_MIN = 9, HCAMD_FMAP_MAX = 10,
+  HCAMD_FMAP_UDIV = 11,
+  HCAMD_FMAP_LT = 12, HCAMD_FMAP_LE = 13, HCAMD_FMAP_EQ = 14, HCAMD_FMAP_NE = 15,
+  HCAMD_FMAP_GE = 16, HCAMD_FMAP_GT = 17,
+  HCAMD_FMAP_NEG = 18, HCAMD_FMAP_ABS = 19, HCAMD_FMAP_SQRT = 20, HCAMD_FMAP_RINT = 21,
+  HCAMD_FMAP_EXP = 22, HCAMD_FMAP_LOG = 23, HCAMD_FMAP_R16 = 24, HCAMD_FMAP_PSQRT = 25,
+  HCAMD_FMAP_POWCHK = 26,
+  HCAMD_FMAP_COUNT = 27
+};
+int hcamdLaunchFMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
+                    const void *const *inputs, const int *inputTypes, const size_t *inputLd,
+                    size_t nInputs, void *out, int outType, size_t ldo, size_t rows,
+                    size_t cols, int storeAll) HCAMD_NOEXCEPT;
 
 /* Map-reduce: *cell += sum over the window of f(in_0 .. in_{n-1}), fp32, with
  * one hardware atomic add per workgroup.  This is the reference's reduction

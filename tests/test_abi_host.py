@@ -50,7 +50,7 @@ def test_jit_symbol_table_has_the_reference_names():
 
 def test_builtin_code_objects_are_gfx950_elf_and_hold_the_kernels():
     mods = rt.builtin_modules()
-    assert set(mods) == {"copy", "elementwise", "map", "imap", "distance", "gather", "softmax", "quantize", "gemm"}
+    assert set(mods) == {"copy", "elementwise", "map", "imap", "fmap", "distance", "gather", "softmax", "quantize", "gemm"}
     src = open(os.path.join(ROOT, "hc_amd", "csrc", "runtime.cpp")).read()
     wanted = set(re.findall(r'"(hcamd_[a-z0-9_]+)"', src))
     wanted = {w for w in wanted if not w.endswith("_")}       # prefixes built at run time

@@ -4,6 +4,8 @@ CPU oracle.  The three copy kernels are the bodies of the reference's own GPU
 end-to-end tests (python/hckernel/tests/test_e2e.py:57-136), imported through
 the reference's package name."""
 
+import zlib
+
 import numpy as np
 import pytest
 import sympy
@@ -1061,3 +1063,162 @@ def test_int32_division_by_zero_deactivates_the_element_and_shift_counts():
     # numpy.ma's own corner: |INT_MIN| overflows in its divisor test, so INT_MIN // 0 stays
     # active with NumPy's quotient 0 (element 1 of the inputs)
     assert (a[1], b[1]) == (-2 ** 31, 0) and hosts[0][1] == 1 and hosts[1][1] == 0
+
+
+def _special_floats(rng, shape, dtype):
+    """Random values with zeros of both signs, infinities, NaNs, huge and tiny
+    magnitudes mixed in, so that divisions fail in every way numpy.ma tests for."""
+    big, tiny = (3.0e38, 1.5e-38) if dtype == np.float32 else (60000.0, 6.2e-5)
+    x = (rng.standard_normal(shape) * 4).astype(dtype)
+    special = np.array([0.0, -0.0, 1.0, -1.0, 2.5, -7.25, big, -big, tiny, np.inf, -np.inf, np.nan,
+                        3.0, -3.0, 0.5], dtype)
+    pick = rng.random(shape) < 0.35
+    x[pick] = special[rng.integers(0, len(special), int(pick.sum()))]
+    return x
+
+
+_FLOAT_OPERATOR_BODIES = {
+    # the tile operators go through numpy.ma: a failed division deactivates its element
+    "a/b": lambda a, b, K: a / b,
+    "a/b*2+1": lambda a, b, K: a / b * K(2) + K(1),
+    "(a+b)/(a-b)": lambda a, b, K: (a + b) / (a - b),
+    "a/3": lambda a, b, K: a / K(3),
+    "a/0": lambda a, b, K: a / K(0),
+    "a*a/b": lambda a, b, K: a * a / b,
+    "a**2/b": lambda a, b, K: a ** K(2) / b,
+    "a**0.5*b": lambda a, b, K: a ** K(0.5) * b,
+    # a NumPy function reads the values, deactivated or not, and returns a plain array
+    "np.divide(a,b)": lambda a, b, K: np.divide(a, b),
+    "np.exp(a/b)": lambda a, b, K: np.exp(a / b),
+    "np.abs(a/b)-b/a": lambda a, b, K: np.abs(a / b) - b / a,
+    "np.abs(a/b*2)": lambda a, b, K: np.abs(a / b * K(2)),
+    "a/b+np.abs(b/a)": lambda a, b, K: a / b + np.abs(b / a),
+    "np.maximum(a/b,b/a)": lambda a, b, K: np.maximum(a / b, b / a),
+    "np.sqrt(a**2)": lambda a, b, K: np.sqrt(a ** K(2)),
+    # // and %, comparisons
+    "a//b": lambda a, b, K: a // b,
+    "a%b": lambda a, b, K: a % b,
+    "a//b*b+a%b": lambda a, b, K: (a // b) * b + a % b,
+    "a%3-b//2": lambda a, b, K: a % K(3) - b // K(2),
+    "np.abs(a//b)": lambda a, b, K: np.abs(a // b),
+    "(a<b)*a": lambda a, b, K: (a < b).astype(K) * a,
+    "-(a/b)": lambda a, b, K: -(a / b),
+    "abs(a/b)": lambda a, b, K: abs(a / b),
+    # NumPy functions with a domain put numpy.ma's fill value where it fails
+    "np.sqrt(a)": lambda a, b, K: np.sqrt(a),
+    "np.log(a)": lambda a, b, K: np.log(a),
+    "np.sqrt(a/b)": lambda a, b, K: np.sqrt(a / b),
+    "a*np.sqrt(b)": lambda a, b, K: a * np.sqrt(b),
+    "np.sqrt(a)*b": lambda a, b, K: np.sqrt(a) * b,
+    "np.log(a)/b": lambda a, b, K: np.log(a) / b,
+    "np.add(a/b,b)": lambda a, b, K: np.add(a / b, b),
+    "np.remainder(a,b)": lambda a, b, K: np.remainder(a, b),
+    "(a/b)*b": lambda a, b, K: (a / b) * b,
+    "np.abs(a)*(b/a)": lambda a, b, K: np.abs(a) * (b / a),
+    "K(2)*(a/b)": lambda a, b, K: K(2) * (a / b),
+    "np.abs(a/b)+K(1)": lambda a, b, K: np.abs(a / b) + K(1),
+    "np.rint(a//b)-a%b": lambda a, b, K: np.rint(a // b) - a % b,
+}
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("name", list(_FLOAT_OPERATOR_BODIES))
+def test_float_tile_operators_deactivate_like_numpy_ma(name, dtype):
+    """/ // % ** on float tiles go through numpy.ma in the reference
+    (python/hckernel/kernel_api.py:157-180): a zero divisor or a quotient that is
+    not finite deactivates the element, the store leaves it alone, and a NumPy
+    function applied afterwards sees the value numpy.ma left there.  Same body on
+    the GPU and on the host executor, bit for bit, including which elements are
+    written at all."""
+    expr = _FLOAT_OPERATOR_BODIES[name]
+    rng = np.random.default_rng(zlib.crc32(name.encode()) % 1000 + np.dtype(dtype).itemsize)
+    R, Cc = sym.R, sym.C
+    shape = (37, 1031) if dtype == np.float32 else (19, 520)
+
+    def body(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT], out: Buffer[R, Cc, DT]):
+        x, y = gr.work_offset
+        gr.store(out[x:, y:], expr(gr.load(a[x:, y:], shape=gr.shape), gr.load(b[x:, y:], shape=gr.shape),
+                                   dtype))
+
+    a, b = _special_floats(rng, shape, dtype), _special_floats(rng, shape, dtype)
+    host = np.full(shape, 7.5, dtype)
+    dout = rt.to_device(host)
+    deco = dict(work_shape=(R, Cc), group_shape=(4, 64))
+    kernel(**deco)(body)(rt.to_device(a), rt.to_device(b), dout)
+    with np.errstate(all="ignore"):
+        sim_kernel(**deco)(body)(a, b, host)
+    got = dout.to_host()
+    nan = np.isnan(host)
+    assert_array_equal(np.isnan(got), nan, err_msg=name)
+    u = np.uint32 if dtype == np.float32 else np.uint16
+    if "exp" in name or "log" in name or "**0.5" in name:
+        # the library exp / log differ from NumPy's in the last bit, and numpy.ma computes
+        # x ** 0.5 with NumPy's power (not correctly rounded) where the GPU takes the square
+        # root; which elements are written, signs, zeros and infinities still have to agree
+        # exactly
+        tiny = float(np.finfo(dtype).tiny)
+        fin = np.isfinite(host) & (np.abs(host) >= tiny)       # results near underflow: absolute
+        assert_array_equal(got[~nan & ~np.isfinite(host)], host[~nan & ~np.isfinite(host)], err_msg=name)
+        assert_allclose(got[~nan & np.isfinite(host) & ~fin].astype(np.float64),
+                        host[~nan & np.isfinite(host) & ~fin].astype(np.float64), rtol=0, atol=tiny)
+        assert_allclose(got[fin].astype(np.float64), host[fin].astype(np.float64),
+                        rtol=4e-7 if dtype == np.float32 else 1e-3, err_msg=name)
+    else:
+        assert_array_equal(got.view(u)[~nan], host.view(u)[~nan], err_msg=name)
+    if name in ("a/b", "a/0", "a**0.5*b", "a//b", "a%b", "a/b+np.abs(b/a)", "abs(a/b)"):
+        assert (host.view(u) == np.array(7.5, dtype).view(u)).sum() > 100   # elements were left alone
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_float_comparisons_store_to_bool_buffers(dtype):
+    N = sym.N
+
+    def body(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], lt: Buffer[N, DT], le: Buffer[N, DT],
+             eq: Buffer[N, DT], ne: Buffer[N, DT], ge: Buffer[N, DT], gt: Buffer[N, DT], mix: Buffer[N, DT]):
+        o, g = gr.work_offset[0], gr.shape[0]
+        ta, tb = gr.load(a[o:], shape=g), gr.load(b[o:], shape=g)
+        gr.store(lt[o:], ta < tb)
+        gr.store(le[o:], ta <= tb)
+        gr.store(eq[o:], ta == tb)
+        gr.store(ne[o:], ta != tb)
+        gr.store(ge[o:], ta >= tb)
+        gr.store(gt[o:], ta > tb)
+        gr.store(mix[o:], ta / tb > dtype(0.5))        # inactive where the division failed
+
+    rng = np.random.default_rng(5)
+    n = 10_007
+    a, b = _special_floats(rng, n, dtype), _special_floats(rng, n, dtype)
+    b[::7] = a[::7]
+    hosts = [np.zeros(n, bool) for _ in range(7)]
+    for h in hosts:
+        h[::3] = True
+    devs = [rt.to_device(h) for h in hosts]
+    kernel(work_shape=N, group_shape=256)(body)(rt.to_device(a), rt.to_device(b), *devs)
+    with np.errstate(all="ignore"):
+        sim_kernel(work_shape=N, group_shape=256)(body)(a, b, *hosts)
+    for d, h, name in zip(devs, hosts, ["lt", "le", "eq", "ne", "ge", "gt", "mix"]):
+        assert_array_equal(d.to_host(), h, err_msg=name)
+
+
+def test_sum_skips_elements_a_division_deactivated():
+    """`acc += (a / b).sum()`: numpy.ma's sum leaves deactivated elements out."""
+    N = sym.N
+
+    def body(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], acc: Buffer[1, DT]):
+        o, g = gr.work_offset[0], gr.shape[0]
+        atomic_ref(acc)[0] += (gr.load(a[o:], shape=g) / gr.load(b[o:], shape=g) + np.float32(1)).sum()
+
+    rng = np.random.default_rng(6)
+    n = 100_003
+    a = rng.standard_normal(n).astype(np.float32)
+    b = rng.integers(-3, 4, n).astype(np.float32)          # a seventh of the divisors are zero
+    host = np.zeros(1, np.float32)
+    dacc = rt.to_device(host)
+    kernel(work_shape=N, group_shape=256)(body)(rt.to_device(a), rt.to_device(b), dacc)
+    ok = b != 0
+    want = (a[ok].astype(np.float64) / b[ok] + 1).sum()
+    assert (~ok).sum() > 10_000
+    assert_allclose(dacc.to_host()[0], want, rtol=1e-5)
+    with np.errstate(all="ignore"):
+        sim_kernel(work_shape=N, group_shape=256)(body)(a, b, host)
+    assert_allclose(host[0], want, rtol=1e-4)

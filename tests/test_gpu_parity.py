@@ -298,6 +298,92 @@ def test_imap_zero_divisors_are_left_alone_and_bad_programs_refused(ctx):
             rt.plan_imap(prog, [x], out).launch(sync=True)
 
 
+def _ma_special(rng, n, dtype):
+    big, tiny = (3.0e38, 1.5e-38) if dtype == np.float32 else (60000.0, 6.2e-5)
+    x = (rng.standard_normal(n) * 4).astype(dtype)
+    special = np.array([0.0, -0.0, 1.0, -1.0, 2.5, -7.25, big, -big, tiny, np.inf, -np.inf, np.nan], dtype)
+    pick = rng.random(n) < 0.4
+    x[pick] = special[rng.integers(0, len(special), int(pick.sum()))]
+    return x
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_fmap_every_operation_against_numpy_ma(ctx, dtype):
+    """hcamdLaunchFMap, one program per opcode, against numpy.ma itself on data full
+    of zeros, infinities and NaNs: the values, and which elements are stored.  The
+    second operand is partly inactive already (a failed division in front of the
+    operation under test), so the rules for inactive operands are covered too."""
+    import numpy.ma as ma
+    rng = np.random.default_rng(321)
+    n = 20_003
+    a, b, c = (_ma_special(rng, n, dtype) for _ in range(3))
+    ty = rt.F32 if dtype == np.float32 else rt.F16
+    half = int(dtype == np.float16)
+    F = lambda name, arg=0, imm=0.0: (name, arg, imm)
+    u = np.uint32 if dtype == np.float32 else np.uint16
+    r16 = [F("r16")] if half else []
+
+    def run(prog, n_in, store_all, out_dtype=None):
+        out = poisoned((n,), out_dtype or dtype)
+        types = [ty] * n_in + [rt.U8 if out_dtype == np.uint8 else ty]
+        rt.plan_fmap(prog, [dev(a), dev(b), dev(c)][:n_in], out, types, store_all).launch(sync=True)
+        return out.to_host()
+
+    def check(name, got, want_ma, store_all):
+        data, mask = ma.getdata(want_ma).astype(dtype), ma.getmaskarray(want_ma)
+        poison = np.full(1, POISON32 if dtype == np.float32 else POISON32 & 0xFFFF, u).view(dtype)[0]
+        want = data.copy() if store_all else np.where(mask, poison, data)
+        nan = np.isnan(want)
+        assert_array_equal(np.isnan(got), nan, err_msg=name)
+        assert_array_equal(got.view(u)[~nan], want.view(u)[~nan], err_msg=name)
+
+    am, bm, cm = (ma.masked_array(x) for x in (a, b, c))
+    with np.errstate(all="ignore"):
+        cases = {
+            "add": am + bm, "sub": am - bm, "mul": am * bm, "div": am / bm, "floordiv": am // bm,
+            "mod": am % bm, "min": np.minimum(am, bm), "max": np.maximum(am, bm), "udiv": np.divide(am, bm)}
+        for name, want in cases.items():
+            arg = half if name in ("div", "floordiv", "min", "max") else 0
+            tail = [] if name in ("div", "floordiv", "min", "max") else r16
+            for store_all in (False, True):
+                check(name, run([F("in", 0), F("in", 1), F(name, arg)] + tail, 2, store_all), want, store_all)
+        # the same operations on a second operand that a division has partly deactivated: b / c
+        q = bm / cm
+        cases2 = {"add": am + q, "sub": am - q, "mul": am * q, "div": am / q, "floordiv": am // q,
+                  "mod": am % q, "max": np.maximum(am, q), "udiv": np.divide(am, q),
+                  "add|2": np.add(am, q), "mul|2": np.multiply(am, q)}
+        for name, want in cases2.items():
+            op, _, fn = name.partition("|")
+            arg = (half if op in ("div", "floordiv", "max") else 0) | (2 if fn else 0)
+            tail = [] if op in ("div", "floordiv", "max") else r16
+            prog = [F("in", 0), F("in", 1), F("in", 2), F("div", half), F(op, arg)] + tail
+            for store_all in (False, True):
+                check("a " + name + " (b/c)", run(prog, 3, store_all), want, store_all)
+        unary = {"neg": -q, "abs": abs(q), "sqrt": np.sqrt(q), "log": None, "rint": np.rint(q),
+                 "psqrt": None}
+        for name, want in unary.items():
+            if want is None:
+                continue
+            prog = [F("in", 1), F("in", 2), F("div", half), F(name)] + ([] if name in ("neg", "abs") else r16)
+            for store_all in (False, True):
+                check(name + "(b/c)", run(prog, 3, store_all), want, store_all)
+        # x ** 2 as numpy.ma.power computes and checks it
+        want = ma.power(am, dtype(2))
+        check("pow2", run([F("in", 0), F("in", 0), F("mul")] + r16 + [F("powchk")], 1, False), want, False)
+        check("pow2", run([F("in", 0), F("in", 0), F("mul")] + r16 + [F("powchk")], 1, True), want, True)
+        # comparisons into a one-byte buffer; inactive elements are left alone
+        for name, want in {"lt": am < q, "le": am <= q, "ge": am >= q, "gt": am > q, "ne": am != bm,
+                           "eq": am == bm}.items():
+            second = [F("in", 1)] if name in ("ne", "eq") else [F("in", 1), F("in", 2), F("div", half)]
+            got = run([F("in", 0)] + second + [F(name)], 3, False, np.uint8)
+            data, mask = ma.getdata(want).astype(np.uint8), ma.getmaskarray(want)
+            assert_array_equal(got, np.where(mask, POISON32 & 0xFF, data), err_msg=name)
+    with pytest.raises(rt.HcRuntimeError, match="underflow"):
+        rt.plan_fmap([F("add")], [dev(a)], poisoned((n,), dtype), [ty, ty]).launch(sync=True)
+    with pytest.raises(rt.HcRuntimeError, match="leaves 2 values"):
+        rt.plan_fmap([F("in", 0), F("in", 0)], [dev(a)], poisoned((n,), dtype), [ty, ty]).launch(sync=True)
+
+
 # ---------------------------------------------------------------------------
 # stream calibration kernels (the yardstick of the memory-bound kernels)
 # ---------------------------------------------------------------------------

@@ -198,7 +198,7 @@ def stack_depth(program):
     sp = deepest = 0
     for name, _, _ in program:
         code = rt.MAP_OPS[name]
-        sp += 1 if code <= 2 else (-1 if code <= 10 else 0)     # the rest: one in, one out
+        sp += 1 if code <= 2 else (-1 if code <= 10 or code in (44, 45) else 0)   # the rest: one in, one out
         deepest = max(deepest, sp)
     assert sp == 1
     return deepest
@@ -221,14 +221,15 @@ def test_elementwise_expressions_compile_to_postfix_programs(ctx):
     # constants fold into immediates; a reversed immediate form where the
     # constant is on the left
     (p,) = kern(lambda a, b, c: (2.0 - a) * b / 4).plan(*arrs, ctx=ctx)
+    # (the tile operator / is numpy.ma's division: the m* forms deactivate failed quotients)
     assert map_program(p) == [("in", 0, 0.0), ("rsubi", 0, 2.0), ("mul_in", 1, 0.0),
-                              ("divi", 0, 4.0)]
+                              ("mdivi", 0, 4.0)]
     assert p.args[6] == 2 and p.args[10:] == (1, 1000)        # two operands, 1 x 1000
     # an operand on one side of a binary operation is read by the operation
     # itself: a - (b*c + a/b) evaluates the right side, then "a minus top"
     (p,) = kern(lambda a, b, c: a - (b * c + a / b)).plan(*arrs, ctx=ctx)
     prog = map_program(p)
-    assert [i[0] for i in prog] == ["in", "mul_in", "in", "div_in", "add", "rsub_in"]
+    assert [i[0] for i in prog] == ["in", "mul_in", "in", "mdiv_in", "add", "rsub_in"]
     assert stack_depth(prog) == 2
     assert p.args[3][prog[-1][1]] == arrs[0].ptr       # operands are numbered by first use
     # the deeper side goes first: (a*b - c*a) / (exp(a) / (b*c + a*a))
@@ -237,7 +238,7 @@ def test_elementwise_expressions_compile_to_postfix_programs(ctx):
     prog = map_program(p)
     assert [i[0] for i in prog] == ["in", "mul_in", "in", "mul_in", "sub",        # numerator
                                     "in", "mul_in", "in", "mul_in", "add",        # b*c + a*a
-                                    "in", "exp", "rdiv", "div"]
+                                    "in", "exp", "rmdiv", "mdiv"]
     assert stack_depth(prog) == 3
     # ufuncs, clip, maximum with NaN propagation left to the kernel
     (p,) = kern(lambda a, b, c: np.clip(np.exp(-np.abs(a)) + np.maximum(b, c), 0, 6)).plan(
@@ -1449,3 +1450,74 @@ def test_thread_variants_are_private_to_the_thread():
     t.join()
     assert seen["ok"]
     rt.set_thread_variant("gemm", -1)
+
+
+def fmap_program(plan):
+    """(opname, arg, imm) triples of a hcamdLaunchFMap plan."""
+    names = {v: k for k, v in rt.FMAP_OPS.items()}
+    prog, n = plan.args[1], plan.args[2]
+    return [(names[prog[i].op], prog[i].arg, prog[i].imm) for i in range(n)]
+
+
+def test_float_operators_follow_numpy_ma_and_pick_the_kernel_that_can(ctx):
+    """The tile operators / // % ** go through numpy.ma in the reference
+    (python/hckernel/kernel_api.py:157-180): failed divisions deactivate their
+    elements.  The fast map kernel keeps one flag per element, which is exact
+    when the result is a tile (deactivated elements are not stored) or when only
+    NumPy functions without a domain sit above the divisions; everything else,
+    // % and comparisons go to the general float map."""
+    N = sym.N
+    f = np.float32
+
+    def plan(expr, out_dt="float32", in_dt="float32"):
+        @kernel(work_shape=N, group_shape=256)
+        def k(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], out: Buffer[N, DT]):
+            o, g = gr.work_offset[0], gr.shape[0]
+            gr.store(out[o:], expr(gr.load(a[o:], shape=g), gr.load(b[o:], shape=g)))
+        (p,) = k.plan(FakeDev((1000,), in_dt), FakeDev((1000,), in_dt), FakeDev((1000,), out_dt), ctx=ctx)
+        return p
+
+    # the operator: numpy.ma's division; the function: domain fill, general map
+    p = plan(lambda a, b: a / b)
+    assert p.fn is rt.hcamdLaunchMap and map_program(p) == [("in", 0, 0.0), ("mdiv_in", 1, 0.0)]
+    p = plan(lambda a, b: np.divide(a, b))
+    assert p.fn is rt.hcamdLaunchFMap and fmap_program(p) == [("in", 0, 0.0), ("in", 1, 0.0), ("udiv", 0, 0.0)]
+    assert p.args[-1] == 1                                  # a bare numpy.ma array: stored in full
+    # fp16 tiles: the quotient is tested after rounding to fp16 (bit 8 of the operand form's arg)
+    p = plan(lambda a, b: a / b + np.float16(1), "float16", "float16")
+    assert map_program(p) == [("in", 0, 0.0), ("mdiv_in", 0x101, 0.0), ("addi", 0, 1.0), ("r16", 0, 0.0)]
+    # a function without a domain above the division: plain arithmetic on what numpy.ma
+    # leaves (the dividend), everything stored
+    p = plan(lambda a, b: np.exp(a / b))
+    assert p.fn is rt.hcamdLaunchMap
+    assert [i[0] for i in map_program(p)] == ["in", "mdiv_in", "exp", "clear"]
+    # numpy.sqrt / numpy.log have domains
+    p = plan(lambda a, b: a * np.sqrt(b) + b * np.log(a))
+    assert p.fn is rt.hcamdLaunchMap
+    assert [i[0] for i in map_program(p)] == ["in", "msqrt", "mul_in", "in", "mlog", "mul_in", "add"]
+    p = plan(lambda a, b: np.sqrt(a) + np.log(b))           # a bare array on the left: stored in full
+    assert p.fn is rt.hcamdLaunchFMap and p.args[-1] == 1
+    # ** : numpy.ma.power's check for results that are not finite
+    p = plan(lambda a, b: a ** f(2) / b)
+    assert [i[0] for i in map_program(p)] == ["in", "mul_in", "powchk", "mdiv_in"]
+    # an operator above a division in a result that is stored in full needs numpy.ma's values
+    p = plan(lambda a, b: np.abs(a / b) - b / a)
+    assert p.fn is rt.hcamdLaunchFMap and p.args[-1] == 1
+    assert [i[0] for i in fmap_program(p)] == ["in", "in", "div", "abs", "in", "in", "div", "sub"]
+    # the same shape as a tile (left operand a tile): deactivated elements are not stored
+    p = plan(lambda a, b: a / b + np.abs(b / a))
+    assert p.fn is rt.hcamdLaunchMap
+    # // % and comparisons
+    p = plan(lambda a, b: (a // b) % f(3))
+    assert p.fn is rt.hcamdLaunchFMap and p.args[-1] == 0
+    assert fmap_program(p) == [("in", 0, 0.0), ("in", 1, 0.0), ("floordiv", 0, 0.0), ("const", 0, 3.0),
+                               ("mod", 0, 0.0)]
+    p = plan(lambda a, b: a < b, out_dt="bool")
+    assert p.fn is rt.hcamdLaunchFMap and p.args[8] == rt.U8
+    assert [i[0] for i in fmap_program(p)] == ["in", "in", "lt"]
+    p = plan(lambda a, b: np.add(a, b) * (a - b))            # + as a function: arg bit 1
+    assert p.fn is rt.hcamdLaunchMap                         # nothing can deactivate anything
+    p = plan(lambda a, b: np.add(a // b, b))
+    assert fmap_program(p)[-1] == ("add", 2, 0.0)
+    with pytest.raises(NoNativeKernel, match="floor_divide"):
+        plan(lambda a, b: np.floor_divide(a, b))
