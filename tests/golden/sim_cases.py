@@ -361,6 +361,76 @@ def case_store_forms(api):
     return rec.out
 
 
+def case_float_activity(api):
+    """What the GPU path's float operators are held to: which elements a failed
+    division, remainder or power deactivates, what value numpy.ma leaves there,
+    what NumPy functions make of such tiles, and what a store writes for each
+    kind of result (a tile: active elements only; what a NumPy function or an
+    operator with such a result on its left returns: everything)."""
+    rec = Recorder()
+    dsts = {}
+    for tag, dt, big, tiny in (("f32", np.float32, 3.0e38, 1.5e-38), ("f16", np.float16, 60000.0, 6.2e-5)):
+        a = np.array([4, -9, 0, -0.0, 7, 5.5, -5.5, big, -big, tiny, np.inf, -np.inf, np.nan, 3, -3, 1,
+                      2.5, -7.25, 0, 1e-3], dt)
+        b = np.array([2, 0, 0, 3, -0.0, -2, 2, 1e-3, big, big, 2, 0, 1, np.nan, np.inf, -np.inf,
+                      0.5, 3, -4, tiny], dt)
+        n = len(a)
+        K = dt
+        bodies = [
+            ("div", lambda x, y: x / y), ("floordiv", lambda x, y: x // y), ("mod", lambda x, y: x % y),
+            ("div_chain", lambda x, y: x / y * K(2) + K(1)),
+            ("pow2", lambda x, y: x ** K(2)), ("pow_half", lambda x, y: x ** K(0.5)),
+            ("pow2_div", lambda x, y: x ** K(2) / y),
+            ("neg_div", lambda x, y: -(x / y)), ("abs_builtin_div", lambda x, y: abs(x / y)),
+            ("np_divide", lambda x, y: np.divide(x, y)), ("np_remainder", lambda x, y: np.remainder(x, y)),
+            ("np_abs_div", lambda x, y: np.abs(x / y)), ("np_sqrt", lambda x, y: np.sqrt(x)),
+            ("np_log", lambda x, y: np.log(x)), ("np_sqrt_div", lambda x, y: np.sqrt(x / y)),
+            ("np_maximum_divs", lambda x, y: np.maximum(x / y, y / x)),
+            ("np_minimum", lambda x, y: np.minimum(x, y)), ("np_maximum", lambda x, y: np.maximum(x, y)),
+            ("np_add_div", lambda x, y: np.add(x / y, y)),
+            ("np_abs_div_times2", lambda x, y: np.abs(x / y * K(2))),
+            ("bare_left_sub", lambda x, y: np.abs(x / y) - y / x),
+            ("bare_left_mul", lambda x, y: np.abs(x) * (y / x)),
+            ("bare_left_div", lambda x, y: np.abs(x) / y),
+            ("bare_right_add", lambda x, y: x / y + np.abs(y / x)),
+            ("tile_times_np_sqrt", lambda x, y: x * np.sqrt(y)),
+            ("np_sqrt_times_tile", lambda x, y: np.sqrt(x) * y),
+            ("bare_plus_scalar", lambda x, y: np.abs(x / y) + K(1)),
+            ("npscalar_left_mul", lambda x, y: K(2) * (x / y)),
+            ("floordiv_mod", lambda x, y: (x // y) * y + x % y),
+            ("rint_floordiv_minus_mod", lambda x, y: np.rint(x // y) - x % y),
+            ("lt", lambda x, y: x < y), ("le", lambda x, y: x <= y), ("eq", lambda x, y: x == y),
+            ("ne", lambda x, y: x != y), ("ge", lambda x, y: x >= y), ("gt", lambda x, y: x > y),
+            ("div_gt", lambda x, y: x / y > K(0.5)),
+            ("lt_as_factor", lambda x, y: (x < y).astype(dt) * x),
+            ("sum_div", lambda x, y: (x / y).sum()), ("np_abs_div_sum", lambda x, y: np.abs(x / y).sum()),
+        ]
+        # tiles four elements wider than the arrays: every tile has a real mask
+        # (the reference cannot read or store a comparison of two tiles that
+        # numpy.ma gave its scalar "no mask", kernel_api.py:93-103,117-119)
+        dst = np.full((len(bodies), n + 4), 7.5, dt)
+        flags = np.zeros((len(bodies), n + 4), bool)
+        flags[:, ::3] = True
+
+        def body(gr, a, b, dst, flags, bodies=bodies, tag=tag, n=n):
+            x, y = gr.load(a, shape=n + 4), gr.load(b, shape=n + 4)
+            for row, (name, fn) in enumerate(bodies):
+                t = rec.attempt(f"{tag}.{name}", lambda: fn(x, y))
+                if t is None or np.ndim(t) == 0 or "_left_" in name:
+                    continue                    # (the reference has no reflected operators)
+                try:
+                    gr.store(flags[row] if np.asarray(t).dtype == bool else dst[row], t)
+                except Exception as e:                  # noqa: BLE001
+                    rec.out[f"{tag}.{name}.store_raises"] = _text(type(e).__name__)
+
+        with np.errstate(all="ignore"), warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            _one_group(api, body, a, b, dst, flags, group=n)
+        rec.array(f"{tag}.dst", dst)
+        rec.array(f"{tag}.flags", flags)
+    return rec.out
+
+
 CASES = {
     "inplace_partial": case_inplace_partial,
     "load_from_masked": case_load_from_masked,
@@ -370,6 +440,7 @@ CASES = {
     "scalar_promotion": case_scalar_promotion,
     "operators": case_operators,
     "store_forms": case_store_forms,
+    "float_activity": case_float_activity,
 }
 
 
