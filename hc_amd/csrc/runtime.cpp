@@ -2834,6 +2834,7 @@ int launchGemm(OlQueue q, bool half, const void *a, size_t lda, const void *bt,
       {"hcamd_gemm_bf16_p256x256_w2x4_hinted", 256, 256, 512},      // 24: half-step order left to the compiler
       {"hcamd_gemm_bf16_p256x256_w2x4_loads_early", 256, 256, 512}, // 25: loads in the first half of the MFMAs
       {"hcamd_gemm_bf16_probe_b_direct", 256, 256, 512},            // 26: measurement only
+      {"hcamd_gemm_bf16_p256x256_w2x2", 256, 256, 256},             // 27: four waves, 128 x 128 each
   };
   constexpr int kGeneral = 6;
   constexpr int kFirstPipelined = 7; // variants from here need K >= 128
