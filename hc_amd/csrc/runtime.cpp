@@ -1431,20 +1431,14 @@ int hcamdLaunchIMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
   }
   if (rows == 0 || cols == 0)
     return 0;
-  if (rows > 65535 && cols > 1) {
-    dev->report("%s: more than 65535 rows", who);
-    return 1;
-  }
-  if (rows > 65535) { // a column vector: walk it as one row when it is dense
+  if (rows > 65535 && cols == 1) { // a column vector: walk it as one row when it is dense
     bool dense = ldo == 1;
     for (size_t i = 0; i < nInputs; ++i)
       dense = dense && inputLd[i] == 1;
-    if (!dense) {
-      dev->report("%s: more than 65535 rows", who);
-      return 1;
+    if (dense) {
+      cols = rows;
+      rows = 1;
     }
-    cols = rows;
-    rows = 1;
   }
   bool vec = outType == HCAMD_I32 && aligned16(out) && (rows == 1 || ldo % 4 == 0);
   for (size_t i = 0; i < nInputs; ++i) {
@@ -1475,9 +1469,19 @@ int hcamdLaunchIMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
   if (!k)
     return 1;
   void *args[] = {&a};
-  const size_t grid[3] = {ceilDiv(ceilDiv(cols, (size_t)4), (size_t)256), rows, 1};
   const size_t block[3] = {256, 1, 1};
-  return launch(queue, k, grid, block, args, 0);
+  // blockIdx.y numbers the rows: at most 65535 of them per launch
+  for (size_t r0 = 0; r0 < rows; r0 += 65535) {
+    const size_t nr = std::min(rows - r0, (size_t)65535);
+    a.rows = nr;
+    for (size_t i = 0; i < nInputs; ++i)
+      a.in[i] = static_cast<const char *>(inputs[i]) + r0 * inputLd[i] * sizeof(int32_t);
+    a.out = static_cast<char *>(out) + r0 * ldo * (outType == HCAMD_U8 ? 1 : sizeof(int32_t));
+    const size_t grid[3] = {ceilDiv(ceilDiv(cols, (size_t)4), (size_t)256), nr, 1};
+    if (int rc = launch(queue, k, grid, block, args, 0))
+      return rc;
+  }
+  return 0;
 }
 
 namespace {
@@ -1544,16 +1548,14 @@ int hcamdLaunchFMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
   }
   if (rows == 0 || cols == 0)
     return 0;
-  if (rows > 65535) { // a column vector: walk it as one row when it is dense
-    bool dense = cols == 1 && ldo == 1;
+  if (rows > 65535 && cols == 1) { // a column vector: walk it as one row when it is dense
+    bool dense = ldo == 1;
     for (size_t i = 0; i < nInputs; ++i)
       dense = dense && inputLd[i] == 1;
-    if (!dense) {
-      dev->report("%s: more than 65535 rows", who);
-      return 1;
+    if (dense) {
+      cols = rows;
+      rows = 1;
     }
-    cols = rows;
-    rows = 1;
   }
   // a row of four-element pieces: fp32 pieces are 16 bytes, fp16 pieces 8
   auto piece_ok = [&](const void *p, int type, size_t ld) {
@@ -1596,9 +1598,21 @@ int hcamdLaunchFMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
   if (!k)
     return 1;
   void *args[] = {&a};
-  const size_t grid[3] = {ceilDiv(ceilDiv(cols, (size_t)4), (size_t)256), rows, 1};
   const size_t block[3] = {256, 1, 1};
-  return launch(queue, k, grid, block, args, 0);
+  const size_t outSize = outType == HCAMD_F32 ? 4 : outType == HCAMD_F16 ? 2 : 1;
+  // blockIdx.y numbers the rows: at most 65535 of them per launch
+  for (size_t r0 = 0; r0 < rows; r0 += 65535) {
+    const size_t nr = std::min(rows - r0, (size_t)65535);
+    a.rows = nr;
+    for (size_t i = 0; i < nInputs; ++i)
+      a.in[i] = static_cast<const char *>(inputs[i]) +
+                r0 * inputLd[i] * (inputTypes[i] == HCAMD_F16 ? 2 : 4);
+    a.out = static_cast<char *>(out) + r0 * ldo * outSize;
+    const size_t grid[3] = {ceilDiv(ceilDiv(cols, (size_t)4), (size_t)256), nr, 1};
+    if (int rc = launch(queue, k, grid, block, args, 0))
+      return rc;
+  }
+  return 0;
 }
 
 int hcamdLaunchMapSum(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,

@@ -298,6 +298,34 @@ def test_imap_zero_divisors_are_left_alone_and_bad_programs_refused(ctx):
             rt.plan_imap(prog, [x], out).launch(sync=True)
 
 
+def test_imap_and_fmap_take_more_rows_than_one_grid_dimension_holds(ctx):
+    """blockIdx.y numbers the rows (at most 65535 per launch): taller windows are walked in blocks."""
+    rows, cols, ld = 70_001, 3, 5
+    rng = np.random.default_rng(9)
+    ai = rng.integers(-1000, 1000, (rows, ld)).astype(np.int32)
+    bi = rng.integers(1, 50, (rows, ld)).astype(np.int32)
+    out = poisoned((rows, ld), np.int32)
+    view = lambda d: _View(d, (rows, cols), 0, (ld, 1))
+    dai, dbi = dev(ai), dev(bi)                      # (a view does not keep its array alive)
+    rt.plan_imap([I("in", 0), I("in", 1), I("floordiv")], [view(dai), view(dbi)], view(out)).launch(sync=True)
+    got = out.to_host()
+    assert_array_equal(got[:, :cols], ai[:, :cols] // bi[:, :cols])
+    assert (got[:, cols:].view(np.uint32) == POISON32).all()
+    af = rng.standard_normal((rows, ld)).astype(np.float32)
+    bf = rng.integers(-2, 3, (rows, ld)).astype(np.float32)
+    outf = poisoned((rows, ld), np.float32)
+    daf, dbf = dev(af), dev(bf)
+    rt.plan_fmap([("in", 0, 0.0), ("in", 1, 0.0), ("div", 0, 0.0)], [view(daf), view(dbf)], view(outf),
+                 [rt.F32, rt.F32, rt.F32]).launch(sync=True)
+    gotf = outf.to_host()
+    ok = bf[:, :cols] != 0
+    with np.errstate(all="ignore"):
+        want = af[:, :cols] / bf[:, :cols]
+    assert_array_equal(gotf[:, :cols][ok], (want + np.float32(0) * af[:, :cols])[ok])
+    assert (gotf[:, :cols][~ok].view(np.uint32) == POISON32).all() and (~ok).sum() > 10_000
+    assert (gotf[:, cols:].view(np.uint32) == POISON32).all()
+
+
 def _ma_special(rng, n, dtype):
     big, tiny = (3.0e38, 1.5e-38) if dtype == np.float32 else (60000.0, 6.2e-5)
     x = (rng.standard_normal(n) * 4).astype(dtype)
