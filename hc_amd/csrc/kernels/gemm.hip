@@ -266,7 +266,7 @@ __device__ __forceinline__ Acc mfma_block(V b, V a, Acc c) {
 // but one before MFMA LF + v * LS; RS == 0 leaves the order to the compiler
 // under sched_group_barrier hints.
 template <class E, int BM, int BN, int WM, int WN, int MF, bool EDGE = false, int EPI = 0,
-          bool PRIO = false, int PROBE = 0, int STAGE = 0, int RS = 0, int LF = 1, int LS = 2>
+          bool PRIO = false, int PROBE = 0, int STAGE = 0, int RS = 0, int LF = 1, int LS = 2, int ORDER = 2>
 __device__ __forceinline__ void gemm_tile_pipelined(
     const E *__restrict__ A, size_t lda, const E *__restrict__ Bt, size_t ldb,
     E *__restrict__ C, size_t ldc, int M, int N, int K) {
@@ -551,10 +551,14 @@ __device__ __forceinline__ void gemm_tile_pipelined(
     static_assert(RF + (kReads - 1) * S / kReads < kMfma, "every LDS read has its MFMA");
     const unsigned char *rbase = lds + rbuf * kStageBytes + (rks ? coff[1][0] : coff[0][0]);
 #pragma unroll
-    for (int i = 0; i < kMI; ++i)
-#pragma unroll
-      for (int j = 0; j < kNI; ++j) {
-        const int slot = i * kNI + j;
+    for (int slot = 0; slot < kMI * kNI; ++slot) {
+      {
+        // ORDER 0: the four Bt blocks under one A block, then the next A block;
+        // 1: the eight A blocks under one Bt block; 2: as 0 in a serpentine (every
+        // other A block takes the Bt blocks in reverse: consecutive MFMAs then
+        // always share an operand; 1 % faster than 0, measured)
+        const int i = ORDER == 1 ? slot % kMI : slot / kNI;
+        const int j = ORDER == 1 ? slot / kMI : ORDER == 2 && (slot / kNI) % 2 ? kNI - 1 - slot % kNI : slot % kNI;
         if (do_read) {
 #pragma unroll
           for (int r = 0; r < kReads; ++r)
@@ -570,6 +574,7 @@ __device__ __forceinline__ void gemm_tile_pipelined(
         acc[i][j] = mfma_block<E, MF>(fb[U][0][j], fa[U][0][i], acc[i][j]);
         __builtin_amdgcn_sched_barrier(0);
       }
+    }
   };
 
   // Order inside a half-step: one LDS read per MFMA from the start, so the last
