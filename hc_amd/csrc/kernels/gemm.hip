@@ -557,8 +557,12 @@ __device__ __forceinline__ void gemm_tile_pipelined(
         // 1: the eight A blocks under one Bt block; 2: as 0 in a serpentine (every
         // other A block takes the Bt blocks in reverse: consecutive MFMAs then
         // always share an operand; 1 % faster than 0, measured)
-        const int i = ORDER == 1 ? slot % kMI : slot / kNI;
-        const int j = ORDER == 1 ? slot / kMI : ORDER == 2 && (slot / kNI) % 2 ? kNI - 1 - slot % kNI : slot % kNI;
+        const int i = ORDER == 1 ? slot % kMI
+                      : ORDER == 3 ? ((slot / kMI) % 2 ? kMI - 1 - slot % kMI : slot % kMI)
+                                   : slot / kNI;
+        const int j = (ORDER == 1 || ORDER == 3) ? slot / kMI
+                      : ORDER == 2 && (slot / kNI) % 2 ? kNI - 1 - slot % kNI
+                                                       : slot % kNI;
         if (do_read) {
 #pragma unroll
           for (int r = 0; r < kReads; ++r)
@@ -851,7 +855,12 @@ HCAMD_GEMM_PS(hcamd_gemm_bf16_p256x256_w2x4_loads_early, __bf16, 256, 256, 2, 4,
 HCAMD_GEMM_PS(hcamd_gemm_bf16_p256x256_w2x4_stage_a, __bf16, 256, 256, 2, 4, 16, 1, 0, 1, 2)
 // four waves with 128 x 128 each (one wave per SIMD, the accumulators in the
 // 256 AGPRs): a third less LDS operand traffic, the same speed within noise
-HCAMD_GEMM_PS(hcamd_gemm_bf16_p256x256_w2x2, __bf16, 256, 256, 2, 2, 16, 0, 24, 1, 4)
+// (plain MFMA order: the serpentine costs this build 30 %)
+extern "C" __global__ __launch_bounds__(256) void hcamd_gemm_bf16_p256x256_w2x2(
+    const __bf16 *A, size_t lda, const __bf16 *Bt, size_t ldb, __bf16 *C, size_t ldc, int M, int N, int K) {
+  gemm_tile_pipelined<__bf16, 256, 256, 2, 2, 16, false, 2, false, 0, 0, 24, 1, 4, 0>(A, lda, Bt, ldb, C, ldc, M,
+                                                                                    N, K);
+}
 // measurement builds whose output is not the product
 HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_mfma_only, 1)
 HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_no_vmwait, 2)
