@@ -847,10 +847,10 @@ class _MapCompiler:
             a, b = t.args
             if _const(b):
                 self.emit(a, out)
-                out.append((fwd + "i", flag, _round_to(b.attrs["value"], t.dtype_name)))
+                out.append((fwd + "i", flag << 8, _round_to(b.attrs["value"], t.dtype_name)))
             elif _const(a):
                 self.emit(b, out)
-                out.append((rev + "i", flag, _round_to(a.attrs["value"], t.dtype_name)))
+                out.append((rev + "i", flag << 8, _round_to(a.attrs["value"], t.dtype_name)))
             elif _leaf(b) is not None:              # operand forms: one dispatch, no push
                 self.emit(a, out)
                 out.append((fwd + "_in", self.operand(_leaf(b)) | (flag << 8), 0.0))
@@ -1349,6 +1349,10 @@ class _RowCompiler(_MapCompiler):
     def program(self, t: Tile, scalar: bool = False) -> list:
         self.prepare(t, scalar)
         self._scalar_mode = scalar
+        # numpy.ma's rules for / ** sqrt log in the element-wise stages (stores
+        # skip, sums and maxima leave out what they deactivate); arithmetic on
+        # row scalars stays plain
+        self.masked = not scalar
         self.need_cache = {}
         if not self.supported(t):
             raise NoNativeKernel(f"{t!r} is not an expression of float32 / float16 tiles, row "
@@ -1357,7 +1361,12 @@ class _RowCompiler(_MapCompiler):
             raise NoNativeKernel("expression needs an evaluation stack deeper than "
                                  f"{rt.MAP_STACK_DEPTH}")
         out: list = []
-        self.emit(t, out)
+        try:
+            self.emit(t, out)
+        except _NeedsEntryMasks:               # numpy.divide as a function: plain arithmetic
+            self.masked = False
+            out = []
+            self.emit(t, out)
         return out
 
     def slot_of(self, t: Tile):
@@ -1430,14 +1439,20 @@ class _RowCompiler(_MapCompiler):
             a, b = t.args
             sa, sb = self.slot_of(a), self.slot_of(b)
             if sb is not None or sa is not None:
+                mdiv = self.masked and t.op == "div" and not t.attrs.get("func")
+                if mdiv:
+                    fwd, rev = "mdiv", "rmdiv"
+                flag = (0x100 if t.dtype_name == "float16" else 0) if mdiv else 0
                 if sb is not None:
                     self.emit(a, out)
-                    out.append((fwd + "_red", sb, 0.0))
+                    out.append((fwd + "_red", sb | flag, 0.0))
                 else:
                     self.emit(b, out)
-                    out.append((rev + "_red", sa, 0.0))
-                if t.dtype_name == "float16" and t.op not in _MAP_EXACT:
+                    out.append((rev + "_red", sa | flag, 0.0))
+                if t.dtype_name == "float16" and t.op not in _MAP_EXACT and not mdiv:
                     out.append(("r16", 0, 0.0))
+                if self.masked and t.attrs.get("pow"):
+                    out.append(("powchk", 0, 0.0))
                 return
         super().emit(t, out)
 
@@ -1487,6 +1502,8 @@ def match_rows(dst_view, value, n_groups):
         comp.stages.append(("store_col", 0, program))
     else:
         program = comp.program(value)
+        if value.attrs.get("plain") and _maybe_masked(value):
+            program.append(("clear", 0, 0.0))  # a bare numpy.ma array: every value is written
         comp.stages.append(("store", 0, program))
     if len(comp.stages) > rt.ROW_MAX_STAGES:
         raise NoNativeKernel(f"the expression needs {len(comp.stages)} passes over the rows "

@@ -84,21 +84,22 @@ enum : uint32_t {
   OP_RSUB_IN = 33, // operand - top
   OP_RDIV_IN = 34, // operand / top
   OP_COUNT = 35,
-  // 35 .. 43 are the row programs' scalar forms (below)
   // The tile operator `/` as numpy.ma computes it: a quotient that is not finite
   // (a zero divisor gives one) deactivates its element, whose value becomes the
-  // dividend.  `arg` bit 8 (MDIV_IN forms) or any `arg` (others): the tile is
-  // fp16 and the quotient is rounded to fp16 before the test.
-  OP_MDIV = 44,
-  OP_RMDIV = 45,
-  OP_MDIVI = 46,
-  OP_RMDIVI = 47,
-  OP_MDIV_IN = 48,
-  OP_RMDIV_IN = 49,
-  OP_CLEAR = 50,  // every element active again (a NumPy function returns a plain array)
-  OP_POWCHK = 51, // numpy.ma.power: a result that is not finite deactivates, value 1e20
-  OP_MSQRT = 52,  // numpy.sqrt of a tile: x < 0 deactivates, value 0
-  OP_MLOG = 53,   // numpy.log of a tile: x <= 0 deactivates, value 1
+  // dividend.  `arg` bit 8 (any `arg` for MDIV / RMDIV): the tile is fp16 and
+  // the quotient is rounded to fp16 before the test.
+  OP_MDIV = 35,
+  OP_RMDIV = 36,
+  OP_MDIVI = 37,
+  OP_RMDIVI = 38,
+  OP_MDIV_IN = 39,
+  OP_RMDIV_IN = 40,
+  OP_CLEAR = 41,  // every element active again (a NumPy function returns a plain array)
+  OP_POWCHK = 42, // numpy.ma.power: a result that is not finite deactivates, value 1e20
+  OP_MSQRT = 43,  // numpy.sqrt of a tile: x < 0 deactivates, value 0
+  OP_MLOG = 44,   // numpy.log of a tile: x <= 0 deactivates, value 1
+  // 45 .. 55 are the row programs' scalar forms (below): the highest opcodes,
+  // so that one comparison finds them
 };
 
 struct Instr {
@@ -308,7 +309,7 @@ __device__ __forceinline__ void do_masked(StackT<N> &r, const RawT<N> &raw, uint
       default: unpack(raw, 3, f16_mask & 8, t); break;
       }
     }
-    const bool half = (OP == OP_MDIVI || OP == OP_RMDIVI) ? arg != 0 : (arg & 0x100u) != 0;
+    const bool half = (arg & 0x100u) != 0;
     if constexpr (OP == OP_MDIVI || OP == OP_MDIV_IN)
       masked_div(r, r.st[SP - 1], r.st[SP - 1], t, half);
     else
@@ -1160,9 +1161,11 @@ constexpr int kMaxStages = 16;
 constexpr int kRowProg = 128;
 constexpr int kRowN = 8; // elements per lane per run of a stage's program (16: registers cost more than the halved dispatch gains)
 enum : uint32_t {
-  OP_RED = 35,     // push row scalar `arg`
-  OP_ADD_RED = 36, // top = top op row scalar `arg`, in the order of OP_ADD_IN..
-  OP_RDIV_RED = 43,
+  OP_RED = 45,     // push row scalar `arg`
+  OP_ADD_RED = 46, // top = top op row scalar `arg`, in the order of OP_ADD_IN..
+  OP_RDIV_RED = 53,
+  OP_MDIV_RED = 54,  // top / row scalar and row scalar / top under numpy.ma's rule
+  OP_RMDIV_RED = 55, // (`arg` bits 0..3: the scalar, bit 8: fp16)
 };
 enum : uint32_t { ST_SUM = 0, ST_MAX = 1, ST_MIN = 2, ST_SCALAR = 3, ST_STORE = 4, ST_STORE_COL = 5 };
 
@@ -1170,7 +1173,8 @@ struct Stage {
   uint16_t begin, end; // instructions [begin, end)
   uint8_t kind, dst;
   uint8_t load_mask; // operands this stage reads
-  uint8_t pad[5];
+  uint8_t masked;    // the program has numpy.ma's division / domain forms: honour the inactive bits
+  uint8_t pad[4];
 };
 
 struct RowArgs {
@@ -1210,6 +1214,7 @@ __device__ __forceinline__ void run_stage(const RowArgs &a, uint32_t begin, uint
                                           const RawT<kRowN> &raw, StackT<kRowN> &r,
                                           uint32_t reds) {
   int sp = 0;
+  r.bad = 0;
   Instr next = a.prog[begin & (kRowProg - 1)];
   for (uint32_t pc = begin; pc < end; ++pc) {
     const Instr cur = next;
@@ -1223,7 +1228,9 @@ __device__ __forceinline__ void run_stage(const RowArgs &a, uint32_t begin, uint
     uint32_t imm_bits = __builtin_bit_cast(uint32_t, cur.imm);
     if (op >= OP_RED) {
       imm_bits = __builtin_amdgcn_readlane(reds, arg & (kMaxRed - 1));
-      op = op == OP_RED ? (uint32_t)OP_CONST : op - OP_ADD_RED + OP_ADDI;
+      op = op == OP_RED        ? (uint32_t)OP_CONST
+           : op >= OP_MDIV_RED ? op - OP_MDIV_RED + OP_MDIVI
+                               : op - OP_ADD_RED + OP_ADDI;
     }
     asm volatile("" : "+s"(op), "+s"(imm_bits));
     const float imm = __builtin_bit_cast(float, imm_bits);
@@ -1379,7 +1386,32 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
       run_stage(a, st.begin, st.end, raw, r, reds);
       // a wave whose lanes all hold whole chunks folds them without masks
       const bool all_whole = __builtin_amdgcn_ballot_w64(at.n_valid != kRowN) == 0;
-      if (kind == ST_STORE) {
+      if (st.masked && per_element) {
+        // a stage with numpy.ma's forms (uniform: the host marks it): elements
+        // that a division or a domain function deactivated are neither stored
+        // nor folded
+        const bool whole_chunk = kind == ST_STORE && ((a.vec_mask >> 8) & 1) && at.n_valid == kRowN &&
+                                 r.bad == 0;
+        if (whole_chunk) {
+#pragma unroll
+          for (int j = 0; j < kRowN / 8; ++j)
+            store_chunk(orow, out_f16, at.first / 8 + j, r.st[0] + 8 * j);
+        }
+#pragma unroll
+        for (int e = 0; e < kRowN; ++e) {
+          const bool take = (uint32_t)e < at.n_valid && !((r.bad >> e) & 1u);
+          if (kind == ST_STORE) {
+            if (take && !whole_chunk)
+              store_elem(orow, out_f16, at.first + e * at.step, r.st[0][e]);
+          } else if (kind == ST_SUM) {
+            acc += take ? r.st[0][e] : 0.0f;
+          } else if (kind == ST_MAX) {
+            acc = take ? nan_max(acc, r.st[0][e]) : acc;
+          } else {
+            acc = take ? nan_min(acc, r.st[0][e]) : acc;
+          }
+        }
+      } else if (kind == ST_STORE) {
         if (((a.vec_mask >> 8) & 1) && at.n_valid == kRowN) {
 #pragma unroll
           for (int j = 0; j < kRowN / 8; ++j)
@@ -1444,10 +1476,10 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
 } // namespace
 
 extern "C" __global__ __launch_bounds__(256)
-__attribute__((amdgpu_waves_per_eu(2, 4))) void hcamd_row_program_w256(const RowArgs a) {
+__attribute__((amdgpu_waves_per_eu(4, 4))) void hcamd_row_program_w256(const RowArgs a) {
   row_program<256>(a);
 }
 extern "C" __global__ __launch_bounds__(256)
-__attribute__((amdgpu_waves_per_eu(2, 4))) void hcamd_row_program_w64(const RowArgs a) {
+__attribute__((amdgpu_waves_per_eu(4, 4))) void hcamd_row_program_w64(const RowArgs a) {
   row_program<64>(a);
 }

@@ -1182,7 +1182,7 @@ int launchMap(OlQueue q, bool sum, const HcamdMapInstr *prog, size_t nInstr,
       return 1;
     }
     const bool maskedOperand = prog[i].op == HCAMD_MAP_MDIV_IN || prog[i].op == HCAMD_MAP_RMDIV_IN;
-    hasMasked = hasMasked || prog[i].op >= HCAMD_MAP_MDIV;
+    hasMasked = hasMasked || (prog[i].op >= HCAMD_MAP_MDIV && prog[i].op <= HCAMD_MAP_MLOG);
     const bool readsOperand =
         prog[i].op == HCAMD_MAP_IN || maskedOperand ||
         (prog[i].op >= HCAMD_MAP_ADD_IN && prog[i].op <= HCAMD_MAP_RDIV_IN);
@@ -1847,7 +1847,9 @@ namespace {
 // Argument block of the row-program kernels (the same layout as in the device code).
 struct RowStageDev {
   uint16_t begin, end;
-  uint8_t kind, dst, loadMask, pad[5];
+  uint8_t kind, dst, loadMask;
+  uint8_t masked; // the stage has numpy.ma's division / domain forms
+  uint8_t pad[4];
 };
 struct RowArgs {
   const void *in[kMapMaxIn];
@@ -1919,28 +1921,38 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
     for (size_t i = pc; i < pc + st.nInstr; ++i) {
       const unsigned op = prog[i].op;
       int pops, pushes;
-      const bool red = op >= HCAMD_MAP_RED && op <= HCAMD_MAP_RDIV_RED;
+      const bool maskedRed = op == HCAMD_MAP_MDIV_RED || op == HCAMD_MAP_RMDIV_RED;
+      if ((op >= HCAMD_MAP_MDIV && op <= HCAMD_MAP_MLOG && op != HCAMD_MAP_CLEAR) || maskedRed)
+        a.stage[s].masked = 1;
+      const bool red = op >= HCAMD_MAP_RED && op <= HCAMD_MAP_RMDIV_RED;
       if (red)
         pops = op == HCAMD_MAP_RED ? 0 : 1, pushes = 1;
+      else if (perElement)
+        mapStackEffectMasked(op, pops, pushes); // numpy.ma's division forms: element-wise stages only
       else
         mapStackEffect(op, pops, pushes);
       if (pops < 0) {
         dev->report("%s: unknown opcode %u at %zu", who, op, i);
         return 1;
       }
-      const bool readsOperand =
-          op == HCAMD_MAP_IN || (op >= HCAMD_MAP_ADD_IN && op <= HCAMD_MAP_RDIV_IN);
+      const bool maskedIn = op == HCAMD_MAP_MDIV_IN || op == HCAMD_MAP_RMDIV_IN;
+      const bool readsOperand = op == HCAMD_MAP_IN || maskedIn ||
+                                (op >= HCAMD_MAP_ADD_IN && op <= HCAMD_MAP_RDIV_IN);
+      const unsigned index = (maskedIn || maskedRed) ? prog[i].arg & 0xffu : prog[i].arg;
       if (readsOperand) {
-        if (!perElement || prog[i].arg >= nInputs) {
+        if (!perElement || index >= nInputs) {
           dev->report("%s: operand %u at %zu (%zu given; scalar stages read none)", who,
-                      prog[i].arg, i, nInputs);
+                      index, i, nInputs);
           return 1;
         }
-        usedIn[s] |= 1u << prog[i].arg;
+        usedIn[s] |= 1u << index;
       }
-      if (red && (prog[i].arg >= HCAMD_ROW_MAX_SCALARS || !((written >> prog[i].arg) & 1))) {
-        dev->report("%s: row scalar %u read at %zu before it is written", who,
-                    prog[i].arg, i);
+      if (maskedRed && !perElement) {
+        dev->report("%s: opcode %u at %zu in a scalar stage", who, op, i);
+        return 1;
+      }
+      if (red && (index >= HCAMD_ROW_MAX_SCALARS || !((written >> index) & 1))) {
+        dev->report("%s: row scalar %u read at %zu before it is written", who, index, i);
         return 1;
       }
       if (sp < pops) {

@@ -515,13 +515,14 @@ MAP_OPS = {"in": 1, "const": 2, "add": 3, "sub": 4, "mul": 5, "div": 6, "max": 7
            "exp": 23, "log": 24, "tanh": 25, "r16": 26, "add_in": 27, "sub_in": 28,
            "mul_in": 29, "div_in": 30, "max_in": 31, "min_in": 32, "rsub_in": 33,
            "rdiv_in": 34,
-           # the tile operator `/` under numpy.ma's rule (element-wise map and its sum only)
-           "mdiv": 44, "rmdiv": 45, "mdivi": 46, "rmdivi": 47, "mdiv_in": 48, "rmdiv_in": 49,
-           "clear": 50, "powchk": 51, "msqrt": 52, "mlog": 53}
+           # the tile operator `/` under numpy.ma's rule, ** and the domain functions
+           "mdiv": 35, "rmdiv": 36, "mdivi": 37, "rmdivi": 38, "mdiv_in": 39, "rmdiv_in": 40,
+           "clear": 41, "powchk": 42, "msqrt": 43, "mlog": 44}
 MAP_MAX_INPUTS, MAP_MAX_INSTRS, MAP_STACK_DEPTH = 4, 32, 4
 # Row programs (hcamdLaunchRowProgram): opcodes that read row scalars, stage kinds, limits
-MAP_OPS.update({"red": 35, "add_red": 36, "sub_red": 37, "mul_red": 38, "div_red": 39,
-                "max_red": 40, "min_red": 41, "rsub_red": 42, "rdiv_red": 43})
+MAP_OPS.update({"red": 45, "add_red": 46, "sub_red": 47, "mul_red": 48, "div_red": 49,
+                "max_red": 50, "min_red": 51, "rsub_red": 52, "rdiv_red": 53,
+                "mdiv_red": 54, "rmdiv_red": 55})
 ROW_KINDS = {"sum": 0, "max": 1, "min": 2, "scalar": 3, "store": 4, "store_col": 5}
 ROW_MAX_STAGES, ROW_MAX_SCALARS, ROW_MAX_INSTRS = 16, 16, 128
 F32, F16, BF16 = 0, 1, 2

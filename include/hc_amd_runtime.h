@@ -321,26 +321,27 @@ enum HcamdMapOp {
   HCAMD_MAP_MIN_IN = 32,
   HCAMD_MAP_RSUB_IN = 33, /* operand - top */
   HCAMD_MAP_RDIV_IN = 34, /* operand / top */
-  /* 35 .. 43: the row programs' scalar forms (enum HcamdRowOp) */
   /* The tile OPERATOR `/`, as numpy.ma computes it
    * (python/hckernel/kernel_api.py:157-180 forwards it to numpy.ma): a quotient
    * that is not finite (a zero divisor gives one) makes its element inactive,
    * nothing is stored or summed for it, and its value becomes 0 + dividend.
    * The forms mirror DIV / RDIV; for an fp16 tile the quotient is rounded to
-   * fp16 before the test: `arg` != 0 says so (the *_IN forms: bit 8 of `arg`,
-   * whose low bits are the operand index).  HCAMD_MAP_DIV and its forms stay
-   * the plain quotient, which is numpy.divide called as a function.  hcamdLaunchMap
-   * and hcamdLaunchMapSum only. */
-  HCAMD_MAP_MDIV = 44,
-  HCAMD_MAP_RMDIV = 45,
-  HCAMD_MAP_MDIVI = 46,
-  HCAMD_MAP_RMDIVI = 47,
-  HCAMD_MAP_MDIV_IN = 48,
-  HCAMD_MAP_RMDIV_IN = 49,
-  HCAMD_MAP_CLEAR = 50,  /* every element active again (ends a program whose result is stored in full) */
-  HCAMD_MAP_POWCHK = 51, /* numpy.ma.power: top not finite -> inactive, value 1e20 */
-  HCAMD_MAP_MSQRT = 52,  /* numpy.sqrt of a tile: x < 0 -> inactive, value 0 */
-  HCAMD_MAP_MLOG = 53    /* numpy.log of a tile: x <= 0 -> inactive, value 1 */
+   * fp16 before the test: bit 8 of `arg` says so (MDIV / RMDIV: any `arg`; the
+   * low bits of the *_IN forms are the operand index).  HCAMD_MAP_DIV and its
+   * forms stay the plain quotient.  hcamdLaunchMap, hcamdLaunchMapSum and the
+   * element-wise stages of hcamdLaunchRowProgram (whose sums, maxima and
+   * minima leave inactive elements out, as numpy.ma's reductions do). */
+  HCAMD_MAP_MDIV = 35,
+  HCAMD_MAP_RMDIV = 36,
+  HCAMD_MAP_MDIVI = 37,
+  HCAMD_MAP_RMDIVI = 38,
+  HCAMD_MAP_MDIV_IN = 39,
+  HCAMD_MAP_RMDIV_IN = 40,
+  HCAMD_MAP_CLEAR = 41,  /* every element active again (ends a program whose result is stored in full) */
+  HCAMD_MAP_POWCHK = 42, /* numpy.ma.power: top not finite -> inactive, value 1e20 */
+  HCAMD_MAP_MSQRT = 43,  /* numpy.sqrt of a tile: x < 0 -> inactive, value 0 */
+  HCAMD_MAP_MLOG = 44    /* numpy.log of a tile: x <= 0 -> inactive, value 1 */
+  /* 45 .. 55: the row programs' scalar forms (enum below) */
 };
 #define HCAMD_MAP_MAX_INPUTS 4
 #define HCAMD_MAP_MAX_INSTRS 32
@@ -516,15 +517,19 @@ enum HcamdRowStageKind {
   HCAMD_ROW_STORE_COL = 5
 };
 enum {
-  HCAMD_MAP_RED = 35,     /* push row scalar `arg` */
-  HCAMD_MAP_ADD_RED = 36, /* top = top + row scalar `arg` */
-  HCAMD_MAP_SUB_RED = 37,
-  HCAMD_MAP_MUL_RED = 38,
-  HCAMD_MAP_DIV_RED = 39,
-  HCAMD_MAP_MAX_RED = 40,
-  HCAMD_MAP_MIN_RED = 41,
-  HCAMD_MAP_RSUB_RED = 42, /* scalar - top */
-  HCAMD_MAP_RDIV_RED = 43  /* scalar / top */
+  HCAMD_MAP_RED = 45,     /* push row scalar `arg` */
+  HCAMD_MAP_ADD_RED = 46, /* top = top + row scalar `arg` */
+  HCAMD_MAP_SUB_RED = 47,
+  HCAMD_MAP_MUL_RED = 48,
+  HCAMD_MAP_DIV_RED = 49,
+  HCAMD_MAP_MAX_RED = 50,
+  HCAMD_MAP_MIN_RED = 51,
+  HCAMD_MAP_RSUB_RED = 52, /* scalar - top */
+  HCAMD_MAP_RDIV_RED = 53, /* scalar / top */
+  /* the tile operator / with a row scalar under numpy.ma's rule (see
+   * HCAMD_MAP_MDIV): `arg` bits 0..3 the scalar, bit 8 the fp16 flag */
+  HCAMD_MAP_MDIV_RED = 54, /* top / scalar */
+  HCAMD_MAP_RMDIV_RED = 55 /* scalar / top */
 };
 #define HCAMD_ROW_MAX_STAGES 16
 #define HCAMD_ROW_MAX_SCALARS 16

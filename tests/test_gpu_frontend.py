@@ -1222,3 +1222,60 @@ def test_sum_skips_elements_a_division_deactivated():
     with np.errstate(all="ignore"):
         sim_kernel(work_shape=N, group_shape=256)(body)(a, b, host)
     assert_allclose(host[0], want, rtol=1e-4)
+
+
+def test_row_programs_leave_deactivated_elements_alone():
+    """Row reductions and stores under numpy.ma's rules: a row divided by its own
+    zero sum is left as it was, a sum leaves out the elements a division or a
+    domain function deactivated, and a result that is a bare numpy.ma array
+    (a NumPy function on the left) is written in full."""
+    M, N, GM = sym.M, sym.N, sym.GM
+    f = np.float32
+
+    def normalise(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[M, N, DT], gshape: GM):
+        m0, mb = gr.work_offset[0], gr.shape[0]
+        t = gr.load(x[m0:, :], shape=(mb, N))
+        gr.store(out[m0:, :], t / t.sum(axis=1, keepdims=True))
+
+    def sum_of_quotients(gr: CurrentGroup, x: Buffer[M, N, DT], y: Buffer[M, N, DT], out: Buffer[M, DT],
+                         gshape: GM):
+        m0, mb = gr.work_offset[0], gr.shape[0]
+        a, b = gr.load(x[m0:, :], shape=(mb, N)), gr.load(y[m0:, :], shape=(mb, N))
+        gr.store(out[m0:], (a / b + f(1)).sum(axis=1))
+
+    def log_then_max(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[M, N, DT], gshape: GM):
+        m0, mb = gr.work_offset[0], gr.shape[0]
+        t = gr.load(x[m0:, :], shape=(mb, N))
+        lg = np.log(t)                                    # 1 where t <= 0, and inactive there
+        gr.store(out[m0:, :], t * lg - (t * lg).max(axis=1, keepdims=True))
+
+    def exp_over_sum(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[M, N, DT], gshape: GM):
+        m0, mb = gr.work_offset[0], gr.shape[0]
+        t = gr.load(x[m0:, :], shape=(mb, N))
+        e = np.exp(t)
+        gr.store(out[m0:, :], e / (t * f(0) + t.sum(axis=1, keepdims=True)))   # a bare array on the left
+
+    rng = np.random.default_rng(12)
+    rows, n = 37, 1000
+    x = rng.standard_normal((rows, n)).astype(f)
+    x[3] = 0
+    x[5, ::2] = 1; x[5, 1::2] = -1                        # sums to zero exactly
+    x[7, :10] = -np.abs(x[7, :10])
+    y = rng.integers(-3, 4, (rows, n)).astype(f)
+    deco = dict(work_shape=M, group_shape=4)
+    for body, ins, shape, tol in ((normalise, (x,), (rows, n), 2e-5), (sum_of_quotients, (x, y), (rows,), 2e-4),
+                                  (log_then_max, (x,), (rows, n), 2e-5), (exp_over_sum, (x,), (rows, n), 2e-5)):
+        host = np.full(shape, 7.5, f)
+        dout = rt.to_device(host)
+        kernel(**deco)(body)(*[rt.to_device(v) for v in ins], dout, 4)
+        assert rt.last_kernel_name().startswith("hcamd_row_program"), body.__name__
+        with np.errstate(all="ignore"):
+            sim_kernel(**deco)(body)(*ins, host, 4)
+        got = dout.to_host()
+        untouched = host == f(7.5)
+        assert_array_equal(got == f(7.5), untouched, err_msg=body.__name__)
+        nan = np.isnan(host)
+        assert_array_equal(np.isnan(got), nan, err_msg=body.__name__)
+        assert_allclose(got[~nan], host[~nan], rtol=tol, atol=tol, err_msg=body.__name__)
+        if body is normalise:
+            assert untouched[3].all() and untouched[5].all() and not untouched[0].any()
