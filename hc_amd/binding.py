@@ -810,6 +810,17 @@ class _MapCompiler:
         if self.masked and t.attrs.get("pow"):
             out.append(("powchk", 0, 0.0))
 
+    def emit_whole(self, t: Tile, out: list):
+        """The program of a whole expression where no other kernel can take
+        over: numpy.ma's forms where this kernel has them, plain arithmetic for
+        what it lacks (numpy.divide called as a function)."""
+        try:
+            self.emit(t, out)
+        except _NeedsEntryMasks:
+            self.masked = False
+            del out[:]
+            self.emit(t, out)
+
     def _emit_node(self, t: Tile, out: list):
         half = t.dtype_name == "float16"
         if _is(t, "load"):
@@ -1612,6 +1623,8 @@ class _ColBodyCompiler(_MapCompiler):
     reductions (`temps`: uid of the reduction -> operand slot), which every row
     uses."""
 
+    masked = True                     # numpy.ma's rules: the folds leave out what / ** sqrt log deactivate
+
     def __init__(self, n_groups, temps):
         super().__init__(n_groups)
         self.temps = temps            # uid -> index into the list of temporaries
@@ -1657,7 +1670,7 @@ def _compile_col_reduce(red: Tile, root: Tile, n_groups, temps):
         raise NoNativeKernel("expression needs an evaluation stack deeper than "
                              f"{rt.MAP_STACK_DEPTH}")
     program: list = []
-    comp.emit(body, program)
+    comp.emit_whole(body, program)
     if len(program) > rt.MAP_MAX_INSTRS or not 1 <= len(comp.inputs) <= rt.MAP_MAX_INPUTS:
         raise NoNativeKernel(f"the reduced expression compiles to {len(program)} operations on "
                              f"{len(comp.inputs)} arrays (at most {rt.MAP_MAX_INSTRS} on "
@@ -1810,7 +1823,9 @@ def match_cols_tile(dst_view, value, n_groups):
         raise NoNativeKernel("expression needs an evaluation stack deeper than "
                              f"{rt.MAP_STACK_DEPTH}")
     program: list = []
-    final.emit(value, program)
+    final.emit_whole(value, program)
+    if value.attrs.get("plain") and _maybe_masked(value):
+        program.append(("clear", 0, 0.0))      # a bare numpy.ma array: every value is written
     if len(program) > rt.MAP_MAX_INSTRS or len(final.inputs) > rt.MAP_MAX_INPUTS:
         raise NoNativeKernel(f"the stored expression compiles to {len(program)} operations on "
                              f"{len(final.inputs)} arrays (at most {rt.MAP_MAX_INSTRS} on "

@@ -938,6 +938,7 @@ struct ColArgs {
   uint32_t interleaved; // columns of a block dealt to the lanes one by one
   uint32_t out_vec;     // the result may be written 16 bytes at a time
   uint32_t n_post;
+  uint32_t masked;      // the program has numpy.ma's division / domain forms: inactive elements are left out
   Instr post[kPostProg];
 };
 
@@ -1048,9 +1049,15 @@ __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, 
       }
       run_program(a, raw, a.f16_mask, r);
       if (row0 + u * kWaves * R + sub < row_end) {
+        if (c.masked) { // uniform
 #pragma unroll
-        for (int e = 0; e < kN; ++e)
-          acc[e] = col_fold(c.kind, acc[e], r.st[0][e]);
+          for (int e = 0; e < kN; ++e)
+            acc[e] = ((r.bad >> e) & 1u) ? acc[e] : col_fold(c.kind, acc[e], r.st[0][e]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < kN; ++e)
+            acc[e] = col_fold(c.kind, acc[e], r.st[0][e]);
+        }
       }
     }
   }

@@ -1627,18 +1627,21 @@ namespace {
 // Second argument block of the column-reduction kernels (device layout).
 struct ColArgs {
   float *partial;
-  uint32_t colsPad, band, kind, lanes, interleaved, outVec, nPost;
+  uint32_t colsPad, band, kind, lanes, interleaved, outVec, nPost, masked;
   HcamdMapInstr post[HCAMD_COLS_MAX_POST];
 };
 
 // Stack discipline of a map program: within bounds, one value left, operands
 // below nInputs.
 bool mapProgramOk(Device *dev, const char *who, const HcamdMapInstr *prog, size_t nInstr,
-                  size_t nInputs) {
+                  size_t nInputs, bool allowMasked = false) {
   int sp = 0;
   for (size_t i = 0; i < nInstr; ++i) {
     int pops, pushes;
-    mapStackEffect(prog[i].op, pops, pushes);
+    if (allowMasked)
+      mapStackEffectMasked(prog[i].op, pops, pushes);
+    else
+      mapStackEffect(prog[i].op, pops, pushes);
     if (pops < 0) {
       dev->report("%s: unknown opcode %u at %zu", who, prog[i].op, i);
       return false;
@@ -1737,7 +1740,7 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
     dev->report("%s: unsupported output type %d", who, outType);
     return 1;
   }
-  if (!mapProgramOk(dev, who, prog, nInstr, nInputs) ||
+  if (!mapProgramOk(dev, who, prog, nInstr, nInputs, true) ||
       (nPost && !mapProgramOk(dev, who, post, nPost, 1)))
     return 1;
   if (cols == 0)
@@ -1815,6 +1818,9 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
   a.n_instr = static_cast<uint32_t>(nInstr);
   std::memcpy(a.prog, prog, nInstr * sizeof(HcamdMapInstr));
   c.kind = static_cast<uint32_t>(kind);
+  for (size_t i = 0; i < nInstr; ++i)
+    if (prog[i].op >= HCAMD_MAP_MDIV && prog[i].op <= HCAMD_MAP_MLOG && prog[i].op != HCAMD_MAP_CLEAR)
+      c.masked = 1; // numpy.ma's forms: the folds leave inactive elements out
   c.colsPad = static_cast<uint32_t>(colsPad);
   c.band = static_cast<uint32_t>(band);
   c.lanes = static_cast<uint32_t>(colLanes(cols));

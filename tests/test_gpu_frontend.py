@@ -1279,3 +1279,34 @@ def test_row_programs_leave_deactivated_elements_alone():
         assert_allclose(got[~nan], host[~nan], rtol=tol, atol=tol, err_msg=body.__name__)
         if body is normalise:
             assert untouched[3].all() and untouched[5].all() and not untouched[0].any()
+
+
+def test_column_reductions_leave_deactivated_elements_out():
+    """`(a / b).sum(axis=0)` and `(a / b).max(axis=0)`: numpy.ma's reductions skip
+    the elements a zero divisor deactivated; same body on the GPU and on the host
+    executor."""
+    M, N, GN = sym.M, sym.N, sym.GN
+
+    def body(fn):
+        def k(gr: CurrentGroup, x: Buffer[M, N, DT], y: Buffer[M, N, DT], out: Buffer[N, DT], gn: GN):
+            n0 = gr.id[0] * GN
+            tx, ty = gr.load(x[:, n0:], shape=(M, GN)), gr.load(y[:, n0:], shape=(M, GN))
+            gr.store(out[n0:], fn(tx, ty))
+        return k
+
+    rng = np.random.default_rng(21)
+    rows, n, gn = 777, 200, 64
+    x = rng.standard_normal((rows, n)).astype(np.float32)
+    y = rng.integers(-2, 3, (rows, n)).astype(np.float32)          # a fifth of the divisors are zero
+    deco = dict(work_shape=cdiv(n, gn), group_shape=1, literals={GN})
+    for name, fn in (("sum", lambda a, b: (a / b).sum(axis=0)), ("max", lambda a, b: (a / b).max(axis=0)),
+                     ("sum_sqrt", lambda a, b: np.sqrt(a * b).sum(axis=0)),
+                     ("min_log", lambda a, b: np.log(a * b).min(axis=0))):
+        want = np.zeros(n, np.float32)
+        with np.errstate(all="ignore"):
+            sim_kernel(**deco)(body(fn))(x, y, want, gn)
+        out = rt.DeviceArray((n,), np.float32).fill_bytes32(0xA5A5A5A5)
+        kernel(**deco)(body(fn))(rt.to_device(x), rt.to_device(y), out, gn)
+        assert rt.last_kernel_name().startswith("hcamd_map"), name
+        assert np.isfinite(want).all(), name
+        assert_allclose(out.to_host(), want, rtol=2e-4, atol=2e-4, err_msg=name)
