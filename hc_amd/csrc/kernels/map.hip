@@ -268,9 +268,9 @@ template <int SP, int OP, int N> __device__ __forceinline__ void do_unary(StackT
 __device__ __forceinline__ bool is_finite(float x) { return __builtin_fabsf(x) < INFINITY; }
 // num / den under numpy.ma's rule, into `dst`
 template <int N>
-__device__ __forceinline__ void masked_div(StackT<N> &r, float *dst, const float *num, const float *den,
-                                           bool half) {
-  uint32_t bad = r.bad;
+__device__ __forceinline__ void masked_div(uint32_t &bad_bits, float *dst, const float *num,
+                                           const float *den, bool half) {
+  uint32_t bad = bad_bits;
 #pragma unroll
   for (int e = 0; e < N; ++e) {
     const float n = num[e];
@@ -284,7 +284,32 @@ __device__ __forceinline__ void masked_div(StackT<N> &r, float *dst, const float
     dst[e] = good ? q : 0.0f + n;
     bad |= good ? 0u : (1u << e);
   }
-  r.bad = bad;
+  bad_bits = bad;
+}
+// numpy.sqrt / numpy.log of a tile: outside the domain the element is
+// deactivated and holds numpy.ma's fill value (0 and 1)
+template <bool LOG, int N> __device__ __forceinline__ void domain_fn(uint32_t &bad_bits, float *x) {
+  uint32_t bad = bad_bits;
+#pragma unroll
+  for (int e = 0; e < N; ++e) {
+    const float v = x[e];
+    const bool out = LOG ? v <= 0.0f : v < 0.0f;
+    const float y = LOG ? logf(v) : __builtin_sqrtf(v);
+    x[e] = out ? (LOG ? 1.0f : 0.0f) : y;
+    bad |= out ? (1u << e) : 0u;
+  }
+  bad_bits = bad;
+}
+// numpy.ma.power: a result that is not finite deactivates, value 1e20
+template <int N> __device__ __forceinline__ void powchk_fn(uint32_t &bad_bits, float *x) {
+  uint32_t bad = bad_bits;
+#pragma unroll
+  for (int e = 0; e < N; ++e) {
+    const bool good = is_finite(x[e]);
+    x[e] = good ? x[e] : 1e20f;
+    bad |= good ? 0u : (1u << e);
+  }
+  bad_bits = bad;
 }
 template <int SP, int OP, int N>
 __device__ __forceinline__ void do_masked(StackT<N> &r, const RawT<N> &raw, uint32_t f16_mask, uint32_t arg,
@@ -292,9 +317,9 @@ __device__ __forceinline__ void do_masked(StackT<N> &r, const RawT<N> &raw, uint
   if constexpr (OP == OP_MDIV || OP == OP_RMDIV) {
     if constexpr (SP >= 2) {
       if constexpr (OP == OP_MDIV)
-        masked_div(r, r.st[SP - 2], r.st[SP - 2], r.st[SP - 1], arg != 0);
+        masked_div<N>(r.bad, r.st[SP - 2], r.st[SP - 2], r.st[SP - 1], arg != 0);
       else
-        masked_div(r, r.st[SP - 2], r.st[SP - 1], r.st[SP - 2], arg != 0);
+        masked_div<N>(r.bad, r.st[SP - 2], r.st[SP - 1], r.st[SP - 2], arg != 0);
     }
   } else if constexpr (SP >= 1) {
     float t[N];
@@ -311,36 +336,18 @@ __device__ __forceinline__ void do_masked(StackT<N> &r, const RawT<N> &raw, uint
     }
     const bool half = (arg & 0x100u) != 0;
     if constexpr (OP == OP_MDIVI || OP == OP_MDIV_IN)
-      masked_div(r, r.st[SP - 1], r.st[SP - 1], t, half);
+      masked_div<N>(r.bad, r.st[SP - 1], r.st[SP - 1], t, half);
     else
-      masked_div(r, r.st[SP - 1], t, r.st[SP - 1], half);
+      masked_div<N>(r.bad, r.st[SP - 1], t, r.st[SP - 1], half);
   }
 }
 template <int SP, bool LOG, int N> __device__ __forceinline__ void do_domain(StackT<N> &r) {
-  if constexpr (SP >= 1) {
-    uint32_t bad = r.bad;
-#pragma unroll
-    for (int e = 0; e < N; ++e) {
-      const float x = r.st[SP - 1][e];
-      const bool out = LOG ? x <= 0.0f : x < 0.0f;
-      const float y = LOG ? logf(x) : __builtin_sqrtf(x);
-      r.st[SP - 1][e] = out ? (LOG ? 1.0f : 0.0f) : y;
-      bad |= out ? (1u << e) : 0u;
-    }
-    r.bad = bad;
-  }
+  if constexpr (SP >= 1)
+    domain_fn<LOG, N>(r.bad, r.st[SP - 1]);
 }
 template <int SP, int N> __device__ __forceinline__ void do_powchk(StackT<N> &r) {
-  if constexpr (SP >= 1) {
-    uint32_t bad = r.bad;
-#pragma unroll
-    for (int e = 0; e < N; ++e) {
-      const bool good = is_finite(r.st[SP - 1][e]);
-      r.st[SP - 1][e] = good ? r.st[SP - 1][e] : 1e20f;
-      bad |= good ? 0u : (1u << e);
-    }
-    r.bad = bad;
-  }
+  if constexpr (SP >= 1)
+    powchk_fn<N>(r.bad, r.st[SP - 1]);
 }
 
 // One instruction with SP entries on the stack; returns the new stack pointer.
@@ -1195,6 +1202,7 @@ struct RowArgs {
   uint32_t vec_mask; // bit i: rows of operand i start on 16-byte boundaries; bit 8: the output
   uint32_t interleaved; // columns are dealt to lanes one by one (then vec_mask is 0)
   uint32_t n_col, n_stages, passes;
+  uint32_t hold, hold_last; // chain kernels: the operand a lane keeps in registers, and the last instruction that reads it
   Stage stage[kMaxStages];
   Instr prog[kRowProg];
 };
@@ -1490,3 +1498,345 @@ extern "C" __global__ __launch_bounds__(256)
 __attribute__((amdgpu_waves_per_eu(4, 4))) void hcamd_row_program_w64(const RowArgs a) {
   row_program<64>(a);
 }
+
+// ---- row programs whose stages are chains ------------------------------------------
+// Most bodies with row reductions compile to stages that never hold two values
+// at once: an operand, then operations that change it in place (`in sub_red exp`,
+// `in sub_red mdiv_red mul_in add_in`).  For those the evaluation stack is one
+// value per element, and a lane can afford all of its row at once: P chunks of
+// eight (P = 1, 2; rows of at most P * LPR chunks, LPR = 64 ... 1024 lanes to a row), so that one dispatch of an
+// instruction works on 8 P elements instead of 8 and the dispatch, which is what
+// bounds the general kernel above, is paid a P-th as often.  The operand most
+// stages read (`hold`) is fetched once, every chunk requested before the first
+// stage starts, and stays in registers; any other operand is fetched by the
+// instruction that names it.  The host decides (hcamdLaunchRowProgram): every
+// stage a chain, whole chunks only (columns a multiple of 8, 16-byte aligned
+// rows), at most 4 chunks per lane; `x x mul` with equal halves arrives as
+// `x sq`.  Everything else is as above: the same stages, row scalars, numpy.ma
+// forms and fixed order of additions (lane order differs from the general
+// kernel's, so sums agree with it to rounding, not bit for bit).
+namespace {
+constexpr uint32_t OP_SQ = 63; // top = top * top; made by the host, not part of the C ABI
+
+template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArgs &a) {
+  constexpr int NE = 8 * P;
+  constexpr int T = LPR < kThreads ? kThreads : LPR; // threads of a workgroup
+  constexpr uint32_t R = T / LPR;                     // rows per workgroup and turn
+  __shared__ float slots[2][T / kWave];
+  __shared__ float red_cells[T / kWave][kMaxRed];
+  const uint32_t t = threadIdx.x, lane = t % LPR;
+  float *cells = red_cells[t / kWave];
+  const uint32_t per_row = (uint32_t)(a.cols / 8);
+  const bool out_f16 = (a.f16_mask >> 8) & 1;
+  uint32_t parity = 0;
+  // A workgroup takes rows in turns, the grid apart: as many workgroups as the
+  // device holds at once, so none waits to be launched behind another.
+  const size_t turns = (a.rows + R - 1) / R;
+  // chunk p of this lane is chunk p * LPR + lane of the row (chunk 0 where the
+  // row has no such chunk: loaded, never used)
+  auto chunk_at = [&](int p) {
+    const uint32_t c = (uint32_t)p * LPR + lane;
+    return c < per_row ? c : 0u;
+  };
+  // The chunks of operand i in row `r` as loaded: 8 fp16 in w[p][0], 8 fp32 in w[p][0..1].
+  auto request = [&](uint32_t i, size_t r, u32x4 (&w)[P][2]) {
+    const void *in = a.in[0];
+    size_t ld = a.ld[0];
+#pragma unroll
+    for (int k = 1; k < kMaxIn; ++k) {
+      in = i == (uint32_t)k ? a.in[k] : in;
+      ld = i == (uint32_t)k ? a.ld[k] : ld;
+    }
+    const bool f16 = (a.f16_mask >> i) & 1;
+    const char *b = static_cast<const char *>(in) + r * ld * (f16 ? 2 : 4);
+    if (f16) {
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        w[p][0] = ldg<false>(reinterpret_cast<const u32x4 *>(b) + chunk_at(p));
+        w[p][1] = u32x4{0u, 0u, 0u, 0u};
+      }
+    } else {
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        const u32x4 *q = reinterpret_cast<const u32x4 *>(b) + 2 * chunk_at(p);
+        w[p][0] = ldg<false>(q);
+        w[p][1] = ldg<false>(q + 1);
+      }
+    }
+  };
+  auto row_of = [&](size_t turn) { // idle lanes compute on row 0 and store nothing
+    const size_t r = turn * R + t / LPR;
+    return r < a.rows ? r : (size_t)0;
+  };
+  // The held operand's row: requested here for the first turn, and for every
+  // later one by the turn before it, as soon as that has read the operand for
+  // the last time (instruction `hold_last`), so that the row arrives while the
+  // rest of the last stage runs.
+  const uint32_t hold = a.hold & (kMaxIn - 1);
+  u32x4 held[P][2];
+  request(hold, row_of(blockIdx.x), held);
+#pragma nounroll
+  for (size_t turn = blockIdx.x; turn < turns; turn += gridDim.x) {
+  const size_t row_at = turn * R + t / LPR;
+  const bool row_live = row_at < a.rows;
+  const size_t row = row_of(turn);
+  // bit p of `live`: chunk p of this lane exists
+  uint32_t live = 0;
+#pragma unroll
+  for (int p = 0; p < P; ++p)
+    live |= (row_live && (uint32_t)p * LPR + lane < per_row) ? 1u << p : 0u;
+
+  if (t % kWave < kMaxRed)
+    cells[t % kWave] = 0.0f;
+#pragma unroll
+  for (int k = 0; k < kMaxIn; ++k)
+    if (k < (int)a.n_col)
+      cells[k] = uniform(load_elem(a.col[k], (a.f16_mask >> (16 + k)) & 1, row));
+
+  char *const orow = static_cast<char *>(a.out) + row * a.ldo * (out_f16 ? 2 : 4);
+
+#pragma nounroll
+  for (uint32_t s = 0; s < a.n_stages; ++s) {
+    const Stage st = a.stage[s];
+    const uint32_t kind = st.kind;
+    // the row scalars, scalar k in lane k
+    const uint32_t reds = __builtin_bit_cast(uint32_t, cells[t & (kMaxRed - 1)]);
+    // the instruction at pc, a scalar form rewritten into the immediate form
+    // with the row scalar as the immediate
+    auto decode = [&](Instr cur, uint32_t &op, float &imm) {
+      op = cur.op;
+      uint32_t imm_bits = __builtin_bit_cast(uint32_t, cur.imm);
+      if (op >= OP_RED && op != OP_SQ) {
+        imm_bits = __builtin_amdgcn_readlane(reds, cur.arg & (kMaxRed - 1));
+        op = op == OP_RED        ? (uint32_t)OP_CONST
+             : op >= OP_MDIV_RED ? op - OP_MDIV_RED + OP_MDIVI
+                                 : op - OP_ADD_RED + OP_ADDI;
+      }
+      asm volatile("" : "+s"(op), "+s"(imm_bits));
+      imm = __builtin_bit_cast(float, imm_bits);
+    };
+    Instr next = a.prog[st.begin & (kRowProg - 1)];
+    if (kind == ST_SCALAR || kind == ST_STORE_COL) {
+      // arithmetic on row scalars: one value
+      float sv = 0.0f;
+#pragma nounroll
+      for (uint32_t pc = st.begin; pc < st.end; ++pc) {
+        const Instr cur = next;
+        next = a.prog[(pc + 1) & (kRowProg - 1)];
+        uint32_t op;
+        float imm;
+        decode(cur, op, imm);
+        switch (op) {
+        case OP_CONST: sv = imm; break;
+        case OP_ADDI: sv = sv + imm; break;
+        case OP_SUBI: sv = sv - imm; break;
+        case OP_MULI: sv = sv * imm; break;
+        case OP_DIVI: sv = sv / imm; break;
+        case OP_MAXI: sv = nan_max(sv, imm); break;
+        case OP_MINI: sv = nan_min(sv, imm); break;
+        case OP_RSUBI: sv = imm - sv; break;
+        case OP_RDIVI: sv = imm / sv; break;
+        case OP_NEG: sv = -sv; break;
+        case OP_ABS: sv = __builtin_fabsf(sv); break;
+        case OP_SQRT: sv = __builtin_sqrtf(sv); break;
+        case OP_RINT: sv = __builtin_rintf(sv); break;
+        case OP_EXP: sv = expf(sv); break;
+        case OP_LOG: sv = logf(sv); break;
+        case OP_TANH: sv = tanh_selects(sv); break;
+        case OP_R16: sv = round16(sv); break;
+        case OP_SQ: sv = sv * sv; break;
+        default: break;
+        }
+      }
+      if (kind == ST_SCALAR)
+        cells[st.dst & (kMaxRed - 1)] = uniform(sv);
+      else if (row_live && lane == 0)
+        store_elem(a.out, out_f16, row * a.ldo, sv);
+      continue;
+    }
+    float v[NE];
+    uint32_t bad = 0;
+#pragma unroll
+    for (int e = 0; e < NE; ++e)
+      v[e] = 0.0f;
+#pragma nounroll
+    for (uint32_t pc = st.begin; pc < st.end; ++pc) {
+      const Instr cur = next;
+      next = a.prog[(pc + 1) & (kRowProg - 1)];
+      const uint32_t arg = cur.arg;
+      uint32_t op;
+      float imm;
+      decode(cur, op, imm);
+      const bool half = (arg & 0x100u) != 0;
+      // Heavy operations run chunk by chunk (the fence keeps the scheduler from
+      // interleaving all 8 P elements, whose temporaries would not fit): four at a time.
+#define HCAMD_CHAIN_EACH(EXPR)                                                    \
+  _Pragma("unroll") for (int g = 0; g < NE / 4; ++g) {                            \
+    _Pragma("unroll") for (int e = 4 * g; e < 4 * g + 4; ++e) { EXPR; }           \
+    __builtin_amdgcn_sched_barrier(0);                                            \
+  }
+      const bool reads = op == OP_IN || (op >= OP_ADD_IN && op <= OP_RDIV_IN) ||
+                         op == OP_MDIV_IN || op == OP_RMDIV_IN;
+      if (reads) {
+        // v = v op operand, the operand straight from where it was loaded to
+        auto apply = [&](auto rhs) {
+          switch (op) {
+          case OP_IN: HCAMD_CHAIN_EACH(v[e] = rhs(e)) break;
+          case OP_ADD_IN: HCAMD_CHAIN_EACH(v[e] = v[e] + rhs(e)) break;
+          case OP_SUB_IN: HCAMD_CHAIN_EACH(v[e] = v[e] - rhs(e)) break;
+          case OP_MUL_IN: HCAMD_CHAIN_EACH(v[e] = v[e] * rhs(e)) break;
+          case OP_DIV_IN: HCAMD_CHAIN_EACH(v[e] = v[e] / rhs(e)) break;
+          case OP_MAX_IN: HCAMD_CHAIN_EACH(v[e] = nan_max(v[e], rhs(e))) break;
+          case OP_MIN_IN: HCAMD_CHAIN_EACH(v[e] = nan_min(v[e], rhs(e))) break;
+          case OP_RSUB_IN: HCAMD_CHAIN_EACH(v[e] = rhs(e) - v[e]) break;
+          case OP_RDIV_IN: HCAMD_CHAIN_EACH(v[e] = rhs(e) / v[e]) break;
+          default: { // the numpy.ma quotients
+            float x[NE];
+#pragma unroll
+            for (int e = 0; e < NE; ++e) x[e] = rhs(e);
+            if (op == OP_MDIV_IN)
+              masked_div<NE>(bad, v, v, x, half);
+            else
+              masked_div<NE>(bad, v, x, v, half);
+          }
+          }
+        };
+        const uint32_t i = arg & (kMaxIn - 1);
+        const bool f16 = (a.f16_mask >> i) & 1;
+        // (the empty asm statements pin conversions and products of the held
+        // operand to the arm that uses them: hoisted out of the stage loop, as
+        // loop invariants, they would each hold 8 P registers for the whole row)
+        auto from = [&](const u32x4 (&w)[P][2]) {
+          if (f16)
+            apply([&](int e) {
+              uint32_t x = w[e / 8][0][(e % 8) / 2];
+              asm volatile("" : "+v"(x));
+              return (float)__builtin_bit_cast(_Float16, (uint16_t)(e % 2 ? x >> 16 : x & 0xffffu));
+            });
+          else
+            apply([&](int e) {
+              uint32_t x = w[e / 8][(e % 8) / 4][e % 4];
+              asm volatile("" : "+v"(x));
+              return __builtin_bit_cast(float, x);
+            });
+        };
+        if (i == hold) {
+          from(held);
+          if (pc == a.hold_last && turn + gridDim.x < turns)
+            request(hold, row_of(turn + gridDim.x), held);
+        } else {
+          u32x4 w[P][2];
+          request(i, row, w);
+          from(w);
+        }
+        continue;
+      }
+      switch (op) {
+      case OP_CONST: HCAMD_CHAIN_EACH(v[e] = imm) break;
+      case OP_ADDI: HCAMD_CHAIN_EACH(v[e] = v[e] + imm) break;
+      case OP_SUBI: HCAMD_CHAIN_EACH(v[e] = v[e] - imm) break;
+      case OP_MULI: HCAMD_CHAIN_EACH(v[e] = v[e] * imm) break;
+      case OP_DIVI: HCAMD_CHAIN_EACH(v[e] = v[e] / imm) break;
+      case OP_MAXI: HCAMD_CHAIN_EACH(v[e] = nan_max(v[e], imm)) break;
+      case OP_MINI: HCAMD_CHAIN_EACH(v[e] = nan_min(v[e], imm)) break;
+      case OP_RSUBI: HCAMD_CHAIN_EACH(v[e] = imm - v[e]) break;
+      case OP_RDIVI: HCAMD_CHAIN_EACH(v[e] = imm / v[e]) break;
+      case OP_NEG: HCAMD_CHAIN_EACH(v[e] = -v[e]) break;
+      case OP_ABS: HCAMD_CHAIN_EACH(v[e] = __builtin_fabsf(v[e])) break;
+      case OP_SQRT: HCAMD_CHAIN_EACH(v[e] = __builtin_sqrtf(v[e])) break;
+      case OP_RINT: HCAMD_CHAIN_EACH(v[e] = __builtin_rintf(v[e])) break;
+      case OP_EXP: HCAMD_CHAIN_EACH(v[e] = expf(v[e])) break;
+      case OP_LOG: HCAMD_CHAIN_EACH(v[e] = logf(v[e])) break;
+      case OP_TANH: HCAMD_CHAIN_EACH(v[e] = tanh_selects(v[e])) break;
+      case OP_R16: HCAMD_CHAIN_EACH(v[e] = round16(v[e])) break;
+      case OP_SQ: HCAMD_CHAIN_EACH(v[e] = v[e] * v[e]) break;
+      case OP_MDIVI:
+      case OP_RMDIVI: {
+        float x[NE];
+#pragma unroll
+        for (int e = 0; e < NE; ++e) x[e] = imm;
+        if (op == OP_MDIVI)
+          masked_div<NE>(bad, v, v, x, half);
+        else
+          masked_div<NE>(bad, v, x, v, half);
+        break;
+      }
+      case OP_CLEAR:
+        bad = 0;
+        break;
+      case OP_POWCHK:
+        powchk_fn<NE>(bad, v);
+        break;
+      case OP_MSQRT:
+        domain_fn<false, NE>(bad, v);
+        break;
+      case OP_MLOG:
+        domain_fn<true, NE>(bad, v);
+        break;
+      default:
+        break;
+      }
+#undef HCAMD_CHAIN_EACH
+    }
+
+    if (kind <= ST_MIN) {
+      float acc = kind == ST_MAX ? -INFINITY : kind == ST_MIN ? INFINITY : 0.0f;
+      // a wave whose lanes all hold P chunks with every element active folds without masks
+      if (__builtin_amdgcn_ballot_w64(bad != 0 || live != (1u << P) - 1u) == 0) {
+        if (kind == ST_SUM) {
+#pragma unroll
+          for (int e = 0; e < NE; ++e) acc += v[e];
+        } else if (kind == ST_MAX) {
+#pragma unroll
+          for (int e = 0; e < NE; ++e) acc = nan_max(acc, v[e]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < NE; ++e) acc = nan_min(acc, v[e]);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < NE; ++e) {
+          const bool take = ((live >> (e / 8)) & 1u) && !((bad >> e) & 1u);
+          if (kind == ST_SUM)
+            acc += take ? v[e] : 0.0f;
+          else if (kind == ST_MAX)
+            acc = take ? nan_max(acc, v[e]) : acc;
+          else
+            acc = take ? nan_min(acc, v[e]) : acc;
+        }
+      }
+      constexpr int W = LPR / kWave;
+      float total;
+      float *mine = slots[parity] + (t / LPR) * W; // the slots of this row's waves
+      if (kind == ST_SUM)
+        total = group_reduce<SumOp, W>(acc, mine);
+      else if (kind == ST_MAX)
+        total = group_reduce<NanMaxOp, W>(acc, mine);
+      else
+        total = group_reduce<NanMinOp, W>(acc, mine);
+      parity ^= 1;
+      cells[st.dst & (kMaxRed - 1)] = total;
+    } else if (kind == ST_STORE) {
+      char *o = orow; // opaque: the element addresses of the masked form are not loop invariants
+      asm volatile("" : "+v"(o));
+#pragma unroll
+      for (int p = 0; p < P; ++p)
+        if ((live >> p) & 1u)
+          store_chunk(o, out_f16, (size_t)p * LPR + lane, v + 8 * p, (bad >> (8 * p)) & 0xffu);
+    }
+  }
+  } // turns
+}
+} // namespace
+
+#define HCAMD_ROW_CHAIN(LPR, P, T)                                                       \
+  extern "C" __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(4, 4)))   \
+  void hcamd_row_program_chain_w##LPR##_p##P(const RowArgs a) {                          \
+    row_chain<LPR, P>(a);                                                                 \
+  }
+HCAMD_ROW_CHAIN(64, 1, 256)
+HCAMD_ROW_CHAIN(64, 2, 256)
+HCAMD_ROW_CHAIN(128, 2, 256)
+HCAMD_ROW_CHAIN(256, 2, 256)
+HCAMD_ROW_CHAIN(512, 2, 512)
+HCAMD_ROW_CHAIN(1024, 2, 1024)

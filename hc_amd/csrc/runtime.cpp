@@ -267,7 +267,7 @@ std::unordered_map<std::string, int> &variants() {
   static std::unordered_map<std::string, int> v{
       {"add", 0},     {"fma", 0},  {"softmax", 0},
       {"quantize", 0}, {"gemm", 0}, {"copy", 0}, {"map", 0},
-      {"gather", 0}, {"gather_fuse", 0}};
+      {"gather", 0}, {"gather_fuse", 0}, {"rows", 0}};
   return v;
 }
 std::mutex g_variantLock; // guards variants()
@@ -1866,9 +1866,59 @@ struct RowArgs {
   size_t rows, cols;
   uint32_t f16Mask, vecMask, interleaved;
   uint32_t nCol, nStages, passes;
+  uint32_t hold, holdLast;
   RowStageDev stage[HCAMD_ROW_MAX_STAGES];
   HcamdMapInstr prog[HCAMD_ROW_MAX_INSTRS];
 };
+
+// A stage program that never holds two values at once, as the chain kernels
+// take it: a push, then operations that change the value in place.  `x x mul`
+// with two equal halves is such a program too, `x sq` (kRowSq exists between
+// this file and the kernel only).  Appends to out[0 .. count) (never more
+// instructions than it read); false: not a chain.
+constexpr unsigned kRowSq = 63;
+bool chainOf(const HcamdMapInstr *p, size_t n, HcamdMapInstr *out, size_t &count) {
+  auto pushes = [](unsigned op) {
+    return op == HCAMD_MAP_IN || op == HCAMD_MAP_CONST || op == HCAMD_MAP_RED;
+  };
+  auto inPlace = [](unsigned op) {
+    return (op >= HCAMD_MAP_ADDI && op <= HCAMD_MAP_RDIV_IN) ||
+           (op >= HCAMD_MAP_MDIVI && op <= HCAMD_MAP_MLOG) ||
+           (op >= HCAMD_MAP_ADD_RED && op <= HCAMD_MAP_RMDIV_RED);
+  };
+  auto chain = [&](const HcamdMapInstr *q, size_t m) {
+    if (m == 0 || !pushes(q[0].op))
+      return false;
+    for (size_t i = 1; i < m; ++i)
+      if (!inPlace(q[i].op))
+        return false;
+    return true;
+  };
+  auto append = [&](const HcamdMapInstr *q, size_t m) {
+    std::memcpy(out + count, q, m * sizeof(HcamdMapInstr));
+    count += m;
+  };
+  if (chain(p, n)) {
+    append(p, n);
+    return true;
+  }
+  size_t k = 0;
+  while (k < n && (pushes(p[k].op) || inPlace(p[k].op)))
+    ++k;
+  if (k == n || p[k].op != HCAMD_MAP_MUL || k < 2 || k % 2)
+    return false;
+  const size_t h = k / 2;
+  if (!chain(p, h) || std::memcmp(p, p + h, h * sizeof(HcamdMapInstr)) != 0)
+    return false;
+  for (size_t i = k + 1; i < n; ++i)
+    if (!inPlace(p[i].op))
+      return false;
+  append(p, h);
+  const HcamdMapInstr sq{static_cast<uint16_t>(kRowSq), 0, 0.0f};
+  append(&sq, 1);
+  append(p + k + 1, n - k - 1);
+  return true;
+}
 } // namespace
 
 int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
@@ -2057,13 +2107,68 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
     a.vecMask = 0;
     a.interleaved = 1;
   }
-  Kernel *k = builtinKernel(dev, "map", lanesPerRow == 64 ? "hcamd_row_program_w64"
-                                                         : "hcamd_row_program_w256");
+  // Rows of whole, aligned chunks, at most 2048 of them, whose stages are all
+  // chains run on the chain kernels: a lane has its whole part of the row at
+  // once, 8 or 16 elements to a dispatch, and the operand that most
+  // instructions read stays in registers (variant 1 of "rows": never).
+  size_t lanes = lanesPerRow, maxGroups = SIZE_MAX, threads = 256;
+  char name[48];
+  std::snprintf(name, sizeof name, "hcamd_row_program_w%zu", lanes);
+  if (variantOf("rows") != 1 && !a.interleaved && cols % 8 == 0 && perRow <= 2048 && nInputs > 0) {
+    HcamdMapInstr chained[HCAMD_ROW_MAX_INSTRS];
+    size_t nChained = 0;
+    uint16_t begin[HCAMD_ROW_MAX_STAGES], end[HCAMD_ROW_MAX_STAGES];
+    bool ok = true;
+    size_t at = 0;
+    for (size_t s = 0; s < nStages && ok; ++s) {
+      begin[s] = static_cast<uint16_t>(nChained);
+      ok = chainOf(prog + at, stages[s].nInstr, chained, nChained);
+      end[s] = static_cast<uint16_t>(nChained);
+      at += stages[s].nInstr;
+    }
+    uint32_t reads[kMapMaxIn] = {};
+    for (size_t i = 0; i < nChained; ++i) {
+      const HcamdMapInstr &in = chained[i];
+      const unsigned op = in.op;
+      if (op == HCAMD_MAP_IN || (op >= HCAMD_MAP_ADD_IN && op <= HCAMD_MAP_RDIV_IN) ||
+          op == HCAMD_MAP_MDIV_IN || op == HCAMD_MAP_RMDIV_IN)
+        ++reads[in.arg & 3u];
+    }
+    size_t hold = 0;
+    for (size_t i = 1; i < nInputs; ++i)
+      if (reads[i] > reads[hold])
+        hold = i;
+    if (ok && reads[hold] > 0) {
+      const unsigned p = perRow <= 64 ? 1 : 2;
+      lanes = 64;
+      while (lanes * p < perRow)
+        lanes *= 2;
+      threads = std::max<size_t>(256, lanes);
+      for (size_t s = 0; s < nStages; ++s) {
+        a.stage[s].begin = begin[s];
+        a.stage[s].end = end[s];
+      }
+      std::memset(a.prog, 0, sizeof a.prog);
+      std::memcpy(a.prog, chained, nChained * sizeof(HcamdMapInstr));
+      a.hold = static_cast<uint32_t>(hold);
+      for (size_t i = 0; i < nChained; ++i) {
+        const unsigned op = chained[i].op;
+        if ((op == HCAMD_MAP_IN || (op >= HCAMD_MAP_ADD_IN && op <= HCAMD_MAP_RDIV_IN) ||
+             op == HCAMD_MAP_MDIV_IN || op == HCAMD_MAP_RMDIV_IN) &&
+            (chained[i].arg & 3u) == hold)
+          a.holdLast = static_cast<uint32_t>(i);
+      }
+      std::snprintf(name, sizeof name, "hcamd_row_program_chain_w%zu_p%u", lanes, p);
+      // these kernels walk the rows themselves: as many workgroups as are resident at once
+      maxGroups = (size_t)computeUnitsOf(dev) * 16 / (threads / 64);
+    }
+  }
+  Kernel *k = builtinKernel(dev, "map", name);
   if (!k)
     return 1;
   void *args[] = {&a};
-  const size_t grid[3] = {ceilDiv(rows, 256 / lanesPerRow), 1, 1};
-  const size_t block[3] = {256, 1, 1};
+  const size_t grid[3] = {std::min(ceilDiv(rows, threads / lanes), maxGroups), 1, 1};
+  const size_t block[3] = {threads, 1, 1};
   return launch(queue, k, grid, block, args, 0);
 }
 

@@ -505,8 +505,15 @@ int hcamdLaunchMapReduceColsNoAlloc(OlQueue q, int kind, const HcamdMapInstr *pr
  * or, with leading dimension 0, one vector of cols elements used for every row;
  * `columns` hold one value per row and fill row scalars 0 .. nColumns-1.
  * A row is handled by one wave (cols <= 4096) or one workgroup; every stage
- * reads the operands it uses again (a row just read is still in L2).  Sums add in an order that
- * depends on the shape only: results are reproducible, and agree with a
+ * reads the operands it uses again (a row just read is still in L2).  Programs
+ * whose stages all change one value in place (an operand, then *I, *_IN, *_RED
+ * and unary forms; `x x MUL` with two equal halves counts) over 16-byte aligned
+ * rows of whole chunks of 8 elements, at most 16384 of them, run on kernels that
+ * keep a lane's whole part of the row in registers: the operand most
+ * instructions read is fetched once per row, and an instruction is dispatched
+ * once for 8 or 16 elements of a lane (variant 1 of the "rows" family keeps the
+ * general kernel).  Sums add in an order that
+ * depends on the shape and the kernel only: results are reproducible, and agree with a
  * sequential fp32 sum to within the usual n * 2^-24 bound. */
 enum HcamdRowStageKind {
   HCAMD_ROW_SUM = 0,
@@ -647,7 +654,7 @@ int hcamdLaunchGemmF16(OlQueue q, const void *a, size_t lda, const void *bt,
 
 /* Chooses between kernel variants of one family by number (0 = default
  * choice by shape).  For tuning and measurement; family names are "add",
- * "fma", "softmax", "quantize", "gemm", "copy", "map", "gather" (block
+ * "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "gather" (block
  * shape), "gather_fuse" (groups per workgroup; read by hcamdGatherGemmCreate).
  * Process-wide, guarded by a lock.  Returns 1 for an unknown family. */
 int hcamdSetVariant(const char *family, int variant) HCAMD_NOEXCEPT;

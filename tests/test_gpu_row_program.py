@@ -59,24 +59,51 @@ def np_softmax(x):
     return e / e.sum(axis=1, keepdims=True)
 
 
-# cols: one wave per row (<= 4096), one workgroup per row, one and several chunks per lane
+def kernel_for(cols, general=False):
+    """The kernel hcamdLaunchRowProgram picks for dense, 16-byte aligned rows whose
+    stages are all chains: a chain kernel for whole chunks up to 2048 of them (one
+    chunk per lane up to 64, else two, on 64 ... 1024 lanes), else the general one
+    (a wave per row up to 4096 columns, else a workgroup)."""
+    per_row = cols // 8
+    if not general and cols % 8 == 0 and per_row <= 2048:
+        p = 1 if per_row <= 64 else 2
+        lanes = 64
+        while lanes * p < per_row:
+            lanes *= 2
+        return f"hcamd_row_program_chain_w{lanes}_p{p}"
+    return "hcamd_row_program_w64" if cols <= 4096 else "hcamd_row_program_w256"
+
+
+@pytest.fixture(params=[0, 1], ids=["chain", "general"])
+def rows_variant(request):
+    """Variant 1 of "rows" keeps every program on the general kernel."""
+    rt.set_variant("rows", request.param)
+    yield request.param
+    rt.set_variant("rows", 0)
+
+
+# cols: one wave per row, one workgroup per row, one and several chunks per lane,
+# whole chunks and not; rows: fewer than the chain kernels' workgroups, and more
+# (their workgroups then take several rows in turns, fetching the next row early)
 @pytest.mark.parametrize("rows,cols", [(1, 1), (30, 25), (7, 8), (5, 512), (9, 513), (33, 2048),
-                                       (17, 4099), (64, 8192), (3, 16384), (2, 16392), (2, 40_001)])
-def test_softmax_as_a_row_program(ctx, rows, cols):
+                                       (17, 4099), (64, 8192), (3, 16384), (2, 16392), (2, 40_001),
+                                       (4501, 512), (4203, 1000), (2051, 2048), (1101, 4096),
+                                       (603, 8192), (301, 16384)])
+def test_softmax_as_a_row_program(ctx, rows, cols, rows_variant):
     rng = np.random.default_rng(cols)
     x = (rng.standard_normal((rows, cols)) * 3).astype(np.float32)
     out = poisoned((rows, cols), np.float32)
-    say("row program softmax", rows, cols)
+    say("row program softmax", rows, cols, rows_variant)
     rt.plan_row_program(SOFTMAX, [rt.to_device(x)], out).launch(sync=True)
     say("  ", rt.last_kernel_name())
-    assert rt.last_kernel_name() == ("hcamd_row_program_w64" if cols <= 4096 else "hcamd_row_program_w256")
+    assert rt.last_kernel_name() == kernel_for(cols, general=rows_variant == 1)
     assert_allclose(out.to_host(), np_softmax(x), rtol=1e-5, atol=1e-30)
 
 
 @pytest.mark.parametrize("cols,dtype", [(300, np.float32), (1000, np.float16), (8192, np.float32),
                                         (4104, np.float16)])
-def test_layer_normalisation_with_weight_and_bias_vectors(ctx, cols, dtype):
-    rows = 50
+def test_layer_normalisation_with_weight_and_bias_vectors(ctx, cols, dtype, rows_variant):
+    rows = 50 if cols != 1000 else 4100      # 4100 rows of 1000: several rows to a workgroup, in turns
     rng = np.random.default_rng(cols)
     x = (rng.standard_normal((rows, cols)) * 2 + 0.5).astype(dtype)
     g = rng.standard_normal(cols).astype(np.float32)
@@ -92,13 +119,14 @@ def test_layer_normalisation_with_weight_and_bias_vectors(ctx, cols, dtype):
     ]
     out = poisoned((rows, cols), np.float32)
     rt.plan_row_program(stages, [rt.to_device(x), rt.to_device(g), rt.to_device(b)], out).launch(sync=True)
+    assert rt.last_kernel_name() == kernel_for(cols, general=rows_variant == 1)   # `x x mul` is a chain too
     x64 = x.astype(np.float64)
     want = (x64 - x64.mean(axis=1, keepdims=True)) / np.sqrt(x64.var(axis=1, keepdims=True) + eps) * g + b
     assert_allclose(out.to_host(), want, rtol=2e-5, atol=2e-5)
 
 
-@pytest.mark.parametrize("rows,cols", [(1000, 7), (129, 1031), (4, 70_001)])
-def test_row_sums_maxima_and_minima_as_per_row_results(ctx, rows, cols):
+@pytest.mark.parametrize("rows,cols", [(1000, 7), (129, 1031), (4, 70_001), (5000, 264), (1300, 3000)])
+def test_row_sums_maxima_and_minima_as_per_row_results(ctx, rows, cols, rows_variant):
     rng = np.random.default_rng(rows)
     x = rng.standard_normal((rows, cols)).astype(np.float32)
     dx = rt.to_device(x)
@@ -117,8 +145,9 @@ def test_row_sums_maxima_and_minima_as_per_row_results(ctx, rows, cols):
                 assert_array_equal(got, want.astype(np.float32))
 
 
-def test_column_operands_fill_row_scalars_and_fp16_results_round_once(ctx):
-    rows, cols = 77, 1000
+@pytest.mark.parametrize("rows", [77, 4300])
+def test_column_operands_fill_row_scalars_and_fp16_results_round_once(ctx, rows, rows_variant):
+    cols = 1000
     rng = np.random.default_rng(5)
     q = rng.integers(-127, 128, (rows, cols)).astype(np.float16)
     scale = rng.uniform(0.01, 2.0, rows).astype(np.float32)
@@ -131,8 +160,9 @@ def test_column_operands_fill_row_scalars_and_fp16_results_round_once(ctx):
     assert_array_equal(out.to_host().view(np.uint16), want.view(np.uint16))
 
 
-def test_windows_of_larger_arrays_and_untouched_surroundings(ctx):
-    rows, cols = 19, 1003
+@pytest.mark.parametrize("cols", [1003, 1000])        # 1000: whole chunks, the chain kernel where rows are aligned
+def test_windows_of_larger_arrays_and_untouched_surroundings(ctx, cols, rows_variant):
+    rows = 19
     rng = np.random.default_rng(6)
     x = rng.standard_normal((rows, cols)).astype(np.float32)
     for ld, off in ((1024, 4), (1011, 3)):            # 16-byte aligned rows, and not
@@ -189,7 +219,7 @@ def test_fp16_rows_off_16_byte_boundaries_interleave_the_lanes(ctx, cols, ld):
                     atol=cols * 2.0 ** -24 * np.abs(p64).sum(axis=1).max() + 1e-30)
 
 
-def test_special_values_follow_numpy(ctx):
+def test_special_values_follow_numpy(ctx, rows_variant):
     x = np.zeros((6, 600), np.float32)
     x[0, 5] = np.nan                    # NaN reaches every result of its row only
     x[1, :] = -np.inf                   # exp(-inf - -inf) = NaN in NumPy too
@@ -224,3 +254,31 @@ def test_malformed_programs_are_refused_before_anything_runs(ctx):
     assert (out.to_host().view(np.uint32) == POISON32).all()
     with pytest.raises(rt.HcRuntimeError, match="shape mismatch"):
         rt.plan_row_program(SOFTMAX, [rt.to_device(np.ones((4, 17), np.float32))], out)
+
+
+def test_numpy_ma_forms_and_partly_empty_lanes_on_the_chain_kernels(ctx, rows_variant):
+    """x / (row sum of y * y) with rows whose sum is zero (numpy.ma leaves such a
+    row as it was), the maximum of log(x) over the positive elements only, and a
+    row length that leaves some lanes of the chain kernel with one chunk or none:
+    both kernels against NumPy, including which elements are written."""
+    rows, cols = 4200, 1112                       # 139 chunks: w128_p2 with 117 idle chunk slots
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    y = rng.standard_normal((rows, cols)).astype(np.float32)
+    y[::7] = 0.0
+    dx, dy = rt.to_device(x), rt.to_device(y)
+    out = poisoned((rows, cols), np.float32)
+    rt.plan_row_program([("sum", 0, [I("in", 1), I("mul_in", 1)]),
+                         ("store", 0, [I("in", 0), I("mdiv_red", 0)])], [dx, dy], out).launch(sync=True)
+    assert rt.last_kernel_name() == kernel_for(cols, general=rows_variant == 1)
+    got = out.to_host()
+    s = (y.astype(np.float64) ** 2).sum(axis=1)
+    dead = s == 0
+    assert dead.sum() == 600
+    assert (got[dead].view(np.uint32) == POISON32).all()
+    assert_allclose(got[~dead], x[~dead] / s[~dead, None], rtol=3e-6)
+    tops = poisoned((rows,), np.float32)
+    rt.plan_row_program([("max", 0, [I("in", 0), I("mlog")]), ("store_col", 0, [I("red", 0)])],
+                        [dx], tops).launch(sync=True)
+    want = np.log(np.where(x > 0, x, np.float32(1e-30)).astype(np.float64)).max(axis=1)
+    assert_allclose(tops.to_host(), want, rtol=2e-6, atol=1e-6)
