@@ -967,6 +967,128 @@ __device__ __forceinline__ void run_post(const ColArgs &c, const Raw &raw, Stack
   }
 }
 
+// ---- chains: programs that never hold two values at once ------------------------
+// An operand (or a constant), then operations that change the value in place:
+// the evaluation stack is one value per element, so one dispatch can work on
+// several chunks of a lane at once (NE = 16 elements) where the general
+// interpreter above affords 8.  The host recognises such programs and folds
+// `x x mul` with two equal halves into `x sq`.
+constexpr uint32_t OP_SQ = 63; // top = top * top; made by the host, not part of the C ABI
+
+// Four elements at a time: the fence keeps the scheduler from interleaving all
+// NE, whose temporaries (a division, an exponential) would not fit.
+#define HCAMD_CHAIN_EACH(EXPR)                                                    \
+  _Pragma("unroll") for (int g = 0; g < NE / 4; ++g) {                            \
+    _Pragma("unroll") for (int e = 4 * g; e < 4 * g + 4; ++e) { EXPR; }           \
+    __builtin_amdgcn_sched_barrier(0);                                            \
+  }
+
+__device__ __forceinline__ bool chain_reads(uint32_t op) {
+  return op == OP_IN || (op >= OP_ADD_IN && op <= OP_RDIV_IN) || op == OP_MDIV_IN ||
+         op == OP_RMDIV_IN;
+}
+// v = v op operand for the instructions that name an operand; rhs(e) is the
+// operand's element e, read straight from where it was loaded to.
+template <int NE, class Rhs>
+__device__ __forceinline__ void chain_operand(uint32_t op, float (&v)[NE], uint32_t &bad, bool half,
+                                              Rhs rhs) {
+  auto apply = [&](auto at) {
+    switch (op) {
+    case OP_IN: HCAMD_CHAIN_EACH(v[e] = at(e)) break;
+    case OP_ADD_IN: HCAMD_CHAIN_EACH(v[e] = v[e] + at(e)) break;
+    case OP_SUB_IN: HCAMD_CHAIN_EACH(v[e] = v[e] - at(e)) break;
+    case OP_MUL_IN: HCAMD_CHAIN_EACH(v[e] = v[e] * at(e)) break;
+    case OP_DIV_IN: HCAMD_CHAIN_EACH(v[e] = v[e] / at(e)) break;
+    case OP_MAX_IN: HCAMD_CHAIN_EACH(v[e] = nan_max(v[e], at(e))) break;
+    case OP_MIN_IN: HCAMD_CHAIN_EACH(v[e] = nan_min(v[e], at(e))) break;
+    case OP_RSUB_IN: HCAMD_CHAIN_EACH(v[e] = at(e) - v[e]) break;
+    case OP_RDIV_IN: HCAMD_CHAIN_EACH(v[e] = at(e) / v[e]) break;
+    default: { // the numpy.ma quotients
+      float x[NE];
+#pragma unroll
+      for (int e = 0; e < NE; ++e) x[e] = at(e);
+      if (op == OP_MDIV_IN)
+        masked_div<NE>(bad, v, v, x, half);
+      else
+        masked_div<NE>(bad, v, x, v, half);
+    }
+    }
+  };
+  rhs(apply);
+}
+// The operand as P chunks of loaded words: 8 fp16 in w[p][0], 8 fp32 in
+// w[p][0..1].  (The empty asm statements pin conversions and products of an
+// operand that stays in registers to the arm that uses them: hoisted out of the
+// surrounding loops, as loop invariants, they would each hold 8 P registers.)
+// `word(p, j, c)` is component c of word j of chunk p.
+template <class Word> __device__ __forceinline__ auto chain_words(Word word, bool f16) {
+  return [word, f16](auto apply) {
+    if (f16)
+      apply([&](int e) {
+        uint32_t x = word(e / 8, 0, (e % 8) / 2);
+        asm volatile("" : "+v"(x));
+        return (float)__builtin_bit_cast(_Float16, (uint16_t)(e % 2 ? x >> 16 : x & 0xffffu));
+      });
+    else
+      apply([&](int e) {
+        uint32_t x = word(e / 8, (e % 8) / 4, e % 4);
+        asm volatile("" : "+v"(x));
+        return __builtin_bit_cast(float, x);
+      });
+  };
+}
+// every other instruction of a chain
+template <int NE>
+__device__ __forceinline__ void chain_plain(uint32_t op, float (&v)[NE], uint32_t &bad, float imm,
+                                            bool half) {
+  switch (op) {
+  case OP_CONST: HCAMD_CHAIN_EACH(v[e] = imm) break;
+  case OP_ADDI: HCAMD_CHAIN_EACH(v[e] = v[e] + imm) break;
+  case OP_SUBI: HCAMD_CHAIN_EACH(v[e] = v[e] - imm) break;
+  case OP_MULI: HCAMD_CHAIN_EACH(v[e] = v[e] * imm) break;
+  case OP_DIVI: HCAMD_CHAIN_EACH(v[e] = v[e] / imm) break;
+  case OP_MAXI: HCAMD_CHAIN_EACH(v[e] = nan_max(v[e], imm)) break;
+  case OP_MINI: HCAMD_CHAIN_EACH(v[e] = nan_min(v[e], imm)) break;
+  case OP_RSUBI: HCAMD_CHAIN_EACH(v[e] = imm - v[e]) break;
+  case OP_RDIVI: HCAMD_CHAIN_EACH(v[e] = imm / v[e]) break;
+  case OP_NEG: HCAMD_CHAIN_EACH(v[e] = -v[e]) break;
+  case OP_ABS: HCAMD_CHAIN_EACH(v[e] = __builtin_fabsf(v[e])) break;
+  case OP_SQRT: HCAMD_CHAIN_EACH(v[e] = __builtin_sqrtf(v[e])) break;
+  case OP_RINT: HCAMD_CHAIN_EACH(v[e] = __builtin_rintf(v[e])) break;
+  case OP_EXP: HCAMD_CHAIN_EACH(v[e] = expf(v[e])) break;
+  case OP_LOG: HCAMD_CHAIN_EACH(v[e] = logf(v[e])) break;
+  case OP_TANH: HCAMD_CHAIN_EACH(v[e] = tanh_selects(v[e])) break;
+  case OP_R16: HCAMD_CHAIN_EACH(v[e] = round16(v[e])) break;
+  case OP_SQ: HCAMD_CHAIN_EACH(v[e] = v[e] * v[e]) break;
+  case OP_MDIVI:
+  case OP_RMDIVI: {
+    float x[NE];
+#pragma unroll
+    for (int e = 0; e < NE; ++e) x[e] = imm;
+    if (op == OP_MDIVI)
+      masked_div<NE>(bad, v, v, x, half);
+    else
+      masked_div<NE>(bad, v, x, v, half);
+    break;
+  }
+  case OP_CLEAR:
+    bad = 0;
+    break;
+  case OP_POWCHK:
+    powchk_fn<NE>(bad, v);
+    break;
+  case OP_MSQRT:
+    domain_fn<false, NE>(bad, v);
+    break;
+  case OP_MLOG:
+    domain_fn<true, NE>(bad, v);
+    break;
+  default:
+    break;
+  }
+}
+#undef HCAMD_CHAIN_EACH
+
 __device__ __forceinline__ float col_fold(uint32_t kind, float a, float b) {
   return kind == COL_SUM ? a + b : kind == COL_MAX ? nan_max(a, b) : nan_min(a, b);
 }
@@ -1003,9 +1125,8 @@ __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, 
   const bool vec = !c.interleaved && __builtin_amdgcn_ballot_w64(n_valid != (uint32_t)kN) == 0;
   Raw raw;
   Stack r;
-#pragma nounroll
-  for (uint32_t row0 = row_begin + wave * R; row0 < row_end; row0 += kWaves * R * U) {
-    u32x4 staged[NIN][U][2];
+  // the rows of the turn that starts at row0, requested (rows past the end: not)
+  auto request = [&](uint32_t row0, u32x4 (&staged)[NIN][U][2]) {
 #pragma unroll
     for (int i = 0; i < NIN; ++i)
       if (i < (int)n_in) {
@@ -1042,6 +1163,11 @@ __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, 
           }
         }
       }
+  };
+#pragma nounroll
+  for (uint32_t row0 = row_begin + wave * R; row0 < row_end; row0 += kWaves * R * U) {
+    u32x4 staged[NIN][U][2];
+    request(row0, staged);
 #pragma nounroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
@@ -1516,8 +1642,6 @@ __attribute__((amdgpu_waves_per_eu(4, 4))) void hcamd_row_program_w64(const RowA
 // forms and fixed order of additions (lane order differs from the general
 // kernel's, so sums agree with it to rounding, not bit for bit).
 namespace {
-constexpr uint32_t OP_SQ = 63; // top = top * top; made by the host, not part of the C ABI
-
 template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArgs &a) {
   constexpr int NE = 8 * P;
   constexpr int T = LPR < kThreads ? kThreads : LPR; // threads of a workgroup
@@ -1668,115 +1792,23 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
       float imm;
       decode(cur, op, imm);
       const bool half = (arg & 0x100u) != 0;
-      // Heavy operations run chunk by chunk (the fence keeps the scheduler from
-      // interleaving all 8 P elements, whose temporaries would not fit): four at a time.
-#define HCAMD_CHAIN_EACH(EXPR)                                                    \
-  _Pragma("unroll") for (int g = 0; g < NE / 4; ++g) {                            \
-    _Pragma("unroll") for (int e = 4 * g; e < 4 * g + 4; ++e) { EXPR; }           \
-    __builtin_amdgcn_sched_barrier(0);                                            \
-  }
-      const bool reads = op == OP_IN || (op >= OP_ADD_IN && op <= OP_RDIV_IN) ||
-                         op == OP_MDIV_IN || op == OP_RMDIV_IN;
-      if (reads) {
-        // v = v op operand, the operand straight from where it was loaded to
-        auto apply = [&](auto rhs) {
-          switch (op) {
-          case OP_IN: HCAMD_CHAIN_EACH(v[e] = rhs(e)) break;
-          case OP_ADD_IN: HCAMD_CHAIN_EACH(v[e] = v[e] + rhs(e)) break;
-          case OP_SUB_IN: HCAMD_CHAIN_EACH(v[e] = v[e] - rhs(e)) break;
-          case OP_MUL_IN: HCAMD_CHAIN_EACH(v[e] = v[e] * rhs(e)) break;
-          case OP_DIV_IN: HCAMD_CHAIN_EACH(v[e] = v[e] / rhs(e)) break;
-          case OP_MAX_IN: HCAMD_CHAIN_EACH(v[e] = nan_max(v[e], rhs(e))) break;
-          case OP_MIN_IN: HCAMD_CHAIN_EACH(v[e] = nan_min(v[e], rhs(e))) break;
-          case OP_RSUB_IN: HCAMD_CHAIN_EACH(v[e] = rhs(e) - v[e]) break;
-          case OP_RDIV_IN: HCAMD_CHAIN_EACH(v[e] = rhs(e) / v[e]) break;
-          default: { // the numpy.ma quotients
-            float x[NE];
-#pragma unroll
-            for (int e = 0; e < NE; ++e) x[e] = rhs(e);
-            if (op == OP_MDIV_IN)
-              masked_div<NE>(bad, v, v, x, half);
-            else
-              masked_div<NE>(bad, v, x, v, half);
-          }
-          }
-        };
+      if (chain_reads(op)) {
         const uint32_t i = arg & (kMaxIn - 1);
         const bool f16 = (a.f16_mask >> i) & 1;
-        // (the empty asm statements pin conversions and products of the held
-        // operand to the arm that uses them: hoisted out of the stage loop, as
-        // loop invariants, they would each hold 8 P registers for the whole row)
-        auto from = [&](const u32x4 (&w)[P][2]) {
-          if (f16)
-            apply([&](int e) {
-              uint32_t x = w[e / 8][0][(e % 8) / 2];
-              asm volatile("" : "+v"(x));
-              return (float)__builtin_bit_cast(_Float16, (uint16_t)(e % 2 ? x >> 16 : x & 0xffffu));
-            });
-          else
-            apply([&](int e) {
-              uint32_t x = w[e / 8][(e % 8) / 4][e % 4];
-              asm volatile("" : "+v"(x));
-              return __builtin_bit_cast(float, x);
-            });
-        };
         if (i == hold) {
-          from(held);
+          chain_operand<NE>(op, v, bad, half,
+                            chain_words([&](int p, int j, int c) { return held[p][j][c]; }, f16));
           if (pc == a.hold_last && turn + gridDim.x < turns)
             request(hold, row_of(turn + gridDim.x), held);
         } else {
           u32x4 w[P][2];
           request(i, row, w);
-          from(w);
+          chain_operand<NE>(op, v, bad, half,
+                            chain_words([&](int p, int j, int c) { return w[p][j][c]; }, f16));
         }
-        continue;
+      } else {
+        chain_plain<NE>(op, v, bad, imm, half);
       }
-      switch (op) {
-      case OP_CONST: HCAMD_CHAIN_EACH(v[e] = imm) break;
-      case OP_ADDI: HCAMD_CHAIN_EACH(v[e] = v[e] + imm) break;
-      case OP_SUBI: HCAMD_CHAIN_EACH(v[e] = v[e] - imm) break;
-      case OP_MULI: HCAMD_CHAIN_EACH(v[e] = v[e] * imm) break;
-      case OP_DIVI: HCAMD_CHAIN_EACH(v[e] = v[e] / imm) break;
-      case OP_MAXI: HCAMD_CHAIN_EACH(v[e] = nan_max(v[e], imm)) break;
-      case OP_MINI: HCAMD_CHAIN_EACH(v[e] = nan_min(v[e], imm)) break;
-      case OP_RSUBI: HCAMD_CHAIN_EACH(v[e] = imm - v[e]) break;
-      case OP_RDIVI: HCAMD_CHAIN_EACH(v[e] = imm / v[e]) break;
-      case OP_NEG: HCAMD_CHAIN_EACH(v[e] = -v[e]) break;
-      case OP_ABS: HCAMD_CHAIN_EACH(v[e] = __builtin_fabsf(v[e])) break;
-      case OP_SQRT: HCAMD_CHAIN_EACH(v[e] = __builtin_sqrtf(v[e])) break;
-      case OP_RINT: HCAMD_CHAIN_EACH(v[e] = __builtin_rintf(v[e])) break;
-      case OP_EXP: HCAMD_CHAIN_EACH(v[e] = expf(v[e])) break;
-      case OP_LOG: HCAMD_CHAIN_EACH(v[e] = logf(v[e])) break;
-      case OP_TANH: HCAMD_CHAIN_EACH(v[e] = tanh_selects(v[e])) break;
-      case OP_R16: HCAMD_CHAIN_EACH(v[e] = round16(v[e])) break;
-      case OP_SQ: HCAMD_CHAIN_EACH(v[e] = v[e] * v[e]) break;
-      case OP_MDIVI:
-      case OP_RMDIVI: {
-        float x[NE];
-#pragma unroll
-        for (int e = 0; e < NE; ++e) x[e] = imm;
-        if (op == OP_MDIVI)
-          masked_div<NE>(bad, v, v, x, half);
-        else
-          masked_div<NE>(bad, v, x, v, half);
-        break;
-      }
-      case OP_CLEAR:
-        bad = 0;
-        break;
-      case OP_POWCHK:
-        powchk_fn<NE>(bad, v);
-        break;
-      case OP_MSQRT:
-        domain_fn<false, NE>(bad, v);
-        break;
-      case OP_MLOG:
-        domain_fn<true, NE>(bad, v);
-        break;
-      default:
-        break;
-      }
-#undef HCAMD_CHAIN_EACH
     }
 
     if (kind <= ST_MIN) {
