@@ -1329,6 +1329,7 @@ struct RowArgs {
   uint32_t interleaved; // columns are dealt to lanes one by one (then vec_mask is 0)
   uint32_t n_col, n_stages, passes;
   uint32_t hold, hold_last; // chain kernels: the operand a lane keeps in registers, and the last instruction that reads it
+  uint32_t kept;            // chain kernels: byte i = the LDS slot (0, 1) that keeps operand i, a vector shared by all rows; 0xff: none
   Stage stage[kMaxStages];
   Instr prog[kRowProg];
 };
@@ -1648,6 +1649,11 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
   constexpr uint32_t R = T / LPR;                     // rows per workgroup and turn
   __shared__ float slots[2][T / kWave];
   __shared__ float red_cells[T / kWave][kMaxRed];
+  // Up to two operands that are one vector for every row (weights, a bias): a
+  // lane reads the same chunks of them in every row, so it fetches them once
+  // and parks them here, each lane its own words (no one else reads them, so
+  // nothing has to be synchronised): 100 cycles away instead of an L2 round trip.
+  __shared__ u32x4 parked[2][P][2][T];
   const uint32_t t = threadIdx.x, lane = t % LPR;
   float *cells = red_cells[t / kWave];
   const uint32_t per_row = (uint32_t)(a.cols / 8);
@@ -1699,6 +1705,19 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
   const uint32_t hold = a.hold & (kMaxIn - 1);
   u32x4 held[P][2];
   request(hold, row_of(blockIdx.x), held);
+#pragma unroll
+  for (int i = 0; i < kMaxIn; ++i) {
+    const uint32_t slot = (a.kept >> (8 * i)) & 0xffu;
+    if (slot < 2u) {
+      u32x4 w[P][2];
+      request((uint32_t)i, 0, w);
+#pragma unroll
+      for (int p = 0; p < P; ++p)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          parked[slot][p][j][t] = w[p][j];
+    }
+  }
 #pragma nounroll
   for (size_t turn = blockIdx.x; turn < turns; turn += gridDim.x) {
   const size_t row_at = turn * R + t / LPR;
@@ -1802,7 +1821,16 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
             request(hold, row_of(turn + gridDim.x), held);
         } else {
           u32x4 w[P][2];
-          request(i, row, w);
+          const uint32_t slot = (a.kept >> (8 * i)) & 0xffu;
+          if (slot < 2u) {
+#pragma unroll
+            for (int p = 0; p < P; ++p)
+#pragma unroll
+              for (int j = 0; j < 2; ++j)
+                w[p][j] = parked[slot][p][j][t];
+          } else {
+            request(i, row, w);
+          }
           chain_operand<NE>(op, v, bad, half,
                             chain_words([&](int p, int j, int c) { return w[p][j][c]; }, f16));
         }

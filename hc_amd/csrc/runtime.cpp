@@ -1866,7 +1866,7 @@ struct RowArgs {
   size_t rows, cols;
   uint32_t f16Mask, vecMask, interleaved;
   uint32_t nCol, nStages, passes;
-  uint32_t hold, holdLast;
+  uint32_t hold, holdLast, kept;
   RowStageDev stage[HCAMD_ROW_MAX_STAGES];
   HcamdMapInstr prog[HCAMD_ROW_MAX_INSTRS];
 };
@@ -2151,6 +2151,14 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       std::memset(a.prog, 0, sizeof a.prog);
       std::memcpy(a.prog, chained, nChained * sizeof(HcamdMapInstr));
       a.hold = static_cast<uint32_t>(hold);
+      // vectors shared by all rows stay in LDS, two at most
+      a.kept = 0xffffffffu;
+      unsigned slot = 0;
+      for (size_t i = 0; i < nInputs && slot < 2; ++i)
+        if (i != hold && reads[i] > 0 && (inputLd[i] == 0 || rows == 1)) {
+          a.kept &= ~(0xffu << (8 * i));
+          a.kept |= slot++ << (8 * i);
+        }
       for (size_t i = 0; i < nChained; ++i) {
         const unsigned op = chained[i].op;
         if ((op == HCAMD_MAP_IN || (op >= HCAMD_MAP_ADD_IN && op <= HCAMD_MAP_RDIV_IN) ||
