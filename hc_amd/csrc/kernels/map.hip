@@ -27,6 +27,8 @@
 // per element.
 #include "common.h"
 
+#include <type_traits>
+
 #pragma clang fp contract(off)
 
 using namespace hcamd;
@@ -267,7 +269,7 @@ template <int SP, int OP, int N> __device__ __forceinline__ void do_unary(StackT
 
 __device__ __forceinline__ bool is_finite(float x) { return __builtin_fabsf(x) < INFINITY; }
 // num / den under numpy.ma's rule, into `dst`
-template <int N>
+template <int N, int B0 = 0> // B0: the bit of element 0
 __device__ __forceinline__ void masked_div(uint32_t &bad_bits, float *dst, const float *num,
                                            const float *den, bool half) {
   uint32_t bad = bad_bits;
@@ -282,7 +284,26 @@ __device__ __forceinline__ void masked_div(uint32_t &bad_bits, float *dst, const
     // the mask that way): a quotient of -0 becomes +0 unless the dividend is negative
     q += 0.0f * n;
     dst[e] = good ? q : 0.0f + n;
+    bad |= good ? 0u : (1u << (B0 + e));
+  }
+  bad_bits = bad;
+}
+// the same with one of the two a scalar (an immediate, a row scalar): v = v / s, or v = s / v
+template <int N, bool REVERSED>
+__device__ __forceinline__ void masked_div_scalar(uint32_t &bad_bits, float *v, float s, bool half) {
+  uint32_t bad = bad_bits;
+#pragma unroll
+  for (int e = 0; e < N; ++e) {
+    const float n = REVERSED ? s : v[e];
+    float q = REVERSED ? s / v[e] : v[e] / s;
+    if (half)
+      q = round16(q);
+    const bool good = is_finite(q);
+    q += 0.0f * n;
+    v[e] = good ? q : 0.0f + n;
     bad |= good ? 0u : (1u << e);
+    if (e % 4 == 3)
+      __builtin_amdgcn_sched_barrier(0);
   }
   bad_bits = bad;
 }
@@ -978,7 +999,7 @@ constexpr uint32_t OP_SQ = 63; // top = top * top; made by the host, not part of
 // Four elements at a time: the fence keeps the scheduler from interleaving all
 // NE, whose temporaries (a division, an exponential) would not fit.
 #define HCAMD_CHAIN_EACH(EXPR)                                                    \
-  _Pragma("unroll") for (int g = 0; g < NE / 4; ++g) {                            \
+  _Pragma("unroll") for (int g = E0 / 4; g < E1 / 4; ++g) {                       \
     _Pragma("unroll") for (int e = 4 * g; e < 4 * g + 4; ++e) { EXPR; }           \
     __builtin_amdgcn_sched_barrier(0);                                            \
   }
@@ -989,7 +1010,8 @@ __device__ __forceinline__ bool chain_reads(uint32_t op) {
 }
 // v = v op operand for the instructions that name an operand; rhs(e) is the
 // operand's element e, read straight from where it was loaded to.
-template <int NE, class Rhs>
+// Elements E0 .. E1-1 of v (all of it, or the part whose operand words are at hand).
+template <int NE, int E0 = 0, int E1 = NE, class Rhs>
 __device__ __forceinline__ void chain_operand(uint32_t op, float (&v)[NE], uint32_t &bad, bool half,
                                               Rhs rhs) {
   auto apply = [&](auto at) {
@@ -1004,13 +1026,13 @@ __device__ __forceinline__ void chain_operand(uint32_t op, float (&v)[NE], uint3
     case OP_RSUB_IN: HCAMD_CHAIN_EACH(v[e] = at(e) - v[e]) break;
     case OP_RDIV_IN: HCAMD_CHAIN_EACH(v[e] = at(e) / v[e]) break;
     default: { // the numpy.ma quotients
-      float x[NE];
+      float x[E1 - E0];
 #pragma unroll
-      for (int e = 0; e < NE; ++e) x[e] = at(e);
+      for (int e = E0; e < E1; ++e) x[e - E0] = at(e);
       if (op == OP_MDIV_IN)
-        masked_div<NE>(bad, v, v, x, half);
+        masked_div<E1 - E0, E0>(bad, v + E0, v + E0, x, half);
       else
-        masked_div<NE>(bad, v, x, v, half);
+        masked_div<E1 - E0, E0>(bad, v + E0, x, v + E0, half);
     }
     }
   };
@@ -1041,6 +1063,7 @@ template <class Word> __device__ __forceinline__ auto chain_words(Word word, boo
 template <int NE>
 __device__ __forceinline__ void chain_plain(uint32_t op, float (&v)[NE], uint32_t &bad, float imm,
                                             bool half) {
+  constexpr int E0 = 0, E1 = NE;
   switch (op) {
   case OP_CONST: HCAMD_CHAIN_EACH(v[e] = imm) break;
   case OP_ADDI: HCAMD_CHAIN_EACH(v[e] = v[e] + imm) break;
@@ -1061,16 +1084,11 @@ __device__ __forceinline__ void chain_plain(uint32_t op, float (&v)[NE], uint32_
   case OP_R16: HCAMD_CHAIN_EACH(v[e] = round16(v[e])) break;
   case OP_SQ: HCAMD_CHAIN_EACH(v[e] = v[e] * v[e]) break;
   case OP_MDIVI:
-  case OP_RMDIVI: {
-    float x[NE];
-#pragma unroll
-    for (int e = 0; e < NE; ++e) x[e] = imm;
-    if (op == OP_MDIVI)
-      masked_div<NE>(bad, v, v, x, half);
-    else
-      masked_div<NE>(bad, v, x, v, half);
+    masked_div_scalar<NE, false>(bad, v, imm, half);
     break;
-  }
+  case OP_RMDIVI:
+    masked_div_scalar<NE, true>(bad, v, imm, half);
+    break;
   case OP_CLEAR:
     bad = 0;
     break;
@@ -1088,6 +1106,30 @@ __device__ __forceinline__ void chain_plain(uint32_t op, float (&v)[NE], uint32_
   }
 }
 #undef HCAMD_CHAIN_EACH
+// one instruction of a chain on one value (the stages that compute with row scalars)
+__device__ __forceinline__ void chain_scalar(uint32_t op, float &sv, float imm) {
+  switch (op) {
+  case OP_CONST: sv = imm; break;
+  case OP_ADDI: sv = sv + imm; break;
+  case OP_SUBI: sv = sv - imm; break;
+  case OP_MULI: sv = sv * imm; break;
+  case OP_DIVI: sv = sv / imm; break;
+  case OP_MAXI: sv = nan_max(sv, imm); break;
+  case OP_MINI: sv = nan_min(sv, imm); break;
+  case OP_RSUBI: sv = imm - sv; break;
+  case OP_RDIVI: sv = imm / sv; break;
+  case OP_NEG: sv = -sv; break;
+  case OP_ABS: sv = __builtin_fabsf(sv); break;
+  case OP_SQRT: sv = __builtin_sqrtf(sv); break;
+  case OP_RINT: sv = __builtin_rintf(sv); break;
+  case OP_EXP: sv = expf(sv); break;
+  case OP_LOG: sv = logf(sv); break;
+  case OP_TANH: sv = tanh_selects(sv); break;
+  case OP_R16: sv = round16(sv); break;
+  case OP_SQ: sv = sv * sv; break;
+  default: break;
+  }
+}
 
 __device__ __forceinline__ float col_fold(uint32_t kind, float a, float b) {
   return kind == COL_SUM ? a + b : kind == COL_MAX ? nan_max(a, b) : nan_min(a, b);
@@ -1328,8 +1370,7 @@ struct RowArgs {
   uint32_t vec_mask; // bit i: rows of operand i start on 16-byte boundaries; bit 8: the output
   uint32_t interleaved; // columns are dealt to lanes one by one (then vec_mask is 0)
   uint32_t n_col, n_stages, passes;
-  uint32_t hold, hold_last; // chain kernels: the operand a lane keeps in registers, and the last instruction that reads it
-  uint32_t kept;            // chain kernels: byte i = the LDS slot (0, 1) that keeps operand i, a vector shared by all rows; 0xff: none
+  uint32_t hold, hold_last; // chain kernels: the operand that stays in LDS for the row, and the last instruction that reads it
   Stage stage[kMaxStages];
   Instr prog[kRowProg];
 };
@@ -1631,45 +1672,52 @@ __attribute__((amdgpu_waves_per_eu(4, 4))) void hcamd_row_program_w64(const RowA
 // at once: an operand, then operations that change it in place (`in sub_red exp`,
 // `in sub_red mdiv_red mul_in add_in`).  For those the evaluation stack is one
 // value per element, and a lane can afford all of its row at once: P chunks of
-// eight (P = 1, 2; rows of at most P * LPR chunks, LPR = 64 ... 1024 lanes to a row), so that one dispatch of an
-// instruction works on 8 P elements instead of 8 and the dispatch, which is what
-// bounds the general kernel above, is paid a P-th as often.  The operand most
-// stages read (`hold`) is fetched once, every chunk requested before the first
-// stage starts, and stays in registers; any other operand is fetched by the
-// instruction that names it.  The host decides (hcamdLaunchRowProgram): every
-// stage a chain, whole chunks only (columns a multiple of 8, 16-byte aligned
-// rows), at most 4 chunks per lane; `x x mul` with equal halves arrives as
-// `x sq`.  Everything else is as above: the same stages, row scalars, numpy.ma
-// forms and fixed order of additions (lane order differs from the general
-// kernel's, so sums agree with it to rounding, not bit for bit).
+// eight (P = 1, 2, 4; rows of at most P * LPR chunks on LPR = 64 ... 1024 lanes),
+// so that one dispatch of an instruction works on 8 P elements instead of 8 and
+// the dispatch, which is what bounds the general kernel above, is paid a P-th as
+// often.  The operand most instructions read (`hold`) is fetched once per row and
+// lives in LDS, each lane its own words (so nothing has to be synchronised),
+// written there by the loads themselves (buffer_load ... lds), which is also how
+// the next row arrives while the last stage still runs: a workgroup takes rows
+// in turns, and requests the next one as soon as this one has been read for the
+// last time.  Every other operand is fetched by the instruction that names it,
+// two chunks at a time.  That leaves the registers to the running values.  The
+// host decides (hcamdLaunchRowProgram): every stage a chain, whole chunks only
+// (columns a multiple of 8, 16-byte aligned rows), at most 4096 chunks; `x x
+// mul` with equal halves arrives as `x sq`.  Everything else is as above: the
+// same stages, row scalars, numpy.ma forms and fixed order of additions (lane
+// order differs from the general kernel's, so sums agree with it to rounding,
+// not bit for bit).
 namespace {
+typedef __attribute__((address_space(3))) void *row_lds_ptr;
+
 template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArgs &a) {
   constexpr int NE = 8 * P;
+  constexpr int CH = P < 2 ? P : 2; // chunks of another operand fetched at a time
   constexpr int T = LPR < kThreads ? kThreads : LPR; // threads of a workgroup
   constexpr uint32_t R = T / LPR;                     // rows per workgroup and turn
   __shared__ float slots[2][T / kWave];
   __shared__ float red_cells[T / kWave][kMaxRed];
-  // Up to two operands that are one vector for every row (weights, a bias): a
-  // lane reads the same chunks of them in every row, so it fetches them once
-  // and parks them here, each lane its own words (no one else reads them, so
-  // nothing has to be synchronised): 100 cycles away instead of an L2 round trip.
-  __shared__ u32x4 parked[2][P][2][T];
+  __shared__ __attribute__((aligned(1024))) u32x4 row_words[P][2][T];
   const uint32_t t = threadIdx.x, lane = t % LPR;
   float *cells = red_cells[t / kWave];
   const uint32_t per_row = (uint32_t)(a.cols / 8);
   const bool out_f16 = (a.f16_mask >> 8) & 1;
   uint32_t parity = 0;
-  // A workgroup takes rows in turns, the grid apart: as many workgroups as the
-  // device holds at once, so none waits to be launched behind another.
   const size_t turns = (a.rows + R - 1) / R;
-  // chunk p of this lane is chunk p * LPR + lane of the row (chunk 0 where the
-  // row has no such chunk: loaded, never used)
-  auto chunk_at = [&](int p) {
-    const uint32_t c = (uint32_t)p * LPR + lane;
+  // (`ln`: the lane's number in its row, handed in through an empty asm statement
+  // where addresses are made: computed from `lane` itself they are loop
+  // invariants, and a dozen hoisted address registers spill)
+  auto chunk_at = [&](int p, uint32_t ln) {
+    const uint32_t c = (uint32_t)p * LPR + ln;
     return c < per_row ? c : 0u;
   };
-  // The chunks of operand i in row `r` as loaded: 8 fp16 in w[p][0], 8 fp32 in w[p][0..1].
-  auto request = [&](uint32_t i, size_t r, u32x4 (&w)[P][2]) {
+  auto row_of = [&](size_t turn) { // idle waves compute on row 0 and store nothing
+    const size_t r = turn * R + t / LPR;
+    return r < a.rows ? r : (size_t)0;
+  };
+  // operand i's chunks p0 .. p0 + CH - 1 of row r, into registers
+  auto request = [&](uint32_t i, size_t r, int p0, u32x4 (&w)[CH][2]) {
     const void *in = a.in[0];
     size_t ld = a.ld[0];
 #pragma unroll
@@ -1679,73 +1727,78 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
     }
     const bool f16 = (a.f16_mask >> i) & 1;
     const char *b = static_cast<const char *>(in) + r * ld * (f16 ? 2 : 4);
-    if (f16) {
+    uint32_t ln = lane;
+    asm volatile("" : "+v"(ln));
 #pragma unroll
-      for (int p = 0; p < P; ++p) {
-        w[p][0] = ldg<false>(reinterpret_cast<const u32x4 *>(b) + chunk_at(p));
+    for (int p = 0; p < CH; ++p) {
+      if (f16) {
+        w[p][0] = ldg<false>(reinterpret_cast<const u32x4 *>(b) + chunk_at(p0 + p, ln));
         w[p][1] = u32x4{0u, 0u, 0u, 0u};
-      }
-    } else {
-#pragma unroll
-      for (int p = 0; p < P; ++p) {
-        const u32x4 *q = reinterpret_cast<const u32x4 *>(b) + 2 * chunk_at(p);
+      } else {
+        const u32x4 *q = reinterpret_cast<const u32x4 *>(b) + 2 * chunk_at(p0 + p, ln);
         w[p][0] = ldg<false>(q);
         w[p][1] = ldg<false>(q + 1);
       }
     }
   };
-  auto row_of = [&](size_t turn) { // idle lanes compute on row 0 and store nothing
-    const size_t r = turn * R + t / LPR;
-    return r < a.rows ? r : (size_t)0;
-  };
-  // The held operand's row: requested here for the first turn, and for every
-  // later one by the turn before it, as soon as that has read the operand for
-  // the last time (instruction `hold_last`), so that the row arrives while the
-  // rest of the last stage runs.
+  // The held operand's row r, from memory straight into this wave's words of
+  // row_words.  A wave belongs to one row (LPR >= 64), so the row's address is
+  // wave-uniform: it goes into the buffer descriptor, the lane's part into the
+  // 32-bit offset (a row is shorter than 2^31 bytes: the host has checked).
   const uint32_t hold = a.hold & (kMaxIn - 1);
-  u32x4 held[P][2];
-  request(hold, row_of(blockIdx.x), held);
+  const bool hold_f16 = (a.f16_mask >> hold) & 1;
+  const void *hold_in = a.in[0];
+  size_t hold_ld = a.ld[0];
 #pragma unroll
-  for (int i = 0; i < kMaxIn; ++i) {
-    const uint32_t slot = (a.kept >> (8 * i)) & 0xffu;
-    if (slot < 2u) {
-      u32x4 w[P][2];
-      request((uint32_t)i, 0, w);
-#pragma unroll
-      for (int p = 0; p < P; ++p)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          parked[slot][p][j][t] = w[p][j];
-    }
+  for (int k = 1; k < kMaxIn; ++k) {
+    hold_in = hold == (uint32_t)k ? a.in[k] : hold_in;
+    hold_ld = hold == (uint32_t)k ? a.ld[k] : hold_ld;
   }
+  auto fetch_row = [&](size_t r) {
+    const uint64_t at = reinterpret_cast<uint64_t>(hold_in) + r * hold_ld * (hold_f16 ? 2 : 4);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)at);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(at >> 32));
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        reinterpret_cast<void *>(((uint64_t)hi << 32) | lo), 0, (int)(a.cols * (hold_f16 ? 2 : 4)),
+        0x00020000);
+    const uint32_t wave_first = __builtin_amdgcn_readfirstlane(t & ~(uint32_t)(kWave - 1));
+    uint32_t ln = lane;
+    asm volatile("" : "+v"(ln));
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      const int off = (int)(chunk_at(p, ln) * (hold_f16 ? 16u : 32u));
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (row_lds_ptr)&row_words[p][0][wave_first], 16, off, 0,
+                                               0, 0);
+      if (!hold_f16)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (row_lds_ptr)&row_words[p][1][wave_first], 16, off,
+                                                 16, 0, 0); // the scalar offset: memory side only
+    }
+  };
+  fetch_row(row_of(blockIdx.x));
 #pragma nounroll
   for (size_t turn = blockIdx.x; turn < turns; turn += gridDim.x) {
   const size_t row_at = turn * R + t / LPR;
   const bool row_live = row_at < a.rows;
   const size_t row = row_of(turn);
-  // bit p of `live`: chunk p of this lane exists
-  uint32_t live = 0;
+  uint32_t live = 0; // bit p: chunk p of this lane exists
 #pragma unroll
   for (int p = 0; p < P; ++p)
     live |= (row_live && (uint32_t)p * LPR + lane < per_row) ? 1u << p : 0u;
-
   if (t % kWave < kMaxRed)
     cells[t % kWave] = 0.0f;
 #pragma unroll
   for (int k = 0; k < kMaxIn; ++k)
     if (k < (int)a.n_col)
       cells[k] = uniform(load_elem(a.col[k], (a.f16_mask >> (16 + k)) & 1, row));
-
   char *const orow = static_cast<char *>(a.out) + row * a.ldo * (out_f16 ? 2 : 4);
+  // the row requested by the turn before (or above) has to be there
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
 #pragma nounroll
   for (uint32_t s = 0; s < a.n_stages; ++s) {
     const Stage st = a.stage[s];
     const uint32_t kind = st.kind;
-    // the row scalars, scalar k in lane k
     const uint32_t reds = __builtin_bit_cast(uint32_t, cells[t & (kMaxRed - 1)]);
-    // the instruction at pc, a scalar form rewritten into the immediate form
-    // with the row scalar as the immediate
     auto decode = [&](Instr cur, uint32_t &op, float &imm) {
       op = cur.op;
       uint32_t imm_bits = __builtin_bit_cast(uint32_t, cur.imm);
@@ -1760,7 +1813,6 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
     };
     Instr next = a.prog[st.begin & (kRowProg - 1)];
     if (kind == ST_SCALAR || kind == ST_STORE_COL) {
-      // arithmetic on row scalars: one value
       float sv = 0.0f;
 #pragma nounroll
       for (uint32_t pc = st.begin; pc < st.end; ++pc) {
@@ -1769,27 +1821,7 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
         uint32_t op;
         float imm;
         decode(cur, op, imm);
-        switch (op) {
-        case OP_CONST: sv = imm; break;
-        case OP_ADDI: sv = sv + imm; break;
-        case OP_SUBI: sv = sv - imm; break;
-        case OP_MULI: sv = sv * imm; break;
-        case OP_DIVI: sv = sv / imm; break;
-        case OP_MAXI: sv = nan_max(sv, imm); break;
-        case OP_MINI: sv = nan_min(sv, imm); break;
-        case OP_RSUBI: sv = imm - sv; break;
-        case OP_RDIVI: sv = imm / sv; break;
-        case OP_NEG: sv = -sv; break;
-        case OP_ABS: sv = __builtin_fabsf(sv); break;
-        case OP_SQRT: sv = __builtin_sqrtf(sv); break;
-        case OP_RINT: sv = __builtin_rintf(sv); break;
-        case OP_EXP: sv = expf(sv); break;
-        case OP_LOG: sv = logf(sv); break;
-        case OP_TANH: sv = tanh_selects(sv); break;
-        case OP_R16: sv = round16(sv); break;
-        case OP_SQ: sv = sv * sv; break;
-        default: break;
-        }
+        chain_scalar(op, sv, imm);
       }
       if (kind == ST_SCALAR)
         cells[st.dst & (kMaxRed - 1)] = uniform(sv);
@@ -1814,25 +1846,28 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
       if (chain_reads(op)) {
         const uint32_t i = arg & (kMaxIn - 1);
         const bool f16 = (a.f16_mask >> i) & 1;
-        if (i == hold) {
-          chain_operand<NE>(op, v, bad, half,
-                            chain_words([&](int p, int j, int c) { return held[p][j][c]; }, f16));
-          if (pc == a.hold_last && turn + gridDim.x < turns)
-            request(hold, row_of(turn + gridDim.x), held);
-        } else {
-          u32x4 w[P][2];
-          const uint32_t slot = (a.kept >> (8 * i)) & 0xffu;
-          if (slot < 2u) {
+        // CH chunks at a time: their words, then the operation on those elements
+        auto part = [&](auto number) {
+          constexpr int h = decltype(number)::value;
+          u32x4 w[CH][2];
+          if (i == hold) {
 #pragma unroll
-            for (int p = 0; p < P; ++p)
+            for (int p = 0; p < CH; ++p)
 #pragma unroll
               for (int j = 0; j < 2; ++j)
-                w[p][j] = parked[slot][p][j][t];
+                w[p][j] = row_words[CH * h + p][j][t];
           } else {
-            request(i, row, w);
+            request(i, row, CH * h, w);
           }
-          chain_operand<NE>(op, v, bad, half,
-                            chain_words([&](int p, int j, int c) { return w[p][j][c]; }, f16));
+          chain_operand<NE, 8 * CH * h, 8 * CH * (h + 1)>(
+              op, v, bad, half, chain_words([&](int p, int j, int c) { return w[p - CH * h][j][c]; }, f16));
+        };
+        part(std::integral_constant<int, 0>{});
+        if constexpr (P > CH)
+          part(std::integral_constant<int, 1>{});
+        if (i == hold && pc == a.hold_last && turn + gridDim.x < turns) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the words have been read
+          fetch_row(row_of(turn + gridDim.x));
         }
       } else {
         chain_plain<NE>(op, v, bad, imm, half);
@@ -1841,7 +1876,6 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
 
     if (kind <= ST_MIN) {
       float acc = kind == ST_MAX ? -INFINITY : kind == ST_MIN ? INFINITY : 0.0f;
-      // a wave whose lanes all hold P chunks with every element active folds without masks
       if (__builtin_amdgcn_ballot_w64(bad != 0 || live != (1u << P) - 1u) == 0) {
         if (kind == ST_SUM) {
 #pragma unroll
@@ -1867,7 +1901,7 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
       }
       constexpr int W = LPR / kWave;
       float total;
-      float *mine = slots[parity] + (t / LPR) * W; // the slots of this row's waves
+      float *mine = slots[parity] + (t / LPR) * W;
       if (kind == ST_SUM)
         total = group_reduce<SumOp, W>(acc, mine);
       else if (kind == ST_MAX)
@@ -1876,27 +1910,31 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
         total = group_reduce<NanMinOp, W>(acc, mine);
       parity ^= 1;
       cells[st.dst & (kMaxRed - 1)] = total;
-    } else if (kind == ST_STORE) {
-      char *o = orow; // opaque: the element addresses of the masked form are not loop invariants
-      asm volatile("" : "+v"(o));
+    } else {
+      char *o = orow;
+      uint32_t ln = lane;
+      asm volatile("" : "+v"(o), "+v"(ln));
 #pragma unroll
       for (int p = 0; p < P; ++p)
         if ((live >> p) & 1u)
-          store_chunk(o, out_f16, (size_t)p * LPR + lane, v + 8 * p, (bad >> (8 * p)) & 0xffu);
+          store_chunk(o, out_f16, (size_t)p * LPR + ln, v + 8 * p, (bad >> (8 * p)) & 0xffu);
     }
   }
   } // turns
 }
 } // namespace
 
+// (one and two chunks per lane leave registers for six waves per SIMD)
 #define HCAMD_ROW_CHAIN(LPR, P, T)                                                       \
-  extern "C" __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(4, 4)))   \
+  extern "C" __global__ __launch_bounds__(T)                                              \
+      __attribute__((amdgpu_waves_per_eu(P <= 2 ? 6 : 4, P <= 2 ? 6 : 4)))                \
   void hcamd_row_program_chain_w##LPR##_p##P(const RowArgs a) {                          \
     row_chain<LPR, P>(a);                                                                 \
   }
 HCAMD_ROW_CHAIN(64, 1, 256)
 HCAMD_ROW_CHAIN(64, 2, 256)
-HCAMD_ROW_CHAIN(128, 2, 256)
-HCAMD_ROW_CHAIN(256, 2, 256)
-HCAMD_ROW_CHAIN(512, 2, 512)
-HCAMD_ROW_CHAIN(1024, 2, 1024)
+HCAMD_ROW_CHAIN(64, 4, 256)
+HCAMD_ROW_CHAIN(128, 4, 256)
+HCAMD_ROW_CHAIN(256, 4, 256)
+HCAMD_ROW_CHAIN(512, 4, 512)
+HCAMD_ROW_CHAIN(1024, 4, 1024)

@@ -1866,7 +1866,7 @@ struct RowArgs {
   size_t rows, cols;
   uint32_t f16Mask, vecMask, interleaved;
   uint32_t nCol, nStages, passes;
-  uint32_t hold, holdLast, kept;
+  uint32_t hold, holdLast;
   RowStageDev stage[HCAMD_ROW_MAX_STAGES];
   HcamdMapInstr prog[HCAMD_ROW_MAX_INSTRS];
 };
@@ -2107,14 +2107,14 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
     a.vecMask = 0;
     a.interleaved = 1;
   }
-  // Rows of whole, aligned chunks, at most 2048 of them, whose stages are all
+  // Rows of whole, aligned chunks, at most 4096 of them, whose stages are all
   // chains run on the chain kernels: a lane has its whole part of the row at
-  // once, 8 or 16 elements to a dispatch, and the operand that most
-  // instructions read stays in registers (variant 1 of "rows": never).
+  // once, 8, 16 or 32 elements to a dispatch, and the operand that most
+  // instructions read stays in LDS for the row (variant 1 of "rows": never).
   size_t lanes = lanesPerRow, maxGroups = SIZE_MAX, threads = 256;
   char name[48];
   std::snprintf(name, sizeof name, "hcamd_row_program_w%zu", lanes);
-  if (variantOf("rows") != 1 && !a.interleaved && cols % 8 == 0 && perRow <= 2048 && nInputs > 0) {
+  if (variantOf("rows") != 1 && !a.interleaved && cols % 8 == 0 && perRow <= 4096 && nInputs > 0) {
     HcamdMapInstr chained[HCAMD_ROW_MAX_INSTRS];
     size_t nChained = 0;
     uint16_t begin[HCAMD_ROW_MAX_STAGES], end[HCAMD_ROW_MAX_STAGES];
@@ -2139,7 +2139,8 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       if (reads[i] > reads[hold])
         hold = i;
     if (ok && reads[hold] > 0) {
-      const unsigned p = perRow <= 64 ? 1 : 2;
+      // one, two or four chunks per lane of a wave, then four on more lanes
+      const unsigned p = perRow <= 64 ? 1 : perRow <= 128 ? 2 : 4;
       lanes = 64;
       while (lanes * p < perRow)
         lanes *= 2;
@@ -2151,14 +2152,6 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       std::memset(a.prog, 0, sizeof a.prog);
       std::memcpy(a.prog, chained, nChained * sizeof(HcamdMapInstr));
       a.hold = static_cast<uint32_t>(hold);
-      // vectors shared by all rows stay in LDS, two at most
-      a.kept = 0xffffffffu;
-      unsigned slot = 0;
-      for (size_t i = 0; i < nInputs && slot < 2; ++i)
-        if (i != hold && reads[i] > 0 && (inputLd[i] == 0 || rows == 1)) {
-          a.kept &= ~(0xffu << (8 * i));
-          a.kept |= slot++ << (8 * i);
-        }
       for (size_t i = 0; i < nChained; ++i) {
         const unsigned op = chained[i].op;
         if ((op == HCAMD_MAP_IN || (op >= HCAMD_MAP_ADD_IN && op <= HCAMD_MAP_RDIV_IN) ||
@@ -2168,7 +2161,7 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       }
       std::snprintf(name, sizeof name, "hcamd_row_program_chain_w%zu_p%u", lanes, p);
       // these kernels walk the rows themselves: as many workgroups as are resident at once
-      maxGroups = (size_t)computeUnitsOf(dev) * 16 / (threads / 64);
+      maxGroups = (size_t)computeUnitsOf(dev) * (p <= 2 ? 24 : 16) / (threads / 64); // 6 or 4 waves per SIMD
     }
   }
   Kernel *k = builtinKernel(dev, "map", name);

@@ -61,12 +61,12 @@ def np_softmax(x):
 
 def kernel_for(cols, general=False):
     """The kernel hcamdLaunchRowProgram picks for dense, 16-byte aligned rows whose
-    stages are all chains: a chain kernel for whole chunks up to 2048 of them (one
-    chunk per lane up to 64, else two, on 64 ... 1024 lanes), else the general one
-    (a wave per row up to 4096 columns, else a workgroup)."""
+    stages are all chains: a chain kernel for whole chunks up to 4096 of them (one,
+    two or four chunks per lane of a wave, then four on 128 ... 1024 lanes), else the
+    general one (a wave per row up to 4096 columns, else a workgroup)."""
     per_row = cols // 8
-    if not general and cols % 8 == 0 and per_row <= 2048:
-        p = 1 if per_row <= 64 else 2
+    if not general and cols % 8 == 0 and per_row <= 4096:
+        p = 1 if per_row <= 64 else 2 if per_row <= 128 else 4
         lanes = 64
         while lanes * p < per_row:
             lanes *= 2
@@ -88,7 +88,7 @@ def rows_variant(request):
 @pytest.mark.parametrize("rows,cols", [(1, 1), (30, 25), (7, 8), (5, 512), (9, 513), (33, 2048),
                                        (17, 4099), (64, 8192), (3, 16384), (2, 16392), (2, 40_001),
                                        (4501, 512), (4203, 1000), (2051, 2048), (1101, 4096),
-                                       (603, 8192), (301, 16384)])
+                                       (603, 8192), (301, 16384), (5, 32768), (300, 32768)])
 def test_softmax_as_a_row_program(ctx, rows, cols, rows_variant):
     rng = np.random.default_rng(cols)
     x = (rng.standard_normal((rows, cols)) * 3).astype(np.float32)
