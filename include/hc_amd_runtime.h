@@ -508,11 +508,11 @@ int hcamdLaunchMapReduceColsNoAlloc(OlQueue q, int kind, const HcamdMapInstr *pr
  * reads the operands it uses again (a row just read is still in L2).  Programs
  * whose stages all change one value in place (an operand, then *I, *_IN, *_RED
  * and unary forms; `x x MUL` with two equal halves counts) over 16-byte aligned
- * rows of whole chunks of 8 elements, at most 16384 of them, run on kernels that
- * keep a lane's whole part of the row in registers: the operand most
- * instructions read is fetched once per row, and an instruction is dispatched
- * once for 8 or 16 elements of a lane (variant 1 of the "rows" family keeps the
- * general kernel).  Sums add in an order that
+ * rows of whole chunks of 8 elements, at most 32768 elements, run on kernels that
+ * take a lane's whole part of the row at once: the operand most instructions
+ * read is fetched once per row (into LDS), and an instruction is dispatched
+ * once for 8, 16 or 32 elements of a lane (variant 1 of the "rows" family keeps
+ * the general kernel).  Sums add in an order that
  * depends on the shape and the kernel only: results are reproducible, and agree with a
  * sequential fp32 sum to within the usual n * 2^-24 bound. */
 enum HcamdRowStageKind {
