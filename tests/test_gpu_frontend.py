@@ -717,7 +717,10 @@ def test_autotune_of_the_convolution_example():
 # ---------------------------------------------------------------------------
 # bodies with reductions along rows -> hcamdLaunchRowProgram
 # ---------------------------------------------------------------------------
-@pytest.mark.parametrize("rows,n", [(37, 200), (64, 4096), (9, 4104), (5, 20_003)])
+# (one, two and four chunks per lane of the chain kernels, 64 ... 1024 lanes to a row, more rows
+# than workgroups; 20,003 columns: the general kernel)
+@pytest.mark.parametrize("rows,n", [(37, 200), (64, 4096), (9, 4104), (5, 20_003), (4400, 1000),
+                                    (12, 16384), (3, 32768)])
 @pytest.mark.parametrize("name", ["layernorm", "rmsnorm_half", "log_softmax_t", "row_norms", "spread",
                                   "unit_rows", "log_sum_exp"])
 def test_row_reduction_bodies_match_the_simulator(name, rows, n):
