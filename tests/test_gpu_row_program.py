@@ -282,3 +282,58 @@ def test_numpy_ma_forms_and_partly_empty_lanes_on_the_chain_kernels(ctx, rows_va
                         [dx], tops).launch(sync=True)
     want = np.log(np.where(x > 0, x, np.float32(1e-30)).astype(np.float64)).max(axis=1)
     assert_allclose(tops.to_host(), want, rtol=2e-6, atol=1e-6)
+
+
+def _every_chain_instruction():
+    """One stored tile per instruction a chain may hold: `in(0)` followed by the
+    instruction (operand 1 for the *_in forms, column 0 for the *_red forms), the
+    numpy.ma forms with and without the fp16 flag, and a program that ends after
+    a form that deactivates elements followed by more arithmetic."""
+    progs = {}
+    for name in ("neg", "abs", "sqrt", "rint", "exp", "log", "tanh", "r16", "clear", "powchk",
+                 "msqrt", "mlog"):
+        progs[name] = [I("in", 0), I(name)]
+    for name in ("add", "sub", "mul", "div", "max", "min", "rsub", "rdiv"):
+        progs[name + "_in"] = [I("in", 0), I(name + "_in", 1)]
+        progs[name + "i"] = [I("in", 0), I(name + "i", 0, 0.75)]
+        progs[name + "_red"] = [I("in", 0), I(name + "_red", 0)]
+    for flag in (0, 0x100):
+        tag = "_h" if flag else ""
+        progs["mdivi" + tag] = [I("in", 0), I("mdivi", flag, 0.0)]           # every element deactivated
+        progs["rmdivi" + tag] = [I("in", 0), I("rmdivi", flag, 2.0)]         # where x is 0
+        progs["mdiv_in" + tag] = [I("in", 0), I("mdiv_in", 1 | flag)]
+        progs["rmdiv_in" + tag] = [I("in", 0), I("rmdiv_in", 1 | flag)]
+        progs["mdiv_red" + tag] = [I("in", 0), I("mdiv_red", flag)]
+        progs["rmdiv_red" + tag] = [I("in", 0), I("rmdiv_red", flag)]
+    progs["square"] = [I("in", 0), I("sub_red", 0), I("in", 0), I("sub_red", 0), I("mul")]
+    progs["after_mask"] = [I("in", 1), I("rmdiv_in", 0), I("addi", 0, 1.0), I("msqrt"), I("mul_in", 1)]
+    progs["const_first"] = [I("const", 0, 3.0), I("sub_in", 0), I("mlog"), I("clear")]
+    return progs
+
+
+@pytest.mark.parametrize("rows,cols,dtype", [(70, 512, np.float32), (300, 1000, np.float16),
+                                             (50, 4096, np.float32), (9, 16384, np.float16)])
+def test_every_instruction_of_a_chain_computes_what_the_general_kernel_computes(ctx, rows, cols, dtype):
+    """Element-wise stages do the same arithmetic on both kernels: the stored tiles
+    are equal bit for bit, including which elements the numpy.ma forms leave
+    untouched, on one, two and four chunks per lane and both storage types."""
+    rng = np.random.default_rng(rows)
+    x = (rng.standard_normal((rows, cols)) * 3).astype(dtype)
+    y = (rng.standard_normal((rows, cols)) * 3).astype(dtype)
+    for a in (x, y):                                   # zeros, negatives are there; add specials
+        a[::3, ::5] = 0
+        a[1, 7], a[2, 9], a[3, 11] = np.inf, -np.inf, np.nan
+    col = rng.standard_normal(rows).astype(np.float32)
+    col[::4] = 0
+    dx, dy, dcol = rt.to_device(x), rt.to_device(y), rt.to_device(col)
+    for name, program in _every_chain_instruction().items():
+        results = []
+        for variant in (0, 1):
+            rt.set_variant("rows", variant)
+            out = poisoned((rows, cols), dtype)
+            rt.plan_row_program([("store", 0, program)], [dx, dy], out, columns=[dcol]).launch(sync=True)
+            assert rt.last_kernel_name() == kernel_for(cols, general=variant == 1), name
+            results.append(out.to_host())
+        rt.set_variant("rows", 0)
+        bits = np.uint32 if dtype == np.float32 else np.uint16
+        assert_array_equal(results[0].view(bits), results[1].view(bits), err_msg=name)
