@@ -819,6 +819,11 @@ HCAMD_MAP_FLAT(hcamd_map_sum_flat_n2u2, 2, 2, false, true)
 HCAMD_MAP_FLAT(hcamd_map_sum_flat_n1u4, 1, 4, false, true)
 HCAMD_MAP_FLAT(hcamd_map_sum_flat_n4u2h, 4, 2, true, true)
 HCAMD_MAP_FLAT(hcamd_map_sum_flat_n2u4h, 2, 4, true, true)
+// The map itself with one or two fp16 operands: a single chunk per lane
+// (hcamd_map_flat below) is 16 or 32 bytes in flight, too few to fill the memory
+// system (8192 x 8192: 56 -> 45 us with one operand).  With fp32 operands the
+// same form measured slower than one chunk per lane (96 -> 107 us).
+HCAMD_MAP_FLAT(hcamd_map_flat_n2u4h, 2, 4, true, false)
 
 // The two commonest reductions without the interpreter: sum(x) and sum(x * y)
 // over flat fp32 arrays (a dot product; y = x gives a sum of squares).  One

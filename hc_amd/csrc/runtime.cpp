@@ -1289,6 +1289,9 @@ int launchMap(OlQueue q, bool sum, const HcamdMapInstr *prog, size_t nInstr,
       u = 2;
     } else if (sum) {
       name = "hcamd_map_sum_flat_n4u1";
+    } else if (half && nInputs <= 2 && variantOf("map") != 3) {
+      name = "hcamd_map_flat_n2u4h"; // (variant 3 of "map": one chunk per lane whatever the operands)
+      u = 4;
     }
     // the reduction: 1024-lane workgroups, one per CU, each striding over the
     // vector and ending in one atomic addition

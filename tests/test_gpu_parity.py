@@ -1036,6 +1036,34 @@ def test_sum_and_dot_of_fp32_vectors_have_their_own_kernels(ctx, n):
             64 * 2.0 ** -24 * np.abs(x).sum()
 
 
+@pytest.mark.parametrize("n", [8, 2049, 8192 + 5, 3 * 8192 * 4 + 123])
+def test_map_of_one_or_two_fp16_operands_takes_four_chunks_per_lane(ctx, n):
+    """Dense fp16 maps with one or two operands: four chunks of 8 per lane in
+    flight (hcamd_map_flat_n2u4h), bit for bit what one chunk per lane gives
+    (variant 3 of "map") and what NumPy gives in fp32 rounded once; fewer than a
+    chunk, a ragged tail, several workgroups."""
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal(n).astype(np.float16)
+    y = rng.standard_normal(n).astype(np.float16)
+    dx, dy = dev(x), dev(y)
+    x32, y32 = x.astype(np.float32), y.astype(np.float32)
+    cases = {"one": ([I("in", 0), I("muli", 0, 2.5), I("addi", 0, 1.0)], [dx],
+                     (x32 * np.float32(2.5) + np.float32(1.0)).astype(np.float16)),
+             "two": ([I("in", 0), I("mul_in", 1), I("sub_in", 0)], [dx, dy],
+                     (x32 * y32 - x32).astype(np.float16))}
+    for name, (program, inputs, want) in cases.items():
+        got = {}
+        for variant in (0, 3):
+            rt.set_variant("map", variant)
+            out = poisoned((n,), np.float16)
+            rt.plan_map(program, inputs, out).launch(sync=True)
+            assert rt.last_kernel_name() == ("hcamd_map_flat_n2u4h" if variant == 0 else "hcamd_map_flat"), name
+            got[variant] = out.to_host()
+        rt.set_variant("map", 0)
+        assert_array_equal(got[0].view(np.uint16), got[3].view(np.uint16), err_msg=name)
+        assert_array_equal(got[0].view(np.uint16), want.view(np.uint16), err_msg=name)
+
+
 def test_map_full_benchmark_size_fma(ctx):
     a, b, c = cf.inputs_c2()
     d = rt.DeviceArray(a.shape, np.float16)
