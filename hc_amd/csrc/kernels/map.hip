@@ -885,6 +885,13 @@ __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcam
   const size_t n_chunks = n / 8;
   const bool out_f16 = (a.f16_mask >> 8) & 1;
   const size_t c = (size_t)blockIdx.x * 256 + threadIdx.x;
+  // All fp32, and the 64 chunks of this wave all there: a lane's eight elements
+  // are two runs of four, 256 elements apart, so that each of its two 16-byte
+  // accesses is one of 64 consecutive ones (1 KiB of whole cache lines per wave
+  // and instruction).  Eight consecutive elements per lane make every
+  // instruction touch 2 KiB of lines and use half of each.
+  const size_t wave_first = c & ~(size_t)63, lane = c & 63;
+  const bool split = (a.f16_mask & 0x1ffu) == 0 && wave_first + 64 <= n_chunks;
   Raw raw;
   if (c < n_chunks) {
 #pragma unroll
@@ -892,6 +899,10 @@ __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcam
       if (i < (int)n_in) {
         if ((a.f16_mask >> i) & 1) {
           raw.w[i][0] = ldg<true>(static_cast<const u32x4 *>(a.in[i]) + c);
+        } else if (split) {
+          const u32x4 *q = static_cast<const u32x4 *>(a.in[i]) + 2 * wave_first + lane;
+          raw.w[i][0] = ldg<true>(q);
+          raw.w[i][1] = ldg<true>(q + 64);
         } else {
           const u32x4 *q = static_cast<const u32x4 *>(a.in[i]) + 2 * c;
           raw.w[i][0] = ldg<true>(q);
@@ -901,8 +912,20 @@ __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcam
   }
   Stack r;
   run_program(a, raw, a.f16_mask, r);
-  if (c < n_chunks)
+  if (split) {
+    float *o = static_cast<float *>(a.out) + 8 * wave_first + 4 * lane;
+    if (r.bad & 0xffu) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (!((r.bad >> e) & 1u))
+          o[(e / 4) * 256 + e % 4] = r.st[0][e];
+    } else {
+      stg<true>(reinterpret_cast<f32x4 *>(o), f32x4{r.st[0][0], r.st[0][1], r.st[0][2], r.st[0][3]});
+      stg<true>(reinterpret_cast<f32x4 *>(o + 256), f32x4{r.st[0][4], r.st[0][5], r.st[0][6], r.st[0][7]});
+    }
+  } else if (c < n_chunks) {
     store_chunk(a.out, out_f16, c, r.st[0], r.bad);
+  }
   if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 255 && n_chunks * 8 < n) {
     gather(a, n_in, raw, [&](int, int e, size_t &off) {
       off = n_chunks * 8 + e;
@@ -1170,6 +1193,12 @@ __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, 
     acc[e] = identity;
   // 16-byte accesses: consecutive columns and a wave of whole chunks
   const bool vec = !c.interleaved && __builtin_amdgcn_ballot_w64(n_valid != (uint32_t)kN) == 0;
+  // All operands fp32: a lane's eight columns are two runs of four, 4 L columns
+  // apart, so that the L lanes of a row read 16 L consecutive bytes with each of
+  // their two accesses (whole cache lines; eight consecutive columns per lane
+  // make every access touch twice the lines and use half of each).
+  const bool split = vec && (a.f16_mask & ((1u << n_in) - 1u)) == 0;
+  const uint32_t run_a = blockIdx.x * L * kN + 4 * cl, run_b = run_a + 4 * L;
   Raw raw;
   Stack r;
   // the rows of the turn that starts at row0, requested (rows past the end: not)
@@ -1184,7 +1213,11 @@ __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, 
           if (row < row_end) {
             const char *base =
                 static_cast<const char *>(a.in[i]) + (size_t)row * a.ld[i] * (f16 ? 2 : 4);
-            if (vec) {
+            if (split) {
+              const u32x4 *q = reinterpret_cast<const u32x4 *>(base) + run_a / 4;
+              staged[i][u][0] = ldg<true>(q);
+              staged[i][u][1] = ldg<true>(q + L);
+            } else if (vec) {
               const u32x4 *q = reinterpret_cast<const u32x4 *>(base) + (f16 ? chunk : 2 * chunk);
               staged[i][u][0] = ldg<true>(q);
               if (!f16)
@@ -1269,8 +1302,8 @@ __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, 
         lo[e] = acc[e];
         hi[e] = acc[4 + e];
       }
-      *reinterpret_cast<f32x4 *>(dst + first) = lo;
-      *reinterpret_cast<f32x4 *>(dst + first + 4) = hi;
+      *reinterpret_cast<f32x4 *>(dst + (split ? run_a : first)) = lo;
+      *reinterpret_cast<f32x4 *>(dst + (split ? run_b : first + 4)) = hi;
     } else {
 #pragma unroll
       for (int e = 0; e < kN; ++e)
@@ -1290,7 +1323,11 @@ __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, 
       r.st[0][e] = acc[e];
   }
   const bool out_f16 = (a.f16_mask >> 8) & 1;
-  if (c.out_vec && !c.interleaved && n_valid == (uint32_t)kN) {
+  if (split) {
+#pragma unroll
+    for (int e = 0; e < kN; ++e)
+      store_elem(a.out, out_f16, (size_t)(e < 4 ? run_a + e : run_b + e - 4), r.st[0][e]);
+  } else if (c.out_vec && !c.interleaved && n_valid == (uint32_t)kN) {
     store_chunk(a.out, out_f16, chunk, r.st[0]);
   } else {
 #pragma unroll
@@ -1376,6 +1413,7 @@ struct RowArgs {
   uint32_t interleaved; // columns are dealt to lanes one by one (then vec_mask is 0)
   uint32_t n_col, n_stages, passes;
   uint32_t hold, hold_last; // chain kernels: the operand that stays in LDS for the row, and the last instruction that reads it
+  uint32_t all_f32;         // chain kernels: every operand in use and the output are fp32
   Stage stage[kMaxStages];
   Instr prog[kRowProg];
 };
@@ -1717,6 +1755,21 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
     const uint32_t c = (uint32_t)p * LPR + ln;
     return c < per_row ? c : 0u;
   };
+  // Everything fp32 (the operands in use and the output; the host says): where
+  // all 64 chunks of a wave exist, a lane's eight elements are two runs of four,
+  // 256 elements apart, so that each of its two 16-byte accesses is one of 64
+  // consecutive ones (whole cache lines; eight consecutive elements per lane
+  // make every access touch 2 KiB of lines and use half of each).  `split(p)`
+  // is the same for every operand, the output and every stage, which is all
+  // that element-wise work and reductions along the row need.
+  const bool all_f32 = a.all_f32 != 0;
+  auto split = [&](int p) {
+    return all_f32 && (uint32_t)p * LPR + (lane & ~(uint32_t)(kWave - 1)) + kWave <= per_row;
+  };
+  // the two 16-byte words of chunk c, in units of 16 bytes from the row's start
+  auto word_at = [&](uint32_t c, bool sp, int j) {
+    return sp ? 2 * (c & ~(uint32_t)(kWave - 1)) + (c & (kWave - 1)) + (uint32_t)j * kWave : 2 * c + (uint32_t)j;
+  };
   auto row_of = [&](size_t turn) { // idle waves compute on row 0 and store nothing
     const size_t r = turn * R + t / LPR;
     return r < a.rows ? r : (size_t)0;
@@ -1740,9 +1793,10 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
         w[p][0] = ldg<false>(reinterpret_cast<const u32x4 *>(b) + chunk_at(p0 + p, ln));
         w[p][1] = u32x4{0u, 0u, 0u, 0u};
       } else {
-        const u32x4 *q = reinterpret_cast<const u32x4 *>(b) + 2 * chunk_at(p0 + p, ln);
-        w[p][0] = ldg<false>(q);
-        w[p][1] = ldg<false>(q + 1);
+        const uint32_t c = chunk_at(p0 + p, ln);
+        const bool sp = split(p0 + p);
+        w[p][0] = ldg<false>(reinterpret_cast<const u32x4 *>(b) + word_at(c, sp, 0));
+        w[p][1] = ldg<false>(reinterpret_cast<const u32x4 *>(b) + word_at(c, sp, 1));
       }
     }
   };
@@ -1771,12 +1825,17 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
     asm volatile("" : "+v"(ln));
 #pragma unroll
     for (int p = 0; p < P; ++p) {
-      const int off = (int)(chunk_at(p, ln) * (hold_f16 ? 16u : 32u));
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (row_lds_ptr)&row_words[p][0][wave_first], 16, off, 0,
-                                               0, 0);
-      if (!hold_f16)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (row_lds_ptr)&row_words[p][1][wave_first], 16, off,
-                                                 16, 0, 0); // the scalar offset: memory side only
+      const uint32_t c = chunk_at(p, ln);
+      if (hold_f16) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (row_lds_ptr)&row_words[p][0][wave_first], 16,
+                                                 (int)(c * 16u), 0, 0, 0);
+      } else {
+        const bool sp = split(p);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (row_lds_ptr)&row_words[p][0][wave_first], 16,
+                                                 (int)(word_at(c, sp, 0) * 16u), 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (row_lds_ptr)&row_words[p][1][wave_first], 16,
+                                                 (int)(word_at(c, sp, 1) * 16u), 0, 0, 0);
+      }
     }
   };
   fetch_row(row_of(blockIdx.x));
@@ -1921,8 +1980,26 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
       asm volatile("" : "+v"(o), "+v"(ln));
 #pragma unroll
       for (int p = 0; p < P; ++p)
-        if ((live >> p) & 1u)
-          store_chunk(o, out_f16, (size_t)p * LPR + ln, v + 8 * p, (bad >> (8 * p)) & 0xffu);
+        if ((live >> p) & 1u) {
+          const uint32_t c = (uint32_t)p * LPR + ln, none = (bad >> (8 * p)) & 0xffu;
+          if (split(p)) { // fp32 output, two runs of four
+            float *dst = reinterpret_cast<float *>(o);
+            const uint32_t e0 = 4 * word_at(c, true, 0), e1 = 4 * word_at(c, true, 1);
+            if (none) {
+#pragma unroll
+              for (int e = 0; e < 8; ++e)
+                if (!((none >> e) & 1u))
+                  dst[(e < 4 ? e0 : e1) + e % 4] = v[8 * p + e];
+            } else {
+              stg<true>(reinterpret_cast<f32x4 *>(dst + e0),
+                        f32x4{v[8 * p], v[8 * p + 1], v[8 * p + 2], v[8 * p + 3]});
+              stg<true>(reinterpret_cast<f32x4 *>(dst + e1),
+                        f32x4{v[8 * p + 4], v[8 * p + 5], v[8 * p + 6], v[8 * p + 7]});
+            }
+          } else {
+            store_chunk(o, out_f16, c, v + 8 * p, none);
+          }
+        }
     }
   }
   } // turns

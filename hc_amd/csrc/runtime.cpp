@@ -1869,7 +1869,7 @@ struct RowArgs {
   size_t rows, cols;
   uint32_t f16Mask, vecMask, interleaved;
   uint32_t nCol, nStages, passes;
-  uint32_t hold, holdLast;
+  uint32_t hold, holdLast, allF32;
   RowStageDev stage[HCAMD_ROW_MAX_STAGES];
   HcamdMapInstr prog[HCAMD_ROW_MAX_INSTRS];
 };
@@ -2155,6 +2155,8 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       std::memset(a.prog, 0, sizeof a.prog);
       std::memcpy(a.prog, chained, nChained * sizeof(HcamdMapInstr));
       a.hold = static_cast<uint32_t>(hold);
+      // storesTile: the output is a tile; a per-row result has no layout to agree with
+      a.allF32 = (a.f16Mask & used & 0xffu) == 0 && (!storesTile || outType == HCAMD_F32) ? 1u : 0u;
       for (size_t i = 0; i < nChained; ++i) {
         const unsigned op = chained[i].op;
         if ((op == HCAMD_MAP_IN || (op >= HCAMD_MAP_ADD_IN && op <= HCAMD_MAP_RDIV_IN) ||
