@@ -592,6 +592,7 @@ __device__ __forceinline__ void map_flat(const MapArgs &a, const uint32_t n_in) 
   const size_t passes = (n_chunks + stride - 1) / stride;
   const bool out_f16 = (a.f16_mask >> 8) & 1;
   size_t c0 = (size_t)blockIdx.x * (kThreads * U) + threadIdx.x;
+  const bool all_f32 = (a.f16_mask & ((1u << n_in) - 1u)) == 0;
   float acc = 0.0f;
   Raw raw;
   Stack r;
@@ -605,11 +606,25 @@ __device__ __forceinline__ void map_flat(const MapArgs &a, const uint32_t n_in) 
           const size_t chunk = c0 + (size_t)u * kThreads;
           if (chunk < n_chunks) {
             const bool f16 = HALF || ((a.f16_mask >> i) & 1);
-            const u32x4 *q = static_cast<const u32x4 *>(a.in[i]) + (f16 ? chunk : 2 * chunk);
-            staged[i][u][0] = ldg<true>(q);
-            if constexpr (!HALF)
-              if (!f16)
-                staged[i][u][1] = ldg<true>(q + 1);
+            bool done = false;
+            if constexpr (SUM && !HALF) {
+              // a sum does not care which elements a lane adds: two runs of four,
+              // 256 elements apart, so that the wave's accesses are whole cache lines
+              if (all_f32 && (chunk | 63) < n_chunks) {
+                const u32x4 *q =
+                    static_cast<const u32x4 *>(a.in[i]) + 2 * (chunk & ~(size_t)63) + (chunk & 63);
+                staged[i][u][0] = ldg<true>(q);
+                staged[i][u][1] = ldg<true>(q + 64);
+                done = true;
+              }
+            }
+            if (!done) {
+              const u32x4 *q = static_cast<const u32x4 *>(a.in[i]) + (f16 ? chunk : 2 * chunk);
+              staged[i][u][0] = ldg<true>(q);
+              if constexpr (!HALF)
+                if (!f16)
+                  staged[i][u][1] = ldg<true>(q + 1);
+            }
           }
         }
       }
