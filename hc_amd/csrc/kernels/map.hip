@@ -900,19 +900,26 @@ __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcam
   const size_t n_chunks = n / 8;
   const bool out_f16 = (a.f16_mask >> 8) & 1;
   const size_t c = (size_t)blockIdx.x * 256 + threadIdx.x;
-  // All fp32, and the 64 chunks of this wave all there: a lane's eight elements
-  // are two runs of four, 256 elements apart, so that each of its two 16-byte
-  // accesses is one of 64 consecutive ones (1 KiB of whole cache lines per wave
-  // and instruction).  Eight consecutive elements per lane make every
+  // fp32 among the operands or as the output, and the 64 chunks of this wave
+  // all there: a lane's eight elements are two runs of four, 256 elements
+  // apart, so that each of its two 16-byte accesses to fp32 data is one of 64
+  // consecutive ones (1 KiB of whole cache lines per wave and instruction;
+  // fp16 data of the same elements: two 8-byte accesses, 512 bytes of whole
+  // lines each).  Eight consecutive fp32 elements per lane make every
   // instruction touch 2 KiB of lines and use half of each.
   const size_t wave_first = c & ~(size_t)63, lane = c & 63;
-  const bool split = (a.f16_mask & 0x1ffu) == 0 && wave_first + 64 <= n_chunks;
+  const uint32_t present = ((1u << n_in) - 1u) | 0x100u;
+  const bool split = (~a.f16_mask & present) != 0 && wave_first + 64 <= n_chunks;
   Raw raw;
   if (c < n_chunks) {
 #pragma unroll
     for (int i = 0; i < kMaxIn; ++i)
       if (i < (int)n_in) {
-        if ((a.f16_mask >> i) & 1) {
+        if (split && ((a.f16_mask >> i) & 1)) {
+          const u32x2 *q = static_cast<const u32x2 *>(a.in[i]) + 2 * wave_first + lane;
+          const u32x2 lo = ldg<true>(q), hi = ldg<true>(q + 64);
+          raw.w[i][0] = u32x4{lo.x, lo.y, hi.x, hi.y};
+        } else if ((a.f16_mask >> i) & 1) {
           raw.w[i][0] = ldg<true>(static_cast<const u32x4 *>(a.in[i]) + c);
         } else if (split) {
           const u32x4 *q = static_cast<const u32x4 *>(a.in[i]) + 2 * wave_first + lane;
@@ -927,7 +934,24 @@ __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcam
   }
   Stack r;
   run_program(a, raw, a.f16_mask, r);
-  if (split) {
+  if (split && out_f16) {
+    _Float16 *o = static_cast<_Float16 *>(a.out) + 8 * wave_first + 4 * lane;
+    if (r.bad & 0xffu) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (!((r.bad >> e) & 1u))
+          o[(e / 4) * 256 + e % 4] = (_Float16)r.st[0][e];
+    } else {
+      f16x4 lo, hi;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        lo[e] = (_Float16)r.st[0][e];
+        hi[e] = (_Float16)r.st[0][4 + e];
+      }
+      stg<true>(reinterpret_cast<f16x4 *>(o), lo);
+      stg<true>(reinterpret_cast<f16x4 *>(o + 256), hi);
+    }
+  } else if (split) {
     float *o = static_cast<float *>(a.out) + 8 * wave_first + 4 * lane;
     if (r.bad & 0xffu) {
 #pragma unroll

@@ -1064,6 +1064,41 @@ def test_map_of_one_or_two_fp16_operands_takes_four_chunks_per_lane(ctx, n):
         assert_array_equal(got[0].view(np.uint16), want.view(np.uint16), err_msg=name)
 
 
+@pytest.mark.parametrize("n", [8, 511, 512 * 3 + 8 * 7 + 3, 1 << 20])
+@pytest.mark.parametrize("types", [(np.float32, np.float32, np.float32), (np.float16, np.float32, np.float16),
+                                   (np.float16, np.float16, np.float32), (np.float32, np.float16, np.float32)])
+def test_map_of_flat_arrays_of_mixed_types(ctx, n, types):
+    """a * b + a over dense vectors of fp16 and fp32 in every combination (the
+    kernel deals elements to lanes differently as soon as one of the three is
+    fp32): bit for bit the fp32 arithmetic of NumPy, rounded once to the output's
+    type; whole waves, a partial last wave, a ragged tail; and with every third
+    divisor zero in a / b under numpy.ma's rule, the poison stays where the
+    quotient is not finite."""
+    ta, tb, to = types
+    rng = np.random.default_rng(n)
+    a = rng.standard_normal(n).astype(ta)
+    b = rng.standard_normal(n).astype(tb)
+    a32, b32 = a.astype(np.float32), b.astype(np.float32)
+    out = poisoned((n,), to)
+    rt.plan_map([I("in", 0), I("mul_in", 1), I("add_in", 0)], [dev(a), dev(b)], out).launch(sync=True)
+    assert rt.last_kernel_name() == ("hcamd_map_flat_n2u4h" if ta == tb == np.float16 else "hcamd_map_flat")
+    want = (a32 * b32 + a32).astype(to)
+    bits = np.uint32 if to == np.float32 else np.uint16
+    assert_array_equal(out.to_host().view(bits), want.view(bits))
+    b[::3] = 0
+    b32 = b.astype(np.float32)
+    out = poisoned((n,), to)
+    rt.plan_map([I("in", 0), I("mdiv_in", 1 | (0x100 if to == np.float16 else 0))], [dev(a), dev(b)],
+                out).launch(sync=True)
+    got = out.to_host()
+    with np.errstate(all="ignore"):
+        q = (a32 / b32).astype(to)
+    dead = ~np.isfinite(q.astype(np.float32))
+    assert dead[::3].all()
+    assert (got.view(bits)[dead] == poison_value(to).view(bits)).all()
+    assert_array_equal(got.view(bits)[~dead], (q + np.float32(0) * a32.astype(to)).astype(to).view(bits)[~dead])
+
+
 def test_map_full_benchmark_size_fma(ctx):
     a, b, c = cf.inputs_c2()
     d = rt.DeviceArray(a.shape, np.float16)
