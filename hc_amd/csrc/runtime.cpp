@@ -1289,7 +1289,7 @@ int launchMap(OlQueue q, bool sum, const HcamdMapInstr *prog, size_t nInstr,
       u = 2;
     } else if (sum) {
       name = "hcamd_map_sum_flat_n4u1";
-    } else if (half && nInputs <= 2 && variantOf("map") != 3) {
+    } else if (half && outType == HCAMD_F16 && nInputs <= 2 && variantOf("map") != 3) {
       name = "hcamd_map_flat_n2u4h"; // (variant 3 of "map": one chunk per lane whatever the operands)
       u = 4;
     }
