@@ -395,6 +395,12 @@ def make_workloads(rt, wl):
         def plan(self, rt, s):
             return rt.plan_map([I("in", 0), I("mul_in", 1), I("add_in", 2)], s[:3], s[3])
 
+    class X7(C1):
+        """a+b on the C1 vectors through the fused map kernel (2 instructions)."""
+
+        def plan(self, rt, s):
+            return rt.plan_map([I("in", 0), I("add_in", 1)], s[:2], s[2])
+
     class X2(Workload):
         """fp32 dot product of the C1 vectors through the map-sum kernel."""
 
@@ -569,6 +575,8 @@ def make_workloads(rt, wl):
                  W.work_c3(), "GB/s"),
         "x6": X6("x6", "column reduction: root mean square down the columns, fp32 4096x8192", "f32",
                  "hbm", W.work_c3() // 2 + 4 * 8192, "GB/s"),
+        "x7": X7("x7", "map kernel: vadd fp32 N=16777259 as a 2-instruction program", "f32", "hbm",
+                 W.work_c1(), "GB/s"),
     }
     # the mix and size of each memory-bound configuration, then the plain streams
     for key, n_reads, write, mib in STREAMS:
@@ -578,7 +586,7 @@ def make_workloads(rt, wl):
     elif wl == "streams":
         keys = [k for k, *_ in STREAMS]
     elif wl == "extra":
-        keys = ["x1", "x2", "x3", "x4", "x5", "x6"]
+        keys = ["x1", "x2", "x3", "x4", "x5", "x6", "x7"]
     else:
         keys = [wl]
     return [table[k] for k in keys]
@@ -653,7 +661,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="all", choices=["all", "streams", "c0", "c1", "c2", "c3", "c4", "c5", "v5", "extra", "x1", "x2", "x3",
-                             "x4", "x5", "x6"] + [k for k, *_ in STREAMS])
+                             "x4", "x5", "x6", "x7"] + [k for k, *_ in STREAMS])
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy CPU baseline")
     ap.add_argument("--variant", action="append", default=[], metavar="FAMILY=N",
                     help="measure kernel variant N of a family (hcamdSetVariant), e.g. gemm=14; "

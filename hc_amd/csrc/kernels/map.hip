@@ -911,20 +911,28 @@ __attribute__((amdgpu_waves_per_eu(HCAMD_MAP_WAVES, HCAMD_MAP_WAVES))) void hcam
   const uint32_t present = ((1u << n_in) - 1u) | 0x100u;
   const bool split = (~a.f16_mask & present) != 0 && wave_first + 64 <= n_chunks;
   Raw raw;
-  if (c < n_chunks) {
+  // (one branch on the layout around all the loads, not one per operand: the
+  // loads of an arm then go out back to back)
+  if (split) {
 #pragma unroll
     for (int i = 0; i < kMaxIn; ++i)
       if (i < (int)n_in) {
-        if (split && ((a.f16_mask >> i) & 1)) {
+        if ((a.f16_mask >> i) & 1) {
           const u32x2 *q = static_cast<const u32x2 *>(a.in[i]) + 2 * wave_first + lane;
           const u32x2 lo = ldg<true>(q), hi = ldg<true>(q + 64);
           raw.w[i][0] = u32x4{lo.x, lo.y, hi.x, hi.y};
-        } else if ((a.f16_mask >> i) & 1) {
-          raw.w[i][0] = ldg<true>(static_cast<const u32x4 *>(a.in[i]) + c);
-        } else if (split) {
+        } else {
           const u32x4 *q = static_cast<const u32x4 *>(a.in[i]) + 2 * wave_first + lane;
           raw.w[i][0] = ldg<true>(q);
           raw.w[i][1] = ldg<true>(q + 64);
+        }
+      }
+  } else if (c < n_chunks) {
+#pragma unroll
+    for (int i = 0; i < kMaxIn; ++i)
+      if (i < (int)n_in) {
+        if ((a.f16_mask >> i) & 1) {
+          raw.w[i][0] = ldg<true>(static_cast<const u32x4 *>(a.in[i]) + c);
         } else {
           const u32x4 *q = static_cast<const u32x4 *>(a.in[i]) + 2 * c;
           raw.w[i][0] = ldg<true>(q);

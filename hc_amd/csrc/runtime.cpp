@@ -1056,12 +1056,16 @@ int hcamdLaunchFmaF16(OlQueue q, const void *a, size_t lda, const void *b,
   const int variant = variantOf("fma");
   if (dense && aligned16(a) && aligned16(b) && aligned16(c) && aligned16(d) &&
       variant != 7) {
+    // 0: the paced kernel (four waves per SIMD, a pause before the store);
+    // 8..12: the same with other paces, for measurement
     static const char *const names[] = {
-        "hcamd_fma_f16_v4_nt", "hcamd_fma_f16_v1",    "hcamd_fma_f16_v2",
-        "hcamd_fma_f16_v4",    "hcamd_fma_f16_v1_nt", "hcamd_fma_f16_v2_nt",
-        "hcamd_fma_f16_v4_nt"};
-    static const int vpt[] = {4, 1, 2, 4, 1, 2, 4};
-    const int v = (variant >= 0 && variant <= 6) ? variant : 0;
+        "hcamd_fma_f16_v1_nt_w4_d6", "hcamd_fma_f16_v1",    "hcamd_fma_f16_v2",
+        "hcamd_fma_f16_v4",          "hcamd_fma_f16_v1_nt", "hcamd_fma_f16_v2_nt",
+        "hcamd_fma_f16_v4_nt",       nullptr,               "hcamd_fma_f16_v1_nt_w4_d0",
+        "hcamd_fma_f16_v1_nt_w4_d3", "hcamd_fma_f16_v1_nt_w4_d12", "hcamd_fma_f16_v1_nt_w5_d12",
+        "hcamd_fma_f16_v1_nt_w6_d8"};
+    static const int vpt[] = {1, 1, 2, 4, 1, 2, 4, 0, 1, 1, 1, 1, 1};
+    const int v = (variant >= 0 && variant <= 12) ? variant : 0;
     size_t n = rows * cols;
     const size_t words = ceilDiv(n, 8);
     void *args[] = {&a, &b, &c, &d, &n};

@@ -509,7 +509,7 @@ def test_fma_bit_exact_all_variants(ctx, shape):
     want = cf.np_fma_f16(a, b, c)
     assert_array_equal(want.view(np.uint16), co.fma_f16(a, b, c).view(np.uint16))
     da, db, dc = dev(a), dev(b), dev(c)
-    for v in range(0, 8):
+    for v in range(0, 13):                              # 0: the paced kernel, 8..12: other paces
         rt.set_variant("fma", v)
         dd = poisoned((shape[0] * shape[1] + 16,), np.float16)
         out_view = _View(dd, shape)
