@@ -124,10 +124,9 @@ HCAMD_COPY_TILED(hcamd_copy2d_tiled_b16, u32x4)
 // lanes owns 1024 consecutive words, two per lane, non-temporal both ways: the
 // structure that measured fastest for every mix.  The launcher passes whole
 // workgroups only (bytes a multiple of 16 KiB).
-template <int R, int W>
+template <int R, int W, int kT = 512, int kVpt = 2, int DELAY = -1>
 __device__ __forceinline__ void stream_mix(const u32x4 *a, const u32x4 *b, const u32x4 *c,
                                            void *out) {
-  constexpr int kT = 512, kVpt = 2;
   const u32x4 *in[3] = {a, b, c};
   const size_t first = (size_t)blockIdx.x * (kT * kVpt) + threadIdx.x;
   u32x4 v[kVpt][R > 0 ? R : 1];
@@ -136,14 +135,22 @@ __device__ __forceinline__ void stream_mix(const u32x4 *a, const u32x4 *b, const
 #pragma unroll
     for (int j = 0; j < kVpt; ++j)
       v[j][r] = ldg<true>(in[r] + first + (size_t)j * kT);
+  if constexpr (DELAY >= 0 && R > 0) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if constexpr (DELAY > 0)
+      __builtin_amdgcn_s_sleep(DELAY);
+  }
   uint32_t total = 0;
 #pragma unroll
   for (int j = 0; j < kVpt; ++j) {
     const uint32_t w = (uint32_t)(first + (size_t)j * kT);
     u32x4 s = R ? v[j][0] : u32x4{w, w, w, w};
-#pragma unroll
-    for (int r = 1; r < R; ++r)
-      s += v[j][r];
+    // (written out: as a loop over r the compiler drops the non-temporal
+    // marking of the store when kVpt is 1)
+    if constexpr (R >= 2)
+      s += v[j][1];
+    if constexpr (R >= 3)
+      s += v[j][2];
     if constexpr (W == 1) {
       stg<true>(static_cast<u32x4 *>(out) + first + (size_t)j * kT, s);
     } else if constexpr (W == 2) {
@@ -176,6 +183,26 @@ HCAMD_STREAM(hcamd_stream_r1w1, 1, 1)
 HCAMD_STREAM(hcamd_stream_r2w1, 2, 1)
 HCAMD_STREAM(hcamd_stream_r3w1, 3, 1)
 HCAMD_STREAM(hcamd_stream_r1w1h, 1, 2)
+
+// The same mixes paced as the fp16 fma kernel is: 256 lanes, one word each, REG
+// the highest register touched (127: four waves per SIMD), DELAY * 64 clocks
+// between the arrival of a wave's words and its store (-1: no wait at all).
+// Only the mixes that both read and write have such forms.
+#define HCAMD_STREAM_PACED(NAME, R, W, REG, DELAY)                             \
+  extern "C" __global__ __launch_bounds__(256) void NAME(                      \
+      const u32x4 *a, const u32x4 *b, const u32x4 *c, void *out) {             \
+    asm volatile("v_mov_b32 v" #REG ", 0" ::: "v" #REG);                       \
+    stream_mix<R, W, 256, 1, DELAY>(a, b, c, out);                             \
+  }
+#define HCAMD_STREAM_PACED_ALL(SUFFIX, REG, DELAY)                             \
+  HCAMD_STREAM_PACED(hcamd_stream_r1w1##SUFFIX, 1, 1, REG, DELAY)              \
+  HCAMD_STREAM_PACED(hcamd_stream_r2w1##SUFFIX, 2, 1, REG, DELAY)              \
+  HCAMD_STREAM_PACED(hcamd_stream_r3w1##SUFFIX, 3, 1, REG, DELAY)              \
+  HCAMD_STREAM_PACED(hcamd_stream_r1w1h##SUFFIX, 1, 2, REG, DELAY)
+HCAMD_STREAM_PACED_ALL(_w4_d6, 127, 6)
+HCAMD_STREAM_PACED_ALL(_w4_d0, 127, 0)
+HCAMD_STREAM_PACED_ALL(_w4_d12, 127, 12)
+HCAMD_STREAM_PACED_ALL(_w8, 63, -1)
 
 // ---------------------------------------------------------------------------
 // Ids as data: out[index(g, l)] = value(g, l), both affine in the group id g and

@@ -267,7 +267,7 @@ std::unordered_map<std::string, int> &variants() {
   static std::unordered_map<std::string, int> v{
       {"add", 0},     {"fma", 0},  {"softmax", 0},
       {"quantize", 0}, {"gemm", 0}, {"copy", 0}, {"map", 0},
-      {"gather", 0}, {"gather_fuse", 0}, {"rows", 0}};
+      {"gather", 0}, {"gather_fuse", 0}, {"rows", 0}, {"stream", 0}};
   return v;
 }
 std::mutex g_variantLock; // guards variants()
@@ -964,6 +964,21 @@ int hcamdLaunchStream(OlQueue q, int nReads, int writeMode, const void *const *i
     return 1;
   }
   void *args[] = {&in[0], &in[1], &in[2], &out};
+  // 256-lane workgroups of one word a lane, paced as the fp16 fma kernel is
+  // (four waves per SIMD and 6, 0 or 12 pauses before the store: "stream"
+  // variants 2, 3, 4) or not paced at all (5).  By shape (variant 0) only three
+  // reads against one write take the paced form: measured 85.8 -> 80.0 us at
+  // 128 MiB a stream; every other mix is slower that way.  Variant 1: the
+  // 512-lane form for every mix.
+  static const char *const paced[] = {"_w4_d6", "_w4_d0", "_w4_d12", "_w8"};
+  int variant = variantOf("stream");
+  if (variant == 0 && nReads == 3)
+    variant = 2;
+  if (variant >= 2 && variant <= 5 && nReads > 0 && writeMode != HCAMD_STREAM_NONE) {
+    char full[64];
+    snprintf(full, sizeof full, "%s%s", name, paced[variant - 2]);
+    return launch1d(queue, "copy", full, bytes / 4096, 256, args);
+  }
   return launch1d(queue, "copy", name, bytes / 16384, 512, args);
 }
 

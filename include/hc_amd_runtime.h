@@ -243,7 +243,11 @@ int hcamdLaunchIdScatter(OlQueue q, void *out, int outType, size_t outRank,
  * HCAMD_STREAM_NONE one 32-bit total per 16 KiB of input (bytes / 4096 out: a
  * read-only stream with a checkable result).  nReads == 0 writes the word
  * index (a fill; HCAMD_STREAM_FULL only).  bytes must be a multiple of 16 KiB,
- * pointers 16-byte aligned. */
+ * pointers 16-byte aligned.  Each mix runs in the form that measured fastest
+ * for it: three reads against one write from workgroups held to four waves per
+ * SIMD that pause between the arrival of their words and their store, the
+ * others from full workgroups that do not ("stream" variants 1..5 force one
+ * form on every mix that reads and writes). */
 enum HcamdStreamWrite { HCAMD_STREAM_NONE = 0, HCAMD_STREAM_FULL = 1, HCAMD_STREAM_HALF = 2 };
 int hcamdLaunchStream(OlQueue q, int nReads, int writeMode, const void *const *inputs,
                       void *out, size_t bytes) HCAMD_NOEXCEPT;
@@ -654,8 +658,9 @@ int hcamdLaunchGemmF16(OlQueue q, const void *a, size_t lda, const void *bt,
 
 /* Chooses between kernel variants of one family by number (0 = default
  * choice by shape).  For tuning and measurement; family names are "add",
- * "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "gather" (block
- * shape), "gather_fuse" (groups per workgroup; read by hcamdGatherGemmCreate).
+ * "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "stream", "gather"
+ * (block shape), "gather_fuse" (groups per workgroup; read by
+ * hcamdGatherGemmCreate).
  * Process-wide, guarded by a lock.  Returns 1 for an unknown family. */
 int hcamdSetVariant(const char *family, int variant) HCAMD_NOEXCEPT;
 /* The same choice for the calling thread only: it takes precedence over

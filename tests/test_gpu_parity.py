@@ -34,10 +34,10 @@ def ctx():
 
 @pytest.fixture(autouse=True)
 def default_variants():
-    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "gather", "gather_fuse"):
+    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "stream", "gather", "gather_fuse"):
         rt.set_variant(fam, 0)
     yield
-    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "gather", "gather_fuse"):
+    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "stream", "gather", "gather_fuse"):
         rt.set_variant(fam, 0)
 
 
@@ -417,7 +417,16 @@ def test_fmap_every_operation_against_numpy_ma(ctx, dtype):
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("n_reads,write", [(1, "full"), (2, "full"), (3, "full"), (0, "full"),
                                             (1, "half"), (1, "none")])
-def test_stream_mixes_compute_what_they_say(ctx, n_reads, write):
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5])
+def test_stream_mixes_compute_what_they_say(ctx, n_reads, write, variant):
+    rt.set_variant("stream", variant)
+    try:
+        _stream_mix(n_reads, write, variant)
+    finally:
+        rt.set_variant("stream", 0)
+
+
+def _stream_mix(n_reads, write, variant):
     nbytes = 5 * 16384
     rng = np.random.default_rng(60 + n_reads)
     ins = [rng.integers(0, 2 ** 32, nbytes // 4, dtype=np.uint32) for _ in range(n_reads)]
@@ -426,6 +435,11 @@ def test_stream_mixes_compute_what_they_say(ctx, n_reads, write):
     out = poisoned((words + pad,), np.uint32)
     rt.plan_stream([dev(x) for x in ins], _View(out, (words,), 0), write).launch(sync=True)
     say("stream", n_reads, write, rt.last_kernel_name())
+    plain = "hcamd_stream_r%dw%d%s" % (n_reads, write != "none", "h" if write == "half" else "")
+    both = n_reads > 0 and write != "none"
+    suffix = {0: "_w4_d6" if n_reads == 3 else "", 1: "", 2: "_w4_d6", 3: "_w4_d0", 4: "_w4_d12",
+              5: "_w8"}[variant] if both else ""
+    assert rt.last_kernel_name() == plain + suffix
     total = np.zeros(nbytes // 4, np.uint32)
     for x in ins:
         total += x
