@@ -2022,9 +2022,11 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
       parity ^= 1;
       cells[st.dst & (kMaxRed - 1)] = total;
     } else {
-      char *o = orow;
-      uint32_t ln = lane;
-      asm volatile("" : "+v"(o), "+v"(ln));
+      // (an offset the compiler cannot see through, not the pointer itself: a
+      // laundered pointer is no longer known to be global and would store flat)
+      uint32_t ln = lane, zero = 0;
+      asm volatile("" : "+v"(zero), "+v"(ln));
+      char *o = orow + zero;
 #pragma unroll
       for (int p = 0; p < P; ++p)
         if ((live >> p) & 1u) {
