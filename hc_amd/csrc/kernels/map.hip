@@ -890,6 +890,89 @@ extern "C" __global__ __launch_bounds__(1024) void hcamd_dot_f32(
   reduce_f32<true>(x, y, cell, n);
 }
 
+// The two commonest reductions down columns without the interpreter: the sums
+// of x and of x * x over the rows of a band of a dense fp32 window, into
+// partial[band][column] (the first of the two launches of a column reduction;
+// the second one, which folds the bands and runs the post program, is the
+// general kernel's).  A lane owns four consecutive columns, a wave 256 (1 KiB of
+// every row it reads), the W waves of a workgroup take the rows of the band
+// in turns, U rows in flight each with an accumulator of its own; the
+// accumulators fold in a fixed order, then the waves through LDS in theirs, so
+// the result is the same from run to run.  The product is rounded before it is
+// added, as the interpreter's multiply-then-fold does.
+template <bool SQ, int W, int U>
+__device__ __forceinline__ void cols_sum_f32(const float *__restrict__ x, size_t ld,
+                                             float *__restrict__ partial, uint32_t cols,
+                                             uint32_t cols_pad, uint32_t rows, uint32_t band) {
+  __shared__ f32x4 fold[W][kWave];
+  const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const uint32_t col = (blockIdx.x * kWave + lane) * 4;
+  const uint32_t first = blockIdx.y * band;
+  const uint32_t end = (uint32_t)min((uint64_t)first + band, (uint64_t)rows);
+  const bool there = col < cols; // cols is a multiple of 4
+  f32x4 acc[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    acc[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  auto add = [](f32x4 &to, const f32x4 v) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      to[e] += SQ ? __fmul_rn(v[e], v[e]) : v[e];
+  };
+  if (there) {
+    const float *p = x + (size_t)(first + wave) * ld + col;
+    uint32_t r = first + wave;
+    for (; r + W * (U - 1) < end; r += W * U, p += (size_t)(W * U) * ld) {
+      f32x4 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        v[u] = ldg<true>(reinterpret_cast<const f32x4 *>(p + (size_t)(W * u) * ld));
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        add(acc[u], v[u]);
+    }
+    // the rows left over, in the accumulators they would have had
+#pragma unroll
+    for (int u = 0; u < U - 1; ++u)
+      if (r + W * u < end)
+        add(acc[u], ldg<true>(reinterpret_cast<const f32x4 *>(p + (size_t)(W * u) * ld)));
+  }
+#pragma unroll
+  for (int step = 1; step < U; step *= 2)
+#pragma unroll
+    for (int u = 0; u + step < U; u += 2 * step)
+      acc[u] += acc[u + step];
+  fold[wave][lane] = acc[0];
+  __syncthreads();
+  if (wave == 0 && there) {
+    f32x4 part[W];
+#pragma unroll
+    for (int w = 0; w < W; ++w)
+      part[w] = fold[w][lane];
+#pragma unroll
+    for (int step = 1; step < W; step *= 2)
+#pragma unroll
+      for (int w = 0; w + step < W; w += 2 * step)
+        part[w] += part[w + step];
+    *reinterpret_cast<f32x4 *>(partial + (size_t)blockIdx.y * cols_pad + col) = part[0];
+  }
+}
+#define HCAMD_COLS_SUM(NAME, SQ, W, U)                                                    \
+  extern "C" __global__ __launch_bounds__(W * 64) void NAME(                              \
+      const float *x, size_t ld, float *partial, uint32_t cols, uint32_t cols_pad,       \
+      uint32_t rows, uint32_t band) {                                                     \
+    cols_sum_f32<SQ, W, U>(x, ld, partial, cols, cols_pad, rows, band);                   \
+  }
+// 16 waves with four rows in flight each measured fastest (root mean square down
+// the columns of 4096 x 8192, both launches: 32.7 us; 4 waves x 8 rows 39.6, 8 x 8
+// 34.5, 16 x 2 32.7; the general kernel 36.8): with a band of 64 rows a wave is
+// done after one round trip, and many short waves keep the memory busier than
+// few long ones.
+HCAMD_COLS_SUM(hcamd_cols_sum_f32, false, 16, 4)
+HCAMD_COLS_SUM(hcamd_cols_sumsq_f32, true, 16, 4)
+HCAMD_COLS_SUM(hcamd_cols_sum_f32_w4u8, false, 4, 8)
+HCAMD_COLS_SUM(hcamd_cols_sumsq_f32_w4u8, true, 4, 8)
+
 // The map itself: one chunk per lane, one pass, no loop around the interpreter
 // (several chunks per pass, or a persistent grid, measured slower here: the
 // stores of one workgroup already overlap the loads of the next).

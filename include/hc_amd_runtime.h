@@ -458,7 +458,10 @@ int hcamdLaunchMapSum(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
  * `workspace` (device memory, 16-byte aligned, at least
  * hcamdMapReduceColsWorkspace(rows, cols) bytes, a function of the shape alone;
  * that is 0 when one launch does it all and workspace may then be null).  The
- * launch allocates nothing. */
+ * launch allocates nothing.  The sums of x and of x * x down a dense fp32 window
+ * of 256 columns or more are the commonest cases and fill their bands with a
+ * kernel that interprets nothing (variant 1 of the "cols" family keeps the
+ * general one). */
 enum HcamdColsKind { HCAMD_COLS_SUM = 0, HCAMD_COLS_MAX = 1, HCAMD_COLS_MIN = 2 };
 #define HCAMD_COLS_MAX_POST 8
 size_t hcamdMapReduceColsWorkspace(size_t rows, size_t cols) HCAMD_NOEXCEPT;
@@ -658,7 +661,7 @@ int hcamdLaunchGemmF16(OlQueue q, const void *a, size_t lda, const void *bt,
 
 /* Chooses between kernel variants of one family by number (0 = default
  * choice by shape).  For tuning and measurement; family names are "add",
- * "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "stream", "gather"
+ * "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "cols", "stream", "gather"
  * (block shape), "gather_fuse" (groups per workgroup; read by
  * hcamdGatherGemmCreate).
  * Process-wide, guarded by a lock.  Returns 1 for an unknown family. */

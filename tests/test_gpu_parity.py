@@ -34,10 +34,10 @@ def ctx():
 
 @pytest.fixture(autouse=True)
 def default_variants():
-    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "stream", "gather", "gather_fuse"):
+    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "stream", "cols", "gather", "gather_fuse"):
         rt.set_variant(fam, 0)
     yield
-    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "stream", "gather", "gather_fuse"):
+    for fam in ("add", "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "stream", "cols", "gather", "gather_fuse"):
         rt.set_variant(fam, 0)
 
 

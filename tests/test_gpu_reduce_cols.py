@@ -120,6 +120,47 @@ def test_windows_of_larger_arrays_vectors_and_fp16_results(ctx, ld, off, dtype):
     assert (got[cols + 1:].view(np.uint16) == POISON32 & 0xFFFF).all()
 
 
+# rows that fill the turns of the waves and rows that do not,
+# column counts on and off the 256 columns of a wave, a window of a wider array
+@pytest.mark.parametrize("rows,cols,ld", [(4096, 8192, 8192), (4100, 256, 256), (1031, 264, 272),
+                                          (2999, 1000, 1000), (517, 4096, 4104), (70_000, 256, 256)])
+def test_sum_and_sum_of_squares_of_a_dense_fp32_window_take_their_own_kernel(ctx, rows, cols, ld):
+    rng = np.random.default_rng(rows + cols)
+    big = np.full((rows, ld), np.nan, np.float32)
+    x = (rng.standard_normal((rows, cols)) + 0.25).astype(np.float32)
+    big[:, :cols] = x
+    dbig = rt.to_device(big)
+    dx = _View(dbig, (rows, cols), 0, (ld, 1))
+    x64 = x.astype(np.float64)
+    sq64 = (x * x).astype(np.float64)  # the product is rounded to fp32 before it is added
+    say("cols_sum", rows, cols, ld)
+    programs = {"sum": ([I("in", 0)], x64), "sumsq": ([I("in", 0), I("in", 0), I("mul")], sq64),
+                "sumsq2": ([I("in", 0), I("mul_in", 0)], sq64)}
+    results = {}
+    for variant in (1, 2, 0):
+        rt.set_variant("cols", variant)
+        try:
+            for name, (prog, terms) in programs.items():
+                out = poisoned((cols + 8,), np.float32)
+                rt.plan_map_reduce_cols("sum", prog, [dx], _View(out, (cols,), 0),
+                                        post=[I("in", 0), I("divi", 0, 2.0)]).launch(sync=True)
+                kernel = rt.last_kernel_name()
+                got = out.to_host()
+                within(got[:cols], terms.sum(axis=0) / 2, sum_bound(terms) / 2)
+                assert (got[cols:].view(np.uint32) == POISON32).all()
+                results[variant, name] = got
+                if variant == 0:
+                    # the launch that finishes is the general kernel's either way
+                    assert kernel == "hcamd_map_reduce_cols_n1u4"
+                    again = poisoned((cols + 8,), np.float32)
+                    rt.plan_map_reduce_cols("sum", prog, [dx], _View(again, (cols,), 0),
+                                            post=[I("in", 0), I("divi", 0, 2.0)]).launch(sync=True)
+                    assert_array_equal(again.to_host().view(np.uint32), got.view(np.uint32))
+        finally:
+            rt.set_variant("cols", 0)
+    assert_array_equal(results[0, "sumsq"].view(np.uint32), results[0, "sumsq2"].view(np.uint32))
+
+
 def test_nan_and_infinities_follow_numpy(ctx):
     rows, cols = 300, 40
     x = np.random.default_rng(1).standard_normal((rows, cols)).astype(np.float32)
