@@ -963,11 +963,13 @@ __device__ __forceinline__ void cols_sum_f32(const float *__restrict__ x, size_t
       uint32_t rows, uint32_t band) {                                                     \
     cols_sum_f32<SQ, W, U>(x, ld, partial, cols, cols_pad, rows, band);                   \
   }
-// 16 waves with four rows in flight each measured fastest (root mean square down
-// the columns of 4096 x 8192, both launches: 32.7 us; 4 waves x 8 rows 39.6, 8 x 8
-// 34.5, 16 x 2 32.7; the general kernel 36.8): with a band of 64 rows a wave is
-// done after one round trip, and many short waves keep the memory busier than
-// few long ones.
+// 16 waves to a workgroup measured fastest, however many rows each has in flight
+// (root mean square down the columns of 4096 x 8192, both launches: 16 waves x 4,
+// 2 or 1 rows 32.7-32.9 us; 8 waves x 8, 4 or 2 rows 34.5-34.9; 4 waves x 8 or 4
+// rows 39.6-42.7; 2 x 8 41.2; the general kernel 36.8): what counts is the number
+// of waves the launch has.  With bands of 64 rows, 16 waves to a band are four
+// times the wave slots of the device, which the waves pass through one after the
+// other; 4 waves to a band fill the slots once and all wait at the same time.
 HCAMD_COLS_SUM(hcamd_cols_sum_f32, false, 16, 4)
 HCAMD_COLS_SUM(hcamd_cols_sumsq_f32, true, 16, 4)
 HCAMD_COLS_SUM(hcamd_cols_sum_f32_w4u8, false, 4, 8)
