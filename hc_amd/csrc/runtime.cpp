@@ -2101,6 +2101,7 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
     dev->report("%s: more than 2^31 rows or 2^32 - 1 columns", who);
     return 1;
   }
+  char name[48];
   const size_t perRow = cols / 8 + (cols % 8 ? 1 : 0);
   // a wave per row up to 4096 columns (at most 8 chunks per lane), else a workgroup
   const size_t lanesPerRow = perRow <= 512 ? 64 : 256;
@@ -2159,12 +2160,58 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
     a.vecMask = 0;
     a.interleaved = 1;
   }
+  // A layer normalisation as the front-end emits it for a body written with
+  // mean and var along axis 1 (five stages: the mean, the centred squares, the
+  // scale, then (x - mean) / s * w + b with numpy.ma's division), on dense fp32
+  // rows of at most 32768 elements with fp32 vectors w and b: a kernel that
+  // interprets nothing (variant 2 of "rows": the chain kernels for this too;
+  // variant 1: the general kernel for everything).
+  {
+    auto is = [&](size_t at, unsigned op, unsigned arg) {
+      return prog[at].op == op && prog[at].arg == arg;
+    };
+    auto stage = [&](size_t s, unsigned kind, unsigned dst, unsigned n) {
+      return stages[s].kind == kind && (kind == HCAMD_ROW_STORE || stages[s].dst == dst) &&
+             stages[s].nInstr == n;
+    };
+    const bool shape =
+        variantOf("rows") == 0 && nStages == 5 && nInputs == 3 && nColumns == 0 && pc == 17 &&
+        stage(0, HCAMD_ROW_SUM, 0, 1) && stage(1, HCAMD_ROW_SCALAR, 1, 2) &&
+        stage(2, HCAMD_ROW_SUM, 2, 5) && stage(3, HCAMD_ROW_SCALAR, 3, 4) &&
+        stage(4, HCAMD_ROW_STORE, 0, 5);
+    if (shape && is(0, HCAMD_MAP_IN, 0) && is(1, HCAMD_MAP_RED, 0) && prog[2].op == HCAMD_MAP_DIVI &&
+        is(3, HCAMD_MAP_IN, 0) && is(4, HCAMD_MAP_SUB_RED, 1) && is(5, HCAMD_MAP_IN, 0) &&
+        is(6, HCAMD_MAP_SUB_RED, 1) && prog[7].op == HCAMD_MAP_MUL && is(8, HCAMD_MAP_RED, 2) &&
+        prog[9].op == HCAMD_MAP_DIVI && prog[10].op == HCAMD_MAP_ADDI &&
+        prog[11].op == HCAMD_MAP_SQRT && is(12, HCAMD_MAP_IN, 0) && is(13, HCAMD_MAP_SUB_RED, 1) &&
+        is(14, HCAMD_MAP_MDIV_RED, 3) && is(15, HCAMD_MAP_MUL_IN, 1) &&
+        is(16, HCAMD_MAP_ADD_IN, 2) && prog[2].imm == prog[9].imm && a.f16Mask == 0 &&
+        inputLd[0] != 0 && inputLd[1] == 0 && inputLd[2] == 0 && (a.vecMask & 0x107u) == 0x107u &&
+        cols % 4 == 0 && cols <= 32768) {
+      const size_t chunks = cols / 4;
+      // two chunks to a lane on up to 512 lanes, then four; 1024 lanes from 2048 chunks on
+      size_t lpr = 64, e = chunks <= 64 ? 1 : 2;
+      while (lpr < 512 && lpr * 2 < chunks)
+        lpr *= 2;
+      if (chunks > 2048)
+        lpr = 1024;
+      while (lpr * e < chunks)
+        e *= 2;
+      std::snprintf(name, sizeof name, "hcamd_layer_norm_f32_w%zu_e%zu", lpr, e);
+      const size_t t = std::max(lpr, (size_t)256);
+      const void *x = inputs[0], *w = inputs[1], *b = inputs[2];
+      size_t ldx = inputLd[0], ldOut = ldo;
+      uint32_t nRows = static_cast<uint32_t>(rows), nCols = static_cast<uint32_t>(cols);
+      float n = prog[2].imm, eps = prog[10].imm;
+      void *args[] = {&x, &ldx, &w, &b, &out, &ldOut, &nRows, &nCols, &n, &eps};
+      return launch1d(queue, "map", name, ceilDiv(rows, t / lpr), t, args);
+    }
+  }
   // Rows of whole, aligned chunks, at most 4096 of them, whose stages are all
   // chains run on the chain kernels: a lane has its whole part of the row at
   // once, 8, 16 or 32 elements to a dispatch, and the operand that most
   // instructions read stays in LDS for the row (variant 1 of "rows": never).
   size_t lanes = lanesPerRow, maxGroups = SIZE_MAX, threads = 256;
-  char name[48];
   std::snprintf(name, sizeof name, "hcamd_row_program_w%zu", lanes);
   if (variantOf("rows") != 1 && !a.interleaved && cols % 8 == 0 && perRow <= 4096 && nInputs > 0) {
     HcamdMapInstr chained[HCAMD_ROW_MAX_INSTRS];

@@ -519,7 +519,13 @@ int hcamdLaunchMapReduceColsNoAlloc(OlQueue q, int kind, const HcamdMapInstr *pr
  * take a lane's whole part of the row at once: the operand most instructions
  * read is fetched once per row (into LDS), and an instruction is dispatched
  * once for 8, 16 or 32 elements of a lane (variant 1 of the "rows" family keeps
- * the general kernel).  Sums add in an order that
+ * the general kernel).  One program has a kernel of its own that interprets
+ * nothing: the layer normalisation (x - mean) / sqrt(var + eps) * w + b in the
+ * five stages the front-end emits for it (sum; RED DIVI; the sum of the
+ * centred squares; RED DIVI ADDI SQRT; IN SUB_RED MDIV_RED MUL_IN ADD_IN) on
+ * dense fp32 rows of at most 32768 elements with fp32 vectors w and b: the same
+ * operations per element, the row read once (variant 2 of "rows" keeps it on
+ * the kernels above).  Sums add in an order that
  * depends on the shape and the kernel only: results are reproducible, and agree with a
  * sequential fp32 sum to within the usual n * 2^-24 bound. */
 enum HcamdRowStageKind {

@@ -734,7 +734,10 @@ def test_row_reduction_bodies_match_the_simulator(name, rows, n):
         _row_bodies(sim_kernel)[name](*host[:-1], want, 8)
     out = rt.DeviceArray(host[-1].shape, host[-1].dtype).fill_bytes32(0xA5A5A5A5)
     _row_bodies(kernel)[name](*[rt.to_device(a) for a in host[:-1]], out, 8)
-    assert rt.last_kernel_name().startswith("hcamd_row_program")
+    # (a layer normalisation over dense fp32 rows of whole chunks has a kernel of its own)
+    assert rt.last_kernel_name().startswith(("hcamd_row_program", "hcamd_layer_norm_f32"))
+    if name == "layernorm" and n % 4 == 0 and n >= 8 and n <= 32768:
+        assert rt.last_kernel_name().startswith("hcamd_layer_norm_f32")
     got = out.to_host()
     if got.dtype == np.float16:
         assert_allclose(got.astype(np.float32), want.astype(np.float32), rtol=1.1e-3)

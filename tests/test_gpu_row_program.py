@@ -125,6 +125,72 @@ def test_layer_normalisation_with_weight_and_bias_vectors(ctx, cols, dtype, rows
     assert_allclose(out.to_host(), want, rtol=2e-5, atol=2e-5)
 
 
+def layer_norm_stages(n, eps):
+    """The five stages the front-end emits for (x - mean) / sqrt(var + eps) * w + b
+    written with mean and var along axis 1 (numpy.ma's division in the last)."""
+    return [("sum", 0, [I("in", 0)]),
+            ("scalar", 1, [I("red", 0), I("divi", 0, n)]),
+            ("sum", 2, [I("in", 0), I("sub_red", 1), I("in", 0), I("sub_red", 1), I("mul")]),
+            ("scalar", 3, [I("red", 2), I("divi", 0, n), I("addi", 0, eps), I("sqrt")]),
+            ("store", 0, [I("in", 0), I("sub_red", 1), I("mdiv_red", 3), I("mul_in", 1), I("add_in", 2)])]
+
+
+def layer_norm_kernel(cols):
+    chunks = cols // 4
+    lpr = 64
+    while lpr < 512 and lpr * 2 < chunks:
+        lpr *= 2
+    if chunks > 2048:
+        lpr = 1024
+    e = 1 if chunks <= 64 else 2
+    while lpr * e < chunks:
+        e *= 2
+    return f"hcamd_layer_norm_f32_w{lpr}_e{e}"
+
+
+# every kernel of the family, rows that leave lanes and chunk slots idle, more rows
+# than a workgroup holds, a window of a wider array
+@pytest.mark.parametrize("rows,cols,ld", [(33, 12, 12), (1001, 256, 256), (77, 300, 300), (515, 1000, 1008),
+                                          (130, 2048, 2048), (67, 4096, 4100), (4096, 8192, 8192),
+                                          (9, 8200, 8200), (5, 20_480, 20_480), (6, 32_768, 32_768)])
+def test_layer_normalisation_as_the_front_end_writes_it_takes_its_own_kernel(ctx, rows, cols, ld):
+    rng = np.random.default_rng(rows + cols)
+    big = np.full((rows, ld), np.nan, np.float32)
+    x = (rng.standard_normal((rows, cols)) * 2 + 0.5).astype(np.float32)
+    if rows > 8:
+        x[3, cols // 2] = np.inf       # the row's mean is not finite: numpy.ma stores nothing of it
+        x[5] = 1.25                    # no variance: eps alone under the root
+    big[:, :cols] = x
+    dbig = rt.to_device(big)
+    dx = _View(dbig, (rows, cols), 0, (ld, 1))
+    g = rng.standard_normal(cols).astype(np.float32)
+    b = rng.standard_normal(cols).astype(np.float32)
+    dg, db = rt.to_device(g), rt.to_device(b)
+    eps = 1e-5
+    stages = layer_norm_stages(float(cols), eps)
+    x64 = x.astype(np.float64)
+    with np.errstate(invalid="ignore"):
+        want = (x64 - x64.mean(axis=1, keepdims=True)) / np.sqrt(x64.var(axis=1, keepdims=True) + eps) * g + b
+    stored = np.isfinite(want)
+    results = {}
+    say("layer norm", rows, cols, ld)
+    for variant in (1, 2, 0):
+        rt.set_variant("rows", variant)
+        try:
+            out = poisoned((rows, cols), np.float32)
+            rt.plan_row_program(stages, [dx, dg, db], out).launch(sync=True)
+            name = rt.last_kernel_name()
+        finally:
+            rt.set_variant("rows", 0)
+        assert name == (layer_norm_kernel(cols) if variant == 0 else kernel_for(cols, general=variant == 1))
+        got = out.to_host()
+        assert_allclose(got[stored], want[stored], rtol=2e-5, atol=2e-5)
+        assert (got[~stored].view(np.uint32) == POISON32).all()
+        results[variant] = got
+    # the same operations per element: only the order of a row's sums differs
+    assert_allclose(results[0][stored], results[2][stored], rtol=3e-6, atol=3e-6)
+
+
 @pytest.mark.parametrize("rows,cols", [(1000, 7), (129, 1031), (4, 70_001), (5000, 264), (1300, 3000)])
 def test_row_sums_maxima_and_minima_as_per_row_results(ctx, rows, cols, rows_variant):
     rng = np.random.default_rng(rows)
