@@ -378,7 +378,7 @@ OlDevice olCreateDevice(const char *desc, OlErrorCallback errCallback,
     dev->colsKernelsReady = true;
     for (const char *name : {"hcamd_map_reduce_cols_n1u4", "hcamd_map_reduce_cols_n2u2",
                              "hcamd_map_reduce_cols_n4u1", "hcamd_cols_sum_f32",
-                             "hcamd_cols_sumsq_f32"})
+                             "hcamd_cols_sumsq_f32", "hcamd_cols_fold_f32"})
       if (!builtinKernel(dev.get(), "map", name))
         dev->colsKernelsReady = false;
   }
@@ -1849,6 +1849,8 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
   c.lanes = static_cast<uint32_t>(colLanes(cols));
   c.interleaved = allVec ? 0u : 1u;
   if (bands == 1) {
+    // few rows: fewer lanes to a row, as in the launch that folds bands
+    c.lanes = static_cast<uint32_t>(colSecondLanes(rows, c.lanes));
     finishing(a, c);
     return launchOne(a, c, nInputs, 1);
   }
@@ -1883,6 +1885,41 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
       return rc;
   } else if (int rc = launchOne(a, c, nInputs, bands)) {
     return rc;
+  }
+  // A sum whose post program only changes the folded value in place (the
+  // division of a mean, the root of a norm) into a dense fp32 result: the bands
+  // fold on a kernel that takes the program as arguments and interprets nothing.
+  struct FoldPost {
+    uint32_t n;
+    uint32_t op[4];
+    float imm[4];
+  } fp{};
+  bool simple = kind == HCAMD_COLS_SUM && outType == HCAMD_F32 && aligned16(out) && cols % 4 == 0 &&
+                nPost <= 5 && variantOf("cols") != 1 &&
+                (nPost == 0 || (post[0].op == HCAMD_MAP_IN && post[0].arg == 0));
+  for (size_t i = 1; i < nPost && simple; ++i) {
+    switch (post[i].op) {
+    case HCAMD_MAP_ADDI: case HCAMD_MAP_SUBI: case HCAMD_MAP_MULI: case HCAMD_MAP_DIVI:
+    case HCAMD_MAP_RSUBI: case HCAMD_MAP_RDIVI: case HCAMD_MAP_NEG: case HCAMD_MAP_ABS:
+    case HCAMD_MAP_SQRT:
+      fp.op[fp.n] = post[i].op;
+      fp.imm[fp.n++] = post[i].imm;
+      break;
+    default:
+      simple = false;
+    }
+  }
+  if (simple) {
+    Kernel *k = builtinKernel(dev, "map", "hcamd_cols_fold_f32");
+    if (!k)
+      return 1;
+    const void *partial = workspace;
+    size_t ld = colsPad;
+    uint32_t nCols = static_cast<uint32_t>(cols), nBands = static_cast<uint32_t>(bands);
+    void *args[] = {&partial, &ld, &out, &nCols, &nBands, &fp};
+    const size_t grid[3] = {ceilDiv(cols, (size_t)256), 1, 1};
+    const size_t block[3] = {1024, 1, 1};
+    return launch(queue, k, grid, block, args, 0);
   }
   // the bands just written are the rows of an fp32 operand
   MapArgs a2{};

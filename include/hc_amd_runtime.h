@@ -460,8 +460,10 @@ int hcamdLaunchMapSum(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
  * that is 0 when one launch does it all and workspace may then be null).  The
  * launch allocates nothing.  The sums of x and of x * x down a dense fp32 window
  * of 256 columns or more are the commonest cases and fill their bands with a
- * kernel that interprets nothing (variant 1 of the "cols" family keeps the
- * general one). */
+ * kernel that interprets nothing, and the bands of any sum whose post program
+ * only changes the folded value in place (at most four of ADDI SUBI MULI DIVI
+ * RSUBI RDIVI NEG ABS SQRT after IN 0) into a dense fp32 result fold on another
+ * (variant 1 of the "cols" family keeps the general one for both). */
 enum HcamdColsKind { HCAMD_COLS_SUM = 0, HCAMD_COLS_MAX = 1, HCAMD_COLS_MIN = 2 };
 #define HCAMD_COLS_MAX_POST 8
 size_t hcamdMapReduceColsWorkspace(size_t rows, size_t cols) HCAMD_NOEXCEPT;

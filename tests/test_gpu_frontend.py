@@ -763,7 +763,8 @@ def test_column_reduction_bodies_match_the_simulator(name, rows, n, gn):
     _col_bodies(sim_kernel)[name](x, y, want, gn)
     out = rt.DeviceArray((n,), np.float32).fill_bytes32(0xA5A5A5A5)
     _col_bodies(kernel)[name](rt.to_device(x), rt.to_device(y), out, gn)
-    assert rt.last_kernel_name().startswith("hcamd_map_reduce_cols")
+    # (the bands of a sum with a simple post program fold on a kernel of their own)
+    assert rt.last_kernel_name().startswith(("hcamd_map_reduce_cols", "hcamd_cols_fold_f32"))
     got = out.to_host()
     if name in ("col_max_abs", "col_min"):
         assert_array_equal(got, want)
@@ -1313,6 +1314,6 @@ def test_column_reductions_leave_deactivated_elements_out():
             sim_kernel(**deco)(body(fn))(x, y, want, gn)
         out = rt.DeviceArray((n,), np.float32).fill_bytes32(0xA5A5A5A5)
         kernel(**deco)(body(fn))(rt.to_device(x), rt.to_device(y), out, gn)
-        assert rt.last_kernel_name().startswith("hcamd_map"), name
+        assert rt.last_kernel_name().startswith(("hcamd_map", "hcamd_cols_fold_f32")), name
         assert np.isfinite(want).all(), name
         assert_allclose(out.to_host(), want, rtol=2e-4, atol=2e-4, err_msg=name)

@@ -149,9 +149,9 @@ def test_sum_and_sum_of_squares_of_a_dense_fp32_window_take_their_own_kernel(ctx
                 within(got[:cols], terms.sum(axis=0) / 2, sum_bound(terms) / 2)
                 assert (got[cols:].view(np.uint32) == POISON32).all()
                 results[variant, name] = got
+                # the bands of a sum with such a post program fold on a kernel of their own
+                assert kernel == ("hcamd_map_reduce_cols_n1u4" if variant == 1 else "hcamd_cols_fold_f32")
                 if variant == 0:
-                    # the launch that finishes is the general kernel's either way
-                    assert kernel == "hcamd_map_reduce_cols_n1u4"
                     again = poisoned((cols + 8,), np.float32)
                     rt.plan_map_reduce_cols("sum", prog, [dx], _View(again, (cols,), 0),
                                             post=[I("in", 0), I("divi", 0, 2.0)]).launch(sync=True)
@@ -159,6 +159,43 @@ def test_sum_and_sum_of_squares_of_a_dense_fp32_window_take_their_own_kernel(ctx
         finally:
             rt.set_variant("cols", 0)
     assert_array_equal(results[0, "sumsq"].view(np.uint32), results[0, "sumsq2"].view(np.uint32))
+
+
+def test_the_bands_of_a_sum_fold_with_every_simple_post_instruction(ctx):
+    """The general kernel fills the bands (two operands, fp16), the fold kernel adds
+    them up and runs the post program; variant 1 of "cols" runs the same on the
+    general kernel alone, and the two agree bit for bit where the sums do."""
+    rows, cols = 3000, 1028
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((rows, cols)).astype(np.float16)
+    y = rng.standard_normal((rows, cols)).astype(np.float16)
+    dx, dy = rt.to_device(x), rt.to_device(y)
+    posts = {"none": [], "mean": [I("in", 0), I("divi", 0, rows)],
+             "all": [I("in", 0), I("rsubi", 0, 2.0), I("abs"), I("sqrt"), I("rdivi", 0, 3.0)],
+             "more": [I("in", 0), I("muli", 0, 0.5), I("subi", 0, 1.0), I("neg"), I("addi", 0, 0.25)],
+             "long": [I("in", 0), I("abs"), I("sqrt"), I("abs"), I("sqrt"), I("neg")],     # five: the general kernel
+             "other": [I("in", 0), I("exp")]}                                             # not simple: the general kernel
+    for name, post in posts.items():
+        got = {}
+        for variant in (1, 0):
+            rt.set_variant("cols", variant)
+            try:
+                out = poisoned((cols + 8,), np.float32)
+                rt.plan_map_reduce_cols("sum", [I("in", 0), I("mul_in", 1)], [dx, dy], _View(out, (cols,), 0),
+                                        post=post).launch(sync=True)
+                kernel = rt.last_kernel_name()
+            finally:
+                rt.set_variant("cols", 0)
+            simple = variant == 0 and name not in ("long", "other")
+            assert kernel == ("hcamd_cols_fold_f32" if simple else "hcamd_map_reduce_cols_n1u4"), name
+            got[variant] = out.to_host()
+            assert (got[variant][cols:].view(np.uint32) == POISON32).all()
+        # the bands are the same; the fold adds them in another order
+        assert_allclose(got[0][:cols], got[1][:cols], rtol=2e-5, atol=1e-5, err_msg=name)
+    terms = (x.astype(np.float32) * y.astype(np.float32)).astype(np.float64)
+    rt.plan_map_reduce_cols("sum", [I("in", 0), I("mul_in", 1)], [dx, dy], _View(out, (cols,), 0),
+                            post=posts["more"]).launch(sync=True)
+    within(out.to_host()[:cols], -(terms.sum(axis=0) * 0.5 - 1.0) + 0.25, sum_bound(terms) + 1e-6)
 
 
 def test_nan_and_infinities_follow_numpy(ctx):
