@@ -99,6 +99,34 @@ HCAMD_COPY_2D(hcamd_copy2d_b4, uint32_t)
 HCAMD_COPY_2D(hcamd_copy2d_b8, uint64_t)
 HCAMD_COPY_2D(hcamd_copy2d_b16, u32x4)
 
+// Windows whose rows are contiguous inside and lie the same way against 16-byte
+// boundaries in both arrays, whatever the element size and however ragged the
+// ends: a lane owns one aligned 16-byte piece of the destination row and moves
+// it whole, or, at the two ends of the row, the bytes of it that belong to the
+// window.  (An int32 window of odd width or offset otherwise moves 4 bytes per
+// lane: 8191 x 8191 of a stride-8200 array 160 us, a uint8 one 1 byte per lane.)
+extern "C" __global__ __launch_bounds__(256) void hcamd_copy2d_rows(
+    const uint8_t *src, ptrdiff_t src_row_bytes, uint8_t *dst, ptrdiff_t dst_row_bytes,
+    size_t rows, size_t row_bytes) {
+  const size_t row = (size_t)blockIdx.y * blockDim.y + threadIdx.y;
+  if (row >= rows)
+    return;
+  const uint8_t *s0 = src + (ptrdiff_t)row * src_row_bytes;
+  uint8_t *d0 = dst + (ptrdiff_t)row * dst_row_bytes;
+  const ptrdiff_t lead = (ptrdiff_t)(reinterpret_cast<uintptr_t>(d0) & 15);
+  const ptrdiff_t piece = (ptrdiff_t)((size_t)blockIdx.x * blockDim.x + threadIdx.x);
+  const ptrdiff_t b0 = piece * 16 - lead, b1 = b0 + 16, end = (ptrdiff_t)row_bytes;
+  if (b0 >= end)
+    return;
+  if (b0 >= 0 && b1 <= end) {
+    stg<true>(reinterpret_cast<u32x4 *>(d0 + b0), ldg<true>(reinterpret_cast<const u32x4 *>(s0 + b0)));
+    return;
+  }
+  const ptrdiff_t lo = b0 < 0 ? 0 : b0, hi = b1 < end ? b1 : end;
+  for (ptrdiff_t b = lo; b < hi; ++b)
+    d0[b] = s0[b];
+}
+
 #define HCAMD_COPY_TILED(NAME, T)                                              \
   extern "C" __global__ __launch_bounds__(1024) void NAME(                     \
       int64_t unroll, int64_t ss0, const T *src, int64_t rows, int64_t cols,   \

@@ -193,20 +193,46 @@ def test_copy_window_smaller_than_destination_leaves_rest_untouched(ctx, itemsiz
     assert_array_equal(small.to_host(), big.to_host()[:5, :9])
 
 
-@pytest.mark.parametrize("cols,lds,ldd,off,kernel", [
-    (100, 132, 136, 0, "b16"), (100, 132, 136, 2, "b8"), (100, 132, 136, 1, "b4"),
-    (102, 132, 136, 0, "b8"), (100, 130, 136, 0, "b8"), (101, 132, 136, 0, "b4"),
-    (128, 129, 128, 0, "b4")])
-def test_copy_windows_use_the_widest_element_their_rows_allow(ctx, cols, lds, ldd, off, kernel):
+@pytest.mark.parametrize("cols,lds,ldd,off,kernel,pieces", [
+    (100, 132, 136, 0, "b16", True), (100, 132, 136, 2, "b8", True), (100, 132, 136, 1, "b4", True),
+    (102, 132, 136, 0, "b8", True), (100, 130, 136, 0, "b8", False), (101, 132, 136, 0, "b4", True),
+    (128, 129, 128, 0, "b4", False)])
+def test_copy_windows_use_the_widest_element_their_rows_allow(ctx, cols, lds, ldd, off, kernel, pieces):
+    """`pieces`: the rows lie the same way against 16-byte boundaries in both arrays,
+    so aligned 16-byte pieces with ragged ends move them (variant 10 of "copy": the
+    widest element the rows are aligned for, as for every other window)."""
     rows = 37
     rng = np.random.default_rng(cols + off)
     a = rng.integers(0, 1 << 30, (rows * lds + 8,)).astype(np.int32)
-    src, dst = dev(a), poisoned((rows * ldd + 8,), np.int32)
-    rt.copy2d(_View(src, (rows, cols), off, (lds, 1)), _View(dst, (rows, cols), off, (ldd, 1)))
-    assert rt.last_kernel_name() == "hcamd_copy2d_" + kernel
     want = np.full((rows * ldd + 8,), poison_value(np.int32), np.int32)
     want[off:off + rows * ldd].reshape(rows, ldd)[:, :cols] = \
         a[off:off + rows * lds].reshape(rows, lds)[:, :cols]
+    for variant in (0, 10):
+        rt.set_variant("copy", variant)
+        src, dst = dev(a), poisoned((rows * ldd + 8,), np.int32)
+        rt.copy2d(_View(src, (rows, cols), off, (lds, 1)), _View(dst, (rows, cols), off, (ldd, 1)))
+        assert rt.last_kernel_name() == "hcamd_copy2d_" + ("rows" if pieces and variant == 0 else kernel)
+        assert_array_equal(dst.to_host(), want)
+
+
+@pytest.mark.parametrize("dtype", [np.uint8, np.int16, np.int32, np.int64])
+@pytest.mark.parametrize("rows,cols,ld,soff,pieces_apart", [
+    (1, 1000, 1000, 3, 1), (5, 64, 80, 1, 0), (300, 1001, 1040, 5, 1), (70_000, 67, 80, 7, 0),
+    (33, 4097, 4112, 0, 1), (9, 100, 112, 15, 1)])
+def test_copy_windows_in_aligned_pieces_with_ragged_ends(ctx, dtype, rows, cols, ld, soff, pieces_apart):
+    """Source and destination offsets that differ by a multiple of 16 bytes, strides
+    that are multiples of 16 bytes, odd widths: every byte of the window arrives and
+    no byte outside it is touched, for every element size."""
+    item = np.dtype(dtype).itemsize
+    doff = soff + pieces_apart * (16 // item)
+    rng = np.random.default_rng(rows + cols)
+    a = rng.integers(0, 120, (rows * ld + 64,)).astype(dtype)
+    src, dst = dev(a), poisoned((rows * ld + 64,), dtype)
+    rt.copy2d(_View(src, (rows, cols), soff, (ld, 1)), _View(dst, (rows, cols), doff, (ld, 1)))
+    if cols * item >= 64 and (rows == 1 or (ld * item) % 16 == 0):
+        assert rt.last_kernel_name() == "hcamd_copy2d_rows"
+    want = np.full((rows * ld + 64,), poison_value(dtype), dtype)
+    want[doff:doff + rows * ld].reshape(rows, ld)[:, :cols] = a[soff:soff + rows * ld].reshape(rows, ld)[:, :cols]
     assert_array_equal(dst.to_host(), want)
 
 
