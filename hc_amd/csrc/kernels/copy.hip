@@ -105,7 +105,11 @@ HCAMD_COPY_2D(hcamd_copy2d_b16, u32x4)
 // it whole, or, at the two ends of the row, the bytes of it that belong to the
 // window.  (An int32 window of odd width or offset otherwise moves 4 bytes per
 // lane: 8191 x 8191 of a stride-8200 array 160 us, a uint8 one 1 byte per lane.)
-extern "C" __global__ __launch_bounds__(256) void hcamd_copy2d_rows(
+// ANY: the source rows lie differently from the destination rows; the 16 bytes of
+// a piece are then read from wherever they are (the compiler is told nothing
+// about their alignment and emits what the target allows for that).
+template <bool ANY>
+__device__ __forceinline__ void copy_rows(
     const uint8_t *src, ptrdiff_t src_row_bytes, uint8_t *dst, ptrdiff_t dst_row_bytes,
     size_t rows, size_t row_bytes) {
   const size_t row = (size_t)blockIdx.y * blockDim.y + threadIdx.y;
@@ -119,12 +123,27 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_copy2d_rows(
   if (b0 >= end)
     return;
   if (b0 >= 0 && b1 <= end) {
-    stg<true>(reinterpret_cast<u32x4 *>(d0 + b0), ldg<true>(reinterpret_cast<const u32x4 *>(s0 + b0)));
+    u32x4 v;
+    if constexpr (ANY)
+      __builtin_memcpy(&v, s0 + b0, 16);
+    else
+      v = ldg<true>(reinterpret_cast<const u32x4 *>(s0 + b0));
+    stg<true>(reinterpret_cast<u32x4 *>(d0 + b0), v);
     return;
   }
   const ptrdiff_t lo = b0 < 0 ? 0 : b0, hi = b1 < end ? b1 : end;
   for (ptrdiff_t b = lo; b < hi; ++b)
     d0[b] = s0[b];
+}
+extern "C" __global__ __launch_bounds__(256) void hcamd_copy2d_rows(
+    const uint8_t *src, ptrdiff_t src_row_bytes, uint8_t *dst, ptrdiff_t dst_row_bytes,
+    size_t rows, size_t row_bytes) {
+  copy_rows<false>(src, src_row_bytes, dst, dst_row_bytes, rows, row_bytes);
+}
+extern "C" __global__ __launch_bounds__(256) void hcamd_copy2d_rows_any(
+    const uint8_t *src, ptrdiff_t src_row_bytes, uint8_t *dst, ptrdiff_t dst_row_bytes,
+    size_t rows, size_t row_bytes) {
+  copy_rows<true>(src, src_row_bytes, dst, dst_row_bytes, rows, row_bytes);
 }
 
 #define HCAMD_COPY_TILED(NAME, T)                                              \

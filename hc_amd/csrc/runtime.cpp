@@ -835,11 +835,13 @@ int hcamdLaunchCopy2D(OlQueue q, size_t elemSize, const void *src,
   // ragged ends where the rows have them, non-temporal both ways (8192 x 8192
   // int32 of a stride-8200 array 92 -> 87 us, 8191 x 8191 at offset 1 160 -> 87 us;
   // variant 10 of "copy" keeps the element-wise kernel).
-  if (ss1 == 1 && ds1 == 1 && variant != 9 && variant != 10 &&
-      cols * elemSize >= 64 &&
-      (reinterpret_cast<uintptr_t>(src) - reinterpret_cast<uintptr_t>(dst)) % 16 == 0 &&
-      (rows == 1 || ((ss0 - ds0) * (ptrdiff_t)elemSize) % 16 == 0)) {
-    Kernel *k = builtinKernel(dev, "copy", "hcamd_copy2d_rows");
+  // Rows that lie differently in the two arrays: the same pieces of the
+  // destination, each read from wherever its 16 bytes are in the source.
+  if (ss1 == 1 && ds1 == 1 && variant != 9 && variant != 10 && cols * elemSize >= 64) {
+    const bool same =
+        (reinterpret_cast<uintptr_t>(src) - reinterpret_cast<uintptr_t>(dst)) % 16 == 0 &&
+        (rows == 1 || ((ss0 - ds0) * (ptrdiff_t)elemSize) % 16 == 0);
+    Kernel *k = builtinKernel(dev, "copy", same ? "hcamd_copy2d_rows" : "hcamd_copy2d_rows_any");
     if (!k)
       return 1;
     size_t rowBytes = cols * elemSize;

@@ -208,10 +208,10 @@ int hcamdDeviceInfo(OlDevice dev, int *computeUnits, int *clockKHz,
  * window [0,min(srcRows,dstRows)) x [0,min(srcCols,dstCols)) and leaves every
  * other byte of dst untouched.  elemSize is 1, 2, 4, 8 or 16.  Strides in
  * elements; either may be non-unit.  Dense windows move as one vector; windows
- * with unit inner strides whose rows lie the same way against 16-byte
- * boundaries in both arrays move in aligned 16-byte pieces with byte-wise ends;
- * other windows with the widest element their rows are aligned for; source and
- * destination must not overlap. */
+ * with unit inner strides move in aligned 16-byte pieces of the destination
+ * rows with byte-wise ends (read with aligned loads where the source rows lie
+ * the same way against 16-byte boundaries, with unaligned ones otherwise);
+ * other windows element by element; source and destination must not overlap. */
 int hcamdLaunchCopy2D(OlQueue q, size_t elemSize, const void *src,
                       size_t srcRows, size_t srcCols, ptrdiff_t srcStride0,
                       ptrdiff_t srcStride1, void *dst, size_t dstRows,

@@ -184,7 +184,13 @@ def test_copy_window_smaller_than_destination_leaves_rest_untouched(ctx, itemsiz
     a = rng.integers(0, 200, (37, 101)).astype(dtype)
     src, dst = dev(a), poisoned((50, 130), dtype)
     rt.copy2d(src, dst)                       # window 37 x 101 of a 50 x 130 array
+    assert rt.last_kernel_name() == "hcamd_copy2d_rows_any"     # rows of 101 and of 130 elements
+    assert_array_equal(dst.to_host(), cf.np_copy_window(a, np.full((50, 130), poison_value(dtype), dtype)))
+    rt.set_variant("copy", 10)                # the element-wise kernel
+    dst = poisoned((50, 130), dtype)
+    rt.copy2d(src, dst)
     assert rt.last_kernel_name() == f"hcamd_copy2d_b{itemsize}"
+    rt.set_variant("copy", 0)
     want = cf.np_copy_window(a, np.full((50, 130), poison_value(dtype), dtype))
     assert_array_equal(dst.to_host(), want)
     big = dev(rng.integers(0, 200, (64, 140)).astype(dtype))
@@ -199,8 +205,9 @@ def test_copy_window_smaller_than_destination_leaves_rest_untouched(ctx, itemsiz
     (128, 129, 128, 0, "b4", False)])
 def test_copy_windows_use_the_widest_element_their_rows_allow(ctx, cols, lds, ldd, off, kernel, pieces):
     """`pieces`: the rows lie the same way against 16-byte boundaries in both arrays,
-    so aligned 16-byte pieces with ragged ends move them (variant 10 of "copy": the
-    widest element the rows are aligned for, as for every other window)."""
+    so aligned 16-byte pieces with ragged ends move them; otherwise the pieces of the
+    destination are read from wherever they lie in the source (variant 10 of "copy":
+    the widest element the rows are aligned for)."""
     rows = 37
     rng = np.random.default_rng(cols + off)
     a = rng.integers(0, 1 << 30, (rows * lds + 8,)).astype(np.int32)
@@ -211,7 +218,8 @@ def test_copy_windows_use_the_widest_element_their_rows_allow(ctx, cols, lds, ld
         rt.set_variant("copy", variant)
         src, dst = dev(a), poisoned((rows * ldd + 8,), np.int32)
         rt.copy2d(_View(src, (rows, cols), off, (lds, 1)), _View(dst, (rows, cols), off, (ldd, 1)))
-        assert rt.last_kernel_name() == "hcamd_copy2d_" + ("rows" if pieces and variant == 0 else kernel)
+        assert rt.last_kernel_name() == "hcamd_copy2d_" + (
+            kernel if variant == 10 else "rows" if pieces else "rows_any")
         assert_array_equal(dst.to_host(), want)
 
 
@@ -233,6 +241,22 @@ def test_copy_windows_in_aligned_pieces_with_ragged_ends(ctx, dtype, rows, cols,
         assert rt.last_kernel_name() == "hcamd_copy2d_rows"
     want = np.full((rows * ld + 64,), poison_value(dtype), dtype)
     want[doff:doff + rows * ld].reshape(rows, ld)[:, :cols] = a[soff:soff + rows * ld].reshape(rows, ld)[:, :cols]
+    assert_array_equal(dst.to_host(), want)
+
+
+@pytest.mark.parametrize("dtype", [np.uint8, np.int16, np.int32, np.int64])
+@pytest.mark.parametrize("rows,cols,lds,ldd,soff,doff", [(1, 1000, 1000, 1000, 3, 8), (300, 1001, 1037, 1040, 5, 2),
+                                                         (20_000, 67, 71, 80, 0, 7), (33, 4097, 4100, 4111, 9, 0)])
+def test_copy_windows_whose_rows_lie_differently_in_the_two_arrays(ctx, dtype, rows, cols, lds, ldd, soff, doff):
+    item = np.dtype(dtype).itemsize
+    rng = np.random.default_rng(rows + cols)
+    a = rng.integers(0, 120, (rows * lds + 64,)).astype(dtype)
+    src, dst = dev(a), poisoned((rows * ldd + 64,), dtype)
+    rt.copy2d(_View(src, (rows, cols), soff, (lds, 1)), _View(dst, (rows, cols), doff, (ldd, 1)))
+    if cols * item >= 64:
+        assert rt.last_kernel_name() in ("hcamd_copy2d_rows", "hcamd_copy2d_rows_any")
+    want = np.full((rows * ldd + 64,), poison_value(dtype), dtype)
+    want[doff:doff + rows * ldd].reshape(rows, ldd)[:, :cols] = a[soff:soff + rows * lds].reshape(rows, lds)[:, :cols]
     assert_array_equal(dst.to_host(), want)
 
 
