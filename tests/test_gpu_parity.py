@@ -260,6 +260,21 @@ def test_copy_windows_whose_rows_lie_differently_in_the_two_arrays(ctx, dtype, r
     assert_array_equal(dst.to_host(), want)
 
 
+@pytest.mark.parametrize("variant", [0, 10])
+def test_copy_from_rows_in_reverse_order(ctx, variant):
+    """A source window whose row stride is negative (the rows of an array bottom up)."""
+    rows, cols, ld = 61, 203, 208
+    a = np.random.default_rng(3).integers(0, 1 << 30, (rows, ld)).astype(np.int32)
+    src, dst = dev(a), poisoned((rows, ld), np.int32)
+    rt.set_variant("copy", variant)
+    rt.copy2d(_View(src, (rows, cols), (rows - 1) * ld + 1, (-ld, 1)), _View(dst, (rows, cols), 2, (ld, 1)))
+    assert rt.last_kernel_name() == ("hcamd_copy2d_rows_any" if variant == 0 else "hcamd_copy2d_b4")
+    want = np.full((rows * ld,), poison_value(np.int32), np.int32)
+    for r in range(rows):
+        want[2 + r * ld:2 + r * ld + cols] = a[rows - 1 - r, 1:1 + cols]
+    assert_array_equal(dst.to_host().reshape(-1), want)
+
+
 def test_copy_large_flat_all_variants(ctx):
     a = np.random.default_rng(1).integers(0, 2 ** 31, 4_000_037, dtype=np.int32)[None, :]
     src = dev(a)
