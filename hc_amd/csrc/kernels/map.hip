@@ -2192,8 +2192,10 @@ HCAMD_ROW_CHAIN(1024, 4, 1024)
 // unstored); only the order in which a row's terms are added differs.  LPR lanes
 // share a row, each with E chunks of four elements LPR chunks apart, the row
 // stays in registers between its three passes, the waves of a row meet in LDS.
+// The same for the three-stage root-mean-square normalisation  s = sqrt(sum(x *
+// x) / n + eps);  out = x / s * w  (hcamd_rms_norm_f32_*: no mean, no bias).
 namespace {
-template <int LPR, int E>
+template <int LPR, int E, bool RMS>
 __device__ __forceinline__ void layer_norm_rows(const float *__restrict__ x, size_t ld,
                                                 const float *__restrict__ w,
                                                 const float *__restrict__ b,
@@ -2219,7 +2221,10 @@ __device__ __forceinline__ void layer_norm_rows(const float *__restrict__ x, siz
 #pragma unroll
     for (int k = 0; k < 4; ++k)
       acc = __fadd_rn(acc, v[e][k]);
-  const float mean = group_reduce<SumOp, W>(acc, slots[0][sub]) / n;
+  // (RMS: no mean is taken off; the mean of the squares, no bias)
+  float mean = 0.0f;
+  if constexpr (!RMS)
+    mean = group_reduce<SumOp, W>(acc, slots[0][sub]) / n;
   acc = -0.0f;
 #pragma unroll
   for (int e = 0; e < E; ++e) {
@@ -2227,7 +2232,7 @@ __device__ __forceinline__ void layer_norm_rows(const float *__restrict__ x, siz
     if (live && c < chunks) {
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
-        const float d = __fsub_rn(v[e][k], mean);
+        const float d = RMS ? v[e][k] : __fsub_rn(v[e][k], mean);
         acc = __fadd_rn(acc, __fmul_rn(d, d));
       }
     }
@@ -2240,16 +2245,19 @@ __device__ __forceinline__ void layer_norm_rows(const float *__restrict__ x, siz
   for (int e = 0; e < E; ++e) {
     const uint32_t c = e * LPR + lane;
     if (c < chunks) {
-      const f32x4 wv = reinterpret_cast<const f32x4 *>(w)[c], bv = reinterpret_cast<const f32x4 *>(b)[c];
+      const f32x4 wv = reinterpret_cast<const f32x4 *>(w)[c];
+      f32x4 bv = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      if constexpr (!RMS)
+        bv = reinterpret_cast<const f32x4 *>(b)[c];
       float y[4];
 #pragma unroll
       for (int k = 0; k < 4; ++k)
-        y[k] = __fsub_rn(v[e][k], mean);
+        y[k] = RMS ? v[e][k] : __fsub_rn(v[e][k], mean);
       uint32_t bad = 0;
       masked_div_scalar<4, false>(bad, y, s, false);
 #pragma unroll
       for (int k = 0; k < 4; ++k)
-        y[k] = __fadd_rn(__fmul_rn(y[k], wv[k]), bv[k]);
+        y[k] = RMS ? __fmul_rn(y[k], wv[k]) : __fadd_rn(__fmul_rn(y[k], wv[k]), bv[k]);
       if (bad == 0) {
         stg<true>(reinterpret_cast<f32x4 *>(orow) + c, f32x4{y[0], y[1], y[2], y[3]});
       } else {
@@ -2267,7 +2275,13 @@ __device__ __forceinline__ void layer_norm_rows(const float *__restrict__ x, siz
       hcamd_layer_norm_f32_w##LPR##_e##E(const float *x, size_t ld, const float *w,      \
                                          const float *b, float *out, size_t ldo,          \
                                          uint32_t rows, uint32_t cols, float n, float eps) { \
-    layer_norm_rows<LPR, E>(x, ld, w, b, out, ldo, rows, cols, n, eps);                   \
+    layer_norm_rows<LPR, E, false>(x, ld, w, b, out, ldo, rows, cols, n, eps);            \
+  }                                                                                       \
+  extern "C" __global__ __launch_bounds__(LPR < 256 ? 256 : LPR) void                     \
+      hcamd_rms_norm_f32_w##LPR##_e##E(const float *x, size_t ld, const float *w,        \
+                                       const float *b, float *out, size_t ldo,            \
+                                       uint32_t rows, uint32_t cols, float n, float eps) { \
+    layer_norm_rows<LPR, E, true>(x, ld, w, b, out, ldo, rows, cols, n, eps);             \
   }
 // (a row of 8192 on 512 lanes with four chunks each: 49.9 us for 4096 rows; on
 // 1024 lanes with two 51.4, on 256 with eight 53.4)

@@ -2237,6 +2237,24 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
     auto is = [&](size_t at, unsigned op, unsigned arg) {
       return prog[at].op == op && prog[at].arg == arg;
     };
+    auto launchNorm = [&](bool rmsForm, const void *x, size_t ldx, const void *w, const void *b,
+                          float n, float eps) {
+      const size_t chunks = cols / 4;
+      // two chunks to a lane on up to 512 lanes, then four; 1024 lanes from 2048 chunks on
+      size_t lpr = 64, e = chunks <= 64 ? 1 : 2;
+      while (lpr < 512 && lpr * 2 < chunks)
+        lpr *= 2;
+      if (chunks > 2048)
+        lpr = 1024;
+      while (lpr * e < chunks)
+        e *= 2;
+      std::snprintf(name, sizeof name, "hcamd_%s_norm_f32_w%zu_e%zu", rmsForm ? "rms" : "layer", lpr, e);
+      const size_t t = std::max(lpr, (size_t)256);
+      size_t ldOut = ldo;
+      uint32_t nRows = static_cast<uint32_t>(rows), nCols = static_cast<uint32_t>(cols);
+      void *args[] = {&x, &ldx, &w, &b, &out, &ldOut, &nRows, &nCols, &n, &eps};
+      return launch1d(queue, "map", name, ceilDiv(rows, t / lpr), t, args);
+    };
     auto stage = [&](size_t s, unsigned kind, unsigned dst, unsigned n) {
       return stages[s].kind == kind && (kind == HCAMD_ROW_STORE || stages[s].dst == dst) &&
              stages[s].nInstr == n;
@@ -2255,24 +2273,20 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
         is(16, HCAMD_MAP_ADD_IN, 2) && prog[2].imm == prog[9].imm && a.f16Mask == 0 &&
         inputLd[0] != 0 && inputLd[1] == 0 && inputLd[2] == 0 && (a.vecMask & 0x107u) == 0x107u &&
         cols % 4 == 0 && cols <= 32768) {
-      const size_t chunks = cols / 4;
-      // two chunks to a lane on up to 512 lanes, then four; 1024 lanes from 2048 chunks on
-      size_t lpr = 64, e = chunks <= 64 ? 1 : 2;
-      while (lpr < 512 && lpr * 2 < chunks)
-        lpr *= 2;
-      if (chunks > 2048)
-        lpr = 1024;
-      while (lpr * e < chunks)
-        e *= 2;
-      std::snprintf(name, sizeof name, "hcamd_layer_norm_f32_w%zu_e%zu", lpr, e);
-      const size_t t = std::max(lpr, (size_t)256);
-      const void *x = inputs[0], *w = inputs[1], *b = inputs[2];
-      size_t ldx = inputLd[0], ldOut = ldo;
-      uint32_t nRows = static_cast<uint32_t>(rows), nCols = static_cast<uint32_t>(cols);
-      float n = prog[2].imm, eps = prog[10].imm;
-      void *args[] = {&x, &ldx, &w, &b, &out, &ldOut, &nRows, &nCols, &n, &eps};
-      return launch1d(queue, "map", name, ceilDiv(rows, t / lpr), t, args);
+      return launchNorm(false, inputs[0], inputLd[0], inputs[1], inputs[2], prog[2].imm, prog[10].imm);
     }
+    // The root-mean-square normalisation  x / sqrt(mean(x * x) + eps) * w  in its
+    // three stages, under the same conditions.
+    const bool rms =
+        variantOf("rows") == 0 && nStages == 3 && nInputs == 2 && nColumns == 0 && pc == 9 &&
+        stage(0, HCAMD_ROW_SUM, 0, 2) && stage(1, HCAMD_ROW_SCALAR, 1, 4) &&
+        stage(2, HCAMD_ROW_STORE, 0, 3);
+    if (rms && is(0, HCAMD_MAP_IN, 0) && is(1, HCAMD_MAP_MUL_IN, 0) && is(2, HCAMD_MAP_RED, 0) &&
+        prog[3].op == HCAMD_MAP_DIVI && prog[4].op == HCAMD_MAP_ADDI && prog[5].op == HCAMD_MAP_SQRT &&
+        is(6, HCAMD_MAP_IN, 0) && is(7, HCAMD_MAP_MDIV_RED, 1) && is(8, HCAMD_MAP_MUL_IN, 1) &&
+        a.f16Mask == 0 && inputLd[0] != 0 && inputLd[1] == 0 && (a.vecMask & 0x103u) == 0x103u &&
+        cols % 4 == 0 && cols <= 32768)
+      return launchNorm(true, inputs[0], inputLd[0], inputs[1], inputs[1], prog[3].imm, prog[4].imm);
   }
   // Rows of whole, aligned chunks, at most 4096 of them, whose stages are all
   // chains run on the chain kernels: a lane has its whole part of the row at

@@ -530,8 +530,10 @@ int hcamdLaunchMapReduceColsNoAlloc(OlQueue q, int kind, const HcamdMapInstr *pr
  * five stages the front-end emits for it (sum; RED DIVI; the sum of the
  * centred squares; RED DIVI ADDI SQRT; IN SUB_RED MDIV_RED MUL_IN ADD_IN) on
  * dense fp32 rows of at most 32768 elements with fp32 vectors w and b: the same
- * operations per element, the row read once (variant 2 of "rows" keeps it on
- * the kernels above).  Sums add in an order that
+ * operations per element, the row read once; and so has the root-mean-square
+ * normalisation x / sqrt(mean(x * x) + eps) * w in its three stages (IN MUL_IN
+ * summed; RED DIVI ADDI SQRT; IN MDIV_RED MUL_IN) under the same conditions
+ * (variant 2 of "rows" keeps both on the kernels above).  Sums add in an order that
  * depends on the shape and the kernel only: results are reproducible, and agree with a
  * sequential fp32 sum to within the usual n * 2^-24 bound. */
 enum HcamdRowStageKind {
