@@ -2195,43 +2195,61 @@ HCAMD_ROW_CHAIN(1024, 4, 1024)
 // The same for the three-stage root-mean-square normalisation  s = sqrt(sum(x *
 // x) / n + eps);  out = x / s * w  (hcamd_rms_norm_f32_*: no mean, no bias).
 namespace {
-template <int LPR, int E, bool RMS>
-__device__ __forceinline__ void layer_norm_rows(const float *__restrict__ x, size_t ld,
+// HALF: x and out are fp16 (a chunk is then eight elements, computed in fp32
+// and rounded once when stored, which is what the trailing R16 of such a
+// program does); w and b stay fp32.
+template <int LPR, int E, bool RMS, bool HALF>
+__device__ __forceinline__ void layer_norm_rows(const void *__restrict__ x, size_t ld,
                                                 const float *__restrict__ w,
                                                 const float *__restrict__ b,
-                                                float *__restrict__ out, size_t ldo,
+                                                void *__restrict__ out, size_t ldo,
                                                 uint32_t rows, uint32_t cols, float n, float eps) {
   constexpr int T = LPR < 256 ? 256 : LPR, RPW = T / LPR, W = LPR / kWave;
+  constexpr int C = HALF ? 8 : 4; // elements of a 16-byte chunk
   __shared__ float slots[2][RPW][W];
   const uint32_t lane = threadIdx.x % LPR, sub = threadIdx.x / LPR;
-  const uint32_t row = blockIdx.x * RPW + sub, chunks = cols / 4;
+  const uint32_t row = blockIdx.x * RPW + sub, chunks = cols / C;
   const bool live = row < rows;
-  const f32x4 *xr = reinterpret_cast<const f32x4 *>(x + (size_t)row * ld);
-  f32x4 v[E];
+  const char *xr = static_cast<const char *>(x) + (size_t)row * ld * (HALF ? 2 : 4);
+  float v[E][C];
   float acc = -0.0f;
 #pragma unroll
   for (int e = 0; e < E; ++e) {
     const uint32_t c = e * LPR + lane;
-    v[e] = f32x4{-0.0f, -0.0f, -0.0f, -0.0f};
-    if (live && c < chunks)
-      v[e] = ldg<true>(xr + c);
+#pragma unroll
+    for (int k = 0; k < C; ++k)
+      v[e][k] = -0.0f;
+    if (live && c < chunks) {
+      if constexpr (HALF) {
+        const f16x8 h = ldg<true>(reinterpret_cast<const f16x8 *>(xr) + c);
+#pragma unroll
+        for (int k = 0; k < C; ++k)
+          v[e][k] = (float)h[k];
+      } else {
+        const f32x4 f = ldg<true>(reinterpret_cast<const f32x4 *>(xr) + c);
+#pragma unroll
+        for (int k = 0; k < C; ++k)
+          v[e][k] = f[k];
+      }
+    }
   }
-#pragma unroll
-  for (int e = 0; e < E; ++e)
-#pragma unroll
-    for (int k = 0; k < 4; ++k)
-      acc = __fadd_rn(acc, v[e][k]);
   // (RMS: no mean is taken off; the mean of the squares, no bias)
   float mean = 0.0f;
-  if constexpr (!RMS)
+  if constexpr (!RMS) {
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+#pragma unroll
+      for (int k = 0; k < C; ++k)
+        acc = __fadd_rn(acc, v[e][k]);
     mean = group_reduce<SumOp, W>(acc, slots[0][sub]) / n;
+  }
   acc = -0.0f;
 #pragma unroll
   for (int e = 0; e < E; ++e) {
     const uint32_t c = e * LPR + lane;
     if (live && c < chunks) {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
+      for (int k = 0; k < C; ++k) {
         const float d = RMS ? v[e][k] : __fsub_rn(v[e][k], mean);
         acc = __fadd_rn(acc, __fmul_rn(d, d));
       }
@@ -2240,49 +2258,71 @@ __device__ __forceinline__ void layer_norm_rows(const float *__restrict__ x, siz
   const float s = __builtin_sqrtf(__fadd_rn(group_reduce<SumOp, W>(acc, slots[1][sub]) / n, eps));
   if (!live)
     return;
-  float *orow = out + (size_t)row * ldo;
+  char *orow = static_cast<char *>(out) + (size_t)row * ldo * (HALF ? 2 : 4);
 #pragma unroll
   for (int e = 0; e < E; ++e) {
     const uint32_t c = e * LPR + lane;
     if (c < chunks) {
-      const f32x4 wv = reinterpret_cast<const f32x4 *>(w)[c];
-      f32x4 bv = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-      if constexpr (!RMS)
-        bv = reinterpret_cast<const f32x4 *>(b)[c];
-      float y[4];
+      float wv[C], bv[C], y[C];
 #pragma unroll
-      for (int k = 0; k < 4; ++k)
+      for (int q = 0; q < C / 4; ++q) {
+        const f32x4 w4 = reinterpret_cast<const f32x4 *>(w)[c * (C / 4) + q];
+        f32x4 b4 = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        if constexpr (!RMS)
+          b4 = reinterpret_cast<const f32x4 *>(b)[c * (C / 4) + q];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          wv[4 * q + k] = w4[k];
+          bv[4 * q + k] = b4[k];
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < C; ++k)
         y[k] = RMS ? v[e][k] : __fsub_rn(v[e][k], mean);
       uint32_t bad = 0;
-      masked_div_scalar<4, false>(bad, y, s, false);
+      masked_div_scalar<C, false>(bad, y, s, false);
 #pragma unroll
-      for (int k = 0; k < 4; ++k)
+      for (int k = 0; k < C; ++k)
         y[k] = RMS ? __fmul_rn(y[k], wv[k]) : __fadd_rn(__fmul_rn(y[k], wv[k]), bv[k]);
-      if (bad == 0) {
-        stg<true>(reinterpret_cast<f32x4 *>(orow) + c, f32x4{y[0], y[1], y[2], y[3]});
-      } else {
+      if constexpr (HALF) {
+        _Float16 *oh = reinterpret_cast<_Float16 *>(orow);
+        if (bad == 0) {
+          f16x8 h;
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
-          if (!((bad >> k) & 1u))
-            orow[4 * c + k] = y[k];
+          for (int k = 0; k < C; ++k)
+            h[k] = (_Float16)y[k];
+          stg<true>(reinterpret_cast<f16x8 *>(orow) + c, h);
+        } else {
+#pragma unroll
+          for (int k = 0; k < C; ++k)
+            if (!((bad >> k) & 1u))
+              oh[C * c + k] = (_Float16)y[k];
+        }
+      } else {
+        float *of = reinterpret_cast<float *>(orow);
+        if (bad == 0) {
+          stg<true>(reinterpret_cast<f32x4 *>(orow) + c, f32x4{y[0], y[1], y[2], y[3]});
+        } else {
+#pragma unroll
+          for (int k = 0; k < C; ++k)
+            if (!((bad >> k) & 1u))
+              of[C * c + k] = y[k];
+        }
       }
     }
   }
 }
 } // namespace
-#define HCAMD_LAYER_NORM(LPR, E)                                                          \
-  extern "C" __global__ __launch_bounds__(LPR < 256 ? 256 : LPR) void                     \
-      hcamd_layer_norm_f32_w##LPR##_e##E(const float *x, size_t ld, const float *w,      \
-                                         const float *b, float *out, size_t ldo,          \
-                                         uint32_t rows, uint32_t cols, float n, float eps) { \
-    layer_norm_rows<LPR, E, false>(x, ld, w, b, out, ldo, rows, cols, n, eps);            \
-  }                                                                                       \
-  extern "C" __global__ __launch_bounds__(LPR < 256 ? 256 : LPR) void                     \
-      hcamd_rms_norm_f32_w##LPR##_e##E(const float *x, size_t ld, const float *w,        \
-                                       const float *b, float *out, size_t ldo,            \
-                                       uint32_t rows, uint32_t cols, float n, float eps) { \
-    layer_norm_rows<LPR, E, true>(x, ld, w, b, out, ldo, rows, cols, n, eps);             \
+#define HCAMD_NORM_KERNEL(NAME, LPR, E, RMS, HALF)                                        \
+  extern "C" __global__ __launch_bounds__(LPR < 256 ? 256 : LPR) void NAME(               \
+      const void *x, size_t ld, const float *w, const float *b, void *out, size_t ldo,    \
+      uint32_t rows, uint32_t cols, float n, float eps) {                                 \
+    layer_norm_rows<LPR, E, RMS, HALF>(x, ld, w, b, out, ldo, rows, cols, n, eps);        \
   }
+#define HCAMD_LAYER_NORM(LPR, E)                                                          \
+  HCAMD_NORM_KERNEL(hcamd_layer_norm_f32_w##LPR##_e##E, LPR, E, false, false)             \
+  HCAMD_NORM_KERNEL(hcamd_rms_norm_f32_w##LPR##_e##E, LPR, E, true, false)                \
+  HCAMD_NORM_KERNEL(hcamd_rms_norm_f16_w##LPR##_e##E, LPR, E, true, true)
 // (a row of 8192 on 512 lanes with four chunks each: 49.9 us for 4096 rows; on
 // 1024 lanes with two 51.4, on 256 with eight 53.4)
 HCAMD_LAYER_NORM(64, 1)

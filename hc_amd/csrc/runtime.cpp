@@ -2238,8 +2238,8 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       return prog[at].op == op && prog[at].arg == arg;
     };
     auto launchNorm = [&](bool rmsForm, const void *x, size_t ldx, const void *w, const void *b,
-                          float n, float eps) {
-      const size_t chunks = cols / 4;
+                          float n, float eps, bool half = false) {
+      const size_t chunks = cols / (half ? 8 : 4);
       // two chunks to a lane on up to 512 lanes, then four; 1024 lanes from 2048 chunks on
       size_t lpr = 64, e = chunks <= 64 ? 1 : 2;
       while (lpr < 512 && lpr * 2 < chunks)
@@ -2248,7 +2248,8 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
         lpr = 1024;
       while (lpr * e < chunks)
         e *= 2;
-      std::snprintf(name, sizeof name, "hcamd_%s_norm_f32_w%zu_e%zu", rmsForm ? "rms" : "layer", lpr, e);
+      std::snprintf(name, sizeof name, "hcamd_%s_norm_%s_w%zu_e%zu", rmsForm ? "rms" : "layer",
+                    half ? "f16" : "f32", lpr, e);
       const size_t t = std::max(lpr, (size_t)256);
       size_t ldOut = ldo;
       uint32_t nRows = static_cast<uint32_t>(rows), nCols = static_cast<uint32_t>(cols);
@@ -2287,6 +2288,19 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
         a.f16Mask == 0 && inputLd[0] != 0 && inputLd[1] == 0 && (a.vecMask & 0x103u) == 0x103u &&
         cols % 4 == 0 && cols <= 32768)
       return launchNorm(true, inputs[0], inputLd[0], inputs[1], inputs[1], prog[3].imm, prog[4].imm);
+    // The same on fp16 rows, computed in fp32 and stored as fp16 (the program
+    // then ends in R16); w stays fp32.
+    const bool rmsHalf =
+        variantOf("rows") == 0 && nStages == 3 && nInputs == 2 && nColumns == 0 && pc == 10 &&
+        stage(0, HCAMD_ROW_SUM, 0, 2) && stage(1, HCAMD_ROW_SCALAR, 1, 4) &&
+        stage(2, HCAMD_ROW_STORE, 0, 4);
+    if (rmsHalf && is(0, HCAMD_MAP_IN, 0) && is(1, HCAMD_MAP_MUL_IN, 0) && is(2, HCAMD_MAP_RED, 0) &&
+        prog[3].op == HCAMD_MAP_DIVI && prog[4].op == HCAMD_MAP_ADDI && prog[5].op == HCAMD_MAP_SQRT &&
+        is(6, HCAMD_MAP_IN, 0) && is(7, HCAMD_MAP_MDIV_RED, 1) && is(8, HCAMD_MAP_MUL_IN, 1) &&
+        prog[9].op == HCAMD_MAP_R16 && a.f16Mask == 0x101u && inputLd[0] != 0 && inputLd[1] == 0 &&
+        (a.vecMask & 0x103u) == 0x103u && cols % 8 == 0 && cols <= 65536)
+      return launchNorm(true, inputs[0], inputLd[0], inputs[1], inputs[1], prog[3].imm, prog[4].imm,
+                        true);
   }
   // Rows of whole, aligned chunks, at most 4096 of them, whose stages are all
   // chains run on the chain kernels: a lane has its whole part of the row at

@@ -532,7 +532,8 @@ int hcamdLaunchMapReduceColsNoAlloc(OlQueue q, int kind, const HcamdMapInstr *pr
  * dense fp32 rows of at most 32768 elements with fp32 vectors w and b: the same
  * operations per element, the row read once; and so has the root-mean-square
  * normalisation x / sqrt(mean(x * x) + eps) * w in its three stages (IN MUL_IN
- * summed; RED DIVI ADDI SQRT; IN MDIV_RED MUL_IN) under the same conditions
+ * summed; RED DIVI ADDI SQRT; IN MDIV_RED MUL_IN; with R16 at the end on fp16
+ * rows of whole chunks of 8 with an fp32 w) under the same conditions
  * (variant 2 of "rows" keeps both on the kernels above).  Sums add in an order that
  * depends on the shape and the kernel only: results are reproducible, and agree with a
  * sequential fp32 sum to within the usual n * 2^-24 bound. */

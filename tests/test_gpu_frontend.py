@@ -734,10 +734,12 @@ def test_row_reduction_bodies_match_the_simulator(name, rows, n):
         _row_bodies(sim_kernel)[name](*host[:-1], want, 8)
     out = rt.DeviceArray(host[-1].shape, host[-1].dtype).fill_bytes32(0xA5A5A5A5)
     _row_bodies(kernel)[name](*[rt.to_device(a) for a in host[:-1]], out, 8)
-    # (a layer normalisation over dense fp32 rows of whole chunks has a kernel of its own)
-    assert rt.last_kernel_name().startswith(("hcamd_row_program", "hcamd_layer_norm_f32"))
+    # (the two normalisations over dense rows of whole chunks have kernels of their own)
+    assert rt.last_kernel_name().startswith(("hcamd_row_program", "hcamd_layer_norm_f32", "hcamd_rms_norm_f16"))
     if name == "layernorm" and n % 4 == 0 and n >= 8 and n <= 32768:
         assert rt.last_kernel_name().startswith("hcamd_layer_norm_f32")
+    if name == "rmsnorm_half" and n % 8 == 0:
+        assert rt.last_kernel_name().startswith("hcamd_rms_norm_f16")
     got = out.to_host()
     if got.dtype == np.float16:
         assert_allclose(got.astype(np.float32), want.astype(np.float32), rtol=1.1e-3)

@@ -135,8 +135,8 @@ def layer_norm_stages(n, eps):
             ("store", 0, [I("in", 0), I("sub_red", 1), I("mdiv_red", 3), I("mul_in", 1), I("add_in", 2)])]
 
 
-def layer_norm_kernel(cols):
-    chunks = cols // 4
+def layer_norm_kernel(cols, per_chunk=4):
+    chunks = cols // per_chunk
     lpr = 64
     while lpr < 512 and lpr * 2 < chunks:
         lpr *= 2
@@ -191,13 +191,17 @@ def test_layer_normalisation_as_the_front_end_writes_it_takes_its_own_kernel(ctx
     assert_allclose(results[0][stored], results[2][stored], rtol=3e-6, atol=3e-6)
 
 
-@pytest.mark.parametrize("rows,cols,ld", [(33, 12, 12), (77, 300, 300), (515, 1000, 1008), (4096, 8192, 8192),
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("rows,cols,ld", [(33, 24, 24), (77, 304, 304), (515, 1000, 1008), (4096, 8192, 8192),
                                           (9, 8200, 8200), (6, 32_768, 32_768)])
-def test_rms_normalisation_as_the_front_end_writes_it_takes_its_own_kernel(ctx, rows, cols, ld):
-    """x / sqrt(mean(x * x) + eps) * w in the three stages the front-end emits."""
+def test_rms_normalisation_as_the_front_end_writes_it_takes_its_own_kernel(ctx, rows, cols, ld, dtype):
+    """x / sqrt(mean(x * x) + eps) * w in the three stages the front-end emits, on
+    fp32 rows and on fp16 rows (computed in fp32, stored as fp16: the program then
+    ends in r16)."""
+    half = dtype == np.float16
     rng = np.random.default_rng(rows + cols)
-    big = np.full((rows, ld), np.nan, np.float32)
-    x = (rng.standard_normal((rows, cols)) * 2 + 0.5).astype(np.float32)
+    big = np.full((rows, ld), np.nan, dtype)
+    x = (rng.standard_normal((rows, cols)) * 2 + 0.5).astype(dtype)
     if rows > 8:
         x[3, cols // 2] = np.inf       # the scale is not finite: x / inf is 0 (stored), inf / inf is not
         x[5] = 0.0
@@ -209,28 +213,31 @@ def test_rms_normalisation_as_the_front_end_writes_it_takes_its_own_kernel(ctx, 
     eps = 1e-6
     stages = [("sum", 0, [I("in", 0), I("mul_in", 0)]),
               ("scalar", 1, [I("red", 0), I("divi", 0, float(cols)), I("addi", 0, eps), I("sqrt")]),
-              ("store", 0, [I("in", 0), I("mdiv_red", 1), I("mul_in", 1)])]
+              ("store", 0, [I("in", 0), I("mdiv_red", 1), I("mul_in", 1)] + ([I("r16")] if half else []))]
     x64 = x.astype(np.float64)
     with np.errstate(invalid="ignore", over="ignore"):
         q = x64 / np.sqrt((x64 * x64).mean(axis=1, keepdims=True) + eps)
         want = q * g
     stored = np.isfinite(q)
+    tol = dict(rtol=1.1e-3, atol=1e-4) if half else dict(rtol=2e-5, atol=2e-5)
     results = {}
     for variant in (1, 2, 0):
         rt.set_variant("rows", variant)
         try:
-            out = poisoned((rows, cols), np.float32)
+            out = poisoned((rows, cols), dtype)
             rt.plan_row_program(stages, [dx, dg], out).launch(sync=True)
             name = rt.last_kernel_name()
         finally:
             rt.set_variant("rows", 0)
-        assert name == (layer_norm_kernel(cols).replace("layer", "rms") if variant == 0
-                        else kernel_for(cols, general=variant == 1))
+        own = layer_norm_kernel(cols, 8 if half else 4).replace("layer", "rms").replace("f32", "f16" if half else "f32")
+        assert name == (own if variant == 0 else kernel_for(cols, general=variant == 1))
         got = out.to_host()
-        assert_allclose(got[stored], want[stored], rtol=2e-5, atol=2e-5)
-        assert (got[~stored].view(np.uint32) == POISON32).all()
-        results[variant] = got
-    assert_allclose(results[0][stored], results[2][stored], rtol=3e-6, atol=3e-6)
+        assert_allclose(got[stored].astype(np.float64), want[stored], **tol)
+        raw = got.view(np.uint16 if half else np.uint32)
+        assert (raw[~stored] == (POISON32 & 0xFFFF if half else POISON32)).all()
+        results[variant] = got.astype(np.float64)
+    assert_allclose(results[0][stored], results[2][stored], **(dict(rtol=1e-3, atol=1e-4) if half else
+                                                               dict(rtol=3e-6, atol=3e-6)))
 
 
 @pytest.mark.parametrize("rows,cols", [(1000, 7), (129, 1031), (4, 70_001), (5000, 264), (1300, 3000)])
