@@ -684,30 +684,63 @@ _MAP_BINARY = {"add": ("add", "add", True), "mul": ("mul", "mul", True),
                "maximum": ("max", "max", True), "minimum": ("min", "min", True),
                "sub": ("sub", "rsub", False), "div": ("div", "rdiv", False)}
 _MAP_UNARY = {"neg": "neg", "abs": "abs", "sqrt": "sqrt", "rint": "rint", "exp": "exp",
-              "log": "log", "tanh": "tanh"}
+              "log": "log", "tanh": "tanh", "masqrt": "masqrt"}
 _MAP_EXACT = {"neg", "abs", "maximum", "minimum", "clip"}   # fp16 in -> fp16 out, no rounding
 _MAP_FLOATS = ("float16", "float32")
+
+
+_REDUCTIONS = ("sum", "max", "min", "count", "norm")
+
+
+def _is_reduction(t: Tile) -> bool:
+    return t.op in _REDUCTIONS and "axes" in t.attrs and len(t.args) == 1
 
 
 def _masks(t: Tile) -> bool:
     """t itself can deactivate elements at run time.  The tile operators / // %
     and ** go through numpy.ma, which deactivates failed divisions and results
     of ** that are not finite; NumPy functions with a domain (sqrt, log, divide)
-    called on tiles deactivate where the domain fails."""
+    called on tiles deactivate where the domain fails.  The division of a mean
+    is numpy.ma's too; a variance is inactive where fewer than ddof + 1 elements
+    were active; numpy.ma.sqrt (the standard deviation's) deactivates results
+    that are not finite."""
+    if t.op == "masqrt":
+        return True
+    if t.op == "vardiv":
+        return not _const(t.args[1])
     if t.attrs.get("func"):
         return t.op in ("sqrt", "log", "div", "floordiv", "mod")
     return t.op in ("div", "floordiv", "mod") or bool(t.attrs.get("pow"))
 
 
 def _maybe_masked(t: Tile, memo=None) -> bool:
-    """Some element of t may be inactive for a reason only the data knows."""
+    """Some element of t may be inactive for a reason only the data knows.  (A
+    fold over elements of which every one may be inactive may be inactive itself;
+    their number never is.)"""
     memo = {} if memo is None else memo
     if t.uid not in memo:
-        if _is(t, "load") or _const(t):
+        if _is(t, "load") or _const(t) or t.op == "count":
             memo[t.uid] = False
         else:
             memo[t.uid] = _masks(t) or any(_maybe_masked(a, memo) for a in t.args if isinstance(a, Tile))
     return memo[t.uid]
+
+
+def _fails_on_finite_data(t: Tile) -> bool:
+    """t can deactivate elements whose operands are ordinary finite numbers: a
+    zero divisor, an argument outside a function's domain, a variance over too
+    few active elements.  (A division by a non-zero constant or by a count, a
+    square and numpy.ma.sqrt of a variance only fail on values that are not
+    finite already, or by overflow.)"""
+    if not _masks(t):
+        return False
+    if t.op == "masqrt" or t.attrs.get("pow"):
+        return False
+    if t.op == "div" and not t.attrs.get("func"):
+        d = t.args[1]
+        if t.attrs.get("ma") or (_const(d) and d.attrs.get("value") != 0.0):
+            return False
+    return True
 
 
 # Operations that compute from their operands' values and change nothing about
@@ -717,17 +750,36 @@ def _maybe_masked(t: Tile, memo=None) -> bool:
 _TRANSPARENT_FUNCS = ("exp", "rint", "tanh", "maximum", "minimum", "add", "sub", "mul", "clip", "neg", "abs")
 
 
-def _values_flow_plainly(t: Tile, clean: bool = True) -> bool:
+def _values_flow_plainly(t: Tile, clean: bool = True, finite: bool = False) -> bool:
     """Every operation that can deactivate elements has only transparent
     operations above it: then the value stored for a deactivated element is
-    what plain arithmetic on the value numpy.ma left there gives."""
+    what plain arithmetic on the value numpy.ma left there gives.  `finite`:
+    only operations that can fail on finite data count."""
     if _is(t, "load") or _const(t):
         return True
-    if _masks(t) and not clean:
+    if _is_reduction(t):
+        # a fold's value does not depend on what its deactivated elements hold;
+        # the fold itself is inactive where all of them are
+        return clean or not _can_fail(t, finite)
+    if (_fails_on_finite_data(t) if finite else _masks(t)) and not clean:
         return False
     transparent = _is(t, "astype", 1) or t.op in ("neg", "abs") or \
         (bool(t.attrs.get("func")) and t.op in _TRANSPARENT_FUNCS)
-    return all(_values_flow_plainly(a, clean and transparent) for a in t.args if isinstance(a, Tile))
+    return all(_values_flow_plainly(a, clean and transparent, finite) for a in t.args if isinstance(a, Tile))
+
+
+def _can_fail(t: Tile, finite: bool, memo=None) -> bool:
+    """_maybe_masked, or (finite) the same restricted to failures on finite data."""
+    if not finite:
+        return _maybe_masked(t)
+    memo = {} if memo is None else memo
+    if t.uid not in memo:
+        if _is(t, "load") or _const(t) or t.op == "count":
+            memo[t.uid] = False
+        else:
+            memo[t.uid] = _fails_on_finite_data(t) or \
+                any(_can_fail(a, True, memo) for a in t.args if isinstance(a, Tile))
+    return memo[t.uid]
 
 
 class _NeedsEntryMasks(Exception):
@@ -751,12 +803,27 @@ def _leaf(t: Tile):
     return None
 
 
+# Flags in `arg` of the instructions of a stage that computes with row scalars
+# (bit 8 is the fp16 flag of the numpy.ma quotients).  What a deactivated row
+# scalar holds is part of the result when it is stored, and numpy.ma leaves the
+# first operand's value there for the tile operators + - * / while NumPy
+# functions compute on the values regardless.
+_FUNC_FORM = 0x200            # the operation was called as a NumPy function
+_SWAPPED = 0x400              # a commutative operation whose running value is the second operand
+
+
 class _MapCompiler:
     """Sethi-Ullman ordering: the operand that needs the deeper stack is
     evaluated first, constants become immediates, so an expression with up to
     eight distinct leaves in a balanced tree fits the four-entry stack."""
 
     masked = False                # emit numpy.ma's division rule (element-wise map and its sum only)
+    _scalar_mode = False          # the program computes with row scalars (row programs only)
+
+    def _form(self, t: Tile, swapped: bool = False) -> int:
+        if not self._scalar_mode:
+            return 0
+        return (_FUNC_FORM if t.attrs.get("func") else 0) | (_SWAPPED if swapped else 0)
 
     def __init__(self, n_groups):
         self.n_groups = n_groups
@@ -784,6 +851,8 @@ class _MapCompiler:
             if all(_const(a) for a in t.args):
                 return False
             return all(self.supported(a) and (_const(a) or a.shape == t.shape) for a in t.args)
+        if _is(t, "vardiv", 2):                  # a variance whose count is a number
+            return _const(t.args[1]) and self.supported(t.args[0])
         return False
 
     def need(self, t: Tile) -> int:
@@ -791,7 +860,7 @@ class _MapCompiler:
             return self.need_cache[t.uid]
         if _is(t, "load") or _const(t):
             n = 1
-        elif len(t.args) == 1:
+        elif len(t.args) == 1 or _is(t, "vardiv", 2):
             n = self.need(t.args[0])
         else:
             a, b = t.args
@@ -817,9 +886,8 @@ class _MapCompiler:
         try:
             self.emit(t, out)
         except _NeedsEntryMasks:
-            self.masked = False
-            del out[:]
-            self.emit(t, out)
+            raise NoNativeKernel("numpy.divide called as a function next to a reduction has no "
+                                 "native code (the / operator has)") from None
 
     def _emit_node(self, t: Tile, out: list):
         half = t.dtype_name == "float16"
@@ -839,6 +907,12 @@ class _MapCompiler:
             out.append(("maxi", 0, _round_to(t.attrs["lo"], t.dtype_name)))
             out.append(("mini", 0, _round_to(t.attrs["hi"], t.dtype_name)))
             return
+        if _is(t, "vardiv", 2):
+            # the sum of the centred squares over a count that is a number: the
+            # variance is active whatever the quotient is
+            self.emit(t.args[0], out)
+            out.append(("divi", 0, _round_to(t.args[1].attrs["value"], t.dtype_name)))
+            return
         mdiv = self.masked and t.op == "div"
         if mdiv and t.attrs.get("func"):
             raise _NeedsEntryMasks()           # numpy.divide as a function: the general map has it
@@ -847,6 +921,8 @@ class _MapCompiler:
             name = _MAP_UNARY[t.op]
             if self.masked and t.attrs.get("func") and name in ("sqrt", "log"):
                 name = "m" + name              # numpy.sqrt / numpy.log of a tile: domain fill
+            if name == "masqrt" and not self.masked:
+                name = "sqrt"                  # stored in full: the same values
             out.append((name, 0, 0.0))
             if self.masked and t.op == "sqrt" and t.attrs.get("pow"):
                 out.append(("addi", 0, 0.0))   # x ** 0.5 of -0 is +0 (the square root's is -0)
@@ -856,12 +932,13 @@ class _MapCompiler:
                 fwd, rev = "mdiv", "rmdiv"
             flag = int(half) if mdiv else 0              # the quotient is tested as fp16
             a, b = t.args
+            same = fwd == rev                       # commutative: the name does not say which side runs
             if _const(b):
                 self.emit(a, out)
-                out.append((fwd + "i", flag << 8, _round_to(b.attrs["value"], t.dtype_name)))
+                out.append((fwd + "i", flag << 8 | self._form(t), _round_to(b.attrs["value"], t.dtype_name)))
             elif _const(a):
                 self.emit(b, out)
-                out.append((rev + "i", flag << 8, _round_to(a.attrs["value"], t.dtype_name)))
+                out.append((rev + "i", flag << 8 | self._form(t, same), _round_to(a.attrs["value"], t.dtype_name)))
             elif _leaf(b) is not None:              # operand forms: one dispatch, no push
                 self.emit(a, out)
                 out.append((fwd + "_in", self.operand(_leaf(b)) | (flag << 8), 0.0))
@@ -871,11 +948,11 @@ class _MapCompiler:
             elif self.need(a) >= self.need(b):
                 self.emit(a, out)
                 self.emit(b, out)
-                out.append((fwd, flag, 0.0))
+                out.append((fwd, flag | self._form(t), 0.0))
             else:
                 self.emit(b, out)
                 self.emit(a, out)
-                out.append((rev, flag, 0.0))
+                out.append((rev, flag | self._form(t, same), 0.0))
         if half and t.op not in _MAP_EXACT and not mdiv:
             out.append(("r16", 0, 0.0))
 
@@ -929,7 +1006,7 @@ def match_map(dst_view, value, n_groups):
 # ---------------------------------------------------------------------------
 # Row programs: elementwise arithmetic mixed with reductions along rows
 # ---------------------------------------------------------------------------
-_ROW_REDUCE = {"sum": "sum", "max": "max", "min": "min"}
+_ROW_REDUCE = {"sum": "sum", "max": "max", "min": "min", "count": "count"}
 
 
 # ---------------------------------------------------------------------------
@@ -1237,7 +1314,7 @@ class _RowCompiler(_MapCompiler):
             return not _is(t, "load") and self._is_scalar_node(t.args[0])
         if _is(t, "astype", 1) or t.op in _MAP_UNARY or _is(t, "clip", 1):
             return self._is_scalar_node(t.args[0])
-        if t.op in _MAP_BINARY and len(t.args) == 2:
+        if (t.op in _MAP_BINARY or t.op == "vardiv") and len(t.args) == 2:
             return all(_const(a) or self._is_scalar_node(a) for a in t.args) and \
                 not all(_const(a) for a in t.args)
         return False
@@ -1304,13 +1381,32 @@ class _RowCompiler(_MapCompiler):
             if _same(uid_t, t):
                 self.slots[t.uid] = slot
                 return slot
-        if t.op == "norm" and t.attrs.get("axes") == (1,):
+        if t.op == "norm" and t.attrs.get("axes") == (1,) and not _maybe_masked(t.args[0]):
             # numpy.linalg.norm along an axis is sqrt(add.reduce(x * x))
             body = t.args[0]
             total = (body * body)._reduce("sum", 1, t.attrs.get("keepdims", False))
             slot = self.scalar(Tile("sqrt", (total,), total.shape, total.dtype_name))
             self.slots[t.uid] = slot
             return slot
+        if _is(t, "vardiv", 2):
+            # numpy.ma's variance: the sum of the centred squares (0 where every
+            # one of them is inactive, whatever made them so) over the count less
+            # ddof; active wherever that is positive, whatever the division did
+            total, count = t.args
+            program = [("red0", self.scalar(total), 0.0)]
+            if _const(count):
+                program.append(("divi", 0, _round_to(count.attrs["value"], "float32")))
+            else:
+                c = self.scalar(count)
+                program += [("mdiv_red", c, 0.0), ("livepos", c, 0.0)]
+            slot = self._new_slot(t)
+            self.stages.append(("scalar", slot, program))
+            self._same_reductions.append((t, slot))
+            return slot
+        if t.op == "norm" and t.attrs.get("axes") == (1,) and _maybe_masked(t.args[0]):
+            raise NoNativeKernel("numpy.linalg.norm of a tile whose elements a division or a domain "
+                                 "function may deactivate: the norm adds up what such elements hold, "
+                                 "which has no native code (use (x * x).sum(axis=1) for the active ones)")
         if t.op in _ROW_REDUCE and t.attrs.get("axes") == (1,):
             body = t.args[0]
             if self.klass(body) != "E":
@@ -1350,7 +1446,7 @@ class _RowCompiler(_MapCompiler):
             if base.uid in self.slots:
                 return
             if base.op in (*_ROW_REDUCE, "norm") and base.attrs.get("axes") == (1,) or \
-                    _is(base, "load"):
+                    _is(base, "load") or _is(base, "vardiv", 2):
                 self.scalar(base)
                 return
             t = base
@@ -1360,10 +1456,10 @@ class _RowCompiler(_MapCompiler):
     def program(self, t: Tile, scalar: bool = False) -> list:
         self.prepare(t, scalar)
         self._scalar_mode = scalar
-        # numpy.ma's rules for / ** sqrt log in the element-wise stages (stores
-        # skip, sums and maxima leave out what they deactivate); arithmetic on
-        # row scalars stays plain
-        self.masked = not scalar
+        # numpy.ma's rules for / ** sqrt log: in the element-wise stages stores
+        # skip, and folds leave out, what they deactivate; a row scalar that they
+        # deactivate deactivates every element and every row scalar computed from it
+        self.masked = True
         self.need_cache = {}
         if not self.supported(t):
             raise NoNativeKernel(f"{t!r} is not an expression of float32 / float16 tiles, row "
@@ -1374,10 +1470,9 @@ class _RowCompiler(_MapCompiler):
         out: list = []
         try:
             self.emit(t, out)
-        except _NeedsEntryMasks:               # numpy.divide as a function: plain arithmetic
-            self.masked = False
-            out = []
-            self.emit(t, out)
+        except _NeedsEntryMasks:
+            raise NoNativeKernel("numpy.divide called as a function next to a reduction along rows "
+                                 "has no native code (the / operator has)") from None
         return out
 
     def slot_of(self, t: Tile):
@@ -1456,10 +1551,10 @@ class _RowCompiler(_MapCompiler):
                 flag = (0x100 if t.dtype_name == "float16" else 0) if mdiv else 0
                 if sb is not None:
                     self.emit(a, out)
-                    out.append((fwd + "_red", sb | flag, 0.0))
+                    out.append((fwd + "_red", sb | flag | self._form(t), 0.0))
                 else:
                     self.emit(b, out)
-                    out.append((rev + "_red", sa | flag, 0.0))
+                    out.append((rev + "_red", sa | flag | self._form(t, fwd == rev), 0.0))
                 if t.dtype_name == "float16" and t.op not in _MAP_EXACT and not mdiv:
                     out.append(("r16", 0, 0.0))
                 if self.masked and t.attrs.get("pow"):
@@ -1507,6 +1602,11 @@ def match_rows(dst_view, value, n_groups):
     if not per_row and value.shape != (rows, n):
         return None
     if per_row:
+        # A per-row result is a bare numpy.ma array: every row is written, a
+        # deactivated one with what numpy.ma left in it, which the stages that
+        # compute with row scalars reproduce (the tile operators leave their
+        # first operand's value, NumPy functions compute regardless; the
+        # instructions say which is which).
         comp.prepare(value, True)
         slot = comp.slot_of(value)
         program = [("red", slot, 0.0)] if slot is not None else comp.program(value, scalar=True)
@@ -1514,6 +1614,10 @@ def match_rows(dst_view, value, n_groups):
     else:
         program = comp.program(value)
         if value.attrs.get("plain") and _maybe_masked(value):
+            if not _values_flow_plainly(value, finite=True):
+                raise NoNativeKernel("the stored value is a bare numpy.ma array, written in full, and "
+                                     "a tile operator follows an operation that can deactivate "
+                                     "elements: what numpy.ma leaves in those has no native code here")
             program.append(("clear", 0, 0.0))  # a bare numpy.ma array: every value is written
         comp.stages.append(("store", 0, program))
     if len(comp.stages) > rt.ROW_MAX_STAGES:
@@ -1662,6 +1766,15 @@ def _compile_col_reduce(red: Tile, root: Tile, n_groups, temps):
     if red.op in ("sum", "norm") and body.dtype_name != "float32":
         raise NoNativeKernel("column sums are computed in float32: cast the tile with "
                              ".astype(np.float32) before adding it up")
+    if red.op == "norm" and _maybe_masked(red.args[0]):
+        raise NoNativeKernel("numpy.linalg.norm of a tile whose elements a division or a domain "
+                             "function may deactivate: the norm adds up what such elements hold, "
+                             "which has no native code (use (x * x).sum(axis=0) for the active ones)")
+    if root is not red and red.op != "sum" and _maybe_masked(red.args[0]):
+        # a maximum / minimum over no active element is deactivated and holds
+        # numpy.ma's fill value: the kernel stores that, but computes nothing from it
+        raise NoNativeKernel(f"arithmetic on the {red.op} down the columns of an expression whose "
+                             "elements may be deactivated has no native code (the fold itself has)")
     comp = _ColBodyCompiler(n_groups, temps)
     if _const(body) or not comp.supported(body):
         raise NoNativeKernel(f"{body!r} is not an elementwise expression of float32 / float16 "
@@ -1693,6 +1806,17 @@ def _compile_col_reduce(red: Tile, root: Tile, n_groups, temps):
     return kind, program, post, comp
 
 
+def _no_fold_read_back_if_it_can_be_deactivated(red: Tile):
+    """A fold down a column whose elements are all inactive is deactivated, and
+    so is everything computed from it; the temporary vectors of the column
+    kernels carry values only."""
+    if _can_fail(red.args[0], finite=True):
+        raise NoNativeKernel("an expression reads back a reduction down the columns of elements that "
+                             "a zero divisor or a domain function may deactivate: a column without "
+                             "active elements would have to deactivate what is computed from it, "
+                             "which has no native code (reductions along rows have)")
+
+
 def match_cols(dst_view, value, n_groups):
     """value = post(reduce(f(tiles...), axis=0)): sums, maxima, minima, means,
     variances, standard deviations and 2-norms down the columns of (rows, N)
@@ -1710,6 +1834,8 @@ def match_cols(dst_view, value, n_groups):
             t = t.args[0]
         elif t.op in _MAP_BINARY and len(t.args) == 2 and _const(t.args[0]) != _const(t.args[1]):
             t = t.args[0] if _const(t.args[1]) else t.args[1]
+        elif _is(t, "vardiv", 2) and _const(t.args[1]):
+            t = t.args[0]
         else:
             return None
     outer = t
@@ -1730,6 +1856,7 @@ def match_cols(dst_view, value, n_groups):
     inner(outer.args[0])
     temps, steps = {}, []
     for red in order:
+        _no_fold_read_back_if_it_can_be_deactivated(red)
         steps.append(_compile_col_reduce(red, red, n_groups, dict(temps)))
         temps[red.uid] = len(temps)
     steps.append(_compile_col_reduce(outer, value, n_groups, dict(temps)))
@@ -1813,6 +1940,7 @@ def match_cols_tile(dst_view, value, n_groups):
         return None
     temps, steps = {}, []
     for red in order:
+        _no_fold_read_back_if_it_can_be_deactivated(red)
         steps.append(_compile_col_reduce(red, red, n_groups, dict(temps)))
         temps[red.uid] = len(temps)
     final = _ColBodyCompiler(n_groups, dict(temps))
@@ -1825,6 +1953,10 @@ def match_cols_tile(dst_view, value, n_groups):
     program: list = []
     final.emit_whole(value, program)
     if value.attrs.get("plain") and _maybe_masked(value):
+        if not _values_flow_plainly(value, finite=True):
+            raise NoNativeKernel("the stored value is a bare numpy.ma array, written in full, and a "
+                                 "tile operator follows an operation that can deactivate elements: "
+                                 "what numpy.ma leaves in those has no native code here")
         program.append(("clear", 0, 0.0))      # a bare numpy.ma array: every value is written
     if len(program) > rt.MAP_MAX_INSTRS or len(final.inputs) > rt.MAP_MAX_INPUTS:
         raise NoNativeKernel(f"the stored expression compiles to {len(program)} operations on "
@@ -2113,6 +2245,17 @@ def simplify(t: Tile, memo=None) -> Tile:
     folded = _assembled_reduce(out)
     if folded is not None:
         out = folded
+    if out.op == "count" and _is_reduction(out) and not _maybe_masked(out.args[0]):
+        # nothing can deactivate an element: the number of active elements is the
+        # number of elements (tiles hold whole rows / columns of their arrays)
+        n = math.prod(out.args[0].shape[a] for a in out.attrs["axes"])
+        out = Tile("const", (), (), "float32", value=float(n), weak=False, exact=n, counted=True)
+    elif out.op == "sub" and len(out.args) == 2 and out.args[0].attrs.get("counted") and \
+            _is(out.args[1], "const"):
+        n = out.args[0].attrs["value"] - out.args[1].attrs["value"]       # count - ddof
+        if n <= 0:
+            raise NoNativeKernel("var/std with ddof: fewer than ddof + 1 elements")
+        out = Tile("const", (), (), "float32", value=float(n), weak=False, exact=int(n), counted=True)
     memo[id(t)] = out
     return out
 

@@ -1128,6 +1128,7 @@ struct ColArgs {
   uint32_t out_vec;     // the result may be written 16 bytes at a time
   uint32_t n_post;
   uint32_t masked;      // the program has numpy.ma's division / domain forms: inactive elements are left out
+  uint32_t fill_empty;  // finishing launch of a maximum / minimum: the identity (no active element) becomes 1e20
   Instr post[kPostProg];
 };
 
@@ -1471,6 +1472,11 @@ __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, 
     }
     return;
   }
+  if (c.fill_empty) { // uniform
+#pragma unroll
+    for (int e = 0; e < kN; ++e)
+      acc[e] = acc[e] == identity ? 1e20f : acc[e];
+  }
   if (c.n_post) {
 #pragma unroll
     for (int e = 0; e < kN; ++e)
@@ -1549,15 +1555,25 @@ enum : uint32_t {
   OP_RDIV_RED = 53,
   OP_MDIV_RED = 54,  // top / row scalar and row scalar / top under numpy.ma's rule
   OP_RMDIV_RED = 55, // (`arg` bits 0..3: the scalar, bit 8: fp16)
+  OP_RED0 = 56,      // push row scalar `arg` as a value, deactivated or not
+  OP_MASQRT = 57,    // numpy.ma.sqrt (scalar stages): not finite or x < 0 deactivates, value x
 };
-enum : uint32_t { ST_SUM = 0, ST_MAX = 1, ST_MIN = 2, ST_SCALAR = 3, ST_STORE = 4, ST_STORE_COL = 5 };
+// flags in `arg` of the instructions of scalar stages (beside bit 8, fp16)
+constexpr uint32_t kFuncForm = 0x200; // called as a NumPy function: computed on the values, deactivated or not
+constexpr uint32_t kSwapped = 0x400;  // commutative operation whose running value is the second operand
+enum : uint32_t {
+  ST_SUM = 0, ST_MAX = 1, ST_MIN = 2, ST_SCALAR = 3, ST_STORE = 4, ST_STORE_COL = 5,
+  ST_COUNT = 6 // the number of active elements of the program's value, as fp32
+};
 
 struct Stage {
   uint16_t begin, end; // instructions [begin, end)
   uint8_t kind, dst;
   uint8_t load_mask; // operands this stage reads
-  uint8_t masked;    // the program has numpy.ma's division / domain forms: honour the inactive bits
-  uint8_t pad[4];
+  uint8_t masked;    // honour the inactive bits: numpy.ma's forms, or a row scalar read that may be deactivated
+  uint16_t red_mask; // row scalars this stage reads that may be deactivated
+  uint8_t live_pos;  // scalar stages: the result is active iff this row scalar is positive (0xff: not used)
+  uint8_t pad;
 };
 
 struct RowArgs {
@@ -1611,11 +1627,11 @@ __device__ __forceinline__ void run_stage(const RowArgs &a, uint32_t begin, uint
     // into the dispatch below and tear its arms apart.
     uint32_t op = cur.op;
     uint32_t imm_bits = __builtin_bit_cast(uint32_t, cur.imm);
-    if (op >= OP_RED) {
+    if (op >= OP_RED && op <= OP_RED0) {
       imm_bits = __builtin_amdgcn_readlane(reds, arg & (kMaxRed - 1));
-      op = op == OP_RED        ? (uint32_t)OP_CONST
-           : op >= OP_MDIV_RED ? op - OP_MDIV_RED + OP_MDIVI
-                               : op - OP_ADD_RED + OP_ADDI;
+      op = (op == OP_RED || op == OP_RED0) ? (uint32_t)OP_CONST
+           : op >= OP_MDIV_RED             ? op - OP_MDIV_RED + OP_MDIVI
+                                           : op - OP_ADD_RED + OP_ADDI;
     }
     asm volatile("" : "+s"(op), "+s"(imm_bits));
     const float imm = __builtin_bit_cast(float, imm_bits);
@@ -1630,6 +1646,168 @@ __device__ __forceinline__ void run_stage(const RowArgs &a, uint32_t begin, uint
     default: asm volatile("; stack depth 4"); sp = step<4>(r, raw, a.f16_mask, op, arg, imm); break;
     }
   }
+}
+
+// A stage that computes with row scalars only (SCALAR, STORE_COL), as numpy.ma
+// computes on values that may be deactivated: every stack entry is a value and a
+// "deactivated" bit.  The tile operators + - * leave their first operand's value
+// in a deactivated result, the quotient leaves the dividend's, NumPy functions
+// compute on the values regardless (numpy.sqrt and numpy.log put their fill value
+// where the domain fails or the argument is deactivated already).  What a
+// deactivated row scalar holds matters where it is stored all the same (a per-row
+// result is a bare numpy.ma array, written in full) and where a variance reads a
+// sum whose terms were all inactive.  Everything here is uniform over the lanes
+// of a row.  `dead`: bit k = row scalar k is deactivated.
+struct ScalarResult {
+  float value;
+  bool dead;
+};
+__device__ __forceinline__ ScalarResult run_scalar_stage(const RowArgs &a, uint32_t begin, uint32_t end,
+                                                         const float *cells, uint32_t dead) {
+  float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+  uint32_t dbits = 0; // bit i: stack entry i is deactivated
+  int sp = 0;
+  auto get = [&](int i) { return i == 0 ? s0 : i == 1 ? s1 : i == 2 ? s2 : s3; };
+  auto put = [&](int i, float v, bool d) {
+    s0 = i == 0 ? v : s0;
+    s1 = i == 1 ? v : s1;
+    s2 = i == 2 ? v : s2;
+    s3 = i == 3 ? v : s3;
+    dbits = (dbits & ~(1u << i)) | (d ? 1u << i : 0u);
+  };
+#pragma nounroll
+  for (uint32_t pc = begin; pc < end; ++pc) {
+    const Instr cur = a.prog[pc & (kRowProg - 1)];
+    const uint32_t op = cur.op, arg = cur.arg;
+    const uint32_t slot = arg & (kMaxRed - 1);
+    if (op == OP_CONST) {
+      put(sp++, cur.imm, false);
+      continue;
+    }
+    if (op == OP_RED || op == OP_RED0) {
+      put(sp++, cells[slot], op == OP_RED && ((dead >> slot) & 1u));
+      continue;
+    }
+    const bool is_unary = (op >= OP_NEG && op <= OP_R16) || op == OP_POWCHK || op == OP_MSQRT ||
+                          op == OP_MLOG || op == OP_MASQRT;
+    if (is_unary) {
+      if (sp < 1)
+        continue;
+      const float v = get(sp - 1);
+      bool d = (dbits >> (sp - 1)) & 1u;
+      float y;
+      switch (op) {
+      case OP_NEG: y = -v; break;
+      case OP_ABS: y = __builtin_fabsf(v); break;
+      case OP_SQRT: y = __builtin_sqrtf(v); break;
+      case OP_RINT: y = __builtin_rintf(v); break;
+      case OP_EXP: y = expf(v); break;
+      case OP_LOG: y = logf(v); break;
+      case OP_TANH: y = tanh_selects(v); break;
+      case OP_R16: y = round16(v); break;
+      case OP_MSQRT: {
+        const bool out = d || v < 0.0f;
+        y = out ? 0.0f : __builtin_sqrtf(v);
+        d = out;
+        break;
+      }
+      case OP_MLOG: {
+        const bool out = d || v <= 0.0f;
+        y = out ? 1.0f : logf(v);
+        d = out;
+        break;
+      }
+      case OP_MASQRT: {
+        const float r = __builtin_sqrtf(v);
+        const bool out = d || !is_finite(r) || v < 0.0f;
+        y = out ? v : r;
+        d = out;
+        break;
+      }
+      default: { // OP_POWCHK
+        const bool out = !is_finite(v);
+        y = out ? 1e20f : v;
+        d = d || out;
+        break;
+      }
+      }
+      put(sp - 1, y, d);
+      continue;
+    }
+    // binary: two stack entries, or the top and an immediate / a row scalar
+    uint32_t base; // OP_ADD .. OP_RDIV, OP_MDIV, OP_RMDIV
+    float other = 0.0f;
+    bool other_dead = false;
+    int at; // where the running value is and the result goes
+    bool half = (arg & 0x100u) != 0; // the quotient is rounded to fp16 before it is tested
+    if ((op >= OP_ADD && op <= OP_RDIV) || op == OP_MDIV || op == OP_RMDIV) {
+      if (sp < 2)
+        continue;
+      base = op;
+      half = (arg & 0x1ffu) != 0;
+      other = get(sp - 1);
+      other_dead = (dbits >> (sp - 1)) & 1u;
+      at = sp - 2;
+      --sp;
+    } else {
+      if (sp < 1)
+        continue;
+      at = sp - 1;
+      if (op >= OP_ADDI && op <= OP_RDIVI) {
+        base = op - OP_ADDI + OP_ADD;
+        other = cur.imm;
+      } else if (op == OP_MDIVI || op == OP_RMDIVI) {
+        base = op - OP_MDIVI + OP_MDIV;
+        other = cur.imm;
+      } else if (op >= OP_ADD_RED && op <= OP_RDIV_RED) {
+        base = op - OP_ADD_RED + OP_ADD;
+        other = cells[slot];
+        other_dead = (dead >> slot) & 1u;
+      } else if (op == OP_MDIV_RED || op == OP_RMDIV_RED) {
+        base = op - OP_MDIV_RED + OP_MDIV;
+        other = cells[slot];
+        other_dead = (dead >> slot) & 1u;
+      } else {
+        continue; // nothing else is valid here (the host has checked)
+      }
+    }
+    float lv = get(at), rv = other; // first and second operand
+    bool ld = (dbits >> at) & 1u, rd = other_dead;
+    const bool reversed = base == OP_RSUB || base == OP_RDIV || base == OP_RMDIV;
+    if (reversed || (arg & kSwapped)) {
+      const float tv = lv;
+      lv = rv, rv = tv;
+      const bool td = ld;
+      ld = rd, rd = td;
+    }
+    const bool gone = ld || rd;
+    float y;
+    bool d = gone;
+    if (base == OP_MDIV || base == OP_RMDIV) {
+      float q = lv / rv;
+      if (half)
+        q = round16(q);
+      const bool good = is_finite(q) && !gone;
+      y = good ? q + 0.0f * lv : 0.0f + lv;
+      d = !good;
+    } else {
+      switch (base) {
+      case OP_ADD: y = lv + rv; break;
+      case OP_SUB:
+      case OP_RSUB: y = lv - rv; break;
+      case OP_MUL: y = lv * rv; break;
+      case OP_DIV:
+      case OP_RDIV: y = lv / rv; break;
+      case OP_MAX: y = nan_max(lv, rv); break;
+      default: y = nan_min(lv, rv); break;
+      }
+      const bool keeps_first = !(arg & kFuncForm) &&
+                               (base == OP_ADD || base == OP_SUB || base == OP_RSUB || base == OP_MUL);
+      y = gone && keeps_first ? lv : y;
+    }
+    put(at, y, d);
+  }
+  return ScalarResult{s0, (dbits & 1u) != 0};
 }
 
 // Where a lane stands in its row during pass p.
@@ -1746,35 +1924,51 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
   char *const orow = static_cast<char *>(a.out) + row * a.ldo * (out_f16 ? 2 : 4);
 
   uint32_t parity = 0;
+  uint32_t dead = 0; // bit k: row scalar k is deactivated (the same in every lane of a row)
 #pragma nounroll
   for (uint32_t s = 0; s < a.n_stages; ++s) {
     const Stage st = a.stage[s];
     const uint32_t kind = st.kind;
-    const bool per_element = kind <= ST_MIN || kind == ST_STORE;
-    const uint32_t n_pass = per_element ? a.passes : 1;
+    if (kind == ST_SCALAR || kind == ST_STORE_COL) {
+      ScalarResult res = run_scalar_stage(a, st.begin, st.end, cells, dead);
+      if (st.live_pos != 0xff)
+        res.dead = !(cells[st.live_pos & (kMaxRed - 1)] > 0.0f);
+      if (kind == ST_SCALAR) {
+        const uint32_t bit = 1u << (st.dst & (kMaxRed - 1));
+        cells[st.dst & (kMaxRed - 1)] = uniform(res.value);
+        dead = res.dead ? dead | bit : dead & ~bit;
+      } else if (row_live && lane == 0) {
+        store_elem(a.out, out_f16, row * a.ldo, res.value);
+      }
+      continue;
+    }
+    const uint32_t n_pass = a.passes;
+    // every element of a stage that reads a deactivated row scalar is inactive
+    const bool row_gone = (dead & st.red_mask) != 0;
     // the row scalars, scalar k in lane k
     const uint32_t reds = __builtin_bit_cast(uint32_t, cells[t & (kMaxRed - 1)]);
     float acc = kind == ST_MAX ? -INFINITY : kind == ST_MIN ? INFINITY : 0.0f;
+    float taken = 0.0f; // active elements folded (stages that honour the inactive bits)
     StackT<kRowN> r;
 #pragma nounroll
     for (uint32_t p = 0; p < n_pass; ++p) {
-      const Place at = per_element ? place(p) : Place{0u, 1u, 0u};
+      const Place at = place(p);
       RawT<kRowN> raw;
-      if (per_element) {
 #pragma unroll
-        for (int i = 0; i < kMaxIn; ++i) {
-          if ((st.load_mask >> i) & 1) {
-            load_chunk(a, i, bases[i], at, raw.w[i]);
-          }
+      for (int i = 0; i < kMaxIn; ++i) {
+        if ((st.load_mask >> i) & 1) {
+          load_chunk(a, i, bases[i], at, raw.w[i]);
         }
       }
       run_stage(a, st.begin, st.end, raw, r, reds);
       // a wave whose lanes all hold whole chunks folds them without masks
       const bool all_whole = __builtin_amdgcn_ballot_w64(at.n_valid != kRowN) == 0;
-      if (st.masked && per_element) {
-        // a stage with numpy.ma's forms (uniform: the host marks it): elements
-        // that a division or a domain function deactivated are neither stored
-        // nor folded
+      if (st.masked) {
+        // a stage with numpy.ma's forms, or one that reads a row scalar that may
+        // be deactivated (uniform: the host marks it): elements that a division
+        // or a domain function deactivated are neither stored nor folded
+        if (row_gone)
+          r.bad = ~0u;
         const bool whole_chunk = kind == ST_STORE && ((a.vec_mask >> 8) & 1) && at.n_valid == kRowN &&
                                  r.bad == 0;
         if (whole_chunk) {
@@ -1792,9 +1986,10 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
             acc += take ? r.st[0][e] : 0.0f;
           } else if (kind == ST_MAX) {
             acc = take ? nan_max(acc, r.st[0][e]) : acc;
-          } else {
+          } else if (kind == ST_MIN) {
             acc = take ? nan_min(acc, r.st[0][e]) : acc;
           }
+          taken += take ? 1.0f : 0.0f;
         }
       } else if (kind == ST_STORE) {
         if (((a.vec_mask >> 8) & 1) && at.n_valid == kRowN) {
@@ -1837,24 +2032,32 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
           for (int e = 0; e < kRowN; ++e)
             acc = (uint32_t)e < at.n_valid ? nan_min(acc, r.st[0][e]) : acc;
         }
+      } else if (kind == ST_COUNT) {
+        taken += (float)at.n_valid; // nothing can be inactive but what lies past the row's end
       }
     }
-    if (kind <= ST_MIN) {
+    if (kind <= ST_MIN || kind == ST_COUNT) {
       constexpr int W = LPR / kWave;
       float total;
-      if (kind == ST_SUM)
-        total = group_reduce<SumOp, W>(acc, slots[parity]);
-      else if (kind == ST_MAX)
+      if (kind == ST_MAX)
         total = group_reduce<NanMaxOp, W>(acc, slots[parity]);
-      else
+      else if (kind == ST_MIN)
         total = group_reduce<NanMinOp, W>(acc, slots[parity]);
+      else
+        total = group_reduce<SumOp, W>(kind == ST_COUNT ? taken : acc, slots[parity]);
       parity ^= 1;
+      const uint32_t bit = 1u << (st.dst & (kMaxRed - 1));
+      if (st.masked && kind != ST_COUNT) {
+        // a fold over no active element at all is deactivated, and holds what
+        // numpy.ma leaves there: 0 for a sum, its fill value for a maximum or minimum
+        const bool none = group_reduce<SumOp, W>(taken, slots[parity]) == 0.0f;
+        parity ^= 1;
+        total = none ? (kind == ST_SUM ? 0.0f : 1e20f) : total;
+        dead = none ? dead | bit : dead & ~bit;
+      } else {
+        dead &= ~bit;
+      }
       cells[st.dst & (kMaxRed - 1)] = total;
-    } else if (kind == ST_SCALAR) {
-      cells[st.dst & (kMaxRed - 1)] = uniform(r.st[0][0]);
-    } else if (kind == ST_STORE_COL) {
-      if (row_live && lane == 0)
-        store_elem(a.out, out_f16, row * a.ldo, r.st[0][0]);
     }
   }
 }
@@ -2183,10 +2386,10 @@ HCAMD_ROW_CHAIN(512, 4, 512)
 HCAMD_ROW_CHAIN(1024, 4, 1024)
 
 // ---- layer normalisation without the interpreter -----------------------------------
-// The five-stage row program  mean = sum(x) / n;  s = sqrt(sum((x - mean) *
-// (x - mean)) / n + eps);  out = (x - mean) / s * w + b  (the division
-// numpy.ma's, as the front-end emits it for a body written with mean and var
-// along axis 1) on dense fp32 rows, with the same operations in the same order
+// The six-stage row program  mean = sum(x) / n;  var = sum((x - mean) *
+// (x - mean)) / n;  s = sqrt(var + eps);  out = (x - mean) / s * w + b  (the
+// mean's division and the last one numpy.ma's, as the front-end emits it for a
+// body written with mean and var along axis 1) on dense fp32 rows, with the same operations in the same order
 // per element as the interpreter performs them (every product and sum rounded
 // on its own, a true division, elements whose quotient is not finite left
 // unstored); only the order in which a row's terms are added differs.  LPR lanes
@@ -2255,8 +2458,12 @@ __device__ __forceinline__ void layer_norm_rows(const void *__restrict__ x, size
       }
     }
   }
-  const float s = __builtin_sqrtf(__fadd_rn(group_reduce<SumOp, W>(acc, slots[1][sub]) / n, eps));
-  if (!live)
+  const float mean_sq = group_reduce<SumOp, W>(acc, slots[1][sub]) / n;
+  const float s = __builtin_sqrtf(__fadd_rn(mean_sq, eps));
+  // The mean is numpy.ma's quotient: one that is not finite is deactivated, and
+  // with it every element computed from it (the variance of such a row is an
+  // active 0, but the row's x - mean are all inactive).
+  if (!live || !is_finite(RMS ? mean_sq : mean))
     return;
   char *orow = static_cast<char *>(out) + (size_t)row * ldo * (HALF ? 2 : 4);
 #pragma unroll

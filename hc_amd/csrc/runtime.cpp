@@ -1681,6 +1681,7 @@ namespace {
 struct ColArgs {
   float *partial;
   uint32_t colsPad, band, kind, lanes, interleaved, outVec, nPost, masked;
+  uint32_t fillEmpty; // the finishing launch: a maximum / minimum over no active element is 1e20
   HcamdMapInstr post[HCAMD_COLS_MAX_POST];
 };
 
@@ -1865,6 +1866,12 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
     ca.nPost = static_cast<uint32_t>(nPost);
     if (nPost)
       std::memcpy(ca.post, post, nPost * sizeof(HcamdMapInstr));
+    // numpy.ma's maximum / minimum of a column without an active element is
+    // deactivated and holds its fill value, which is what a per-column result,
+    // a bare numpy.ma array written in full, then stores.  (The fold's identity
+    // stands for "no active element": a column whose active values are all
+    // -inf (+inf) is taken for an empty one.)
+    ca.fillEmpty = c.masked && kind != HCAMD_COLS_SUM ? 1u : 0u;
   };
   a.rows = rows;
   a.cols = cols;
@@ -1973,8 +1980,10 @@ namespace {
 struct RowStageDev {
   uint16_t begin, end;
   uint8_t kind, dst, loadMask;
-  uint8_t masked; // the stage has numpy.ma's division / domain forms
-  uint8_t pad[4];
+  uint8_t masked;   // honour the inactive bits: numpy.ma's forms, or a row scalar read that may be deactivated
+  uint16_t redMask; // row scalars this stage reads that may be deactivated
+  uint8_t livePos;  // scalar stages: the result is active iff this row scalar is positive (0xff: not used)
+  uint8_t pad;
 };
 struct RowArgs {
   const void *in[kMapMaxIn];
@@ -2069,13 +2078,18 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
   }
   RowArgs a{};
   // Every stage must keep the stack within bounds, leave one value, and read
-  // only operands that exist and row scalars that have been written.
+  // only operands that exist and row scalars that have been written.  Along
+  // the way: which row scalars the data can deactivate (a fold over elements
+  // that numpy.ma's forms can deactivate, a scalar stage with such a form, and
+  // everything computed from one of those), and which stages read them.
   uint32_t written = (1u << nColumns) - 1u;
+  uint32_t deadable = 0;
+  bool tracking = false; // some row scalar may be deactivated, or active elements are counted
   uint32_t usedIn[HCAMD_ROW_MAX_STAGES] = {};
   size_t pc = 0;
   for (size_t s = 0; s < nStages; ++s) {
     const HcamdRowStage &st = stages[s];
-    if (st.kind > HCAMD_ROW_STORE_COL || st.nInstr == 0 ||
+    if (st.kind > HCAMD_ROW_COUNT || st.nInstr == 0 ||
         pc + st.nInstr > HCAMD_ROW_MAX_INSTRS) {
       dev->report("%s: stage %zu: kind %u with %u instructions (%d in all allowed)", who,
                   s, st.kind, st.nInstr, HCAMD_ROW_MAX_INSTRS);
@@ -2086,26 +2100,41 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       dev->report("%s: the last stage, and only the last, must store", who);
       return 1;
     }
-    const bool perElement = st.kind <= HCAMD_ROW_MIN || st.kind == HCAMD_ROW_STORE;
+    const bool perElement = !(st.kind == HCAMD_ROW_SCALAR || st.kind == HCAMD_ROW_STORE_COL);
     if (!stores && st.dst >= HCAMD_ROW_MAX_SCALARS) {
       dev->report("%s: stage %zu writes row scalar %u (%d exist)", who, s, st.dst,
                   HCAMD_ROW_MAX_SCALARS);
       return 1;
     }
     int sp = 0;
-    for (size_t i = pc; i < pc + st.nInstr; ++i) {
+    bool hasForms = false;
+    uint32_t readsDeadable = 0;
+    a.stage[s].livePos = 0xff;
+    size_t stageEnd = pc + st.nInstr;
+    if (prog[stageEnd - 1].op == HCAMD_MAP_LIVEPOS) {
+      const unsigned index = prog[stageEnd - 1].arg & 0xffu;
+      if (perElement || st.nInstr < 2 || index >= HCAMD_ROW_MAX_SCALARS || !((written >> index) & 1)) {
+        dev->report("%s: stage %zu: LIVEPOS closes a scalar stage and names a row scalar that "
+                    "has been written", who, s);
+        return 1;
+      }
+      a.stage[s].livePos = static_cast<uint8_t>(index);
+      --stageEnd;
+    }
+    for (size_t i = pc; i < stageEnd; ++i) {
       const unsigned op = prog[i].op;
       int pops, pushes;
       const bool maskedRed = op == HCAMD_MAP_MDIV_RED || op == HCAMD_MAP_RMDIV_RED;
-      if ((op >= HCAMD_MAP_MDIV && op <= HCAMD_MAP_MLOG && op != HCAMD_MAP_CLEAR) || maskedRed)
-        a.stage[s].masked = 1;
-      const bool red = op >= HCAMD_MAP_RED && op <= HCAMD_MAP_RMDIV_RED;
+      if ((op >= HCAMD_MAP_MDIV && op <= HCAMD_MAP_MLOG && op != HCAMD_MAP_CLEAR) || maskedRed ||
+          op == HCAMD_MAP_MASQRT)
+        hasForms = true;
+      const bool red = op >= HCAMD_MAP_RED && op <= HCAMD_MAP_RED0;
       if (red)
-        pops = op == HCAMD_MAP_RED ? 0 : 1, pushes = 1;
-      else if (perElement)
-        mapStackEffectMasked(op, pops, pushes); // numpy.ma's division forms: element-wise stages only
+        pops = (op == HCAMD_MAP_RED || op == HCAMD_MAP_RED0) ? 0 : 1, pushes = 1;
+      else if (op == HCAMD_MAP_MASQRT && !perElement)
+        pops = 1, pushes = 1;
       else
-        mapStackEffect(op, pops, pushes);
+        mapStackEffectMasked(op, pops, pushes);
       if (pops < 0) {
         dev->report("%s: unknown opcode %u at %zu", who, op, i);
         return 1;
@@ -2113,7 +2142,8 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       const bool maskedIn = op == HCAMD_MAP_MDIV_IN || op == HCAMD_MAP_RMDIV_IN;
       const bool readsOperand = op == HCAMD_MAP_IN || maskedIn ||
                                 (op >= HCAMD_MAP_ADD_IN && op <= HCAMD_MAP_RDIV_IN);
-      const unsigned index = (maskedIn || maskedRed) ? prog[i].arg & 0xffu : prog[i].arg;
+      // (bits 8 and up of `arg` are flags: fp16, and in scalar stages the form of the operation)
+      const unsigned index = (maskedIn || red) ? prog[i].arg & 0xffu : prog[i].arg;
       if (readsOperand) {
         if (!perElement || index >= nInputs) {
           dev->report("%s: operand %u at %zu (%zu given; scalar stages read none)", who,
@@ -2122,14 +2152,20 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
         }
         usedIn[s] |= 1u << index;
       }
-      if (maskedRed && !perElement) {
-        dev->report("%s: opcode %u at %zu in a scalar stage", who, op, i);
+      if (op == HCAMD_MAP_RED0 && perElement) {
+        dev->report("%s: opcode %u at %zu outside a scalar stage", who, op, i);
+        return 1;
+      }
+      if (perElement && !red && !maskedIn && (prog[i].arg & ~0x1ffu)) {
+        dev->report("%s: flags 0x%x at %zu outside a scalar stage", who, prog[i].arg, i);
         return 1;
       }
       if (red && (index >= HCAMD_ROW_MAX_SCALARS || !((written >> index) & 1))) {
         dev->report("%s: row scalar %u read at %zu before it is written", who, index, i);
         return 1;
       }
+      if (red && op != HCAMD_MAP_RED0)
+        readsDeadable |= (1u << index) & deadable;
       if (sp < pops) {
         dev->report("%s: stack underflow at %zu", who, i);
         return 1;
@@ -2145,11 +2181,20 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       return 1;
     }
     a.stage[s].begin = static_cast<uint16_t>(pc);
-    a.stage[s].end = static_cast<uint16_t>(pc + st.nInstr);
+    a.stage[s].end = static_cast<uint16_t>(stageEnd);
     a.stage[s].kind = static_cast<uint8_t>(st.kind);
     a.stage[s].dst = static_cast<uint8_t>(st.dst);
-    if (!stores)
+    a.stage[s].redMask = static_cast<uint16_t>(readsDeadable);
+    a.stage[s].masked = (hasForms || readsDeadable) ? 1 : 0;
+    const bool canDie = (stores || st.kind == HCAMD_ROW_COUNT) ? false
+                        : perElement                           ? (hasForms || readsDeadable)
+                                                   : (hasForms || readsDeadable || a.stage[s].livePos != 0xff);
+    if (!stores) {
       written |= 1u << st.dst;
+      deadable = canDie ? deadable | (1u << st.dst) : deadable & ~(1u << st.dst);
+    }
+    // (a STORE_COL stage that can fail stores what numpy.ma leaves: the scalar interpreter's business too)
+    tracking = tracking || canDie || st.kind == HCAMD_ROW_COUNT || (!perElement && (hasForms || readsDeadable));
     pc += st.nInstr;
   }
   std::memcpy(a.prog, prog, pc * sizeof(HcamdMapInstr));
@@ -2228,11 +2273,12 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
     a.interleaved = 1;
   }
   // A layer normalisation as the front-end emits it for a body written with
-  // mean and var along axis 1 (five stages: the mean, the centred squares, the
-  // scale, then (x - mean) / s * w + b with numpy.ma's division), on dense fp32
-  // rows of at most 32768 elements with fp32 vectors w and b: a kernel that
-  // interprets nothing (variant 2 of "rows": the chain kernels for this too;
-  // variant 1: the general kernel for everything).
+  // mean and var along axis 1 (six stages: the mean, the centred squares, the
+  // variance, the scale, then (x - mean) / s * w + b; the mean's division and the
+  // last one numpy.ma's), on dense fp32 rows of at most 32768 elements with
+  // fp32 vectors w and b: a kernel that interprets nothing, and stores nothing
+  // to a row whose mean is not finite, as the stages demand (variant 2 of
+  // "rows": the general kernel for this too; variant 1: for everything).
   {
     auto is = [&](size_t at, unsigned op, unsigned arg) {
       return prog[at].op == op && prog[at].arg == arg;
@@ -2261,29 +2307,33 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
              stages[s].nInstr == n;
     };
     const bool shape =
-        variantOf("rows") == 0 && nStages == 5 && nInputs == 3 && nColumns == 0 && pc == 17 &&
+        variantOf("rows") == 0 && nStages == 6 && nInputs == 3 && nColumns == 0 && pc == 18 &&
         stage(0, HCAMD_ROW_SUM, 0, 1) && stage(1, HCAMD_ROW_SCALAR, 1, 2) &&
-        stage(2, HCAMD_ROW_SUM, 2, 5) && stage(3, HCAMD_ROW_SCALAR, 3, 4) &&
-        stage(4, HCAMD_ROW_STORE, 0, 5);
-    if (shape && is(0, HCAMD_MAP_IN, 0) && is(1, HCAMD_MAP_RED, 0) && prog[2].op == HCAMD_MAP_DIVI &&
+        stage(2, HCAMD_ROW_SUM, 2, 5) && stage(3, HCAMD_ROW_SCALAR, 3, 2) &&
+        stage(4, HCAMD_ROW_SCALAR, 4, 3) && stage(5, HCAMD_ROW_STORE, 0, 5);
+    if (shape && is(0, HCAMD_MAP_IN, 0) && is(1, HCAMD_MAP_RED, 0) && is(2, HCAMD_MAP_MDIVI, 0) &&
         is(3, HCAMD_MAP_IN, 0) && is(4, HCAMD_MAP_SUB_RED, 1) && is(5, HCAMD_MAP_IN, 0) &&
-        is(6, HCAMD_MAP_SUB_RED, 1) && prog[7].op == HCAMD_MAP_MUL && is(8, HCAMD_MAP_RED, 2) &&
-        prog[9].op == HCAMD_MAP_DIVI && prog[10].op == HCAMD_MAP_ADDI &&
-        prog[11].op == HCAMD_MAP_SQRT && is(12, HCAMD_MAP_IN, 0) && is(13, HCAMD_MAP_SUB_RED, 1) &&
-        is(14, HCAMD_MAP_MDIV_RED, 3) && is(15, HCAMD_MAP_MUL_IN, 1) &&
-        is(16, HCAMD_MAP_ADD_IN, 2) && prog[2].imm == prog[9].imm && a.f16Mask == 0 &&
+        is(6, HCAMD_MAP_SUB_RED, 1) && is(7, HCAMD_MAP_MUL, 0) && is(8, HCAMD_MAP_RED0, 2) &&
+        is(9, HCAMD_MAP_DIVI, 0) && is(10, HCAMD_MAP_RED, 3) && is(11, HCAMD_MAP_ADDI, 0) &&
+        is(12, HCAMD_MAP_MSQRT, 0) && is(13, HCAMD_MAP_IN, 0) && is(14, HCAMD_MAP_SUB_RED, 1) &&
+        is(15, HCAMD_MAP_MDIV_RED, 4) && is(16, HCAMD_MAP_MUL_IN, 1) &&
+        is(17, HCAMD_MAP_ADD_IN, 2) && prog[2].imm == prog[9].imm && prog[11].imm >= 0.0f &&
+        a.f16Mask == 0 &&
         inputLd[0] != 0 && inputLd[1] == 0 && inputLd[2] == 0 && (a.vecMask & 0x107u) == 0x107u &&
         cols % 4 == 0 && cols <= 32768) {
-      return launchNorm(false, inputs[0], inputLd[0], inputs[1], inputs[2], prog[2].imm, prog[10].imm);
+      return launchNorm(false, inputs[0], inputLd[0], inputs[1], inputs[2], prog[2].imm, prog[11].imm);
     }
     // The root-mean-square normalisation  x / sqrt(mean(x * x) + eps) * w  in its
-    // three stages, under the same conditions.
+    // three stages, under the same conditions (a row whose mean of squares is not
+    // finite is left alone).
     const bool rms =
         variantOf("rows") == 0 && nStages == 3 && nInputs == 2 && nColumns == 0 && pc == 9 &&
         stage(0, HCAMD_ROW_SUM, 0, 2) && stage(1, HCAMD_ROW_SCALAR, 1, 4) &&
         stage(2, HCAMD_ROW_STORE, 0, 3);
-    if (rms && is(0, HCAMD_MAP_IN, 0) && is(1, HCAMD_MAP_MUL_IN, 0) && is(2, HCAMD_MAP_RED, 0) &&
-        prog[3].op == HCAMD_MAP_DIVI && prog[4].op == HCAMD_MAP_ADDI && prog[5].op == HCAMD_MAP_SQRT &&
+    const bool rmsScale = is(2, HCAMD_MAP_RED, 0) && is(3, HCAMD_MAP_MDIVI, 0) &&
+                          is(4, HCAMD_MAP_ADDI, 0) && is(5, HCAMD_MAP_MSQRT, 0) &&
+                          prog[4].imm >= 0.0f;
+    if (rms && is(0, HCAMD_MAP_IN, 0) && is(1, HCAMD_MAP_MUL_IN, 0) && rmsScale &&
         is(6, HCAMD_MAP_IN, 0) && is(7, HCAMD_MAP_MDIV_RED, 1) && is(8, HCAMD_MAP_MUL_IN, 1) &&
         a.f16Mask == 0 && inputLd[0] != 0 && inputLd[1] == 0 && (a.vecMask & 0x103u) == 0x103u &&
         cols % 4 == 0 && cols <= 32768)
@@ -2294,8 +2344,7 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
         variantOf("rows") == 0 && nStages == 3 && nInputs == 2 && nColumns == 0 && pc == 10 &&
         stage(0, HCAMD_ROW_SUM, 0, 2) && stage(1, HCAMD_ROW_SCALAR, 1, 4) &&
         stage(2, HCAMD_ROW_STORE, 0, 4);
-    if (rmsHalf && is(0, HCAMD_MAP_IN, 0) && is(1, HCAMD_MAP_MUL_IN, 0) && is(2, HCAMD_MAP_RED, 0) &&
-        prog[3].op == HCAMD_MAP_DIVI && prog[4].op == HCAMD_MAP_ADDI && prog[5].op == HCAMD_MAP_SQRT &&
+    if (rmsHalf && is(0, HCAMD_MAP_IN, 0) && is(1, HCAMD_MAP_MUL_IN, 0) && rmsScale &&
         is(6, HCAMD_MAP_IN, 0) && is(7, HCAMD_MAP_MDIV_RED, 1) && is(8, HCAMD_MAP_MUL_IN, 1) &&
         prog[9].op == HCAMD_MAP_R16 && a.f16Mask == 0x101u && inputLd[0] != 0 && inputLd[1] == 0 &&
         (a.vecMask & 0x103u) == 0x103u && cols % 8 == 0 && cols <= 65536)
@@ -2308,7 +2357,8 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
   // instructions read stays in LDS for the row (variant 1 of "rows": never).
   size_t lanes = lanesPerRow, maxGroups = SIZE_MAX, threads = 256;
   std::snprintf(name, sizeof name, "hcamd_row_program_w%zu", lanes);
-  if (variantOf("rows") != 1 && !a.interleaved && cols % 8 == 0 && perRow <= 4096 && nInputs > 0) {
+  if (variantOf("rows") != 1 && !tracking && !a.interleaved && cols % 8 == 0 && perRow <= 4096 &&
+      nInputs > 0) {
     HcamdMapInstr chained[HCAMD_ROW_MAX_INSTRS];
     size_t nChained = 0;
     uint16_t begin[HCAMD_ROW_MAX_STAGES], end[HCAMD_ROW_MAX_STAGES];

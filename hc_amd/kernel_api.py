@@ -787,9 +787,11 @@ class Tile:
                 return plain(x * x)
             return plain(Tile(op, (x,), x.shape, x.dtype_name))
         a, b = inputs
-        if isinstance(a, np.generic) and isinstance(b, Tile):
+        if isinstance(a, np.generic) and isinstance(b, Tile) and not b.attrs.get("plain"):
             # `np.float32(2) * tile`: the scalar's operator arrives here; it is the
-            # tile's reflected operator (which the reference's tile type lacks)
+            # tile's reflected operator (which the reference's tile type lacks).
+            # (Next to a bare numpy.ma array the scalar's operator is the NumPy
+            # function: computed on the values, deactivated or not.)
             refl = {"add": "__radd__", "sub": "__rsub__", "mul": "__rmul__", "div": "__rtruediv__",
                     "floordiv": "__rfloordiv__", "mod": "__rmod__", "lt": "__gt__", "le": "__ge__",
                     "gt": "__lt__", "ge": "__le__", "eq": "__eq__", "ne": "__ne__"}.get(op)
@@ -849,35 +851,53 @@ class Tile:
         axes = tuple(a % len(self.shape) for a in axes)
         shape = tuple((1 if i in axes else n) for i, n in enumerate(self.shape)) if keepdims \
             else tuple(n for i, n in enumerate(self.shape) if i not in axes)
-        return Tile(op, (self,), shape, self.dtype_name, axes=axes, keepdims=bool(keepdims))
+        # (plain: a reduction of a tile is a bare numpy.ma array, not a tile,
+        # python/hckernel/kernel_api.py:150-151)
+        return Tile(op, (self,), shape, self.dtype_name, axes=axes, keepdims=bool(keepdims), plain=True)
 
     def max(self, axis=None, keepdims=False): return self._reduce("max", axis, keepdims)
     def min(self, axis=None, keepdims=False): return self._reduce("min", axis, keepdims)
     def sum(self, axis=None, keepdims=False): return self._reduce("sum", axis, keepdims)
 
-    # mean, var and std are spelled out the way NumPy computes them
-    # (numpy/_core/_methods.py: _mean, _var), so that the host executor and the
-    # traced program round at the same places.
-    def _count(self, axis):
-        axes = range(len(self.shape)) if axis is None else \
-            ((axis,) if isinstance(axis, int) else axis)
-        return math.prod(self.shape[a % len(self.shape)] for a in axes)
+    # mean, var and std as numpy.ma computes them on a tile (numpy/ma/core.py:
+    # MaskedArray.mean / var / std; a tile's mask is always an array, so the
+    # masked branches run): the mean is the sum over the active elements divided
+    # by their number, a domained division that deactivates a result that is not
+    # finite; the variance divides the sum of the centred squares by that number
+    # less ddof and is active wherever that is positive, whatever the division
+    # did; the standard deviation is numpy.ma.sqrt of it.  `count` is a
+    # reduction node of its own (the number of active elements, as fp32);
+    # hc_amd.binding turns it into a constant where nothing can deactivate an
+    # element.
+    def _count(self, axis, keepdims):
+        r = self._reduce("count", axis, keepdims)
+        r.dtype_name = "float32"
+        return r
 
     def mean(self, axis=None, keepdims=False):
-        if self.dtype_name == "float16":        # NumPy adds up fp16 data in fp32
-            total = self.astype("float32")._reduce("sum", axis, keepdims)
-            return (total / self._count(axis)).astype("float16")
-        return self._reduce("sum", axis, keepdims) / self._count(axis)
+        half = self.dtype_name == "float16"     # NumPy adds up fp16 data in fp32
+        x = self.astype("float32") if half else self
+        if x.dtype_name != "float32":
+            raise TraceError("mean of a tile: float32 and float16 tiles only (cast first)")
+        total = x._reduce("sum", axis, keepdims)
+        r = Tile("div", (total, x._count(axis, keepdims)), total.shape, "float32", ma=True, plain=True)
+        return r.astype("float16") if half else r
 
     def var(self, axis=None, keepdims=False, ddof=0):
         if self.dtype_name != "float32":
             raise TraceError("var/std of a tile: float32 tiles only (cast first)")
-        centred = self - self._reduce("sum", axis, True) / self._count(axis)
-        return (centred * centred)._reduce("sum", axis, keepdims) / max(self._count(axis) - ddof, 0)
+        if not isinstance(ddof, (int, np.integer)) or ddof < 0:
+            raise TraceError("var/std of a tile: ddof must be a non-negative integer")
+        centred = self - self.mean(axis, True)
+        total = (centred * centred)._reduce("sum", axis, keepdims)
+        count = self._count(axis, keepdims)
+        if ddof:
+            count = count - np.float32(ddof)
+        return Tile("vardiv", (total, count), total.shape, "float32", plain=True)
 
     def std(self, axis=None, keepdims=False, ddof=0):
         v = self.var(axis, keepdims, ddof)
-        return Tile("sqrt", (v,), v.shape, v.dtype_name)
+        return Tile("masqrt", (v,), v.shape, v.dtype_name, plain=True)
 
     def __pow__(self, e):
         if isinstance(e, (int, float, np.generic)) and not isinstance(e, bool):
@@ -896,7 +916,7 @@ class Tile:
         name = dtype_name(dt)
         if name == self.dtype_name:
             return self
-        return Tile("astype", (self,), self.shape, name)
+        return Tile("astype", (self,), self.shape, name, **self._plain_kw())
 
     @property
     def T(self):
@@ -931,7 +951,7 @@ class Tile:
                 next(dims)
         norm = tuple("new" if k is None else
                      (k.start, k.stop, k.step) if isinstance(k, slice) else int(k) for k in key)
-        return Tile("slice", (self,), shape, self.dtype_name, key=norm)
+        return Tile("slice", (self,), shape, self.dtype_name, key=norm, **self._plain_kw())
 
     def __setitem__(self, key, value):
         """`tile[key] = value` with a static key: the tile object becomes the
@@ -968,7 +988,7 @@ class Tile:
             shape = tuple(math.prod(self.shape) // known if s == -1 else s for s in shape)
         if math.prod(shape) != math.prod(self.shape):
             raise TraceError("reshape changes the number of elements")
-        return Tile("reshape", (self,), shape, self.dtype_name)
+        return Tile("reshape", (self,), shape, self.dtype_name, **self._plain_kw())
 
     def __bool__(self):
         raise TraceError("the value of a tile is not known while the kernel is traced; "

@@ -522,8 +522,11 @@ MAP_MAX_INPUTS, MAP_MAX_INSTRS, MAP_STACK_DEPTH = 4, 32, 4
 # Row programs (hcamdLaunchRowProgram): opcodes that read row scalars, stage kinds, limits
 MAP_OPS.update({"red": 45, "add_red": 46, "sub_red": 47, "mul_red": 48, "div_red": 49,
                 "max_red": 50, "min_red": 51, "rsub_red": 52, "rdiv_red": 53,
-                "mdiv_red": 54, "rmdiv_red": 55})
-ROW_KINDS = {"sum": 0, "max": 1, "min": 2, "scalar": 3, "store": 4, "store_col": 5}
+                "mdiv_red": 54, "rmdiv_red": 55,
+                # push a row scalar as a value, deactivated or not; numpy.ma.sqrt;
+                # (last in a stage) the result is active iff row scalar `arg` is positive
+                "red0": 56, "masqrt": 57, "livepos": 58})
+ROW_KINDS = {"sum": 0, "max": 1, "min": 2, "scalar": 3, "store": 4, "store_col": 5, "count": 6}
 ROW_MAX_STAGES, ROW_MAX_SCALARS, ROW_MAX_INSTRS = 16, 16, 128
 F32, F16, BF16 = 0, 1, 2
 

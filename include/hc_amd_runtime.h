@@ -511,9 +511,34 @@ int hcamdLaunchMapReduceColsNoAlloc(OlQueue q, int kind, const HcamdMapInstr *pr
  *                  scalar `dst`
  *   STORE          the value at every element is stored to out[row, col]
  *   STORE_COL      as SCALAR, stored to out[row * ldo]
+ *   COUNT          the number of active elements of the value (see below) becomes
+ *                  row scalar `dst` (fp32)
  * Exactly one stage stores, and it is the last.  Programs read row scalars with
  * HCAMD_MAP_RED (push) and the *_RED forms (top = top op scalar), only scalars
  * that an earlier stage or a column operand has written.
+ * Activity follows numpy.ma, to which the reference's tiles forward their
+ * operators and reductions (python/hckernel/kernel_api.py:150-180).  Elements
+ * that the masked forms (HCAMD_MAP_MDIV .. MLOG) deactivate are neither stored
+ * nor folded, and are not counted.  A fold over a row without any active
+ * element is a deactivated row scalar (holding 0 for a sum, 1e20 for a maximum
+ * or minimum); so is the result of a SCALAR stage in which a masked form fails
+ * (a quotient that is not finite, a root of a negative number) or that reads a
+ * deactivated row scalar.  Every element of a stage that reads a deactivated
+ * row scalar is inactive.  STORE_COL stores every row, a deactivated one with
+ * the value numpy.ma leaves in it: in SCALAR / STORE_COL stages + - * leave
+ * their first operand's value there, the quotient leaves the dividend, NumPy
+ * functions compute regardless (sqrt and log give their fill values 0 and 1).
+ * For that, `arg` of the instructions of those stages carries two more flags:
+ * 0x200, the operation was called as a NumPy function; 0x400, a commutative
+ * operation whose running value (the stack top of an immediate or *_RED form,
+ * the deeper entry of a stack form) is its second operand.  HCAMD_MAP_RED0
+ * pushes a row scalar's value whether deactivated or not (numpy.ma's variance
+ * reads the sum of the centred squares that way: 0 if all of them were
+ * inactive); HCAMD_MAP_MASQRT is numpy.ma.sqrt (the standard deviation's: a
+ * result that is not finite deactivates and leaves the argument);
+ * HCAMD_MAP_LIVEPOS, as the last instruction of a SCALAR stage, replaces the
+ * result's activity: active iff row scalar `arg` is positive (a variance is
+ * active where count - ddof is).
  * Operands: `inputs` are rows x cols tiles with a leading dimension in elements,
  * or, with leading dimension 0, one vector of cols elements used for every row;
  * `columns` hold one value per row and fill row scalars 0 .. nColumns-1.
@@ -527,14 +552,16 @@ int hcamdLaunchMapReduceColsNoAlloc(OlQueue q, int kind, const HcamdMapInstr *pr
  * once for 8, 16 or 32 elements of a lane (variant 1 of the "rows" family keeps
  * the general kernel).  One program has a kernel of its own that interprets
  * nothing: the layer normalisation (x - mean) / sqrt(var + eps) * w + b in the
- * five stages the front-end emits for it (sum; RED DIVI; the sum of the
- * centred squares; RED DIVI ADDI SQRT; IN SUB_RED MDIV_RED MUL_IN ADD_IN) on
- * dense fp32 rows of at most 32768 elements with fp32 vectors w and b: the same
- * operations per element, the row read once; and so has the root-mean-square
- * normalisation x / sqrt(mean(x * x) + eps) * w in its three stages (IN MUL_IN
- * summed; RED DIVI ADDI SQRT; IN MDIV_RED MUL_IN; with R16 at the end on fp16
- * rows of whole chunks of 8 with an fp32 w) under the same conditions
- * (variant 2 of "rows" keeps both on the kernels above).  Sums add in an order that
+ * six stages the front-end emits for it (sum; RED MDIVI; the sum of the
+ * centred squares; RED0 DIVI; RED ADDI MSQRT; IN SUB_RED MDIV_RED MUL_IN
+ * ADD_IN) on dense fp32 rows of at most 32768 elements with fp32 vectors w and
+ * b: the same operations per element, the row read once, nothing stored to a
+ * row whose mean is not finite; and so has the root-mean-square normalisation
+ * x / sqrt(mean(x * x) + eps) * w in its three stages (IN MUL_IN summed; RED
+ * MDIVI ADDI MSQRT; IN MDIV_RED MUL_IN; with R16 at the end on fp16 rows of
+ * whole chunks of 8 with an fp32 w) under the same conditions (variant 2 of
+ * "rows" keeps both on the kernels above).  Programs in which a row scalar can
+ * be deactivated, or that count, run on the general kernel.  Sums add in an order that
  * depends on the shape and the kernel only: results are reproducible, and agree with a
  * sequential fp32 sum to within the usual n * 2^-24 bound. */
 enum HcamdRowStageKind {
@@ -543,7 +570,8 @@ enum HcamdRowStageKind {
   HCAMD_ROW_MIN = 2,
   HCAMD_ROW_SCALAR = 3,
   HCAMD_ROW_STORE = 4,
-  HCAMD_ROW_STORE_COL = 5
+  HCAMD_ROW_STORE_COL = 5,
+  HCAMD_ROW_COUNT = 6
 };
 enum {
   HCAMD_MAP_RED = 45,     /* push row scalar `arg` */
@@ -558,7 +586,10 @@ enum {
   /* the tile operator / with a row scalar under numpy.ma's rule (see
    * HCAMD_MAP_MDIV): `arg` bits 0..3 the scalar, bit 8 the fp16 flag */
   HCAMD_MAP_MDIV_RED = 54, /* top / scalar */
-  HCAMD_MAP_RMDIV_RED = 55 /* scalar / top */
+  HCAMD_MAP_RMDIV_RED = 55, /* scalar / top */
+  HCAMD_MAP_RED0 = 56,    /* SCALAR / STORE_COL stages: push row scalar `arg`, deactivated or not */
+  HCAMD_MAP_MASQRT = 57,  /* SCALAR / STORE_COL stages: numpy.ma.sqrt */
+  HCAMD_MAP_LIVEPOS = 58  /* closes a SCALAR stage: active iff row scalar `arg` > 0 */
 };
 #define HCAMD_ROW_MAX_STAGES 16
 #define HCAMD_ROW_MAX_SCALARS 16

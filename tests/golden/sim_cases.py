@@ -431,7 +431,101 @@ def case_float_activity(api):
     return rec.out
 
 
+def case_masked_reductions(api):
+    """Reductions along rows and down columns over elements that a zero divisor
+    deactivated, row / column scalars that are deactivated themselves (a
+    quotient of two sums with a zero divisor, numpy.sqrt of a negative sum, a
+    mean that is not finite), arithmetic on those, and what a store then writes:
+    tiles skip deactivated elements, per-row results (bare numpy.ma arrays) are
+    written in full with what numpy.ma left under the mask."""
+    rec = Recorder()
+    f = np.float32
+    rng = np.random.default_rng(11)
+    a = rng.integers(-6, 7, (6, 5)).astype(f) / f(2)
+    b = rng.integers(-3, 4, (6, 5)).astype(f)
+    b[1, :] = 0                                     # every quotient of the row is deactivated
+    b[4, :] = [1.5, -1.5, 2, -2, 0]                 # adds up to zero
+    b[2, :] = -np.abs(b[2, :]) - f(1)               # a negative sum
+    a[5, 2] = np.inf                                # a mean that is not finite
+    tiles = {
+        "ratio": lambda ta, tb: ta * (ta.sum(axis=1, keepdims=True) / tb.sum(axis=1, keepdims=True)),
+        "centre": lambda ta, tb: (ta / tb) - (ta / tb).mean(axis=1, keepdims=True),
+        "divsqrt": lambda ta, tb: ta / np.sqrt(tb.sum(axis=1, keepdims=True)),
+        "mullog": lambda ta, tb: ta * np.log(tb.sum(axis=1, keepdims=True)),
+        "xvar": lambda ta, tb: tb * ta.var(axis=1, keepdims=True),
+        "xstd": lambda ta, tb: tb * ta.std(axis=1, keepdims=True),
+        "xmaskedvar": lambda ta, tb: tb * (ta / tb).var(axis=1, keepdims=True, ddof=2),
+        "rms": lambda ta, tb: ta / np.sqrt(np.mean(np.square(ta), axis=1, keepdims=True) + f(1e-6)) * tb,
+        "layernorm": lambda ta, tb: (ta - ta.mean(axis=1, keepdims=True)) /
+        np.sqrt(ta.var(axis=1, keepdims=True) + f(1e-5)) * tb,
+        "over_max": lambda ta, tb: ta / (ta / tb).max(axis=1, keepdims=True),
+        "col_centre": lambda ta, tb: ta - ta.mean(axis=0, keepdims=True),
+        "col_over_sum": lambda ta, tb: ta / tb.sum(axis=0, keepdims=True),
+    }
+    rows = {
+        "mean": lambda ta, tb: (ta / tb).mean(axis=1),
+        "sum": lambda ta, tb: (ta / tb).sum(axis=1),
+        "max": lambda ta, tb: (ta / tb).max(axis=1),
+        "min": lambda ta, tb: (ta / tb).min(axis=1),
+        "var": lambda ta, tb: (ta / tb).var(axis=1),
+        "std1": lambda ta, tb: (ta / tb).std(axis=1, ddof=1),
+        "plain_mean": lambda ta, tb: ta.mean(axis=1),
+        "plain_var": lambda ta, tb: ta.var(axis=1),
+        "plain_std": lambda ta, tb: ta.std(axis=1),
+        "sqrt_sum": lambda ta, tb: np.sqrt(tb.sum(axis=1)),
+        "sum_ratio": lambda ta, tb: ta.sum(axis=1) / tb.sum(axis=1),
+        "one_plus_ratio": lambda ta, tb: f(1) + ta.sum(axis=1) / tb.sum(axis=1),
+        "python_one_plus_ratio": lambda ta, tb: 1.0 + ta.sum(axis=1) / tb.sum(axis=1),
+        "ratio_times_two": lambda ta, tb: ta.sum(axis=1) / tb.sum(axis=1) * f(2),
+        "two_ratios": lambda ta, tb: (ta.sum(axis=1) / tb.sum(axis=1) + f(1)) *
+        (tb.max(axis=1) / ta.sum(axis=1) - f(2)),
+        "neg_sqrt_ratio": lambda ta, tb: -np.sqrt(ta.sum(axis=1) / tb.sum(axis=1)),
+        "max_plus_log": lambda ta, tb: ta.max(axis=1) + np.log(tb.sum(axis=1)),
+        "log_plus_max": lambda ta, tb: np.log(tb.sum(axis=1)) + ta.max(axis=1),
+        "exp_of_mean": lambda ta, tb: np.exp((ta / tb).mean(axis=1)),
+    }
+    cols = {
+        "col_sum": lambda ta, tb: (ta / tb).sum(axis=0),
+        "col_max": lambda ta, tb: (ta / tb).max(axis=0),
+        "col_min_log": lambda ta, tb: np.log(ta * tb).min(axis=0),
+        "col_mean": lambda ta, tb: ta.mean(axis=0),
+        "col_var": lambda ta, tb: ta.var(axis=0),
+        "col_std": lambda ta, tb: ta.std(axis=0, ddof=1),
+    }
+    bt = b.copy()
+    bt[:, 3] = 0                                    # a column without an active quotient
+    dst_t = np.full((len(tiles), 6, 5), POISON, f)
+    dst_r = np.full((len(rows), 6), POISON, f)
+    dst_c = np.full((len(cols), 5), POISON, f)
+
+    def body(gr, a, b, bt, dst_t, dst_r, dst_c):
+        for i, (name, fn) in enumerate(tiles.items()):
+            ta, tb = gr.load(a, shape=(8, 5)), gr.load(b, shape=(8, 5))
+            t = rec.attempt("tile." + name, lambda: fn(ta, tb))
+            if t is not None:
+                gr.store(dst_t[i], t)
+        for i, (name, fn) in enumerate(rows.items()):
+            ta, tb = gr.load(a, shape=(8, 5)), gr.load(b, shape=(8, 5))
+            t = rec.attempt("row." + name, lambda: fn(ta, tb))
+            if t is not None:
+                gr.store(dst_r[i], t)
+        for i, (name, fn) in enumerate(cols.items()):
+            ta, tb = gr.load(a, shape=(6, 8)), gr.load(bt, shape=(6, 8))
+            t = rec.attempt("col." + name, lambda: fn(ta, tb))
+            if t is not None:
+                gr.store(dst_c[i], t)
+
+    with np.errstate(all="ignore"), warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        _one_group(api, body, a, b, bt, dst_t, dst_r, dst_c)
+    rec.array("dst_tiles", dst_t)
+    rec.array("dst_rows", dst_r)
+    rec.array("dst_cols", dst_c)
+    return rec.out
+
+
 CASES = {
+    "masked_reductions": case_masked_reductions,
     "inplace_partial": case_inplace_partial,
     "load_from_masked": case_load_from_masked,
     "domain_masking": case_domain_masking,

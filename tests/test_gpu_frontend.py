@@ -747,6 +747,58 @@ def test_row_reduction_bodies_match_the_simulator(name, rows, n):
         assert_allclose(got, want, rtol=2e-5, atol=2e-6)
 
 
+# (a wave per row with and without 16-byte rows, a workgroup per row, rows past the last group)
+@pytest.mark.parametrize("rows,n", [(8, 5), (37, 200), (21, 1031), (9, 4104), (70, 4608)])
+def test_reductions_over_deactivated_elements_follow_numpy_ma_on_the_gpu(rows, n):
+    """Row reductions over elements the data deactivates (zero divisors), row
+    scalars that are deactivated themselves (a quotient of sums with a zero
+    divisor, a root of a negative sum, a mean that is not finite), and what
+    follows from them, on the GPU and on the CPU simulator: the same elements
+    written (the rest keep the poison), the same values to the bound of sums
+    added in another order, per-row results of deactivated rows included."""
+    from test_kernel_frontend import POISON, _masked_row_bodies, _masked_row_case
+    gpu, sim = _masked_row_bodies(kernel), _masked_row_bodies(sim_kernel)
+    a, b = _masked_row_case(rows, n, seed=rows)
+    da, db = rt.to_device(a), rt.to_device(b)
+    for name, (body, per_row) in gpu.items():
+        shape = (rows,) if per_row else (rows, n)
+        want = np.full(shape, POISON)
+        with np.errstate(all="ignore"):
+            sim[name][0](a, b, want, 8)
+        out = rt.to_device(np.full(shape, POISON))
+        body(da, db, out, 8)
+        assert rt.last_kernel_name().startswith("hcamd_row_program_w"), (name, rt.last_kernel_name())
+        got = out.to_host()
+        assert_array_equal(got == POISON, want == POISON, err_msg=name)
+        assert_array_equal(np.isnan(got), np.isnan(want), err_msg=name)
+        assert_allclose(got, want, rtol=1e-4, atol=1e-5, err_msg=name)
+
+
+@pytest.mark.parametrize("name", ["layernorm"])
+@pytest.mark.parametrize("rows,n", [(64, 4096), (37, 200), (5, 20_003)])
+def test_normalisations_leave_rows_with_a_mean_that_is_not_finite_alone(name, rows, n):
+    """numpy.ma's mean of a row with an inf or a NaN is deactivated: nothing of
+    that row is stored, by the kernels of their own (dense rows of whole
+    chunks) as by the general one."""
+    from test_kernel_frontend import _row_bodies, _row_case
+    host = _row_case(name, rows, n, seed=rows)
+    x = host[0]
+    x[1, n // 3] = np.inf
+    x[2, 0] = np.nan
+    want = np.full(host[-1].shape, -77, host[-1].dtype)
+    with np.errstate(all="ignore"):
+        _row_bodies(sim_kernel)[name](*host[:-1], want, 8)
+    out = rt.to_device(np.full(host[-1].shape, -77, host[-1].dtype))
+    _row_bodies(kernel)[name](*[rt.to_device(v) for v in host[:-1]], out, 8)
+    got = out.to_host()
+    assert (want[1] == -77).all() and (want[2] == -77).all() and (want[0] != -77).all()
+    assert_array_equal(got == -77, want == -77)
+    if got.dtype == np.float16:
+        assert_allclose(got.astype(np.float32), want.astype(np.float32), rtol=1.1e-3)
+    else:
+        assert_allclose(got, want, rtol=2e-5, atol=2e-6)
+
+
 @pytest.mark.parametrize("rows,n,gn", [(37, 200, 64), (3000, 4096, 512), (70_000, 24, 24),
                                        (513, 1031, 1031)])
 @pytest.mark.parametrize("name", ["col_sums", "col_max_abs", "col_min", "col_means", "col_norms",
@@ -842,7 +894,7 @@ def test_random_row_expressions_match_the_simulator():
         try:
             random_row_body(kernel, expr, per_row)(*[rt.to_device(a) for a in host[:-1]], out, 8)
         except NoNativeKernel as exc:
-            assert any(w in str(exc) for w in ("stack", "row scalars", "operations", "passes",
+            assert any(w in str(exc) for w in ("stack", "row scalars", "operations", "passes", "numpy.ma leaves",
                                                "arrays")), (text, str(exc))
             continue
         assert rt.last_kernel_name().startswith("hcamd_row_program"), text
@@ -1307,6 +1359,8 @@ def test_column_reductions_leave_deactivated_elements_out():
     rows, n, gn = 777, 200, 64
     x = rng.standard_normal((rows, n)).astype(np.float32)
     y = rng.integers(-2, 3, (rows, n)).astype(np.float32)          # a fifth of the divisors are zero
+    y[:, 7] = 0              # a column without an active quotient: numpy.ma stores 0 for its sum, 1e20 for its maximum
+    y[:, 130] = 0
     deco = dict(work_shape=cdiv(n, gn), group_shape=1, literals={GN})
     for name, fn in (("sum", lambda a, b: (a / b).sum(axis=0)), ("max", lambda a, b: (a / b).max(axis=0)),
                      ("sum_sqrt", lambda a, b: np.sqrt(a * b).sum(axis=0)),

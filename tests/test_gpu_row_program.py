@@ -126,13 +126,16 @@ def test_layer_normalisation_with_weight_and_bias_vectors(ctx, cols, dtype, rows
 
 
 def layer_norm_stages(n, eps):
-    """The five stages the front-end emits for (x - mean) / sqrt(var + eps) * w + b
-    written with mean and var along axis 1 (numpy.ma's division in the last)."""
+    """The six stages the front-end emits for (x - mean) / sqrt(var + eps) * w + b
+    written with mean and var along axis 1: the mean's division and the last one
+    are numpy.ma's, the variance reads the sum of the centred squares as a value
+    (0 where the mean, and with it every centred square, is deactivated)."""
     return [("sum", 0, [I("in", 0)]),
-            ("scalar", 1, [I("red", 0), I("divi", 0, n)]),
+            ("scalar", 1, [I("red", 0), I("mdivi", 0, n)]),
             ("sum", 2, [I("in", 0), I("sub_red", 1), I("in", 0), I("sub_red", 1), I("mul")]),
-            ("scalar", 3, [I("red", 2), I("divi", 0, n), I("addi", 0, eps), I("sqrt")]),
-            ("store", 0, [I("in", 0), I("sub_red", 1), I("mdiv_red", 3), I("mul_in", 1), I("add_in", 2)])]
+            ("scalar", 3, [I("red0", 2), I("divi", 0, n)]),
+            ("scalar", 4, [I("red", 3), I("addi", 0, eps), I("msqrt")]),
+            ("store", 0, [I("in", 0), I("sub_red", 1), I("mdiv_red", 4), I("mul_in", 1), I("add_in", 2)])]
 
 
 def layer_norm_kernel(cols, per_chunk=4):
@@ -182,7 +185,8 @@ def test_layer_normalisation_as_the_front_end_writes_it_takes_its_own_kernel(ctx
             name = rt.last_kernel_name()
         finally:
             rt.set_variant("rows", 0)
-        assert name == (layer_norm_kernel(cols) if variant == 0 else kernel_for(cols, general=variant == 1))
+        # (a program whose row scalars the data can deactivate: the general kernel, or its own)
+        assert name == (layer_norm_kernel(cols) if variant == 0 else kernel_for(cols, general=True))
         got = out.to_host()
         assert_allclose(got[stored], want[stored], rtol=2e-5, atol=2e-5)
         assert (got[~stored].view(np.uint32) == POISON32).all()
@@ -203,7 +207,7 @@ def test_rms_normalisation_as_the_front_end_writes_it_takes_its_own_kernel(ctx, 
     big = np.full((rows, ld), np.nan, dtype)
     x = (rng.standard_normal((rows, cols)) * 2 + 0.5).astype(dtype)
     if rows > 8:
-        x[3, cols // 2] = np.inf       # the scale is not finite: x / inf is 0 (stored), inf / inf is not
+        x[3, cols // 2] = np.inf       # the mean of the squares is not finite: numpy.ma stores nothing of the row
         x[5] = 0.0
     big[:, :cols] = x
     dbig = rt.to_device(big)
@@ -212,13 +216,13 @@ def test_rms_normalisation_as_the_front_end_writes_it_takes_its_own_kernel(ctx, 
     dg = rt.to_device(g)
     eps = 1e-6
     stages = [("sum", 0, [I("in", 0), I("mul_in", 0)]),
-              ("scalar", 1, [I("red", 0), I("divi", 0, float(cols)), I("addi", 0, eps), I("sqrt")]),
+              ("scalar", 1, [I("red", 0), I("mdivi", 0, float(cols)), I("addi", 0, eps), I("msqrt")]),
               ("store", 0, [I("in", 0), I("mdiv_red", 1), I("mul_in", 1)] + ([I("r16")] if half else []))]
     x64 = x.astype(np.float64)
     with np.errstate(invalid="ignore", over="ignore"):
         q = x64 / np.sqrt((x64 * x64).mean(axis=1, keepdims=True) + eps)
         want = q * g
-    stored = np.isfinite(q)
+    stored = np.isfinite(q) & np.isfinite((x64 * x64).mean(axis=1, keepdims=True))
     tol = dict(rtol=1.1e-3, atol=1e-4) if half else dict(rtol=2e-5, atol=2e-5)
     results = {}
     for variant in (1, 2, 0):
@@ -230,7 +234,7 @@ def test_rms_normalisation_as_the_front_end_writes_it_takes_its_own_kernel(ctx, 
         finally:
             rt.set_variant("rows", 0)
         own = layer_norm_kernel(cols, 8 if half else 4).replace("layer", "rms").replace("f32", "f16" if half else "f32")
-        assert name == (own if variant == 0 else kernel_for(cols, general=variant == 1))
+        assert name == (own if variant == 0 else kernel_for(cols, general=True))
         got = out.to_host()
         assert_allclose(got[stored].astype(np.float64), want[stored], **tol)
         raw = got.view(np.uint16 if half else np.uint32)

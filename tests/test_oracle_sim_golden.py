@@ -7,7 +7,9 @@ or document of the reference fixes: in-place operators on partially active
 tiles, loads from tiles that are already masked, domain masking of / // % **,
 NumPy functions and reductions applied to tiles, compressed() and repr, Python
 and NumPy scalars next to a tile, every installed operator on int32, float32
-and bool tiles, and stores of numpy.ma results.
+and bool tiles, stores of numpy.ma results, and reductions (sum, max, min,
+mean, var, std) over elements that a zero divisor deactivated, together with
+arithmetic on the deactivated row and column scalars that come out of them.
 
 Rule: wherever the reference returned a value, the oracle returns the same
 bytes (dtype, shape, content).  Where the reference raised there is no result
@@ -101,3 +103,33 @@ def test_headline_behaviours(golden):
     #      in a 0-d float64 array), a NumPy scalar of the tile's type does not
     assert _text(g["scalar_promotion/f32.mul_pyfloat.dtype"]) == "float64"
     assert _text(g["scalar_promotion/f32.mul_npf32.dtype"]) == "float32"
+
+
+def test_headline_behaviours_of_reductions_over_deactivated_elements(golden):
+    """What numpy.ma does where elements or whole rows are deactivated (rows of the
+    case: 1 has zero divisors only, 2 a negative divisor sum, 4 divisors that add
+    up to zero, 5 an inf in the dividend)."""
+    g = golden
+    rows = g["masked_reductions/dst_rows"]
+    names = ["mean", "sum", "max", "min", "var", "std1", "plain_mean", "plain_var", "plain_std", "sqrt_sum",
+             "sum_ratio", "one_plus_ratio", "python_one_plus_ratio"]
+    r = {n: rows[i] for i, n in enumerate(names)}
+    # a per-row result is stored in full; a fold without active elements holds 0
+    # (sum, and the mean and variance made of it) or numpy.ma's fill value 1e20
+    assert r["sum"][1] == 0 and r["mean"][1] == 0 and r["var"][1] == 0
+    assert r["max"][1] == np.float32(1e20) and r["min"][1] == np.float32(1e20)
+    # the mean divides by the number of active elements: one of row 0's five divisors is zero
+    assert r["mean"][0] * 4 == r["sum"][0]
+    # a mean that is not finite is deactivated, the variance of that row is an active 0
+    assert np.isinf(r["plain_mean"][5]) and r["plain_var"][5] == 0 and r["plain_std"][5] == 0
+    # numpy.sqrt of a negative sum: deactivated, fill value 0
+    assert r["sqrt_sum"][2] == 0
+    # a deactivated quotient holds the dividend; a NumPy scalar's + computes on it
+    # (1 + dividend), a Python scalar's leaves its own first operand (1)
+    assert r["sum_ratio"][4] == -1.5 and r["one_plus_ratio"][4] == -0.5 and r["python_one_plus_ratio"][4] == 1.0
+    # tiles computed from a deactivated row scalar are not stored
+    tiles = g["masked_reductions/dst_tiles"]
+    assert (tiles[0][[0, 1, 4, 5]] == sim_cases.POISON).all() and (tiles[0][[2, 3]] != sim_cases.POISON).all()
+    # down columns: a column without an active quotient
+    cols = g["masked_reductions/dst_cols"]
+    assert cols[0][3] == 0 and cols[1][3] == np.float32(1e20)
