@@ -129,9 +129,11 @@ def autotune(kernel, *args, max_trials: int = 64, iters: int = 10, warmup: int =
                 continue
             family, numbers = _FAMILIES[what]
             chosen = 0
+            # (this thread's choice only: whatever the process has selected with
+            # hcamdSetVariant stays as it is, and is what other threads keep running)
             try:
                 for v in numbers:
-                    rt.set_variant(family, v)
+                    rt.set_thread_variant(family, v)
                     try:
                         us = _time(best_plans, ctx, iters, warmup)
                     except rt.HcRuntimeError:
@@ -139,7 +141,7 @@ def autotune(kernel, *args, max_trials: int = 64, iters: int = 10, warmup: int =
                     if us < best_us:
                         best_us, chosen = us, v
             finally:
-                rt.set_variant(family, 0)
+                rt.set_thread_variant(family, -1)
             if chosen:
                 variants[family] = chosen
     return TunedParams(best, variants, ctx.info().get("arch", ""), round(best_us, 3))

@@ -850,6 +850,11 @@ class _MapCompiler:
         if t.op in _MAP_BINARY and len(t.args) == 2:
             if all(_const(a) for a in t.args):
                 return False
+            if t.op in ("maximum", "minimum") and t.dtype_name == "float16":
+                # NumPy's fp16 maximum / minimum return the first of two equal values
+                # (+0 and -0), the fp32 ones, which this kernel has, the second:
+                # the general float map has both
+                return False
             return all(self.supported(a) and (_const(a) or a.shape == t.shape) for a in t.args)
         if _is(t, "vardiv", 2):                  # a variance whose count is a number
             return _const(t.args[1]) and self.supported(t.args[0])

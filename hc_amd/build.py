@@ -2,6 +2,10 @@
 
     python -m hc_amd.build            # everything
     python -m hc_amd.build gemm       # one kernel module, then relink
+    python -m hc_amd.build --probes   # everything, with the measurement builds
+                                      # of the GEMM (kernels whose output is not
+                                      # the product; hc_amd_bench.h), which a
+                                      # default build leaves out
 
 Outputs (all under hc_amd/_native/, none tracked by git):
     build/<module>.hsaco      gfx950 code objects, one per kernels/<module>.hip
@@ -67,10 +71,17 @@ def _run(cmd: list[str]) -> None:
         print(err, file=sys.stderr)
 
 
+PROBES = False          # set by --probes: compile the measurement builds too
+
+
+def _defines() -> list[str]:
+    return ["-DHCAMD_PROBES"] if PROBES else []
+
+
 def build_kernel_module(name: str, keep_asm: bool = False) -> Path:
     src = CSRC / "kernels" / f"{name}.hip"
     out = BUILD / f"{name}.hsaco"
-    cmd = [_hipcc(), "--genco", "--no-gpu-bundle-output", *DEVICE_FLAGS,
+    cmd = [_hipcc(), "--genco", "--no-gpu-bundle-output", *DEVICE_FLAGS, *_defines(),
            *MODULE_FLAGS.get(name, []), "-I", str(CSRC / "kernels"),
            "-o", str(out), str(src)]
     if keep_asm:
@@ -100,7 +111,7 @@ def build_runtime() -> Path:
     rocm = _rocm_root()
     cxx = shutil.which("g++") or "g++"
     scratch = build_scratch()
-    _run([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall",
+    _run([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", *_defines(),
           "-D__HIP_PLATFORM_AMD__", "-I", str(rocm / "include"),
           "-I", str(INCLUDE), "-I", str(CSRC), f"-Wa,-I{BUILD}",
           str(CSRC / "runtime.cpp"), str(CSRC / "blobs.S"), str(scratch),
@@ -130,7 +141,9 @@ def build_all(modules: tuple[str, ...] = KERNEL_MODULES, keep_asm: bool = False)
 
 
 def main(argv: list[str]) -> int:
+    global PROBES
     keep = "--asm" in argv
+    PROBES = "--probes" in argv
     names = tuple(a for a in argv if not a.startswith("--")) or KERNEL_MODULES
     unknown = [n for n in names if n not in KERNEL_MODULES]
     if unknown:

@@ -861,7 +861,9 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_gemm_bf16_p256x256_w2x2(
   gemm_tile_pipelined<__bf16, 256, 256, 2, 2, 16, false, 2, false, 0, 0, 24, 1, 4, 0>(A, lda, Bt, ldb, C, ldc, M,
                                                                                     N, K);
 }
-// measurement builds whose output is not the product
+// measurement builds whose output is not the product: compiled only into a
+// library built with `python -m hc_amd.build --probes`
+#ifdef HCAMD_PROBES
 HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_mfma_only, 1)
 HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_no_vmwait, 2)
 HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_no_barrier, 3)
@@ -869,6 +871,7 @@ HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_no_ldsread, 4)
 HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_no_loads, 5)
 HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_loads_to_regs, 6)
 HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_b_direct, __bf16, 256, 256, 2, 4, 16, 2, false, 7)
+#endif
 HCAMD_GEMM_PE(hcamd_gemm_bf16_p256x256_w2x4_edge, __bf16, 256, 256, 2, 4, 16)
 HCAMD_GEMM_PE(hcamd_gemm_f16_p256x256_w2x4_edge, _Float16, 256, 256, 2, 4, 16)
 HCAMD_GEMM_PE(hcamd_gemm_bf16_p128x128_w2x2_edge, __bf16, 128, 128, 2, 2, 16)

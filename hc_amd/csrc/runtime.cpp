@@ -3,8 +3,10 @@
 // directly on the HIP module API: hipModuleLoadData, hipModuleGetFunction,
 // hipModuleLaunchKernel, one stream per queue, hipMalloc.  The signatures and
 // the reference interfaces they replace are documented in
-// include/hc_amd_runtime.h.
+// include/hc_amd_runtime.h; the measurement entry points are declared in
+// include/hc_amd_bench.h.
 #include "hc_amd_runtime.h"
+#include "hc_amd_bench.h"
 #include "internal.h"
 
 #include <hip/hip_runtime_api.h>
@@ -725,8 +727,31 @@ int hcamdDeviceInfo(OlDevice dev, int *computeUnits, int *clockKHz,
   return 0;
 }
 
+namespace {
+// Variants 17..22 and 26 of "gemm" are measurement builds of the default kernel
+// with one part of its loop taken out: what they leave in C is not the product.
+// They exist only in a library built with HCAMD_PROBES defined (`python -m
+// hc_amd.build --probes`); any other build refuses to select them.
+bool variantIsAbsentProbe(const char *family, int variant) {
+#ifdef HCAMD_PROBES
+  (void)family, (void)variant;
+  return false;
+#else
+  return std::strcmp(family, "gemm") == 0 && ((variant >= 17 && variant <= 22) || variant == 26);
+#endif
+}
+} // namespace
+
+int hcamdProbesBuilt(void) noexcept {
+#ifdef HCAMD_PROBES
+  return 1;
+#else
+  return 0;
+#endif
+}
+
 int hcamdSetVariant(const char *family, int variant) noexcept {
-  if (!family)
+  if (!family || variantIsAbsentProbe(family, variant))
     return 1;
   std::lock_guard<std::mutex> guard(g_variantLock);
   auto &v = variants();
@@ -738,7 +763,7 @@ int hcamdSetVariant(const char *family, int variant) noexcept {
 }
 
 int hcamdSetThreadVariant(const char *family, int variant) noexcept {
-  if (!family)
+  if (!family || variantIsAbsentProbe(family, variant))
     return 1;
   {
     std::lock_guard<std::mutex> guard(g_variantLock);
@@ -3191,6 +3216,11 @@ int launchGemm(OlQueue q, bool half, const void *a, size_t lda, const void *bt,
     const char *name;
     int bm, bn, threads;
   };
+#ifdef HCAMD_PROBES
+#define HCAMD_PROBE_NAME(n) n
+#else
+#define HCAMD_PROBE_NAME(n) nullptr // not in this build (and hcamdSetVariant refuses the number)
+#endif
   static const Tiled tiled[] = {
       {"hcamd_gemm_bf16_256x256_w2x4_s0", 256, 256, 512}, // 1
       {"hcamd_gemm_bf16_256x256_w2x4_s1", 256, 256, 512},
@@ -3208,16 +3238,16 @@ int launchGemm(OlQueue q, bool half, const void *a, size_t lda, const void *bt,
       {"hcamd_gemm_bf16_p256x256_w2x4_direct", 256, 256, 512}, // 14: 8-byte stores from the accumulators
       {"hcamd_gemm_bf16_p256x256_w2x4_lds", 256, 256, 512},    // 15: through LDS, plain stores
       {"hcamd_gemm_bf16_p256x256_w2x4_prio", 256, 256, 512},   // 16: raised priority in the MFMA bursts
-      {"hcamd_gemm_bf16_probe_mfma_only", 256, 256, 512},      // 17: measurement only, output is not the product
-      {"hcamd_gemm_bf16_probe_no_vmwait", 256, 256, 512},      // 18..21: likewise
-      {"hcamd_gemm_bf16_probe_no_barrier", 256, 256, 512},
-      {"hcamd_gemm_bf16_probe_no_ldsread", 256, 256, 512},
-      {"hcamd_gemm_bf16_probe_no_loads", 256, 256, 512},
-      {"hcamd_gemm_bf16_probe_loads_to_regs", 256, 256, 512}, // 22
+      {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_mfma_only"), 256, 256, 512},      // 17: measurement only, output is not the product
+      {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_no_vmwait"), 256, 256, 512},      // 18..21: likewise
+      {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_no_barrier"), 256, 256, 512},
+      {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_no_ldsread"), 256, 256, 512},
+      {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_no_loads"), 256, 256, 512},
+      {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_loads_to_regs"), 256, 256, 512}, // 22
       {"hcamd_gemm_bf16_p256x256_w2x4_stage_a", 256, 256, 512},     // 23: A panel through registers
       {"hcamd_gemm_bf16_p256x256_w2x4_hinted", 256, 256, 512},      // 24: half-step order left to the compiler
       {"hcamd_gemm_bf16_p256x256_w2x4_loads_early", 256, 256, 512}, // 25: loads in the first half of the MFMAs
-      {"hcamd_gemm_bf16_probe_b_direct", 256, 256, 512},            // 26: measurement only
+      {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_b_direct"), 256, 256, 512},            // 26: measurement only
       {"hcamd_gemm_bf16_p256x256_w2x2", 256, 256, 256},             // 27: four waves, 128 x 128 each
   };
   constexpr int kGeneral = 6;

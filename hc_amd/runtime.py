@@ -93,7 +93,9 @@ class AffineId(C.Structure):
 hcamdLaunchIdScatter = _sig(_rt, "hcamdLaunchIdScatter", _int, _vp, _vp, _int, _sz, _sz_p,
                             C.POINTER(_ssz), C.POINTER(AffineId), C.POINTER(AffineId), _sz, _sz_p,
                             _sz_p, _int)
+# (the measurement entry points of include/hc_amd_bench.h)
 hcamdLaunchStream = _sig(_rt, "hcamdLaunchStream", _int, _vp, _int, _int, C.POINTER(_vp), _vp, _sz)
+hcamdProbesBuilt = _sig(_rt, "hcamdProbesBuilt", _int)
 hcamdLaunchAddF32 = _sig(_rt, "hcamdLaunchAddF32", _int, _vp, _vp, _vp, _vp, _sz)
 hcamdLaunchFmaF16 = _sig(_rt, "hcamdLaunchFmaF16", _int, _vp, _vp, _sz, _vp, _sz, _vp,
                          _sz, _vp, _sz, _sz, _sz)
@@ -983,15 +985,29 @@ def gemm_bf16(a, bt, c, sync: bool = True) -> None:
     plan_gemm_bf16(a, bt, c).launch(sync)
 
 
+def probes_built() -> bool:
+    """The library holds the measurement builds of the GEMM (built with
+    `python -m hc_amd.build --probes`); see hc_amd_bench.h."""
+    return bool(hcamdProbesBuilt())
+
+
+def _variant_error(family: str, variant: int) -> HcRuntimeError:
+    if family == "gemm" and (17 <= variant <= 22 or variant == 26) and not probes_built():
+        return HcRuntimeError(f"gemm variant {variant} is a measurement build whose output is not the "
+                              "product; this library was built without them (python -m hc_amd.build "
+                              "--probes builds them)")
+    return HcRuntimeError(f"unknown kernel family {family!r}")
+
+
 def set_variant(family: str, variant: int) -> None:
     if hcamdSetVariant(family.encode(), int(variant)):
-        raise HcRuntimeError(f"unknown kernel family {family!r}")
+        raise _variant_error(family, int(variant))
 
 
 def set_thread_variant(family: str, variant: int) -> None:
     """The choice for this thread only (variant < 0 removes it)."""
     if hcamdSetThreadVariant(family.encode(), int(variant)):
-        raise HcRuntimeError(f"unknown kernel family {family!r}")
+        raise _variant_error(family, int(variant))
 
 
 def last_kernel_name() -> str:

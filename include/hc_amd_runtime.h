@@ -238,24 +238,6 @@ int hcamdLaunchIdScatter(OlQueue q, void *out, int outType, size_t outRank,
                          const size_t *groupCount, const size_t *groupShape,
                          int perItem) HCAMD_NOEXCEPT;
 
-/* Stream calibration (no counterpart in the reference): what HBM delivers for
- * a mix of read and write streams with nothing else in the way, the yardstick
- * the memory-bound kernels are held to.  nReads (0..3) vectors of `bytes` bytes
- * are added in 32-bit lanes, word by word; writeMode selects what leaves:
- * HCAMD_STREAM_FULL the sum (bytes out), HCAMD_STREAM_HALF the xor of each sum
- * word's halves (bytes / 2 out: the 2:1 ratio of the int8 quantiser),
- * HCAMD_STREAM_NONE one 32-bit total per 16 KiB of input (bytes / 4096 out: a
- * read-only stream with a checkable result).  nReads == 0 writes the word
- * index (a fill; HCAMD_STREAM_FULL only).  bytes must be a multiple of 16 KiB,
- * pointers 16-byte aligned.  Each mix runs in the form that measured fastest
- * for it: three reads against one write from workgroups held to four waves per
- * SIMD that pause between the arrival of their words and their store, the
- * others from full workgroups that do not ("stream" variants 1..5 force one
- * form on every mix that reads and writes). */
-enum HcamdStreamWrite { HCAMD_STREAM_NONE = 0, HCAMD_STREAM_FULL = 1, HCAMD_STREAM_HALF = 2 };
-int hcamdLaunchStream(OlQueue q, int nReads, int writeMode, const void *const *inputs,
-                      void *out, size_t bytes) HCAMD_NOEXCEPT;
-
 /* The same copy launched with the reference's own geometry and kernel argument
  * list (tests/Transforms/gpu-to-gpu-runtime.mlir:34-37): grid =
  * (ceil(cols/(bx*unroll)), ceil(rows/by), 1), block = (bx, by, 1), one element
@@ -710,7 +692,11 @@ int hcamdLaunchGemmF16(OlQueue q, const void *a, size_t lda, const void *bt,
  * "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "cols", "stream", "gather"
  * (block shape), "gather_fuse" (groups per workgroup; read by
  * hcamdGatherGemmCreate).
- * Process-wide, guarded by a lock.  Returns 1 for an unknown family. */
+ * Process-wide, guarded by a lock.  Returns 1 for an unknown family, and for
+ * the numbers of the measurement builds of the "gemm" family (17..22 and 26,
+ * whose output is not the product) unless the library was built with them
+ * (hc_amd_bench.h).  Every variant a default build accepts computes the same
+ * result as variant 0. */
 int hcamdSetVariant(const char *family, int variant) HCAMD_NOEXCEPT;
 /* The same choice for the calling thread only: it takes precedence over
  * hcamdSetVariant for launches made by this thread and is invisible to others

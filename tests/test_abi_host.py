@@ -35,6 +35,28 @@ def test_runtime_exports_every_declared_symbol():
         assert hasattr(py_runtime.runtime_lib, n), n
 
 
+def test_measurement_entry_points_have_a_header_of_their_own_and_probes_stay_out_of_a_default_build():
+    names = declared_functions("hc_amd_bench.h")
+    assert set(names) == {"hcamdLaunchStream", "hcamdProbesBuilt"}
+    assert not set(names) & set(declared_functions("hc_amd_runtime.h"))
+    for n in names:
+        assert hasattr(py_runtime.runtime_lib, n), n
+    blob = C.string_at(*rt.builtin_modules()["gemm"])
+    if rt.probes_built():
+        assert b"hcamd_gemm_bf16_probe_mfma_only\x00" in blob
+        return
+    # a default build holds no kernel whose output is not the product, and
+    # refuses the numbers that would select one
+    assert b"hcamd_gemm_bf16_probe" not in blob
+    for v in (17, 18, 19, 20, 21, 22, 26):
+        assert rt.hcamdSetVariant(b"gemm", v) == 1 and rt.hcamdSetThreadVariant(b"gemm", v) == 1
+        with pytest.raises(rt.HcRuntimeError, match="--probes"):
+            rt.set_variant("gemm", v)
+    for v in (0, 7, 16, 23, 25, 27):
+        assert rt.hcamdSetVariant(b"gemm", v) == 0
+    rt.set_variant("gemm", 0)
+
+
 def test_pyabi_exports_every_declared_symbol():
     names = declared_functions("hc_amd_pyabi.h")
     assert {"hcgpuConvertPyArray", "hcgpuConvertPyInt64", "hcgpuSetRuntimeSearchPaths"} <= set(names)
@@ -54,6 +76,8 @@ def test_builtin_code_objects_are_gfx950_elf_and_hold_the_kernels():
     src = open(os.path.join(ROOT, "hc_amd", "csrc", "runtime.cpp")).read()
     wanted = set(re.findall(r'"(hcamd_[a-z0-9_]+)"', src))
     wanted = {w for w in wanted if not w.endswith("_")}       # prefixes built at run time
+    if not rt.probes_built():                                 # measurement builds: only with --probes
+        wanted = {w for w in wanted if not w.startswith("hcamd_gemm_bf16_probe_")}
     found = set()
     for name, (addr, n) in mods.items():
         blob = C.string_at(addr, n)
