@@ -259,7 +259,8 @@ __device__ __forceinline__ Acc mfma_block(V b, V a, Acc c) {
 // waits or barriers; 2: no wait for the loads at the barrier; 3: no barrier;
 // 4: no LDS operand reads; 5: no loads; 6: the loads fetch into a register
 // instead of LDS; 7: the Bt operand blocks are fetched in MFMA layout straight
-// into registers).  STAGE sends a panel through registers (buffer load, then
+// into registers; 8: the tile is not stored; 9: two K tiles only, i.e. launch,
+// prologue and epilogue without the loop between them).  STAGE sends a panel through registers (buffer load, then
 // ds_write) instead of the load that writes LDS itself.  RS != 0 writes each
 // half-step out in hand order, one fenced slot per MFMA: the LDS reads of the
 // next half-step's operands over the first RS MFMAs, load v of the next tile
@@ -300,7 +301,7 @@ __device__ __forceinline__ void gemm_tile_pipelined(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int wave_m = (wave / WN) * kWaveM;
   const int wave_n = (wave % WN) * kWaveN;
-  const int KT = EDGE ? (K + kBK - 1) / kBK : K / kBK; // host guarantees KT >= 2
+  const int KT = PROBE == 9 ? 2 : EDGE ? (K + kBK - 1) / kBK : K / kBK; // host guarantees KT >= 2
   // EDGE: whole 16-byte chunks of the last K tile that hold data (8 = all)
   const int tail_chunks = EDGE && K % kBK ? (K % kBK) / 8 : 8;
 
@@ -762,7 +763,10 @@ __device__ __forceinline__ void gemm_tile_pipelined(
       const int r = r0 + rr;
       const u32x4 v = *reinterpret_cast<const u32x4 *>(mine + r * kRowB + pc * 16);
       E *dst = C + (size_t)(tm * BM + wave_m + r) * ldc + tn * BN + wave_n + ((pc ^ (r & (kCPR - 1))) * 8);
-      if constexpr (EPI == 2)
+      if constexpr (PROBE == 8) {
+        if (v[0] == 0x7fc07fc1u) // (never: keeps the read of the tile alive)
+          *reinterpret_cast<u32x4 *>(dst) = v;
+      } else if constexpr (EPI == 2)
         __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst));
       else
         *reinterpret_cast<u32x4 *>(dst) = v;
@@ -871,6 +875,8 @@ HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_no_ldsread, 4)
 HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_no_loads, 5)
 HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_loads_to_regs, 6)
 HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_b_direct, __bf16, 256, 256, 2, 4, 16, 2, false, 7)
+HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_no_stores, 8)
+HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_two_tiles, 9)
 #endif
 HCAMD_GEMM_PE(hcamd_gemm_bf16_p256x256_w2x4_edge, __bf16, 256, 256, 2, 4, 16)
 HCAMD_GEMM_PE(hcamd_gemm_f16_p256x256_w2x4_edge, _Float16, 256, 256, 2, 4, 16)

@@ -728,7 +728,7 @@ int hcamdDeviceInfo(OlDevice dev, int *computeUnits, int *clockKHz,
 }
 
 namespace {
-// Variants 17..22 and 26 of "gemm" are measurement builds of the default kernel
+// Variants 17..22, 26, 28 and 29 of "gemm" are measurement builds of the default kernel
 // with one part of its loop taken out: what they leave in C is not the product.
 // They exist only in a library built with HCAMD_PROBES defined (`python -m
 // hc_amd.build --probes`); any other build refuses to select them.
@@ -737,7 +737,8 @@ bool variantIsAbsentProbe(const char *family, int variant) {
   (void)family, (void)variant;
   return false;
 #else
-  return std::strcmp(family, "gemm") == 0 && ((variant >= 17 && variant <= 22) || variant == 26);
+  return std::strcmp(family, "gemm") == 0 &&
+         ((variant >= 17 && variant <= 22) || variant == 26 || variant == 28 || variant == 29);
 #endif
 }
 } // namespace
@@ -3249,6 +3250,8 @@ int launchGemm(OlQueue q, bool half, const void *a, size_t lda, const void *bt,
       {"hcamd_gemm_bf16_p256x256_w2x4_loads_early", 256, 256, 512}, // 25: loads in the first half of the MFMAs
       {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_b_direct"), 256, 256, 512},            // 26: measurement only
       {"hcamd_gemm_bf16_p256x256_w2x2", 256, 256, 256},             // 27: four waves, 128 x 128 each
+      {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_no_stores"), 256, 256, 512}, // 28: measurement only
+      {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_two_tiles"), 256, 256, 512}, // 29: measurement only
   };
   constexpr int kGeneral = 6;
   constexpr int kFirstPipelined = 7; // variants from here need K >= 128

@@ -36,9 +36,10 @@ int hcamdLaunchStream(OlQueue q, int nReads, int writeMode, const void *const *i
                       void *out, size_t bytes) HCAMD_NOEXCEPT;
 
 /* 1 if the library holds the measurement builds of the bf16 GEMM ("gemm"
- * variants 17..22 and 26: the default 256 x 256 kernel with its MFMAs only,
- * without its waits on loads, without its barriers, without its LDS reads,
- * without its loads, with its loads to registers, with B read directly).  What
+ * variants 17..22, 26, 28 and 29: the default 256 x 256 kernel with its MFMAs
+ * only, without its waits on loads, without its barriers, without its LDS
+ * reads, without its loads, with its loads to registers, with B read directly,
+ * without its stores, with two K tiles only).  What
  * those leave in C is NOT the product.  They are compiled only when the
  * library is built with `python -m hc_amd.build --probes` (HCAMD_PROBES); any
  * other build returns 0 here, holds none of them, and hcamdSetVariant /

@@ -48,7 +48,7 @@ def test_measurement_entry_points_have_a_header_of_their_own_and_probes_stay_out
     # a default build holds no kernel whose output is not the product, and
     # refuses the numbers that would select one
     assert b"hcamd_gemm_bf16_probe" not in blob
-    for v in (17, 18, 19, 20, 21, 22, 26):
+    for v in (17, 18, 19, 20, 21, 22, 26, 28, 29):
         assert rt.hcamdSetVariant(b"gemm", v) == 1 and rt.hcamdSetThreadVariant(b"gemm", v) == 1
         with pytest.raises(rt.HcRuntimeError, match="--probes"):
             rt.set_variant("gemm", v)
@@ -272,3 +272,27 @@ def test_product_never_imports_the_oracle():
                 text = open(os.path.join(base, f)).read()
                 assert not re.search(r"^\s*(from|import)\s+oracle\b", text, re.M), f
                 assert "liboracle" not in text, f
+
+
+def test_package_face_leaves_the_simulator_to_the_next_hckernel_on_the_path(tmp_path):
+    """`hckernel/` defines the GPU decorator and the runtime face only; a module it
+    does not define (the reference's kernel_sim, and the kernel_api that module
+    imports relatively) comes from the next `hckernel` directory on the path.
+    (A stand-in directory plays the reference's package here.)"""
+    import subprocess
+    import sys
+    other = tmp_path / "elsewhere" / "hckernel"
+    other.mkdir(parents=True)
+    (other / "__init__.py").write_text("")
+    (other / "kernel_api.py").write_text("WHOSE = 'the other package'\n")
+    (other / "kernel_sim.py").write_text("from .kernel_api import WHOSE\n")
+    (other / "kernel.py").write_text("WHOSE = 'shadowed'\n")
+    code = ("import hckernel.kernel as k, hckernel.kernel_sim as s, hckernel.py_runtime as p\n"
+            "import hc_amd.kernel, hc_amd.py_runtime\n"
+            "assert k.kernel is hc_amd.kernel.kernel and p.runtime_lib is hc_amd.py_runtime.runtime_lib\n"
+            "assert s.WHOSE == 'the other package', s.__file__\n"
+            "import sys; assert not any(m == 'oracle' or m.startswith('oracle.') for m in sys.modules)\n")
+    env = dict(os.environ, PYTHONPATH=os.pathsep.join([ROOT, str(other.parent)]))
+    done = subprocess.run([sys.executable, "-B", "-c", code], env=env, cwd=str(tmp_path),
+                          capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr
