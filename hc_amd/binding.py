@@ -819,9 +819,10 @@ class _MapCompiler:
 
     masked = False                # emit numpy.ma's division rule (element-wise map and its sum only)
     _scalar_mode = False          # the program computes with row scalars (row programs only)
+    _frozen = False               # the stage keeps what numpy.ma leaves in deactivated elements
 
     def _form(self, t: Tile, swapped: bool = False) -> int:
-        if not self._scalar_mode:
+        if not (self._scalar_mode or self._frozen):
             return 0
         return (_FUNC_FORM if t.attrs.get("func") else 0) | (_SWAPPED if swapped else 0)
 
@@ -946,10 +947,10 @@ class _MapCompiler:
                 out.append((rev + "i", flag << 8 | self._form(t, same), _round_to(a.attrs["value"], t.dtype_name)))
             elif _leaf(b) is not None:              # operand forms: one dispatch, no push
                 self.emit(a, out)
-                out.append((fwd + "_in", self.operand(_leaf(b)) | (flag << 8), 0.0))
+                out.append((fwd + "_in", self.operand(_leaf(b)) | (flag << 8) | self._form(t), 0.0))
             elif _leaf(a) is not None:
                 self.emit(b, out)
-                out.append((rev + "_in", self.operand(_leaf(a)) | (flag << 8), 0.0))
+                out.append((rev + "_in", self.operand(_leaf(a)) | (flag << 8) | self._form(t, same), 0.0))
             elif self.need(a) >= self.need(b):
                 self.emit(a, out)
                 self.emit(b, out)
@@ -1458,9 +1459,10 @@ class _RowCompiler(_MapCompiler):
         for a in t.args:
             self.prepare(a, scalar)
 
-    def program(self, t: Tile, scalar: bool = False) -> list:
+    def program(self, t: Tile, scalar: bool = False, frozen: bool = False) -> list:
         self.prepare(t, scalar)
         self._scalar_mode = scalar
+        self._frozen = frozen
         # numpy.ma's rules for / ** sqrt log: in the element-wise stages stores
         # skip, and folds leave out, what they deactivate; a row scalar that they
         # deactivate deactivates every element and every row scalar computed from it
@@ -1568,6 +1570,16 @@ class _RowCompiler(_MapCompiler):
         super().emit(t, out)
 
 
+_PUSHES = ("in", "const", "red", "red0")
+_STACK_BINARY = {n for fwd, rev, _ in _MAP_BINARY.values() for n in (fwd, rev)} | {"mdiv", "rmdiv"}
+
+
+def _is_chain(program) -> bool:
+    """A push, then operations that change that one value in place."""
+    return bool(program) and program[0][0] in _PUSHES and all(
+        name not in _PUSHES and name not in _STACK_BINARY for name, _, _ in program[1:])
+
+
 def match_rows(dst_view, value, n_groups):
     """Elementwise expressions with reductions along the rows, e.g.
     (x - x.mean(axis=1, keepdims=True)) / x.std(axis=1, keepdims=True) or
@@ -1619,11 +1631,26 @@ def match_rows(dst_view, value, n_groups):
     else:
         program = comp.program(value)
         if value.attrs.get("plain") and _maybe_masked(value):
-            if not _values_flow_plainly(value, finite=True):
-                raise NoNativeKernel("the stored value is a bare numpy.ma array, written in full, and "
-                                     "a tile operator follows an operation that can deactivate "
-                                     "elements: what numpy.ma leaves in those has no native code here")
-            program.append(("clear", 0, 0.0))  # a bare numpy.ma array: every value is written
+            # a bare numpy.ma array: every value is written, a deactivated one
+            # with what numpy.ma left in it
+            if _values_flow_plainly(value):
+                program.append(("clear", 0, 0.0))      # plain arithmetic gives those values
+            else:
+                # a tile operator follows an operation that can deactivate: it
+                # leaves its first operand's value there, which a stage that
+                # changes one running value in place can do element by element
+                frozen = comp.program(value, frozen=True)
+                if _is_chain(frozen):
+                    program = frozen + [("frozen", 0, 0.0)]
+                elif _values_flow_plainly(value, finite=True):
+                    # (exact wherever the operands are finite: what can fail here
+                    # fails on values that are not finite already, or by overflow)
+                    program.append(("clear", 0, 0.0))
+                else:
+                    raise NoNativeKernel("the stored value is a bare numpy.ma array, written in full, "
+                                         "and a tile operator follows an operation that can deactivate "
+                                         "elements: what numpy.ma leaves in those is only reproduced "
+                                         "for expressions that update one running value")
         comp.stages.append(("store", 0, program))
     if len(comp.stages) > rt.ROW_MAX_STAGES:
         raise NoNativeKernel(f"the expression needs {len(comp.stages)} passes over the rows "

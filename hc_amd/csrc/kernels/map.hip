@@ -1423,9 +1423,11 @@ __device__ __forceinline__ void reduce_cols(const MapArgs &a, const ColArgs &c, 
       run_program(a, raw, a.f16_mask, r);
       if (row0 + u * kWaves * R + sub < row_end) {
         if (c.masked) { // uniform
+          // (numpy.ma adds up a sum's deactivated elements as +0: a column of them is +0, not the identity -0)
 #pragma unroll
           for (int e = 0; e < kN; ++e)
-            acc[e] = ((r.bad >> e) & 1u) ? acc[e] : col_fold(c.kind, acc[e], r.st[0][e]);
+            acc[e] = ((r.bad >> e) & 1u) ? (c.kind == COL_SUM ? acc[e] + 0.0f : acc[e])
+                                         : col_fold(c.kind, acc[e], r.st[0][e]);
         } else {
 #pragma unroll
           for (int e = 0; e < kN; ++e)
@@ -1573,7 +1575,7 @@ struct Stage {
   uint8_t masked;    // honour the inactive bits: numpy.ma's forms, or a row scalar read that may be deactivated
   uint16_t red_mask; // row scalars this stage reads that may be deactivated
   uint8_t live_pos;  // scalar stages: the result is active iff this row scalar is positive (0xff: not used)
-  uint8_t pad;
+  uint8_t frozen;    // STORE stages: deactivated elements are stored too, with what numpy.ma leaves in them
 };
 
 struct RowArgs {
@@ -1648,16 +1650,103 @@ __device__ __forceinline__ void run_stage(const RowArgs &a, uint32_t begin, uint
   }
 }
 
+// One value as numpy.ma computes with it: the value and whether it is deactivated.
+// The tile operators + - * leave their first operand's value in a deactivated
+// result, the quotient leaves the dividend's, NumPy functions compute on the
+// values regardless (numpy.sqrt and numpy.log put their fill value where the
+// domain fails or the argument is deactivated already).
+struct MaValue {
+  float v;
+  bool dead;
+};
+// `op`: one of the unary opcodes (OP_NEG .. OP_R16, OP_POWCHK, OP_MSQRT, OP_MLOG, OP_MASQRT)
+__device__ __forceinline__ bool ma_is_unary(uint32_t op) {
+  return (op >= OP_NEG && op <= OP_R16) || op == OP_POWCHK || op == OP_MSQRT || op == OP_MLOG ||
+         op == OP_MASQRT;
+}
+__device__ __forceinline__ MaValue ma_unary(uint32_t op, MaValue x) {
+  const float v = x.v;
+  switch (op) {
+  case OP_NEG: return {-v, x.dead};
+  case OP_ABS: return {__builtin_fabsf(v), x.dead};
+  case OP_SQRT: return {__builtin_sqrtf(v), x.dead};
+  case OP_RINT: return {__builtin_rintf(v), x.dead};
+  case OP_EXP: return {expf(v), x.dead};
+  case OP_LOG: return {logf(v), x.dead};
+  case OP_TANH: return {tanh_selects(v), x.dead};
+  case OP_R16: return {round16(v), x.dead};
+  case OP_MSQRT: {
+    const bool out = x.dead || v < 0.0f;
+    return {out ? 0.0f : __builtin_sqrtf(v), out};
+  }
+  case OP_MLOG: {
+    const bool out = x.dead || v <= 0.0f;
+    return {out ? 1.0f : logf(v), out};
+  }
+  case OP_MASQRT: {
+    const float r = __builtin_sqrtf(v);
+    const bool out = x.dead || !is_finite(r) || v < 0.0f;
+    return {out ? v : r, out};
+  }
+  default: { // OP_POWCHK
+    const bool out = !is_finite(v);
+    return {out ? 1e20f : v, x.dead || out};
+  }
+  }
+}
+// `base`: OP_ADD .. OP_RDIV, OP_MDIV, OP_RMDIV with `run` the running value (the
+// deeper stack entry, or the top of an immediate / operand / row-scalar form) and
+// `other` the other operand; `flags`: kFuncForm, kSwapped; `half`: the quotient
+// is rounded to fp16 before it is tested.
+__device__ __forceinline__ MaValue ma_binary(uint32_t base, uint32_t flags, bool half, MaValue run,
+                                             MaValue other) {
+  MaValue l = run, r = other; // first and second operand
+  const bool reversed = base == OP_RSUB || base == OP_RDIV || base == OP_RMDIV;
+  if (reversed || (flags & kSwapped)) {
+    l = other;
+    r = run;
+  }
+  const bool gone = l.dead || r.dead;
+  if (base == OP_MDIV || base == OP_RMDIV) {
+    float q = l.v / r.v;
+    if (half)
+      q = round16(q);
+    const bool good = is_finite(q) && !gone;
+    return {good ? q + 0.0f * l.v : 0.0f + l.v, !good};
+  }
+  float y;
+  switch (base) {
+  case OP_ADD: y = l.v + r.v; break;
+  case OP_SUB:
+  case OP_RSUB: y = l.v - r.v; break;
+  case OP_MUL: y = l.v * r.v; break;
+  case OP_DIV:
+  case OP_RDIV: y = l.v / r.v; break;
+  case OP_MAX: y = nan_max(l.v, r.v); break;
+  default: y = nan_min(l.v, r.v); break;
+  }
+  const bool keeps_first =
+      !(flags & kFuncForm) && (base == OP_ADD || base == OP_SUB || base == OP_RSUB || base == OP_MUL);
+  return {gone && keeps_first ? l.v : y, gone};
+}
+// The plain binary operation behind an immediate, operand or row-scalar form
+// (0: `op` is none of them).
+__device__ __forceinline__ uint32_t ma_base_of(uint32_t op) {
+  if (op >= OP_ADDI && op <= OP_RDIVI) return op - OP_ADDI + OP_ADD;
+  if (op >= OP_ADD_IN && op <= OP_RDIV_IN) return op - OP_ADD_IN + OP_ADD;
+  if (op >= OP_ADD_RED && op <= OP_RDIV_RED) return op - OP_ADD_RED + OP_ADD;
+  if (op == OP_MDIVI || op == OP_MDIV_IN || op == OP_MDIV_RED) return OP_MDIV;
+  if (op == OP_RMDIVI || op == OP_RMDIV_IN || op == OP_RMDIV_RED) return OP_RMDIV;
+  return 0u;
+}
+
 // A stage that computes with row scalars only (SCALAR, STORE_COL), as numpy.ma
 // computes on values that may be deactivated: every stack entry is a value and a
-// "deactivated" bit.  The tile operators + - * leave their first operand's value
-// in a deactivated result, the quotient leaves the dividend's, NumPy functions
-// compute on the values regardless (numpy.sqrt and numpy.log put their fill value
-// where the domain fails or the argument is deactivated already).  What a
-// deactivated row scalar holds matters where it is stored all the same (a per-row
-// result is a bare numpy.ma array, written in full) and where a variance reads a
-// sum whose terms were all inactive.  Everything here is uniform over the lanes
-// of a row.  `dead`: bit k = row scalar k is deactivated.
+// "deactivated" bit.  What a deactivated row scalar holds matters where it is
+// stored all the same (a per-row result is a bare numpy.ma array, written in
+// full) and where a variance reads a sum whose terms were all inactive.
+// Everything here is uniform over the lanes of a row.  `dead`: bit k = row
+// scalar k is deactivated.
 struct ScalarResult {
   float value;
   bool dead;
@@ -1667,13 +1756,15 @@ __device__ __forceinline__ ScalarResult run_scalar_stage(const RowArgs &a, uint3
   float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
   uint32_t dbits = 0; // bit i: stack entry i is deactivated
   int sp = 0;
-  auto get = [&](int i) { return i == 0 ? s0 : i == 1 ? s1 : i == 2 ? s2 : s3; };
-  auto put = [&](int i, float v, bool d) {
-    s0 = i == 0 ? v : s0;
-    s1 = i == 1 ? v : s1;
-    s2 = i == 2 ? v : s2;
-    s3 = i == 3 ? v : s3;
-    dbits = (dbits & ~(1u << i)) | (d ? 1u << i : 0u);
+  auto get = [&](int i) {
+    return MaValue{i == 0 ? s0 : i == 1 ? s1 : i == 2 ? s2 : s3, ((dbits >> i) & 1u) != 0};
+  };
+  auto put = [&](int i, MaValue x) {
+    s0 = i == 0 ? x.v : s0;
+    s1 = i == 1 ? x.v : s1;
+    s2 = i == 2 ? x.v : s2;
+    s3 = i == 3 ? x.v : s3;
+    dbits = (dbits & ~(1u << i)) | (x.dead ? 1u << i : 0u);
   };
 #pragma nounroll
   for (uint32_t pc = begin; pc < end; ++pc) {
@@ -1681,133 +1772,88 @@ __device__ __forceinline__ ScalarResult run_scalar_stage(const RowArgs &a, uint3
     const uint32_t op = cur.op, arg = cur.arg;
     const uint32_t slot = arg & (kMaxRed - 1);
     if (op == OP_CONST) {
-      put(sp++, cur.imm, false);
-      continue;
+      put(sp++, {cur.imm, false});
+    } else if (op == OP_RED || op == OP_RED0) {
+      put(sp++, {cells[slot], op == OP_RED && ((dead >> slot) & 1u)});
+    } else if (ma_is_unary(op)) {
+      if (sp >= 1)
+        put(sp - 1, ma_unary(op, get(sp - 1)));
+    } else if ((op >= OP_ADD && op <= OP_RDIV) || op == OP_MDIV || op == OP_RMDIV) {
+      if (sp >= 2) { // (any `arg` but the form flags marks an fp16 quotient)
+        put(sp - 2, ma_binary(op, arg, (arg & 0x1ffu) != 0, get(sp - 2), get(sp - 1)));
+        --sp;
+      }
+    } else if (const uint32_t base = ma_base_of(op); base != 0 && sp >= 1) {
+      const bool red = op >= OP_ADD_RED;
+      const MaValue other{red ? cells[slot] : cur.imm, red && ((dead >> slot) & 1u)};
+      put(sp - 1, ma_binary(base, arg, (arg & 0x100u) != 0, get(sp - 1), other));
     }
-    if (op == OP_RED || op == OP_RED0) {
-      put(sp++, cells[slot], op == OP_RED && ((dead >> slot) & 1u));
-      continue;
-    }
-    const bool is_unary = (op >= OP_NEG && op <= OP_R16) || op == OP_POWCHK || op == OP_MSQRT ||
-                          op == OP_MLOG || op == OP_MASQRT;
-    if (is_unary) {
-      if (sp < 1)
-        continue;
-      const float v = get(sp - 1);
-      bool d = (dbits >> (sp - 1)) & 1u;
-      float y;
-      switch (op) {
-      case OP_NEG: y = -v; break;
-      case OP_ABS: y = __builtin_fabsf(v); break;
-      case OP_SQRT: y = __builtin_sqrtf(v); break;
-      case OP_RINT: y = __builtin_rintf(v); break;
-      case OP_EXP: y = expf(v); break;
-      case OP_LOG: y = logf(v); break;
-      case OP_TANH: y = tanh_selects(v); break;
-      case OP_R16: y = round16(v); break;
-      case OP_MSQRT: {
-        const bool out = d || v < 0.0f;
-        y = out ? 0.0f : __builtin_sqrtf(v);
-        d = out;
-        break;
-      }
-      case OP_MLOG: {
-        const bool out = d || v <= 0.0f;
-        y = out ? 1.0f : logf(v);
-        d = out;
-        break;
-      }
-      case OP_MASQRT: {
-        const float r = __builtin_sqrtf(v);
-        const bool out = d || !is_finite(r) || v < 0.0f;
-        y = out ? v : r;
-        d = out;
-        break;
-      }
-      default: { // OP_POWCHK
-        const bool out = !is_finite(v);
-        y = out ? 1e20f : v;
-        d = d || out;
-        break;
-      }
-      }
-      put(sp - 1, y, d);
-      continue;
-    }
-    // binary: two stack entries, or the top and an immediate / a row scalar
-    uint32_t base; // OP_ADD .. OP_RDIV, OP_MDIV, OP_RMDIV
-    float other = 0.0f;
-    bool other_dead = false;
-    int at; // where the running value is and the result goes
-    bool half = (arg & 0x100u) != 0; // the quotient is rounded to fp16 before it is tested
-    if ((op >= OP_ADD && op <= OP_RDIV) || op == OP_MDIV || op == OP_RMDIV) {
-      if (sp < 2)
-        continue;
-      base = op;
-      half = (arg & 0x1ffu) != 0;
-      other = get(sp - 1);
-      other_dead = (dbits >> (sp - 1)) & 1u;
-      at = sp - 2;
-      --sp;
-    } else {
-      if (sp < 1)
-        continue;
-      at = sp - 1;
-      if (op >= OP_ADDI && op <= OP_RDIVI) {
-        base = op - OP_ADDI + OP_ADD;
-        other = cur.imm;
-      } else if (op == OP_MDIVI || op == OP_RMDIVI) {
-        base = op - OP_MDIVI + OP_MDIV;
-        other = cur.imm;
-      } else if (op >= OP_ADD_RED && op <= OP_RDIV_RED) {
-        base = op - OP_ADD_RED + OP_ADD;
-        other = cells[slot];
-        other_dead = (dead >> slot) & 1u;
-      } else if (op == OP_MDIV_RED || op == OP_RMDIV_RED) {
-        base = op - OP_MDIV_RED + OP_MDIV;
-        other = cells[slot];
-        other_dead = (dead >> slot) & 1u;
-      } else {
-        continue; // nothing else is valid here (the host has checked)
-      }
-    }
-    float lv = get(at), rv = other; // first and second operand
-    bool ld = (dbits >> at) & 1u, rd = other_dead;
-    const bool reversed = base == OP_RSUB || base == OP_RDIV || base == OP_RMDIV;
-    if (reversed || (arg & kSwapped)) {
-      const float tv = lv;
-      lv = rv, rv = tv;
-      const bool td = ld;
-      ld = rd, rd = td;
-    }
-    const bool gone = ld || rd;
-    float y;
-    bool d = gone;
-    if (base == OP_MDIV || base == OP_RMDIV) {
-      float q = lv / rv;
-      if (half)
-        q = round16(q);
-      const bool good = is_finite(q) && !gone;
-      y = good ? q + 0.0f * lv : 0.0f + lv;
-      d = !good;
-    } else {
-      switch (base) {
-      case OP_ADD: y = lv + rv; break;
-      case OP_SUB:
-      case OP_RSUB: y = lv - rv; break;
-      case OP_MUL: y = lv * rv; break;
-      case OP_DIV:
-      case OP_RDIV: y = lv / rv; break;
-      case OP_MAX: y = nan_max(lv, rv); break;
-      default: y = nan_min(lv, rv); break;
-      }
-      const bool keeps_first = !(arg & kFuncForm) &&
-                               (base == OP_ADD || base == OP_SUB || base == OP_RSUB || base == OP_MUL);
-      y = gone && keeps_first ? lv : y;
-    }
-    put(at, y, d);
   }
   return ScalarResult{s0, (dbits & 1u) != 0};
+}
+
+// A STORE stage that keeps what numpy.ma leaves in deactivated elements (the
+// stored value is a bare numpy.ma array, written in full, and a tile operator
+// follows an operation that can deactivate): the same rules, element by
+// element, for a program that pushes one value and changes it in place.  The
+// host sends only such programs here; their instructions carry the form flags.
+__device__ __forceinline__ void run_frozen_stage(const RowArgs &a, uint32_t begin, uint32_t end,
+                                                 const RawT<kRowN> &raw, StackT<kRowN> &r,
+                                                 const float *cells, uint32_t dead) {
+  float(&v)[kRowN] = r.st[0];
+  uint32_t bad = 0;
+  auto operand = [&](uint32_t i, float *t) {
+    switch (i & 3u) {
+    case 0: unpack(raw, 0, a.f16_mask & 1, t); break;
+    case 1: unpack(raw, 1, a.f16_mask & 2, t); break;
+    case 2: unpack(raw, 2, a.f16_mask & 4, t); break;
+    default: unpack(raw, 3, a.f16_mask & 8, t); break;
+    }
+  };
+#pragma nounroll
+  for (uint32_t pc = begin; pc < end; ++pc) {
+    const Instr cur = a.prog[pc & (kRowProg - 1)];
+    const uint32_t op = cur.op, arg = cur.arg;
+    const uint32_t slot = arg & (kMaxRed - 1);
+    if (op == OP_IN) {
+      operand(arg, v);
+    } else if (op == OP_CONST || op == OP_RED || op == OP_RED0) {
+      const float x = op == OP_CONST ? cur.imm : cells[slot];
+#pragma unroll
+      for (int e = 0; e < kRowN; ++e)
+        v[e] = x;
+      bad = (op == OP_RED && ((dead >> slot) & 1u)) ? ~0u : 0u;
+    } else if (op == OP_CLEAR) {
+      bad = 0;
+    } else if (ma_is_unary(op)) {
+#pragma unroll
+      for (int e = 0; e < kRowN; ++e) {
+        const MaValue y = ma_unary(op, {v[e], ((bad >> e) & 1u) != 0});
+        v[e] = y.v;
+        bad = (bad & ~(1u << e)) | (y.dead ? 1u << e : 0u);
+      }
+    } else if (const uint32_t base = ma_base_of(op); base != 0) {
+      float t[kRowN];
+      bool other_dead = false;
+      if ((op >= OP_ADD_IN && op <= OP_RDIV_IN) || op == OP_MDIV_IN || op == OP_RMDIV_IN) {
+        operand(arg, t);
+      } else {
+        const bool red = op >= OP_ADD_RED;
+        other_dead = red && ((dead >> slot) & 1u);
+#pragma unroll
+        for (int e = 0; e < kRowN; ++e)
+          t[e] = red ? cells[slot] : cur.imm;
+      }
+#pragma unroll
+      for (int e = 0; e < kRowN; ++e) {
+        const MaValue y = ma_binary(base, arg, (arg & 0x100u) != 0, {v[e], ((bad >> e) & 1u) != 0},
+                                    {t[e], other_dead});
+        v[e] = y.v;
+        bad = (bad & ~(1u << e)) | (y.dead ? 1u << e : 0u);
+      }
+    }
+  }
+  r.bad = 0; // every element is stored
 }
 
 // Where a lane stands in its row during pass p.
@@ -1960,14 +2006,17 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
           load_chunk(a, i, bases[i], at, raw.w[i]);
         }
       }
-      run_stage(a, st.begin, st.end, raw, r, reds);
+      if (st.frozen)
+        run_frozen_stage(a, st.begin, st.end, raw, r, cells, dead);
+      else
+        run_stage(a, st.begin, st.end, raw, r, reds);
       // a wave whose lanes all hold whole chunks folds them without masks
       const bool all_whole = __builtin_amdgcn_ballot_w64(at.n_valid != kRowN) == 0;
       if (st.masked) {
         // a stage with numpy.ma's forms, or one that reads a row scalar that may
         // be deactivated (uniform: the host marks it): elements that a division
         // or a domain function deactivated are neither stored nor folded
-        if (row_gone)
+        if (row_gone && !st.frozen)
           r.bad = ~0u;
         const bool whole_chunk = kind == ST_STORE && ((a.vec_mask >> 8) & 1) && at.n_valid == kRowN &&
                                  r.bad == 0;
@@ -2406,7 +2455,8 @@ __device__ __forceinline__ void layer_norm_rows(const void *__restrict__ x, size
                                                 const float *__restrict__ w,
                                                 const float *__restrict__ b,
                                                 void *__restrict__ out, size_t ldo,
-                                                uint32_t rows, uint32_t cols, float n, float eps) {
+                                                uint32_t rows, uint32_t cols, float n, float eps,
+                                                uint32_t frozen) {
   constexpr int T = LPR < 256 ? 256 : LPR, RPW = T / LPR, W = LPR / kWave;
   constexpr int C = HALF ? 8 : 4; // elements of a 16-byte chunk
   __shared__ float slots[2][RPW][W];
@@ -2462,8 +2512,11 @@ __device__ __forceinline__ void layer_norm_rows(const void *__restrict__ x, size
   const float s = __builtin_sqrtf(__fadd_rn(mean_sq, eps));
   // The mean is numpy.ma's quotient: one that is not finite is deactivated, and
   // with it every element computed from it (the variance of such a row is an
-  // active 0, but the row's x - mean are all inactive).
-  if (!live || !is_finite(RMS ? mean_sq : mean))
+  // active 0, but the row's x - mean are all inactive).  `frozen` (the stored
+  // expression is a bare numpy.ma array, written in full): deactivated
+  // elements are stored too, with what numpy.ma leaves in them, the dividend.
+  const bool row_gone = !is_finite(RMS ? mean_sq : mean);
+  if (!live || (row_gone && !frozen))
     return;
   char *orow = static_cast<char *>(out) + (size_t)row * ldo * (HALF ? 2 : 4);
 #pragma unroll
@@ -2487,10 +2540,18 @@ __device__ __forceinline__ void layer_norm_rows(const void *__restrict__ x, size
       for (int k = 0; k < C; ++k)
         y[k] = RMS ? v[e][k] : __fsub_rn(v[e][k], mean);
       uint32_t bad = 0;
-      masked_div_scalar<C, false>(bad, y, s, false);
+      float kept[C];
 #pragma unroll
       for (int k = 0; k < C; ++k)
+        kept[k] = 0.0f + y[k];
+      masked_div_scalar<C, false>(bad, y, s, false);
+      bad = row_gone ? ~0u : bad;
+#pragma unroll
+      for (int k = 0; k < C; ++k) {
         y[k] = RMS ? __fmul_rn(y[k], wv[k]) : __fadd_rn(__fmul_rn(y[k], wv[k]), bv[k]);
+        y[k] = frozen && ((bad >> k) & 1u) ? kept[k] : y[k];
+      }
+      bad = frozen ? 0u : bad;
       if constexpr (HALF) {
         _Float16 *oh = reinterpret_cast<_Float16 *>(orow);
         if (bad == 0) {
@@ -2523,8 +2584,8 @@ __device__ __forceinline__ void layer_norm_rows(const void *__restrict__ x, size
 #define HCAMD_NORM_KERNEL(NAME, LPR, E, RMS, HALF)                                        \
   extern "C" __global__ __launch_bounds__(LPR < 256 ? 256 : LPR) void NAME(               \
       const void *x, size_t ld, const float *w, const float *b, void *out, size_t ldo,    \
-      uint32_t rows, uint32_t cols, float n, float eps) {                                 \
-    layer_norm_rows<LPR, E, RMS, HALF>(x, ld, w, b, out, ldo, rows, cols, n, eps);        \
+      uint32_t rows, uint32_t cols, float n, float eps, uint32_t frozen) {                \
+    layer_norm_rows<LPR, E, RMS, HALF>(x, ld, w, b, out, ldo, rows, cols, n, eps, frozen); \
   }
 #define HCAMD_LAYER_NORM(LPR, E)                                                          \
   HCAMD_NORM_KERNEL(hcamd_layer_norm_f32_w##LPR##_e##E, LPR, E, false, false)             \

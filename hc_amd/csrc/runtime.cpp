@@ -2009,7 +2009,7 @@ struct RowStageDev {
   uint8_t masked;   // honour the inactive bits: numpy.ma's forms, or a row scalar read that may be deactivated
   uint16_t redMask; // row scalars this stage reads that may be deactivated
   uint8_t livePos;  // scalar stages: the result is active iff this row scalar is positive (0xff: not used)
-  uint8_t pad;
+  uint8_t frozen;   // STORE stages: deactivated elements are stored too, with what numpy.ma leaves in them
 };
 struct RowArgs {
   const void *in[kMapMaxIn];
@@ -2147,6 +2147,16 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       a.stage[s].livePos = static_cast<uint8_t>(index);
       --stageEnd;
     }
+    bool frozen = false;
+    if (prog[stageEnd - 1].op == HCAMD_MAP_FROZEN) {
+      if (st.kind != HCAMD_ROW_STORE || st.nInstr < 2) {
+        dev->report("%s: stage %zu: FROZEN closes a STORE stage", who, s);
+        return 1;
+      }
+      frozen = true;
+      a.stage[s].frozen = 1;
+      --stageEnd;
+    }
     for (size_t i = pc; i < stageEnd; ++i) {
       const unsigned op = prog[i].op;
       int pops, pushes;
@@ -2169,7 +2179,7 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       const bool readsOperand = op == HCAMD_MAP_IN || maskedIn ||
                                 (op >= HCAMD_MAP_ADD_IN && op <= HCAMD_MAP_RDIV_IN);
       // (bits 8 and up of `arg` are flags: fp16, and in scalar stages the form of the operation)
-      const unsigned index = (maskedIn || red) ? prog[i].arg & 0xffu : prog[i].arg;
+      const unsigned index = (maskedIn || red || frozen) ? prog[i].arg & 0xffu : prog[i].arg;
       if (readsOperand) {
         if (!perElement || index >= nInputs) {
           dev->report("%s: operand %u at %zu (%zu given; scalar stages read none)", who,
@@ -2182,8 +2192,8 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
         dev->report("%s: opcode %u at %zu outside a scalar stage", who, op, i);
         return 1;
       }
-      if (perElement && !red && !maskedIn && (prog[i].arg & ~0x1ffu)) {
-        dev->report("%s: flags 0x%x at %zu outside a scalar stage", who, prog[i].arg, i);
+      if (perElement && !frozen && !red && !maskedIn && (prog[i].arg & ~0x1ffu)) {
+        dev->report("%s: flags 0x%x at %zu outside a scalar or frozen stage", who, prog[i].arg, i);
         return 1;
       }
       if (red && (index >= HCAMD_ROW_MAX_SCALARS || !((written >> index) & 1))) {
@@ -2197,8 +2207,8 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
         return 1;
       }
       sp += pushes - pops;
-      if (sp > kMapDepth) {
-        dev->report("%s: stack deeper than %d at %zu", who, kMapDepth, i);
+      if (sp > (frozen ? 1 : kMapDepth)) {
+        dev->report("%s: stack deeper than %d at %zu", who, frozen ? 1 : kMapDepth, i);
         return 1;
       }
     }
@@ -2211,7 +2221,7 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
     a.stage[s].kind = static_cast<uint8_t>(st.kind);
     a.stage[s].dst = static_cast<uint8_t>(st.dst);
     a.stage[s].redMask = static_cast<uint16_t>(readsDeadable);
-    a.stage[s].masked = (hasForms || readsDeadable) ? 1 : 0;
+    a.stage[s].masked = (hasForms || readsDeadable || frozen) ? 1 : 0;
     const bool canDie = (stores || st.kind == HCAMD_ROW_COUNT) ? false
                         : perElement                           ? (hasForms || readsDeadable)
                                                    : (hasForms || readsDeadable || a.stage[s].livePos != 0xff);
@@ -2220,7 +2230,8 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       deadable = canDie ? deadable | (1u << st.dst) : deadable & ~(1u << st.dst);
     }
     // (a STORE_COL stage that can fail stores what numpy.ma leaves: the scalar interpreter's business too)
-    tracking = tracking || canDie || st.kind == HCAMD_ROW_COUNT || (!perElement && (hasForms || readsDeadable));
+    tracking = tracking || canDie || frozen || st.kind == HCAMD_ROW_COUNT ||
+               (!perElement && (hasForms || readsDeadable));
     pc += st.nInstr;
   }
   std::memcpy(a.prog, prog, pc * sizeof(HcamdMapInstr));
@@ -2310,7 +2321,7 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       return prog[at].op == op && prog[at].arg == arg;
     };
     auto launchNorm = [&](bool rmsForm, const void *x, size_t ldx, const void *w, const void *b,
-                          float n, float eps, bool half = false) {
+                          float n, float eps, bool half = false, uint32_t frozen = 0) {
       const size_t chunks = cols / (half ? 8 : 4);
       // two chunks to a lane on up to 512 lanes, then four; 1024 lanes from 2048 chunks on
       size_t lpr = 64, e = chunks <= 64 ? 1 : 2;
@@ -2325,7 +2336,7 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       const size_t t = std::max(lpr, (size_t)256);
       size_t ldOut = ldo;
       uint32_t nRows = static_cast<uint32_t>(rows), nCols = static_cast<uint32_t>(cols);
-      void *args[] = {&x, &ldx, &w, &b, &out, &ldOut, &nRows, &nCols, &n, &eps};
+      void *args[] = {&x, &ldx, &w, &b, &out, &ldOut, &nRows, &nCols, &n, &eps, &frozen};
       return launch1d(queue, "map", name, ceilDiv(rows, t / lpr), t, args);
     };
     auto stage = [&](size_t s, unsigned kind, unsigned dst, unsigned n) {
@@ -2366,16 +2377,19 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       return launchNorm(true, inputs[0], inputLd[0], inputs[1], inputs[1], prog[3].imm, prog[4].imm);
     // The same on fp16 rows, computed in fp32 and stored as fp16 (the program
     // then ends in R16); w stays fp32.
+    // (with FROZEN at the end when the body computes from x.astype(float32), a
+    // bare numpy.ma array: every element is stored, a deactivated one as x)
+    const bool rmsFrozen = pc == 11 && prog[10].op == HCAMD_MAP_FROZEN;
     const bool rmsHalf =
-        variantOf("rows") == 0 && nStages == 3 && nInputs == 2 && nColumns == 0 && pc == 10 &&
-        stage(0, HCAMD_ROW_SUM, 0, 2) && stage(1, HCAMD_ROW_SCALAR, 1, 4) &&
-        stage(2, HCAMD_ROW_STORE, 0, 4);
+        variantOf("rows") == 0 && nStages == 3 && nInputs == 2 && nColumns == 0 &&
+        (pc == 10 || rmsFrozen) && stage(0, HCAMD_ROW_SUM, 0, 2) && stage(1, HCAMD_ROW_SCALAR, 1, 4) &&
+        stage(2, HCAMD_ROW_STORE, 0, rmsFrozen ? 5 : 4);
     if (rmsHalf && is(0, HCAMD_MAP_IN, 0) && is(1, HCAMD_MAP_MUL_IN, 0) && rmsScale &&
         is(6, HCAMD_MAP_IN, 0) && is(7, HCAMD_MAP_MDIV_RED, 1) && is(8, HCAMD_MAP_MUL_IN, 1) &&
-        prog[9].op == HCAMD_MAP_R16 && a.f16Mask == 0x101u && inputLd[0] != 0 && inputLd[1] == 0 &&
+        is(9, HCAMD_MAP_R16, 0) && a.f16Mask == 0x101u && inputLd[0] != 0 && inputLd[1] == 0 &&
         (a.vecMask & 0x103u) == 0x103u && cols % 8 == 0 && cols <= 65536)
       return launchNorm(true, inputs[0], inputLd[0], inputs[1], inputs[1], prog[3].imm, prog[4].imm,
-                        true);
+                        true, rmsFrozen ? 1u : 0u);
   }
   // Rows of whole, aligned chunks, at most 4096 of them, whose stages are all
   // chains run on the chain kernels: a lane has its whole part of the row at

@@ -690,9 +690,10 @@ class Tile:
         o = Tile.wrap(other)
         a, b = (o, self) if reflected else (self, o)
         r = Tile(op, (a, b), _broadcast(a.shape, b.shape), _result_dtype(a, b))
-        if a.attrs.get("plain"):
+        if a.attrs.get("plain") or (a.op == "const" and b.attrs.get("plain")):
             # the left operand is what a NumPy function returned: in the reference a
-            # bare numpy.ma array, whose operator gives another one (stored in full)
+            # bare numpy.ma array, whose operator gives another one (stored in full);
+            # so does the reflected operator of a bare array next to a number
             r.attrs["plain"] = True
         return r
 
@@ -914,9 +915,11 @@ class Tile:
 
     def astype(self, dt):
         name = dtype_name(dt)
-        if name == self.dtype_name:
+        if name == self.dtype_name and self.attrs.get("plain"):
             return self
-        return Tile("astype", (self,), self.shape, name, **self._plain_kw())
+        # (a tile's astype is numpy.ma's, python/hckernel/kernel_api.py:150-151:
+        # the result is a bare numpy.ma array, not a tile)
+        return Tile("astype", (self,), self.shape, name, plain=True)
 
     @property
     def T(self):

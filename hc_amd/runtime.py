@@ -527,7 +527,10 @@ MAP_OPS.update({"red": 45, "add_red": 46, "sub_red": 47, "mul_red": 48, "div_red
                 "mdiv_red": 54, "rmdiv_red": 55,
                 # push a row scalar as a value, deactivated or not; numpy.ma.sqrt;
                 # (last in a stage) the result is active iff row scalar `arg` is positive
-                "red0": 56, "masqrt": 57, "livepos": 58})
+                "red0": 56, "masqrt": 57, "livepos": 58,
+                # (last in a STORE stage) every element is stored, a deactivated
+                # one with the value numpy.ma leaves in it
+                "frozen": 59})
 ROW_KINDS = {"sum": 0, "max": 1, "min": 2, "scalar": 3, "store": 4, "store_col": 5, "count": 6}
 ROW_MAX_STAGES, ROW_MAX_SCALARS, ROW_MAX_INSTRS = 16, 16, 128
 F32, F16, BF16 = 0, 1, 2

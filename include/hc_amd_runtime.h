@@ -520,7 +520,12 @@ int hcamdLaunchMapReduceColsNoAlloc(OlQueue q, int kind, const HcamdMapInstr *pr
  * result that is not finite deactivates and leaves the argument);
  * HCAMD_MAP_LIVEPOS, as the last instruction of a SCALAR stage, replaces the
  * result's activity: active iff row scalar `arg` is positive (a variance is
- * active where count - ddof is).
+ * active where count - ddof is).  HCAMD_MAP_FROZEN, as the last instruction of
+ * a STORE stage, makes that stage store every element, a deactivated one with
+ * the value numpy.ma leaves in it (the stored expression is a bare numpy.ma
+ * array and a tile operator follows an operation that can deactivate): the
+ * stage's program must push one value and change it in place, and its
+ * instructions carry the two form flags like those of SCALAR stages.
  * Operands: `inputs` are rows x cols tiles with a leading dimension in elements,
  * or, with leading dimension 0, one vector of cols elements used for every row;
  * `columns` hold one value per row and fill row scalars 0 .. nColumns-1.
@@ -571,7 +576,8 @@ enum {
   HCAMD_MAP_RMDIV_RED = 55, /* scalar / top */
   HCAMD_MAP_RED0 = 56,    /* SCALAR / STORE_COL stages: push row scalar `arg`, deactivated or not */
   HCAMD_MAP_MASQRT = 57,  /* SCALAR / STORE_COL stages: numpy.ma.sqrt */
-  HCAMD_MAP_LIVEPOS = 58  /* closes a SCALAR stage: active iff row scalar `arg` > 0 */
+  HCAMD_MAP_LIVEPOS = 58, /* closes a SCALAR stage: active iff row scalar `arg` > 0 */
+  HCAMD_MAP_FROZEN = 59   /* closes a STORE stage: every element is stored (see above) */
 };
 #define HCAMD_ROW_MAX_STAGES 16
 #define HCAMD_ROW_MAX_SCALARS 16

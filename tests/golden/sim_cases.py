@@ -459,6 +459,16 @@ def case_masked_reductions(api):
         "layernorm": lambda ta, tb: (ta - ta.mean(axis=1, keepdims=True)) /
         np.sqrt(ta.var(axis=1, keepdims=True) + f(1e-5)) * tb,
         "over_max": lambda ta, tb: ta / (ta / tb).max(axis=1, keepdims=True),
+        # tile.astype gives a bare numpy.ma array: what is computed from it is
+        # stored in full, deactivated elements with what numpy.ma leaves in them
+        "bare_scaled_quotient": lambda ta, tb: (ta.astype(f) / tb.astype(f)) * f(3) - f(1),
+        "bare_rms": lambda ta, tb: ta.astype(f) / np.sqrt(np.mean(np.square(ta.astype(f)), axis=1, keepdims=True)
+                                                          + f(1e-6)) * tb.astype(f),
+        "bare_centre_over_sum": lambda ta, tb: (ta.astype(f) - ta.astype(f).mean(axis=1, keepdims=True)) /
+        tb.astype(f).sum(axis=1, keepdims=True),
+        "bare_one_minus_quotient": lambda ta, tb: f(1) - ta.astype(f) / tb.astype(f),
+        "bare_python_one_minus_quotient": lambda ta, tb: 1.0 - ta.astype(f) / tb.astype(f),
+        "bare_sqrt_of_quotient": lambda ta, tb: np.sqrt(ta.astype(f) / tb.astype(f)) + f(2),
         "col_centre": lambda ta, tb: ta - ta.mean(axis=0, keepdims=True),
         "col_over_sum": lambda ta, tb: ta / tb.sum(axis=0, keepdims=True),
     }

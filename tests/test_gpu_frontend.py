@@ -774,19 +774,25 @@ def test_reductions_over_deactivated_elements_follow_numpy_ma_on_the_gpu(rows, n
             sim[name][0](a, b, want, 8)
         out = rt.to_device(np.full(shape, POISON))
         body(da, db, out, 8)
-        assert rt.last_kernel_name().startswith("hcamd_row_program_w"), (name, rt.last_kernel_name())
+        elementwise = name in ("bare_scaled_quotient", "bare_one_minus_quotient",
+                               "bare_python_one_minus_quotient", "bare_sqrt_of_quotient")
+        assert rt.last_kernel_name().startswith(("hcamd_fmap", "hcamd_map") if elementwise
+                                                else "hcamd_row_program_w"), (name, rt.last_kernel_name())
         got = out.to_host()
         assert_array_equal(got == POISON, want == POISON, err_msg=name)
         assert_array_equal(np.isnan(got), np.isnan(want), err_msg=name)
         assert_allclose(got, want, rtol=1e-4, atol=1e-5, err_msg=name)
 
 
-@pytest.mark.parametrize("name", ["layernorm"])
+@pytest.mark.parametrize("name", ["layernorm", "rmsnorm_half"])
 @pytest.mark.parametrize("rows,n", [(64, 4096), (37, 200), (5, 20_003)])
-def test_normalisations_leave_rows_with_a_mean_that_is_not_finite_alone(name, rows, n):
-    """numpy.ma's mean of a row with an inf or a NaN is deactivated: nothing of
-    that row is stored, by the kernels of their own (dense rows of whole
-    chunks) as by the general one."""
+def test_normalisations_of_rows_with_a_mean_that_is_not_finite(name, rows, n):
+    """numpy.ma's mean of a row with an inf or a NaN is deactivated.  The layer
+    normalisation computes from a tile: nothing of such a row is stored.  The
+    root-mean-square one computes from x.astype(float32), a bare numpy.ma
+    array, and is written in full: such a row gets what numpy.ma leaves in a
+    deactivated quotient, the dividend x.  The kernels of their own (dense rows
+    of whole chunks) and the general one do the same."""
     from test_kernel_frontend import _row_bodies, _row_case
     host = _row_case(name, rows, n, seed=rows)
     x = host[0]
@@ -798,8 +804,13 @@ def test_normalisations_leave_rows_with_a_mean_that_is_not_finite_alone(name, ro
     out = rt.to_device(np.full(host[-1].shape, -77, host[-1].dtype))
     _row_bodies(kernel)[name](*[rt.to_device(v) for v in host[:-1]], out, 8)
     got = out.to_host()
-    assert (want[1] == -77).all() and (want[2] == -77).all() and (want[0] != -77).all()
+    if name == "layernorm":
+        assert (want[1] == -77).all() and (want[2] == -77).all() and (want[0] != -77).all()
+    else:
+        assert_array_equal(want[1].view(np.uint16), x[1].view(np.uint16))
+        assert_array_equal(want[2].view(np.uint16), x[2].view(np.uint16))
     assert_array_equal(got == -77, want == -77)
+    assert_array_equal(np.isnan(got), np.isnan(want))
     if got.dtype == np.float16:
         assert_allclose(got.astype(np.float32), want.astype(np.float32), rtol=1.1e-3)
     else:

@@ -840,9 +840,15 @@ def run_row_stages(stages, inputs, columns=(), out_dtype=np.float32, init=None):
             stack = []                    # values; scalar stages: (value, dead)
             bad = np.zeros((rows, n), bool)
             live_slot = None
+            # a frozen stage keeps what numpy.ma leaves in deactivated elements
+            # (one running value; the instructions carry the form flags)
+            frozen = program[-1][0] == "frozen"
             for name, arg, imm in program:
                 if name == "livepos":
                     live_slot = arg & 0xff
+                    continue
+                if name == "frozen":
+                    bad[:] = False
                     continue
                 if scalar_stage:
                     half, func, swapped = bool(arg & 0x100), bool(arg & FUNC), bool(arg & SWAPPED)
@@ -903,7 +909,10 @@ def run_row_stages(stages, inputs, columns=(), out_dtype=np.float32, init=None):
                 elif name in unary:
                     stack.append(unary[name](stack.pop()).astype(f))
                 elif name in ("msqrt", "mlog", "powchk"):
-                    v, failed = domain(name, stack.pop())
+                    x = stack.pop()
+                    if frozen and name != "powchk":
+                        x = np.where(bad, f(-1), x)       # deactivated already: the fill value too
+                    v, failed = domain(name, x)
                     stack.append(v)
                     bad |= failed
                 elif name in ("add", "sub", "mul", "div", "max", "min", "rsub", "rdiv", "mdiv", "rmdiv"):
@@ -923,17 +932,23 @@ def run_row_stages(stages, inputs, columns=(), out_dtype=np.float32, init=None):
                     if form == "i":
                         b = np.full((rows, n), imm, f)
                     elif form == "_red":
-                        b = np.broadcast_to(red[arg & 0xff][0], (rows, n))
-                        bad |= red[arg & 0xff][1]
+                        b = np.broadcast_to(red[arg & 0xf][0], (rows, n))
+                        bad = bad | red[arg & 0xf][1]
                     else:
-                        b = np.broadcast_to(inputs[arg & 0xff].astype(f), (rows, n))
+                        b = np.broadcast_to(inputs[arg & 0x3].astype(f), (rows, n))
                     if op.startswith("r"):
                         op, a, b = op[1:], b, a
+                    elif frozen and arg & SWAPPED:
+                        a, b = b, a
                     if op == "mdiv":
                         v, failed = quotient(a, b, half)
-                        bad |= failed
+                        if frozen:
+                            v = np.where(bad, f(0) + a, v)
+                        bad = bad | failed
                     else:
                         v = plain[op](a, b).astype(f)
+                        if frozen and not arg & FUNC and op in ("add", "sub", "mul"):
+                            v = np.where(bad, a, v)           # numpy.ma keeps the first operand's value
                     stack.append(v)
             (top,) = stack
             if scalar_stage:
@@ -1137,6 +1152,17 @@ def _masked_row_bodies(deco):
         "zscore": zscore,
         "square_of_sum": lambda ta, tb: ta * (tb * f(1e10)).sum(axis=1, keepdims=True) ** 2,
         "over_max": lambda ta, tb: ta / (ta / tb).max(axis=1, keepdims=True),
+        # tile.astype gives a bare numpy.ma array: what is computed from it is stored in
+        # full, deactivated elements with what numpy.ma leaves in them
+        "bare_scaled_quotient": lambda ta, tb: (ta.astype(f) / tb.astype(f)) * f(3) - f(1),
+        "bare_rms": lambda ta, tb: ta.astype(f) / np.sqrt(np.mean(np.square(ta.astype(f)), axis=1, keepdims=True)
+                                                          + f(1e-6)) * tb.astype(f),
+        "bare_centre_over_sum": lambda ta, tb: (ta.astype(f) - ta.astype(f).mean(axis=1, keepdims=True)) /
+        tb.astype(f).sum(axis=1, keepdims=True),
+        "bare_one_minus_quotient": lambda ta, tb: f(1) - ta.astype(f) / tb.astype(f),
+        "bare_python_one_minus_quotient": lambda ta, tb: 1.0 - ta.astype(f) / tb.astype(f),
+        "bare_sqrt_of_quotient": lambda ta, tb: np.sqrt(ta.astype(f) / tb.astype(f)) + f(2),
+        "bare_quotient_over_row_sum": lambda ta, tb: tb.astype(f) / ta.astype(f).sum(axis=1, keepdims=True) * ta,
     }
     rows = {
         "mean": lambda ta, tb: (ta / tb).mean(axis=1),
@@ -1199,6 +1225,13 @@ def test_reductions_over_deactivated_elements_follow_numpy_ma(ctx, rows, n):
             sim[name][0](a, b, want, 8)
         fake = [FakeDev(a.shape, "float32"), FakeDev(b.shape, "float32"), FakeDev(shape, "float32")]
         (p,) = body.plan(*fake, 8, ctx=ctx)
+        if p.fn is not rt.hcamdLaunchRowProgram:
+            # no reduction in the body: the fast map where the values flow plainly, else the
+            # general float map, which tracks activity per operand (their parity is a GPU test)
+            assert p.fn in (rt.hcamdLaunchFMap, rt.hcamdLaunchMap) and name in (
+                "bare_scaled_quotient", "bare_one_minus_quotient", "bare_python_one_minus_quotient",
+                "bare_sqrt_of_quotient"), name
+            continue
         by_ptr = {fake[0].ptr: a, fake[1].ptr: b}
         operands = [by_ptr[p.args[4][i]] for i in range(p.args[7])]      # in the order of first use
         with np.errstate(all="ignore"):
