@@ -1052,7 +1052,7 @@ def match_imap(dst_view, value, n_groups):
         operation whose operands may be exchanged evaluates the deeper one first)."""
         if id(t) in needs:
             return needs[id(t)]
-        if _is(t, "astype", 1) or (t.op in _IMAP_UNARY and len(t.args) == 1):
+        if _is(t, "astype", 1) or _is(t, "active", 1) or (t.op in _IMAP_UNARY and len(t.args) == 1):
             n = need(t.args[0])
         elif t.op in _IMAP_BINARY and len(t.args) == 2:
             a, b = need(t.args[0]), need(t.args[1])
@@ -1098,8 +1098,18 @@ def match_imap(dst_view, value, n_groups):
             return ok
         if _is(t, "astype", 1) and t.dtype_name == "int32" and t.args[0].dtype_name == "bool":
             return emit(t.args[0])                 # 0 / 1 as int32: the same bits
+        if _is(t, "active", 1):
+            # tile.mask: the kernel keeps one activity flag per element, that of
+            # the whole expression so far, so the mask is taken of a whole expression
+            if t is not top_active:
+                raise NoNativeKernel("tile.mask inside a larger integer expression has no native code "
+                                     "(the mask of the stored expression has)")
+            ok = emit(t.args[0])
+            program.append(("active", 0, 0))
+            return ok
         return False
 
+    top_active = value.args[0] if _is(value, "astype", 1) and _is(value.args[0], "active", 1) else value
     is_cmp = value.dtype_name == "bool"
     if value.dtype_name not in ("int32", "bool") or (out_dt == "bool") != is_cmp and out_dt == "bool":
         return None
@@ -1197,6 +1207,10 @@ def match_fmap(dst_view, value, n_groups):
             ok = emit(src)
             if half and src.dtype_name == "float32":
                 program.append(("r16", 0, 0.0))
+            return ok
+        if _is(t, "active", 1):
+            ok = emit(t.args[0])                   # tile.mask: the entry's activity as 0 / 1
+            program.append(("active", 0, 0.0))
             return ok
         if _is(t, "clip", 1):
             ok = emit(t.args[0])

@@ -31,6 +31,8 @@
 //     it is inactive), FOP_POWCHK what numpy.ma.power does afterwards: a result
 //     that is not finite becomes inactive with the value 1e20.
 //   * comparisons give 0 / 1 and are false for NaN except !=.
+//   * FOP_ACTIVE is `tile.mask`: 1 where the element is active, 0 where not, a
+//     plain array (every element active again).
 // The store skips inactive elements, or with store_all writes every value: a
 // NumPy function returns a bare numpy.ma array, which the reference's store
 // copies in full.
@@ -53,6 +55,7 @@ enum : uint32_t {
   FOP_LT = 12, FOP_LE = 13, FOP_EQ = 14, FOP_NE = 15, FOP_GE = 16, FOP_GT = 17,
   FOP_NEG = 18, FOP_ABS = 19, FOP_SQRT = 20, FOP_RINT = 21, FOP_EXP = 22, FOP_LOG = 23,
   FOP_R16 = 24, FOP_PSQRT = 25, FOP_POWCHK = 26,
+  FOP_ACTIVE = 27, // `tile.mask`: 1 where the element is active in the entry, else 0; active again
 };
 
 struct Instr {
@@ -184,6 +187,11 @@ __device__ __forceinline__ float unary(uint32_t op, float a, bool &ok) {
   case FOP_EXP: return expf(a);
   case FOP_R16: return round16(a);
   case FOP_PSQRT: return ok ? __builtin_sqrtf(a) + 0.0f : a; // pow(-0, 0.5) is +0
+  case FOP_ACTIVE: {
+    const float r = ok ? 1.0f : 0.0f;
+    ok = true;
+    return r;
+  }
   default: // FOP_POWCHK
     if (!finite(a)) {
       ok = false;

@@ -33,6 +33,7 @@ enum : uint32_t {
   IOP_AND = 10, IOP_OR = 11, IOP_XOR = 12, IOP_SHL = 13, IOP_SHR = 14,
   IOP_LT = 15, IOP_LE = 16, IOP_EQ = 17, IOP_NE = 18, IOP_GE = 19, IOP_GT = 20,
   IOP_NEG = 21, IOP_ABS = 22, IOP_NOT = 23, IOP_LNOT = 24,
+  IOP_ACTIVE = 25, // 1 where the element is still active, else 0; the element is active again
 };
 
 struct Instr {
@@ -162,6 +163,14 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_imap_i32(IMapArgs a) {
         if (op == IOP_IN)
           x = arg == 0 ? v[0][e] : arg == 1 ? v[1][e] : arg == 2 ? v[2][e] : v[3][e];
         t0[e] = x;
+      }
+    } else if (op == IOP_ACTIVE) {
+      // `tile.mask`: a plain array of which elements are active, every one of
+      // them a value that is stored
+#pragma unroll
+      for (int e = 0; e < kV; ++e) {
+        t0[e] = ok[e] ? 1 : 0;
+        ok[e] = true;
       }
     } else if (op >= IOP_NEG) {
 #pragma unroll

@@ -703,8 +703,16 @@ class Tile:
     def __rsub__(self, o): return self._binary(o, "sub", True)
     def __mul__(self, o): return self._binary(o, "mul")
     def __rmul__(self, o): return self._binary(o, "mul", True)
-    def __truediv__(self, o): return self._binary(o, "div")
-    def __rtruediv__(self, o): return self._binary(o, "div", True)
+    def __truediv__(self, o): return self._true_divide(o, False)
+    def __rtruediv__(self, o): return self._true_divide(o, True)
+
+    def _true_divide(self, o, reflected):
+        r = self._binary(o, "div", reflected)
+        if _RANK[r.dtype_name] < 5:
+            raise TraceError("tile / tile on integer tiles is float64 in NumPy, for which there is no "
+                             "native kernel (use // for the integer quotient)")
+        return r
+
     def __neg__(self): return Tile("neg", (self,), self.shape, self.dtype_name, **self._plain_kw())
     def __abs__(self): return Tile("abs", (self,), self.shape, self.dtype_name, **self._plain_kw())
 
@@ -752,12 +760,18 @@ class Tile:
 
     @property
     def mask(self):
-        raise TraceError("tile.mask: which elements are active depends on the data (division by "
-                         "zero) and on the group; it is not available while the body is traced")
+        """Which elements are active (True = active: the reference inverts
+        numpy.ma's polarity, python/hckernel/kernel_api.py:117-119).  A plain
+        bool array, every element of which is a value: stored in full."""
+        if self.attrs.get("plain"):
+            raise TraceError("the mask of a bare numpy.ma array (the result of a NumPy function, a "
+                             "reduction or astype) has numpy.ma's polarity, not a tile's: no native code")
+        return Tile("active", (self,), self.shape, "bool", plain=True)
 
     def compressed(self):
-        raise TraceError("tile.compressed(): the number of active elements is not known while the "
-                         "body is traced")
+        raise TraceError("tile.compressed(): a 1-D array of the active elements only; its length "
+                         "depends on the data, which a traced body cannot express (store the tile "
+                         "and tile.mask instead)")
 
     def __matmul__(self, o):
         return _dot(self, Tile.wrap(o))

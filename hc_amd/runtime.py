@@ -606,7 +606,8 @@ def plan_map_sum(program, inputs, cell, index: int = 0, types=None) -> Plan:
 U8 = 5
 IMAP_OPS = {"in": 1, "const": 2, "add": 3, "sub": 4, "mul": 5, "floordiv": 6, "mod": 7, "min": 8,
             "max": 9, "and": 10, "or": 11, "xor": 12, "shl": 13, "shr": 14, "lt": 15, "le": 16,
-            "eq": 17, "ne": 18, "ge": 19, "gt": 20, "neg": 21, "abs": 22, "not": 23, "lnot": 24}
+            "eq": 17, "ne": 18, "ge": 19, "gt": 20, "neg": 21, "abs": 22, "not": 23, "lnot": 24,
+            "active": 25}
 
 
 def plan_imap(program, inputs, out, out_bool=False) -> Plan:
@@ -643,7 +644,7 @@ def plan_imap(program, inputs, out, out_bool=False) -> Plan:
 FMAP_OPS = {"in": 1, "const": 2, "add": 3, "sub": 4, "mul": 5, "div": 6, "floordiv": 7, "mod": 8,
             "min": 9, "max": 10, "udiv": 11, "lt": 12, "le": 13, "eq": 14, "ne": 15, "ge": 16,
             "gt": 17, "neg": 18, "abs": 19, "sqrt": 20, "rint": 21, "exp": 22, "log": 23, "r16": 24,
-            "psqrt": 25, "powchk": 26}
+            "psqrt": 25, "powchk": 26, "active": 27}
 FMAP_MAX_INSTRS = 48
 
 

@@ -366,7 +366,9 @@ enum HcamdIMapOp {
   HCAMD_IMAP_LT = 15, HCAMD_IMAP_LE = 16, HCAMD_IMAP_EQ = 17, HCAMD_IMAP_NE = 18,
   HCAMD_IMAP_GE = 19, HCAMD_IMAP_GT = 20,
   HCAMD_IMAP_NEG = 21, HCAMD_IMAP_ABS = 22, HCAMD_IMAP_NOT = 23, HCAMD_IMAP_LNOT = 24,
-  HCAMD_IMAP_COUNT = 25
+  HCAMD_IMAP_ACTIVE = 25, /* top = 1 where the element is still active, else 0; the element is active again
+                             (`tile.mask`, python/hckernel/kernel_api.py:117-119) */
+  HCAMD_IMAP_COUNT = 26
 };
 int hcamdLaunchIMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
                     const void *const *inputs, const size_t *inputLd, size_t nInputs,
@@ -411,7 +413,8 @@ enum HcamdFMapOp {
   HCAMD_FMAP_NEG = 18, HCAMD_FMAP_ABS = 19, HCAMD_FMAP_SQRT = 20, HCAMD_FMAP_RINT = 21,
   HCAMD_FMAP_EXP = 22, HCAMD_FMAP_LOG = 23, HCAMD_FMAP_R16 = 24, HCAMD_FMAP_PSQRT = 25,
   HCAMD_FMAP_POWCHK = 26,
-  HCAMD_FMAP_COUNT = 27
+  HCAMD_FMAP_ACTIVE = 27, /* top = 1 where the element is active in it, else 0; active again (`tile.mask`) */
+  HCAMD_FMAP_COUNT = 28
 };
 int hcamdLaunchFMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
                     const void *const *inputs, const int *inputTypes, const size_t *inputLd,

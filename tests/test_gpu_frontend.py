@@ -1113,6 +1113,47 @@ def test_random_int32_expression_trees_equal_the_host_executor(seed):
     assert_array_equal(dout.to_host(), host, err_msg=desc)
 
 
+def test_tile_mask_is_stored_as_a_plain_bool_array():
+    """`tile.mask` (python/hckernel/kernel_api.py:117-119: True = active) of
+    float and int32 expressions that the data deactivates here and there: the
+    same bytes as the simulator stores, every element written."""
+    N = sym.N
+
+    def fbody(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], q: Buffer[N, DT], m: Buffer[N, DT],
+              m2: Buffer[N, DT]):
+        o = gr.work_offset[0]
+        ta, tb = gr.load(a[o:], shape=gr.shape), gr.load(b[o:], shape=gr.shape)
+        t = ta / tb
+        gr.store(q[o:], t)
+        gr.store(m[o:], t.mask)
+        gr.store(m2[o:], ((ta - tb) / (t * tb)).mask)
+
+    def ibody(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], q: Buffer[N, DT], m: Buffer[N, DT],
+              m2: Buffer[N, DT]):
+        o = gr.work_offset[0]
+        ta, tb = gr.load(a[o:], shape=gr.shape), gr.load(b[o:], shape=gr.shape)
+        gr.store(q[o:], ta // tb)
+        gr.store(m[o:], (ta % tb + ta).mask)
+        gr.store(m2[o:], ta.mask)
+
+    rng = np.random.default_rng(8)
+    n = 1003
+    for dtype, body in ((np.float32, fbody), (np.float16, fbody), (np.int32, ibody)):
+        a = rng.integers(-4, 5, n).astype(dtype)
+        b = rng.integers(-2, 3, n).astype(dtype)
+        if dtype != np.int32:
+            a[5], b[9] = np.inf, np.nan
+        want = [np.full(n, 7, dtype), np.full(n, 7, np.bool_), np.full(n, 7, np.bool_)]
+        with np.errstate(all="ignore"):
+            sim_kernel(work_shape=N, group_shape=256)(body)(a, b, *want)
+        got = [rt.to_device(np.full(n, 7, dtype)), rt.to_device(np.full(n, 7, np.bool_)),
+               rt.to_device(np.full(n, 7, np.bool_))]
+        kernel(work_shape=N, group_shape=256)(body)(rt.to_device(a), rt.to_device(b), *got)
+        assert 0 < want[1].sum() < n                       # some elements are deactivated, some are not
+        for g, w in zip(got, want):
+            assert_array_equal(g.to_host().view(np.uint8), w.view(np.uint8))
+
+
 def test_fp16_maximum_and_minimum_of_signed_zeros_follow_numpy():
     """NumPy's fp16 maximum / minimum return the first of two equal values, its
     fp32 ones the second: +0 against -0 shows it.  Bits must equal the simulator's

@@ -183,8 +183,10 @@ def test_integer_tile_operators_bind_to_the_integer_map(ctx):
 
     with pytest.raises(NoNativeKernel):
         truediv.plan(a, b, out, ctx=ctx)
-    with pytest.raises(NoNativeKernel, match="mask"):
-        uses_mask.plan(a, out, ctx=ctx)
+    with pytest.raises(NoNativeKernel, match="float64 in NumPy"):
+        truediv.plan(a, b, out, ctx=ctx)
+    (p,) = uses_mask.plan(a, out, ctx=ctx)              # tile.mask: 0 / 1, every element stored
+    assert p.fn is rt.hcamdLaunchIMap and imap_program(p) == [("in", 0, 0), ("active", 0, 0)]
 
 
 def map_program(plan):
@@ -1239,6 +1241,33 @@ def test_reductions_over_deactivated_elements_follow_numpy_ma(ctx, rows, n):
         np.testing.assert_array_equal(got == POISON, want == POISON, err_msg=name)
         np.testing.assert_array_equal(np.isnan(got), np.isnan(want), err_msg=name)
         np.testing.assert_allclose(got, want, rtol=3e-5, atol=1e-6, err_msg=name)
+
+
+def test_what_a_traced_tile_cannot_give_says_why(ctx):
+    N = sym.N
+
+    def body(fn, out_dtype):
+        @kernel(work_shape=N, group_shape=256)
+        def k(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], out: Buffer[N, DT]):
+            o = gr.work_offset[0]
+            gr.store(out[o:], fn(gr.load(a[o:], shape=gr.shape), gr.load(b[o:], shape=gr.shape)))
+        return k
+
+    f32, i32 = FakeDev((1000,), "float32"), FakeDev((1000,), "int32")
+    with pytest.raises(NoNativeKernel, match="length depends on the data"):
+        body(lambda a, b: (a / b).compressed(), "float32").plan(f32, f32, FakeDev((1000,), "float32"), ctx=ctx)
+    with pytest.raises(NoNativeKernel, match="float64 in NumPy"):
+        body(lambda a, b: a / b, "float32").plan(i32, i32, FakeDev((1000,), "float32"), ctx=ctx)
+    with pytest.raises(NoNativeKernel, match="polarity"):
+        body(lambda a, b: np.exp(a).mask, "bool").plan(f32, f32, FakeDev((1000,), "bool"), ctx=ctx)
+    with pytest.raises(NoNativeKernel, match="inside a larger integer expression"):
+        body(lambda a, b: (a // b).mask.astype(np.int32) + (a % b), "int32").plan(
+            i32, i32, FakeDev((1000,), "int32"), ctx=ctx)
+    # the mask of a whole expression binds: one more instruction, a one-byte output
+    (p,) = body(lambda a, b: (a / b).mask, "bool").plan(f32, f32, FakeDev((1000,), "bool"), ctx=ctx)
+    assert p.fn is rt.hcamdLaunchFMap and fmap_program(p)[-1][0] == "active"
+    (p,) = body(lambda a, b: (a // b).mask, "bool").plan(i32, i32, FakeDev((1000,), "bool"), ctx=ctx)
+    assert p.fn is rt.hcamdLaunchIMap and imap_program(p)[-1][0] == "active"
 
 
 def test_row_bodies_without_native_code_say_why(ctx):
