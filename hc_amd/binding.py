@@ -1148,16 +1148,10 @@ _FMAP_MIRROR = {"add": "add", "mul": "mul", "max": "max", "min": "min", "eq": "e
 _FMAP_COMPARE = ("lt", "le", "eq", "ne", "ge", "gt")
 
 
-def match_fmap(dst_view, value, n_groups):
-    """An expression of fp32 / fp16 loads of one window, constants, the tile
-    operators and NumPy functions, stored to an fp32, fp16 or (for a
-    comparison) bool buffer, with activity tracked per operand."""
-    out_dt = dst_view.base.dtype_name
-    if out_dt not in _MAP_FLOATS + ("bool",):
-        return None
-    if (value.dtype_name == "bool") != (out_dt == "bool") or \
-            (value.dtype_name != "bool" and value.dtype_name not in _MAP_FLOATS):
-        return None
+def _compile_fmap(value, mapped=False):
+    """The program of the general float map for `value`: (loads, program), or
+    None if value is not a float expression that kernel takes.  Leaves are
+    loads (with `mapped`, loads through a mapping too)."""
     loads, program, needs, memo = [], [], {}, {}
 
     def fdtype(t):
@@ -1166,13 +1160,13 @@ def match_fmap(dst_view, value, n_groups):
     def need(t):
         if t.uid in needs:
             return needs[t.uid]
-        if _is(t, "load") or _const(t):
+        if _is(t, "load") or _is(t, "mapped_load") or _const(t):
             n = 1
         elif len(t.args) == 1:
             n = need(t.args[0])
         elif len(t.args) == 2:
             a, b = need(t.args[0]), need(t.args[1])
-            if _FMAP_BINARY.get(t.op) in _FMAP_MIRROR and not _maybe_masked(t, memo):
+            if _FMAP_BINARY.get(t.op) in _FMAP_MIRROR and not mapped and not _maybe_masked(t, memo):
                 n = max(a, b) if a != b else a + 1
             else:
                 n = max(a, b + 1)
@@ -1185,7 +1179,7 @@ def match_fmap(dst_view, value, n_groups):
         """Appends the code for t; False if t is not a float expression this kernel takes."""
         half = t.dtype_name == "float16"
         func = bool(t.attrs.get("func"))
-        if _is(t, "load"):
+        if _is(t, "load") or (mapped and _is(t, "mapped_load")):
             if t.dtype_name not in _MAP_FLOATS:
                 return False
             for i, u in enumerate(loads):
@@ -1237,7 +1231,9 @@ def match_fmap(dst_view, value, n_groups):
                 raise NoNativeKernel("numpy.floor_divide called as a function has no native code "
                                      "(the // operator has)")
             a, b = t.args
-            if op in _FMAP_MIRROR and not _maybe_masked(t, memo) and need(b) > need(a):
+            # (operands are only exchanged where no element can be inactive: the first
+            # operand's value is what numpy.ma leaves in a deactivated result)
+            if op in _FMAP_MIRROR and not mapped and not _maybe_masked(t, memo) and need(b) > need(a):
                 a, b, op = b, a, _FMAP_MIRROR[op]
             for x in (a, b):
                 if _const(x):
@@ -1264,7 +1260,7 @@ def match_fmap(dst_view, value, n_groups):
             program.append(("powchk", 0, 0.0))
         return ok
 
-    if _is(value, "load") or _const(value):
+    if _is(value, "load") or _is(value, "mapped_load") or _const(value):
         return None
     if not emit(value) or not loads:
         return None
@@ -1273,6 +1269,23 @@ def match_fmap(dst_view, value, n_groups):
     if len(program) > rt.FMAP_MAX_INSTRS:
         raise NoNativeKernel(f"float expression too long ({len(program)} operations, at most "
                              f"{rt.FMAP_MAX_INSTRS})")
+    return loads, list(program)
+
+
+def match_fmap(dst_view, value, n_groups):
+    """An expression of fp32 / fp16 loads of one window, constants, the tile
+    operators and NumPy functions, stored to an fp32, fp16 or (for a
+    comparison) bool buffer, with activity tracked per operand."""
+    out_dt = dst_view.base.dtype_name
+    if out_dt not in _MAP_FLOATS + ("bool",):
+        return None
+    if (value.dtype_name == "bool") != (out_dt == "bool") or \
+            (value.dtype_name != "bool" and value.dtype_name not in _MAP_FLOATS):
+        return None
+    compiled = _compile_fmap(value)
+    if compiled is None:
+        return None
+    loads, prog = compiled
     wins = [window_of(t.attrs["view"], t.shape, n_groups) for t in loads]
     wins.append(window_of(dst_view, value.shape, n_groups))
     w = _check_same_window(wins)
@@ -1280,13 +1293,127 @@ def match_fmap(dst_view, value, n_groups):
         raise NoNativeKernel("only 1-D and 2-D buffers have native kernels")
     types = [rt.F16 if t.dtype_name == "float16" else rt.F32 for t in loads]
     types.append({"float32": rt.F32, "float16": rt.F16, "bool": rt.U8}[out_dt])
-    prog = list(program)
     store_all = bool(value.attrs.get("plain"))     # a bare numpy.ma array is written in full
 
     def make(mem, ctx):
         arrays = [_Arr(_sub(mem[x.buffer], w.extent), ctx) for x in wins]
         return [rt.plan_fmap(prog, arrays[:-1], arrays[-1], types, store_all)]
     make.program = prog
+    return make
+
+
+def _element_tables(func, shape, ndim, name):
+    """An index mapping evaluated on a whole tile: [elements, ndim] int64, the
+    index inside the window of every tile element in row-major order (None:
+    the identity of an unmapped load or store)."""
+    import numpy as np
+    grids = np.indices(shape, dtype=np.int64)
+    if func is None:
+        if ndim != len(shape):
+            raise NoNativeKernel(f"{name}: a tile of rank {len(shape)} on a buffer of rank {ndim}")
+        mapped = tuple(grids)
+    else:
+        try:
+            mapped = func(*grids)
+        except TraceError:
+            raise
+        except Exception as exc:
+            raise NoNativeKernel(f"{name}: the mapping cannot be evaluated on index arrays "
+                                 f"({type(exc).__name__}: {exc})") from exc
+        if not isinstance(mapped, tuple):
+            mapped = (mapped,)
+        if len(mapped) != ndim:
+            raise NoNativeKernel(f"{name}: the mapping must return {ndim} indices")
+    out = np.zeros((math.prod(shape), ndim), np.int64)
+    for d, m in enumerate(mapped):
+        try:
+            full = np.broadcast_to(np.asarray(m), shape)
+            if full.dtype == object or full.dtype.kind == "f":
+                as_int = np.array([int(v) for v in full.ravel()], dtype=np.int64).reshape(shape)
+                if not all(v == w for v, w in zip(full.ravel(), as_int.ravel())):
+                    raise NoNativeKernel(f"{name}: the mapping gives fractional indices")
+                full = as_int
+            out[:, d] = full.astype(np.int64).ravel()
+        except (TypeError, ValueError) as exc:
+            raise NoNativeKernel(f"{name}: mapping result of dimension {d} is not an integer "
+                                 f"array ({exc})") from exc
+    return out
+
+
+_GATHER_MAP_MAX_DESTS = 1 << 24
+
+
+def match_gather_map(dst_view, value, n_groups, out_func=None, force=False):
+    """store(f(tiles...)) where a tile is loaded through a mapping, or the store
+    goes through one: gathered copies, elementwise expressions of gathered
+    tiles, scattered stores (python/hckernel/kernel_api.py:304-310,319-335)."""
+    import numpy as np
+
+    def has_mapped(t, seen):
+        if t.uid in seen:
+            return False
+        seen.add(t.uid)
+        return _is(t, "mapped_load") or any(has_mapped(a, seen) for a in t.args)
+
+    if not force and not has_mapped(value, set()):
+        return None
+    if len(value.shape) not in (1, 2, 3):
+        raise NoNativeKernel("tiles loaded or stored through a mapping have 1 to 3 dimensions")
+    out_dt = dst_view.base.dtype_name
+    leaf = value.args[0] if _is(value, "astype", 1) and value.dtype_name == value.args[0].dtype_name else value
+    copy_bytes = 0
+    if (_is(leaf, "load") or _is(leaf, "mapped_load")) and leaf.dtype_name == out_dt:
+        # a gathered / scattered copy: any element type
+        loads, program = [leaf], []
+        copy_bytes = leaf.attrs["view"].base.dtype.itemsize if hasattr(leaf.attrs["view"].base.dtype, "itemsize") else 2
+        if copy_bytes not in (1, 2, 4, 8):
+            raise NoNativeKernel(f"copies through a mapping move elements of 1, 2, 4 or 8 bytes")
+    else:
+        if out_dt not in _MAP_FLOATS + ("bool",) or (value.dtype_name == "bool") != (out_dt == "bool") or \
+                (value.dtype_name != "bool" and value.dtype_name not in _MAP_FLOATS):
+            raise NoNativeKernel("expressions of tiles loaded or stored through a mapping are bound "
+                                 "for float32 / float16 tiles (copies for every type)")
+        compiled = _compile_fmap(value, mapped=True)
+        if compiled is None:
+            raise NoNativeKernel(f"{value!r}: not an elementwise float expression of tiles")
+        loads, program = compiled
+    shape = value.shape
+    for t in loads:
+        if t.shape != shape:
+            raise NoNativeKernel("the tiles of an expression with mapped loads must have one shape")
+    total = math.prod(n_groups)
+    operands = []
+    for t, func in [(t, t.attrs.get("mapping")) for t in loads] + [(None, out_func)]:
+        view = dst_view if t is None else t.attrs["view"]
+        base = view.base
+        operands.append((tuple(int(v) for v in base.shape), tuple(int(v) for v in base.strides),
+                         _group_starts(view, n_groups), _element_tables(func, shape, base.ndim, base.name)))
+    # two active elements of the output must not land on one address: the
+    # reference stores them one after the other, a launch in no order
+    o_shape, o_strides, o_starts, o_index = operands[-1]
+    if total * o_index.shape[0] > _GATHER_MAP_MAX_DESTS:
+        raise NoNativeKernel(f"{dst_view.base.name}: {total} groups of {o_index.shape[0]} elements are "
+                             "too many to check that no two of them are stored to one place")
+    idx = o_starts[:, None, :] + o_index[None, :, :]
+    inside = ((o_index[None, :, :] >= 0) & (idx < np.asarray(o_shape, np.int64))).all(axis=2)
+    dest = (idx * np.asarray(o_strides, np.int64)).sum(axis=2)[inside]
+    if len(np.unique(dest)) != dest.size:
+        raise NoNativeKernel(f"{dst_view.base.name}: two tile elements (of one group or of two) are "
+                             "stored to one place; their order is the reference's group order, which "
+                             "a launch does not keep")
+    indices = [t.attrs["view"].base.index for t in loads] + [dst_view.base.index]
+    types = [rt.F16 if t.dtype_name == "float16" else rt.F32 for t in loads]
+    out_type = {"float32": rt.F32, "float16": rt.F16, "bool": rt.U8}.get(out_dt, rt.F32)
+    store_all = bool(value.attrs.get("plain")) and not copy_bytes
+    cache = {}
+
+    def make(mem, ctx):
+        g = cache.get(id(ctx))
+        if g is None:
+            g = cache[id(ctx)] = rt.GatherMap(ctx, operands, total, math.prod(shape))
+        arrays = [_Arr(mem[i], ctx) for i in indices]
+        return [rt.plan_gather_map(g, program, arrays[:-1], arrays[-1], types, out_type, store_all, copy_bytes)]
+    make.program = program
     return make
 
 
@@ -2322,6 +2449,14 @@ def match_id_store(proxy, index, value, per_item, n_groups, group_shape):
     return make
 
 
+def _has_dot(t: Tile, seen=None) -> bool:
+    seen = set() if seen is None else seen
+    if t.uid in seen:
+        return False
+    seen.add(t.uid)
+    return t.op == "dot" or any(_has_dot(a, seen) for a in t.args)
+
+
 def bind(stores, n_groups, atomics=(), mapped_stores=(), id_stores=(), group_shape=()):
     """stores: list of (BufferView, Tile) from one traced execution; atomics:
     list of (BufferProxy, index, Tile) atomic additions; mapped_stores: list of
@@ -2342,15 +2477,20 @@ def bind(stores, n_groups, atomics=(), mapped_stores=(), id_stores=(), group_sha
                                      "atomically has no native kernel")
             return [mk for proxy, index, value in atomics
                     for mk in match_sum(proxy, index, value, n_groups)]
-        makers = id_makers + [match_gather_gemm(view, value, n_groups, func, plain=False)
-                              for view, value, func in mapped_stores]
+        makers = list(id_makers)
+        for view, value, func in mapped_stores:
+            value = simplify(value, memo)
+            if _has_dot(value):
+                makers.append(match_gather_gemm(view, value, n_groups, func, plain=False))
+            else:
+                makers.append(match_gather_map(view, value, n_groups, func, force=True))
         q = match_quantize(stores, n_groups)
         if q is not None:
             return makers + [q]
         for view, value in stores:
             for matcher in (match_copy, match_imap, match_add, match_fma, match_softmax, match_gemm,
-                            match_gather_gemm, match_pairwise, match_cols, match_cols_tile, match_rows,
-                            match_map, match_fmap):
+                            match_gather_gemm, match_gather_map, match_pairwise, match_cols,
+                            match_cols_tile, match_rows, match_map, match_fmap):
                 mk = matcher(view, value, n_groups)
                 if mk is not None:
                     makers.append(mk)

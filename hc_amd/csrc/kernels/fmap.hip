@@ -327,3 +327,116 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_fmap(FMapArgs a) {
     }
   }
 }
+
+// ---- elementwise expressions of gathered tiles ------------------------------------
+// out_g[mo(e)] = f(in0_g[m0(e)], ...) for every group g and tile element e: what
+// a body computes that loads its tiles through index mappings, or stores one
+// through a mapping, outside a matrix product (CurrentGroup.load / store with
+// mapping=..., python/hckernel/kernel_api.py:304-310,319-335).  x_g is the
+// window of buffer x that starts at starts[g][d] along dimension d; element e
+// of a tile sits at index[e][d] of the window and is active if 0 <= index[e][d]
+// < shape[d] - starts[g][d] for every d (the reference's bounds test; an
+// unmapped operand has the identity table).  Inactive operand elements are
+// zeros that deactivate what is computed from them under the rules above;
+// inactive output positions are not written, and neither are deactivated
+// results unless store_all.  One tile element per lane: the accesses are
+// gathers, so there is nothing to vectorise.
+namespace {
+struct GatherMapOperand {
+  const int32_t *starts; // [groups][4]
+  const int32_t *index;  // [tile elements][4]
+  uint32_t shape[4];     // 1 for the dimensions the buffer does not have
+  uint32_t strides[4];   // in elements
+};
+struct GatherMapArgs {
+  const void *in[kMaxIn];
+  void *out;
+  GatherMapOperand op[kMaxIn + 1]; // the inputs, then the output
+  uint32_t n_in, tile_elems, chunks; // chunks: workgroups per group
+  uint32_t f16_mask;  // bit i: operand i is fp16
+  uint32_t out_type;  // 0 fp32, 1 fp16, 2 one byte of 0 / 1
+  uint32_t store_all; // write deactivated results too
+  uint32_t copy_bytes; // != 0: no program, operand 0 is copied as elements of this many bytes
+  uint32_t n_instr;
+  Instr prog[kMaxProg];
+};
+// offset of element e of group g in elements, or -1 if the element is inactive
+__device__ __forceinline__ int64_t gather_offset(const GatherMapOperand &o, uint32_t g, uint32_t e) {
+  int64_t at = 0;
+  bool inside = true;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const int32_t st = o.starts[(size_t)g * 4 + d], ix = o.index[(size_t)e * 4 + d];
+    inside = inside && ix >= 0 && (int64_t)ix < (int64_t)o.shape[d] - st;
+    at += ((int64_t)st + ix) * o.strides[d];
+  }
+  return inside ? at : -1;
+}
+} // namespace
+
+extern "C" __global__ __launch_bounds__(256) void hcamd_gather_fmap(GatherMapArgs a) {
+  const uint32_t g = blockIdx.x / a.chunks;
+  const uint32_t e = (blockIdx.x % a.chunks) * 256 + threadIdx.x;
+  if (e >= a.tile_elems)
+    return;
+  const int64_t dst = gather_offset(a.op[a.n_in], g, e);
+  if (dst < 0)
+    return;
+  if (a.copy_bytes) {
+    const int64_t src = gather_offset(a.op[0], g, e);
+    if (src < 0)
+      return;
+    switch (a.copy_bytes) {
+    case 1: static_cast<uint8_t *>(a.out)[dst] = static_cast<const uint8_t *>(a.in[0])[src]; break;
+    case 2: static_cast<uint16_t *>(a.out)[dst] = static_cast<const uint16_t *>(a.in[0])[src]; break;
+    case 4: static_cast<uint32_t *>(a.out)[dst] = static_cast<const uint32_t *>(a.in[0])[src]; break;
+    default: static_cast<uint64_t *>(a.out)[dst] = static_cast<const uint64_t *>(a.in[0])[src]; break;
+    }
+    return;
+  }
+  float v[kMaxIn];
+  bool act[kMaxIn];
+#pragma unroll
+  for (int i = 0; i < kMaxIn; ++i) {
+    v[i] = 0.0f;
+    act[i] = false;
+    if (i < (int)a.n_in) {
+      const int64_t at = gather_offset(a.op[i], g, e);
+      act[i] = at >= 0;
+      if (at >= 0)
+        v[i] = ((a.f16_mask >> i) & 1) ? (float)static_cast<const _Float16 *>(a.in[i])[at]
+                                        : static_cast<const float *>(a.in[i])[at];
+    }
+  }
+  float t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
+  bool k0 = true, k1 = true, k2 = true, k3 = true;
+  for (uint32_t pc = 0; pc < a.n_instr; ++pc) {
+    const uint32_t op = a.prog[pc].op, arg = a.prog[pc].arg;
+    if (op == FOP_IN || op == FOP_CONST) {
+      t3 = t2, t2 = t1, t1 = t0;
+      k3 = k2, k2 = k1, k1 = k0;
+      t0 = a.prog[pc].imm;
+      k0 = true;
+      if (op == FOP_IN) {
+        t0 = arg == 0 ? v[0] : arg == 1 ? v[1] : arg == 2 ? v[2] : v[3];
+        k0 = arg == 0 ? act[0] : arg == 1 ? act[1] : arg == 2 ? act[2] : act[3];
+      }
+    } else if (op >= FOP_NEG) {
+      t0 = unary(op, t0, k0);
+    } else {
+      bool ok = k1 && k0;
+      t0 = binary(op, t1, t0, arg, ok);
+      k0 = ok;
+      t1 = t2, t2 = t3;
+      k1 = k2, k2 = k3;
+    }
+  }
+  if (!(k0 || a.store_all))
+    return;
+  if (a.out_type == 2)
+    static_cast<uint8_t *>(a.out)[dst] = (uint8_t)(t0 != 0.0f);
+  else if (a.out_type == 1)
+    static_cast<_Float16 *>(a.out)[dst] = (_Float16)t0;
+  else
+    static_cast<float *>(a.out)[dst] = t0;
+}

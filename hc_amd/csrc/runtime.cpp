@@ -3004,6 +3004,226 @@ void hcamdGatherGemmRelease(HcamdGatherGemm plan) noexcept {
   delete plan;
 }
 
+// ---------------------------------------------------------------------------
+// Elementwise expressions of gathered tiles
+// ---------------------------------------------------------------------------
+struct HcamdGatherMap_ {
+  Device *device = nullptr;
+  int32_t *tables = nullptr; // one device allocation: per operand starts[groups][4], index[elems][4]
+  size_t offStarts[kMapMaxIn + 1] = {}, offIndex[kMapMaxIn + 1] = {};
+  uint32_t shape[kMapMaxIn + 1][4] = {}, strides[kMapMaxIn + 1][4] = {};
+  size_t nInputs = 0, nGroups = 0, tileElems = 0;
+};
+
+namespace {
+// argument block of hcamd_gather_fmap (the same layout as in the device code)
+struct GatherMapOperandDev {
+  const int32_t *starts;
+  const int32_t *index;
+  uint32_t shape[4];
+  uint32_t strides[4];
+};
+struct GatherMapArgs {
+  const void *in[kMapMaxIn];
+  void *out;
+  GatherMapOperandDev op[kMapMaxIn + 1];
+  uint32_t nIn, tileElems, chunks;
+  uint32_t f16Mask, outType, storeAll, copyBytes, nInstr;
+  HcamdMapInstr prog[48];
+};
+} // namespace
+
+HcamdGatherMap hcamdGatherMapCreate(OlQueue q, const HcamdGatherMapOperand *operands, size_t nInputs,
+                                    size_t nGroups, size_t tileElems) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return nullptr;
+  Device *dev = queue->device;
+  const char *who = "hcamdGatherMapCreate";
+  if (!operands || nInputs < 1 || nInputs > kMapMaxIn || nGroups == 0 || tileElems == 0 ||
+      nGroups > 0x7fffffffull || tileElems > ((size_t)1 << 24)) {
+    dev->report("%s: %zu operands (1..%zu), %zu groups, %zu tile elements", who, nInputs, kMapMaxIn,
+                nGroups, tileElems);
+    return nullptr;
+  }
+  const size_t chunks = ceilDiv(tileElems, (size_t)256);
+  if (nGroups * chunks > 0x7fffffffull) {
+    dev->report("%s: %zu groups of %zu elements are more workgroups than a launch holds", who,
+                nGroups, tileElems);
+    return nullptr;
+  }
+  auto *plan = new (std::nothrow) HcamdGatherMap_;
+  if (!plan) {
+    dev->report("%s: out of host memory", who);
+    return nullptr;
+  }
+  plan->device = dev;
+  plan->nInputs = nInputs;
+  plan->nGroups = nGroups;
+  plan->tileElems = tileElems;
+  size_t total = 0;
+  for (size_t o = 0; o <= nInputs; ++o) {
+    const HcamdGatherMapOperand &op = operands[o];
+    if (op.ndim < 1 || op.ndim > 4 || !op.starts || !op.index) {
+      dev->report("%s: operand %zu: rank %d or null table", who, o, op.ndim);
+      delete plan;
+      return nullptr;
+    }
+    size_t span = 1;
+    for (int d = 0; d < 4; ++d) {
+      const size_t n = d < op.ndim ? op.shape[d] : 1, st = d < op.ndim ? op.strides[d] : 0;
+      if (n == 0 || n > 0x7fffffffull || st > 0x7fffffffull) {
+        dev->report("%s: operand %zu: empty or larger than 2^31 along dimension %d", who, o, d);
+        delete plan;
+        return nullptr;
+      }
+      plan->shape[o][d] = (uint32_t)n;
+      plan->strides[o][d] = (uint32_t)st;
+      span += (n - 1) * st;
+    }
+    if (span > 0x7fffffffull) {
+      dev->report("%s: operand %zu spans more than 2^31 elements", who, o);
+      delete plan;
+      return nullptr;
+    }
+    for (size_t g = 0; g < nGroups * (size_t)op.ndim; ++g)
+      if (op.starts[g] < 0) {
+        dev->report("%s: operand %zu: negative window start", who, o);
+        delete plan;
+        return nullptr;
+      }
+    plan->offStarts[o] = total;
+    total += nGroups * 4;
+    plan->offIndex[o] = total;
+    total += tileElems * 4;
+  }
+  std::vector<int32_t> host;
+  try {
+    host.assign(total, 0);
+  } catch (...) {
+    dev->report("%s: out of host memory", who);
+    delete plan;
+    return nullptr;
+  }
+  for (size_t o = 0; o <= nInputs; ++o) {
+    const HcamdGatherMapOperand &op = operands[o];
+    for (size_t g = 0; g < nGroups; ++g)
+      for (int d = 0; d < op.ndim; ++d)
+        host[plan->offStarts[o] + g * 4 + d] = op.starts[g * op.ndim + d];
+    for (size_t e = 0; e < tileElems; ++e)
+      for (int d = 0; d < op.ndim; ++d)
+        host[plan->offIndex[o] + e * 4 + d] = op.index[e * op.ndim + d];
+  }
+  if (dev->makeCurrent() ||
+      HIP_CHECK(dev, hipMalloc(reinterpret_cast<void **>(&plan->tables), total * sizeof(int32_t)))) {
+    delete plan;
+    return nullptr;
+  }
+  if (HIP_CHECK(dev, hipMemcpy(plan->tables, host.data(), total * sizeof(int32_t), hipMemcpyHostToDevice))) {
+    (void)hipFree(plan->tables);
+    delete plan;
+    return nullptr;
+  }
+  return plan;
+}
+
+int hcamdGatherMapLaunch(OlQueue q, HcamdGatherMap plan, const HcamdMapInstr *prog, size_t nInstr,
+                         const void *const *inputs, const int *inputTypes, void *out, int outType,
+                         int storeAll, size_t copyBytes) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  const char *who = "hcamdGatherMapLaunch";
+  if (!plan || plan->device != dev || !inputs || !out) {
+    dev->report("%s: null pointer, or a plan of another device", who);
+    return 1;
+  }
+  GatherMapArgs a{};
+  if (copyBytes) {
+    if (copyBytes != 1 && copyBytes != 2 && copyBytes != 4 && copyBytes != 8) {
+      dev->report("%s: copies move elements of 1, 2, 4 or 8 bytes", who);
+      return 1;
+    }
+    a.copyBytes = (uint32_t)copyBytes;
+  } else {
+    if (!prog || !inputTypes || nInstr == 0 || nInstr > 48) {
+      dev->report("%s: program of %zu instructions (1..48)", who, nInstr);
+      return 1;
+    }
+    if (outType != HCAMD_F32 && outType != HCAMD_F16 && outType != HCAMD_U8) {
+      dev->report("%s: unsupported output type %d", who, outType);
+      return 1;
+    }
+    int sp = 0;
+    for (size_t i = 0; i < nInstr; ++i) {
+      const unsigned op = prog[i].op;
+      if (op == HCAMD_FMAP_END || op >= HCAMD_FMAP_COUNT) {
+        dev->report("%s: bad opcode %u at %zu", who, op, i);
+        return 1;
+      }
+      if (op == HCAMD_FMAP_IN && prog[i].arg >= plan->nInputs) {
+        dev->report("%s: operand %u at %zu (only %zu given)", who, prog[i].arg, i, plan->nInputs);
+        return 1;
+      }
+      const bool push = op == HCAMD_FMAP_IN || op == HCAMD_FMAP_CONST;
+      const bool unary = op >= HCAMD_FMAP_NEG;
+      if (sp < (push ? 0 : unary ? 1 : 2)) {
+        dev->report("%s: stack underflow at %zu", who, i);
+        return 1;
+      }
+      sp += push ? 1 : unary ? 0 : -1;
+      if (sp > 4) {
+        dev->report("%s: stack deeper than 4 at %zu", who, i);
+        return 1;
+      }
+      a.prog[i] = prog[i];
+    }
+    if (sp != 1) {
+      dev->report("%s: program leaves %d values, expected 1", who, sp);
+      return 1;
+    }
+    a.nInstr = (uint32_t)nInstr;
+    a.outType = outType == HCAMD_F32 ? 0u : outType == HCAMD_F16 ? 1u : 2u;
+    a.storeAll = storeAll ? 1u : 0u;
+  }
+  for (size_t i = 0; i <= plan->nInputs; ++i) {
+    if (i < plan->nInputs) {
+      if (!inputs[i]) {
+        dev->report("%s: null pointer", who);
+        return 1;
+      }
+      if (!copyBytes && inputTypes[i] != HCAMD_F32 && inputTypes[i] != HCAMD_F16) {
+        dev->report("%s: unsupported operand type %d", who, inputTypes[i]);
+        return 1;
+      }
+      a.in[i] = inputs[i];
+      if (!copyBytes && inputTypes[i] == HCAMD_F16)
+        a.f16Mask |= 1u << i;
+    }
+    a.op[i].starts = plan->tables + plan->offStarts[i];
+    a.op[i].index = plan->tables + plan->offIndex[i];
+    for (int d = 0; d < 4; ++d) {
+      a.op[i].shape[d] = plan->shape[i][d];
+      a.op[i].strides[d] = plan->strides[i][d];
+    }
+  }
+  a.out = out;
+  a.nIn = (uint32_t)plan->nInputs;
+  a.tileElems = (uint32_t)plan->tileElems;
+  a.chunks = (uint32_t)ceilDiv(plan->tileElems, (size_t)256);
+  void *args[] = {&a};
+  return launch1d(queue, "fmap", "hcamd_gather_fmap", plan->nGroups * a.chunks, 256, args);
+}
+
+void hcamdGatherMapRelease(HcamdGatherMap plan) noexcept {
+  if (!plan)
+    return;
+  if (!plan->device->makeCurrent() && plan->tables)
+    (void)hipFree(plan->tables);
+  delete plan;
+}
+
 int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,
                           size_t ldy, size_t rows, size_t cols) noexcept {
   auto *queue = static_cast<Queue *>(q);

@@ -162,6 +162,16 @@ hcamdGatherGemmCreate = _sig(_rt, "hcamdGatherGemmCreate", _vp, _vp, C.POINTER(G
 hcamdGatherGemmLaunchF32 = _sig(_rt, "hcamdGatherGemmLaunchF32", _int, _vp, _vp, _vp, _vp, _vp)
 hcamdGatherGemmLaunch = _sig(_rt, "hcamdGatherGemmLaunch", _int, _vp, _vp, _int, _vp, _vp, _vp)
 hcamdGatherGemmRelease = _sig(_rt, "hcamdGatherGemmRelease", None, _vp)
+class GatherMapOperand(C.Structure):
+    """HcamdGatherMapOperand of include/hc_amd_runtime.h."""
+    _fields_ = [("ndim", _int), ("shape", _sz * 4), ("strides", _sz * 4),
+                ("starts", C.POINTER(C.c_int32)), ("index", C.POINTER(C.c_int32))]
+
+
+hcamdGatherMapCreate = _sig(_rt, "hcamdGatherMapCreate", _vp, _vp, C.POINTER(GatherMapOperand), _sz, _sz, _sz)
+hcamdGatherMapLaunch = _sig(_rt, "hcamdGatherMapLaunch", _int, _vp, _vp, _vp, _sz, C.POINTER(_vp),
+                            C.POINTER(_int), _vp, _int, _int, _sz)
+hcamdGatherMapRelease = _sig(_rt, "hcamdGatherMapRelease", None, _vp)
 hcamdConvertPyArray = _sig(_py, "hcamdConvertPyArray", _int, C.py_object, _int, _vp,
                            _sz_p, C.c_char_p, _sz)
 hcamdConvertPyInt64 = _sig(_py, "hcamdConvertPyInt64", _int, C.py_object,
@@ -875,6 +885,69 @@ class GatherGemm:
                 hcamdGatherGemmRelease(handle)
             except Exception:       # interpreter shutdown: the library may be gone
                 pass
+
+
+class GatherMap:
+    """Device tables of an elementwise expression of gathered tiles
+    (hcamdGatherMapCreate).  `operands`: the inputs, then the output, each
+    (shape, strides, starts [n_groups, ndim], index [tile elements, ndim]);
+    shape / strides of the whole buffer in elements."""
+
+    def __init__(self, ctx, operands, n_groups: int, tile_elems: int):
+        self.ctx, self.handle = ctx, None
+        self.layouts = [(tuple(int(v) for v in o[0]), tuple(int(v) for v in o[1])) for o in operands]
+        ops, keep = (GatherMapOperand * len(operands))(), []
+        for op, (shape, strides, starts, index) in zip(ops, operands):
+            op.ndim = len(shape)
+            if not 1 <= op.ndim <= 4:
+                raise HcRuntimeError("gathered operands have 1 to 4 dimensions")
+            for d in range(op.ndim):
+                op.shape[d], op.strides[d] = int(shape[d]), int(strides[d])
+            tabs = []
+            for t in (starts, index):
+                t = np.ascontiguousarray(t, dtype=np.int64).reshape(-1, op.ndim)
+                if t.size and (t.max() > 0x7fffffff or t.min() < -0x80000000):
+                    raise HcRuntimeError("gather index out of the 32-bit range")
+                t = t.astype(np.int32)
+                keep.append(t)
+                tabs.append(t.ctypes.data_as(C.POINTER(C.c_int32)))
+            op.starts, op.index = tabs
+        h = hcamdGatherMapCreate(ctx.queue, ops, len(operands) - 1, n_groups, tile_elems)
+        if not h:
+            ctx.check(1, "hcamdGatherMapCreate")
+        self.handle = h
+
+    def __del__(self):
+        handle, self.handle = getattr(self, "handle", None), None
+        if handle:
+            try:
+                hcamdGatherMapRelease(handle)
+            except Exception:       # interpreter shutdown: the library may be gone
+                pass
+
+
+def plan_gather_map(tables: GatherMap, program, inputs, out, types, out_type, store_all=False,
+                    copy_bytes=0) -> Plan:
+    """One launch of a GatherMap: `program` is a program of the general float map
+    ((opname, arg, imm) triples), or empty with copy_bytes the element size of a
+    gathered / scattered copy."""
+    inputs = list(inputs)
+    ctx = _ctx_of(*inputs, out)
+    ms = [as_memref(x) for x in inputs] + [as_memref(out)]
+    for m, lay in zip(ms, tables.layouts):
+        if (tuple(m.shape), tuple(m.strides)) != lay:
+            raise HcRuntimeError(f"gather_map: an operand has shape {m.shape} strides {m.strides}, "
+                                 f"the tables were built for {lay[0]} {lay[1]}")
+    n_in = len(inputs)
+    prog = (MapInstr * max(len(program), 1))()
+    for i, (name, arg, imm) in enumerate(program):
+        prog[i].op, prog[i].arg, prog[i].imm = FMAP_OPS[name], int(arg), float(imm)
+    ptrs = (_vp * max(n_in, 1))(*[m.ptr for m in ms[:-1]])
+    tys = (_int * max(n_in, 1))(*types[:n_in])
+    return Plan(ctx, hcamdGatherMapLaunch,
+                (ctx.queue, tables.handle, prog, len(program), ptrs, tys, ms[-1].ptr, int(out_type),
+                 int(bool(store_all)), int(copy_bytes)), "hcamdGatherMapLaunch",
+                (tables, inputs, out, prog, ptrs, tys))
 
 
 def plan_gather_gemm(tables: GatherGemm, a, b, out, dtype: str = "float32") -> Plan:

@@ -660,6 +660,42 @@ int hcamdGatherGemmLaunch(OlQueue q, HcamdGatherGemm plan, int elemType,
                           void *out) HCAMD_NOEXCEPT;
 void hcamdGatherGemmRelease(HcamdGatherGemm plan) HCAMD_NOEXCEPT;
 
+/* Elementwise expressions of gathered tiles -- what a body computes that loads
+ * tiles through index mappings, or stores one through a mapping, outside a
+ * matrix product (CurrentGroup.load / store with mapping=...,
+ * python/hckernel/kernel_api.py:304-310,319-335):
+ *
+ *     out_g[mo(e)] = f(in0_g[m0(e)], in1_g[m1(e)], ...)     for every group g, tile element e
+ *
+ * x_g is the window of buffer x that starts at starts[g][d] along dimension d;
+ * element e of a tile (row-major) sits at index[e][d] of the window and is
+ * active if 0 <= index[e][d] < shape[d] - starts[g][d] for every d, the
+ * reference's bounds test; an operand without a mapping has the identity table.
+ * f is a program of hcamdLaunchFMap with its activity rules: an inactive operand
+ * element is a zero that deactivates what is computed from it; an inactive
+ * output position is not written, and neither is a deactivated result unless
+ * storeAll.  With copyBytes != 0 (1, 2, 4 or 8) there is no program: operand 0
+ * is copied element by element whatever its type (a gathered / scattered copy).
+ * Two active out elements of one launch must not share a destination (their
+ * order is not defined).  `operands` holds the nInputs inputs, then the output;
+ * all pointers in it are host memory and are not kept.  Create allocates device
+ * memory for the tables and synchronises; Launch neither allocates nor
+ * synchronises. */
+typedef struct HcamdGatherMapOperand {
+  int ndim;              /* 1..4 */
+  size_t shape[4];       /* elements per dimension of the whole buffer */
+  size_t strides[4];     /* in elements */
+  const int32_t *starts; /* [nGroups][ndim], >= 0 */
+  const int32_t *index;  /* [tileElems][ndim] */
+} HcamdGatherMapOperand;
+typedef struct HcamdGatherMap_ *HcamdGatherMap;
+HcamdGatherMap hcamdGatherMapCreate(OlQueue q, const HcamdGatherMapOperand *operands, size_t nInputs,
+                                    size_t nGroups, size_t tileElems) HCAMD_NOEXCEPT;
+int hcamdGatherMapLaunch(OlQueue q, HcamdGatherMap plan, const HcamdMapInstr *prog, size_t nInstr,
+                         const void *const *inputs, const int *inputTypes, void *out, int outType,
+                         int storeAll, size_t copyBytes) HCAMD_NOEXCEPT;
+void hcamdGatherMapRelease(HcamdGatherMap plan) HCAMD_NOEXCEPT;
+
 /* Row softmax, fp32: y[r,:] = exp(x[r,:]-max(x[r,:])) / sum(exp(...)).
  * Expression of python/hckernel/tests/test_examples.py:330-335. */
 int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,

@@ -1113,6 +1113,79 @@ def test_random_int32_expression_trees_equal_the_host_executor(seed):
     assert_array_equal(dout.to_host(), host, err_msg=desc)
 
 
+def _gather_bodies(deco, make_mapping):
+    """Bodies that load tiles through index mappings, or store one through a
+    mapping, outside a matrix product (python/hckernel/kernel_api.py:304-310,
+    319-335): indices that leave the window are inactive elements."""
+    R, Cc = sym.R, sym.C
+    TM, TN = 8, 16
+    transpose = make_mapping(lambda i, j: (j, i))
+    shifted = make_mapping(lambda i, j: (i - 1, j + 2))
+    spread = make_mapping(lambda i, j: (2 * i, j))
+    diagonal = make_mapping(lambda i, j: (i, (i + j) % TN))
+
+    @deco(work_shape=(R, Cc), group_shape=(TM, TN))
+    def gathered_copy(gr: CurrentGroup, a: Buffer[Cc, R, DT], out: Buffer[R, Cc, DT]):
+        x, y = gr.work_offset
+        gr.store(out[x:, y:], gr.load(a[y:, x:], shape=(TM, TN), mapping=transpose))
+
+    @deco(work_shape=(R, Cc), group_shape=(TM, TN))
+    def gathered_expression(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT], out: Buffer[R, Cc, DT]):
+        x, y = gr.work_offset
+        ta = gr.load(a[x:, y:], shape=(TM, TN), mapping=shifted)
+        tb = gr.load(b[x:, y:], shape=(TM, TN))
+        gr.store(out[x:, y:], (ta * np.float32(2) + tb) / gr.load(b[x:, y:], shape=(TM, TN), mapping=diagonal))
+
+    @deco(work_shape=(R, Cc), group_shape=(TM, TN))
+    def scattered_store(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT], out: Buffer[2 * R, Cc, DT]):
+        x, y = gr.work_offset
+        t = gr.load(a[x:, y:], shape=(TM, TN)) - gr.load(b[x:, y:], shape=(TM, TN))
+        gr.store(out[2 * x:, y:], t, mapping=spread)
+
+    @deco(work_shape=(R, Cc), group_shape=(TM, TN))
+    def function_of_gathered(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT], out: Buffer[R, Cc, DT]):
+        x, y = gr.work_offset
+        ta = gr.load(a[x:, y:], shape=(TM, TN), mapping=shifted)
+        gr.store(out[x:, y:], np.exp(ta) + gr.load(b[x:, y:], shape=(TM, TN)))     # a bare array: stored in full
+
+    return {"gathered_copy": gathered_copy, "gathered_expression": gathered_expression,
+            "scattered_store": scattered_store, "function_of_gathered": function_of_gathered}
+
+
+@pytest.mark.parametrize("rows,cols", [(16, 32), (37, 50), (8, 16)])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.int32])
+def test_mapped_loads_and_stores_outside_a_product_match_the_simulator(rows, cols, dtype):
+    """The same bodies on the GPU and on the simulator, on arrays that do not
+    fill their last tiles: bit for bit, including which elements are left alone
+    (indices past the window, deactivated quotients)."""
+    gpu, sim = _gather_bodies(kernel, create_mapping), _gather_bodies(sim_kernel, __import__("oracle.hcsim", fromlist=["x"]).create_mapping)
+    rng = np.random.default_rng(rows + cols)
+    a = rng.integers(-5, 6, (rows, cols)).astype(dtype)
+    b = rng.integers(-2, 3, (rows, cols)).astype(dtype)
+    at = np.ascontiguousarray(a.T)
+    cases = {"gathered_copy": ([at], (rows, cols))}
+    if dtype != np.int32:
+        cases.update({"gathered_expression": ([a, b], (rows, cols)), "scattered_store": ([a, b], (2 * rows, cols)),
+                      "function_of_gathered": ([a, b], (rows, cols))})
+    for name, (ins, shape) in cases.items():
+        want = np.full(shape, 7, dtype)
+        with np.errstate(all="ignore"):
+            sim[name](*ins, want)
+        out = rt.to_device(np.full(shape, 7, dtype))
+        gpu[name](*[rt.to_device(v) for v in ins], out)
+        assert rt.last_kernel_name() == "hcamd_gather_fmap", name
+        got = out.to_host()
+        if name == "function_of_gathered":          # exp: the last bit may differ
+            assert_array_equal(got == 7, want == 7, err_msg=name)
+            assert_allclose(got.astype(np.float64), want.astype(np.float64), rtol=2e-3 if dtype == np.float16 else 1e-6,
+                            err_msg=name)
+        else:
+            bits = {2: np.uint16, 4: np.uint32}[np.dtype(dtype).itemsize]
+            assert_array_equal(got.view(bits), want.view(bits), err_msg=name)
+        if name in ("gathered_expression", "scattered_store"):
+            assert (want == 7).any(), name               # something is left alone
+
+
 def test_tile_mask_is_stored_as_a_plain_bool_array():
     """`tile.mask` (python/hckernel/kernel_api.py:117-119: True = active) of
     float and int32 expressions that the data deactivates here and there: the

@@ -724,6 +724,83 @@ def test_mappings_that_no_table_can_express_are_refused(ctx, monkeypatch):
         make(lambda i, j: (i, j if j < 3 else 0))
 
 
+class MapTablesOnly:
+    """Stands in for hc_amd.runtime.GatherMap: keeps the host tables and runs
+    them in NumPy."""
+    last = None
+
+    def __init__(self, ctx, operands, n_groups, tile_elems):
+        self.ctx, self.handle = ctx, 0xABCE
+        self.operands, self.n_groups, self.tile_elems = operands, n_groups, tile_elems
+        self.layouts = [(tuple(o[0]), tuple(o[1])) for o in operands]
+        MapTablesOnly.last = self
+
+    def gather(self, k, arr, g):
+        """(values, active) of operand k's tile for group g (HcamdGatherMapOperand:
+        element e sits at index[e] of the window that starts at starts[g] and is
+        active while every index is inside it)."""
+        shape, _, starts, index = self.operands[k]
+        ok = ((index >= 0) & (index < np.asarray(shape) - starts[g])).all(-1)
+        src = np.where(ok[:, None], index + starts[g], 0)
+        return np.where(ok, arr[tuple(src[:, d] for d in range(len(shape)))], 0), ok, src
+
+
+def test_mapped_loads_and_stores_outside_a_product_bind_to_the_gathered_map(ctx, monkeypatch):
+    from hc_amd.kernel import create_mapping
+    monkeypatch.setattr(rt, "GatherMap", MapTablesOnly)
+    R, Cc = sym.R, sym.C
+    rows, cols, TM, TN = 19, 21, 4, 8
+
+    def body(load_func=None, store_func=None, fn=lambda t, u: t * np.float32(3) - u, stretch=1):
+        lm = create_mapping(load_func) if load_func else None
+        sm = create_mapping(store_func) if store_func else None
+
+        @kernel(work_shape=(R, Cc), group_shape=(TM, TN))
+        def k(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT], out: Buffer[sym.RO, sym.CO, DT]):
+            x, y = gr.work_offset
+            t = gr.load(a[x:, y:], shape=(TM, TN), mapping=lm)
+            u = gr.load(b[x:, y:], shape=(TM, TN))
+            gr.store(out[stretch * x:, y:], fn(t, u), mapping=sm)
+        return k
+
+    def plan(k, dtype="float32", out_shape=(rows, cols)):
+        return k.plan(FakeDev((rows, cols), dtype), FakeDev((rows, cols), dtype), FakeDev(out_shape, dtype), ctx=ctx)
+
+    # a gathered expression: the tables say where every tile element comes from
+    (p,) = plan(body(load_func=lambda i, j: (i + 1, j - 1)))
+    assert p.fn is rt.hcamdGatherMapLaunch
+    names = {v: k for k, v in rt.FMAP_OPS.items()}
+    prog = [(names[p.args[2][i].op], p.args[2][i].arg, p.args[2][i].imm) for i in range(p.args[3])]
+    assert prog == [("in", 0, 0.0), ("const", 0, 3.0), ("mul", 0, 0.0), ("in", 1, 0.0), ("sub", 0, 0.0)]
+    t = MapTablesOnly.last
+    assert (t.n_groups, t.tile_elems) == (5 * 3, TM * TN)
+    rng = np.random.default_rng(0)
+    a = rng.standard_normal((rows, cols)).astype(np.float32)
+    g = 4                                              # group (1, 1): rows 4.., columns 8..
+    vals, ok, src = t.gather(0, a, g)
+    assert tuple(t.operands[0][2][g]) == (4, 8)
+    assert_eq = np.testing.assert_array_equal
+    assert_eq(ok.reshape(TM, TN)[:, 0], False)          # column index -1: outside the window
+    assert_eq(vals.reshape(TM, TN)[:, 1:], a[5:9, 8:15])
+    # a scattered store past the destination's end is not written: the bounds test is the table's
+    (p,) = plan(body(store_func=lambda i, j: (2 * i, j), stretch=2), out_shape=(2 * rows - 1, cols))
+    t = MapTablesOnly.last
+    _, ok, dst = t.gather(2, np.zeros((2 * rows - 1, cols)), 14)   # the last group: from row 32 of 37
+    assert ok.reshape(TM, TN)[:, 0].tolist() == [True, True, True, False]
+    # a copy takes any element type
+    (p,) = plan(body(load_func=lambda i, j: (i, j), fn=lambda t, u: t), dtype="int32")
+    assert p.args[-1] == 4 and p.args[3] == 0
+    # what has no native code says why
+    with pytest.raises(NoNativeKernel, match="stored to one place"):
+        plan(body(store_func=lambda i, j: (i // 2, j)))
+    with pytest.raises(NoNativeKernel, match="float32 / float16"):
+        plan(body(load_func=lambda i, j: (i, j)), dtype="int32")
+    with pytest.raises(NoNativeKernel, match="must return 2 indices"):
+        plan(body(load_func=lambda i, j: (i, j, 0)))
+    with pytest.raises(NoNativeKernel, match="cannot be evaluated"):
+        plan(body(load_func=lambda i, j: (i, j if j < 3 else 0)))
+
+
 def test_offsets_with_division_are_for_mapped_accesses_only(ctx):
     W, H = sym.W, sym.H
 
