@@ -2442,6 +2442,63 @@ def match_id_store(proxy, index, value, per_item, n_groups, group_shape):
     out_type = {"int32": rt.I32, "int64": rt.I64, "float32": rt.F32}[proxy.dtype_name]
     idx = [(i.const, i.g, i.l) for i in index]
     val = (value.const, value.g, value.l)
+    rank = len(group_shape)
+    # (the last Python dimension is the launch's x; the others are y and z)
+    for d in range(rank - 1):
+        if n_groups[d] > 65535:
+            raise NoNativeKernel(f"{n_groups[d]} groups along dimension {d}: a launch takes at most 65535 "
+                                 "along every dimension but the last")
+    extents = [(n, s if per_item else 1) for n, s in zip(n_groups, group_shape)]
+
+    def span(c, g, l):
+        """Smallest and largest value of c + sum g[k] * gid[k] + sum l[k] * lid[k]."""
+        lo = hi = c
+        for k in range(rank):
+            for coef, n in ((g[k], extents[k][0]), (l[k], extents[k][1])):
+                lo += min(0, coef * (n - 1))
+                hi += max(0, coef * (n - 1))
+        return lo, hi
+
+    for d, (c, g, l) in enumerate(idx):
+        if span(c, g, l)[0] < 0:
+            raise NoNativeKernel(f"{proxy.name}: the index along dimension {d} goes below 0 for some "
+                                 "work-item; NumPy counts such an index from the end, the kernel does not")
+    # Two work-items that store different values to one element: the simulator
+    # keeps the last one's, a launch whichever comes last.
+    import numpy as np
+    stores = math.prod(n * s for n, s in extents)
+    if stores <= 1 << 22:
+        ids = np.indices([n for n, _ in extents] + [s for _, s in extents], dtype=np.int64).reshape(2 * rank, -1)
+
+        def values(c, g, l):
+            return c + sum(g[k] * ids[k] + l[k] * ids[rank + k] for k in range(rank))
+        dest = np.zeros(stores, np.int64)
+        for (c, g, l), n in zip(idx, proxy.shape):
+            dest = dest * int(n) + np.clip(values(c, g, l), 0, int(n) - 1)
+        order = np.argsort(dest, kind="stable")
+        same = dest[order][1:] == dest[order][:-1]
+        v = values(*val)[order]
+        if (same & (v[1:] != v[:-1])).any():
+            raise NoNativeKernel(f"{proxy.name}: two work-items store different values to one element; "
+                                 "the simulator keeps the last one's, a launch whichever finishes last")
+    else:
+        # too many to enumerate: every (group id, local id) pair must walk a
+        # dimension of its own as a global id does (coefficients s * n, s)
+        used = set()
+        ok = True
+        for c, g, l in idx:
+            nz = [k for k in range(rank) if g[k] or l[k]]
+            if len(nz) > 1 or (nz and nz[0] in used):
+                ok = False
+            for k in nz:
+                used.add(k)
+                lk = extents[k][1]
+                if not ((l[k] != 0 and g[k] == l[k] * lk) or (lk == 1 and g[k] != 0)):
+                    ok = False
+        moving = [k for k in range(rank) if extents[k][0] > 1 or extents[k][1] > 1]
+        if not ok or any(k not in used for k in moving):
+            raise NoNativeKernel(f"{proxy.name}: {stores} stores are too many to check that no two of them "
+                                 "put different values into one element, and the index is not a global id")
 
     def make(mem, ctx):
         return [rt.plan_id_scatter(_Arr(mem[proxy.index], ctx), idx, val, n_groups, group_shape,

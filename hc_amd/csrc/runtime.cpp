@@ -373,14 +373,16 @@ OlDevice olCreateDevice(const char *desc, OlErrorCallback errCallback,
   // Set-up for the entry point that allocates nothing: this GPU's address of the
   // static scratch array, and the kernels it launches.  A failure here only
   // makes that entry point refuse; every other one works without either.
+  // (Its failure is not this call's: the device is created, and the entry point
+  // says why it cannot run when it is called.)
   char why[200] = {0};
-  if (hcamdInternalScratchSetup(dev->index, why, sizeof(why))) {
-    dev->report("%s", why);
-  } else {
+  if (!hcamdInternalScratchSetup(dev->index, why, sizeof(why))) {
     dev->colsKernelsReady = true;
+    // every kernel a column reduction can launch, whatever the "cols" variant
     for (const char *name : {"hcamd_map_reduce_cols_n1u4", "hcamd_map_reduce_cols_n2u2",
                              "hcamd_map_reduce_cols_n4u1", "hcamd_cols_sum_f32",
-                             "hcamd_cols_sumsq_f32", "hcamd_cols_fold_f32"})
+                             "hcamd_cols_sumsq_f32", "hcamd_cols_sum_f32_w4u8",
+                             "hcamd_cols_sumsq_f32_w4u8", "hcamd_cols_fold_f32"})
       if (!builtinKernel(dev.get(), "map", name))
         dev->colsKernelsReady = false;
   }
@@ -956,6 +958,11 @@ int hcamdLaunchIdScatter(OlQueue q, void *out, int outType, size_t outRank,
     return 0;
   if (threads > 1024) {
     dev->report("%s: a group of %zu work-items (at most 1024 fit one workgroup)", who, threads);
+    return 1;
+  }
+  if (grid[1] > 65535 || grid[2] > 65535 || grid[0] > 0x7fffffffull) {
+    dev->report("%s: %zu x %zu x %zu groups (at most 65535 along every dimension but the last)", who,
+                grid[2], grid[1], grid[0]);
     return 1;
   }
   for (size_t d = 0; d < outRank; ++d) {

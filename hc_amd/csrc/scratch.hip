@@ -58,7 +58,8 @@ int hcamdLaunchMapReduceColsNoAlloc(OlQueue q, int kind, const HcamdMapInstr *pr
     return 1;
   void *ptr = device < kMaxDevices ? g_scratchOn[device] : nullptr;
   if (!ptr) {
-    hcamdInternalReport(q, "%s: no scratch array on device %d", who, device);
+    hcamdInternalReport(q, "%s: no scratch array on device %d (its address is looked up when the "
+                           "device is created, for device indices below %d)", who, device, kMaxDevices);
     return 1;
   }
   if (!hcamdInternalColsKernelsReady(q)) {

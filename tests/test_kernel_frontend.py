@@ -1756,6 +1756,44 @@ def test_workitem_scope_binds_ids_and_elementwise_statements(ctx):
     with pytest.raises(NoNativeKernel, match="wi.global_id"):
         shifted.plan(x, z, ctx=ctx)
 
+    # stores of ids whose outcome would depend on the order of the work-items, or
+    # on NumPy's wrap-around of negative indices, are refused
+    def id_body(index, value, group=64):
+        @kernel(work_shape=N, group_shape=group)
+        def k(gr: CurrentGroup, out: Buffer[N, DT]):
+            @gr.workitems
+            def inner(wi: CurrentWorkitem):
+                out[index(gr, wi)] = value(gr, wi)
+
+            inner()
+        return k
+
+    o = FakeDev((256,), "int32")
+    with pytest.raises(NoNativeKernel, match="different values to one element"):
+        id_body(lambda gr, wi: gr.id[0], lambda gr, wi: wi.local_id()[0]).plan(o, ctx=ctx)
+    with pytest.raises(NoNativeKernel, match="goes below 0"):
+        id_body(lambda gr, wi: wi.global_id()[0] - 1, lambda gr, wi: wi.local_id()[0]).plan(o, ctx=ctx)
+    # the same element from every work-item of a group, but the same value: fine
+    (p,) = id_body(lambda gr, wi: gr.id[0], lambda gr, wi: gr.id[0] * 3).plan(o, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchIdScatter
+    # more stores than can be enumerated: a global id is still known to be one-to-one
+    big = FakeDev((1 << 24,), "int32")
+    (p,) = id_body(lambda gr, wi: wi.global_id()[0], lambda gr, wi: wi.local_id()[0], group=256).plan(big, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchIdScatter
+    with pytest.raises(NoNativeKernel, match="too many to check"):
+        id_body(lambda gr, wi: wi.global_id()[0] - gr.id[0], lambda gr, wi: wi.local_id()[0], group=256).plan(big, ctx=ctx)
+
+    @kernel(work_shape=(N, 8), group_shape=(1, 8))
+    def tall(gr: CurrentGroup, out: Buffer[N, 8, DT]):
+        @gr.workitems
+        def inner(wi: CurrentWorkitem):
+            out[wi.global_id()] = wi.local_id()[1]
+
+        inner()
+
+    with pytest.raises(NoNativeKernel, match="at most 65535"):
+        tall.plan(FakeDev((70_000, 8), "int32"), ctx=ctx)
+
 
 def test_vload_needs_a_static_shape(ctx):
     """docs/langref.md:226-243 of the reference: a vector's shape must be known at

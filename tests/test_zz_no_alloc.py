@@ -56,6 +56,41 @@ def test_two_calls_in_a_row_equal_the_workspace_entry_point():
         assert np.allclose(got.view(np.float32), ref, rtol=1e-5)
 
 
+def test_launches_leave_the_free_device_memory_as_it_is():
+    """The entry point allocates nothing: the free device memory the HIP runtime
+    reports is the same before and after its launches, under every variant of the
+    column-reduction kernels (their kernels are all resolved when the device is
+    created, so no code object is loaded on the way either)."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+
+    def free_bytes():
+        free, total = C.c_size_t(), C.c_size_t()
+        assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+        return free.value
+
+    rng = np.random.default_rng(25)
+    x_host = rng.standard_normal((150_000, 256)).astype(np.float32)
+    x = rt.to_device(x_host)
+    out = rt.DeviceArray((256,), np.float32)
+    plan = rt.plan_map_reduce_cols("sum", [I("in", 0), I("mul_in", 0)], [x], out)
+    noalloc = rt.Plan(plan.ctx, rt.hcamdLaunchMapReduceColsNoAlloc, tuple(plan.args[:-2]),
+                      "hcamdLaunchMapReduceColsNoAlloc", plan.keep)
+    plan.ctx.synchronize()
+    try:
+        for variant in (0, 1, 2):
+            rt.set_variant("cols", variant)
+            say("no-alloc column reduction: free memory around launches, cols variant", variant)
+            before = free_bytes()
+            for _ in range(3):
+                noalloc.launch(sync=True)
+            assert free_bytes() == before, variant
+            ref = (x_host.astype(np.float64) ** 2).sum(axis=0)
+            assert np.allclose(out.to_host(), ref, rtol=1e-5)
+    finally:
+        rt.set_variant("cols", 0)
+
+
 def test_one_launch_windows_and_refusals():
     rng = np.random.default_rng(24)
     x = rng.standard_normal((64, 1000)).astype(np.float32)      # no bands: scratch unused
