@@ -498,7 +498,7 @@ def make_workloads(rt, wl):
     class X5(Workload):
         """Layer normalisation with weight and bias over the rows of the C3 matrix,
         written as a kernel body with mean and var along axis 1 and launched
-        through the @kernel front-end (a five-stage row program)."""
+        through the @kernel front-end (a six-stage row program)."""
 
         def setup(self, rt):
             from hc_amd.examples import layer_norm
