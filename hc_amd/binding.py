@@ -2418,6 +2418,21 @@ def simplify(t: Tile, memo=None) -> Tile:
     folded = _assembled_reduce(out)
     if folded is not None:
         out = folded
+    if _is(out, "slice", 1) and _const(out.args[0]) and _const_value(out.args[0]) is not None:
+        # part of an allocated tile (CurrentGroup.vec with a shape): the same constant
+        out = _const_tile(out.shape, out.dtype_name, out.args[0])
+    elif _is(out, "update", 2) and _const(out.args[0]) and \
+            all(k == (0, n) for k, n in zip(out.attrs["key"], out.shape)):
+        # `tile[:] = value` on a freshly allocated tile (python/hckernel/kernel_api.py:125-131:
+        # value where it is active, the allocator's fill elsewhere, every element active)
+        old, value = out.args
+        if _const(value) and _const_value(value) is not None:
+            out = _const_tile(out.shape, out.dtype_name, value)
+        elif value.shape == out.shape and not value.attrs.get("plain"):
+            filled = value if value.dtype_name == out.dtype_name else \
+                Tile("astype", (value,), out.shape, out.dtype_name)
+            memo.setdefault("overlays", []).append(filled)
+            out = filled
     if out.op == "count" and _is_reduction(out) and not _maybe_masked(out.args[0]):
         # nothing can deactivate an element: the number of active elements is the
         # number of elements (tiles hold whole rows / columns of their arrays)
@@ -2431,6 +2446,89 @@ def simplify(t: Tile, memo=None) -> Tile:
         out = Tile("const", (), (), "float32", value=float(n), weak=False, exact=int(n), counted=True)
     memo[id(t)] = out
     return out
+
+
+def _const_value(t: Tile):
+    """The number a constant tile holds (exactly, for integers), or None."""
+    if _is(t, "full") and t.args:
+        t = t.args[0]
+    v = t.attrs.get("exact")
+    return t.attrs.get("value") if v is None else v
+
+
+def _const_tile(shape, dtype, like: Tile) -> Tile:
+    v = _const_value(like)
+    c = Tile("const", (), (), dtype, value=float(v), weak=False,
+             **({"exact": int(v)} if float(v).is_integer() else {}))
+    return Tile("full", (c,), tuple(shape), dtype, value=float(v))
+
+
+def _overlay_guard(view, value, overlays, n_groups):
+    """A tile filled by `tile[:] = loaded` is active everywhere and holds the
+    allocator's fill where the loaded tile is not; that is the loaded tile
+    itself as long as the store's window is no larger than the loads'."""
+    if not any(_contains(value, o) for o in overlays):
+        return
+    dst = window_of(view, value.shape, n_groups)
+    for t in _walk(value):
+        if _is(t, "load"):
+            w = window_of(t.attrs["view"], t.shape, n_groups)
+            if w.extent != dst.extent or w.driver != dst.driver:
+                raise NoNativeKernel(
+                    f"{view.base.name}: a tile filled by assignment is stored to a window larger than "
+                    "what was loaded into it; the elements beyond would receive the allocator's "
+                    "initial value, which no native kernel writes")
+
+
+def _walk(t: Tile, seen=None):
+    seen = set() if seen is None else seen
+    if id(t) in seen:
+        return
+    seen.add(id(t))
+    yield t
+    for a in t.args:
+        if isinstance(a, Tile):
+            yield from _walk(a, seen)
+
+
+def _contains(t: Tile, node: Tile) -> bool:
+    return any(u is node for u in _walk(t))
+
+
+_FILL_TYPES = {"float32": 4, "float16": 2, "int32": 4, "bool": 1}
+
+
+def match_fill(dst_view, value, n_groups):
+    """A constant tile (CurrentGroup.full / zeros / ones / empty, or arithmetic
+    on constants that folded to one) stored to a window: a program that only
+    pushes the constant, with no operand."""
+    if not _const(value) or value.shape == ():
+        return None
+    v = _const_value(value)
+    out_dt = dst_view.base.dtype_name
+    if v is None or out_dt not in _FILL_TYPES:
+        return None
+    w = window_of(dst_view, value.shape, n_groups)
+    if len(w.extent) > 2:
+        raise NoNativeKernel("only 1-D and 2-D buffers have native kernels")
+    if out_dt in ("int32", "bool"):
+        iv = int(bool(v)) if out_dt == "bool" else int(v)
+        if float(v) != iv and out_dt == "int32":
+            raise NoNativeKernel(f"constant {v} stored to an int32 buffer")
+        if not -2 ** 31 <= iv < 2 ** 31:
+            raise NoNativeKernel(f"constant {v} is not an int32")
+        program = [("const", 0, iv)]
+
+        def make(mem, ctx):
+            return [rt.plan_imap(program, [], _Arr(_sub(mem[w.buffer], w.extent), ctx), out_bool=out_dt == "bool")]
+    else:
+        program = [("const", 0, _round_to(float(v), out_dt))]
+        types = [rt.F16 if out_dt == "float16" else rt.F32]
+
+        def make(mem, ctx):
+            return [rt.plan_map(program, [], _Arr(_sub(mem[w.buffer], w.extent), ctx), types)]
+    make.program = program
+    return make
 
 
 def match_id_store(proxy, index, value, per_item, n_groups, group_shape):
@@ -2524,6 +2622,8 @@ def bind(stores, n_groups, atomics=(), mapped_stores=(), id_stores=(), group_sha
         raise NoNativeKernel("the kernel body stores nothing")
     memo = {}
     stores = [(view, simplify(value, memo)) for view, value in stores]
+    for view, value in stores:
+        _overlay_guard(view, value, memo.get("overlays", ()), n_groups)
     id_makers = [match_id_store(p, i, v, per, n_groups, group_shape) for p, i, v, per in id_stores]
     if id_stores and not (stores or atomics or mapped_stores):
         return id_makers
@@ -2545,7 +2645,7 @@ def bind(stores, n_groups, atomics=(), mapped_stores=(), id_stores=(), group_sha
         if q is not None:
             return makers + [q]
         for view, value in stores:
-            for matcher in (match_copy, match_imap, match_add, match_fma, match_softmax, match_gemm,
+            for matcher in (match_fill, match_copy, match_imap, match_add, match_fma, match_softmax, match_gemm,
                             match_gather_gemm, match_gather_map, match_pairwise, match_cols,
                             match_cols_tile, match_rows, match_map, match_fmap):
                 mk = matcher(view, value, n_groups)

@@ -1227,6 +1227,61 @@ def test_tile_mask_is_stored_as_a_plain_bool_array():
             assert_array_equal(g.to_host().view(np.uint8), w.view(np.uint8))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.int32])
+def test_allocated_tiles_as_values(dtype):
+    """CurrentGroup.full / zeros / ones / empty and their v-forms
+    (python/hckernel/kernel_api.py:347-376,433-434) as values: a constant tile
+    stored as it is (1-D, a ragged 2-D window, a bool buffer), as an operand, as an
+    accumulator that loads are added to, and as a tile that is filled by
+    assignment; the bytes the simulator leaves, untouched elements included."""
+    N, M = sym.N, sym.M
+    T = dtype
+
+    def one_d(gr: CurrentGroup, a: Buffer[N, DT], c: Buffer[N, DT], s: Buffer[N, DT], acc: Buffer[N, DT],
+              filled: Buffer[N, DT], flag: Buffer[N, DT]):
+        o = gr.work_offset[0]
+        x = gr.load(a[o:], shape=gr.shape)
+        gr.store(c[o:], gr.full(gr.shape, dtype=T, fill_value=42))
+        gr.store(s[o:], x * gr.vfull(gr.shape, dtype=T, fill_value=3) + gr.ones(gr.shape, dtype=T))
+        t = gr.vzeros(gr.shape, dtype=T)
+        t += x
+        t += gr.vload(a[o:], shape=gr.shape)
+        gr.store(acc[o:], t)
+        e = gr.empty(gr.shape, dtype=T)
+        e[:] = x - gr.vones(gr.shape, dtype=T)
+        gr.store(filled[o:], gr.vec(e))
+        gr.store(flag[o:], gr.zeros(gr.shape, dtype=np.bool_))
+
+    n = 1003
+    rng = np.random.default_rng(21)
+    a = rng.integers(-50, 50, n).astype(dtype)
+    want = [np.full(n, 7, dtype) for _ in range(4)] + [np.full(n, 1, np.bool_)]
+    sim_kernel(work_shape=N, group_shape=256)(one_d)(a, *want)
+    got = [rt.to_device(np.full(n, 7, dtype)) for _ in range(4)] + [rt.to_device(np.full(n, 1, np.bool_))]
+    kernel(work_shape=N, group_shape=256)(one_d)(rt.to_device(a), *got)
+    for g, w in zip(got, want):
+        assert_array_equal(g.to_host().view(np.uint8), w.view(np.uint8))
+
+    def two_d(gr: CurrentGroup, c: Buffer[M, N, DT]):
+        i, j = gr.work_offset
+        gr.store(c[i:, j:], gr.full(gr.shape, dtype=T, fill_value=5))
+
+    want2 = np.full((61, 123), 9, dtype)            # ragged against the 8 x 32 groups
+    sim_kernel(work_shape=(M, N), group_shape=(8, 32))(two_d)(want2)
+    dev = rt.to_device(np.full((61, 123), 9, dtype))
+    kernel(work_shape=(M, N), group_shape=(8, 32))(two_d)(dev)
+    assert_array_equal(dev.to_host(), want2)
+    assert (want2 == 5).all()
+    torch = pytest.importorskip("torch")
+    if torch.cuda.is_available():
+        # a window of a larger tensor: the rest must stay as it was
+        big = torch.full((70, 131), 9, dtype=getattr(torch, np.dtype(dtype).name), device="cuda")
+        torch.cuda.synchronize()
+        kernel(work_shape=(M, N), group_shape=(8, 32))(two_d)(big[3:64, 2:125])
+        host = big.cpu().numpy()
+        assert (host[3:64, 2:125] == 5).all() and (host == 9).sum() == 70 * 131 - 61 * 123
+
+
 def test_fp16_maximum_and_minimum_of_signed_zeros_follow_numpy():
     """NumPy's fp16 maximum / minimum return the first of two equal values, its
     fp32 ones the second: +0 against -0 shows it.  Bits must equal the simulator's

@@ -1347,6 +1347,54 @@ def test_what_a_traced_tile_cannot_give_says_why(ctx):
     assert p.fn is rt.hcamdLaunchIMap and imap_program(p)[-1][0] == "active"
 
 
+def test_allocated_tiles_bind_as_constants_and_assignment_targets(ctx):
+    """CurrentGroup.full / zeros / ones / empty / vec (python/hckernel/kernel_api.py:347-376):
+    a constant tile stored as it is is a program that pushes the constant and reads
+    nothing; `tile[:] = value` on a fresh tile is the value; a part of a constant
+    tile is the constant."""
+    N = sym.N
+
+    def body(fn):
+        @kernel(work_shape=N, group_shape=256)
+        def k(gr: CurrentGroup, a: Buffer[N, DT], out: Buffer[N, DT]):
+            o = gr.work_offset[0]
+            gr.store(out[o:], fn(gr, gr.load(a[o:], shape=gr.shape)))
+        return k
+
+    f32, f16, i32 = (FakeDev((1000,), t) for t in ("float32", "float16", "int32"))
+    (p,) = body(lambda gr, x: gr.full(gr.shape, dtype=np.float32, fill_value=2.5)).plan(f32, f32, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchMap and map_program(p) == [("const", 0, 2.5)] and p.args[6] == 0   # no operand
+    (p,) = body(lambda gr, x: gr.vones(gr.shape, dtype=np.float16)).plan(f16, f16, ctx=ctx)
+    assert map_program(p) == [("const", 0, 1.0)]
+    (p,) = body(lambda gr, x: gr.full(gr.shape, dtype=np.int32, fill_value=-7)).plan(i32, i32, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchIMap and imap_program(p) == [("const", 0, -7)]
+    (p,) = body(lambda gr, x: gr.zeros(gr.shape, dtype=np.bool_)).plan(i32, FakeDev((1000,), "bool"), ctx=ctx)
+    assert p.fn is rt.hcamdLaunchIMap and imap_program(p) == [("const", 0, 0)]
+    with pytest.raises(NoNativeKernel, match="int32 buffer"):
+        body(lambda gr, x: gr.full(gr.shape, dtype=np.int32, fill_value=0.5)).plan(i32, i32, ctx=ctx)
+
+    def filled(gr, x):
+        t = gr.empty(gr.shape, dtype=np.float32)
+        t[:] = x * np.float32(2)
+        return gr.vec(t)
+    (p,) = body(filled).plan(f32, f32, ctx=ctx)
+    assert map_program(p) == [("in", 0, 0.0), ("muli", 0, 2.0)]
+    # stored to a larger window the tile would carry the allocator's fill beyond the loaded part
+    M = sym.M
+
+    @kernel(work_shape=M, group_shape=256)
+    def wider(gr: CurrentGroup, a: Buffer[N, DT], out: Buffer[M, DT]):
+        o = gr.work_offset[0]
+        gr.store(out[o:], filled(gr, gr.load(a[o:], shape=gr.shape)))
+    with pytest.raises(NoNativeKernel, match=r"allocator's\s+initial value"):
+        wider.plan(f32, FakeDev((1200,), "float32"), ctx=ctx)
+
+    def part_of_constant(gr, x):
+        return x + gr.vec(gr.full((512,), dtype=np.float32, fill_value=3), shape=gr.shape)
+    (p,) = body(part_of_constant).plan(f32, f32, ctx=ctx)
+    assert map_program(p) == [("in", 0, 0.0), ("addi", 0, 3.0)]
+
+
 def test_row_bodies_without_native_code_say_why(ctx):
     M, N, GM = sym.M, sym.N, sym.GM
 
