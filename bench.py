@@ -48,7 +48,7 @@ PREWARM_SECONDS = 0.4        # untimed, per workload, before the W warm-up steps
 # commands listed in profiles/hbm_traffic_pmc.txt; a figure is reported only
 # while the kernel that ran is the kernel that was measured.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-TRAFFIC_WORKLOADS = ("c0", "c1", "c2", "c3", "c4", "c5", "x6")
+TRAFFIC_WORKLOADS = ("c0", "c1", "c2", "c3", "c4", "c5", "x5", "x6", "x8")
 C0_KIB = 256 * 1024          # c0 reads and writes 256 MiB
 
 
@@ -71,14 +71,24 @@ def traffic_from(dirname, launches):
     import csv
 
     def per_launch(w, counter):
+        # a step of a workload may be several kernels (x6: bands, then their fold):
+        # their counters add up, and the record is keyed by the last one, which is
+        # the name the bench line carries
         total = collections.defaultdict(float)
+        last = None
         with open(os.path.join(dirname, f"{w}_{counter}_counter_collection.csv")) as f:
-            for r in csv.DictReader(f):
-                k = r["Kernel_Name"]
-                if k.startswith("hcamd_") and "fill" not in k:
-                    total[k] += float(r["Counter_Value"])
-        (kernel, value), = total.items()       # one kernel per workload
-        return kernel, value / launches
+            rows = sorted(csv.DictReader(f), key=lambda r: int(r.get("Dispatch_Id", 0)))
+        for r in rows:
+            k = r["Kernel_Name"]
+            if k.startswith("hcamd_") and "fill" not in k:
+                total[k] += float(r["Counter_Value"])
+                last = k
+        if last is None:
+            raise OSError(f"no kernel of the library in the {counter} file of {w}")
+        kernels.setdefault(w, sorted(total))
+        return last, sum(total.values()) / launches
+
+    kernels = {}
 
     _, f0 = per_launch("c0", "FETCH_SIZE")
     _, w0 = per_launch("c0", "WRITE_SIZE")
@@ -95,7 +105,8 @@ def traffic_from(dirname, launches):
         except OSError:
             continue
         out["workloads"][w] = {
-            "kernel": kernel, "FETCH_SIZE_KiB": round(fetch, 1), "WRITE_SIZE_KiB": round(write, 1),
+            "kernel": kernel, "kernels": kernels[w],
+            "FETCH_SIZE_KiB": round(fetch, 1), "WRITE_SIZE_KiB": round(write, 1),
             "bytes": int((fetch * scale["FETCH_SIZE"] + write * scale["WRITE_SIZE"]) * 1024)}
     with open(TRAFFIC_FILE, "w") as f:
         json.dump(out, f, indent=1, sort_keys=True)
@@ -553,6 +564,35 @@ def make_workloads(rt, wl):
         def cpu(self):
             return _best_of(lambda: self._numpy(self.x), 2), "full size, NumPy fp32", 1
 
+    class X8(Workload):
+        """Root-mean-square normalisation with an fp32 weight over the rows of the C4
+        matrix (fp16 in, fp32 math, fp16 out), written as a kernel body and
+        launched through the @kernel front-end."""
+
+        def setup(self, rt):
+            from hc_amd.examples import rms_norm_f16
+            self.kernel = rms_norm_f16()
+            (self.x,) = W.inputs_c4()
+            self.g = np.random.default_rng(9).standard_normal(self.x.shape[1]).astype(np.float32)
+            return [(rt.to_device(self.x), rt.to_device(self.g), rt.DeviceArray(self.x.shape, np.float16))
+                    for _ in range(ROTATE)]
+
+        def plan(self, rt, s):
+            (p,) = self.kernel.plan_rows(*s)
+            return p
+
+        def _numpy(self, x):
+            return x / np.sqrt((x * x).mean(axis=1, keepdims=True) + x.dtype.type(1e-6)) * self.g.astype(x.dtype)
+
+        def check(self, rt, s):
+            got, want = s[2].to_host().astype(np.float64), self._numpy(self.x.astype(np.float64))
+            ok = np.allclose(got, want, rtol=1.1e-3, atol=1e-6)
+            return {"parity": "one fp16 ulp (rtol 1.1e-3) vs fp64" if ok else "MISMATCH", "ok": bool(ok)}
+
+        def cpu(self):
+            return _best_of(lambda: self._numpy(self.x.astype(np.float32)).astype(np.float16), 2), \
+                "full size, NumPy fp32", 1
+
     table = {
         "c0": C0("c0", "copy 256 MiB int32 (calibration)", "u32", "hbm", 2 * 4 * 64 * 1024 * 1024,
                  "GB/s"),
@@ -577,6 +617,8 @@ def make_workloads(rt, wl):
                  "hbm", W.work_c3() // 2 + 4 * 8192, "GB/s"),
         "x7": X7("x7", "map kernel: vadd fp32 N=16777259 as a 2-instruction program", "f32", "hbm",
                  W.work_c1(), "GB/s"),
+        "x8": X8("x8", "row program: rms norm fp16 16384x4096 with an fp32 weight (fp32 math)", "f16", "hbm",
+                 2 * 2 * 16384 * 4096 + 4 * 4096, "GB/s"),
     }
     # the mix and size of each memory-bound configuration, then the plain streams
     for key, n_reads, write, mib in STREAMS:
@@ -586,7 +628,7 @@ def make_workloads(rt, wl):
     elif wl == "streams":
         keys = [k for k, *_ in STREAMS]
     elif wl == "extra":
-        keys = ["x1", "x2", "x3", "x4", "x5", "x6", "x7"]
+        keys = ["x1", "x2", "x3", "x4", "x5", "x6", "x7", "x8"]
     else:
         keys = [wl]
     return [table[k] for k in keys]
@@ -661,7 +703,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="all", choices=["all", "streams", "c0", "c1", "c2", "c3", "c4", "c5", "v5", "extra", "x1", "x2", "x3",
-                             "x4", "x5", "x6", "x7"] + [k for k, *_ in STREAMS])
+                             "x4", "x5", "x6", "x7", "x8"] + [k for k, *_ in STREAMS])
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy CPU baseline")
     ap.add_argument("--variant", action="append", default=[], metavar="FAMILY=N",
                     help="measure kernel variant N of a family (hcamdSetVariant), e.g. gemm=14; "

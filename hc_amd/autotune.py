@@ -31,7 +31,7 @@ _FAMILIES = {
     "hcamdLaunchAddF32": ("add", tuple(range(1, 9))),
     "hcamdLaunchFmaF16": ("fma", tuple(range(1, 7))),
     "hcamdLaunchCopy2D": ("copy", tuple(range(1, 9))),
-    "hcamdLaunchSoftmaxF32": ("softmax", (0, 3, 4, 5, 6, 7, 8, 9, 10)),
+    "hcamdLaunchSoftmaxF32": ("softmax", (0, 3, 4, 5, 6, 7, 8, 9, 10, 11)),
     "hcamdLaunchQuantizeF16I8": ("quantize", (0, 2, 3, 4, 7, 8, 9, 10, 11)),
     "hcamdLaunchGemmBF16": ("gemm", (1, 2, 3, 4, 5, 7, 8, 9, 10, 11, 12)),
     "hcamdGatherGemmLaunchF32": ("gather", (1, 2, 3, 4, 5, 6)),

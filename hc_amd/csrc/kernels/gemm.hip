@@ -877,6 +877,19 @@ HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_loads_to_regs, 6)
 HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_b_direct, __bf16, 256, 256, 2, 4, 16, 2, false, 7)
 HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_no_stores, 8)
 HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_two_tiles, 9)
+// other hand orders of the four-wave shape (these do compute the product; they are
+// here because only measurements select them): LDS reads over the first 48 MFMAs
+// of a half-step's 64; a load every second MFMA; the eight A blocks under one Bt block
+#define HCAMD_GEMM_W2X2(NAME, RS, LF, LS, ORDER)                                \
+  extern "C" __global__ __launch_bounds__(256) void NAME(                       \
+      const __bf16 *A, size_t lda, const __bf16 *Bt, size_t ldb, __bf16 *C,     \
+      size_t ldc, int M, int N, int K) {                                        \
+    gemm_tile_pipelined<__bf16, 256, 256, 2, 2, 16, false, 2, false, 0, 0, RS,  \
+                        LF, LS, ORDER>(A, lda, Bt, ldb, C, ldc, M, N, K);       \
+  }
+HCAMD_GEMM_W2X2(hcamd_gemm_bf16_probe_w2x2_reads48, 48, 1, 4, 0)
+HCAMD_GEMM_W2X2(hcamd_gemm_bf16_probe_w2x2_loads2, 24, 1, 2, 0)
+HCAMD_GEMM_W2X2(hcamd_gemm_bf16_probe_w2x2_a_inner, 24, 1, 4, 1)
 #endif
 HCAMD_GEMM_PE(hcamd_gemm_bf16_p256x256_w2x4_edge, __bf16, 256, 256, 2, 4, 16)
 HCAMD_GEMM_PE(hcamd_gemm_f16_p256x256_w2x4_edge, _Float16, 256, 256, 2, 4, 16)

@@ -964,15 +964,15 @@ __device__ __forceinline__ void cols_sum_f32(const float *__restrict__ x, size_t
       *reinterpret_cast<f32x4 *>(partial + (size_t)blockIdx.y * cols_pad + col) = total;  \
     });                                                                                   \
   }
-// 16 waves to a workgroup measured fastest, however many rows each has in flight
-// (root mean square down the columns of 4096 x 8192, both launches: 16 waves x 4,
-// 2 or 1 rows 32.7-32.9 us; 8 waves x 8, 4 or 2 rows 34.5-34.9; 4 waves x 8 or 4
-// rows 39.6-42.7; 2 x 8 41.2; the general kernel 36.8): what counts is the number
-// of waves the launch has.  With bands of 64 rows, 16 waves to a band are four
-// times the wave slots of the device, which the waves pass through one after the
-// other; 4 waves to a band fill the slots once and all wait at the same time.
-HCAMD_COLS_SUM(hcamd_cols_sum_f32, false, 16, 4)
-HCAMD_COLS_SUM(hcamd_cols_sumsq_f32, true, 16, 4)
+// 16 waves to a workgroup measured fastest, and many short bands (root mean
+// square down the columns of 4096 x 8192, both launches; bands of 32 / 48 / 64
+// rows): 16 waves x 1 row in flight 24.1 / 24.2 / 27.8 us, 16 x 2 24.5 / 24.7 /
+// 27.0, 16 x 4 24.7 / 24.5 / 27.0, 8 x 2 24.7 / 24.3 / 29.9, 4 x 4 27.5 / 25.7 /
+// 37.5, 2 x 8 28.3 / 26.1 / 35.9: what counts is the number of waves the launch
+// has, each with a row or two to fetch (a read-only stream of the same bytes
+// takes 19.9 us, this kernel's launch alone 21.1-21.5 us).
+HCAMD_COLS_SUM(hcamd_cols_sum_f32, false, 16, 2)
+HCAMD_COLS_SUM(hcamd_cols_sumsq_f32, true, 16, 2)
 HCAMD_COLS_SUM(hcamd_cols_sum_f32_w4u8, false, 4, 8)
 HCAMD_COLS_SUM(hcamd_cols_sumsq_f32_w4u8, true, 4, 8)
 

@@ -731,7 +731,8 @@ int hcamdDeviceInfo(OlDevice dev, int *computeUnits, int *clockKHz,
 
 namespace {
 // Variants 17..22, 26, 28 and 29 of "gemm" are measurement builds of the default kernel
-// with one part of its loop taken out: what they leave in C is not the product.
+// with one part of its loop taken out: what they leave in C is not the product
+// (30..32 are further hand orders of variant 27 that only measurements select).
 // They exist only in a library built with HCAMD_PROBES defined (`python -m
 // hc_amd.build --probes`); any other build refuses to select them.
 bool variantIsAbsentProbe(const char *family, int variant) {
@@ -740,7 +741,7 @@ bool variantIsAbsentProbe(const char *family, int variant) {
   return false;
 #else
   return std::strcmp(family, "gemm") == 0 &&
-         ((variant >= 17 && variant <= 22) || variant == 26 || variant == 28 || variant == 29);
+         ((variant >= 17 && variant <= 22) || variant == 26 || (variant >= 28 && variant <= 32));
 #endif
 }
 } // namespace
@@ -1779,6 +1780,21 @@ void colBands(size_t rows, size_t cols, size_t &bands, size_t &band) {
   bands = ceilDiv(rows, band);
 }
 
+// The sums of x and of x * x over a dense fp32 window have band kernels of their
+// own (hcamd_cols_sum_f32, hcamd_cols_sumsq_f32), which run fastest with many
+// short bands: about sixteen workgroups of sixteen waves for each compute
+// unit, 32 rows or more to a band (root mean square down 4096 x 8192, both
+// launches: bands of 32 rows 24.1 us, of 64 rows 27.0 us; the partial sums are
+// then 1/32 of the window).
+bool colDenseShape(size_t cols) { return cols % 8 == 0 && cols >= 256; }
+void colBandsDense(size_t rows, size_t cols, size_t &bands, size_t &band) {
+  const size_t blocks = ceilDiv(cols, (size_t)256);
+  const size_t wanted = ceilDiv((size_t)4096, blocks);
+  bands = std::max(std::min(wanted, rows / 32), (size_t)1);
+  band = ceilDiv(ceilDiv(rows, bands), (size_t)32) * 32;
+  bands = ceilDiv(rows, band);
+}
+
 // The bands of the first launch are the rows of the second, which always
 // finishes: it spreads its few rows over the lanes of a wave (fewer lanes per
 // row), so that a wave has them all in flight in one or two turns.
@@ -1794,6 +1810,12 @@ size_t hcamdMapReduceColsWorkspace(size_t rows, size_t cols) noexcept {
     return 0;
   size_t bands, band;
   colBands(rows, cols, bands, band);
+  if (bands > 1 && colDenseShape(cols)) {
+    // (whichever kernel the program gets: the caller sizes the workspace by the shape alone)
+    size_t denseBands, denseBand;
+    colBandsDense(rows, cols, denseBands, denseBand);
+    bands = std::max(bands, denseBands);
+  }
   return bands > 1 ? bands * ceilDiv(cols, (size_t)8) * 8 * sizeof(float) : 0;
 }
 
@@ -1871,6 +1893,19 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
   const size_t colsPad = ceilDiv(cols, (size_t)8) * 8;
   size_t bands, band;
   colBands(rows, cols, bands, band);
+  // The sums of x and of x * x over a dense fp32 window at least a wave's 256
+  // columns wide have a kernel of their own for the first launch (variant 1 of
+  // "cols" keeps the general one): 4096 x 8192, both launches, 36.8 -> 32.7 us,
+  // and 24.1 us with the shorter bands that kernel likes.
+  const bool plain = nInstr == 1 && prog[0].op == HCAMD_MAP_IN;
+  const bool square = (nInstr == 3 && prog[0].op == HCAMD_MAP_IN && prog[1].op == HCAMD_MAP_IN &&
+                       prog[2].op == HCAMD_MAP_MUL) ||
+                      (nInstr == 2 && prog[0].op == HCAMD_MAP_IN && prog[1].op == HCAMD_MAP_MUL_IN);
+  const bool denseSum = bands > 1 && (plain || square) && kind == HCAMD_COLS_SUM && nInputs == 1 &&
+                        inputTypes[0] == HCAMD_F32 && inputLd[0] != 0 && allVec && colDenseShape(cols) &&
+                        variantOf("cols") != 1;
+  if (denseSum)
+    colBandsDense(rows, cols, bands, band);
   const size_t floats = bands > 1 ? bands * colsPad : 0;
   if (floats && (!workspace || !aligned16(workspace) || workspaceBytes < floats * sizeof(float))) {
     dev->report("%s: workspace of %zu bytes, 16-byte aligned, needed (%zu given)", who,
@@ -1925,15 +1960,7 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
     return launchOne(a, c, nInputs, 1);
   }
   c.partial = static_cast<float *>(workspace);
-  // The sums of x and of x * x over a dense fp32 window at least a wave's 256
-  // columns wide have a kernel of their own for the first launch (variant 1 of
-  // "cols" keeps the general one): 4096 x 8192, both launches, 36.8 -> 32.7 us.
-  const bool plain = nInstr == 1 && prog[0].op == HCAMD_MAP_IN;
-  const bool square = (nInstr == 3 && prog[0].op == HCAMD_MAP_IN && prog[1].op == HCAMD_MAP_IN &&
-                       prog[2].op == HCAMD_MAP_MUL) ||
-                      (nInstr == 2 && prog[0].op == HCAMD_MAP_IN && prog[1].op == HCAMD_MAP_MUL_IN);
-  if ((plain || square) && kind == HCAMD_COLS_SUM && nInputs == 1 && inputTypes[0] == HCAMD_F32 &&
-      inputLd[0] != 0 && allVec && cols % 8 == 0 && cols >= 256 && variantOf("cols") != 1) {
+  if (denseSum) {
     // (variant 2: four waves to a workgroup with eight rows in flight each)
     const bool few = variantOf("cols") == 2;
     const size_t lanes = few ? 256 : 1024;
@@ -3297,6 +3324,10 @@ int hcamdLaunchSoftmaxF32(OlQueue q, const float *x, size_t ldx, float *y,
       // full rows: 1024 lanes per row, two 16-byte words per lane
       return launch1d(queue, "softmax", "hcamd_softmax_f32_g1024_v2_full_nt", rows, 1024,
                       args);
+    if (cols == 8192 && variant == 11)
+      // the same with one exchange of (maximum, sum) pairs between the waves
+      return launch1d(queue, "softmax", "hcamd_softmax_f32_g1024_v2_one_exchange_nt", rows, 1024,
+                      args);
     if (cols == 8192 && ((variant == 10 && rows >= 8 * cus) ||
                          (variant >= 5 && variant <= 9))) {
       // Full rows and enough of them: the persistent kernel, a fixed number of
@@ -3493,6 +3524,9 @@ int launchGemm(OlQueue q, bool half, const void *a, size_t lda, const void *bt,
       {"hcamd_gemm_bf16_p256x256_w2x2", 256, 256, 256},             // 27: four waves, 128 x 128 each
       {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_no_stores"), 256, 256, 512}, // 28: measurement only
       {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_two_tiles"), 256, 256, 512}, // 29: measurement only
+      {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_w2x2_reads48"), 256, 256, 256}, // 30..32: other hand orders of 27
+      {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_w2x2_loads2"), 256, 256, 256},  //         (the product, measurement builds only)
+      {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_w2x2_a_inner"), 256, 256, 256},
   };
   constexpr int kGeneral = 6;
   constexpr int kFirstPipelined = 7; // variants from here need K >= 128

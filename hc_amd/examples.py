@@ -69,6 +69,27 @@ def layer_norm(eps: float = 1e-5, rows_per_group: int = 8):
     return body
 
 
+def rms_norm_f16(eps: float = 1e-6, rows_per_group: int = 8):
+    """out = x / sqrt(mean(x * x) + eps) * weight along the rows of a float16
+    matrix, computed in float32 (the weight is float32) and stored as float16:
+    the second normalisation that is common enough to have a kernel of its own
+    behind the row-program entry point."""
+    M, N, GM = sym.M, sym.N, sym.GM
+    f = np.float32
+
+    @kernel(work_shape=M, group_shape=GM)
+    def body(gr: CurrentGroup, x: Buffer[M, N, DT], weight: Buffer[N, DT], out: Buffer[M, N, DT], gshape: GM):
+        m0, mb = gr.work_offset[0], gr.shape[0]
+        t = gr.load(x[m0:, :], shape=(mb, N)).astype(f)
+        ms = np.mean(np.square(t), axis=1, keepdims=True)
+        gr.store(out[m0:, :], (t / np.sqrt(ms + f(eps)) * gr.load(weight[:], shape=(N,))).astype(np.float16))
+
+    def plan(x, weight, out, **kw):
+        return body.plan(x, weight, out, rows_per_group, **kw)
+    body.plan_rows = plan
+    return body
+
+
 def column_rms(eps: float = 1e-6, cols_per_group: int = 512):
     """out[c] = sqrt(mean(x[:, c] ** 2) + eps) down the columns of a float32
     matrix: a body that reduces tiles holding whole columns along axis 0 (the

@@ -738,8 +738,8 @@ int hcamdLaunchGemmF16(OlQueue q, const void *a, size_t lda, const void *bt,
  * (block shape), "gather_fuse" (groups per workgroup; read by
  * hcamdGatherGemmCreate).
  * Process-wide, guarded by a lock.  Returns 1 for an unknown family, and for
- * the numbers of the measurement builds of the "gemm" family (17..22, 26, 28, 29,
- * whose output is not the product) unless the library was built with them
+ * the numbers of the measurement builds of the "gemm" family (17..22, 26, 28..32:
+ * most of them leave something other than the product in C) unless the library was built with them
  * (hc_amd_bench.h).  Every variant a default build accepts computes the same
  * result as variant 0. */
 int hcamdSetVariant(const char *family, int variant) HCAMD_NOEXCEPT;

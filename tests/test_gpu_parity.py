@@ -1214,7 +1214,7 @@ def test_softmax_variants_and_strided_rows(ctx):
     (x,) = cf.inputs_c3((rows, ld))
     want = cf.np_softmax(x[:, :cols])
     dx = dev(x)
-    for v in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10):
+    for v in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11):
         rt.set_variant("softmax", v)
         dy = poisoned((rows, ld), np.float32)
         rt.softmax_f32(_View(dx, (rows, cols), 0, (ld, 1)), _View(dy, (rows, cols), 0, (ld, 1)))
@@ -1235,7 +1235,7 @@ def test_softmax_variants_and_strided_rows(ctx):
         assert (out[:, 1 + width:].view(np.uint32) == POISON32).all()
 
 
-@pytest.mark.parametrize("cols,variant", [(1024, 0), (8192, 0), (8192, 5), (1023, 0), (8191, 0),
+@pytest.mark.parametrize("cols,variant", [(1024, 0), (8192, 0), (8192, 5), (8192, 11), (1023, 0), (8191, 0),
                                           (12345, 0), (20000, 0), (50257, 0), (70001, 0), (20000, 2), (8192, 1)])
 def test_softmax_extreme_and_special_rows(ctx, cols, variant):
     f = np.float32
@@ -1261,7 +1261,7 @@ def test_softmax_extreme_and_special_rows(ctx, cols, variant):
     assert y[5, 3] == 1.0 and y[5].sum() == 1.0
 
 
-@pytest.mark.parametrize("cols,variant", [(1000, 0), (4096, 0), (8192, 0), (8192, 5), (4095, 0),
+@pytest.mark.parametrize("cols,variant", [(1000, 0), (4096, 0), (8192, 0), (8192, 5), (8192, 11), (4095, 0),
                                           (20001, 0), (40000, 0), (66000, 0)])
 def test_softmax_rows_of_huge_magnitude(ctx, cols, variant):
     # a row's maximum may be far from 0: only differences matter
@@ -1590,7 +1590,8 @@ def test_gemm_all_variants_and_padded_output(ctx):
     want = cf.np_gemm_bf16(ab, bb, np.float32)
     sigma = 0.02 * 0.02 * 16
     bits0 = None
-    for v in list(range(0, 17)) + [23, 24, 25, 27]:   # 17..22 and 26 are measurement probes whose output is not the product
+    # (17..22, 26, 28 and 29 are measurement builds whose output is not the product; 30..32 exist with them only)
+    for v in list(range(0, 17)) + [23, 24, 25, 27] + ([30, 31, 32] if rt.probes_built() else []):
         rt.set_variant("gemm", v)
         bits = run_gemm(ab, bb, ldc_pad=8)
         got = cf.bf16_bits_to_f32(bits)
@@ -1598,7 +1599,7 @@ def test_gemm_all_variants_and_padded_output(ctx):
         assert_allclose(got, want, rtol=GEMM_RTOL, atol=1e-2 * sigma)
         if v == 0:
             bits0 = bits
-        if v in (7, 14, 15, 16, 23, 24, 25, 27):   # the same sums with other epilogues / priorities / load paths
+        if v in (7, 14, 15, 16, 23, 24, 25, 27, 30, 31, 32):   # the same sums with other epilogues / priorities / load paths / orders
             assert_array_equal(bits, bits0)
 
 
