@@ -10,11 +10,66 @@ from __future__ import annotations
 
 import numpy as np
 
-# Shapes, seeded inputs and the bf16 bit-pattern helpers are shared with the
-# benchmark and live in the package; re-exported here for the tests.
-from hc_amd.workloads import (C1_N, C2_SHAPE, C3_SHAPE, C4_SHAPE, C5_MNK,  # noqa: F401
-                              bf16_bits_to_f32, f32_to_bf16_bits, inputs_c1,
-                              inputs_c2, inputs_c3, inputs_c4, inputs_c5)
+# Shapes, seeded inputs and bf16 bit patterns are stated here on their own: the
+# package under test has the same figures in hc_amd/workloads.py for its
+# benchmark, and tests/test_oracle_closed_forms.py holds the two against each
+# other, so that a slip in either shows up instead of being shared.
+C1_N = 16_777_259
+C2_SHAPE = (8191, 8193)
+C3_SHAPE = (4096, 8192)
+C4_SHAPE = (16384, 4096)
+C5_MNK = (4096, 4096, 4096)
+
+
+def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """fp32 -> bf16 bit patterns, round to nearest, ties to even; NaN stays a
+    quiet NaN.  Written as a comparison of the discarded half word with one half
+    unit in the last place, not as the carry trick the package uses."""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    keep, rest = u >> 16, u & 0xFFFF
+    up = (rest > 0x8000) | ((rest == 0x8000) & ((keep & 1) == 1))
+    out = keep + up                       # a carry out of the mantissa is the next exponent (or inf)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    return np.where(nan, keep | 0x40, out).astype(np.uint16)
+
+
+def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    wide = np.zeros(np.shape(b) + (2,), np.uint16)
+    wide[..., 1 if np.little_endian else 0] = b
+    return wide.view(np.float32)[..., 0]
+
+
+def inputs_c1(n: int = C1_N, seed: int = 1):
+    rng = np.random.default_rng(seed)
+    a = rng.uniform(-1.0, 1.0, n).astype(np.float32)
+    b = rng.uniform(-1.0, 1.0, n).astype(np.float32)
+    return a, b
+
+
+def inputs_c2(shape=C2_SHAPE, seed: int = 2):
+    rng = np.random.default_rng(seed)
+    return tuple(rng.standard_normal(shape, dtype=np.float32).astype(np.float16) for _ in range(3))
+
+
+def inputs_c3(shape=C3_SHAPE, seed: int = 3):
+    rng = np.random.default_rng(seed)
+    return (np.float32(3.0) * rng.standard_normal(shape, dtype=np.float32),)
+
+
+def inputs_c4(shape=C4_SHAPE, seed: int = 4):
+    rng = np.random.default_rng(seed)
+    n = rng.standard_normal(shape, dtype=np.float32)
+    outlier = rng.random(shape, dtype=np.float32) < np.float32(0.01)
+    return ((n * np.where(outlier, np.float32(50.0), np.float32(1.0))).astype(np.float16),)
+
+
+def inputs_c5(mnk=C5_MNK, seed: int = 5):
+    """A[M,K] and Bt[N,K] as bf16 bit patterns (B is column-major)."""
+    m, n, k = mnk
+    rng = np.random.default_rng(seed)
+    a = np.float32(0.02) * rng.standard_normal((m, k), dtype=np.float32)
+    bt = np.float32(0.02) * rng.standard_normal((n, k), dtype=np.float32)
+    return f32_to_bf16_bits(a), f32_to_bf16_bits(bt)
 
 
 # ---------------------------------------------------------------------------

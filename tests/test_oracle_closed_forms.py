@@ -73,6 +73,30 @@ def test_bf16_rounding_two_statements_and_ties():
         assert np.isnan(cf.bf16_bits_to_f32(b[2:3]))[0]
 
 
+def test_the_benchmark_builds_the_inputs_the_oracle_describes():
+    """The package keeps its own statement of the shapes, the seeded inputs and
+    the bf16 bit patterns for its benchmark (hc_amd/workloads.py); the oracle's
+    are written independently.  Same figures, same bytes."""
+    from hc_amd import workloads as W
+    assert (W.C1_N, W.C2_SHAPE, W.C3_SHAPE, W.C4_SHAPE, W.C5_MNK) == \
+        (cf.C1_N, cf.C2_SHAPE, cf.C3_SHAPE, cf.C4_SHAPE, cf.C5_MNK)
+    for ours, theirs in ((cf.inputs_c1(1001), W.inputs_c1(1001)), (cf.inputs_c2((37, 41)), W.inputs_c2((37, 41))),
+                         (cf.inputs_c3((9, 64)), W.inputs_c3((9, 64))), (cf.inputs_c4((33, 128)), W.inputs_c4((33, 128))),
+                         (cf.inputs_c5((64, 32, 128)), W.inputs_c5((64, 32, 128)))):
+        assert len(ours) == len(theirs)
+        for a, b in zip(ours, theirs):
+            assert a.dtype == b.dtype and a.shape == b.shape
+            assert_array_equal(a.view(np.uint8), b.view(np.uint8))
+    # every fp32 whose upper half word is one of 4096 and whose lower one is any of 65536
+    hi = np.random.default_rng(2).integers(0, 1 << 16, 4096).astype(np.uint32)
+    hi[:8] = (0x7F7F, 0xFF7F, 0x7F80, 0xFF80, 0x7FC0, 0x0000, 0x8000, 0x007F)
+    x = ((hi[:, None] << 16) | np.arange(1 << 16, dtype=np.uint32)[None, :]).view(np.float32)
+    assert_array_equal(cf.f32_to_bf16_bits(x), W.f32_to_bf16_bits(x))
+    bits = np.arange(1 << 16, dtype=np.uint16)
+    assert_array_equal(cf.bf16_bits_to_f32(bits).view(np.uint32), W.bf16_bits_to_f32(bits).view(np.uint32))
+    assert_array_equal(cf.bf16_bits_to_f32(bits).view(np.uint32), bits.astype(np.uint32) << 16)
+
+
 # ---------------------------------------------------------------------------
 # W1 / W2
 # ---------------------------------------------------------------------------
