@@ -1302,11 +1302,21 @@ def match_fmap(dst_view, value, n_groups):
     return make
 
 
+class _Table:
+    """The index table of a load that the binder derived itself: [elements,
+    ndim] indices inside the window (compared by identity)."""
+
+    def __init__(self, array):
+        self.array = array
+
+
 def _element_tables(func, shape, ndim, name):
     """An index mapping evaluated on a whole tile: [elements, ndim] int64, the
     index inside the window of every tile element in row-major order (None:
     the identity of an unmapped load or store)."""
     import numpy as np
+    if isinstance(func, _Table):
+        return func.array
     grids = np.indices(shape, dtype=np.int64)
     if func is None:
         if ndim != len(shape):
@@ -1415,6 +1425,136 @@ def match_gather_map(dst_view, value, n_groups, out_func=None, force=False):
         return [rt.plan_gather_map(g, program, arrays[:-1], arrays[-1], types, out_type, store_all, copy_bytes)]
     make.program = program
     return make
+
+
+def _gathered_form(value):
+    """`value` rewritten so that every leaf is a load of value's own shape
+    through an index table, with the shape-changing nodes between the loads and
+    the result (broadcasts of smaller tiles, transposes, slices, reshapes)
+    folded into the tables; None if value is not such an expression."""
+    import numpy as np
+    root = tuple(value.shape)
+    elems = math.prod(root)
+    memo = {}
+
+    def rebuild(t, args):
+        return Tile(t.op, tuple(args), root, t.dtype_name, **t.attrs)
+
+    def go(t, coords):
+        # coords[d][e]: along dimension d of t, the element of t that element e of the result reads
+        key = (t.uid, coords.tobytes())
+        if key in memo:
+            return memo[key]
+        out = None
+        if _is(t, "const"):
+            out = t
+        elif _is(t, "full"):
+            out = Tile("full", t.args, root, t.dtype_name, **t.attrs)
+        elif _is(t, "load") or _is(t, "mapped_load"):
+            view = t.attrs["view"]
+            if _is(t, "load"):
+                mapped = tuple(coords)
+            else:
+                func = t.attrs["mapping"]
+                if isinstance(func, _Table):
+                    flat = np.ravel_multi_index(tuple(coords), t.shape)
+                    mapped = tuple(func.array[flat, d] for d in range(func.array.shape[1]))
+                else:
+                    mapped = tuple(_element_tables(func, t.shape, view.base.ndim, view.base.name).T)
+                    flat = np.ravel_multi_index(tuple(coords), t.shape)
+                    mapped = tuple(m[flat] for m in mapped)
+            table = np.stack([np.asarray(m, np.int64).reshape(elems) for m in mapped], axis=1)
+            out = Tile("mapped_load", (), root, t.dtype_name, view=view, mapping=_Table(table))
+        elif _is(t, "transpose", 1):
+            out = go(t.args[0], coords[::-1])
+        elif _is(t, "reshape", 1):
+            flat = np.ravel_multi_index(tuple(coords), t.shape)
+            out = go(t.args[0], np.stack(np.unravel_index(flat, t.args[0].shape)))
+        elif _is(t, "slice", 1):
+            src = t.args[0]
+            child, at, dim = [], 0, 0
+            for k in t.attrs["key"]:
+                if k == "new":
+                    at += 1                            # a new axis of t: no axis of the source
+                elif isinstance(k, tuple):
+                    start, _, step = slice(*k).indices(src.shape[dim])
+                    child.append(start + step * coords[at])
+                    at += 1
+                    dim += 1
+                else:
+                    child.append(np.full(elems, k % src.shape[dim], np.int64))
+                    dim += 1
+            out = go(src, np.stack(child)) if len(child) == len(src.shape) else None
+        elif t.op in _REDUCTIONS or t.op in ("dot", "norm", "window", "update"):
+            out = None
+        elif len(t.args) in (1, 2) and all(isinstance(a, Tile) for a in t.args):
+            args = []
+            for a in t.args:
+                if a.shape == ():
+                    args.append(go(a, np.zeros((0, elems), np.int64)) if not _const(a) else a)
+                    continue
+                lead = len(t.shape) - len(a.shape)
+                if lead < 0:
+                    return None
+                sub = [coords[lead + d] if a.shape[d] == t.shape[lead + d] else np.zeros(elems, np.int64)
+                       for d in range(len(a.shape))]
+                args.append(go(a, np.stack(sub)))
+            out = None if any(a is None for a in args) else rebuild(t, args)
+        memo[key] = out
+        return out
+
+    return go(value, np.indices(root, dtype=np.int64).reshape(len(root), elems))
+
+
+def _strip_views(t: Tile) -> Tile:
+    while (_is(t, "transpose", 1) or _is(t, "slice", 1) or _is(t, "reshape", 1)) and isinstance(t.args[0], Tile):
+        t = t.args[0]
+    return t
+
+
+def match_general_windows(dst_view, value, n_groups):
+    """The last resort for an elementwise expression whose loads do not walk
+    the store's window the way the tiled kernels need: windows shifted by a
+    constant (stencils), smaller tiles broadcast over larger ones (a row or a
+    column vector next to a 2-D tile), transposed, sliced or reshaped tiles.
+    Every load becomes a gathered operand of hcamdGatherMap with the index
+    table the expression implies (python/hckernel/kernel_api.py:297-342: the
+    same bounds test per element)."""
+    import numpy as np
+    if len(value.shape) not in (1, 2, 3) or len(value.shape) != dst_view.base.ndim:
+        return None
+    out_dt = dst_view.base.dtype_name
+    copy = _is(_strip_views(value), "load") and value.dtype_name == out_dt
+    if not copy and (out_dt not in _MAP_FLOATS + ("bool",) or
+                     any(_is(t, "load") and t.dtype_name not in _MAP_FLOATS for t in _walk(value))):
+        return None                              # (copies move any element type)
+    lowered = _gathered_form(value)
+    if lowered is None:
+        return None
+    if value.attrs.get("plain") or lowered.attrs.get("plain"):
+        # A bare numpy.ma array is stored in full: where a load was outside its
+        # buffer the reference writes the value it initialises tiles with.
+        total = math.prod(n_groups)
+        elems = math.prod(value.shape)
+        if total * elems > _GATHER_MAP_MAX_DESTS:
+            raise NoNativeKernel(f"{dst_view.base.name}: too many elements to check that the stored array "
+                                 "has no element that was loaded from outside its buffer")
+        d_starts = _group_starts(dst_view, n_groups)
+        d_index = np.indices(value.shape, dtype=np.int64).reshape(len(value.shape), elems).T
+        d_shape = np.asarray(dst_view.base.shape, np.int64)
+        stored = ((d_starts[:, None, :] + d_index[None, :, :]) < d_shape).all(axis=2)
+        for t in _walk(lowered):
+            if _is(t, "mapped_load"):
+                view = t.attrs["view"]
+                idx = _group_starts(view, n_groups)[:, None, :] + t.attrs["mapping"].array[None, :, :]
+                inside = ((t.attrs["mapping"].array[None, :, :] >= 0) &
+                          (idx < np.asarray(view.base.shape, np.int64))).all(axis=2)
+                if (stored & ~inside).any():
+                    raise NoNativeKernel(
+                        f"{dst_view.base.name}: the stored value is a bare array (a NumPy function or "
+                        f"attribute of a tile), written in full, and some of its elements were loaded from "
+                        f"outside {view.base.name}; the reference writes its fill value there")
+    return match_gather_map(dst_view, lowered, n_groups, force=True)
 
 
 class _RowCompiler(_MapCompiler):
@@ -2645,14 +2785,27 @@ def bind(stores, n_groups, atomics=(), mapped_stores=(), id_stores=(), group_sha
         if q is not None:
             return makers + [q]
         for view, value in stores:
-            for matcher in (match_fill, match_copy, match_imap, match_add, match_fma, match_softmax, match_gemm,
-                            match_gather_gemm, match_gather_map, match_pairwise, match_cols,
-                            match_cols_tile, match_rows, match_map, match_fmap):
-                mk = matcher(view, value, n_groups)
-                if mk is not None:
-                    makers.append(mk)
-                    break
-            else:
+            try:
+                for matcher in (match_fill, match_copy, match_imap, match_add, match_fma, match_softmax,
+                                match_gemm, match_gather_gemm, match_gather_map, match_pairwise, match_cols,
+                                match_cols_tile, match_rows, match_map, match_fmap, match_general_windows):
+                    mk = matcher(view, value, n_groups)
+                    if mk is not None:
+                        makers.append(mk)
+                        break
+                else:
+                    mk = None
+            except NoNativeKernel as refusal:
+                # a kernel that walks one window refused the shape of the accesses
+                # (shifted, broadcast or transposed tiles): the gathered form may take it
+                try:
+                    mk = match_general_windows(view, value, n_groups)
+                except NoNativeKernel:
+                    raise refusal from None
+                if mk is None:
+                    raise
+                makers.append(mk)
+            if mk is None:
                 raise NoNativeKernel(
                     f"no hand-written kernel matches the value stored to {view.base.name} "
                     f"({value!r}); bound patterns: copy, a+b (fp32), a*b+c (fp16 storage, fp32 "

@@ -939,7 +939,9 @@ class Tile:
     def T(self):
         if len(self.shape) != 2:
             raise TraceError(".T needs a 2-D tile")
-        return Tile("transpose", (self,), self.shape[::-1], self.dtype_name)
+        # (an attribute the reference's wrapper forwards to numpy.ma,
+        # python/hckernel/kernel_api.py:150-151: the result is a bare array)
+        return Tile("transpose", (self,), self.shape[::-1], self.dtype_name, plain=True)
 
     @property
     def dtype(self):

@@ -1186,6 +1186,85 @@ def test_mapped_loads_and_stores_outside_a_product_match_the_simulator(rows, col
             assert (want == 7).any(), name               # something is left alone
 
 
+def _window_bodies(deco):
+    """Elementwise bodies whose loads do not walk the store's window: a window
+    shifted by a constant, a row vector and a column vector next to a 2-D tile,
+    a transposed tile, a slice of a wider tile, a reshaped one."""
+    M, N = sym.M, sym.N
+
+    @deco(work_shape=N, group_shape=64)
+    def stencil(gr: CurrentGroup, x: Buffer[N, DT], out: Buffer[N, DT]):
+        o = gr.work_offset[0]
+        left, mid, right = (gr.load(x[o + k:], shape=gr.shape) for k in (0, 1, 2))
+        gr.store(out[o:], (left + right) * x.dtype.type(0.5) - mid)
+
+    @deco(work_shape=(M, N), group_shape=(8, 32))
+    def bias_and_scale(gr: CurrentGroup, x: Buffer[M, N, DT], b: Buffer[N, DT], s: Buffer[M, DT],
+                       out: Buffer[M, N, DT]):
+        i, j = gr.work_offset
+        t = gr.load(x[i:, j:], shape=gr.shape)
+        row = gr.load(b[j:], shape=gr.shape[1])
+        col = gr.load(s[i:], shape=gr.shape[0])
+        gr.store(out[i:, j:], (t + row) * col[:, None] / row[None, :])
+
+    @deco(work_shape=(M, N), group_shape=(8, 32))
+    def transposed(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[N, M, DT]):
+        i, j = gr.work_offset
+        gr.store(out[j:, i:], gr.load(x[i:, j:], shape=gr.shape).T)
+
+    @deco(work_shape=(M, N), group_shape=(8, 32))
+    def symmetric_part(gr: CurrentGroup, x: Buffer[M, N, DT], y: Buffer[N, M, DT], out: Buffer[M, N, DT]):
+        i, j = gr.work_offset
+        a = gr.load(x[i:, j:], shape=gr.shape)
+        bt = gr.load(y[j:, i:], shape=gr.shape[::-1])
+        gr.store(out[i:, j:], a * x.dtype.type(0.5) + bt.T * x.dtype.type(0.5))
+
+    @deco(work_shape=(M, N), group_shape=(8, 32))
+    def sliced(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[M, N, DT]):
+        i, j = gr.work_offset
+        wide = gr.load(x[i:, j:], shape=(gr.shape[0] + 1, gr.shape[1] + 1))
+        gr.store(out[i:, j:], wide[1:, 1:] - wide[:-1, :-1])
+
+    @deco(work_shape=(M, N), group_shape=(8, 32))
+    def reshaped(gr: CurrentGroup, x: Buffer[M, N, DT], flat: Buffer[sym.L, DT], out: Buffer[M, N, DT]):
+        i, j = gr.work_offset
+        v = gr.load(flat[:], shape=(8 * 32,))
+        gr.store(out[i:, j:], gr.load(x[i:, j:], shape=gr.shape) + v.reshape(8, 32))
+
+    return {"stencil": stencil, "bias_and_scale": bias_and_scale, "transposed": transposed,
+            "symmetric_part": symmetric_part, "sliced": sliced, "reshaped": reshaped}
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("rows,cols", [(16, 64), (37, 50), (5, 131)])
+def test_loads_that_do_not_walk_the_window_of_the_store_match_the_simulator(rows, cols, dtype):
+    """Shifted, broadcast, transposed, sliced and reshaped tiles in elementwise
+    bodies go to the gathered map with index tables the binder derives; the
+    same bytes as the simulator writes, elements it leaves alone included
+    (loads past the end of an array, zero divisors)."""
+    gpu, sim = _window_bodies(kernel), _window_bodies(sim_kernel)
+    rng = np.random.default_rng(rows * cols)
+    x = rng.integers(-6, 7, (rows, cols)).astype(dtype)
+    y = rng.integers(-6, 7, (cols, rows)).astype(dtype)
+    b = rng.integers(-2, 3, cols).astype(dtype)          # zeros: deactivated quotients
+    sc = rng.integers(-3, 4, rows).astype(dtype)
+    flat = rng.integers(-6, 7, 8 * 32 - 3).astype(dtype)  # shorter than the tile it is reshaped into
+    cases = {"stencil": ([x.reshape(-1)], (rows * cols,)), "bias_and_scale": ([x, b, sc], (rows, cols)),
+             "transposed": ([x], (cols, rows)), "symmetric_part": ([x, y], (rows, cols)),
+             "sliced": ([x], (rows, cols)), "reshaped": ([x, flat], (rows, cols))}
+    bits = {2: np.uint16, 4: np.uint32}[np.dtype(dtype).itemsize]
+    for name, (ins, shape) in cases.items():
+        want = np.full(shape, 7, dtype)
+        with np.errstate(all="ignore"):
+            sim[name](*ins, want)
+        out = rt.to_device(np.full(shape, 7, dtype))
+        gpu[name](*[rt.to_device(v) for v in ins], out)
+        assert rt.last_kernel_name() == "hcamd_gather_fmap", name
+        assert_array_equal(out.to_host().view(bits), want.view(bits), err_msg=name)
+        if name in ("stencil", "bias_and_scale", "sliced", "reshaped"):
+            assert (want == 7).any(), name                 # something is left alone
+
+
 def test_tile_mask_is_stored_as_a_plain_bool_array():
     """`tile.mask` (python/hckernel/kernel_api.py:117-119: True = active) of
     float and int32 expressions that the data deactivates here and there: the

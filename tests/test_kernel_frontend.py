@@ -391,13 +391,13 @@ def test_symbol_conflicts_and_rank_errors_are_reported():
                                                                FakeDev((3, 4), "int32"))
 
 
-def test_bodies_without_a_native_kernel_fail_loudly(ctx):
+def test_bodies_without_a_native_kernel_fail_loudly(ctx, monkeypatch):
     N = sym.N
 
     @kernel(work_shape=N, group_shape=64)
     def shifted(gr: CurrentGroup, a: Buffer[N, DT], c: Buffer[N, DT]):
         o = gr.work_offset[0]
-        gr.store(c[o:], gr.load(a[o + 1:], shape=gr.shape[0]))       # not a disjoint tiling
+        gr.store(c[o:], gr.load(a[o + 1:], shape=gr.shape[0]))       # not a disjoint tiling: a gathered copy
 
     @kernel(work_shape=N, group_shape=64)
     def scaled(gr: CurrentGroup, a: Buffer[N, DT], c: Buffer[N, DT]):
@@ -416,9 +416,13 @@ def test_bodies_without_a_native_kernel_fail_loudly(ctx):
         inner()
 
     a, c = FakeDev((1000,), "float32"), FakeDev((1000,), "float32")
-    for k in (shifted, scaled, nothing, scoped):
+    for k in (scaled, nothing, scoped):
         with pytest.raises(NoNativeKernel):
             k.plan(a, c, ctx=ctx)
+    monkeypatch.setattr(rt, "GatherMap", MapTablesOnly)
+    (p,) = shifted.plan(a, c, ctx=ctx)
+    assert p.fn is rt.hcamdGatherMapLaunch and p.args[-1] == 4          # copy mode, 4-byte elements
+    assert MapTablesOnly.last.operands[0][2][:2, 0].tolist() == [1, 65]
 
 
 def test_decorator_argument_checks():
@@ -799,6 +803,120 @@ def test_mapped_loads_and_stores_outside_a_product_bind_to_the_gathered_map(ctx,
         plan(body(load_func=lambda i, j: (i, j, 0)))
     with pytest.raises(NoNativeKernel, match="cannot be evaluated"):
         plan(body(load_func=lambda i, j: (i, j if j < 3 else 0)))
+
+
+def run_gathered_plan(p, tables, host_of, out):
+    """A gathered-map plan in NumPy: operands gathered by the host tables
+    (host_of: device address -> host array), the program on (value, active)
+    pairs (the operations these tests use), active elements inside the
+    destination stored."""
+    names = {v: k for k, v in rt.FMAP_OPS.items()}
+    prog = [(names[p.args[2][i].op], p.args[2][i].arg, p.args[2][i].imm) for i in range(p.args[3])]
+    arrays = [host_of[p.args[4][i]] for i in range(len(tables.operands) - 1)]
+    for g in range(tables.n_groups):
+        stack = []
+        for op, arg, imm in prog:
+            if op == "in":
+                v, ok, _ = tables.gather(arg, arrays[arg], g)
+                stack.append((v.astype(np.float32), ok))
+            elif op == "const":
+                stack.append((np.full(tables.tile_elems, imm, np.float32), np.ones(tables.tile_elems, bool)))
+            else:
+                (b, bok), (a, aok) = stack.pop(), stack.pop()
+                with np.errstate(all="ignore"):
+                    v = {"add": a + b, "sub": a - b, "mul": a * b, "div": a / b}[op]
+                ok = aok & bok
+                if op == "div":
+                    ok &= (b != 0) & np.isfinite(v)
+                stack.append((v.astype(np.float32), ok))
+        (v, ok), = stack
+        _, inside, dst = tables.gather(len(arrays), out, g)
+        keep = ok & inside
+        out[tuple(dst[keep, d] for d in range(out.ndim))] = v[keep]
+
+
+def test_loads_that_do_not_walk_the_window_of_the_store_become_gathered_operands(ctx, monkeypatch):
+    """Windows shifted by a constant, row and column vectors broadcast over a
+    2-D tile, transposed, sliced and reshaped tiles: no kernel that walks one
+    window takes them; the binder derives an index table per load and hands the
+    expression to the gathered map.  The tables, run in NumPy, give what the
+    simulator gives."""
+    from oracle.hcsim import kernel as sim_kernel
+    monkeypatch.setattr(rt, "GatherMap", MapTablesOnly)
+    M, N = sym.M, sym.N
+    f = np.float32
+
+    def bodies(deco):
+        @deco(work_shape=N, group_shape=16)
+        def shifted(gr: CurrentGroup, x: Buffer[N, DT], out: Buffer[N, DT]):
+            o = gr.work_offset[0]
+            gr.store(out[o:], gr.load(x[o + 1:], shape=gr.shape) - gr.load(x[o:], shape=gr.shape))
+
+        @deco(work_shape=(M, N), group_shape=(4, 8))
+        def broadcast(gr: CurrentGroup, x: Buffer[M, N, DT], b: Buffer[N, DT], s: Buffer[M, DT], out: Buffer[M, N, DT]):
+            i, j = gr.work_offset
+            t = gr.load(x[i:, j:], shape=gr.shape)
+            gr.store(out[i:, j:], (t + gr.load(b[j:], shape=gr.shape[1])) / gr.load(s[i:], shape=gr.shape[0])[:, None])
+
+        @deco(work_shape=(M, N), group_shape=(4, 8))
+        def transposed(gr: CurrentGroup, x: Buffer[M, N, DT], y: Buffer[N, M, DT], out: Buffer[N, M, DT]):
+            i, j = gr.work_offset
+            t = gr.load(x[i:, j:], shape=gr.shape)
+            gr.store(out[j:, i:], gr.load(y[j:, i:], shape=gr.shape[::-1]) * t.T)
+
+        @deco(work_shape=(M, N), group_shape=(4, 8))
+        def sliced(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[M, N, DT]):
+            i, j = gr.work_offset
+            wide = gr.load(x[i:, j:], shape=(5, 9))
+            gr.store(out[i:, j:], wide[1:, 1:] - wide[:-1, :-1].reshape(32).reshape(4, 8))
+        return {"shifted": shifted, "broadcast": broadcast, "transposed": transposed, "sliced": sliced}
+
+    rng = np.random.default_rng(5)
+    rows, cols = 11, 21
+    x = rng.integers(-5, 6, (rows, cols)).astype(f)
+    y = rng.integers(-5, 6, (cols, rows)).astype(f)
+    b = rng.integers(-5, 6, cols).astype(f)
+    sc = rng.integers(-1, 2, rows).astype(f)                 # zeros: rows whose quotients are deactivated
+    cases = {"shifted": ([x.reshape(-1)], (rows * cols,)), "broadcast": ([x, b, sc], (rows, cols)),
+             "transposed": ([x, y], (cols, rows)), "sliced": ([x], (rows, cols))}
+    gpu, sim = bodies(kernel), bodies(sim_kernel)
+    for name, (ins, shape) in cases.items():
+        want = np.full(shape, 77, f)
+        with np.errstate(all="ignore"):
+            sim[name](*ins, want)
+        fake = [FakeDev(v.shape, "float32") for v in ins]
+        (p,) = gpu[name].plan(*fake, FakeDev(shape, "float32"), ctx=ctx)
+        assert p.fn is rt.hcamdGatherMapLaunch, name
+        got = np.full(shape, 77, f)
+        run_gathered_plan(p, MapTablesOnly.last, {d.ptr: v for d, v in zip(fake, ins)}, got)
+        np.testing.assert_array_equal(got, want, err_msg=name)
+        assert (want == 77).any() or name == "transposed", name
+    # the shifted window is a window start, the broadcast vector a table that ignores a dimension
+    (p,) = gpu["shifted"].plan(FakeDev((200,), "float32"), FakeDev((200,), "float32"), ctx=ctx)
+    t = MapTablesOnly.last
+    assert t.operands[0][2][:3, 0].tolist() == [1, 17, 33] and t.operands[1][2][:3, 0].tolist() == [0, 16, 32]
+    (p,) = gpu["broadcast"].plan(FakeDev((12, 21), "float32"), FakeDev((21,), "float32"), FakeDev((12,), "float32"),
+                                 FakeDev((12, 21), "float32"), ctx=ctx)
+    t = MapTablesOnly.last
+    assert t.operands[1][3][:, 0].tolist() == list(range(8)) * 4         # the row vector: the column index
+    assert t.operands[2][3][:, 0].tolist() == [r for r in range(4) for _ in range(8)]
+    # a bare array (a transposed tile is one) is stored in full: refused where that would write what the
+    # reference initialises tiles with
+    T2 = sym.T2
+
+    @kernel(work_shape=(M, N), group_shape=(4, 8))
+    def wider(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[T2, T2, DT]):
+        i, j = gr.work_offset
+        gr.store(out[j:, i:], gr.load(x[i:, j:], shape=gr.shape).T)
+    with pytest.raises(NoNativeKernel, match="written in full"):
+        wider.plan(FakeDev((11, 21), "float32"), FakeDev((24, 24), "float32"), ctx=ctx)
+    # other element types: copies only
+    @kernel(work_shape=(M, N), group_shape=(4, 8))
+    def int_transpose(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[N, M, DT]):
+        i, j = gr.work_offset
+        gr.store(out[j:, i:], gr.load(x[i:, j:], shape=gr.shape).T)
+    (p,) = int_transpose.plan(FakeDev((11, 21), "int32"), FakeDev((21, 11), "int32"), ctx=ctx)
+    assert p.fn is rt.hcamdGatherMapLaunch and p.args[-1] == 4 and p.args[3] == 0      # a copy of 4-byte elements
 
 
 def test_offsets_with_division_are_for_mapped_accesses_only(ctx):
