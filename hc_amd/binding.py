@@ -184,6 +184,35 @@ def match_copy(dst_view, value, n_groups):
     return make
 
 
+def match_transpose(dst_view, value, n_groups):
+    """store(out[j:, i:], load(x[i:, j:], shape).T): a tile's `.T` written to the
+    transposed window.  The tiles of all groups add up to one transposed copy
+    of the window, whatever the group shape.  `.T` of a tile is a bare numpy.ma
+    array in the reference (python/hckernel/kernel_api.py:150-151) and is stored
+    in full, so the window must not reach past what was loaded."""
+    if not (_is(value, "transpose", 1) and _is(value.args[0], "load") and len(value.shape) == 2):
+        return None
+    load = value.args[0]
+    src = load.attrs["view"]
+    if src.base.dtype_name != dst_view.base.dtype_name or \
+            getattr(src.base.dtype, "itemsize", 2) not in (1, 2, 4, 8):
+        return None
+    ws = window_of(src, load.shape, n_groups)
+    wd = window_of(dst_view, value.shape, n_groups)
+    if wd.driver != ws.driver[::-1]:
+        raise NoNativeKernel("the transposed tile is stored to a window that is not the loaded one transposed")
+    if wd.extent[0] > ws.extent[1] or wd.extent[1] > ws.extent[0]:
+        raise NoNativeKernel(
+            f"{dst_view.base.name}: the transposed tile is a bare array, written in full, and its window reaches "
+            f"past what was loaded from {src.base.name}; the reference writes its fill value there")
+    rows, cols = wd.extent[1], wd.extent[0]          # of the source window
+
+    def make(mem, ctx):
+        return [rt.plan_transpose2d(_Arr(_sub(mem[ws.buffer], (rows, cols)), ctx),
+                                    _Arr(_sub(mem[wd.buffer], (cols, rows)), ctx))]
+    return make
+
+
 def match_add(dst_view, value, n_groups):
     value = _strip_cast(value, dst_view.base.dtype_name)
     if not (_is(value, "add", 2) and all(_is(a, "load") for a in value.args)):
@@ -1401,16 +1430,25 @@ def match_gather_map(dst_view, value, n_groups, out_func=None, force=False):
     # two active elements of the output must not land on one address: the
     # reference stores them one after the other, a launch in no order
     o_shape, o_strides, o_starts, o_index = operands[-1]
-    if total * o_index.shape[0] > _GATHER_MAP_MAX_DESTS:
-        raise NoNativeKernel(f"{dst_view.base.name}: {total} groups of {o_index.shape[0]} elements are "
-                             "too many to check that no two of them are stored to one place")
-    idx = o_starts[:, None, :] + o_index[None, :, :]
-    inside = ((o_index[None, :, :] >= 0) & (idx < np.asarray(o_shape, np.int64))).all(axis=2)
-    dest = (idx * np.asarray(o_strides, np.int64)).sum(axis=2)[inside]
-    if len(np.unique(dest)) != dest.size:
-        raise NoNativeKernel(f"{dst_view.base.name}: two tile elements (of one group or of two) are "
-                             "stored to one place; their order is the reference's group order, which "
-                             "a launch does not keep")
+    disjoint = False
+    if out_func is None:
+        # an unmapped store whose windows tile the destination: every element has a place of its own
+        try:
+            window_of(dst_view, shape, n_groups)
+            disjoint = True
+        except NoNativeKernel:
+            pass
+    if not disjoint:
+        if total * o_index.shape[0] > _GATHER_MAP_MAX_DESTS:
+            raise NoNativeKernel(f"{dst_view.base.name}: {total} groups of {o_index.shape[0]} elements are "
+                                 "too many to check that no two of them are stored to one place")
+        idx = o_starts[:, None, :] + o_index[None, :, :]
+        inside = ((o_index[None, :, :] >= 0) & (idx < np.asarray(o_shape, np.int64))).all(axis=2)
+        dest = (idx * np.asarray(o_strides, np.int64)).sum(axis=2)[inside]
+        if len(np.unique(dest)) != dest.size:
+            raise NoNativeKernel(f"{dst_view.base.name}: two tile elements (of one group or of two) are "
+                                 "stored to one place; their order is the reference's group order, which "
+                                 "a launch does not keep")
     indices = [t.attrs["view"].base.index for t in loads] + [dst_view.base.index]
     types = [rt.F16 if t.dtype_name == "float16" else rt.F32 for t in loads]
     out_type = {"float32": rt.F32, "float16": rt.F16, "bool": rt.U8}.get(out_dt, rt.F32)
@@ -1536,19 +1574,22 @@ def match_general_windows(dst_view, value, n_groups):
         # buffer the reference writes the value it initialises tiles with.
         total = math.prod(n_groups)
         elems = math.prod(value.shape)
-        if total * elems > _GATHER_MAP_MAX_DESTS:
+        if total * elems > 16 * _GATHER_MAP_MAX_DESTS:
             raise NoNativeKernel(f"{dst_view.base.name}: too many elements to check that the stored array "
                                  "has no element that was loaded from outside its buffer")
         d_starts = _group_starts(dst_view, n_groups)
         d_index = np.indices(value.shape, dtype=np.int64).reshape(len(value.shape), elems).T
         d_shape = np.asarray(dst_view.base.shape, np.int64)
-        stored = ((d_starts[:, None, :] + d_index[None, :, :]) < d_shape).all(axis=2)
-        for t in _walk(lowered):
-            if _is(t, "mapped_load"):
-                view = t.attrs["view"]
-                idx = _group_starts(view, n_groups)[:, None, :] + t.attrs["mapping"].array[None, :, :]
-                inside = ((t.attrs["mapping"].array[None, :, :] >= 0) &
-                          (idx < np.asarray(view.base.shape, np.int64))).all(axis=2)
+        loads = [t for t in _walk(lowered) if _is(t, "mapped_load")]
+        starts = [_group_starts(t.attrs["view"], n_groups) for t in loads]
+        step = max(1, (1 << 21) // elems)               # groups at a time: a few tens of MB of indices
+        for g0 in range(0, total, step):
+            g1 = min(total, g0 + step)
+            stored = ((d_starts[g0:g1, None, :] + d_index[None, :, :]) < d_shape).all(axis=2)
+            for t, st in zip(loads, starts):
+                view, table = t.attrs["view"], t.attrs["mapping"].array
+                idx = st[g0:g1, None, :] + table[None, :, :]
+                inside = ((table[None, :, :] >= 0) & (idx < np.asarray(view.base.shape, np.int64))).all(axis=2)
                 if (stored & ~inside).any():
                     raise NoNativeKernel(
                         f"{dst_view.base.name}: the stored value is a bare array (a NumPy function or "
@@ -1887,7 +1928,12 @@ def match_rows(dst_view, value, n_groups):
                 return r
         return None
 
-    if not has_row_reduce(value, set()):
+    # Without a reduction the same stages serve a 2-D tile next to a row vector
+    # or a per-row operand (a bias, a per-row scale): nothing then ties a tile to
+    # whole rows, and the groups may cut the columns too.
+    broadcast_only = not has_row_reduce(value, set())
+    if broadcast_only and not (len(value.shape) == 2 and
+                               any(_is(t, "load") and len(t.shape) == 1 for t in _walk(value))):
         return None
     x = first_tile(value)
     if x is None:
@@ -1947,18 +1993,27 @@ def match_rows(dst_view, value, n_groups):
     for i, (_, _, t) in enumerate(comp.inputs):
         w = window_of(t.attrs["view"], t.shape, n_groups)
         if comp.kinds[i] == "tile":
-            if len(w.extent) != 2 or w.driver[1] is not None or \
-                    w.extent[1] != t.attrs["view"].base.shape[1] or w.extent[1] != n:
+            if len(w.extent) != 2 or (not broadcast_only and (
+                    w.driver[1] is not None or w.extent[1] != t.attrs["view"].base.shape[1] or
+                    w.extent[1] != n)):
                 raise NoNativeKernel("row reductions need tiles that hold whole rows")
             if tile_win is not None and (w.extent != tile_win.extent or w.driver != tile_win.driver):
                 raise NoNativeKernel("the tiles of a row expression must walk the same rows")
             tile_win = tile_win or w
-        else:
-            if any(d is not None for d in w.driver) or math.prod(w.extent) != n:
-                raise NoNativeKernel("a vector used by every row must be loaded whole by every group")
         wins.append(w)
     if tile_win is None:
         return None
+    width = tile_win.extent[1]                 # columns of the window (n when tiles hold whole rows)
+    for i, w in enumerate(wins):
+        if comp.kinds[i] != "tile":
+            # a vector every row uses: loaded whole by every group, or cut along the
+            # columns exactly as the tiles are
+            one_d = [d for d, e in enumerate(w.extent) if e != 1]
+            if math.prod(w.extent) != width or len(one_d) > 1 or \
+                    any(w.driver[d] is not None for d in range(len(w.extent)) if d not in one_d) or \
+                    (one_d and w.driver[one_d[0]] != tile_win.driver[1]):
+                raise NoNativeKernel("a vector used by every row must cover the columns of the tiles: loaded "
+                                     "whole by every group, or cut along the columns as the tiles are")
     col_wins = []
     for _, _, t in comp.columns:
         w = window_of(t.attrs["view"], t.shape, n_groups)
@@ -1989,7 +2044,7 @@ def match_rows(dst_view, value, n_groups):
             if comp.kinds[i] == "tile":
                 ins.append(_Arr(_sub(m, w.extent), ctx))
             else:
-                ins.append(_Arr(rt.Memref(m.ptr, (n,), (m.strides[-1],), m.itemsize), ctx))
+                ins.append(_Arr(rt.Memref(m.ptr, (width,), (m.strides[-1],), m.itemsize), ctx))
         cols = []
         for w in col_wins:
             m = mem[w.buffer]
@@ -2786,7 +2841,7 @@ def bind(stores, n_groups, atomics=(), mapped_stores=(), id_stores=(), group_sha
             return makers + [q]
         for view, value in stores:
             try:
-                for matcher in (match_fill, match_copy, match_imap, match_add, match_fma, match_softmax,
+                for matcher in (match_fill, match_copy, match_transpose, match_imap, match_add, match_fma, match_softmax,
                                 match_gemm, match_gather_gemm, match_gather_map, match_pairwise, match_cols,
                                 match_cols_tile, match_rows, match_map, match_fmap, match_general_windows):
                     mk = matcher(view, value, n_groups)
@@ -2798,10 +2853,14 @@ def bind(stores, n_groups, atomics=(), mapped_stores=(), id_stores=(), group_sha
             except NoNativeKernel as refusal:
                 # a kernel that walks one window refused the shape of the accesses
                 # (shifted, broadcast or transposed tiles): the gathered form may take it
-                try:
-                    mk = match_general_windows(view, value, n_groups)
-                except NoNativeKernel:
-                    raise refusal from None
+                mk = None
+                for fallback in (match_rows, match_general_windows):
+                    try:
+                        mk = fallback(view, value, n_groups)
+                    except NoNativeKernel:
+                        mk = None
+                    if mk is not None:
+                        break
                 if mk is None:
                     raise
                 makers.append(mk)

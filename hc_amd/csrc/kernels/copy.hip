@@ -159,6 +159,45 @@ HCAMD_COPY_TILED(hcamd_copy2d_tiled_b8, uint64_t)
 HCAMD_COPY_TILED(hcamd_copy2d_tiled_b16, u32x4)
 
 // ---------------------------------------------------------------------------
+// dst[c][r] = src[r][c] over a rows x cols window of src (what a body stores
+// that writes a tile's .T to the transposed window): 64 x 64 elements per
+// workgroup through LDS, read along the rows of src and written along the rows
+// of dst, 64 lanes to a row piece both ways; a pad column keeps the column
+// reads of the LDS tile off one bank.  Leading dimensions in elements.
+// ---------------------------------------------------------------------------
+namespace {
+template <class T>
+__device__ __forceinline__ void transpose_tile(const T *__restrict__ src, size_t lds, T *__restrict__ dst,
+                                               size_t ldd, uint32_t rows, uint32_t cols) {
+  __shared__ T tile[64][65];
+  const uint32_t tx = threadIdx.x % 64, ty = threadIdx.x / 64;   // 64 x 4 lanes
+  const uint32_t r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+#pragma unroll
+  for (uint32_t k = 0; k < 64; k += 4) {
+    const uint32_t r = r0 + ty + k, c = c0 + tx;
+    if (r < rows && c < cols)
+      tile[ty + k][tx] = src[(size_t)r * lds + c];
+  }
+  __syncthreads();
+#pragma unroll
+  for (uint32_t k = 0; k < 64; k += 4) {
+    const uint32_t c = c0 + ty + k, r = r0 + tx;                 // a row of dst is a column of src
+    if (c < cols && r < rows)
+      dst[(size_t)c * ldd + r] = tile[tx][ty + k];
+  }
+}
+} // namespace
+#define HCAMD_TRANSPOSE(NAME, T)                                                            \
+  extern "C" __global__ __launch_bounds__(256) void NAME(const T *src, size_t lds, T *dst,   \
+                                                         size_t ldd, uint32_t rows, uint32_t cols) { \
+    transpose_tile<T>(src, lds, dst, ldd, rows, cols);                                      \
+  }
+HCAMD_TRANSPOSE(hcamd_transpose2d_b1, uint8_t)
+HCAMD_TRANSPOSE(hcamd_transpose2d_b2, uint16_t)
+HCAMD_TRANSPOSE(hcamd_transpose2d_b4, uint32_t)
+HCAMD_TRANSPOSE(hcamd_transpose2d_b8, uint64_t)
+
+// ---------------------------------------------------------------------------
 // Stream calibration: what HBM delivers for a given mix of read and write
 // streams when nothing else is in the way.  R input vectors of 16-byte words
 // are added lane by lane (32-bit wrap-around) and

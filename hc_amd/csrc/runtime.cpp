@@ -790,6 +790,49 @@ const char *hcamdLastKernelName(void) noexcept { return t_lastKernel; }
 // ---------------------------------------------------------------------------
 // Typed launchers
 // ---------------------------------------------------------------------------
+int hcamdLaunchTranspose2D(OlQueue q, size_t elemSize, const void *src, size_t srcLd, void *dst,
+                           size_t dstLd, size_t rows, size_t cols) noexcept {
+  auto *queue = static_cast<Queue *>(q);
+  if (!queue)
+    return 1;
+  Device *dev = queue->device;
+  const char *name = elemSize == 1   ? "hcamd_transpose2d_b1"
+                     : elemSize == 2 ? "hcamd_transpose2d_b2"
+                     : elemSize == 4 ? "hcamd_transpose2d_b4"
+                     : elemSize == 8 ? "hcamd_transpose2d_b8"
+                                     : nullptr;
+  if (!name) {
+    dev->report("hcamdLaunchTranspose2D: unsupported element size %zu", elemSize);
+    return 1;
+  }
+  if (rows == 0 || cols == 0)
+    return 0;
+  if (!src || !dst) {
+    dev->report("hcamdLaunchTranspose2D: null pointer");
+    return 1;
+  }
+  if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) % elemSize) {
+    dev->report("hcamdLaunchTranspose2D: pointer not aligned to the element size");
+    return 1;
+  }
+  if ((rows > 1 && srcLd < cols) || (cols > 1 && dstLd < rows)) {
+    dev->report("hcamdLaunchTranspose2D: leading dimension smaller than a row");
+    return 1;
+  }
+  if (rows > 0xffffffffull || cols > 0xffffffffull || ceilDiv(rows, (size_t)64) > 65535) {
+    dev->report("hcamdLaunchTranspose2D: window of %zu x %zu (at most 4,194,240 rows)", rows, cols);
+    return 1;
+  }
+  Kernel *k = builtinKernel(dev, "copy", name);
+  if (!k)
+    return 1;
+  uint32_t nRows = static_cast<uint32_t>(rows), nCols = static_cast<uint32_t>(cols);
+  void *args[] = {&src, &srcLd, &dst, &dstLd, &nRows, &nCols};
+  const size_t grid[3] = {ceilDiv(cols, (size_t)64), ceilDiv(rows, (size_t)64), 1};
+  const size_t block[3] = {256, 1, 1};
+  return launch(queue, k, grid, block, args, 0);
+}
+
 int hcamdLaunchCopy2D(OlQueue q, size_t elemSize, const void *src,
                       size_t srcRows, size_t srcCols, ptrdiff_t ss0,
                       ptrdiff_t ss1, void *dst, size_t dstRows, size_t dstCols,

@@ -81,6 +81,7 @@ hcamdDeviceInfo = _sig(_rt, "hcamdDeviceInfo", _int, _vp, C.POINTER(_int),
 hcamdSetVariant = _sig(_rt, "hcamdSetVariant", _int, C.c_char_p, _int)
 hcamdSetThreadVariant = _sig(_rt, "hcamdSetThreadVariant", _int, C.c_char_p, _int)
 hcamdLastKernelName = _sig(_rt, "hcamdLastKernelName", C.c_char_p)
+hcamdLaunchTranspose2D = _sig(_rt, "hcamdLaunchTranspose2D", _int, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz)
 hcamdLaunchCopy2D = _sig(_rt, "hcamdLaunchCopy2D", _int, _vp, _sz, _vp, _sz, _sz,
                          _ssz, _ssz, _vp, _sz, _sz, _ssz, _ssz)
 hcamdLaunchCopy2DTiled = _sig(_rt, "hcamdLaunchCopy2DTiled", _int, _vp, _sz, _vp, _vp,
@@ -413,6 +414,19 @@ def plan_copy2d(src, dst) -> Plan:
                 (ctx.queue, s.itemsize, s.ptr, s.shape[0], s.shape[1], s.strides[0],
                  s.strides[1], d.ptr, d.shape[0], d.shape[1], d.strides[0], d.strides[1]),
                 "hcamdLaunchCopy2D", (src, dst))
+
+
+def plan_transpose2d(src, dst) -> Plan:
+    """dst[c, r] = src[r, c] over the part of src that fits dst transposed (see
+    hcamdLaunchTranspose2D); unit inner strides, equal element sizes."""
+    ctx = _ctx_of(src, dst)
+    s, d = as_memref(src, 2), as_memref(dst, 2)
+    if s.itemsize != d.itemsize or s.strides[1] != 1 or d.strides[1] != 1:
+        raise HcRuntimeError("transpose2d: unit inner stride and equal element size required")
+    rows, cols = min(s.shape[0], d.shape[1]), min(s.shape[1], d.shape[0])
+    return Plan(ctx, hcamdLaunchTranspose2D,
+                (ctx.queue, s.itemsize, s.ptr, s.strides[0], d.ptr, d.strides[0], rows, cols),
+                "hcamdLaunchTranspose2D", (src, dst))
 
 
 def plan_copy2d_tiled(src, dst, block_x: int, block_y: int, unroll: int = 1) -> Plan:

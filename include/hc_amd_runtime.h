@@ -218,6 +218,16 @@ int hcamdLaunchCopy2D(OlQueue q, size_t elemSize, const void *src,
                       size_t dstCols, ptrdiff_t dstStride0,
                       ptrdiff_t dstStride1) HCAMD_NOEXCEPT;
 
+/* dst[c][r] = src[r][c] for r < rows, c < cols: what a body stores that
+ * writes a loaded tile's `.T` to the transposed window (an attribute the
+ * reference's tile wrapper forwards to numpy.ma,
+ * python/hckernel/kernel_api.py:150-151).  elemSize is 1, 2, 4 or 8; leading
+ * dimensions in elements, unit inner strides; 64 x 64 elements per workgroup
+ * through LDS; every other byte of dst stays as it was; source and destination
+ * must not overlap. */
+int hcamdLaunchTranspose2D(OlQueue q, size_t elemSize, const void *src, size_t srcLd, void *dst,
+                           size_t dstLd, size_t rows, size_t cols) HCAMD_NOEXCEPT;
+
 /* Ids as data: out[index] = value for every work-item (perItem != 0) or once per
  * group, with index (one per dimension of out) and value affine in the group id
  * and the local id: x = c + sum_k g[k] * group_id[k] + sum_k l[k] * local_id[k],

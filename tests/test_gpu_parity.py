@@ -260,6 +260,27 @@ def test_copy_windows_whose_rows_lie_differently_in_the_two_arrays(ctx, dtype, r
     assert_array_equal(dst.to_host(), want)
 
 
+@pytest.mark.parametrize("dtype", [np.uint8, np.float16, np.float32, np.int64])
+@pytest.mark.parametrize("rows,cols,lds,ldd,soff,doff", [(1, 1, 1, 1, 0, 0), (64, 64, 64, 64, 0, 0), (37, 50, 50, 37, 0, 0),
+                                                          (100, 130, 141, 107, 3, 5), (5, 1000, 1000, 8, 0, 1),
+                                                          (1000, 3, 4, 1000, 1, 0)])
+def test_transposed_copy_of_windows(ctx, dtype, rows, cols, lds, ldd, soff, doff):
+    """hcamdLaunchTranspose2D: every element size, windows of larger arrays,
+    extents that do not fill the 64 x 64 tiles; everything outside the window
+    keeps the poison."""
+    rng = np.random.default_rng(rows + cols)
+    src = rng.integers(0, 200, (rows, lds)).astype(dtype)
+    dsrc = dev(np.concatenate([np.zeros(soff, dtype), src.reshape(-1)]))
+    ddst = poisoned((cols * ldd + doff,), dtype)
+    rt.plan_transpose2d(_View(dsrc, (rows, cols), soff, (lds, 1)), _View(ddst, (cols, rows), doff, (ldd, 1))).launch()
+    assert rt.last_kernel_name() == f"hcamd_transpose2d_b{np.dtype(dtype).itemsize}"
+    got = ddst.to_host()
+    want = np.full(cols * ldd + doff, poison_value(dtype), dtype)
+    body = want[doff:].reshape(cols, ldd)
+    body[:, :rows] = src[:, :cols].T
+    assert_array_equal(got.view(np.uint8), want.view(np.uint8))
+
+
 @pytest.mark.parametrize("variant", [0, 10])
 def test_copy_from_rows_in_reverse_order(ctx, variant):
     """A source window whose row stride is negative (the rows of an array bottom up)."""

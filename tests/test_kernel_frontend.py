@@ -886,17 +886,31 @@ def test_loads_that_do_not_walk_the_window_of_the_store_become_gathered_operands
             sim[name](*ins, want)
         fake = [FakeDev(v.shape, "float32") for v in ins]
         (p,) = gpu[name].plan(*fake, FakeDev(shape, "float32"), ctx=ctx)
-        assert p.fn is rt.hcamdGatherMapLaunch, name
-        got = np.full(shape, 77, f)
-        run_gathered_plan(p, MapTablesOnly.last, {d.ptr: v for d, v in zip(fake, ins)}, got)
+        if name == "broadcast":
+            # a row vector and a per-row operand next to a tile: one store stage of a row
+            # program over the whole window, whatever the groups' tiling
+            assert p.fn is rt.hcamdLaunchRowProgram and p.args[-2:] == (rows, cols)
+            assert (p.args[7], p.args[10]) == (2, 1)          # the tile and the vector; one per-row operand
+            got = run_row_stages(row_stages(p), [x, b], [sc], f, init=np.full(shape, 77, f))
+        else:
+            assert p.fn is rt.hcamdGatherMapLaunch, name
+            got = np.full(shape, 77, f)
+            run_gathered_plan(p, MapTablesOnly.last, {d.ptr: v for d, v in zip(fake, ins)}, got)
         np.testing.assert_array_equal(got, want, err_msg=name)
         assert (want == 77).any() or name == "transposed", name
     # the shifted window is a window start, the broadcast vector a table that ignores a dimension
     (p,) = gpu["shifted"].plan(FakeDev((200,), "float32"), FakeDev((200,), "float32"), ctx=ctx)
     t = MapTablesOnly.last
     assert t.operands[0][2][:3, 0].tolist() == [1, 17, 33] and t.operands[1][2][:3, 0].tolist() == [0, 16, 32]
-    (p,) = gpu["broadcast"].plan(FakeDev((12, 21), "float32"), FakeDev((21,), "float32"), FakeDev((12,), "float32"),
-                                 FakeDev((12, 21), "float32"), ctx=ctx)
+    # (a vector that the row program cannot take, here one shorter than the tiles are wide, stays gathered)
+    @kernel(work_shape=(M, N), group_shape=(4, 8))
+    def short_vector(gr: CurrentGroup, x: Buffer[M, N, DT], b: Buffer[sym.NB, DT], s: Buffer[M, DT], out: Buffer[M, N, DT]):
+        i, j = gr.work_offset
+        t = gr.load(x[i:, j:], shape=gr.shape)
+        gr.store(out[i:, j:], (t + gr.load(b[j:], shape=gr.shape[1])) * gr.load(s[i:], shape=gr.shape[0])[:, None])
+    (p,) = short_vector.plan(FakeDev((12, 21), "float32"), FakeDev((19,), "float32"), FakeDev((12,), "float32"),
+                             FakeDev((12, 21), "float32"), ctx=ctx)
+    assert p.fn is rt.hcamdGatherMapLaunch
     t = MapTablesOnly.last
     assert t.operands[1][3][:, 0].tolist() == list(range(8)) * 4         # the row vector: the column index
     assert t.operands[2][3][:, 0].tolist() == [r for r in range(4) for _ in range(8)]
@@ -915,8 +929,17 @@ def test_loads_that_do_not_walk_the_window_of_the_store_become_gathered_operands
     def int_transpose(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[N, M, DT]):
         i, j = gr.work_offset
         gr.store(out[j:, i:], gr.load(x[i:, j:], shape=gr.shape).T)
+    # a tile's .T alone, stored to the transposed window, is one transposed copy of the whole window
     (p,) = int_transpose.plan(FakeDev((11, 21), "int32"), FakeDev((21, 11), "int32"), ctx=ctx)
-    assert p.fn is rt.hcamdGatherMapLaunch and p.args[-1] == 4 and p.args[3] == 0      # a copy of 4-byte elements
+    assert p.fn is rt.hcamdLaunchTranspose2D and p.args[1] == 4 and p.args[-2:] == (11, 21)
+    (p,) = int_transpose.plan(FakeDev((11, 21), "int8", ld=32), FakeDev((21, 11), "int8", ld=16), ctx=ctx)
+    assert p.args[1] == 1 and p.args[-2:] == (11, 21) and (p.args[3], p.args[5]) == (32, 16)
+    @kernel(work_shape=(M, N), group_shape=(4, 8))
+    def wider_transpose(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[N, T2, DT]):
+        i, j = gr.work_offset
+        gr.store(out[j:, i:], gr.load(x[i:, j:], shape=gr.shape).T)
+    with pytest.raises(NoNativeKernel, match="written in full"):
+        wider_transpose.plan(FakeDev((11, 21), "int32"), FakeDev((21, 12), "int32"), ctx=ctx)
 
 
 def test_offsets_with_division_are_for_mapped_accesses_only(ctx):
