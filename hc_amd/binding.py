@@ -32,7 +32,7 @@ import math
 from dataclasses import dataclass
 
 from . import runtime as rt
-from .kernel_api import (Affine, BufferView, ItemIndex, Tile, TraceError, same_index,
+from .kernel_api import (Affine, BufferProxy, BufferView, ItemIndex, Tile, TraceError, same_index,
                          same_starts)
 
 
@@ -2799,6 +2799,111 @@ def match_id_store(proxy, index, value, per_item, n_groups, group_shape):
     return make
 
 
+_CELL_FOLDS = ("sum", "max", "min")
+
+
+def match_group_cells(proxy, index, value, accumulate, n_groups):
+    """`out[c + k * group_id] = f(tile.sum(), tile.max(), ...)`, or `+=` through
+    atomic_ref: one number per group, from reductions of whole 1-D tiles that cut
+    their arrays into consecutive pieces (the first stage of a two-stage
+    reduction).  The groups' tiles are the rows of a (groups, tile) view of the
+    arrays, the results a per-row output of a row program; a last tile that its
+    array does not fill is a second launch over the shorter row."""
+    if len(n_groups) != 1 or proxy.ndim != 1 or len(index) != 1:
+        raise NoNativeKernel("one result per group is bound for 1-D work shapes and 1-D result arrays")
+    if proxy.dtype_name not in _MAP_FLOATS:
+        raise NoNativeKernel(f"{proxy.name}: per-group results are stored to float32 / float16 arrays")
+    (at,) = index
+    co = _coeffs(at, 1)[0]
+    groups = n_groups[0]
+    if co != 1 or at.const < 0 or at.const + groups > proxy.shape[0] or proxy.strides[0] != 1:
+        raise NoNativeKernel(f"{proxy.name}[{at!r}]: per-group results go to consecutive elements inside a "
+                             "dense array (the group id plus a constant)")
+    loads = [t for t in _walk(value) if _is(t, "load")]
+    if not loads or any(len(t.shape) != 1 or t.shape != loads[0].shape for t in loads):
+        raise NoNativeKernel("per-group results are bound for reductions of 1-D tiles of one length")
+    tile = loads[0].shape[0]
+    n = None
+    for t in loads:
+        v = t.attrs["view"]
+        st = v.starts[0]
+        if not (isinstance(st, Affine) and st.const == 0 and _coeffs(st, 1)[0] == tile):
+            raise NoNativeKernel(f"{v.base.name}: the tiles of a per-group reduction must cut the array into "
+                                 "consecutive pieces (group_id * tile_length)")
+        if n is not None and v.base.shape[0] != n:
+            raise NoNativeKernel("the arrays of a per-group reduction must have one length")
+        n = v.base.shape[0]
+    full, rest = divmod(n, tile)
+    if groups != full + (1 if rest else 0):
+        raise NoNativeKernel(f"{groups} groups of {tile} elements over arrays of {n}: a group without an element "
+                             "has nothing to reduce (numpy.ma gives it a masked value)")
+
+    def lifted(width, rows):
+        """The expression over (1, width) row tiles of (rows, width) views; the
+        views are what `views` maps argument indices to."""
+        memo, views = {}, {}
+
+        def view_of(base, shape, strides, start):
+            p2 = BufferProxy(base.index, base.name, shape, strides, base.dtype_name, None)
+            views[base.index] = (shape, strides)
+            return BufferView(p2, start)
+
+        def go(t):
+            if t.uid in memo:
+                return memo[t.uid]
+            if _const(t):
+                out = t if t.shape == () else _const_tile((1, width), t.dtype_name, t)
+            elif _is(t, "load"):
+                base = t.attrs["view"].base
+                v2 = view_of(base, (rows, width), (tile * base.strides[0], base.strides[0]),
+                             (Affine(0, (1,)), Affine(0, (0,))))
+                out = Tile("load", (), (1, width), t.dtype_name, view=v2)
+            elif t.op in _CELL_FOLDS and len(t.args) == 1 and len(t.args[0].shape) == 1 and t.shape == ():
+                out = Tile(t.op, (go(t.args[0]),), (1,), t.dtype_name,
+                           **{**t.attrs, "axes": (1,), "keepdims": False})
+            elif t.op in _REDUCTIONS or t.op in ("norm", "dot", "slice", "reshape", "transpose", "update", "window"):
+                raise NoNativeKernel(f"{t!r}: per-group results are built from sum, max and min of whole 1-D "
+                                     "tiles and arithmetic on them")
+            else:
+                args = tuple(go(a) if isinstance(a, Tile) else a for a in t.args)
+                shape = (1,) if t.shape == () else (1, width)
+                out = Tile(t.op, args, shape, t.dtype_name, **t.attrs)
+            memo[t.uid] = out
+            return out
+
+        v2 = go(value)
+        out_stride = co * proxy.strides[0]
+        dst = view_of(proxy, (rows,), (out_stride,), (Affine(0, (1,)),))
+        if accumulate:
+            old = Tile("load", (), (1,), proxy.dtype_name, view=dst)
+            v2 = Tile("add", (old, v2), (1,), proxy.dtype_name, plain=True)
+        mk = match_rows(dst, v2, (rows,))
+        if mk is None:
+            raise NoNativeKernel(f"{value!r}: not a reduction of tiles that a row program computes")
+        return mk, views
+
+    parts = []                                    # (maker, views, first row)
+    if full:
+        parts.append(lifted(tile, full) + (0,))
+    if rest:
+        parts.append(lifted(rest, 1) + (full,))
+
+    def make(mem, ctx):
+        plans = []
+        for mk, views, row0 in parts:
+            patched = list(mem)
+            for i, (shape, strides) in views.items():
+                m = mem[i]
+                if i == proxy.index and len(shape) == 1:
+                    offset = at.const * m.strides[0] + row0 * strides[0]
+                else:
+                    offset = row0 * tile * m.strides[0]
+                patched[i] = rt.Memref(m.ptr + offset * m.itemsize, shape, strides, m.itemsize)
+            plans += mk(patched, ctx)
+        return plans
+    return make
+
+
 def _has_dot(t: Tile, seen=None) -> bool:
     seen = set() if seen is None else seen
     if t.uid in seen:
@@ -2807,29 +2912,31 @@ def _has_dot(t: Tile, seen=None) -> bool:
     return t.op == "dot" or any(_has_dot(a, seen) for a in t.args)
 
 
-def bind(stores, n_groups, atomics=(), mapped_stores=(), id_stores=(), group_shape=()):
+def bind(stores, n_groups, atomics=(), mapped_stores=(), id_stores=(), group_shape=(), cell_stores=()):
     """stores: list of (BufferView, Tile) from one traced execution; atomics:
     list of (BufferProxy, index, Tile) atomic additions; mapped_stores: list of
     (BufferView, Tile, index function); id_stores: (BufferProxy, index, value,
     per work-item?) element stores of ids.  Returns a list of plan makers;
     raises NoNativeKernel when nothing matches."""
-    if not stores and not atomics and not mapped_stores and not id_stores:
+    if not stores and not atomics and not mapped_stores and not id_stores and not cell_stores:
         raise NoNativeKernel("the kernel body stores nothing")
     memo = {}
     stores = [(view, simplify(value, memo)) for view, value in stores]
     for view, value in stores:
         _overlay_guard(view, value, memo.get("overlays", ()), n_groups)
     id_makers = [match_id_store(p, i, v, per, n_groups, group_shape) for p, i, v, per in id_stores]
-    if id_stores and not (stores or atomics or mapped_stores):
+    if id_stores and not (stores or atomics or mapped_stores or cell_stores):
         return id_makers
     try:
         if atomics:
-            if stores or mapped_stores:
+            if stores or mapped_stores or cell_stores:
                 raise NoNativeKernel("a body that both stores tiles and accumulates "
                                      "atomically has no native kernel")
             return [mk for proxy, index, value in atomics
                     for mk in match_sum(proxy, index, value, n_groups)]
         makers = list(id_makers)
+        for proxy, index, value, accumulate in cell_stores:
+            makers.append(match_group_cells(proxy, index, simplify(value, memo), accumulate, n_groups))
         for view, value, func in mapped_stores:
             value = simplify(value, memo)
             if _has_dot(value):

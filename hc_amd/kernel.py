@@ -276,7 +276,7 @@ class GpuKernel:
                 if isinstance(p, BufferProxy):
                     p.obj = None
         return bind(group_obj.stores, n_groups, group_obj.atomics, group_obj.mapped_stores,
-                    group_obj.id_stores, group)
+                    group_obj.id_stores, group, group_obj.cell_stores)
 
     def plan(self, *args, ctx=None):
         """Everything a call does short of launching: returns the list of

@@ -106,11 +106,10 @@ class AtomicRef:
             index = index[0]
         if isinstance(index, Affine):
             if not index.is_const:
-                raise TraceError("atomic updates of an element chosen by the group id have no "
-                                 "native kernel yet")
+                return _AtomicCell(self, index)       # a cell of the group's own: see record()
             index = index.const
         if not isinstance(index, (int, np.integer)):
-            raise TraceError("atomic_ref(buffer)[i]: i must be an integer")
+            raise TraceError("atomic_ref(buffer)[i]: i must be an integer or built from the group id")
         return _AtomicCell(self, int(index))
 
     def __setitem__(self, index, value):
@@ -121,6 +120,11 @@ class AtomicRef:
         group = getattr(self.proxy, "group", None)
         if group is None:
             raise TraceError("atomic_ref outside a kernel body")
+        if isinstance(index, Affine):
+            # `ref[f(group id)] += value`: every group adds to an element that the
+            # index picks for it
+            group.cell_stores.append((self.proxy, (index,), Tile.wrap(value), True))
+            return
         group.atomics.append((self.proxy, index, Tile.wrap(value)))
 
 
@@ -1041,6 +1045,7 @@ class CurrentGroup:
                          for i in range(rank))
         self.stores = []          # (BufferView, Tile) in program order
         self.atomics = []         # (BufferProxy, element index, Tile) atomic additions
+        self.cell_stores = []     # (BufferProxy, index of Affine, scalar Tile, add to the old value?)
         self.mapped_stores = []   # (BufferView, Tile, index function) scattered stores
         self.id_stores = []       # (BufferProxy, ItemIndex per dim, value ItemIndex, per work-item?)
         self._ring = []           # greenlets of the subgroup scope that is running
@@ -1236,9 +1241,15 @@ class CurrentGroup:
                                  "is stored at wi.global_id() only")
             self.store(proxy[tuple(slice(o, None) for o in self.work_offset)], value)
             return
+        if isinstance(value, Tile) and value.shape == () and not self._in_workitems and \
+                all(not any(i.l) for i in index):
+            # `out[f(group id)] = tile.sum()`: one result per group
+            rank = len(self._shape)
+            self.cell_stores.append((proxy, tuple(Affine(i.const, i.g[:rank]) for i in index), value, False))
+            return
         if isinstance(value, Tile):
-            raise TraceError("only ids, numbers and per-work-item values may be assigned to a "
-                             "buffer element")
+            raise TraceError("only ids, numbers, per-work-item values and (at group level) reductions "
+                             "of whole tiles may be assigned to a buffer element")
         rank = len(self._shape)
         if isinstance(value, (float, np.floating)) and float(value) != int(value):
             raise TraceError("only integers and ids may be assigned to a buffer element")

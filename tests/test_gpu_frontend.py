@@ -1268,6 +1268,52 @@ def test_loads_that_do_not_walk_the_window_of_the_store_match_the_simulator(rows
             assert (want == 7).any(), name                 # something is left alone
 
 
+@pytest.mark.parametrize("n,tile", [(1000, 256), (1024, 256), (77, 64), (5000, 1024), (300, 512)])
+def test_one_result_per_group_from_reductions_of_whole_tiles(n, tile):
+    """`out[group id] = tile.sum()` and `atomic_ref(out)[f(group id)] += ...`:
+    the first stage of a two-stage reduction, every group with an element of
+    its own; against the simulator, the last tile shorter than the others,
+    elements no group owns left as they were."""
+    N, G = sym.N, sym.G
+
+    def bodies(deco):
+        @deco(work_shape=N, group_shape=tile)
+        def sums(gr: CurrentGroup, x: Buffer[N, DT], out: Buffer[G, DT]):
+            o = gr.work_offset[0]
+            t = gr.load(x[o:], shape=gr.shape)
+            out[gr.id[0]] = (t * t).sum()
+
+        @deco(work_shape=N, group_shape=tile)
+        def spread(gr: CurrentGroup, x: Buffer[N, DT], y: Buffer[N, DT], out: Buffer[G, DT]):
+            o = gr.work_offset[0]
+            t, u = gr.load(x[o:], shape=gr.shape), gr.load(y[o:], shape=gr.shape)
+            atomic_ref(out)[gr.id[0] + 2] += (t + u).max() - np.minimum(t, u).min()
+        return sums, spread
+
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal(n).astype(np.float32)
+    y = rng.standard_normal(n).astype(np.float32)
+    groups = -(-n // tile)
+    (g_sums, g_spread), (s_sums, s_spread) = bodies(kernel), bodies(sim_kernel)
+    want = np.full(groups + 3, 7, np.float32)
+    s_sums(x, want)
+    out = rt.to_device(np.full(groups + 3, 7, np.float32))
+    g_sums(rt.to_device(x), out)
+    assert rt.last_kernel_name().startswith("hcamd_row_program")
+    got = out.to_host()
+    assert_allclose(got, want, rtol=2e-6 * np.sqrt(tile))
+    assert (got[groups:] == 7).all()
+    start = rng.standard_normal(groups + 5).astype(np.float32)
+    want = start.copy()
+    s_spread(x, y, want)
+    out = rt.to_device(start)
+    g_spread(rt.to_device(x), rt.to_device(y), out)
+    got = out.to_host()
+    assert_allclose(got, want, rtol=1e-6, atol=1e-6)
+    assert_array_equal(got[:2], start[:2])
+    assert_array_equal(got[groups + 2:], start[groups + 2:])
+
+
 def test_tile_mask_is_stored_as_a_plain_bool_array():
     """`tile.mask` (python/hckernel/kernel_api.py:117-119: True = active) of
     float and int32 expressions that the data deactivates here and there: the

@@ -483,9 +483,21 @@ def test_reference_reduction_bodies_bind_to_the_map_sum_kernel(ctx):
     def assigned(gr: CurrentGroup, a: Buffer[WS, DT], result: Buffer[4, DT]):
         atomic_ref(result)[0] = gr.load(a[gr.work_offset[0]:], shape=gr.shape[0]).sum()
 
-    for k in (per_group, not_a_sum, assigned):
+    for k in (not_a_sum, assigned):
         with pytest.raises(NoNativeKernel):
             k.plan(a, res4, ctx=ctx)
+    # an element per group: the groups' tiles are the rows of a row program with a per-row result
+    # (20 elements in tiles of 256: one short row)
+    (p,) = per_group.plan(a, res4, ctx=ctx)
+    assert p.fn is rt.hcamdLaunchRowProgram and p.args[-2:] == (1, 20)
+    # (slot 0: the element's old value, read as a per-row operand; slot 1: the row's sum)
+    assert row_stages(p) == [("sum", 1, [("in", 0, 0.0)]), ("store_col", 0, [("red", 0, 0.0), ("add_red", 1, 0.0)])]
+    big = FakeDev((1000,), "float32")
+    plans = per_group.plan(big, res4, ctx=ctx)
+    assert [q.args[-2:] for q in plans] == [(3, 256), (1, 232)]
+    assert plans[1].args[4][0] == big.ptr + 3 * 256 * 4 and plans[1].args[11] == res4.ptr + 3 * 4
+    with pytest.raises(NoNativeKernel, match="consecutive elements"):
+        per_group.plan(FakeDev((2000,), "float32"), res4, ctx=ctx)         # eight groups, four elements
     with pytest.raises(NoNativeKernel, match="float32"):
         reduction_1.plan(a, FakeDev((1,), "float16"), 8, ctx=ctx)
 
