@@ -1025,6 +1025,11 @@ class Tile:
 
 
 def _dot(a: Tile, b: Tile) -> Tile:
+    if len(a.shape) == 2 and len(b.shape) == 1 and a.shape[1] == b.shape[0]:
+        # matrix times vector: the rows' sums of products (NumPy computes on the
+        # data, where an inactive element is the 0 a load puts there,
+        # python/hckernel/kernel_api.py:223-224,301-303: the same sum)
+        return a._binary(b, "mul")._reduce("sum", 1, False)
     if len(a.shape) != 2 or len(b.shape) != 2 or a.shape[1] != b.shape[0]:
         raise TraceError(f"dot of shapes {a.shape} and {b.shape}")
     return Tile("dot", (a, b), (a.shape[0], b.shape[1]), promote(a.dtype_name, b.dtype_name))

@@ -1314,6 +1314,30 @@ def test_one_result_per_group_from_reductions_of_whole_tiles(n, tile):
     assert_array_equal(got[groups + 2:], start[groups + 2:])
 
 
+@pytest.mark.parametrize("rows,k", [(64, 128), (37, 1000), (300, 4097)])
+def test_matrix_times_vector_is_a_row_sum_of_products(rows, k):
+    """numpy.dot of a (rows, K) tile and a (K,) tile: the row program's sum of
+    products along the rows; against the simulator's numpy.dot to the bound of a
+    sum of K fp32 products added in another order."""
+    M, K = sym.M, sym.K
+
+    def body(gr: CurrentGroup, a: Buffer[M, K, DT], v: Buffer[K, DT], out: Buffer[M, DT]):
+        i = gr.work_offset[0]
+        gr.store(out[i:], np.dot(gr.load(a[i:, :], shape=(gr.shape[0], K)), gr.load(v[:], shape=(K,))))
+
+    rng = np.random.default_rng(k)
+    a = rng.standard_normal((rows, k)).astype(np.float32)
+    v = rng.standard_normal(k).astype(np.float32)
+    want = np.full(rows, 7, np.float32)
+    sim_kernel(work_shape=M, group_shape=8)(body)(a, v, want)
+    out = rt.to_device(np.full(rows, 7, np.float32))
+    kernel(work_shape=M, group_shape=8)(body)(rt.to_device(a), rt.to_device(v), out)
+    assert rt.last_kernel_name().startswith("hcamd_row_program")
+    bound = 4 * np.finfo(np.float32).eps * (np.abs(a) @ np.abs(v))
+    assert (np.abs(out.to_host() - want) <= bound).all()
+    assert_allclose(out.to_host(), a.astype(np.float64) @ v.astype(np.float64), atol=float(bound.max()))
+
+
 def test_tile_mask_is_stored_as_a_plain_bool_array():
     """`tile.mask` (python/hckernel/kernel_api.py:117-119: True = active) of
     float and int32 expressions that the data deactivates here and there: the
