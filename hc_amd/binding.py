@@ -748,8 +748,8 @@ def _maybe_masked(t: Tile, memo=None) -> bool:
     their number never is.)"""
     memo = {} if memo is None else memo
     if t.uid not in memo:
-        if _is(t, "load") or _const(t) or t.op == "count":
-            memo[t.uid] = False
+        if _is(t, "load") or _const(t) or t.op in ("count", "where"):
+            memo[t.uid] = False                  # (numpy.where returns a plain array)
         else:
             memo[t.uid] = _masks(t) or any(_maybe_masked(a, memo) for a in t.args if isinstance(a, Tile))
     return memo[t.uid]
@@ -803,8 +803,8 @@ def _can_fail(t: Tile, finite: bool, memo=None) -> bool:
         return _maybe_masked(t)
     memo = {} if memo is None else memo
     if t.uid not in memo:
-        if _is(t, "load") or _const(t) or t.op == "count":
-            memo[t.uid] = False
+        if _is(t, "load") or _const(t) or t.op in ("count", "where"):
+            memo[t.uid] = False                  # (numpy.where returns a plain array)
         else:
             memo[t.uid] = _fails_on_finite_data(t) or \
                 any(_can_fail(a, True, memo) for a in t.args if isinstance(a, Tile))
@@ -1171,7 +1171,8 @@ def match_imap(dst_view, value, n_groups):
 _FMAP_BINARY = {"add": "add", "sub": "sub", "mul": "mul", "div": "div", "floordiv": "floordiv",
                 "mod": "mod", "maximum": "max", "minimum": "min", "lt": "lt", "le": "le", "eq": "eq",
                 "ne": "ne", "ge": "ge", "gt": "gt"}
-_FMAP_UNARY = {"neg": "neg", "abs": "abs", "sqrt": "sqrt", "rint": "rint", "exp": "exp", "log": "log"}
+_FMAP_UNARY = {"neg": "neg", "abs": "abs", "sqrt": "sqrt", "rint": "rint", "exp": "exp", "log": "log",
+               "tanh": "tanh"}
 _FMAP_MIRROR = {"add": "add", "mul": "mul", "max": "max", "min": "min", "eq": "eq", "ne": "ne",
                 "lt": "gt", "gt": "lt", "le": "ge", "ge": "le"}
 _FMAP_COMPARE = ("lt", "le", "eq", "ne", "ge", "gt")
@@ -1186,11 +1187,20 @@ def _compile_fmap(value, mapped=False):
     def fdtype(t):
         return t.attrs.get("operand_dtype", t.dtype_name) if t.op in _FMAP_COMPARE else t.dtype_name
 
+    def int_leaf(t):
+        """The int32 load behind `load.astype(float32)`: converted when it is read."""
+        if _is(t, "astype", 1) and t.dtype_name == "float32" and t.args[0].dtype_name == "int32" and \
+                (_is(t.args[0], "load") or (mapped and _is(t.args[0], "mapped_load"))):
+            return t.args[0]
+        return None
+
     def need(t):
         if t.uid in needs:
             return needs[t.uid]
-        if _is(t, "load") or _is(t, "mapped_load") or _const(t):
+        if _is(t, "load") or _is(t, "mapped_load") or _const(t) or int_leaf(t) is not None:
             n = 1
+        elif _is(t, "where", 3):
+            n = max(need(t.args[0]), 1 + need(t.args[1]), 2 + need(t.args[2]))
         elif len(t.args) == 1:
             n = need(t.args[0])
         elif len(t.args) == 2:
@@ -1208,8 +1218,10 @@ def _compile_fmap(value, mapped=False):
         """Appends the code for t; False if t is not a float expression this kernel takes."""
         half = t.dtype_name == "float16"
         func = bool(t.attrs.get("func"))
+        if int_leaf(t) is not None:
+            t = int_leaf(t)
         if _is(t, "load") or (mapped and _is(t, "mapped_load")):
-            if t.dtype_name not in _MAP_FLOATS:
+            if t.dtype_name not in _MAP_FLOATS + ("int32",):
                 return False
             for i, u in enumerate(loads):
                 if _same(u, t):
@@ -1230,6 +1242,16 @@ def _compile_fmap(value, mapped=False):
             ok = emit(src)
             if half and src.dtype_name == "float32":
                 program.append(("r16", 0, 0.0))
+            return ok
+        if _is(t, "where", 3):
+            if t.dtype_name not in _MAP_FLOATS:
+                return False
+            for x in t.args:
+                if _const(x):
+                    program.append(("const", 0, _round_to(x.attrs["value"], t.dtype_name)))
+                else:
+                    ok = emit(x) and ok
+            program.append(("select", 0, 0.0))
             return ok
         if _is(t, "active", 1):
             ok = emit(t.args[0])                   # tile.mask: the entry's activity as 0 / 1
@@ -1320,7 +1342,7 @@ def match_fmap(dst_view, value, n_groups):
     w = _check_same_window(wins)
     if len(w.extent) > 2:
         raise NoNativeKernel("only 1-D and 2-D buffers have native kernels")
-    types = [rt.F16 if t.dtype_name == "float16" else rt.F32 for t in loads]
+    types = [{"float16": rt.F16, "int32": rt.I32}.get(t.dtype_name, rt.F32) for t in loads]
     types.append({"float32": rt.F32, "float16": rt.F16, "bool": rt.U8}[out_dt])
     store_all = bool(value.attrs.get("plain"))     # a bare numpy.ma array is written in full
 
@@ -1450,7 +1472,7 @@ def match_gather_map(dst_view, value, n_groups, out_func=None, force=False):
                                  "stored to one place; their order is the reference's group order, which "
                                  "a launch does not keep")
     indices = [t.attrs["view"].base.index for t in loads] + [dst_view.base.index]
-    types = [rt.F16 if t.dtype_name == "float16" else rt.F32 for t in loads]
+    types = [{"float16": rt.F16, "int32": rt.I32}.get(t.dtype_name, rt.F32) for t in loads]
     out_type = {"float32": rt.F32, "float16": rt.F16, "bool": rt.U8}.get(out_dt, rt.F32)
     store_all = bool(value.attrs.get("plain")) and not copy_bytes
     cache = {}
@@ -1525,7 +1547,7 @@ def _gathered_form(value):
             out = go(src, np.stack(child)) if len(child) == len(src.shape) else None
         elif t.op in _REDUCTIONS or t.op in ("dot", "norm", "window", "update"):
             out = None
-        elif len(t.args) in (1, 2) and all(isinstance(a, Tile) for a in t.args):
+        elif len(t.args) in (1, 2, 3) and all(isinstance(a, Tile) for a in t.args):
             args = []
             for a in t.args:
                 if a.shape == ():
@@ -1564,7 +1586,7 @@ def match_general_windows(dst_view, value, n_groups):
     out_dt = dst_view.base.dtype_name
     copy = _is(_strip_views(value), "load") and value.dtype_name == out_dt
     if not copy and (out_dt not in _MAP_FLOATS + ("bool",) or
-                     any(_is(t, "load") and t.dtype_name not in _MAP_FLOATS for t in _walk(value))):
+                     any(_is(t, "load") and t.dtype_name not in _MAP_FLOATS + ("int32",) for t in _walk(value))):
         return None                              # (copies move any element type)
     lowered = _gathered_form(value)
     if lowered is None:

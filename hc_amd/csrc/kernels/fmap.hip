@@ -32,7 +32,9 @@
 //     that is not finite becomes inactive with the value 1e20.
 //   * comparisons give 0 / 1 and are false for NaN except !=.
 //   * FOP_ACTIVE is `tile.mask`: 1 where the element is active, 0 where not, a
-//     plain array (every element active again).
+//     plain array (every element active again).  FOP_SELECT is numpy.where: a
+//     plain array too, chosen from the values whatever their activity.
+//   * an int32 operand is converted when it is read (tile.astype(float32)).
 // The store skips inactive elements, or with store_all writes every value: a
 // NumPy function returns a bare numpy.ma array, which the reference's store
 // copies in full.
@@ -56,6 +58,10 @@ enum : uint32_t {
   FOP_NEG = 18, FOP_ABS = 19, FOP_SQRT = 20, FOP_RINT = 21, FOP_EXP = 22, FOP_LOG = 23,
   FOP_R16 = 24, FOP_PSQRT = 25, FOP_POWCHK = 26,
   FOP_ACTIVE = 27, // `tile.mask`: 1 where the element is active in the entry, else 0; active again
+  FOP_TANH = 28,
+  // numpy.where(c, a, b) with c, a, b the three top entries (b on top): NumPy takes the
+  // values whatever their activity and returns a plain array, so the result is active
+  FOP_SELECT = 29,
 };
 
 struct Instr {
@@ -70,7 +76,7 @@ struct FMapArgs {
   size_t ld[kMaxIn];
   size_t ldo;
   size_t rows, cols;
-  uint32_t f16_mask; // bit i: operand i is fp16
+  uint32_t f16_mask; // bit i: operand i is fp16; bit 8 + i: operand i is int32 (converted when read)
   uint32_t out_type; // 0 fp32, 1 fp16, 2 one byte of 0 / 1
   uint32_t vec;      // every row of every operand and of the output starts 16-byte aligned
   uint32_t store_all; // write inactive elements too
@@ -185,6 +191,7 @@ __device__ __forceinline__ float unary(uint32_t op, float a, bool &ok) {
     return logf(a);
   case FOP_RINT: return __builtin_rintf(a);
   case FOP_EXP: return expf(a);
+  case FOP_TANH: return tanh_selects(a);
   case FOP_R16: return round16(a);
   case FOP_PSQRT: return ok ? __builtin_sqrtf(a) + 0.0f : a; // pow(-0, 0.5) is +0
   case FOP_ACTIVE: {
@@ -229,6 +236,11 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_fmap(FMapArgs a) {
         for (int e = 0; e < kV; ++e)
           v[i][e] = col0 + e < a.cols ? (float)p[e] : 0.0f;
       }
+    } else if ((a.f16_mask >> (8 + i)) & 1) {
+      const int32_t *p = static_cast<const int32_t *>(a.in[i]) + row * a.ld[i] + col0;
+#pragma unroll
+      for (int e = 0; e < kV; ++e)
+        v[i][e] = col0 + e < a.cols ? (float)p[e] : 0.0f;
     } else {
       const float *p = static_cast<const float *>(a.in[i]) + row * a.ld[i] + col0;
       if (a.vec && whole) {
@@ -268,6 +280,14 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_fmap(FMapArgs a) {
           x = arg == 0 ? v[0][e] : arg == 1 ? v[1][e] : arg == 2 ? v[2][e] : v[3][e];
         t0[e] = x;
         k0[e] = true;
+      }
+    } else if (op == FOP_SELECT) {
+#pragma unroll
+      for (int e = 0; e < kV; ++e) {
+        t0[e] = t2[e] != 0.0f ? t1[e] : t0[e];
+        k0[e] = true;
+        t1[e] = t3[e];
+        k1[e] = k3[e];
       }
     } else if (op >= FOP_NEG) {
 #pragma unroll
@@ -353,7 +373,7 @@ struct GatherMapArgs {
   void *out;
   GatherMapOperand op[kMaxIn + 1]; // the inputs, then the output
   uint32_t n_in, tile_elems, chunks; // chunks: workgroups per group
-  uint32_t f16_mask;  // bit i: operand i is fp16
+  uint32_t f16_mask;  // bit i: operand i is fp16; bit 8 + i: operand i is int32 (converted when read)
   uint32_t out_type;  // 0 fp32, 1 fp16, 2 one byte of 0 / 1
   uint32_t store_all; // write deactivated results too
   uint32_t copy_bytes; // != 0: no program, operand 0 is copied as elements of this many bytes
@@ -404,8 +424,9 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_gather_fmap(GatherMapArg
       const int64_t at = gather_offset(a.op[i], g, e);
       act[i] = at >= 0;
       if (at >= 0)
-        v[i] = ((a.f16_mask >> i) & 1) ? (float)static_cast<const _Float16 *>(a.in[i])[at]
-                                        : static_cast<const float *>(a.in[i])[at];
+        v[i] = ((a.f16_mask >> i) & 1)         ? (float)static_cast<const _Float16 *>(a.in[i])[at]
+               : ((a.f16_mask >> (8 + i)) & 1) ? (float)static_cast<const int32_t *>(a.in[i])[at]
+                                               : static_cast<const float *>(a.in[i])[at];
     }
   }
   float t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
@@ -421,6 +442,11 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_gather_fmap(GatherMapArg
         t0 = arg == 0 ? v[0] : arg == 1 ? v[1] : arg == 2 ? v[2] : v[3];
         k0 = arg == 0 ? act[0] : arg == 1 ? act[1] : arg == 2 ? act[2] : act[3];
       }
+    } else if (op == FOP_SELECT) {
+      t0 = t2 != 0.0f ? t1 : t0;
+      k0 = true;
+      t1 = t3;
+      k1 = k3;
     } else if (op >= FOP_NEG) {
       t0 = unary(op, t0, k0);
     } else {

@@ -141,29 +141,6 @@ template <int OP> __device__ __forceinline__ float binary(float a, float b) {
   if constexpr (OP == OP_RDIV) return b / a;
   return a;
 }
-// tanh without a branch.  The library routine chooses between its two formulas
-// with a per-lane branch, and one per-lane branch inside the interpreter is
-// enough for the compiler to linearise the whole dispatch around it (every arm
-// becomes a block that is stepped over, and all stack registers are copied at
-// every join).  Both formulas are evaluated here and one is selected:
-// |x| < 1: x + x^3 P(x^2), P fitted to (tanh(t)/t - 1)/t^2 (1.1 ulp);
-// otherwise 1 - 2/(exp(2|x|) + 1) (1.1 ulp); the sign is copied from x, and a
-// NaN comes out of the second formula as a NaN.
-__device__ __forceinline__ float tanh_selects(float x) {
-  const float t = __builtin_fabsf(x);
-  const float z = t * t;
-  float p = -0.00035845194361172616f;
-  p = __builtin_fmaf(p, z, 0.0023013644386082888f);
-  p = __builtin_fmaf(p, z, -0.007946105673909187f);
-  p = __builtin_fmaf(p, z, 0.021486656740307808f);
-  p = __builtin_fmaf(p, z, -0.05387980118393898f);
-  p = __builtin_fmaf(p, z, 0.13332344591617584f);
-  p = __builtin_fmaf(p, z, -0.33333295583724976f);
-  const float small = __builtin_fmaf(t * z, p, t);
-  const float big = 1.0f - 2.0f / (expf(2.0f * t) + 1.0f);
-  return __builtin_copysignf(t < 1.0f ? small : big, x);
-}
-
 template <int OP> __device__ __forceinline__ float unary(float a) {
   if constexpr (OP == OP_NEG) return -a;
   if constexpr (OP == OP_ABS) return __builtin_fabsf(a);

@@ -1660,12 +1660,13 @@ int hcamdLaunchFMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
       return 1;
     }
     const bool push = op == HCAMD_FMAP_IN || op == HCAMD_FMAP_CONST;
-    const bool unary = op >= HCAMD_FMAP_NEG;
-    if (sp < (push ? 0 : unary ? 1 : 2)) {
+    const bool select = op == HCAMD_FMAP_SELECT; // three entries in, one out
+    const bool unary = op >= HCAMD_FMAP_NEG && !select;
+    if (sp < (push ? 0 : unary ? 1 : select ? 3 : 2)) {
       dev->report("%s: stack underflow at %zu", who, i);
       return 1;
     }
-    sp += push ? 1 : unary ? 0 : -1;
+    sp += push ? 1 : unary ? 0 : select ? -2 : -1;
     if (sp > 4) {
       dev->report("%s: stack deeper than 4 at %zu", who, i);
       return 1;
@@ -1698,7 +1699,7 @@ int hcamdLaunchFMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
       dev->report("%s: null pointer", who);
       return 1;
     }
-    if (inputTypes[i] != HCAMD_F32 && inputTypes[i] != HCAMD_F16) {
+    if (inputTypes[i] != HCAMD_F32 && inputTypes[i] != HCAMD_F16 && inputTypes[i] != HCAMD_I32) {
       dev->report("%s: unsupported operand type %d", who, inputTypes[i]);
       return 1;
     }
@@ -1710,6 +1711,8 @@ int hcamdLaunchFMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
     a.ld[i] = inputLd[i];
     if (inputTypes[i] == HCAMD_F16)
       a.f16_mask |= 1u << i;
+    if (inputTypes[i] == HCAMD_I32)
+      a.f16_mask |= 1u << (8 + i); // converted to fp32 when read
     vec = vec && piece_ok(inputs[i], inputTypes[i], inputLd[i]);
   }
   if (rows > 1 && ldo < cols) {
@@ -3244,12 +3247,13 @@ int hcamdGatherMapLaunch(OlQueue q, HcamdGatherMap plan, const HcamdMapInstr *pr
         return 1;
       }
       const bool push = op == HCAMD_FMAP_IN || op == HCAMD_FMAP_CONST;
-      const bool unary = op >= HCAMD_FMAP_NEG;
-      if (sp < (push ? 0 : unary ? 1 : 2)) {
+      const bool select = op == HCAMD_FMAP_SELECT; // three entries in, one out
+      const bool unary = op >= HCAMD_FMAP_NEG && !select;
+      if (sp < (push ? 0 : unary ? 1 : select ? 3 : 2)) {
         dev->report("%s: stack underflow at %zu", who, i);
         return 1;
       }
-      sp += push ? 1 : unary ? 0 : -1;
+      sp += push ? 1 : unary ? 0 : select ? -2 : -1;
       if (sp > 4) {
         dev->report("%s: stack deeper than 4 at %zu", who, i);
         return 1;
@@ -3270,13 +3274,16 @@ int hcamdGatherMapLaunch(OlQueue q, HcamdGatherMap plan, const HcamdMapInstr *pr
         dev->report("%s: null pointer", who);
         return 1;
       }
-      if (!copyBytes && inputTypes[i] != HCAMD_F32 && inputTypes[i] != HCAMD_F16) {
+      if (!copyBytes && inputTypes[i] != HCAMD_F32 && inputTypes[i] != HCAMD_F16 &&
+          inputTypes[i] != HCAMD_I32) {
         dev->report("%s: unsupported operand type %d", who, inputTypes[i]);
         return 1;
       }
       a.in[i] = inputs[i];
       if (!copyBytes && inputTypes[i] == HCAMD_F16)
         a.f16Mask |= 1u << i;
+      if (!copyBytes && inputTypes[i] == HCAMD_I32)
+        a.f16Mask |= 1u << (8 + i); // converted to fp32 when read
     }
     a.op[i].starts = plan->tables + plan->offStarts[i];
     a.op[i].index = plan->tables + plan->offIndex[i];

@@ -853,6 +853,14 @@ class Tile:
             if len(args) > 1:
                 kw["axis"] = args[1]
             return getattr(Tile.wrap(args[0]), name)(**kw)
+        if name == "where" and len(args) == 3:
+            # numpy.where converts its arguments to plain arrays (the values, whatever
+            # their activity) and returns one
+            c, a, b = (Tile.wrap(v) for v in args)
+            if c.dtype_name != "bool":
+                raise TraceError("numpy.where: the condition must be a comparison of tiles")
+            shape = _broadcast(_broadcast(c.shape, a.shape), b.shape)
+            return Tile("where", (c, a, b), shape, _result_dtype(a, b), plain=True, func=True)
         if name == "transpose" and len(args) == 1:
             return Tile.wrap(args[0]).T
         if name == "norm" and kwargs.get("ord", args[1] if len(args) > 1 else None) is None:

@@ -668,15 +668,15 @@ def plan_imap(program, inputs, out, out_bool=False) -> Plan:
 FMAP_OPS = {"in": 1, "const": 2, "add": 3, "sub": 4, "mul": 5, "div": 6, "floordiv": 7, "mod": 8,
             "min": 9, "max": 10, "udiv": 11, "lt": 12, "le": 13, "eq": 14, "ne": 15, "ge": 16,
             "gt": 17, "neg": 18, "abs": 19, "sqrt": 20, "rint": 21, "exp": 22, "log": 23, "r16": 24,
-            "psqrt": 25, "powchk": 26, "active": 27}
+            "psqrt": 25, "powchk": 26, "active": 27, "tanh": 28, "select": 29}
 FMAP_MAX_INSTRS = 48
 
 
 def plan_fmap(program, inputs, out, types, store_all=False) -> Plan:
     """out = f(inputs...) over fp32 / fp16 windows with numpy.ma's activity rules
     (see hcamdLaunchFMap).  `program` is a postfix list of (opname, arg, float
-    immediate); `types` lists F32 / F16 for the inputs followed by F32, F16 or
-    U8 (a one-byte-per-element array that receives 0 / 1) for the output;
+    immediate); `types` lists F32 / F16 / I32 (converted when read) for the inputs
+    followed by F32, F16 or U8 (a one-byte-per-element array that receives 0 / 1) for the output;
     store_all writes inactive elements too."""
     inputs = list(inputs)
     ctx = _ctx_of(*inputs, out)
@@ -686,7 +686,7 @@ def plan_fmap(program, inputs, out, types, store_all=False) -> Plan:
     ms = []
     for x, ty in zip(inputs, types):
         m = as_memref(x)
-        _expect(m, {F32: 4, F16: 2}[ty], "fmap operand")
+        _expect(m, {F32: 4, F16: 2, I32: 4}[ty], "fmap operand")
         r, c, _ = _rows_cols(m)
         if (r, c) != (rows, cols):
             raise HcRuntimeError("fmap: shape mismatch")

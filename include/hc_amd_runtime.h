@@ -407,7 +407,8 @@ int hcamdLaunchIMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
  *                the second (`arg` bit 0, fp16 tiles: the first, as NumPy's half
  *                loops do)
  *   the rest     computed from the values, activity kept; comparisons give 0 / 1
- * Every rounding to fp16 other than DIV / FLOORDIV's is an explicit
+ * An operand of type HCAMD_I32 is converted to fp32 when it is read (a tile's
+ * astype(float32)).  Every rounding to fp16 other than DIV / FLOORDIV's is an explicit
  * HCAMD_FMAP_R16.  outType is HCAMD_F32, HCAMD_F16, or HCAMD_U8 (one byte of
  * 0 / 1, a bool buffer).  Inactive elements are not stored, unless storeAll is
  * set: a NumPy function returns a bare numpy.ma array, which the reference's
@@ -424,7 +425,12 @@ enum HcamdFMapOp {
   HCAMD_FMAP_EXP = 22, HCAMD_FMAP_LOG = 23, HCAMD_FMAP_R16 = 24, HCAMD_FMAP_PSQRT = 25,
   HCAMD_FMAP_POWCHK = 26,
   HCAMD_FMAP_ACTIVE = 27, /* top = 1 where the element is active in it, else 0; active again (`tile.mask`) */
-  HCAMD_FMAP_COUNT = 28
+  HCAMD_FMAP_TANH = 28,
+  /* numpy.where(c, a, b) with c, a, b the three top entries (b on top): the
+   * values are taken whatever their activity and the result is active, a plain
+   * array as NumPy returns one */
+  HCAMD_FMAP_SELECT = 29,
+  HCAMD_FMAP_COUNT = 30
 };
 int hcamdLaunchFMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
                     const void *const *inputs, const int *inputTypes, const size_t *inputLd,

@@ -534,6 +534,74 @@ def case_masked_reductions(api):
     return rec.out
 
 
+def case_shapes_and_selections(api):
+    """What a store writes for tiles whose shape was changed on the way (a
+    transposed tile, a row vector and a per-row operand broadcast over a 2-D
+    tile, a matrix times a vector), for numpy.where and numpy.tanh of tiles, for
+    an int32 tile converted with astype, and for one result per group assigned
+    to a buffer element; loads reach past their arrays, divisors hold zeros."""
+    rec = Recorder()
+    f = np.float32
+    rng = np.random.default_rng(13)
+    x = rng.integers(-4, 5, (5, 6)).astype(f)
+    y = rng.integers(-2, 3, (5, 6)).astype(f)
+    row = rng.integers(-2, 3, 6).astype(f)
+    col = rng.integers(-2, 3, 5).astype(f)
+    xi = rng.integers(-9, 10, (5, 6)).astype(np.int32)
+    vec = rng.integers(-3, 4, 6).astype(f)
+    forms = {
+        "where_of_tiles": lambda a, b, r, c, ai: np.where(a > b, a, b),
+        "where_with_numbers": lambda a, b, r, c, ai: np.where(a * b >= f(0), a, f(-1)),
+        "where_of_quotient": lambda a, b, r, c, ai: np.where(b != f(0), a / b, f(9)),
+        "tanh_of_quotient": lambda a, b, r, c, ai: np.tanh(a / b),
+        "tanh_times_tile": lambda a, b, r, c, ai: a * np.tanh(b),
+        "row_vector": lambda a, b, r, c, ai: a + r,
+        "col_vector": lambda a, b, r, c, ai: a * c[:, None],
+        "both_vectors": lambda a, b, r, c, ai: (a + r) / c[:, None],
+        "vector_first": lambda a, b, r, c, ai: r / a,
+        "int_astype": lambda a, b, r, c, ai: ai.astype(f) * f(0.5),
+        "int_astype_plus_tile": lambda a, b, r, c, ai: a + ai.astype(f),
+    }
+    dst = np.full((len(forms), 7, 7), POISON, f)
+    dst_t = np.full((2, 8, 7), POISON, f)              # taller than the transposed tile's active part
+    dst_v = np.full((2, 7), POISON, f)
+    cells = np.full(6, POISON, f)
+
+    def body(gr, x, y, row, col, xi, vec, dst, dst_t, dst_v, cells):
+        for i, (name, fn) in enumerate(forms.items()):
+            a, b = gr.load(x, shape=(7, 8)), gr.load(y, shape=(7, 8))
+            r, c = gr.load(row, shape=8), gr.load(col, shape=7)
+            ai = gr.load(xi, shape=(7, 8))
+            t = rec.attempt(name, lambda: fn(a, b, r, c, ai))
+            if t is not None:
+                gr.store(dst[i], t)
+        a = gr.load(x, shape=(7, 8))
+        t = rec.attempt("transposed", lambda: a.T)
+        if t is not None:
+            gr.store(dst_t[0], t)
+        t = rec.attempt("transposed_sum", lambda: a.T + gr.load(y, shape=(7, 8)).T)
+        if t is not None:
+            gr.store(dst_t[1], t)
+        v = gr.load(vec, shape=8)
+        t = rec.attempt("matrix_times_vector", lambda: np.dot(a, v))
+        if t is not None:
+            gr.store(dst_v[0], t)
+        t = rec.attempt("rows_sum_of_products", lambda: (a * v).sum(axis=1))
+        if t is not None:
+            gr.store(dst_v[1], t)
+        cells[gr.id[0] + 1] = (a * a).sum()
+        cells[gr.id[0] + 3] += a.max() - a.min()
+
+    with np.errstate(all="ignore"), warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        _one_group(api, body, x, y, row, col, xi, vec, dst, dst_t, dst_v, cells)
+    rec.array("dst", dst)
+    rec.array("dst_transposed", dst_t)
+    rec.array("dst_vectors", dst_v)
+    rec.array("cells", cells)
+    return rec.out
+
+
 CASES = {
     "masked_reductions": case_masked_reductions,
     "inplace_partial": case_inplace_partial,
@@ -545,6 +613,7 @@ CASES = {
     "operators": case_operators,
     "store_forms": case_store_forms,
     "float_activity": case_float_activity,
+    "shapes_and_selections": case_shapes_and_selections,
 }
 
 

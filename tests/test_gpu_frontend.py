@@ -1338,6 +1338,62 @@ def test_matrix_times_vector_is_a_row_sum_of_products(rows, k):
     assert_allclose(out.to_host(), a.astype(np.float64) @ v.astype(np.float64), atol=float(bound.max()))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_selections_conversions_and_tanh_match_the_simulator(dtype):
+    """numpy.where of tiles (a plain array chosen from the values, whatever their
+    activity), numpy.tanh next to operations that deactivate, and an int32 tile
+    converted with astype inside a float expression: the simulator's bytes,
+    elements it leaves alone included (tanh to 1.5 ulp)."""
+    M, N = sym.M, sym.N
+    f = dtype
+    forms = {
+        "where_of_tiles": lambda a, b, ai: np.where(a > b, a, b),
+        "where_with_numbers": lambda a, b, ai: np.where(a * b >= f(0), a, f(-1)),
+        "where_of_quotient": lambda a, b, ai: np.where(b != f(0), a / b, f(9)),
+        "where_nested": lambda a, b, ai: np.where(a < b, np.where(a < f(0), -a, a), b * f(2)),
+        "tanh_of_quotient": lambda a, b, ai: np.tanh(a / b),
+        "tanh_times_tile": lambda a, b, ai: a * np.tanh(b),
+        "tanh_and_domain": lambda a, b, ai: np.sqrt(np.abs(a)) + np.tanh(b) - np.square(a),
+    }
+    if dtype == np.float32:
+        forms.update({"int_astype": lambda a, b, ai: ai.astype(f) * f(0.5),
+                      "int_astype_plus_tile": lambda a, b, ai: a + ai.astype(f),
+                      "int_in_where": lambda a, b, ai: np.where(ai.astype(f) > a, b, ai.astype(f))})
+
+    def make(deco, fn):
+        @deco(work_shape=(M, N), group_shape=(8, 32))
+        def body(gr: CurrentGroup, x: Buffer[M, N, DT], y: Buffer[M, N, DT], xi: Buffer[M, N, DT],
+                 out: Buffer[M, N, DT]):
+            i, j = gr.work_offset
+            a, b = gr.load(x[i:, j:], shape=gr.shape), gr.load(y[i:, j:], shape=gr.shape)
+            gr.store(out[i:, j:], fn(a, b, gr.load(xi[i:, j:], shape=gr.shape)))
+        return body
+
+    rng = np.random.default_rng(31)
+    rows, cols = 37, 50
+    x = (rng.integers(-8, 9, (rows, cols)) / 4).astype(dtype)
+    y = (rng.integers(-3, 4, (rows, cols)) / 2).astype(dtype)          # zeros among the divisors
+    x[3, 4], y[5, 6], x[7, 7] = np.inf, np.nan, -0.0
+    xi = rng.integers(-9, 10, (rows, cols)).astype(np.int32)
+    bits = {2: np.uint16, 4: np.uint32}[np.dtype(dtype).itemsize]
+    for name, fn in forms.items():
+        want = np.full((rows, cols), 7, dtype)
+        with np.errstate(all="ignore"):
+            make(sim_kernel, fn)(x, y, xi, want)
+        out = rt.to_device(np.full((rows, cols), 7, dtype))
+        make(kernel, fn)(rt.to_device(x), rt.to_device(y), rt.to_device(xi), out)
+        got = out.to_host()
+        if "tanh" in name:
+            assert_array_equal(got == 7, want == 7, err_msg=name)
+            assert_array_equal(np.isnan(got), np.isnan(want), err_msg=name)
+            ok = ~np.isnan(want)
+            assert_allclose(got[ok].astype(np.float64), want[ok].astype(np.float64),
+                            rtol=1.1e-3 if dtype == np.float16 else 4e-7,
+                            atol=0 if dtype == np.float16 else 5e-7, err_msg=name)   # (sums of terms near +-2)
+        else:
+            assert_array_equal(got.view(bits), want.view(bits), err_msg=name)
+
+
 def test_tile_mask_is_stored_as_a_plain_bool_array():
     """`tile.mask` (python/hckernel/kernel_api.py:117-119: True = active) of
     float and int32 expressions that the data deactivates here and there: the

@@ -421,6 +421,51 @@ def _ma_special(rng, n, dtype):
     return x
 
 
+def test_fmap_select_tanh_and_int32_operands(ctx):
+    """hcamdLaunchFMap: SELECT takes its values whatever their activity and gives an
+    active result (numpy.where returns a plain array), an int32 operand is
+    converted when it is read, TANH keeps the activity; a ragged 2-D window, the
+    rest of the output untouched."""
+    rng = np.random.default_rng(99)
+    rows, cols, ld = 13, 1001, 1010
+    a = rng.standard_normal((rows, ld)).astype(np.float32)
+    b = rng.integers(-2, 3, (rows, ld)).astype(np.float32)
+    k = rng.integers(-(2 ** 31), 2 ** 31 - 1, (rows, ld), dtype=np.int64).astype(np.int32)
+    F = lambda name, arg=0, imm=0.0: (name, arg, imm)
+    da, db, dk = dev(a), dev(b), dev(k)
+    win = lambda d: _View(d, (rows, cols), 0, (ld, 1))
+    # where(b != 0, a / b, float(k)): the quotient's deactivated elements are not taken anyway
+    prog = [F("in", 1), F("const", 0, 0.0), F("ne"), F("in", 0), F("in", 1), F("div"), F("in", 2), F("select")]
+    out = poisoned((rows, ld), np.float32)
+    rt.plan_fmap(prog, [win(da), win(db), win(dk)], win(out), [rt.F32, rt.F32, rt.I32, rt.F32]).launch()
+    got = out.to_host()
+    with np.errstate(all="ignore"):
+        want = np.where(b != 0, a / b, k.astype(np.float32))
+    assert_array_equal(got[:, :cols].view(np.uint32), want[:, :cols].view(np.uint32))
+    assert (got[:, cols:].view(np.uint32) == POISON32).all()
+    # where(a / b > 0, 1, 2) on a deactivated condition: NumPy sees the value numpy.ma left (the dividend)
+    prog = [F("in", 0), F("in", 1), F("div"), F("const", 0, 0.0), F("gt"), F("const", 0, 1.0), F("const", 0, 2.0),
+            F("select")]
+    out = poisoned((rows, ld), np.float32)
+    rt.plan_fmap(prog, [win(da), win(db)], win(out), [rt.F32, rt.F32, rt.F32]).launch()
+    import numpy.ma as ma
+    with np.errstate(all="ignore"):
+        q = ma.array(a) / ma.array(b)
+        want = np.where(np.asarray(q > 0), np.float32(1), np.float32(2))
+    assert_array_equal(out.to_host()[:, :cols], want[:, :cols])
+    # tanh(a / b): deactivated elements are not stored
+    prog = [F("in", 0), F("in", 1), F("div"), F("tanh")]
+    out = poisoned((rows, ld), np.float32)
+    rt.plan_fmap(prog, [win(da), win(db)], win(out), [rt.F32, rt.F32, rt.F32]).launch()
+    got = out.to_host()[:, :cols]
+    live = b[:, :cols] != 0
+    assert (got[~live].view(np.uint32) == POISON32).all()
+    assert_allclose(got[live], np.tanh(a[:, :cols][live] / b[:, :cols][live]), rtol=4e-7, atol=1e-7)
+    # a program that pops more than the stack holds is refused
+    with pytest.raises(rt.HcRuntimeError, match="underflow"):
+        rt.plan_fmap([F("in", 0), F("in", 1), F("select")], [win(da), win(db)], win(out), [rt.F32, rt.F32, rt.F32]).launch()
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 def test_fmap_every_operation_against_numpy_ma(ctx, dtype):
     """hcamdLaunchFMap, one program per opcode, against numpy.ma itself on data full
