@@ -738,7 +738,7 @@ def _masks(t: Tile) -> bool:
     if t.op == "vardiv":
         return not _const(t.args[1])
     if t.attrs.get("func"):
-        return t.op in ("sqrt", "log", "div", "floordiv", "mod")
+        return t.op in ("sqrt", "log", "log2", "log10", "div", "floordiv", "mod")
     return t.op in ("div", "floordiv", "mod") or bool(t.attrs.get("pow"))
 
 
@@ -1172,7 +1172,9 @@ _FMAP_BINARY = {"add": "add", "sub": "sub", "mul": "mul", "div": "div", "floordi
                 "mod": "mod", "maximum": "max", "minimum": "min", "lt": "lt", "le": "le", "eq": "eq",
                 "ne": "ne", "ge": "ge", "gt": "gt"}
 _FMAP_UNARY = {"neg": "neg", "abs": "abs", "sqrt": "sqrt", "rint": "rint", "exp": "exp", "log": "log",
-               "tanh": "tanh"}
+               "tanh": "tanh", "floor": "floor", "ceil": "ceil", "trunc": "trunc", "sign": "sign",
+               "exp2": "exp2", "log2": "log2", "log10": "log10", "log1p": "log1p", "expm1": "expm1",
+               "sin": "sin", "cos": "cos", "reciprocal": "reciprocal"}
 _FMAP_MIRROR = {"add": "add", "mul": "mul", "max": "max", "min": "min", "eq": "eq", "ne": "ne",
                 "lt": "gt", "gt": "lt", "le": "ge", "ge": "le"}
 _FMAP_COMPARE = ("lt", "le", "eq", "ne", "ge", "gt")

@@ -62,6 +62,10 @@ enum : uint32_t {
   // numpy.where(c, a, b) with c, a, b the three top entries (b on top): NumPy takes the
   // values whatever their activity and returns a plain array, so the result is active
   FOP_SELECT = 29,
+  // more NumPy functions of one operand: computed from the values, activity kept;
+  // log2 and log10 have numpy.ma's domain like log (inactive with the value 1)
+  FOP_FLOOR = 30, FOP_CEIL = 31, FOP_TRUNC = 32, FOP_SIGN = 33, FOP_EXP2 = 34, FOP_LOG2 = 35,
+  FOP_LOG10 = 36, FOP_LOG1P = 37, FOP_EXPM1 = 38, FOP_SIN = 39, FOP_COS = 40, FOP_RECIP = 41,
 };
 
 struct Instr {
@@ -189,7 +193,25 @@ __device__ __forceinline__ float unary(uint32_t op, float a, bool &ok) {
       return 1.0f;
     }
     return logf(a);
+  case FOP_LOG2:
+  case FOP_LOG10:
+    if (!ok || a <= 0.0f) {
+      ok = false;
+      return 1.0f;
+    }
+    return op == FOP_LOG2 ? log2f(a) : log10f(a);
   case FOP_RINT: return __builtin_rintf(a);
+  case FOP_FLOOR: return __builtin_floorf(a);
+  case FOP_CEIL: return __builtin_ceilf(a);
+  case FOP_TRUNC: return __builtin_truncf(a);
+  // numpy.sign: -1, 0 (the operand's zero is not kept: +0), 1, NaN for NaN
+  case FOP_SIGN: return a > 0.0f ? 1.0f : a < 0.0f ? -1.0f : a == 0.0f ? 0.0f : a;
+  case FOP_EXP2: return exp2f(a);
+  case FOP_LOG1P: return log1pf(a);
+  case FOP_EXPM1: return expm1f(a);
+  case FOP_SIN: return sinf(a);
+  case FOP_COS: return cosf(a);
+  case FOP_RECIP: return 1.0f / a;
   case FOP_EXP: return expf(a);
   case FOP_TANH: return tanh_selects(a);
   case FOP_R16: return round16(a);

@@ -635,7 +635,10 @@ _UFUNC_OPS = {"floor_divide": "floordiv", "remainder": "mod", "mod": "mod", "bit
               "add": "add", "subtract": "sub", "multiply": "mul", "true_divide": "div",
               "divide": "div", "exp": "exp", "absolute": "abs", "fabs": "abs", "rint": "rint",
               "negative": "neg", "maximum": "maximum", "minimum": "minimum", "sqrt": "sqrt",
-              "log": "log", "tanh": "tanh", "square": "square", "power": "power"}
+              "log": "log", "tanh": "tanh", "square": "square", "power": "power",
+              "floor": "floor", "ceil": "ceil", "trunc": "trunc", "sign": "sign", "exp2": "exp2",
+              "log2": "log2", "log10": "log10", "log1p": "log1p", "expm1": "expm1", "sin": "sin",
+              "cos": "cos", "reciprocal": "reciprocal"}
 
 
 def _result_dtype(a: "Tile", b: "Tile") -> str:

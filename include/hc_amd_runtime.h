@@ -430,7 +430,12 @@ enum HcamdFMapOp {
    * values are taken whatever their activity and the result is active, a plain
    * array as NumPy returns one */
   HCAMD_FMAP_SELECT = 29,
-  HCAMD_FMAP_COUNT = 30
+  /* more NumPy functions of one operand, computed from the values with the
+   * activity kept; LOG2 and LOG10 have numpy.ma's domain like LOG */
+  HCAMD_FMAP_FLOOR = 30, HCAMD_FMAP_CEIL = 31, HCAMD_FMAP_TRUNC = 32, HCAMD_FMAP_SIGN = 33,
+  HCAMD_FMAP_EXP2 = 34, HCAMD_FMAP_LOG2 = 35, HCAMD_FMAP_LOG10 = 36, HCAMD_FMAP_LOG1P = 37,
+  HCAMD_FMAP_EXPM1 = 38, HCAMD_FMAP_SIN = 39, HCAMD_FMAP_COS = 40, HCAMD_FMAP_RECIP = 41,
+  HCAMD_FMAP_COUNT = 42
 };
 int hcamdLaunchFMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
                     const void *const *inputs, const int *inputTypes, const size_t *inputLd,

@@ -602,6 +602,35 @@ def case_shapes_and_selections(api):
     return rec.out
 
 
+def case_more_functions(api):
+    """NumPy functions of one operand on tiles, on values and on quotients with
+    deactivated elements: what numpy.ma gives (the function of the values, the
+    activity kept; its fill value where a domain fails) and what a store writes."""
+    rec = Recorder()
+    f = np.float32
+    x = np.array([[-2.5, -1.0, -0.5, -0.0, 0.0, 0.5, 1.0, 2.5], [3.75, -3.25, 100.0, -100.0, 1e-3, -1e-3, 7.0, -7.0]], f)
+    y = np.array([[1.0, 0.0, 2.0, 0.0, -1.0, 4.0, 0.0, 0.5], [2.0, -2.0, 0.0, 8.0, 0.0, 1.0, -0.5, 0.0]], f)
+    names = ["floor", "ceil", "trunc", "sign", "exp2", "log2", "log10", "log1p", "expm1", "sin", "cos", "reciprocal"]
+    dst = np.full((2 * len(names), 3, 9), POISON, f)
+
+    def body(gr, x, y, dst):
+        for i, name in enumerate(names):
+            fn = getattr(np, name)
+            a, b = gr.load(x, shape=(3, 9)), gr.load(y, shape=(3, 9))
+            t = rec.attempt(name + "_of_tile", lambda: fn(a))
+            if t is not None:
+                gr.store(dst[2 * i], t)
+            t = rec.attempt(name + "_of_quotient", lambda: fn(a / b) + a)
+            if t is not None:
+                gr.store(dst[2 * i + 1], t)
+
+    with np.errstate(all="ignore"), warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        _one_group(api, body, x, y, dst)
+    rec.array("dst", dst)
+    return rec.out
+
+
 CASES = {
     "masked_reductions": case_masked_reductions,
     "inplace_partial": case_inplace_partial,
@@ -614,6 +643,7 @@ CASES = {
     "store_forms": case_store_forms,
     "float_activity": case_float_activity,
     "shapes_and_selections": case_shapes_and_selections,
+    "more_functions": case_more_functions,
 }
 
 

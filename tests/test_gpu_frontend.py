@@ -1394,6 +1394,55 @@ def test_selections_conversions_and_tanh_match_the_simulator(dtype):
             assert_array_equal(got.view(bits), want.view(bits), err_msg=name)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_more_numpy_functions_of_tiles(dtype):
+    """floor, ceil, trunc, sign, exp2, log2, log10, log1p, expm1, sin, cos and
+    reciprocal of tiles and of quotients with deactivated elements, through the
+    general float map: the same elements written as the simulator writes (numpy.ma
+    keeps the activity, log2 / log10 have its domain), exact functions bit for
+    bit, the others to a few units in the last place."""
+    N = sym.N
+    exact = ("floor", "ceil", "trunc", "sign", "reciprocal")
+    names = exact + ("exp2", "log2", "log10", "log1p", "expm1", "sin", "cos")
+
+    def make(deco, fn, quotient):
+        @deco(work_shape=N, group_shape=256)
+        def body(gr: CurrentGroup, x: Buffer[N, DT], y: Buffer[N, DT], out: Buffer[N, DT]):
+            o = gr.work_offset[0]
+            a, b = gr.load(x[o:], shape=gr.shape), gr.load(y[o:], shape=gr.shape)
+            gr.store(out[o:], a + fn(a / b) if quotient else fn(a))      # (a tile on the left: a tile again)
+        return body
+
+    rng = np.random.default_rng(17)
+    n = 3001
+    x = (rng.integers(-40, 41, n) / 8).astype(dtype)
+    y = (rng.integers(-2, 3, n) / 2).astype(dtype)
+    x[:6] = [np.inf, -np.inf, np.nan, 0.0, -0.0, 1.0]
+    y[:6] = [1.0, 2.0, 1.0, 1.0, 1.0, 0.0]
+    bits = {2: np.uint16, 4: np.uint32}[np.dtype(dtype).itemsize]
+    for name in names:
+        for quotient in (False, True):
+            fn = getattr(np, name)
+            want = np.full(n, 7, dtype)
+            with np.errstate(all="ignore"):
+                make(sim_kernel, fn, quotient)(x, y, want)
+            out = rt.to_device(np.full(n, 7, dtype))
+            make(kernel, fn, quotient)(rt.to_device(x), rt.to_device(y), out)
+            assert rt.last_kernel_name() == "hcamd_fmap", name
+            got = out.to_host()
+            tag = f"{name} quotient={quotient}"
+            if name in exact:
+                assert_array_equal(got.view(bits), want.view(bits), err_msg=tag)
+            else:
+                assert_array_equal(np.isnan(got), np.isnan(want), err_msg=tag)
+                ok = ~np.isnan(want)
+                assert_allclose(got[ok].astype(np.float64), want[ok].astype(np.float64),
+                                rtol=2e-3 if dtype == np.float16 else 1e-6,
+                                atol=2e-3 if dtype == np.float16 else 1e-6, err_msg=tag)
+            if quotient:
+                assert ((want == 7) & (y == 0)).sum() > 100, tag          # deactivated quotients are left alone
+
+
 def test_tile_mask_is_stored_as_a_plain_bool_array():
     """`tile.mask` (python/hckernel/kernel_api.py:117-119: True = active) of
     float and int32 expressions that the data deactivates here and there: the
