@@ -631,6 +631,45 @@ def case_more_functions(api):
     return rec.out
 
 
+def case_numpy_scalar_on_the_left(api):
+    """`numpy.float32(2) / tile` and the like: the tile type has no reflected
+    operators, so the NumPy scalar's own operator decides what happens."""
+    rec = Recorder()
+    f = np.float32
+    x = np.array([1.0, 0.0, -0.0, np.inf, np.nan, 4.0, -2.0, 0.5], f)
+    y = np.array([2.0, 0.0, 1.0, 1.0, 1.0, 0.0, 0.0, -1.0], f)
+    forms = {
+        "div": lambda a, b: f(2.0) / a,
+        "mul": lambda a, b: f(2.0) * a,
+        "sub": lambda a, b: f(2.0) - a,
+        "add": lambda a, b: f(1.0) + a,
+        "floordiv": lambda a, b: f(2.0) // a,
+        "mod": lambda a, b: f(2.0) % a,
+        "pow": lambda a, b: f(2.0) ** a,
+        "lt": lambda a, b: f(1.0) < a,
+        "div_quotient": lambda a, b: f(2.0) / (a / b),
+        "mul_quotient": lambda a, b: f(2.0) * (a / b),
+        "add_quotient_then_tile": lambda a, b: (f(1.0) + (a / b)) * a,
+        "div_then_tile_op": lambda a, b: (f(2.0) / a) + a,
+        "tile_then_div": lambda a, b: a + (f(2.0) / a),
+    }
+    dst = np.full((len(forms), 8), POISON, f)
+    dstb = np.full(8, True)
+
+    def body(gr, x, y, dst, dstb):
+        for i, (name, fn) in enumerate(forms.items()):
+            a, b = gr.load(x[:7], shape=8), gr.load(y[:7], shape=8)
+            t = rec.attempt(name, lambda: fn(a, b))
+            if t is not None:
+                gr.store(dstb if name == "lt" else dst[i], t)
+
+    with np.errstate(all="ignore"), warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        _one_group(api, body, x, y, dst, dstb)
+    rec.array("dst_bool", dstb)          # (the arithmetic forms raise in the reference: nothing to compare)
+    return rec.out
+
+
 CASES = {
     "masked_reductions": case_masked_reductions,
     "inplace_partial": case_inplace_partial,
@@ -644,6 +683,7 @@ CASES = {
     "float_activity": case_float_activity,
     "shapes_and_selections": case_shapes_and_selections,
     "more_functions": case_more_functions,
+    "numpy_scalar_on_the_left": case_numpy_scalar_on_the_left,
 }
 
 

@@ -35,12 +35,14 @@ GOLDEN = os.path.join(HERE, "golden", "sim_golden.json")
 # The reference raises, the oracle returns a value:
 #  * an operand that is not a tile on the left of an operator: the reference
 #    installs no reflected methods (kernel_api.py:185-195), so `2 * tile`
-#    is a TypeError there; the oracle gives the commuted result.
+#    is a TypeError there, and so is `numpy.float32(2) / tile` (every arithmetic
+#    operator of a NumPy scalar; its comparisons are reflected by Python and
+#    work); the oracle gives the commuted result.
 #  * `int_tile ** 2`: numpy.ma returns its scalar "no mask", which the
 #    reference's mask property cannot invert (kernel_api.py:93-103); the oracle
 #    treats it as all active.
 #  * len(tile): no __len__ on the reference's wrapper type.
-ORACLE_DEFINES = ("_left_", "domain_masking/int_pow", "compressed_repr/len")
+ORACLE_DEFINES = ("_left_", "domain_masking/int_pow", "compressed_repr/len", "numpy_scalar_on_the_left/")
 
 
 def _text(a):
