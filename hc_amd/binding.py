@@ -733,6 +733,8 @@ def _masks(t: Tile) -> bool:
     is numpy.ma's too; a variance is inactive where fewer than ddof + 1 elements
     were active; numpy.ma.sqrt (the standard deviation's) deactivates results
     that are not finite."""
+    if t.attrs.get("ieee"):
+        return False                         # plain NumPy arrays: NumPy's own arithmetic
     if t.op == "masqrt":
         return True
     if t.op == "vardiv":
@@ -792,7 +794,7 @@ def _values_flow_plainly(t: Tile, clean: bool = True, finite: bool = False) -> b
         return clean or not _can_fail(t, finite)
     if (_fails_on_finite_data(t) if finite else _masks(t)) and not clean:
         return False
-    transparent = _is(t, "astype", 1) or t.op in ("neg", "abs") or \
+    transparent = _is(t, "astype", 1) or t.op in ("neg", "abs") or bool(t.attrs.get("ieee")) or \
         (bool(t.attrs.get("func")) and t.op in _TRANSPARENT_FUNCS)
     return all(_values_flow_plainly(a, clean and transparent, finite) for a in t.args if isinstance(a, Tile))
 
@@ -885,10 +887,31 @@ class _MapCompiler:
                 # (+0 and -0), the fp32 ones, which this kernel has, the second:
                 # the general float map has both
                 return False
-            return all(self.supported(a) and (_const(a) or a.shape == t.shape) for a in t.args)
+            if not all(self.supported(a) and (_const(a) or a.shape == t.shape) for a in t.args):
+                return False
+            # of two equal values (+0 and -0) NumPy's maximum / minimum return the second:
+            # the operands must reach the kernel in the order they were written
+            return t.op not in ("maximum", "minimum") or self._keeps_order(t)
         if _is(t, "vardiv", 2):                  # a variance whose count is a number
             return _const(t.args[1]) and self.supported(t.args[0])
         return False
+
+    def _keeps_order(self, t: Tile) -> bool:
+        """emit() hands t's operands to the kernel in the order they were written
+        (it evaluates the deeper side first and has operand and immediate forms
+        that take the running value as the first operand)."""
+        a, b = t.args
+        if self._scalar_mode or self._frozen:
+            return True                               # (those stages say which operand came first)
+        if _const(b):
+            return True
+        if _const(a):
+            return a.attrs.get("value") != 0          # only zeros of two signs are equal and differ
+        if _leaf(b) is not None:
+            return True
+        if _leaf(a) is not None:
+            return False
+        return self.need(a) >= self.need(b)
 
     def need(self, t: Tile) -> int:
         if t.uid in self.need_cache:
@@ -913,6 +936,8 @@ class _MapCompiler:
         self._emit_node(t, out)
         if self.masked and t.attrs.get("pow"):
             out.append(("powchk", 0, 0.0))
+            if t.dtype_name == "float16":
+                out.append(("r16", 0, 0.0))        # numpy.ma's fill value 1e20 is infinite as fp16
 
     def emit_whole(self, t: Tile, out: list):
         """The program of a whole expression where no other kernel can take
@@ -948,13 +973,13 @@ class _MapCompiler:
             self.emit(t.args[0], out)
             out.append(("divi", 0, _round_to(t.args[1].attrs["value"], t.dtype_name)))
             return
-        mdiv = self.masked and t.op == "div"
+        mdiv = self.masked and t.op == "div" and not t.attrs.get("ieee")
         if mdiv and t.attrs.get("func"):
             raise _NeedsEntryMasks()           # numpy.divide as a function: the general map has it
         if t.op in _MAP_UNARY:
             self.emit(t.args[0], out)
             name = _MAP_UNARY[t.op]
-            if self.masked and t.attrs.get("func") and name in ("sqrt", "log"):
+            if self.masked and t.attrs.get("func") and name in ("sqrt", "log") and not t.attrs.get("ieee"):
                 name = "m" + name              # numpy.sqrt / numpy.log of a tile: domain fill
             if name == "masqrt" and not self.masked:
                 name = "sqrt"                  # stored in full: the same values
@@ -1120,6 +1145,10 @@ def match_imap(dst_view, value, n_groups):
             if t.attrs.get("operand_dtype", t.dtype_name) != "int32":
                 return False
             op = _IMAP_BINARY[t.op]
+            if t.attrs.get("right_values") and _maybe_masked(b):
+                raise NoNativeKernel("a NumPy function's result on the left of % & | ^ << >> sees the values "
+                                     "of the tile on the right, whatever their activity: no native code for "
+                                     "integer tiles that can be inactive")
             if op in mirrored and need(b) > need(a):
                 a, b, op = b, a, mirrored[op]
             ok = emit(a) and emit(b)
@@ -1203,6 +1232,8 @@ def _compile_fmap(value, mapped=False):
             n = 1
         elif _is(t, "where", 3):
             n = max(need(t.args[0]), 1 + need(t.args[1]), 2 + need(t.args[2]))
+        elif _is(t, "clip", 1):
+            n = max(need(t.args[0]), 2)          # the bounds are pushed next to the value
         elif len(t.args) == 1:
             n = need(t.args[0])
         elif len(t.args) == 2:
@@ -1220,6 +1251,7 @@ def _compile_fmap(value, mapped=False):
         """Appends the code for t; False if t is not a float expression this kernel takes."""
         half = t.dtype_name == "float16"
         func = bool(t.attrs.get("func"))
+        plain_numpy = 4 if t.attrs.get("ieee") else 0      # operands are plain arrays: NumPy's own arithmetic
         if int_leaf(t) is not None:
             t = int_leaf(t)
         if _is(t, "load") or (mapped and _is(t, "mapped_load")):
@@ -1272,7 +1304,7 @@ def _compile_fmap(value, mapped=False):
                 name = "psqrt"                 # x ** 0.5; numpy.sqrt(x) has a domain instead
             elif name in ("sqrt", "log") and not func:
                 return False
-            program.append((name, 0, 0.0))
+            program.append((name, plain_numpy, 0.0))
             if half and t.op not in _MAP_EXACT:
                 program.append(("r16", 0, 0.0))
         elif t.op in _FMAP_BINARY and len(t.args) == 2:
@@ -1280,37 +1312,45 @@ def _compile_fmap(value, mapped=False):
             if dt not in _MAP_FLOATS:
                 return False
             op = _FMAP_BINARY[t.op]
-            if func and op == "floordiv":
+            if func and op == "floordiv" and not plain_numpy:
                 raise NoNativeKernel("numpy.floor_divide called as a function has no native code "
                                      "(the // operator has)")
             a, b = t.args
             # (operands are only exchanged where no element can be inactive: the first
             # operand's value is what numpy.ma leaves in a deactivated result)
+            swapped = 0
             if op in _FMAP_MIRROR and not mapped and not _maybe_masked(t, memo) and need(b) > need(a):
                 a, b, op = b, a, _FMAP_MIRROR[op]
+                swapped = 8                    # which of two equal values min / max return depends on the order
             for x in (a, b):
                 if _const(x):
                     program.append(("const", 0, _round_to(x.attrs["value"], dt)))
                 else:
                     ok = emit(x) and ok
             half_op = dt == "float16"
-            if op == "div" and func:
+            # a bare numpy.ma array % tile: the tile's values, whatever their activity
+            values_only = 16 if t.attrs.get("right_values") else 0
+            if plain_numpy and op in ("div", "floordiv", "mod"):
+                program.append((op, plain_numpy, 0.0))
+            elif op == "div" and func:
                 program.append(("udiv", 0, 0.0))
             elif op in ("div", "floordiv"):
                 program.append((op, int(half_op), 0.0))
             elif op in ("add", "sub", "mul"):
                 program.append((op, 2 if func else 0, 0.0))
             elif op in ("min", "max"):
-                program.append((op, int(half_op), 0.0))
+                program.append((op, int(half_op) | swapped, 0.0))
             else:
-                program.append((op, 0, 0.0))
+                program.append((op, values_only | (2 if func else 0), 0.0))
             if half_op and t.op not in _MAP_EXACT and t.op not in _FMAP_COMPARE and \
-                    not (op in ("div", "floordiv") and not func):
+                    not (op in ("div", "floordiv") and not func and not plain_numpy):
                 program.append(("r16", 0, 0.0))
         else:
             return False
         if t.attrs.get("pow"):
             program.append(("powchk", 0, 0.0))
+            if half:
+                program.append(("r16", 0, 0.0))    # numpy.ma's fill value 1e20 is infinite as fp16
         return ok
 
     if _is(value, "load") or _is(value, "mapped_load") or _const(value):
@@ -1898,7 +1938,7 @@ class _RowCompiler(_MapCompiler):
             a, b = t.args
             sa, sb = self.slot_of(a), self.slot_of(b)
             if sb is not None or sa is not None:
-                mdiv = self.masked and t.op == "div" and not t.attrs.get("func")
+                mdiv = self.masked and t.op == "div" and not t.attrs.get("func") and not t.attrs.get("ieee")
                 if mdiv:
                     fwd, rev = "mdiv", "rmdiv"
                 flag = (0x100 if t.dtype_name == "float16" else 0) if mdiv else 0
@@ -1912,6 +1952,8 @@ class _RowCompiler(_MapCompiler):
                     out.append(("r16", 0, 0.0))
                 if self.masked and t.attrs.get("pow"):
                     out.append(("powchk", 0, 0.0))
+                    if t.dtype_name == "float16":
+                        out.append(("r16", 0, 0.0))
                 return
         super().emit(t, out)
 

@@ -30,11 +30,20 @@
 //   * ** : FOP_PSQRT is the square root of x ** 0.5 (the operand's value where
 //     it is inactive), FOP_POWCHK what numpy.ma.power does afterwards: a result
 //     that is not finite becomes inactive with the value 1e20.
-//   * comparisons give 0 / 1 and are false for NaN except !=.
+//   * comparisons give 0 / 1 and are false for NaN except !=.  Under an inactive
+//     result the tile operators == and != leave 1 / 0 where both operands are
+//     inactive and 0 / 1 where one is (numpy.ma compares the activity there);
+//     `arg` bit 1 (numpy.equal / not_equal called as functions) compares the values.
 //   * FOP_ACTIVE is `tile.mask`: 1 where the element is active, 0 where not, a
 //     plain array (every element active again).  FOP_SELECT is numpy.where: a
 //     plain array too, chosen from the values whatever their activity.
 //   * an int32 operand is converted when it is read (tile.astype(float32)).
+//   * `arg` bit 4 on a binary operation: the second operand's activity does not
+//     count (a bare numpy.ma array % tile, and the other operators numpy.ma does
+//     not define itself: ndarray's operator converts the tile to its values).
+//   * `arg` bit 2: the operands are plain NumPy arrays (what numpy.where, numpy.dot
+//     and tile.mask return, and arithmetic of those), so the operation is NumPy's
+//     own: IEEE quotients, remainders, roots and logarithms, nothing deactivated.
 // The store skips inactive elements, or with store_all writes every value: a
 // NumPy function returns a bare numpy.ma array, which the reference's store
 // copies in full.
@@ -142,8 +151,10 @@ __device__ __forceinline__ bool unsafe_divide(float a, float b) {
 }
 
 // one binary operation; ok comes in as "active in both operands"
-__device__ __forceinline__ float binary(uint32_t op, float a, float b, uint32_t arg, bool &ok) {
+__device__ __forceinline__ float binary(uint32_t op, float a, float b, uint32_t arg, bool &ok,
+                                        bool both_inactive) {
   const bool half = arg & 1u, as_function = arg & 2u;
+  const bool plain = arg & 4u; // plain arrays: NumPy's own arithmetic
   switch (op) {
   case FOP_ADD: return (ok || as_function) ? a + b : a;
   case FOP_SUB: return (ok || as_function) ? a - b : a;
@@ -151,6 +162,8 @@ __device__ __forceinline__ float binary(uint32_t op, float a, float b, uint32_t 
   case FOP_DIV:
   case FOP_FLOORDIV: {
     float r = op == FOP_DIV ? a / b : np_floor_divide(a, b);
+    if (plain)
+      return r;
     if (half)
       r = round16(r);
     if (!ok || b == 0.0f || !finite(r)) {
@@ -161,41 +174,50 @@ __device__ __forceinline__ float binary(uint32_t op, float a, float b, uint32_t 
   }
   case FOP_MOD:
   case FOP_UDIV:
-    if (unsafe_divide(a, b)) {
+    if (!plain && unsafe_divide(a, b)) {
       ok = false;
       return 1.0f;
     }
     return op == FOP_MOD ? np_remainder(a, b) : a / b;
-  // NumPy's half loops keep the first of two equal values, its float loops the second
-  case FOP_MIN: return half ? ((a <= b || a != a) ? a : b) : nan_min(a, b);
-  case FOP_MAX: return half ? ((a >= b || a != a) ? a : b) : nan_max(a, b);
+  // NumPy's half loops keep the first of two equal values, its float loops the
+  // second; `arg` bit 3: the program evaluated the operands in the other order
+  case FOP_MIN:
+  case FOP_MAX: {
+    const float x = (arg & 8u) ? b : a, y = (arg & 8u) ? a : b;
+    if (op == FOP_MIN)
+      return half ? ((x <= y || x != x) ? x : y) : nan_min(x, y);
+    return half ? ((x >= y || x != x) ? x : y) : nan_max(x, y);
+  }
   case FOP_LT: return a < b ? 1.0f : 0.0f;
   case FOP_LE: return a <= b ? 1.0f : 0.0f;
-  case FOP_EQ: return a == b ? 1.0f : 0.0f;
-  case FOP_NE: return a != b ? 1.0f : 0.0f;
+  // numpy.ma's == and != leave "both inactive" / "one inactive" under an
+  // inactive result; numpy.equal / not_equal as functions compare the values
+  case FOP_EQ: return (ok || as_function) ? (a == b ? 1.0f : 0.0f) : (both_inactive ? 1.0f : 0.0f);
+  case FOP_NE: return (ok || as_function) ? (a != b ? 1.0f : 0.0f) : (both_inactive ? 0.0f : 1.0f);
   case FOP_GE: return a >= b ? 1.0f : 0.0f;
   default: return a > b ? 1.0f : 0.0f; // FOP_GT
   }
 }
-__device__ __forceinline__ float unary(uint32_t op, float a, bool &ok) {
+__device__ __forceinline__ float unary(uint32_t op, float a, uint32_t arg, bool &ok) {
+  const bool plain = arg & 4u; // a plain array: NumPy's own function, NaN and infinities included
   switch (op) {
   case FOP_NEG: return -a;
   case FOP_ABS: return __builtin_fabsf(a);
   case FOP_SQRT:
-    if (!ok || a < 0.0f) {
+    if (!plain && (!ok || a < 0.0f)) {
       ok = false;
       return 0.0f;
     }
     return __builtin_sqrtf(a);
   case FOP_LOG:
-    if (!ok || a <= 0.0f) {
+    if (!plain && (!ok || a <= 0.0f)) {
       ok = false;
       return 1.0f;
     }
     return logf(a);
   case FOP_LOG2:
   case FOP_LOG10:
-    if (!ok || a <= 0.0f) {
+    if (!plain && (!ok || a <= 0.0f)) {
       ok = false;
       return 1.0f;
     }
@@ -314,12 +336,13 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_fmap(FMapArgs a) {
     } else if (op >= FOP_NEG) {
 #pragma unroll
       for (int e = 0; e < kV; ++e)
-        t0[e] = unary(op, t0[e], k0[e]);
+        t0[e] = unary(op, t0[e], arg, k0[e]);
     } else {
 #pragma unroll
       for (int e = 0; e < kV; ++e) {
-        bool ok = k1[e] && k0[e];
-        t0[e] = binary(op, t1[e], t0[e], arg, ok);
+        const bool second = k0[e] || (arg & 16u);
+        bool ok = k1[e] && second;
+        t0[e] = binary(op, t1[e], t0[e], arg, ok, !k1[e] && !second);
         k0[e] = ok;
         t1[e] = t2[e];
         t2[e] = t3[e];
@@ -470,10 +493,11 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_gather_fmap(GatherMapArg
       t1 = t3;
       k1 = k3;
     } else if (op >= FOP_NEG) {
-      t0 = unary(op, t0, k0);
+      t0 = unary(op, t0, arg, k0);
     } else {
-      bool ok = k1 && k0;
-      t0 = binary(op, t1, t0, arg, ok);
+      const bool second = k0 || (arg & 16u);
+      bool ok = k1 && second;
+      t0 = binary(op, t1, t0, arg, ok, !k1 && !second);
       k0 = ok;
       t1 = t2, t2 = t3;
       k1 = k2, k2 = k3;

@@ -693,11 +693,26 @@ class Tile:
                         exact=int(x) if isinstance(x, (bool, int, np.integer)) else None)
         raise TraceError(f"cannot use {type(x).__name__} in a tile expression")
 
-    def _binary(self, other, op, reflected=False):
+    def _binary(self, other, op, reflected=False, as_function=False):
         o = Tile.wrap(other)
         a, b = (o, self) if reflected else (self, o)
         r = Tile(op, (a, b), _broadcast(a.shape, b.shape), _result_dtype(a, b))
-        if a.attrs.get("plain") or (a.op == "const" and b.attrs.get("plain")):
+        if _all_ndarrays(a, b):
+            # plain NumPy arrays (numpy.where's result, tile.mask) and numbers:
+            # NumPy's own arithmetic, IEEE results, another plain array
+            r.attrs.update(plain=True, ndarray=True, ieee=True)
+        elif a.attrs.get("ndarray") and not b.attrs.get("plain") and not as_function:
+            # NumPy defers to the tile, whose type has no reflected operators
+            # (python/hckernel/kernel_api.py:158-206)
+            raise TypeError(f"unsupported operand type(s) for {op}: a plain NumPy array (the result of "
+                            f"numpy.where or tile.mask) and a tile; write the tile first")
+        elif a.attrs.get("plain") or (a.op == "const" and b.attrs.get("plain")):
+            if a.attrs.get("plain") and not b.attrs.get("plain") and b.op != "const" and \
+                    op in _NOT_NUMPY_MA_OPERATORS and not as_function:
+                # numpy.ma does not define this operator itself: ndarray's runs the
+                # NumPy function with the tile converted to its values, whatever
+                # their activity (python/hckernel/kernel_api.py:150-151)
+                r.attrs["right_values"] = True
             # the left operand is what a NumPy function returned: in the reference a
             # bare numpy.ma array, whose operator gives another one (stored in full);
             # so does the reflected operator of a bare array next to a number
@@ -724,6 +739,8 @@ class Tile:
     def __abs__(self): return Tile("abs", (self,), self.shape, self.dtype_name, **self._plain_kw())
 
     def _plain_kw(self):
+        if self.attrs.get("ndarray"):
+            return {"plain": True, "ndarray": True}
         return {"plain": True} if self.attrs.get("plain") else {}
 
     # The rest of the operators the reference's wrapper forwards to NumPy
@@ -749,7 +766,11 @@ class Tile:
         o = Tile.wrap(other)
         r = Tile(op, (self, o), _broadcast(self.shape, o.shape), "bool",
                  operand_dtype=_result_dtype(self, o))
-        if self.attrs.get("plain"):
+        if _all_ndarrays(self, o):
+            r.attrs.update(plain=True, ndarray=True)
+        elif self.attrs.get("ndarray") and not o.attrs.get("plain"):
+            pass                                # the tile's mirrored comparison: a tile
+        elif self.attrs.get("plain"):
             r.attrs["plain"] = True
         return r
 
@@ -773,7 +794,7 @@ class Tile:
         if self.attrs.get("plain"):
             raise TraceError("the mask of a bare numpy.ma array (the result of a NumPy function, a "
                              "reduction or astype) has numpy.ma's polarity, not a tile's: no native code")
-        return Tile("active", (self,), self.shape, "bool", plain=True)
+        return Tile("active", (self,), self.shape, "bool", plain=True, ndarray=True)
 
     def compressed(self):
         raise TraceError("tile.compressed(): a 1-D array of the active elements only; its length "
@@ -801,6 +822,9 @@ class Tile:
         def plain(t: "Tile") -> "Tile":
             t.attrs["plain"] = t.attrs["func"] = True
             t.attrs.pop("pow", None)
+            if _all_ndarrays(*(Tile.wrap(v) for v in inputs)):
+                # a NumPy function of plain arrays is plain NumPy: no domains, IEEE results
+                t.attrs["ndarray"] = t.attrs["ieee"] = True
             return t
 
         if len(inputs) == 1:
@@ -809,16 +833,22 @@ class Tile:
                 return plain(x * x)
             return plain(Tile(op, (x,), x.shape, x.dtype_name))
         a, b = inputs
+        if isinstance(a, np.ndarray) and a.ndim == 0:
+            a = a[()]                           # (a NumPy scalar's comparison arrives as a 0-d array)
         if isinstance(a, np.generic) and isinstance(b, Tile) and not b.attrs.get("plain"):
-            # `np.float32(2) * tile`: the scalar's operator arrives here; it is the
-            # tile's reflected operator (which the reference's tile type lacks).
-            # (Next to a bare numpy.ma array the scalar's operator is the NumPy
-            # function: computed on the values, deactivated or not.)
-            refl = {"add": "__radd__", "sub": "__rsub__", "mul": "__rmul__", "div": "__rtruediv__",
-                    "floordiv": "__rfloordiv__", "mod": "__rmod__", "lt": "__gt__", "le": "__ge__",
-                    "gt": "__lt__", "ge": "__le__", "eq": "__eq__", "ne": "__ne__"}.get(op)
-            if refl is not None:
+            # `np.float32(2) * tile`: the scalar's operator arrives here.  The
+            # reference's tile type has no reflected operators and is no array, so
+            # there the arithmetic operators raise TypeError and the comparisons
+            # fall back to the tile's own, mirrored.  (Next to a bare numpy.ma array
+            # the scalar's operator is the NumPy function: computed on the values,
+            # deactivated or not.)
+            refl = {"lt": "__gt__", "le": "__ge__", "gt": "__lt__", "ge": "__le__", "eq": "__eq__",
+                    "ne": "__ne__"}.get(op)
+            if refl is not None and _called_by_an_operator():
                 return getattr(b, refl)(a)
+            if _called_by_an_operator():
+                    raise TypeError(f"unsupported operand type(s) for numpy.{ufunc.__name__}: "
+                                f"'{type(a).__name__}' and a tile (write the tile first, or a Python number)")
         if op == "power":
             r = Tile.wrap(a) ** b
             if r is a:                          # exponent 1: a new node, the same values
@@ -828,8 +858,8 @@ class Tile:
             a, b = Tile.wrap(a), Tile.wrap(b)
             return plain(a._compare(b, op))
         if isinstance(a, Tile):
-            return plain(a._binary(b, op))
-        return plain(Tile.wrap(b)._binary(a, op, reflected=True))
+            return plain(a._binary(b, op, as_function=True))
+        return plain(Tile.wrap(b)._binary(a, op, reflected=True, as_function=True))
 
     def __array_function__(self, func, types, args, kwargs):
         name = func.__name__
@@ -839,8 +869,8 @@ class Tile:
             x = Tile.wrap(args[0])
             lo = kwargs.get("a_min", args[1] if len(args) > 1 else None)
             hi = kwargs.get("a_max", args[2] if len(args) > 2 else None)
-            return Tile("clip", (x,), x.shape, x.dtype_name, lo=float(lo), hi=float(hi), plain=True,
-                        func=True)
+            return Tile("clip", (x,), x.shape, x.dtype_name, lo=float(lo), hi=float(hi), func=True,
+                        **{"plain": True, **x._plain_kw()})
         if name in ("amax", "max", "sum", "amin", "min"):
             x = Tile.wrap(args[0])
             return x._reduce({"amax": "max", "amin": "min"}.get(name, name),
@@ -863,7 +893,7 @@ class Tile:
             if c.dtype_name != "bool":
                 raise TraceError("numpy.where: the condition must be a comparison of tiles")
             shape = _broadcast(_broadcast(c.shape, a.shape), b.shape)
-            return Tile("where", (c, a, b), shape, _result_dtype(a, b), plain=True, func=True)
+            return Tile("where", (c, a, b), shape, _result_dtype(a, b), plain=True, func=True, ndarray=True)
         if name == "transpose" and len(args) == 1:
             return Tile.wrap(args[0]).T
         if name == "norm" and kwargs.get("ord", args[1] if len(args) > 1 else None) is None:
@@ -883,7 +913,8 @@ class Tile:
             else tuple(n for i, n in enumerate(self.shape) if i not in axes)
         # (plain: a reduction of a tile is a bare numpy.ma array, not a tile,
         # python/hckernel/kernel_api.py:150-151)
-        return Tile(op, (self,), shape, self.dtype_name, axes=axes, keepdims=bool(keepdims), plain=True)
+        return Tile(op, (self,), shape, self.dtype_name, axes=axes, keepdims=bool(keepdims),
+                    **{"plain": True, **self._plain_kw()})
 
     def max(self, axis=None, keepdims=False): return self._reduce("max", axis, keepdims)
     def min(self, axis=None, keepdims=False): return self._reduce("min", axis, keepdims)
@@ -910,7 +941,11 @@ class Tile:
         if x.dtype_name != "float32":
             raise TraceError("mean of a tile: float32 and float16 tiles only (cast first)")
         total = x._reduce("sum", axis, keepdims)
-        r = Tile("div", (total, x._count(axis, keepdims)), total.shape, "float32", ma=True, plain=True)
+        if self.attrs.get("ndarray"):           # numpy.mean of a plain array: the sum over the number
+            r = Tile("div", (total, x._count(axis, keepdims)), total.shape, "float32", plain=True,
+                     ndarray=True, ieee=True)
+        else:
+            r = Tile("div", (total, x._count(axis, keepdims)), total.shape, "float32", ma=True, plain=True)
         return r.astype("float16") if half else r
 
     def var(self, axis=None, keepdims=False, ddof=0):
@@ -930,6 +965,13 @@ class Tile:
         return Tile("masqrt", (v,), v.shape, v.dtype_name, plain=True)
 
     def __pow__(self, e):
+        if isinstance(e, (int, float, np.generic)) and not isinstance(e, bool) and self.attrs.get("ndarray"):
+            # a plain array: ndarray.__pow__ calls numpy.square, numpy.sqrt for these exponents
+            if float(e) == 2.0:
+                return self * self
+            if float(e) == 0.5:
+                return Tile("sqrt", (self,), self.shape, self.dtype_name, func=True, ieee=True,
+                            **self._plain_kw())
         if isinstance(e, (int, float, np.generic)) and not isinstance(e, bool):
             # pow=True: numpy.ma.power deactivates results that are not finite
             if float(e) == 2.0:
@@ -948,7 +990,7 @@ class Tile:
             return self
         # (a tile's astype is numpy.ma's, python/hckernel/kernel_api.py:150-151:
         # the result is a bare numpy.ma array, not a tile)
-        return Tile("astype", (self,), self.shape, name, plain=True)
+        return Tile("astype", (self,), self.shape, name, **{"plain": True, **self._plain_kw()})
 
     @property
     def T(self):
@@ -956,7 +998,8 @@ class Tile:
             raise TraceError(".T needs a 2-D tile")
         # (an attribute the reference's wrapper forwards to numpy.ma,
         # python/hckernel/kernel_api.py:150-151: the result is a bare array)
-        return Tile("transpose", (self,), self.shape[::-1], self.dtype_name, plain=True)
+        return Tile("transpose", (self,), self.shape[::-1], self.dtype_name,
+                    **{"plain": True, **self._plain_kw()})
 
     @property
     def dtype(self):
@@ -1033,6 +1076,29 @@ class Tile:
 
     def __repr__(self):
         return f"<tile {self.op} {self.shape} {self.dtype_name}>"
+
+
+def _called_by_an_operator() -> bool:
+    """The NumPy function that reached Tile.__array_ufunc__ was started by an
+    operator of a NumPy scalar (`numpy.float32(2) * tile`), not written as a
+    call (`numpy.multiply(numpy.float32(2), tile)`).  NumPy gives no other way
+    to tell the two apart, and the reference raises for the first only: the
+    instruction the body's frame is at says which it is."""
+    import dis
+    import sys
+    frame = sys._getframe(2)                   # the caller of __array_ufunc__'s caller (NumPy has no frame)
+    name = dis.opname[frame.f_code.co_code[frame.f_lasti]]
+    return name.startswith(("BINARY_", "INPLACE_", "COMPARE_OP"))
+
+
+_NOT_NUMPY_MA_OPERATORS = ("mod", "and", "or", "xor", "shl", "shr")
+
+
+def _all_ndarrays(*operands: Tile) -> bool:
+    """Plain NumPy arrays and numbers only, at least one array: no numpy.ma
+    array among them, so NumPy's own arithmetic applies."""
+    return any(t.attrs.get("ndarray") for t in operands) and \
+        all(t.attrs.get("ndarray") or t.op == "const" for t in operands)
 
 
 def _dot(a: Tile, b: Tile) -> Tile:

@@ -407,6 +407,18 @@ int hcamdLaunchIMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
  *                the second (`arg` bit 0, fp16 tiles: the first, as NumPy's half
  *                loops do)
  *   the rest     computed from the values, activity kept; comparisons give 0 / 1
+ *   EQ NE        under an inactive result: 1 / 0 where both operands are inactive,
+ *                0 / 1 where one is (numpy.ma compares the activity there);
+ *                `arg` bit 1: numpy.equal / not_equal as functions, the values
+ *   `arg` bit 3  on MIN MAX: the program evaluated the operands in the other
+ *                order (which of two equal values wins depends on the order)
+ *   `arg` bit 4  on a binary operation: the second operand's activity does not
+ *                count (a bare numpy.ma array % tile: ndarray's operator converts
+ *                the tile to its values)
+ *   `arg` bit 2  on DIV FLOORDIV MOD UDIV SQRT LOG LOG2 LOG10: the operands are
+ *                plain NumPy arrays (results of numpy.where, numpy.dot, tile.mask
+ *                and arithmetic of those), so the operation is NumPy's own: IEEE
+ *                results, nothing deactivated
  * An operand of type HCAMD_I32 is converted to fp32 when it is read (a tile's
  * astype(float32)).  Every rounding to fp16 other than DIV / FLOORDIV's is an explicit
  * HCAMD_FMAP_R16.  outType is HCAMD_F32, HCAMD_F16, or HCAMD_U8 (one byte of

@@ -98,6 +98,21 @@ def _install_operators():
             return Tile(fn(self._m, _as_ma(other)))
 
         def reflected(self, other):
+            # The reference's wrapper has no reflected operators
+            # (kernel_api.py:158-206).  What is on the left decides:
+            #  * a Python number: an extension of this executor (a TypeError there);
+            #  * a NumPy scalar or a plain ndarray (numpy.where's result): NumPy
+            #    defers to the wrapper, finds no reflected operator: TypeError;
+            #  * a bare numpy.ma array arrives here only for the operators
+            #    numpy.ma does not define itself (% & | ^ << >>): there ndarray's
+            #    operator runs the ufunc with the wrapper converted through
+            #    numpy.ma's __array__ (kernel_api.py:150-151), that is on the
+            #    tile's values, whatever their activity, and the result is a
+            #    bare numpy.ma array again.
+            if isinstance(other, ma.MaskedArray):
+                return fn(other, self._m.data)
+            if isinstance(other, (np.generic, np.ndarray)):
+                raise TypeError(f"unsupported operand type(s): '{type(other).__name__}' and a tile")
             return Tile(fn(_as_ma(other), self._m))
 
         def inplace(self, other):

@@ -670,7 +670,106 @@ def case_numpy_scalar_on_the_left(api):
     return rec.out
 
 
+def _w(a, b):
+    return np.where(a < b, a, b)
+
+def _v(a, b):
+    return np.where(a < b, b, a)
+
+PLAIN_AND_BARE_FORMS = {
+    # plain arrays and numbers
+    "w_div_number": lambda a, b: _w(a, b) / np.float32(-0.125),
+    "w_div_zero": lambda a, b: _w(a, b) / np.float32(0),
+    "w_floordiv_v": lambda a, b: _w(a, b) // _v(a, b),
+    "w_mod_number": lambda a, b: _w(a, b) % np.float32(2),
+    "w_mod_v": lambda a, b: _w(a, b) % _v(a, b),
+    "sqrt_w": lambda a, b: np.sqrt(_w(a, b)),
+    "log_w": lambda a, b: np.log(_w(a, b)),
+    "w_pow_half": lambda a, b: _w(a, b) ** np.float32(0.5),
+    "w_pow_two": lambda a, b: _w(a, b) ** np.float32(2),
+    "number_div_w": lambda a, b: np.float32(2) / _w(a, b),
+    "pynumber_minus_w": lambda a, b: 2 - _w(a, b),
+    "divide_w_v": lambda a, b: np.divide(_w(a, b), _v(a, b)),
+    "neg_abs_w": lambda a, b: -abs(_w(a, b)),
+    "w_lt_number": lambda a, b: _w(a, b) < np.float32(0),
+    "w_sum": lambda a, b: _w(a, b).sum(),
+    "where_of_quotient_then_div": lambda a, b: np.where(a < b, a / b, b) / np.float32(0),
+    # plain arrays next to tiles
+    "w_add_tile": lambda a, b: _w(a, b) + a,
+    "w_div_tile": lambda a, b: _w(a, b) / a,
+    "w_floordiv_tile": lambda a, b: _w(a, b) // a,
+    "w_mod_tile": lambda a, b: _w(a, b) % a,
+    "tile_add_w": lambda a, b: a + _w(a, b),
+    "tile_div_w": lambda a, b: a / _w(a, b),
+    "tile_floordiv_w": lambda a, b: a // _w(a, b),
+    "tile_mod_w": lambda a, b: a % _w(a, b),
+    "w_lt_tile": lambda a, b: _w(a, b) < a,
+    "tile_lt_w": lambda a, b: a < _w(a, b),
+    "divide_tile_w": lambda a, b: np.divide(a, _w(a, b)),
+    "divide_w_tile": lambda a, b: np.divide(_w(a, b), a),
+    "maximum_w_tile": lambda a, b: np.maximum(_w(a, b), a),
+    "where_of_w_and_tile": lambda a, b: np.where(_w(a, b) > a, _w(a, b), a),
+    "mask_and_mask": lambda a, b: (a / b).mask & (b / a).mask,
+    "where_of_mask": lambda a, b: np.where((a / b).mask, a, b),
+    # plain arrays next to bare numpy.ma arrays
+    "w_div_bare": lambda a, b: _w(a, b) / np.abs(a),
+    "w_mod_bare": lambda a, b: _w(a, b) % np.abs(a),
+    "bare_div_w": lambda a, b: np.abs(a) / _w(a, b),
+    "bare_mod_w": lambda a, b: np.abs(a) % _w(a, b),
+    # bare numpy.ma arrays next to tiles
+    "bare_add_tile": lambda a, b: np.abs(a) + b,
+    "bare_div_tile": lambda a, b: np.abs(a) / b,
+    "bare_floordiv_tile": lambda a, b: np.abs(a) // b,
+    "bare_mod_tile": lambda a, b: np.abs(a) % b,
+    "sqrt_mod_tile": lambda a, b: np.sqrt(a * a) % b,
+    "tile_mod_bare": lambda a, b: a % np.abs(b),
+    "tile_floordiv_bare": lambda a, b: a // np.abs(b),
+    "bare_lt_tile": lambda a, b: np.abs(a) < b,
+    "bare_pow_half": lambda a, b: np.negative(a) ** np.float32(0.5),
+    "bare_mod_number": lambda a, b: np.abs(a) % np.float32(2),
+    "bare_mod_zero": lambda a, b: np.abs(a) % np.float32(0),
+    "tile_mod_zero": lambda a, b: a % np.float32(0),
+    "tile_mod_product": lambda a, b: a % (np.float32(0) * b),
+    "quotient_mod_tile": lambda a, b: (a / b) % b,
+}
+
+
+def case_plain_and_bare_arrays_next_to_tiles(api):
+    """What follows numpy.where (a plain NumPy array) and a NumPy function of a
+    tile (a bare numpy.ma array) when they meet numbers, each other and tiles,
+    on either side of the operators and in NumPy functions: which arithmetic
+    runs (NumPy's own, numpy.ma's operator, numpy.ma's wrapped function), what
+    kind of value comes back, what raises, and what a store writes."""
+    rec = Recorder()
+    f = np.float32
+    x = np.array([1.0, 0.0, -0.0, np.inf, np.nan, 4.0, -2.0, 0.5, -1.0, 3.0, -np.inf, 2.5], f)
+    y = np.array([2.0, 0.0, 1.0, 1.0, 1.0, 0.0, 0.0, -1.0, 1.0, -2.0, 2.0, 0.0], f)
+
+    forms = PLAIN_AND_BARE_FORMS
+    dst = np.full((len(forms), 12), POISON, f)
+    dstb = np.full((len(forms), 12), True)
+
+    def body(gr, x, y, dst, dstb):
+        for i, (name, fn) in enumerate(forms.items()):
+            a, b = gr.load(x[:11], shape=12), gr.load(y[:11], shape=12)
+            t = rec.attempt(name, lambda: fn(a, b))
+            if t is None or np.ndim(t) != 1:
+                continue
+            if t.dtype == f:
+                gr.store(dst[i], t)
+            elif t.dtype == bool:
+                gr.store(dstb[i], t)
+
+    with np.errstate(all="ignore"), warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        _one_group(api, body, x, y, dst, dstb, group=12)
+    rec.array("dst", dst)
+    rec.array("dst_bool", dstb)
+    return rec.out
+
+
 CASES = {
+    "plain_and_bare_arrays_next_to_tiles": case_plain_and_bare_arrays_next_to_tiles,
     "masked_reductions": case_masked_reductions,
     "inplace_partial": case_inplace_partial,
     "load_from_masked": case_load_from_masked,

@@ -1,0 +1,103 @@
+"""Random elementwise kernel bodies that lean on numpy.ma's rules: zero
+divisors, domains of functions, numpy.where, bare arrays and plain arrays next
+to tiles, signed zeros, NaN and infinities in the data.  Shared by the CPU test
+that runs the binder's programs in a NumPy restatement of the kernel and by the
+GPU test that runs them on the device; both compare with the host executor."""
+
+import numpy as np
+
+# functions whose results may differ from NumPy's in the last bits (tile ** 0.5
+# is numpy.power's powf there, a correctly rounded square root here)
+INEXACT = ("exp", "log", "tanh", "sin", "cos", "expm1", "log1p", "exp2", "log2", "log10", "** K(0.5)")
+
+
+def expression(rng, depth, K):
+    """(function of three tiles, its source text); K is the tiles' NumPy type."""
+    def gen(d):
+        if d == 0 or rng.random() < 0.15:
+            return rng.choice(["a", "b", "c"])
+        kind = rng.integers(0, 20)
+        x = gen(d - 1)
+        if kind <= 2:
+            return f"({x} {rng.choice(['+', '-', '*'])} {gen(d - 1)})"
+        if kind == 3:
+            return f"({x} / {gen(d - 1)})"
+        if kind == 4:
+            return f"({x} // {gen(d - 1)})"
+        if kind == 5:
+            return f"({x} % {gen(d - 1)})"
+        if kind == 6:
+            return f"np.{rng.choice(['maximum', 'minimum'])}({x}, {gen(d - 1)})"
+        if kind == 7:
+            return f"(-{x})"
+        if kind == 8:
+            return f"np.abs({x})"
+        if kind == 9:
+            return f"np.sqrt({x})"
+        if kind == 10:
+            return f"np.log({x})"
+        if kind == 11:
+            cmp = rng.choice(['<', '<=', '>', '>=', '==', '!='])
+            return f"np.where({gen(d - 1)} {cmp} {gen(d - 1)}, {x}, {gen(d - 1)})"
+        if kind == 12:
+            return f"({x} ** K({rng.choice(['2', '0.5'])}))"
+        if kind == 13:
+            return f"np.{rng.choice(['floor', 'ceil', 'trunc', 'sign', 'rint', 'reciprocal'])}({x})"
+        if kind == 14:
+            return f"np.{rng.choice(['tanh', 'sin', 'cos'])}({x})"
+        if kind == 15:
+            return f"({x} {rng.choice(['//', '%', '/'])} K({rng.choice(['0.5', '2.0', '-1.25', '0.0'])}))"
+        if kind == 16:
+            return f"np.{rng.choice(['divide', 'multiply', 'add', 'subtract'])}({x}, {gen(d - 1)})"
+        if kind == 17:
+            return f"np.clip({x}, -1.5, 2.25)"
+        if kind == 18:
+            return f"np.square({x})"
+        return f"({x} {rng.choice(['+', '-', '*', '/'])} K({rng.choice(['0.5', '4.0', '-0.125', '0.0'])}))"
+
+    text = gen(depth)
+    while text in ("a", "b", "c"):
+        text = gen(depth)
+    return eval(f"lambda a, b, c: {text}", {"np": np, "K": K}), text
+
+
+def special_values(rng, shape, dtype):
+    """Small multiples of 0.5 (so that sums and products are exact) with zeros
+    of both signs, infinities and NaN sprinkled in."""
+    v = (rng.integers(-6, 7, shape) / 2).astype(dtype)
+    flat = v.reshape(-1)
+    idx = rng.integers(0, flat.size, max(1, flat.size // 50))
+    flat[idx] = rng.choice(np.array([np.inf, -np.inf, np.nan, 0.0, -0.0], dtype), idx.size)
+    return v
+
+
+def case(seed):
+    """(function, text, dtype, three operand arrays of shape `shape`, shape kind)."""
+    rng = np.random.default_rng(seed)
+    dtype = [np.float32, np.float16][seed % 2]
+    fn, text = expression(rng, int(rng.integers(1, 4)), dtype)
+    shape = (1003,) if seed % 3 == 0 else (37, 131)
+    return fn, text, dtype, [special_values(rng, shape, dtype) for _ in range(3)], shape
+
+
+def difference(got, want, text):
+    """None if `got` equals `want`: the same NaNs, the same bits elsewhere
+    (a few ulp where `text` calls a function whose last bits may differ)."""
+    dtype = want.dtype
+    nan = np.isnan(want)
+    if not (np.isnan(got) == nan).all():
+        i = tuple(np.argwhere(np.isnan(got) != nan)[0])
+        return f"NaN pattern differs at {i}: got {got[i]} want {want[i]}"
+    if any(w in text for w in INEXACT):
+        tol = dict(rtol=2e-3, atol=2e-3) if dtype == np.float16 else dict(rtol=2e-6, atol=1e-6)
+        ok = np.isclose(got.astype(np.float64), want.astype(np.float64), equal_nan=True, **tol)
+        if not ok.all():
+            i = tuple(np.argwhere(~ok)[0])
+            return f"values differ at {i}: got {got[i]} want {want[i]}"
+        return None
+    u = np.uint32 if dtype == np.float32 else np.uint16
+    bad = (got.view(u) != want.view(u)) & ~nan
+    if bad.any():
+        i = tuple(np.argwhere(bad)[0])
+        return f"bits differ at {i}: got {got[i]} want {want[i]}"
+    return None

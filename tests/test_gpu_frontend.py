@@ -1105,6 +1105,12 @@ def test_random_int32_expression_trees_equal_the_host_executor(seed):
             if "too deep" in str(e) or "too long" in str(e):
                 continue
             raise
+        except TypeError:
+            # a NumPy scalar on the left of a tile: a TypeError in the reference too
+            # (its tile type has no reflected operators), and in the host executor
+            with pytest.raises(TypeError), np.errstate(all="ignore"):
+                sim_kernel(work_shape=(R, Cc), group_shape=(4, 64))(body)(*ins, host)
+            continue
         break
     else:
         pytest.fail("no tree that fits the integer map in 20 draws")
@@ -1652,7 +1658,7 @@ _FLOAT_OPERATOR_BODIES = {
     "np.remainder(a,b)": lambda a, b, K: np.remainder(a, b),
     "(a/b)*b": lambda a, b, K: (a / b) * b,
     "np.abs(a)*(b/a)": lambda a, b, K: np.abs(a) * (b / a),
-    "K(2)*(a/b)": lambda a, b, K: K(2) * (a / b),
+    "(a/b)*K(2)": lambda a, b, K: (a / b) * K(2),
     "np.abs(a/b)+K(1)": lambda a, b, K: np.abs(a / b) + K(1),
     "np.rint(a//b)-a%b": lambda a, b, K: np.rint(a // b) - a % b,
 }
@@ -1849,3 +1855,115 @@ def test_column_reductions_leave_deactivated_elements_out():
         assert rt.last_kernel_name().startswith(("hcamd_map", "hcamd_cols_fold_f32")), name
         assert np.isfinite(want).all(), name
         assert_allclose(out.to_host(), want, rtol=2e-4, atol=2e-4, err_msg=name)
+
+
+# forms of the fixture's case that have no native kernel: a scalar result, `&`
+# of two plain bool arrays
+_PLAIN_AND_BARE_REFUSED = {"w_sum", "mask_and_mask"}
+
+
+def test_plain_and_bare_arrays_next_to_tiles_match_the_reference_simulator():
+    """numpy.where returns a plain NumPy array and a NumPy function of a tile a
+    bare numpy.ma array; what they do next to numbers, each other and tiles
+    (NumPy's own arithmetic, numpy.ma's operators, TypeError for a plain array
+    or a NumPy scalar on the left of a tile) is pinned by vectors written by the
+    reference simulator (tests/golden/sim_cases.py,
+    case_plain_and_bare_arrays_next_to_tiles); the same bodies run here through
+    @kernel and every stored value is compared with those vectors bit for bit
+    (numpy.log: 2 ulp)."""
+    import os
+    import sys
+    sys.path.insert(0, os.path.join(os.path.dirname(__file__), "golden"))
+    import sim_cases
+    from hc_amd.binding import NoNativeKernel
+    golden = sim_cases.load(os.path.join(os.path.dirname(__file__), "golden", "sim_golden.json"))
+    case = "plain_and_bare_arrays_next_to_tiles/"
+    f = np.float32
+    x = np.array([1.0, 0.0, -0.0, np.inf, np.nan, 4.0, -2.0, 0.5, -1.0, 3.0, -np.inf, 2.5], f)
+    y = np.array([2.0, 0.0, 1.0, 1.0, 1.0, 0.0, 0.0, -1.0, 1.0, -2.0, 2.0, 0.0], f)
+    N = sym.N
+    dx, dy = rt.to_device(x[:11].copy()), rt.to_device(y[:11].copy())
+    refused = set()
+    for i, (name, fn) in enumerate(sim_cases.PLAIN_AND_BARE_FORMS.items()):
+        is_bool = case + name + ".dtype" in golden and bytes(golden[case + name + ".dtype"]) == b"bool"
+        # (the arrays end one element before the tiles do, as in the fixture: the
+        # last element of every tile is inactive)
+        want = golden[case + ("dst_bool" if is_bool else "dst")][i][:11]
+        out = rt.to_device(np.full(11, True) if is_bool else np.full(11, sim_cases.POISON, f))
+
+        @kernel(work_shape=N, group_shape=12)
+        def body(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], out: Buffer[N, typename.DT2]):
+            gr.store(out[0:], fn(gr.load(a[0:], shape=12), gr.load(b[0:], shape=12)))
+
+        if case + name + ".raises" in golden:
+            with pytest.raises(TypeError):
+                body(dx, dy, out)
+            continue
+        try:
+            body(dx, dy, out)
+        except NoNativeKernel:
+            refused.add(name)
+            continue
+        got = out.to_host()
+        if name == "log_w":
+            assert_array_equal(np.isnan(got), np.isnan(want), err_msg=name)
+            assert_allclose(got, want, rtol=3e-7, err_msg=name)
+        elif is_bool:
+            assert_array_equal(got, want, err_msg=name)
+        else:
+            nan = np.isnan(want)
+            assert_array_equal(np.isnan(got), nan, err_msg=f"{name}: got {got.tolist()} want {want.tolist()}")
+            assert_array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan],
+                               err_msg=f"{name}: got {got.tolist()} want {want.tolist()}")
+    assert refused == _PLAIN_AND_BARE_REFUSED, refused
+
+
+def test_random_bodies_match_the_simulator():
+    """Random elementwise bodies that lean on numpy.ma's rules
+    (tests/random_bodies.py: zero divisors, domains, numpy.where, bare and plain
+    arrays next to tiles, signed zeros, NaN, infinities), 1-D and 2-D, fp32 and
+    fp16, on the device against the host executor: the same NaNs, the same bits
+    elsewhere (a few ulp for transcendental functions).  Whatever kernel the
+    binder picks runs; a body either side refuses is refused by both or has no
+    native kernel."""
+    import warnings
+    import random_bodies
+    from hc_amd.binding import NoNativeKernel
+    N, M = sym.N, sym.M
+    tally = {"ok": 0, "refused": 0, "both raise": 0}
+    for seed in range(600):
+        fn, text, dtype, vals, shape = random_bodies.case(seed)
+        if len(shape) == 1:
+            def body(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], c: Buffer[N, DT], out: Buffer[N, DT]):
+                o = gr.work_offset[0]
+                gr.store(out[o:], fn(*(gr.load(v[o:], shape=gr.shape) for v in (a, b, c))))
+            deco = dict(work_shape=N, group_shape=256)
+        else:
+            def body(gr: CurrentGroup, a: Buffer[M, N, DT], b: Buffer[M, N, DT], c: Buffer[M, N, DT],
+                     out: Buffer[M, N, DT]):
+                i, j = gr.work_offset
+                gr.store(out[i:, j:], fn(*(gr.load(v[i:, j:], shape=gr.shape) for v in (a, b, c))))
+            deco = dict(work_shape=(M, N), group_shape=(4, 64))
+        want = np.full(shape, 7.5, dtype)
+        sim_raises = False
+        try:
+            with np.errstate(all="ignore"), warnings.catch_warnings():
+                warnings.simplefilter("ignore")
+                sim_kernel(**deco)(body)(*vals, want)
+        except TypeError:                      # a NumPy scalar or plain array on the left of a tile
+            sim_raises = True
+        out = rt.to_device(np.full(shape, 7.5, dtype))
+        try:
+            kernel(**deco)(body)(*[rt.to_device(v) for v in vals], out)
+        except NoNativeKernel:
+            tally["refused"] += 1
+            continue
+        except TypeError:
+            assert sim_raises, f"seed {seed}: {text}: only the front-end raises TypeError"
+            tally["both raise"] += 1
+            continue
+        assert not sim_raises, f"seed {seed}: {text}: only the simulator raises TypeError"
+        diff = random_bodies.difference(out.to_host(), want, text)
+        assert diff is None, f"seed {seed}: {text} ({np.dtype(dtype).name}, {rt.last_kernel_name()}): {diff}"
+        tally["ok"] += 1
+    assert tally["ok"] > 400, tally

@@ -543,6 +543,56 @@ def test_fmap_every_operation_against_numpy_ma(ctx, dtype):
         rt.plan_fmap([F("in", 0), F("in", 0)], [dev(a)], poisoned((n,), dtype), [ty, ty]).launch(sync=True)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_fmap_every_opcode_and_flag_against_its_numpy_restatement(ctx, dtype):
+    """hcamdLaunchFMap against tests/fmap_emulator.py (the rules of the kernel's
+    header in NumPy, which the CPU tests run the binder's programs with), for
+    every opcode under every flag it reads: bit 0 fp16, bit 1 called as a
+    function, bit 2 plain arrays, bit 3 operands evaluated in the other order,
+    bit 4 the second operand's activity does not count.  Operands are quotients
+    with zero divisors, so both carry inactive elements; stored where active and
+    in full."""
+    from fmap_emulator import run_fmap
+    rng = np.random.default_rng(77)
+    n = 6_007
+    a, b, c = (_ma_special(rng, n, dtype) for _ in range(3))
+    ty = rt.F32 if dtype == np.float32 else rt.F16
+    half = int(dtype == np.float16)
+    u = np.uint32 if dtype == np.float32 else np.uint16
+    F = lambda name, arg=0, imm=0.0: (name, arg, imm)
+    r16 = [F("r16")] if half else []
+    left = [F("in", 0), F("in", 1), F("div", half)]            # a / b: inactive where b == 0 ...
+    right = [F("in", 2), F("in", 0), F("div", half)]           # c / a
+    inexact = {"exp", "log", "tanh", "exp2", "log2", "log10", "log1p", "expm1", "sin", "cos"}
+    binary = ["add", "sub", "mul", "div", "floordiv", "mod", "min", "max", "udiv", "lt", "le", "eq", "ne", "ge", "gt"]
+    unary = [k for k in rt.FMAP_OPS if k not in binary + ["end", "in", "const", "select"]]
+    programs = []
+    for name in binary:
+        for arg in (0, 1, 2, 4, 8, 16, 2 | 16, 1 | 8):
+            programs.append((f"{name}|{arg}", left + right + [F(name, arg)] + r16))
+    for name in unary:
+        for arg in (0, 4):
+            programs.append((f"{name}|{arg}", left + [F(name, arg)] + r16))
+            programs.append((f"{name}|{arg} of an operand", [F("in", 0), F(name, arg)] + r16))
+    programs.append(("select", left + right + [F("lt")] + left + right + [F("select")]))
+    da, db, dc = dev(a), dev(b), dev(c)
+    for label, prog in programs:
+        for store_all in (False, True):
+            say("fmap", np.dtype(dtype).name, label, store_all)
+            out = poisoned((n,), dtype)
+            rt.plan_fmap(prog, [da, db, dc], out, [ty, ty, ty, ty], store_all).launch(sync=True)
+            got = out.to_host()
+            want = np.full(1, POISON32 if dtype == np.float32 else POISON32 & 0xFFFF, u).view(dtype).repeat(n)
+            run_fmap(prog, [a, b, c], store_all, want)
+            nan = np.isnan(want)
+            assert_array_equal(np.isnan(got), nan, err_msg=label)
+            if label.split("|")[0] in inexact:
+                assert_allclose(got[~nan].astype(np.float64), want[~nan].astype(np.float64),
+                                rtol=2e-3 if half else 1e-6, atol=2e-3 if half else 1e-7, err_msg=label)
+            else:
+                assert_array_equal(got.view(u)[~nan], want.view(u)[~nan], err_msg=label)
+
+
 # ---------------------------------------------------------------------------
 # stream calibration kernels (the yardstick of the memory-bound kernels)
 # ---------------------------------------------------------------------------

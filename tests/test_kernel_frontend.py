@@ -1491,7 +1491,7 @@ def test_what_a_traced_tile_cannot_give_says_why(ctx):
     with pytest.raises(NoNativeKernel, match="polarity"):
         body(lambda a, b: np.exp(a).mask, "bool").plan(f32, f32, FakeDev((1000,), "bool"), ctx=ctx)
     with pytest.raises(NoNativeKernel, match="inside a larger integer expression"):
-        body(lambda a, b: (a // b).mask.astype(np.int32) + (a % b), "int32").plan(
+        body(lambda a, b: (a % b) + (a // b).mask.astype(np.int32), "int32").plan(
             i32, i32, FakeDev((1000,), "int32"), ctx=ctx)
     # the mask of a whole expression binds: one more instruction, a one-byte output
     (p,) = body(lambda a, b: (a / b).mask, "bool").plan(f32, f32, FakeDev((1000,), "bool"), ctx=ctx)
@@ -2155,3 +2155,43 @@ def test_float_operators_follow_numpy_ma_and_pick_the_kernel_that_can(ctx):
     assert fmap_program(p)[-1] == ("add", 2, 0.0)
     with pytest.raises(NoNativeKernel, match="floor_divide"):
         plan(lambda a, b: np.floor_divide(a, b))
+
+
+def test_results_of_numpy_where_are_plain_arrays_with_numpys_own_arithmetic(ctx):
+    """numpy.where (and tile.mask) return plain NumPy arrays in the reference:
+    operators and functions of those alone are NumPy's own (IEEE quotients,
+    NaN for a root of a negative number, nothing deactivated: `arg` bit 2),
+    next to a tile the tile's reflected operator runs and the result is a tile
+    again (stored where active), and a NumPy scalar on the left of a tile is a
+    TypeError as it is there."""
+    N = sym.N
+    f = np.float32
+
+    def plan(expr):
+        @kernel(work_shape=N, group_shape=256)
+        def k(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], out: Buffer[N, DT]):
+            o, g = gr.work_offset[0], gr.shape[0]
+            gr.store(out[o:], expr(gr.load(a[o:], shape=g), gr.load(b[o:], shape=g)))
+        (p,) = k.plan(FakeDev((1000,), "float32"), FakeDev((1000,), "float32"), FakeDev((1000,), "float32"),
+                      ctx=ctx)
+        return p
+
+    p = plan(lambda a, b: np.where(a < b, a, b) / f(-0.125))
+    assert fmap_program(p)[-2:] == [("const", 0, -0.125), ("div", 4, 0.0)] and p.args[-1] == 1
+    p = plan(lambda a, b: np.sqrt(np.where(a < b, a, b)) % f(2))
+    assert fmap_program(p)[-3:] == [("sqrt", 4, 0.0), ("const", 0, 2.0), ("mod", 4, 0.0)] and p.args[-1] == 1
+    p = plan(lambda a, b: np.where(a < b, a, b) ** f(0.5) // np.where(a < b, b, a))
+    assert [i[:2] for i in fmap_program(p) if i[0] in ("sqrt", "psqrt", "floordiv", "powchk")] == \
+        [("sqrt", 4), ("floordiv", 4)]
+    # next to a tile: on the right numpy.ma's operator, and a tile again; on the left NumPy
+    # defers to the tile, which has no reflected operators
+    with pytest.raises(TypeError):
+        plan(lambda a, b: np.where(a < b, a, b) // a)
+    p = plan(lambda a, b: a / np.where(a < b, a, b))
+    assert fmap_program(p)[-1] == ("div", 0, 0.0) and p.args[-1] == 0
+    # next to what a NumPy function of a tile returned: numpy.ma's operator, stored in full
+    p = plan(lambda a, b: np.where(a < b, a, b) / np.exp(a))
+    assert fmap_program(p)[-1] == ("div", 0, 0.0) and p.args[-1] == 1
+    for op in ("+", "-", "*", "/", "//", "%", "**"):
+        with pytest.raises(TypeError):
+            plan(eval(f"lambda a, b: f(2) {op} a", {"f": f}))

@@ -42,7 +42,7 @@ GOLDEN = os.path.join(HERE, "golden", "sim_golden.json")
 #    reference's mask property cannot invert (kernel_api.py:93-103); the oracle
 #    treats it as all active.
 #  * len(tile): no __len__ on the reference's wrapper type.
-ORACLE_DEFINES = ("_left_", "domain_masking/int_pow", "compressed_repr/len", "numpy_scalar_on_the_left/")
+ORACLE_DEFINES = ("_left_", "domain_masking/int_pow", "compressed_repr/len")
 
 
 def _text(a):
