@@ -765,8 +765,8 @@ def _fails_on_finite_data(t: Tile) -> bool:
     finite already, or by overflow.)"""
     if not _masks(t):
         return False
-    if t.op == "masqrt" or t.attrs.get("pow"):
-        return False
+    if t.op == "masqrt" or (t.attrs.get("pow") and t.op != "sqrt"):
+        return False                         # (x ** 0.5 fails on every negative x)
     if t.op == "div" and not t.attrs.get("func"):
         d = t.args[1]
         if t.attrs.get("ma") or (_const(d) and d.attrs.get("value") != 0.0):
@@ -841,6 +841,7 @@ def _leaf(t: Tile):
 # functions compute on the values regardless.
 _FUNC_FORM = 0x200            # the operation was called as a NumPy function
 _SWAPPED = 0x400              # a commutative operation whose running value is the second operand
+_KEEP_DEAD = 0x800            # a unary operation that leaves a deactivated value as it is (x ** 0.5)
 
 
 class _MapCompiler:
@@ -983,7 +984,9 @@ class _MapCompiler:
                 name = "m" + name              # numpy.sqrt / numpy.log of a tile: domain fill
             if name == "masqrt" and not self.masked:
                 name = "sqrt"                  # stored in full: the same values
-            out.append((name, 0, 0.0))
+            keep = _KEEP_DEAD if (self._scalar_mode or self._frozen) and t.op == "sqrt" and \
+                t.attrs.get("pow") else 0      # x ** 0.5: numpy.ma.power keeps an inactive operand's value
+            out.append((name, keep, 0.0))
             if self.masked and t.op == "sqrt" and t.attrs.get("pow"):
                 out.append(("addi", 0, 0.0))   # x ** 0.5 of -0 is +0 (the square root's is -0)
         else:
@@ -1938,6 +1941,8 @@ class _RowCompiler(_MapCompiler):
             a, b = t.args
             sa, sb = self.slot_of(a), self.slot_of(b)
             if sb is not None or sa is not None:
+                if self.masked and t.op == "div" and t.attrs.get("func") and not t.attrs.get("ieee"):
+                    raise _NeedsEntryMasks()       # numpy.divide as a function: its own domain and fill value
                 mdiv = self.masked and t.op == "div" and not t.attrs.get("func") and not t.attrs.get("ieee")
                 if mdiv:
                     fwd, rev = "mdiv", "rmdiv"

@@ -1540,6 +1540,8 @@ enum : uint32_t {
 // flags in `arg` of the instructions of scalar stages (beside bit 8, fp16)
 constexpr uint32_t kFuncForm = 0x200; // called as a NumPy function: computed on the values, deactivated or not
 constexpr uint32_t kSwapped = 0x400;  // commutative operation whose running value is the second operand
+constexpr uint32_t kKeepDead = 0x800; // unary operation that leaves a deactivated value as it is (x ** 0.5:
+                                      // numpy.ma.power keeps its operand where that is inactive)
 enum : uint32_t {
   ST_SUM = 0, ST_MAX = 1, ST_MIN = 2, ST_SCALAR = 3, ST_STORE = 4, ST_STORE_COL = 5,
   ST_COUNT = 6 // the number of active elements of the program's value, as fp32
@@ -1641,8 +1643,10 @@ __device__ __forceinline__ bool ma_is_unary(uint32_t op) {
   return (op >= OP_NEG && op <= OP_R16) || op == OP_POWCHK || op == OP_MSQRT || op == OP_MLOG ||
          op == OP_MASQRT;
 }
-__device__ __forceinline__ MaValue ma_unary(uint32_t op, MaValue x) {
+__device__ __forceinline__ MaValue ma_unary(uint32_t op, MaValue x, uint32_t arg) {
   const float v = x.v;
+  if ((arg & kKeepDead) && x.dead)
+    return x;
   switch (op) {
   case OP_NEG: return {-v, x.dead};
   case OP_ABS: return {__builtin_fabsf(v), x.dead};
@@ -1754,7 +1758,7 @@ __device__ __forceinline__ ScalarResult run_scalar_stage(const RowArgs &a, uint3
       put(sp++, {cells[slot], op == OP_RED && ((dead >> slot) & 1u)});
     } else if (ma_is_unary(op)) {
       if (sp >= 1)
-        put(sp - 1, ma_unary(op, get(sp - 1)));
+        put(sp - 1, ma_unary(op, get(sp - 1), arg));
     } else if ((op >= OP_ADD && op <= OP_RDIV) || op == OP_MDIV || op == OP_RMDIV) {
       if (sp >= 2) { // (any `arg` but the form flags marks an fp16 quotient)
         put(sp - 2, ma_binary(op, arg, (arg & 0x1ffu) != 0, get(sp - 2), get(sp - 1)));
@@ -1805,7 +1809,7 @@ __device__ __forceinline__ void run_frozen_stage(const RowArgs &a, uint32_t begi
     } else if (ma_is_unary(op)) {
 #pragma unroll
       for (int e = 0; e < kRowN; ++e) {
-        const MaValue y = ma_unary(op, {v[e], ((bad >> e) & 1u) != 0});
+        const MaValue y = ma_unary(op, {v[e], ((bad >> e) & 1u) != 0}, arg);
         v[e] = y.v;
         bad = (bad & ~(1u << e)) | (y.dead ? 1u << e : 0u);
       }

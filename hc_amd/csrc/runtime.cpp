@@ -2282,6 +2282,11 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       }
       if (red && op != HCAMD_MAP_RED0)
         readsDeadable |= (1u << index) & deadable;
+      // CLEAR makes every element active again: a deactivated row scalar read
+      // before it (the operand of a NumPy function, computed on its value) does
+      // not take the row out of the store
+      if (op == HCAMD_MAP_CLEAR && perElement)
+        readsDeadable = 0;
       if (sp < pops) {
         dev->report("%s: stack underflow at %zu", who, i);
         return 1;

@@ -546,10 +546,12 @@ int hcamdLaunchMapReduceColsNoAlloc(OlQueue q, int kind, const HcamdMapInstr *pr
  * the value numpy.ma leaves in it: in SCALAR / STORE_COL stages + - * leave
  * their first operand's value there, the quotient leaves the dividend, NumPy
  * functions compute regardless (sqrt and log give their fill values 0 and 1).
- * For that, `arg` of the instructions of those stages carries two more flags:
+ * For that, `arg` of the instructions of those stages carries three more flags:
  * 0x200, the operation was called as a NumPy function; 0x400, a commutative
  * operation whose running value (the stack top of an immediate or *_RED form,
- * the deeper entry of a stack form) is its second operand.  HCAMD_MAP_RED0
+ * the deeper entry of a stack form) is its second operand; 0x800, a unary
+ * operation that leaves a deactivated value as it is (the square root of
+ * x ** 0.5: numpy.ma.power keeps its operand where that is inactive).  HCAMD_MAP_RED0
  * pushes a row scalar's value whether deactivated or not (numpy.ma's variance
  * reads the sum of the centred squares that way: 0 if all of them were
  * inactive); HCAMD_MAP_MASQRT is numpy.ma.sqrt (the standard deviation's: a

@@ -101,3 +101,74 @@ def difference(got, want, text):
         i = tuple(np.argwhere(bad)[0])
         return f"bits differ at {i}: got {got[i]} want {want[i]}"
     return None
+
+
+def row_expression(rng, K):
+    """(function of two 2-D tiles, its text, result is one value per row): an
+    elementwise expression of the tiles and of row scalars (sum, max, min, mean,
+    var, std along axis 1 of smaller elementwise expressions)."""
+    red_count = [0]
+
+    def scalar(d):
+        red = rng.choice(["sum", "max", "min", "mean", "var", "std"])
+        inner = elem(d, False)
+        if red in ("var", "std"):
+            ddof = rng.choice(["", ", ddof=1"])
+            return f"{inner}.{red}(axis=1, keepdims=True{ddof})"
+        return f"{inner}.{red}(axis=1, keepdims=True)"
+
+    def elem(d, scalars):
+        if d == 0 or rng.random() < 0.2:
+            if scalars and red_count[0] < 3 and rng.random() < 0.45:
+                red_count[0] += 1
+                return scalar(max(d - 1, 0))
+            return rng.choice(["ta", "tb"])
+        kind = rng.integers(0, 12)
+        x = elem(d - 1, scalars)
+        if kind <= 2:
+            return f"({x} {rng.choice(['+', '-', '*'])} {elem(d - 1, scalars)})"
+        if kind <= 4:
+            return f"({x} / {elem(d - 1, scalars)})"
+        if kind == 5:
+            return f"np.{rng.choice(['maximum', 'minimum'])}({x}, {elem(d - 1, scalars)})"
+        if kind == 6:
+            return f"np.{rng.choice(['sqrt', 'log', 'abs', 'exp', 'tanh', 'square'])}({x})"
+        if kind == 7:
+            return f"(-{x})"
+        if kind == 8:
+            return f"({x} ** K({rng.choice(['2', '0.5'])}))"
+        if kind == 9:
+            return f"({x} {rng.choice(['+', '-', '*', '/'])} K({rng.choice(['0.5', '2.0', '-1.25', '0.0'])}))"
+        if kind == 10:
+            return f"{x}.astype(K)"
+        return f"np.{rng.choice(['divide', 'multiply', 'add', 'subtract'])}({x}, {elem(d - 1, scalars)})"
+
+    per_row = rng.random() < 0.3
+    while True:
+        red_count[0] = 0
+        if per_row:
+            inner = elem(int(rng.integers(1, 3)), False)
+            text = f"{inner}.{rng.choice(['sum', 'max', 'min', 'mean', 'var', 'std'])}(axis=1)"
+            if rng.random() < 0.4:
+                text = f"({text} {rng.choice(['+', '*', '/'])} {elem(1, False)}.{rng.choice(['sum', 'max', 'mean'])}(axis=1))"
+            break
+        text = elem(int(rng.integers(1, 4)), True)
+        if red_count[0]:
+            break
+    return eval(f"lambda ta, tb: {text}", {"np": np, "K": K}), text, per_row
+
+
+def row_case(seed):
+    """(function, text, per_row, two operand arrays of shape (rows, n))."""
+    rng = np.random.default_rng(seed)
+    fn, text, per_row = row_expression(rng, np.float32)
+    rows, n = [(9, 5), (13, 200), (6, 1031)][seed % 3]
+    vals = [special_values(rng, (rows, n), np.float32) for _ in range(2)]
+    # numpy.ma's mean / var / std of a bare array take NumPy's own path while no element of
+    # the whole tile is masked and numpy.ma's otherwise, which on rows with infinities or NaN
+    # gives different values and activity: data-dependent across rows, outside what the row
+    # kernels model (a documented deviation), so those bodies get finite data
+    if seed % 2 or any(w in text for w in ("mean(", "var(", "std(")):
+        for v in vals:
+            v[~np.isfinite(v)] = 0.5
+    return fn, text, per_row, vals

@@ -1,6 +1,7 @@
-"""The programs the binder emits for the general float map, run on the CPU by a
-NumPy restatement of the kernel's rules (tests/fmap_emulator.py), against the
-host executor, on random bodies (tests/random_bodies.py).  This checks the
+"""The programs the binder emits for the general float map and for row programs,
+run on the CPU by NumPy restatements of the kernels' rules (tests/fmap_emulator.py,
+run_row_stages of tests/test_kernel_frontend.py), against the host executor, on
+random bodies (tests/random_bodies.py).  This checks the
 front-end and the binder (which arithmetic a node means, which flags an
 instruction carries, operand order) without a GPU; that the kernel follows the
 same rules is checked on the GPU, by the same bodies among others."""
@@ -17,7 +18,9 @@ from oracle.hcsim import kernel as sim_kernel
 
 import random_bodies
 from fmap_emulator import run_fmap
-from test_kernel_frontend import FakeDev, MapTablesOnly, ctx, fmap_program   # noqa: F401  (ctx: a fixture)
+from test_kernel_frontend import (FakeDev, MapTablesOnly, POISON, ctx, fmap_program,   # noqa: F401  (ctx: a fixture)
+                                  row_stages, run_row_stages)
+from hc_amd.kernel_api import TraceError
 
 DT = typename.DT
 N, M = sym.N, sym.M
@@ -71,3 +74,60 @@ def test_random_bodies_mean_what_the_simulator_computes(ctx, monkeypatch):
         assert diff is None, f"seed {seed}: {text} ({np.dtype(dtype).name}): {diff}\n{fmap_program(p)}"
         tally["ok"] += 1
     assert tally["ok"] > SEEDS // 3, tally
+
+
+ROW_SEEDS = 800
+
+
+def row_body(deco, fn, per_row):
+    GM = sym.GM
+    if per_row:
+        @deco(work_shape=M, group_shape=GM)
+        def k(gr: CurrentGroup, a: Buffer[M, N, DT], b: Buffer[M, N, DT], out: Buffer[M, DT], g: GM):
+            m0, mb = gr.work_offset[0], gr.shape[0]
+            gr.store(out[m0:], fn(gr.load(a[m0:, :], shape=(mb, N)), gr.load(b[m0:, :], shape=(mb, N))))
+    else:
+        @deco(work_shape=M, group_shape=GM)
+        def k(gr: CurrentGroup, a: Buffer[M, N, DT], b: Buffer[M, N, DT], out: Buffer[M, N, DT], g: GM):
+            m0, mb = gr.work_offset[0], gr.shape[0]
+            gr.store(out[m0:, :], fn(gr.load(a[m0:, :], shape=(mb, N)), gr.load(b[m0:, :], shape=(mb, N))))
+    return k
+
+
+def test_random_row_bodies_mean_what_the_simulator_computes(ctx, monkeypatch):
+    """Elementwise expressions of two tiles and of sums, maxima, minima, means,
+    variances and standard deviations along their rows: the stages the binder
+    emits, run in NumPy with the row kernel's rules, store the elements the
+    simulator stores, NaN where it has NaN, and the same values to 1e-4 (sums
+    are added up in another order)."""
+    monkeypatch.setattr(rt, "GatherMap", MapTablesOnly)
+    tally = {"ok": 0, "refused": 0, "another kernel": 0}
+    for seed in range(ROW_SEEDS):
+        fn, text, per_row, (a, b) = random_bodies.row_case(seed)
+        shape = (a.shape[0],) if per_row else a.shape
+        want = np.full(shape, POISON)
+        with np.errstate(all="ignore"), warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            row_body(sim_kernel, fn, per_row)(a, b, want, 4)
+        fake = [FakeDev(a.shape, "float32"), FakeDev(b.shape, "float32"), FakeDev(shape, "float32")]
+        try:
+            plans = row_body(kernel, fn, per_row).plan(*fake, 4, ctx=ctx)
+        except (NoNativeKernel, TraceError):
+            tally["refused"] += 1
+            continue
+        if len(plans) != 1 or plans[0].fn is not rt.hcamdLaunchRowProgram:
+            tally["another kernel"] += 1
+            continue
+        (p,) = plans
+        by_ptr = {fake[0].ptr: a, fake[1].ptr: b}
+        operands = [by_ptr[p.args[4][i]] for i in range(p.args[7])]
+        with np.errstate(all="ignore"):
+            got = run_row_stages(row_stages(p), operands, (), np.float32, init=np.full(shape, POISON))
+        if got.shape != want.shape and got.ndim == 1 and (want[:, 1:] == POISON).all():
+            want = want[:, 0]                  # a (rows, 1) value stored to the window: its first column
+        where = f"seed {seed}: {text}\n{row_stages(p)}"
+        np.testing.assert_array_equal(got == POISON, want == POISON, err_msg=where)
+        np.testing.assert_array_equal(np.isnan(got), np.isnan(want), err_msg=where)
+        np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4, err_msg=where)
+        tally["ok"] += 1
+    assert tally["ok"] > ROW_SEEDS // 2, tally

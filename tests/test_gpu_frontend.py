@@ -1967,3 +1967,39 @@ def test_random_bodies_match_the_simulator():
         assert diff is None, f"seed {seed}: {text} ({np.dtype(dtype).name}, {rt.last_kernel_name()}): {diff}"
         tally["ok"] += 1
     assert tally["ok"] > 400, tally
+
+
+def test_random_row_bodies_match_the_simulator():
+    """Random elementwise expressions of two tiles and of reductions along their
+    rows (tests/random_bodies.py: sums, maxima, minima, means, variances,
+    standard deviations; divisions by zero, roots of negative numbers, NumPy
+    functions next to operators; data with zeros of both signs, and infinities
+    and NaN where no mean, var or std is taken) on the device against the host
+    executor: the same elements stored, NaN where it has NaN, values to 1e-4."""
+    import warnings
+    import random_bodies
+    from hc_amd.binding import NoNativeKernel
+    from hc_amd.kernel_api import TraceError
+    from test_fmap_programs_against_oracle import row_body
+    poison = np.float32(-77.0)
+    tally = {"ok": 0, "refused": 0}
+    for seed in range(500):
+        fn, text, per_row, (a, b) = random_bodies.row_case(seed)
+        shape = (a.shape[0],) if per_row else a.shape
+        want = np.full(shape, poison)
+        with np.errstate(all="ignore"), warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            row_body(sim_kernel, fn, per_row)(a, b, want, 4)
+        out = rt.to_device(np.full(shape, poison))
+        try:
+            row_body(kernel, fn, per_row)(rt.to_device(a), rt.to_device(b), out, 4)
+        except (NoNativeKernel, TraceError):
+            tally["refused"] += 1
+            continue
+        got = out.to_host()
+        where = f"seed {seed}: {text} ({rt.last_kernel_name()})"
+        assert_array_equal(got == poison, want == poison, err_msg=where)
+        assert_array_equal(np.isnan(got), np.isnan(want), err_msg=where)
+        assert_allclose(got, want, rtol=1e-4, atol=1e-4, err_msg=where)
+        tally["ok"] += 1
+    assert tally["ok"] > 400, tally

@@ -1024,7 +1024,7 @@ def run_row_stages(stages, inputs, columns=(), out_dtype=np.float32, init=None):
     rows = next(x.shape[0] for x in inputs if x.ndim == 2)
     n = next(x.shape[1] for x in inputs if x.ndim == 2)
     red = {k: (c.astype(f).reshape(rows, 1), np.zeros((rows, 1), bool)) for k, c in enumerate(columns)}
-    FUNC, SWAPPED = 0x200, 0x400
+    FUNC, SWAPPED, KEEP_DEAD = 0x200, 0x400, 0x800
     plain = {"add": lambda a, b: a + b, "sub": lambda a, b: a - b, "mul": lambda a, b: a * b,
              "div": lambda a, b: a / b, "max": np.maximum, "min": np.minimum}
     unary = {"neg": np.negative, "abs": np.abs, "sqrt": np.sqrt, "rint": np.rint, "exp": np.exp,
@@ -1094,7 +1094,8 @@ def run_row_stages(stages, inputs, columns=(), out_dtype=np.float32, init=None):
                         continue
                     if name in unary:
                         v, d = stack.pop()
-                        stack.append((unary[name](v).astype(f), d))
+                        keep = d if arg & KEEP_DEAD else never     # x ** 0.5 keeps a deactivated operand
+                        stack.append((np.where(keep, v, unary[name](v)).astype(f), d))
                         continue
                     if name in ("msqrt", "mlog", "masqrt", "powchk"):
                         v, d = stack.pop()
@@ -1139,7 +1140,9 @@ def run_row_stages(stages, inputs, columns=(), out_dtype=np.float32, init=None):
                 elif name == "clear":
                     bad[:] = False
                 elif name in unary:
-                    stack.append(unary[name](stack.pop()).astype(f))
+                    x = stack.pop()
+                    y = unary[name](x).astype(f)
+                    stack.append(np.where(bad, x, y) if frozen and arg & KEEP_DEAD else y)
                 elif name in ("msqrt", "mlog", "powchk"):
                     x = stack.pop()
                     if frozen and name != "powchk":
