@@ -2136,7 +2136,11 @@ def match_rows(dst_view, value, n_groups):
 class _PostCompiler(_MapCompiler):
     """Compiles what is done to a reduction's result (a chain of unary
     operations, casts and operations with constants) with that result as
-    operand 0."""
+    operand 0.  numpy.ma's forms: the result is a bare array, written whatever
+    its activity, with numpy.ma's fill values and dividends where an operation
+    fails."""
+
+    masked = True
 
     def __init__(self, n_groups, root: Tile):
         super().__init__(n_groups)
@@ -2151,6 +2155,11 @@ class _PostCompiler(_MapCompiler):
     def emit(self, t: Tile, out: list):
         if t is self.root:
             out.append(("in", 0, 0.0))
+        elif _is(t, "masqrt", 1):
+            # the standard deviation's numpy.ma.sqrt: where it fails (a variance that is
+            # not finite) it leaves its argument, which is what the root of that is
+            self.emit(t.args[0], out)
+            out.append(("sqrt", 0, 0.0))
         else:
             super().emit(t, out)
 
@@ -2235,6 +2244,10 @@ def _compile_col_reduce(red: Tile, root: Tile, n_groups, temps):
         if not pc.supported(root):
             raise NoNativeKernel(f"{root!r}: what follows a column reduction must be float32 / "
                                  "float16 arithmetic with constants")
+        if not _values_flow_plainly(root, finite=True):      # (as for rows: overflow and inf / NaN data aside)
+            raise NoNativeKernel(f"{root!r}: an operator follows an operation on a column reduction that "
+                                 "can fail (a division, a root, a logarithm); the stored value would be what "
+                                 "numpy.ma leaves under the deactivated result, which has no native code")
         tail: list = []
         pc.emit(root, tail)
         post = post + tail[1:] if post else tail

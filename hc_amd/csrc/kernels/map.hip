@@ -1266,6 +1266,20 @@ __device__ __forceinline__ void chain_scalar(uint32_t op, float &sv, float imm) 
   case OP_TANH: sv = tanh_selects(sv); break;
   case OP_R16: sv = round16(sv); break;
   case OP_SQ: sv = sv * sv; break;
+  // numpy.ma's forms, for a value that is stored whatever becomes of its activity:
+  // a failed quotient leaves the dividend, the functions their fill values
+  case OP_MDIVI: {
+    const float q = sv / imm;
+    sv = is_finite(q) ? q + 0.0f * sv : 0.0f + sv;
+    break;
+  }
+  case OP_RMDIVI: {
+    const float q = imm / sv;
+    sv = is_finite(q) ? q + 0.0f * imm : 0.0f + imm;
+    break;
+  }
+  case OP_MSQRT: sv = sv < 0.0f ? 0.0f : __builtin_sqrtf(sv); break;
+  case OP_MLOG: sv = sv <= 0.0f ? 1.0f : logf(sv); break;
   default: break;
   }
 }

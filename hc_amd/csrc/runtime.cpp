@@ -1896,7 +1896,7 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
     return 1;
   }
   if (!mapProgramOk(dev, who, prog, nInstr, nInputs, true) ||
-      (nPost && !mapProgramOk(dev, who, post, nPost, 1)))
+      (nPost && !mapProgramOk(dev, who, post, nPost, 1, true)))
     return 1;
   if (cols == 0)
     return 0;
@@ -2044,7 +2044,12 @@ int hcamdLaunchMapReduceCols(OlQueue q, int kind, const HcamdMapInstr *prog, siz
     switch (post[i].op) {
     case HCAMD_MAP_ADDI: case HCAMD_MAP_SUBI: case HCAMD_MAP_MULI: case HCAMD_MAP_DIVI:
     case HCAMD_MAP_RSUBI: case HCAMD_MAP_RDIVI: case HCAMD_MAP_NEG: case HCAMD_MAP_ABS:
-    case HCAMD_MAP_SQRT:
+    case HCAMD_MAP_SQRT: case HCAMD_MAP_MSQRT: case HCAMD_MAP_MLOG:
+      fp.op[fp.n] = post[i].op;
+      fp.imm[fp.n++] = post[i].imm;
+      break;
+    case HCAMD_MAP_MDIVI: case HCAMD_MAP_RMDIVI: // (the fp16 flag of `arg`: an fp32 result has none)
+      simple = (post[i].arg & 0x100u) == 0;
       fp.op[fp.n] = post[i].op;
       fp.imm[fp.n++] = post[i].imm;
       break;

@@ -172,3 +172,58 @@ def row_case(seed):
         for v in vals:
             v[~np.isfinite(v)] = 0.5
     return fn, text, per_row, vals
+
+
+def col_expression(rng, K):
+    """(function of two (M, GN) tiles holding whole columns, its text): reductions
+    down the columns of elementwise expressions, combined per column."""
+    def elem(d):
+        if d == 0 or rng.random() < 0.25:
+            return rng.choice(["ta", "tb"])
+        kind = rng.integers(0, 9)
+        x = elem(d - 1)
+        if kind <= 2:
+            return f"({x} {rng.choice(['+', '-', '*'])} {elem(d - 1)})"
+        if kind == 3:
+            return f"({x} / {elem(d - 1)})"
+        if kind == 4:
+            return f"np.{rng.choice(['maximum', 'minimum'])}({x}, {elem(d - 1)})"
+        if kind == 5:
+            return f"np.{rng.choice(['sqrt', 'log', 'abs', 'exp', 'square'])}({x})"
+        if kind == 6:
+            return f"(-{x})"
+        if kind == 7:
+            return f"({x} ** K({rng.choice(['2', '0.5'])}))"
+        return f"({x} {rng.choice(['+', '-', '*', '/'])} K({rng.choice(['0.5', '2.0', '-1.25', '0.0'])}))"
+
+    def fold():
+        red = rng.choice(["sum", "max", "min", "mean", "var", "std"])
+        extra = rng.choice(["", ", ddof=1"]) if red in ("var", "std") else ""
+        return f"{elem(int(rng.integers(0, 3)))}.{red}(axis=0{extra})"
+
+    text = fold()
+    bare_fold = text
+    shape = rng.integers(0, 6)
+    if shape == 0:
+        text = f"np.{rng.choice(['sqrt', 'abs', 'log'])}({text})"
+    elif shape == 1:
+        text = f"({text} {rng.choice(['*', '+', '/'])} K({rng.choice(['0.5', '2.0', '0.0'])}))"
+    elif shape == 2:
+        text = f"({text} {rng.choice(['+', '-', '*', '/'])} {fold()})"
+    elif shape == 3:
+        text = f"np.sqrt({text} / K(7) + K(1e-6))"
+    return eval(f"lambda ta, tb: {text}", {"np": np, "K": K}), text, text == bare_fold
+
+
+def col_case(seed):
+    """(function, text, two operand arrays (rows, n), columns per group)."""
+    rng = np.random.default_rng(seed)
+    fn, text, fold_only = col_expression(rng, np.float32)
+    (rows, n), gn = [((37, 70), 32), ((300, 200), 64), ((5, 64), 64)][seed % 3]
+    vals = [special_values(rng, (rows, n), np.float32) for _ in range(2)]
+    # (see row_case; what follows a fold is plain arithmetic where a column holds infinities
+    # or NaN and numpy.ma's there: the documented deviation, so those bodies get finite data too)
+    if seed % 2 or not fold_only or any(w in text for w in ("mean(", "var(", "std(")):
+        for v in vals:
+            v[~np.isfinite(v)] = 0.5
+    return fn, text, vals, gn

@@ -2003,3 +2003,45 @@ def test_random_row_bodies_match_the_simulator():
         assert_allclose(got, want, rtol=1e-4, atol=1e-4, err_msg=where)
         tally["ok"] += 1
     assert tally["ok"] > 400, tally
+
+
+def test_random_column_bodies_match_the_simulator():
+    """Random reductions down the columns of elementwise expressions, with what
+    may follow them per column (tests/random_bodies.py: a root, a logarithm, a
+    division by zero, a second fold), on the device against the host executor:
+    the same NaNs, values to 1e-4.  numpy.sqrt / numpy.log of a fold give
+    numpy.ma's fill values where the domain fails and a failed division leaves
+    its dividend, as the result is a bare array that is written in full."""
+    import warnings
+    import random_bodies
+    from hc_amd.binding import NoNativeKernel
+    from hc_amd.kernel_api import TraceError
+    M, N, GN = sym.M, sym.N, sym.GN
+    poison = np.float32(-77.0)
+    tally = {"ok": 0, "refused": 0}
+    for seed in range(400):
+        fn, text, (a, b), gn = random_bodies.col_case(seed)
+        n = a.shape[1]
+
+        def body(gr: CurrentGroup, x: Buffer[M, N, DT], y: Buffer[M, N, DT], out: Buffer[N, DT], g: GN):
+            n0 = gr.id[0] * GN
+            gr.store(out[n0:], fn(gr.load(x[:, n0:], shape=(M, GN)), gr.load(y[:, n0:], shape=(M, GN))))
+
+        deco = dict(work_shape=cdiv(n, gn), group_shape=1, literals={GN})
+        want = np.full(n, poison)
+        with np.errstate(all="ignore"), warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            sim_kernel(**deco)(body)(a, b, want, gn)
+        out = rt.to_device(np.full(n, poison))
+        try:
+            kernel(**deco)(body)(rt.to_device(a), rt.to_device(b), out, gn)
+        except (NoNativeKernel, TraceError):
+            tally["refused"] += 1
+            continue
+        got = out.to_host()
+        where = f"seed {seed}: {text} ({rt.last_kernel_name()})"
+        assert_array_equal(got == poison, want == poison, err_msg=where)
+        assert_array_equal(np.isnan(got), np.isnan(want), err_msg=where)
+        assert_allclose(got, want, rtol=1e-4, atol=1e-4, err_msg=where)
+        tally["ok"] += 1
+    assert tally["ok"] > 200, tally
