@@ -2025,7 +2025,9 @@ def match_rows(dst_view, value, n_groups):
         comp.prepare(value, True)
         slot = comp.slot_of(value)
         program = [("red", slot, 0.0)] if slot is not None else comp.program(value, scalar=True)
-        comp.stages.append(("store_col", 0, program))
+        # (a tile instead -- a per-row operand on the left of the tile operators -- keeps
+        # its deactivated rows out of the store: dst 1)
+        comp.stages.append(("store_col", 0 if value.attrs.get("plain") else 1, program))
     else:
         program = comp.program(value)
         if value.attrs.get("plain") and _maybe_masked(value):

@@ -1519,7 +1519,7 @@ HCAMD_REDUCE_COLS(hcamd_map_reduce_cols_n1u4, 1, 4)
 //                    scalar `dst`
 //   STORE            the program's value at every element is stored to the
 //                    output tile
-//   STORE_COL        as SCALAR, stored to out[row * ldo]
+//   STORE_COL        as SCALAR, stored to out[row * ldo] (dst 1: unless the row's result is deactivated)
 //
 // A program reaches row scalars through the RED opcodes, which are rewritten on
 // the fly into the immediate forms of the interpreter with the scalar as the
@@ -1978,7 +1978,8 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
         const uint32_t bit = 1u << (st.dst & (kMaxRed - 1));
         cells[st.dst & (kMaxRed - 1)] = uniform(res.value);
         dead = res.dead ? dead | bit : dead & ~bit;
-      } else if (row_live && lane == 0) {
+      } else if (row_live && lane == 0 && !(st.dst && res.dead)) {
+        // (dst 1: the value is a tile, whose deactivated rows are not stored)
         store_elem(a.out, out_f16, row * a.ldo, res.value);
       }
       continue;

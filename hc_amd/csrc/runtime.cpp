@@ -2321,6 +2321,7 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
     }
     // (a STORE_COL stage that can fail stores what numpy.ma leaves: the scalar interpreter's business too)
     tracking = tracking || canDie || frozen || st.kind == HCAMD_ROW_COUNT ||
+               (st.kind == HCAMD_ROW_STORE_COL && st.dst != 0) ||
                (!perElement && (hasForms || readsDeadable));
     pc += st.nInstr;
   }

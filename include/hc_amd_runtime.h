@@ -528,7 +528,9 @@ int hcamdLaunchMapReduceColsNoAlloc(OlQueue q, int kind, const HcamdMapInstr *pr
  *   SCALAR         the program reads row scalars only; its value becomes row
  *                  scalar `dst`
  *   STORE          the value at every element is stored to out[row, col]
- *   STORE_COL      as SCALAR, stored to out[row * ldo]
+ *   STORE_COL      as SCALAR, stored to out[row * ldo]; with dst = 1 a row whose
+ *                  result is deactivated is not stored (the value is a tile: a
+ *                  per-row operand on the left of the tile operators)
  *   COUNT          the number of active elements of the value (see below) becomes
  *                  row scalar `dst` (fp32)
  * Exactly one stage stores, and it is the last.  Programs read row scalars with

@@ -103,15 +103,18 @@ def difference(got, want, text):
     return None
 
 
-def row_expression(rng, K):
+def row_expression(rng, K, leaves=("ta", "tb")):
     """(function of two 2-D tiles, its text, result is one value per row): an
     elementwise expression of the tiles and of row scalars (sum, max, min, mean,
-    var, std along axis 1 of smaller elementwise expressions)."""
+    var, std along axis 1 of smaller elementwise expressions).  `leaves` may
+    name more operands (a row vector `w`, a per-row operand `s[:, None]`)."""
     red_count = [0]
 
     def scalar(d):
         red = rng.choice(["sum", "max", "min", "mean", "var", "std"])
         inner = elem(d, False)
+        while "ta" not in inner and "tb" not in inner:      # (a reduction needs a 2-D tile under it)
+            inner = elem(d, False)
         if red in ("var", "std"):
             ddof = rng.choice(["", ", ddof=1"])
             return f"{inner}.{red}(axis=1, keepdims=True{ddof})"
@@ -122,7 +125,7 @@ def row_expression(rng, K):
             if scalars and red_count[0] < 3 and rng.random() < 0.45:
                 red_count[0] += 1
                 return scalar(max(d - 1, 0))
-            return rng.choice(["ta", "tb"])
+            return rng.choice(list(leaves))
         kind = rng.integers(0, 12)
         x = elem(d - 1, scalars)
         if kind <= 2:
@@ -148,14 +151,33 @@ def row_expression(rng, K):
         red_count[0] = 0
         if per_row:
             inner = elem(int(rng.integers(1, 3)), False)
+            if "ta" not in inner and "tb" not in inner:
+                continue
             text = f"{inner}.{rng.choice(['sum', 'max', 'min', 'mean', 'var', 'std'])}(axis=1)"
             if rng.random() < 0.4:
-                text = f"({text} {rng.choice(['+', '*', '/'])} {elem(1, False)}.{rng.choice(['sum', 'max', 'mean'])}(axis=1))"
+                other = elem(1, False)
+                if "ta" in other or "tb" in other:
+                    text = f"({text} {rng.choice(['+', '*', '/'])} {other}.{rng.choice(['sum', 'max', 'mean'])}(axis=1))"
+            if rng.random() < 0.3 and "s[:, None]" in leaves:
+                text = f"(s {rng.choice(['+', '*', '/', '-'])} {text})"
             break
         text = elem(int(rng.integers(1, 4)), True)
         if red_count[0]:
             break
-    return eval(f"lambda ta, tb: {text}", {"np": np, "K": K}), text, per_row
+    return eval(f"lambda ta, tb, w=None, s=None: {text}", {"np": np, "K": K}), text, per_row
+
+
+def vector_case(seed):
+    """(function of a tile, a second tile, a row vector w and a per-row operand s,
+    text, per_row, the four arrays): row_case with operands that broadcast."""
+    rng = np.random.default_rng(seed)
+    fn, text, per_row = row_expression(rng, np.float32, ("ta", "ta", "tb", "w", "s[:, None]"))
+    rows, n = [(9, 5), (13, 200), (6, 1031)][seed % 3]
+    vals = [special_values(rng, shape, np.float32) for shape in ((rows, n), (rows, n), (n,), (rows,))]
+    if seed % 2 or any(x in text for x in ("mean(", "var(", "std(")):
+        for v in vals:
+            v[~np.isfinite(v)] = 0.5
+    return fn, text, per_row, vals
 
 
 def row_case(seed):

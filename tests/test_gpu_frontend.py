@@ -2045,3 +2045,56 @@ def test_random_column_bodies_match_the_simulator():
         assert_allclose(got, want, rtol=1e-4, atol=1e-4, err_msg=where)
         tally["ok"] += 1
     assert tally["ok"] > 200, tally
+
+
+def test_random_bodies_with_a_row_vector_and_a_per_row_operand_match_the_simulator():
+    """The random row bodies with two more operands that broadcast: a row vector
+    (a weight, a bias) and a per-row operand (a scale per row), as in the
+    reference's normalisation and softmax-with-temperature bodies.  A per-row
+    result that is a tile (the per-row operand on the left of the tile operators)
+    keeps its deactivated rows out of the store."""
+    import warnings
+    import random_bodies
+    from hc_amd.binding import NoNativeKernel
+    from hc_amd.kernel_api import TraceError
+    M, N, GM = sym.M, sym.N, sym.GM
+    poison = np.float32(-77.0)
+
+    def bodies(deco, fn, per_row):
+        if per_row:
+            @deco(work_shape=M, group_shape=GM)
+            def k(gr: CurrentGroup, a: Buffer[M, N, DT], b: Buffer[M, N, DT], w: Buffer[N, DT], s: Buffer[M, DT],
+                  out: Buffer[M, DT], g: GM):
+                m0, mb = gr.work_offset[0], gr.shape[0]
+                gr.store(out[m0:], fn(gr.load(a[m0:, :], shape=(mb, N)), gr.load(b[m0:, :], shape=(mb, N)),
+                                      gr.load(w[:], shape=(N,)), gr.load(s[m0:], shape=(mb,))))
+        else:
+            @deco(work_shape=M, group_shape=GM)
+            def k(gr: CurrentGroup, a: Buffer[M, N, DT], b: Buffer[M, N, DT], w: Buffer[N, DT], s: Buffer[M, DT],
+                  out: Buffer[M, N, DT], g: GM):
+                m0, mb = gr.work_offset[0], gr.shape[0]
+                gr.store(out[m0:, :], fn(gr.load(a[m0:, :], shape=(mb, N)), gr.load(b[m0:, :], shape=(mb, N)),
+                                         gr.load(w[:], shape=(N,)), gr.load(s[m0:], shape=(mb,))))
+        return k
+
+    tally = {"ok": 0, "refused": 0}
+    for seed in range(400):
+        fn, text, per_row, vals = random_bodies.vector_case(seed)
+        shape = (vals[0].shape[0],) if per_row else vals[0].shape
+        want = np.full(shape, poison)
+        with np.errstate(all="ignore"), warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            bodies(sim_kernel, fn, per_row)(*vals, want, 4)
+        out = rt.to_device(np.full(shape, poison))
+        try:
+            bodies(kernel, fn, per_row)(*[rt.to_device(v) for v in vals], out, 4)
+        except (NoNativeKernel, TraceError):
+            tally["refused"] += 1
+            continue
+        got = out.to_host()
+        where = f"seed {seed}: {text} ({rt.last_kernel_name()})"
+        assert_array_equal(got == poison, want == poison, err_msg=where)
+        assert_array_equal(np.isnan(got), np.isnan(want), err_msg=where)
+        assert_allclose(got, want, rtol=1e-4, atol=1e-4, err_msg=where)
+        tally["ok"] += 1
+    assert tally["ok"] > 300, tally

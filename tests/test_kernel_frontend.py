@@ -1193,6 +1193,8 @@ def run_row_stages(stages, inputs, columns=(), out_dtype=np.float32, init=None):
                     dead = ~(red[live_slot][0] > 0)
                 if kind == "scalar":
                     red[dst] = (v, dead)
+                elif dst == 1 and result is not None:      # a tile: deactivated rows are not stored
+                    result = np.where(dead.reshape(rows), result, v.reshape(rows).astype(out_dtype))
                 else:
                     result = v.reshape(rows).astype(out_dtype)
                 continue
