@@ -133,12 +133,21 @@ def _row_reduce(t: Tile, op: str):
 # ---------------------------------------------------------------------------
 # Patterns.  Each returns a function(memrefs, ctx) -> list[rt.Plan] or None.
 # ---------------------------------------------------------------------------
-def _check_same_window(wins):
+def _check_same_window(wins, value: Tile = None):
+    """The window every operand and the output walk.  With `value` (what is
+    stored) a tile -- operators of loads, stored where active -- the arrays may
+    end at different places: an element is active only where every load was
+    inside its array, and stored only where the output has it, so the common
+    part of the windows is the whole of the work.  (A bare array is written in
+    full, with the 0 a load puts outside its array: the windows must agree.)"""
     w0 = wins[0]
+    shrink = value is not None and not value.attrs.get("plain")
+    extent = w0.extent
     for w in wins[1:]:
-        if w.extent != w0.extent or w.driver != w0.driver:
+        if w.driver != w0.driver or len(w.extent) != len(extent) or (w.extent != extent and not shrink):
             raise NoNativeKernel("loads and the store walk different windows")
-    return w0
+        extent = tuple(min(a, b) for a, b in zip(extent, w.extent))
+    return Window(w0.buffer, extent, w0.driver, w0.tile) if extent != w0.extent else w0
 
 
 def _region2d(extent):
@@ -221,7 +230,7 @@ def match_add(dst_view, value, n_groups):
         return None
     wins = [window_of(a.attrs["view"], a.shape, n_groups) for a in value.args]
     wins.append(window_of(dst_view, value.shape, n_groups))
-    w = _check_same_window(wins)
+    w = _check_same_window(wins, value)
 
     general = match_map(dst_view, value, n_groups)
 
@@ -1053,7 +1062,7 @@ def match_map(dst_view, value, n_groups):
         return None
     wins = [window_of(t.attrs["view"], t.shape, n_groups) for _, _, t in comp.inputs]
     wins.append(window_of(dst_view, value.shape, n_groups))
-    w = _check_same_window(wins)
+    w = _check_same_window(wins, value)
     if len(w.extent) > 2:
         raise NoNativeKernel("only 1-D and 2-D buffers have native kernels")
     types = [rt.F16 if t.dtype_name == "float16" else rt.F32 for _, _, t in comp.inputs]
@@ -1111,6 +1120,8 @@ def match_imap(dst_view, value, n_groups):
             return needs[id(t)]
         if _is(t, "astype", 1) or _is(t, "active", 1) or (t.op in _IMAP_UNARY and len(t.args) == 1):
             n = need(t.args[0])
+        elif _is(t, "where", 3):
+            n = max(need(t.args[0]), 1 + need(t.args[1]), 2 + need(t.args[2]))
         elif t.op in _IMAP_BINARY and len(t.args) == 2:
             a, b = need(t.args[0]), need(t.args[1])
             if _IMAP_BINARY[t.op] in mirrored:
@@ -1159,6 +1170,22 @@ def match_imap(dst_view, value, n_groups):
             return ok
         if _is(t, "astype", 1) and t.dtype_name == "int32" and t.args[0].dtype_name == "bool":
             return emit(t.args[0])                 # 0 / 1 as int32: the same bits
+        if _is(t, "where", 3) and t.dtype_name == "int32":
+            # numpy.where picks from the values and returns a plain array.  The kernel
+            # keeps one activity flag per element and, under a failed // or %, the
+            # value numpy.ma leaves (the dividend, 1): enough for the selection of a
+            # whole stored value from operands that are such a quotient or cannot fail
+            # (`numpy.where(b != 0, a // b, 0)`), not for arithmetic on top of them.
+            def leaves_numpy_mas_value(x):
+                return not _maybe_masked(x) or (x.op in ("floordiv", "mod") and not x.attrs.get("func") and
+                                                not any(_maybe_masked(z) for z in x.args))
+            if t is not value or _maybe_masked(t.args[0]) or not all(leaves_numpy_mas_value(x) for x in t.args[1:]):
+                raise NoNativeKernel("numpy.where of integer tiles: only as the whole stored value, chosen by a "
+                                     "condition that cannot be deactivated from operands that are a // or % "
+                                     "of such values or cannot be deactivated either")
+            ok = all([emit(x) for x in t.args])
+            program.append(("select", 0, 0))
+            return ok
         if _is(t, "active", 1):
             # tile.mask: the kernel keeps one activity flag per element, that of
             # the whole expression so far, so the mask is taken of a whole expression
@@ -1184,7 +1211,7 @@ def match_imap(dst_view, value, n_groups):
         return None                                # a plain copy
     wins = [window_of(t.attrs["view"], t.shape, n_groups) for t in loads]
     wins.append(window_of(dst_view, value.shape, n_groups))
-    w = _check_same_window(wins)
+    w = _check_same_window(wins, value)
     if len(w.extent) > 2:
         raise NoNativeKernel("only 1-D and 2-D buffers have native kernels")
     prog = list(program)
@@ -1384,7 +1411,7 @@ def match_fmap(dst_view, value, n_groups):
     loads, prog = compiled
     wins = [window_of(t.attrs["view"], t.shape, n_groups) for t in loads]
     wins.append(window_of(dst_view, value.shape, n_groups))
-    w = _check_same_window(wins)
+    w = _check_same_window(wins, value)
     if len(w.extent) > 2:
         raise NoNativeKernel("only 1-D and 2-D buffers have native kernels")
     types = [{"float16": rt.F16, "int32": rt.I32}.get(t.dtype_name, rt.F32) for t in loads]
@@ -1636,9 +1663,11 @@ def match_general_windows(dst_view, value, n_groups):
     lowered = _gathered_form(value)
     if lowered is None:
         return None
-    if value.attrs.get("plain") or lowered.attrs.get("plain"):
+    if copy and (value.attrs.get("plain") or lowered.attrs.get("plain")):
         # A bare numpy.ma array is stored in full: where a load was outside its
-        # buffer the reference writes the value it initialises tiles with.
+        # buffer the reference writes the value it initialises tiles with (0), which
+        # the copying form of the kernel, that moves elements, does not.  (A computed
+        # value is computed from that 0 by the kernel as by the reference.)
         total = math.prod(n_groups)
         elems = math.prod(value.shape)
         if total * elems > 16 * _GATHER_MAP_MAX_DESTS:

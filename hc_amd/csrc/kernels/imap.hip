@@ -14,6 +14,9 @@
 //   * << and >> with a count outside 0..31 give 0 (>> of a negative value: -1),
 //     which is what NumPy defines; >> is arithmetic;
 //   * comparisons give 0 / 1.
+//   * IOP_SELECT is numpy.where: it picks from the values, whatever became of
+//     their activity (the dividend under a failed //, 1 under a failed %), and
+//     the result is a plain array, every element of which is stored.
 // The evaluation stack has four entries held in four fixed registers per
 // element (top of stack in t0; a push moves the others down, a pop moves them
 // up), so no register is ever indexed.  A lane owns four consecutive elements
@@ -34,6 +37,7 @@ enum : uint32_t {
   IOP_LT = 15, IOP_LE = 16, IOP_EQ = 17, IOP_NE = 18, IOP_GE = 19, IOP_GT = 20,
   IOP_NEG = 21, IOP_ABS = 22, IOP_NOT = 23, IOP_LNOT = 24,
   IOP_ACTIVE = 25, // 1 where the element is still active, else 0; the element is active again
+  IOP_SELECT = 26, // numpy.where(c, a, b) with c, a, b the three top entries (b on top): the element is active again
 };
 
 struct Instr {
@@ -58,11 +62,13 @@ __device__ __forceinline__ int32_t wrap_add(int32_t a, int32_t b) { return (int3
 __device__ __forceinline__ int32_t wrap_sub(int32_t a, int32_t b) { return (int32_t)((uint32_t)a - (uint32_t)b); }
 __device__ __forceinline__ int32_t wrap_mul(int32_t a, int32_t b) { return (int32_t)((uint32_t)a * (uint32_t)b); }
 
-// floor division and the remainder that goes with it; ok is cleared for b == 0
+// floor division and the remainder that goes with it; ok is cleared for b == 0,
+// and the value is what numpy.ma leaves under the deactivated result (the
+// dividend of //, the fill value 1 of %), which numpy.where may pick up
 __device__ __forceinline__ int32_t floor_div(int32_t a, int32_t b, bool &ok) {
   if (b == 0) {
     ok = ok && a == INT32_MIN;
-    return 0;
+    return a == INT32_MIN ? 0 : a;
   }
   if (b == -1)
     return wrap_sub(0, a); // INT_MIN / -1 wraps instead of trapping
@@ -74,7 +80,7 @@ __device__ __forceinline__ int32_t floor_div(int32_t a, int32_t b, bool &ok) {
 __device__ __forceinline__ int32_t floor_mod(int32_t a, int32_t b, bool &ok) {
   if (b == 0) {
     ok = ok && a == INT32_MIN;
-    return 0;
+    return a == INT32_MIN ? 0 : 1;
   }
   if (b == -1)
     return 0;
@@ -170,6 +176,14 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_imap_i32(IMapArgs a) {
 #pragma unroll
       for (int e = 0; e < kV; ++e) {
         t0[e] = ok[e] ? 1 : 0;
+        ok[e] = true;
+      }
+    } else if (op == IOP_SELECT) {
+      // numpy.where returns a plain array: chosen from the values, every element active
+#pragma unroll
+      for (int e = 0; e < kV; ++e) {
+        t0[e] = t2[e] != 0 ? t1[e] : t0[e];
+        t1[e] = t3[e];
         ok[e] = true;
       }
     } else if (op >= IOP_NEG) {

@@ -1541,12 +1541,13 @@ int hcamdLaunchIMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
       return 1;
     }
     const bool push = op == HCAMD_IMAP_IN || op == HCAMD_IMAP_CONST;
-    const bool unary = op >= HCAMD_IMAP_NEG;
-    if (sp < (push ? 0 : unary ? 1 : 2)) {
+    const bool select = op == HCAMD_IMAP_SELECT; // three entries in, one out
+    const bool unary = op >= HCAMD_IMAP_NEG && !select;
+    if (sp < (push ? 0 : unary ? 1 : select ? 3 : 2)) {
       dev->report("%s: stack underflow at %zu", who, i);
       return 1;
     }
-    sp += push ? 1 : unary ? 0 : -1;
+    sp += push ? 1 : unary ? 0 : select ? -2 : -1;
     if (sp > 4) {
       dev->report("%s: stack deeper than 4 at %zu", who, i);
       return 1;

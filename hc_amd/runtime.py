@@ -631,7 +631,7 @@ U8 = 5
 IMAP_OPS = {"in": 1, "const": 2, "add": 3, "sub": 4, "mul": 5, "floordiv": 6, "mod": 7, "min": 8,
             "max": 9, "and": 10, "or": 11, "xor": 12, "shl": 13, "shr": 14, "lt": 15, "le": 16,
             "eq": 17, "ne": 18, "ge": 19, "gt": 20, "neg": 21, "abs": 22, "not": 23, "lnot": 24,
-            "active": 25}
+            "active": 25, "select": 26}
 
 
 def plan_imap(program, inputs, out, out_bool=False) -> Plan:

@@ -378,7 +378,11 @@ enum HcamdIMapOp {
   HCAMD_IMAP_NEG = 21, HCAMD_IMAP_ABS = 22, HCAMD_IMAP_NOT = 23, HCAMD_IMAP_LNOT = 24,
   HCAMD_IMAP_ACTIVE = 25, /* top = 1 where the element is still active, else 0; the element is active again
                              (`tile.mask`, python/hckernel/kernel_api.py:117-119) */
-  HCAMD_IMAP_COUNT = 26
+  /* numpy.where(c, a, b) with c, a, b the three top entries (b on top): picked from
+   * the values (the dividend under a failed //, 1 under a failed %); the element
+   * is active again, as NumPy returns a plain array */
+  HCAMD_IMAP_SELECT = 26,
+  HCAMD_IMAP_COUNT = 27
 };
 int hcamdLaunchIMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
                     const void *const *inputs, const size_t *inputLd, size_t nInputs,

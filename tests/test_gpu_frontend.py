@@ -2098,3 +2098,45 @@ def test_random_bodies_with_a_row_vector_and_a_per_row_operand_match_the_simulat
         assert_allclose(got, want, rtol=1e-4, atol=1e-4, err_msg=where)
         tally["ok"] += 1
     assert tally["ok"] > 300, tally
+
+
+def test_numpy_where_of_int32_tiles():
+    """numpy.where of integer tiles as the stored value (the guarded division
+    `numpy.where(b != 0, a // b, 0)` among them): picked from the values, the
+    dividend under a failed //, 1 under a failed %, every element stored; same
+    bodies on the host executor.  Arithmetic on top of a quotient inside the
+    selection is refused."""
+    from hc_amd.binding import NoNativeKernel
+    N = sym.N
+    I = np.int32
+    rng = np.random.default_rng(31)
+    n = 5003
+    a = rng.integers(-40, 41, n).astype(I)
+    b = rng.integers(-3, 4, n).astype(I)            # a seventh of the divisors are zero
+    a[:3] = [np.iinfo(I).min, np.iinfo(I).min, 7]
+    b[:3] = [0, -1, 0]
+    forms = {
+        "guarded": lambda x, y: np.where(y != I(0), x // y, I(0)),
+        "unguarded": lambda x, y: np.where(x < y, x // y, x % y),
+        "plain": lambda x, y: np.where(x * y > I(10), x - y, y),
+        "numbers": lambda x, y: np.where(x >= y, I(1), I(-1)),
+    }
+    for name, fn in forms.items():
+        def body(gr: CurrentGroup, x: Buffer[N, DT], y: Buffer[N, DT], out: Buffer[N, DT]):
+            o = gr.work_offset[0]
+            gr.store(out[o:], fn(gr.load(x[o:], shape=gr.shape), gr.load(y[o:], shape=gr.shape)))
+        want = np.full(n, -777, I)
+        with np.errstate(all="ignore"):
+            sim_kernel(work_shape=N, group_shape=256)(body)(a, b, want)
+        out = rt.to_device(np.full(n, -777, I))
+        kernel(work_shape=N, group_shape=256)(body)(rt.to_device(a), rt.to_device(b), out)
+        assert rt.last_kernel_name() == "hcamd_imap_i32"
+        assert_array_equal(out.to_host(), want, err_msg=name)
+        assert (want != -777).all()
+
+    def on_top(gr: CurrentGroup, x: Buffer[N, DT], y: Buffer[N, DT], out: Buffer[N, DT]):
+        o = gr.work_offset[0]
+        tx, ty = gr.load(x[o:], shape=gr.shape), gr.load(y[o:], shape=gr.shape)
+        gr.store(out[o:], np.where(tx < ty, tx // ty + I(1), ty))
+    with pytest.raises(NoNativeKernel, match="numpy.where of integer tiles"):
+        kernel(work_shape=N, group_shape=256)(on_top)(rt.to_device(a), rt.to_device(b), rt.to_device(a))

@@ -421,6 +421,30 @@ def _ma_special(rng, n, dtype):
     return x
 
 
+def test_imap_select_picks_from_values_numpy_ma_leaves(ctx):
+    """hcamdLaunchIMap, SELECT (numpy.where): the three top entries, condition
+    deepest; the element is active again, and under a failed // or % it finds
+    what numpy.ma leaves there (the dividend, 1; INT_MIN // 0 stays NumPy's 0)."""
+    I = np.int32
+    a = np.array([7, -7, 0, 5, np.iinfo(I).min, 9, -3, 4, 11], I)
+    b = np.array([0, 0, 0, 2, 0, -4, 3, 0, 5], I)
+    F = lambda name, arg=0, imm=0: (name, arg, imm)
+    da, db = dev(a), dev(b)
+    for op, left in (("floordiv", np.array([7, -7, 0, 2, 0, -3, -1, 4, 2], I)),
+                     ("mod", np.array([1, 1, 1, 1, 0, -3, 0, 1, 1], I))):
+        out = poisoned((9,), I)
+        # where(1, a op b, -5): everything comes from the quotient / remainder
+        rt.plan_imap([F("const", 0, 1), F("in", 0), F("in", 1), F(op), F("const", 0, -5), F("select")],
+                     [da, db], out).launch(sync=True)
+        assert_array_equal(out.to_host(), left, err_msg=op)
+    out = poisoned((9,), I)
+    rt.plan_imap([F("in", 1), F("const", 0, 0), F("ne"), F("in", 0), F("in", 1), F("floordiv"), F("const", 0, 0),
+                  F("select")], [da, db], out).launch(sync=True)
+    assert_array_equal(out.to_host(), np.array([0, 0, 0, 2, 0, -3, -1, 0, 2], I))
+    with pytest.raises(rt.HcRuntimeError, match="underflow"):
+        rt.plan_imap([F("in", 0), F("in", 1), F("select")], [da, db], out).launch(sync=True)
+
+
 def test_fmap_select_tanh_and_int32_operands(ctx):
     """hcamdLaunchFMap: SELECT takes its values whatever their activity and gives an
     active result (numpy.where returns a plain array), an int32 operand is
