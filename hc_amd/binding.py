@@ -761,6 +761,8 @@ def _maybe_masked(t: Tile, memo=None) -> bool:
     if t.uid not in memo:
         if _is(t, "load") or _const(t) or t.op in ("count", "where"):
             memo[t.uid] = False                  # (numpy.where returns a plain array)
+        elif _is(t, "merge", 2):
+            memo[t.uid] = _maybe_masked(t.args[0], memo)     # active wherever the tile was
         else:
             memo[t.uid] = _masks(t) or any(_maybe_masked(a, memo) for a in t.args if isinstance(a, Tile))
     return memo[t.uid]
@@ -1264,6 +1266,8 @@ def _compile_fmap(value, mapped=False):
             n = max(need(t.args[0]), 1 + need(t.args[1]), 2 + need(t.args[2]))
         elif _is(t, "clip", 1):
             n = max(need(t.args[0]), 2)          # the bounds are pushed next to the value
+        elif _is(t, "merge", 2):
+            n = max(need(t.args[0]), need(t.args[1]) + 1)
         elif len(t.args) == 1:
             n = need(t.args[0])
         elif len(t.args) == 2:
@@ -1320,6 +1324,16 @@ def _compile_fmap(value, mapped=False):
         if _is(t, "active", 1):
             ok = emit(t.args[0])                   # tile.mask: the entry's activity as 0 / 1
             program.append(("active", 0, 0.0))
+            return ok
+        if _is(t, "merge", 2):
+            if t.dtype_name not in _MAP_FLOATS:
+                return False
+            for x in t.args:
+                if _const(x):
+                    program.append(("const", 0, _round_to(_const_value(x), t.dtype_name)))
+                else:
+                    ok = emit(x) and ok
+            program.append(("merge", 0, 0.0))
             return ok
         if _is(t, "clip", 1):
             ok = emit(t.args[0])
@@ -2731,18 +2745,36 @@ def simplify(t: Tile, memo=None) -> Tile:
     if _is(out, "slice", 1) and _const(out.args[0]) and _const_value(out.args[0]) is not None:
         # part of an allocated tile (CurrentGroup.vec with a shape): the same constant
         out = _const_tile(out.shape, out.dtype_name, out.args[0])
-    elif _is(out, "update", 2) and _const(out.args[0]) and \
-            all(k == (0, n) for k, n in zip(out.attrs["key"], out.shape)):
-        # `tile[:] = value` on a freshly allocated tile (python/hckernel/kernel_api.py:125-131:
-        # value where it is active, the allocator's fill elsewhere, every element active)
+    elif _is(out, "update", 2) and all(k == (0, n) for k, n in zip(out.attrs["key"], out.shape)):
+        # `tile[:] = value`, which is also what the in-place operators do
+        # (python/hckernel/kernel_api.py:123-145): a tile's active elements are taken
+        # and become active, the rest of the tile stays as it is; anything else (a number,
+        # a bare array) overwrites the whole tile and activates it.
         old, value = out.args
         if _const(value) and _const_value(value) is not None:
             out = _const_tile(out.shape, out.dtype_name, value)
-        elif value.shape == out.shape and not value.attrs.get("plain"):
+        elif value.shape == out.shape:
             filled = value if value.dtype_name == out.dtype_name else \
-                Tile("astype", (value,), out.shape, out.dtype_name)
-            memo.setdefault("overlays", []).append(filled)
-            out = filled
+                Tile("astype", (value,), out.shape, out.dtype_name, **value._plain_kw())
+            if value.attrs.get("plain"):
+                if not _const(old) and out.dtype_name in _MAP_FLOATS:
+                    # every element is overwritten with the bare array's value, whatever its
+                    # activity there, and is active: a selection that always takes the value
+                    one = Tile("const", (), (), out.dtype_name, value=1.0, weak=False)
+                    zero = Tile("const", (), (), out.dtype_name, value=0.0, weak=False)
+                    out = Tile("where", (one, filled, zero), out.shape, out.dtype_name)
+            elif _maybe_masked(value) and out.dtype_name in _MAP_FLOATS:
+                # elements the data can deactivate keep what the tile held
+                out = Tile("merge", (old, filled), out.shape, out.dtype_name)
+            elif _const(old):
+                # on a freshly allocated tile: value where it is active, the allocator's fill
+                # elsewhere, every element active (a load that reaches past its array is what
+                # can be inactive: the store's window must not reach further than the loads')
+                if _has_elementwise_load(filled):
+                    memo.setdefault("overlays", []).append(filled)
+                out = filled
+            else:
+                out = filled                     # active wherever the tile was: nothing is kept
     if out.op == "count" and _is_reduction(out) and not _maybe_masked(out.args[0]):
         # nothing can deactivate an element: the number of active elements is the
         # number of elements (tiles hold whole rows / columns of their arrays)
@@ -2756,6 +2788,17 @@ def simplify(t: Tile, memo=None) -> Tile:
         out = Tile("const", (), (), "float32", value=float(n), weak=False, exact=int(n), counted=True)
     memo[id(t)] = out
     return out
+
+
+def _has_elementwise_load(t: Tile) -> bool:
+    """A load whose activity reaches t element by element (not through a matrix
+    product, numpy.where, tile.mask or a reduction, whose results are active
+    everywhere)."""
+    if _is(t, "load") or _is(t, "mapped_load"):
+        return True
+    if t.op in ("dot", "where", "active") or _is_reduction(t):
+        return False
+    return any(_has_elementwise_load(a) for a in t.args if isinstance(a, Tile))
 
 
 def _const_value(t: Tile):
@@ -3048,7 +3091,7 @@ def bind(stores, n_groups, atomics=(), mapped_stores=(), id_stores=(), group_sha
                 raise NoNativeKernel("a body that both stores tiles and accumulates "
                                      "atomically has no native kernel")
             return [mk for proxy, index, value in atomics
-                    for mk in match_sum(proxy, index, value, n_groups)]
+                    for mk in match_sum(proxy, index, simplify(value, memo), n_groups)]
         makers = list(id_makers)
         for proxy, index, value, accumulate in cell_stores:
             makers.append(match_group_cells(proxy, index, simplify(value, memo), accumulate, n_groups))

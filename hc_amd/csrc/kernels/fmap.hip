@@ -75,6 +75,10 @@ enum : uint32_t {
   // log2 and log10 have numpy.ma's domain like log (inactive with the value 1)
   FOP_FLOOR = 30, FOP_CEIL = 31, FOP_TRUNC = 32, FOP_SIGN = 33, FOP_EXP2 = 34, FOP_LOG2 = 35,
   FOP_LOG10 = 36, FOP_LOG1P = 37, FOP_EXPM1 = 38, FOP_SIN = 39, FOP_COS = 40, FOP_RECIP = 41,
+  // `tile[:] = value` and the in-place operators (tile op= x is tile[:] = tile op x): of the
+  // two top entries (the tile below, the value on top) the value where it is active, the
+  // tile's own element elsewhere; active where either is
+  FOP_MERGE = 42,
 };
 
 struct Instr {
@@ -333,6 +337,16 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_fmap(FMapArgs a) {
         t1[e] = t3[e];
         k1[e] = k3[e];
       }
+    } else if (op == FOP_MERGE) {
+#pragma unroll
+      for (int e = 0; e < kV; ++e) {
+        t0[e] = k0[e] ? t0[e] : t1[e];
+        k0[e] = k0[e] || k1[e];
+        t1[e] = t2[e];
+        t2[e] = t3[e];
+        k1[e] = k2[e];
+        k2[e] = k3[e];
+      }
     } else if (op >= FOP_NEG) {
 #pragma unroll
       for (int e = 0; e < kV; ++e)
@@ -487,6 +501,11 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_gather_fmap(GatherMapArg
         t0 = arg == 0 ? v[0] : arg == 1 ? v[1] : arg == 2 ? v[2] : v[3];
         k0 = arg == 0 ? act[0] : arg == 1 ? act[1] : arg == 2 ? act[2] : act[3];
       }
+    } else if (op == FOP_MERGE) {
+      t0 = k0 ? t0 : t1;
+      k0 = k0 || k1;
+      t1 = t2, t2 = t3;
+      k1 = k2, k2 = k3;
     } else if (op == FOP_SELECT) {
       t0 = t2 != 0.0f ? t1 : t0;
       k0 = true;

@@ -1662,7 +1662,7 @@ int hcamdLaunchFMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
     }
     const bool push = op == HCAMD_FMAP_IN || op == HCAMD_FMAP_CONST;
     const bool select = op == HCAMD_FMAP_SELECT; // three entries in, one out
-    const bool unary = op >= HCAMD_FMAP_NEG && !select;
+    const bool unary = op >= HCAMD_FMAP_NEG && !select && op != HCAMD_FMAP_MERGE; // (MERGE: two in, one out)
     if (sp < (push ? 0 : unary ? 1 : select ? 3 : 2)) {
       dev->report("%s: stack underflow at %zu", who, i);
       return 1;
@@ -3260,7 +3260,7 @@ int hcamdGatherMapLaunch(OlQueue q, HcamdGatherMap plan, const HcamdMapInstr *pr
       }
       const bool push = op == HCAMD_FMAP_IN || op == HCAMD_FMAP_CONST;
       const bool select = op == HCAMD_FMAP_SELECT; // three entries in, one out
-      const bool unary = op >= HCAMD_FMAP_NEG && !select;
+      const bool unary = op >= HCAMD_FMAP_NEG && !select && op != HCAMD_FMAP_MERGE; // (MERGE: two in, one out)
       if (sp < (push ? 0 : unary ? 1 : select ? 3 : 2)) {
         dev->report("%s: stack underflow at %zu", who, i);
         return 1;

@@ -16,6 +16,7 @@ from __future__ import annotations
 import functools
 import itertools
 import math
+import weakref
 import operator
 from collections.abc import Iterable
 from fractions import Fraction
@@ -671,11 +672,22 @@ class Tile:
     __array_priority__ = 1000
     _counter = 0
 
+    # every node made so far, so that `tile[key] = value` (which changes the tile
+    # object in place, as the reference does) can leave what was computed from
+    # the tile before reading what the tile held then
+    _made = weakref.WeakSet()
+
     def __init__(self, op, args=(), shape=(), dtype="float32", **attrs):
         self.op, self.args, self.shape = op, tuple(args), tuple(int(s) for s in shape)
         self.dtype_name, self.attrs = dtype, attrs
         Tile._counter += 1
         self.uid = Tile._counter
+        Tile._made.add(self)
+
+    def snapshot(self) -> "Tile":
+        """What the tile holds now, as a node that a later assignment to the tile
+        does not change (a store records this)."""
+        return Tile(self.op, self.args, self.shape, self.dtype_name, **self.attrs)
 
     # -- construction helpers ----------------------------------------------------
     @staticmethod
@@ -734,6 +746,30 @@ class Tile:
             raise TraceError("tile / tile on integer tiles is float64 in NumPy, for which there is no "
                              "native kernel (use // for the integer quotient)")
         return r
+
+    # In-place operators are `tile[:] = tile op other` in the reference
+    # (python/hckernel/kernel_api.py:142-145): the assignment takes the result's
+    # active elements only, so an element whose result is inactive (a zero divisor,
+    # an operand that is inactive there) keeps its value and its activity.
+    def _in_place(self, other, method):
+        if self.attrs.get("plain"):
+            raise TraceError("an in-place operator on the result of a NumPy function, a reduction or astype "
+                             "is numpy.ma's own in-place operator, which has no native code (write x = x op y)")
+        self[:] = method(self, other)
+        return self
+
+    def __iadd__(self, o): return self._in_place(o, Tile.__add__)
+    def __isub__(self, o): return self._in_place(o, Tile.__sub__)
+    def __imul__(self, o): return self._in_place(o, Tile.__mul__)
+    def __itruediv__(self, o): return self._in_place(o, Tile.__truediv__)
+    def __ifloordiv__(self, o): return self._in_place(o, Tile.__floordiv__)
+    def __imod__(self, o): return self._in_place(o, Tile.__mod__)
+    def __ipow__(self, o): return self._in_place(o, Tile.__pow__)
+    def __iand__(self, o): return self._in_place(o, Tile.__and__)
+    def __ior__(self, o): return self._in_place(o, Tile.__or__)
+    def __ixor__(self, o): return self._in_place(o, Tile.__xor__)
+    def __ilshift__(self, o): return self._in_place(o, Tile.__lshift__)
+    def __irshift__(self, o): return self._in_place(o, Tile.__rshift__)
 
     def __neg__(self): return Tile("neg", (self,), self.shape, self.dtype_name, **self._plain_kw())
     def __abs__(self): return Tile("abs", (self,), self.shape, self.dtype_name, **self._plain_kw())
@@ -1051,8 +1087,15 @@ class Tile:
                 if not -n <= i < n:
                     raise TraceError(f"tile assignment: index {i} out of range for extent {n}")
                 norm.append(i % n)
-        old = Tile(self.op, self.args, self.shape, self.dtype_name, **self.attrs)
-        self.op, self.args = "update", (old, Tile.wrap(value))
+        if self.attrs.get("plain"):
+            raise TraceError("assignment into the result of a NumPy function, a reduction or astype (a bare "
+                             "numpy.ma array) is numpy.ma's own __setitem__, which has no native code")
+        old = self.snapshot()
+        for node in list(Tile._made):           # what was computed from the tile so far keeps reading the old contents
+            if node is not old and any(a is self for a in node.args):
+                node.args = tuple(old if a is self else a for a in node.args)
+        value = Tile.wrap(value)
+        self.op, self.args = "update", (old, old if value is self else value)
         self.attrs = {"key": tuple(norm)}
         Tile._counter += 1
         self.uid = Tile._counter
@@ -1197,12 +1240,12 @@ class CurrentGroup:
         if mapping is not None:
             if not isinstance(mapping, Mapping):
                 raise TraceError("mapping must come from create_mapping")
-            self.mapped_stores.append((view, Tile.wrap(src), mapping.func))
+            self.mapped_stores.append((view, Tile.wrap(src).snapshot(), mapping.func))
             return
         if not view.affine:
             raise TraceError("window offsets that use // or % of the group id are supported "
                              "on mapped loads and stores only")
-        self.stores.append((view, Tile.wrap(src)))
+        self.stores.append((view, Tile.wrap(src).snapshot()))
 
     # -- allocators ------------------------------------------------------------------
     def _alloc(self, shape, dtype, value):

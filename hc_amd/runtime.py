@@ -670,7 +670,7 @@ FMAP_OPS = {"in": 1, "const": 2, "add": 3, "sub": 4, "mul": 5, "div": 6, "floord
             "gt": 17, "neg": 18, "abs": 19, "sqrt": 20, "rint": 21, "exp": 22, "log": 23, "r16": 24,
             "psqrt": 25, "powchk": 26, "active": 27, "tanh": 28, "select": 29,
             "floor": 30, "ceil": 31, "trunc": 32, "sign": 33, "exp2": 34, "log2": 35, "log10": 36,
-            "log1p": 37, "expm1": 38, "sin": 39, "cos": 40, "reciprocal": 41}
+            "log1p": 37, "expm1": 38, "sin": 39, "cos": 40, "reciprocal": 41, "merge": 42}
 FMAP_MAX_INSTRS = 48
 
 

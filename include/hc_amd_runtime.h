@@ -451,7 +451,12 @@ enum HcamdFMapOp {
   HCAMD_FMAP_FLOOR = 30, HCAMD_FMAP_CEIL = 31, HCAMD_FMAP_TRUNC = 32, HCAMD_FMAP_SIGN = 33,
   HCAMD_FMAP_EXP2 = 34, HCAMD_FMAP_LOG2 = 35, HCAMD_FMAP_LOG10 = 36, HCAMD_FMAP_LOG1P = 37,
   HCAMD_FMAP_EXPM1 = 38, HCAMD_FMAP_SIN = 39, HCAMD_FMAP_COS = 40, HCAMD_FMAP_RECIP = 41,
-  HCAMD_FMAP_COUNT = 42
+  /* `tile[:] = value` and the in-place operators of the reference's tiles
+   * (python/hckernel/kernel_api.py:123-145: tile op= x is tile[:] = tile op x): of the
+   * two top entries (the tile below, the value on top) the value where it is active, the
+   * tile's own element elsewhere; active where either is */
+  HCAMD_FMAP_MERGE = 42,
+  HCAMD_FMAP_COUNT = 43
 };
 int hcamdLaunchFMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
                     const void *const *inputs, const int *inputTypes, const size_t *inputLd,

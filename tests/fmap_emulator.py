@@ -31,6 +31,10 @@ def run_fmap(program, inputs, store_all, out):
                 (c, _), (a, _), (b, _) = stack[-3:]
                 del stack[-3:]
                 stack.append((np.where(c != 0, a, b), np.ones(shape, bool)))
+            elif name == "merge":             # tile[:] = value: the value where active, the tile's own elsewhere
+                (a, ka), (b, kb) = stack[-2:]
+                del stack[-2:]
+                stack.append((np.where(kb, b, a), ka | kb))
             elif name in _UNARY:
                 a, ok = stack.pop()
                 stack.append(_UNARY[name](a, ok.copy(), plain))

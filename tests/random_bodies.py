@@ -249,3 +249,61 @@ def col_case(seed):
         for v in vals:
             v[~np.isfinite(v)] = 0.5
     return fn, text, vals, gn
+
+
+def statement_body(seed, api):
+    """(kernel body, its text, decorator arguments, two operand arrays): a short
+    random sequence of statements on two loaded tiles and perhaps an allocated
+    one -- in-place operators, `tile[:] = value`, rebinding to an expression or a
+    NumPy function -- that ends with a store of one of the tiles.  `api` is the
+    module that supplies CurrentGroup, Buffer, sym, typename (the kernel API)."""
+    rng = np.random.default_rng(seed)
+    two_d = seed % 2 == 0
+    names = ["x", "y"]
+    lines = []
+    if rng.random() < 0.6:
+        kind = rng.choice(["zeros", "ones", "full", "empty"])
+        lines.append(f"z = gr.{kind}(gr.shape, np.float32{', K(0.5)' if kind == 'full' else ''})")
+        names.append("z")
+
+    def operand():
+        r = rng.random()
+        if r < 0.5:
+            return rng.choice(names)
+        if r < 0.7:
+            return f"K({rng.choice(['0.5', '2.0', '-1.25', '0.0'])})"
+        return f"({rng.choice(names)} {rng.choice(['+', '-', '*', '/'])} {rng.choice(names)})"
+
+    for _ in range(int(rng.integers(1, 5))):
+        v = rng.choice(names)
+        r = rng.random()
+        if r < 0.45:
+            lines.append(f"{v} {rng.choice(['+=', '-=', '*=', '/='])} {operand()}")
+        elif r < 0.65:
+            lines.append(f"{v}[:] = {operand()}")
+        elif r < 0.8:
+            lines.append(f"{v} = {operand()} {rng.choice(['+', '*', '-'])} {operand()}")
+        else:
+            lines.append(f"{v} = np.{rng.choice(['abs', 'exp', 'sqrt'])}({v})")
+    out = rng.choice(names)
+    M, N, DT = api.sym.M, api.sym.N, api.typename.DT
+    if two_d:
+        head = ["def body(gr: CurrentGroup, a: Buffer[M, N, DT], b: Buffer[M, N, DT], out: Buffer[M, N, DT]):",
+                "    i, j = gr.work_offset",
+                "    x = gr.load(a[i:, j:], shape=gr.shape)", "    y = gr.load(b[i:, j:], shape=gr.shape)"]
+        tail = [f"    gr.store(out[i:, j:], {out})"]
+        shape, deco = (37, 131), dict(work_shape=(M, N), group_shape=(4, 64))
+    else:
+        head = ["def body(gr: CurrentGroup, a: Buffer[N, DT], b: Buffer[N, DT], out: Buffer[N, DT]):",
+                "    o = gr.work_offset[0]",
+                "    x = gr.load(a[o:], shape=gr.shape)", "    y = gr.load(b[o:], shape=gr.shape)"]
+        tail = [f"    gr.store(out[o:], {out})"]
+        shape, deco = (1003,), dict(work_shape=N, group_shape=256)
+    env = {"np": np, "K": np.float32, "CurrentGroup": api.CurrentGroup, "Buffer": api.Buffer, "M": M, "N": N,
+           "DT": DT}
+    exec("\n".join(head + ["    " + line for line in lines] + tail), env)
+    vals = [special_values(rng, shape, np.float32) for _ in range(2)]
+    if seed % 4 < 2:
+        for v in vals:
+            v[~np.isfinite(v)] = 0.5
+    return env["body"], "; ".join(lines) + f" -> {out}", deco, vals

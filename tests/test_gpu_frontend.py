@@ -2140,3 +2140,48 @@ def test_numpy_where_of_int32_tiles():
         gr.store(out[o:], np.where(tx < ty, tx // ty + I(1), ty))
     with pytest.raises(NoNativeKernel, match="numpy.where of integer tiles"):
         kernel(work_shape=N, group_shape=256)(on_top)(rt.to_device(a), rt.to_device(b), rt.to_device(a))
+
+
+def test_random_statement_sequences_match_the_simulator():
+    """In-place operators and `tile[:] = value` (python/hckernel/kernel_api.py:123-145:
+    tile op= x is tile[:] = tile op x, which takes the value's active elements
+    only -- an element whose result is deactivated keeps its value and its
+    activity), allocated tiles, rebinding: random sequences of such statements
+    on the device against the host executor, bit for bit (exp: a few ulp)."""
+    import sys
+    import warnings
+    import random_bodies
+    from hc_amd.binding import NoNativeKernel
+    from hc_amd.kernel_api import TraceError
+    api = sys.modules["hckernel.kernel"]
+    tally = {"ok": 0, "refused": 0, "both raise": 0}
+    for seed in range(600):
+        body, text, deco, vals = random_bodies.statement_body(seed, api)
+        want = np.full(vals[0].shape, np.float32(-77))
+        sim_raises = False
+        try:
+            with np.errstate(all="ignore"), warnings.catch_warnings():
+                warnings.simplefilter("ignore")
+                sim_kernel(**deco)(body)(*vals, want)
+        except TypeError:
+            sim_raises = True
+        out = rt.to_device(np.full(vals[0].shape, np.float32(-77)))
+        try:
+            kernel(**deco)(body)(*[rt.to_device(v) for v in vals], out)
+        except (NoNativeKernel, TraceError):
+            tally["refused"] += 1
+            continue
+        except TypeError:
+            assert sim_raises, f"seed {seed}: {text}: only the front-end raises TypeError"
+            tally["both raise"] += 1
+            continue
+        assert not sim_raises, f"seed {seed}: {text}: only the simulator raises TypeError"
+        got = out.to_host()
+        if "exp" in text:                      # exp of exp amplifies the last bits
+            assert_array_equal(np.isnan(got), np.isnan(want), err_msg=f"seed {seed}: {text}")
+            assert_allclose(got, want, rtol=2e-5, atol=1e-6, err_msg=f"seed {seed}: {text}")
+        else:
+            diff = random_bodies.difference(got, want, text)
+            assert diff is None, f"seed {seed}: {text} ({rt.last_kernel_name()}): {diff}"
+        tally["ok"] += 1
+    assert tally["ok"] > 300, tally

@@ -588,7 +588,8 @@ def test_fmap_every_opcode_and_flag_against_its_numpy_restatement(ctx, dtype):
     left = [F("in", 0), F("in", 1), F("div", half)]            # a / b: inactive where b == 0 ...
     right = [F("in", 2), F("in", 0), F("div", half)]           # c / a
     inexact = {"exp", "log", "tanh", "exp2", "log2", "log10", "log1p", "expm1", "sin", "cos"}
-    binary = ["add", "sub", "mul", "div", "floordiv", "mod", "min", "max", "udiv", "lt", "le", "eq", "ne", "ge", "gt"]
+    binary = ["add", "sub", "mul", "div", "floordiv", "mod", "min", "max", "udiv", "lt", "le", "eq", "ne", "ge", "gt",
+              "merge"]
     unary = [k for k in rt.FMAP_OPS if k not in binary + ["end", "in", "const", "select"]]
     programs = []
     for name in binary:
