@@ -759,8 +759,8 @@ def _maybe_masked(t: Tile, memo=None) -> bool:
     their number never is.)"""
     memo = {} if memo is None else memo
     if t.uid not in memo:
-        if _is(t, "load") or _const(t) or t.op in ("count", "where"):
-            memo[t.uid] = False                  # (numpy.where returns a plain array)
+        if _is(t, "load") or _const(t) or t.op in ("count", "where", "active"):
+            memo[t.uid] = False                  # (numpy.where and tile.mask return plain arrays)
         elif _is(t, "merge", 2):
             memo[t.uid] = _maybe_masked(t.args[0], memo)     # active wherever the tile was
         else:
@@ -1205,7 +1205,20 @@ def match_imap(dst_view, value, n_groups):
         return None
     if not emit(value) or not loads:
         return None
-    if need(value) > 4:
+    depth = need(value)
+    if value.attrs.get("plain") and _maybe_masked(value) and not _is(value, "where", 3):
+        # A bare numpy.ma array is written in full, with what numpy.ma leaves under a
+        # deactivated element.  The kernel keeps one activity flag per element and the
+        # leftovers of // and % (the dividend, 1): where only NumPy functions, negation
+        # and abs sit above them the plain arithmetic gives numpy.ma's values, and an
+        # always-true selection makes every element active again.
+        if not _values_flow_plainly(value):
+            raise NoNativeKernel(f"{dst_view.base.name}: the stored value is a bare array (a NumPy function of "
+                                 "integer tiles), written in full, with an operator above a // or % that can "
+                                 "fail: what numpy.ma leaves there has no native code for integer tiles")
+        program[:] = [("const", 0, 1)] + program + [("const", 0, 0), ("select", 0, 0)]
+        depth += 1
+    if depth > 4:
         raise NoNativeKernel("integer expression too deep for the four-entry stack")
     if len(program) > 32:
         raise NoNativeKernel(f"integer expression too long ({len(program)} operations, at most 32)")
@@ -2763,9 +2776,11 @@ def simplify(t: Tile, memo=None) -> Tile:
                     one = Tile("const", (), (), out.dtype_name, value=1.0, weak=False)
                     zero = Tile("const", (), (), out.dtype_name, value=0.0, weak=False)
                     out = Tile("where", (one, filled, zero), out.shape, out.dtype_name)
-            elif _maybe_masked(value) and out.dtype_name in _MAP_FLOATS:
-                # elements the data can deactivate keep what the tile held
-                out = Tile("merge", (old, filled), out.shape, out.dtype_name)
+            elif _maybe_masked(value):
+                # elements the data can deactivate keep what the tile held (the general float
+                # map has that; integer tiles stay an assignment, which no kernel takes)
+                if out.dtype_name in _MAP_FLOATS:
+                    out = Tile("merge", (old, filled), out.shape, out.dtype_name)
             elif _const(old):
                 # on a freshly allocated tile: value where it is active, the allocator's fill
                 # elsewhere, every element active (a load that reaches past its array is what

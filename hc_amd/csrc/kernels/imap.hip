@@ -8,9 +8,10 @@
 //   * // rounds towards minus infinity and % takes the sign of the divisor;
 //   * an element whose divisor is zero becomes INACTIVE, as numpy.ma makes it,
 //     and stays inactive through everything computed from it: nothing is stored
-//     for it.  (One exception, numpy.ma's own: its test is
+//     for it.  (Two exceptions, numpy.ma's own: its test is
 //     |a| * tiny >= |b|, and |INT_MIN| overflows to a negative number, so
-//     INT_MIN // 0 and INT_MIN % 0 stay active with NumPy's result 0.)
+//     INT_MIN // 0 and INT_MIN % 0 stay active with NumPy's result 0, and a
+//     divisor INT_MIN deactivates whatever the dividend is.)
 //   * << and >> with a count outside 0..31 give 0 (>> of a negative value: -1),
 //     which is what NumPy defines; >> is arithmetic;
 //   * comparisons give 0 / 1.
@@ -70,6 +71,10 @@ __device__ __forceinline__ int32_t floor_div(int32_t a, int32_t b, bool &ok) {
     ok = ok && a == INT32_MIN;
     return a == INT32_MIN ? 0 : a;
   }
+  if (b == INT32_MIN) { // numpy.ma's test sees |INT_MIN| as a negative number: always deactivated
+    ok = false;
+    return a;
+  }
   if (b == -1)
     return wrap_sub(0, a); // INT_MIN / -1 wraps instead of trapping
   int32_t q = a / b;
@@ -81,6 +86,10 @@ __device__ __forceinline__ int32_t floor_mod(int32_t a, int32_t b, bool &ok) {
   if (b == 0) {
     ok = ok && a == INT32_MIN;
     return a == INT32_MIN ? 0 : 1;
+  }
+  if (b == INT32_MIN) {
+    ok = false;
+    return 1;
   }
   if (b == -1)
     return 0;

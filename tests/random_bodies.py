@@ -307,3 +307,65 @@ def statement_body(seed, api):
         for v in vals:
             v[~np.isfinite(v)] = 0.5
     return env["body"], "; ".join(lines) + f" -> {out}", deco, vals
+
+
+def int_statement_body(seed, api):
+    """(kernel body, its text, decorator arguments, two int32 operand arrays): a
+    few statements on two loaded int32 tiles (in-place operators, assignment,
+    rebinding) and a stored expression of + - * // % & | ^ << >> minimum maximum
+    abs negation and numpy.where; divisors hold zeros, every fifth case INT_MIN
+    and INT_MAX."""
+    rng = np.random.default_rng(seed)
+    I = np.int32
+    names = ["x", "y"]
+
+    def expr(d):
+        if d == 0 or rng.random() < 0.25:
+            return rng.choice(names)
+        k = rng.integers(0, 12)
+        x = expr(d - 1)
+        if k <= 2:
+            return f"({x} {rng.choice(['+', '-', '*'])} {expr(d - 1)})"
+        if k == 3:
+            return f"({x} // {expr(d - 1)})"
+        if k == 4:
+            return f"({x} % {expr(d - 1)})"
+        if k == 5:
+            return f"({x} {rng.choice(['&', '|', '^'])} {expr(d - 1)})"
+        if k == 6:
+            return f"({x} {rng.choice(['<<', '>>'])} ({expr(d - 1)} & I(7)))"
+        if k == 7:
+            return f"np.{rng.choice(['maximum', 'minimum'])}({x}, {expr(d - 1)})"
+        if k == 8:
+            return f"{rng.choice(['-', 'abs'])}({x})"
+        if k == 9:
+            return f"({x} {rng.choice(['+', '*', '//', '%', '-'])} I({rng.choice(['2', '-3', '0', '7'])}))"
+        if k == 10:
+            cmp = rng.choice(['<', '==', '!=', '>='])
+            return f"np.where({expr(d - 1)} {cmp} {expr(d - 1)}, {x}, {expr(d - 1)})"
+        return f"np.abs({x})"
+
+    lines = []
+    for _ in range(int(rng.integers(0, 3))):
+        v = rng.choice(names)
+        r = rng.random()
+        if r < 0.5:
+            lines.append(f"{v} {rng.choice(['+=', '-=', '*=', '//=', '%=', '&='])} {expr(1)}")
+        elif r < 0.7:
+            lines.append(f"{v}[:] = {expr(1)}")
+        else:
+            lines.append(f"{v} = {expr(2)}")
+    final = expr(int(rng.integers(0, 3)))
+    M, N, DT = api.sym.M, api.sym.N, api.typename.DT
+    src = ["def body(gr: CurrentGroup, a: Buffer[M, N, DT], b: Buffer[M, N, DT], out: Buffer[M, N, DT]):",
+           "    i, j = gr.work_offset", "    x = gr.load(a[i:, j:], shape=gr.shape)",
+           "    y = gr.load(b[i:, j:], shape=gr.shape)"] + ["    " + line for line in lines] + \
+          [f"    gr.store(out[i:, j:], {final})"]
+    env = {"np": np, "I": I, "CurrentGroup": api.CurrentGroup, "Buffer": api.Buffer, "M": M, "N": N, "DT": DT}
+    exec("\n".join(src), env)
+    shape = (37, 131)
+    vals = [rng.integers(-9, 10, shape).astype(I) for _ in range(2)]
+    if seed % 5 == 0:
+        vals[0][rng.random(shape) < 0.05] = np.iinfo(I).min
+        vals[1][rng.random(shape) < 0.05] = np.iinfo(I).max
+    return env["body"], "; ".join(lines) + f" -> {final}", dict(work_shape=(M, N), group_shape=(4, 64)), vals

@@ -2185,3 +2185,41 @@ def test_random_statement_sequences_match_the_simulator():
             assert diff is None, f"seed {seed}: {text} ({rt.last_kernel_name()}): {diff}"
         tally["ok"] += 1
     assert tally["ok"] > 300, tally
+
+
+def test_random_int32_statement_sequences_match_the_simulator():
+    """Random statements and expressions of int32 tiles (tests/random_bodies.py) on
+    the device against the host executor, exactly: zero divisors, INT_MIN as a
+    dividend and as a divisor (numpy.ma's test deactivates every quotient by
+    INT_MIN), bare arrays written in full with numpy.ma's leftovers, numpy.where."""
+    import sys
+    import warnings
+    import random_bodies
+    from hc_amd.binding import NoNativeKernel
+    from hc_amd.kernel_api import TraceError
+    api = sys.modules["hckernel.kernel"]
+    tally = {"ok": 0, "refused": 0, "both raise": 0}
+    for seed in range(600):
+        body, text, deco, vals = random_bodies.int_statement_body(seed, api)
+        want = np.full(vals[0].shape, np.int32(-777))
+        sim_raises = False
+        try:
+            with np.errstate(all="ignore"), warnings.catch_warnings():
+                warnings.simplefilter("ignore")
+                sim_kernel(**deco)(body)(*vals, want)
+        except TypeError:
+            sim_raises = True
+        out = rt.to_device(np.full(vals[0].shape, np.int32(-777)))
+        try:
+            kernel(**deco)(body)(*[rt.to_device(v) for v in vals], out)
+        except (NoNativeKernel, TraceError):
+            tally["refused"] += 1
+            continue
+        except TypeError:
+            assert sim_raises, f"seed {seed}: {text}: only the front-end raises TypeError"
+            tally["both raise"] += 1
+            continue
+        assert not sim_raises, f"seed {seed}: {text}: only the simulator raises TypeError"
+        assert_array_equal(out.to_host(), want, err_msg=f"seed {seed}: {text}")
+        tally["ok"] += 1
+    assert tally["ok"] > 350, tally
