@@ -759,7 +759,7 @@ def _maybe_masked(t: Tile, memo=None) -> bool:
     their number never is.)"""
     memo = {} if memo is None else memo
     if t.uid not in memo:
-        if _is(t, "load") or _const(t) or t.op in ("count", "where", "active"):
+        if _is(t, "load") or _const(t) or t.op in ("count", "where", "active", "activated"):
             memo[t.uid] = False                  # (numpy.where and tile.mask return plain arrays)
         elif _is(t, "merge", 2):
             memo[t.uid] = _maybe_masked(t.args[0], memo)     # active wherever the tile was
@@ -816,8 +816,10 @@ def _can_fail(t: Tile, finite: bool, memo=None) -> bool:
         return _maybe_masked(t)
     memo = {} if memo is None else memo
     if t.uid not in memo:
-        if _is(t, "load") or _const(t) or t.op in ("count", "where"):
+        if _is(t, "load") or _const(t) or t.op in ("count", "where", "active", "activated"):
             memo[t.uid] = False                  # (numpy.where returns a plain array)
+        elif _is(t, "merge", 2):
+            memo[t.uid] = _can_fail(t.args[0], True, memo)
         else:
             memo[t.uid] = _fails_on_finite_data(t) or \
                 any(_can_fail(a, True, memo) for a in t.args if isinstance(a, Tile))
@@ -1281,6 +1283,8 @@ def _compile_fmap(value, mapped=False):
             n = max(need(t.args[0]), 2)          # the bounds are pushed next to the value
         elif _is(t, "merge", 2):
             n = max(need(t.args[0]), need(t.args[1]) + 1)
+        elif _is(t, "activated", 1):
+            n = need(t.args[0]) + 1
         elif len(t.args) == 1:
             n = need(t.args[0])
         elif len(t.args) == 2:
@@ -1337,6 +1341,15 @@ def _compile_fmap(value, mapped=False):
         if _is(t, "active", 1):
             ok = emit(t.args[0])                   # tile.mask: the entry's activity as 0 / 1
             program.append(("active", 0, 0.0))
+            return ok
+        if _is(t, "activated", 1):
+            # the values whatever their activity, every element active: a selection that always takes them
+            if t.dtype_name not in _MAP_FLOATS or _const(t.args[0]):
+                return False
+            program.append(("const", 0, 1.0))
+            ok = emit(t.args[0])
+            program.append(("const", 0, 0.0))
+            program.append(("select", 0, 0.0))
             return ok
         if _is(t, "merge", 2):
             if t.dtype_name not in _MAP_FLOATS:
@@ -2773,14 +2786,22 @@ def simplify(t: Tile, memo=None) -> Tile:
                 if not _const(old) and out.dtype_name in _MAP_FLOATS:
                     # every element is overwritten with the bare array's value, whatever its
                     # activity there, and is active: a selection that always takes the value
-                    one = Tile("const", (), (), out.dtype_name, value=1.0, weak=False)
-                    zero = Tile("const", (), (), out.dtype_name, value=0.0, weak=False)
-                    out = Tile("where", (one, filled, zero), out.shape, out.dtype_name)
+                    out = Tile("activated", (filled,), out.shape, out.dtype_name)
             elif _maybe_masked(value):
                 # elements the data can deactivate keep what the tile held (the general float
                 # map has that; integer tiles stay an assignment, which no kernel takes)
                 if out.dtype_name in _MAP_FLOATS:
-                    out = Tile("merge", (old, filled), out.shape, out.dtype_name)
+                    if filled.op in ("add", "sub", "mul", "div", "floordiv") and not filled.attrs.get("func") \
+                            and len(filled.args) == 2 and _same(filled.args[0], old) and not _maybe_masked(old) \
+                            and any(_is_reduction(x) for x in _walk(filled)):
+                        # tile op= x on a tile that is active everywhere: numpy.ma leaves the first
+                        # operand (the dividend) under a deactivated result, which is the tile's
+                        # own element, so the merged tile is the result's values, all active.
+                        # (Only where a reduction keeps the general map, which has the merge
+                        # itself, away: numpy.ma leaves 0 + dividend, so a kept -0 becomes +0.)
+                        out = Tile("activated", (filled,), out.shape, out.dtype_name)
+                    else:
+                        out = Tile("merge", (old, filled), out.shape, out.dtype_name)
             elif _const(old):
                 # on a freshly allocated tile: value where it is active, the allocator's fill
                 # elsewhere, every element active (a load that reaches past its array is what
@@ -2803,6 +2824,31 @@ def simplify(t: Tile, memo=None) -> Tile:
         out = Tile("const", (), (), "float32", value=float(n), weak=False, exact=int(n), counted=True)
     memo[id(t)] = out
     return out
+
+
+def _without_activations_for_data_that_is_not_finite(t: Tile, memo=None) -> Tile:
+    """t with `activated(x)` replaced by x wherever only overflow or data that is
+    not finite can deactivate an element of x: what the kernels for reductions,
+    which cannot represent the activation, compute instead (elsewhere they give
+    plain arithmetic on such data too)."""
+    memo = {} if memo is None else memo
+    if id(t) not in memo:
+        args = tuple(_without_activations_for_data_that_is_not_finite(a, memo) if isinstance(a, Tile) else a
+                     for a in t.args)
+        out = t if all(a is b for a, b in zip(args, t.args)) else Tile(t.op, args, t.shape, t.dtype_name, **t.attrs)
+        if _is(out, "activated", 1) and not _can_fail(out.args[0], True):
+            out = out.args[0]
+        memo[id(t)] = out
+    return memo[id(t)]
+
+
+def _stored_in_full_if_activated(value: Tile) -> Tile:
+    """A stored tile all of whose elements an assignment activated, with the values
+    numpy.ma left in them, is to the kernels what a bare array is: written in full."""
+    if _is(value, "activated", 1) and not _const(value.args[0]):
+        inner = value.args[0]
+        return Tile(inner.op, inner.args, inner.shape, inner.dtype_name, **{**inner.attrs, "plain": True})
+    return value
 
 
 def _has_elementwise_load(t: Tile) -> bool:
@@ -3094,7 +3140,9 @@ def bind(stores, n_groups, atomics=(), mapped_stores=(), id_stores=(), group_sha
     if not stores and not atomics and not mapped_stores and not id_stores and not cell_stores:
         raise NoNativeKernel("the kernel body stores nothing")
     memo = {}
-    stores = [(view, simplify(value, memo)) for view, value in stores]
+    stores = [(view, _stored_in_full_if_activated(simplify(value, memo))) for view, value in stores]
+    stores = [(view, _without_activations_for_data_that_is_not_finite(value)
+               if any(_is_reduction(t) for t in _walk(value)) else value) for view, value in stores]
     for view, value in stores:
         _overlay_guard(view, value, memo.get("overlays", ()), n_groups)
     id_makers = [match_id_store(p, i, v, per, n_groups, group_shape) for p, i, v, per in id_stores]

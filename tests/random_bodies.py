@@ -369,3 +369,49 @@ def int_statement_body(seed, api):
         vals[0][rng.random(shape) < 0.05] = np.iinfo(I).min
         vals[1][rng.random(shape) < 0.05] = np.iinfo(I).max
     return env["body"], "; ".join(lines) + f" -> {final}", dict(work_shape=(M, N), group_shape=(4, 64)), vals
+
+
+def row_statement_body(seed, api):
+    """(kernel body, text, decorator arguments, two operand arrays, group rows): a
+    few statements on two tiles that hold whole rows -- in-place operators with row
+    scalars (`t -= t.max(axis=1, keepdims=True)`, `t /= u.sum(axis=1, keepdims=True)`),
+    rebinding to NumPy functions -- and a store of a tile or of an expression."""
+    rng = np.random.default_rng(seed)
+    names = ["t", "u"]
+
+    def scalar():
+        red = rng.choice(["sum", "max", "min", "mean", "std"])
+        return f"{rng.choice(names)}.{red}(axis=1, keepdims=True)"
+
+    def operand():
+        r = rng.random()
+        if r < 0.45:
+            return scalar()
+        if r < 0.65:
+            return rng.choice(names)
+        if r < 0.8:
+            return f"K({rng.choice(['0.5', '2.0', '-1.25', '0.0'])})"
+        return f"({rng.choice(names)} {rng.choice(['+', '-', '*'])} {scalar()})"
+
+    lines = []
+    for _ in range(int(rng.integers(1, 4))):
+        v = rng.choice(names)
+        r = rng.random()
+        if r < 0.6:
+            lines.append(f"{v} {rng.choice(['+=', '-=', '*=', '/='])} {operand()}")
+        elif r < 0.75:
+            lines.append(f"{v} = np.{rng.choice(['exp', 'abs', 'sqrt', 'tanh'])}({v})")
+        else:
+            lines.append(f"{v} = {v} {rng.choice(['+', '-', '*', '/'])} {operand()}")
+    final = rng.choice(names) if rng.random() < 0.6 else f"({rng.choice(names)} {rng.choice(['+', '*', '/'])} {operand()})"
+    M, N, GM, DT = api.sym.M, api.sym.N, api.sym.GM, api.typename.DT
+    src = ["def body(gr: CurrentGroup, a: Buffer[M, N, DT], b: Buffer[M, N, DT], out: Buffer[M, N, DT], g: GM):",
+           "    m0, mb = gr.work_offset[0], gr.shape[0]",
+           "    t = gr.load(a[m0:, :], shape=(mb, N))", "    u = gr.load(b[m0:, :], shape=(mb, N))"] + \
+          ["    " + line for line in lines] + [f"    gr.store(out[m0:, :], {final})"]
+    env = {"np": np, "K": np.float32, "CurrentGroup": api.CurrentGroup, "Buffer": api.Buffer, "M": M, "N": N,
+           "GM": GM, "DT": DT}
+    exec("\n".join(src), env)
+    rows, n = [(9, 5), (13, 200), (6, 1031)][seed % 3]
+    vals = [(rng.integers(-6, 7, (rows, n)) / 2).astype(np.float32) for _ in range(2)]   # finite (see row_case)
+    return env["body"], "; ".join(lines) + f" -> {final}", dict(work_shape=M, group_shape=GM), vals

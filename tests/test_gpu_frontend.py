@@ -2223,3 +2223,37 @@ def test_random_int32_statement_sequences_match_the_simulator():
         assert_array_equal(out.to_host(), want, err_msg=f"seed {seed}: {text}")
         tally["ok"] += 1
     assert tally["ok"] > 350, tally
+
+
+def test_random_statement_sequences_in_row_bodies_match_the_simulator():
+    """In-place operators with row scalars (`t -= t.max(axis=1, keepdims=True)`,
+    `t /= u.sum(axis=1, keepdims=True)`: where the divisor is zero the element
+    keeps its value and stays active), rebinding to NumPy functions, then a store:
+    random sequences on the device against the host executor."""
+    import sys
+    import warnings
+    import random_bodies
+    from hc_amd.binding import NoNativeKernel
+    from hc_amd.kernel_api import TraceError
+    api = sys.modules["hckernel.kernel"]
+    poison = np.float32(-7777.25)
+    tally = {"ok": 0, "refused": 0}
+    for seed in range(300):
+        body, text, deco, vals = random_bodies.row_statement_body(seed, api)
+        want = np.full(vals[0].shape, poison)
+        with np.errstate(all="ignore"), warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            sim_kernel(**deco)(body)(*vals, want, 4)
+        out = rt.to_device(np.full(vals[0].shape, poison))
+        try:
+            kernel(**deco)(body)(*[rt.to_device(v) for v in vals], out, 4)
+        except (NoNativeKernel, TraceError):
+            tally["refused"] += 1
+            continue
+        got = out.to_host()
+        where = f"seed {seed}: {text} ({rt.last_kernel_name()})"
+        assert_array_equal(got == poison, want == poison, err_msg=where)
+        assert_array_equal(np.isnan(got), np.isnan(want), err_msg=where)
+        assert_allclose(got, want, rtol=1e-4, atol=1e-4, err_msg=where)
+        tally["ok"] += 1
+    assert tally["ok"] > 200, tally
