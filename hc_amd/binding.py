@@ -2280,6 +2280,9 @@ def _compile_col_reduce(red: Tile, root: Tile, n_groups, temps):
     """(kind, program, post, compiler) of root = post(red), red a reduction
     along axis 0."""
     body = red.args[0]
+    if red.op == "count":
+        raise NoNativeKernel("the number of active elements down the columns (the mean, var or std of an "
+                             "expression whose elements can be deactivated) has no native code")
     if red.op == "norm":          # numpy.linalg.norm along an axis is sqrt(add.reduce(x * x))
         body = body * body
     if red.op in ("sum", "norm") and body.dtype_name != "float32":
@@ -2409,10 +2412,10 @@ def match_cols(dst_view, value, n_groups):
     ftype = lambda name: rt.F16 if name == "float16" else rt.F32
     n_cols = w.extent[1]
 
-    def make(mem, ctx):
+    def make(mem, ctx, into=None):
         import numpy as np
         mo = mem[wo.buffer]
-        if n_cols > 1 and mo.strides[-1] != 1:
+        if n_cols > 1 and mo.strides[-1] != 1 and into is None:
             raise NoNativeKernel("the per-column result must be contiguous")
         vectors = [rt.DeviceArray((n_cols,), np.float32, ctx) for _ in order]
         plans = []
@@ -2427,6 +2430,8 @@ def match_cols(dst_view, value, n_groups):
                     types.append(ftype(tl.dtype_name))
             if i < len(order):
                 out, out_type = vectors[i], rt.F32
+            elif into is not None:
+                out, out_type = into, rt.F32
             else:
                 out = _Arr(rt.Memref(mo.ptr, (n_cols,), (1,), mo.itemsize), ctx)
                 out_type = ftype(dst_view.base.dtype_name)
@@ -2434,6 +2439,103 @@ def match_cols(dst_view, value, n_groups):
         return plans
     make.program, make.post, make.kind = steps[-1][1], steps[-1][2], steps[-1][0]
     make.steps = [(k, pr, po) for k, pr, po, _ in steps]
+    make.columns = (w.extent[1], w.driver[1])
+    return make
+
+
+def _cols_chain_root(t: Tile):
+    """The column reduction under t if only what match_cols takes as a post program
+    sits between them (operations with constants, functions of one operand)."""
+    while not _is_col_reduce(t):
+        if len(t.args) == 1 and (_is(t, "astype", 1) or t.op in _MAP_UNARY or _is(t, "clip", 1)):
+            t = t.args[0]
+        elif t.op in _MAP_BINARY and len(t.args) == 2 and _const(t.args[0]) != _const(t.args[1]):
+            t = t.args[0] if _const(t.args[1]) else t.args[1]
+        elif _is(t, "vardiv", 2) and _const(t.args[1]):
+            t = t.args[0]
+        else:
+            return None
+    return t
+
+
+def match_cols_combined(dst_view, value, n_groups):
+    """An elementwise expression of several reductions down the columns
+    (`x.sum(axis=0) / y.sum(axis=0)`, `(x * x).mean(axis=0) - x.mean(axis=0) ** 2`):
+    every reduction with what follows it alone runs as match_cols would run it,
+    into a temporary vector of one element per column, and the general float map
+    combines the vectors.  The reductions' results are bare numpy.ma arrays, so
+    the combination follows numpy.ma's rules and is written in full; a fold that
+    the data could deactivate (a column without active elements) has no activity
+    to hand on and is refused."""
+    if dst_view.base.dtype_name not in _MAP_FLOATS or len(value.shape) != 1 or \
+            value.dtype_name not in _MAP_FLOATS or _cols_chain_root(value) is not None:
+        return None
+    units, fakes = [], {}
+
+    def split(t: Tile) -> Tile:
+        """t with every unit replaced by a load of its temporary vector."""
+        if _const(t):
+            return t
+        if t.shape != value.shape:
+            raise NoNativeKernel(f"{t!r} inside an expression of column reductions: only per-column values "
+                                 "combine")
+        if _cols_chain_root(t) is not None:
+            for u, fake in units:
+                if _same(u, t):
+                    return fake
+            proxy = type("TemporaryVector", (), {"index": -1 - len(units), "name": f"column vector {len(units)}",
+                                                 "shape": t.shape, "dtype_name": "float32", "ndim": 1})()
+            view = type("TemporaryView", (), {"base": proxy, "starts": ()})()
+            fake = Tile("load", (), t.shape, "float32", view=view)
+            if t.dtype_name != "float32":
+                fake = Tile("astype", (fake,), t.shape, t.dtype_name, plain=True)
+            units.append((t, fake))
+            return fake
+        if _is(t, "load") or not t.args:
+            raise NoNativeKernel(f"{t!r} next to column reductions: only reductions down the columns and "
+                                 "numbers combine")
+        args = tuple(split(a) if isinstance(a, Tile) else a for a in t.args)
+        return Tile(t.op, args, t.shape, t.dtype_name, **t.attrs)
+
+    if not any(_is_col_reduce(t) for t in _walk(value)):
+        return None
+    combined = split(value)
+    if len(units) < 2:
+        return None
+    makers = []
+    for u, _ in units:
+        for red in (t for t in _walk(u) if _is_col_reduce(t)):
+            _no_fold_read_back_if_it_can_be_deactivated(red)
+        mk = match_cols(dst_view, u, n_groups)
+        if mk is None:
+            raise NoNativeKernel(f"{u!r}: not a reduction down the columns that has a native kernel")
+        makers.append(mk)
+    if len({mk.columns for mk in makers}) != 1:
+        raise NoNativeKernel("the column reductions of one expression must walk the same columns")
+    compiled = _compile_fmap(combined)
+    if compiled is None:
+        raise NoNativeKernel(f"{value!r}: not an expression of column reductions that the general float map takes")
+    loads, prog = compiled
+    order = [next(i for i, (_, fake) in enumerate(units)
+                  if (fake if _is(fake, "load") else fake.args[0]) is ld) for ld in loads]
+    wo = window_of(dst_view, value.shape, n_groups)
+    n_cols = makers[0].columns[0]
+    out_type = {"float32": rt.F32, "float16": rt.F16}[dst_view.base.dtype_name]
+
+    def make(mem, ctx):
+        import numpy as np
+        mo = mem[wo.buffer]
+        if n_cols > 1 and mo.strides[-1] != 1:
+            raise NoNativeKernel("the per-column result must be contiguous")
+        vectors = [rt.DeviceArray((n_cols,), np.float32, ctx) for _ in units]
+        plans = []
+        for mk, vec in zip(makers, vectors):
+            plans += mk(mem, ctx, into=vec)
+        out = _Arr(rt.Memref(mo.ptr, (n_cols,), (1,), mo.itemsize), ctx)
+        plans.append(rt.plan_fmap(prog, [vectors[i] for i in order], out, [rt.F32] * len(order) + [out_type],
+                                  store_all=True))
+        return plans
+    make.program = prog
     return make
 
 
@@ -3171,7 +3273,7 @@ def bind(stores, n_groups, atomics=(), mapped_stores=(), id_stores=(), group_sha
             try:
                 for matcher in (match_fill, match_copy, match_transpose, match_imap, match_add, match_fma, match_softmax,
                                 match_gemm, match_gather_gemm, match_gather_map, match_pairwise, match_cols,
-                                match_cols_tile, match_rows, match_map, match_fmap, match_general_windows):
+                                match_cols_combined, match_cols_tile, match_rows, match_map, match_fmap, match_general_windows):
                     mk = matcher(view, value, n_groups)
                     if mk is not None:
                         makers.append(mk)

@@ -2257,3 +2257,39 @@ def test_random_statement_sequences_in_row_bodies_match_the_simulator():
         assert_allclose(got, want, rtol=1e-4, atol=1e-4, err_msg=where)
         tally["ok"] += 1
     assert tally["ok"] > 200, tally
+
+
+def test_expressions_of_several_column_reductions():
+    """`(x * x).mean(axis=0) - x.mean(axis=0) ** 2` and the like: every reduction
+    down the columns runs into a temporary vector and the general float map
+    combines them under numpy.ma's rules (a zero divisor leaves the dividend,
+    the result is written in full); same bodies on the host executor."""
+    M, N, GN = sym.M, sym.N, sym.GN
+    f = np.float32
+    rng = np.random.default_rng(77)
+    rows, n, gn = 300, 200, 64
+    x = rng.standard_normal((rows, n)).astype(f)
+    y = (np.abs(rng.standard_normal((rows, n))) + 0.1).astype(f)       # (sums without cancellation)
+    y[:, 5] = 0                                  # a column whose sum is zero: a / 0 leaves a
+    forms = {
+        "variance": lambda a, b: (a * a).mean(axis=0) - a.mean(axis=0) ** f(2),
+        "ratio": lambda a, b: a.sum(axis=0) / b.sum(axis=0),
+        "range": lambda a, b: a.max(axis=0) - a.min(axis=0),
+        "cosine": lambda a, b: (a * b).sum(axis=0) / np.sqrt((a * a).sum(axis=0) * (b * b).sum(axis=0)),
+        "same_twice": lambda a, b: a.sum(axis=0) * a.sum(axis=0) + b.std(axis=0),
+    }
+    for name, fn in forms.items():
+        def body(gr: CurrentGroup, a: Buffer[M, N, DT], b: Buffer[M, N, DT], out: Buffer[N, DT], g: GN):
+            n0 = gr.id[0] * GN
+            gr.store(out[n0:], fn(gr.load(a[:, n0:], shape=(M, GN)), gr.load(b[:, n0:], shape=(M, GN))))
+        deco = dict(work_shape=cdiv(n, gn), group_shape=1, literals={GN})
+        want = np.full(n, f(-77))
+        with np.errstate(all="ignore"):
+            sim_kernel(**deco)(body)(x, y, want, gn)
+        out = rt.to_device(np.full(n, f(-77)))
+        kernel(**deco)(body)(rt.to_device(x), rt.to_device(y), out, gn)
+        assert rt.last_kernel_name() == "hcamd_fmap", name
+        got = out.to_host()
+        assert (got != f(-77)).all(), name
+        assert_array_equal(np.isnan(got), np.isnan(want), err_msg=name)
+        assert_allclose(got, want, rtol=2e-4, atol=2e-4, err_msg=name)
