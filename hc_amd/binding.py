@@ -1535,7 +1535,15 @@ def match_gather_map(dst_view, value, n_groups, out_func=None, force=False):
     out_dt = dst_view.base.dtype_name
     leaf = value.args[0] if _is(value, "astype", 1) and value.dtype_name == value.args[0].dtype_name else value
     copy_bytes = 0
-    if (_is(leaf, "load") or _is(leaf, "mapped_load")) and leaf.dtype_name == out_dt:
+    # A bare numpy.ma array stored through a mapping goes element by element
+    # (python/hckernel/kernel_api.py:331-334): a deactivated element is the
+    # masked constant, which NumPy converts to NaN in a float array, to False
+    # in a bool array and refuses to convert to an integer.
+    masked_constants = out_func is not None and bool(value.attrs.get("plain"))
+    if masked_constants and out_dt not in _MAP_FLOATS + ("bool",):
+        raise NoNativeKernel(f"{dst_view.base.name}: a numpy.ma array stored through a mapping writes its "
+                             "deactivated elements as masked constants, which only float and bool arrays take")
+    if (_is(leaf, "load") or _is(leaf, "mapped_load")) and leaf.dtype_name == out_dt and not masked_constants:
         # a gathered / scattered copy: any element type
         loads, program = [leaf], []
         copy_bytes = leaf.attrs["view"].base.dtype.itemsize if hasattr(leaf.attrs["view"].base.dtype, "itemsize") else 2
@@ -1586,7 +1594,7 @@ def match_gather_map(dst_view, value, n_groups, out_func=None, force=False):
     indices = [t.attrs["view"].base.index for t in loads] + [dst_view.base.index]
     types = [{"float16": rt.F16, "int32": rt.I32}.get(t.dtype_name, rt.F32) for t in loads]
     out_type = {"float32": rt.F32, "float16": rt.F16, "bool": rt.U8}.get(out_dt, rt.F32)
-    store_all = bool(value.attrs.get("plain")) and not copy_bytes
+    store_all = 0 if copy_bytes or not value.attrs.get("plain") else 2 if masked_constants else 1
     cache = {}
 
     def make(mem, ctx):

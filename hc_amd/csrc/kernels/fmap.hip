@@ -434,7 +434,7 @@ struct GatherMapArgs {
   uint32_t n_in, tile_elems, chunks; // chunks: workgroups per group
   uint32_t f16_mask;  // bit i: operand i is fp16; bit 8 + i: operand i is int32 (converted when read)
   uint32_t out_type;  // 0 fp32, 1 fp16, 2 one byte of 0 / 1
-  uint32_t store_all; // write deactivated results too
+  uint32_t store_all; // write deactivated results too: 1 as computed, 2 as NaN (0 in a bool buffer)
   uint32_t copy_bytes; // != 0: no program, operand 0 is copied as elements of this many bytes
   uint32_t n_instr;
   Instr prog[kMaxProg];
@@ -524,6 +524,8 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_gather_fmap(GatherMapArg
   }
   if (!(k0 || a.store_all))
     return;
+  if (!k0 && a.store_all == 2)
+    t0 = a.out_type == 2 ? 0.0f : __builtin_nanf("");
   if (a.out_type == 2)
     static_cast<uint8_t *>(a.out)[dst] = (uint8_t)(t0 != 0.0f);
   else if (a.out_type == 1)

@@ -3278,7 +3278,11 @@ int hcamdGatherMapLaunch(OlQueue q, HcamdGatherMap plan, const HcamdMapInstr *pr
     }
     a.nInstr = (uint32_t)nInstr;
     a.outType = outType == HCAMD_F32 ? 0u : outType == HCAMD_F16 ? 1u : 2u;
-    a.storeAll = storeAll ? 1u : 0u;
+    if (storeAll < 0 || storeAll > 2) {
+      dev->report("%s: storeAll is 0, 1 or 2", who);
+      return 1;
+    }
+    a.storeAll = (uint32_t)storeAll;
   }
   for (size_t i = 0; i <= plan->nInputs; ++i) {
     if (i < plan->nInputs) {

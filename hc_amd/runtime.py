@@ -962,7 +962,7 @@ def plan_gather_map(tables: GatherMap, program, inputs, out, types, out_type, st
     tys = (_int * max(n_in, 1))(*types[:n_in])
     return Plan(ctx, hcamdGatherMapLaunch,
                 (ctx.queue, tables.handle, prog, len(program), ptrs, tys, ms[-1].ptr, int(out_type),
-                 int(bool(store_all)), int(copy_bytes)), "hcamdGatherMapLaunch",
+                 int(store_all), int(copy_bytes)), "hcamdGatherMapLaunch",
                 (tables, inputs, out, prog, ptrs, tys))
 
 

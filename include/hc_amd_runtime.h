@@ -720,7 +720,10 @@ void hcamdGatherGemmRelease(HcamdGatherGemm plan) HCAMD_NOEXCEPT;
  * f is a program of hcamdLaunchFMap with its activity rules: an inactive operand
  * element is a zero that deactivates what is computed from it; an inactive
  * output position is not written, and neither is a deactivated result unless
- * storeAll.  With copyBytes != 0 (1, 2, 4 or 8) there is no program: operand 0
+ * storeAll: 1 writes the value the program leaves there, 2 writes NaN (a float
+ * out) or 0 (a bool out), which is what NumPy makes of numpy.ma's masked
+ * constant when the reference stores a bare numpy.ma array through a mapping
+ * (python/hckernel/kernel_api.py:331-334).  With copyBytes != 0 (1, 2, 4 or 8) there is no program: operand 0
  * is copied element by element whatever its type (a gathered / scattered copy).
  * Two active out elements of one launch must not share a destination (their
  * order is not defined).  `operands` holds the nInputs inputs, then the output;

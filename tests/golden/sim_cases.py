@@ -768,7 +768,54 @@ def case_plain_and_bare_arrays_next_to_tiles(api):
     return rec.out
 
 
+def case_mapped_loads_and_stores(api):
+    """Tiles loaded and stored through index mappings
+    (python/hckernel/kernel_api.py:296-335): which elements a mapped load
+    activates, what a mapped store writes for a tile, for a bare numpy.ma array
+    (its deactivated elements are numpy.ma's masked constant) and for a plain
+    array, into float32, float16, bool and int32 destinations."""
+    rec = Recorder()
+    x = (np.arange(24, dtype=np.float32).reshape(4, 6) - 7)
+    y = np.array([[1, 0, 2, 0, -1, 3]] * 4, np.float32)
+    shifted = api.create_mapping(lambda i, j: (i - 1, j + 2))
+    transpose = api.create_mapping(lambda i, j: (j, i))
+    dst = {n: np.full((5, 8), POISON, np.float32) for n in ("tile", "bare", "bare_unmapped", "plain", "quotient")}
+    dst16 = np.full((5, 8), POISON, np.float16)
+    dstb = np.full((5, 8), True)
+    dsti = np.full((5, 8), POISON, np.int32)
+
+    def body(gr, x, y, tile, bare, bare_unmapped, plain, quotient, dst16, dstb, dsti):
+        t = gr.load(x, shape=(4, 8), mapping=transpose)      # rows 0..3 of x's columns: a 4 x 4 part is active
+        rec.tile("transposed", t)
+        s = gr.load(x, shape=(4, 8), mapping=shifted)
+        rec.tile("shifted", s)
+        u = gr.load(x, shape=(4, 8))
+        gr.store(tile, u, mapping=shifted)
+        r = np.sqrt(u)                                     # a bare numpy.ma array: negative and inactive elements masked
+        rec.tile("sqrt", r)
+        gr.store(bare, r, mapping=shifted)
+        gr.store(bare_unmapped, r)
+        gr.store(plain, np.where(u.mask, u.data, 5), mapping=shifted)
+        q = u / gr.load(y, shape=(4, 8))
+        rec.tile("quotient", q)
+        gr.store(quotient, q, mapping=shifted)
+        gr.store(dst16, r.astype(np.float16), mapping=shifted)
+        gr.store(dstb, np.less(r, 2.5), mapping=shifted)
+        rec.attempt("int_destination", lambda: gr.store(dsti, r.astype(np.int32), mapping=shifted))
+
+    with np.errstate(all="ignore"), warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        _one_group(api, body, x, y, *dst.values(), dst16, dstb, dsti)
+    for n, a in dst.items():
+        rec.array("dst_" + n, a)
+    rec.array("dst_float16", dst16)
+    rec.array("dst_bool", dstb)
+    rec.array("dst_int32", dsti)
+    return rec.out
+
+
 CASES = {
+    "mapped_loads_and_stores": case_mapped_loads_and_stores,
     "plain_and_bare_arrays_next_to_tiles": case_plain_and_bare_arrays_next_to_tiles,
     "masked_reductions": case_masked_reductions,
     "inplace_partial": case_inplace_partial,

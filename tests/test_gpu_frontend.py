@@ -1154,8 +1154,22 @@ def _gather_bodies(deco, make_mapping):
         ta = gr.load(a[x:, y:], shape=(TM, TN), mapping=shifted)
         gr.store(out[x:, y:], np.exp(ta) + gr.load(b[x:, y:], shape=(TM, TN)))     # a bare array: stored in full
 
+    @deco(work_shape=(R, Cc), group_shape=(TM, TN))
+    def bare_array_scattered(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT], out: Buffer[R, Cc, DT]):
+        # numpy.ma's own array, element by element: a deactivated element is the
+        # masked constant, which NumPy turns into NaN (kernel_api.py:331-334)
+        x, y = gr.work_offset
+        ta = gr.load(a[x:, y:], shape=(TM, TN), mapping=diagonal)
+        gr.store(out[x:, y:], np.sqrt(ta) / gr.load(b[x:, y:], shape=(TM, TN)), mapping=shifted)
+
+    @deco(work_shape=(R, Cc), group_shape=(TM, TN))
+    def bare_copy_scattered(gr: CurrentGroup, a: Buffer[R, Cc, DT], b: Buffer[R, Cc, DT], out: Buffer[R, Cc, DT]):
+        x, y = gr.work_offset
+        gr.store(out[x:, y:], gr.load(a[x:, y:], shape=(TM, TN)).astype(a.dtype), mapping=shifted)
+
     return {"gathered_copy": gathered_copy, "gathered_expression": gathered_expression,
-            "scattered_store": scattered_store, "function_of_gathered": function_of_gathered}
+            "scattered_store": scattered_store, "function_of_gathered": function_of_gathered,
+            "bare_array_scattered": bare_array_scattered, "bare_copy_scattered": bare_copy_scattered}
 
 
 @pytest.mark.parametrize("rows,cols", [(16, 32), (37, 50), (8, 16)])
@@ -1172,7 +1186,8 @@ def test_mapped_loads_and_stores_outside_a_product_match_the_simulator(rows, col
     cases = {"gathered_copy": ([at], (rows, cols))}
     if dtype != np.int32:
         cases.update({"gathered_expression": ([a, b], (rows, cols)), "scattered_store": ([a, b], (2 * rows, cols)),
-                      "function_of_gathered": ([a, b], (rows, cols))})
+                      "function_of_gathered": ([a, b], (rows, cols)),
+                      "bare_array_scattered": ([a, b], (rows, cols)), "bare_copy_scattered": ([a, b], (rows, cols))})
     for name, (ins, shape) in cases.items():
         want = np.full(shape, 7, dtype)
         with np.errstate(all="ignore"):
@@ -1190,6 +1205,8 @@ def test_mapped_loads_and_stores_outside_a_product_match_the_simulator(rows, col
             assert_array_equal(got.view(bits), want.view(bits), err_msg=name)
         if name in ("gathered_expression", "scattered_store"):
             assert (want == 7).any(), name               # something is left alone
+        if name.startswith("bare_") and (rows, cols) == (37, 50):
+            assert np.isnan(want).any() and (want == 7).any(), name     # masked constants, and places no index reaches
 
 
 def _window_bodies(deco):
