@@ -890,6 +890,11 @@ HCAMD_GEMM_PZ(hcamd_gemm_bf16_probe_two_tiles, 9)
 HCAMD_GEMM_W2X2(hcamd_gemm_bf16_probe_w2x2_reads48, 48, 1, 4, 0)
 HCAMD_GEMM_W2X2(hcamd_gemm_bf16_probe_w2x2_loads2, 24, 1, 2, 0)
 HCAMD_GEMM_W2X2(hcamd_gemm_bf16_probe_w2x2_a_inner, 24, 1, 4, 1)
+// the bare MFMA stream with the accumulators stored straight from registers, in
+// 16 x 16 x 32 and in 32 x 32 x 16 blocks (half the operand registers read per
+// multiply-add): what the block shape alone does to the clock
+HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_mfma16_direct, __bf16, 256, 256, 2, 4, 16, 0, false, 1)
+HCAMD_GEMM_PX(hcamd_gemm_bf16_probe_mfma32_direct, __bf16, 256, 256, 2, 4, 32, 0, false, 1)
 #endif
 HCAMD_GEMM_PE(hcamd_gemm_bf16_p256x256_w2x4_edge, __bf16, 256, 256, 2, 4, 16)
 HCAMD_GEMM_PE(hcamd_gemm_f16_p256x256_w2x4_edge, _Float16, 256, 256, 2, 4, 16)

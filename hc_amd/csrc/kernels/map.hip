@@ -2514,6 +2514,20 @@ __device__ __forceinline__ void layer_norm_rows(const void *__restrict__ x, size
   const bool row_gone = !is_finite(RMS ? mean_sq : mean);
   if (!live || (row_gone && !frozen))
     return;
+  // Dividing a whole row by one scalar: s_inv = 1.0 / (double)s is formed once
+  // and a quotient is float(double(y) * s_inv).  That is the correctly rounded
+  // fp32 quotient whenever it is a normal number: the product is within 2^-52
+  // (relative) of y / s, and a quotient of two 24-bit significands that is not
+  // itself representable lies at least 2^-49 (relative) from every fp32 value and
+  // from every midpoint between two, so both round the same way.  A chunk whose
+  // quotients are all normal numbers, or zeros that come from zero dividends
+  // (s > 0: the quotient keeps the dividend's sign, and numpy.ma's 0 * dividend
+  // added to it changes nothing), has nothing deactivated and takes the short
+  // way; any other chunk (a quotient that is not finite, or below the normal
+  // range, where fp32 values lie further apart and an exact tie is possible) is
+  // divided the long way with numpy.ma's bookkeeping.
+  const double s_inv = 1.0 / (double)s;
+  const bool s_plain = s > 0.0f && !row_gone;
   char *orow = static_cast<char *>(out) + (size_t)row * ldo * (HALF ? 2 : 4);
 #pragma unroll
   for (int e = 0; e < E; ++e) {
@@ -2535,6 +2549,36 @@ __device__ __forceinline__ void layer_norm_rows(const void *__restrict__ x, size
 #pragma unroll
       for (int k = 0; k < C; ++k)
         y[k] = RMS ? v[e][k] : __fsub_rn(v[e][k], mean);
+      float quo[C];
+      uint32_t lo = 255u, hi = 0u;
+#pragma unroll
+      for (int k = 0; k < C; ++k) {
+        quo[k] = (float)((double)y[k] * s_inv);
+        const uint32_t ex = (__builtin_bit_cast(uint32_t, quo[k]) >> 23) & 255u;
+        lo = ex < lo ? ex : lo;
+        hi = ex > hi ? ex : hi;
+      }
+      bool plain = s_plain && hi != 255u;
+      if (plain && lo == 0u) {
+#pragma unroll
+        for (int k = 0; k < C; ++k)
+          plain = plain && (((__builtin_bit_cast(uint32_t, quo[k]) >> 23) & 255u) != 0u || y[k] == 0.0f);
+      }
+      if (plain) {
+#pragma unroll
+        for (int k = 0; k < C; ++k)
+          y[k] = RMS ? __fmul_rn(quo[k], wv[k]) : __fadd_rn(__fmul_rn(quo[k], wv[k]), bv[k]);
+        if constexpr (HALF) {
+          f16x8 h;
+#pragma unroll
+          for (int k = 0; k < C; ++k)
+            h[k] = (_Float16)y[k];
+          stg<true>(reinterpret_cast<f16x8 *>(orow) + c, h);
+        } else {
+          stg<true>(reinterpret_cast<f32x4 *>(orow) + c, f32x4{y[0], y[1], y[2], y[3]});
+        }
+        continue;
+      }
       uint32_t bad = 0;
       float kept[C];
 #pragma unroll
@@ -2591,6 +2635,8 @@ __device__ __forceinline__ void layer_norm_rows(const void *__restrict__ x, size
 // 1024 lanes with two 51.4, on 256 with eight 53.4)
 HCAMD_LAYER_NORM(64, 1)
 HCAMD_LAYER_NORM(64, 2)
+HCAMD_LAYER_NORM(128, 4)
+HCAMD_LAYER_NORM(512, 1)
 HCAMD_LAYER_NORM(128, 2)
 HCAMD_LAYER_NORM(256, 2)
 HCAMD_LAYER_NORM(512, 2)

@@ -269,7 +269,7 @@ std::unordered_map<std::string, int> &variants() {
   static std::unordered_map<std::string, int> v{
       {"add", 0},     {"fma", 0},  {"softmax", 0},
       {"quantize", 0}, {"gemm", 0}, {"copy", 0}, {"map", 0},
-      {"gather", 0}, {"gather_fuse", 0}, {"rows", 0}, {"stream", 0}, {"cols", 0}};
+      {"gather", 0}, {"gather_fuse", 0}, {"rows", 0}, {"stream", 0}, {"cols", 0}, {"norm", 0}};
   return v;
 }
 std::mutex g_variantLock; // guards variants()
@@ -730,8 +730,8 @@ int hcamdDeviceInfo(OlDevice dev, int *computeUnits, int *clockKHz,
 }
 
 namespace {
-// Variants 17..22, 26, 28 and 29 of "gemm" are measurement builds of the default kernel
-// with one part of its loop taken out: what they leave in C is not the product
+// Variants 17..22, 26, 28, 29, 33 and 34 of "gemm" are measurement builds of the default
+// kernel with one part of its loop taken out: what they leave in C is not the product
 // (30..32 are further hand orders of variant 27 that only measurements select).
 // They exist only in a library built with HCAMD_PROBES defined (`python -m
 // hc_amd.build --probes`); any other build refuses to select them.
@@ -741,7 +741,7 @@ bool variantIsAbsentProbe(const char *family, int variant) {
   return false;
 #else
   return std::strcmp(family, "gemm") == 0 &&
-         ((variant >= 17 && variant <= 22) || variant == 26 || (variant >= 28 && variant <= 32));
+         ((variant >= 17 && variant <= 22) || variant == 26 || (variant >= 28 && variant <= 34));
 #endif
 }
 } // namespace
@@ -2423,6 +2423,11 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
         lpr = 1024;
       while (lpr * e < chunks)
         e *= 2;
+      // variants of "norm", for measurements: 1 twice the lanes to a row, 2 half of them
+      if (variantOf("norm") == 1 && lpr < 1024 && e > 1)
+        lpr *= 2, e /= 2;
+      else if (variantOf("norm") == 2 && lpr > 64 && e < 8)
+        lpr /= 2, e *= 2;
       std::snprintf(name, sizeof name, "hcamd_%s_norm_%s_w%zu_e%zu", rmsForm ? "rms" : "layer",
                     half ? "f16" : "f32", lpr, e);
       const size_t t = std::max(lpr, (size_t)256);
@@ -3593,6 +3598,8 @@ int launchGemm(OlQueue q, bool half, const void *a, size_t lda, const void *bt,
       {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_w2x2_reads48"), 256, 256, 256}, // 30..32: other hand orders of 27
       {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_w2x2_loads2"), 256, 256, 256},  //         (the product, measurement builds only)
       {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_w2x2_a_inner"), 256, 256, 256},
+      {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_mfma16_direct"), 256, 256, 512}, // 33, 34: measurement only
+      {HCAMD_PROBE_NAME("hcamd_gemm_bf16_probe_mfma32_direct"), 256, 256, 512},
   };
   constexpr int kGeneral = 6;
   constexpr int kFirstPipelined = 7; // variants from here need K >= 128

@@ -1085,7 +1085,7 @@ def probes_built() -> bool:
 
 
 def _variant_error(family: str, variant: int) -> HcRuntimeError:
-    if family == "gemm" and (17 <= variant <= 22 or variant in (26, 28, 29, 30, 31, 32)) and not probes_built():
+    if family == "gemm" and (17 <= variant <= 22 or variant in (26, 28, 29, 30, 31, 32, 33, 34)) and not probes_built():
         return HcRuntimeError(f"gemm variant {variant} is a measurement build whose output is not the "
                               "product; this library was built without them (python -m hc_amd.build "
                               "--probes builds them)")

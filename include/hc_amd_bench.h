@@ -39,9 +39,11 @@ int hcamdLaunchStream(OlQueue q, int nReads, int writeMode, const void *const *i
  * variants 17..22, 26, 28 and 29: the default 256 x 256 kernel with its MFMAs
  * only, without its waits on loads, without its barriers, without its LDS
  * reads, without its loads, with its loads to registers, with B read directly,
- * without its stores, with two K tiles only; and 30..32, further hand orders of
- * the four-wave kernel of variant 27 that only measurements select).  What
- * 17..29 of them leave in C is NOT the product.  They are compiled only when the
+ * without its stores, with two K tiles only; 30..32, further hand orders of
+ * the four-wave kernel of variant 27 that only measurements select; 33 and 34,
+ * the MFMAs only in 16 x 16 x 32 and in 32 x 32 x 16 blocks with C stored
+ * straight from the accumulators).  What 17..29, 33 and 34 leave in C is NOT
+ * the product.  They are compiled only when the
  * library is built with `python -m hc_amd.build --probes` (HCAMD_PROBES); any
  * other build returns 0 here, holds none of them, and hcamdSetVariant /
  * hcamdSetThreadVariant return 1 for their numbers. */

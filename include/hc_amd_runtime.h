@@ -783,11 +783,12 @@ int hcamdLaunchGemmF16(OlQueue q, const void *a, size_t lda, const void *bt,
 
 /* Chooses between kernel variants of one family by number (0 = default
  * choice by shape).  For tuning and measurement; family names are "add",
- * "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "cols", "stream", "gather"
+ * "fma", "softmax", "quantize", "gemm", "copy", "map", "rows", "cols", "stream", "norm"
+ * (lanes to a row in the normalisation kernels: 1 twice, 2 half as many), "gather"
  * (block shape), "gather_fuse" (groups per workgroup; read by
  * hcamdGatherGemmCreate).
  * Process-wide, guarded by a lock.  Returns 1 for an unknown family, and for
- * the numbers of the measurement builds of the "gemm" family (17..22, 26, 28..32:
+ * the numbers of the measurement builds of the "gemm" family (17..22, 26, 28..34:
  * most of them leave something other than the product in C) unless the library was built with them
  * (hc_amd_bench.h).  Every variant a default build accepts computes the same
  * result as variant 0. */

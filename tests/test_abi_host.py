@@ -48,7 +48,7 @@ def test_measurement_entry_points_have_a_header_of_their_own_and_probes_stay_out
     # a default build holds no kernel whose output is not the product, and
     # refuses the numbers that would select one
     assert b"hcamd_gemm_bf16_probe" not in blob
-    for v in (17, 18, 19, 20, 21, 22, 26, 28, 29, 30, 31, 32):
+    for v in (17, 18, 19, 20, 21, 22, 26, 28, 29, 30, 31, 32, 33, 34):
         assert rt.hcamdSetVariant(b"gemm", v) == 1 and rt.hcamdSetThreadVariant(b"gemm", v) == 1
         with pytest.raises(rt.HcRuntimeError, match="--probes"):
             rt.set_variant("gemm", v)
