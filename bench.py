@@ -406,6 +406,26 @@ def make_workloads(rt, wl):
         def plan(self, rt, s):
             return rt.plan_map([I("in", 0), I("mul_in", 1), I("add_in", 2)], s[:3], s[3])
 
+    class X9(C2):
+        """max(sqrt(|a*b+c|) * a - b, 0) * 0.5 on the C2 arrays: a 9-instruction program that never
+        holds two values at once, which the map entry point runs on its chain kernel."""
+        PROGRAM = [("in", 0), ("mul_in", 1), ("add_in", 2), ("abs", 0), ("sqrt", 0), ("mul_in", 0), ("sub_in", 1),
+                   ("maxi", 0, 0.0), ("muli", 0, 0.5)]
+
+        def plan(self, rt, s):
+            return rt.plan_map([I(*p) for p in self.PROGRAM], s[:3], s[3])
+
+        def numpy_result(self):
+            a, b, c = (v.astype(np.float32) for v in (self.a, self.b, self.c))
+            return (np.maximum(np.sqrt(np.abs(a * b + c)) * a - b, np.float32(0)) * np.float32(0.5)).astype(np.float16)
+
+        def check(self, rt, s):
+            ok = np.array_equal(s[3].to_host().view(np.uint16), self.numpy_result().view(np.uint16))
+            return {"parity": "bit-exact vs NumPy (fp32 steps, one rounding to fp16)" if ok else "MISMATCH", "ok": bool(ok)}
+
+        def cpu(self):
+            return _best_of(self.numpy_result, 2), "full size, NumPy fp32 expression", 1
+
     class X7(C1):
         """a+b on the C1 vectors through the fused map kernel (2 instructions)."""
 
@@ -619,6 +639,8 @@ def make_workloads(rt, wl):
                  W.work_c1(), "GB/s"),
         "x8": X8("x8", "row program: rms norm fp16 16384x4096 with an fp32 weight (fp32 math)", "f16", "hbm",
                  2 * 2 * 16384 * 4096 + 4 * 4096, "GB/s"),
+        "x9": X9("x9", "map kernel: a 9-instruction chain on the fp16 8191x8193 arrays", "f16", "hbm",
+                 W.work_c2(), "GB/s"),
     }
     # the mix and size of each memory-bound configuration, then the plain streams
     for key, n_reads, write, mib in STREAMS:
@@ -628,7 +650,7 @@ def make_workloads(rt, wl):
     elif wl == "streams":
         keys = [k for k, *_ in STREAMS]
     elif wl == "extra":
-        keys = ["x1", "x2", "x3", "x4", "x5", "x6", "x7", "x8"]
+        keys = ["x1", "x2", "x3", "x4", "x5", "x6", "x7", "x8", "x9"]
     else:
         keys = [wl]
     return [table[k] for k in keys]
@@ -703,7 +725,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="all", choices=["all", "streams", "c0", "c1", "c2", "c3", "c4", "c5", "v5", "extra", "x1", "x2", "x3",
-                             "x4", "x5", "x6", "x7", "x8"] + [k for k, *_ in STREAMS])
+                             "x4", "x5", "x6", "x7", "x8", "x9"] + [k for k, *_ in STREAMS])
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy CPU baseline")
     ap.add_argument("--variant", action="append", default=[], metavar="FAMILY=N",
                     help="measure kernel variant N of a family (hcamdSetVariant), e.g. gemm=14; "

@@ -2430,6 +2430,152 @@ HCAMD_ROW_CHAIN(256, 4, 256)
 HCAMD_ROW_CHAIN(512, 4, 512)
 HCAMD_ROW_CHAIN(1024, 4, 1024)
 
+// ---- the flat map for chains ---------------------------------------------------------
+// A program that never holds two values at once (an operand or a constant, then
+// operations that change the value in place) on dense arrays: one dispatch of
+// the chain interpreter works on sixteen elements of a lane, and there is one
+// level of dispatch instead of two (the general interpreter also branches on the
+// stack depth), so an interpreted instruction costs a third of the scalar issue
+// per element.  A workgroup owns 4096 consecutive elements; a lane's sixteen are
+// four runs of four, 1024 elements apart (16-byte accesses to fp32 arrays, 8-byte
+// ones to fp16 arrays, whole cache lines per wave either way), or, when every
+// array is fp16 (ALLH), two runs of eight, 2048 elements apart (16-byte
+// accesses).  The elements past the last whole region go through the general
+// interpreter in one more workgroup, the first of the grid: it takes longer than
+// the others and would otherwise finish alone after them.
+namespace {
+template <int NIN, bool ALLH>
+__device__ __forceinline__ void map_chain(const MapArgs &a, const uint32_t n_in) {
+  constexpr int NE = 16, P = 2;
+  const size_t n = a.cols;
+  const size_t regions = n / 4096;
+  const uint32_t t = threadIdx.x;
+  const bool out_f16 = (a.f16_mask >> 8) & 1;
+  const uint32_t extra = n % 4096 ? 1u : 0u;
+  if (extra && blockIdx.x == 0) {
+    Raw raw;
+    Stack r;
+#pragma nounroll
+    for (size_t first = regions * 4096 + (size_t)t * 8; first < n; first += 256 * 8) {
+      gather(a, n_in, raw, [&](int, int e, size_t &off) {
+        off = first + e;
+        return off < n;
+      });
+      run_program(a, raw, 0, r);
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (first + e < n && !((r.bad >> e) & 1u))
+          store_elem(a.out, out_f16, first + e, r.st[0][e]);
+    }
+    return;
+  }
+  const size_t base = (size_t)(blockIdx.x - extra) * 4096;
+  u32x4 w[NIN][P][2];
+#pragma unroll
+  for (int i = 0; i < NIN; ++i)
+    if (i < (int)n_in) {
+      if constexpr (ALLH) {
+        const u32x4 *q = static_cast<const u32x4 *>(a.in[i]) + base / 8 + t;
+#pragma unroll
+        for (int p = 0; p < P; ++p)
+          w[i][p][0] = ldg<true>(q + p * 256);
+      } else if ((a.f16_mask >> i) & 1) {
+        const u32x2 *q = static_cast<const u32x2 *>(a.in[i]) + base / 4 + t;
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+          const u32x2 lo = ldg<true>(q + (2 * p) * 256), hi = ldg<true>(q + (2 * p + 1) * 256);
+          w[i][p][0] = u32x4{lo.x, lo.y, hi.x, hi.y};
+        }
+      } else {
+        const u32x4 *q = static_cast<const u32x4 *>(a.in[i]) + base / 4 + t;
+#pragma unroll
+        for (int p = 0; p < P; ++p)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            w[i][p][j] = ldg<true>(q + (2 * p + j) * 256);
+      }
+    }
+  float v[NE];
+  uint32_t bad = 0;
+#pragma unroll
+  for (int e = 0; e < NE; ++e)
+    v[e] = 0.0f;
+  Instr next = a.prog[0];
+#pragma nounroll
+  for (uint32_t pc = 0; pc < a.n_instr; ++pc) {
+    const Instr cur = next;
+    next = a.prog[(pc + 1) & (kMaxProg - 1)];
+    const uint32_t op = cur.op, arg = cur.arg;
+    const float imm = cur.imm;
+    const bool half = (arg & 0x100u) != 0;
+    if (chain_reads(op)) {
+      auto use = [&](auto number) {
+        constexpr int I = decltype(number)::value;
+        if constexpr (I < NIN)
+          chain_operand<NE>(op, v, bad, half,
+                            chain_words([&](int p, int j, int c) { return w[I][p][j][c]; },
+                                        ALLH || ((a.f16_mask >> I) & 1)));
+      };
+      switch (arg & 3u) {
+      case 0: use(std::integral_constant<int, 0>{}); break;
+      case 1: use(std::integral_constant<int, 1>{}); break;
+      case 2: use(std::integral_constant<int, 2>{}); break;
+      default: use(std::integral_constant<int, 3>{}); break;
+      }
+    } else {
+      chain_plain<NE>(op, v, bad, imm, half);
+    }
+  }
+  if constexpr (ALLH) {
+    _Float16 *o = static_cast<_Float16 *>(a.out) + base + (size_t)t * 8;
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      if ((bad >> (8 * p)) & 0xffu) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (!((bad >> (8 * p + e)) & 1u))
+            o[p * 2048 + e] = (_Float16)v[8 * p + e];
+      } else {
+        f16x8 h;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          h[e] = (_Float16)v[8 * p + e];
+        stg<true>(reinterpret_cast<f16x8 *>(o + p * 2048), h);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const size_t at = base + (size_t)g * 1024 + (size_t)t * 4;
+      const uint32_t bits = (bad >> (4 * g)) & 0xfu;
+      if (bits) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (!((bits >> e) & 1u))
+            store_elem(a.out, out_f16, at + e, v[4 * g + e]);
+      } else if (out_f16) {
+        f16x4 h;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          h[e] = (_Float16)v[4 * g + e];
+        stg<true>(reinterpret_cast<f16x4 *>(static_cast<_Float16 *>(a.out) + at), h);
+      } else {
+        stg<true>(reinterpret_cast<f32x4 *>(static_cast<float *>(a.out) + at),
+                  f32x4{v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3]});
+      }
+    }
+  }
+}
+} // namespace
+#define HCAMD_MAP_CHAIN(NAME, NIN, ALLH)                                                  \
+  extern "C" __global__ __launch_bounds__(256) void NAME(const MapArgs a, const uint32_t n_in) { \
+    map_chain<NIN, ALLH>(a, n_in);                                                        \
+  }
+HCAMD_MAP_CHAIN(hcamd_map_chain_n2, 2, false)
+HCAMD_MAP_CHAIN(hcamd_map_chain_n4, 4, false)
+HCAMD_MAP_CHAIN(hcamd_map_chain_n2h, 2, true)
+HCAMD_MAP_CHAIN(hcamd_map_chain_n4h, 4, true)
+
 // ---- layer normalisation without the interpreter -----------------------------------
 // The six-stage row program  mean = sum(x) / n;  var = sum((x - mean) *
 // (x - mean)) / n;  s = sqrt(var + eps);  out = (x - mean) / s * w + b  (the

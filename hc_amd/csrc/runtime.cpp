@@ -1420,6 +1420,23 @@ int launchMap(OlQueue q, bool sum, const HcamdMapInstr *prog, size_t nInstr,
       name = "hcamd_map_flat_n2u4h"; // (variant 3 of "map": one chunk per lane whatever the operands)
       u = 4;
     }
+    // A chain (an operand or a constant first, then only operations that change
+    // the value in place) of five instructions or more runs on the chain
+    // interpreter, sixteen elements of a lane to a dispatch (variant 4 of "map":
+    // every chain; 5: none).
+    if (!sum && a.cols >= 4096 && variantOf("map") != 5 && variantOf("map") != 3 &&
+        (nInstr >= 5 || variantOf("map") == 4)) {
+      bool chain = prog[0].op == HCAMD_MAP_IN || prog[0].op == HCAMD_MAP_CONST;
+      for (size_t pc = 1; pc < nInstr && chain; ++pc)
+        chain = !(prog[pc].op <= HCAMD_MAP_RDIV || prog[pc].op == HCAMD_MAP_MDIV ||
+                  prog[pc].op == HCAMD_MAP_RMDIV);
+      if (chain) {
+        const bool allHalf = half && outType == HCAMD_F16;
+        const char *chainName = nInputs <= 2 ? (allHalf ? "hcamd_map_chain_n2h" : "hcamd_map_chain_n2")
+                                             : (allHalf ? "hcamd_map_chain_n4h" : "hcamd_map_chain_n4");
+        return launch1d(queue, "map", chainName, a.cols / 4096 + (a.cols % 4096 ? 1 : 0), 256, args);
+      }
+    }
     // the reduction: 1024-lane workgroups, one per CU, each striding over the
     // vector and ending in one atomic addition
     const size_t threads = sum ? 1024 : 256;

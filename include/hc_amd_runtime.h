@@ -282,7 +282,11 @@ int hcamdLaunchFmaF16(OlQueue q, const void *a, size_t lda, const void *b,
  * propagate NaN like numpy.maximum / numpy.minimum; the store rounds to
  * nearest even.  Operands are fp32 or fp16, each with its own leading
  * dimension in elements.  The program is validated on the host; a malformed
- * one is an error, not a launch. */
+ * one is an error, not a launch.  On dense arrays a program of five
+ * instructions or more that never holds two values at once (IN or CONST first,
+ * then no further push and no two-value operation) runs on a kernel that
+ * interprets sixteen elements of a lane per dispatch; the results are the same
+ * bit for bit (variant 4 of the "map" family: every such program, 5: none). */
 enum HcamdElemType { HCAMD_F32 = 0, HCAMD_F16 = 1, HCAMD_BF16 = 2, HCAMD_I32 = 3, HCAMD_I64 = 4,
                      HCAMD_U8 = 5 };
 enum HcamdMapOp {

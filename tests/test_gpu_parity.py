@@ -1003,6 +1003,45 @@ def test_map_fma_program_equals_the_fma_kernel(ctx, shape, variant):
     assert_array_equal(want.view(np.uint16), co.fma_f16(a, b, c).view(np.uint16))
 
 
+@pytest.mark.parametrize("n", [4096, 4097, 3 * 4096 + 4095, 1 << 20])
+@pytest.mark.parametrize("types", [(np.float16,) * 5, (np.float32,) * 5,
+                                   (np.float16, np.float32, np.float32, np.float16, np.float16),
+                                   (np.float32, np.float16, np.float16, np.float32, np.float32)])
+@pytest.mark.parametrize("n_in", [1, 2, 4])
+def test_map_chains_equal_the_general_interpreter(ctx, n, types, n_in):
+    """A program that never holds two values at once runs on the chain kernels
+    (sixteen elements of a lane to a dispatch) on dense arrays: bit for bit what
+    the general interpreter stores, the same elements left alone (zero divisors
+    of the numpy.ma division, roots and logarithms outside their domain), and
+    nothing written past the end."""
+    rng = np.random.default_rng(n + n_in)
+    ins = [rng.integers(-3, 4, n + 8).astype(np.float64) * 0.5 for _ in range(4)]
+    program = [I("in", 0), I("mul_in", (1) % n_in), I("add_in", (2) % n_in), I("abs"), I("sqrt"),
+               I("mdiv_in", (3) % n_in | (0x100 if types[4] == np.float16 else 0)), I("sub_in", 0), I("maxi", 0, -1.5),
+               I("msqrt"), I("muli", 0, 0.5), I("rsubi", 0, 2.0), I("exp")]
+    devs = [dev(x.astype(t)) for x, t in zip(ins, types)]
+    views = [_View(d, (n,), 0, (1,)) for d in devs[:n_in]]
+    got = {}
+    for variant, prefix in ((0, "hcamd_map_chain_n"), (5, "hcamd_map_flat")):
+        out = poisoned((n + 8,), types[4])
+        rt.set_variant("map", variant)
+        try:
+            rt.plan_map(program, views, _View(out, (n,), 0, (1,))).launch(sync=True)
+        finally:
+            rt.set_variant("map", 0)
+        assert rt.last_kernel_name().startswith(prefix), rt.last_kernel_name()
+        if variant == 0:
+            all_half = all(t == np.float16 for t in types[:n_in] + types[4:])
+            assert rt.last_kernel_name() == f"hcamd_map_chain_n{2 if n_in <= 2 else 4}{'h' if all_half else ''}"
+        got[variant] = out.to_host()
+    bits = np.uint16 if types[4] == np.float16 else np.uint32
+    assert_array_equal(got[0].view(bits), got[5].view(bits))
+    p = poison_value(types[4])
+    assert (got[0][n:].view(bits) == p.view(bits)).all()
+    left_alone = got[0][:n].view(bits) == p.view(bits)
+    assert left_alone.any() and not left_alone.all()
+
+
 def test_map_window_of_larger_arrays_leaves_the_rest_untouched(ctx):
     rows, cols = 37, 1031
     a, b, c = cf.inputs_c2((rows, cols))
