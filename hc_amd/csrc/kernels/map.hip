@@ -2777,8 +2777,10 @@ __device__ __forceinline__ void layer_norm_rows(const void *__restrict__ x, size
   HCAMD_NORM_KERNEL(hcamd_layer_norm_f32_w##LPR##_e##E, LPR, E, false, false)             \
   HCAMD_NORM_KERNEL(hcamd_rms_norm_f32_w##LPR##_e##E, LPR, E, true, false)                \
   HCAMD_NORM_KERNEL(hcamd_rms_norm_f16_w##LPR##_e##E, LPR, E, true, true)
-// (a row of 8192 on 512 lanes with four chunks each: 49.9 us for 4096 rows; on
-// 1024 lanes with two 51.4, on 256 with eight 53.4)
+// (a row of 8192 on 512 lanes with four chunks each: 48.3 us for 4096 rows; on
+// 1024 lanes with two 50.1, on 256 with eight 51.1; with the weights and biases
+// requested behind the row instead of where they are used 50.8: the registers
+// that hold them cost a workgroup per compute unit)
 HCAMD_LAYER_NORM(64, 1)
 HCAMD_LAYER_NORM(64, 2)
 HCAMD_LAYER_NORM(128, 4)
@@ -2787,5 +2789,7 @@ HCAMD_LAYER_NORM(128, 2)
 HCAMD_LAYER_NORM(256, 2)
 HCAMD_LAYER_NORM(512, 2)
 HCAMD_LAYER_NORM(512, 4)
+HCAMD_LAYER_NORM(256, 8)
+HCAMD_LAYER_NORM(1024, 2)
 HCAMD_LAYER_NORM(1024, 4)
 HCAMD_LAYER_NORM(1024, 8)

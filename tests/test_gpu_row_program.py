@@ -244,6 +244,46 @@ def test_rms_normalisation_as_the_front_end_writes_it_takes_its_own_kernel(ctx, 
                                                                dict(rtol=3e-6, atol=3e-6)))
 
 
+def test_rms_normalisation_divides_exactly_where_quotients_leave_the_normal_range(ctx):
+    """The normalisation kernels divide by the row's scale through one
+    double-precision reciprocal and go the long way for quotients below the
+    normal range, where that shortcut can break a tie the wrong way.  Rows built
+    so that the scale is exactly 3 * 2^34 whatever the order of the sums (one
+    element 3 * 2^40, every other square underflows to nothing), with elements
+    3 * m * 2^-120 whose quotients m * 2^-154 need rounding to multiples of
+    2^-149, half of them exact ties; zeros of both signs keep their sign.  Every
+    kernel must store the IEEE quotient bit for bit."""
+    rows, cols = 6, 4096
+    m = np.arange(cols, dtype=np.float64)
+    x = np.empty((rows, cols), np.float32)
+    for r in range(rows):
+        x[r] = (3.0 * (m * (2 * r + 1) % 4099) * 2.0 ** -120).astype(np.float32)
+        x[r, 1::7] *= -1
+        x[r, 5] = 0.0
+        x[r, 6] = -0.0
+        x[r, 0] = 3.0 * 2.0 ** 40
+    s = np.float32(3.0 * 2.0 ** 34)
+    assert np.sqrt((x.astype(np.float64) ** 2).sum(axis=1) / cols).astype(np.float32).tolist() == [float(s)] * rows
+    want = x / s
+    assert (np.abs(want[:, 1:]) < np.float32(1.17549435e-38)).all() and (want[:, 1:] != 0).sum() > rows * 4000
+    # some quotients are exact ties between two subnormal numbers
+    assert ((x[:, 1:].astype(np.float64) / float(s) / 2.0 ** -150) % 2 == 1).sum() > 100
+    stages = [("sum", 0, [I("in", 0), I("mul_in", 0)]),
+              ("scalar", 1, [I("red", 0), I("mdivi", 0, float(cols)), I("addi", 0, 0.0), I("msqrt")]),
+              ("store", 0, [I("in", 0), I("mdiv_red", 1), I("mul_in", 1)])]
+    dx, dg = rt.to_device(x), rt.to_device(np.ones(cols, np.float32))
+    for variant in (1, 2, 0):
+        rt.set_variant("rows", variant)
+        try:
+            out = poisoned((rows, cols), np.float32)
+            rt.plan_row_program(stages, [dx, dg], out).launch(sync=True)
+            name = rt.last_kernel_name()
+        finally:
+            rt.set_variant("rows", 0)
+        assert name.startswith("hcamd_rms_norm_f32") == (variant == 0)
+        assert_array_equal(out.to_host().view(np.uint32), want.view(np.uint32), err_msg=name)
+
+
 @pytest.mark.parametrize("rows,cols", [(1000, 7), (129, 1031), (4, 70_001), (5000, 264), (1300, 3000)])
 def test_row_sums_maxima_and_minima_as_per_row_results(ctx, rows, cols, rows_variant):
     rng = np.random.default_rng(rows)
