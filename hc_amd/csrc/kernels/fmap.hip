@@ -51,13 +51,13 @@
 // elements per lane (one 16-byte fp32 or 8-byte fp16 access per operand where
 // rows allow it).  This is a correctness path for HBM-bound work, not tuned.
 #include "common.h"
+#include <type_traits>
 
 using namespace hcamd;
 
 namespace {
 constexpr int kMaxIn = 4;
 constexpr int kMaxProg = 48;
-constexpr int kV = 4;
 
 enum : uint32_t {
   FOP_END = 0, FOP_IN = 1, FOP_CONST = 2,
@@ -257,57 +257,66 @@ __device__ __forceinline__ float unary(uint32_t op, float a, uint32_t arg, bool 
 }
 } // namespace
 
-extern "C" __global__ __launch_bounds__(256) void hcamd_fmap(FMapArgs a) {
+// V elements of a lane to a dispatch of the interpreter, consecutive in the row
+// and moved in pieces of four (16 bytes of fp32, 8 of fp16).
+namespace {
+template <int V> __device__ __forceinline__ void fmap_row_pieces(const FMapArgs &a) {
   const size_t row = blockIdx.y;
-  const size_t col0 = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * kV;
+  const size_t col0 = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
   if (col0 >= a.cols)
     return;
-  const bool whole = col0 + kV <= a.cols;
-  float v[kMaxIn][kV];
+  const bool whole = col0 + V <= a.cols;
+  float v[kMaxIn][V];
 #pragma unroll
   for (int i = 0; i < kMaxIn; ++i) {
     if (!a.in[i]) { // uniform: operands are packed from 0
 #pragma unroll
-      for (int e = 0; e < kV; ++e)
+      for (int e = 0; e < V; ++e)
         v[i][e] = 0.0f;
       continue;
     }
     if ((a.f16_mask >> i) & 1) {
       const _Float16 *p = static_cast<const _Float16 *>(a.in[i]) + row * a.ld[i] + col0;
       if (a.vec && whole) {
-        const f16x4 w = *reinterpret_cast<const f16x4 *>(p);
 #pragma unroll
-        for (int e = 0; e < kV; ++e)
-          v[i][e] = (float)w[e];
+        for (int g = 0; g < V / 4; ++g) {
+          const f16x4 w = ldg<true>(reinterpret_cast<const f16x4 *>(p) + g);
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            v[i][4 * g + e] = (float)w[e];
+        }
       } else {
 #pragma unroll
-        for (int e = 0; e < kV; ++e)
+        for (int e = 0; e < V; ++e)
           v[i][e] = col0 + e < a.cols ? (float)p[e] : 0.0f;
       }
     } else if ((a.f16_mask >> (8 + i)) & 1) {
       const int32_t *p = static_cast<const int32_t *>(a.in[i]) + row * a.ld[i] + col0;
 #pragma unroll
-      for (int e = 0; e < kV; ++e)
+      for (int e = 0; e < V; ++e)
         v[i][e] = col0 + e < a.cols ? (float)p[e] : 0.0f;
     } else {
       const float *p = static_cast<const float *>(a.in[i]) + row * a.ld[i] + col0;
       if (a.vec && whole) {
-        const f32x4 w = *reinterpret_cast<const f32x4 *>(p);
 #pragma unroll
-        for (int e = 0; e < kV; ++e)
-          v[i][e] = w[e];
+        for (int g = 0; g < V / 4; ++g) {
+          const f32x4 w = ldg<true>(reinterpret_cast<const f32x4 *>(p) + g);
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            v[i][4 * g + e] = w[e];
+        }
       } else {
 #pragma unroll
-        for (int e = 0; e < kV; ++e)
+        for (int e = 0; e < V; ++e)
           v[i][e] = col0 + e < a.cols ? p[e] : 0.0f;
       }
     }
   }
   // the stack and, beside every entry, whether the element is still active in it
-  float t0[kV], t1[kV], t2[kV], t3[kV];
-  bool k0[kV], k1[kV], k2[kV], k3[kV];
+  float t0[V], t1[V], t2[V], t3[V];
+  bool k0[V], k1[V], k2[V], k3[V];
 #pragma unroll
-  for (int e = 0; e < kV; ++e) {
+  for (int e = 0; e < V; ++e) {
     t0[e] = t1[e] = t2[e] = t3[e] = 0.0f;
     k0[e] = k1[e] = k2[e] = k3[e] = true;
   }
@@ -316,7 +325,7 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_fmap(FMapArgs a) {
     const float imm = a.prog[pc].imm;
     if (op == FOP_IN || op == FOP_CONST) {
 #pragma unroll
-      for (int e = 0; e < kV; ++e) {
+      for (int e = 0; e < V; ++e) {
         t3[e] = t2[e];
         t2[e] = t1[e];
         t1[e] = t0[e];
@@ -331,7 +340,7 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_fmap(FMapArgs a) {
       }
     } else if (op == FOP_SELECT) {
 #pragma unroll
-      for (int e = 0; e < kV; ++e) {
+      for (int e = 0; e < V; ++e) {
         t0[e] = t2[e] != 0.0f ? t1[e] : t0[e];
         k0[e] = true;
         t1[e] = t3[e];
@@ -339,7 +348,7 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_fmap(FMapArgs a) {
       }
     } else if (op == FOP_MERGE) {
 #pragma unroll
-      for (int e = 0; e < kV; ++e) {
+      for (int e = 0; e < V; ++e) {
         t0[e] = k0[e] ? t0[e] : t1[e];
         k0[e] = k0[e] || k1[e];
         t1[e] = t2[e];
@@ -348,64 +357,110 @@ extern "C" __global__ __launch_bounds__(256) void hcamd_fmap(FMapArgs a) {
         k2[e] = k3[e];
       }
     } else if (op >= FOP_NEG) {
+      // one branch on the operation for all the elements of the lane: inside
+      // `each` the operation is a constant and the function's own switch folds
+      auto each = [&](auto tag) {
+        constexpr uint32_t OP = decltype(tag)::value;
 #pragma unroll
-      for (int e = 0; e < kV; ++e)
-        t0[e] = unary(op, t0[e], arg, k0[e]);
-    } else {
-#pragma unroll
-      for (int e = 0; e < kV; ++e) {
-        const bool second = k0[e] || (arg & 16u);
-        bool ok = k1[e] && second;
-        t0[e] = binary(op, t1[e], t0[e], arg, ok, !k1[e] && !second);
-        k0[e] = ok;
-        t1[e] = t2[e];
-        t2[e] = t3[e];
-        k1[e] = k2[e];
-        k2[e] = k3[e];
+        for (int e = 0; e < V; ++e)
+          t0[e] = unary(OP, t0[e], arg, k0[e]);
+      };
+#define HCAMD_FMAP_CASE(X)                                                       \
+  case X:                                                                        \
+    each(std::integral_constant<uint32_t, X>{});                                 \
+    break;
+      switch (op) {
+        HCAMD_FMAP_CASE(FOP_NEG) HCAMD_FMAP_CASE(FOP_ABS) HCAMD_FMAP_CASE(FOP_SQRT) HCAMD_FMAP_CASE(FOP_RINT)
+        HCAMD_FMAP_CASE(FOP_EXP) HCAMD_FMAP_CASE(FOP_LOG) HCAMD_FMAP_CASE(FOP_R16) HCAMD_FMAP_CASE(FOP_PSQRT)
+        HCAMD_FMAP_CASE(FOP_ACTIVE) HCAMD_FMAP_CASE(FOP_TANH) HCAMD_FMAP_CASE(FOP_FLOOR) HCAMD_FMAP_CASE(FOP_CEIL)
+        HCAMD_FMAP_CASE(FOP_TRUNC) HCAMD_FMAP_CASE(FOP_SIGN) HCAMD_FMAP_CASE(FOP_EXP2) HCAMD_FMAP_CASE(FOP_LOG2)
+        HCAMD_FMAP_CASE(FOP_LOG10) HCAMD_FMAP_CASE(FOP_LOG1P) HCAMD_FMAP_CASE(FOP_EXPM1) HCAMD_FMAP_CASE(FOP_SIN)
+        HCAMD_FMAP_CASE(FOP_COS) HCAMD_FMAP_CASE(FOP_RECIP)
+      default:
+        each(std::integral_constant<uint32_t, FOP_POWCHK>{});
+        break;
       }
+    } else {
+      auto each = [&](auto tag) {
+        constexpr uint32_t OP = decltype(tag)::value;
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          const bool second = k0[e] || (arg & 16u);
+          bool ok = k1[e] && second;
+          t0[e] = binary(OP, t1[e], t0[e], arg, ok, !k1[e] && !second);
+          k0[e] = ok;
+          t1[e] = t2[e];
+          t2[e] = t3[e];
+          k1[e] = k2[e];
+          k2[e] = k3[e];
+        }
+      };
+      switch (op) {
+        HCAMD_FMAP_CASE(FOP_ADD) HCAMD_FMAP_CASE(FOP_SUB) HCAMD_FMAP_CASE(FOP_MUL) HCAMD_FMAP_CASE(FOP_DIV)
+        HCAMD_FMAP_CASE(FOP_FLOORDIV) HCAMD_FMAP_CASE(FOP_MOD) HCAMD_FMAP_CASE(FOP_MIN) HCAMD_FMAP_CASE(FOP_MAX)
+        HCAMD_FMAP_CASE(FOP_UDIV) HCAMD_FMAP_CASE(FOP_LT) HCAMD_FMAP_CASE(FOP_LE) HCAMD_FMAP_CASE(FOP_EQ)
+        HCAMD_FMAP_CASE(FOP_NE) HCAMD_FMAP_CASE(FOP_GE)
+      default:
+        each(std::integral_constant<uint32_t, FOP_GT>{});
+        break;
+      }
+#undef HCAMD_FMAP_CASE
     }
   }
-  bool ok[kV];
+  bool ok[V];
 #pragma unroll
-  for (int e = 0; e < kV; ++e)
+  for (int e = 0; e < V; ++e)
     ok[e] = k0[e] || a.store_all != 0;
-  const bool all_ok = ok[0] && ok[1] && ok[2] && ok[3];
+  bool all_ok = true;
+#pragma unroll
+  for (int e = 0; e < V; ++e)
+    all_ok = all_ok && ok[e];
   if (a.out_type == 2) {
     uint8_t *o = static_cast<uint8_t *>(a.out) + row * a.ldo + col0;
 #pragma unroll
-    for (int e = 0; e < kV; ++e)
+    for (int e = 0; e < V; ++e)
       if (col0 + e < a.cols && ok[e])
         o[e] = (uint8_t)(t0[e] != 0.0f);
   } else if (a.out_type == 1) {
     _Float16 *o = static_cast<_Float16 *>(a.out) + row * a.ldo + col0;
     if (a.vec && whole && all_ok) {
-      f16x4 w;
 #pragma unroll
-      for (int e = 0; e < kV; ++e)
-        w[e] = (_Float16)t0[e];
-      *reinterpret_cast<f16x4 *>(o) = w;
+      for (int g = 0; g < V / 4; ++g) {
+        f16x4 w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          w[e] = (_Float16)t0[4 * g + e];
+        stg<true>(reinterpret_cast<f16x4 *>(o) + g, w);
+      }
     } else {
 #pragma unroll
-      for (int e = 0; e < kV; ++e)
+      for (int e = 0; e < V; ++e)
         if (col0 + e < a.cols && ok[e])
           o[e] = (_Float16)t0[e];
     }
   } else {
     float *o = static_cast<float *>(a.out) + row * a.ldo + col0;
     if (a.vec && whole && all_ok) {
-      f32x4 w;
 #pragma unroll
-      for (int e = 0; e < kV; ++e)
-        w[e] = t0[e];
-      *reinterpret_cast<f32x4 *>(o) = w;
+      for (int g = 0; g < V / 4; ++g) {
+        f32x4 w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          w[e] = t0[4 * g + e];
+        stg<true>(reinterpret_cast<f32x4 *>(o) + g, w);
+      }
     } else {
 #pragma unroll
-      for (int e = 0; e < kV; ++e)
+      for (int e = 0; e < V; ++e)
         if (col0 + e < a.cols && ok[e])
           o[e] = t0[e];
     }
   }
 }
+} // namespace
+extern "C" __global__ __launch_bounds__(256) void hcamd_fmap(FMapArgs a) { fmap_row_pieces<4>(a); }
+// eight elements of a lane to a dispatch, for rows of 2048 columns or more
+extern "C" __global__ __launch_bounds__(256) void hcamd_fmap_v8(FMapArgs a) { fmap_row_pieces<8>(a); }
 
 // ---- elementwise expressions of gathered tiles ------------------------------------
 // out_g[mo(e)] = f(in0_g[m0(e)], ...) for every group g and tile element e: what

@@ -1745,7 +1745,10 @@ int hcamdLaunchFMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
   a.vec = vec ? 1u : 0u;
   a.store_all = storeAll ? 1u : 0u;
   a.n_instr = (uint32_t)nInstr;
-  Kernel *k = builtinKernel(dev, "fmap", "hcamd_fmap");
+  // eight elements of a lane to a dispatch where the rows are long enough to
+  // give a workgroup its 2048 and move in whole pieces
+  const size_t perLane = vec && cols >= 2048 ? 8 : 4;
+  Kernel *k = builtinKernel(dev, "fmap", perLane == 8 ? "hcamd_fmap_v8" : "hcamd_fmap");
   if (!k)
     return 1;
   void *args[] = {&a};
@@ -1759,7 +1762,7 @@ int hcamdLaunchFMap(OlQueue q, const HcamdMapInstr *prog, size_t nInstr,
       a.in[i] = static_cast<const char *>(inputs[i]) +
                 r0 * inputLd[i] * (inputTypes[i] == HCAMD_F16 ? 2 : 4);
     a.out = static_cast<char *>(out) + r0 * ldo * outSize;
-    const size_t grid[3] = {ceilDiv(ceilDiv(cols, (size_t)4), (size_t)256), nr, 1};
+    const size_t grid[3] = {ceilDiv(ceilDiv(cols, perLane), (size_t)256), nr, 1};
     if (int rc = launch(queue, k, grid, block, args, 0))
       return rc;
   }
