@@ -1427,7 +1427,14 @@ def _compile_fmap(value, mapped=False):
         return None
     if not emit(value) or not loads:
         return None
-    if need(value) > 4:
+    # (the estimate, then the program as emitted: merges and selections of shared
+    # subexpressions can hold more entries than the tree's shape says)
+    depth = deepest = 0
+    for name, _, _ in program:
+        depth += 1 if name in ("in", "const") else -2 if name == "select" else \
+            -1 if name == "merge" or rt.FMAP_OPS[name] < rt.FMAP_OPS["neg"] else 0
+        deepest = max(deepest, depth)
+    if need(value) > 4 or deepest > 4:
         raise NoNativeKernel("float expression too deep for the four-entry stack of the general map")
     if len(program) > rt.FMAP_MAX_INSTRS:
         raise NoNativeKernel(f"float expression too long ({len(program)} operations, at most "

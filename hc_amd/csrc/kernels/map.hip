@@ -1245,6 +1245,15 @@ __device__ __forceinline__ void chain_plain(uint32_t op, float (&v)[NE], uint32_
   }
 }
 #undef HCAMD_CHAIN_EACH
+// an operation on a row scalar that numpy.ma would deactivate the result of
+__device__ __forceinline__ bool chain_scalar_fails(uint32_t op, float sv, float imm) {
+  return op == OP_MDIVI    ? !is_finite(sv / imm)
+         : op == OP_RMDIVI ? !is_finite(imm / sv)
+         : op == OP_MSQRT  ? sv < 0.0f
+         : op == OP_MLOG   ? sv <= 0.0f
+         : op == OP_POWCHK ? !is_finite(sv)
+                           : false;
+}
 // one instruction of a chain on one value (the stages that compute with row scalars)
 __device__ __forceinline__ void chain_scalar(uint32_t op, float &sv, float imm) {
   switch (op) {
@@ -1586,6 +1595,13 @@ struct RowArgs {
   uint32_t all_f32;         // chain kernels: every operand in use and the output are fp32
   Stage stage[kMaxStages];
   Instr prog[kRowProg];
+  // Two launches for programs whose row scalars can be deactivated (a quotient
+  // that is not finite, a root or a logarithm outside its domain): the chain
+  // kernels, which keep no such books, run every row, store nothing of a row on
+  // which an operation on a row scalar failed and say so in deferred[row]; the
+  // general kernel then runs the rows marked in only[] (the same array).
+  uint8_t *deferred;
+  const uint8_t *only;
 };
 
 struct NanMaxOp {
@@ -1931,7 +1947,9 @@ template <int LPR> __device__ __forceinline__ void row_program(const RowArgs &a)
   const uint32_t t = threadIdx.x, lane = t % LPR;
   float *cells = red_cells[t / kWave];
   const size_t row_at = (size_t)blockIdx.x * (kThreads / LPR) + t / LPR;
-  const bool row_live = row_at < a.rows;
+  const bool row_live = row_at < a.rows && (!a.only || a.only[row_at]);
+  if (LPR == kThreads && a.only && !row_live)
+    return; // (one row to a workgroup: the branch is uniform)
   const size_t row = row_live ? row_at : 0; // idle lanes compute on row 0 and store nothing
   const uint32_t whole = (uint32_t)(a.cols / kRowN), rem = (uint32_t)(a.cols % kRowN);
   const uint32_t per_row = whole + (rem ? 1u : 0u);
@@ -2255,6 +2273,7 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
 #pragma unroll
   for (int p = 0; p < P; ++p)
     live |= (row_live && (uint32_t)p * LPR + lane < per_row) ? 1u << p : 0u;
+  bool died = false; // an operation on a row scalar of this row failed (the same in every lane of the row)
   if (t % kWave < kMaxRed)
     cells[t % kWave] = 0.0f;
 #pragma unroll
@@ -2292,11 +2311,12 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
         uint32_t op;
         float imm;
         decode(cur, op, imm);
+        died = died || chain_scalar_fails(op, sv, imm);
         chain_scalar(op, sv, imm);
       }
       if (kind == ST_SCALAR)
         cells[st.dst & (kMaxRed - 1)] = uniform(sv);
-      else if (row_live && lane == 0)
+      else if (row_live && lane == 0 && !(a.deferred && died))
         store_elem(a.out, out_f16, row * a.ldo, sv);
       continue;
     }
@@ -2387,9 +2407,10 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
       uint32_t ln = lane, zero = 0;
       asm volatile("" : "+v"(zero), "+v"(ln));
       char *o = orow + zero;
+      const bool skip = a.deferred && died;
 #pragma unroll
       for (int p = 0; p < P; ++p)
-        if ((live >> p) & 1u) {
+        if (((live >> p) & 1u) && !skip) {
           const uint32_t c = (uint32_t)p * LPR + ln, none = (bad >> (8 * p)) & 0xffu;
           if (split(p)) { // fp32 output, two runs of four
             float *dst = reinterpret_cast<float *>(o);
@@ -2411,6 +2432,8 @@ template <int LPR, int P> __device__ __forceinline__ void row_chain(const RowArg
         }
     }
   }
+  if (a.deferred && row_live && lane == 0)
+    a.deferred[row_at] = died ? 1 : 0;
   } // turns
 }
 } // namespace

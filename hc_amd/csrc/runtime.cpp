@@ -75,6 +75,10 @@ struct Device {
   int index = 0;
   int computeUnits = 0; // filled in on first use
   bool colsKernelsReady = false; // the column-reduction kernels were resolved at creation
+  // one byte per row for the row programs that take two launches (which rows the
+  // first one left to the second); allocated on first use, grown when needed
+  void *rowMarks = nullptr;
+  size_t rowMarksBytes = 0;
   // built-in modules and kernels, loaded on first use
   std::unordered_map<std::string, hipModule_t> modules;
   std::unordered_map<std::string, struct Kernel *> kernels;
@@ -391,7 +395,10 @@ OlDevice olCreateDevice(const char *desc, OlErrorCallback errCallback,
 
 void olReleaseDevice(OlDevice dev) noexcept {
   OL_TRACE();
-  delete static_cast<Device *>(dev);
+  auto *device = static_cast<Device *>(dev);
+  if (device && device->rowMarks)
+    (void)hipFree(device->rowMarks);
+  delete device;
 }
 
 OlModule olCreateModule(OlDevice dev, const void *data,
@@ -2129,6 +2136,8 @@ struct RowArgs {
   uint32_t hold, holdLast, allF32;
   RowStageDev stage[HCAMD_ROW_MAX_STAGES];
   HcamdMapInstr prog[HCAMD_ROW_MAX_INSTRS];
+  uint8_t *deferred;   // chain kernels: one byte per row, 1 = left to the general kernel
+  const uint8_t *only; // general kernel: the rows to run (null: all)
 };
 
 // A stage program that never holds two values at once, as the chain kernels
@@ -2217,6 +2226,10 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
   uint32_t written = (1u << nColumns) - 1u;
   uint32_t deadable = 0;
   bool tracking = false; // some row scalar may be deactivated, or active elements are counted
+  // ... for a reason other than an operation on row scalars that can fail (a
+  // quotient, a root, a logarithm): counted folds, folds over elements that can be
+  // deactivated, frozen stores, per-row results that are tiles
+  bool trackingBeyondScalars = false;
   uint32_t usedIn[HCAMD_ROW_MAX_STAGES] = {};
   size_t pc = 0;
   for (size_t s = 0; s < nStages; ++s) {
@@ -2344,6 +2357,9 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
     tracking = tracking || canDie || frozen || st.kind == HCAMD_ROW_COUNT ||
                (st.kind == HCAMD_ROW_STORE_COL && st.dst != 0) ||
                (!perElement && (hasForms || readsDeadable));
+    trackingBeyondScalars = trackingBeyondScalars || frozen || st.kind == HCAMD_ROW_COUNT ||
+                            (st.kind == HCAMD_ROW_STORE_COL && st.dst != 0) ||
+                            (perElement && !stores && hasForms) || a.stage[s].livePos != 0xff;
     pc += st.nInstr;
   }
   std::memcpy(a.prog, prog, pc * sizeof(HcamdMapInstr));
@@ -2514,7 +2530,18 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
   // instructions read stays in LDS for the row (variant 1 of "rows": never).
   size_t lanes = lanesPerRow, maxGroups = SIZE_MAX, threads = 256;
   std::snprintf(name, sizeof name, "hcamd_row_program_w%zu", lanes);
-  if (variantOf("rows") != 1 && !tracking && !a.interleaved && cols % 8 == 0 && perRow <= 4096 &&
+  // A program whose only deactivations are failed operations on row scalars
+  // takes two launches: the chain kernel for every row, which leaves a row alone
+  // and marks it when such an operation fails on it, then the general kernel for
+  // the marked rows (variant 3 of "rows": the general kernel alone, as for
+  // every other program that needs the books).
+  const bool twoLaunches = tracking && !trackingBeyondScalars && variantOf("rows") == 0;
+  RowArgs general = a;
+  char generalName[64];
+  std::snprintf(generalName, sizeof generalName, "%s", name);
+  const size_t generalLanes = lanes;
+  bool chainTaken = false;
+  if (variantOf("rows") != 1 && (!tracking || twoLaunches) && !a.interleaved && cols % 8 == 0 && perRow <= 4096 &&
       nInputs > 0) {
     HcamdMapInstr chained[HCAMD_ROW_MAX_INSTRS];
     size_t nChained = 0;
@@ -2565,7 +2592,27 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
       std::snprintf(name, sizeof name, "hcamd_row_program_chain_w%zu_p%u", lanes, p);
       // these kernels walk the rows themselves: as many workgroups as are resident at once
       maxGroups = (size_t)computeUnitsOf(dev) * (p <= 2 ? 24 : 16) / (threads / 64); // 6 or 4 waves per SIMD
+      chainTaken = true;
     }
+  }
+  if (tracking && !chainTaken) // (the rewrite above is for the chain kernels only)
+    a = general;
+  if (tracking && chainTaken) {
+    // one byte per row, kept with the device and grown when a launch has more rows
+    if (dev->rowMarksBytes < rows) {
+      if (dev->rowMarks)
+        (void)hipFree(dev->rowMarks);
+      dev->rowMarks = nullptr;
+      dev->rowMarksBytes = 0;
+      const size_t want = std::max(rows, (size_t)1 << 16);
+      if (hipMalloc(&dev->rowMarks, want) != hipSuccess) {
+        dev->report("%s: no device memory for %zu row marks", who, want);
+        return 1;
+      }
+      dev->rowMarksBytes = want;
+    }
+    a.deferred = static_cast<uint8_t *>(dev->rowMarks);
+    general.only = static_cast<const uint8_t *>(dev->rowMarks);
   }
   Kernel *k = builtinKernel(dev, "map", name);
   if (!k)
@@ -2573,7 +2620,17 @@ int hcamdLaunchRowProgram(OlQueue q, const HcamdMapInstr *prog,
   void *args[] = {&a};
   const size_t grid[3] = {std::min(ceilDiv(rows, threads / lanes), maxGroups), 1, 1};
   const size_t block[3] = {threads, 1, 1};
-  return launch(queue, k, grid, block, args, 0);
+  if (int rc = launch(queue, k, grid, block, args, 0))
+    return rc;
+  if (!(tracking && chainTaken))
+    return 0;
+  Kernel *kg = builtinKernel(dev, "map", generalName);
+  if (!kg)
+    return 1;
+  void *gargs[] = {&general};
+  const size_t ggrid[3] = {ceilDiv(rows, (size_t)256 / generalLanes), 1, 1};
+  const size_t gblock[3] = {256, 1, 1};
+  return launch(queue, kg, ggrid, gblock, gargs, 0);
 }
 
 int hcamdLaunchPairwiseDistF32(OlQueue q, const float *a, size_t lda,

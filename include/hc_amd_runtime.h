@@ -589,8 +589,13 @@ int hcamdLaunchMapReduceColsNoAlloc(OlQueue q, int kind, const HcamdMapInstr *pr
  * rows of whole chunks of 8 elements, at most 32768 elements, run on kernels that
  * take a lane's whole part of the row at once: the operand most instructions
  * read is fetched once per row (into LDS), and an instruction is dispatched
- * once for 8, 16 or 32 elements of a lane (variant 1 of the "rows" family keeps
- * the general kernel).  One program has a kernel of its own that interprets
+ * once for 8, 16 or 32 elements of a lane; a program in which only operations
+ * on row scalars can deactivate anything (a quotient, a root, a logarithm, a
+ * power) runs there too, followed by a launch of the general kernel for the
+ * rows on which one did, which the first launch leaves untouched and marks in
+ * a byte array the device keeps (variant 3 of "rows": the general kernel alone
+ * for such programs; variant 1 of the "rows" family keeps the general kernel
+ * for every program).  One program has a kernel of its own that interprets
  * nothing: the layer normalisation (x - mean) / sqrt(var + eps) * w + b in the
  * six stages the front-end emits for it (sum; RED MDIVI; the sum of the
  * centred squares; RED0 DIVI; RED ADDI MSQRT; IN SUB_RED MDIV_RED MUL_IN
