@@ -593,7 +593,10 @@ int hcamdLaunchMapReduceColsNoAlloc(OlQueue q, int kind, const HcamdMapInstr *pr
  * on row scalars can deactivate anything (a quotient, a root, a logarithm, a
  * power) runs there too, followed by a launch of the general kernel for the
  * rows on which one did, which the first launch leaves untouched and marks in
- * a byte array the device keeps (variant 3 of "rows": the general kernel alone
+ * a byte array the device keeps (one byte per row, at least 64 KiB: the first
+ * such launch on a device allocates it with hipMalloc and a launch with more
+ * rows than any before replaces it, so callers that cannot allocate, a stream
+ * under capture among them, select variant 3 of "rows": the general kernel alone
  * for such programs; variant 1 of the "rows" family keeps the general kernel
  * for every program).  One program has a kernel of its own that interprets
  * nothing: the layer normalisation (x - mean) / sqrt(var + eps) * w + b in the
