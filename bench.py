@@ -584,6 +584,33 @@ def make_workloads(rt, wl):
         def cpu(self):
             return _best_of(lambda: self._numpy(self.x), 2), "full size, NumPy fp32", 1
 
+    class X10(Workload):
+        """Log-softmax over the rows of the C3 matrix, written as a kernel body and launched through
+        the @kernel front-end: a row program with a logarithm of a row scalar, which runs as two
+        launches (the chain kernel for every row, the general kernel for rows it left alone)."""
+
+        def setup(self, rt):
+            from hc_amd.examples import log_softmax
+            self.kernel = log_softmax()
+            (self.x,) = W.inputs_c3()
+            return [(rt.to_device(self.x), rt.DeviceArray(self.x.shape, np.float32)) for _ in range(ROTATE)]
+
+        def plan(self, rt, s):
+            (p,) = self.kernel.plan_rows(*s)
+            return p
+
+        def _numpy(self, x):
+            c = x - x.max(axis=1, keepdims=True)
+            return c - np.log(np.exp(c).sum(axis=1, keepdims=True))
+
+        def check(self, rt, s):
+            got, want = s[1].to_host(), self._numpy(self.x.astype(np.float64))
+            ok = np.allclose(got, want, rtol=2e-5, atol=2e-5)
+            return {"parity": "rtol 2e-5, atol 2e-5 vs fp64" if ok else "MISMATCH", "ok": bool(ok)}
+
+        def cpu(self):
+            return _best_of(lambda: self._numpy(self.x), 2), "full size, NumPy fp32", 1
+
     class X8(Workload):
         """Root-mean-square normalisation with an fp32 weight over the rows of the C4
         matrix (fp16 in, fp32 math, fp16 out), written as a kernel body and
@@ -639,6 +666,8 @@ def make_workloads(rt, wl):
                  W.work_c1(), "GB/s"),
         "x8": X8("x8", "row program: rms norm fp16 16384x4096 with an fp32 weight (fp32 math)", "f16", "hbm",
                  2 * 2 * 16384 * 4096 + 4 * 4096, "GB/s"),
+        "x10": X10("x10", "row program: log-softmax fp32 4096x8192 (two launches)", "f32", "hbm",
+                   W.work_c3(), "GB/s"),
         "x9": X9("x9", "map kernel: a 9-instruction chain on the fp16 8191x8193 arrays", "f16", "hbm",
                  W.work_c2(), "GB/s"),
     }
@@ -650,7 +679,7 @@ def make_workloads(rt, wl):
     elif wl == "streams":
         keys = [k for k, *_ in STREAMS]
     elif wl == "extra":
-        keys = ["x1", "x2", "x3", "x4", "x5", "x6", "x7", "x8", "x9"]
+        keys = ["x1", "x2", "x3", "x4", "x5", "x6", "x7", "x8", "x9", "x10"]
     else:
         keys = [wl]
     return [table[k] for k in keys]
@@ -725,7 +754,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="all", choices=["all", "streams", "c0", "c1", "c2", "c3", "c4", "c5", "v5", "extra", "x1", "x2", "x3",
-                             "x4", "x5", "x6", "x7", "x8", "x9"] + [k for k, *_ in STREAMS])
+                             "x4", "x5", "x6", "x7", "x8", "x9", "x10"] + [k for k, *_ in STREAMS])
     ap.add_argument("--no-cpu", action="store_true", help="skip the NumPy CPU baseline")
     ap.add_argument("--variant", action="append", default=[], metavar="FAMILY=N",
                     help="measure kernel variant N of a family (hcamdSetVariant), e.g. gemm=14; "

@@ -69,6 +69,26 @@ def layer_norm(eps: float = 1e-5, rows_per_group: int = 8):
     return body
 
 
+def log_softmax(rows_per_group: int = 8):
+    """out = (x - max(x)) - log(sum(exp(x - max(x)))) along the rows of a float32
+    matrix: a row program in which a NumPy function of a row scalar (the
+    logarithm of the sum, which numpy.ma deactivates outside its domain) stands
+    between the reductions and the store."""
+    M, N, GM = sym.M, sym.N, sym.GM
+
+    @kernel(work_shape=M, group_shape=GM)
+    def body(gr: CurrentGroup, x: Buffer[M, N, DT], out: Buffer[M, N, DT], gshape: GM):
+        m0, mb = gr.work_offset[0], gr.shape[0]
+        t = gr.load(x[m0:, :], shape=(mb, N))
+        c = t - t.max(axis=1, keepdims=True)
+        gr.store(out[m0:, :], c - np.log(np.exp(c).sum(axis=1, keepdims=True)))
+
+    def plan(x, out, **kw):
+        return body.plan(x, out, rows_per_group, **kw)
+    body.plan_rows = plan
+    return body
+
+
 def rms_norm_f16(eps: float = 1e-6, rows_per_group: int = 8):
     """out = x / sqrt(mean(x * x) + eps) * weight along the rows of a float16
     matrix, computed in float32 (the weight is float32) and stored as float16:
